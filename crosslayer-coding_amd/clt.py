@@ -1,0 +1,363 @@
+"""CrossLayerTranscoder for one MI355X.
+
+Drop-in for the forward path of the reference class (clt/models/clt.py:22-425): same
+constructor, ``encode`` / ``decode`` / ``forward`` / ``get_feature_activations`` /
+``get_preactivations`` / ``_encode_all_layers`` / ``get_decoder_norms`` / ``jumprelu``,
+same sub-module and parameter names (so ``state_dict()`` and safetensors checkpoints are
+interchangeable), same log-and-return-zeros handling of bad inputs.
+
+``forward`` never materialises dense activations: one MFMA launch projects all layers,
+the selection kernels turn the pre-activations into survivor lists, and the sparse
+decoder writes every target layer.  ``get_feature_activations`` densifies those lists
+because its callers index [tokens, features] tensors.
+
+The kernels implement inference: results carry no autograd graph.
+"""
+
+from __future__ import annotations
+
+import logging
+from typing import Any, Dict, List, Optional, Tuple, Union
+
+import torch
+
+from . import _native as nat
+from . import engine
+from .activations import resolve_token_k
+from .base import BaseTranscoder
+from .config import CLTConfig
+from .decoder import Decoder
+from .encoder import Encoder
+from .engine import SurvivorList, Workspace
+from .parallel import require_single_rank
+from .registry import get_activation_fn
+from .theta import ThetaManager
+
+logger = logging.getLogger(__name__)
+
+
+class _NullTimer:
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        return False
+
+
+class CrossLayerTranscoder(BaseTranscoder):
+    device: torch.device
+    dtype: torch.dtype
+
+    def __init__(self, config: CLTConfig, process_group=None, device: Optional[torch.device] = None,
+                 profiler: Optional[Any] = None):
+        super().__init__(config)
+        require_single_rank(process_group)
+        self.process_group = process_group
+        self.world_size, self.rank = 1, 0
+        self.profiler = profiler
+        self.dtype = self._resolve_dtype(config.clt_dtype)
+        if device is not None:
+            self.device = torch.device(device)
+        else:
+            self.device = torch.device("cuda" if torch.cuda.is_available() else "cpu")
+        logger.info(f"CLT TP model initialized on rank {self.rank} with device {self.device} and dtype {self.dtype}")
+        self.encoder_module = Encoder(config, process_group, self.device, self.dtype)
+        self.decoder_module = Decoder(config, process_group, self.device, self.dtype)
+        self.theta_manager = ThetaManager(config, process_group, self.device, self.dtype)
+        self._ws: Optional[Workspace] = None
+
+    # ---- small helpers ---------------------------------------------------------------
+    def _resolve_dtype(self, dtype_input: Optional[Union[str, torch.dtype]]) -> torch.dtype:
+        if isinstance(dtype_input, torch.dtype):
+            return dtype_input
+        if isinstance(dtype_input, str):
+            cand = getattr(torch, dtype_input, None)
+            if isinstance(cand, torch.dtype):
+                return cand
+            logger.warning(f"Unsupported CLT dtype string: '{dtype_input}'. Defaulting to float32.")
+        return torch.float32
+
+    def _workspace(self) -> Workspace:
+        dev = self.encoder_module.encoders[0].weight.device
+        if self._ws is None or self._ws.device != dev:
+            self._ws = Workspace(dev)
+        return self._ws
+
+    def _timed(self, name: str):
+        return self.profiler.timer(name) if self.profiler else _NullTimer()
+
+    def _record(self, name: str, timer) -> None:
+        if self.profiler and hasattr(timer, "elapsed"):
+            self.profiler.record(name, timer.elapsed)
+
+    def _sync_device(self) -> None:
+        """Follow the parameters after ``module.to(...)``."""
+        w = self.encoder_module.encoders[0].weight
+        if w.device != self.device or w.dtype != self.dtype:
+            self.device, self.dtype = w.device, w.dtype
+            for m in (self.encoder_module, self.decoder_module, self.theta_manager):
+                m.device, m.dtype = w.device, w.dtype
+
+    def release_workspace(self) -> None:
+        """Free the cached scratch buffers (pre-activations, selection workspace)."""
+        if self._ws is not None:
+            self._ws.release()
+
+    # ---- reference API: thin delegations ------------------------------------------------
+    def jumprelu(self, x: torch.Tensor, layer_idx: int) -> torch.Tensor:
+        return self.theta_manager.jumprelu(x, layer_idx)
+
+    def get_preactivations(self, x: torch.Tensor, layer_idx: int) -> torch.Tensor:
+        self._sync_device()
+        return self.encoder_module.get_preactivations(x, layer_idx)
+
+    def _encode_all_layers(self, inputs: Dict[int, torch.Tensor]
+                           ) -> Tuple[Dict[int, torch.Tensor], List[Tuple[int, int, int]]]:
+        self._sync_device()
+        return self.encoder_module.encode_all_layers(inputs)
+
+    def decode(self, a: Dict[int, torch.Tensor], layer_idx: int,
+               source_inputs: Optional[Dict[int, torch.Tensor]] = None) -> torch.Tensor:
+        self._sync_device()
+        return self.decoder_module.decode(a, layer_idx, source_inputs)
+
+    def get_decoder_norms(self) -> torch.Tensor:
+        self._sync_device()
+        return self.decoder_module.get_decoder_norms()
+
+    @property
+    def log_threshold(self) -> Optional[torch.nn.Parameter]:
+        tm = getattr(self, "theta_manager", None)
+        return tm.log_threshold if tm is not None else None
+
+    @log_threshold.setter
+    def log_threshold(self, new_param: Optional[torch.nn.Parameter]) -> None:
+        if getattr(self, "theta_manager", None) is None:
+            raise AttributeError("ThetaManager is not initialised; cannot set log_threshold.")
+        self.theta_manager.log_threshold = new_param
+
+    def estimate_theta_posthoc(self, *args, **kwargs):
+        return self.theta_manager.estimate_theta_posthoc(*args, **kwargs)
+
+    def convert_to_jumprelu_inplace(self, *args, **kwargs):
+        return self.theta_manager.convert_to_jumprelu_inplace(*args, **kwargs)
+
+    # ---- encode (per-layer activations) ---------------------------------------------------
+    def encode(self, x: torch.Tensor, layer_idx: int) -> torch.Tensor:
+        """Activations [tokens, F] of one layer for relu / jumprelu; for the top-k family the
+        reference logs an error and returns zeros here (clt.py:135-149), and so does this."""
+        self._sync_device()
+        x = x.to(device=self.device, dtype=self.dtype)
+        preact = self.get_preactivations(x, layer_idx)
+        F = self.config.num_features
+
+        def zeros(rows: int) -> torch.Tensor:
+            return torch.zeros((rows, F), device=self.device, dtype=self.dtype)
+
+        if preact.numel() == 0:
+            logger.warning(f"Rank {self.rank}: Received empty preactivations for encode layer {layer_idx}.")
+            rows = x.shape[0] if x.dim() == 2 else x.shape[0] * x.shape[1] if x.dim() == 3 else 0
+            return zeros(rows)
+        if preact.shape[-1] != F:
+            logger.warning(
+                f"Rank {self.rank}: Received invalid preactivations shape {preact.shape} for encode layer {layer_idx}.")
+            return zeros(preact.shape[0])
+        fn = self.config.activation_fn
+        try:
+            if fn == "jumprelu":
+                return self.theta_manager.jumprelu(preact, layer_idx)
+            if fn == "relu":
+                return get_activation_fn("relu")(self, preact, layer_idx)
+            logger.error(
+                f"Rank {self.rank}: Unsupported activation function '{fn}' encountered in encode method path. "
+                f"Expected jumprelu or relu.")
+        except ValueError as e:
+            logger.error(f"Rank {self.rank}: Error getting activation function '{fn}' for layer {layer_idx}: {e}")
+        return zeros(preact.shape[0])
+
+    # ---- survivors: the fused encode + select ------------------------------------------------
+    def _select(self, pre: torch.Tensor) -> SurvivorList:
+        """Selection over a slab pre [n, T, F] of the layers present, per the config."""
+        cfg = self.config
+        ws = self._workspace()
+        fn = cfg.activation_fn
+        glob = cfg.topk_mode != "per_layer"
+        if fn == "batchtopk":
+            with self._timed("batchtopk_activation") as tm:
+                surv = engine.batchtopk_select(pre, int(cfg.batchtopk_k), glob, ws)
+            self._record("batchtopk_activation", tm)
+            return surv
+        if fn == "topk":
+            n, _, F = pre.shape
+            kk = resolve_token_k(float(cfg.topk_k), n * F if glob else F)
+            with self._timed("topk_activation") as tm:
+                surv = engine.tokentopk_select(pre, kk, glob, ws)
+            self._record("topk_activation", tm)
+            return surv
+        raise AssertionError(fn)
+
+    def _survivors(self, inputs: Dict[int, torch.Tensor]):
+        """(layers, T, survivor list over those layers) or None when the inputs need the
+        reference's per-layer fallbacks."""
+        self._sync_device()
+        cfg = self.config
+        layers = sorted(inputs.keys())
+        if not layers:
+            return None
+        fn = cfg.activation_fn
+        # pre-activation slab: reused scratch, it never leaves this function
+        x0 = inputs[layers[0]]
+        if x0.dim() not in (2, 3):
+            return None
+        T = x0.shape[0] if x0.dim() == 2 else x0.shape[0] * x0.shape[1]
+        n = len(layers)
+        ws = self._workspace()
+        pre_buf = ws.typed("pre", (n, T, cfg.num_features), self.dtype) if T > 0 else None
+        slab = self.encoder_module.encode_slab(inputs, out=pre_buf)
+        if slab is None:
+            return None
+        _, pre = slab
+        if fn in ("batchtopk", "topk"):
+            surv = self._select(pre)
+        elif fn == "jumprelu":
+            theta = self.theta_manager.thresholds(self.dtype)
+            if layers != list(range(cfg.num_layers)):
+                theta = theta.index_select(0, torch.tensor(layers, device=theta.device)).contiguous()
+            surv = engine.threshold_select(pre, theta, nat.PRED_GE_THETA, ws)
+        elif fn == "relu":
+            surv = engine.threshold_select(pre, None, nat.PRED_GT_ZERO, ws)
+        else:
+            return None
+        return layers, T, surv
+
+    def _expand_layers(self, layers: List[int], surv: SurvivorList) -> SurvivorList:
+        """Re-index a list over the present layers to all num_layers (absent layers: empty rows)."""
+        L, T = self.config.num_layers, surv.T
+        if layers == list(range(L)):
+            return surv
+        counts = torch.zeros(L * T, dtype=torch.int64, device=surv.row_ptr.device)
+        per_row = (surv.row_ptr[1:] - surv.row_ptr[:-1]).to(torch.int64)
+        for i, l in enumerate(layers):
+            counts[l * T:(l + 1) * T] = per_row[i * T:(i + 1) * T]
+        row_ptr = torch.zeros(L * T + 1, dtype=torch.int32, device=counts.device)
+        row_ptr[1:] = torch.cumsum(counts, 0).to(torch.int32)
+        return SurvivorList(row_ptr, surv.col, surv.val, T, surv.F, L, surv.dtype)
+
+    # ---- get_feature_activations -------------------------------------------------------------
+    def get_feature_activations(self, inputs: Dict[int, torch.Tensor]) -> Dict[int, torch.Tensor]:
+        """Dense activations per layer (clt.py:220-277)."""
+        self._sync_device()
+        cfg = self.config
+        topk_family = cfg.activation_fn in ("batchtopk", "topk")
+        res = self._survivors(inputs)
+        if res is not None:
+            layers, T, surv = res
+            dense = engine.densify(surv, out_f32=(cfg.activation_fn == "jumprelu"))
+            return {l: dense[i] for i, l in enumerate(layers)}
+        # inputs that need the per-layer fallbacks
+        proc = {l: x.to(device=self.device, dtype=self.dtype) for l, x in inputs.items()}
+        if not topk_family:
+            return {l: self.encode(proc[l], l) for l in sorted(proc.keys())}
+        return self._topk_from_preacts(inputs, proc)
+
+    def _topk_from_preacts(self, inputs, proc) -> Dict[int, torch.Tensor]:
+        """Top-k family when some layer took a fallback: follows the helper's zero-filling of
+        empty or mismatched layers (activations.py:250-297) on a stacked copy."""
+        cfg = self.config
+        F = cfg.num_features
+        pre_dict, _ = self._encode_all_layers(proc)
+        if not pre_dict:
+            out = {}
+            for l, x in inputs.items():
+                rows = x.shape[0] * x.shape[1] if x.dim() == 3 else x.shape[0] if x.dim() == 2 else 0
+                out[l] = torch.zeros((rows, F), device=self.device, dtype=self.dtype)
+            return out
+        first = next((p for p in pre_dict.values() if p.numel() > 0), None)
+        if first is None:
+            logger.warning(f"Rank {self.rank}: No valid preactivations found in dict for BatchTopK. Returning empty dict.")
+            return {l: torch.empty((0, F), device=self.device, dtype=self.dtype) for l in pre_dict}
+        T = first.shape[0]
+        layers = [l for l in range(cfg.num_layers) if l in pre_dict]
+        slabs = []
+        for l in layers:
+            p = pre_dict[l]
+            if p.numel() == 0:
+                p = torch.zeros((T, F), device=self.device, dtype=self.dtype)
+            elif p.shape[0] != T:
+                logger.warning(
+                    f"Rank {self.rank} Layer {l}: Mismatched batch dim ({p.shape[0]} vs {T}). Using zeros.")
+                p = torch.zeros((T, F), device=self.device, dtype=self.dtype)
+            slabs.append(p)
+        if not layers:
+            return {l: torch.empty((T, F), device=self.device, dtype=self.dtype) for l in pre_dict}
+        pre = torch.stack(slabs).contiguous()
+        dense = engine.densify(self._select(pre))
+        return {l: dense[i] for i, l in enumerate(layers)}
+
+    # ---- forward ---------------------------------------------------------------------------
+    def forward(self, inputs: Dict[int, torch.Tensor]) -> Dict[int, torch.Tensor]:
+        """Reconstruction of every layer present in ``inputs`` (clt.py:186-218)."""
+        self._sync_device()
+        cfg = self.config
+        L, d = cfg.num_layers, cfg.d_model
+        res = self._survivors(inputs)
+        if res is not None:
+            layers, T, surv = res
+            full = self._expand_layers(layers, surv)
+            src_mask = 0
+            for l in layers:
+                src_mask |= 1 << l
+            skip = (self.decoder_module.skip_all_targets(inputs, src_mask, T) if cfg.skip_connection else None)
+            targets = [t for t in range(L) if t in inputs]
+            out = self.decoder_module.decode_survivors(full, src_mask, min(targets), max(targets) + 1, skip_add=skip)
+            return {t: out[t] for t in targets}
+        # fallback wiring over dense activations
+        acts = self.get_feature_activations(inputs)
+        recs: Dict[int, torch.Tensor] = {}
+        for t in range(L):
+            rel = {s: v for s, v in acts.items() if s <= t and v.numel() > 0}
+            if t in inputs and rel:
+                src = {s: inputs[s] for s in range(t + 1) if s in inputs} if cfg.skip_connection else None
+                recs[t] = self.decode(rel, t, src)
+            elif t in inputs:
+                x = inputs[t]
+                rows = 0
+                if x.dim() >= 1:
+                    rows = x.shape[0] * x.shape[1] if x.dim() == 3 else x.shape[0]
+                else:
+                    logger.warning(
+                        f"Rank {self.rank}: Could not determine batch size for fallback tensor in forward layer "
+                        f"{t} from input shape {x.shape}. Using 0.")
+                recs[t] = torch.zeros((rows, d), device=self.device, dtype=self.dtype)
+        return recs
+
+    # ---- checkpoints -----------------------------------------------------------------------
+    def load_state_dict(self, state_dict: Dict[str, torch.Tensor], strict: bool = True):
+        """nn.Module.load_state_dict plus the reference's migrations (clt.py:347-425): an untied
+        checkpoint loaded into a per_source model keeps the diagonal "s->s" decoders, and
+        feature_offset / feature_scale saved under encoder_module move to decoder_module."""
+        sd = dict(state_dict)
+        if self.config.decoder_tying == "per_source" and any("decoders." in k and "->" in k for k in sd):
+            logger.warning(
+                "Loading old untied decoder checkpoint into tied decoder model. "
+                "This will use weights from the first target layer for each source layer.")
+            new_sd = {}
+            for k, v in sd.items():
+                if "decoders." in k and "->" in k:
+                    parts = k.split(".")
+                    i = parts.index("decoders") + 1
+                    s, t = (int(p) for p in parts[i].split("->"))
+                    if s == t:
+                        new_sd[".".join(parts[:i] + [str(s), parts[-1]])] = v
+                else:
+                    new_sd[k] = v
+            sd = new_sd
+        for i in range(self.config.num_layers):
+            for name in ("feature_offset", "feature_scale"):
+                old, new = f"encoder_module.{name}.{i}", f"decoder_module.{name}.{i}"
+                if old in sd and new not in sd:
+                    logger.info(f"Migrating {old} to {new}")
+                    sd[new] = sd.pop(old)
+        result = super().load_state_dict(sd, strict=strict)
+        self.decoder_module.invalidate_packed()
+        return result

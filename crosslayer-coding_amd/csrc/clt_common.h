@@ -1,0 +1,84 @@
+// Shared device/host helpers for the gfx950 CLT kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "../../include/clt_hip.h"
+
+#define CLT_WAVE 64
+
+typedef uint16_t bf16_t;  // raw bfloat16 bits
+
+// ---------------------------------------------------------------- conversions
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) {
+  return __uint_as_float(b << 16);
+}
+
+// round-to-nearest-even, NaN kept quiet (same rule torch uses for float->bfloat16)
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return u >> 16;
+}
+
+__device__ __forceinline__ float round_to_bf16(float f) {
+  return bf16_bits_to_f32(f32_to_bf16_bits(f));
+}
+
+// Element traits: T is float or bf16_t (raw bits).
+template <typename T> struct Elem;
+template <> struct Elem<float> {
+  static constexpr int VEC = 4;       // elements per 16-byte vector
+  static constexpr int KEYBITS = 32;  // bits of the ranking key
+  __device__ static __forceinline__ float to_f32(float v) { return v; }
+  __device__ static __forceinline__ float from_f32(float v) { return v; }
+  __device__ static __forceinline__ float round(float v) { return v; }
+  __device__ static __forceinline__ uint32_t raw(float v) { return __float_as_uint(v); }
+  __device__ static __forceinline__ float from_raw(uint32_t r) { return __uint_as_float(r); }
+};
+template <> struct Elem<bf16_t> {
+  static constexpr int VEC = 8;
+  static constexpr int KEYBITS = 16;
+  __device__ static __forceinline__ float to_f32(bf16_t v) { return bf16_bits_to_f32(v); }
+  __device__ static __forceinline__ bf16_t from_f32(float v) { return (bf16_t)f32_to_bf16_bits(v); }
+  __device__ static __forceinline__ float round(float v) { return round_to_bf16(v); }
+  __device__ static __forceinline__ uint32_t raw(bf16_t v) { return v; }
+  __device__ static __forceinline__ bf16_t from_raw(uint32_t r) { return (bf16_t)r; }
+};
+
+// ---------------------------------------------------------------- ranking keys
+// Order-preserving unsigned key: ascending float order, -0.0 == +0.0, NaN on top.
+__device__ __forceinline__ uint32_t rank_key32(float x) {
+  uint32_t u = __float_as_uint(x);
+  if (x != x) return 0xFFFFFFFFu;
+  if (u == 0x80000000u) u = 0u;
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+// Key of width KB (16: for values that are exactly representable in bf16).
+template <int KB> __device__ __forceinline__ uint32_t rank_key(float x) {
+  return KB == 32 ? rank_key32(x) : (rank_key32(x) >> 16);
+}
+// Float whose key is `key` (the lowest such float for 16-bit keys).
+template <int KB> __device__ __host__ __forceinline__ uint32_t key_to_f32_bits(uint32_t key) {
+  uint32_t k32 = KB == 32 ? key : ((key << 16) | ((key & 0x8000u) ? 0u : 0xFFFFu));
+  return (k32 & 0x80000000u) ? (k32 & 0x7FFFFFFFu) : ~k32;
+}
+
+// ---------------------------------------------------------------- wave helpers
+__device__ __forceinline__ int lane_id() { return threadIdx.x & (CLT_WAVE - 1); }
+
+// number of set bits of `mask` strictly below this lane
+__device__ __forceinline__ uint32_t mbcnt64(uint64_t mask) {
+  return __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32),
+                                   __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
+}
+
+__device__ __forceinline__ uint64_t ballot64(bool p) { return __ballot(p); }
+
+// ---------------------------------------------------------------- host helpers
+static inline int clt_check_launch() {
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? CLT_OK : CLT_ERR_LAUNCH;
+}
+static inline bool clt_aligned16(const void *p) { return (((uintptr_t)p) & 15u) == 0; }
+static inline int64_t clt_ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }

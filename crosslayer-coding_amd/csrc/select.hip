@@ -1,0 +1,771 @@
+// BatchTopK selection and threshold activations -> compact survivor lists.
+//
+// BatchTopK (reference clt/models/activations.py:11-36, 261-357) is an exact
+// "K largest of N" with deterministic ties.  N is 1e8..1e9 and K is ~1 % of it, so
+// the work is one streaming read of the pre-activations:
+//
+//   sample   a hashed sample of the ranking values gives a conservative cut key
+//            (about 2x K elements lie above it);
+//   pass     ONE read of every row (one wavefront per row, 16-byte loads): elements
+//            at or above the cut are appended, in column order (wave ballot +
+//            mbcnt prefix), to a per-row candidate segment and counted into an LDS
+//            histogram of (key - cut);
+//   scan     a single block walks the histogram from the top and finds the bin that
+//            holds the K-th largest key; bins are one key wide near the cut (16-bit
+//            keys) so this usually ends the search, otherwise further levels
+//            re-histogram the candidates only;
+//   count / allot / emit   work on the candidate segments: survivors per row, the
+//            tie budget handed out in flat-index order, then the ordered write of
+//            (feature, value) pairs.
+//
+// A row whose candidates overflow its segment is re-read from the dense matrix by
+// the later stages, and a cut that turns out too high (fewer than K candidates)
+// makes the pass run again with the lowest cut, so the result is exact for any
+// input; only the speed depends on the sample being representative.
+#include "clt_common.h"
+
+namespace {
+
+constexpr int NBINS = 2048;
+constexpr uint32_t FINE16 = 1984;  // 16-bit keys: bins [0,FINE16) are one key wide
+constexpr int SAMPLE_N = 16384;
+constexpr int SCAN_THREADS = 1024;
+
+enum : uint32_t { ST_RUN = 0, ST_RETRY = 1, ST_DONE = 2 };
+
+struct SelState {
+  uint32_t cut_key;   // candidates have key >= cut_key
+  uint32_t status;    // ST_*
+  uint32_t level;     // level whose histogram is being accumulated
+  uint32_t flo, fhi;  // levels >= 1: inclusive range of (key - cut_key) still in play
+  uint32_t bbase;     // levels >= 1: bin = (diff - bbase) >> shift
+  uint32_t shift;
+  uint32_t thr_key;   // result: key of the K-th largest element
+  unsigned long long k_rem;       // still to take from the active range
+  unsigned long long tie_budget;  // result: how many elements equal to thr_key survive
+};
+
+template <int KB> __device__ __forceinline__ uint32_t min_key() {
+  return KB == 32 ? 0x007FFFFFu : 0x007Fu;  // key(-inf); nothing ranks below it
+}
+template <int KB> __device__ __forceinline__ uint32_t bin_level0(uint32_t diff) {
+  if (KB == 16) return diff < FINE16 ? diff : FINE16 + (diff >> 10);
+  return diff >> 21;
+}
+
+// ---- ranking value ---------------------------------------------------------------
+struct RankRaw {
+  __device__ __forceinline__ float operator()(float x, int64_t) const { return x; }
+};
+// z-score in the model dtype: round(round(x - mean) / denom)  (activations.py:283)
+template <typename T> struct RankZ {
+  const float *mean, *denom;  // this layer's rows of the [L][F] statistics
+  __device__ __forceinline__ float operator()(float x, int64_t col) const {
+    float a = Elem<T>::round(x - mean[col]);
+    return Elem<T>::round(a / denom[col]);
+  }
+};
+template <typename T, bool GLOBAL> struct RankOf;
+template <typename T> struct RankOf<T, false> {
+  typedef RankRaw type;
+  __device__ static RankRaw make(const float *, const float *, int64_t, int64_t) { return RankRaw(); }
+};
+template <typename T> struct RankOf<T, true> {
+  typedef RankZ<T> type;
+  __device__ static RankZ<T> make(const float *mean, const float *denom, int64_t l, int64_t F) {
+    RankZ<T> r; r.mean = mean + l * F; r.denom = denom + l * F; return r;
+  }
+};
+
+// ---- vector loads -----------------------------------------------------------------
+template <typename T, int V> struct VecLoad;
+template <> struct VecLoad<float, 4> {
+  __device__ static __forceinline__ void load(const float *p, float (&x)[4], uint32_t (&raw)[4]) {
+    float4 v = *reinterpret_cast<const float4 *>(p);
+    x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) raw[j] = __float_as_uint(x[j]);
+  }
+};
+template <> struct VecLoad<float, 1> {
+  __device__ static __forceinline__ void load(const float *p, float (&x)[1], uint32_t (&raw)[1]) {
+    x[0] = *p; raw[0] = __float_as_uint(x[0]);
+  }
+};
+template <> struct VecLoad<bf16_t, 8> {
+  __device__ static __forceinline__ void load(const bf16_t *p, float (&x)[8], uint32_t (&raw)[8]) {
+    uint4 v = *reinterpret_cast<const uint4 *>(p);
+    uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      raw[2 * j] = w[j] & 0xFFFFu; raw[2 * j + 1] = w[j] >> 16;
+      x[2 * j] = __uint_as_float(w[j] << 16); x[2 * j + 1] = __uint_as_float(w[j] & 0xFFFF0000u);
+    }
+  }
+};
+template <> struct VecLoad<bf16_t, 1> {
+  __device__ static __forceinline__ void load(const bf16_t *p, float (&x)[1], uint32_t (&raw)[1]) {
+    raw[0] = *p; x[0] = bf16_bits_to_f32(raw[0]);
+  }
+};
+
+// exclusive prefix over the wave (lane order, then bit order) of the set bits of m
+template <int V> __device__ __forceinline__ uint32_t wave_mask_prefix(uint32_t m, uint32_t &total) {
+  uint32_t pre = 0; total = 0;
+#pragma unroll
+  for (int j = 0; j < V; ++j) {
+    uint64_t b = ballot64((m >> j) & 1u);
+    pre += mbcnt64(b);
+    total += (uint32_t)__popcll(b);
+  }
+  return pre;
+}
+
+// ---- block scan helper --------------------------------------------------------------
+// Walks hist[nb-1] .. hist[0] and finds the bin where the running count first reaches k.
+// All SCAN_THREADS threads call it; returns false when the histogram holds fewer than k.
+__device__ bool block_find_from_top(const uint32_t *hist, int nb, unsigned long long k,
+                                    int &bin_out, unsigned long long &above_out,
+                                    unsigned long long &total_out) {
+  __shared__ unsigned long long wsum[SCAN_THREADS / CLT_WAVE];
+  __shared__ int s_bin;
+  __shared__ unsigned long long s_above, s_total;
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  int b0 = nb - 1 - 2 * tid, b1 = nb - 2 - 2 * tid;
+  unsigned long long h0 = b0 >= 0 ? hist[b0] : 0, h1 = b1 >= 0 ? hist[b1] : 0;
+  unsigned long long s = h0 + h1, inc = s;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    unsigned long long y = __shfl_up(inc, o);
+    if (lane >= o) inc += y;
+  }
+  if (tid == 0) { s_bin = -1; s_above = 0; }
+  if (lane == 63) wsum[wv] = inc;
+  __syncthreads();
+  unsigned long long base = 0, tot = 0;
+  for (int i = 0; i < SCAN_THREADS / CLT_WAVE; ++i) {
+    unsigned long long w = wsum[i];
+    if (i < wv) base += w;
+    tot += w;
+  }
+  unsigned long long excl = base + inc - s, incl = base + inc;
+  if (k > 0 && excl < k && k <= incl) {
+    if (excl + h0 >= k) { s_bin = b0; s_above = excl; }
+    else { s_bin = b1; s_above = excl + h0; }
+  }
+  if (tid == 0) s_total = tot;
+  __syncthreads();
+  bin_out = s_bin; above_out = s_above; total_out = s_total;
+  bool ok = s_bin >= 0;
+  __syncthreads();
+  return ok;
+}
+
+// ---- kernels ------------------------------------------------------------------------
+__global__ void k_fill_u32(uint32_t *p, uint32_t v, int64_t n) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  for (; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = v;
+}
+
+__device__ __forceinline__ uint64_t hash_index(uint64_t i, uint64_t n) {
+  uint64_t x = (i + 1) * 0x9E3779B97F4A7C15ull;
+  x ^= x >> 29; x *= 0xBF58476D1CE4E5B9ull; x ^= x >> 32;
+  return __umul64hi(x, n);
+}
+
+// One block per problem: conservative cut key from a hashed sample.
+template <typename T, bool GLOBAL>
+__global__ __launch_bounds__(SCAN_THREADS) void k_sample_cut(
+    const T *pre, int64_t Tn, int64_t F, int64_t L, int64_t lstride, const float *mean,
+    const float *denom, unsigned long long N, unsigned long long K, SelState *st) {
+  constexpr int KB = Elem<T>::KEYBITS;
+  constexpr int PER = SAMPLE_N / SCAN_THREADS;
+  __shared__ uint32_t lh[NBINS];
+  const int p = blockIdx.x, tid = threadIdx.x;
+  const unsigned long long ns = N < (unsigned long long)SAMPLE_N ? N : (unsigned long long)SAMPLE_N;
+  uint32_t keys[PER];
+  bool valid[PER];
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    unsigned long long si = (unsigned long long)tid + (unsigned long long)i * SCAN_THREADS;
+    valid[i] = si < ns;
+    keys[i] = 0;
+    if (valid[i]) {
+      unsigned long long idx = (ns == N) ? si : hash_index(si, N);
+      int64_t l, t, f;
+      if (GLOBAL) { int64_t rowlen = L * F; t = idx / rowlen; int64_t rem = idx - t * rowlen; l = rem / F; f = rem - l * F; }
+      else { l = p; t = idx / F; f = idx - t * F; }
+      float x = Elem<T>::to_f32(pre[l * lstride + t * F + f]);
+      typename RankOf<T, GLOBAL>::type rk = RankOf<T, GLOBAL>::make(mean, denom, l, F);
+      keys[i] = rank_key<KB>(rk(x, f));
+    }
+  }
+  // rank (1-based from the top) of the sample element used as the cut
+  unsigned long long r;
+  if (ns == N) r = K;
+  else {
+    double e = (double)K / (double)N * (double)ns;
+    r = (unsigned long long)(1.25 * e + 6.0 * sqrt(e) + 16.0) + 1;
+  }
+  uint32_t cut = min_key<KB>();
+  if (r <= ns && r > 0) {
+    constexpr int NLEV = KB == 32 ? 3 : 2;
+    const int shifts[3] = {KB == 32 ? 21 : 5, KB == 32 ? 10 : 0, 0};
+    const int widths[3] = {11, KB == 32 ? 11 : 5, 10};
+    uint32_t prefix = 0, prefix_mask = 0;  // decided high bits
+    unsigned long long k_rem = r;
+    for (int lev = 0; lev < NLEV; ++lev) {
+      for (int i = tid; i < NBINS; i += SCAN_THREADS) lh[i] = 0;
+      __syncthreads();
+      const int sh = shifts[lev];
+      const uint32_t dm = (1u << widths[lev]) - 1u;
+#pragma unroll
+      for (int i = 0; i < PER; ++i)
+        if (valid[i] && (keys[i] & prefix_mask) == prefix) atomicAdd(&lh[(keys[i] >> sh) & dm], 1u);
+      __syncthreads();
+      int bin; unsigned long long above, total;
+      block_find_from_top(lh, (int)dm + 1, k_rem, bin, above, total);
+      if (bin < 0) bin = 0;  // cannot happen (r <= ns); keep the cut low if it does
+      k_rem -= above;
+      prefix |= (uint32_t)bin << sh;
+      prefix_mask |= dm << sh;
+    }
+    cut = prefix;
+    if (cut < min_key<KB>()) cut = min_key<KB>();
+  }
+  if (tid == 0) {
+    SelState s;
+    s.cut_key = cut; s.status = ST_RUN; s.level = 0; s.flo = 0; s.fhi = 0; s.bbase = 0; s.shift = 0;
+    s.thr_key = 0; s.k_rem = K; s.tie_budget = 0;
+    st[p] = s;
+  }
+}
+
+// The streaming pass: one wavefront per row.
+template <typename T, int V, bool GLOBAL>
+__global__ __launch_bounds__(256) void k_select_pass(
+    const T *pre, int64_t Tn, int64_t F, int64_t L, int64_t lstride, const float *mean,
+    const float *denom, const SelState *st, uint32_t *hist, uint32_t *seg_count, uint2 *seg,
+    int cap, int phase) {
+  constexpr int KB = Elem<T>::KEYBITS;
+  __shared__ uint32_t lh[NBINS];
+  const int l = blockIdx.y, p = GLOBAL ? 0 : l;
+  const uint32_t status = st[p].status;
+  if (phase == 0 ? status != ST_RUN : status != ST_RETRY) return;
+  const uint32_t cut_key = st[p].cut_key;
+  const float cutf = __uint_as_float(key_to_f32_bits<KB>(cut_key));
+  for (int i = threadIdx.x; i < NBINS; i += blockDim.x) lh[i] = 0;
+  __syncthreads();
+  const int lane = lane_id(), wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
+  typename RankOf<T, GLOBAL>::type rk = RankOf<T, GLOBAL>::make(mean, denom, l, F);
+  for (int64_t t = (int64_t)blockIdx.x * nwv + wv; t < Tn; t += (int64_t)gridDim.x * nwv) {
+    const int64_t r = (int64_t)l * Tn + t;
+    const T *row = pre + l * lstride + t * F;
+    uint2 *sg = seg + r * cap;
+    uint32_t n = 0;
+    for (int64_t c0 = 0; c0 < F; c0 += 64 * V) {
+      const int64_t col = c0 + (int64_t)lane * V;
+      float x[V], rv[V]; uint32_t raw[V];
+      uint32_t m = 0;
+      if (col < F) {
+        VecLoad<T, V>::load(row + col, x, raw);
+#pragma unroll
+        for (int j = 0; j < V; ++j) { rv[j] = rk(x[j], col + j); if (!(rv[j] < cutf)) m |= 1u << j; }
+      }
+      if (ballot64(m != 0) == 0) continue;
+#pragma unroll
+      for (int j = 0; j < V; ++j)
+        if ((m >> j) & 1u) {
+          uint32_t key = rank_key<KB>(rv[j]);
+          if (key < cut_key) m &= ~(1u << j);
+          else atomicAdd(&lh[bin_level0<KB>(key - cut_key)], 1u);
+        }
+      uint32_t total, pre_cnt = wave_mask_prefix<V>(m, total);
+#pragma unroll
+      for (int j = 0; j < V; ++j)
+        if ((m >> j) & 1u) {
+          uint32_t pos = n + pre_cnt + __popc(m & ((1u << j) - 1u));
+          if (pos < (uint32_t)cap) sg[pos] = make_uint2((uint32_t)(col + j), raw[j]);
+        }
+      n += total;
+    }
+    if (lane == 0) seg_count[r] = n;
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < NBINS; i += blockDim.x) {
+    uint32_t c = lh[i];
+    if (c) atomicAdd(&hist[(int64_t)p * NBINS + i], c);
+  }
+}
+
+// One block per problem: consume the histogram of the current level.
+template <int KB>
+__global__ __launch_bounds__(SCAN_THREADS) void k_select_scan(SelState *st, uint32_t *hist, int phase, int level) {
+  __shared__ uint32_t lh[NBINS];
+  const int p = blockIdx.x, tid = threadIdx.x;
+  SelState s = st[p];
+  // phase 0: first look at level 0; phase 1: level 0 again after a retry pass; phase 2: levels >= 1
+  if (phase == 0 && !(s.status == ST_RUN && s.level == 0)) return;
+  if (phase == 1 && s.status != ST_RETRY) return;
+  if (phase == 2 && !(s.status == ST_RUN && (int)s.level == level)) return;
+  uint32_t *h = hist + (int64_t)p * NBINS;
+  for (int i = tid; i < NBINS; i += SCAN_THREADS) { lh[i] = h[i]; h[i] = 0; }
+  __syncthreads();
+  int bin; unsigned long long above, total;
+  bool found = block_find_from_top(lh, NBINS, s.k_rem, bin, above, total);
+  if (tid != 0) return;
+  if (!found) {
+    // fewer candidates than K: the sampled cut was too high -> run the pass again from the bottom
+    s.status = ST_RETRY; s.cut_key = min_key<KB>(); s.level = 0;
+    st[p] = s;
+    return;
+  }
+  s.k_rem -= above;
+  if (s.level == 0) {
+    if (KB == 16) {
+      if ((uint32_t)bin < FINE16) { s.thr_key = s.cut_key + bin; s.tie_budget = s.k_rem; s.status = ST_DONE; }
+      else {
+        uint32_t c = (uint32_t)bin - FINE16;
+        s.bbase = c << 10; s.flo = s.bbase > FINE16 ? s.bbase : FINE16; s.fhi = s.bbase + 1023u;
+        s.shift = 0; s.level = 1; s.status = ST_RUN;
+      }
+    } else {
+      s.bbase = (uint32_t)bin << 21; s.flo = s.bbase; s.fhi = s.bbase + ((1u << 21) - 1u);
+      s.shift = 10; s.level = 1; s.status = ST_RUN;
+    }
+  } else {
+    if (s.shift == 0) { s.thr_key = s.cut_key + s.bbase + bin; s.tie_budget = s.k_rem; s.status = ST_DONE; }
+    else {
+      s.bbase = s.bbase + ((uint32_t)bin << s.shift); s.flo = s.bbase; s.fhi = s.bbase + ((1u << s.shift) - 1u);
+      s.shift = 0; s.level = s.level + 1;
+    }
+  }
+  st[p] = s;
+}
+
+// Visit the candidates of one row (segment, or the dense row when the segment
+// overflowed) with one wavefront.  `f(active, col, raw, key)` is called once per wave step
+// with one element per lane (active=false for idle lanes), in ascending column order
+// across steps and lanes.
+template <typename T, bool GLOBAL, typename Fn>
+__device__ __forceinline__ void visit_candidates(
+    const T *pre, int64_t Tn, int64_t F, int64_t lstride, int l, int64_t t,
+    typename RankOf<T, GLOBAL>::type rk, uint32_t cut_key, const uint32_t *seg_count,
+    const uint2 *seg, int cap, Fn f) {
+  constexpr int KB = Elem<T>::KEYBITS;
+  const int lane = lane_id();
+  const int64_t r = (int64_t)l * Tn + t;
+  const uint32_t n = seg_count[r];
+  if (n <= (uint32_t)cap) {
+    const uint2 *sg = seg + r * cap;
+    for (uint32_t i0 = 0; i0 < n; i0 += 64) {
+      uint32_t i = i0 + lane;
+      bool act = i < n;
+      uint2 e = act ? sg[i] : make_uint2(0, 0);
+      uint32_t key = 0;
+      if (act) key = rank_key<KB>(rk(Elem<T>::to_f32(Elem<T>::from_raw(e.y)), (int64_t)e.x));
+      f(act, e.x, e.y, key);
+    }
+  } else {
+    const T *row = pre + l * lstride + t * F;
+    for (int64_t c0 = 0; c0 < F; c0 += 64) {
+      int64_t col = c0 + lane;
+      bool act = col < F;
+      uint32_t raw = 0, key = 0;
+      if (act) {
+        T v = row[col];
+        raw = Elem<T>::raw(v);
+        key = rank_key<KB>(rk(Elem<T>::to_f32(v), col));
+        act = key >= cut_key;
+      }
+      f(act, (uint32_t)col, raw, key);
+    }
+  }
+}
+
+// Levels >= 1: histogram of the candidates inside the active key range.
+template <typename T, bool GLOBAL>
+__global__ __launch_bounds__(256) void k_select_level(
+    const T *pre, int64_t Tn, int64_t F, int64_t L, int64_t lstride, const float *mean,
+    const float *denom, const SelState *st, uint32_t *hist, const uint32_t *seg_count,
+    const uint2 *seg, int cap, int level) {
+  __shared__ uint32_t lh[NBINS];
+  const int l = blockIdx.y, p = GLOBAL ? 0 : l;
+  const SelState s = st[p];
+  if (!(s.status == ST_RUN && (int)s.level == level)) return;
+  for (int i = threadIdx.x; i < NBINS; i += blockDim.x) lh[i] = 0;
+  __syncthreads();
+  const int wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
+  typename RankOf<T, GLOBAL>::type rk = RankOf<T, GLOBAL>::make(mean, denom, l, F);
+  for (int64_t t = (int64_t)blockIdx.x * nwv + wv; t < Tn; t += (int64_t)gridDim.x * nwv) {
+    visit_candidates<T, GLOBAL>(pre, Tn, F, lstride, l, t, rk, s.cut_key, seg_count, seg, cap,
+      [&](bool act, uint32_t, uint32_t, uint32_t key) {
+        if (act) {
+          uint32_t diff = key - s.cut_key;
+          if (diff >= s.flo && diff <= s.fhi) atomicAdd(&lh[(diff - s.bbase) >> s.shift], 1u);
+        }
+      });
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < NBINS; i += blockDim.x) {
+    uint32_t c = lh[i];
+    if (c) atomicAdd(&hist[(int64_t)p * NBINS + i], c);
+  }
+}
+
+// Per row: how many candidates beat the threshold key and how many equal it.
+template <typename T, bool GLOBAL>
+__global__ __launch_bounds__(256) void k_select_count(
+    const T *pre, int64_t Tn, int64_t F, int64_t L, int64_t lstride, const float *mean,
+    const float *denom, const SelState *st, const uint32_t *seg_count, const uint2 *seg,
+    int cap, uint32_t *row_gt, uint32_t *row_eq) {
+  const int l = blockIdx.y, p = GLOBAL ? 0 : l;
+  const SelState s = st[p];
+  const int wv = threadIdx.x >> 6, nwv = blockDim.x >> 6, lane = lane_id();
+  typename RankOf<T, GLOBAL>::type rk = RankOf<T, GLOBAL>::make(mean, denom, l, F);
+  for (int64_t t = (int64_t)blockIdx.x * nwv + wv; t < Tn; t += (int64_t)gridDim.x * nwv) {
+    uint32_t ngt = 0, neq = 0;
+    visit_candidates<T, GLOBAL>(pre, Tn, F, lstride, l, t, rk, s.cut_key, seg_count, seg, cap,
+      [&](bool act, uint32_t, uint32_t, uint32_t key) {
+        ngt += (uint32_t)__popcll(ballot64(act && key > s.thr_key));
+        neq += (uint32_t)__popcll(ballot64(act && key == s.thr_key));
+      });
+    if (lane == 0) { row_gt[(int64_t)l * Tn + t] = ngt; row_eq[(int64_t)l * Tn + t] = neq; }
+  }
+}
+
+__device__ __forceinline__ unsigned long long block_excl_scan_u64(unsigned long long v, unsigned long long &total) {
+  __shared__ unsigned long long ws[SCAN_THREADS / CLT_WAVE];
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  unsigned long long inc = v;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    unsigned long long y = __shfl_up(inc, o);
+    if (lane >= o) inc += y;
+  }
+  __syncthreads();
+  if (lane == 63) ws[wv] = inc;
+  __syncthreads();
+  unsigned long long base = 0, tot = 0;
+  for (int i = 0; i < (int)(blockDim.x >> 6); ++i) { unsigned long long w = ws[i]; if (i < wv) base += w; tot += w; }
+  total = tot;
+  return base + inc - v;
+}
+
+// One block per problem: hand the tie budget out in flat-index order; in per-layer mode
+// also write this layer's part of row_ptr (every layer keeps exactly K rows' worth).
+template <bool GLOBAL>
+__global__ __launch_bounds__(SCAN_THREADS) void k_select_allot(
+    const SelState *st, int64_t Tn, int64_t L, const uint32_t *row_gt, const uint32_t *row_eq,
+    uint32_t *allot, uint32_t *keep, int32_t *row_ptr, unsigned long long K) {
+  const int p = blockIdx.x, tid = threadIdx.x;
+  const unsigned long long budget = st[p].tie_budget;
+  const int64_t nrows = GLOBAL ? Tn * L : Tn;
+  unsigned long long eq_run = 0, keep_run = 0;
+  for (int64_t i0 = 0; i0 < nrows; i0 += SCAN_THREADS) {
+    int64_t i = i0 + tid;
+    int64_t r = -1;
+    if (i < nrows) r = GLOBAL ? ((i % L) * Tn + i / L) : ((int64_t)p * Tn + i);
+    unsigned long long eq = r >= 0 ? row_eq[r] : 0, gt = r >= 0 ? row_gt[r] : 0, tot;
+    unsigned long long before = eq_run + block_excl_scan_u64(eq, tot);
+    eq_run += tot;
+    unsigned long long a = before >= budget ? 0 : (budget - before < eq ? budget - before : eq);
+    unsigned long long kp = gt + a;
+    if (r >= 0) { allot[r] = (uint32_t)a; keep[r] = (uint32_t)kp; }
+    if (!GLOBAL) {
+      unsigned long long kt;
+      unsigned long long kbefore = keep_run + block_excl_scan_u64(kp, kt);
+      keep_run += kt;
+      if (r >= 0) row_ptr[r] = (int32_t)((unsigned long long)p * K + kbefore);
+    }
+  }
+  if (!GLOBAL && tid == 0 && p == (int)gridDim.x - 1) row_ptr[(int64_t)gridDim.x * Tn] = (int32_t)((unsigned long long)gridDim.x * K);
+}
+
+// Single block: row_ptr = exclusive scan of keep[] in storage order (row = layer*T + token).
+__global__ __launch_bounds__(SCAN_THREADS) void k_rowptr_scan(const uint32_t *keep, int64_t R, int32_t *row_ptr) {
+  const int tid = threadIdx.x;
+  const int64_t per = (R + SCAN_THREADS - 1) / SCAN_THREADS;
+  const int64_t b = (int64_t)tid * per, e = b + per < R ? b + per : R;
+  unsigned long long s = 0;
+  for (int64_t i = b; i < e; ++i) s += keep[i];
+  unsigned long long tot;
+  unsigned long long run = block_excl_scan_u64(s, tot);
+  for (int64_t i = b; i < e; ++i) { row_ptr[i] = (int32_t)run; run += keep[i]; }
+  if (tid == 0) row_ptr[R] = (int32_t)tot;
+}
+
+// Ordered write of the survivors of each row.
+template <typename T, bool GLOBAL>
+__global__ __launch_bounds__(256) void k_select_emit(
+    const T *pre, int64_t Tn, int64_t F, int64_t L, int64_t lstride, const float *mean,
+    const float *denom, const SelState *st, const uint32_t *seg_count, const uint2 *seg, int cap,
+    const uint32_t *allot, const int32_t *row_ptr, int32_t *col_out, T *val_out) {
+  const int l = blockIdx.y, p = GLOBAL ? 0 : l;
+  const SelState s = st[p];
+  const int wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
+  typename RankOf<T, GLOBAL>::type rk = RankOf<T, GLOBAL>::make(mean, denom, l, F);
+  for (int64_t t = (int64_t)blockIdx.x * nwv + wv; t < Tn; t += (int64_t)gridDim.x * nwv) {
+    const int64_t r = (int64_t)l * Tn + t;
+    const int64_t base = row_ptr[r];
+    const uint32_t my_allot = allot[r];
+    uint32_t kept = 0, ties = 0;
+    visit_candidates<T, GLOBAL>(pre, Tn, F, lstride, l, t, rk, s.cut_key, seg_count, seg, cap,
+      [&](bool act, uint32_t col, uint32_t raw, uint32_t key) {
+        bool eq = act && key == s.thr_key;
+        uint64_t beq = ballot64(eq);
+        bool keepit = act && (key > s.thr_key || (eq && ties + mbcnt64(beq) < my_allot));
+        uint64_t bk = ballot64(keepit);
+        if (keepit) {
+          int64_t pos = base + kept + mbcnt64(bk);
+          col_out[pos] = (int32_t)col;
+          val_out[pos] = Elem<T>::from_raw(raw);
+        }
+        kept += (uint32_t)__popcll(bk);
+        ties += (uint32_t)__popcll(beq);
+      });
+  }
+}
+
+// ---- threshold activations ----------------------------------------------------------
+template <typename T, int PRED> __device__ __forceinline__ bool pred_keep(float x, float th) {
+  if (PRED == CLT_PRED_GE_THETA) return x >= th;
+  if (PRED == CLT_PRED_GT_ZERO) return x > 0.0f;
+  return x != 0.0f;
+}
+
+template <typename T, int V, int PRED, bool EMIT>
+__global__ __launch_bounds__(256) void k_threshold(
+    const T *pre, int64_t Tn, int64_t F, int64_t L, int64_t lstride, const T *theta,
+    uint32_t *row_cnt, const int32_t *row_ptr, int32_t *col_out, T *val_out) {
+  const int l = blockIdx.y;
+  const int lane = lane_id(), wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
+  const T *th_row = PRED == CLT_PRED_GE_THETA ? theta + (int64_t)l * F : nullptr;
+  for (int64_t t = (int64_t)blockIdx.x * nwv + wv; t < Tn; t += (int64_t)gridDim.x * nwv) {
+    const int64_t r = (int64_t)l * Tn + t;
+    const T *row = pre + l * lstride + t * F;
+    const int64_t base = EMIT ? (int64_t)row_ptr[r] : 0;
+    uint32_t n = 0;
+    for (int64_t c0 = 0; c0 < F; c0 += 64 * V) {
+      const int64_t col = c0 + (int64_t)lane * V;
+      float x[V]; uint32_t raw[V];
+      uint32_t m = 0;
+      if (col < F) {
+        VecLoad<T, V>::load(row + col, x, raw);
+        float th[V];
+        if (PRED == CLT_PRED_GE_THETA) { uint32_t traw[V]; VecLoad<T, V>::load(th_row + col, th, traw); }
+#pragma unroll
+        for (int j = 0; j < V; ++j) if (pred_keep<T, PRED>(x[j], PRED == CLT_PRED_GE_THETA ? th[j] : 0.0f)) m |= 1u << j;
+      }
+      if (EMIT) {
+        if (ballot64(m != 0) == 0) continue;
+        uint32_t total, pre_cnt = wave_mask_prefix<V>(m, total);
+#pragma unroll
+        for (int j = 0; j < V; ++j)
+          if ((m >> j) & 1u) {
+            int64_t pos = base + n + pre_cnt + __popc(m & ((1u << j) - 1u));
+            col_out[pos] = (int32_t)(col + j);
+            val_out[pos] = Elem<T>::from_raw(raw[j]);
+          }
+        n += total;
+      } else {
+        n += __popc(m);
+      }
+    }
+    if (!EMIT) {
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) n += __shfl_xor(n, o);
+      if (lane == 0) row_cnt[r] = n;
+    }
+  }
+}
+
+// ---- host side ------------------------------------------------------------------------
+struct SelLayout {
+  size_t off_state, off_hist, off_segcnt, off_gt, off_eq, off_allot, off_keep, off_seg, total;
+  int cap, nprob;
+};
+
+static int seg_capacity(int64_t T, int64_t F, int64_t L, int64_t k, int mode) {
+  // expected candidates per row are about 2x the survivors per row
+  double per_row = mode == CLT_TOPK_GLOBAL ? (double)k / (double)L : (double)k;
+  int64_t want = (int64_t)(4.0 * per_row) + 1;
+  int64_t cap = 64;
+  while (cap < want && cap < 4096) cap <<= 1;
+  return (int)cap;
+}
+
+static SelLayout sel_layout(int64_t T, int64_t F, int64_t L, int64_t k, int mode) {
+  SelLayout lo;
+  lo.nprob = mode == CLT_TOPK_GLOBAL ? 1 : (int)L;
+  lo.cap = seg_capacity(T, F, L, k, mode);
+  const size_t R = (size_t)(L * T);
+  size_t o = 0;
+  auto take = [&](size_t bytes) { size_t at = o; o += (bytes + 255) & ~(size_t)255; return at; };
+  lo.off_state = take(sizeof(SelState) * (size_t)lo.nprob);
+  lo.off_hist = take(sizeof(uint32_t) * NBINS * (size_t)lo.nprob);
+  lo.off_segcnt = take(4 * R);
+  lo.off_gt = take(4 * R);
+  lo.off_eq = take(4 * R);
+  lo.off_allot = take(4 * R);
+  lo.off_keep = take(4 * R);
+  lo.off_seg = take(8 * R * (size_t)lo.cap);
+  lo.total = o;
+  return lo;
+}
+
+template <typename T, int V, bool GLOBAL>
+static int run_batchtopk(const T *pre, int64_t Tn, int64_t F, int64_t L, int64_t lstride, int64_t k,
+                         const float *mean, const float *denom, int32_t *row_ptr, int32_t *col, T *val,
+                         char *ws, hipStream_t stream) {
+  constexpr int KB = Elem<T>::KEYBITS;
+  const int mode = GLOBAL ? CLT_TOPK_GLOBAL : CLT_TOPK_PER_LAYER;
+  const SelLayout lo = sel_layout(Tn, F, L, k, mode);
+  SelState *st = (SelState *)(ws + lo.off_state);
+  uint32_t *hist = (uint32_t *)(ws + lo.off_hist);
+  uint32_t *segcnt = (uint32_t *)(ws + lo.off_segcnt);
+  uint32_t *rgt = (uint32_t *)(ws + lo.off_gt), *req = (uint32_t *)(ws + lo.off_eq);
+  uint32_t *allot = (uint32_t *)(ws + lo.off_allot), *keep = (uint32_t *)(ws + lo.off_keep);
+  uint2 *seg = (uint2 *)(ws + lo.off_seg);
+  const unsigned long long N = (unsigned long long)Tn * (unsigned long long)F * (GLOBAL ? (unsigned long long)L : 1ull);
+  unsigned long long K = (unsigned long long)k * (unsigned long long)Tn;
+  if (K > N) K = N;
+  const int nprob = lo.nprob;
+  k_fill_u32<<<64, 256, 0, stream>>>(hist, 0u, (int64_t)NBINS * nprob);
+  k_sample_cut<T, GLOBAL><<<nprob, SCAN_THREADS, 0, stream>>>(pre, Tn, F, L, lstride, mean, denom, N, K, st);
+  int gx = (int)clt_ceil_div(Tn, 4);
+  int maxgx = (int)clt_ceil_div(256 * 8, L);  // about 8 blocks per CU over all layers
+  if (maxgx < 1) maxgx = 1;
+  if (gx > maxgx) gx = maxgx;
+  dim3 grid(gx, (unsigned)L);
+  for (int phase = 0; phase < 2; ++phase) {
+    k_select_pass<T, V, GLOBAL><<<grid, 256, 0, stream>>>(pre, Tn, F, L, lstride, mean, denom, st, hist, segcnt, seg, lo.cap, phase);
+    k_select_scan<KB><<<nprob, SCAN_THREADS, 0, stream>>>(st, hist, phase, 0);
+  }
+  const int nlev = KB == 32 ? 3 : 2;
+  for (int level = 1; level < nlev; ++level) {
+    k_select_level<T, GLOBAL><<<grid, 256, 0, stream>>>(pre, Tn, F, L, lstride, mean, denom, st, hist, segcnt, seg, lo.cap, level);
+    k_select_scan<KB><<<nprob, SCAN_THREADS, 0, stream>>>(st, hist, 2, level);
+  }
+  k_select_count<T, GLOBAL><<<grid, 256, 0, stream>>>(pre, Tn, F, L, lstride, mean, denom, st, segcnt, seg, lo.cap, rgt, req);
+  k_select_allot<GLOBAL><<<nprob, SCAN_THREADS, 0, stream>>>(st, Tn, L, rgt, req, allot, keep, row_ptr, K);
+  if (GLOBAL) k_rowptr_scan<<<1, SCAN_THREADS, 0, stream>>>(keep, L * Tn, row_ptr);
+  k_select_emit<T, GLOBAL><<<grid, 256, 0, stream>>>(pre, Tn, F, L, lstride, mean, denom, st, segcnt, seg, lo.cap, allot, row_ptr, col, val);
+  return clt_check_launch();
+}
+
+template <typename T, bool GLOBAL>
+static int run_batchtopk_v(const T *pre, int64_t Tn, int64_t F, int64_t L, int64_t lstride, int64_t k,
+                           const float *mean, const float *denom, int32_t *row_ptr, int32_t *col, T *val,
+                           char *ws, hipStream_t stream) {
+  constexpr int VV = Elem<T>::VEC;
+  bool vec = (F % VV == 0) && clt_aligned16(pre) && ((lstride * (int64_t)sizeof(T)) % 16 == 0);
+  if (vec) return run_batchtopk<T, VV, GLOBAL>(pre, Tn, F, L, lstride, k, mean, denom, row_ptr, col, val, ws, stream);
+  return run_batchtopk<T, 1, GLOBAL>(pre, Tn, F, L, lstride, k, mean, denom, row_ptr, col, val, ws, stream);
+}
+
+template <typename T, int V, int PRED>
+static int run_threshold(bool emit, const T *pre, int64_t Tn, int64_t F, int64_t L, int64_t lstride,
+                         const T *theta, uint32_t *row_cnt, int32_t *row_ptr, int32_t *col, T *val,
+                         hipStream_t stream) {
+  int gx = (int)clt_ceil_div(Tn, 4);
+  int maxgx = (int)clt_ceil_div(256 * 8, L);
+  if (maxgx < 1) maxgx = 1;
+  if (gx > maxgx) gx = maxgx;
+  dim3 grid(gx, (unsigned)L);
+  if (!emit) {
+    k_threshold<T, V, PRED, false><<<grid, 256, 0, stream>>>(pre, Tn, F, L, lstride, theta, row_cnt, nullptr, nullptr, nullptr);
+    k_rowptr_scan<<<1, SCAN_THREADS, 0, stream>>>(row_cnt, L * Tn, row_ptr);
+  } else {
+    k_threshold<T, V, PRED, true><<<grid, 256, 0, stream>>>(pre, Tn, F, L, lstride, theta, nullptr, row_ptr, col, val);
+  }
+  return clt_check_launch();
+}
+
+template <typename T>
+static int dispatch_threshold(bool emit, const void *pre, int64_t Tn, int64_t F, int64_t L, int64_t lstride,
+                              const void *theta, int pred, uint32_t *row_cnt, int32_t *row_ptr,
+                              int32_t *col, void *val, hipStream_t stream) {
+  constexpr int VV = Elem<T>::VEC;
+  bool vec = (F % VV == 0) && clt_aligned16(pre) && ((lstride * (int64_t)sizeof(T)) % 16 == 0) &&
+             (pred != CLT_PRED_GE_THETA || clt_aligned16(theta));
+  const T *p = (const T *)pre; const T *th = (const T *)theta; T *v = (T *)val;
+#define CLT_TH(PR)                                                                                       \
+  return vec ? run_threshold<T, VV, PR>(emit, p, Tn, F, L, lstride, th, row_cnt, row_ptr, col, v, stream) \
+             : run_threshold<T, 1, PR>(emit, p, Tn, F, L, lstride, th, row_cnt, row_ptr, col, v, stream)
+  if (pred == CLT_PRED_GE_THETA) { CLT_TH(CLT_PRED_GE_THETA); }
+  if (pred == CLT_PRED_GT_ZERO) { CLT_TH(CLT_PRED_GT_ZERO); }
+  CLT_TH(CLT_PRED_NONZERO);
+#undef CLT_TH
+}
+
+}  // namespace
+
+extern "C" size_t clt_batchtopk_workspace_bytes(int64_t T, int64_t F, int64_t L, int64_t k, int mode, int dtype) {
+  (void)dtype;
+  if (T <= 0 || F <= 0 || L <= 0) return 256;
+  if (k < 0) k = 0;
+  return sel_layout(T, F, L, k, mode).total;
+}
+
+extern "C" int clt_batchtopk_select(const void *pre, int64_t T, int64_t F, int64_t L, int64_t pre_layer_stride,
+                                    int64_t k, int mode, const float *mean, const float *denom, int dtype,
+                                    int32_t *row_ptr, int32_t *col, void *val, void *workspace,
+                                    size_t workspace_bytes, void *stream) {
+  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (T < 0 || F < 0 || L <= 0 || L > 65535 || !row_ptr) return CLT_ERR_ARG;
+  if (mode != CLT_TOPK_PER_LAYER && mode != CLT_TOPK_GLOBAL) return CLT_ERR_ARG;
+  hipStream_t s = (hipStream_t)stream;
+  const int64_t R = L * T;
+  if (k <= 0 || T == 0 || F == 0) {
+    k_fill_u32<<<64, 256, 0, s>>>((uint32_t *)row_ptr, 0u, R + 1);
+    return clt_check_launch();
+  }
+  if (!pre || !col || !val || !workspace) return CLT_ERR_ARG;
+  if (mode == CLT_TOPK_GLOBAL && (!mean || !denom)) return CLT_ERR_ARG;
+  if ((double)T * (double)F * (double)L >= 4294967296.0) return CLT_ERR_RANGE;
+  if (workspace_bytes < clt_batchtopk_workspace_bytes(T, F, L, k, mode, dtype)) return CLT_ERR_WORKSPACE;
+  if ((((uintptr_t)workspace) & 255u) != 0) return CLT_ERR_ALIGN;
+  char *ws = (char *)workspace;
+  if (dtype == CLT_BF16) {
+    if (mode == CLT_TOPK_GLOBAL)
+      return run_batchtopk_v<bf16_t, true>((const bf16_t *)pre, T, F, L, pre_layer_stride, k, mean, denom, row_ptr, col, (bf16_t *)val, ws, s);
+    return run_batchtopk_v<bf16_t, false>((const bf16_t *)pre, T, F, L, pre_layer_stride, k, mean, denom, row_ptr, col, (bf16_t *)val, ws, s);
+  }
+  if (mode == CLT_TOPK_GLOBAL)
+    return run_batchtopk_v<float, true>((const float *)pre, T, F, L, pre_layer_stride, k, mean, denom, row_ptr, col, (float *)val, ws, s);
+  return run_batchtopk_v<float, false>((const float *)pre, T, F, L, pre_layer_stride, k, mean, denom, row_ptr, col, (float *)val, ws, s);
+}
+
+extern "C" int clt_threshold_count(const void *pre, int64_t T, int64_t F, int64_t L, int64_t pre_layer_stride,
+                                   const void *theta, int pred, int dtype, int32_t *row_ptr, void *workspace,
+                                   size_t workspace_bytes, void *stream) {
+  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (T < 0 || F < 0 || L <= 0 || L > 65535 || !row_ptr) return CLT_ERR_ARG;
+  if (pred < 0 || pred > 2 || (pred == CLT_PRED_GE_THETA && !theta)) return CLT_ERR_ARG;
+  hipStream_t s = (hipStream_t)stream;
+  const int64_t R = L * T;
+  if (T == 0 || F == 0) {
+    k_fill_u32<<<64, 256, 0, s>>>((uint32_t *)row_ptr, 0u, R + 1);
+    return clt_check_launch();
+  }
+  if (!pre || !workspace) return CLT_ERR_ARG;
+  if ((double)T * (double)F * (double)L >= 2147483648.0) return CLT_ERR_RANGE;
+  if (workspace_bytes < (size_t)R * 4) return CLT_ERR_WORKSPACE;
+  uint32_t *cnt = (uint32_t *)workspace;
+  if (dtype == CLT_BF16) return dispatch_threshold<bf16_t>(false, pre, T, F, L, pre_layer_stride, theta, pred, cnt, row_ptr, nullptr, nullptr, s);
+  return dispatch_threshold<float>(false, pre, T, F, L, pre_layer_stride, theta, pred, cnt, row_ptr, nullptr, nullptr, s);
+}
+
+extern "C" int clt_threshold_emit(const void *pre, int64_t T, int64_t F, int64_t L, int64_t pre_layer_stride,
+                                  const void *theta, int pred, int dtype, const int32_t *row_ptr, int32_t *col,
+                                  void *val, void *stream) {
+  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (T < 0 || F < 0 || L <= 0 || L > 65535 || !row_ptr) return CLT_ERR_ARG;
+  if (pred < 0 || pred > 2 || (pred == CLT_PRED_GE_THETA && !theta)) return CLT_ERR_ARG;
+  if (T == 0 || F == 0) return CLT_OK;
+  if (!pre || !col || !val) return CLT_ERR_ARG;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == CLT_BF16) return dispatch_threshold<bf16_t>(true, pre, T, F, L, pre_layer_stride, theta, pred, nullptr, (int32_t *)row_ptr, col, val, s);
+  return dispatch_threshold<float>(true, pre, T, F, L, pre_layer_stride, theta, pred, nullptr, (int32_t *)row_ptr, col, val, s);
+}

@@ -1,0 +1,286 @@
+"""Decoder stack: rec[t] = sum over sources s <= t of a[s] . W_dec + bias.
+
+Interface and parameter layout of the reference's ``Decoder``
+(clt/models/decoder.py:14-485): ``decoders`` is a ModuleDict keyed "s->t" (untied) or
+a ModuleList (per_source / per_target tying) of layers whose ``weight`` is [d_model, F];
+optional ``skip_weights``, ``feature_offset``, ``feature_scale``; ``decode`` and
+``get_decoder_norms`` with the same arguments, log messages and zero fallbacks.
+
+Internally every decoder matrix also exists as a feature-major [F, d_model] copy in one
+slab, so that the contribution of an active feature is one contiguous read, and the
+activations are handled as survivor lists (non-zeros only).
+"""
+
+from __future__ import annotations
+
+import logging
+import weakref
+from typing import Dict, List, Optional, Tuple
+
+import torch
+import torch.nn as nn
+
+from . import _native as nat
+from . import engine
+from .engine import SurvivorList
+from .parallel import RowParallelLinear, require_single_rank
+
+logger = logging.getLogger(__name__)
+
+
+def merge_layer_lists(parts: List[Tuple[int, SurvivorList]], L: int, T: int, F: int,
+                      dtype: torch.dtype, device: torch.device) -> SurvivorList:
+    """One survivor list over L layers from single-layer lists given as (layer, list),
+    layers ascending; layers that are not given get empty rows."""
+    counts = torch.zeros(L * T, dtype=torch.int64, device=device)
+    cols, vals = [], []
+    for s, sl in parts:
+        counts[s * T:(s + 1) * T] = (sl.row_ptr[1:] - sl.row_ptr[:-1]).to(torch.int64)
+        cols.append(sl.col)
+        vals.append(sl.val)
+    row_ptr = torch.zeros(L * T + 1, dtype=torch.int32, device=device)
+    row_ptr[1:] = torch.cumsum(counts, 0).to(torch.int32)
+    col = torch.cat(cols) if cols else torch.empty(0, dtype=torch.int32, device=device)
+    val = torch.cat(vals) if vals else torch.empty(0, dtype=dtype, device=device)
+    return SurvivorList(row_ptr, col, val, T, F, L, dtype)
+
+
+class Decoder(nn.Module):
+    def __init__(self, config, process_group, device: torch.device, dtype: torch.dtype):
+        super().__init__()
+        require_single_rank(process_group)
+        self.config = config
+        self.process_group = process_group
+        self.device = device
+        self.dtype = dtype
+        self.world_size, self.rank = 1, 0
+        L, F, d = config.num_layers, config.num_features, config.d_model
+        tied = config.decoder_tying in ("per_source", "per_target")
+
+        def make():
+            return RowParallelLinear(F, d, bias=True, process_group=process_group, d_model_for_init=d,
+                                     num_layers_for_init=L, device=device, dtype=dtype)
+
+        if tied:
+            self.decoders = nn.ModuleList(make() for _ in range(L))
+            for dec in self.decoders:  # tied decoders start at zero (decoder.py:80-86)
+                nn.init.zeros_(dec.weight)
+                nn.init.zeros_(dec.bias_param)
+        else:
+            self.decoders = nn.ModuleDict({f"{s}->{t}": make() for s in range(L) for t in range(s, L)})
+
+        def square():
+            return nn.Parameter(torch.zeros(d, d, device=device, dtype=dtype))
+
+        if config.skip_connection:
+            if tied:
+                self.skip_weights = nn.ParameterList(square() for _ in range(L))
+            else:
+                self.skip_weights = nn.ParameterDict({f"{s}->{t}": square() for s in range(L) for t in range(s, L)})
+        else:
+            self.skip_weights = None
+
+        # per-target affine on the selected features, tied decoders only (decoder.py:141-172)
+        self.feature_offset = None
+        self.feature_scale = None
+        if tied and config.enable_feature_offset:
+            self.feature_offset = nn.ParameterList(
+                nn.Parameter(torch.zeros(F, device=device, dtype=dtype)) for _ in range(L))
+        if tied and config.enable_feature_scale:
+            self.feature_scale = nn.ParameterList(
+                nn.Parameter(torch.ones(F, device=device, dtype=dtype) if i == 0
+                             else torch.full((F,), 0.1, device=device, dtype=dtype)) for i in range(L))
+
+        self.register_buffer("_cached_decoder_norms", None, persistent=False)
+        self._slab: Optional[torch.Tensor] = None
+        self._slab_keys: List[Optional[tuple]] = []
+        self._norm_key = None
+        self._bias_cache: Dict[int, Tuple[tuple, torch.Tensor]] = {}
+        self._compact_cache: Dict[int, tuple] = {}
+
+    # ---- decoder bookkeeping -------------------------------------------------------
+    def _ordered(self) -> List[RowParallelLinear]:
+        """Decoder layers in slot order (untied: "0->0", "0->1", ..., as created)."""
+        if isinstance(self.decoders, nn.ModuleDict):
+            L = self.config.num_layers
+            return [self.decoders[f"{s}->{t}"] for s in range(L) for t in range(s, L)]
+        return list(self.decoders)
+
+    def _slots(self) -> List[Tuple[int, int]]:
+        """(source, target) fed by each slot; tied decoders report (i, i)."""
+        L = self.config.num_layers
+        if self.config.decoder_tying == "none":
+            return [(s, t) for s in range(L) for t in range(s, L)]
+        return [(i, i) for i in range(L)]
+
+    def packed(self) -> torch.Tensor:
+        """[n_dec, F, d] feature-major slab; matrices whose parameter changed are repacked."""
+        decs = self._ordered()
+        w0 = decs[0].weight
+        F, d = self.config.num_features, self.config.d_model
+        if (self._slab is None or self._slab.device != w0.device or self._slab.dtype != w0.dtype
+                or self._slab.shape[0] != len(decs)):
+            self._slab = torch.empty(len(decs), F, d, device=w0.device, dtype=w0.dtype)
+            self._slab_keys = [None] * len(decs)
+            self.device, self.dtype = w0.device, w0.dtype
+        for i, dec in enumerate(decs):
+            w = dec.weight
+            key = (w.data_ptr(), w._version)
+            if self._slab_keys[i] != key:
+                engine.pack_decoder(w.detach().contiguous(), self._slab[i])
+                self._slab_keys[i] = key
+        return self._slab
+
+    def invalidate_packed(self) -> None:
+        """Force a repack on next use (needed only after writes that bypass autograd
+        version counting, e.g. through ``.data``)."""
+        self._slab_keys = [None] * len(self._slab_keys)
+        self._bias_cache.clear()
+        self._cached_decoder_norms = None
+
+    def bias_sum(self, src_mask: int) -> torch.Tensor:
+        """[L, d] fp32: for every target the sum of the biases of the decoders that run for
+        it - one per contributing source (decoder.py:294-295 / parallel.py:380-381), or the
+        target's own decoder for per_target tying (decoder.py:250-251)."""
+        decs = self._ordered()
+        key = tuple((dec.bias_param.data_ptr(), dec.bias_param._version) for dec in decs)
+        hit = self._bias_cache.get(src_mask)
+        if hit is not None and hit[0] == key:
+            return hit[1]
+        L, d = self.config.num_layers, self.config.d_model
+        B = torch.stack([dec.bias_param.detach().float() for dec in decs])
+        tying = self.config.decoder_tying
+        if tying == "per_target":
+            out = B.contiguous()
+        else:
+            out = torch.zeros(L, d, dtype=torch.float32, device=B.device)
+            if tying == "none":
+                for i, (s, t) in enumerate(self._slots()):
+                    if (src_mask >> s) & 1:
+                        out[t] += B[i]
+            else:
+                run = torch.zeros(d, dtype=torch.float32, device=B.device)
+                for t in range(L):
+                    if (src_mask >> t) & 1:
+                        run = run + B[t]
+                    out[t] = run
+        if len(self._bias_cache) > 64:
+            self._bias_cache.clear()
+        self._bias_cache[src_mask] = (key, out)
+        return out
+
+    def _affine(self):
+        L = self.config.num_layers
+        off = torch.stack([p.detach() for p in self.feature_offset]).contiguous() if self.feature_offset is not None else None
+        sc = torch.stack([p.detach() for p in self.feature_scale]).contiguous() if self.feature_scale is not None else None
+        assert off is None or off.shape[0] == L
+        return off, sc
+
+    def _skip_term(self, x2d: torch.Tensor, w_skip: torch.Tensor) -> torch.Tensor:
+        """x @ w_skip.T in fp32 (decoder.py:310, 332) through the encoder's MFMA kernel."""
+        x = x2d.detach().to(device=self.device, dtype=self.dtype).reshape(1, -1, self.config.d_model).contiguous()
+        return engine.encode(x, w_skip.detach().unsqueeze(0).contiguous(), None)[0].float()
+
+    # ---- fused path ------------------------------------------------------------------
+    def decode_survivors(self, surv: SurvivorList, src_mask: int, t_begin: int = 0, t_end: Optional[int] = None,
+                         skip_add: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Reconstructions [L, T, d] (rows outside [t_begin, t_end) are not written)."""
+        off, sc = self._affine()
+        return engine.decode_sparse(surv, self.packed(), self.config.decoder_tying, self.config.d_model,
+                                    bias_sum=self.bias_sum(src_mask), feat_offset=off, feat_scale=sc,
+                                    skip_add=skip_add, t_begin=t_begin, t_end=t_end, src_mask=src_mask)
+
+    def skip_all_targets(self, inputs: Dict[int, torch.Tensor], src_mask: int, T: int) -> Optional[torch.Tensor]:
+        """[L, T, d] fp32 skip-connection terms for every target present in ``inputs``."""
+        if self.skip_weights is None:
+            return None
+        L, d = self.config.num_layers, self.config.d_model
+        out = torch.zeros(L, T, d, dtype=torch.float32, device=self.device)
+        for t in range(L):
+            if t not in inputs:
+                continue
+            if self.config.decoder_tying == "none":
+                for s in range(t + 1):
+                    if (src_mask >> s) & 1 and s in inputs and f"{s}->{t}" in self.skip_weights:
+                        out[t] += self._skip_term(inputs[s], self.skip_weights[f"{s}->{t}"])
+            else:
+                out[t] += self._skip_term(inputs[t], self.skip_weights[t])
+        return out
+
+    # ---- reference interface -----------------------------------------------------------
+    def _compact(self, a2d: torch.Tensor, orig: torch.Tensor) -> SurvivorList:
+        ent = self._compact_cache.get(id(orig))
+        if ent is not None and ent[0]() is orig and ent[1] == orig._version:
+            return ent[2]
+        sl = engine.threshold_select(a2d.detach().contiguous().unsqueeze(0), None, nat.PRED_NONZERO)
+        if len(self._compact_cache) > 4 * self.config.num_layers + 8:
+            self._compact_cache.clear()
+        try:
+            self._compact_cache[id(orig)] = (weakref.ref(orig), orig._version, sl)
+        except TypeError:
+            pass
+        return sl
+
+    def decode(self, a: Dict[int, torch.Tensor], layer_idx: int,
+               source_inputs: Optional[Dict[int, torch.Tensor]] = None) -> torch.Tensor:
+        """Reconstruction [tokens, d_model] of ``layer_idx`` from dense activations ``a``."""
+        cfg = self.config
+        d, F = cfg.d_model, cfg.num_features
+        keys = sorted(a.keys())
+        if not keys:
+            logger.warning(f"Rank {self.rank}: No activation keys available in decode method for layer {layer_idx}")
+            return torch.zeros((0, d), device=self.device, dtype=self.dtype)
+        batch = 0
+        for k in keys:
+            if a[k].numel() > 0:
+                batch = a[k].shape[0] if a[k].dim() <= 2 else a[k].numel() // a[k].shape[-1]
+                break
+        if batch == 0:
+            return torch.zeros((0, d), device=self.device, dtype=self.dtype)
+        parts: List[Tuple[int, SurvivorList]] = []
+        src_mask = 0
+        for s in range(layer_idx + 1):
+            if s not in a:
+                continue
+            act = a[s]
+            if act.numel() == 0:
+                continue
+            if act.shape[-1] != F:
+                logger.warning(
+                    f"Rank {self.rank}: Activation tensor for layer {s} has incorrect feature dimension "
+                    f"{act.shape[-1]}, expected {F}. Skipping decode contribution.")
+                continue
+            a2 = act.to(device=self.device, dtype=self.dtype).reshape(-1, F)
+            if a2.shape[0] != batch:
+                raise ValueError(f"activation rows {a2.shape[0]} of layer {s} do not match batch {batch}")
+            nat.require_device(a2, "decode")
+            parts.append((s, self._compact(a2, act)))
+            src_mask |= 1 << s
+        L = cfg.num_layers
+        surv = merge_layer_lists(parts, L, batch, F, self.dtype, self.device)
+        skip = None
+        if self.skip_weights is not None and source_inputs is not None:
+            acc = torch.zeros(batch, d, dtype=torch.float32, device=self.device)
+            if cfg.decoder_tying == "none":
+                for s, _ in parts:
+                    if s in source_inputs and f"{s}->{layer_idx}" in self.skip_weights:
+                        acc += self._skip_term(source_inputs[s], self.skip_weights[f"{s}->{layer_idx}"])
+            elif layer_idx in source_inputs:
+                acc += self._skip_term(source_inputs[layer_idx], self.skip_weights[layer_idx])
+            skip = torch.zeros(L, batch, d, dtype=torch.float32, device=self.device)
+            skip[layer_idx] = acc
+        out = self.decode_survivors(surv, src_mask, layer_idx, layer_idx + 1, skip_add=skip)
+        return out[layer_idx]
+
+    def get_decoder_norms(self) -> torch.Tensor:
+        """[L, F] L2 norm of each feature's decoder vectors over the decoders its source
+        feeds (decoder.py:374-485); cached until ``_cached_decoder_norms`` is cleared or a
+        decoder weight changes."""
+        decs = self._ordered()
+        key = tuple((dec.weight.data_ptr(), dec.weight._version) for dec in decs)
+        if self._cached_decoder_norms is not None and self._norm_key == key:
+            return self._cached_decoder_norms
+        norms = engine.decoder_norms(self.packed(), self.config.num_layers, self.config.decoder_tying)
+        self._cached_decoder_norms = norms
+        self._norm_key = key
+        return norms

@@ -1,0 +1,258 @@
+"""Tensor-level entry points over the C ABI: stacked encode, selection into survivor
+lists, sparse decode.  torch supplies device memory and the current stream; every
+computation is a HIP kernel of libclt_hip.so.
+
+Layouts
+    x          [L, T, d]      inputs, one slab per layer
+    w_enc      [L, F, d]      encoder weights (nn.Linear layout)
+    pre        [L, T, F]      pre-activations
+    survivors  SurvivorList   rows r = layer * T + token; (col, val) sorted by col in a row
+    w_packed   [n_dec, F, d]  decoder weights, feature-major
+    out        [L, T, d]      reconstructions
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, Optional
+
+import torch
+
+from . import _native as nat
+
+
+@dataclass
+class SurvivorList:
+    """Compact activations of L layers x T tokens (CSR by row = layer*T + token)."""
+
+    row_ptr: torch.Tensor  # int32 [L*T + 1]
+    col: torch.Tensor      # int32 [nnz]   feature index
+    val: torch.Tensor      # model dtype [nnz]   raw pre-activation
+    T: int
+    F: int
+    L: int
+    dtype: torch.dtype
+
+    @property
+    def nnz(self) -> int:
+        return int(self.row_ptr[-1].item())
+
+
+class Workspace:
+    """Grow-only device buffers reused across calls on one stream."""
+
+    def __init__(self, device: torch.device):
+        self.device = device
+        self._bufs: Dict[str, torch.Tensor] = {}
+
+    def get(self, name: str, nbytes: int) -> torch.Tensor:
+        buf = self._bufs.get(name)
+        if buf is None or buf.numel() < nbytes:
+            self._bufs.pop(name, None)
+            buf = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=self.device)
+            self._bufs[name] = buf
+        return buf
+
+    def typed(self, name: str, shape, dtype: torch.dtype) -> torch.Tensor:
+        n = 1
+        for s in shape:
+            n *= int(s)
+        item = torch.empty((), dtype=dtype).element_size()
+        buf = self.get(name, n * item)
+        return buf[: n * item].view(dtype).view(*shape)
+
+    def release(self) -> None:
+        self._bufs.clear()
+
+
+def _stream(t: torch.Tensor) -> int:
+    return nat.current_stream(t.device)
+
+
+def encode(x: torch.Tensor, w: torch.Tensor, b: Optional[torch.Tensor],
+           out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """pre[l] = x[l] @ w[l].T + b[l] for stacked layers (parallel.py:286 per layer)."""
+    nat.require_device(x, "encode")
+    L, T, d = x.shape
+    F = w.shape[1]
+    assert w.shape == (L, F, d) and x.dtype == w.dtype
+    assert x.stride(2) == 1 and x.stride(1) == d and w.stride(2) == 1 and w.stride(1) == d
+    if out is None:
+        out = torch.empty((L, T, F), dtype=x.dtype, device=x.device)
+    assert out.shape == (L, T, F) and out.stride(2) == 1 and out.stride(1) == F
+    if b is not None:
+        assert b.shape == (L, F) and b.stride(1) == 1 and b.dtype == x.dtype
+    lib = nat.load()
+    code = lib.clt_encode(nat.ptr(x), nat.ptr(w), nat.ptr(b), nat.ptr(out), T, d, F, L,
+                          x.stride(0), w.stride(0), b.stride(0) if b is not None else 0, out.stride(0),
+                          nat.dtype_code(x.dtype), _stream(x))
+    nat.check(code, "clt_encode")
+    return out
+
+
+def colstats(pre: torch.Tensor):
+    """(mean, denom) fp32 [L, F] of the global ranking z-score (activations.py:281-283)."""
+    nat.require_device(pre, "colstats")
+    L, T, F = pre.shape
+    mean = torch.empty((L, F), dtype=torch.float32, device=pre.device)
+    denom = torch.empty((L, F), dtype=torch.float32, device=pre.device)
+    code = nat.load().clt_colstats(nat.ptr(pre), nat.ptr(mean), nat.ptr(denom), T, F, L, pre.stride(0),
+                                   nat.dtype_code(pre.dtype), _stream(pre))
+    nat.check(code, "clt_colstats")
+    return mean, denom
+
+
+def _check_pre(pre: torch.Tensor):
+    nat.require_device(pre, "select")
+    L, T, F = pre.shape
+    assert pre.stride(2) == 1 and (pre.stride(1) == F or T <= 1)
+    return L, T, F
+
+
+def batchtopk_select(pre: torch.Tensor, k: int, global_mode: bool, ws: Optional[Workspace] = None,
+                     stats=None) -> SurvivorList:
+    """BatchTopK survivors of pre [L, T, F] (activations.py:11-36 per layer, 261-357 global)."""
+    L, T, F = _check_pre(pre)
+    dev = pre.device
+    k = int(k)
+    if global_mode:
+        total = min(k * T, T * F * L) if k > 0 else 0
+    else:
+        total = L * min(k * T, T * F) if k > 0 else 0
+    row_ptr = torch.empty(L * T + 1, dtype=torch.int32, device=dev)
+    col = torch.empty(max(total, 1), dtype=torch.int32, device=dev)
+    val = torch.empty(max(total, 1), dtype=pre.dtype, device=dev)
+    mode = nat.TOPK_GLOBAL if global_mode else nat.TOPK_PER_LAYER
+    lib = nat.load()
+    mean = denom = None
+    if global_mode and total > 0:
+        mean, denom = stats if stats is not None else colstats(pre)
+    nbytes = lib.clt_batchtopk_workspace_bytes(T, F, L, max(k, 0), mode, nat.dtype_code(pre.dtype))
+    wbuf = (ws or Workspace(dev)).get("select", nbytes)
+    code = lib.clt_batchtopk_select(nat.ptr(pre), T, F, L, pre.stride(0), k, mode, nat.ptr(mean), nat.ptr(denom),
+                                    nat.dtype_code(pre.dtype), nat.ptr(row_ptr), nat.ptr(col), nat.ptr(val),
+                                    nat.ptr(wbuf), wbuf.numel(), _stream(pre))
+    nat.check(code, "clt_batchtopk_select")
+    return SurvivorList(row_ptr, col[:total], val[:total], T, F, L, pre.dtype)
+
+
+def tokentopk_select(pre: torch.Tensor, kk: int, global_mode: bool, ws: Optional[Workspace] = None,
+                     stats=None) -> SurvivorList:
+    """TokenTopK survivors, kk already resolved to a count (activations.py:99-128, 391-491)."""
+    L, T, F = _check_pre(pre)
+    dev = pre.device
+    kk = int(kk)
+    total = T * min(kk, L * F) if global_mode else L * T * min(kk, F)
+    total = max(total, 0)
+    row_ptr = torch.empty(L * T + 1, dtype=torch.int32, device=dev)
+    col = torch.empty(max(total, 1), dtype=torch.int32, device=dev)
+    val = torch.empty(max(total, 1), dtype=pre.dtype, device=dev)
+    mode = nat.TOPK_GLOBAL if global_mode else nat.TOPK_PER_LAYER
+    lib = nat.load()
+    mean = denom = None
+    if global_mode and total > 0:
+        mean, denom = stats if stats is not None else colstats(pre)
+    nbytes = lib.clt_tokentopk_workspace_bytes(T, F, L, max(kk, 0), mode, nat.dtype_code(pre.dtype))
+    wbuf = (ws or Workspace(dev)).get("select", nbytes)
+    code = lib.clt_tokentopk_select(nat.ptr(pre), T, F, L, pre.stride(0), kk, mode, nat.ptr(mean), nat.ptr(denom),
+                                    nat.dtype_code(pre.dtype), nat.ptr(row_ptr), nat.ptr(col), nat.ptr(val),
+                                    nat.ptr(wbuf), wbuf.numel(), _stream(pre))
+    nat.check(code, "clt_tokentopk_select")
+    return SurvivorList(row_ptr, col[:total], val[:total], T, F, L, pre.dtype)
+
+
+def threshold_select(pre: torch.Tensor, theta: Optional[torch.Tensor], pred: int,
+                     ws: Optional[Workspace] = None) -> SurvivorList:
+    """JumpReLU (x >= theta), ReLU (x > 0) or non-zero compaction of pre [L, T, F].
+
+    Two kernels with one 4-byte read-back in between: the survivor total sizes col/val.
+    """
+    L, T, F = _check_pre(pre)
+    dev = pre.device
+    lib = nat.load()
+    code_dt = nat.dtype_code(pre.dtype)
+    if theta is not None:
+        assert theta.shape == (L, F) and theta.dtype == pre.dtype and theta.is_contiguous()
+    row_ptr = torch.empty(L * T + 1, dtype=torch.int32, device=dev)
+    wbuf = (ws or Workspace(dev)).get("threshold", max(L * T * 4, 256))
+    code = lib.clt_threshold_count(nat.ptr(pre), T, F, L, pre.stride(0), nat.ptr(theta), pred, code_dt,
+                                   nat.ptr(row_ptr), nat.ptr(wbuf), wbuf.numel(), _stream(pre))
+    nat.check(code, "clt_threshold_count")
+    total = int(row_ptr[-1].item())
+    col = torch.empty(max(total, 1), dtype=torch.int32, device=dev)
+    val = torch.empty(max(total, 1), dtype=pre.dtype, device=dev)
+    code = lib.clt_threshold_emit(nat.ptr(pre), T, F, L, pre.stride(0), nat.ptr(theta), pred, code_dt,
+                                  nat.ptr(row_ptr), nat.ptr(col), nat.ptr(val), _stream(pre))
+    nat.check(code, "clt_threshold_emit")
+    return SurvivorList(row_ptr, col[:total], val[:total], T, F, L, pre.dtype)
+
+
+def pack_decoder(w_ref: torch.Tensor, out: torch.Tensor) -> None:
+    """[d, F] checkpoint layout -> [F, d] feature-major (one matrix)."""
+    nat.require_device(w_ref, "pack_decoder")
+    d, F = w_ref.shape
+    assert w_ref.is_contiguous() and out.shape == (F, d) and out.is_contiguous() and out.dtype == w_ref.dtype
+    code = nat.load().clt_pack_decoder(nat.ptr(w_ref), nat.ptr(out), d, F, 1, d * F, d * F,
+                                       nat.dtype_code(w_ref.dtype), _stream(w_ref))
+    nat.check(code, "clt_pack_decoder")
+
+
+def decode_sparse(surv: SurvivorList, w_packed: torch.Tensor, tying: str, d: int,
+                  bias_sum: Optional[torch.Tensor] = None, feat_offset: Optional[torch.Tensor] = None,
+                  feat_scale: Optional[torch.Tensor] = None, skip_add: Optional[torch.Tensor] = None,
+                  t_begin: int = 0, t_end: Optional[int] = None, src_mask: Optional[int] = None,
+                  out: Optional[torch.Tensor] = None, out_f32: bool = False) -> torch.Tensor:
+    """Reconstructions [L, T, d] for targets [t_begin, t_end) (decoder.py:176-340)."""
+    nat.require_device(w_packed, "decode_sparse")
+    L, T, F = surv.L, surv.T, surv.F
+    t_end = L if t_end is None else t_end
+    if src_mask is None:
+        src_mask = (1 << L) - 1
+    dev = w_packed.device
+    odt = torch.float32 if out_f32 else surv.dtype
+    if out is None:
+        out = torch.empty((L, T, d), dtype=odt, device=dev)
+    assert out.shape == (L, T, d) and out.is_contiguous() and out.dtype == odt
+    assert w_packed.is_contiguous() and w_packed.dtype == surv.dtype and w_packed.shape[1:] == (F, d)
+    for a in (bias_sum, skip_add):
+        assert a is None or (a.dtype == torch.float32 and a.is_contiguous())
+    for a in (feat_offset, feat_scale):
+        assert a is None or (a.dtype == surv.dtype and a.is_contiguous() and a.shape == (L, F))
+    code = nat.load().clt_decode_sparse(
+        nat.ptr(surv.row_ptr), nat.ptr(surv.col), nat.ptr(surv.val), nat.ptr(w_packed), nat.ptr(bias_sum),
+        nat.ptr(feat_offset), nat.ptr(feat_scale), nat.ptr(skip_add), nat.ptr(out), T, d, F, L,
+        nat.TYING[tying], t_begin, t_end, src_mask & ((1 << 64) - 1), nat.dtype_code(surv.dtype),
+        1 if out_f32 else 0, _stream(w_packed))
+    nat.check(code, "clt_decode_sparse")
+    return out
+
+
+def densify(surv: SurvivorList, out_f32: bool = False, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Dense [L, T, F] activations (value or 0) from a survivor list (activations.py:65, 347)."""
+    dev = surv.row_ptr.device
+    odt = torch.float32 if (out_f32 or surv.dtype == torch.float32) else surv.dtype
+    if out is None:
+        out = torch.empty((surv.L, surv.T, surv.F), dtype=odt, device=dev)
+    assert out.stride(2) == 1 and (out.stride(1) == surv.F or surv.T <= 1) and out.dtype == odt
+    code = nat.load().clt_densify(nat.ptr(surv.row_ptr), nat.ptr(surv.col), nat.ptr(surv.val), nat.ptr(out),
+                                  surv.T, surv.F, surv.L, out.stride(0), nat.dtype_code(surv.dtype),
+                                  1 if odt == torch.float32 else 0, nat.current_stream(dev))
+    nat.check(code, "clt_densify")
+    return out
+
+
+def decoder_norms(w_packed: torch.Tensor, L: int, tying: str) -> torch.Tensor:
+    """[L, F] per-feature decoder norms in the model dtype (decoder.py:374-485)."""
+    nat.require_device(w_packed, "decoder_norms")
+    _, F, d = w_packed.shape
+    out = torch.empty((L, F), dtype=w_packed.dtype, device=w_packed.device)
+    code = nat.load().clt_decoder_norms(nat.ptr(w_packed), nat.ptr(out), d, F, L, nat.TYING[tying],
+                                        nat.dtype_code(w_packed.dtype), _stream(w_packed))
+    nat.check(code, "clt_decoder_norms")
+    return out
+
+
+def survivor_rows(surv: SurvivorList) -> torch.Tensor:
+    """Row index (layer*T + token) of every survivor, int64 [nnz]."""
+    counts = (surv.row_ptr[1:] - surv.row_ptr[:-1]).to(torch.int64)
+    return torch.repeat_interleave(torch.arange(surv.L * surv.T, device=counts.device), counts)

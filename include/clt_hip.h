@@ -1,0 +1,208 @@
+/*
+ * clt_hip.h - C ABI of libclt_hip.so, the gfx950 (MI355X) implementation of the
+ * cross-layer-transcoder forward path: encoder projection, BatchTopK / TokenTopK /
+ * JumpReLU selection into a compact survivor list, and sparse cross-layer decode.
+ *
+ * The reference (curt-tigges/crosslayer-coding) has no native boundary for this
+ * path: it issues stock ATen ops from Python.  Each entry point below names the
+ * reference call site (file:line, relative to the reference checkout) whose work
+ * it replaces.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless its name ends in _host;
+ *   - sizes and strides are int64 element counts (strides between layers);
+ *   - `dtype` is CLT_F32 or CLT_BF16 and names the model dtype (inputs, weights,
+ *     pre-activations, survivor values, outputs unless said otherwise);
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream);
+ *   - functions launch asynchronously on `stream` and return CLT_OK or a negative
+ *     error code; nothing is allocated or freed inside;
+ *   - rows of the survivor list ("CSR") are numbered r = layer * T + token;
+ *     row_ptr has L*T+1 int32 entries, col holds feature indices in ascending
+ *     order inside a row, val the raw pre-activation values in the model dtype.
+ */
+#ifndef CLT_HIP_H
+#define CLT_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CLT_F32 0
+#define CLT_BF16 1
+
+#define CLT_OK 0
+#define CLT_ERR_ARG (-1)       /* null pointer, negative size, unsupported combination */
+#define CLT_ERR_DTYPE (-2)     /* dtype is not CLT_F32 / CLT_BF16 */
+#define CLT_ERR_WORKSPACE (-3) /* workspace smaller than clt_*_workspace_bytes() says */
+#define CLT_ERR_LAUNCH (-4)    /* HIP reported an error when launching */
+#define CLT_ERR_ALIGN (-5)     /* a pointer or row pitch is not 16-byte aligned */
+#define CLT_ERR_RANGE (-6)     /* a size exceeds what the kernels index (see each call) */
+
+/* decoder tying, reference clt/config/clt_config.py:41 */
+#define CLT_TYING_NONE 0
+#define CLT_TYING_PER_SOURCE 1
+#define CLT_TYING_PER_TARGET 2
+
+/* selection scope, reference clt/config/clt_config.py:31 */
+#define CLT_TOPK_PER_LAYER 0
+#define CLT_TOPK_GLOBAL 1
+
+/* predicates of clt_threshold_count / clt_threshold_emit */
+#define CLT_PRED_GE_THETA 0 /* x >= theta[layer][feature]   (JumpReLU) */
+#define CLT_PRED_GT_ZERO 1  /* x > 0                        (ReLU)     */
+#define CLT_PRED_NONZERO 2  /* x != 0                       (compaction of a dense tensor) */
+
+/* Library version (major*10000 + minor*100 + patch). */
+int clt_version(void);
+
+/* Static text for an error code. */
+const char *clt_error_string(int code);
+
+/*
+ * Encoder projection for L layers in one launch:
+ *   pre[l][t][f] = sum_k x[l][t][k] * w[l][f][k] + b[l][f]
+ * x [L][T][d], w [L][F][d] (nn.Linear layout), b [L][F] or NULL, pre [L][T][F].
+ * fp32 accumulation, one rounding to the model dtype.
+ * Replaces F.linear in ColumnParallelLinear.forward (clt/models/parallel.py:286)
+ * as called by Encoder.get_preactivations (clt/models/encoder.py:101), for every
+ * layer that Encoder.encode_all_layers walks (clt/models/encoder.py:151-162).
+ */
+int clt_encode(const void *x, const void *w, const void *b, void *pre,
+               int64_t T, int64_t d, int64_t F, int64_t L,
+               int64_t x_layer_stride, int64_t w_layer_stride,
+               int64_t b_layer_stride, int64_t pre_layer_stride,
+               int dtype, void *stream);
+
+/*
+ * Per-feature ranking statistics of the global BatchTopK / TokenTopK helper:
+ *   mean[l][f]  = mean over tokens of pre[l][:, f]
+ *   denom[l][f] = unbiased std over tokens + 1e-6
+ * both rounded to the model dtype as the reference's tensors are, stored as fp32.
+ * Replaces preact.mean(dim=0) / preact.std(dim=0) (clt/models/activations.py:281-283).
+ */
+int clt_colstats(const void *pre, float *mean, float *denom,
+                 int64_t T, int64_t F, int64_t L, int64_t pre_layer_stride,
+                 int dtype, void *stream);
+
+/*
+ * BatchTopK selection into a survivor list.
+ *   mode CLT_TOPK_PER_LAYER: for each layer, the min(k*T, T*F) largest of its T*F
+ *     pre-activations (ranking on the raw value), i.e. BatchTopK._compute_mask
+ *     (clt/models/activations.py:11-36) as applied per layer by
+ *     batchtopk_per_layer_activation (clt/activations/registry.py:43-72).
+ *   mode CLT_TOPK_GLOBAL: the min(k*T, T*L*F) largest over all layers, ranked on
+ *     (x - mean[l][f]) / denom[l][f] evaluated in the model dtype; the raw value
+ *     is what is kept: _apply_batch_topk_helper (clt/models/activations.py:261-357).
+ * Ties at the threshold go to the lowest flat index of the [T, F] (per layer) or
+ * [T, L*F] (global) block; -0.0 == +0.0; NaN ranks above +inf.
+ * Outputs: row_ptr [L*T+1], col / val with room for the survivor total
+ * (L * min(k*T, T*F) per-layer, min(k*T, T*L*F) global).
+ * Limits: T*F*L < 2^32, F % 8 == 0 for bf16 / F % 4 == 0 for fp32 on the fast
+ * path (other F take a scalar path), pre rows 16-byte aligned on the fast path.
+ */
+size_t clt_batchtopk_workspace_bytes(int64_t T, int64_t F, int64_t L, int64_t k,
+                                     int mode, int dtype);
+int clt_batchtopk_select(const void *pre, int64_t T, int64_t F, int64_t L,
+                         int64_t pre_layer_stride, int64_t k, int mode,
+                         const float *mean, const float *denom, int dtype,
+                         int32_t *row_ptr, int32_t *col, void *val,
+                         void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * TokenTopK selection: per token row, the kk largest of its F (per layer) or L*F
+ * (global, ranked on the z-score as above) entries.  kk is the already resolved
+ * integer count (fraction/ceil rule of clt/models/activations.py:108-116).
+ * Replaces TokenTopK._compute_mask (clt/models/activations.py:99-128) and
+ * _apply_token_topk_helper (clt/models/activations.py:391-491).
+ */
+size_t clt_tokentopk_workspace_bytes(int64_t T, int64_t F, int64_t L, int64_t kk,
+                                     int mode, int dtype);
+int clt_tokentopk_select(const void *pre, int64_t T, int64_t F, int64_t L,
+                         int64_t pre_layer_stride, int64_t kk, int mode,
+                         const float *mean, const float *denom, int dtype,
+                         int32_t *row_ptr, int32_t *col, void *val,
+                         void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Threshold activations (JumpReLU, ReLU) and compaction of a dense activation
+ * tensor, in two calls because the survivor total is data dependent:
+ *   clt_threshold_count fills row_ptr [L*T+1] (row_ptr[L*T] = total);
+ *   the caller sizes col/val from the total and calls clt_threshold_emit.
+ * theta [L][F] in the model dtype (already exp()'d and rounded), used by
+ * CLT_PRED_GE_THETA only.  Replaces JumpReLU.forward
+ * (clt/models/activations.py:177-180) as called by ThetaManager.jumprelu
+ * (clt/models/theta.py:70-79), F.relu (clt/activations/registry.py:30-33), and
+ * the `activation_tensor != 0` scans of Decoder.decode (clt/models/decoder.py:230, 270).
+ * workspace: (L*T) * 4 bytes.
+ */
+int clt_threshold_count(const void *pre, int64_t T, int64_t F, int64_t L,
+                        int64_t pre_layer_stride, const void *theta, int pred,
+                        int dtype, int32_t *row_ptr, void *workspace,
+                        size_t workspace_bytes, void *stream);
+int clt_threshold_emit(const void *pre, int64_t T, int64_t F, int64_t L,
+                       int64_t pre_layer_stride, const void *theta, int pred,
+                       int dtype, const int32_t *row_ptr, int32_t *col, void *val,
+                       void *stream);
+
+/*
+ * Repack decoder weights from the checkpoint layout [d][F] (nn.Linear weight of
+ * RowParallelLinear, clt/models/parallel.py:66-70) to feature-major [F][d], so a
+ * feature's decoder vector is one contiguous run.  n_dec matrices, element strides.
+ */
+int clt_pack_decoder(const void *w_ref, void *w_packed, int64_t d, int64_t F,
+                     int64_t n_dec, int64_t in_stride, int64_t out_stride,
+                     int dtype, void *stream);
+
+/*
+ * Sparse cross-layer decode for targets t in [t_begin, t_end):
+ *   out[t][tok][:] = sum over sources s <= t with bit s of src_mask set,
+ *                    over survivors (f, v) of row s*T+tok:
+ *                        v' * w_packed[slot(s,t)][f][:]
+ *                    + bias_sum[t][:] (+ skip_add[t][tok][:])
+ *   v' = v, or (v + feat_offset[t][f]) * feat_scale[t][f] (model-dtype rounding
+ *   after each step, zeros left untouched) when those arrays are given.
+ *   slot(s,t): CLT_TYING_NONE       s*L - s*(s-1)/2 + (t-s)  (order of "s->t" keys)
+ *              CLT_TYING_PER_SOURCE s
+ *              CLT_TYING_PER_TARGET t
+ * fp32 accumulation; out [L][T][d] in the model dtype (out_f32 = 0) or fp32.
+ * bias_sum [L][d] fp32 or NULL, feat_offset / feat_scale [L][F] model dtype or
+ * NULL, skip_add [L][T][d] fp32 or NULL.
+ * Replaces Decoder.decode (clt/models/decoder.py:176-340) and the
+ * RowParallelLinear.forward calls inside it (clt/models/parallel.py:366, 380-381),
+ * for all targets that CrossLayerTranscoder.forward loops over
+ * (clt/models/clt.py:192-199).
+ * Limits: L <= 64; d % 8 == 0 (bf16) / d % 4 == 0 (fp32) on the fast path.
+ */
+int clt_decode_sparse(const int32_t *row_ptr, const int32_t *col, const void *val,
+                      const void *w_packed, const float *bias_sum,
+                      const void *feat_offset, const void *feat_scale,
+                      const float *skip_add, void *out,
+                      int64_t T, int64_t d, int64_t F, int64_t L,
+                      int tying, int64_t t_begin, int64_t t_end, uint64_t src_mask,
+                      int dtype, int out_f32, void *stream);
+
+/*
+ * Dense materialisation of a survivor list: out[l][t][f] = value or 0.
+ * out_f32 selects fp32 output (JumpReLU returns fp32, activations.py:180).
+ * Replaces `x * mask.to(x.dtype)` (clt/models/activations.py:65, 347).
+ */
+int clt_densify(const int32_t *row_ptr, const int32_t *col, const void *val,
+                void *out, int64_t T, int64_t F, int64_t L, int64_t out_layer_stride,
+                int dtype, int out_f32, void *stream);
+
+/*
+ * Per-feature decoder norms from packed weights:
+ *   norms[s][f] = sqrt(sum over decoders fed by source s of ||w[f][:]||^2)
+ * fp32 accumulation, rounded to the model dtype.
+ * Replaces Decoder.get_decoder_norms (clt/models/decoder.py:374-485).
+ */
+int clt_decoder_norms(const void *w_packed, void *norms, int64_t d, int64_t F,
+                      int64_t L, int tying, int dtype, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CLT_HIP_H */

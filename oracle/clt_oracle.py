@@ -1,0 +1,426 @@
+"""CPU oracle for the cross-layer-transcoder forward path.
+
+TEST INFRASTRUCTURE ONLY.  This module restates, with plain torch-CPU / numpy
+operations, the algorithm the reference runs on its forward path.  It exists so
+that the HIP kernels can be checked against it; nothing that ships (the package,
+its C-ABI library) may import or call it.  Only ``tests/``, the smoke check and
+the ``cpu_baseline`` leg of the benchmark use it, and there only as the checker
+or as the timed CPU baseline.
+
+Every function cites the reference lines it follows (paths relative to the
+reference checkout).
+
+How each function is pinned (see ``tests/test_oracle_*.py``):
+
+* ``batchtopk_mask`` / ``batchtopk_forward``  - the reference's known-answer
+  vectors (tests/unit/models/test_activations.py:10-25, 28-63, 66-111) plus a
+  brute-force full-sort selector on small random inputs with forced ties.
+* ``tokentopk_mask``  - known answers (test_activations.py:158-283).
+* ``jumprelu_forward``  - known answer (test_activations.py:304-315) and the
+  ``where(x >= theta, x, 0)`` identity (tests/unit/models/test_theta.py:79-92).
+* ``encoder_preactivations``  - affine map checked against a float64 numpy
+  contraction (the reference pins it against nn.Linear,
+  tests/integration/test_tp_equivalence.py:316-343).
+* ``decode``  - additivity over sources (tests/unit/models/test_decoder.py:62-81),
+  zero weights give zero output (tests/unit/models/test_tied_decoders.py:138-166),
+  and a float64 numpy per-element loop on tiny shapes.
+* ``global_batchtopk``  - closed form of the z-score on hand-computable columns;
+  the reference has no golden numbers for it: PARITY UNPINNED beyond that
+  closed form (its tests only check shapes, test_clt_encode_decode.py:70-116).
+* ``forward``  - composition of the above; the reference has no golden tensors
+  for a full forward: PARITY UNPINNED beyond shape/keys and the pins of its parts.
+
+Tie rule.  ``torch.topk(sorted=False)`` leaves the choice among equal ranking
+values unspecified (reference activations.py:28).  This oracle fixes it the way
+the HIP kernels do: among equal ranking values the lowest flat index wins, where
+-0.0 and +0.0 are equal and every NaN ranks above +inf (as torch.topk orders them).
+"""
+
+from __future__ import annotations
+
+import math
+from typing import Dict, List, Optional, Tuple
+
+import numpy as np
+import torch
+import torch.nn.functional as F
+
+
+# ---------------------------------------------------------------------------
+# ranking keys
+# ---------------------------------------------------------------------------
+
+def ranking_key_u32(x: torch.Tensor) -> np.ndarray:
+    """Order-preserving unsigned key of a float tensor (flattened).
+
+    key(a) > key(b)  <=>  a ranks above b under torch.topk's ordering
+    (activations.py:28): ascending float order, -0.0 == +0.0, NaN above +inf.
+    bf16/fp16 inputs are widened to fp32 first (exact), so one 32-bit key law
+    covers every dtype.
+    """
+    xf = x.detach().to(torch.float32).reshape(-1).contiguous()
+    bits = xf.numpy().view(np.uint32).copy()
+    nan = np.isnan(xf.numpy())
+    bits[bits == np.uint32(0x80000000)] = np.uint32(0)  # -0.0 -> +0.0
+    neg = (bits >> np.uint32(31)).astype(bool)
+    key = np.where(neg, ~bits, bits | np.uint32(0x80000000)).astype(np.uint32)
+    key[nan] = np.uint32(0xFFFFFFFF)
+    return key
+
+
+def _select_flat(key: np.ndarray, k_total: int) -> np.ndarray:
+    """Flat indices of the k_total largest keys, ties to the lowest index."""
+    if k_total <= 0:
+        return np.zeros(0, dtype=np.int64)
+    # stable ascending sort of the inverted key = descending key, ties by index
+    order = np.argsort(~key, kind="stable")
+    return order[:k_total]
+
+
+# ---------------------------------------------------------------------------
+# activations  (reference clt/models/activations.py)
+# ---------------------------------------------------------------------------
+
+def batchtopk_mask(x: torch.Tensor, k_per_token: int,
+                   x_for_ranking: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """BatchTopK._compute_mask (activations.py:11-36).
+
+    k_total = min(k * B, numel) survivors over the whole flattened block,
+    ranked on ``x_for_ranking`` when given, else on ``x``; k <= 0 or an empty
+    tensor gives an all-False mask.
+    """
+    B = x.size(0)
+    if k_per_token <= 0 or x.numel() == 0:
+        return torch.zeros_like(x, dtype=torch.bool)
+    k_total = min(int(k_per_token) * B, x.numel())
+    rank = x_for_ranking if x_for_ranking is not None else x
+    idx = _select_flat(ranking_key_u32(rank), k_total)
+    mask = np.zeros(x.numel(), dtype=bool)
+    mask[idx] = True
+    return torch.from_numpy(mask).view(x.shape)
+
+
+def batchtopk_forward(x: torch.Tensor, k: float,
+                      x_for_ranking: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """BatchTopK.forward (activations.py:39-65): x * mask, negatives kept."""
+    mask = batchtopk_mask(x, int(k), x_for_ranking)
+    return x * mask.to(x.dtype)
+
+
+def tokentopk_k(k_float: float, f_total: int) -> int:
+    """k rule of TokenTopK._compute_mask (activations.py:108-116).
+
+    0 < k < 1 is a fraction of the row (rounded up, computed in fp32 like the
+    reference's torch.tensor(k * F)), k >= 1 is an integer count, k <= 0 keeps
+    nothing; always capped at the row length.
+    """
+    if f_total == 0 or k_float <= 0:
+        return 0
+    if k_float < 1:
+        kk = int(math.ceil(float(np.float32(k_float * f_total))))
+    else:
+        kk = int(k_float)
+    return min(kk, f_total)
+
+
+def tokentopk_mask(x: torch.Tensor, k_float: float,
+                   x_for_ranking: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """TokenTopK._compute_mask (activations.py:99-128): row-wise top-k."""
+    if x.numel() == 0:
+        return torch.zeros_like(x, dtype=torch.bool)
+    n_rows, f_total = x.shape
+    kk = tokentopk_k(k_float, f_total)
+    if kk <= 0:
+        return torch.zeros_like(x, dtype=torch.bool)
+    rank = x_for_ranking if x_for_ranking is not None else x
+    key = ranking_key_u32(rank).reshape(n_rows, f_total)
+    mask = np.zeros((n_rows, f_total), dtype=bool)
+    for r in range(n_rows):
+        mask[r, _select_flat(key[r], kk)] = True
+    return torch.from_numpy(mask)
+
+
+def tokentopk_forward(x: torch.Tensor, k: float,
+                      x_for_ranking: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """TokenTopK.forward (activations.py:131-156)."""
+    return x * tokentopk_mask(x, k, x_for_ranking).to(x.dtype)
+
+
+def jumprelu_forward(x: torch.Tensor, threshold: torch.Tensor) -> torch.Tensor:
+    """JumpReLU.forward (activations.py:177-180): (x >= theta).float() * x.
+
+    The product is fp32 whatever the input dtype, as in the reference.
+    """
+    return (x >= threshold).float() * x
+
+
+def theta_from_log(log_threshold_row: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """ThetaManager.jumprelu's threshold (theta.py:78): exp, then cast to the
+    model dtype *before* the comparison."""
+    return torch.exp(log_threshold_row).to(dtype)
+
+
+# ---------------------------------------------------------------------------
+# encoder  (reference clt/models/encoder.py:54-131, parallel.py:282-294)
+# ---------------------------------------------------------------------------
+
+def encoder_preactivations(x: torch.Tensor, weight: torch.Tensor,
+                           bias: Optional[torch.Tensor]) -> torch.Tensor:
+    """pre = x . W^T + b with W [F, d_model] (parallel.py:286); a 3-D input is
+    flattened to [B*S, d_model] first (encoder.py:67-75)."""
+    if x.dim() == 3:
+        x = x.reshape(-1, x.shape[-1])
+    return F.linear(x, weight, bias)
+
+
+# ---------------------------------------------------------------------------
+# global BatchTopK / TokenTopK helper  (activations.py:229-357, 360-491)
+# ---------------------------------------------------------------------------
+
+def zscore_for_ranking(pre: torch.Tensor) -> torch.Tensor:
+    """Per-feature z-score used for ranking only (activations.py:281-283):
+    (x - mean_0) / (std_0 + 1e-6) with the unbiased std over the batch axis,
+    every intermediate kept in the tensor's own dtype."""
+    mean = pre.mean(dim=0, keepdim=True)
+    std = pre.std(dim=0, keepdim=True)
+    return (pre - mean) / (std + 1e-6)
+
+
+def global_batchtopk(preacts: Dict[int, torch.Tensor], num_layers: int,
+                     k: int) -> Dict[int, torch.Tensor]:
+    """_apply_batch_topk_helper at world_size 1 (activations.py:261-357).
+
+    Layers are concatenated in range(num_layers) order to [T, sum F], the
+    ranking tensor is the per-layer z-score, k*T survivors are taken over the
+    whole block, the mask multiplies the raw values.
+    """
+    layers = [l for l in range(num_layers) if l in preacts]
+    if not layers:
+        return {}
+    orig = torch.cat([preacts[l] for l in layers], dim=1)
+    norm = torch.cat([zscore_for_ranking(preacts[l]) for l in layers], dim=1)
+    mask = batchtopk_mask(orig, int(k), norm)
+    act = orig * mask.to(orig.dtype)
+    out, off = {}, 0
+    for l in layers:
+        f = preacts[l].shape[1]
+        out[l] = act[:, off:off + f]
+        off += f
+    return out
+
+
+def global_tokentopk(preacts: Dict[int, torch.Tensor], num_layers: int,
+                     k: float) -> Dict[int, torch.Tensor]:
+    """_apply_token_topk_helper at world_size 1 (activations.py:391-491)."""
+    layers = [l for l in range(num_layers) if l in preacts]
+    if not layers:
+        return {}
+    orig = torch.cat([preacts[l] for l in layers], dim=1)
+    norm = torch.cat([zscore_for_ranking(preacts[l]) for l in layers], dim=1)
+    mask = tokentopk_mask(orig, float(k), norm)
+    act = orig * mask.to(orig.dtype)
+    out, off = {}, 0
+    for l in layers:
+        f = preacts[l].shape[1]
+        out[l] = act[:, off:off + f]
+        off += f
+    return out
+
+
+# ---------------------------------------------------------------------------
+# decoder  (reference clt/models/decoder.py:176-340, parallel.py:335-383)
+# ---------------------------------------------------------------------------
+
+def _affine_on_nonzero(a: torch.Tensor, offset: Optional[torch.Tensor],
+                       scale: Optional[torch.Tensor]) -> torch.Tensor:
+    """decoder.py:228-245 / 268-285: (a + offset[f]) * scale[f] on the non-zero
+    entries only, offset first, each step rounded in the tensor dtype."""
+    if offset is None and scale is None:
+        return a
+    nz = a != 0
+    if not bool(nz.any()):
+        return a
+    a = a.clone()
+    rows, cols = nz.nonzero(as_tuple=True)
+    if offset is not None:
+        a[rows, cols] += offset[cols]
+    if scale is not None:
+        a[rows, cols] *= scale[cols]
+    return a
+
+
+def decode(acts: Dict[int, torch.Tensor], layer_idx: int, *, tying: str,
+           weights: Dict[str, torch.Tensor], biases: Dict[str, torch.Tensor],
+           d_model: int, num_features: int, dtype: torch.dtype,
+           feature_offset: Optional[List[torch.Tensor]] = None,
+           feature_scale: Optional[List[torch.Tensor]] = None,
+           skip_weights: Optional[Dict[str, torch.Tensor]] = None,
+           source_inputs: Optional[Dict[int, torch.Tensor]] = None) -> torch.Tensor:
+    """Decoder.decode (decoder.py:176-340).
+
+    ``weights`` / ``biases`` are keyed like the reference's module names:
+    "s->t" for untied decoders, "i" for tied ones; each weight is stored
+    [d_model, F] (parallel.py:66-70).  The cross-source sum runs in ``dtype``
+    exactly as the reference does (decoder.py:206, 316); the bias is added
+    once per decoder call (parallel.py:380-381).
+    """
+    keys = sorted(acts.keys())
+    if not keys:
+        return torch.zeros((0, d_model), dtype=dtype)
+    batch = 0
+    for kk in keys:
+        if acts[kk].numel() > 0:
+            batch = acts[kk].shape[0]
+            break
+    rec = torch.zeros((batch, d_model), dtype=dtype)
+
+    def usable(s):
+        if s not in acts:
+            return None
+        a = acts[s].to(dtype)
+        if a.numel() == 0 or a.shape[-1] != num_features:
+            return None
+        return a
+
+    if tying == "per_target":
+        summed = torch.zeros((batch, num_features), dtype=dtype)
+        for s in range(layer_idx + 1):
+            a = usable(s)
+            if a is None:
+                continue
+            off = feature_offset[layer_idx] if feature_offset is not None else None
+            sc = feature_scale[layer_idx] if feature_scale is not None else None
+            summed += _affine_on_nonzero(a, off, sc)
+        rec = F.linear(summed, weights[str(layer_idx)]) + biases[str(layer_idx)]
+    else:
+        for s in range(layer_idx + 1):
+            a = usable(s)
+            if a is None:
+                continue
+            if tying == "per_source":
+                off = feature_offset[layer_idx] if feature_offset is not None else None
+                sc = feature_scale[layer_idx] if feature_scale is not None else None
+                a = _affine_on_nonzero(a, off, sc)
+                name = str(s)
+            else:
+                name = f"{s}->{layer_idx}"
+            dec = F.linear(a, weights[name]) + biases[name]
+            if (tying == "none" and skip_weights is not None and source_inputs is not None
+                    and s in source_inputs and f"{s}->{layer_idx}" in skip_weights):
+                src = source_inputs[s].to(dtype)
+                src2 = src.reshape(-1, src.shape[-1])
+                dec = dec + src2 @ skip_weights[f"{s}->{layer_idx}"].T
+            rec = rec + dec
+    if tying in ("per_source", "per_target"):
+        if (skip_weights is not None and source_inputs is not None
+                and layer_idx in source_inputs):
+            src = source_inputs[layer_idx].to(dtype)
+            src2 = src.reshape(-1, src.shape[-1])
+            rec = rec + src2 @ skip_weights[str(layer_idx)].T
+    return rec
+
+
+def decoder_norms(weights: Dict[str, torch.Tensor], num_layers: int,
+                  num_features: int, tying: str, dtype: torch.dtype) -> torch.Tensor:
+    """Decoder.get_decoder_norms at world_size 1 (decoder.py:374-485):
+    norms[s, f] = sqrt(sum over the decoders source s feeds of ||W[:, f]||^2),
+    squared norms accumulated in fp32, result cast to the model dtype."""
+    out = torch.zeros(num_layers, num_features, dtype=dtype)
+    for s in range(num_layers):
+        acc = torch.zeros(num_features, dtype=torch.float32)
+        if tying == "per_source":
+            names = [str(s)]
+        elif tying == "per_target":
+            names = [str(t) for t in range(s, num_layers)]
+        else:
+            names = [f"{s}->{t}" for t in range(s, num_layers)]
+        for n in names:
+            acc += torch.norm(weights[n], dim=0).pow(2).to(torch.float32)
+        out[s] = torch.sqrt(acc).to(dtype)
+    return out
+
+
+# ---------------------------------------------------------------------------
+# whole forward  (reference clt/models/clt.py:186-277)
+# ---------------------------------------------------------------------------
+
+def feature_activations(inputs: Dict[int, torch.Tensor], *, enc_w: List[torch.Tensor],
+                        enc_b: List[torch.Tensor], activation_fn: str, dtype: torch.dtype,
+                        num_layers: int, k: Optional[float] = None,
+                        topk_mode: str = "global",
+                        log_threshold: Optional[torch.Tensor] = None
+                        ) -> Dict[int, torch.Tensor]:
+    """get_feature_activations (clt.py:220-277).
+
+    ``topk_mode="per_layer"`` follows the registry's per-layer functions
+    (clt/activations/registry.py:43-98): the mask is computed per layer on the
+    raw pre-activation.  (In the reference snapshot that mode is routed to
+    ``encode`` and ends in the zero fallback, clt.py:227-234 and 135-149; the
+    per-layer selection itself is what the registry defines.)
+    """
+    xs = {l: inputs[l].to(dtype) for l in inputs}
+    pre = {l: encoder_preactivations(xs[l], enc_w[l], enc_b[l]) for l in sorted(xs)}
+    if activation_fn == "batchtopk":
+        if topk_mode == "per_layer":
+            return {l: batchtopk_forward(pre[l], float(int(k)), pre[l]) for l in pre}
+        return global_batchtopk(pre, num_layers, int(k))
+    if activation_fn == "topk":
+        if topk_mode == "per_layer":
+            return {l: tokentopk_forward(pre[l], float(k), pre[l]) for l in pre}
+        return global_tokentopk(pre, num_layers, float(k))
+    if activation_fn == "jumprelu":
+        return {l: jumprelu_forward(pre[l], theta_from_log(log_threshold[l], dtype)) for l in pre}
+    if activation_fn == "relu":
+        return {l: F.relu(pre[l]) for l in pre}
+    raise ValueError(activation_fn)
+
+
+def forward(inputs: Dict[int, torch.Tensor], *, enc_w, enc_b, dec_w, dec_b,
+            activation_fn: str, dtype: torch.dtype, num_layers: int, d_model: int,
+            num_features: int, tying: str = "none", k: Optional[float] = None,
+            topk_mode: str = "global", log_threshold=None, feature_offset=None,
+            feature_scale=None, skip_weights=None
+            ) -> Tuple[Dict[int, torch.Tensor], Dict[int, torch.Tensor]]:
+    """CrossLayerTranscoder.forward (clt.py:186-218); returns (reconstructions,
+    activations)."""
+    acts = feature_activations(inputs, enc_w=enc_w, enc_b=enc_b, activation_fn=activation_fn,
+                               dtype=dtype, num_layers=num_layers, k=k, topk_mode=topk_mode,
+                               log_threshold=log_threshold)
+    recs: Dict[int, torch.Tensor] = {}
+    for t in range(num_layers):
+        rel = {s: a for s, a in acts.items() if s <= t and a.numel() > 0}
+        if t in inputs and rel:
+            src = ({s: inputs[s] for s in range(t + 1) if s in inputs}
+                   if skip_weights is not None else None)
+            recs[t] = decode(rel, t, tying=tying, weights=dec_w, biases=dec_b, d_model=d_model,
+                             num_features=num_features, dtype=dtype,
+                             feature_offset=feature_offset, feature_scale=feature_scale,
+                             skip_weights=skip_weights, source_inputs=src)
+        elif t in inputs:
+            x = inputs[t]
+            b = x.shape[0] * x.shape[1] if x.dim() == 3 else x.shape[0]
+            recs[t] = torch.zeros((b, d_model), dtype=dtype)
+    return recs, acts
+
+
+# ---------------------------------------------------------------------------
+# float64 references used to pin the torch restatements above
+# ---------------------------------------------------------------------------
+
+def affine_f64(x: np.ndarray, w: np.ndarray, b: Optional[np.ndarray]) -> np.ndarray:
+    """x . w^T + b in float64 (w is [out, in])."""
+    y = x.astype(np.float64) @ w.astype(np.float64).T
+    if b is not None:
+        y = y + b.astype(np.float64)
+    return y
+
+
+def rel_l2(a: torch.Tensor, b: torch.Tensor) -> float:
+    """||a - b|| / ||b|| in float64 (0 when both are all-zero)."""
+    a64 = a.detach().to(torch.float64).cpu()
+    b64 = b.detach().to(torch.float64).cpu()
+    den = float(torch.linalg.vector_norm(b64))
+    num = float(torch.linalg.vector_norm(a64 - b64))
+    if den == 0.0:
+        return 0.0 if num == 0.0 else float("inf")
+    return num / den

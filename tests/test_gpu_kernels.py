@@ -1,0 +1,302 @@
+"""Parity of the HIP kernels (called through the C ABI) with the CPU oracle.
+
+Tolerances: survivor sets, column order and values bit-exact; encoder pre-activations and
+reconstructions rel-L2 <= 1e-2 in bf16 and <= 1e-5 in fp32.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import crosslayer_coding_amd as cca
+from crosslayer_coding_amd import _native as nat
+from crosslayer_coding_amd import engine
+from oracle import clt_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float32: 1e-5, torch.bfloat16: 1e-2}
+
+
+def dense_from(surv):
+    return engine.densify(surv).cpu()
+
+
+def check_rows_sorted(surv):
+    rp = surv.row_ptr.cpu().numpy()
+    col = surv.col.cpu().numpy()
+    assert rp[0] == 0 and np.all(np.diff(rp) >= 0) and rp[-1] == len(col)
+    for r in range(len(rp) - 1):
+        seg = col[rp[r]:rp[r + 1]]
+        assert np.all(np.diff(seg) > 0), f"row {r} not strictly ascending"
+
+
+# ---- encoder --------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("L,T,d,F", [(1, 30, 8, 16), (2, 300, 64, 136), (3, 257, 96, 260), (1, 5, 7, 9), (2, 512, 768, 512)])
+def test_encode_parity(dev, dtype, L, T, d, F):
+    g = torch.Generator().manual_seed(L * 1000 + T)
+    x = torch.randn(L, T, d, generator=g).to(dtype)
+    w = (torch.randn(L, F, d, generator=g) / math.sqrt(d)).to(dtype)
+    b = torch.randn(L, F, generator=g).to(dtype)
+    got = engine.encode(x.to(dev), w.to(dev), b.to(dev)).cpu()
+    for l in range(L):
+        ref = orc.encoder_preactivations(x[l], w[l], b[l])
+        ref64 = torch.from_numpy(orc.affine_f64(x[l].float().numpy(), w[l].float().numpy(), b[l].float().numpy()))
+        assert orc.rel_l2(got[l], ref) <= TOL[dtype]
+        assert orc.rel_l2(got[l], ref64) <= TOL[dtype]
+    nob = engine.encode(x.to(dev), w.to(dev), None).cpu()
+    assert orc.rel_l2(nob[0], orc.encoder_preactivations(x[0], w[0], None)) <= TOL[dtype]
+
+
+# ---- BatchTopK per layer ---------------------------------------------------------------------
+def run_select(pre, k, dev, global_mode=False):
+    surv = engine.batchtopk_select(pre.to(dev), k, global_mode)
+    torch.cuda.synchronize()
+    return surv
+
+
+def oracle_per_layer(pre, k):
+    return torch.stack([orc.batchtopk_forward(pre[l], float(k), pre[l]) for l in range(pre.shape[0])])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("L,T,F,k", [(1, 2, 4, 2), (2, 64, 256, 8), (3, 100, 1000, 17), (1, 33, 77, 5),
+                                     (2, 16, 64, 64), (2, 16, 64, 100), (1, 1, 8, 3), (2, 512, 2048, 40)])
+def test_batchtopk_per_layer_bit_exact(dev, dtype, L, T, F, k):
+    g = torch.Generator().manual_seed(T * 7 + F)
+    pre = torch.randn(L, T, F, generator=g).to(dtype)
+    surv = run_select(pre, k, dev)
+    check_rows_sorted(surv)
+    assert surv.nnz == L * min(k * T, T * F)
+    got = dense_from(surv)
+    ref = oracle_per_layer(pre, k)
+    assert torch.equal(got, ref)
+
+
+def test_batchtopk_reference_known_answer(dev):
+    # reference tests/unit/models/test_activations.py:10-25 : survivors at flat indices {3,4,7,2}
+    x = torch.tensor([[[1.0, 2.0, 3.0, 4.0], [5.0, 1.0, 2.5, 3.5]]])
+    surv = run_select(x, 2, dev)
+    rows = engine.survivor_rows(surv).cpu() * 4 + surv.col.cpu().long()
+    assert sorted(rows.tolist()) == [2, 3, 4, 7]
+    assert torch.equal(dense_from(surv)[0], torch.tensor([[0.0, 0.0, 3.0, 4.0], [5.0, 0.0, 0.0, 3.5]]))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_batchtopk_heavy_ties_lowest_index(dev, dtype):
+    g = torch.Generator().manual_seed(11)
+    pre = (torch.randint(-4, 5, (2, 96, 520), generator=g).float() * 0.25).to(dtype)
+    for k in (3, 50, 300):
+        surv = run_select(pre, k, dev)
+        check_rows_sorted(surv)
+        assert torch.equal(dense_from(surv).to(dtype), oracle_per_layer(pre, k))
+        # zero-valued survivors vanish in the dense form: compare the index sets as well
+        for l in range(2):
+            m = orc.batchtopk_mask(pre[l], k, pre[l])
+            rows = engine.survivor_rows(surv).cpu()
+            sel = (rows >= l * 96) & (rows < (l + 1) * 96)
+            flat = (rows[sel] - l * 96) * 520 + surv.col.cpu().long()[sel]
+            assert torch.equal(torch.sort(flat).values, m.view(-1).nonzero().view(-1))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_batchtopk_special_values(dev, dtype):
+    g = torch.Generator().manual_seed(5)
+    pre = torch.randn(1, 40, 128, generator=g).to(dtype)
+    pre[0, 0, 0], pre[0, 1, 5] = float("nan"), float("inf")
+    pre[0, 2, 7], pre[0, 3, 9] = float("-inf"), -0.0
+    pre[0, 5, :64] = 0.0
+    pre[0, 6, :64] = -0.0
+    for k in (1, 20, 100, 128):
+        surv = run_select(pre, k, dev)
+        m = orc.batchtopk_mask(pre[0], k, pre[0])
+        rows = engine.survivor_rows(surv).cpu()
+        flat = rows * 128 + surv.col.cpu().long()
+        assert torch.equal(torch.sort(flat).values, m.view(-1).nonzero().view(-1)), k
+
+
+def test_batchtopk_all_equal_and_constant_rows(dev):
+    pre = torch.full((2, 50, 96), 1.5)
+    surv = run_select(pre, 10, dev)
+    # all tie: the lowest flat indices win -> the first 500 elements of each layer
+    got = dense_from(surv)
+    ref = oracle_per_layer(pre, 10)
+    assert torch.equal(got, ref) and int((got != 0).sum()) == 2 * 500
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_batchtopk_outlier_rows_overflow_segments(dev, dtype):
+    # a few rows hold nearly all survivors: their candidate segments overflow and are re-read
+    g = torch.Generator().manual_seed(9)
+    L, T, F, k = 2, 256, 4096, 16
+    pre = torch.randn(L, T, F, generator=g)
+    pre[:, 3] += 6.0
+    pre[0, 200] += 8.0
+    pre = pre.to(dtype)
+    surv = run_select(pre, k, dev)
+    check_rows_sorted(surv)
+    assert torch.equal(dense_from(surv), oracle_per_layer(pre, k))
+
+
+def test_batchtopk_k_zero_and_empty(dev):
+    pre = torch.randn(2, 8, 16)
+    surv = run_select(pre, 0, dev)
+    assert surv.nnz == 0 and int(surv.row_ptr.abs().sum()) == 0
+    surv = engine.batchtopk_select(torch.empty(2, 0, 16, device=dev), 3, False)
+    assert surv.nnz == 0
+
+
+# ---- BatchTopK global ------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("L,T,F,k", [(2, 2, 2, 1), (3, 64, 128, 6), (4, 200, 520, 12)])
+def test_batchtopk_global(dev, dtype, L, T, F, k):
+    g = torch.Generator().manual_seed(L + T + F)
+    pre = (torch.randn(L, T, F, generator=g) * (1 + torch.arange(L).view(L, 1, 1))).to(dtype)
+    surv = run_select(pre, k, dev, global_mode=True)
+    check_rows_sorted(surv)
+    assert surv.nnz == min(k * T, T * F * L)
+    got = dense_from(surv)
+    ref = orc.global_batchtopk({l: pre[l] for l in range(L)}, L, k)
+    ref = torch.stack([ref[l] for l in range(L)])
+    # ranking uses per-feature mean/std reductions, whose last-bit rounding differs between
+    # implementations: elements whose z-score is within a relative 2^-6 (bf16) / 1e-5 (fp32)
+    # of the threshold may legitimately differ; everything else must agree exactly.
+    z = torch.cat([orc.zscore_for_ranking(pre[l]) for l in range(L)], dim=1).double()
+    flat = z.reshape(-1)
+    kth = torch.topk(flat, min(k * T, flat.numel())).values[-1]
+    band = (2.0 ** -6 if dtype == torch.bfloat16 else 1e-5) * max(abs(float(kth)), 1e-3)
+    zl = torch.stack([z[:, l * F:(l + 1) * F] for l in range(L)])
+    sure = (zl - kth).abs() > band
+    assert torch.equal((got != 0) & sure, (ref != 0) & sure)
+    assert torch.equal(got[got != 0], torch.stack([pre[l] for l in range(L)])[got != 0])
+    if dtype == torch.float32 and (L, T, F) == (2, 2, 2):
+        assert torch.equal(got, ref)
+
+
+def test_batchtopk_global_closed_form(dev):
+    # hand-computed case of tests/test_oracle_pins.py::test_zscore_closed_form_and_global_selection
+    pre = torch.tensor([[[0.0, 5.0], [2.0, 5.0]], [[10.0, -1.0], [10.0, 3.0]]])
+    got = dense_from(run_select(pre, 1, dev, global_mode=True))
+    assert torch.equal(got[0], torch.tensor([[0.0, 0.0], [2.0, 0.0]]))
+    assert torch.equal(got[1], torch.tensor([[0.0, 0.0], [0.0, 3.0]]))
+
+
+# ---- threshold activations ---------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("L,T,F", [(1, 7, 7), (2, 100, 264), (3, 64, 1000)])
+def test_jumprelu_and_relu_exact(dev, dtype, L, T, F):
+    g = torch.Generator().manual_seed(T + F)
+    pre = torch.randn(L, T, F, generator=g).to(dtype)
+    log_t = torch.log(torch.rand(L, F, generator=g) + 0.3)
+    theta = torch.stack([orc.theta_from_log(log_t[l], dtype) for l in range(L)])
+    pre[0, 0, 0] = theta[0, 0]                     # equality must pass
+    surv = engine.threshold_select(pre.to(dev), theta.to(dev), nat.PRED_GE_THETA)
+    check_rows_sorted(surv)
+    got = engine.densify(surv, out_f32=True).cpu()
+    ref = torch.stack([orc.jumprelu_forward(pre[l], theta[l]) for l in range(L)])
+    assert got.dtype == torch.float32 and torch.equal(got, ref)
+    assert got[0, 0, 0] == theta[0, 0].float()
+    relu = engine.densify(engine.threshold_select(pre.to(dev), None, nat.PRED_GT_ZERO)).cpu()
+    assert torch.equal(relu, torch.relu(pre))
+    nz = engine.densify(engine.threshold_select(relu.to(dev), None, nat.PRED_NONZERO)).cpu()
+    assert torch.equal(nz, relu)
+
+
+def test_jumprelu_reference_known_answer(dev):
+    # reference tests/unit/models/test_activations.py:304-315
+    x = torch.tensor([-2.0, -1.0, -0.4, 0.0, 0.4, 1.0, 2.0], device=dev)
+    out = cca.JumpReLU.apply(x, torch.tensor([0.5], device=dev), 1.0)
+    assert torch.equal(out.cpu(), torch.tensor([0.0, 0.0, 0.0, 0.0, 0.0, 1.0, 2.0]))
+
+
+# ---- pack / densify / norms -------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_pack_is_transpose(dev, dtype):
+    w = torch.randn(70, 130).to(dtype)
+    out = torch.empty(130, 70, dtype=dtype, device=dev)
+    engine.pack_decoder(w.to(dev), out)
+    assert torch.equal(out.cpu(), w.T.contiguous())
+
+
+# ---- sparse decode -------------------------------------------------------------------------------
+def make_decoder(L, d, F, tying, dtype, g):
+    names = [f"{s}->{t}" for s in range(L) for t in range(s, L)] if tying == "none" else [str(i) for i in range(L)]
+    w = {n: (torch.randn(d, F, generator=g) / math.sqrt(F)).to(dtype) for n in names}
+    b = {n: torch.randn(d, generator=g).to(dtype) for n in names}
+    return names, w, b
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("tying", ["none", "per_source", "per_target"])
+@pytest.mark.parametrize("L,T,d,F", [(2, 30, 8, 16), (3, 70, 768, 256), (4, 33, 100, 72), (3, 20, 2048, 64)])
+def test_decode_sparse_parity(dev, dtype, tying, L, T, d, F):
+    g = torch.Generator().manual_seed(L * 31 + d)
+    names, w, b = make_decoder(L, d, F, tying, dtype, g)
+    acts = torch.randn(L, T, F, generator=g) * (torch.rand(L, T, F, generator=g) < 0.1)
+    acts = acts.to(dtype)
+    tied = tying != "none"
+    off = torch.randn(L, F, generator=g).to(dtype) if tied else None
+    sc = torch.randn(L, F, generator=g).to(dtype) if tied else None
+    surv = engine.threshold_select(acts.to(dev), None, nat.PRED_NONZERO)
+    slab = torch.empty(len(names), F, d, dtype=dtype, device=dev)
+    for i, n in enumerate(names):
+        engine.pack_decoder(w[n].to(dev), slab[i])
+    B = torch.stack([b[n].float() for n in names])
+    bias_sum = torch.zeros(L, d)
+    for t in range(L):
+        if tying == "none":
+            for s in range(t + 1):
+                bias_sum[t] += B[names.index(f"{s}->{t}")]
+        elif tying == "per_source":
+            bias_sum[t] = B[: t + 1].sum(0)
+        else:
+            bias_sum[t] = B[t]
+    got = engine.decode_sparse(surv, slab, tying, d, bias_sum=bias_sum.to(dev),
+                               feat_offset=off.to(dev) if tied else None,
+                               feat_scale=sc.to(dev) if tied else None).cpu()
+    for t in range(L):
+        ref = orc.decode({s: acts[s] for s in range(L)}, t, tying=tying, weights=w, biases=b, d_model=d,
+                         num_features=F, dtype=dtype,
+                         feature_offset=list(off) if tied else None, feature_scale=list(sc) if tied else None)
+        assert orc.rel_l2(got[t], ref) <= TOL[dtype], (t, orc.rel_l2(got[t], ref))
+    # fp32 output and a source subset
+    mask = 0b101 if L >= 3 else 0b01
+    sub = engine.decode_sparse(surv, slab, tying, d, src_mask=mask, out_f32=True).cpu()
+    t = L - 1
+    zero_b = {n: torch.zeros_like(v) for n, v in b.items()}
+    ref = orc.decode({s: acts[s] for s in range(L) if (mask >> s) & 1}, t, tying=tying, weights=w, biases=zero_b,
+                     d_model=d, num_features=F, dtype=torch.float32)
+    if tying != "per_target":
+        assert sub.dtype == torch.float32 and orc.rel_l2(sub[t], ref) <= TOL[dtype]
+
+
+def test_decode_linearity_property(dev):
+    # decode(2 * a) - bias == 2 * (decode(a) - bias), exact in fp32 for power-of-two scaling
+    g = torch.Generator().manual_seed(2)
+    L, T, d, F = 3, 64, 768, 512
+    names, w, b = make_decoder(L, d, F, "none", torch.float32, g)
+    acts = torch.randn(L, T, F, generator=g) * (torch.rand(L, T, F, generator=g) < 0.05)
+    slab = torch.empty(len(names), F, d, device=dev)
+    for i, n in enumerate(names):
+        engine.pack_decoder(w[n].to(dev), slab[i])
+    s1 = engine.threshold_select(acts.to(dev), None, nat.PRED_NONZERO)
+    s2 = engine.threshold_select((2 * acts).to(dev), None, nat.PRED_NONZERO)
+    o1 = engine.decode_sparse(s1, slab, "none", d)
+    o2 = engine.decode_sparse(s2, slab, "none", d)
+    assert torch.equal(o2, 2 * o1)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("tying", ["none", "per_source", "per_target"])
+def test_decoder_norms(dev, dtype, tying):
+    g = torch.Generator().manual_seed(8)
+    L, d, F = 3, 40, 50
+    names, w, _ = make_decoder(L, d, F, tying, dtype, g)
+    slab = torch.empty(len(names), F, d, dtype=dtype, device=dev)
+    for i, n in enumerate(names):
+        engine.pack_decoder(w[n].to(dev), slab[i])
+    got = engine.decoder_norms(slab, L, tying).cpu()
+    ref = orc.decoder_norms(w, L, F, tying, dtype)
+    assert orc.rel_l2(got, ref) <= TOL[dtype]

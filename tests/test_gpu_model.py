@@ -1,0 +1,194 @@
+"""CrossLayerTranscoder (host mirror over the HIP kernels) against the CPU oracle's forward."""
+import logging
+
+import pytest
+import torch
+
+import crosslayer_coding_amd as cca
+from crosslayer_coding_amd import synth
+from oracle import clt_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float32: 1e-5, torch.bfloat16: 1e-2}
+
+
+def oracle_forward(wl, sd, x, **extra):
+    dtype = getattr(torch, wl.dtype)
+    L = wl.num_layers
+    enc_w = [sd[f"encoder_module.encoders.{l}.weight"] for l in range(L)]
+    enc_b = [sd[f"encoder_module.encoders.{l}.bias_param"] for l in range(L)]
+    names = synth.decoder_names(wl)
+    dec_w = {n: sd[f"decoder_module.decoders.{n}.weight"] for n in names}
+    dec_b = {n: sd[f"decoder_module.decoders.{n}.bias_param"] for n in names}
+    return orc.forward({l: x[l] for l in range(L)}, enc_w=enc_w, enc_b=enc_b, dec_w=dec_w, dec_b=dec_b,
+                       activation_fn=wl.activation_fn, dtype=dtype, num_layers=L, d_model=wl.d_model,
+                       num_features=wl.num_features, tying=wl.decoder_tying, k=wl.k, topk_mode=wl.topk_mode,
+                       log_threshold=sd.get("theta_manager.log_threshold"), **extra)
+
+
+def build(wl, dev, bias_noise=True):
+    x = synth.make_inputs(wl, "cpu")
+    sd = synth.make_state_dict(wl, "cpu", inputs=x)
+    if bias_noise:
+        g = torch.Generator().manual_seed(77)
+        for k in list(sd):
+            if k.endswith("bias_param") and "decoder" in k:
+                sd[k] = (torch.randn(sd[k].shape, generator=g) * 0.1).to(sd[k].dtype)
+    model = cca.CrossLayerTranscoder(wl.config(), None, dev)
+    model.load_state_dict(sd)
+    return model, sd, x
+
+
+BASE = synth.Workload("tiny", 9, 3, 64, 256, 96, "float32", k=8)
+CASES = [
+    BASE,
+    BASE.scaled("tiny-bf16", dtype="bfloat16"),
+    BASE.scaled("tiny-global", topk_mode="global"),
+    BASE.scaled("tiny-jump", activation_fn="jumprelu", k=None),
+    BASE.scaled("tiny-jump-bf16", activation_fn="jumprelu", k=None, dtype="bfloat16"),
+    BASE.scaled("tiny-relu", activation_fn="relu", k=None),
+    BASE.scaled("tiny-per-target", decoder_tying="per_target", dtype="bfloat16"),
+    BASE.scaled("tiny-per-source", decoder_tying="per_source"),
+    BASE.scaled("ref-shape", num_layers=2, d_model=8, num_features=16, tokens=30, k=3),   # the reference's own test shape
+    BASE.scaled("mid", num_layers=4, d_model=768, num_features=2048, tokens=300, k=20, dtype="bfloat16"),
+]
+
+
+@pytest.mark.parametrize("wl", CASES, ids=lambda w: w.name)
+def test_forward_matches_oracle(dev, wl):
+    dtype = getattr(torch, wl.dtype)
+    model, sd, x = build(wl, dev)
+    inputs = {l: x[l].to(dev) for l in range(wl.num_layers)}
+    recs = model(inputs)
+    ref_recs, ref_acts = oracle_forward(wl, sd, x)
+    assert sorted(recs) == sorted(ref_recs)
+    for t in recs:
+        assert recs[t].shape == ref_recs[t].shape and recs[t].dtype == dtype
+        err = orc.rel_l2(recs[t], ref_recs[t])
+        assert err <= TOL[dtype], (t, err)
+    acts = model.get_feature_activations(inputs)
+    assert sorted(acts) == sorted(ref_acts)
+    if dtype == torch.float32 and wl.topk_mode == "per_layer" or wl.activation_fn in ("relu",):
+        pass
+    for l in acts:
+        assert acts[l].shape == ref_acts[l].shape
+        assert acts[l].dtype == ref_acts[l].dtype
+    # selection parity is judged on identical pre-activations: feed the oracle the GPU's own
+    pre, _ = model._encode_all_layers(inputs)
+    pre_cpu = {l: p.cpu() for l, p in pre.items()}
+    if wl.activation_fn == "batchtopk" and wl.topk_mode == "per_layer":
+        for l in acts:
+            assert torch.equal(acts[l].cpu(), orc.batchtopk_forward(pre_cpu[l], float(wl.k), pre_cpu[l]))
+    elif wl.activation_fn == "jumprelu":
+        lt = sd["theta_manager.log_threshold"]
+        for l in acts:
+            assert torch.equal(acts[l].cpu(), orc.jumprelu_forward(pre_cpu[l], orc.theta_from_log(lt[l], dtype)))
+    elif wl.activation_fn == "relu":
+        for l in acts:
+            assert torch.equal(acts[l].cpu(), torch.relu(pre_cpu[l]))
+    for l in pre:
+        assert orc.rel_l2(pre[l], orc.encoder_preactivations(x[l], sd[f"encoder_module.encoders.{l}.weight"],
+                                                              sd[f"encoder_module.encoders.{l}.bias_param"])) <= TOL[dtype]
+
+
+def test_decode_api_matches_forward(dev):
+    wl = BASE
+    model, sd, x = build(wl, dev)
+    inputs = {l: x[l].to(dev) for l in range(wl.num_layers)}
+    acts = model.get_feature_activations(inputs)
+    recs = model(inputs)
+    for t in range(wl.num_layers):
+        rel = {s: a for s, a in acts.items() if s <= t}
+        out = model.decode(rel, t)
+        assert orc.rel_l2(out, recs[t]) <= 1e-6
+    # additivity over sources (reference tests/unit/models/test_decoder.py:62-81)
+    zero_bias = {k: torch.zeros_like(v) for k, v in sd.items() if k.endswith("bias_param") and "decoder" in k}
+    model.load_state_dict({**sd, **zero_bias})
+    full = model.decode(acts, 2)
+    parts = sum(model.decode({s: acts[s]}, 2) for s in range(3))
+    assert orc.rel_l2(parts, full) <= 1e-5
+
+
+def test_encode_api_and_fallbacks(dev, caplog):
+    wl = BASE.scaled("j", activation_fn="jumprelu", k=None)
+    model, sd, x = build(wl, dev)
+    out = model.encode(x[1].to(dev), 1)
+    pre = model.get_preactivations(x[1].to(dev), 1).cpu()
+    assert out.dtype == torch.float32
+    assert torch.equal(out.cpu(), orc.jumprelu_forward(pre, orc.theta_from_log(sd["theta_manager.log_threshold"][1], torch.float32)))
+    # 3-D input is flattened (reference tests/unit/models/test_encoder.py:50-73)
+    x3 = x[0][:90].view(3, 30, wl.d_model).to(dev)
+    assert model.get_preactivations(x3, 0).shape == (90, wl.num_features)
+    # wrong d_model -> zeros + warning (test_encoder.py:89-103)
+    with caplog.at_level(logging.WARNING):
+        bad = model.get_preactivations(torch.randn(5, wl.d_model + 1, device=dev), 0)
+    assert bad.shape == (5, wl.num_features) and float(bad.abs().sum()) == 0
+    assert "Input d_model" in caplog.text
+    caplog.clear()
+    # out-of-range layer -> zeros + error (test_encoder.py:105-117)
+    with caplog.at_level(logging.ERROR):
+        bad = model.get_preactivations(x[0].to(dev), 99)
+    assert bad.shape == (wl.tokens, wl.num_features) and float(bad.abs().sum()) == 0
+    assert "Invalid layer index" in caplog.text
+    # 1-D input (test_encoder.py:145-162)
+    bad = model.get_preactivations(torch.randn(wl.d_model, device=dev), 0)
+    assert bad.shape == (wl.d_model, wl.num_features)
+    # empty activation dict (test_decoder.py:83-92)
+    assert model.decode({}, 0).shape == (0, wl.d_model)
+
+
+def test_forward_subset_of_layers_and_bad_layer(dev):
+    wl = BASE
+    model, sd, x = build(wl, dev)
+    inputs = {0: x[0].to(dev), 2: x[2].to(dev)}
+    recs = model(inputs)
+    ref, _ = oracle_forward(wl, sd, {0: x[0], 2: x[2]}) if False else (None, None)
+    assert sorted(recs) == [0, 2]
+    L = wl.num_layers
+    enc_w = [sd[f"encoder_module.encoders.{l}.weight"] for l in range(L)]
+    enc_b = [sd[f"encoder_module.encoders.{l}.bias_param"] for l in range(L)]
+    names = synth.decoder_names(wl)
+    ref, _ = orc.forward({0: x[0], 2: x[2]}, enc_w=enc_w, enc_b=enc_b,
+                         dec_w={n: sd[f"decoder_module.decoders.{n}.weight"] for n in names},
+                         dec_b={n: sd[f"decoder_module.decoders.{n}.bias_param"] for n in names},
+                         activation_fn="batchtopk", dtype=torch.float32, num_layers=L, d_model=wl.d_model,
+                         num_features=wl.num_features, k=wl.k, topk_mode="per_layer")
+    for t in recs:
+        assert orc.rel_l2(recs[t], ref[t]) <= 1e-5
+
+
+def test_state_dict_round_trip_and_tied_migration(dev, tmp_path):
+    from safetensors.torch import load_file, save_file
+
+    wl = BASE.scaled("s", num_layers=2, d_model=8, num_features=16, tokens=10, k=3)
+    model, sd, x = build(wl, dev)
+    path = str(tmp_path / "clt.safetensors")
+    save_file({k: v.contiguous() for k, v in model.state_dict().items()}, path)
+    loaded = load_file(path)
+    assert set(loaded) == set(sd)
+    for k in sd:
+        assert loaded[k].shape == sd[k].shape and torch.equal(loaded[k], sd[k])
+    m2 = cca.CrossLayerTranscoder(wl.config(), None, dev)
+    m2.load_state_dict(loaded)
+    inputs = {l: x[l].to(dev) for l in range(2)}
+    a, b = model(inputs), m2(inputs)
+    assert all(torch.equal(a[t], b[t]) for t in a)
+    # untied checkpoint into a per_source model keeps the diagonal decoders
+    tied_cfg = wl.scaled("t", decoder_tying="per_source").config()
+    m3 = cca.CrossLayerTranscoder(tied_cfg, None, dev)
+    m3.load_state_dict(loaded, strict=False)
+    assert torch.equal(m3.decoder_module.decoders[1].weight.cpu(), sd["decoder_module.decoders.1->1.weight"])
+
+
+def test_model_to_device_keeps_results(dev):
+    wl = BASE.scaled("m", tokens=40)
+    x = synth.make_inputs(wl, "cpu")
+    sd = synth.make_state_dict(wl, "cpu")
+    model = cca.CrossLayerTranscoder(wl.config(), None, torch.device("cpu"))
+    model.load_state_dict(sd)
+    model = model.to(dev)
+    recs = model({l: x[l].to(dev) for l in range(wl.num_layers)})
+    ref, _ = oracle_forward(wl, sd, x)
+    for t in recs:
+        assert orc.rel_l2(recs[t], ref[t]) <= 1e-5

@@ -1,0 +1,236 @@
+"""Pins the CPU oracle: the reference's own known-answer vectors, brute force on small
+inputs, and closed forms.  Vector sources are cited per test (paths relative to the
+reference checkout)."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import clt_oracle as orc
+
+
+# ---- BatchTopK: reference tests/unit/models/test_activations.py -------------------------
+def test_batchtopk_mask_known_answer():
+    # test_activations.py:10-25 : indices {3, 4, 7, 2}
+    x = torch.tensor([[1.0, 2.0, 3.0, 4.0], [5.0, 1.0, 2.5, 3.5]])
+    mask = orc.batchtopk_mask(x, 2)
+    expect = torch.zeros(8, dtype=torch.bool)
+    expect[torch.tensor([3, 4, 7, 2])] = True
+    assert mask.dtype == torch.bool and mask.shape == x.shape
+    assert torch.equal(mask.view(-1), expect)
+
+
+def test_batchtopk_edge_cases():
+    # test_activations.py:28-63
+    x = torch.randn(2, 4)
+    assert orc.batchtopk_mask(x, 0).sum() == 0
+    assert bool(orc.batchtopk_mask(x, 4).all())
+    assert bool(orc.batchtopk_mask(x, 5).all())
+    assert orc.batchtopk_mask(torch.empty(0, 4), 2).shape == (0, 4)
+    assert orc.batchtopk_mask(torch.empty(2, 0), 2).shape == (2, 0)
+
+
+def test_batchtopk_forward_known_answer():
+    # test_activations.py:66-90 : [[0,0,3,4],[5,0,0,3.5]]
+    x = torch.tensor([[1.0, 2.0, 3.0, 4.0], [5.0, 1.0, 2.5, 3.5]])
+    out = orc.batchtopk_forward(x, 2.0)
+    assert torch.equal(out, torch.tensor([[0.0, 0.0, 3.0, 4.0], [5.0, 0.0, 0.0, 3.5]]))
+
+
+def test_batchtopk_ranking_override_known_answer():
+    # test_activations.py:92-111 : the second row is selected, the values come from x
+    x = torch.tensor([[1.0, 2.0, 3.0, 4.0], [0.0, 0.0, 0.0, 0.0]])
+    r = torch.tensor([[0.0, 0.0, 0.0, 0.0], [5.0, 6.0, 7.0, 8.0]])
+    mask = orc.batchtopk_mask(x, 2, r)
+    assert torch.equal(mask, torch.tensor([[False] * 4, [True] * 4]))
+    assert torch.equal(orc.batchtopk_forward(x, 2.0, r), torch.zeros(2, 4))
+
+
+def test_batchtopk_keeps_negatives():
+    x = torch.tensor([[-1.0, -2.0, -3.0]])
+    assert torch.equal(orc.batchtopk_forward(x, 2.0), torch.tensor([[-1.0, -2.0, 0.0]]))
+
+
+def _brute_force_topk(values, k_total):
+    """Independent selector: python sort on (value desc, index asc) with explicit float rules."""
+    def sort_key(iv):
+        i, v = iv
+        if math.isnan(v):
+            return (0, 0.0, i)       # NaN first (largest)
+        return (1, -(v + 0.0), i)    # -0.0 + 0.0 == +0.0
+    order = sorted(enumerate(values), key=sort_key)
+    return sorted(i for i, _ in order[:k_total])
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_batchtopk_matches_brute_force_with_ties(seed):
+    g = torch.Generator().manual_seed(seed)
+    B, F, k = 7, 13, 3
+    x = torch.randint(-3, 4, (B, F), generator=g).float() * 0.5   # heavy ties
+    if seed % 2:
+        x[0, 0], x[1, 1] = float("nan"), float("inf")
+        x[2, 2], x[3, 3] = -0.0, 0.0
+    got = orc.batchtopk_mask(x, k).view(-1).nonzero().view(-1).tolist()
+    assert got == _brute_force_topk(x.view(-1).tolist(), k * B)
+
+
+def test_batchtopk_invariants_bf16():
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(32, 64, generator=g).to(torch.bfloat16)
+    mask = orc.batchtopk_mask(x, 5)
+    assert int(mask.sum()) == 5 * 32
+    assert float(x[mask].float().min()) >= float(x[~mask].float().max())
+
+
+# ---- TokenTopK: test_activations.py:158-283 ------------------------------------------------
+def test_tokentopk_known_answers():
+    x = torch.tensor([[1.0, 2.0, 3.0, 4.0], [5.0, 1.0, 2.5, 3.5]])
+    assert torch.equal(orc.tokentopk_mask(x, 0.5),
+                       torch.tensor([[False, False, True, True], [True, False, False, True]]))
+    assert torch.equal(orc.tokentopk_mask(x, 1.0),
+                       torch.tensor([[False, False, False, True], [True, False, False, False]]))
+    assert orc.tokentopk_mask(x, 0.0).sum() == 0 and orc.tokentopk_mask(x, -0.5).sum() == 0
+    assert bool(orc.tokentopk_mask(x, 4.0).all()) and bool(orc.tokentopk_mask(x, 5.0).all())
+    y = torch.randn(2, 5)
+    assert orc.tokentopk_mask(y, 0.6).sum(dim=1).tolist() == [3, 3]   # ceil(3.0)
+    assert orc.tokentopk_mask(y, 0.5).sum(dim=1).tolist() == [3, 3]   # ceil(2.5)
+    assert orc.tokentopk_mask(torch.empty(0, 4), 0.5).shape == (0, 4)
+
+
+def test_tokentopk_ranking_override_known_answer():
+    # test_activations.py:255-272
+    x = torch.tensor([[1.0, 2.0, 3.0, 4.0], [10.0, 10.0, 10.0, 10.0]])
+    r = torch.tensor([[4.0, 3.0, 2.0, 1.0], [1.0, 2.0, 3.0, 4.0]])
+    assert torch.equal(orc.tokentopk_forward(x, 0.5, r), torch.tensor([[1.0, 2.0, 0.0, 0.0], [0.0, 0.0, 10.0, 10.0]]))
+
+
+# ---- JumpReLU: test_activations.py:304-315, test_theta.py:79-92 --------------------------------
+def test_jumprelu_known_answer():
+    x = torch.tensor([-2.0, -1.0, -0.4, 0.0, 0.4, 1.0, 2.0])
+    out = orc.jumprelu_forward(x, torch.tensor([0.5]))
+    assert torch.equal(out, torch.tensor([0.0, 0.0, 0.0, 0.0, 0.0, 1.0, 2.0]))
+    assert out.dtype == torch.float32
+
+
+def test_jumprelu_is_where_ge_theta_and_fp32():
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(10, 16, generator=g).to(torch.bfloat16)
+    log_t = torch.full((16,), math.log(0.5))
+    theta = orc.theta_from_log(log_t, torch.bfloat16)
+    out = orc.jumprelu_forward(x, theta)
+    assert out.dtype == torch.float32
+    assert torch.equal(out, torch.where(x >= theta, x, torch.zeros_like(x)).float())
+    x[0, 0] = theta[0]      # equality passes (>=)
+    assert orc.jumprelu_forward(x, theta)[0, 0] == theta[0].float()
+
+
+# ---- encoder: affine map ---------------------------------------------------------------------
+def test_encoder_matches_float64_contraction():
+    g = torch.Generator().manual_seed(1)
+    x, w, b = torch.randn(9, 8, generator=g), torch.randn(16, 8, generator=g), torch.randn(16, generator=g)
+    got = orc.encoder_preactivations(x, w, b)
+    ref = orc.affine_f64(x.numpy(), w.numpy(), b.numpy())
+    assert np.allclose(got.numpy(), ref, rtol=1e-5, atol=1e-5)
+    assert orc.encoder_preactivations(x.view(3, 3, 8), w, b).shape == (9, 16)
+    # transposed-operand mistake would fail this: a one-hot input picks a weight column
+    e = torch.zeros(1, 8); e[0, 2] = 1.0
+    assert torch.allclose(orc.encoder_preactivations(e, w, None)[0], w[:, 2])
+
+
+# ---- global helper: closed form of the z-score -----------------------------------------------
+def test_zscore_closed_form_and_global_selection():
+    # column 0: values 0,2 -> mean 1, unbiased std sqrt(2); column 1 constant -> std 0 -> /1e-6
+    pre = torch.tensor([[0.0, 5.0], [2.0, 5.0]])
+    z = orc.zscore_for_ranking(pre)
+    s = math.sqrt(2.0)
+    assert torch.allclose(z[:, 0], torch.tensor([-1.0 / (s + 1e-6), 1.0 / (s + 1e-6)]))
+    assert torch.equal(z[:, 1], torch.zeros(2))
+    # two layers, k=1 per token -> 2 survivors over the [2, 4] block ranked on z, raw values kept
+    pre0 = torch.tensor([[0.0, 5.0], [2.0, 5.0]])
+    pre1 = torch.tensor([[10.0, -1.0], [10.0, 3.0]])
+    out = orc.global_batchtopk({0: pre0, 1: pre1}, 2, 1)
+    # z: layer0 col0 = -.707/+.707, col1 = 0,0 ; layer1 col0 = 0,0, col1 = -.707/+.707
+    # top-2 z are (t=1,l=0,f=0) and (t=1,l=1,f=1); the large raw 10.0 is not selected
+    assert torch.equal(out[0], torch.tensor([[0.0, 0.0], [2.0, 0.0]]))
+    assert torch.equal(out[1], torch.tensor([[0.0, 0.0], [0.0, 3.0]]))
+
+
+# ---- decoder -------------------------------------------------------------------------------------
+def _dec_params(L, d, F, tying, g, dtype=torch.float32):
+    names = [f"{s}->{t}" for s in range(L) for t in range(s, L)] if tying == "none" else [str(i) for i in range(L)]
+    w = {n: torch.randn(d, F, generator=g).to(dtype) for n in names}
+    b = {n: torch.randn(d, generator=g).to(dtype) for n in names}
+    return w, b
+
+
+def test_decode_additivity_and_loop_reference():
+    # additivity over sources: reference tests/unit/models/test_decoder.py:62-81
+    g = torch.Generator().manual_seed(2)
+    L, d, F, T = 3, 4, 6, 5
+    w, b = _dec_params(L, d, F, "none", g)
+    a = {s: torch.randn(T, F, generator=g) * (torch.rand(T, F, generator=g) > 0.5) for s in range(L)}
+    kw = dict(tying="none", weights=w, biases=b, d_model=d, num_features=F, dtype=torch.float32)
+    full = orc.decode(a, 2, **kw)
+    parts = sum(orc.decode({s: a[s]}, 2, **kw) for s in range(3))
+    assert torch.allclose(full, parts, atol=1e-5)
+    # explicit float64 loops (target 1: sources 0 and 1, one bias per decoder)
+    ref = np.zeros((T, d))
+    for s in (0, 1):
+        W = w[f"{s}->1"].double().numpy()
+        for tok in range(T):
+            for f in range(F):
+                ref[tok] += float(a[s][tok, f]) * W[:, f]
+        ref += b[f"{s}->1"].double().numpy()
+    assert np.allclose(orc.decode(a, 1, **kw).numpy(), ref, atol=1e-5)
+    assert orc.decode({}, 1, **kw).shape == (0, d)                    # test_decoder.py:83-92
+    bad = dict(a); bad[1] = torch.randn(T, F + 1)                      # test_decoder.py:94-112
+    assert torch.allclose(orc.decode(bad, 1, **kw), orc.decode({0: a[0]}, 1, **kw))
+
+
+def test_decode_tied_variants():
+    g = torch.Generator().manual_seed(4)
+    L, d, F, T = 3, 4, 6, 5
+    a = {s: torch.randn(T, F, generator=g) * (torch.rand(T, F, generator=g) > 0.5) for s in range(L)}
+    # zero-initialised tied decoders give zero output (test_tied_decoders.py:138-166)
+    zw = {str(i): torch.zeros(d, F) for i in range(L)}
+    zb = {str(i): torch.zeros(d) for i in range(L)}
+    for tying in ("per_source", "per_target"):
+        out = orc.decode(a, 2, tying=tying, weights=zw, biases=zb, d_model=d, num_features=F, dtype=torch.float32)
+        assert torch.equal(out, torch.zeros(T, d))
+    w, b = _dec_params(L, d, F, "per_target", g)
+    off = [torch.randn(F, generator=g) for _ in range(L)]
+    sc = [torch.randn(F, generator=g) for _ in range(L)]
+    out = orc.decode(a, 1, tying="per_target", weights=w, biases=b, d_model=d, num_features=F,
+                     dtype=torch.float32, feature_offset=off, feature_scale=sc)
+    summed = torch.zeros(T, F)
+    for s in (0, 1):
+        summed += torch.where(a[s] != 0, (a[s] + off[1]) * sc[1], torch.zeros(()))
+    assert torch.allclose(out, summed @ w["1"].T + b["1"], atol=1e-5)
+    out_ps = orc.decode(a, 1, tying="per_source", weights=w, biases=b, d_model=d, num_features=F,
+                        dtype=torch.float32, feature_offset=off, feature_scale=sc)
+    ref = sum(torch.where(a[s] != 0, (a[s] + off[1]) * sc[1], torch.zeros(())) @ w[str(s)].T + b[str(s)] for s in (0, 1))
+    assert torch.allclose(out_ps, ref, atol=1e-5)
+
+
+def test_decoder_norms_closed_form():
+    L, d, F = 2, 2, 2
+    w = {"0->0": torch.tensor([[3.0, 0.0], [4.0, 1.0]]), "0->1": torch.tensor([[0.0, 2.0], [0.0, 0.0]]),
+         "1->1": torch.tensor([[1.0, 1.0], [1.0, 1.0]])}
+    n = orc.decoder_norms(w, L, F, "none", torch.float32)
+    assert torch.allclose(n, torch.tensor([[5.0, math.sqrt(5.0)], [math.sqrt(2.0), math.sqrt(2.0)]]))
+
+
+def test_forward_wiring_small():
+    g = torch.Generator().manual_seed(5)
+    L, d, F, T = 2, 8, 16, 30
+    enc_w = [torch.randn(F, d, generator=g) for _ in range(L)]
+    enc_b = [torch.randn(F, generator=g) for _ in range(L)]
+    w, b = _dec_params(L, d, F, "none", g)
+    x = {l: torch.randn(T, d, generator=g) for l in range(L)}
+    recs, acts = orc.forward(x, enc_w=enc_w, enc_b=enc_b, dec_w=w, dec_b=b, activation_fn="batchtopk",
+                             dtype=torch.float32, num_layers=L, d_model=d, num_features=F, k=3, topk_mode="global")
+    assert set(recs) == {0, 1} and recs[0].shape == (T, d) and acts[1].shape == (T, F)
+    assert sum(int((a != 0).sum()) for a in acts.values()) == 3 * T
+    r1 = acts[0] @ w["0->1"].T + b["0->1"] + acts[1] @ w["1->1"].T + b["1->1"]
+    assert torch.allclose(recs[1], r1, atol=1e-5)
