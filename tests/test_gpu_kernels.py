@@ -267,7 +267,7 @@ def test_decode_sparse_parity(dev, dtype, tying, L, T, d, F):
     t = L - 1
     zero_b = {n: torch.zeros_like(v) for n, v in b.items()}
     ref = orc.decode({s: acts[s] for s in range(L) if (mask >> s) & 1}, t, tying=tying, weights=w, biases=zero_b,
-                     d_model=d, num_features=F, dtype=torch.float32)
+                     d_model=d, num_features=F, dtype=dtype)
     if tying != "per_target":
         assert sub.dtype == torch.float32 and orc.rel_l2(sub[t], ref) <= TOL[dtype]
 
