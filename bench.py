@@ -1,0 +1,211 @@
+#!/usr/bin/env python3
+"""CLT forward benchmark on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1] [--no-cpu]
+
+One step = one forward pass (encoder projection of all layers -> BatchTopK selection ->
+sparse cross-layer decode of all targets) over one synthetic batch that is already
+resident in HBM.  Prints ONE JSON line: whole-forward tokens/s, the roofline of the
+dominant kernel (the sparse decode) measured with HIP events around its launch, the
+per-stage figures, and a CPU baseline (the reference's dense algorithm, restated in
+``oracle/``, timed on the host cores on a bounded sample of the same workload).
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, GB/s
+MFMA_BF16_PEAK_TF = 2500.0  # dense bf16, TFLOP/s
+MFMA_FP32_PEAK_TF = 157.3
+
+
+def algorithmic_work(wl, nnz_rows_pairs: int, nnz_total: int):
+    """Algorithmic flops / bytes per forward, by stage (e = bytes per element)."""
+    e = 2 if wl.dtype == "bfloat16" else 4
+    L, T, d, F = wl.num_layers, wl.tokens, wl.d_model, wl.num_features
+    P = nnz_rows_pairs  # (token, feature, source->target) triples that fetch a decoder vector
+    n_dec = L * (L + 1) // 2 if wl.decoder_tying == "none" else L
+    return {
+        "encoder_flop": 2.0 * T * d * F * L,
+        "select_bytes": float(L * T * F * e + nnz_total * (4 + e)),
+        "decode_gathered_bytes": float(P * d * e + P * (4 + e) + L * T * d * e),
+        "decode_compulsory_bytes": float(n_dec * F * d * e + P * (4 + e) + L * T * d * e),
+    }
+
+
+def gpu_events(n):
+    return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
+
+
+def run_gpu(args):
+    import crosslayer_coding_amd as cca
+    from crosslayer_coding_amd import engine, synth
+
+    wl = synth.WORKLOADS[args.workload]
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    cca._native.load(build_if_missing=False)
+    model, inputs, slab = synth.build_model(wl, dev)
+    model.eval()
+    L, T = wl.num_layers, wl.tokens
+
+    for _ in range(args.warmup):
+        out = model(inputs)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        out = model(inputs)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall / args.steps * 1e3
+    del out
+
+    # per-stage durations: the same three launches, bracketed by events on the launch stream
+    enc, dec = model.encoder_module, model.decoder_module
+    ws = model._workspace()
+    pre_buf = ws.typed("pre", (L, T, wl.num_features), model.dtype)
+    glob = wl.topk_mode != "per_layer"
+    src_mask = (1 << L) - 1
+    st = {"encode": 0.0, "select": 0.0, "decode": 0.0}
+    surv = None
+    for _ in range(args.steps):
+        ev = gpu_events(4)
+        ev[0].record()
+        _, pre = enc.encode_slab(inputs, out=pre_buf)
+        ev[1].record()
+        if wl.activation_fn == "batchtopk":
+            surv = engine.batchtopk_select(pre, wl.k, glob, ws)
+        else:
+            surv = model._survivors(inputs)[2]
+        ev[2].record()
+        rec = dec.decode_survivors(surv, src_mask)
+        ev[3].record()
+        torch.cuda.synchronize()
+        st["encode"] += ev[0].elapsed_time(ev[1])
+        st["select"] += ev[1].elapsed_time(ev[2])
+        st["decode"] += ev[2].elapsed_time(ev[3])
+    for k in st:
+        st[k] /= args.steps
+    del rec
+
+    counts = (surv.row_ptr[1:] - surv.row_ptr[:-1]).view(L, T).sum(dim=1).tolist()
+    nnz_total = int(sum(counts))
+    # every survivor of source s fetches one decoder vector for each target t >= s
+    pairs = int(sum(counts[s] * (L - s) for s in range(L)))
+    work = algorithmic_work(wl, pairs, nnz_total)
+    enc_tf = work["encoder_flop"] / (st["encode"] * 1e-3) / 1e12
+    sel_gbs = work["select_bytes"] / (st["select"] * 1e-3) / 1e9
+    dec_gbs = work["decode_gathered_bytes"] / (st["decode"] * 1e-3) / 1e9
+    dec_c_gbs = work["decode_compulsory_bytes"] / (st["decode"] * 1e-3) / 1e9
+    mfma_peak = MFMA_BF16_PEAK_TF if wl.dtype == "bfloat16" else MFMA_FP32_PEAK_TF
+    result = {
+        "metric": "CLT forward tokens/sec at GPT-2-small x32 BatchTopK k=200; % of roofline per stage",
+        "value": T * args.steps / wall,
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if wl.dtype == "bfloat16" else "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": f"{wl.name}: CLT forward, L={L} d_model={wl.d_model} F={wl.num_features} T={T} "
+                        f"{wl.activation_fn} k={wl.k} ({wl.topk_mode}), decoders {wl.decoder_tying}",
+            "global_batch_tokens": T,
+            "survivors_per_layer": counts[0],
+        },
+        "roofline": {
+            "kernel": "k_decode (sparse cross-layer decode, all targets in one launch)",
+            "bound": "hbm",
+            "achieved": dec_gbs,
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": dec_gbs / HBM_PEAK_GBS,
+            "traffic": None,
+            "algorithmic_bytes_per_launch": work["decode_gathered_bytes"],
+            "avg_launch_ms": st["decode"],
+        },
+        "stages": {
+            "encoder": {"ms": st["encode"], "bound": "mfma", "achieved": enc_tf, "peak": mfma_peak,
+                        "unit": "TFLOP/s", "frac": enc_tf / mfma_peak},
+            "select": {"ms": st["select"], "bound": "hbm", "achieved": sel_gbs, "peak": HBM_PEAK_GBS,
+                       "unit": "GB/s", "frac": sel_gbs / HBM_PEAK_GBS},
+            "decode": {"ms": st["decode"], "bound": "hbm", "achieved": dec_gbs, "peak": HBM_PEAK_GBS,
+                       "unit": "GB/s", "frac": dec_gbs / HBM_PEAK_GBS,
+                       "compulsory_GBps": dec_c_gbs, "compulsory_frac": dec_c_gbs / HBM_PEAK_GBS},
+        },
+    }
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(wl, model, slab, args.cpu_tokens)
+    return result
+
+
+def cpu_baseline(wl, model, slab, tokens):
+    """The reference's dense forward (F.linear encoder, torch.topk mask, one dense F.linear
+    per decoder, sum in the model dtype) from ``oracle/``, on the first ``tokens`` tokens of
+    the same batch with the same weights, on the host cores."""
+    from oracle import clt_oracle as orc
+
+    L = wl.num_layers
+    dtype = getattr(torch, wl.dtype)
+    sd = {k: v.detach().cpu() for k, v in model.state_dict().items()}
+    enc_w = [sd[f"encoder_module.encoders.{l}.weight"] for l in range(L)]
+    enc_b = [sd[f"encoder_module.encoders.{l}.bias_param"] for l in range(L)]
+    from crosslayer_coding_amd import synth
+
+    names = synth.decoder_names(wl)
+    dec_w = {n: sd[f"decoder_module.decoders.{n}.weight"] for n in names}
+    dec_b = {n: sd[f"decoder_module.decoders.{n}.bias_param"] for n in names}
+    x = {l: slab[l, :tokens].detach().cpu() for l in range(L)}
+    cores = torch.get_num_threads()
+    t0 = time.perf_counter()
+    orc.forward(x, enc_w=enc_w, enc_b=enc_b, dec_w=dec_w, dec_b=dec_b, activation_fn=wl.activation_fn,
+                dtype=dtype, num_layers=L, d_model=wl.d_model, num_features=wl.num_features,
+                tying=wl.decoder_tying, k=wl.k, topk_mode=wl.topk_mode,
+                log_threshold=sd.get("theta_manager.log_threshold"), timed_baseline=True)
+    dt = time.perf_counter() - t0
+    return {
+        "value": tokens / dt,
+        "unit": "tokens/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"one dense forward of the first {tokens} tokens of the {wl.name} batch "
+                  f"(same weights, {wl.dtype}, torch {torch.__version__} CPU ops, {dt:.1f} s)",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="c1")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-tokens", type=int, default=1024)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures the one-GPU forward path; this build has no multi-GPU path "
+              f"(asked for --gpus {args.gpus})", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a ROCm GPU", file=sys.stderr)
+        sys.exit(2)
+    print(json.dumps(run_gpu(args)))
+
+
+if __name__ == "__main__":
+    main()

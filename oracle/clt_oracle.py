@@ -100,10 +100,27 @@ def batchtopk_mask(x: torch.Tensor, k_per_token: int,
     return torch.from_numpy(mask).view(x.shape)
 
 
-def batchtopk_forward(x: torch.Tensor, k: float,
-                      x_for_ranking: Optional[torch.Tensor] = None) -> torch.Tensor:
+def batchtopk_mask_topk(x: torch.Tensor, k_per_token: int,
+                        x_for_ranking: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The same mask through the reference's own op sequence - torch.topk(sorted=False)
+    then an index write (activations.py:21-32).  Ties fall wherever torch.topk puts them,
+    so this variant is used for the timed CPU baseline only, never as the parity checker."""
+    B = x.size(0)
+    if k_per_token <= 0 or x.numel() == 0:
+        return torch.zeros_like(x, dtype=torch.bool)
+    k_total = min(int(k_per_token) * B, x.numel())
+    rank = x_for_ranking if x_for_ranking is not None else x
+    _, idx = torch.topk(rank.reshape(-1), k_total, sorted=False)
+    mask = torch.zeros(x.numel(), dtype=torch.bool)
+    mask[idx] = True
+    return mask.view_as(x)
+
+
+def batchtopk_forward(x: torch.Tensor, k: float, x_for_ranking: Optional[torch.Tensor] = None,
+                      timed_baseline: bool = False) -> torch.Tensor:
     """BatchTopK.forward (activations.py:39-65): x * mask, negatives kept."""
-    mask = batchtopk_mask(x, int(k), x_for_ranking)
+    fn = batchtopk_mask_topk if timed_baseline else batchtopk_mask
+    mask = fn(x, int(k), x_for_ranking)
     return x * mask.to(x.dtype)
 
 
@@ -187,7 +204,7 @@ def zscore_for_ranking(pre: torch.Tensor) -> torch.Tensor:
 
 
 def global_batchtopk(preacts: Dict[int, torch.Tensor], num_layers: int,
-                     k: int) -> Dict[int, torch.Tensor]:
+                     k: int, timed_baseline: bool = False) -> Dict[int, torch.Tensor]:
     """_apply_batch_topk_helper at world_size 1 (activations.py:261-357).
 
     Layers are concatenated in range(num_layers) order to [T, sum F], the
@@ -199,7 +216,7 @@ def global_batchtopk(preacts: Dict[int, torch.Tensor], num_layers: int,
         return {}
     orig = torch.cat([preacts[l] for l in layers], dim=1)
     norm = torch.cat([zscore_for_ranking(preacts[l]) for l in layers], dim=1)
-    mask = batchtopk_mask(orig, int(k), norm)
+    mask = (batchtopk_mask_topk if timed_baseline else batchtopk_mask)(orig, int(k), norm)
     act = orig * mask.to(orig.dtype)
     out, off = {}, 0
     for l in layers:
@@ -348,8 +365,8 @@ def feature_activations(inputs: Dict[int, torch.Tensor], *, enc_w: List[torch.Te
                         enc_b: List[torch.Tensor], activation_fn: str, dtype: torch.dtype,
                         num_layers: int, k: Optional[float] = None,
                         topk_mode: str = "global",
-                        log_threshold: Optional[torch.Tensor] = None
-                        ) -> Dict[int, torch.Tensor]:
+                        log_threshold: Optional[torch.Tensor] = None,
+                        timed_baseline: bool = False) -> Dict[int, torch.Tensor]:
     """get_feature_activations (clt.py:220-277).
 
     ``topk_mode="per_layer"`` follows the registry's per-layer functions
@@ -362,8 +379,8 @@ def feature_activations(inputs: Dict[int, torch.Tensor], *, enc_w: List[torch.Te
     pre = {l: encoder_preactivations(xs[l], enc_w[l], enc_b[l]) for l in sorted(xs)}
     if activation_fn == "batchtopk":
         if topk_mode == "per_layer":
-            return {l: batchtopk_forward(pre[l], float(int(k)), pre[l]) for l in pre}
-        return global_batchtopk(pre, num_layers, int(k))
+            return {l: batchtopk_forward(pre[l], float(int(k)), pre[l], timed_baseline) for l in pre}
+        return global_batchtopk(pre, num_layers, int(k), timed_baseline)
     if activation_fn == "topk":
         if topk_mode == "per_layer":
             return {l: tokentopk_forward(pre[l], float(k), pre[l]) for l in pre}
@@ -379,13 +396,13 @@ def forward(inputs: Dict[int, torch.Tensor], *, enc_w, enc_b, dec_w, dec_b,
             activation_fn: str, dtype: torch.dtype, num_layers: int, d_model: int,
             num_features: int, tying: str = "none", k: Optional[float] = None,
             topk_mode: str = "global", log_threshold=None, feature_offset=None,
-            feature_scale=None, skip_weights=None
+            feature_scale=None, skip_weights=None, timed_baseline: bool = False
             ) -> Tuple[Dict[int, torch.Tensor], Dict[int, torch.Tensor]]:
     """CrossLayerTranscoder.forward (clt.py:186-218); returns (reconstructions,
     activations)."""
     acts = feature_activations(inputs, enc_w=enc_w, enc_b=enc_b, activation_fn=activation_fn,
                                dtype=dtype, num_layers=num_layers, k=k, topk_mode=topk_mode,
-                               log_threshold=log_threshold)
+                               log_threshold=log_threshold, timed_baseline=timed_baseline)
     recs: Dict[int, torch.Tensor] = {}
     for t in range(num_layers):
         rel = {s: a for s, a in acts.items() if s <= t and a.numel() > 0}
