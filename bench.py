@@ -89,7 +89,7 @@ def run_gpu(args):
         else:
             surv = model._survivors(inputs)[2]
         ev[2].record()
-        rec = dec.decode_survivors(surv, src_mask)
+        rec = dec.decode_survivors(surv, src_mask, ws=ws)
         ev[3].record()
         torch.cuda.synchronize()
         st["encode"] += ev[0].elapsed_time(ev[1])

@@ -309,7 +309,8 @@ class CrossLayerTranscoder(BaseTranscoder):
                 src_mask |= 1 << l
             skip = (self.decoder_module.skip_all_targets(inputs, src_mask, T) if cfg.skip_connection else None)
             targets = [t for t in range(L) if t in inputs]
-            out = self.decoder_module.decode_survivors(full, src_mask, min(targets), max(targets) + 1, skip_add=skip)
+            out = self.decoder_module.decode_survivors(full, src_mask, min(targets), max(targets) + 1, skip_add=skip,
+                                                       ws=self._workspace())
             return {t: out[t] for t in targets}
         # fallback wiring over dense activations
         acts = self.get_feature_activations(inputs)

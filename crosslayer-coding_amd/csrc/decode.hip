@@ -10,25 +10,31 @@
 
 namespace {
 
+// Row layout seen by one wavefront: NF full chunks of 64 lanes x 16 bytes, then an optional
+// tail chunk - TAIL 1: 64 lanes x 8 bytes (exactly fills the row), TAIL 2: a 16-byte chunk
+// in which only the leading lanes are inside the row.
 template <typename T> struct WVec;
 template <> struct WVec<float> {
-  static constexpr int V = 4;
-  __device__ static __forceinline__ void fma(float (&acc)[4], const float *p, float v) {
-    float4 w = *reinterpret_cast<const float4 *>(p);
-    acc[0] = fmaf(v, w.x, acc[0]); acc[1] = fmaf(v, w.y, acc[1]);
-    acc[2] = fmaf(v, w.z, acc[2]); acc[3] = fmaf(v, w.w, acc[3]);
+  static constexpr int V = 4;   // elements per 16 bytes
+  __device__ static __forceinline__ void fma16(float *acc, const uint4 &w, float v) {
+    acc[0] = fmaf(v, __uint_as_float(w.x), acc[0]); acc[1] = fmaf(v, __uint_as_float(w.y), acc[1]);
+    acc[2] = fmaf(v, __uint_as_float(w.z), acc[2]); acc[3] = fmaf(v, __uint_as_float(w.w), acc[3]);
+  }
+  __device__ static __forceinline__ void fma8(float *acc, const uint2 &w, float v) {
+    acc[0] = fmaf(v, __uint_as_float(w.x), acc[0]); acc[1] = fmaf(v, __uint_as_float(w.y), acc[1]);
   }
 };
 template <> struct WVec<bf16_t> {
   static constexpr int V = 8;
-  __device__ static __forceinline__ void fma(float (&acc)[8], const bf16_t *p, float v) {
-    uint4 w = *reinterpret_cast<const uint4 *>(p);
-    uint32_t u[4] = {w.x, w.y, w.z, w.w};
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      acc[2 * j] = fmaf(v, __uint_as_float(u[j] << 16), acc[2 * j]);
-      acc[2 * j + 1] = fmaf(v, __uint_as_float(u[j] & 0xFFFF0000u), acc[2 * j + 1]);
-    }
+  __device__ static __forceinline__ void fma32(float *acc, uint32_t u, float v) {
+    acc[0] = fmaf(v, __uint_as_float(u << 16), acc[0]);
+    acc[1] = fmaf(v, __uint_as_float(u & 0xFFFF0000u), acc[1]);
+  }
+  __device__ static __forceinline__ void fma16(float *acc, const uint4 &w, float v) {
+    fma32(acc, w.x, v); fma32(acc + 2, w.y, v); fma32(acc + 4, w.z, v); fma32(acc + 6, w.w, v);
+  }
+  __device__ static __forceinline__ void fma8(float *acc, const uint2 &w, float v) {
+    fma32(acc, w.x, v); fma32(acc + 2, w.y, v);
   }
 };
 
@@ -38,35 +44,76 @@ __device__ __forceinline__ int64_t decoder_slot(int tying, int64_t s, int64_t t,
   return s * L - (s * (s - 1)) / 2 + (t - s);
 }
 
-// One wavefront per (target, token).  CH = number of 64-lane x V-element chunks that cover d.
-template <typename T, int CH, bool AFFINE>
+// Fetch UU decoder vectors (all requests issued before the first multiply) and accumulate.
+template <typename T, int NF, int TAIL, int UU>
+__device__ __forceinline__ void decode_batch(float *acc, const T *wbase, int64_t d, int32_t my_col, float my_val,
+                                             int i0, int n, int lane, int64_t tail_off, bool tail_on) {
+  constexpr int V = WVec<T>::V;
+  uint4 wq[UU][NF > 0 ? NF : 1];
+  uint4 wt16[UU];
+  uint2 wt8[UU];
+  float v[UU];
+#pragma unroll
+  for (int u = 0; u < UU; ++u) {
+    const int idx = (i0 + u) < n ? (i0 + u) : (n - 1);   // clamp: a repeated fetch, weight 0
+    const int32_t f = __builtin_amdgcn_readlane(my_col, idx);
+    const float vv = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(my_val), idx));
+    v[u] = (i0 + u) < n ? vv : 0.0f;
+    const T *wrow = wbase + (int64_t)f * d;
+#pragma unroll
+    for (int c = 0; c < NF; ++c) wq[u][c] = *reinterpret_cast<const uint4 *>(wrow + (int64_t)c * 64 * V + (int64_t)lane * V);
+    if (TAIL == 1) wt8[u] = *reinterpret_cast<const uint2 *>(wrow + tail_off);
+    if (TAIL == 2) wt16[u] = tail_on ? *reinterpret_cast<const uint4 *>(wrow + tail_off) : make_uint4(0, 0, 0, 0);
+  }
+#pragma unroll
+  for (int u = 0; u < UU; ++u) {
+#pragma unroll
+    for (int c = 0; c < NF; ++c) WVec<T>::fma16(acc + c * V, wq[u][c], v[u]);
+    if (TAIL == 1) WVec<T>::fma8(acc + NF * V, wt8[u], v[u]);
+    if (TAIL == 2) WVec<T>::fma16(acc + NF * V, wt16[u], v[u]);
+  }
+}
+
+// One wavefront per (target, token) - or per (target, token, feature slice) when SLICED.
+// The survivors of a row are taken 64 at a time into registers (one per lane) and consumed
+// U at a time, so U row fetches are in flight per wavefront.
+//
+// SLICED: the feature axis is cut into `ns` slices and block b works on slice b % ns.
+// Workgroups are handed to the XCDs round-robin, so with ns = 8 each XCD sees one slice of
+// every decoder matrix (1/8 of its rows) for ALL tokens: the slice stays in that XCD's L2
+// while the tokens stream past.  Each wavefront writes an fp32 partial row; k_decode_reduce
+// adds the slices in a fixed order (deterministic) and applies bias / skip / rounding.
+template <typename T, int NF, int TAIL, int U, bool AFFINE, bool SLICED>
 __global__ __launch_bounds__(256) void k_decode(
     const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ col, const T *__restrict__ val,
     const T *__restrict__ wp, const float *__restrict__ bias_sum, const T *__restrict__ foff,
     const T *__restrict__ fscale, const float *__restrict__ skip_add, void *__restrict__ out,
     int64_t Tn, int64_t d, int64_t F, int64_t L, int tying, int64_t t_begin, int64_t t_end,
-    uint64_t src_mask, int out_f32) {
+    uint64_t src_mask, int out_f32, const int32_t *__restrict__ sptr, float *__restrict__ partial, int ns) {
   constexpr int V = WVec<T>::V;
+  constexpr int HV = V / 2;                       // elements per 8 bytes
+  constexpr int NACC = NF * V + (TAIL == 1 ? HV : TAIL == 2 ? V : 0);
   const int lane = lane_id(), wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
   const int64_t blocks_per_t = (Tn + nwv - 1) / nwv;
+  const int64_t bid = SLICED ? (int64_t)blockIdx.x / ns : (int64_t)blockIdx.x;
+  const int slice = SLICED ? (int)(blockIdx.x % ns) : 0;
   // heaviest targets (most sources) first
-  const int64_t t = t_end - 1 - (int64_t)blockIdx.x / blocks_per_t;
-  const int64_t tok = ((int64_t)blockIdx.x % blocks_per_t) * nwv + wv;
+  const int64_t t = t_end - 1 - bid / blocks_per_t;
+  const int64_t tok = (bid % blocks_per_t) * nwv + wv;
   if (tok >= Tn) return;
-  float acc[CH][V];
+  float acc[NACC];
 #pragma unroll
-  for (int c = 0; c < CH; ++c)
-#pragma unroll
-    for (int j = 0; j < V; ++j) acc[c][j] = 0.0f;
-  bool lane_on[CH];
-#pragma unroll
-  for (int c = 0; c < CH; ++c) lane_on[c] = (int64_t)(c * 64 + lane) * V < d;
+  for (int j = 0; j < NACC; ++j) acc[j] = 0.0f;
+  const int64_t tail_off = TAIL == 1 ? (int64_t)NF * 64 * V + (int64_t)lane * HV : (int64_t)NF * 64 * V + (int64_t)lane * V;
+  const bool tail_on = TAIL == 1 ? true : (TAIL == 2 ? tail_off < d : false);
 
   for (int64_t s = 0; s <= t; ++s) {
     if (!((src_mask >> s) & 1ull)) continue;
     const int64_t r = s * Tn + tok;
-    const int32_t b = row_ptr[r], e = row_ptr[r + 1];
-    const T *wbase = wp + decoder_slot(tying, s, t, L) * F * d + (int64_t)lane * V;
+    int32_t b, e;
+    if (SLICED) { b = sptr[r * (ns + 1) + slice]; e = sptr[r * (ns + 1) + slice + 1]; }
+    else { b = row_ptr[r]; e = row_ptr[r + 1]; }
+    const T *wbase = wp + decoder_slot(tying, s, t, L) * F * d;
     for (int32_t j0 = b; j0 < e; j0 += 64) {
       const int n = (e - j0) < 64 ? (e - j0) : 64;
       int32_t my_col = 0; float my_val = 0.0f;
@@ -78,36 +125,85 @@ __global__ __launch_bounds__(256) void k_decode(
           if (fscale) my_val = Elem<T>::round(my_val * Elem<T>::to_f32(fscale[t * F + my_col]));
         }
       }
-#pragma unroll 4
-      for (int i = 0; i < n; ++i) {
-        const int32_t f = __builtin_amdgcn_readlane(my_col, i);
-        const float v = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(my_val), i));
-        const T *wrow = wbase + (int64_t)f * d;
-#pragma unroll
-        for (int c = 0; c < CH; ++c)
-          if (lane_on[c]) WVec<T>::fma(acc[c], wrow + c * 64 * V, v);
-      }
+      int i0 = 0;
+      for (; i0 + U <= n; i0 += U) decode_batch<T, NF, TAIL, U>(acc, wbase, d, my_col, my_val, i0, n, lane, tail_off, tail_on);
+      for (; i0 < n; i0 += 2) decode_batch<T, NF, TAIL, 2>(acc, wbase, d, my_col, my_val, i0, n, lane, tail_off, tail_on);
     }
   }
+  if (SLICED) {
+    float *prow = partial + (((int64_t)slice * L + t) * Tn + tok) * d;
 #pragma unroll
-  for (int c = 0; c < CH; ++c) {
-    if (!lane_on[c]) continue;
-    const int64_t o = (int64_t)(c * 64 + lane) * V;
-    float y[V];
+    for (int c = 0; c < NF; ++c) {
+      float *pp = prow + (int64_t)c * 64 * V + (int64_t)lane * V;
 #pragma unroll
-    for (int j = 0; j < V; ++j) {
-      y[j] = acc[c][j];
-      if (bias_sum) y[j] += bias_sum[t * d + o + j];
-      if (skip_add) y[j] += skip_add[(t * Tn + tok) * d + o + j];
+      for (int j = 0; j < V; j += 4) *reinterpret_cast<float4 *>(pp + j) = make_float4(acc[c * V + j], acc[c * V + j + 1], acc[c * V + j + 2], acc[c * V + j + 3]);
     }
-    if (out_f32) {
-      float *po = (float *)out + (t * Tn + tok) * d + o;
+    if (TAIL == 1) {
 #pragma unroll
-      for (int j = 0; j < V; ++j) po[j] = y[j];
-    } else {
-      T *po = (T *)out + (t * Tn + tok) * d + o;
+      for (int j = 0; j < HV; ++j) prow[tail_off + j] = acc[NF * V + j];
+    }
+    if (TAIL == 2 && tail_on) {
 #pragma unroll
-      for (int j = 0; j < V; ++j) po[j] = Elem<T>::from_f32(y[j]);
+      for (int j = 0; j < V; ++j) prow[tail_off + j] = acc[NF * V + j];
+    }
+    return;
+  }
+  // epilogue: bias, skip term, one write of the output row
+  auto emit = [&](int64_t o, const float *a, int cnt, bool on) {
+    if (!on) return;
+    for (int j = 0; j < cnt; ++j) {
+      float y = a[j];
+      if (bias_sum) y += bias_sum[t * d + o + j];
+      if (skip_add) y += skip_add[(t * Tn + tok) * d + o + j];
+      if (out_f32) ((float *)out)[(t * Tn + tok) * d + o + j] = y;
+      else ((T *)out)[(t * Tn + tok) * d + o + j] = Elem<T>::from_f32(y);
+    }
+  };
+#pragma unroll
+  for (int c = 0; c < NF; ++c) emit((int64_t)c * 64 * V + (int64_t)lane * V, acc + c * V, V, true);
+  if (TAIL == 1) emit(tail_off, acc + NF * V, HV, true);
+  if (TAIL == 2) emit(tail_off, acc + NF * V, V, tail_on);
+}
+
+// sptr[r][j] = first survivor of row r whose feature index is >= j * F / ns  (j = 0..ns)
+__global__ void k_slice_ptr(const int32_t *row_ptr, const int32_t *col, int64_t R, int64_t F, int ns, int32_t *sptr) {
+  const int64_t total = R * (ns + 1);
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t r = i / (ns + 1);
+    const int j = (int)(i - r * (ns + 1));
+    const int32_t bound = (int32_t)(((int64_t)j * F) / ns);
+    int32_t lo = row_ptr[r], hi = row_ptr[r + 1];
+    while (lo < hi) {
+      int32_t mid = lo + ((hi - lo) >> 1);
+      if (col[mid] < bound) lo = mid + 1; else hi = mid;
+    }
+    sptr[i] = lo;
+  }
+}
+
+// out[t][tok][:] = sum over slices (fixed order) + bias + skip, rounded once.  4 elements per thread.
+template <typename T>
+__global__ void k_decode_reduce(const float *__restrict__ partial, const float *__restrict__ bias_sum,
+                                const float *__restrict__ skip_add, void *__restrict__ out, int64_t Tn, int64_t d,
+                                int64_t L, int64_t t_begin, int64_t t_end, int ns, int out_f32) {
+  const int64_t per_t = Tn * d, span = (t_end - t_begin) * per_t, slice_stride = L * per_t;
+  for (int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4; i < span; i += (int64_t)gridDim.x * blockDim.x * 4) {
+    const int64_t g = t_begin * per_t + i;          // index into [L][T][d]
+    float4 a = *reinterpret_cast<const float4 *>(partial + g);
+    for (int sl = 1; sl < ns; ++sl) {
+      float4 b = *reinterpret_cast<const float4 *>(partial + sl * slice_stride + g);
+      a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+    }
+    const int64_t t = g / per_t, o = g % d;
+    if (bias_sum) { a.x += bias_sum[t * d + o]; a.y += bias_sum[t * d + o + 1]; a.z += bias_sum[t * d + o + 2]; a.w += bias_sum[t * d + o + 3]; }
+    if (skip_add) { float4 k = *reinterpret_cast<const float4 *>(skip_add + g); a.x += k.x; a.y += k.y; a.z += k.z; a.w += k.w; }
+    if (out_f32) *reinterpret_cast<float4 *>((float *)out + g) = a;
+    else if (sizeof(T) == 4) *reinterpret_cast<float4 *>((float *)out + g) = a;
+    else {
+      uint2 o2;
+      o2.x = f32_to_bf16_bits(a.x) | (f32_to_bf16_bits(a.y) << 16);
+      o2.y = f32_to_bf16_bits(a.z) | (f32_to_bf16_bits(a.w) << 16);
+      *reinterpret_cast<uint2 *>((bf16_t *)out + g) = o2;
     }
   }
 }
@@ -217,52 +313,93 @@ __global__ __launch_bounds__(256) void k_norms(const T *wp, T *norms, int64_t d,
   }
 }
 
+constexpr int DEC_SLICES = 8;  // one feature slice per XCD of an MI355X
+
+static size_t decode_ws_bytes(int64_t Tn, int64_t d, int64_t L) {
+  size_t part = ((size_t)DEC_SLICES * L * Tn * d * 4 + 255) & ~(size_t)255;
+  size_t sp = ((size_t)L * Tn * (DEC_SLICES + 1) * 4 + 255) & ~(size_t)255;
+  return part + sp;
+}
+
 template <typename T>
 static int launch_decode(const int32_t *row_ptr, const int32_t *col, const void *val, const void *wp,
                          const float *bias_sum, const void *foff, const void *fscale, const float *skip_add,
                          void *out, int64_t Tn, int64_t d, int64_t F, int64_t L, int tying, int64_t t_begin,
-                         int64_t t_end, uint64_t src_mask, int out_f32, hipStream_t stream) {
+                         int64_t t_end, uint64_t src_mask, int out_f32, void *workspace, size_t workspace_bytes,
+                         hipStream_t stream) {
   constexpr int V = WVec<T>::V;
   const int nwv = 4;
   const int64_t blocks_per_t = clt_ceil_div(Tn, nwv);
-  const int64_t nblk = blocks_per_t * (t_end - t_begin);
+  const bool can_slice = workspace && workspace_bytes >= decode_ws_bytes(Tn, d, L) && (d % 4 == 0) &&
+                         F >= 64 * DEC_SLICES && ((((uintptr_t)workspace) & 255u) == 0);
+  const int ns = can_slice ? DEC_SLICES : 1;
+  int32_t *sptr = nullptr; float *partial = nullptr;
+  if (can_slice) {
+    partial = (float *)workspace;
+    sptr = (int32_t *)((char *)workspace + (((size_t)DEC_SLICES * L * Tn * d * 4 + 255) & ~(size_t)255));
+  }
+  const int64_t nblk = blocks_per_t * (t_end - t_begin) * ns;
   if (nblk <= 0) return CLT_OK;
   if (nblk > 2147483647LL) return CLT_ERR_RANGE;
   const bool affine = foff || fscale;
-  const bool fast = (d % V == 0) && clt_aligned16(wp) && d <= 64 * V * 8;
-#define CLT_DEC(CHN)                                                                                          \
-  do {                                                                                                        \
-    if (affine)                                                                                               \
-      k_decode<T, CHN, true><<<(unsigned)nblk, 256, 0, stream>>>(row_ptr, col, (const T *)val, (const T *)wp, \
-          bias_sum, (const T *)foff, (const T *)fscale, skip_add, out, Tn, d, F, L, tying, t_begin, t_end,     \
-          src_mask, out_f32);                                                                                 \
-    else                                                                                                      \
-      k_decode<T, CHN, false><<<(unsigned)nblk, 256, 0, stream>>>(row_ptr, col, (const T *)val, (const T *)wp,\
-          bias_sum, nullptr, nullptr, skip_add, out, Tn, d, F, L, tying, t_begin, t_end, src_mask, out_f32);  \
+  const int64_t chunk = 64 * V;
+  const int64_t nf = d / chunk, rem = d % chunk;
+  const bool fast = (d % V == 0) && clt_aligned16(wp) && nf <= 4 && (nf > 0 || rem > 0);
+  if (can_slice && !fast) return launch_decode<T>(row_ptr, col, val, wp, bias_sum, foff, fscale, skip_add, out, Tn, d, F,
+                                                  L, tying, t_begin, t_end, src_mask, out_f32, nullptr, 0, stream);
+  if (can_slice) k_slice_ptr<<<1024, 256, 0, stream>>>(row_ptr, col, L * Tn, F, ns, sptr);
+#define CLT_DEC_ARGS(FO, FS)                                                                                    \
+  row_ptr, col, (const T *)val, (const T *)wp, bias_sum, FO, FS, skip_add, out, Tn, d, F, L, tying, t_begin,    \
+      t_end, src_mask, out_f32, sptr, partial, ns
+#define CLT_DEC(NFN, TL, UN)                                                                                    \
+  do {                                                                                                          \
+    if (affine && can_slice)                                                                                    \
+      k_decode<T, NFN, TL, UN, true, true><<<(unsigned)nblk, 256, 0, stream>>>(CLT_DEC_ARGS((const T *)foff, (const T *)fscale)); \
+    else if (affine)                                                                                            \
+      k_decode<T, NFN, TL, UN, true, false><<<(unsigned)nblk, 256, 0, stream>>>(CLT_DEC_ARGS((const T *)foff, (const T *)fscale)); \
+    else if (can_slice)                                                                                         \
+      k_decode<T, NFN, TL, UN, false, true><<<(unsigned)nblk, 256, 0, stream>>>(CLT_DEC_ARGS(nullptr, nullptr)); \
+    else                                                                                                        \
+      k_decode<T, NFN, TL, UN, false, false><<<(unsigned)nblk, 256, 0, stream>>>(CLT_DEC_ARGS(nullptr, nullptr)); \
+  } while (0)
+#define CLT_DEC_TAIL(NFN, UN)                              \
+  do {                                                     \
+    if (rem == 0) CLT_DEC(NFN, 0, UN);                     \
+    else if (rem * 2 == chunk) CLT_DEC(NFN, 1, UN);        \
+    else CLT_DEC(NFN, 2, UN);                              \
   } while (0)
   if (fast) {
-    const int64_t ch = clt_ceil_div(d, 64 * V);
-    if (ch <= 1) CLT_DEC(1);
-    else if (ch == 2) CLT_DEC(2);
-    else if (ch == 3) CLT_DEC(3);
-    else if (ch == 4) CLT_DEC(4);
-    else if (ch <= 6) CLT_DEC(6);
-    else CLT_DEC(8);
+    if (nf == 0) CLT_DEC(0, 2, 8);
+    else if (nf == 1) CLT_DEC_TAIL(1, 8);
+    else if (nf == 2) CLT_DEC_TAIL(2, 6);
+    else if (nf == 3) CLT_DEC_TAIL(3, 4);
+    else if (rem == 0) CLT_DEC(4, 0, 4);
+    else CLT_DEC(4, 2, 3);
   } else {
     k_decode_generic<T><<<(unsigned)nblk, 256, 0, stream>>>(row_ptr, col, (const T *)val, (const T *)wp, bias_sum,
         (const T *)foff, (const T *)fscale, skip_add, out, Tn, d, F, L, tying, t_begin, t_end, src_mask, out_f32);
   }
+#undef CLT_DEC_TAIL
 #undef CLT_DEC
+#undef CLT_DEC_ARGS
+  if (can_slice)
+    k_decode_reduce<T><<<2048, 256, 0, stream>>>(partial, bias_sum, skip_add, out, Tn, d, L, t_begin, t_end, ns, out_f32);
   return clt_check_launch();
 }
 
 }  // namespace
 
+extern "C" size_t clt_decode_workspace_bytes(int64_t T, int64_t d, int64_t F, int64_t L) {
+  (void)F;
+  if (T <= 0 || d <= 0 || L <= 0) return 256;
+  return decode_ws_bytes(T, d, L);
+}
+
 extern "C" int clt_decode_sparse(const int32_t *row_ptr, const int32_t *col, const void *val, const void *w_packed,
                                  const float *bias_sum, const void *feat_offset, const void *feat_scale,
                                  const float *skip_add, void *out, int64_t T, int64_t d, int64_t F, int64_t L,
                                  int tying, int64_t t_begin, int64_t t_end, uint64_t src_mask, int dtype,
-                                 int out_f32, void *stream) {
+                                 int out_f32, void *workspace, size_t workspace_bytes, void *stream) {
   if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
   if (T < 0 || d <= 0 || F <= 0 || L <= 0 || L > 64) return CLT_ERR_ARG;
   if (t_begin < 0 || t_end > L || t_begin > t_end) return CLT_ERR_ARG;
@@ -271,8 +408,8 @@ extern "C" int clt_decode_sparse(const int32_t *row_ptr, const int32_t *col, con
   if (!row_ptr || !w_packed || !out) return CLT_ERR_ARG;
   hipStream_t s = (hipStream_t)stream;
   if (dtype == CLT_BF16)
-    return launch_decode<bf16_t>(row_ptr, col, val, w_packed, bias_sum, feat_offset, feat_scale, skip_add, out, T, d, F, L, tying, t_begin, t_end, src_mask, out_f32, s);
-  return launch_decode<float>(row_ptr, col, val, w_packed, bias_sum, feat_offset, feat_scale, skip_add, out, T, d, F, L, tying, t_begin, t_end, src_mask, out_f32, s);
+    return launch_decode<bf16_t>(row_ptr, col, val, w_packed, bias_sum, feat_offset, feat_scale, skip_add, out, T, d, F, L, tying, t_begin, t_end, src_mask, out_f32, workspace, workspace_bytes, s);
+  return launch_decode<float>(row_ptr, col, val, w_packed, bias_sum, feat_offset, feat_scale, skip_add, out, T, d, F, L, tying, t_begin, t_end, src_mask, out_f32, workspace, workspace_bytes, s);
 }
 
 extern "C" int clt_pack_decoder(const void *w_ref, void *w_packed, int64_t d, int64_t F, int64_t n_dec,

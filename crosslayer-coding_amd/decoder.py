@@ -183,12 +183,12 @@ class Decoder(nn.Module):
 
     # ---- fused path ------------------------------------------------------------------
     def decode_survivors(self, surv: SurvivorList, src_mask: int, t_begin: int = 0, t_end: Optional[int] = None,
-                         skip_add: Optional[torch.Tensor] = None) -> torch.Tensor:
+                         skip_add: Optional[torch.Tensor] = None, ws=None) -> torch.Tensor:
         """Reconstructions [L, T, d] (rows outside [t_begin, t_end) are not written)."""
         off, sc = self._affine()
         return engine.decode_sparse(surv, self.packed(), self.config.decoder_tying, self.config.d_model,
                                     bias_sum=self.bias_sum(src_mask), feat_offset=off, feat_scale=sc,
-                                    skip_add=skip_add, t_begin=t_begin, t_end=t_end, src_mask=src_mask)
+                                    skip_add=skip_add, t_begin=t_begin, t_end=t_end, src_mask=src_mask, ws=ws)
 
     def skip_all_targets(self, inputs: Dict[int, torch.Tensor], src_mask: int, T: int) -> Optional[torch.Tensor]:
         """[L, T, d] fp32 skip-connection terms for every target present in ``inputs``."""

@@ -65,6 +65,10 @@ class Workspace:
         self._bufs.clear()
 
 
+# below this many (token, target) rows one wavefront per row already underfills the GPU
+SLICED_DECODE_MIN_ROWS = 8192
+
+
 def _stream(t: torch.Tensor) -> int:
     return nat.current_stream(t.device)
 
@@ -201,8 +205,11 @@ def decode_sparse(surv: SurvivorList, w_packed: torch.Tensor, tying: str, d: int
                   bias_sum: Optional[torch.Tensor] = None, feat_offset: Optional[torch.Tensor] = None,
                   feat_scale: Optional[torch.Tensor] = None, skip_add: Optional[torch.Tensor] = None,
                   t_begin: int = 0, t_end: Optional[int] = None, src_mask: Optional[int] = None,
-                  out: Optional[torch.Tensor] = None, out_f32: bool = False) -> torch.Tensor:
-    """Reconstructions [L, T, d] for targets [t_begin, t_end) (decoder.py:176-340)."""
+                  out: Optional[torch.Tensor] = None, out_f32: bool = False,
+                  ws: Optional[Workspace] = None) -> torch.Tensor:
+    """Reconstructions [L, T, d] for targets [t_begin, t_end) (decoder.py:176-340).
+
+    With a workspace and a batch large enough to fill the GPU the XCD-sliced kernel is used."""
     nat.require_device(w_packed, "decode_sparse")
     L, T, F = surv.L, surv.T, surv.F
     t_end = L if t_end is None else t_end
@@ -218,11 +225,16 @@ def decode_sparse(surv: SurvivorList, w_packed: torch.Tensor, tying: str, d: int
         assert a is None or (a.dtype == torch.float32 and a.is_contiguous())
     for a in (feat_offset, feat_scale):
         assert a is None or (a.dtype == surv.dtype and a.is_contiguous() and a.shape == (L, F))
-    code = nat.load().clt_decode_sparse(
+    lib = nat.load()
+    wbuf, wbytes = None, 0
+    if ws is not None and T * (t_end - t_begin) >= SLICED_DECODE_MIN_ROWS:
+        wbytes = lib.clt_decode_workspace_bytes(T, d, F, L)
+        wbuf = ws.get("decode", wbytes)
+    code = lib.clt_decode_sparse(
         nat.ptr(surv.row_ptr), nat.ptr(surv.col), nat.ptr(surv.val), nat.ptr(w_packed), nat.ptr(bias_sum),
         nat.ptr(feat_offset), nat.ptr(feat_scale), nat.ptr(skip_add), nat.ptr(out), T, d, F, L,
         nat.TYING[tying], t_begin, t_end, src_mask & ((1 << 64) - 1), nat.dtype_code(surv.dtype),
-        1 if out_f32 else 0, _stream(w_packed))
+        1 if out_f32 else 0, nat.ptr(wbuf), wbytes, _stream(w_packed))
     nat.check(code, "clt_decode_sparse")
     return out
 

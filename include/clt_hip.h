@@ -175,14 +175,21 @@ int clt_pack_decoder(const void *w_ref, void *w_packed, int64_t d, int64_t F,
  * for all targets that CrossLayerTranscoder.forward loops over
  * (clt/models/clt.py:192-199).
  * Limits: L <= 64; d % 8 == 0 (bf16) / d % 4 == 0 (fp32) on the fast path.
+ * workspace: NULL runs one wavefront per (target, token) over all features.  With a
+ * workspace of clt_decode_workspace_bytes() the feature axis is cut into 8 slices, one per
+ * XCD, so that each slice of a decoder matrix stays in one L2 while all tokens pass; the
+ * per-slice fp32 partial rows are then summed in a fixed order.  Both give the same result
+ * up to fp32 summation order.
  */
+size_t clt_decode_workspace_bytes(int64_t T, int64_t d, int64_t F, int64_t L);
 int clt_decode_sparse(const int32_t *row_ptr, const int32_t *col, const void *val,
                       const void *w_packed, const float *bias_sum,
                       const void *feat_offset, const void *feat_scale,
                       const float *skip_add, void *out,
                       int64_t T, int64_t d, int64_t F, int64_t L,
                       int tying, int64_t t_begin, int64_t t_end, uint64_t src_mask,
-                      int dtype, int out_f32, void *stream);
+                      int dtype, int out_f32, void *workspace, size_t workspace_bytes,
+                      void *stream);
 
 /*
  * Dense materialisation of a survivor list: out[l][t][f] = value or 0.

@@ -40,7 +40,8 @@ def test_workspace_queries_and_argument_errors_need_no_gpu():
     assert lib.clt_encode(None, None, None, None, 4, 8, 16, 1, 0, 0, 0, 0, 7, None) == -2
     assert lib.clt_encode(None, None, None, None, 4, 8, 16, 1, 0, 0, 0, 0, 0, None) == -1
     assert lib.clt_decode_sparse(None, None, None, None, None, None, None, None, None,
-                                 4, 8, 16, 65, 0, 0, 1, 1, 0, 0, None) == -1
+                                 4, 8, 16, 65, 0, 0, 1, 1, 0, 0, None, 0, None) == -1
+    assert lib.clt_decode_workspace_bytes(4096, 768, 24576, 12) >= 8 * 12 * 4096 * 768 * 4
     assert lib.clt_pack_decoder(None, None, 8, 16, 1, 0, 0, 0, None) == -1
 
 

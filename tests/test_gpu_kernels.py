@@ -272,6 +272,41 @@ def test_decode_sparse_parity(dev, dtype, tying, L, T, d, F):
         assert sub.dtype == torch.float32 and orc.rel_l2(sub[t], ref) <= TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("tying", ["none", "per_target"])
+def test_decode_sliced_matches_single_pass(dev, dtype, tying):
+    # the XCD-sliced kernel (workspace given) against the one-wavefront-per-row kernel and the oracle
+    g = torch.Generator().manual_seed(21)
+    L, T, d, F = 3, 160, 768, 1024
+    names, w, b = make_decoder(L, d, F, tying, dtype, g)
+    acts = (torch.randn(L, T, F, generator=g) * (torch.rand(L, T, F, generator=g) < 0.05)).to(dtype)
+    acts[0, 5] = 0                                     # an empty row
+    acts[1, 7, :] = torch.randn(F, generator=g).to(dtype)   # a full row (more than 64 per slice)
+    surv = engine.threshold_select(acts.to(dev), None, nat.PRED_NONZERO)
+    slab = torch.empty(len(names), F, d, dtype=dtype, device=dev)
+    for i, n in enumerate(names):
+        engine.pack_decoder(w[n].to(dev), slab[i])
+    bias = torch.randn(L, d, generator=g)
+    skip = torch.randn(L, T, d, generator=g)
+    ws = engine.Workspace(dev)
+    old = engine.SLICED_DECODE_MIN_ROWS
+    try:
+        engine.SLICED_DECODE_MIN_ROWS = 1
+        sliced = engine.decode_sparse(surv, slab, tying, d, bias_sum=bias.to(dev), skip_add=skip.to(dev), ws=ws)
+        sliced32 = engine.decode_sparse(surv, slab, tying, d, out_f32=True, t_begin=1, t_end=3, src_mask=0b110, ws=ws)
+    finally:
+        engine.SLICED_DECODE_MIN_ROWS = old
+    single = engine.decode_sparse(surv, slab, tying, d, bias_sum=bias.to(dev), skip_add=skip.to(dev))
+    single32 = engine.decode_sparse(surv, slab, tying, d, out_f32=True, t_begin=1, t_end=3, src_mask=0b110)
+    assert orc.rel_l2(sliced, single) <= (1e-6 if dtype == torch.float32 else 4e-3)
+    assert orc.rel_l2(sliced32[1:], single32[1:]) <= 1e-6
+    zero_b = {n: torch.zeros(d, dtype=dtype) for n in names}
+    for t in range(L):
+        ref = orc.decode({s: acts[s] for s in range(L)}, t, tying=tying, weights=w, biases=zero_b, d_model=d,
+                         num_features=F, dtype=dtype).float() + bias[t] + skip[t]
+        assert orc.rel_l2(sliced[t], ref) <= TOL[dtype]
+
+
 def test_decode_linearity_property(dev):
     # decode(2 * a) - bias == 2 * (decode(a) - bias), exact in fp32 for power-of-two scaling
     g = torch.Generator().manual_seed(2)
