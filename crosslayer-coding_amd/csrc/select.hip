@@ -6,22 +6,23 @@
 //
 //   sample   a hashed sample of the ranking values gives a conservative cut key
 //            (about 2x K elements lie above it);
-//   pass     ONE read of every row (one wavefront per row, 16-byte loads): elements
-//            at or above the cut are appended, in column order (wave ballot +
-//            mbcnt prefix), to a per-row candidate segment and counted into an LDS
-//            histogram of (key - cut);
+//   pass     ONE read of every row (one wavefront per row, four 16-byte loads in flight
+//            per lane): elements at or above the cut are collected, in column order (wave
+//            ballot + mbcnt prefix), in an LDS buffer of the wavefront, counted into an
+//            LDS histogram of (key - cut), and flushed in coalesced extents to a
+//            candidate pool (one atomic per extent; a row's extents are chained);
 //   scan     a single block walks the histogram from the top and finds the bin that
 //            holds the K-th largest key; bins are one key wide near the cut (16-bit
 //            keys) so this usually ends the search, otherwise further levels
 //            re-histogram the candidates only;
-//   count / allot / emit   work on the candidate segments: survivors per row, the
-//            tie budget handed out in flat-index order, then the ordered write of
+//   count / allot / emit   work on the candidate pool: survivors per row, the tie
+//            budget handed out in flat-index order, then the ordered write of
 //            (feature, value) pairs.
 //
-// A row whose candidates overflow its segment is re-read from the dense matrix by
-// the later stages, and a cut that turns out too high (fewer than K candidates)
-// makes the pass run again with the lowest cut, so the result is exact for any
-// input; only the speed depends on the sample being representative.
+// A row that could not get pool space is re-read from the dense matrix by the later
+// stages, and a cut that turns out too high (fewer than K candidates) makes the pass run
+// again with the lowest cut, so the result is exact for any input; only the speed depends
+// on the sample being representative.
 #include "clt_common.h"
 
 namespace {
@@ -29,7 +30,12 @@ namespace {
 constexpr int NBINS = 2048;
 constexpr uint32_t FINE16 = 1984;  // 16-bit keys: bins [0,FINE16) are one key wide
 constexpr int SAMPLE_N = 16384;
+constexpr int SAMPLE_BLOCKS = 16;        // blocks per problem that gather the sample
 constexpr int SCAN_THREADS = 1024;
+constexpr int WBUF = 512;                // candidate entries buffered in LDS per wavefront
+constexpr int PASS_NV = 4;               // 16-byte loads in flight per lane in the pass
+constexpr uint32_t ROW_NONE = 0xFFFFFFFFu;   // row has no candidates
+constexpr uint32_t ROW_DENSE = 0xFFFFFFFEu;  // row did not fit the pool: read it from the matrix
 
 enum : uint32_t { ST_RUN = 0, ST_RETRY = 1, ST_DONE = 2 };
 
@@ -173,34 +179,47 @@ __device__ __forceinline__ uint64_t hash_index(uint64_t i, uint64_t n) {
   return __umul64hi(x, n);
 }
 
-// One block per problem: conservative cut key from a hashed sample.
+// SAMPLE_BLOCKS blocks per problem: ranking keys of a hashed sample.
 template <typename T, bool GLOBAL>
-__global__ __launch_bounds__(SCAN_THREADS) void k_sample_cut(
+__global__ __launch_bounds__(256) void k_sample_keys(
     const T *pre, int64_t Tn, int64_t F, int64_t L, int64_t lstride, const float *mean,
-    const float *denom, unsigned long long N, unsigned long long K, SelState *st) {
+    const float *denom, unsigned long long N, uint32_t *sample) {
   constexpr int KB = Elem<T>::KEYBITS;
+  const int p = blockIdx.y;
+  const unsigned long long ns = N < (unsigned long long)SAMPLE_N ? N : (unsigned long long)SAMPLE_N;
+  for (unsigned long long si = (unsigned long long)blockIdx.x * blockDim.x + threadIdx.x; si < ns;
+       si += (unsigned long long)gridDim.x * blockDim.x) {
+    unsigned long long idx = (ns == N) ? si : hash_index(si, N);
+    int64_t l, t, f;
+    if (GLOBAL) { int64_t rowlen = L * F; t = idx / rowlen; int64_t rem = idx - t * rowlen; l = rem / F; f = rem - l * F; }
+    else { l = p; t = idx / F; f = idx - t * F; }
+    float x = Elem<T>::to_f32(pre[l * lstride + t * F + f]);
+    typename RankOf<T, GLOBAL>::type rk = RankOf<T, GLOBAL>::make(mean, denom, l, F);
+    sample[(int64_t)p * SAMPLE_N + si] = rank_key<KB>(rk(x, f));
+  }
+}
+
+// One block per problem: the cut key = the r-th largest sample key, r chosen so that the
+// expected number of elements above the cut is about 1.25 K plus six standard deviations.
+// Also resets the problem's histogram, pool counter and state.
+template <int KB>
+__global__ __launch_bounds__(SCAN_THREADS) void k_sample_cut(
+    const uint32_t *sample, unsigned long long N, unsigned long long K, SelState *st, uint32_t *hist,
+    uint32_t *pool_count) {
   constexpr int PER = SAMPLE_N / SCAN_THREADS;
   __shared__ uint32_t lh[NBINS];
   const int p = blockIdx.x, tid = threadIdx.x;
   const unsigned long long ns = N < (unsigned long long)SAMPLE_N ? N : (unsigned long long)SAMPLE_N;
+  for (int i = tid; i < NBINS; i += SCAN_THREADS) hist[(int64_t)p * NBINS + i] = 0;
+  if (tid == 0) pool_count[p] = 0;
   uint32_t keys[PER];
   bool valid[PER];
 #pragma unroll
   for (int i = 0; i < PER; ++i) {
     unsigned long long si = (unsigned long long)tid + (unsigned long long)i * SCAN_THREADS;
     valid[i] = si < ns;
-    keys[i] = 0;
-    if (valid[i]) {
-      unsigned long long idx = (ns == N) ? si : hash_index(si, N);
-      int64_t l, t, f;
-      if (GLOBAL) { int64_t rowlen = L * F; t = idx / rowlen; int64_t rem = idx - t * rowlen; l = rem / F; f = rem - l * F; }
-      else { l = p; t = idx / F; f = idx - t * F; }
-      float x = Elem<T>::to_f32(pre[l * lstride + t * F + f]);
-      typename RankOf<T, GLOBAL>::type rk = RankOf<T, GLOBAL>::make(mean, denom, l, F);
-      keys[i] = rank_key<KB>(rk(x, f));
-    }
+    keys[i] = valid[i] ? sample[(int64_t)p * SAMPLE_N + si] : 0u;
   }
-  // rank (1-based from the top) of the sample element used as the cut
   unsigned long long r;
   if (ns == N) r = K;
   else {
@@ -241,55 +260,169 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_sample_cut(
   }
 }
 
-// The streaming pass: one wavefront per row.
+// Inclusive prefix sum over the 64 lanes of a wavefront with DPP row shifts / broadcasts.
+__device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v) {
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x111, 0xf, 0xf, false);  // row_shr:1
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x112, 0xf, 0xf, false);  // row_shr:2
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x114, 0xf, 0xf, false);  // row_shr:4
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x118, 0xf, 0xf, false);  // row_shr:8
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x142, 0xa, 0xf, false);  // row_bcast:15
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x143, 0xc, 0xf, false);  // row_bcast:31
+  return v;
+}
+
+// 16 bytes of a row as loaded, and the float value of element j of it.
+template <typename T> __device__ __forceinline__ float vec_elem(const uint4 &w, int j);
+template <> __device__ __forceinline__ float vec_elem<float>(const uint4 &w, int j) {
+  return __uint_as_float(j == 0 ? w.x : j == 1 ? w.y : j == 2 ? w.z : w.w);
+}
+template <> __device__ __forceinline__ float vec_elem<bf16_t>(const uint4 &w, int j) {
+  const uint32_t u = (j >> 1) == 0 ? w.x : (j >> 1) == 1 ? w.y : (j >> 1) == 2 ? w.z : w.w;
+  return __uint_as_float((j & 1) ? (u & 0xFFFF0000u) : (u << 16));
+}
+
+// The streaming pass: one wavefront per row.  A step covers PASS_NV vectors of 64 lanes x 16
+// bytes.  Lanes keep a bit per element that reaches the cut; when any lane has one, the raw
+// vectors are staged in LDS (column order), two packed prefix scans give every candidate its
+// place in column order, each lane writes the columns of its set bits, and then the lanes
+// finish the candidates in parallel (value, histogram).
 template <typename T, int V, bool GLOBAL>
 __global__ __launch_bounds__(256) void k_select_pass(
     const T *pre, int64_t Tn, int64_t F, int64_t L, int64_t lstride, const float *mean,
-    const float *denom, const SelState *st, uint32_t *hist, uint32_t *seg_count, uint2 *seg,
-    int cap, int phase) {
+    const float *denom, const SelState *st, uint32_t *hist, uint32_t *pool_count, uint2 *pool,
+    unsigned long long pool_cap, uint32_t *row_first, int phase) {
   constexpr int KB = Elem<T>::KEYBITS;
+  static_assert(PASS_NV == 4, "the packed prefix below holds four 16-bit fields");
+  constexpr int STEP = PASS_NV * 64 * V;  // elements per step
   __shared__ uint32_t lh[NBINS];
+  __shared__ uint2 wbuf_all[4][WBUF];
+  __shared__ __attribute__((aligned(16))) T stage_all[4][STEP];
   const int l = blockIdx.y, p = GLOBAL ? 0 : l;
   const uint32_t status = st[p].status;
   if (phase == 0 ? status != ST_RUN : status != ST_RETRY) return;
   const uint32_t cut_key = st[p].cut_key;
-  const float cutf = __uint_as_float(key_to_f32_bits<KB>(cut_key));
+  const uint32_t cut_bits = key_to_f32_bits<KB>(cut_key);
+  const float cutf = __uint_as_float(cut_bits);
+  const bool cut_nan = (cut_bits & 0x7FFFFFFFu) > 0x7F800000u;  // only NaNs reach such a cut
   for (int i = threadIdx.x; i < NBINS; i += blockDim.x) lh[i] = 0;
   __syncthreads();
   const int lane = lane_id(), wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
+  uint2 *wbuf = wbuf_all[wv];
+  T *stage = stage_all[wv];
+  uint2 *mypool = pool + (unsigned long long)p * pool_cap;
   typename RankOf<T, GLOBAL>::type rk = RankOf<T, GLOBAL>::make(mean, denom, l, F);
   for (int64_t t = (int64_t)blockIdx.x * nwv + wv; t < Tn; t += (int64_t)gridDim.x * nwv) {
     const int64_t r = (int64_t)l * Tn + t;
     const T *row = pre + l * lstride + t * F;
-    uint2 *sg = seg + r * cap;
-    uint32_t n = 0;
-    for (int64_t c0 = 0; c0 < F; c0 += 64 * V) {
-      const int64_t col = c0 + (int64_t)lane * V;
-      float x[V], rv[V]; uint32_t raw[V];
-      uint32_t m = 0;
-      if (col < F) {
-        VecLoad<T, V>::load(row + col, x, raw);
+    uint32_t n_buf = 0, first = ROW_NONE, prev = ROW_NONE;
+    bool dense = false;
+    auto flush = [&]() {
+      if (n_buf == 0) return;
+      if (!dense) {
+        uint32_t off = 0;
+        if (lane == 0) off = atomicAdd(&pool_count[p], n_buf + 1u);
+        off = __builtin_amdgcn_readfirstlane(off);
+        if ((unsigned long long)off + n_buf + 1ull > pool_cap) dense = true;
+        else {
+          if (lane == 0) {
+            mypool[off] = make_uint2(ROW_NONE, n_buf);           // extent header: (next, count)
+            if (prev != ROW_NONE) mypool[prev].x = off;
+          }
+          if (prev == ROW_NONE) first = off;
+          prev = off;
+          for (uint32_t i = lane; i < n_buf; i += 64) mypool[off + 1u + i] = wbuf[i];
+        }
+      }
+      n_buf = 0;
+    };
+    for (int64_t c0 = 0; c0 < F; c0 += STEP) {
+      uint4 w[PASS_NV];
+      bool on[PASS_NV];
 #pragma unroll
-        for (int j = 0; j < V; ++j) { rv[j] = rk(x[j], col + j); if (!(rv[j] < cutf)) m |= 1u << j; }
+      for (int q = 0; q < PASS_NV; ++q) {
+        const int64_t col = c0 + (int64_t)q * 64 * V + (int64_t)lane * V;
+        on[q] = col < F;
+        w[q] = make_uint4(0, 0, 0, 0);
+        if (on[q]) {
+          if (V > 1) w[q] = *reinterpret_cast<const uint4 *>(row + col);
+          else w[q].x = sizeof(T) == 2 ? ((uint32_t)Elem<T>::raw(row[col]) << 16) : (uint32_t)Elem<T>::raw(row[col]);
+        }
+      }
+      uint32_t m = 0;  // bit q*V + j: element j of vector q reaches the cut
+#pragma unroll
+      for (int q = 0; q < PASS_NV; ++q) {
+        const int64_t col = c0 + (int64_t)q * 64 * V + (int64_t)lane * V;
+        if (on[q]) {
+#pragma unroll
+          for (int j = 0; j < V; ++j) {
+            const float xv = V > 1 ? vec_elem<T>(w[q], j) : __uint_as_float(w[q].x);
+            const float rv = rk(xv, col + j);
+            const bool c = cut_nan ? (rv != rv) : !(rv < cutf);
+            m |= (c ? 1u : 0u) << (q * V + j);
+          }
+        }
       }
       if (ballot64(m != 0) == 0) continue;
+      // stage the step in column order: stage[col - c0]
 #pragma unroll
-      for (int j = 0; j < V; ++j)
-        if ((m >> j) & 1u) {
-          uint32_t key = rank_key<KB>(rv[j]);
-          if (key < cut_key) m &= ~(1u << j);
-          else atomicAdd(&lh[bin_level0<KB>(key - cut_key)], 1u);
+      for (int q = 0; q < PASS_NV; ++q) {
+        if (V > 1) *reinterpret_cast<uint4 *>(stage + (q * 64 + lane) * V) = w[q];
+        else stage[q * 64 + lane] = Elem<T>::from_raw(sizeof(T) == 2 ? (w[q].x >> 16) : w[q].x);
+      }
+      // per-vector counts, packed 16 bits each, prefix-summed over the lanes
+      constexpr uint32_t FM = (1u << V) - 1u;
+      const uint32_t cA = __popc(m & FM) | (__popc((m >> V) & FM) << 16);
+      const uint32_t cB = __popc((m >> (2 * V)) & FM) | (__popc((m >> (3 * V)) & FM) << 16);
+      const uint32_t iA = wave_inclusive_scan(cA), iB = wave_inclusive_scan(cB);
+      const uint32_t tA = __builtin_amdgcn_readlane(iA, 63), tB = __builtin_amdgcn_readlane(iB, 63);
+      const uint32_t t0 = tA & 0xFFFFu, t1 = tA >> 16, t2 = tB & 0xFFFFu, t3 = tB >> 16;
+      const uint32_t total = t0 + t1 + t2 + t3;
+      if (n_buf + total > (uint32_t)WBUF) flush();
+      const bool fits = total <= (uint32_t)WBUF;
+      if (!fits) dense = true;   // a step denser than the buffer: leave this row to the dense readers
+      // start of each vector's candidates in the buffer, plus this lane's exclusive prefix
+      const uint32_t sA = (iA - cA) + (n_buf | ((n_buf + t0) << 16));
+      const uint32_t sB = (iB - cB) + ((n_buf + t0 + t1) | ((n_buf + t0 + t1 + t2) << 16));
+      const uint32_t c0u = (uint32_t)c0;
+      if (fits) {
+        // each lane drops the step-relative column of its candidates at their ordered slots
+        uint32_t mm = m;
+        while (ballot64(mm != 0)) {
+          if (mm) {
+            const int bit = __ffs(mm) - 1;
+            mm &= mm - 1u;
+            const int q = bit / V;
+            const uint32_t sw = q < 2 ? sA : sB;
+            const uint32_t start = (q & 1) ? (sw >> 16) : (sw & 0xFFFFu);
+            const uint32_t below = __popc(m & ((1u << bit) - 1u) & (FM << (q * V)));
+            wbuf[start + below].x = (uint32_t)(q * 64 * V + lane * V + (bit % V));
+          }
         }
-      uint32_t total, pre_cnt = wave_mask_prefix<V>(m, total);
-#pragma unroll
-      for (int j = 0; j < V; ++j)
-        if ((m >> j) & 1u) {
-          uint32_t pos = n + pre_cnt + __popc(m & ((1u << j) - 1u));
-          if (pos < (uint32_t)cap) sg[pos] = make_uint2((uint32_t)(col + j), raw[j]);
+        // the lanes finish the new entries in parallel
+        for (uint32_t i = lane; i < total; i += 64) {
+          const uint32_t rel = wbuf[n_buf + i].x;
+          const T rawv = stage[rel];
+          const uint32_t col = c0u + rel;
+          const uint32_t key = rank_key<KB>(rk(Elem<T>::to_f32(rawv), (int64_t)col));
+          atomicAdd(&lh[bin_level0<KB>(key - cut_key)], 1u);
+          wbuf[n_buf + i] = make_uint2(col, Elem<T>::raw(rawv));
         }
-      n += total;
+        n_buf += total;
+      } else {
+        uint32_t mm = m;   // histogram only
+        while (ballot64(mm != 0)) {
+          if (mm) {
+            const int bit = __ffs(mm) - 1;
+            mm &= mm - 1u;
+            const uint32_t rel = (uint32_t)((bit / V) * 64 * V + lane * V + (bit % V));
+            const uint32_t key = rank_key<KB>(rk(Elem<T>::to_f32(stage[rel]), (int64_t)(c0u + rel)));
+            atomicAdd(&lh[bin_level0<KB>(key - cut_key)], 1u);
+          }
+        }
+      }
     }
-    if (lane == 0) seg_count[r] = n;
+    flush();
+    if (lane == 0) row_first[r] = dense ? ROW_DENSE : first;
   }
   __syncthreads();
   for (int i = threadIdx.x; i < NBINS; i += blockDim.x) {
@@ -300,7 +433,7 @@ __global__ __launch_bounds__(256) void k_select_pass(
 
 // One block per problem: consume the histogram of the current level.
 template <int KB>
-__global__ __launch_bounds__(SCAN_THREADS) void k_select_scan(SelState *st, uint32_t *hist, int phase, int level) {
+__global__ __launch_bounds__(SCAN_THREADS) void k_select_scan(SelState *st, uint32_t *hist, uint32_t *pool_count, int phase, int level) {
   __shared__ uint32_t lh[NBINS];
   const int p = blockIdx.x, tid = threadIdx.x;
   SelState s = st[p];
@@ -317,6 +450,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_select_scan(SelState *st, uint
   if (!found) {
     // fewer candidates than K: the sampled cut was too high -> run the pass again from the bottom
     s.status = ST_RETRY; s.cut_key = min_key<KB>(); s.level = 0;
+    pool_count[p] = 0;  // the retry pass refills the pool from scratch
     st[p] = s;
     return;
   }
@@ -343,42 +477,49 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_select_scan(SelState *st, uint
   st[p] = s;
 }
 
-// Visit the candidates of one row (segment, or the dense row when the segment
-// overflowed) with one wavefront.  `f(active, col, raw, key)` is called once per wave step
-// with one element per lane (active=false for idle lanes), in ascending column order
-// across steps and lanes.
+// Visit the candidates of one row (its chain of pool extents, or the dense row when the
+// row got no pool space) with one wavefront.  `f(active, col, raw, key)` is called once per
+// wave step with one element per lane (active=false for idle lanes), in ascending column
+// order across steps and lanes.
 template <typename T, bool GLOBAL, typename Fn>
 __device__ __forceinline__ void visit_candidates(
     const T *pre, int64_t Tn, int64_t F, int64_t lstride, int l, int64_t t,
-    typename RankOf<T, GLOBAL>::type rk, uint32_t cut_key, const uint32_t *seg_count,
-    const uint2 *seg, int cap, Fn f) {
+    typename RankOf<T, GLOBAL>::type rk, uint32_t cut_key, const uint32_t *row_first,
+    const uint2 *mypool, Fn f) {
   constexpr int KB = Elem<T>::KEYBITS;
   const int lane = lane_id();
   const int64_t r = (int64_t)l * Tn + t;
-  const uint32_t n = seg_count[r];
-  if (n <= (uint32_t)cap) {
-    const uint2 *sg = seg + r * cap;
-    for (uint32_t i0 = 0; i0 < n; i0 += 64) {
-      uint32_t i = i0 + lane;
-      bool act = i < n;
-      uint2 e = act ? sg[i] : make_uint2(0, 0);
-      uint32_t key = 0;
-      if (act) key = rank_key<KB>(rk(Elem<T>::to_f32(Elem<T>::from_raw(e.y)), (int64_t)e.x));
-      f(act, e.x, e.y, key);
+  uint32_t off = row_first[r];
+  if (off != ROW_DENSE) {
+    while (off != ROW_NONE) {
+      const uint2 hdr = mypool[off];
+      const uint2 *sg = mypool + off + 1u;
+      for (uint32_t i0 = 0; i0 < hdr.y; i0 += 64) {
+        uint32_t i = i0 + lane;
+        bool act = i < hdr.y;
+        uint2 e = act ? sg[i] : make_uint2(0, 0);
+        uint32_t key = 0;
+        if (act) key = rank_key<KB>(rk(Elem<T>::to_f32(Elem<T>::from_raw(e.y)), (int64_t)e.x));
+        f(act, e.x, e.y, key);
+      }
+      off = hdr.x;
     }
   } else {
+    constexpr int NQ = 8;  // independent loads in flight; each covers 64 consecutive columns
     const T *row = pre + l * lstride + t * F;
-    for (int64_t c0 = 0; c0 < F; c0 += 64) {
-      int64_t col = c0 + lane;
-      bool act = col < F;
-      uint32_t raw = 0, key = 0;
-      if (act) {
-        T v = row[col];
-        raw = Elem<T>::raw(v);
-        key = rank_key<KB>(rk(Elem<T>::to_f32(v), col));
-        act = key >= cut_key;
+    for (int64_t c0 = 0; c0 < F; c0 += 64 * NQ) {
+      T v[NQ];
+#pragma unroll
+      for (int q = 0; q < NQ; ++q) { int64_t col = c0 + q * 64 + lane; v[q] = col < F ? row[col] : T(0); }
+#pragma unroll
+      for (int q = 0; q < NQ; ++q) {
+        const int64_t col = c0 + q * 64 + lane;
+        if (c0 + q * 64 >= F) break;
+        bool act = col < F;
+        uint32_t raw = Elem<T>::raw(v[q]), key = 0;
+        if (act) { key = rank_key<KB>(rk(Elem<T>::to_f32(v[q]), col)); act = key >= cut_key; }
+        f(act, (uint32_t)col, raw, key);
       }
-      f(act, (uint32_t)col, raw, key);
     }
   }
 }
@@ -387,8 +528,8 @@ __device__ __forceinline__ void visit_candidates(
 template <typename T, bool GLOBAL>
 __global__ __launch_bounds__(256) void k_select_level(
     const T *pre, int64_t Tn, int64_t F, int64_t L, int64_t lstride, const float *mean,
-    const float *denom, const SelState *st, uint32_t *hist, const uint32_t *seg_count,
-    const uint2 *seg, int cap, int level) {
+    const float *denom, const SelState *st, uint32_t *hist, const uint32_t *row_first,
+    const uint2 *pool, unsigned long long pool_cap, int level) {
   __shared__ uint32_t lh[NBINS];
   const int l = blockIdx.y, p = GLOBAL ? 0 : l;
   const SelState s = st[p];
@@ -398,7 +539,7 @@ __global__ __launch_bounds__(256) void k_select_level(
   const int wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
   typename RankOf<T, GLOBAL>::type rk = RankOf<T, GLOBAL>::make(mean, denom, l, F);
   for (int64_t t = (int64_t)blockIdx.x * nwv + wv; t < Tn; t += (int64_t)gridDim.x * nwv) {
-    visit_candidates<T, GLOBAL>(pre, Tn, F, lstride, l, t, rk, s.cut_key, seg_count, seg, cap,
+    visit_candidates<T, GLOBAL>(pre, Tn, F, lstride, l, t, rk, s.cut_key, row_first, pool + (unsigned long long)p * pool_cap,
       [&](bool act, uint32_t, uint32_t, uint32_t key) {
         if (act) {
           uint32_t diff = key - s.cut_key;
@@ -417,15 +558,15 @@ __global__ __launch_bounds__(256) void k_select_level(
 template <typename T, bool GLOBAL>
 __global__ __launch_bounds__(256) void k_select_count(
     const T *pre, int64_t Tn, int64_t F, int64_t L, int64_t lstride, const float *mean,
-    const float *denom, const SelState *st, const uint32_t *seg_count, const uint2 *seg,
-    int cap, uint32_t *row_gt, uint32_t *row_eq) {
+    const float *denom, const SelState *st, const uint32_t *row_first, const uint2 *pool,
+    unsigned long long pool_cap, uint32_t *row_gt, uint32_t *row_eq) {
   const int l = blockIdx.y, p = GLOBAL ? 0 : l;
   const SelState s = st[p];
   const int wv = threadIdx.x >> 6, nwv = blockDim.x >> 6, lane = lane_id();
   typename RankOf<T, GLOBAL>::type rk = RankOf<T, GLOBAL>::make(mean, denom, l, F);
   for (int64_t t = (int64_t)blockIdx.x * nwv + wv; t < Tn; t += (int64_t)gridDim.x * nwv) {
     uint32_t ngt = 0, neq = 0;
-    visit_candidates<T, GLOBAL>(pre, Tn, F, lstride, l, t, rk, s.cut_key, seg_count, seg, cap,
+    visit_candidates<T, GLOBAL>(pre, Tn, F, lstride, l, t, rk, s.cut_key, row_first, pool + (unsigned long long)p * pool_cap,
       [&](bool act, uint32_t, uint32_t, uint32_t key) {
         ngt += (uint32_t)__popcll(ballot64(act && key > s.thr_key));
         neq += (uint32_t)__popcll(ballot64(act && key == s.thr_key));
@@ -499,8 +640,8 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_rowptr_scan(const uint32_t *ke
 template <typename T, bool GLOBAL>
 __global__ __launch_bounds__(256) void k_select_emit(
     const T *pre, int64_t Tn, int64_t F, int64_t L, int64_t lstride, const float *mean,
-    const float *denom, const SelState *st, const uint32_t *seg_count, const uint2 *seg, int cap,
-    const uint32_t *allot, const int32_t *row_ptr, int32_t *col_out, T *val_out) {
+    const float *denom, const SelState *st, const uint32_t *row_first, const uint2 *pool,
+    unsigned long long pool_cap, const uint32_t *allot, const int32_t *row_ptr, int32_t *col_out, T *val_out) {
   const int l = blockIdx.y, p = GLOBAL ? 0 : l;
   const SelState s = st[p];
   const int wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
@@ -510,7 +651,7 @@ __global__ __launch_bounds__(256) void k_select_emit(
     const int64_t base = row_ptr[r];
     const uint32_t my_allot = allot[r];
     uint32_t kept = 0, ties = 0;
-    visit_candidates<T, GLOBAL>(pre, Tn, F, lstride, l, t, rk, s.cut_key, seg_count, seg, cap,
+    visit_candidates<T, GLOBAL>(pre, Tn, F, lstride, l, t, rk, s.cut_key, row_first, pool + (unsigned long long)p * pool_cap,
       [&](bool act, uint32_t col, uint32_t raw, uint32_t key) {
         bool eq = act && key == s.thr_key;
         uint64_t beq = ballot64(eq);
@@ -582,34 +723,37 @@ __global__ __launch_bounds__(256) void k_threshold(
 
 // ---- host side ------------------------------------------------------------------------
 struct SelLayout {
-  size_t off_state, off_hist, off_segcnt, off_gt, off_eq, off_allot, off_keep, off_seg, total;
-  int cap, nprob;
+  size_t off_state, off_hist, off_poolcnt, off_sample, off_first, off_gt, off_eq, off_allot, off_keep, off_pool, total;
+  unsigned long long pool_cap;  // entries per problem
+  int nprob;
 };
-
-static int seg_capacity(int64_t T, int64_t F, int64_t L, int64_t k, int mode) {
-  // expected candidates per row are about 2x the survivors per row
-  double per_row = mode == CLT_TOPK_GLOBAL ? (double)k / (double)L : (double)k;
-  int64_t want = (int64_t)(4.0 * per_row) + 1;
-  int64_t cap = 64;
-  while (cap < want && cap < 4096) cap <<= 1;
-  return (int)cap;
-}
 
 static SelLayout sel_layout(int64_t T, int64_t F, int64_t L, int64_t k, int mode) {
   SelLayout lo;
   lo.nprob = mode == CLT_TOPK_GLOBAL ? 1 : (int)L;
-  lo.cap = seg_capacity(T, F, L, k, mode);
   const size_t R = (size_t)(L * T);
+  const unsigned long long rows_p = mode == CLT_TOPK_GLOBAL ? (unsigned long long)R : (unsigned long long)T;
+  const unsigned long long N = (unsigned long long)T * F * (mode == CLT_TOPK_GLOBAL ? L : 1);
+  unsigned long long K = (unsigned long long)k * T;
+  if (K > N) K = N;
+  // about 2x K candidates are expected; every extent also stores one header entry
+  unsigned long long cap = 4ull * K + 2ull * rows_p + 4096ull;
+  const unsigned long long hard = N + 2ull * rows_p + 4096ull;
+  if (cap > hard) cap = hard;
+  if (cap > 0xFFF00000ull) cap = 0xFFF00000ull;
+  lo.pool_cap = cap;
   size_t o = 0;
   auto take = [&](size_t bytes) { size_t at = o; o += (bytes + 255) & ~(size_t)255; return at; };
   lo.off_state = take(sizeof(SelState) * (size_t)lo.nprob);
   lo.off_hist = take(sizeof(uint32_t) * NBINS * (size_t)lo.nprob);
-  lo.off_segcnt = take(4 * R);
+  lo.off_poolcnt = take(4 * (size_t)lo.nprob);
+  lo.off_sample = take(4 * (size_t)SAMPLE_N * (size_t)lo.nprob);
+  lo.off_first = take(4 * R);
   lo.off_gt = take(4 * R);
   lo.off_eq = take(4 * R);
   lo.off_allot = take(4 * R);
   lo.off_keep = take(4 * R);
-  lo.off_seg = take(8 * R * (size_t)lo.cap);
+  lo.off_pool = take(8 * (size_t)cap * (size_t)lo.nprob);
   lo.total = o;
   return lo;
 }
@@ -623,34 +767,41 @@ static int run_batchtopk(const T *pre, int64_t Tn, int64_t F, int64_t L, int64_t
   const SelLayout lo = sel_layout(Tn, F, L, k, mode);
   SelState *st = (SelState *)(ws + lo.off_state);
   uint32_t *hist = (uint32_t *)(ws + lo.off_hist);
-  uint32_t *segcnt = (uint32_t *)(ws + lo.off_segcnt);
+  uint32_t *poolcnt = (uint32_t *)(ws + lo.off_poolcnt);
+  uint32_t *sample = (uint32_t *)(ws + lo.off_sample);
+  uint32_t *first = (uint32_t *)(ws + lo.off_first);
   uint32_t *rgt = (uint32_t *)(ws + lo.off_gt), *req = (uint32_t *)(ws + lo.off_eq);
   uint32_t *allot = (uint32_t *)(ws + lo.off_allot), *keep = (uint32_t *)(ws + lo.off_keep);
-  uint2 *seg = (uint2 *)(ws + lo.off_seg);
+  uint2 *pool = (uint2 *)(ws + lo.off_pool);
   const unsigned long long N = (unsigned long long)Tn * (unsigned long long)F * (GLOBAL ? (unsigned long long)L : 1ull);
   unsigned long long K = (unsigned long long)k * (unsigned long long)Tn;
   if (K > N) K = N;
   const int nprob = lo.nprob;
-  k_fill_u32<<<64, 256, 0, stream>>>(hist, 0u, (int64_t)NBINS * nprob);
-  k_sample_cut<T, GLOBAL><<<nprob, SCAN_THREADS, 0, stream>>>(pre, Tn, F, L, lstride, mean, denom, N, K, st);
-  int gx = (int)clt_ceil_div(Tn, 4);
-  int maxgx = (int)clt_ceil_div(256 * 8, L);  // about 8 blocks per CU over all layers
-  if (maxgx < 1) maxgx = 1;
-  if (gx > maxgx) gx = maxgx;
+  k_sample_keys<T, GLOBAL><<<dim3(SAMPLE_BLOCKS, nprob), 256, 0, stream>>>(pre, Tn, F, L, lstride, mean, denom, N, sample);
+  k_sample_cut<KB><<<nprob, SCAN_THREADS, 0, stream>>>(sample, N, K, st, hist, poolcnt);
+  // two rows per wavefront: many more blocks than fit at once, so rows of very different
+  // candidate counts balance out over the CUs
+  int gx = (int)clt_ceil_div(Tn, 8);
+  if (gx > 65535 * 8) gx = 65535 * 8;
   dim3 grid(gx, (unsigned)L);
   for (int phase = 0; phase < 2; ++phase) {
-    k_select_pass<T, V, GLOBAL><<<grid, 256, 0, stream>>>(pre, Tn, F, L, lstride, mean, denom, st, hist, segcnt, seg, lo.cap, phase);
-    k_select_scan<KB><<<nprob, SCAN_THREADS, 0, stream>>>(st, hist, phase, 0);
+    k_select_pass<T, V, GLOBAL><<<grid, 256, 0, stream>>>(pre, Tn, F, L, lstride, mean, denom, st, hist, poolcnt, pool, lo.pool_cap, first, phase);
+    k_select_scan<KB><<<nprob, SCAN_THREADS, 0, stream>>>(st, hist, poolcnt, phase, 0);
   }
+  int gx2 = (int)clt_ceil_div(Tn, 4);
+  int maxgx2 = (int)clt_ceil_div(256 * 8, L);
+  if (maxgx2 < 1) maxgx2 = 1;
+  if (gx2 > maxgx2) gx2 = maxgx2;
+  dim3 grid2(gx2, (unsigned)L);
   const int nlev = KB == 32 ? 3 : 2;
   for (int level = 1; level < nlev; ++level) {
-    k_select_level<T, GLOBAL><<<grid, 256, 0, stream>>>(pre, Tn, F, L, lstride, mean, denom, st, hist, segcnt, seg, lo.cap, level);
-    k_select_scan<KB><<<nprob, SCAN_THREADS, 0, stream>>>(st, hist, 2, level);
+    k_select_level<T, GLOBAL><<<grid2, 256, 0, stream>>>(pre, Tn, F, L, lstride, mean, denom, st, hist, first, pool, lo.pool_cap, level);
+    k_select_scan<KB><<<nprob, SCAN_THREADS, 0, stream>>>(st, hist, poolcnt, 2, level);
   }
-  k_select_count<T, GLOBAL><<<grid, 256, 0, stream>>>(pre, Tn, F, L, lstride, mean, denom, st, segcnt, seg, lo.cap, rgt, req);
+  k_select_count<T, GLOBAL><<<grid2, 256, 0, stream>>>(pre, Tn, F, L, lstride, mean, denom, st, first, pool, lo.pool_cap, rgt, req);
   k_select_allot<GLOBAL><<<nprob, SCAN_THREADS, 0, stream>>>(st, Tn, L, rgt, req, allot, keep, row_ptr, K);
   if (GLOBAL) k_rowptr_scan<<<1, SCAN_THREADS, 0, stream>>>(keep, L * Tn, row_ptr);
-  k_select_emit<T, GLOBAL><<<grid, 256, 0, stream>>>(pre, Tn, F, L, lstride, mean, denom, st, segcnt, seg, lo.cap, allot, row_ptr, col, val);
+  k_select_emit<T, GLOBAL><<<grid2, 256, 0, stream>>>(pre, Tn, F, L, lstride, mean, denom, st, first, pool, lo.pool_cap, allot, row_ptr, col, val);
   return clt_check_launch();
 }
 

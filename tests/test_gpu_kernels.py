@@ -140,6 +140,25 @@ def test_batchtopk_outlier_rows_overflow_segments(dev, dtype):
     assert torch.equal(dense_from(surv), oracle_per_layer(pre, k))
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_batchtopk_candidate_pool_overflow_falls_back_to_dense_rows(dev, dtype):
+    # half of all values tie at the top: the sampled cut admits ~500x more candidates than the
+    # pool holds, so most rows are re-read from the matrix; the result must not change
+    g = torch.Generator().manual_seed(13)
+    L, T, F, k = 2, 512, 2048, 4
+    pre = torch.randn(L, T, F, generator=g).clamp(max=0.0)
+    pre[1] = pre[1].clamp(min=-0.5)
+    pre = pre.to(dtype)
+    surv = run_select(pre, k, dev)
+    check_rows_sorted(surv)
+    for l in range(L):
+        m = orc.batchtopk_mask(pre[l], k, pre[l])
+        rows = engine.survivor_rows(surv).cpu()
+        sel = (rows >= l * T) & (rows < (l + 1) * T)
+        flat = (rows[sel] - l * T) * F + surv.col.cpu().long()[sel]
+        assert torch.equal(torch.sort(flat).values, m.view(-1).nonzero().view(-1))
+
+
 def test_batchtopk_k_zero_and_empty(dev):
     pre = torch.randn(2, 8, 16)
     surv = run_select(pre, 0, dev)
