@@ -1,16 +1,21 @@
 // Encoder projection  pre[l] = x[l] . W[l]^T + b[l]   (reference clt/models/parallel.py:286)
 //
 // MFMA kernel for gfx950.  Both operands are K-contiguous (x is [T][d], W is [F][d]), so
-// one loader serves both: 16-byte chunks go global -> registers -> LDS, where rows are
-// 128 bytes and the chunk index is XOR-swizzled with the row so that the 16-byte
-// fragment reads of a wavefront spread over the banks.  The matrix-core "A" operand is
-// the W tile and "B" the x tile, so every lane ends up with 4 consecutive features of one
-// token per accumulator group and stores them with one 8-byte (bf16) / 16-byte (fp32) write.
+// one loader serves both.
 //
-//   block tile  256 tokens x 128 features, 4 wavefronts (2 x 2), wave tile 128 x 64
-//   k step      128 bytes of K per LDS stage (64 bf16 / 32 fp32), next stage prefetched
-//               into registers while the current one is multiplied
-//   bf16        v_mfma_f32_32x32x16_bf16, fp32 accumulate, one rounding at the store
+//   block tile  256 tokens x 256 features, 4 wavefronts (2 x 2), wave tile 128 x 128:
+//               256 fp32 accumulators per lane, one wavefront per SIMD, one block per CU
+//   k step      128 bytes of K per LDS stage (64 bf16 / 32 fp32), two stages of 64 KB
+//   loads       global_load_lds_dwordx4: 16 bytes per lane straight into LDS, no staging
+//               registers.  LDS rows are 128 bytes; chunk c of row r lives at chunk position
+//               c ^ ((r >> 1) & 7), which the loader realises by permuting which global chunk
+//               each lane fetches, so the 16-byte fragment reads of a wavefront spread over
+//               all banks
+//   math        the matrix-core "A" operand is the W tile and "B" the x tile, so a lane ends
+//               up with 4 consecutive features of one token per accumulator group
+//   epilogue    bias add, rounding, then the tile goes through LDS so that the stores are
+//               16 bytes per lane and 256 contiguous bytes per token
+//   bf16        v_mfma_f32_32x32x16_bf16, fp32 accumulate, one rounding (v_cvt_pk_bf16_f32)
 //   fp32        v_mfma_f32_32x32x2_f32
 #include "clt_common.h"
 
@@ -20,12 +25,10 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
 
 constexpr int BM = 256;   // tokens per block
-constexpr int BN = 128;   // features per block
+constexpr int BN = 256;   // features per block
 constexpr int ROWB = 128; // bytes of K per LDS row
-constexpr int XCH = BM * 8 / 256;  // 16-byte chunks of the x tile per thread
-constexpr int WCH = BN * 8 / 256;
+constexpr int STAGE = (BM + BN) * ROWB;  // bytes of one LDS stage
 
-__device__ __forceinline__ int lds_off(int row, int ch) { return row * ROWB + ((ch ^ (row & 7)) << 4); }
 
 template <typename T> struct Mma;
 template <> struct Mma<bf16_t> {
@@ -43,110 +46,213 @@ template <> struct Mma<float> {
   }
 };
 
+// 16 bytes per lane from global memory straight into LDS: lane i of the wavefront lands at
+// lds_base + 16 * i (lds_base must be wave-uniform).
+__device__ __forceinline__ void load16_to_lds(const void *gsrc, void *lds_base) {
+  __builtin_amdgcn_global_load_lds(gsrc, (__attribute__((address_space(3))) void *)lds_base, 16, 0, 0);
+}
+
+typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+
+// two fp32 -> packed bf16 (round to nearest even; one v_cvt_pk_bf16_f32)
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+  f32x2_t v = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+}
+
+// Requires K % (256 / sizeof(T)) == 0 (an even number of LDS stages), M >= BM and N >= BN.  A tile that
+// would stick out of the matrix is shifted back inside (its overlap with the neighbour is
+// computed twice and stored twice with identical values), so no load or store is predicated.
+//
+// Block -> tile map: workgroups go to the 8 XCDs round-robin, so block b runs on XCD b % 8.
+// When the feature tiles split evenly, XCD x takes the feature tiles n = x, x+8, ... and walks
+// all token tiles of one n before the next: a W tile is fetched by one XCD only and the x slab
+// of the layer stays in that XCD's L2.
 template <typename T>
-__global__ __launch_bounds__(256, 2) void k_encode_mfma(
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void k_encode_mfma(
     const T *__restrict__ x, const T *__restrict__ w, const T *__restrict__ bias, T *__restrict__ pre,
     int M, int K, int N, int tiles_m, int tiles_n, int64_t xs, int64_t wstr, int64_t bs, int64_t ps) {
   constexpr int CE = 16 / (int)sizeof(T);  // elements per 16-byte chunk
   constexpr int BK = ROWB / (int)sizeof(T);
-  __shared__ __attribute__((aligned(16))) unsigned char lds[(BM + BN) * ROWB];
-  unsigned char *xsm = lds, *wsm = lds + BM * ROWB;
+  // Two separate stage buffers (not one array with an offset): the compiler can then tell that
+  // a fragment read of one stage does not depend on the direct-to-LDS loads in flight into the
+  // other, and does not wait for them.
+  __shared__ __attribute__((aligned(16))) unsigned char stage0[STAGE];
+  __shared__ __attribute__((aligned(16))) unsigned char stage1[STAGE];
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave & 1, wn = wave >> 1;
   int bid = blockIdx.x;
   const int per_layer = tiles_m * tiles_n;
   const int layer = bid / per_layer;
   bid -= layer * per_layer;
-  const int tn = bid / tiles_m, tm = bid - tn * tiles_m;  // token tiles vary fastest
-  const int m0 = tm * BM, n0 = tn * BN;
-  const T *xl = x + (int64_t)layer * xs;
-  const T *wl = w + (int64_t)layer * wstr;
+  int tn, tm;
+  if ((tiles_n & 7) == 0) {
+    const int xcd = bid & 7, idx = bid >> 3;
+    tm = idx % tiles_m;
+    tn = (idx / tiles_m) * 8 + xcd;
+  } else {
+    tn = bid / tiles_m; tm = bid - tn * tiles_m;
+  }
+  int m0 = tm * BM, n0 = tn * BN;
+  if (m0 + BM > M) m0 = M - BM;
+  if (n0 + BN > N) n0 = N - BN;
 
-  const int lrow = tid >> 3, lch = tid & 7;  // loader: row (+32 per step) and chunk of this thread
-  uint4 xr[XCH], wr[WCH];
-  auto load_stage = [&](int k0) {
-    const int kk = k0 + lch * CE;
-    const bool kin = kk + CE <= K;
+  // ---- loader: wave `wave` brings in rows [64*wave, 64*wave+64) of both tiles, 8 rows (1 KB)
+  // per instruction.  Lane l lands at row l>>3, chunk position l&7 of its 8-row group and
+  // therefore fetches global chunk (l&7) ^ ((row >> 1) & 7).
+  const int lr = lane >> 3, lp = lane & 7;
+  const int offE = lr * K + ((lp ^ (lane >> 4)) * CE);          // 8-row groups starting at a multiple of 16
+  const int offO = lr * K + ((lp ^ ((lane >> 4) | 4)) * CE);    // ... at 8 mod 16
+  const T *xt = x + (int64_t)layer * xs + (int64_t)(m0 + wave * 64) * K;
+  const T *wt = w + (int64_t)layer * wstr + (int64_t)(n0 + wave * 64) * K;
+  auto issue_stage = [&](unsigned char *stage, int k0) {
+    unsigned char *xs_l = stage + wave * 64 * ROWB;
+    unsigned char *ws_l = xs_l + BM * ROWB;
 #pragma unroll
-    for (int i = 0; i < XCH; ++i) {
-      const int row = m0 + lrow + i * 32;
-      xr[i] = (kin && row < M) ? *reinterpret_cast<const uint4 *>(xl + (int64_t)row * K + kk) : make_uint4(0, 0, 0, 0);
-    }
-#pragma unroll
-    for (int i = 0; i < WCH; ++i) {
-      const int row = n0 + lrow + i * 32;
-      wr[i] = (kin && row < N) ? *reinterpret_cast<const uint4 *>(wl + (int64_t)row * K + kk) : make_uint4(0, 0, 0, 0);
+    for (int t = 0; t < 8; ++t) {
+      const int off = (t & 1) ? offO : offE;
+      load16_to_lds(xt + (int64_t)t * 8 * K + k0 + off, xs_l + t * 8 * ROWB);
+      load16_to_lds(wt + (int64_t)t * 8 * K + k0 + off, ws_l + t * 8 * ROWB);
     }
   };
-  auto store_stage = [&]() {
-#pragma unroll
-    for (int i = 0; i < XCH; ++i) *reinterpret_cast<uint4 *>(xsm + lds_off(lrow + i * 32, lch)) = xr[i];
-#pragma unroll
-    for (int i = 0; i < WCH; ++i) *reinterpret_cast<uint4 *>(wsm + lds_off(lrow + i * 32, lch)) = wr[i];
-  };
 
-  f32x16_t acc[4][2];
+  // ---- fragment reader: row l31 of each 32-row group; chunk (kk*2 + lh) at its swizzled position
+  const int l31 = lane & 31, lh = lane >> 5;
+  const int xrow = (wm * 128 + l31) * ROWB;             // + i * 32 * ROWB
+  const int wrow = BM * ROWB + (wn * 128 + l31) * ROWB; // + j * 32 * ROWB
+  int koff[4];
+#pragma unroll
+  for (int kk = 0; kk < 4; ++kk) koff[kk] = ((kk * 2 + lh) ^ ((l31 >> 1) & 7)) << 4;
+
+  f32x16_t acc[4][4];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < 4; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-  const int l31 = lane & 31, lh = lane >> 5;
-  load_stage(0);
-  for (int k0 = 0; k0 < K; k0 += BK) {
-    store_stage();
-    __syncthreads();
-    if (k0 + BK < K) load_stage(k0 + BK);
+  // Software pipeline over the K stages.  Fragments are double-buffered in registers (fa/fb)
+  // and read one k-step ahead of the matrix ops that use them.  There is one barrier per
+  // stage, placed before the LAST k-step of a stage: at that point this wavefront's loads of
+  // the next stage have landed and its LDS reads of the current stage are complete, so after
+  // the barrier the next stage may be read (its first fragments are fetched under the last
+  // k-step's matrix ops) and the current one may be overwritten by the stage after next.
+  const int nk = K / BK;
+  uint4 fa[8], fb[8];   // [0..3] x fragments, [4..7] W fragments
+  auto load_frags = [&](uint4 (&f)[8], const unsigned char *sb, int kk) {
 #pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
-      const int ch = kk * 2 + lh;
-      uint4 xa[4], wa[2];
+    for (int i = 0; i < 4; ++i) f[i] = *reinterpret_cast<const uint4 *>(sb + xrow + i * 32 * ROWB + koff[kk]);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) xa[i] = *reinterpret_cast<const uint4 *>(xsm + lds_off(wm * 128 + i * 32 + l31, ch));
+    for (int j = 0; j < 4; ++j) f[4 + j] = *reinterpret_cast<const uint4 *>(sb + wrow + j * 32 * ROWB + koff[kk]);
+  };
+  auto mma16 = [&](const uint4 (&f)[8]) {
 #pragma unroll
-      for (int j = 0; j < 2; ++j) wa[j] = *reinterpret_cast<const uint4 *>(wsm + lds_off(wn * 64 + j * 32 + l31, ch));
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int j = 0; j < 4; ++j) Mma<T>::run(acc[i][j], f[4 + j], f[i]);
+  };
+  // interleave hint: pairs of matrix ops with one LDS read between them
+  auto mix_ds = [&]() {
 #pragma unroll
-        for (int j = 0; j < 2; ++j) Mma<T>::run(acc[i][j], wa[j], xa[i]);
+    for (int g = 0; g < 8; ++g) {
+      __builtin_amdgcn_sched_group_barrier(0x008, sizeof(T) == 2 ? 2 : 8, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
     }
+  };
+  // one stage except its last k-step, the barrier, then the last k-step overlapped with the
+  // loads of the stage after next (into `cur`) and the first fragments of `nxt`
+  auto body = [&](unsigned char *cur, unsigned char *nxt, int kt) {
+    load_frags(fb, cur, 1); mma16(fa); mix_ds();
+    load_frags(fa, cur, 2); mma16(fb); mix_ds();
+    load_frags(fb, cur, 3); mma16(fa); mix_ds();
+    __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
-  }
+    // past the end of K the last stage is fetched again (never read)
+    const int kn = kt + 2 < nk ? kt + 2 : nk - 1;
+    issue_stage(cur, kn * BK);
+    load_frags(fa, nxt, 0);
+    mma16(fb);
+#pragma unroll
+    for (int g = 0; g < 16; ++g) {
+      __builtin_amdgcn_sched_group_barrier(0x008, sizeof(T) == 2 ? 1 : 4, 0);
+      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+  };
+  issue_stage(stage0, 0);
+  __builtin_amdgcn_s_waitcnt(0);
+  __syncthreads();
+  issue_stage(stage1, BK);
+  load_frags(fa, stage0, 0);
+  // nk is even (checked by the launcher).  The last two bodies fetch the final stage again and
+  // read fragments that are never used: cheaper than a differently shaped last iteration.
+  for (int kt = 0; kt < nk; kt += 2) { body(stage0, stage1, kt); body(stage1, stage0, kt + 1); }
+  __builtin_amdgcn_s_waitcnt(0);   // no direct-to-LDS load may be in flight when the block retires
 
-  // epilogue: lane owns token (l31) and, per accumulator group rg, features 8*rg + 4*lh + 0..3
+  // ---- epilogue.  The accumulator layout gives a lane 4 consecutive features of one token,
+  // i.e. 8-byte pieces scattered over 32 rows per store - slow to write.  Each wavefront
+  // therefore parks its 128 x 128 tile in LDS (the stage buffers are free now; 32 KB per
+  // wavefront for bf16, two passes of 64 features for fp32) and writes it out row by row,
+  // 16 bytes per lane, 256 contiguous bytes per token.
+  __syncthreads();   // every wavefront is done with the last stage
   T *pl = pre + (int64_t)layer * ps;
   const T *bl = bias ? bias + (int64_t)layer * bs : nullptr;
+  unsigned char *park = (wave < 2 ? stage0 : stage1) + (wave & 1) * (STAGE / 2);
+  constexpr int NPASS = sizeof(T) == 2 ? 1 : 2;           // feature halves per pass
+  constexpr int JP = 4 / NPASS;                            // 32-feature groups per pass
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
+  for (int pass = 0; pass < NPASS; ++pass) {
+    // rows of 256 bytes (128 bf16 / 64 fp32), 16-byte slots XOR-swizzled with the token
 #pragma unroll
-    for (int rg = 0; rg < 4; ++rg) {
-      const int n = n0 + wn * 64 + j * 32 + rg * 8 + lh * 4;
-      if (n >= N) continue;
-      float bv[4] = {0.f, 0.f, 0.f, 0.f};
-      if (bl) {
+    for (int jj = 0; jj < JP; ++jj) {
+      const int j = pass * JP + jj;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) bv[q] = Elem<T>::to_f32(bl[n + q]);
-      }
+      for (int rg = 0; rg < 4; ++rg) {
+        const int nl = jj * 32 + rg * 8 + lh * 4;          // feature inside this pass
+        const int n = n0 + wn * 128 + j * 32 + rg * 8 + lh * 4;
+        float bv[4] = {0.f, 0.f, 0.f, 0.f};
+        if (bl) {
+          if (sizeof(T) == 4) {
+            float4 b4 = *reinterpret_cast<const float4 *>(bl + n);
+            bv[0] = b4.x; bv[1] = b4.y; bv[2] = b4.z; bv[3] = b4.w;
+          } else {
+            uint2 b2 = *reinterpret_cast<const uint2 *>(bl + n);
+            bv[0] = __uint_as_float(b2.x << 16); bv[1] = __uint_as_float(b2.x & 0xFFFF0000u);
+            bv[2] = __uint_as_float(b2.y << 16); bv[3] = __uint_as_float(b2.y & 0xFFFF0000u);
+          }
+        }
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int m = m0 + wm * 128 + i * 32 + l31;
-        if (m >= M) continue;
-        float y[4];
+        for (int i = 0; i < 4; ++i) {
+          const int ml = i * 32 + l31;                     // token inside the wave tile
+          float y[4];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) y[q] = acc[i][j][rg * 4 + q] + bv[q];
-        T *po = pl + (int64_t)m * N + n;
-        if (sizeof(T) == 4) {
-          *reinterpret_cast<float4 *>(po) = make_float4(y[0], y[1], y[2], y[3]);
-        } else {
-          uint2 o;
-          o.x = f32_to_bf16_bits(y[0]) | (f32_to_bf16_bits(y[1]) << 16);
-          o.y = f32_to_bf16_bits(y[2]) | (f32_to_bf16_bits(y[3]) << 16);
-          *reinterpret_cast<uint2 *>(po) = o;
+          for (int q = 0; q < 4; ++q) y[q] = acc[i][j][rg * 4 + q] + bv[q];
+          if (sizeof(T) == 4) {
+            const int slot = (nl >> 2) ^ (ml & 15);
+            *reinterpret_cast<float4 *>(park + ml * 256 + slot * 16) = make_float4(y[0], y[1], y[2], y[3]);
+          } else {
+            const int slot = (nl >> 3) ^ (ml & 15);
+            uint2 o;
+            o.x = pack_bf16x2(y[0], y[1]);
+            o.y = pack_bf16x2(y[2], y[3]);
+            *reinterpret_cast<uint2 *>(park + ml * 256 + slot * 16 + (nl & 4) * 2) = o;
+          }
         }
       }
+    }
+    // the wavefront reads its own tile back: lane -> (row = it*4 + lane/16, slot = lane%16)
+    constexpr int EPS = 16 / (int)sizeof(T);               // elements per 16-byte slot
+#pragma unroll 4
+    for (int it = 0; it < 32; ++it) {
+      const int ml = it * 4 + (lane >> 4), sl = lane & 15;
+      const uint4 v = *reinterpret_cast<const uint4 *>(park + ml * 256 + ((sl ^ (ml & 15)) * 16));
+      const int m = m0 + wm * 128 + ml;
+      const int n = n0 + wn * 128 + pass * (128 / NPASS) + sl * EPS;
+      *reinterpret_cast<uint4 *>(pl + (int64_t)m * N + n) = v;
     }
   }
 }
@@ -170,10 +276,10 @@ template <typename T>
 static int launch_encode(const void *x, const void *w, const void *b, void *pre, int64_t T_, int64_t d, int64_t F,
                          int64_t L, int64_t xs, int64_t wstr, int64_t bs, int64_t ps, hipStream_t stream) {
   constexpr int CE = 16 / (int)sizeof(T);
-  const bool fast = (d % CE == 0) && (F % 4 == 0) && clt_aligned16(x) && clt_aligned16(w) && clt_aligned16(pre) &&
+  const bool fast = (d % (2 * ROWB / (int)sizeof(T)) == 0) && (F % 4 == 0) && T_ >= BM && F >= BN && clt_aligned16(x) && clt_aligned16(w) && clt_aligned16(pre) &&
                     (xs % CE == 0) && (wstr % CE == 0) && (ps % 4 == 0) && (ps * (int64_t)sizeof(T)) % 16 == 0 &&
                     (F * (int64_t)sizeof(T)) % 8 == 0 && T_ < (1 << 30) && F < (1 << 30) && d < (1 << 30) &&
-                    (!b || (((uintptr_t)b) % 8 == 0 && bs % 4 == 0));
+                    (!b || (((uintptr_t)b) % 16 == 0 && bs % 8 == 0));
   if (fast) {
     const int64_t tm = clt_ceil_div(T_, BM), tn = clt_ceil_div(F, BN);
     const int64_t nblk = tm * tn * L;
