@@ -74,22 +74,27 @@ __device__ __forceinline__ void decode_batch(float *acc, const T *wbase, int64_t
   }
 }
 
-// One wavefront per (target, token) - or per (target, token, feature slice) when SLICED.
-// The survivors of a row are taken 64 at a time into registers (one per lane) and consumed
-// U at a time, so U row fetches are in flight per wavefront.
+// One wavefront per (target, token): walks all sources s <= t, accumulates in registers,
+// writes the output row once.  Used for small batches.
 //
-// SLICED: the feature axis is cut into `ns` slices and block b works on slice b % ns.
-// Workgroups are handed to the XCDs round-robin, so with ns = 8 each XCD sees one slice of
-// every decoder matrix (1/8 of its rows) for ALL tokens: the slice stays in that XCD's L2
-// while the tokens stream past.  Each wavefront writes an fp32 partial row; k_decode_reduce
-// adds the slices in a fixed order (deterministic) and applies bias / skip / rounding.
+// SLICED (large batches): one launch per source layer `src`; one wavefront per
+// (target >= src, token, feature slice).  The feature axis is cut into `ns` slices and block b
+// works on slice b % ns.  Workgroups are handed to the XCDs round-robin, so with ns = 8 each
+// XCD sees one slice of a decoder matrix (1/8 of its rows); blocks are ordered target-major,
+// so at any moment the wavefronts resident on an XCD gather from ONE slice of ONE matrix
+// (a few MB, L2-resident) while all tokens stream past - every row is fetched from HBM once
+// and then hit ~T*k/F times in L2.  The price is that a (target, token, slice) accumulator
+// cannot stay in registers across launches: it lives as an fp32 partial row that each launch
+// reads, updates and writes back (skipped when the token has no survivor in the slice).
+// k_decode_reduce finally adds the slices in a fixed order and applies bias / skip / rounding.
 template <typename T, int NF, int TAIL, int U, bool AFFINE, bool SLICED>
 __global__ __launch_bounds__(256) void k_decode(
     const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ col, const T *__restrict__ val,
     const T *__restrict__ wp, const float *__restrict__ bias_sum, const T *__restrict__ foff,
     const T *__restrict__ fscale, const float *__restrict__ skip_add, void *__restrict__ out,
     int64_t Tn, int64_t d, int64_t F, int64_t L, int tying, int64_t t_begin, int64_t t_end,
-    uint64_t src_mask, int out_f32, const int32_t *__restrict__ sptr, float *__restrict__ partial, int ns) {
+    uint64_t src_mask, int out_f32, const int32_t *__restrict__ sptr, float *__restrict__ partial, int ns,
+    int src) {
   constexpr int V = WVec<T>::V;
   constexpr int HV = V / 2;                       // elements per 8 bytes
   constexpr int NACC = NF * V + (TAIL == 1 ? HV : TAIL == 2 ? V : 0);
@@ -97,8 +102,8 @@ __global__ __launch_bounds__(256) void k_decode(
   const int64_t blocks_per_t = (Tn + nwv - 1) / nwv;
   const int64_t bid = SLICED ? (int64_t)blockIdx.x / ns : (int64_t)blockIdx.x;
   const int slice = SLICED ? (int)(blockIdx.x % ns) : 0;
-  // heaviest targets (most sources) first
-  const int64_t t = t_end - 1 - bid / blocks_per_t;
+  // single pass: heaviest targets (most sources) first; sliced: targets in ascending order
+  const int64_t t = SLICED ? t_begin + bid / blocks_per_t : t_end - 1 - bid / blocks_per_t;
   const int64_t tok = (bid % blocks_per_t) * nwv + wv;
   if (tok >= Tn) return;
   float acc[NACC];
@@ -107,12 +112,7 @@ __global__ __launch_bounds__(256) void k_decode(
   const int64_t tail_off = TAIL == 1 ? (int64_t)NF * 64 * V + (int64_t)lane * HV : (int64_t)NF * 64 * V + (int64_t)lane * V;
   const bool tail_on = TAIL == 1 ? true : (TAIL == 2 ? tail_off < d : false);
 
-  for (int64_t s = 0; s <= t; ++s) {
-    if (!((src_mask >> s) & 1ull)) continue;
-    const int64_t r = s * Tn + tok;
-    int32_t b, e;
-    if (SLICED) { b = sptr[r * (ns + 1) + slice]; e = sptr[r * (ns + 1) + slice + 1]; }
-    else { b = row_ptr[r]; e = row_ptr[r + 1]; }
+  auto gather_rows = [&](int64_t s, int32_t b, int32_t e) {
     const T *wbase = wp + decoder_slot(tying, s, t, L) * F * d;
     for (int32_t j0 = b; j0 < e; j0 += 64) {
       const int n = (e - j0) < 64 ? (e - j0) : 64;
@@ -129,24 +129,62 @@ __global__ __launch_bounds__(256) void k_decode(
       for (; i0 + U <= n; i0 += U) decode_batch<T, NF, TAIL, U>(acc, wbase, d, my_col, my_val, i0, n, lane, tail_off, tail_on);
       for (; i0 < n; i0 += 2) decode_batch<T, NF, TAIL, 2>(acc, wbase, d, my_col, my_val, i0, n, lane, tail_off, tail_on);
     }
-  }
+  };
+
   if (SLICED) {
+    const int64_t r = (int64_t)src * Tn + tok;
+    const int32_t b = sptr[r * (ns + 1) + slice], e = sptr[r * (ns + 1) + slice + 1];
+    // the first source that feeds target t initialises the partial row, later ones update it
+    const uint64_t below = src_mask & ((1ull << src) - 1ull);
+    const bool first = below == 0;
+    if (b == e && !first) return;
     float *prow = partial + (((int64_t)slice * L + t) * Tn + tok) * d;
+    float old[NACC];
+#pragma unroll
+    for (int j = 0; j < NACC; ++j) old[j] = 0.0f;
+    if (!first) {   // requested before the gathers so that its latency hides behind them
+#pragma unroll
+      for (int c = 0; c < NF; ++c) {
+        const float *pp = prow + (int64_t)c * 64 * V + (int64_t)lane * V;
+#pragma unroll
+        for (int j = 0; j < V; j += 4) {
+          float4 q = *reinterpret_cast<const float4 *>(pp + j);
+          old[c * V + j] = q.x; old[c * V + j + 1] = q.y; old[c * V + j + 2] = q.z; old[c * V + j + 3] = q.w;
+        }
+      }
+      if (TAIL == 1) {
+#pragma unroll
+        for (int j = 0; j < HV; ++j) old[NF * V + j] = prow[tail_off + j];
+      }
+      if (TAIL == 2 && tail_on) {
+#pragma unroll
+        for (int j = 0; j < V; ++j) old[NF * V + j] = prow[tail_off + j];
+      }
+    }
+    gather_rows(src, b, e);
 #pragma unroll
     for (int c = 0; c < NF; ++c) {
       float *pp = prow + (int64_t)c * 64 * V + (int64_t)lane * V;
 #pragma unroll
-      for (int j = 0; j < V; j += 4) *reinterpret_cast<float4 *>(pp + j) = make_float4(acc[c * V + j], acc[c * V + j + 1], acc[c * V + j + 2], acc[c * V + j + 3]);
+      for (int j = 0; j < V; j += 4)
+        *reinterpret_cast<float4 *>(pp + j) = make_float4(old[c * V + j] + acc[c * V + j], old[c * V + j + 1] + acc[c * V + j + 1],
+                                                          old[c * V + j + 2] + acc[c * V + j + 2], old[c * V + j + 3] + acc[c * V + j + 3]);
     }
     if (TAIL == 1) {
 #pragma unroll
-      for (int j = 0; j < HV; ++j) prow[tail_off + j] = acc[NF * V + j];
+      for (int j = 0; j < HV; ++j) prow[tail_off + j] = old[NF * V + j] + acc[NF * V + j];
     }
     if (TAIL == 2 && tail_on) {
 #pragma unroll
-      for (int j = 0; j < V; ++j) prow[tail_off + j] = acc[NF * V + j];
+      for (int j = 0; j < V; ++j) prow[tail_off + j] = old[NF * V + j] + acc[NF * V + j];
     }
     return;
+  }
+
+  for (int64_t s = 0; s <= t; ++s) {
+    if (!((src_mask >> s) & 1ull)) continue;
+    const int64_t r = s * Tn + tok;
+    gather_rows(s, row_ptr[r], row_ptr[r + 1]);
   }
   // epilogue: bias, skip term, one write of the output row
   auto emit = [&](int64_t o, const float *a, int cnt, bool on) {
@@ -185,16 +223,19 @@ __global__ void k_slice_ptr(const int32_t *row_ptr, const int32_t *col, int64_t 
 template <typename T>
 __global__ void k_decode_reduce(const float *__restrict__ partial, const float *__restrict__ bias_sum,
                                 const float *__restrict__ skip_add, void *__restrict__ out, int64_t Tn, int64_t d,
-                                int64_t L, int64_t t_begin, int64_t t_end, int ns, int out_f32) {
+                                int64_t L, int64_t t_begin, int64_t t_end, int ns, int out_f32, uint64_t src_mask) {
   const int64_t per_t = Tn * d, span = (t_end - t_begin) * per_t, slice_stride = L * per_t;
   for (int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4; i < span; i += (int64_t)gridDim.x * blockDim.x * 4) {
     const int64_t g = t_begin * per_t + i;          // index into [L][T][d]
-    float4 a = *reinterpret_cast<const float4 *>(partial + g);
-    for (int sl = 1; sl < ns; ++sl) {
-      float4 b = *reinterpret_cast<const float4 *>(partial + sl * slice_stride + g);
-      a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
-    }
     const int64_t t = g / per_t, o = g % d;
+    float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (src_mask & ((2ull << t) - 1ull)) {            // some source <= t wrote partial rows
+      a = *reinterpret_cast<const float4 *>(partial + g);
+      for (int sl = 1; sl < ns; ++sl) {
+        float4 b = *reinterpret_cast<const float4 *>(partial + sl * slice_stride + g);
+        a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+      }
+    }
     if (bias_sum) { a.x += bias_sum[t * d + o]; a.y += bias_sum[t * d + o + 1]; a.z += bias_sum[t * d + o + 2]; a.w += bias_sum[t * d + o + 3]; }
     if (skip_add) { float4 k = *reinterpret_cast<const float4 *>(skip_add + g); a.x += k.x; a.y += k.y; a.z += k.z; a.w += k.w; }
     if (out_f32) *reinterpret_cast<float4 *>((float *)out + g) = a;
@@ -338,7 +379,7 @@ static int launch_decode(const int32_t *row_ptr, const int32_t *col, const void 
     partial = (float *)workspace;
     sptr = (int32_t *)((char *)workspace + (((size_t)DEC_SLICES * L * Tn * d * 4 + 255) & ~(size_t)255));
   }
-  const int64_t nblk = blocks_per_t * (t_end - t_begin) * ns;
+  int64_t nblk = blocks_per_t * (t_end - t_begin);
   if (nblk <= 0) return CLT_OK;
   if (nblk > 2147483647LL) return CLT_ERR_RANGE;
   const bool affine = foff || fscale;
@@ -349,8 +390,8 @@ static int launch_decode(const int32_t *row_ptr, const int32_t *col, const void 
                                                   L, tying, t_begin, t_end, src_mask, out_f32, nullptr, 0, stream);
   if (can_slice) k_slice_ptr<<<1024, 256, 0, stream>>>(row_ptr, col, L * Tn, F, ns, sptr);
 #define CLT_DEC_ARGS(FO, FS)                                                                                    \
-  row_ptr, col, (const T *)val, (const T *)wp, bias_sum, FO, FS, skip_add, out, Tn, d, F, L, tying, t_begin,    \
-      t_end, src_mask, out_f32, sptr, partial, ns
+  row_ptr, col, (const T *)val, (const T *)wp, bias_sum, FO, FS, skip_add, out, Tn, d, F, L, tying, tb,         \
+      t_end, src_mask, out_f32, sptr, partial, ns, src
 #define CLT_DEC(NFN, TL, UN)                                                                                    \
   do {                                                                                                          \
     if (affine && can_slice)                                                                                    \
@@ -369,13 +410,26 @@ static int launch_decode(const int32_t *row_ptr, const int32_t *col, const void 
     else CLT_DEC(NFN, 2, UN);                              \
   } while (0)
   if (fast) {
-    if (nf == 0) CLT_DEC(0, 2, 8);
-    else if (nf == 1) CLT_DEC_TAIL(1, 8);
-    else if (nf == 2) CLT_DEC_TAIL(2, 6);
-    else if (nf == 3) CLT_DEC_TAIL(3, 4);
-    else if (rem == 0) CLT_DEC(4, 0, 4);
-    else CLT_DEC(4, 2, 3);
+    // sliced: one launch per source layer, targets max(src, t_begin) .. t_end-1
+    const int n_launch = can_slice ? (int)t_end : 1;
+    for (int src = 0; src < n_launch; ++src) {
+      int64_t tb = t_begin;
+      if (can_slice) {
+        if (!((src_mask >> src) & 1ull)) continue;
+        if (src > tb) tb = src;
+        nblk = blocks_per_t * (t_end - tb) * ns;
+        if (nblk <= 0) continue;
+        if (nblk > 2147483647LL) return CLT_ERR_RANGE;
+      }
+      if (nf == 0) CLT_DEC(0, 2, 8);
+      else if (nf == 1) CLT_DEC_TAIL(1, 8);
+      else if (nf == 2) CLT_DEC_TAIL(2, 6);
+      else if (nf == 3) CLT_DEC_TAIL(3, 4);
+      else if (rem == 0) CLT_DEC(4, 0, 4);
+      else CLT_DEC(4, 2, 3);
+    }
   } else {
+    const int64_t tb = t_begin; const int src = 0; (void)tb; (void)src;
     k_decode_generic<T><<<(unsigned)nblk, 256, 0, stream>>>(row_ptr, col, (const T *)val, (const T *)wp, bias_sum,
         (const T *)foff, (const T *)fscale, skip_add, out, Tn, d, F, L, tying, t_begin, t_end, src_mask, out_f32);
   }
@@ -383,7 +437,7 @@ static int launch_decode(const int32_t *row_ptr, const int32_t *col, const void 
 #undef CLT_DEC
 #undef CLT_DEC_ARGS
   if (can_slice)
-    k_decode_reduce<T><<<2048, 256, 0, stream>>>(partial, bias_sum, skip_add, out, Tn, d, L, t_begin, t_end, ns, out_f32);
+    k_decode_reduce<T><<<2048, 256, 0, stream>>>(partial, bias_sum, skip_add, out, Tn, d, L, t_begin, t_end, ns, out_f32, src_mask);
   return clt_check_launch();
 }
 
