@@ -24,8 +24,25 @@ template <> struct WVec<float> {
     acc[0] = fmaf(v, __uint_as_float(w.x), acc[0]); acc[1] = fmaf(v, __uint_as_float(w.y), acc[1]);
   }
 };
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+
 template <> struct WVec<bf16_t> {
   static constexpr int V = 8;
+  // Two survivors at once: for each pair of bf16 weights in a 32-bit word, a byte permute puts
+  // the same element of both rows side by side and v_dot2c_f32_bf16 multiplies them with the two
+  // activation values (bf16 pair `vv`) and accumulates in fp32 - one op per element instead of two.
+  __device__ static __forceinline__ void dot32(float *acc, uint32_t a, uint32_t b, bf16x2_t vv) {
+    const uint32_t lo = __builtin_amdgcn_perm(b, a, 0x05040100u);   // (a.lo16, b.lo16)
+    const uint32_t hi = __builtin_amdgcn_perm(b, a, 0x07060302u);   // (a.hi16, b.hi16)
+    acc[0] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, lo), vv, acc[0], false);
+    acc[1] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, hi), vv, acc[1], false);
+  }
+  __device__ static __forceinline__ void dot16(float *acc, const uint4 &a, const uint4 &b, bf16x2_t vv) {
+    dot32(acc, a.x, b.x, vv); dot32(acc + 2, a.y, b.y, vv); dot32(acc + 4, a.z, b.z, vv); dot32(acc + 6, a.w, b.w, vv);
+  }
+  __device__ static __forceinline__ void dot8(float *acc, const uint2 &a, const uint2 &b, bf16x2_t vv) {
+    dot32(acc, a.x, b.x, vv); dot32(acc + 2, a.y, b.y, vv);
+  }
   __device__ static __forceinline__ void fma32(float *acc, uint32_t u, float v) {
     acc[0] = fmaf(v, __uint_as_float(u << 16), acc[0]);
     acc[1] = fmaf(v, __uint_as_float(u & 0xFFFF0000u), acc[1]);
@@ -44,35 +61,83 @@ __device__ __forceinline__ int64_t decoder_slot(int tying, int64_t s, int64_t t,
   return s * L - (s * (s - 1)) / 2 + (t - s);
 }
 
-// Fetch UU decoder vectors (all requests issued before the first multiply) and accumulate.
-template <typename T, int NF, int TAIL, int UU>
-__device__ __forceinline__ void decode_batch(float *acc, const T *wbase, int64_t d, int32_t my_col, float my_val,
-                                             int i0, int n, int lane, int64_t tail_off, bool tail_on) {
-  constexpr int V = WVec<T>::V;
+// UU decoder vectors in flight: the row pieces of one lane plus the (wave-uniform) weights.
+template <typename T, int NF, int TAIL, int UU> struct RowBatch {
   uint4 wq[UU][NF > 0 ? NF : 1];
   uint4 wt16[UU];
   uint2 wt8[UU];
   float v[UU];
+
+  // request rows i0 .. i0+UU-1 of the 64 survivors held one per lane in (my_col, my_val)
+  __device__ __forceinline__ void load(const T *wbase, int64_t d, int32_t my_col, float my_val, int i0, int n,
+                                       int lane, int64_t tail_off, bool tail_on) {
+    constexpr int V = WVec<T>::V;
 #pragma unroll
-  for (int u = 0; u < UU; ++u) {
-    const int idx = (i0 + u) < n ? (i0 + u) : (n - 1);   // clamp: a repeated fetch, weight 0
-    const int32_t f = __builtin_amdgcn_readlane(my_col, idx);
-    const float vv = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(my_val), idx));
-    v[u] = (i0 + u) < n ? vv : 0.0f;
-    const T *wrow = wbase + (int64_t)f * d;
+    for (int u = 0; u < UU; ++u) {
+      const int idx = (i0 + u) < n ? (i0 + u) : (n - 1);   // clamp: a repeated fetch, weight 0
+      const int32_t f = __builtin_amdgcn_readlane(my_col, idx);
+      const float vv = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(my_val), idx));
+      v[u] = (i0 + u) < n ? vv : 0.0f;
+      const T *wrow = wbase + (int64_t)f * d;
 #pragma unroll
-    for (int c = 0; c < NF; ++c) wq[u][c] = *reinterpret_cast<const uint4 *>(wrow + (int64_t)c * 64 * V + (int64_t)lane * V);
-    if (TAIL == 1) wt8[u] = *reinterpret_cast<const uint2 *>(wrow + tail_off);
-    if (TAIL == 2) wt16[u] = tail_on ? *reinterpret_cast<const uint4 *>(wrow + tail_off) : make_uint4(0, 0, 0, 0);
+      for (int c = 0; c < NF; ++c) wq[u][c] = *reinterpret_cast<const uint4 *>(wrow + (int64_t)c * 64 * V + (int64_t)lane * V);
+      if (TAIL == 1) wt8[u] = *reinterpret_cast<const uint2 *>(wrow + tail_off);
+      if (TAIL == 2) wt16[u] = tail_on ? *reinterpret_cast<const uint4 *>(wrow + tail_off) : make_uint4(0, 0, 0, 0);
+    }
   }
+
+  __device__ __forceinline__ void consume(float *acc) const {
+    constexpr int V = WVec<T>::V;
+    if constexpr (sizeof(T) == 2 && (UU % 2) == 0) {
+      // bf16: the activation values are exact bf16 numbers, so two of them fit one dot2 operand
 #pragma unroll
-  for (int u = 0; u < UU; ++u) {
+      for (int u = 0; u < UU; u += 2) {
+        const uint32_t vb = (__float_as_uint(v[u]) >> 16) | (__float_as_uint(v[u + 1]) & 0xFFFF0000u);
+        const bf16x2_t vv = __builtin_bit_cast(bf16x2_t, vb);
 #pragma unroll
-    for (int c = 0; c < NF; ++c) WVec<T>::fma16(acc + c * V, wq[u][c], v[u]);
-    if (TAIL == 1) WVec<T>::fma8(acc + NF * V, wt8[u], v[u]);
-    if (TAIL == 2) WVec<T>::fma16(acc + NF * V, wt16[u], v[u]);
+        for (int c = 0; c < NF; ++c) WVec<T>::dot16(acc + c * V, wq[u][c], wq[u + 1][c], vv);
+        if (TAIL == 1) WVec<T>::dot8(acc + NF * V, wt8[u], wt8[u + 1], vv);
+        if (TAIL == 2) WVec<T>::dot16(acc + NF * V, wt16[u], wt16[u + 1], vv);
+      }
+    } else {
+#pragma unroll
+      for (int u = 0; u < UU; ++u) {
+#pragma unroll
+        for (int c = 0; c < NF; ++c) WVec<T>::fma16(acc + c * V, wq[u][c], v[u]);
+        if (TAIL == 1) WVec<T>::fma8(acc + NF * V, wt8[u], v[u]);
+        if (TAIL == 2) WVec<T>::fma16(acc + NF * V, wt16[u], v[u]);
+      }
+    }
+  }
+};
+
+// Fetch UU decoder vectors (all requests issued before the first multiply) and accumulate.
+template <typename T, int NF, int TAIL, int UU>
+__device__ __forceinline__ void decode_batch(float *acc, const T *wbase, int64_t d, int32_t my_col, float my_val,
+                                             int i0, int n, int lane, int64_t tail_off, bool tail_on) {
+  RowBatch<T, NF, TAIL, UU> rb;
+  rb.load(wbase, d, my_col, my_val, i0, n, lane, tail_off, tail_on);
+  rb.consume(acc);
+}
+
+// Up to 64 survivors (one per lane) with two batches in flight: while one batch is multiplied
+// the next one is already on its way.
+template <typename T, int NF, int TAIL, int UU>
+__device__ __forceinline__ void decode_chunk_pipelined(float *acc, const T *wbase, int64_t d, int32_t my_col,
+                                                       float my_val, int n, int lane, int64_t tail_off, bool tail_on) {
+  RowBatch<T, NF, TAIL, UU> ra, rb;
+  ra.load(wbase, d, my_col, my_val, 0, n, lane, tail_off, tail_on);
+  for (int i0 = 0; i0 < n; i0 += 2 * UU) {
+    if (i0 + UU < n) rb.load(wbase, d, my_col, my_val, i0 + UU, n, lane, tail_off, tail_on);
+    ra.consume(acc);
+    if (i0 + UU < n) {
+      if (i0 + 2 * UU < n) ra.load(wbase, d, my_col, my_val, i0 + 2 * UU, n, lane, tail_off, tail_on);
+      rb.consume(acc);
+    }
   }
 }
+
+constexpr int SLICED_NTOK = 4;   // tokens per wavefront in the sliced kernel
 
 // One wavefront per (target, token): walks all sources s <= t, accumulates in registers,
 // writes the output row once.  Used for small batches.
@@ -99,13 +164,14 @@ __global__ __launch_bounds__(256) void k_decode(
   constexpr int HV = V / 2;                       // elements per 8 bytes
   constexpr int NACC = NF * V + (TAIL == 1 ? HV : TAIL == 2 ? V : 0);
   const int lane = lane_id(), wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
-  const int64_t blocks_per_t = (Tn + nwv - 1) / nwv;
+  const int64_t tok_per_blk = SLICED ? (int64_t)nwv * SLICED_NTOK : (int64_t)nwv;
+  const int64_t blocks_per_t = (Tn + tok_per_blk - 1) / tok_per_blk;
   const int64_t bid = SLICED ? (int64_t)blockIdx.x / ns : (int64_t)blockIdx.x;
   const int slice = SLICED ? (int)(blockIdx.x % ns) : 0;
   // single pass: heaviest targets (most sources) first; sliced: targets in ascending order
   const int64_t t = SLICED ? t_begin + bid / blocks_per_t : t_end - 1 - bid / blocks_per_t;
   const int64_t tok = (bid % blocks_per_t) * nwv + wv;
-  if (tok >= Tn) return;
+  if (!SLICED && tok >= Tn) return;
   float acc[NACC];
 #pragma unroll
   for (int j = 0; j < NACC; ++j) acc[j] = 0.0f;
@@ -132,51 +198,86 @@ __global__ __launch_bounds__(256) void k_decode(
   };
 
   if (SLICED) {
-    const int64_t r = (int64_t)src * Tn + tok;
-    const int32_t b = sptr[r * (ns + 1) + slice], e = sptr[r * (ns + 1) + slice + 1];
-    // the first source that feeds target t initialises the partial row, later ones update it
+    // this wavefront: tokens tok*NTOK .. +NTOK-1 of source `src`, slice `slice`, target t.
+    // Their slice bounds are fetched at once (one lane per token), and the survivor list of the
+    // next token is requested before the current token's rows are gathered.
+    const int64_t tok0 = tok * SLICED_NTOK;
+    if (tok0 >= Tn) return;
     const uint64_t below = src_mask & ((1ull << src) - 1ull);
-    const bool first = below == 0;
-    if (b == e && !first) return;
-    float *prow = partial + (((int64_t)slice * L + t) * Tn + tok) * d;
-    float old[NACC];
+    const bool first = below == 0;   // the first source initialises the partial rows
+    int32_t mb = 0, me = 0;
+    if (lane < SLICED_NTOK && tok0 + lane < Tn) {
+      const int64_t r = (int64_t)src * Tn + tok0 + lane;
+      mb = sptr[r * (ns + 1) + slice];
+      me = sptr[r * (ns + 1) + slice + 1];
+    }
+    const T *wbase = wp + decoder_slot(tying, src, t, L) * F * d;
+    int32_t nb = __builtin_amdgcn_readlane(mb, 0), ne = __builtin_amdgcn_readlane(me, 0);
+    int32_t nxt_col = 0; T nxt_val = T(0);
+    if (lane < ne - nb) { nxt_col = col[nb + lane]; nxt_val = val[nb + lane]; }
 #pragma unroll
-    for (int j = 0; j < NACC; ++j) old[j] = 0.0f;
-    if (!first) {   // requested before the gathers so that its latency hides behind them
+    for (int i = 0; i < SLICED_NTOK; ++i) {
+      const int32_t b = nb, e = ne;
+      const int32_t cur_col = nxt_col; const T cur_val = nxt_val;
+      if (i + 1 < SLICED_NTOK) {
+        nb = __builtin_amdgcn_readlane(mb, i + 1); ne = __builtin_amdgcn_readlane(me, i + 1);
+        nxt_col = 0; nxt_val = T(0);
+        if (lane < ne - nb) { nxt_col = col[nb + lane]; nxt_val = val[nb + lane]; }
+      }
+      if (tok0 + i >= Tn) break;
+      if (b == e && !first) continue;
+      float *prow = partial + (((int64_t)slice * L + t) * Tn + tok0 + i) * d;
+      float old[NACC];
+#pragma unroll
+      for (int j = 0; j < NACC; ++j) { old[j] = 0.0f; acc[j] = 0.0f; }
+      if (!first) {   // requested before the gathers so that its latency hides behind them
+#pragma unroll
+        for (int c = 0; c < NF; ++c) {
+          const float *pp = prow + (int64_t)c * 64 * V + (int64_t)lane * V;
+#pragma unroll
+          for (int j = 0; j < V; j += 4) {
+            float4 q = *reinterpret_cast<const float4 *>(pp + j);
+            old[c * V + j] = q.x; old[c * V + j + 1] = q.y; old[c * V + j + 2] = q.z; old[c * V + j + 3] = q.w;
+          }
+        }
+        if (TAIL == 1) {
+#pragma unroll
+          for (int j = 0; j < HV; ++j) old[NF * V + j] = prow[tail_off + j];
+        }
+        if (TAIL == 2 && tail_on) {
+#pragma unroll
+          for (int j = 0; j < V; ++j) old[NF * V + j] = prow[tail_off + j];
+        }
+      }
+      for (int32_t j0 = b; j0 < e; j0 += 64) {
+        const int n = (e - j0) < 64 ? (e - j0) : 64;
+        int32_t my_col = cur_col; float my_val = Elem<T>::to_f32(cur_val);
+        if (j0 > b) {   // more than 64 survivors in this slice: fetch the next 64
+          my_col = 0; my_val = 0.0f;
+          if (lane < n) { my_col = col[j0 + lane]; my_val = Elem<T>::to_f32(val[j0 + lane]); }
+        }
+        if (AFFINE && my_val != 0.0f) {
+          if (foff) my_val = Elem<T>::round(my_val + Elem<T>::to_f32(foff[t * F + my_col]));
+          if (fscale) my_val = Elem<T>::round(my_val * Elem<T>::to_f32(fscale[t * F + my_col]));
+        }
+        decode_chunk_pipelined<T, NF, TAIL, (U > 6 ? 6 : U)>(acc, wbase, d, my_col, my_val, n, lane, tail_off, tail_on);
+      }
 #pragma unroll
       for (int c = 0; c < NF; ++c) {
-        const float *pp = prow + (int64_t)c * 64 * V + (int64_t)lane * V;
+        float *pp = prow + (int64_t)c * 64 * V + (int64_t)lane * V;
 #pragma unroll
-        for (int j = 0; j < V; j += 4) {
-          float4 q = *reinterpret_cast<const float4 *>(pp + j);
-          old[c * V + j] = q.x; old[c * V + j + 1] = q.y; old[c * V + j + 2] = q.z; old[c * V + j + 3] = q.w;
-        }
+        for (int j = 0; j < V; j += 4)
+          *reinterpret_cast<float4 *>(pp + j) = make_float4(old[c * V + j] + acc[c * V + j], old[c * V + j + 1] + acc[c * V + j + 1],
+                                                            old[c * V + j + 2] + acc[c * V + j + 2], old[c * V + j + 3] + acc[c * V + j + 3]);
       }
       if (TAIL == 1) {
 #pragma unroll
-        for (int j = 0; j < HV; ++j) old[NF * V + j] = prow[tail_off + j];
+        for (int j = 0; j < HV; ++j) prow[tail_off + j] = old[NF * V + j] + acc[NF * V + j];
       }
       if (TAIL == 2 && tail_on) {
 #pragma unroll
-        for (int j = 0; j < V; ++j) old[NF * V + j] = prow[tail_off + j];
+        for (int j = 0; j < V; ++j) prow[tail_off + j] = old[NF * V + j] + acc[NF * V + j];
       }
-    }
-    gather_rows(src, b, e);
-#pragma unroll
-    for (int c = 0; c < NF; ++c) {
-      float *pp = prow + (int64_t)c * 64 * V + (int64_t)lane * V;
-#pragma unroll
-      for (int j = 0; j < V; j += 4)
-        *reinterpret_cast<float4 *>(pp + j) = make_float4(old[c * V + j] + acc[c * V + j], old[c * V + j + 1] + acc[c * V + j + 1],
-                                                          old[c * V + j + 2] + acc[c * V + j + 2], old[c * V + j + 3] + acc[c * V + j + 3]);
-    }
-    if (TAIL == 1) {
-#pragma unroll
-      for (int j = 0; j < HV; ++j) prow[tail_off + j] = old[NF * V + j] + acc[NF * V + j];
-    }
-    if (TAIL == 2 && tail_on) {
-#pragma unroll
-      for (int j = 0; j < V; ++j) prow[tail_off + j] = old[NF * V + j] + acc[NF * V + j];
     }
     return;
   }
@@ -417,7 +518,7 @@ static int launch_decode(const int32_t *row_ptr, const int32_t *col, const void 
       if (can_slice) {
         if (!((src_mask >> src) & 1ull)) continue;
         if (src > tb) tb = src;
-        nblk = blocks_per_t * (t_end - tb) * ns;
+        nblk = clt_ceil_div(Tn, nwv * SLICED_NTOK) * (t_end - tb) * ns;
         if (nblk <= 0) continue;
         if (nblk > 2147483647LL) return CLT_ERR_RANGE;
       }
@@ -426,7 +527,7 @@ static int launch_decode(const int32_t *row_ptr, const int32_t *col, const void 
       else if (nf == 2) CLT_DEC_TAIL(2, 6);
       else if (nf == 3) CLT_DEC_TAIL(3, 4);
       else if (rem == 0) CLT_DEC(4, 0, 4);
-      else CLT_DEC(4, 2, 3);
+      else CLT_DEC(4, 2, 2);
     }
   } else {
     const int64_t tb = t_begin; const int src = 0; (void)tb; (void)src;
