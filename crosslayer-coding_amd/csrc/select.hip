@@ -721,6 +721,171 @@ __global__ __launch_bounds__(256) void k_threshold(
   }
 }
 
+// ---- TokenTopK ------------------------------------------------------------------------
+// Row-wise top-k (reference clt/models/activations.py:99-128, 391-491).  A "problem" is one
+// token row: F entries of one layer (per-layer mode) or the L*F entries of all layers ranked
+// on the z-score (global mode).  One block per problem finds the kk-th largest key by MSD
+// radix select over the row (11-bit digits, LDS histogram), then counts per (layer, token)
+// row how many entries beat the threshold and hands the tie budget out in column order
+// (layers in ascending order in global mode).  A second kernel writes the survivors in order.
+template <typename T, bool GLOBAL>
+__global__ __launch_bounds__(SCAN_THREADS) void k_token_threshold(
+    const T *pre, int64_t Tn, int64_t F, int64_t L, int64_t lstride, const float *mean,
+    const float *denom, unsigned long long kk, uint32_t *thr_key, uint32_t *allot, uint32_t *keep) {
+  constexpr int KB = Elem<T>::KEYBITS;
+  constexpr int NLEV = KB == 32 ? 3 : 2;
+  __shared__ uint32_t lh[NBINS];
+  __shared__ uint32_t cnt_gt[64], cnt_eq[64];
+  const int tid = threadIdx.x;
+  // per-layer: problem = (layer, token); global: problem = token
+  const int64_t prob = blockIdx.x;
+  const int64_t l0 = GLOBAL ? 0 : prob / Tn, t = GLOBAL ? prob : prob - l0 * Tn;
+  const int nl = GLOBAL ? (int)L : 1;
+  const int shifts[3] = {KB == 32 ? 21 : 5, KB == 32 ? 10 : 0, 0};
+  const int widths[3] = {11, KB == 32 ? 11 : 5, 10};
+  uint32_t prefix = 0, prefix_mask = 0;
+  unsigned long long k_rem = kk;
+  for (int lev = 0; lev < NLEV; ++lev) {
+    for (int i = tid; i < NBINS; i += SCAN_THREADS) lh[i] = 0;
+    __syncthreads();
+    const int sh = shifts[lev];
+    const uint32_t dm = (1u << widths[lev]) - 1u;
+    for (int li = 0; li < nl; ++li) {
+      const int64_t l = l0 + li;
+      const T *row = pre + l * lstride + t * F;
+      typename RankOf<T, GLOBAL>::type rk = RankOf<T, GLOBAL>::make(mean, denom, l, F);
+      for (int64_t f = tid; f < F; f += SCAN_THREADS) {
+        const uint32_t key = rank_key<KB>(rk(Elem<T>::to_f32(row[f]), f));
+        if ((key & prefix_mask) == prefix) atomicAdd(&lh[(key >> sh) & dm], 1u);
+      }
+    }
+    __syncthreads();
+    int bin; unsigned long long above, total;
+    block_find_from_top(lh, (int)dm + 1, k_rem, bin, above, total);
+    if (bin < 0) bin = 0;   // kk <= row length, so the bin exists
+    k_rem -= above;
+    prefix |= (uint32_t)bin << sh;
+    prefix_mask |= dm << sh;
+  }
+  const uint32_t thr = prefix;          // key of the kk-th largest entry; k_rem ties survive
+  if (tid < 64) { cnt_gt[tid] = 0; cnt_eq[tid] = 0; }
+  __syncthreads();
+  for (int li = 0; li < nl; ++li) {
+    const int64_t l = l0 + li;
+    const T *row = pre + l * lstride + t * F;
+    typename RankOf<T, GLOBAL>::type rk = RankOf<T, GLOBAL>::make(mean, denom, l, F);
+    uint32_t g = 0, e = 0;
+    for (int64_t f = tid; f < F; f += SCAN_THREADS) {
+      const uint32_t key = rank_key<KB>(rk(Elem<T>::to_f32(row[f]), f));
+      g += key > thr; e += key == thr;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) { g += __shfl_xor(g, o); e += __shfl_xor(e, o); }
+    if ((tid & 63) == 0) { atomicAdd(&cnt_gt[li], g); atomicAdd(&cnt_eq[li], e); }
+  }
+  __syncthreads();
+  if (tid == 0) {
+    thr_key[prob] = thr;
+    unsigned long long budget = k_rem;
+    for (int li = 0; li < nl; ++li) {
+      const int64_t r = (l0 + li) * Tn + t;
+      const unsigned long long a = budget < cnt_eq[li] ? budget : cnt_eq[li];
+      budget -= a;
+      allot[r] = (uint32_t)a;
+      keep[r] = cnt_gt[li] + (uint32_t)a;
+    }
+  }
+}
+
+// One wavefront per (layer, token) row: survivors in ascending column order.
+template <typename T, int V, bool GLOBAL>
+__global__ __launch_bounds__(256) void k_token_emit(
+    const T *pre, int64_t Tn, int64_t F, int64_t L, int64_t lstride, const float *mean,
+    const float *denom, const uint32_t *thr_key, const uint32_t *allot, const int32_t *row_ptr,
+    int32_t *col_out, T *val_out) {
+  constexpr int KB = Elem<T>::KEYBITS;
+  const int l = blockIdx.y;
+  const int lane = lane_id(), wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
+  typename RankOf<T, GLOBAL>::type rk = RankOf<T, GLOBAL>::make(mean, denom, l, F);
+  for (int64_t t = (int64_t)blockIdx.x * nwv + wv; t < Tn; t += (int64_t)gridDim.x * nwv) {
+    const int64_t r = (int64_t)l * Tn + t;
+    const uint32_t thr = thr_key[GLOBAL ? t : r];
+    const uint32_t my_allot = allot[r];
+    const int64_t base = row_ptr[r];
+    const T *row = pre + l * lstride + t * F;
+    uint32_t kept = 0, ties = 0;
+    for (int64_t c0 = 0; c0 < F; c0 += 64 * V) {
+      const int64_t col = c0 + (int64_t)lane * V;
+      float x[V]; uint32_t raw[V];
+      uint32_t mg = 0, me = 0;
+      if (col < F) {
+        VecLoad<T, V>::load(row + col, x, raw);
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+          const uint32_t key = rank_key<KB>(rk(x[j], col + j));
+          if (key > thr) mg |= 1u << j;
+          if (key == thr) me |= 1u << j;
+        }
+      }
+      if (ballot64((mg | me) != 0) == 0) continue;
+      // ties first: their rank in column order decides which of them survive
+      uint32_t te, pe = wave_mask_prefix<V>(me, te);
+      uint32_t mk = mg;
+#pragma unroll
+      for (int j = 0; j < V; ++j)
+        if ((me >> j) & 1u) {
+          const uint32_t rank = ties + pe + __popc(me & ((1u << j) - 1u));
+          if (rank < my_allot) mk |= 1u << j;
+        }
+      ties += te;
+      uint32_t tk, pk = wave_mask_prefix<V>(mk, tk);
+#pragma unroll
+      for (int j = 0; j < V; ++j)
+        if ((mk >> j) & 1u) {
+          const int64_t pos = base + kept + pk + __popc(mk & ((1u << j) - 1u));
+          col_out[pos] = (int32_t)(col + j);
+          val_out[pos] = Elem<T>::from_raw(raw[j]);
+        }
+      kept += tk;
+    }
+  }
+}
+
+struct TokLayout { size_t off_thr, off_allot, off_keep, total; };
+static TokLayout tok_layout(int64_t T, int64_t L) {
+  TokLayout lo; size_t o = 0;
+  auto take = [&](size_t bytes) { size_t at = o; o += (bytes + 255) & ~(size_t)255; return at; };
+  lo.off_thr = take(4 * (size_t)(L * T));
+  lo.off_allot = take(4 * (size_t)(L * T));
+  lo.off_keep = take(4 * (size_t)(L * T));
+  lo.total = o;
+  return lo;
+}
+
+template <typename T, bool GLOBAL>
+static int run_tokentopk(const T *pre, int64_t Tn, int64_t F, int64_t L, int64_t lstride, int64_t kk,
+                         const float *mean, const float *denom, int32_t *row_ptr, int32_t *col, T *val,
+                         char *ws, hipStream_t stream) {
+  constexpr int VV = Elem<T>::VEC;
+  const TokLayout lo = tok_layout(Tn, L);
+  uint32_t *thr = (uint32_t *)(ws + lo.off_thr), *allot = (uint32_t *)(ws + lo.off_allot);
+  uint32_t *keep = (uint32_t *)(ws + lo.off_keep);
+  const int64_t nprob = GLOBAL ? Tn : L * Tn;
+  if (nprob > 2147483647LL) return CLT_ERR_RANGE;
+  k_token_threshold<T, GLOBAL><<<(unsigned)nprob, SCAN_THREADS, 0, stream>>>(pre, Tn, F, L, lstride, mean, denom,
+                                                                           (unsigned long long)kk, thr, allot, keep);
+  k_rowptr_scan<<<1, SCAN_THREADS, 0, stream>>>(keep, L * Tn, row_ptr);
+  int gx = (int)clt_ceil_div(Tn, 4);
+  int maxgx = (int)clt_ceil_div(256 * 8, L);
+  if (maxgx < 1) maxgx = 1;
+  if (gx > maxgx) gx = maxgx;
+  dim3 grid(gx, (unsigned)L);
+  const bool vec = (F % VV == 0) && clt_aligned16(pre) && ((lstride * (int64_t)sizeof(T)) % 16 == 0);
+  if (vec) k_token_emit<T, VV, GLOBAL><<<grid, 256, 0, stream>>>(pre, Tn, F, L, lstride, mean, denom, thr, allot, row_ptr, col, val);
+  else k_token_emit<T, 1, GLOBAL><<<grid, 256, 0, stream>>>(pre, Tn, F, L, lstride, mean, denom, thr, allot, row_ptr, col, val);
+  return clt_check_launch();
+}
+
 // ---- host side ------------------------------------------------------------------------
 struct SelLayout {
   size_t off_state, off_hist, off_poolcnt, off_sample, off_first, off_gt, off_eq, off_allot, off_keep, off_pool, total;
@@ -919,4 +1084,40 @@ extern "C" int clt_threshold_emit(const void *pre, int64_t T, int64_t F, int64_t
   hipStream_t s = (hipStream_t)stream;
   if (dtype == CLT_BF16) return dispatch_threshold<bf16_t>(true, pre, T, F, L, pre_layer_stride, theta, pred, nullptr, (int32_t *)row_ptr, col, val, s);
   return dispatch_threshold<float>(true, pre, T, F, L, pre_layer_stride, theta, pred, nullptr, (int32_t *)row_ptr, col, val, s);
+}
+
+extern "C" size_t clt_tokentopk_workspace_bytes(int64_t T, int64_t F, int64_t L, int64_t kk, int mode, int dtype) {
+  (void)F; (void)kk; (void)mode; (void)dtype;
+  if (T <= 0 || L <= 0) return 256;
+  return tok_layout(T, L).total;
+}
+
+extern "C" int clt_tokentopk_select(const void *pre, int64_t T, int64_t F, int64_t L, int64_t pre_layer_stride,
+                                    int64_t kk, int mode, const float *mean, const float *denom, int dtype,
+                                    int32_t *row_ptr, int32_t *col, void *val, void *workspace,
+                                    size_t workspace_bytes, void *stream) {
+  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (T < 0 || F < 0 || L <= 0 || L > 64 || !row_ptr) return CLT_ERR_ARG;
+  if (mode != CLT_TOPK_PER_LAYER && mode != CLT_TOPK_GLOBAL) return CLT_ERR_ARG;
+  hipStream_t s = (hipStream_t)stream;
+  const int64_t R = L * T;
+  if (kk <= 0 || T == 0 || F == 0) {
+    k_fill_u32<<<64, 256, 0, s>>>((uint32_t *)row_ptr, 0u, R + 1);
+    return clt_check_launch();
+  }
+  if (!pre || !col || !val || !workspace) return CLT_ERR_ARG;
+  if (mode == CLT_TOPK_GLOBAL && (!mean || !denom)) return CLT_ERR_ARG;
+  if ((double)T * (double)F * (double)L >= 2147483648.0) return CLT_ERR_RANGE;
+  if (workspace_bytes < clt_tokentopk_workspace_bytes(T, F, L, kk, mode, dtype)) return CLT_ERR_WORKSPACE;
+  const int64_t rowlen = mode == CLT_TOPK_GLOBAL ? L * F : F;
+  if (kk > rowlen) kk = rowlen;
+  char *ws = (char *)workspace;
+  if (dtype == CLT_BF16) {
+    if (mode == CLT_TOPK_GLOBAL)
+      return run_tokentopk<bf16_t, true>((const bf16_t *)pre, T, F, L, pre_layer_stride, kk, mean, denom, row_ptr, col, (bf16_t *)val, ws, s);
+    return run_tokentopk<bf16_t, false>((const bf16_t *)pre, T, F, L, pre_layer_stride, kk, mean, denom, row_ptr, col, (bf16_t *)val, ws, s);
+  }
+  if (mode == CLT_TOPK_GLOBAL)
+    return run_tokentopk<float, true>((const float *)pre, T, F, L, pre_layer_stride, kk, mean, denom, row_ptr, col, (float *)val, ws, s);
+  return run_tokentopk<float, false>((const float *)pre, T, F, L, pre_layer_stride, kk, mean, denom, row_ptr, col, (float *)val, ws, s);
 }

@@ -202,6 +202,68 @@ def test_batchtopk_global_closed_form(dev):
     assert torch.equal(got[1], torch.tensor([[0.0, 0.0], [0.0, 3.0]]))
 
 
+# ---- TokenTopK -----------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("L,T,F,kk", [(1, 2, 4, 2), (2, 40, 256, 7), (3, 33, 1000, 50), (1, 5, 77, 77), (2, 9, 64, 100)])
+def test_tokentopk_per_layer_bit_exact(dev, dtype, L, T, F, kk):
+    g = torch.Generator().manual_seed(T * 3 + F)
+    pre = torch.randn(L, T, F, generator=g)
+    pre[0, 0, : F // 2] = 0.5                      # ties inside a row
+    pre = pre.to(dtype)
+    surv = engine.tokentopk_select(pre.to(dev), kk, False)
+    check_rows_sorted(surv)
+    assert surv.nnz == L * T * min(kk, F)
+    for l in range(L):
+        m = orc.tokentopk_mask(pre[l], float(kk), pre[l])
+        rows = engine.survivor_rows(surv).cpu()
+        sel = (rows >= l * T) & (rows < (l + 1) * T)
+        flat = (rows[sel] - l * T) * F + surv.col.cpu().long()[sel]
+        assert torch.equal(torch.sort(flat).values, m.view(-1).nonzero().view(-1))
+    assert torch.equal(dense_from(surv).to(dtype), torch.stack([orc.tokentopk_forward(pre[l], float(kk), pre[l]) for l in range(L)]))
+
+
+def test_tokentopk_reference_known_answers(dev):
+    # reference tests/unit/models/test_activations.py:158-190, 255-272
+    x = torch.tensor([[1.0, 2.0, 3.0, 4.0], [5.0, 1.0, 2.5, 3.5]], device=dev)
+    m = cca.TokenTopK._compute_mask(x, 0.5).cpu()
+    assert torch.equal(m, torch.tensor([[False, False, True, True], [True, False, False, True]]))
+    m = cca.TokenTopK._compute_mask(x, 1.0).cpu()
+    assert torch.equal(m, torch.tensor([[False, False, False, True], [True, False, False, False]]))
+    assert cca.TokenTopK._compute_mask(x, 0.0).sum() == 0 and bool(cca.TokenTopK._compute_mask(x, 5.0).all())
+    xx = torch.tensor([[1.0, 2.0, 3.0, 4.0], [10.0, 10.0, 10.0, 10.0]], device=dev)
+    r = torch.tensor([[4.0, 3.0, 2.0, 1.0], [1.0, 2.0, 3.0, 4.0]], device=dev)
+    out = cca.TokenTopK.apply(xx, 0.5, True, r).cpu()
+    assert torch.equal(out, torch.tensor([[1.0, 2.0, 0.0, 0.0], [0.0, 0.0, 10.0, 10.0]]))
+    # BatchTopK operator surface too (test_activations.py:66-152)
+    xb = torch.tensor([[1.0, 2.0, 3.0, 4.0], [5.0, 1.0, 2.5, 3.5]], device=dev, requires_grad=True)
+    ob = cca.BatchTopK.apply(xb, 2.0, True, None)
+    assert torch.equal(ob.detach().cpu(), torch.tensor([[0.0, 0.0, 3.0, 4.0], [5.0, 0.0, 0.0, 3.5]]))
+    gout = torch.ones_like(ob)
+    ob.backward(gout)
+    assert torch.equal(xb.grad.cpu(), torch.tensor([[0.0, 0.0, 1.0, 1.0], [1.0, 0.0, 0.0, 1.0]]))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_tokentopk_global(dev, dtype):
+    g = torch.Generator().manual_seed(4)
+    L, T, F, kk = 3, 50, 128, 9
+    pre = (torch.randn(L, T, F, generator=g) * (1 + torch.arange(L).view(L, 1, 1))).to(dtype)
+    surv = engine.tokentopk_select(pre.to(dev), kk, True)
+    check_rows_sorted(surv)
+    assert surv.nnz == T * kk
+    got = dense_from(surv)
+    per_tok = (engine.survivor_rows(surv).cpu() % T).bincount(minlength=T)
+    assert torch.equal(per_tok, torch.full((T,), kk))
+    ref = orc.global_tokentopk({l: pre[l] for l in range(L)}, L, float(kk))
+    ref = torch.stack([ref[l] for l in range(L)])
+    z = torch.stack([orc.zscore_for_ranking(pre[l]) for l in range(L)]).double()       # [L, T, F]
+    zt = z.permute(1, 0, 2).reshape(T, L * F)
+    kth = torch.topk(zt, kk, dim=1).values[:, -1]                                        # per token
+    band = (2.0 ** -6 if dtype == torch.bfloat16 else 1e-5) * kth.abs().clamp(min=1e-3)
+    sure = (z - kth.view(1, T, 1)).abs() > band.view(1, T, 1)
+    assert torch.equal((got != 0) & sure, (ref != 0) & sure)
+
+
 # ---- threshold activations ---------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("L,T,F", [(1, 7, 7), (2, 100, 264), (3, 64, 1000)])

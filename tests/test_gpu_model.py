@@ -50,6 +50,8 @@ CASES = [
     BASE.scaled("tiny-relu", activation_fn="relu", k=None),
     BASE.scaled("tiny-per-target", decoder_tying="per_target", dtype="bfloat16"),
     BASE.scaled("tiny-per-source", decoder_tying="per_source"),
+    BASE.scaled("tiny-topk", activation_fn="topk", k=6),
+    BASE.scaled("tiny-topk-global", activation_fn="topk", k=6, topk_mode="global", dtype="bfloat16"),
     BASE.scaled("ref-shape", num_layers=2, d_model=8, num_features=16, tokens=30, k=3),   # the reference's own test shape
     BASE.scaled("mid", num_layers=4, d_model=768, num_features=2048, tokens=300, k=20, dtype="bfloat16"),
 ]
@@ -87,6 +89,9 @@ def test_forward_matches_oracle(dev, wl):
     elif wl.activation_fn == "relu":
         for l in acts:
             assert torch.equal(acts[l].cpu(), torch.relu(pre_cpu[l]))
+    elif wl.activation_fn == "topk" and wl.topk_mode == "per_layer":
+        for l in acts:
+            assert torch.equal(acts[l].cpu(), orc.tokentopk_forward(pre_cpu[l], float(wl.k), pre_cpu[l]))
     for l in pre:
         assert orc.rel_l2(pre[l], orc.encoder_preactivations(x[l], sd[f"encoder_module.encoders.{l}.weight"],
                                                               sd[f"encoder_module.encoders.{l}.bias_param"])) <= TOL[dtype]
