@@ -1066,7 +1066,7 @@ extern "C" int clt_threshold_count(const void *pre, int64_t T, int64_t F, int64_
     return clt_check_launch();
   }
   if (!pre || !workspace) return CLT_ERR_ARG;
-  if ((double)T * (double)F * (double)L >= 2147483648.0) return CLT_ERR_RANGE;
+  if (F >= 2147483648LL || R >= 2147483647LL) return CLT_ERR_RANGE;   // the survivor total must also stay below 2^31
   if (workspace_bytes < (size_t)R * 4) return CLT_ERR_WORKSPACE;
   uint32_t *cnt = (uint32_t *)workspace;
   if (dtype == CLT_BF16) return dispatch_threshold<bf16_t>(false, pre, T, F, L, pre_layer_stride, theta, pred, cnt, row_ptr, nullptr, nullptr, s);
@@ -1107,7 +1107,7 @@ extern "C" int clt_tokentopk_select(const void *pre, int64_t T, int64_t F, int64
   }
   if (!pre || !col || !val || !workspace) return CLT_ERR_ARG;
   if (mode == CLT_TOPK_GLOBAL && (!mean || !denom)) return CLT_ERR_ARG;
-  if ((double)T * (double)F * (double)L >= 2147483648.0) return CLT_ERR_RANGE;
+  if ((double)T * (double)L * (double)(kk < F * L ? kk : F * L) >= 2147483648.0 || F >= 2147483648LL) return CLT_ERR_RANGE;
   if (workspace_bytes < clt_tokentopk_workspace_bytes(T, F, L, kk, mode, dtype)) return CLT_ERR_WORKSPACE;
   const int64_t rowlen = mode == CLT_TOPK_GLOBAL ? L * F : F;
   if (kk > rowlen) kk = rowlen;
