@@ -44,6 +44,23 @@ def algorithmic_work(wl, nnz_rows_pairs: int, nnz_total: int):
     }
 
 
+# HBM bytes per k_decode launch (FETCH_SIZE + WRITE_SIZE of `rocprofv3 --pmc`, each scaled by
+# what the same counter reads for the known-size copy at the end of this script), keyed by
+# (workload, launches per step).  Filled from the counter runs kept under profiles/.
+MEASURED_TRAFFIC = {("c1", 12): (1871269.0 + 512104.0) * 1024.0}
+
+
+def copy_probe(dev):
+    """A plain elementwise kernel that reads 256 MiB and writes 256 MiB: the yardstick the
+    FETCH_SIZE / WRITE_SIZE counters of a profiled run are scaled by."""
+    n = 64 * 1024 * 1024
+    src = torch.ones(n, dtype=torch.int32, device=dev)
+    dst = torch.empty_like(src)
+    torch.neg(src, out=dst)
+    torch.cuda.synchronize()
+    return int(dst[0].item())
+
+
 def gpu_events(n):
     return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
 
@@ -108,6 +125,12 @@ def run_gpu(args):
     sel_gbs = work["select_bytes"] / (st["select"] * 1e-3) / 1e9
     dec_gbs = work["decode_gathered_bytes"] / (st["decode"] * 1e-3) / 1e9
     dec_c_gbs = work["decode_compulsory_bytes"] / (st["decode"] * 1e-3) / 1e9
+    # the decode of a large batch is one k_decode launch per source layer (plus one small
+    # slice-pointer kernel before and one reduce kernel after, timed with them); a small batch
+    # is a single launch
+    n_dec_launch = L if T * L >= engine.SLICED_DECODE_MIN_ROWS else 1
+    dec_kernel_desc = (f"k_decode (sparse cross-layer decode; {n_dec_launch} launch(es) per step; the per-launch "
+                       "figures are the step's decode stage divided by that count)")
     mfma_peak = MFMA_BF16_PEAK_TF if wl.dtype == "bfloat16" else MFMA_FP32_PEAK_TF
     result = {
         "metric": "CLT forward tokens/sec at GPT-2-small x32 BatchTopK k=200; % of roofline per stage",
@@ -129,15 +152,16 @@ def run_gpu(args):
             "survivors_per_layer": counts[0],
         },
         "roofline": {
-            "kernel": "k_decode (sparse cross-layer decode, all targets in one launch)",
+            "kernel": dec_kernel_desc,
             "bound": "hbm",
             "achieved": dec_gbs,
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": dec_gbs / HBM_PEAK_GBS,
-            "traffic": None,
-            "algorithmic_bytes_per_launch": work["decode_gathered_bytes"],
-            "avg_launch_ms": st["decode"],
+            "traffic": MEASURED_TRAFFIC.get((wl.name, n_dec_launch)),
+            "algorithmic_bytes_per_launch": work["decode_gathered_bytes"] / n_dec_launch,
+            "avg_launch_ms": st["decode"] / n_dec_launch,
+            "launches_per_step": n_dec_launch,
         },
         "stages": {
             "encoder": {"ms": st["encode"], "bound": "mfma", "achieved": enc_tf, "peak": mfma_peak,
@@ -149,6 +173,8 @@ def run_gpu(args):
                        "compulsory_GBps": dec_c_gbs, "compulsory_frac": dec_c_gbs / HBM_PEAK_GBS},
         },
     }
+    if args.copy_probe:
+        copy_probe(dev)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(wl, model, slab, args.cpu_tokens)
     return result
@@ -195,7 +221,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c1")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--cpu-tokens", type=int, default=1024)
+    ap.add_argument("--cpu-tokens", type=int, default=4096)
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run one 256 MiB elementwise copy (counter yardstick for profiled runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures the one-GPU forward path; this build has no multi-GPU path "
