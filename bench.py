@@ -75,6 +75,7 @@ def run_gpu(args):
     cca._native.load(build_if_missing=False)
     model, inputs, slab = synth.build_model(wl, dev)
     model.eval()
+    model.fuse_encode_select = not args.no_fuse
     L, T = wl.num_layers, wl.tokens
 
     for _ in range(args.warmup):
@@ -96,15 +97,25 @@ def run_gpu(args):
     src_mask = (1 << L) - 1
     st = {"encode": 0.0, "select": 0.0, "decode": 0.0}
     surv = None
+    _, x_slab, w_slab, b_slab = enc.prepare_slab(inputs)
+    fused = (wl.activation_fn == "batchtopk" and not glob and model.fuse_encode_select
+             and engine.encode_collect_supported(x_slab, w_slab, b_slab, wl.k))
     for _ in range(args.steps):
         ev = gpu_events(4)
         ev[0].record()
-        _, pre = enc.encode_slab(inputs, out=pre_buf)
-        ev[1].record()
-        if wl.activation_fn == "batchtopk":
-            surv = engine.batchtopk_select(pre, wl.k, glob, ws)
+        if fused:
+            # encoder whose epilogue keeps the candidates only (plus the sample before it and the
+            # first histogram after it), then the exact selection on the candidates
+            handle = engine.encode_collect(x_slab, w_slab, b_slab, wl.k, pre_buf, ws)
+            ev[1].record()
+            surv = engine.collect_select(handle)
         else:
-            surv = model._survivors(inputs)[2]
+            pre = engine.encode(x_slab, w_slab, b_slab, out=pre_buf)
+            ev[1].record()
+            if wl.activation_fn == "batchtopk":
+                surv = engine.batchtopk_select(pre, wl.k, glob, ws)
+            else:
+                surv = model._survivors(inputs)[2]
         ev[2].record()
         rec = dec.decode_survivors(surv, src_mask, ws=ws)
         ev[3].record()
@@ -150,6 +161,7 @@ def run_gpu(args):
                         f"{wl.activation_fn} k={wl.k} ({wl.topk_mode}), decoders {wl.decoder_tying}",
             "global_batch_tokens": T,
             "survivors_per_layer": counts[0],
+            "encode_select": "fused (candidates collected in the encoder epilogue)" if fused else "separate kernels",
         },
         "roofline": {
             "kernel": dec_kernel_desc,
@@ -222,6 +234,7 @@ def main():
     ap.add_argument("--workload", default="c1")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-tokens", type=int, default=4096)
+    ap.add_argument("--no-fuse", action="store_true", help="separate encoder and selection kernels")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one 256 MiB elementwise copy (counter yardstick for profiled runs)")
     args = ap.parse_args()

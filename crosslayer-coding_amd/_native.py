@@ -35,6 +35,10 @@ _SIGNATURES = {
     "clt_colstats": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
     "clt_batchtopk_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64, _int, _int]),
     "clt_batchtopk_select": (_int, [_vp, _i64, _i64, _i64, _i64, _i64, _int, _vp, _vp, _int, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "clt_encode_collect_supported": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _int]),
+    "clt_encode_collect_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64, _i64, _int]),
+    "clt_encode_collect": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _int, _vp, _sz, _vp]),
+    "clt_collect_select": (_int, [_vp, _i64, _i64, _i64, _i64, _i64, _int, _vp, _vp, _vp, _vp, _sz, _vp]),
     "clt_tokentopk_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64, _int, _int]),
     "clt_tokentopk_select": (_int, [_vp, _i64, _i64, _i64, _i64, _i64, _int, _vp, _vp, _int, _vp, _vp, _vp, _vp, _sz, _vp]),
     "clt_threshold_count": (_int, [_vp, _i64, _i64, _i64, _i64, _vp, _int, _int, _vp, _vp, _sz, _vp]),

@@ -55,6 +55,9 @@ class CrossLayerTranscoder(BaseTranscoder):
         self.process_group = process_group
         self.world_size, self.rank = 1, 0
         self.profiler = profiler
+        # per-layer BatchTopK: let the encoder epilogue collect the candidates (same result, one
+        # dense write and one dense read less); False forces the separate encode + select kernels
+        self.fuse_encode_select = True
         self.dtype = self._resolve_dtype(config.clt_dtype)
         if device is not None:
             self.device = torch.device(device)
@@ -213,10 +216,19 @@ class CrossLayerTranscoder(BaseTranscoder):
         n = len(layers)
         ws = self._workspace()
         pre_buf = ws.typed("pre", (n, T, cfg.num_features), self.dtype) if T > 0 else None
-        slab = self.encoder_module.encode_slab(inputs, out=pre_buf)
-        if slab is None:
+        prep = self.encoder_module.prepare_slab(inputs)
+        if prep is None:
             return None
-        _, pre = slab
+        _, x_slab, w_slab, b_slab = prep
+        if fn == "batchtopk" and cfg.topk_mode == "per_layer" and self.fuse_encode_select:
+            # the encoder keeps only the candidates above a sampled cut; nothing dense is written
+            k = int(cfg.batchtopk_k)
+            if engine.encode_collect_supported(x_slab, w_slab, b_slab, k):
+                with self._timed("batchtopk_activation") as tm:
+                    surv = engine.collect_select(engine.encode_collect(x_slab, w_slab, b_slab, k, pre_buf, ws))
+                self._record("batchtopk_activation", tm)
+                return layers, T, surv
+        pre = engine.encode(x_slab, w_slab, b_slab, out=pre_buf)
         if fn in ("batchtopk", "topk"):
             surv = self._select(pre)
         elif fn == "jumprelu":

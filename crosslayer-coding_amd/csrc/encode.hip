@@ -17,7 +17,7 @@
 //               16 bytes per lane and 256 contiguous bytes per token
 //   bf16        v_mfma_f32_32x32x16_bf16, fp32 accumulate, one rounding (v_cvt_pk_bf16_f32)
 //   fp32        v_mfma_f32_32x32x2_f32
-#include "clt_common.h"
+#include "select_state.h"
 
 namespace {
 
@@ -61,6 +61,52 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
 
+// element j of a 16-byte slot as a float / as raw bits
+template <typename T> __device__ __forceinline__ float slot_elem(const uint4 &w, int j);
+template <> __device__ __forceinline__ float slot_elem<float>(const uint4 &w, int j) {
+  return __uint_as_float(j == 0 ? w.x : j == 1 ? w.y : j == 2 ? w.z : w.w);
+}
+template <> __device__ __forceinline__ float slot_elem<bf16_t>(const uint4 &w, int j) {
+  const uint32_t u = (j >> 1) == 0 ? w.x : (j >> 1) == 1 ? w.y : (j >> 1) == 2 ? w.z : w.w;
+  return __uint_as_float((j & 1) ? (u & 0xFFFF0000u) : (u << 16));
+}
+template <typename T> __device__ __forceinline__ uint32_t slot_raw(const uint4 &w, int j);
+template <> __device__ __forceinline__ uint32_t slot_raw<float>(const uint4 &w, int j) {
+  return j == 0 ? w.x : j == 1 ? w.y : j == 2 ? w.z : w.w;
+}
+template <> __device__ __forceinline__ uint32_t slot_raw<bf16_t>(const uint4 &w, int j) {
+  const uint32_t u = (j >> 1) == 0 ? w.x : (j >> 1) == 1 ? w.y : (j >> 1) == 2 ? w.z : w.w;
+  return (j & 1) ? (u >> 16) : (u & 0xFFFFu);
+}
+
+// packed 16-bit helpers (two elements per 32-bit word)
+typedef short i16x2_t __attribute__((ext_vector_type(2)));
+typedef unsigned short u16x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pk_sub_sat16(uint32_t a, uint32_t b) {   // signed saturating a - b
+  return __builtin_bit_cast(uint32_t, __builtin_elementwise_sub_sat(__builtin_bit_cast(i16x2_t, a), __builtin_bit_cast(i16x2_t, b)));
+}
+__device__ __forceinline__ uint32_t pk_sign16(uint32_t a) {                 // 0xFFFF where the half is negative
+  return __builtin_bit_cast(uint32_t, __builtin_bit_cast(i16x2_t, a) >> (short)15);
+}
+__device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
+  return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(u16x2_t, a), __builtin_bit_cast(u16x2_t, b)));
+}
+
+// inclusive prefix sums with DPP row shifts: inside each row of 16 lanes / over the wavefront
+__device__ __forceinline__ uint32_t row16_inclusive_scan(uint32_t v) {
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x111, 0xf, 0xf, false);  // row_shr:1
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x112, 0xf, 0xf, false);  // row_shr:2
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x114, 0xf, 0xf, false);  // row_shr:4
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x118, 0xf, 0xf, false);  // row_shr:8
+  return v;
+}
+__device__ __forceinline__ uint32_t wave_inclusive_scan32(uint32_t v) {
+  v = row16_inclusive_scan(v);
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x142, 0xa, 0xf, false);  // row_bcast:15
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x143, 0xc, 0xf, false);  // row_bcast:31
+  return v;
+}
+
 // Requires K % (256 / sizeof(T)) == 0 (an even number of LDS stages), M >= BM and N >= BN.  A tile that
 // would stick out of the matrix is shifted back inside (its overlap with the neighbour is
 // computed twice and stored twice with identical values), so no load or store is predicated.
@@ -69,10 +115,17 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
 // When the feature tiles split evenly, XCD x takes the feature tiles n = x, x+8, ... and walks
 // all token tiles of one n before the next: a W tile is fetched by one XCD only and the x slab
 // of the layer stays in that XCD's L2.
-template <typename T>
+//
+// COLLECT 0 stores the tile.  COLLECT 1 / 2 store nothing: the epilogue compares every element
+// with the layer's cut value (1) or its feature's threshold (2) and appends the ones that reach
+// it, as (feature, raw value) entries ordered by (token, feature), to one extent of the layer's
+// candidate pool per wavefront and feature segment (see CollectArgs).  These modes need
+// M % BM == 0 and N % BN == 0 (a shifted tile would report its overlap twice).
+template <typename T, int COLLECT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void k_encode_mfma(
     const T *__restrict__ x, const T *__restrict__ w, const T *__restrict__ bias, T *__restrict__ pre,
-    int M, int K, int N, int tiles_m, int tiles_n, int64_t xs, int64_t wstr, int64_t bs, int64_t ps) {
+    int M, int K, int N, int tiles_m, int tiles_n, int64_t xs, int64_t wstr, int64_t bs, int64_t ps,
+    const SelState *__restrict__ gate, CollectArgs ca) {
   constexpr int CE = 16 / (int)sizeof(T);  // elements per 16-byte chunk
   constexpr int BK = ROWB / (int)sizeof(T);
   // Two separate stage buffers (not one array with an offset): the compiler can then tell that
@@ -88,6 +141,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   const int per_layer = tiles_m * tiles_n;
   const int layer = bid / per_layer;
   bid -= layer * per_layer;
+  if (COLLECT == 0 && gate && gate[layer].status != ST_RETRY) return;
   int tn, tm;
   if ((tiles_n & 7) == 0) {
     const int xcd = bid & 7, idx = bid >> 3;
@@ -246,13 +300,137 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     }
     // the wavefront reads its own tile back: lane -> (row = it*4 + lane/16, slot = lane%16)
     constexpr int EPS = 16 / (int)sizeof(T);               // elements per 16-byte slot
+    if constexpr (COLLECT == 0) {
 #pragma unroll 4
-    for (int it = 0; it < 32; ++it) {
-      const int ml = it * 4 + (lane >> 4), sl = lane & 15;
-      const uint4 v = *reinterpret_cast<const uint4 *>(park + ml * 256 + ((sl ^ (ml & 15)) * 16));
-      const int m = m0 + wm * 128 + ml;
-      const int n = n0 + wn * 128 + pass * (128 / NPASS) + sl * EPS;
-      *reinterpret_cast<uint4 *>(pl + (int64_t)m * N + n) = v;
+      for (int it = 0; it < 32; ++it) {
+        const int ml = it * 4 + (lane >> 4), sl = lane & 15;
+        const uint4 v = *reinterpret_cast<const uint4 *>(park + ml * 256 + ((sl ^ (ml & 15)) * 16));
+        const int m = m0 + wm * 128 + ml;
+        const int n = n0 + wn * 128 + pass * (128 / NPASS) + sl * EPS;
+        *reinterpret_cast<uint4 *>(pl + (int64_t)m * N + n) = v;
+      }
+    } else {
+      // lane -> token row (two rows per lane, 64 apart): counting and ordering inside a row
+      // need no cross-lane work, and the per-row bookkeeping is written 64 rows at a time
+      constexpr int KB = Elem<T>::KEYBITS;
+      constexpr int SEGW = 128 / NPASS;                    // features per segment (16 slots)
+      constexpr int NW = SEGW / 32;                        // 32-bit mask words per row
+      const int ncol0 = n0 + wn * 128 + pass * SEGW;       // first feature of the segment
+      uint32_t cut_bits = 0;
+      if constexpr (COLLECT == 1) cut_bits = key_to_f32_bits<KB>(ca.st[layer].cut_key);
+      const bool cut_nan = (cut_bits & 0x7FFFFFFFu) > 0x7F800000u;   // only NaNs reach such a cut
+      const float cutf = __uint_as_float(cut_bits);
+      uint32_t W[2][NW];
+      uint32_t cnt[2];
+      // generic: float compares, element by element; bit c of a row's mask = column c
+      auto scan_generic = [&]() {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const int ml = h * 64 + lane;
+#pragma unroll
+          for (int i = 0; i < NW; ++i) W[h][i] = 0;
+#pragma unroll
+          for (int sl = 0; sl < 16; ++sl) {
+            const uint4 v = *reinterpret_cast<const uint4 *>(park + ml * 256 + ((sl ^ (ml & 15)) * 16));
+            uint4 tv = make_uint4(0, 0, 0, 0);
+            if constexpr (COLLECT == 2)
+              tv = *reinterpret_cast<const uint4 *>((const T *)ca.theta + (int64_t)layer * ca.theta_stride + ncol0 + sl * EPS);
+            uint32_t m = 0;
+#pragma unroll
+            for (int j = 0; j < EPS; ++j) {
+              const float xv = slot_elem<T>(v, j);
+              bool c;
+              if constexpr (COLLECT == 1) c = cut_nan ? (xv != xv) : !(xv < cutf);
+              else c = xv >= slot_elem<T>(tv, j);
+              m |= (c ? 1u : 0u) << j;
+            }
+            W[h][(sl * EPS) >> 5] |= m << ((sl * EPS) & 31);
+          }
+        }
+      };
+      bool done = false;
+      if constexpr (COLLECT == 1 && sizeof(T) == 2) {
+        // bf16 and a positive cut: x >= cut  <=>  bits(x) >= bits(cut) as signed 16-bit integers
+        // (negative values have the sign bit), two elements per operation: the sign of the
+        // saturated difference (cut - 1) - x marks a candidate.  NaNs with the sign bit set would
+        // be missed, so the unsigned maximum of all raw values is tracked; if it shows one, the
+        // tile is redone with float compares.
+        const uint32_t cb = cut_bits >> 16;
+        if (cb >= 1u && cb <= 0x7F80u) {
+          const uint32_t cm1 = (cb - 1u) | ((cb - 1u) << 16);
+          uint32_t mx = 0;
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            const int ml = h * 64 + lane;
+#pragma unroll
+            for (int i = 0; i < NW; ++i) W[h][i] = 0;
+#pragma unroll
+            for (int sl = 0; sl < 16; ++sl) {
+              const uint4 v = *reinterpret_cast<const uint4 *>(park + ml * 256 + ((sl ^ (ml & 15)) * 16));
+              const uint32_t w4[4] = {v.x, v.y, v.z, v.w};
+              uint32_t a = 0;
+#pragma unroll
+              for (int k = 0; k < 4; ++k) {
+                const uint32_t sg = pk_sign16(pk_sub_sat16(cm1, w4[k]));      // 0xFFFF per candidate half
+                a |= sg & ((1u << (2 * k)) | (0x20000u << (2 * k)));         // element 2k -> bit 2k, 2k+1 -> bit 16+2k+1
+                mx = pk_max_u16(mx, w4[k]);
+              }
+              const uint32_t m = (a | (a >> 16)) & 0xFFu;
+              W[h][sl >> 2] |= m << ((sl & 3) * 8);
+            }
+          }
+          const bool neg_nan = (mx & 0xFFFFu) > 0xFF80u || (mx >> 16) > 0xFF80u;
+          done = __ballot(neg_nan) == 0;
+        }
+      }
+      if (!done) scan_generic();
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        cnt[h] = 0;
+#pragma unroll
+        for (int i = 0; i < NW; ++i) cnt[h] += __popc(W[h][i]);
+      }
+      const uint32_t incl0 = wave_inclusive_scan32(cnt[0]), incl1 = wave_inclusive_scan32(cnt[1]);
+      const uint32_t tot0 = __builtin_amdgcn_readlane(incl0, 63), tot1 = __builtin_amdgcn_readlane(incl1, 63);
+      const uint32_t total = tot0 + tot1;
+      const int nseg = N / SEGW;
+      const int seg = ncol0 / SEGW;
+      const int nrb = M >> 7, rowblk = (m0 + wm * 128) >> 7;
+      const uint32_t tile = (uint32_t)seg * (uint32_t)nrb + (uint32_t)rowblk;
+      uint32_t off = tile * ca.caps;                       // the tile's fixed slot
+      bool ok = true;
+      if (total > ca.caps) {                               // rare: an extent behind the slots
+        const unsigned long long fixed = (unsigned long long)nseg * nrb * ca.caps;
+        uint32_t a = 0;
+        if (lane == 0) a = atomicAdd(&ca.pool_count[layer], total);
+        a = __builtin_amdgcn_readfirstlane(a);
+        ok = fixed + a + total <= ca.pool_cap;
+        off = (uint32_t)(fixed + a);
+        if (!ok && lane == 0) atomicOr(&ca.st[layer].overflow, 1u);
+      }
+      uint2 *mypool = ca.pool + (unsigned long long)layer * ca.pool_cap;
+      if (lane == 0) ca.tile_meta[(int64_t)layer * nseg * nrb + tile] = make_uint2(off, ok ? total : 0u);
+      uint2 *meta = ca.seg_meta + ((int64_t)layer * nseg + seg) * M + m0 + wm * 128;
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int ml = h * 64 + lane;
+        uint32_t pos = off + (h ? tot0 + incl1 - cnt[1] : incl0 - cnt[0]);
+        meta[ml] = ok ? make_uint2(pos, cnt[h]) : make_uint2(0u, 0u);
+        if (!ok) continue;
+#pragma unroll
+        for (int i = 0; i < NW; ++i) {
+          uint32_t w = W[h][i];
+          while (__ballot(w != 0)) {
+            if (w) {
+              const int c = i * 32 + (__ffs(w) - 1);       // column inside the segment
+              w &= w - 1u;
+              const int sl = c / EPS, j = c % EPS;
+              const T rawv = *reinterpret_cast<const T *>(park + ml * 256 + ((sl ^ (ml & 15)) * 16) + j * (int)sizeof(T));
+              mypool[pos++] = make_uint2((uint32_t)(ncol0 + c), Elem<T>::raw(rawv));
+            }
+          }
+        }
+      }
     }
   }
 }
@@ -273,20 +451,37 @@ __global__ void k_encode_generic(const T *x, const T *w, const T *bias, T *pre, 
 }
 
 template <typename T>
-static int launch_encode(const void *x, const void *w, const void *b, void *pre, int64_t T_, int64_t d, int64_t F,
-                         int64_t L, int64_t xs, int64_t wstr, int64_t bs, int64_t ps, hipStream_t stream) {
+static bool encode_fast_ok(const void *x, const void *w, const void *b, const void *pre, int64_t T_, int64_t d,
+                           int64_t F, int64_t xs, int64_t wstr, int64_t bs, int64_t ps) {
   constexpr int CE = 16 / (int)sizeof(T);
-  const bool fast = (d % (2 * ROWB / (int)sizeof(T)) == 0) && (F % 4 == 0) && T_ >= BM && F >= BN && clt_aligned16(x) && clt_aligned16(w) && clt_aligned16(pre) &&
-                    (xs % CE == 0) && (wstr % CE == 0) && (ps % 4 == 0) && (ps * (int64_t)sizeof(T)) % 16 == 0 &&
-                    (F * (int64_t)sizeof(T)) % 8 == 0 && T_ < (1 << 30) && F < (1 << 30) && d < (1 << 30) &&
-                    (!b || (((uintptr_t)b) % 16 == 0 && bs % 8 == 0));
+  return (d % (2 * ROWB / (int)sizeof(T)) == 0) && (F % 4 == 0) && T_ >= BM && F >= BN && clt_aligned16(x) &&
+         clt_aligned16(w) && clt_aligned16(pre) && (xs % CE == 0) && (wstr % CE == 0) && (ps % 4 == 0) &&
+         (ps * (int64_t)sizeof(T)) % 16 == 0 && (F * (int64_t)sizeof(T)) % 8 == 0 && T_ < (1 << 30) &&
+         F < (1 << 30) && d < (1 << 30) && (!b || (((uintptr_t)b) % 16 == 0 && bs % 8 == 0));
+}
+
+template <typename T>
+static int launch_encode(const void *x, const void *w, const void *b, void *pre, int64_t T_, int64_t d, int64_t F,
+                         int64_t L, int64_t xs, int64_t wstr, int64_t bs, int64_t ps, int collect,
+                         const SelState *gate, const CollectArgs *ca, hipStream_t stream) {
+  const bool fast = encode_fast_ok<T>(x, w, b, collect ? nullptr : pre, T_, d, F, xs, wstr, bs, collect ? 16 : ps);
+  if (collect && !(fast && T_ % BM == 0 && F % BN == 0)) return CLT_ERR_ARG;
   if (fast) {
     const int64_t tm = clt_ceil_div(T_, BM), tn = clt_ceil_div(F, BN);
     const int64_t nblk = tm * tn * L;
     if (nblk > 2147483647LL) return CLT_ERR_RANGE;
-    k_encode_mfma<T><<<(unsigned)nblk, 256, 0, stream>>>((const T *)x, (const T *)w, (const T *)b, (T *)pre, (int)T_,
-                                                         (int)d, (int)F, (int)tm, (int)tn, xs, wstr, bs, ps);
+    CollectArgs none = {};
+    const CollectArgs a = ca ? *ca : none;
+#define CLT_ENC(C)                                                                                               \
+  k_encode_mfma<T, C><<<(unsigned)nblk, 256, 0, stream>>>((const T *)x, (const T *)w, (const T *)b, (T *)pre,    \
+                                                          (int)T_, (int)d, (int)F, (int)tm, (int)tn, xs, wstr,   \
+                                                          bs, ps, gate, a)
+    if (collect == 0) CLT_ENC(0);
+    else if (collect == 1) CLT_ENC(1);
+    else CLT_ENC(2);
+#undef CLT_ENC
   } else {
+    // the gate is ignored here: recomputing a layer that did not ask for it is harmless
     k_encode_generic<T><<<256 * 8, 256, 0, stream>>>((const T *)x, (const T *)w, (const T *)b, (T *)pre, T_, d, F, L,
                                                      xs, wstr, bs, ps);
   }
@@ -295,6 +490,20 @@ static int launch_encode(const void *x, const void *w, const void *b, void *pre,
 
 }  // namespace
 
+int clt_launch_encode(const void *x, const void *w, const void *b, void *pre, int64_t T, int64_t d, int64_t F,
+                      int64_t L, int64_t xs, int64_t wstr, int64_t bs, int64_t ps, int dtype, int collect,
+                      const SelState *gate, const CollectArgs *ca, hipStream_t stream) {
+  if (dtype == CLT_BF16) return launch_encode<bf16_t>(x, w, b, pre, T, d, F, L, xs, wstr, bs, ps, collect, gate, ca, stream);
+  return launch_encode<float>(x, w, b, pre, T, d, F, L, xs, wstr, bs, ps, collect, gate, ca, stream);
+}
+
+bool clt_encode_can_collect(const void *x, const void *w, const void *b, int64_t T, int64_t d, int64_t F,
+                            int64_t xs, int64_t wstr, int64_t bs, int dtype) {
+  const bool fast = dtype == CLT_BF16 ? encode_fast_ok<bf16_t>(x, w, b, nullptr, T, d, F, xs, wstr, bs, 16)
+                                      : encode_fast_ok<float>(x, w, b, nullptr, T, d, F, xs, wstr, bs, 16);
+  return fast && T % BM == 0 && F % BN == 0;
+}
+
 extern "C" int clt_encode(const void *x, const void *w, const void *b, void *pre, int64_t T, int64_t d, int64_t F,
                           int64_t L, int64_t x_layer_stride, int64_t w_layer_stride, int64_t b_layer_stride,
                           int64_t pre_layer_stride, int dtype, void *stream) {
@@ -302,8 +511,6 @@ extern "C" int clt_encode(const void *x, const void *w, const void *b, void *pre
   if (T < 0 || d <= 0 || F <= 0 || L <= 0) return CLT_ERR_ARG;
   if (T == 0) return CLT_OK;
   if (!x || !w || !pre) return CLT_ERR_ARG;
-  hipStream_t s = (hipStream_t)stream;
-  if (dtype == CLT_BF16)
-    return launch_encode<bf16_t>(x, w, b, pre, T, d, F, L, x_layer_stride, w_layer_stride, b_layer_stride, pre_layer_stride, s);
-  return launch_encode<float>(x, w, b, pre, T, d, F, L, x_layer_stride, w_layer_stride, b_layer_stride, pre_layer_stride, s);
+  return clt_launch_encode(x, w, b, pre, T, d, F, L, x_layer_stride, w_layer_stride, b_layer_stride,
+                           pre_layer_stride, dtype, 0, nullptr, nullptr, (hipStream_t)stream);
 }

@@ -23,33 +23,20 @@
 // stages, and a cut that turns out too high (fewer than K candidates) makes the pass run
 // again with the lowest cut, so the result is exact for any input; only the speed depends
 // on the sample being representative.
-#include "clt_common.h"
+#include "select_state.h"
 
 namespace {
 
 constexpr int NBINS = 2048;
 constexpr uint32_t FINE16 = 1984;  // 16-bit keys: bins [0,FINE16) are one key wide
 constexpr int SAMPLE_N = 16384;
+constexpr int SAMPLE_TOK = 64;           // tokens of the sample taken before the pre-activations exist
 constexpr int SAMPLE_BLOCKS = 16;        // blocks per problem that gather the sample
 constexpr int SCAN_THREADS = 1024;
 constexpr int WBUF = 512;                // candidate entries buffered in LDS per wavefront
 constexpr int PASS_NV = 4;               // 16-byte loads in flight per lane in the pass
 constexpr uint32_t ROW_NONE = 0xFFFFFFFFu;   // row has no candidates
 constexpr uint32_t ROW_DENSE = 0xFFFFFFFEu;  // row did not fit the pool: read it from the matrix
-
-enum : uint32_t { ST_RUN = 0, ST_RETRY = 1, ST_DONE = 2 };
-
-struct SelState {
-  uint32_t cut_key;   // candidates have key >= cut_key
-  uint32_t status;    // ST_*
-  uint32_t level;     // level whose histogram is being accumulated
-  uint32_t flo, fhi;  // levels >= 1: inclusive range of (key - cut_key) still in play
-  uint32_t bbase;     // levels >= 1: bin = (diff - bbase) >> shift
-  uint32_t shift;
-  uint32_t thr_key;   // result: key of the K-th largest element
-  unsigned long long k_rem;       // still to take from the active range
-  unsigned long long tie_budget;  // result: how many elements equal to thr_key survive
-};
 
 template <int KB> __device__ __forceinline__ uint32_t min_key() {
   return KB == 32 ? 0x007FFFFFu : 0x007Fu;  // key(-inf); nothing ranks below it
@@ -205,13 +192,13 @@ __global__ __launch_bounds__(256) void k_sample_keys(
 template <int KB>
 __global__ __launch_bounds__(SCAN_THREADS) void k_sample_cut(
     const uint32_t *sample, unsigned long long N, unsigned long long K, SelState *st, uint32_t *hist,
-    uint32_t *pool_count) {
+    uint32_t *pool_count, uint32_t *pool2_count, uint32_t path) {
   constexpr int PER = SAMPLE_N / SCAN_THREADS;
   __shared__ uint32_t lh[NBINS];
   const int p = blockIdx.x, tid = threadIdx.x;
   const unsigned long long ns = N < (unsigned long long)SAMPLE_N ? N : (unsigned long long)SAMPLE_N;
   for (int i = tid; i < NBINS; i += SCAN_THREADS) hist[(int64_t)p * NBINS + i] = 0;
-  if (tid == 0) pool_count[p] = 0;
+  if (tid == 0) { pool_count[p] = 0; if (pool2_count) pool2_count[p] = 0; }
   uint32_t keys[PER];
   bool valid[PER];
 #pragma unroll
@@ -224,7 +211,10 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_sample_cut(
   if (ns == N) r = K;
   else {
     double e = (double)K / (double)N * (double)ns;
-    r = (unsigned long long)(1.25 * e + 6.0 * sqrt(e) + 16.0) + 1;
+    // the sample taken from a token x feature grid (PATH_TILES) is less even than a hashed
+    // one: leave it more room
+    r = path == PATH_TILES ? (unsigned long long)(1.5 * e + 8.0 * sqrt(e) + 16.0) + 1
+                           : (unsigned long long)(1.25 * e + 6.0 * sqrt(e) + 16.0) + 1;
   }
   uint32_t cut = min_key<KB>();
   if (r <= ns && r > 0) {
@@ -255,7 +245,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_sample_cut(
   if (tid == 0) {
     SelState s;
     s.cut_key = cut; s.status = ST_RUN; s.level = 0; s.flo = 0; s.fhi = 0; s.bbase = 0; s.shift = 0;
-    s.thr_key = 0; s.k_rem = K; s.tie_budget = 0;
+    s.thr_key = 0; s.k_rem = K; s.tie_budget = 0; s.path = path; s.overflow = 0;
     st[p] = s;
   }
 }
@@ -447,9 +437,10 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_select_scan(SelState *st, uint
   int bin; unsigned long long above, total;
   bool found = block_find_from_top(lh, NBINS, s.k_rem, bin, above, total);
   if (tid != 0) return;
+  if (s.overflow) found = false;   // the collecting encoder dropped candidates: start over from the matrix
   if (!found) {
     // fewer candidates than K: the sampled cut was too high -> run the pass again from the bottom
-    s.status = ST_RETRY; s.cut_key = min_key<KB>(); s.level = 0;
+    s.status = ST_RETRY; s.cut_key = min_key<KB>(); s.level = 0; s.path = PATH_ROWS; s.overflow = 0;
     pool_count[p] = 0;  // the retry pass refills the pool from scratch
     st[p] = s;
     return;
@@ -533,7 +524,7 @@ __global__ __launch_bounds__(256) void k_select_level(
   __shared__ uint32_t lh[NBINS];
   const int l = blockIdx.y, p = GLOBAL ? 0 : l;
   const SelState s = st[p];
-  if (!(s.status == ST_RUN && (int)s.level == level)) return;
+  if (!(s.status == ST_RUN && (int)s.level == level) || s.path != PATH_ROWS) return;
   for (int i = threadIdx.x; i < NBINS; i += blockDim.x) lh[i] = 0;
   __syncthreads();
   const int wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
@@ -562,6 +553,7 @@ __global__ __launch_bounds__(256) void k_select_count(
     unsigned long long pool_cap, uint32_t *row_gt, uint32_t *row_eq) {
   const int l = blockIdx.y, p = GLOBAL ? 0 : l;
   const SelState s = st[p];
+  if (s.path != PATH_ROWS) return;
   const int wv = threadIdx.x >> 6, nwv = blockDim.x >> 6, lane = lane_id();
   typename RankOf<T, GLOBAL>::type rk = RankOf<T, GLOBAL>::make(mean, denom, l, F);
   for (int64_t t = (int64_t)blockIdx.x * nwv + wv; t < Tn; t += (int64_t)gridDim.x * nwv) {
@@ -641,9 +633,12 @@ template <typename T, bool GLOBAL>
 __global__ __launch_bounds__(256) void k_select_emit(
     const T *pre, int64_t Tn, int64_t F, int64_t L, int64_t lstride, const float *mean,
     const float *denom, const SelState *st, const uint32_t *row_first, const uint2 *pool,
-    unsigned long long pool_cap, const uint32_t *allot, const int32_t *row_ptr, int32_t *col_out, T *val_out) {
+    unsigned long long pool_cap, const uint32_t *allot, const int32_t *row_ptr, int32_t *col_out, T *val_out,
+    const uint2 *pool2, unsigned long long pool2_cap) {
   const int l = blockIdx.y, p = GLOBAL ? 0 : l;
   const SelState s = st[p];
+  // candidates collected by the encoder were regrouped per row into the second pool
+  if (s.path == PATH_TILES) { pool = pool2; pool_cap = pool2_cap; }
   const int wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
   typename RankOf<T, GLOBAL>::type rk = RankOf<T, GLOBAL>::make(mean, denom, l, F);
   for (int64_t t = (int64_t)blockIdx.x * nwv + wv; t < Tn; t += (int64_t)gridDim.x * nwv) {
@@ -665,6 +660,171 @@ __global__ __launch_bounds__(256) void k_select_emit(
         kept += (uint32_t)__popcll(bk);
         ties += (uint32_t)__popcll(beq);
       });
+  }
+}
+
+// ---- candidates collected by the encoder epilogue (PATH_TILES) -------------------------
+// Ranking keys of a sample taken BEFORE the pre-activations exist: SAMPLE_TOK hashed tokens x
+// SAMPLE_N / SAMPLE_TOK hashed features per layer, each value computed as a plain dot product
+// (fp32 accumulation, rounded to the model dtype).  It only has to give a cut of the right
+// size; the selection stays exact whatever the cut is.
+template <typename T>
+__global__ __launch_bounds__(256) void k_sample_dot(
+    const T *__restrict__ x, const T *__restrict__ w, const T *__restrict__ b, int64_t Tn, int64_t d, int64_t F,
+    int64_t xs, int64_t wstr, int64_t bs, uint32_t *sample) {
+  constexpr int KB = Elem<T>::KEYBITS;
+  constexpr int V = Elem<T>::VEC;
+  constexpr int NFEAT = SAMPLE_N / SAMPLE_TOK;
+  constexpr int NJ = 4;   // features in flight per wavefront
+  const int l = blockIdx.y, ti = blockIdx.x;
+  const int lane = lane_id(), wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
+  const int64_t tok = (int64_t)hash_index((uint64_t)ti * 131u + (uint64_t)l * 7919u, (uint64_t)Tn);
+  const T *xr = x + (int64_t)l * xs + tok * d;
+  const int64_t nch = d / V;   // 16-byte chunks per row (the collecting encoder needs d % V == 0)
+  for (int j0 = wv * NJ; j0 < NFEAT; j0 += nwv * NJ) {
+    const T *wr[NJ];
+    int64_t f[NJ];
+    float acc[NJ];
+#pragma unroll
+    for (int q = 0; q < NJ; ++q) {
+      f[q] = (int64_t)hash_index((uint64_t)(j0 + q) * 257u + (uint64_t)ti * 65537u + (uint64_t)l * 104729u + 1u, (uint64_t)F);
+      wr[q] = w + (int64_t)l * wstr + f[q] * d;
+      acc[q] = 0.0f;
+    }
+    for (int64_t c = lane; c < nch; c += 64) {
+      const uint4 xv = *reinterpret_cast<const uint4 *>(xr + c * V);
+      uint4 wq[NJ];
+#pragma unroll
+      for (int q = 0; q < NJ; ++q) wq[q] = *reinterpret_cast<const uint4 *>(wr[q] + c * V);
+#pragma unroll
+      for (int q = 0; q < NJ; ++q)
+#pragma unroll
+        for (int e = 0; e < V; ++e) acc[q] = fmaf(vec_elem<T>(xv, e), vec_elem<T>(wq[q], e), acc[q]);
+    }
+#pragma unroll
+    for (int q = 0; q < NJ; ++q) {
+      float a = acc[q];
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) a += __shfl_xor(a, o);
+      if (lane == 0) {
+        if (b) a += Elem<T>::to_f32(b[(int64_t)l * bs + f[q]]);
+        sample[(int64_t)l * SAMPLE_N + (int64_t)ti * NFEAT + j0 + q] = rank_key<KB>(Elem<T>::round(a));
+      }
+    }
+  }
+}
+
+// Histogram of the collected candidates of every layer that is at `level`: one wavefront per
+// tile extent.
+template <typename T>
+__global__ __launch_bounds__(256) void k_pool_hist(const SelState *st, const uint2 *tile_meta, int ntile,
+                                                   const uint2 *pool, unsigned long long pool_cap, uint32_t *hist,
+                                                   int level) {
+  constexpr int KB = Elem<T>::KEYBITS;
+  __shared__ uint32_t lh[NBINS];
+  const int p = blockIdx.y;
+  const SelState s = st[p];
+  if (s.path != PATH_TILES || s.status != ST_RUN || (int)s.level != level) return;
+  for (int i = threadIdx.x; i < NBINS; i += blockDim.x) lh[i] = 0;
+  __syncthreads();
+  const int lane = lane_id(), wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
+  const uint2 *mypool = pool + (unsigned long long)p * pool_cap;
+  for (int i = blockIdx.x * nwv + wv; i < ntile; i += gridDim.x * nwv) {
+    const uint2 tm = tile_meta[(int64_t)p * ntile + i];
+    for (uint32_t e = lane; e < tm.y; e += 64) {
+      const uint32_t key = rank_key<KB>(Elem<T>::to_f32(Elem<T>::from_raw(mypool[tm.x + e].y)));
+      const uint32_t diff = key - s.cut_key;
+      if (level == 0) atomicAdd(&lh[bin_level0<KB>(diff)], 1u);
+      else if (diff >= s.flo && diff <= s.fhi) atomicAdd(&lh[(diff - s.bbase) >> s.shift], 1u);
+    }
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < NBINS; i += blockDim.x) {
+    uint32_t c = lh[i];
+    if (c) atomicAdd(&hist[(int64_t)p * NBINS + i], c);
+  }
+}
+
+// One wavefront per row: walks the row's runs in all feature segments (lane -> consecutive
+// segments, so lane order is feature order), counts the entries above / equal to the threshold
+// key and copies them, in feature order, to one extent of the second pool (same extent format
+// as the streaming pass writes: a header entry (next, count), then the entries).
+// SPL = segments per lane.  The first GE entries of each run are fetched in one batch and kept
+// in registers; only a run longer than that is walked again for the copy.
+template <typename T, int SPL>
+__global__ __launch_bounds__(256) void k_row_gather(
+    int64_t Tn, const SelState *st, const uint2 *seg_meta, int nseg, const uint2 *pool, unsigned long long pool_cap,
+    uint32_t *pool2_count, uint2 *pool2, unsigned long long pool2_cap, uint32_t *row_first, uint32_t *row_gt,
+    uint32_t *row_eq) {
+  constexpr int KB = Elem<T>::KEYBITS;
+  constexpr int GE = 4;
+  const int l = blockIdx.y;
+  const SelState s = st[l];
+  if (s.path != PATH_TILES || s.status != ST_DONE) return;
+  const int lane = lane_id(), wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
+  const uint2 *mypool = pool + (unsigned long long)l * pool_cap;
+  uint2 *mypool2 = pool2 + (unsigned long long)l * pool2_cap;
+  const uint2 *meta_l = seg_meta + (int64_t)l * nseg * Tn;
+  auto key_of = [&](const uint2 &e) { return rank_key<KB>(Elem<T>::to_f32(Elem<T>::from_raw(e.y))); };
+  for (int64_t t = (int64_t)blockIdx.x * nwv + wv; t < Tn; t += (int64_t)gridDim.x * nwv) {
+    uint2 m[SPL];
+#pragma unroll
+    for (int q = 0; q < SPL; ++q) {
+      const int g = lane * SPL + q;
+      m[q] = g < nseg ? meta_l[(int64_t)g * Tn + t] : make_uint2(0u, 0u);
+    }
+    uint2 ent[SPL][GE];
+#pragma unroll
+    for (int q = 0; q < SPL; ++q)
+#pragma unroll
+      for (int e = 0; e < GE; ++e) ent[q][e] = (uint32_t)e < m[q].y ? mypool[m[q].x + e] : make_uint2(0u, 0u);
+    uint32_t ngt = 0, neq = 0;
+    bool longrun = false;
+#pragma unroll
+    for (int q = 0; q < SPL; ++q) {
+#pragma unroll
+      for (int e = 0; e < GE; ++e)
+        if ((uint32_t)e < m[q].y) {
+          const uint32_t key = key_of(ent[q][e]);
+          ngt += key > s.thr_key ? 1u : 0u;
+          neq += key == s.thr_key ? 1u : 0u;
+        }
+      for (uint32_t e = GE; e < m[q].y; ++e) {
+        const uint32_t key = key_of(mypool[m[q].x + e]);
+        ngt += key > s.thr_key ? 1u : 0u;
+        neq += key == s.thr_key ? 1u : 0u;
+        longrun = true;
+      }
+    }
+    const uint32_t n = ngt + neq;
+    // both prefix sums in one scan: totals stay below 2^16 per field only if the row is short
+    // enough, so scan them separately
+    const uint32_t incl = wave_inclusive_scan(n);
+    const uint32_t total = __builtin_amdgcn_readlane(incl, 63);
+    const uint32_t tot_gt = __builtin_amdgcn_readlane(wave_inclusive_scan(ngt), 63);
+    const int64_t r = (int64_t)l * Tn + t;
+    uint32_t off = 0;
+    if (total > 0 && lane == 0) off = atomicAdd(&pool2_count[l], total + 1u);
+    off = __builtin_amdgcn_readfirstlane(off);
+    if (lane == 0) {
+      row_gt[r] = tot_gt; row_eq[r] = total - tot_gt;
+      row_first[r] = total > 0 ? off : ROW_NONE;
+      if (total > 0) mypool2[off] = make_uint2(ROW_NONE, total);
+    }
+    if (n > 0) {
+      uint32_t pos = off + 1u + incl - n;
+#pragma unroll
+      for (int q = 0; q < SPL; ++q) {
+#pragma unroll
+        for (int e = 0; e < GE; ++e)
+          if ((uint32_t)e < m[q].y && key_of(ent[q][e]) >= s.thr_key) mypool2[pos++] = ent[q][e];
+        if (longrun)
+          for (uint32_t e = GE; e < m[q].y; ++e) {
+            const uint2 en = mypool[m[q].x + e];
+            if (key_of(en) >= s.thr_key) mypool2[pos++] = en;
+          }
+      }
+    }
   }
 }
 
@@ -943,7 +1103,7 @@ static int run_batchtopk(const T *pre, int64_t Tn, int64_t F, int64_t L, int64_t
   if (K > N) K = N;
   const int nprob = lo.nprob;
   k_sample_keys<T, GLOBAL><<<dim3(SAMPLE_BLOCKS, nprob), 256, 0, stream>>>(pre, Tn, F, L, lstride, mean, denom, N, sample);
-  k_sample_cut<KB><<<nprob, SCAN_THREADS, 0, stream>>>(sample, N, K, st, hist, poolcnt);
+  k_sample_cut<KB><<<nprob, SCAN_THREADS, 0, stream>>>(sample, N, K, st, hist, poolcnt, nullptr, PATH_ROWS);
   // two rows per wavefront: many more blocks than fit at once, so rows of very different
   // candidate counts balance out over the CUs
   int gx = (int)clt_ceil_div(Tn, 8);
@@ -966,7 +1126,7 @@ static int run_batchtopk(const T *pre, int64_t Tn, int64_t F, int64_t L, int64_t
   k_select_count<T, GLOBAL><<<grid2, 256, 0, stream>>>(pre, Tn, F, L, lstride, mean, denom, st, first, pool, lo.pool_cap, rgt, req);
   k_select_allot<GLOBAL><<<nprob, SCAN_THREADS, 0, stream>>>(st, Tn, L, rgt, req, allot, keep, row_ptr, K);
   if (GLOBAL) k_rowptr_scan<<<1, SCAN_THREADS, 0, stream>>>(keep, L * Tn, row_ptr);
-  k_select_emit<T, GLOBAL><<<grid2, 256, 0, stream>>>(pre, Tn, F, L, lstride, mean, denom, st, first, pool, lo.pool_cap, allot, row_ptr, col, val);
+  k_select_emit<T, GLOBAL><<<grid2, 256, 0, stream>>>(pre, Tn, F, L, lstride, mean, denom, st, first, pool, lo.pool_cap, allot, row_ptr, col, val, nullptr, 0);
   return clt_check_launch();
 }
 
@@ -1015,7 +1175,187 @@ static int dispatch_threshold(bool emit, const void *pre, int64_t Tn, int64_t F,
 #undef CLT_TH
 }
 
+// ---- encoder-collected candidates: workspace and the two halves of the fused path ---------
+struct TileLayout {
+  SelLayout sel;
+  size_t off_tmeta, off_meta, off_tpool, off_pool2, off_pool2cnt, off_tcount, total;
+  unsigned long long tpool_cap, pool2_cap;   // entries per layer
+  uint32_t caps;                             // entries per fixed tile slot
+  int nseg, ntile;
+};
+
+static TileLayout tile_layout(int64_t T, int64_t F, int64_t L, int64_t k, int dtype) {
+  TileLayout tl;
+  tl.sel = sel_layout(T, F, L, k, CLT_TOPK_PER_LAYER);
+  const int segw = dtype == CLT_BF16 ? 128 : 64;
+  tl.nseg = (int)(F / segw);
+  tl.ntile = tl.nseg * (int)(T / 128);
+  // about 2.3x K candidates are expected, i.e. 2.3 * k / F of a tile's 128 * segw elements; a
+  // slot holds three times that (at least 64, at most the whole tile)
+  unsigned long long caps = (unsigned long long)(3.0 * 2.3 * (double)k / (double)F * 128.0 * segw) + 64ull;
+  if (caps > 128ull * segw) caps = 128ull * segw;
+  tl.caps = (uint32_t)caps;
+  const unsigned long long N = (unsigned long long)T * F;
+  unsigned long long K = (unsigned long long)k * T;
+  if (K > N) K = N;
+  unsigned long long dyn = 2ull * K + 4096ull;
+  if (dyn > N) dyn = N;
+  tl.tpool_cap = (unsigned long long)tl.ntile * caps + dyn;
+  tl.pool2_cap = (tl.tpool_cap < N ? tl.tpool_cap : N) + (unsigned long long)T;   // + one header per row
+  size_t o = tl.sel.total;
+  auto take = [&](size_t bytes) { size_t at = o; o += (bytes + 255) & ~(size_t)255; return at; };
+  tl.off_tmeta = take(8 * (size_t)tl.ntile * (size_t)L);
+  tl.off_meta = take(8 * (size_t)tl.nseg * (size_t)T * (size_t)L);
+  tl.off_tpool = take(8 * (size_t)tl.tpool_cap * (size_t)L);
+  tl.off_pool2 = take(8 * (size_t)tl.pool2_cap * (size_t)L);
+  tl.off_pool2cnt = take(4 * (size_t)L);
+  tl.off_tcount = take(4 * (size_t)L);
+  tl.total = o;
+  return tl;
+}
+
+template <typename T>
+static int run_encode_collect(const void *x, const void *w, const void *b, void *pre, int64_t Tn, int64_t d,
+                              int64_t F, int64_t L, int64_t xs, int64_t wstr, int64_t bs, int64_t ps, int64_t k,
+                              int dtype, char *ws, hipStream_t stream) {
+  constexpr int KB = Elem<T>::KEYBITS;
+  const TileLayout tl = tile_layout(Tn, F, L, k, dtype);
+  const SelLayout &lo = tl.sel;
+  SelState *st = (SelState *)(ws + lo.off_state);
+  uint32_t *hist = (uint32_t *)(ws + lo.off_hist);
+  uint32_t *poolcnt = (uint32_t *)(ws + lo.off_poolcnt);
+  uint32_t *sample = (uint32_t *)(ws + lo.off_sample);
+  const unsigned long long N = (unsigned long long)Tn * (unsigned long long)F;
+  unsigned long long K = (unsigned long long)k * (unsigned long long)Tn;
+  if (K > N) K = N;
+  k_sample_dot<T><<<dim3(SAMPLE_TOK, (unsigned)L), 256, 0, stream>>>((const T *)x, (const T *)w, (const T *)b, Tn, d, F,
+                                                                      xs, wstr, bs, sample);
+  // (the second counter array handed to k_sample_cut is [pool2 counters | tile-pool counters])
+  k_sample_cut<KB><<<(unsigned)L, SCAN_THREADS, 0, stream>>>(sample, N, K, st, hist, poolcnt,
+                                                              (uint32_t *)(ws + tl.off_pool2cnt), PATH_TILES);
+  k_fill_u32<<<1, 256, 0, stream>>>((uint32_t *)(ws + tl.off_tcount), 0u, L);
+  uint2 *tpool = (uint2 *)(ws + tl.off_tpool);
+  CollectArgs ca;
+  ca.st = st; ca.pool_count = (uint32_t *)(ws + tl.off_tcount); ca.pool = tpool; ca.pool_cap = tl.tpool_cap;
+  ca.tile_meta = (uint2 *)(ws + tl.off_tmeta); ca.seg_meta = (uint2 *)(ws + tl.off_meta); ca.caps = tl.caps;
+  ca.theta = nullptr; ca.theta_stride = 0;
+  int rc = clt_launch_encode(x, w, b, nullptr, Tn, d, F, L, xs, wstr, bs, ps, dtype, 1, nullptr, &ca, stream);
+  if (rc != CLT_OK) return rc;
+  k_pool_hist<T><<<dim3(256, (unsigned)L), 256, 0, stream>>>(st, ca.tile_meta, tl.ntile, tpool, tl.tpool_cap, hist, 0);
+  k_select_scan<KB><<<(unsigned)L, SCAN_THREADS, 0, stream>>>(st, hist, poolcnt, 0, 0);
+  // layers whose cut failed (too few candidates, or no pool space left) get their pre-activations
+  // written out and go through the streaming pass; the launch does nothing for the others
+  return clt_launch_encode(x, w, b, pre, Tn, d, F, L, xs, wstr, bs, ps, dtype, 0, st, nullptr, stream);
+}
+
+template <typename T>
+static int run_collect_select(const T *pre, int64_t Tn, int64_t F, int64_t L, int64_t lstride, int64_t k, int dtype,
+                              int32_t *row_ptr, int32_t *col, T *val, char *ws, hipStream_t stream) {
+  constexpr int KB = Elem<T>::KEYBITS;
+  constexpr int VV = Elem<T>::VEC;
+  const TileLayout tl = tile_layout(Tn, F, L, k, dtype);
+  const SelLayout &lo = tl.sel;
+  SelState *st = (SelState *)(ws + lo.off_state);
+  uint32_t *hist = (uint32_t *)(ws + lo.off_hist);
+  uint32_t *poolcnt = (uint32_t *)(ws + lo.off_poolcnt);
+  uint32_t *first = (uint32_t *)(ws + lo.off_first);
+  uint32_t *rgt = (uint32_t *)(ws + lo.off_gt), *req = (uint32_t *)(ws + lo.off_eq);
+  uint32_t *allot = (uint32_t *)(ws + lo.off_allot), *keep = (uint32_t *)(ws + lo.off_keep);
+  uint2 *pool = (uint2 *)(ws + lo.off_pool);
+  uint2 *pool2 = (uint2 *)(ws + tl.off_pool2);
+  uint32_t *pool2cnt = (uint32_t *)(ws + tl.off_pool2cnt);
+  const uint2 *meta = (const uint2 *)(ws + tl.off_meta);
+  const uint2 *tmeta = (const uint2 *)(ws + tl.off_tmeta);
+  const uint2 *tpool = (const uint2 *)(ws + tl.off_tpool);
+  const unsigned long long N = (unsigned long long)Tn * (unsigned long long)F;
+  unsigned long long K = (unsigned long long)k * (unsigned long long)Tn;
+  if (K > N) K = N;
+  int gx = (int)clt_ceil_div(Tn, 8);
+  if (gx > 65535 * 8) gx = 65535 * 8;
+  // retry of the layers whose cut failed: streaming pass from the bottom key over `pre`
+  k_select_pass<T, VV, false><<<dim3(gx, (unsigned)L), 256, 0, stream>>>(pre, Tn, F, L, lstride, nullptr, nullptr, st, hist,
+                                                                        poolcnt, pool, lo.pool_cap, first, 1);
+  k_select_scan<KB><<<(unsigned)L, SCAN_THREADS, 0, stream>>>(st, hist, poolcnt, 1, 0);
+  int gx2 = (int)clt_ceil_div(Tn, 4);
+  int maxgx2 = (int)clt_ceil_div(256 * 8, L);
+  if (maxgx2 < 1) maxgx2 = 1;
+  if (gx2 > maxgx2) gx2 = maxgx2;
+  dim3 grid2(gx2, (unsigned)L);
+  const int nlev = KB == 32 ? 3 : 2;
+  for (int level = 1; level < nlev; ++level) {
+    k_pool_hist<T><<<dim3(256, (unsigned)L), 256, 0, stream>>>(st, tmeta, tl.ntile, tpool, tl.tpool_cap, hist, level);
+    k_select_level<T, false><<<grid2, 256, 0, stream>>>(pre, Tn, F, L, lstride, nullptr, nullptr, st, hist, first, pool, lo.pool_cap, level);
+    k_select_scan<KB><<<(unsigned)L, SCAN_THREADS, 0, stream>>>(st, hist, poolcnt, 2, level);
+  }
+  // one wavefront per row, all rows at once: these two kernels wait on scattered small reads
+  dim3 grid3((unsigned)clt_ceil_div(Tn, 4), (unsigned)L);
+  const int spl = (tl.nseg + 63) / 64;
+#define CLT_GATHER(S) k_row_gather<T, S><<<grid3, 256, 0, stream>>>(Tn, st, meta, tl.nseg, tpool, tl.tpool_cap, pool2cnt, pool2, tl.pool2_cap, first, rgt, req)
+  if (spl <= 1) CLT_GATHER(1);
+  else if (spl == 2) CLT_GATHER(2);
+  else if (spl == 3) CLT_GATHER(3);
+  else if (spl == 4) CLT_GATHER(4);
+  else if (spl <= 8) CLT_GATHER(8);
+  else return CLT_ERR_RANGE;
+#undef CLT_GATHER
+  k_select_count<T, false><<<grid2, 256, 0, stream>>>(pre, Tn, F, L, lstride, nullptr, nullptr, st, first, pool, lo.pool_cap, rgt, req);
+  k_select_allot<false><<<(unsigned)L, SCAN_THREADS, 0, stream>>>(st, Tn, L, rgt, req, allot, keep, row_ptr, K);
+  k_select_emit<T, false><<<grid3, 256, 0, stream>>>(pre, Tn, F, L, lstride, nullptr, nullptr, st, first, pool, lo.pool_cap, allot,
+                                                     row_ptr, col, val, pool2, tl.pool2_cap);
+  return clt_check_launch();
+}
+
 }  // namespace
+
+extern "C" int clt_encode_collect_supported(const void *x, const void *w, const void *b, int64_t T, int64_t d,
+                                            int64_t F, int64_t L, int64_t x_layer_stride, int64_t w_layer_stride,
+                                            int64_t b_layer_stride, int64_t k, int dtype) {
+  if (dtype != CLT_F32 && dtype != CLT_BF16) return 0;
+  if (T <= 0 || d <= 0 || F <= 0 || L <= 0 || L > 65535 || k <= 0 || !x || !w) return 0;
+  if ((double)T * (double)F >= 4294967296.0) return 0;
+  if (F / (dtype == CLT_BF16 ? 128 : 64) > 512) return 0;            // feature segments one wavefront can walk
+  if (tile_layout(T, F, L, k, dtype).tpool_cap >= 0xFFF00000ull) return 0;
+  return clt_encode_can_collect(x, w, b, T, d, F, x_layer_stride, w_layer_stride, b_layer_stride, dtype) ? 1 : 0;
+}
+
+extern "C" size_t clt_encode_collect_workspace_bytes(int64_t T, int64_t d, int64_t F, int64_t L, int64_t k, int dtype) {
+  (void)d;
+  if (T <= 0 || F <= 0 || L <= 0) return 256;
+  if (k < 0) k = 0;
+  return tile_layout(T, F, L, k, dtype).total;
+}
+
+extern "C" int clt_encode_collect(const void *x, const void *w, const void *b, void *pre, int64_t T, int64_t d,
+                                  int64_t F, int64_t L, int64_t x_layer_stride, int64_t w_layer_stride,
+                                  int64_t b_layer_stride, int64_t pre_layer_stride, int64_t k, int dtype,
+                                  void *workspace, size_t workspace_bytes, void *stream) {
+  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (!pre || !workspace) return CLT_ERR_ARG;
+  if (!clt_encode_collect_supported(x, w, b, T, d, F, L, x_layer_stride, w_layer_stride, b_layer_stride, k, dtype))
+    return CLT_ERR_ARG;
+  if (workspace_bytes < clt_encode_collect_workspace_bytes(T, d, F, L, k, dtype)) return CLT_ERR_WORKSPACE;
+  if ((((uintptr_t)workspace) & 255u) != 0) return CLT_ERR_ALIGN;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == CLT_BF16)
+    return run_encode_collect<bf16_t>(x, w, b, pre, T, d, F, L, x_layer_stride, w_layer_stride, b_layer_stride,
+                                      pre_layer_stride, k, dtype, (char *)workspace, s);
+  return run_encode_collect<float>(x, w, b, pre, T, d, F, L, x_layer_stride, w_layer_stride, b_layer_stride,
+                                   pre_layer_stride, k, dtype, (char *)workspace, s);
+}
+
+extern "C" int clt_collect_select(const void *pre, int64_t T, int64_t F, int64_t L, int64_t pre_layer_stride, int64_t k,
+                                  int dtype, int32_t *row_ptr, int32_t *col, void *val, void *workspace,
+                                  size_t workspace_bytes, void *stream) {
+  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (T <= 0 || F <= 0 || L <= 0 || L > 65535 || k <= 0) return CLT_ERR_ARG;
+  if (!pre || !row_ptr || !col || !val || !workspace) return CLT_ERR_ARG;
+  if (workspace_bytes < clt_encode_collect_workspace_bytes(T, 0, F, L, k, dtype)) return CLT_ERR_WORKSPACE;
+  if ((((uintptr_t)workspace) & 255u) != 0) return CLT_ERR_ALIGN;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == CLT_BF16)
+    return run_collect_select<bf16_t>((const bf16_t *)pre, T, F, L, pre_layer_stride, k, dtype, row_ptr, col, (bf16_t *)val, (char *)workspace, s);
+  return run_collect_select<float>((const float *)pre, T, F, L, pre_layer_stride, k, dtype, row_ptr, col, (float *)val, (char *)workspace, s);
+}
 
 extern "C" size_t clt_batchtopk_workspace_bytes(int64_t T, int64_t F, int64_t L, int64_t k, int mode, int dtype) {
   (void)dtype;

@@ -128,6 +128,15 @@ class Encoder(nn.Module):
     def encode_slab(self, inputs: Dict[int, torch.Tensor], out: Optional[torch.Tensor] = None):
         """All given layers in one launch.  Returns (sorted layers, pre [n, T, F]) or None when
         some input needs the per-layer fallbacks (bad shape, unequal token counts, bad index)."""
+        prep = self.prepare_slab(inputs)
+        if prep is None:
+            return None
+        layers, x_slab, ws, bs = prep
+        return layers, engine.encode(x_slab, ws, bs, out=out)
+
+    def prepare_slab(self, inputs: Dict[int, torch.Tensor]):
+        """(sorted layers, x [n, T, d], weights [n, F, d], biases [n, F]) of the given layers, or
+        None when some input needs the per-layer fallbacks."""
         layers = sorted(inputs.keys())
         if not layers:
             return None
@@ -151,7 +160,7 @@ class Encoder(nn.Module):
         else:
             idx = torch.tensor(layers, device=w.device)
             ws, bs = w.index_select(0, idx), b.index_select(0, idx)
-        return layers, engine.encode(x_slab, ws, bs, out=out)
+        return layers, x_slab, ws, bs
 
 
 def _as_slab(flats: List[torch.Tensor]) -> torch.Tensor:

@@ -140,6 +140,54 @@ def batchtopk_select(pre: torch.Tensor, k: int, global_mode: bool, ws: Optional[
     return SurvivorList(row_ptr, col[:total], val[:total], T, F, L, pre.dtype)
 
 
+def encode_collect_supported(x: torch.Tensor, w: torch.Tensor, b: Optional[torch.Tensor], k: int) -> bool:
+    """True when encode_collect can run these shapes (else: encode, then batchtopk_select)."""
+    if not x.is_cuda or k <= 0:
+        return False
+    L, T, d = x.shape
+    F = w.shape[1]
+    return bool(nat.load().clt_encode_collect_supported(
+        nat.ptr(x), nat.ptr(w), nat.ptr(b), T, d, F, L, x.stride(0), w.stride(0),
+        b.stride(0) if b is not None else 0, int(k), nat.dtype_code(x.dtype)))
+
+
+def encode_collect(x: torch.Tensor, w: torch.Tensor, b: Optional[torch.Tensor], k: int, pre_scratch: torch.Tensor,
+                   ws: Workspace):
+    """First half of the fused per-layer BatchTopK path: the encoder projection whose epilogue
+    keeps only the candidates above a sampled cut (encoder.py:151-162 + activations.py:11-36).
+    Returns the handle that collect_select needs."""
+    nat.require_device(x, "encode_collect")
+    L, T, d = x.shape
+    F = w.shape[1]
+    assert w.shape == (L, F, d) and x.dtype == w.dtype and pre_scratch.shape == (L, T, F)
+    assert pre_scratch.dtype == x.dtype and pre_scratch.stride(2) == 1 and pre_scratch.stride(1) == F
+    lib = nat.load()
+    dt = nat.dtype_code(x.dtype)
+    nbytes = lib.clt_encode_collect_workspace_bytes(T, d, F, L, int(k), dt)
+    wbuf = ws.get("collect", nbytes)
+    code = lib.clt_encode_collect(nat.ptr(x), nat.ptr(w), nat.ptr(b), nat.ptr(pre_scratch), T, d, F, L,
+                                  x.stride(0), w.stride(0), b.stride(0) if b is not None else 0,
+                                  pre_scratch.stride(0), int(k), dt, nat.ptr(wbuf), wbuf.numel(), _stream(x))
+    nat.check(code, "clt_encode_collect")
+    return (pre_scratch, int(k), wbuf)
+
+
+def collect_select(handle) -> SurvivorList:
+    """Second half: exact per-layer BatchTopK on the collected candidates."""
+    pre, k, wbuf = handle
+    L, T, F = pre.shape
+    dev = pre.device
+    total = L * min(k * T, T * F)
+    row_ptr = torch.empty(L * T + 1, dtype=torch.int32, device=dev)
+    col = torch.empty(max(total, 1), dtype=torch.int32, device=dev)
+    val = torch.empty(max(total, 1), dtype=pre.dtype, device=dev)
+    code = nat.load().clt_collect_select(nat.ptr(pre), T, F, L, pre.stride(0), k, nat.dtype_code(pre.dtype),
+                                         nat.ptr(row_ptr), nat.ptr(col), nat.ptr(val), nat.ptr(wbuf), wbuf.numel(),
+                                         _stream(pre))
+    nat.check(code, "clt_collect_select")
+    return SurvivorList(row_ptr, col[:total], val[:total], T, F, L, pre.dtype)
+
+
 def tokentopk_select(pre: torch.Tensor, kk: int, global_mode: bool, ws: Optional[Workspace] = None,
                      stats=None) -> SurvivorList:
     """TokenTopK survivors, kk already resolved to a count (activations.py:99-128, 391-491)."""

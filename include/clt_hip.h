@@ -112,6 +112,42 @@ int clt_batchtopk_select(const void *pre, int64_t T, int64_t F, int64_t L,
                          void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * Encoder projection and per-layer BatchTopK in one path, without writing the dense
+ * pre-activations: the encoder's epilogue compares every value with a per-layer cut found
+ * from a small sample beforehand and appends the ones that reach it to a candidate pool; the
+ * exact selection (same result as clt_encode followed by clt_batchtopk_select with
+ * CLT_TOPK_PER_LAYER, same tie rule) then runs on the pool only.
+ *   clt_encode_collect   sample, cut, encoder with the collecting epilogue, first histogram
+ *   clt_collect_select   threshold, tie allotment, ordered write of row_ptr / col / val
+ * Both calls take the same workspace (clt_encode_collect_workspace_bytes) and must run on
+ * the same stream, clt_collect_select after clt_encode_collect.
+ * `pre` [L][T][F] is scratch: it is written only for a layer whose cut turned out unusable
+ * (fewer than k*T candidates, or no pool space left), which then takes the streaming route.
+ * clt_encode_collect_supported returns 1 when the shapes qualify (T % 256 == 0,
+ * F % 256 == 0, d % 128 == 0 for bf16 / d % 64 == 0 for fp32, 16-byte aligned rows, k > 0),
+ * else 0; callers then use clt_encode + clt_batchtopk_select.
+ * Replaces the same reference calls as clt_encode and clt_batchtopk_select
+ * (clt/models/encoder.py:151-162, clt/activations/registry.py:43-72,
+ * clt/models/activations.py:11-36).
+ */
+int clt_encode_collect_supported(const void *x, const void *w, const void *b,
+                                 int64_t T, int64_t d, int64_t F, int64_t L,
+                                 int64_t x_layer_stride, int64_t w_layer_stride,
+                                 int64_t b_layer_stride, int64_t k, int dtype);
+size_t clt_encode_collect_workspace_bytes(int64_t T, int64_t d, int64_t F, int64_t L,
+                                          int64_t k, int dtype);
+int clt_encode_collect(const void *x, const void *w, const void *b, void *pre,
+                       int64_t T, int64_t d, int64_t F, int64_t L,
+                       int64_t x_layer_stride, int64_t w_layer_stride,
+                       int64_t b_layer_stride, int64_t pre_layer_stride,
+                       int64_t k, int dtype, void *workspace, size_t workspace_bytes,
+                       void *stream);
+int clt_collect_select(const void *pre, int64_t T, int64_t F, int64_t L,
+                       int64_t pre_layer_stride, int64_t k, int dtype,
+                       int32_t *row_ptr, int32_t *col, void *val,
+                       void *workspace, size_t workspace_bytes, void *stream);
+
+/*
  * TokenTopK selection: per token row, the kk largest of its F (per layer) or L*F
  * (global, ranked on the z-score as above) entries.  kk is the already resolved
  * integer count (fraction/ceil rule of clt/models/activations.py:108-116).
@@ -175,11 +211,12 @@ int clt_pack_decoder(const void *w_ref, void *w_packed, int64_t d, int64_t F,
  * for all targets that CrossLayerTranscoder.forward loops over
  * (clt/models/clt.py:192-199).
  * Limits: L <= 64; d % 8 == 0 (bf16) / d % 4 == 0 (fp32) on the fast path.
- * workspace: NULL runs one wavefront per (target, token) over all features.  With a
- * workspace of clt_decode_workspace_bytes() the feature axis is cut into 8 slices, one per
- * XCD, so that each slice of a decoder matrix stays in one L2 while all tokens pass; the
- * per-slice fp32 partial rows are then summed in a fixed order.  Both give the same result
- * up to fp32 summation order.
+ * workspace: NULL runs one wavefront per (target, token) over all features and sources.
+ * With a workspace of clt_decode_workspace_bytes() the feature axis is cut into 8 slices,
+ * one per XCD, and there is one launch per source layer, so that each slice of a decoder
+ * matrix stays in one L2 while all tokens pass; partial sums live as fp32 rows per (slice,
+ * target, token) in the workspace and are added in a fixed order at the end.  Both give the
+ * same result up to fp32 summation order.
  */
 size_t clt_decode_workspace_bytes(int64_t T, int64_t d, int64_t F, int64_t L);
 int clt_decode_sparse(const int32_t *row_ptr, const int32_t *col, const void *val,

@@ -168,6 +168,78 @@ def test_batchtopk_k_zero_and_empty(dev):
 
 
 # ---- BatchTopK global ------------------------------------------------------------------------
+# ---- encoder with the collecting epilogue + BatchTopK on the candidates --------------------
+def fused_vs_separate(x, w, b, k, dev):
+    """The fused path must give the survivor list of encode -> batchtopk_select, bit for bit."""
+    xd, wd, bd = x.to(dev), w.to(dev), (b.to(dev) if b is not None else None)
+    assert engine.encode_collect_supported(xd, wd, bd, k)
+    pre = engine.encode(xd, wd, bd)
+    ref = engine.batchtopk_select(pre, k, False)
+    ws = engine.Workspace(xd.device)
+    scratch = torch.full_like(pre, float("nan"))
+    got = engine.collect_select(engine.encode_collect(xd, wd, bd, k, scratch, ws))
+    torch.cuda.synchronize()
+    assert torch.equal(got.row_ptr.cpu(), ref.row_ptr.cpu())
+    assert torch.equal(got.col.cpu(), ref.col.cpu())
+    assert torch.equal(got.val.cpu().view(torch.int16 if x.dtype == torch.bfloat16 else torch.int32),
+                       ref.val.cpu().view(torch.int16 if x.dtype == torch.bfloat16 else torch.int32))
+    return pre.cpu(), got
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("L,T,d,F,k", [(1, 256, 128, 256, 3), (2, 512, 256, 1024, 20), (3, 256, 768, 512, 64),
+                                       (2, 768, 128, 2048, 200)])
+def test_encode_collect_matches_separate_and_oracle(dev, dtype, L, T, d, F, k):
+    g = torch.Generator().manual_seed(L * 31 + T + F + k)
+    x = torch.randn(L, T, d, generator=g).to(dtype)
+    w = (torch.randn(L, F, d, generator=g) / math.sqrt(d)).to(dtype)
+    b = (0.1 * torch.randn(L, F, generator=g)).to(dtype)
+    pre, got = fused_vs_separate(x, w, b, k, dev)
+    check_rows_sorted(got)
+    assert got.nnz == L * min(k * T, T * F)
+    assert torch.equal(dense_from(got), oracle_per_layer(pre, k))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_encode_collect_heavy_ties(dev, dtype):
+    # small-integer inputs and weights: the pre-activations are exact small integers, so
+    # thousands of them tie at the threshold and the lowest flat indices must win
+    g = torch.Generator().manual_seed(5)
+    L, T, d, F, k = 2, 512, 128, 1024, 30
+    x = torch.randint(-1, 2, (L, T, d), generator=g).to(dtype)
+    w = torch.randint(-1, 2, (L, F, d), generator=g).to(dtype)
+    pre, got = fused_vs_separate(x, w, None, k, dev)
+    assert torch.equal(dense_from(got), oracle_per_layer(pre, k))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_encode_collect_unusable_cut_takes_streaming_route(dev, dtype):
+    # almost every pre-activation is exactly 0 and K reaches into the zeros: every element
+    # reaches the sampled cut, the candidate pool overflows, and the layer must be redone from
+    # the dense pre-activations (written to the scratch buffer for that purpose)
+    g = torch.Generator().manual_seed(9)
+    L, T, d, F, k = 2, 512, 128, 2048, 8
+    x = torch.zeros(L, T, d)
+    x[:, ::64] = torch.randn(L, T // 64, d, generator=g)
+    w = (torch.randn(L, F, d, generator=g) / math.sqrt(d))
+    pre, got = fused_vs_separate(x.to(dtype), w.to(dtype), None, k, dev)
+    assert got.nnz == L * k * T
+    assert torch.equal(dense_from(got), oracle_per_layer(pre, k))
+
+
+def test_encode_collect_all_selected_and_shape_gate(dev):
+    g = torch.Generator().manual_seed(2)
+    L, T, d, F = 1, 256, 128, 256
+    x = torch.randn(L, T, d, generator=g).to(torch.bfloat16)
+    w = torch.randn(L, F, d, generator=g).to(torch.bfloat16)
+    pre, got = fused_vs_separate(x, w, None, F + 5, dev)          # k >= F: everything survives
+    assert got.nnz == T * F
+    # shapes the collecting epilogue does not take
+    assert not engine.encode_collect_supported(x[:, :200].contiguous().to(dev), w.to(dev), None, 4)
+    assert not engine.encode_collect_supported(x.to(dev), w[:, :136].contiguous().to(dev), None, 4)
+    assert not engine.encode_collect_supported(x.to(dev), w.to(dev), None, 0)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("L,T,F,k", [(2, 2, 2, 1), (3, 64, 128, 6), (4, 200, 520, 12)])
 def test_batchtopk_global(dev, dtype, L, T, F, k):
