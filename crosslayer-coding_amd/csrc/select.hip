@@ -192,13 +192,13 @@ __global__ __launch_bounds__(256) void k_sample_keys(
 template <int KB>
 __global__ __launch_bounds__(SCAN_THREADS) void k_sample_cut(
     const uint32_t *sample, unsigned long long N, unsigned long long K, SelState *st, uint32_t *hist,
-    uint32_t *pool_count, uint32_t *pool2_count, uint32_t path) {
+    uint32_t *pool_count, uint32_t *aux_count, uint32_t path) {
   constexpr int PER = SAMPLE_N / SCAN_THREADS;
   __shared__ uint32_t lh[NBINS];
   const int p = blockIdx.x, tid = threadIdx.x;
   const unsigned long long ns = N < (unsigned long long)SAMPLE_N ? N : (unsigned long long)SAMPLE_N;
   for (int i = tid; i < NBINS; i += SCAN_THREADS) hist[(int64_t)p * NBINS + i] = 0;
-  if (tid == 0) { pool_count[p] = 0; if (pool2_count) pool2_count[p] = 0; }
+  if (tid == 0) { pool_count[p] = 0; if (aux_count) aux_count[p] = 0; }
   uint32_t keys[PER];
   bool valid[PER];
 #pragma unroll
@@ -633,12 +633,10 @@ template <typename T, bool GLOBAL>
 __global__ __launch_bounds__(256) void k_select_emit(
     const T *pre, int64_t Tn, int64_t F, int64_t L, int64_t lstride, const float *mean,
     const float *denom, const SelState *st, const uint32_t *row_first, const uint2 *pool,
-    unsigned long long pool_cap, const uint32_t *allot, const int32_t *row_ptr, int32_t *col_out, T *val_out,
-    const uint2 *pool2, unsigned long long pool2_cap) {
+    unsigned long long pool_cap, const uint32_t *allot, const int32_t *row_ptr, int32_t *col_out, T *val_out) {
   const int l = blockIdx.y, p = GLOBAL ? 0 : l;
   const SelState s = st[p];
-  // candidates collected by the encoder were regrouped per row into the second pool
-  if (s.path == PATH_TILES) { pool = pool2; pool_cap = pool2_cap; }
+  if (s.path != PATH_ROWS) return;
   const int wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
   typename RankOf<T, GLOBAL>::type rk = RankOf<T, GLOBAL>::make(mean, denom, l, F);
   for (int64_t t = (int64_t)blockIdx.x * nwv + wv; t < Tn; t += (int64_t)gridDim.x * nwv) {
@@ -681,7 +679,9 @@ __global__ __launch_bounds__(256) void k_sample_dot(
   const int64_t tok = (int64_t)hash_index((uint64_t)ti * 131u + (uint64_t)l * 7919u, (uint64_t)Tn);
   const T *xr = x + (int64_t)l * xs + tok * d;
   const int64_t nch = d / V;   // 16-byte chunks per row (the collecting encoder needs d % V == 0)
-  for (int j0 = wv * NJ; j0 < NFEAT; j0 += nwv * NJ) {
+  // blockIdx.z cuts the features of this token into gridDim.z groups
+  const int jper = NFEAT / (int)gridDim.z, jb = (int)blockIdx.z * jper;
+  for (int j0 = jb + wv * NJ; j0 < jb + jper; j0 += nwv * NJ) {
     const T *wr[NJ];
     int64_t f[NJ];
     float acc[NJ];
@@ -731,11 +731,17 @@ __global__ __launch_bounds__(256) void k_pool_hist(const SelState *st, const uin
   const uint2 *mypool = pool + (unsigned long long)p * pool_cap;
   for (int i = blockIdx.x * nwv + wv; i < ntile; i += gridDim.x * nwv) {
     const uint2 tm = tile_meta[(int64_t)p * ntile + i];
-    for (uint32_t e = lane; e < tm.y; e += 64) {
-      const uint32_t key = rank_key<KB>(Elem<T>::to_f32(Elem<T>::from_raw(mypool[tm.x + e].y)));
-      const uint32_t diff = key - s.cut_key;
-      if (level == 0) atomicAdd(&lh[bin_level0<KB>(diff)], 1u);
-      else if (diff >= s.flo && diff <= s.fhi) atomicAdd(&lh[(diff - s.bbase) >> s.shift], 1u);
+    for (uint32_t e0 = 0; e0 < tm.y; e0 += 256) {
+      uint32_t raw[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) { const uint32_t e = e0 + q * 64 + lane; raw[q] = e < tm.y ? mypool[tm.x + e].y : 0u; }
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        if (e0 + q * 64 + lane >= tm.y) continue;
+        const uint32_t diff = rank_key<KB>(Elem<T>::to_f32(Elem<T>::from_raw(raw[q]))) - s.cut_key;
+        if (level == 0) atomicAdd(&lh[bin_level0<KB>(diff)], 1u);
+        else if (diff >= s.flo && diff <= s.fhi) atomicAdd(&lh[(diff - s.bbase) >> s.shift], 1u);
+      }
     }
   }
   __syncthreads();
@@ -745,87 +751,111 @@ __global__ __launch_bounds__(256) void k_pool_hist(const SelState *st, const uin
   }
 }
 
-// One wavefront per row: walks the row's runs in all feature segments (lane -> consecutive
-// segments, so lane order is feature order), counts the entries above / equal to the threshold
-// key and copies them, in feature order, to one extent of the second pool (same extent format
-// as the streaming pass writes: a header entry (next, count), then the entries).
-// SPL = segments per lane.  The first GE entries of each run are fetched in one batch and kept
-// in registers; only a run longer than that is walked again for the copy.
-template <typename T, int SPL>
-__global__ __launch_bounds__(256) void k_row_gather(
-    int64_t Tn, const SelState *st, const uint2 *seg_meta, int nseg, const uint2 *pool, unsigned long long pool_cap,
-    uint32_t *pool2_count, uint2 *pool2, unsigned long long pool2_cap, uint32_t *row_first, uint32_t *row_gt,
-    uint32_t *row_eq) {
+// The three kernels below finish the selection on the encoder-collected candidates.  They all
+// map a wavefront to 64 consecutive token rows of one feature segment (lane = row): the rows'
+// bookkeeping entries are adjacent in seg_meta and their runs are adjacent in the tile extent,
+// so every access of a wavefront is (nearly) contiguous.
+//
+// k_tile_count: per (row, segment), how many entries beat the threshold key / equal it.
+// Grid: x = blocks of 256 rows, y = segment, z = layer.
+constexpr int TILE_NE = 4;   // entries of a run fetched in one batch
+template <typename T>
+__global__ __launch_bounds__(256) void k_tile_count(
+    int Tn, const SelState *st, const uint2 *seg_meta, int nseg, const uint2 *pool, unsigned long long pool_cap,
+    uint8_t *cgt, uint8_t *ceq) {
   constexpr int KB = Elem<T>::KEYBITS;
-  constexpr int GE = 4;
+  const int l = blockIdx.z, seg = blockIdx.y;
+  const SelState s = st[l];
+  if (s.path != PATH_TILES || s.status != ST_DONE) return;
+  const uint2 *mypool = pool + (unsigned long long)l * pool_cap;
+  const int row = blockIdx.x * 256 + threadIdx.x;
+  if (row >= Tn) return;
+  const int64_t at = ((int64_t)l * nseg + seg) * Tn + row;
+  const uint2 m = seg_meta[at];
+  uint32_t raw[TILE_NE];
+#pragma unroll
+  for (int e = 0; e < TILE_NE; ++e) raw[e] = (uint32_t)e < m.y ? mypool[m.x + e].y : 0u;
+  uint32_t ngt = 0, neq = 0;
+#pragma unroll
+  for (int e = 0; e < TILE_NE; ++e)
+    if ((uint32_t)e < m.y) {
+      const uint32_t key = rank_key<KB>(Elem<T>::to_f32(Elem<T>::from_raw(raw[e])));
+      ngt += key > s.thr_key ? 1u : 0u;
+      neq += key == s.thr_key ? 1u : 0u;
+    }
+  for (uint32_t e = TILE_NE; e < m.y; ++e) {
+    const uint32_t key = rank_key<KB>(Elem<T>::to_f32(Elem<T>::from_raw(mypool[m.x + e].y)));
+    ngt += key > s.thr_key ? 1u : 0u;
+    neq += key == s.thr_key ? 1u : 0u;
+  }
+  cgt[at] = (uint8_t)ngt; ceq[at] = (uint8_t)neq;   // a run has at most 128 entries
+}
+
+// k_row_prefix: per row, exclusive prefix of those counts over the segments, and the row totals.
+__global__ __launch_bounds__(256) void k_row_prefix(
+    int64_t Tn, const SelState *st, int nseg, const uint8_t *cgt, const uint8_t *ceq, uint32_t *pgt, uint32_t *peq,
+    uint32_t *row_gt, uint32_t *row_eq) {
   const int l = blockIdx.y;
   const SelState s = st[l];
   if (s.path != PATH_TILES || s.status != ST_DONE) return;
-  const int lane = lane_id(), wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
-  const uint2 *mypool = pool + (unsigned long long)l * pool_cap;
-  uint2 *mypool2 = pool2 + (unsigned long long)l * pool2_cap;
-  const uint2 *meta_l = seg_meta + (int64_t)l * nseg * Tn;
-  auto key_of = [&](const uint2 &e) { return rank_key<KB>(Elem<T>::to_f32(Elem<T>::from_raw(e.y))); };
-  for (int64_t t = (int64_t)blockIdx.x * nwv + wv; t < Tn; t += (int64_t)gridDim.x * nwv) {
-    uint2 m[SPL];
+  const int64_t row = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (row >= Tn) return;
+  uint32_t g = 0, q = 0;
+  const int64_t base = (int64_t)l * nseg * Tn + row;
+  int seg = 0;
+  for (; seg + 8 <= nseg; seg += 8) {
+    uint32_t a[8], b[8];
 #pragma unroll
-    for (int q = 0; q < SPL; ++q) {
-      const int g = lane * SPL + q;
-      m[q] = g < nseg ? meta_l[(int64_t)g * Tn + t] : make_uint2(0u, 0u);
-    }
-    uint2 ent[SPL][GE];
+    for (int i = 0; i < 8; ++i) { a[i] = cgt[base + (int64_t)(seg + i) * Tn]; b[i] = ceq[base + (int64_t)(seg + i) * Tn]; }
 #pragma unroll
-    for (int q = 0; q < SPL; ++q)
-#pragma unroll
-      for (int e = 0; e < GE; ++e) ent[q][e] = (uint32_t)e < m[q].y ? mypool[m[q].x + e] : make_uint2(0u, 0u);
-    uint32_t ngt = 0, neq = 0;
-    bool longrun = false;
-#pragma unroll
-    for (int q = 0; q < SPL; ++q) {
-#pragma unroll
-      for (int e = 0; e < GE; ++e)
-        if ((uint32_t)e < m[q].y) {
-          const uint32_t key = key_of(ent[q][e]);
-          ngt += key > s.thr_key ? 1u : 0u;
-          neq += key == s.thr_key ? 1u : 0u;
-        }
-      for (uint32_t e = GE; e < m[q].y; ++e) {
-        const uint32_t key = key_of(mypool[m[q].x + e]);
-        ngt += key > s.thr_key ? 1u : 0u;
-        neq += key == s.thr_key ? 1u : 0u;
-        longrun = true;
-      }
-    }
-    const uint32_t n = ngt + neq;
-    // both prefix sums in one scan: totals stay below 2^16 per field only if the row is short
-    // enough, so scan them separately
-    const uint32_t incl = wave_inclusive_scan(n);
-    const uint32_t total = __builtin_amdgcn_readlane(incl, 63);
-    const uint32_t tot_gt = __builtin_amdgcn_readlane(wave_inclusive_scan(ngt), 63);
-    const int64_t r = (int64_t)l * Tn + t;
-    uint32_t off = 0;
-    if (total > 0 && lane == 0) off = atomicAdd(&pool2_count[l], total + 1u);
-    off = __builtin_amdgcn_readfirstlane(off);
-    if (lane == 0) {
-      row_gt[r] = tot_gt; row_eq[r] = total - tot_gt;
-      row_first[r] = total > 0 ? off : ROW_NONE;
-      if (total > 0) mypool2[off] = make_uint2(ROW_NONE, total);
-    }
-    if (n > 0) {
-      uint32_t pos = off + 1u + incl - n;
-#pragma unroll
-      for (int q = 0; q < SPL; ++q) {
-#pragma unroll
-        for (int e = 0; e < GE; ++e)
-          if ((uint32_t)e < m[q].y && key_of(ent[q][e]) >= s.thr_key) mypool2[pos++] = ent[q][e];
-        if (longrun)
-          for (uint32_t e = GE; e < m[q].y; ++e) {
-            const uint2 en = mypool[m[q].x + e];
-            if (key_of(en) >= s.thr_key) mypool2[pos++] = en;
-          }
-      }
+    for (int i = 0; i < 8; ++i) {
+      pgt[base + (int64_t)(seg + i) * Tn] = g; peq[base + (int64_t)(seg + i) * Tn] = q;
+      g += a[i]; q += b[i];
     }
   }
+  for (; seg < nseg; ++seg) {
+    const uint32_t a = cgt[base + (int64_t)seg * Tn], b = ceq[base + (int64_t)seg * Tn];
+    pgt[base + (int64_t)seg * Tn] = g; peq[base + (int64_t)seg * Tn] = q;
+    g += a; q += b;
+  }
+  row_gt[(int64_t)l * Tn + row] = g; row_eq[(int64_t)l * Tn + row] = q;
+}
+
+// k_tile_emit: the ordered write.  An entry's place in its row = the row's start + the entries
+// kept in earlier segments (all that beat the key, and ties while the row's allotment lasts) +
+// the entries kept before it in its own run.
+template <typename T>
+__global__ __launch_bounds__(256) void k_tile_emit(
+    int Tn, const SelState *st, const uint2 *seg_meta, int nseg, const uint2 *pool, unsigned long long pool_cap,
+    const uint32_t *pgt, const uint32_t *peq, const uint32_t *allot, const int32_t *row_ptr, int32_t *col_out,
+    T *val_out) {
+  constexpr int KB = Elem<T>::KEYBITS;
+  const int l = blockIdx.z, seg = blockIdx.y;
+  const SelState s = st[l];
+  if (s.path != PATH_TILES || s.status != ST_DONE) return;
+  const uint2 *mypool = pool + (unsigned long long)l * pool_cap;
+  const int row = blockIdx.x * 256 + threadIdx.x;
+  if (row >= Tn) return;
+  const int64_t at = ((int64_t)l * nseg + seg) * Tn + row;
+  const uint2 m = seg_meta[at];
+  if (m.y == 0) return;
+  const int64_t r = (int64_t)l * Tn + row;
+  uint2 en[TILE_NE];
+#pragma unroll
+  for (int e = 0; e < TILE_NE; ++e) en[e] = (uint32_t)e < m.y ? mypool[m.x + e] : make_uint2(0u, 0u);
+  const uint32_t al = allot[r];
+  uint32_t tie = peq[at];
+  int64_t pos = (int64_t)row_ptr[r] + pgt[at] + (tie < al ? tie : al);
+  auto put = [&](const uint2 &e2) {
+    const uint32_t key = rank_key<KB>(Elem<T>::to_f32(Elem<T>::from_raw(e2.y)));
+    bool keepit = key > s.thr_key;
+    if (key == s.thr_key) { keepit = tie < al; ++tie; }
+    if (keepit) { col_out[pos] = (int32_t)e2.x; val_out[pos] = Elem<T>::from_raw(e2.y); ++pos; }
+  };
+#pragma unroll
+  for (int e = 0; e < TILE_NE; ++e)
+    if ((uint32_t)e < m.y) put(en[e]);
+  for (uint32_t e = TILE_NE; e < m.y; ++e) put(mypool[m.x + e]);
 }
 
 // ---- threshold activations ----------------------------------------------------------
@@ -1126,7 +1156,7 @@ static int run_batchtopk(const T *pre, int64_t Tn, int64_t F, int64_t L, int64_t
   k_select_count<T, GLOBAL><<<grid2, 256, 0, stream>>>(pre, Tn, F, L, lstride, mean, denom, st, first, pool, lo.pool_cap, rgt, req);
   k_select_allot<GLOBAL><<<nprob, SCAN_THREADS, 0, stream>>>(st, Tn, L, rgt, req, allot, keep, row_ptr, K);
   if (GLOBAL) k_rowptr_scan<<<1, SCAN_THREADS, 0, stream>>>(keep, L * Tn, row_ptr);
-  k_select_emit<T, GLOBAL><<<grid2, 256, 0, stream>>>(pre, Tn, F, L, lstride, mean, denom, st, first, pool, lo.pool_cap, allot, row_ptr, col, val, nullptr, 0);
+  k_select_emit<T, GLOBAL><<<grid2, 256, 0, stream>>>(pre, Tn, F, L, lstride, mean, denom, st, first, pool, lo.pool_cap, allot, row_ptr, col, val);
   return clt_check_launch();
 }
 
@@ -1178,8 +1208,8 @@ static int dispatch_threshold(bool emit, const void *pre, int64_t Tn, int64_t F,
 // ---- encoder-collected candidates: workspace and the two halves of the fused path ---------
 struct TileLayout {
   SelLayout sel;
-  size_t off_tmeta, off_meta, off_tpool, off_pool2, off_pool2cnt, off_tcount, total;
-  unsigned long long tpool_cap, pool2_cap;   // entries per layer
+  size_t off_tmeta, off_meta, off_tpool, off_cgt, off_ceq, off_pgt, off_peq, off_tcount, total;
+  unsigned long long tpool_cap;              // entries per layer
   uint32_t caps;                             // entries per fixed tile slot
   int nseg, ntile;
 };
@@ -1201,14 +1231,16 @@ static TileLayout tile_layout(int64_t T, int64_t F, int64_t L, int64_t k, int dt
   unsigned long long dyn = 2ull * K + 4096ull;
   if (dyn > N) dyn = N;
   tl.tpool_cap = (unsigned long long)tl.ntile * caps + dyn;
-  tl.pool2_cap = (tl.tpool_cap < N ? tl.tpool_cap : N) + (unsigned long long)T;   // + one header per row
   size_t o = tl.sel.total;
   auto take = [&](size_t bytes) { size_t at = o; o += (bytes + 255) & ~(size_t)255; return at; };
   tl.off_tmeta = take(8 * (size_t)tl.ntile * (size_t)L);
   tl.off_meta = take(8 * (size_t)tl.nseg * (size_t)T * (size_t)L);
   tl.off_tpool = take(8 * (size_t)tl.tpool_cap * (size_t)L);
-  tl.off_pool2 = take(8 * (size_t)tl.pool2_cap * (size_t)L);
-  tl.off_pool2cnt = take(4 * (size_t)L);
+  const size_t cells = (size_t)tl.nseg * (size_t)T * (size_t)L;   // (row, segment) pairs
+  tl.off_cgt = take(cells);
+  tl.off_ceq = take(cells);
+  tl.off_pgt = take(4 * cells);
+  tl.off_peq = take(4 * cells);
   tl.off_tcount = take(4 * (size_t)L);
   tl.total = o;
   return tl;
@@ -1228,12 +1260,10 @@ static int run_encode_collect(const void *x, const void *w, const void *b, void 
   const unsigned long long N = (unsigned long long)Tn * (unsigned long long)F;
   unsigned long long K = (unsigned long long)k * (unsigned long long)Tn;
   if (K > N) K = N;
-  k_sample_dot<T><<<dim3(SAMPLE_TOK, (unsigned)L), 256, 0, stream>>>((const T *)x, (const T *)w, (const T *)b, Tn, d, F,
+  k_sample_dot<T><<<dim3(SAMPLE_TOK, (unsigned)L, 8), 256, 0, stream>>>((const T *)x, (const T *)w, (const T *)b, Tn, d, F,
                                                                       xs, wstr, bs, sample);
-  // (the second counter array handed to k_sample_cut is [pool2 counters | tile-pool counters])
   k_sample_cut<KB><<<(unsigned)L, SCAN_THREADS, 0, stream>>>(sample, N, K, st, hist, poolcnt,
-                                                              (uint32_t *)(ws + tl.off_pool2cnt), PATH_TILES);
-  k_fill_u32<<<1, 256, 0, stream>>>((uint32_t *)(ws + tl.off_tcount), 0u, L);
+                                                              (uint32_t *)(ws + tl.off_tcount), PATH_TILES);
   uint2 *tpool = (uint2 *)(ws + tl.off_tpool);
   CollectArgs ca;
   ca.st = st; ca.pool_count = (uint32_t *)(ws + tl.off_tcount); ca.pool = tpool; ca.pool_cap = tl.tpool_cap;
@@ -1262,8 +1292,6 @@ static int run_collect_select(const T *pre, int64_t Tn, int64_t F, int64_t L, in
   uint32_t *rgt = (uint32_t *)(ws + lo.off_gt), *req = (uint32_t *)(ws + lo.off_eq);
   uint32_t *allot = (uint32_t *)(ws + lo.off_allot), *keep = (uint32_t *)(ws + lo.off_keep);
   uint2 *pool = (uint2 *)(ws + lo.off_pool);
-  uint2 *pool2 = (uint2 *)(ws + tl.off_pool2);
-  uint32_t *pool2cnt = (uint32_t *)(ws + tl.off_pool2cnt);
   const uint2 *meta = (const uint2 *)(ws + tl.off_meta);
   const uint2 *tmeta = (const uint2 *)(ws + tl.off_tmeta);
   const uint2 *tpool = (const uint2 *)(ws + tl.off_tpool);
@@ -1287,21 +1315,16 @@ static int run_collect_select(const T *pre, int64_t Tn, int64_t F, int64_t L, in
     k_select_level<T, false><<<grid2, 256, 0, stream>>>(pre, Tn, F, L, lstride, nullptr, nullptr, st, hist, first, pool, lo.pool_cap, level);
     k_select_scan<KB><<<(unsigned)L, SCAN_THREADS, 0, stream>>>(st, hist, poolcnt, 2, level);
   }
-  // one wavefront per row, all rows at once: these two kernels wait on scattered small reads
-  dim3 grid3((unsigned)clt_ceil_div(Tn, 4), (unsigned)L);
-  const int spl = (tl.nseg + 63) / 64;
-#define CLT_GATHER(S) k_row_gather<T, S><<<grid3, 256, 0, stream>>>(Tn, st, meta, tl.nseg, tpool, tl.tpool_cap, pool2cnt, pool2, tl.pool2_cap, first, rgt, req)
-  if (spl <= 1) CLT_GATHER(1);
-  else if (spl == 2) CLT_GATHER(2);
-  else if (spl == 3) CLT_GATHER(3);
-  else if (spl == 4) CLT_GATHER(4);
-  else if (spl <= 8) CLT_GATHER(8);
-  else return CLT_ERR_RANGE;
-#undef CLT_GATHER
+  dim3 grid3((unsigned)clt_ceil_div(Tn, 256), (unsigned)tl.nseg, (unsigned)L);
+  uint8_t *cgt = (uint8_t *)(ws + tl.off_cgt), *ceq = (uint8_t *)(ws + tl.off_ceq);
+  uint32_t *pgt = (uint32_t *)(ws + tl.off_pgt), *peq = (uint32_t *)(ws + tl.off_peq);
+  k_tile_count<T><<<grid3, 256, 0, stream>>>((int)Tn, st, meta, tl.nseg, tpool, tl.tpool_cap, cgt, ceq);
+  k_row_prefix<<<dim3((unsigned)clt_ceil_div(Tn, 64), (unsigned)L), 64, 0, stream>>>(Tn, st, tl.nseg, cgt, ceq, pgt, peq, rgt, req);
   k_select_count<T, false><<<grid2, 256, 0, stream>>>(pre, Tn, F, L, lstride, nullptr, nullptr, st, first, pool, lo.pool_cap, rgt, req);
   k_select_allot<false><<<(unsigned)L, SCAN_THREADS, 0, stream>>>(st, Tn, L, rgt, req, allot, keep, row_ptr, K);
-  k_select_emit<T, false><<<grid3, 256, 0, stream>>>(pre, Tn, F, L, lstride, nullptr, nullptr, st, first, pool, lo.pool_cap, allot,
-                                                     row_ptr, col, val, pool2, tl.pool2_cap);
+  k_tile_emit<T><<<grid3, 256, 0, stream>>>((int)Tn, st, meta, tl.nseg, tpool, tl.tpool_cap, pgt, peq, allot, row_ptr, col, val);
+  k_select_emit<T, false><<<grid2, 256, 0, stream>>>(pre, Tn, F, L, lstride, nullptr, nullptr, st, first, pool, lo.pool_cap, allot,
+                                                     row_ptr, col, val);
   return clt_check_launch();
 }
 
@@ -1313,7 +1336,6 @@ extern "C" int clt_encode_collect_supported(const void *x, const void *w, const 
   if (dtype != CLT_F32 && dtype != CLT_BF16) return 0;
   if (T <= 0 || d <= 0 || F <= 0 || L <= 0 || L > 65535 || k <= 0 || !x || !w) return 0;
   if ((double)T * (double)F >= 4294967296.0) return 0;
-  if (F / (dtype == CLT_BF16 ? 128 : 64) > 512) return 0;            // feature segments one wavefront can walk
   if (tile_layout(T, F, L, k, dtype).tpool_cap >= 0xFFF00000ull) return 0;
   return clt_encode_can_collect(x, w, b, T, d, F, x_layer_stride, w_layer_stride, b_layer_stride, dtype) ? 1 : 0;
 }
