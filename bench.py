@@ -47,7 +47,7 @@ def algorithmic_work(wl, nnz_rows_pairs: int, nnz_total: int):
 # HBM bytes per k_decode launch (FETCH_SIZE + WRITE_SIZE of `rocprofv3 --pmc`, each scaled by
 # what the same counter reads for the known-size copy at the end of this script), keyed by
 # (workload, launches per step).  Filled from the counter runs kept under profiles/.
-MEASURED_TRAFFIC = {("c1", 12): (1871269.0 + 512104.0) * 1024.0}
+MEASURED_TRAFFIC = {("c1", 12): (1869520.0 + 512102.0) * 1024.0}
 
 
 def copy_probe(dev):
@@ -177,9 +177,14 @@ def run_gpu(args):
         },
         "stages": {
             "encoder": {"ms": st["encode"], "bound": "mfma", "achieved": enc_tf, "peak": mfma_peak,
-                        "unit": "TFLOP/s", "frac": enc_tf / mfma_peak},
+                        "unit": "TFLOP/s", "frac": enc_tf / mfma_peak,
+                        "note": ("includes the sample / cut before and the candidate histogram after the projection"
+                                 if fused else "projection only")},
             "select": {"ms": st["select"], "bound": "hbm", "achieved": sel_gbs, "peak": HBM_PEAK_GBS,
-                       "unit": "GB/s", "frac": sel_gbs / HBM_PEAK_GBS},
+                       "unit": "GB/s", "frac": sel_gbs / HBM_PEAK_GBS,
+                       "note": ("algorithmic bytes = one read of the ranking values + the survivor write; in the fused "
+                                "path the ranking values are compared in the encoder epilogue and never reach HBM, so "
+                                "this stage only touches the candidates") if fused else "separate streaming pass"},
             "decode": {"ms": st["decode"], "bound": "hbm", "achieved": dec_gbs, "peak": HBM_PEAK_GBS,
                        "unit": "GB/s", "frac": dec_gbs / HBM_PEAK_GBS,
                        "compulsory_GBps": dec_c_gbs, "compulsory_frac": dec_c_gbs / HBM_PEAK_GBS},
