@@ -100,6 +100,9 @@ def run_gpu(args):
     _, x_slab, w_slab, b_slab = enc.prepare_slab(inputs)
     fused = (wl.activation_fn == "batchtopk" and not glob and model.fuse_encode_select
              and engine.encode_collect_supported(x_slab, w_slab, b_slab, wl.k))
+    theta = model.theta_manager.thresholds(model.dtype) if wl.activation_fn == "jumprelu" else None
+    fused_thr = (wl.activation_fn == "jumprelu" and model.fuse_encode_select
+                 and engine.encode_threshold(x_slab, w_slab, b_slab, theta, ws, model._density_ppm) is not None)
     for _ in range(args.steps):
         ev = gpu_events(4)
         ev[0].record()
@@ -109,11 +112,18 @@ def run_gpu(args):
             handle = engine.encode_collect(x_slab, w_slab, b_slab, wl.k, pre_buf, ws)
             ev[1].record()
             surv = engine.collect_select(handle)
+        elif fused_thr:
+            # projection with the thresholds applied in the epilogue, survivor list laid out from
+            # the pool: one call, all of it counted as the encoder stage
+            surv = engine.encode_threshold(x_slab, w_slab, b_slab, theta, ws, model._density_ppm)
+            ev[1].record()
         else:
             pre = engine.encode(x_slab, w_slab, b_slab, out=pre_buf)
             ev[1].record()
             if wl.activation_fn == "batchtopk":
                 surv = engine.batchtopk_select(pre, wl.k, glob, ws)
+            elif wl.activation_fn == "jumprelu":
+                surv = engine.threshold_select(pre, theta, cca._native.PRED_GE_THETA, ws)
             else:
                 surv = model._survivors(inputs)[2]
         ev[2].record()
@@ -161,7 +171,9 @@ def run_gpu(args):
                         f"{wl.activation_fn} k={wl.k} ({wl.topk_mode}), decoders {wl.decoder_tying}",
             "global_batch_tokens": T,
             "survivors_per_layer": counts[0],
-            "encode_select": "fused (candidates collected in the encoder epilogue)" if fused else "separate kernels",
+            "encode_select": ("fused (candidates collected in the encoder epilogue)" if fused else
+                              "fused (thresholds applied in the encoder epilogue; the select stage is empty)"
+                              if fused_thr else "separate kernels"),
         },
         "roofline": {
             "kernel": dec_kernel_desc,
@@ -180,11 +192,13 @@ def run_gpu(args):
                         "unit": "TFLOP/s", "frac": enc_tf / mfma_peak,
                         "note": ("includes the sample / cut before and the candidate histogram after the projection"
                                  if fused else "projection only")},
-            "select": {"ms": st["select"], "bound": "hbm", "achieved": sel_gbs, "peak": HBM_PEAK_GBS,
-                       "unit": "GB/s", "frac": sel_gbs / HBM_PEAK_GBS,
+            "select": {"ms": st["select"], "bound": "hbm", "achieved": None if fused_thr else sel_gbs,
+                       "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": None if fused_thr else sel_gbs / HBM_PEAK_GBS,
                        "note": ("algorithmic bytes = one read of the ranking values + the survivor write; in the fused "
                                 "path the ranking values are compared in the encoder epilogue and never reach HBM, so "
-                                "this stage only touches the candidates") if fused else "separate streaming pass"},
+                                "this stage only touches the candidates") if fused else
+                               "empty: the survivor list is written by the encoder stage" if fused_thr else
+                               "separate streaming pass"},
             "decode": {"ms": st["decode"], "bound": "hbm", "achieved": dec_gbs, "peak": HBM_PEAK_GBS,
                        "unit": "GB/s", "frac": dec_gbs / HBM_PEAK_GBS,
                        "compulsory_GBps": dec_c_gbs, "compulsory_frac": dec_c_gbs / HBM_PEAK_GBS},

@@ -58,6 +58,7 @@ class CrossLayerTranscoder(BaseTranscoder):
         # per-layer BatchTopK: let the encoder epilogue collect the candidates (same result, one
         # dense write and one dense read less); False forces the separate encode + select kernels
         self.fuse_encode_select = True
+        self._density_ppm = 20000   # JumpReLU survivor density the candidate pool is sized for
         self.dtype = self._resolve_dtype(config.clt_dtype)
         if device is not None:
             self.device = torch.device(device)
@@ -228,6 +229,17 @@ class CrossLayerTranscoder(BaseTranscoder):
                     surv = engine.collect_select(engine.encode_collect(x_slab, w_slab, b_slab, k, pre_buf, ws))
                 self._record("batchtopk_activation", tm)
                 return layers, T, surv
+        if fn == "jumprelu" and self.fuse_encode_select:
+            # thresholds applied in the encoder epilogue; the pool is sized from the density seen last
+            theta = self.theta_manager.thresholds(self.dtype)
+            if layers != list(range(cfg.num_layers)):
+                theta = theta.index_select(0, torch.tensor(layers, device=theta.device)).contiguous()
+            surv = engine.encode_threshold(x_slab, w_slab, b_slab, theta, ws, self._density_ppm)
+            if surv is not None:
+                seen = int(1e6 * surv.nnz / max(1, n * T * cfg.num_features))
+                self._density_ppm = max(2000, 2 * seen)
+                return layers, T, surv
+            self._density_ppm = min(1000000, 4 * self._density_ppm)
         pre = engine.encode(x_slab, w_slab, b_slab, out=pre_buf)
         if fn in ("batchtopk", "topk"):
             surv = self._select(pre)

@@ -349,15 +349,35 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         }
       };
       bool done = false;
-      if constexpr (COLLECT == 1 && sizeof(T) == 2) {
-        // bf16 and a positive cut: x >= cut  <=>  bits(x) >= bits(cut) as signed 16-bit integers
-        // (negative values have the sign bit), two elements per operation: the sign of the
-        // saturated difference (cut - 1) - x marks a candidate.  NaNs with the sign bit set would
-        // be missed, so the unsigned maximum of all raw values is tracked; if it shows one, the
-        // tile is redone with float compares.
-        const uint32_t cb = cut_bits >> 16;
-        if (cb >= 1u && cb <= 0x7F80u) {
-          const uint32_t cm1 = (cb - 1u) | ((cb - 1u) << 16);
+      if constexpr (sizeof(T) == 2) {
+        // bf16 and a positive cut / threshold: x >= c  <=>  bits(x) >= bits(c) as signed 16-bit
+        // integers (negative values have the sign bit), two elements per operation: the sign of
+        // the saturated difference (c - 1) - x marks a candidate.  NaNs would be treated wrongly
+        // (a top-k cut must take them all, also those with the sign bit set; a threshold must take
+        // none), so the unsigned maximum of the raw values is tracked and the tile is redone with
+        // float compares if it shows one.
+        bool fast_ok;
+        uint32_t cm1 = 0;
+        const T *theta_seg = nullptr;
+        if constexpr (COLLECT == 1) {
+          const uint32_t cb = cut_bits >> 16;
+          fast_ok = cb >= 1u && cb <= 0x7F80u;
+          cm1 = (cb - 1u) | ((cb - 1u) << 16);
+        } else {
+          theta_seg = (const T *)ca.theta + (int64_t)layer * ca.theta_stride + ncol0;
+          bool bad = false;
+          if (lane < 16) {   // every threshold of the segment must be a positive number
+            const uint4 tv = *reinterpret_cast<const uint4 *>(theta_seg + lane * 8);
+            const uint32_t t4[4] = {tv.x, tv.y, tv.z, tv.w};
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+              const uint32_t lo = t4[k] & 0xFFFFu, hi = t4[k] >> 16;
+              bad = bad || lo < 1u || lo > 0x7F80u || hi < 1u || hi > 0x7F80u;
+            }
+          }
+          fast_ok = __ballot(bad) == 0;
+        }
+        if (fast_ok) {
           uint32_t mx = 0;
 #pragma unroll
           for (int h = 0; h < 2; ++h) {
@@ -368,19 +388,25 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             for (int sl = 0; sl < 16; ++sl) {
               const uint4 v = *reinterpret_cast<const uint4 *>(park + ml * 256 + ((sl ^ (ml & 15)) * 16));
               const uint32_t w4[4] = {v.x, v.y, v.z, v.w};
+              uint32_t c4[4] = {cm1, cm1, cm1, cm1};
+              if constexpr (COLLECT == 2) {
+                const uint4 tv = *reinterpret_cast<const uint4 *>(theta_seg + sl * 8);   // same address in all lanes
+                c4[0] = tv.x - 0x00010001u; c4[1] = tv.y - 0x00010001u; c4[2] = tv.z - 0x00010001u; c4[3] = tv.w - 0x00010001u;
+              }
               uint32_t a = 0;
 #pragma unroll
               for (int k = 0; k < 4; ++k) {
-                const uint32_t sg = pk_sign16(pk_sub_sat16(cm1, w4[k]));      // 0xFFFF per candidate half
+                const uint32_t sg = pk_sign16(pk_sub_sat16(c4[k], w4[k]));   // 0xFFFF per candidate half
                 a |= sg & ((1u << (2 * k)) | (0x20000u << (2 * k)));         // element 2k -> bit 2k, 2k+1 -> bit 16+2k+1
-                mx = pk_max_u16(mx, w4[k]);
+                mx = pk_max_u16(mx, COLLECT == 1 ? w4[k] : (w4[k] & 0x7FFF7FFFu));
               }
               const uint32_t m = (a | (a >> 16)) & 0xFFu;
               W[h][sl >> 2] |= m << ((sl & 3) * 8);
             }
           }
-          const bool neg_nan = (mx & 0xFFFFu) > 0xFF80u || (mx >> 16) > 0xFF80u;
-          done = __ballot(neg_nan) == 0;
+          const uint32_t nan_above = COLLECT == 1 ? 0xFF80u : 0x7F80u;
+          const bool nan_seen = (mx & 0xFFFFu) > nan_above || (mx >> 16) > nan_above;
+          done = __ballot(nan_seen) == 0;
         }
       }
       if (!done) scan_generic();

@@ -858,6 +858,63 @@ __global__ __launch_bounds__(256) void k_tile_emit(
   for (uint32_t e = TILE_NE; e < m.y; ++e) put(mypool[m.x + e]);
 }
 
+// ---- threshold activation on encoder-collected entries (every entry is a survivor) ----------
+// Per row: exclusive prefix of the run lengths over the segments, and the row total.
+__global__ __launch_bounds__(256) void k_row_prefix_meta(int64_t Tn, int nseg, const uint2 *seg_meta, uint32_t *pfx,
+                                                         uint32_t *row_cnt) {
+  const int l = blockIdx.y;
+  const int64_t row = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (row >= Tn) return;
+  uint32_t g = 0;
+  const int64_t base = (int64_t)l * nseg * Tn + row;
+  int seg = 0;
+  for (; seg + 8 <= nseg; seg += 8) {
+    uint32_t a[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) a[i] = seg_meta[base + (int64_t)(seg + i) * Tn].y;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { pfx[base + (int64_t)(seg + i) * Tn] = g; g += a[i]; }
+  }
+  for (; seg < nseg; ++seg) {
+    const uint32_t a = seg_meta[base + (int64_t)seg * Tn].y;
+    pfx[base + (int64_t)seg * Tn] = g; g += a;
+  }
+  row_cnt[(int64_t)l * Tn + row] = g;
+}
+
+// row_ptr[R] = -1 when some layer ran out of pool space (the caller then takes the separate route)
+__global__ void k_thresh_finish(const SelState *st, int L, int32_t *row_ptr, int64_t R) {
+  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+  bool over = false;
+  for (int l = 0; l < L; ++l) over = over || st[l].overflow != 0;
+  if (over) row_ptr[R] = -1;
+}
+
+// Grid: x = blocks of 256 rows, y = segment, z = layer.
+template <typename T>
+__global__ __launch_bounds__(256) void k_tile_emit_all(
+    int Tn, const uint2 *seg_meta, int nseg, const uint2 *pool, unsigned long long pool_cap, const uint32_t *pfx,
+    const int32_t *row_ptr, int32_t *col_out, T *val_out) {
+  const int l = blockIdx.z, seg = blockIdx.y;
+  const uint2 *mypool = pool + (unsigned long long)l * pool_cap;
+  const int row = blockIdx.x * 256 + threadIdx.x;
+  if (row >= Tn) return;
+  const int64_t at = ((int64_t)l * nseg + seg) * Tn + row;
+  const uint2 m = seg_meta[at];
+  if (m.y == 0) return;
+  uint2 en[TILE_NE];
+#pragma unroll
+  for (int e = 0; e < TILE_NE; ++e) en[e] = (uint32_t)e < m.y ? mypool[m.x + e] : make_uint2(0u, 0u);
+  int64_t pos = (int64_t)row_ptr[(int64_t)l * Tn + row] + pfx[at];
+#pragma unroll
+  for (int e = 0; e < TILE_NE; ++e)
+    if ((uint32_t)e < m.y) { col_out[pos] = (int32_t)en[e].x; val_out[pos] = Elem<T>::from_raw(en[e].y); ++pos; }
+  for (uint32_t e = TILE_NE; e < m.y; ++e) {
+    const uint2 e2 = mypool[m.x + e];
+    col_out[pos] = (int32_t)e2.x; val_out[pos] = Elem<T>::from_raw(e2.y); ++pos;
+  }
+}
+
 // ---- threshold activations ----------------------------------------------------------
 template <typename T, int PRED> __device__ __forceinline__ bool pred_keep(float x, float th) {
   if (PRED == CLT_PRED_GE_THETA) return x >= th;
@@ -1328,7 +1385,113 @@ static int run_collect_select(const T *pre, int64_t Tn, int64_t F, int64_t L, in
   return clt_check_launch();
 }
 
+// ---- JumpReLU on the encoder epilogue -----------------------------------------------------------
+struct ThreshLayout {
+  size_t off_state, off_tcount, off_tmeta, off_meta, off_tpool, off_pfx, off_rowcnt, total;
+  unsigned long long tpool_cap;
+  uint32_t caps;
+  int nseg, ntile;
+};
+
+static ThreshLayout thresh_layout(int64_t T, int64_t F, int64_t L, int64_t density_ppm, int dtype) {
+  ThreshLayout tl;
+  const int segw = dtype == CLT_BF16 ? 128 : 64;
+  tl.nseg = (int)(F / segw);
+  tl.ntile = tl.nseg * (int)(T / 128);
+  const double dens = (double)(density_ppm < 1 ? 1 : density_ppm) * 1e-6;
+  // a fixed slot holds three times the expected entries of a tile (at least 64, at most the tile)
+  unsigned long long caps = (unsigned long long)(3.0 * dens * 128.0 * segw) + 64ull;
+  if (caps > 128ull * segw) caps = 128ull * segw;
+  tl.caps = (uint32_t)caps;
+  const unsigned long long N = (unsigned long long)T * F;
+  unsigned long long dyn = (unsigned long long)(2.0 * dens * (double)N) + 4096ull;
+  if (dyn > N) dyn = N;
+  tl.tpool_cap = (unsigned long long)tl.ntile * caps + dyn;
+  size_t o = 0;
+  auto take = [&](size_t bytes) { size_t at = o; o += (bytes + 255) & ~(size_t)255; return at; };
+  tl.off_state = take(sizeof(SelState) * (size_t)L);
+  tl.off_tcount = take(4 * (size_t)L);
+  tl.off_tmeta = take(8 * (size_t)tl.ntile * (size_t)L);
+  tl.off_meta = take(8 * (size_t)tl.nseg * (size_t)T * (size_t)L);
+  tl.off_tpool = take(8 * (size_t)tl.tpool_cap * (size_t)L);
+  tl.off_pfx = take(4 * (size_t)tl.nseg * (size_t)T * (size_t)L);
+  tl.off_rowcnt = take(4 * (size_t)T * (size_t)L);
+  tl.total = o;
+  return tl;
+}
+
 }  // namespace
+
+extern "C" int clt_encode_threshold_supported(const void *x, const void *w, const void *b, const void *theta,
+                                              int64_t T, int64_t d, int64_t F, int64_t L, int64_t x_layer_stride,
+                                              int64_t w_layer_stride, int64_t b_layer_stride,
+                                              int64_t theta_layer_stride, int64_t density_ppm, int dtype) {
+  if (dtype != CLT_F32 && dtype != CLT_BF16) return 0;
+  if (T <= 0 || d <= 0 || F <= 0 || L <= 0 || L > 65535 || !x || !w || !theta) return 0;
+  if ((double)T * (double)F >= 4294967296.0 || (double)T * (double)L >= 2147483647.0) return 0;
+  if (!clt_aligned16(theta) || (theta_layer_stride * (dtype == CLT_BF16 ? 2 : 4)) % 16 != 0) return 0;
+  if (thresh_layout(T, F, L, density_ppm, dtype).tpool_cap >= 0xFFF00000ull) return 0;
+  return clt_encode_can_collect(x, w, b, T, d, F, x_layer_stride, w_layer_stride, b_layer_stride, dtype) ? 1 : 0;
+}
+
+extern "C" size_t clt_encode_threshold_workspace_bytes(int64_t T, int64_t d, int64_t F, int64_t L,
+                                                       int64_t density_ppm, int dtype) {
+  (void)d;
+  if (T <= 0 || F <= 0 || L <= 0) return 256;
+  return thresh_layout(T, F, L, density_ppm, dtype).total;
+}
+
+extern "C" int clt_encode_threshold_count(const void *x, const void *w, const void *b, const void *theta, int64_t T,
+                                          int64_t d, int64_t F, int64_t L, int64_t x_layer_stride,
+                                          int64_t w_layer_stride, int64_t b_layer_stride,
+                                          int64_t theta_layer_stride, int64_t density_ppm, int dtype,
+                                          int32_t *row_ptr, void *workspace, size_t workspace_bytes, void *stream) {
+  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (!row_ptr || !workspace) return CLT_ERR_ARG;
+  if (!clt_encode_threshold_supported(x, w, b, theta, T, d, F, L, x_layer_stride, w_layer_stride, b_layer_stride,
+                                      theta_layer_stride, density_ppm, dtype))
+    return CLT_ERR_ARG;
+  const ThreshLayout tl = thresh_layout(T, F, L, density_ppm, dtype);
+  if (workspace_bytes < tl.total) return CLT_ERR_WORKSPACE;
+  if ((((uintptr_t)workspace) & 255u) != 0) return CLT_ERR_ALIGN;
+  hipStream_t s = (hipStream_t)stream;
+  char *ws = (char *)workspace;
+  SelState *st = (SelState *)(ws + tl.off_state);
+  // state (only the overflow flags are used) and the pool counters start at zero; they are adjacent
+  k_fill_u32<<<8, 256, 0, s>>>((uint32_t *)(ws + tl.off_state), 0u, (int64_t)((tl.off_tmeta - tl.off_state) / 4));
+  CollectArgs ca;
+  ca.st = st; ca.pool_count = (uint32_t *)(ws + tl.off_tcount); ca.pool = (uint2 *)(ws + tl.off_tpool);
+  ca.pool_cap = tl.tpool_cap; ca.tile_meta = (uint2 *)(ws + tl.off_tmeta); ca.seg_meta = (uint2 *)(ws + tl.off_meta);
+  ca.caps = tl.caps; ca.theta = theta; ca.theta_stride = theta_layer_stride;
+  int rc = clt_launch_encode(x, w, b, nullptr, T, d, F, L, x_layer_stride, w_layer_stride, b_layer_stride, 0, dtype, 2,
+                             nullptr, &ca, s);
+  if (rc != CLT_OK) return rc;
+  uint32_t *rowcnt = (uint32_t *)(ws + tl.off_rowcnt);
+  k_row_prefix_meta<<<dim3((unsigned)clt_ceil_div(T, 64), (unsigned)L), 64, 0, s>>>(T, tl.nseg, ca.seg_meta,
+                                                                                    (uint32_t *)(ws + tl.off_pfx), rowcnt);
+  k_rowptr_scan<<<1, SCAN_THREADS, 0, s>>>(rowcnt, L * T, row_ptr);
+  k_thresh_finish<<<1, 64, 0, s>>>(st, (int)L, row_ptr, L * T);
+  return clt_check_launch();
+}
+
+extern "C" int clt_encode_threshold_emit(int64_t T, int64_t F, int64_t L, int64_t density_ppm, int dtype,
+                                         const int32_t *row_ptr, int32_t *col, void *val, void *workspace,
+                                         size_t workspace_bytes, void *stream) {
+  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (T <= 0 || F <= 0 || L <= 0 || L > 65535 || !row_ptr || !col || !val || !workspace) return CLT_ERR_ARG;
+  const ThreshLayout tl = thresh_layout(T, F, L, density_ppm, dtype);
+  if (workspace_bytes < tl.total) return CLT_ERR_WORKSPACE;
+  hipStream_t s = (hipStream_t)stream;
+  char *ws = (char *)workspace;
+  dim3 grid((unsigned)clt_ceil_div(T, 256), (unsigned)tl.nseg, (unsigned)L);
+  if (dtype == CLT_BF16)
+    k_tile_emit_all<bf16_t><<<grid, 256, 0, s>>>((int)T, (const uint2 *)(ws + tl.off_meta), tl.nseg, (const uint2 *)(ws + tl.off_tpool),
+                                                  tl.tpool_cap, (const uint32_t *)(ws + tl.off_pfx), row_ptr, col, (bf16_t *)val);
+  else
+    k_tile_emit_all<float><<<grid, 256, 0, s>>>((int)T, (const uint2 *)(ws + tl.off_meta), tl.nseg, (const uint2 *)(ws + tl.off_tpool),
+                                                 tl.tpool_cap, (const uint32_t *)(ws + tl.off_pfx), row_ptr, col, (float *)val);
+  return clt_check_launch();
+}
 
 extern "C" int clt_encode_collect_supported(const void *x, const void *w, const void *b, int64_t T, int64_t d,
                                             int64_t F, int64_t L, int64_t x_layer_stride, int64_t w_layer_stride,

@@ -239,6 +239,40 @@ def threshold_select(pre: torch.Tensor, theta: Optional[torch.Tensor], pred: int
     return SurvivorList(row_ptr, col[:total], val[:total], T, F, L, pre.dtype)
 
 
+def encode_threshold(x: torch.Tensor, w: torch.Tensor, b: Optional[torch.Tensor], theta: torch.Tensor,
+                     ws: Workspace, density_ppm: int = 20000) -> Optional[SurvivorList]:
+    """Encoder projection + JumpReLU (x >= theta) without dense pre-activations
+    (parallel.py:286 + theta.py:70-79).  Returns None when the shapes do not qualify or the
+    survivors exceeded what ``density_ppm`` provides for: the caller then runs ``encode`` and
+    ``threshold_select``."""
+    nat.require_device(x, "encode_threshold")
+    L, T, d = x.shape
+    F = w.shape[1]
+    assert w.shape == (L, F, d) and x.dtype == w.dtype
+    assert theta.shape == (L, F) and theta.dtype == x.dtype and theta.stride(1) == 1
+    lib = nat.load()
+    dt = nat.dtype_code(x.dtype)
+    strides = (x.stride(0), w.stride(0), b.stride(0) if b is not None else 0, theta.stride(0))
+    if not lib.clt_encode_threshold_supported(nat.ptr(x), nat.ptr(w), nat.ptr(b), nat.ptr(theta), T, d, F, L,
+                                              *strides, int(density_ppm), dt):
+        return None
+    nbytes = lib.clt_encode_threshold_workspace_bytes(T, d, F, L, int(density_ppm), dt)
+    wbuf = ws.get("collect_threshold", nbytes)
+    row_ptr = torch.empty(L * T + 1, dtype=torch.int32, device=x.device)
+    code = lib.clt_encode_threshold_count(nat.ptr(x), nat.ptr(w), nat.ptr(b), nat.ptr(theta), T, d, F, L, *strides,
+                                          int(density_ppm), dt, nat.ptr(row_ptr), nat.ptr(wbuf), wbuf.numel(), _stream(x))
+    nat.check(code, "clt_encode_threshold_count")
+    total = int(row_ptr[-1].item())
+    if total < 0:
+        return None
+    col = torch.empty(max(total, 1), dtype=torch.int32, device=x.device)
+    val = torch.empty(max(total, 1), dtype=x.dtype, device=x.device)
+    code = lib.clt_encode_threshold_emit(T, F, L, int(density_ppm), dt, nat.ptr(row_ptr), nat.ptr(col), nat.ptr(val),
+                                         nat.ptr(wbuf), wbuf.numel(), _stream(x))
+    nat.check(code, "clt_encode_threshold_emit")
+    return SurvivorList(row_ptr, col[:total], val[:total], T, F, L, x.dtype)
+
+
 def pack_decoder(w_ref: torch.Tensor, out: torch.Tensor) -> None:
     """[d, F] checkpoint layout -> [F, d] feature-major (one matrix)."""
     nat.require_device(w_ref, "pack_decoder")

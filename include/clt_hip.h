@@ -184,6 +184,39 @@ int clt_threshold_emit(const void *pre, int64_t T, int64_t F, int64_t L,
                        void *stream);
 
 /*
+ * Encoder projection and JumpReLU in one path, without writing the dense pre-activations:
+ * the encoder's epilogue compares every value with its feature's threshold and appends the
+ * survivors to a pool; the survivor list is then laid out from the pool.  Same result as
+ * clt_encode followed by clt_threshold_count / clt_threshold_emit with CLT_PRED_GE_THETA.
+ *   clt_encode_threshold_count  projection + collection, fills row_ptr [L*T+1];
+ *                               row_ptr[L*T] = survivor total, or -1 when the pool was too
+ *                               small (then use the separate calls)
+ *   clt_encode_threshold_emit   writes col / val (sized from the total) from the pool
+ * theta [L][F] in the model dtype (already exp()'d and rounded).  density_ppm is the caller's
+ * estimate of the survivor density in parts per million; it sizes the pool (three times that
+ * per 128 x 128 tile plus twice that overall) and must be the same in all three calls.
+ * clt_encode_threshold_supported: same shape conditions as clt_encode_collect_supported.
+ * Replaces F.linear (clt/models/parallel.py:286) + ThetaManager.jumprelu
+ * (clt/models/theta.py:70-79, clt/models/activations.py:177-180) for all layers.
+ */
+int clt_encode_threshold_supported(const void *x, const void *w, const void *b, const void *theta,
+                                   int64_t T, int64_t d, int64_t F, int64_t L,
+                                   int64_t x_layer_stride, int64_t w_layer_stride,
+                                   int64_t b_layer_stride, int64_t theta_layer_stride,
+                                   int64_t density_ppm, int dtype);
+size_t clt_encode_threshold_workspace_bytes(int64_t T, int64_t d, int64_t F, int64_t L,
+                                            int64_t density_ppm, int dtype);
+int clt_encode_threshold_count(const void *x, const void *w, const void *b, const void *theta,
+                               int64_t T, int64_t d, int64_t F, int64_t L,
+                               int64_t x_layer_stride, int64_t w_layer_stride,
+                               int64_t b_layer_stride, int64_t theta_layer_stride,
+                               int64_t density_ppm, int dtype, int32_t *row_ptr,
+                               void *workspace, size_t workspace_bytes, void *stream);
+int clt_encode_threshold_emit(int64_t T, int64_t F, int64_t L, int64_t density_ppm, int dtype,
+                              const int32_t *row_ptr, int32_t *col, void *val,
+                              void *workspace, size_t workspace_bytes, void *stream);
+
+/*
  * Repack decoder weights from the checkpoint layout [d][F] (nn.Linear weight of
  * RowParallelLinear, clt/models/parallel.py:66-70) to feature-major [F][d], so a
  * feature's decoder vector is one contiguous run.  n_dec matrices, element strides.

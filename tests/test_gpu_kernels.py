@@ -167,6 +167,72 @@ def test_batchtopk_k_zero_and_empty(dev):
     assert surv.nnz == 0
 
 
+# ---- encoder with the per-feature-threshold epilogue (JumpReLU) ---------------------------------
+def threshold_fused_vs_separate(x, w, b, theta, dev, density_ppm=200000):
+    xd, wd, td = x.to(dev), w.to(dev), theta.to(dev)
+    bd = b.to(dev) if b is not None else None
+    pre = engine.encode(xd, wd, bd)
+    ref = engine.threshold_select(pre, td, nat.PRED_GE_THETA)
+    got = engine.encode_threshold(xd, wd, bd, td, engine.Workspace(xd.device), density_ppm)
+    torch.cuda.synchronize()
+    return pre.cpu(), ref, got
+
+
+def assert_same_list(got, ref, dtype):
+    iv = torch.int16 if dtype == torch.bfloat16 else torch.int32
+    assert torch.equal(got.row_ptr.cpu(), ref.row_ptr.cpu())
+    assert torch.equal(got.col.cpu(), ref.col.cpu())
+    assert torch.equal(got.val.cpu().view(iv), ref.val.cpu().view(iv))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("L,T,d,F", [(1, 256, 128, 256), (2, 512, 256, 1024), (3, 256, 768, 512)])
+def test_encode_threshold_matches_separate_and_oracle(dev, dtype, L, T, d, F):
+    g = torch.Generator().manual_seed(L * 17 + T + F)
+    x = torch.randn(L, T, d, generator=g).to(dtype)
+    w = (torch.randn(L, F, d, generator=g) / math.sqrt(d)).to(dtype)
+    b = (0.1 * torch.randn(L, F, generator=g)).to(dtype)
+    theta = torch.exp(0.5 * torch.randn(L, F, generator=g) + 0.3).to(dtype)
+    pre, ref, got = threshold_fused_vs_separate(x, w, b, theta, dev)
+    assert got is not None
+    assert_same_list(got, ref, dtype)
+    check_rows_sorted(got)
+    dense = engine.densify(got, out_f32=True).cpu()
+    for l in range(L):
+        assert torch.equal(dense[l], orc.jumprelu_forward(pre[l], theta[l]))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_encode_threshold_special_thresholds_and_values(dev, dtype):
+    # zero / huge / infinite thresholds and NaN, +-inf, -0.0 pre-activations (reached through
+    # crafted inputs: one-hot weights copy input values into the pre-activations)
+    g = torch.Generator().manual_seed(4)
+    L, T, d, F = 1, 256, 128, 256
+    x = torch.randn(L, T, d, generator=g)
+    x[0, 3, 0] = float("nan"); x[0, 5, 1] = float("inf"); x[0, 7, 2] = float("-inf"); x[0, 9, 3] = -0.0
+    w = torch.zeros(L, F, d)
+    for f in range(F):
+        w[0, f, f % d] = 1.0                       # pre[t, f] = x[t, f % d] (plus NaN/inf propagation rules)
+    theta = torch.exp(0.5 * torch.randn(L, F, generator=g))
+    theta[0, 0] = 0.0; theta[0, 1] = float("inf"); theta[0, 2] = 3e38; theta[0, 130] = 0.0
+    pre, ref, got = threshold_fused_vs_separate(x.to(dtype), w.to(dtype), None, theta.to(dtype), dev)
+    assert got is not None
+    assert_same_list(got, ref, dtype)
+
+
+def test_encode_threshold_pool_too_small_reports_it(dev):
+    g = torch.Generator().manual_seed(6)
+    L, T, d, F = 1, 256, 128, 256
+    x = torch.randn(L, T, d, generator=g).to(torch.bfloat16)
+    w = (torch.randn(L, F, d, generator=g) / math.sqrt(d)).to(torch.bfloat16)
+    theta = torch.full((L, F), 1e-3).to(torch.bfloat16)          # about half of all values survive
+    pre, ref, got = threshold_fused_vs_separate(x, w, None, theta, dev, density_ppm=1)
+    assert got is None
+    pre, ref, got = threshold_fused_vs_separate(x, w, None, theta, dev, density_ppm=600000)
+    assert got is not None and got.nnz == ref.nnz
+    assert_same_list(got, ref, torch.bfloat16)
+
+
 # ---- BatchTopK global ------------------------------------------------------------------------
 # ---- encoder with the collecting epilogue + BatchTopK on the candidates --------------------
 def fused_vs_separate(x, w, b, k, dev):
