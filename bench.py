@@ -70,6 +70,8 @@ def run_gpu(args):
     from crosslayer_coding_amd import engine, synth
 
     wl = synth.WORKLOADS[args.workload]
+    if args.topk_mode and args.topk_mode != wl.topk_mode:
+        wl = wl.scaled(f"{wl.name}-{args.topk_mode}", topk_mode=args.topk_mode)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     cca._native.load(build_if_missing=False)
@@ -254,6 +256,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-tokens", type=int, default=4096)
     ap.add_argument("--no-fuse", action="store_true", help="separate encoder and selection kernels")
+    ap.add_argument("--topk-mode", choices=["per_layer", "global"], default=None,
+                    help="override the workload's BatchTopK scope (global = the reference's default helper)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one 256 MiB elementwise copy (counter yardstick for profiled runs)")
     args = ap.parse_args()

@@ -271,6 +271,27 @@ template <> __device__ __forceinline__ float vec_elem<bf16_t>(const uint4 &w, in
   return __uint_as_float((j & 1) ? (u & 0xFFFF0000u) : (u << 16));
 }
 
+// Global ranking: for every (layer, feature) the lowest value x whose z-score reaches the cut
+// key (binary search over the ordered keys of the element type; the z-score with its two
+// roundings is monotone in x).  NaN when only a NaN reaches the cut.
+template <typename T>
+__global__ __launch_bounds__(256) void k_col_cut(const float *mean, const float *denom, const SelState *st, int64_t F,
+                                                 int64_t L, T *xcut) {
+  constexpr int KB = Elem<T>::KEYBITS;
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= L * F) return;
+  const uint32_t cut_key = st[0].cut_key;
+  RankZ<T> rk; rk.mean = mean; rk.denom = denom;   // indexed with the flat (layer, feature) position
+  uint32_t lo = min_key<KB>(), hi = KB == 32 ? 0xFFFFFFFFu : 0xFFFFu;
+  while (lo < hi) {
+    const uint32_t mid = lo + ((hi - lo) >> 1);
+    const float xv = __uint_as_float(key_to_f32_bits<KB>(mid));
+    if (rank_key<KB>(rk(xv, i)) >= cut_key) hi = mid; else lo = mid + 1u;
+  }
+  const uint32_t bits = key_to_f32_bits<KB>(lo);
+  xcut[i] = Elem<T>::from_raw(sizeof(T) == 2 ? (bits >> 16) : bits);
+}
+
 // The streaming pass: one wavefront per row.  A step covers PASS_NV vectors of 64 lanes x 16
 // bytes.  Lanes keep a bit per element that reaches the cut; when any lane has one, the raw
 // vectors are staged in LDS (column order), two packed prefix scans give every candidate its
@@ -280,7 +301,7 @@ template <typename T, int V, bool GLOBAL>
 __global__ __launch_bounds__(256) void k_select_pass(
     const T *pre, int64_t Tn, int64_t F, int64_t L, int64_t lstride, const float *mean,
     const float *denom, const SelState *st, uint32_t *hist, uint32_t *pool_count, uint2 *pool,
-    unsigned long long pool_cap, uint32_t *row_first, int phase) {
+    unsigned long long pool_cap, uint32_t *row_first, int phase, const T *xcut) {
   constexpr int KB = Elem<T>::KEYBITS;
   static_assert(PASS_NV == 4, "the packed prefix below holds four 16-bit fields");
   constexpr int STEP = PASS_NV * 64 * V;  // elements per step
@@ -339,15 +360,24 @@ __global__ __launch_bounds__(256) void k_select_pass(
         }
       }
       uint32_t m = 0;  // bit q*V + j: element j of vector q reaches the cut
+      // global ranking, first pass: the z-score is monotone in x, so "z reaches the cut" is
+      // "x reaches the column's own bound" (k_col_cut), one compare instead of a division
+      const bool by_column = GLOBAL && V > 1 && phase == 0 && xcut != nullptr;
 #pragma unroll
       for (int q = 0; q < PASS_NV; ++q) {
         const int64_t col = c0 + (int64_t)q * 64 * V + (int64_t)lane * V;
         if (on[q]) {
+          uint4 xc = make_uint4(0, 0, 0, 0);
+          if (by_column) xc = *reinterpret_cast<const uint4 *>(xcut + (int64_t)l * F + col);
 #pragma unroll
           for (int j = 0; j < V; ++j) {
             const float xv = V > 1 ? vec_elem<T>(w[q], j) : __uint_as_float(w[q].x);
-            const float rv = rk(xv, col + j);
-            const bool c = cut_nan ? (rv != rv) : !(rv < cutf);
+            bool c;
+            if (by_column) c = xv >= vec_elem<T>(xc, j) || xv != xv;
+            else {
+              const float rv = rk(xv, col + j);
+              c = cut_nan ? (rv != rv) : !(rv < cutf);
+            }
             m |= (c ? 1u : 0u) << (q * V + j);
           }
         }
@@ -1135,7 +1165,7 @@ static int run_tokentopk(const T *pre, int64_t Tn, int64_t F, int64_t L, int64_t
 
 // ---- host side ------------------------------------------------------------------------
 struct SelLayout {
-  size_t off_state, off_hist, off_poolcnt, off_sample, off_first, off_gt, off_eq, off_allot, off_keep, off_pool, total;
+  size_t off_state, off_hist, off_poolcnt, off_sample, off_first, off_gt, off_eq, off_allot, off_keep, off_xcut, off_pool, total;
   unsigned long long pool_cap;  // entries per problem
   int nprob;
 };
@@ -1165,6 +1195,7 @@ static SelLayout sel_layout(int64_t T, int64_t F, int64_t L, int64_t k, int mode
   lo.off_eq = take(4 * R);
   lo.off_allot = take(4 * R);
   lo.off_keep = take(4 * R);
+  lo.off_xcut = take(mode == CLT_TOPK_GLOBAL ? 4 * (size_t)F * (size_t)L : 0);   // per-column bounds, element type
   lo.off_pool = take(8 * (size_t)cap * (size_t)lo.nprob);
   lo.total = o;
   return lo;
@@ -1196,8 +1227,13 @@ static int run_batchtopk(const T *pre, int64_t Tn, int64_t F, int64_t L, int64_t
   int gx = (int)clt_ceil_div(Tn, 8);
   if (gx > 65535 * 8) gx = 65535 * 8;
   dim3 grid(gx, (unsigned)L);
+  T *xcut = nullptr;
+  if (GLOBAL && V > 1) {
+    xcut = (T *)(ws + lo.off_xcut);
+    k_col_cut<T><<<(unsigned)clt_ceil_div(L * F, 256), 256, 0, stream>>>(mean, denom, st, F, L, xcut);
+  }
   for (int phase = 0; phase < 2; ++phase) {
-    k_select_pass<T, V, GLOBAL><<<grid, 256, 0, stream>>>(pre, Tn, F, L, lstride, mean, denom, st, hist, poolcnt, pool, lo.pool_cap, first, phase);
+    k_select_pass<T, V, GLOBAL><<<grid, 256, 0, stream>>>(pre, Tn, F, L, lstride, mean, denom, st, hist, poolcnt, pool, lo.pool_cap, first, phase, xcut);
     k_select_scan<KB><<<nprob, SCAN_THREADS, 0, stream>>>(st, hist, poolcnt, phase, 0);
   }
   int gx2 = (int)clt_ceil_div(Tn, 4);
@@ -1359,7 +1395,7 @@ static int run_collect_select(const T *pre, int64_t Tn, int64_t F, int64_t L, in
   if (gx > 65535 * 8) gx = 65535 * 8;
   // retry of the layers whose cut failed: streaming pass from the bottom key over `pre`
   k_select_pass<T, VV, false><<<dim3(gx, (unsigned)L), 256, 0, stream>>>(pre, Tn, F, L, lstride, nullptr, nullptr, st, hist,
-                                                                        poolcnt, pool, lo.pool_cap, first, 1);
+                                                                        poolcnt, pool, lo.pool_cap, first, 1, nullptr);
   k_select_scan<KB><<<(unsigned)L, SCAN_THREADS, 0, stream>>>(st, hist, poolcnt, 1, 0);
   int gx2 = (int)clt_ceil_div(Tn, 4);
   int maxgx2 = (int)clt_ceil_div(256 * 8, L);

@@ -37,6 +37,74 @@ __global__ __launch_bounds__(256) void k_colstats(const T *pre, float *mean, flo
   }
 }
 
+// Vector version: one pass.  A block covers 32 x V columns (V = elements per 16 bytes) with 8
+// row lanes; sums of (x - p) and (x - p)^2 are kept in double, with the column's first value as
+// the pivot p, so the single pass loses nothing to cancellation when the mean is far from zero.
+template <typename T>
+__global__ __launch_bounds__(256) void k_colstats_vec(const T *pre, float *mean, float *denom, int64_t Tn, int64_t F,
+                                                      int64_t lstride) {
+  constexpr int V = Elem<T>::VEC;
+  constexpr int NU = 4;   // loads in flight per thread
+  __shared__ double red[2][8][32 * V];
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+  const int64_t l = blockIdx.y, f0 = ((int64_t)blockIdx.x * 32 + tx) * V;
+  const T *base = pre + l * lstride;
+  const bool on = f0 < F;
+  double s1[V], s2[V];
+  float piv[V];
+#pragma unroll
+  for (int j = 0; j < V; ++j) { s1[j] = 0.0; s2[j] = 0.0; piv[j] = 0.0f; }
+  auto unpack = [](const uint4 &w, float (&x)[V]) {
+    if constexpr (sizeof(T) == 2) {
+      const uint32_t u[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) { x[2 * j] = __uint_as_float(u[j] << 16); x[2 * j + 1] = __uint_as_float(u[j] & 0xFFFF0000u); }
+    } else {
+      x[0] = __uint_as_float(w.x); x[1] = __uint_as_float(w.y); x[2] = __uint_as_float(w.z); x[3] = __uint_as_float(w.w);
+    }
+  };
+  if (on) {
+    unpack(*reinterpret_cast<const uint4 *>(base + f0), piv);
+    for (int64_t t0 = ty; t0 < Tn; t0 += 8 * NU) {
+      uint4 w[NU];
+#pragma unroll
+      for (int u = 0; u < NU; ++u) {
+        const int64_t t = t0 + (int64_t)u * 8;
+        w[u] = t < Tn ? *reinterpret_cast<const uint4 *>(base + t * F + f0) : make_uint4(0, 0, 0, 0);
+      }
+#pragma unroll
+      for (int u = 0; u < NU; ++u) {
+        if (t0 + (int64_t)u * 8 >= Tn) break;
+        float x[V];
+        unpack(w[u], x);
+#pragma unroll
+        for (int j = 0; j < V; ++j) { const double dl = (double)x[j] - (double)piv[j]; s1[j] += dl; s2[j] = fma(dl, dl, s2[j]); }
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < V; ++j) { red[0][ty][tx * V + j] = s1[j]; red[1][ty][tx * V + j] = s2[j]; }
+  __syncthreads();
+  // 256 threads finish the 32 * V columns: thread c < 32 * V takes column c
+  const int c = threadIdx.x;
+  if (c < 32 * V) {
+    const int64_t f = (int64_t)blockIdx.x * 32 * V + c;
+    if (f < F) {
+      double a = 0.0, q = 0.0;
+#pragma unroll
+      for (int r = 0; r < 8; ++r) { a += red[0][r][c]; q += red[1][r][c]; }
+      const double p = (double)Elem<T>::to_f32(base[f]);
+      const double n = (double)Tn;
+      const double mu = p + a / n;
+      double var = (q - a * a / n) / (n - 1.0);   // T == 1 gives NaN, as torch.std does
+      if (var < 0.0) var = 0.0;
+      mean[l * F + f] = Elem<T>::round((float)mu);
+      const float sd = Elem<T>::round((float)sqrt(var));
+      denom[l * F + f] = Elem<T>::round(sd + 1e-6f);
+    }
+  }
+}
+
 }  // namespace
 
 extern "C" int clt_version(void) { return 100; }
@@ -58,8 +126,15 @@ extern "C" int clt_colstats(const void *pre, float *mean, float *denom, int64_t 
                             int64_t pre_layer_stride, int dtype, void *stream) {
   if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
   if (T <= 0 || F <= 0 || L <= 0 || L > 65535 || !pre || !mean || !denom) return CLT_ERR_ARG;
-  dim3 grid((unsigned)clt_ceil_div(F, 64), (unsigned)L);
   hipStream_t s = (hipStream_t)stream;
+  const int V = dtype == CLT_BF16 ? 8 : 4;
+  if (F % V == 0 && clt_aligned16(pre) && (pre_layer_stride % V) == 0) {
+    dim3 gridv((unsigned)clt_ceil_div(F, 32 * V), (unsigned)L);
+    if (dtype == CLT_BF16) k_colstats_vec<bf16_t><<<gridv, 256, 0, s>>>((const bf16_t *)pre, mean, denom, T, F, pre_layer_stride);
+    else k_colstats_vec<float><<<gridv, 256, 0, s>>>((const float *)pre, mean, denom, T, F, pre_layer_stride);
+    return clt_check_launch();
+  }
+  dim3 grid((unsigned)clt_ceil_div(F, 64), (unsigned)L);
   if (dtype == CLT_BF16) k_colstats<bf16_t><<<grid, 256, 0, s>>>((const bf16_t *)pre, mean, denom, T, F, pre_layer_stride);
   else k_colstats<float><<<grid, 256, 0, s>>>((const float *)pre, mean, denom, T, F, pre_layer_stride);
   return clt_check_launch();
