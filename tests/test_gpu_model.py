@@ -54,6 +54,12 @@ CASES = [
     BASE.scaled("tiny-topk-global", activation_fn="topk", k=6, topk_mode="global", dtype="bfloat16"),
     BASE.scaled("ref-shape", num_layers=2, d_model=8, num_features=16, tokens=30, k=3),   # the reference's own test shape
     BASE.scaled("mid", num_layers=4, d_model=768, num_features=2048, tokens=300, k=20, dtype="bfloat16"),
+    # shapes that take the routes fused into the encoder epilogue (T % 256 == 0, F % 256 == 0)
+    BASE.scaled("fused-topk", num_layers=3, d_model=128, num_features=512, tokens=256, k=12),
+    BASE.scaled("fused-topk-bf16", num_layers=3, d_model=256, num_features=1024, tokens=512, k=24, dtype="bfloat16"),
+    BASE.scaled("fused-jump", num_layers=3, d_model=128, num_features=512, tokens=256, activation_fn="jumprelu", k=None),
+    BASE.scaled("fused-jump-bf16", num_layers=3, d_model=256, num_features=1024, tokens=512, activation_fn="jumprelu",
+                k=None, dtype="bfloat16"),
 ]
 
 
@@ -95,6 +101,26 @@ def test_forward_matches_oracle(dev, wl):
     for l in pre:
         assert orc.rel_l2(pre[l], orc.encoder_preactivations(x[l], sd[f"encoder_module.encoders.{l}.weight"],
                                                               sd[f"encoder_module.encoders.{l}.bias_param"])) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("fn", ["batchtopk", "jumprelu"])
+def test_fused_routes_equal_separate_kernels_in_the_model(dev, fn):
+    # same model, same inputs: with and without the encoder-epilogue routes, all layers and a subset
+    wl = BASE.scaled("f", num_layers=3, d_model=256, num_features=1024, tokens=512, k=24 if fn == "batchtopk" else None,
+                     activation_fn=fn, dtype="bfloat16")
+    model, sd, x = build(wl, dev)
+    for layers in ([0, 1, 2], [0, 2]):
+        inputs = {l: x[l].to(dev) for l in layers}
+        model.fuse_encode_select = True
+        a1 = model.get_feature_activations(inputs)
+        r1 = model(inputs)
+        model.fuse_encode_select = False
+        a2 = model.get_feature_activations(inputs)
+        r2 = model(inputs)
+        assert sorted(a1) == sorted(a2) == layers
+        for l in layers:
+            assert torch.equal(a1[l], a2[l])
+            assert torch.equal(r1[l], r2[l])
 
 
 def test_decode_api_matches_forward(dev):
