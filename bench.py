@@ -154,6 +154,7 @@ def run_gpu(args):
     n_dec_launch = L if T * L >= engine.SLICED_DECODE_MIN_ROWS else 1
     dec_kernel_desc = (f"k_decode (sparse cross-layer decode; {n_dec_launch} launch(es) per step; the per-launch "
                        "figures are the step's decode stage divided by that count)")
+    traffic = MEASURED_TRAFFIC.get((wl.name, n_dec_launch))
     mfma_peak = MFMA_BF16_PEAK_TF if wl.dtype == "bfloat16" else MFMA_FP32_PEAK_TF
     result = {
         "metric": "CLT forward tokens/sec at GPT-2-small x32 BatchTopK k=200; % of roofline per stage",
@@ -184,7 +185,11 @@ def run_gpu(args):
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": dec_gbs / HBM_PEAK_GBS,
-            "traffic": MEASURED_TRAFFIC.get((wl.name, n_dec_launch)),
+            "traffic": traffic,
+            "traffic_GBps": (traffic / (st["decode"] / n_dec_launch * 1e-3) / 1e9) if traffic else None,
+            "note": ("achieved = gathered bytes (every active (token, feature, source->target) fetches one decoder row) per "
+                     "launch / launch time; it exceeds the HBM peak because most rows are served by the L2s; traffic = "
+                     "HBM bytes per launch from FETCH_SIZE + WRITE_SIZE"),
             "algorithmic_bytes_per_launch": work["decode_gathered_bytes"] / n_dec_launch,
             "avg_launch_ms": st["decode"] / n_dec_launch,
             "launches_per_step": n_dec_launch,
