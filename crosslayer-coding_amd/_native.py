@@ -33,6 +33,8 @@ _SIGNATURES = {
     "clt_error_string": (ctypes.c_char_p, [_int]),
     "clt_encode": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _int, _vp]),
     "clt_colstats": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
+    "clt_colstats_full": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
+    "clt_selected_min_accumulate": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp, _vp, _vp, _sz, _vp]),
     "clt_batchtopk_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64, _int, _int]),
     "clt_batchtopk_select": (_int, [_vp, _i64, _i64, _i64, _i64, _i64, _int, _vp, _vp, _int, _vp, _vp, _vp, _vp, _sz, _vp]),
     "clt_encode_collect_supported": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _int]),

@@ -140,11 +140,23 @@ class CrossLayerTranscoder(BaseTranscoder):
             raise AttributeError("ThetaManager is not initialised; cannot set log_threshold.")
         self.theta_manager.log_threshold = new_param
 
-    def estimate_theta_posthoc(self, *args, **kwargs):
-        return self.theta_manager.estimate_theta_posthoc(*args, **kwargs)
+    @torch.no_grad()
+    def estimate_theta_posthoc(self, data_iter, num_batches: Optional[int] = None, default_theta_value: float = 1e6,
+                               device: Optional[torch.device] = None) -> torch.Tensor:
+        """Estimate theta post-hoc using a specified number of batches (clt.py:282-307).  The
+        estimation runs where the model lives; ``device`` is accepted for signature parity."""
+        if device is not None and torch.device(device) != self.theta_manager.device:
+            logger.info(f"Rank {self.rank}: theta estimation stays on {self.theta_manager.device} (asked for {device}).")
+        return self.theta_manager.estimate_theta_posthoc(
+            encode_all_layers_fn=self.encoder_module.encode_all_layers, data_iter=data_iter, num_batches=num_batches,
+            default_theta_value=default_theta_value)
 
-    def convert_to_jumprelu_inplace(self, *args, **kwargs):
-        return self.theta_manager.convert_to_jumprelu_inplace(*args, **kwargs)
+    @torch.no_grad()
+    def convert_to_jumprelu_inplace(self, default_theta_value: float = 1e6) -> None:
+        """BatchTopK / TokenTopK -> JumpReLU from the estimated statistics (clt.py:309-318); the
+        ThetaManager updates the config object it shares with the model."""
+        self.theta_manager.convert_to_jumprelu_inplace(default_theta_value=default_theta_value)
+        logger.info(f"Rank {self.rank}: CLT model config updated by ThetaManager. New activation_fn='{self.config.activation_fn}'.")
 
     # ---- encode (per-layer activations) ---------------------------------------------------
     def encode(self, x: torch.Tensor, layer_idx: int) -> torch.Tensor:

@@ -888,6 +888,40 @@ __global__ __launch_bounds__(256) void k_tile_emit(
   for (uint32_t e = TILE_NE; e < m.y; ++e) put(mypool[m.x + e]);
 }
 
+// ---- post-hoc threshold estimation: per-feature minimum of the selected z-scores ---------------
+// keys[l][f] = min over the survivors (l, token, f, v) with v > 0 of key32(z(v)), z evaluated in
+// the model dtype like the ranking value (reference clt/models/theta.py:127-139, which takes the
+// minimum of the NORMALISED pre-activations where the gated activation is positive).
+template <typename T>
+__global__ __launch_bounds__(256) void k_selected_min(const int32_t *row_ptr, const int32_t *col, const T *val,
+                                                      const float *mean, const float *denom, int64_t Tn, int64_t F,
+                                                      int64_t L, uint32_t *keys) {
+  const int lane = lane_id(), wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
+  const int64_t R = L * Tn;
+  for (int64_t r = (int64_t)blockIdx.x * nwv + wv; r < R; r += (int64_t)gridDim.x * nwv) {
+    const int64_t l = r / Tn;
+    RankZ<T> rk; rk.mean = mean + l * F; rk.denom = denom + l * F;
+    for (int32_t j = row_ptr[r] + lane; j < row_ptr[r + 1]; j += 64) {
+      const float v = Elem<T>::to_f32(val[j]);
+      if (v > 0.0f) atomicMin(&keys[l * F + col[j]], rank_key32(rk(v, col[j])));
+    }
+  }
+}
+
+// sum[l][f] += min, count[l][f] += 1 where a finite minimum was seen (both buffers in the model
+// dtype, every addition rounded to it: theta.py:163-167).
+template <typename T>
+__global__ void k_selected_min_accumulate(const uint32_t *keys, int64_t n, T *sum, T *count) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+    const uint32_t k = keys[i];
+    const float z = __uint_as_float(key_to_f32_bits<32>(k));
+    if (k != 0xFFFFFFFFu && z == z && fabsf(z) != __uint_as_float(0x7F800000u)) {
+      sum[i] = Elem<T>::from_f32(Elem<T>::to_f32(sum[i]) + z);
+      count[i] = Elem<T>::from_f32(Elem<T>::to_f32(count[i]) + 1.0f);
+    }
+  }
+}
+
 // ---- threshold activation on encoder-collected entries (every entry is a survivor) ----------
 // Per row: exclusive prefix of the run lengths over the segments, and the row total.
 __global__ __launch_bounds__(256) void k_row_prefix_meta(int64_t Tn, int nseg, const uint2 *seg_meta, uint32_t *pfx,
@@ -1645,6 +1679,26 @@ extern "C" int clt_threshold_emit(const void *pre, int64_t T, int64_t F, int64_t
   hipStream_t s = (hipStream_t)stream;
   if (dtype == CLT_BF16) return dispatch_threshold<bf16_t>(true, pre, T, F, L, pre_layer_stride, theta, pred, nullptr, (int32_t *)row_ptr, col, val, s);
   return dispatch_threshold<float>(true, pre, T, F, L, pre_layer_stride, theta, pred, nullptr, (int32_t *)row_ptr, col, val, s);
+}
+
+extern "C" int clt_selected_min_accumulate(const int32_t *row_ptr, const int32_t *col, const void *val, const float *mean,
+                                           const float *denom, int64_t T, int64_t F, int64_t L, int dtype, void *sum,
+                                           void *count, void *workspace, size_t workspace_bytes, void *stream) {
+  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (T <= 0 || F <= 0 || L <= 0 || !row_ptr || !mean || !denom || !sum || !count || !workspace) return CLT_ERR_ARG;
+  if (workspace_bytes < (size_t)L * (size_t)F * 4) return CLT_ERR_WORKSPACE;
+  hipStream_t s = (hipStream_t)stream;
+  uint32_t *keys = (uint32_t *)workspace;
+  const int64_t n = L * F;
+  k_fill_u32<<<256, 256, 0, s>>>(keys, 0xFFFFFFFFu, n);
+  if (dtype == CLT_BF16) {
+    k_selected_min<bf16_t><<<2048, 256, 0, s>>>(row_ptr, col, (const bf16_t *)val, mean, denom, T, F, L, keys);
+    k_selected_min_accumulate<bf16_t><<<256, 256, 0, s>>>(keys, n, (bf16_t *)sum, (bf16_t *)count);
+  } else {
+    k_selected_min<float><<<2048, 256, 0, s>>>(row_ptr, col, (const float *)val, mean, denom, T, F, L, keys);
+    k_selected_min_accumulate<float><<<256, 256, 0, s>>>(keys, n, (float *)sum, (float *)count);
+  }
+  return clt_check_launch();
 }
 
 extern "C" size_t clt_tokentopk_workspace_bytes(int64_t T, int64_t F, int64_t L, int64_t kk, int mode, int dtype) {

@@ -7,8 +7,8 @@ namespace {
 // One block = 64 feature columns x 4 row groups; two passes over the column
 // (mean, then centred sum of squares) with double accumulation.
 template <typename T>
-__global__ __launch_bounds__(256) void k_colstats(const T *pre, float *mean, float *denom, int64_t Tn, int64_t F,
-                                                  int64_t lstride) {
+__global__ __launch_bounds__(256) void k_colstats(const T *pre, float *mean, float *denom, float *stdv, int64_t Tn,
+                                                  int64_t F, int64_t lstride) {
   __shared__ double red[4][64];
   __shared__ double smean[64];
   const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
@@ -34,6 +34,7 @@ __global__ __launch_bounds__(256) void k_colstats(const T *pre, float *mean, flo
     float sd = Elem<T>::round((float)sqrt(var));
     mean[l * F + f] = m;
     denom[l * F + f] = Elem<T>::round(sd + 1e-6f);
+    if (stdv) stdv[l * F + f] = sd;
   }
 }
 
@@ -41,8 +42,8 @@ __global__ __launch_bounds__(256) void k_colstats(const T *pre, float *mean, flo
 // row lanes; sums of (x - p) and (x - p)^2 are kept in double, with the column's first value as
 // the pivot p, so the single pass loses nothing to cancellation when the mean is far from zero.
 template <typename T>
-__global__ __launch_bounds__(256) void k_colstats_vec(const T *pre, float *mean, float *denom, int64_t Tn, int64_t F,
-                                                      int64_t lstride) {
+__global__ __launch_bounds__(256) void k_colstats_vec(const T *pre, float *mean, float *denom, float *stdv, int64_t Tn,
+                                                      int64_t F, int64_t lstride) {
   constexpr int V = Elem<T>::VEC;
   constexpr int NU = 4;   // loads in flight per thread
   __shared__ double red[2][8][32 * V];
@@ -101,6 +102,7 @@ __global__ __launch_bounds__(256) void k_colstats_vec(const T *pre, float *mean,
       mean[l * F + f] = Elem<T>::round((float)mu);
       const float sd = Elem<T>::round((float)sqrt(var));
       denom[l * F + f] = Elem<T>::round(sd + 1e-6f);
+      if (stdv) stdv[l * F + f] = sd;
     }
   }
 }
@@ -122,20 +124,31 @@ extern "C" const char *clt_error_string(int code) {
   }
 }
 
-extern "C" int clt_colstats(const void *pre, float *mean, float *denom, int64_t T, int64_t F, int64_t L,
-                            int64_t pre_layer_stride, int dtype, void *stream) {
+static int run_colstats(const void *pre, float *mean, float *denom, float *stdv, int64_t T, int64_t F, int64_t L,
+                        int64_t pre_layer_stride, int dtype, void *stream) {
   if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
   if (T <= 0 || F <= 0 || L <= 0 || L > 65535 || !pre || !mean || !denom) return CLT_ERR_ARG;
   hipStream_t s = (hipStream_t)stream;
   const int V = dtype == CLT_BF16 ? 8 : 4;
   if (F % V == 0 && clt_aligned16(pre) && (pre_layer_stride % V) == 0) {
     dim3 gridv((unsigned)clt_ceil_div(F, 32 * V), (unsigned)L);
-    if (dtype == CLT_BF16) k_colstats_vec<bf16_t><<<gridv, 256, 0, s>>>((const bf16_t *)pre, mean, denom, T, F, pre_layer_stride);
-    else k_colstats_vec<float><<<gridv, 256, 0, s>>>((const float *)pre, mean, denom, T, F, pre_layer_stride);
+    if (dtype == CLT_BF16) k_colstats_vec<bf16_t><<<gridv, 256, 0, s>>>((const bf16_t *)pre, mean, denom, stdv, T, F, pre_layer_stride);
+    else k_colstats_vec<float><<<gridv, 256, 0, s>>>((const float *)pre, mean, denom, stdv, T, F, pre_layer_stride);
     return clt_check_launch();
   }
   dim3 grid((unsigned)clt_ceil_div(F, 64), (unsigned)L);
-  if (dtype == CLT_BF16) k_colstats<bf16_t><<<grid, 256, 0, s>>>((const bf16_t *)pre, mean, denom, T, F, pre_layer_stride);
-  else k_colstats<float><<<grid, 256, 0, s>>>((const float *)pre, mean, denom, T, F, pre_layer_stride);
+  if (dtype == CLT_BF16) k_colstats<bf16_t><<<grid, 256, 0, s>>>((const bf16_t *)pre, mean, denom, stdv, T, F, pre_layer_stride);
+  else k_colstats<float><<<grid, 256, 0, s>>>((const float *)pre, mean, denom, stdv, T, F, pre_layer_stride);
   return clt_check_launch();
+}
+
+extern "C" int clt_colstats(const void *pre, float *mean, float *denom, int64_t T, int64_t F, int64_t L,
+                            int64_t pre_layer_stride, int dtype, void *stream) {
+  return run_colstats(pre, mean, denom, nullptr, T, F, L, pre_layer_stride, dtype, stream);
+}
+
+extern "C" int clt_colstats_full(const void *pre, float *mean, float *stdv, float *denom, int64_t T, int64_t F,
+                                 int64_t L, int64_t pre_layer_stride, int dtype, void *stream) {
+  if (!stdv) return CLT_ERR_ARG;
+  return run_colstats(pre, mean, denom, stdv, T, F, L, pre_layer_stride, dtype, stream);
 }

@@ -106,6 +106,35 @@ def colstats(pre: torch.Tensor):
     return mean, denom
 
 
+def colstats_full(pre: torch.Tensor):
+    """(mean, std, denom) fp32 [L, F]: colstats plus the unbiased std itself (theta.py:305-318)."""
+    L, T, F = _check_pre(pre)
+    mean = torch.empty((L, F), dtype=torch.float32, device=pre.device)
+    std = torch.empty_like(mean)
+    denom = torch.empty_like(mean)
+    code = nat.load().clt_colstats_full(nat.ptr(pre), nat.ptr(mean), nat.ptr(std), nat.ptr(denom), T, F, L,
+                                        pre.stride(0), nat.dtype_code(pre.dtype), _stream(pre))
+    nat.check(code, "clt_colstats_full")
+    return mean, std, denom
+
+
+def selected_min_accumulate(surv: SurvivorList, mean: torch.Tensor, denom: torch.Tensor, sum_buf: torch.Tensor,
+                            count_buf: torch.Tensor, ws: Optional[Workspace] = None) -> None:
+    """sum_buf / count_buf [L, F] (model dtype) += the per-feature minimum z-score of the positive
+    survivors of this batch / 1 (theta.py:82-173)."""
+    L, F = surv.L, surv.F
+    assert sum_buf.shape == (L, F) and count_buf.shape == (L, F)
+    assert sum_buf.dtype == surv.dtype and count_buf.dtype == surv.dtype
+    assert sum_buf.is_contiguous() and count_buf.is_contiguous()
+    dev = surv.row_ptr.device
+    wbuf = (ws or Workspace(dev)).get("selected_min", L * F * 4)
+    code = nat.load().clt_selected_min_accumulate(
+        nat.ptr(surv.row_ptr), nat.ptr(surv.col), nat.ptr(surv.val), nat.ptr(mean), nat.ptr(denom), surv.T, F, L,
+        nat.dtype_code(surv.dtype), nat.ptr(sum_buf), nat.ptr(count_buf), nat.ptr(wbuf), wbuf.numel(),
+        nat.current_stream(dev))
+    nat.check(code, "clt_selected_min_accumulate")
+
+
 def _check_pre(pre: torch.Tensor):
     nat.require_device(pre, "select")
     L, T, F = pre.shape

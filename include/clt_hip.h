@@ -88,6 +88,29 @@ int clt_colstats(const void *pre, float *mean, float *denom,
                  int dtype, void *stream);
 
 /*
+ * As clt_colstats, and also stdv[l][f] = the unbiased std itself (rounded to the model dtype,
+ * stored as fp32), which the post-hoc threshold estimation averages over batches
+ * (clt/models/theta.py:305-318).
+ */
+int clt_colstats_full(const void *pre, float *mean, float *stdv, float *denom,
+                      int64_t T, int64_t F, int64_t L, int64_t pre_layer_stride,
+                      int dtype, void *stream);
+
+/*
+ * One batch of the post-hoc threshold estimation
+ * (ThetaManager._update_min_selected_preactivations, clt/models/theta.py:82-173): for every
+ * (layer, feature), the minimum over the survivors with a positive value of their z-score
+ * (x - mean) / denom evaluated in the model dtype; where that minimum is finite,
+ * sum[l][f] += min and count[l][f] += 1 (both [L][F] in the model dtype, each addition
+ * rounded to it).  workspace: L*F*4 bytes.
+ */
+int clt_selected_min_accumulate(const int32_t *row_ptr, const int32_t *col, const void *val,
+                                const float *mean, const float *denom,
+                                int64_t T, int64_t F, int64_t L, int dtype,
+                                void *sum, void *count,
+                                void *workspace, size_t workspace_bytes, void *stream);
+
+/*
  * BatchTopK selection into a survivor list.
  *   mode CLT_TOPK_PER_LAYER: for each layer, the min(k*T, T*F) largest of its T*F
  *     pre-activations (ranking on the raw value), i.e. BatchTopK._compute_mask

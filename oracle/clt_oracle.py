@@ -27,6 +27,10 @@ How each function is pinned (see ``tests/test_oracle_*.py``):
 * ``global_batchtopk``  - closed form of the z-score on hand-computable columns;
   the reference has no golden numbers for it: PARITY UNPINNED beyond that
   closed form (its tests only check shapes, test_clt_encode_decode.py:70-116).
+* ``theta_estimate_posthoc`` / ``theta_convert``  - a hand-computed two-feature case and the
+  properties the reference's own test asserts (tests/unit/models/test_theta.py:110-175:
+  thresholds finite and positive, higher for the features that were selected); the
+  reference holds no golden numbers for them: PARITY UNPINNED beyond that.
 * ``forward``  - composition of the above; the reference has no golden tensors
   for a full forward: PARITY UNPINNED beyond shape/keys and the pins of its parts.
 
@@ -418,6 +422,74 @@ def forward(inputs: Dict[int, torch.Tensor], *, enc_w, enc_b, dec_w, dec_b,
             b = x.shape[0] * x.shape[1] if x.dim() == 3 else x.shape[0]
             recs[t] = torch.zeros((b, d_model), dtype=dtype)
     return recs, acts
+
+
+# ---------------------------------------------------------------------------
+# post-hoc theta estimation and BatchTopK -> JumpReLU conversion
+# ---------------------------------------------------------------------------
+
+def theta_estimate_posthoc(batches: List[Dict[int, torch.Tensor]], *, activation_fn: str, k: float,
+                           num_layers: int, num_features: int, dtype: torch.dtype):
+    """ThetaManager.estimate_theta_posthoc up to the conversion (theta.py:175-416), for
+    batches of pre-activation dicts in which every layer is present with the same token
+    count.  Per batch: per-layer mean / unbiased std over the tokens and the z-score
+    (theta.py:305-307), the averaged statistics (:314-318), the global BatchTopK / TokenTopK
+    gate ranked on the z-score with the raw values kept (:350-391), and
+    _update_min_selected_preactivations (:82-173): per feature the minimum of the z-scores where
+    the gated activation is positive; where it is finite, sum += min and count += 1.
+    Returns (sum, count, avg_means, avg_stds), all [L, F] in ``dtype``."""
+    L, F_ = num_layers, num_features
+    ssum = torch.zeros((L, F_), dtype=dtype)
+    scnt = torch.zeros((L, F_), dtype=dtype)
+    mus = torch.zeros((L, F_), dtype=dtype)
+    sigmas = torch.zeros((L, F_), dtype=dtype)
+    nb = torch.zeros(L, dtype=torch.long)
+    for pre in batches:
+        orig, norm = [], []
+        for l in range(L):
+            p = pre[l].to(dtype)
+            mean = p.mean(dim=0, keepdim=True)
+            std = p.std(dim=0, keepdim=True)
+            orig.append(p)
+            norm.append((p - mean) / (std + 1e-6))
+            mus[l] += mean.squeeze(0)
+            sigmas[l] += std.squeeze(0)
+            nb[l] += 1
+        gating = torch.cat(orig, dim=1)
+        ranking = torch.cat(norm, dim=1)
+        if activation_fn == "batchtopk":
+            gated = batchtopk_forward(gating, float(int(k)), ranking)
+        else:
+            gated = tokentopk_forward(gating, float(k), ranking)
+        for l in range(L):
+            z = ranking[:, l * F_:(l + 1) * F_]
+            active = gated[:, l * F_:(l + 1) * F_] > 0
+            if active.any():
+                per_feature_min = torch.where(active, z, torch.full_like(z, float("inf"))).amin(dim=0)
+                valid = torch.isfinite(per_feature_min)
+                ssum[l, valid] += per_feature_min[valid]
+                scnt[l, valid] += 1
+    active_batches = nb.unsqueeze(-1).clamp_min(1.0)
+    mus /= active_batches
+    sigmas /= active_batches
+    return ssum, scnt, mus, sigmas
+
+
+def theta_convert(ssum: torch.Tensor, scnt: torch.Tensor, mus: torch.Tensor, sigmas: torch.Tensor) -> torch.Tensor:
+    """ThetaManager.convert_to_jumprelu_inplace at world_size 1 (theta.py:466-573): per layer the
+    mean of the finite positive per-feature normalised thetas (fallback 1e-5), un-normalised
+    with sigma.clamp_min(1e-6) and mu, clamped below at 1e-7; returns log(theta) [L, F]."""
+    theta_raw = torch.zeros_like(ssum)
+    for l in range(ssum.shape[0]):
+        active = scnt[l] > 0
+        per_feature = torch.full_like(ssum[l], float("inf"))
+        if active.any():
+            per_feature[active] = ssum[l][active] / scnt[l][active].clamp_min(1.0)
+        pos = per_feature[torch.isfinite(per_feature) & (per_feature > 0)]
+        scalar = pos.mean().item() if pos.numel() > 0 else 1e-5
+        theta_raw[l] = scalar * sigmas[l].clamp_min(1e-6) + mus[l]
+    theta_raw.clamp_min_(1e-7)
+    return torch.log(theta_raw)
 
 
 # ---------------------------------------------------------------------------

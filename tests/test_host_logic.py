@@ -3,6 +3,8 @@ registry, construction-time behaviour.  CPU only; nothing here computes on a dev
 import json
 import math
 
+import logging
+
 import pytest
 import torch
 
@@ -131,8 +133,9 @@ def test_cpu_fallback_shapes_without_kernels(caplog):
     out = m.get_preactivations(torch.randn(2, 3, 4, 8), 0)    # 4-D
     assert out.shape == (2, 16)
     assert m.decode({}, 0).shape == (0, 8)
-    with pytest.raises(NotImplementedError):
-        m.estimate_theta_posthoc(None)
+    # conversion before any estimation: no statistics yet (reference tests/unit/models/test_theta.py:104-108)
+    with pytest.raises(RuntimeError, match="Required buffer"):
+        m.convert_to_jumprelu_inplace()
 
 
 def test_workload_table_matches_baseline_shapes():
@@ -147,3 +150,15 @@ def test_workload_table_matches_baseline_shapes():
     sd = synth.make_state_dict(small)
     assert float(sd["encoder_module.encoders.0.weight"].abs().max()) <= 1 / math.sqrt(16)
     assert sd["decoder_module.decoders.0->1.weight"].shape == (16, 32)
+
+
+def test_convert_to_jumprelu_requires_estimation_first():
+    # reference tests/unit/models/test_theta.py:104-108
+    import pytest
+    from crosslayer_coding_amd.config import CLTConfig
+    from crosslayer_coding_amd.theta import ThetaManager
+
+    cfg = CLTConfig(num_layers=2, d_model=8, num_features=4, activation_fn="batchtopk", batchtopk_k=2)
+    tm = ThetaManager(cfg, None, torch.device("cpu"), torch.float32)
+    with pytest.raises(RuntimeError, match="Required buffer .* not found"):
+        tm.convert_to_jumprelu_inplace()

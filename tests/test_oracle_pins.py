@@ -234,3 +234,36 @@ def test_forward_wiring_small():
     assert sum(int((a != 0).sum()) for a in acts.values()) == 3 * T
     r1 = acts[0] @ w["0->1"].T + b["0->1"] + acts[1] @ w["1->1"].T + b["1->1"]
     assert torch.allclose(recs[1], r1, atol=1e-5)
+
+
+# ---- post-hoc theta estimation: hand-computed case + the reference test's properties ------------
+def test_theta_estimation_hand_computed():
+    # one layer, two features, four tokens, k = 1 per token -> 4 survivors over the [4, 2] block.
+    # feature 0: 10, 11, 12, 13  (mean 11.5, unbiased std sqrt(5/3)); feature 1: 0, 0, 0, 4 (mean 1, std 2)
+    pre = {0: torch.tensor([[10.0, 0.0], [11.0, 0.0], [12.0, 0.0], [13.0, 4.0]])}
+    s, c, mu, sg = orc.theta_estimate_posthoc([pre], activation_fn="batchtopk", k=1, num_layers=1, num_features=2,
+                                              dtype=torch.float32)
+    sd0 = math.sqrt(5.0 / 3.0)
+    z0 = [(v - 11.5) / (sd0 + 1e-6) for v in (10.0, 11.0, 12.0, 13.0)]      # -1.16, -0.39, 0.39, 1.16
+    z1 = [(v - 1.0) / (2.0 + 1e-6) for v in (0.0, 0.0, 0.0, 4.0)]           # -0.5, -0.5, -0.5, 1.5
+    # the four largest z-scores: 1.5 (f1,t3), 1.16 (f0,t3), 0.39 (f0,t2), then -0.39 (f0,t1)
+    assert c.tolist() == [[1.0, 1.0]]
+    assert abs(float(s[0, 0]) - z0[1]) < 1e-6 and abs(float(s[0, 1]) - z1[3]) < 1e-6
+    assert torch.allclose(mu, torch.tensor([[11.5, 1.0]])) and torch.allclose(sg, torch.tensor([[sd0, 2.0]]))
+    # conversion: feature 0's theta is negative, so the layer scalar is the mean of the positive ones = z1[3]
+    log_t = orc.theta_convert(s, c, mu, sg)
+    expect = torch.tensor([[z1[3] * sd0 + 11.5, z1[3] * 2.0 + 1.0]])
+    assert torch.allclose(torch.exp(log_t), expect, rtol=1e-5)
+
+
+def test_theta_estimation_reference_test_properties():
+    # reference tests/unit/models/test_theta.py:110-175: consistently selected features end up with
+    # higher thresholds than the others; all thresholds finite and positive
+    g = torch.Generator().manual_seed(0)
+    l0 = torch.cat([torch.randn(4, 2, generator=g) + 5, torch.randn(4, 2, generator=g)], dim=1)
+    l1 = torch.cat([torch.randn(4, 2, generator=g), torch.randn(4, 2, generator=g) + 5], dim=1)
+    s, c, mu, sg = orc.theta_estimate_posthoc([{0: l0, 1: l1}], activation_fn="batchtopk", k=2, num_layers=2,
+                                              num_features=4, dtype=torch.float32)
+    theta = torch.exp(orc.theta_convert(s, c, mu, sg))
+    assert bool(torch.isfinite(theta).all()) and bool((theta > 0).all())
+    assert bool((theta[0, :2].min() > theta[0, 2:].max())) and bool((theta[1, 2:].min() > theta[1, :2].max()))
