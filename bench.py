@@ -218,6 +218,38 @@ def run_gpu(args):
     return result
 
 
+def run_theta(args):
+    """Post-hoc theta estimation (reference clt/models/theta.py:175-430) over ``steps`` batches of the
+    workload's inputs; one step = one batch: encoder, per-feature statistics, global BatchTopK ranked
+    on the z-score, per-feature minimum of the selected z-scores."""
+    import crosslayer_coding_amd as cca
+    from crosslayer_coding_amd import synth
+
+    wl = synth.WORKLOADS[args.workload].scaled(args.workload + "-global", topk_mode="global")
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    cca._native.load(build_if_missing=False)
+    model, inputs, _ = synth.build_model(wl, dev)
+    model.eval()
+    data = [(inputs, None)] * (args.warmup + args.steps)
+    k, fn = model.config.batchtopk_k, model.config.activation_fn
+    model.estimate_theta_posthoc(data[:args.warmup], num_batches=args.warmup)
+    model.config.activation_fn, model.config.batchtopk_k = fn, k       # estimate again from the same starting point
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    model.estimate_theta_posthoc(data[:args.steps], num_batches=args.steps)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return {
+        "metric": "post-hoc theta estimation tokens/sec (encoder + statistics + global BatchTopK + selected minimum)",
+        "value": wl.tokens * args.steps / wall, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": wall / args.steps * 1e3, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16" if wl.dtype == "bfloat16" else "f32", "data": "synthetic",
+        "config": {"workload": f"{wl.name}: theta estimation, L={wl.num_layers} d_model={wl.d_model} "
+                               f"F={wl.num_features} T={wl.tokens} batchtopk k={wl.k} (global)"},
+    }
+
+
 def cpu_baseline(wl, model, slab, tokens):
     """The reference's dense forward (F.linear encoder, torch.topk mask, one dense F.linear
     per decoder, sum in the model dtype) from ``oracle/``, on the first ``tokens`` tokens of
@@ -263,6 +295,9 @@ def main():
     ap.add_argument("--no-fuse", action="store_true", help="separate encoder and selection kernels")
     ap.add_argument("--topk-mode", choices=["per_layer", "global"], default=None,
                     help="override the workload's BatchTopK scope (global = the reference's default helper)")
+    ap.add_argument("--theta-estimation", action="store_true",
+                    help="time batches of the post-hoc theta estimation (encoder, column statistics, global "
+                         "selection, per-feature minimum) instead of the forward")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one 256 MiB elementwise copy (counter yardstick for profiled runs)")
     args = ap.parse_args()
@@ -273,7 +308,7 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a ROCm GPU", file=sys.stderr)
         sys.exit(2)
-    print(json.dumps(run_gpu(args)))
+    print(json.dumps(run_theta(args) if args.theta_estimation else run_gpu(args)))
 
 
 if __name__ == "__main__":

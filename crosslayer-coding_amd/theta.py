@@ -134,10 +134,11 @@ class ThetaManager(nn.Module):
             slab, good = got
             L, T, F = slab.shape
             mean, std, denom = engine.colstats_full(slab)
-            for l in good:   # averaged normalisation statistics, accumulated in the model dtype (theta.py:314-318)
-                self._avg_layer_means.data[l] += mean[l].to(self.dtype)
-                self._avg_layer_stds.data[l] += std[l].to(self.dtype)
-                self._processed_batches_for_stats.data[l] += 1
+            # averaged normalisation statistics, accumulated in the model dtype (theta.py:314-318)
+            sel = slice(None) if len(good) == L else torch.tensor(good, device=self.device)
+            self._avg_layer_means.data[sel] += mean[sel].to(self.dtype)
+            self._avg_layer_stds.data[sel] += std[sel].to(self.dtype)
+            self._processed_batches_for_stats.data[sel] += 1
             if len(good) < L:   # zero-filled layers rank on zeros: mean 0, denominator std 1 + 1e-6 (theta.py:281-282)
                 bad = [l for l in range(L) if l not in good]
                 mean[bad] = 0.0
