@@ -158,6 +158,51 @@ class CrossLayerTranscoder(BaseTranscoder):
         self.theta_manager.convert_to_jumprelu_inplace(default_theta_value=default_theta_value)
         logger.info(f"Rank {self.rank}: CLT model config updated by ThetaManager. New activation_fn='{self.config.activation_fn}'.")
 
+    # ---- loss and gradients --------------------------------------------------------------------
+    @torch.no_grad()
+    def loss_and_gradients(self, inputs: Dict[int, torch.Tensor], targets: Dict[int, torch.Tensor]):
+        """MSE reconstruction loss (sum over layers of the per-layer mean, losses.py:45-92) and the
+        gradients torch autograd gives the reference for it, computed from the survivor list:
+        returns (loss [fp32 scalar tensor], {state-dict key: fp32 gradient in the parameter's shape}).
+        Needs every layer present, equal token counts, untied decoders, a top-k or JumpReLU /
+        ReLU activation without skip connections or feature affine terms."""
+        cfg = self.config
+        L, d, F = cfg.num_layers, cfg.d_model, cfg.num_features
+        if cfg.decoder_tying != "none" or cfg.skip_connection or getattr(cfg, "enable_feature_offset", False) \
+                or getattr(cfg, "enable_feature_scale", False):
+            raise NotImplementedError("gradients are built for untied decoders without skip / feature affine terms")
+        if sorted(inputs) != list(range(L)) or sorted(targets) != list(range(L)):
+            raise ValueError("loss_and_gradients needs inputs and targets for every layer")
+        res = self._survivors(inputs)
+        if res is None:
+            raise ValueError("inputs do not form one [layers, tokens, d_model] batch")
+        layers, T, surv = res
+        ws = self._workspace()
+        mask = (1 << L) - 1
+        rec = self.decoder_module.decode_survivors(surv, mask, ws=ws)
+        tgt = torch.stack([targets[l].to(device=self.device, dtype=self.dtype).reshape(-1, d) for l in range(L)])
+        loss_l, g, bias_grad = engine.mse_loss_grad(rec, tgt.contiguous(), ws)
+        w_packed = self.decoder_module.packed()
+        dval = engine.decode_backward_values(surv, w_packed, g, cfg.decoder_tying, mask)
+        lists = engine.feature_lists(surv, ws)
+        dw_dec = engine.decoder_weight_grad(lists, surv, g, cfg.decoder_tying)
+        _, x_slab, _, _ = self.encoder_module.prepare_slab(inputs)
+        dw_enc, db_enc = engine.encoder_weight_grad(lists, dval, x_slab.contiguous(), F)
+        grads: Dict[str, torch.Tensor] = {}
+        for l in range(L):
+            grads[f"encoder_module.encoders.{l}.weight"] = dw_enc[l]
+            grads[f"encoder_module.encoders.{l}.bias_param"] = db_enc[l]
+        slot = 0
+        for s_ in range(L):
+            for t in range(s_, L):
+                grads[f"decoder_module.decoders.{s_}->{t}.weight"] = dw_dec[slot].t()     # [d, F] view of the packed gradient
+                grads[f"decoder_module.decoders.{s_}->{t}.bias_param"] = bias_grad[t]
+                slot += 1
+        if cfg.activation_fn == "jumprelu":
+            # the threshold's own gradient (activations.py:183-220) needs the dense neighbourhood of theta
+            grads["theta_manager.log_threshold"] = None
+        return loss_l.sum(), grads
+
     # ---- encode (per-layer activations) ---------------------------------------------------
     def encode(self, x: torch.Tensor, layer_idx: int) -> torch.Tensor:
         """Activations [tokens, F] of one layer for relu / jumprelu; for the top-k family the

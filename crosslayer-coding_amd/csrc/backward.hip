@@ -1,0 +1,418 @@
+// Backward pass of the forward path for the MSE reconstruction loss (reference
+// clt/training/losses.py:45-92 through torch autograd: F.linear backward, the straight-through
+// gate of BatchTopK, clt/models/activations.py:66-96).  Everything stays sparse:
+//
+//   loss / g      g[t] = 2 (rec[t] - target[t]) / (T d), per-layer mean squared error
+//   values        d val[j] = sum over targets t >= s of  g[t][token] . W[s->t][feature]   for every
+//                 survivor j = (s, token, feature): the gradient that reaches the encoder through
+//                 the straight-through gate (zero for everything that was not selected)
+//   feature lists the survivor list regrouped by (layer, feature): which tokens fired it
+//   decoder dW    dW[s->t][feature][:] = sum over its tokens of  val * g[t][token][:]
+//   encoder dW    dW_enc[s][feature][:] = sum over its tokens of  dval * x[s][token][:],
+//                 db_enc[s][feature] = sum of dval
+//   decoder db    db[t][:] = sum over tokens of g[t][token][:]
+//
+// Row vectors are spread over a wavefront in groups of four elements: lane l holds elements
+// c * 256 + 4 l .. + 3 of chunk c (NC4 chunks cover d <= 2048; d % 4 == 0).
+#include "clt_common.h"
+
+namespace {
+
+constexpr int BW_THREADS = 256;
+
+__device__ __forceinline__ int64_t bw_decoder_slot(int tying, int64_t s, int64_t t, int64_t L) {
+  if (tying == CLT_TYING_PER_SOURCE) return s;
+  if (tying == CLT_TYING_PER_TARGET) return t;
+  return s * L - (s * (s - 1)) / 2 + (t - s);
+}
+
+template <typename T> __device__ __forceinline__ float4 load4(const T *p);
+template <> __device__ __forceinline__ float4 load4<float>(const float *p) { return *reinterpret_cast<const float4 *>(p); }
+template <> __device__ __forceinline__ float4 load4<bf16_t>(const bf16_t *p) {
+  const uint2 u = *reinterpret_cast<const uint2 *>(p);
+  return make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xFFFF0000u), __uint_as_float(u.y << 16),
+                     __uint_as_float(u.y & 0xFFFF0000u));
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+  return v;
+}
+
+// ---- loss and its gradient -------------------------------------------------------------------
+// loss_acc[l] += sum of squared differences (double); g[l][t][:] = 2 (rec - target) / (T d)
+template <typename T>
+__global__ __launch_bounds__(BW_THREADS) void k_mse_grad(const T *rec, const T *target, int64_t per_layer, float scale,
+                                                          float *g, double *loss_acc) {
+  __shared__ double red[BW_THREADS / 64];
+  const int l = blockIdx.y;
+  const T *r = rec + (int64_t)l * per_layer, *y = target + (int64_t)l * per_layer;
+  float *gl = g + (int64_t)l * per_layer;
+  double acc = 0.0;
+  for (int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4; i < per_layer; i += (int64_t)gridDim.x * blockDim.x * 4) {
+    const float4 a = load4<T>(r + i), b = load4<T>(y + i);
+    const float d0 = a.x - b.x, d1 = a.y - b.y, d2 = a.z - b.z, d3 = a.w - b.w;
+    *reinterpret_cast<float4 *>(gl + i) = make_float4(scale * d0, scale * d1, scale * d2, scale * d3);
+    acc += (double)d0 * d0 + (double)d1 * d1 + (double)d2 * d2 + (double)d3 * d3;
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    double s = 0.0;
+    for (int i = 0; i < BW_THREADS / 64; ++i) s += red[i];
+    atomicAdd(&loss_acc[l], s);
+  }
+}
+
+__global__ void k_loss_finish(const double *loss_acc, int L, double inv_count, float *loss) {
+  const int l = blockIdx.x * blockDim.x + threadIdx.x;
+  if (l < L) loss[l] = (float)(loss_acc[l] * inv_count);
+}
+
+__global__ void k_zero_u32(uint32_t *p, int64_t n) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = 0u;
+}
+
+__global__ void k_zero_f64(double *p, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0.0;
+}
+
+// ---- column sums over tokens (decoder bias gradients), deterministic two-stage --------------------
+constexpr int CS_SPLIT = 32;
+__global__ __launch_bounds__(BW_THREADS) void k_colsum_partial(const float *g, int64_t Tn, int64_t d, float *part) {
+  const int l = blockIdx.y, sp = blockIdx.z;
+  const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= d) return;
+  const int64_t per = (Tn + CS_SPLIT - 1) / CS_SPLIT, t0 = sp * per, t1 = t0 + per < Tn ? t0 + per : Tn;
+  float acc = 0.0f;
+  for (int64_t t = t0; t < t1; ++t) acc += g[((int64_t)l * Tn + t) * d + c];
+  part[((int64_t)sp * gridDim.y + l) * d + c] = acc;
+}
+__global__ __launch_bounds__(BW_THREADS) void k_colsum_finish(const float *part, int64_t d, int L, float *out) {
+  const int l = blockIdx.y;
+  const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= d) return;
+  float acc = 0.0f;
+  for (int sp = 0; sp < CS_SPLIT; ++sp) acc += part[((int64_t)sp * L + l) * d + c];
+  out[(int64_t)l * d + c] = acc;
+}
+
+// ---- gradient with respect to the survivor values ---------------------------------------------------
+// One wavefront per source row (s, token): its survivors sit one per lane; for every target the
+// row g[t][token] is held in registers and each survivor's decoder vector is fetched and dotted
+// with it (four survivors in flight).
+template <typename T, int NC4>
+__global__ __launch_bounds__(BW_THREADS) void k_decode_bwd_values(
+    const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ col, const T *__restrict__ wp,
+    const float *__restrict__ g, int64_t Tn, int64_t d, int64_t F, int64_t L, int tying, uint64_t src_mask,
+    float *__restrict__ dval) {
+  const int lane = lane_id(), wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
+  const int64_t R = L * Tn;
+  for (int64_t r = (int64_t)blockIdx.x * nwv + wv; r < R; r += (int64_t)gridDim.x * nwv) {
+    const int64_t s = r / Tn, tok = r - s * Tn;
+    const bool src_on = (src_mask >> s) & 1ull;
+    for (int32_t j0 = row_ptr[r]; j0 < row_ptr[r + 1]; j0 += 64) {
+      const int n = (row_ptr[r + 1] - j0) < 64 ? (row_ptr[r + 1] - j0) : 64;
+      const int32_t my_col = lane < n ? col[j0 + lane] : 0;
+      float acc = 0.0f;
+      if (src_on) {
+        for (int64_t t = s; t < L; ++t) {
+          float4 gv[NC4];
+#pragma unroll
+          for (int c = 0; c < NC4; ++c) {
+            const int64_t e = (int64_t)c * 256 + lane * 4;
+            gv[c] = e < d ? *reinterpret_cast<const float4 *>(g + (t * Tn + tok) * d + e) : make_float4(0.f, 0.f, 0.f, 0.f);
+          }
+          const T *wbase = wp + bw_decoder_slot(tying, s, t, L) * F * d;
+          for (int i0 = 0; i0 < n; i0 += 4) {
+            float4 w[4][NC4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+              const int idx = i0 + u < n ? i0 + u : n - 1;
+              const T *wrow = wbase + (int64_t)__builtin_amdgcn_readlane(my_col, idx) * d;
+#pragma unroll
+              for (int c = 0; c < NC4; ++c) {
+                const int64_t e = (int64_t)c * 256 + lane * 4;
+                w[u][c] = e < d ? load4<T>(wrow + e) : make_float4(0.f, 0.f, 0.f, 0.f);
+              }
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+              float p = 0.0f;
+#pragma unroll
+              for (int c = 0; c < NC4; ++c)
+                p = fmaf(w[u][c].x, gv[c].x, fmaf(w[u][c].y, gv[c].y, fmaf(w[u][c].z, gv[c].z, fmaf(w[u][c].w, gv[c].w, p))));
+              p = wave_sum(p);
+              if (i0 + u < n && lane == i0 + u) acc += p;
+            }
+          }
+        }
+      }
+      if (lane < n) dval[j0 + lane] = acc;
+    }
+  }
+}
+
+// ---- feature lists: the survivor list regrouped by (layer, feature) ----------------------------------
+__global__ __launch_bounds__(BW_THREADS) void k_csc_count(const int32_t *row_ptr, const int32_t *col, int64_t Tn, int64_t F,
+                                                           int64_t L, uint32_t *cnt) {
+  const int lane = lane_id(), wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
+  const int64_t R = L * Tn;
+  for (int64_t r = (int64_t)blockIdx.x * nwv + wv; r < R; r += (int64_t)gridDim.x * nwv) {
+    const int64_t l = r / Tn;
+    for (int32_t j = row_ptr[r] + lane; j < row_ptr[r + 1]; j += 64) atomicAdd(&cnt[l * F + col[j]], 1u);
+  }
+}
+
+// single block: ptr = exclusive scan of cnt (n entries), ptr[n] = total; cnt is reset to zero (it
+// serves as the fill cursor next)
+__global__ __launch_bounds__(1024) void k_csc_scan(uint32_t *cnt, int64_t n, int32_t *ptr) {
+  __shared__ unsigned long long ws[16];
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int64_t per = (n + 1023) / 1024, b = (int64_t)tid * per, e = b + per < n ? b + per : n;
+  unsigned long long s = 0;
+  for (int64_t i = b; i < e; ++i) s += cnt[i];
+  unsigned long long inc = s;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    unsigned long long y = __shfl_up(inc, o);
+    if (lane >= o) inc += y;
+  }
+  if (lane == 63) ws[wv] = inc;
+  __syncthreads();
+  unsigned long long base = 0, tot = 0;
+  for (int i = 0; i < 16; ++i) { if (i < wv) base += ws[i]; tot += ws[i]; }
+  unsigned long long run = base + inc - s;
+  for (int64_t i = b; i < e; ++i) { ptr[i] = (int32_t)run; run += cnt[i]; cnt[i] = 0; }
+  if (tid == 0) ptr[n] = (int32_t)tot;
+}
+
+__global__ __launch_bounds__(BW_THREADS) void k_csc_fill(const int32_t *row_ptr, const int32_t *col, int64_t Tn, int64_t F,
+                                                          int64_t L, const int32_t *ptr, uint32_t *cursor, int32_t *tok_out,
+                                                          int32_t *src_out) {
+  const int lane = lane_id(), wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
+  const int64_t R = L * Tn;
+  for (int64_t r = (int64_t)blockIdx.x * nwv + wv; r < R; r += (int64_t)gridDim.x * nwv) {
+    const int64_t l = r / Tn, tok = r - l * Tn;
+    for (int32_t j = row_ptr[r] + lane; j < row_ptr[r + 1]; j += 64) {
+      const int64_t key = l * F + col[j];
+      const uint32_t pos = atomicAdd(&cursor[key], 1u);
+      tok_out[ptr[key] + pos] = (int32_t)tok;
+      src_out[ptr[key] + pos] = j;
+    }
+  }
+}
+
+// Lists of up to 64 entries are put in token order (the fill order depends on scheduling), so
+// that the sums over a list always run in the same order; longer lists stay as filled.
+__global__ __launch_bounds__(BW_THREADS) void k_csc_order(const int32_t *ptr, int64_t nlist, int32_t *tok, int32_t *src) {
+  const int lane = lane_id(), wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
+  for (int64_t q = (int64_t)blockIdx.x * nwv + wv; q < nlist; q += (int64_t)gridDim.x * nwv) {
+    const int32_t b = ptr[q], n = ptr[q + 1] - b;
+    if (n < 2 || n > 64) continue;
+    const int32_t mt = lane < n ? tok[b + lane] : 0x7FFFFFFF, ms = lane < n ? src[b + lane] : 0;
+    int rank = 0;
+    for (int i = 0; i < n; ++i) rank += __builtin_amdgcn_readlane(mt, i) < mt ? 1 : 0;   // tokens of one list are distinct
+    if (lane < n) { tok[b + rank] = mt; src[b + rank] = ms; }
+  }
+}
+
+// ---- weight gradients: one wavefront per output row ---------------------------------------------------
+// out_row[:] = sum over the list of (layer, feature) of coef[entry] * src[token][:]
+//   DECODER: wavefront (s, f, t >= s): coef = survivor value, src = g[t], out = dW[slot(s,t)][f]
+//   encoder: wavefront (s, f):         coef = dval,           src = x[s], out = dW_enc[s][f], rowsum = db_enc[s][f]
+template <typename SrcT, typename CoefT, int NC4, bool DECODER>
+__global__ __launch_bounds__(BW_THREADS) void k_feature_outer(
+    const int32_t *__restrict__ ptr, const int32_t *__restrict__ ltok, const int32_t *__restrict__ lsrc,
+    const CoefT *__restrict__ coef, const SrcT *__restrict__ src, float *__restrict__ out, float *__restrict__ rowsum,
+    int64_t Tn, int64_t d, int64_t F, int64_t L) {
+  const int lane = lane_id(), wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
+  const int64_t per_layer_rows = DECODER ? F * L : F;   // upper bound used to enumerate (f, t) pairs of a layer
+  const int64_t total = L * per_layer_rows;
+  for (int64_t w = (int64_t)blockIdx.x * nwv + wv; w < total; w += (int64_t)gridDim.x * nwv) {
+    const int64_t s = w / per_layer_rows, rem = w - s * per_layer_rows;
+    int64_t f, t;
+    if (DECODER) { t = rem / F; f = rem - t * F; if (t < s) continue; }
+    else { f = rem; t = s; }
+    const int64_t q = s * F + f;
+    const int32_t b = ptr[q], e = ptr[q + 1];
+    const SrcT *sbase = src + (DECODER ? t : s) * Tn * d;
+    float4 acc[NC4];
+#pragma unroll
+    for (int c = 0; c < NC4; ++c) acc[c] = make_float4(0.f, 0.f, 0.f, 0.f);
+    float csum = 0.0f;
+    for (int32_t i0 = b; i0 < e; i0 += 64) {
+      const int n = (e - i0) < 64 ? (e - i0) : 64;
+      int32_t mt = 0; float mc = 0.0f;
+      if (lane < n) { mt = ltok[i0 + lane]; mc = Elem<CoefT>::to_f32(coef[lsrc[i0 + lane]]); }
+      for (int i = 0; i < n; i += 2) {
+        float4 v[2][NC4]; float cf[2];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const int idx = i + u < n ? i + u : n - 1;
+          const SrcT *row = sbase + (int64_t)__builtin_amdgcn_readlane(mt, idx) * d;
+          cf[u] = i + u < n ? __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(mc), idx)) : 0.0f;
+#pragma unroll
+          for (int c = 0; c < NC4; ++c) {
+            const int64_t el = (int64_t)c * 256 + lane * 4;
+            v[u][c] = el < d ? load4<SrcT>(row + el) : make_float4(0.f, 0.f, 0.f, 0.f);
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          csum += cf[u];
+#pragma unroll
+          for (int c = 0; c < NC4; ++c) {
+            acc[c].x = fmaf(cf[u], v[u][c].x, acc[c].x); acc[c].y = fmaf(cf[u], v[u][c].y, acc[c].y);
+            acc[c].z = fmaf(cf[u], v[u][c].z, acc[c].z); acc[c].w = fmaf(cf[u], v[u][c].w, acc[c].w);
+          }
+        }
+      }
+    }
+    float *orow = out + (DECODER ? (bw_decoder_slot(CLT_TYING_NONE, s, t, L) * F + f) : q) * d;
+#pragma unroll
+    for (int c = 0; c < NC4; ++c) {
+      const int64_t el = (int64_t)c * 256 + lane * 4;
+      if (el < d) *reinterpret_cast<float4 *>(orow + el) = acc[c];
+    }
+    if (!DECODER && rowsum && lane == 0) rowsum[q] = csum;
+  }
+}
+
+static bool bw_shape_ok(int64_t d) { return d > 0 && d % 4 == 0 && d <= 2048; }
+
+}  // namespace
+
+extern "C" size_t clt_mse_workspace_bytes(int64_t T, int64_t d, int64_t L) {
+  (void)T;
+  if (d <= 0 || L <= 0) return 256;
+  return (((size_t)L * 8 + 255) & ~(size_t)255) + (size_t)CS_SPLIT * (size_t)L * (size_t)d * 4;
+}
+
+extern "C" int clt_mse_loss_grad(const void *rec, const void *target, int64_t T, int64_t d, int64_t L, int dtype,
+                                 float *loss_per_layer, float *g, float *bias_grad, void *workspace,
+                                 size_t workspace_bytes, void *stream) {
+  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (T <= 0 || d <= 0 || L <= 0 || L > 65535 || !rec || !target || !loss_per_layer || !g || !workspace) return CLT_ERR_ARG;
+  if ((T * d) % 4 != 0) return CLT_ERR_ARG;
+  if (workspace_bytes < clt_mse_workspace_bytes(T, d, L)) return CLT_ERR_WORKSPACE;
+  if ((((uintptr_t)workspace) & 255u) != 0) return CLT_ERR_ALIGN;
+  hipStream_t s = (hipStream_t)stream;
+  double *acc = (double *)workspace;
+  float *part = (float *)((char *)workspace + (((size_t)L * 8 + 255) & ~(size_t)255));
+  k_zero_f64<<<(unsigned)clt_ceil_div(L, 256), 256, 0, s>>>(acc, (int)L);
+  const int64_t per_layer = T * d;
+  const float scale = (float)(2.0 / (double)per_layer);
+  dim3 grid(512, (unsigned)L);
+  if (dtype == CLT_BF16) k_mse_grad<bf16_t><<<grid, BW_THREADS, 0, s>>>((const bf16_t *)rec, (const bf16_t *)target, per_layer, scale, g, acc);
+  else k_mse_grad<float><<<grid, BW_THREADS, 0, s>>>((const float *)rec, (const float *)target, per_layer, scale, g, acc);
+  k_loss_finish<<<(unsigned)clt_ceil_div(L, 256), 256, 0, s>>>(acc, (int)L, 1.0 / (double)per_layer, loss_per_layer);
+  if (bias_grad) {
+    k_colsum_partial<<<dim3((unsigned)clt_ceil_div(d, BW_THREADS), (unsigned)L, CS_SPLIT), BW_THREADS, 0, s>>>(g, T, d, part);
+    k_colsum_finish<<<dim3((unsigned)clt_ceil_div(d, BW_THREADS), (unsigned)L), BW_THREADS, 0, s>>>(part, d, (int)L, bias_grad);
+  }
+  return clt_check_launch();
+}
+
+extern "C" int clt_decode_backward_values(const int32_t *row_ptr, const int32_t *col, const void *w_packed, const float *g,
+                                          int64_t T, int64_t d, int64_t F, int64_t L, int tying, uint64_t src_mask,
+                                          int dtype, float *dval, void *stream) {
+  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (T <= 0 || F <= 0 || L <= 0 || L > 64 || tying < 0 || tying > 2) return CLT_ERR_ARG;
+  if (!row_ptr || !w_packed || !g || !dval) return CLT_ERR_ARG;
+  if (!bw_shape_ok(d)) return CLT_ERR_RANGE;
+  hipStream_t s = (hipStream_t)stream;
+  const int nc4 = (int)clt_ceil_div(d, 256);
+  const unsigned nb = 256 * 16;
+#define CLT_BWV(TT, N) k_decode_bwd_values<TT, N><<<nb, BW_THREADS, 0, s>>>(row_ptr, col, (const TT *)w_packed, g, T, d, F, L, tying, src_mask, dval)
+#define CLT_BWV_N(TT)                                                                       \
+  do {                                                                                      \
+    switch (nc4) {                                                                          \
+      case 1: CLT_BWV(TT, 1); break; case 2: CLT_BWV(TT, 2); break; case 3: CLT_BWV(TT, 3); break; \
+      case 4: CLT_BWV(TT, 4); break; case 5: CLT_BWV(TT, 5); break; case 6: CLT_BWV(TT, 6); break; \
+      case 7: CLT_BWV(TT, 7); break; default: CLT_BWV(TT, 8); break;                        \
+    }                                                                                       \
+  } while (0)
+  if (dtype == CLT_BF16) CLT_BWV_N(bf16_t); else CLT_BWV_N(float);
+#undef CLT_BWV_N
+#undef CLT_BWV
+  return clt_check_launch();
+}
+
+extern "C" size_t clt_feature_lists_workspace_bytes(int64_t F, int64_t L) {
+  if (F <= 0 || L <= 0) return 256;
+  return (size_t)L * (size_t)F * 4;
+}
+
+extern "C" int clt_feature_lists(const int32_t *row_ptr, const int32_t *col, int64_t T, int64_t F, int64_t L,
+                                 int32_t *list_ptr, int32_t *list_tok, int32_t *list_src, void *workspace,
+                                 size_t workspace_bytes, void *stream) {
+  if (T <= 0 || F <= 0 || L <= 0 || L > 65535 || !row_ptr || !list_ptr || !workspace) return CLT_ERR_ARG;
+  if ((double)L * (double)F >= 2147483647.0) return CLT_ERR_RANGE;
+  if (workspace_bytes < clt_feature_lists_workspace_bytes(F, L)) return CLT_ERR_WORKSPACE;
+  hipStream_t s = (hipStream_t)stream;
+  uint32_t *cnt = (uint32_t *)workspace;
+  const int64_t n = L * F;
+  const unsigned nb = 256 * 8;
+  k_zero_u32<<<nb, BW_THREADS, 0, s>>>(cnt, n);
+  k_csc_count<<<nb, BW_THREADS, 0, s>>>(row_ptr, col, T, F, L, cnt);
+  k_csc_scan<<<1, 1024, 0, s>>>(cnt, n, list_ptr);
+  if (list_tok && list_src) {
+    k_csc_fill<<<nb, BW_THREADS, 0, s>>>(row_ptr, col, T, F, L, list_ptr, cnt, list_tok, list_src);
+    k_csc_order<<<nb, BW_THREADS, 0, s>>>(list_ptr, n, list_tok, list_src);
+  }
+  return clt_check_launch();
+}
+
+extern "C" int clt_decoder_weight_grad(const int32_t *list_ptr, const int32_t *list_tok, const int32_t *list_src,
+                                       const void *val, const float *g, float *dw_packed, int64_t T, int64_t d, int64_t F,
+                                       int64_t L, int tying, int dtype, void *stream) {
+  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (tying != CLT_TYING_NONE) return CLT_ERR_ARG;   // tied decoders sum over several (source, target) pairs: not built
+  if (T <= 0 || F <= 0 || L <= 0 || L > 64 || !list_ptr || !list_tok || !list_src || !val || !g || !dw_packed) return CLT_ERR_ARG;
+  if (!bw_shape_ok(d)) return CLT_ERR_RANGE;
+  hipStream_t s = (hipStream_t)stream;
+  const int nc4 = (int)clt_ceil_div(d, 256);
+  const unsigned nb = 256 * 32;
+#define CLT_DW(CT, N) k_feature_outer<float, CT, N, true><<<nb, BW_THREADS, 0, s>>>(list_ptr, list_tok, list_src, (const CT *)val, g, dw_packed, nullptr, T, d, F, L)
+#define CLT_DW_N(CT)                                                                       \
+  do {                                                                                     \
+    switch (nc4) {                                                                         \
+      case 1: CLT_DW(CT, 1); break; case 2: CLT_DW(CT, 2); break; case 3: CLT_DW(CT, 3); break; \
+      case 4: CLT_DW(CT, 4); break; case 5: CLT_DW(CT, 5); break; case 6: CLT_DW(CT, 6); break; \
+      case 7: CLT_DW(CT, 7); break; default: CLT_DW(CT, 8); break;                         \
+    }                                                                                      \
+  } while (0)
+  if (dtype == CLT_BF16) CLT_DW_N(bf16_t); else CLT_DW_N(float);
+#undef CLT_DW_N
+#undef CLT_DW
+  return clt_check_launch();
+}
+
+extern "C" int clt_encoder_weight_grad(const int32_t *list_ptr, const int32_t *list_tok, const int32_t *list_src,
+                                       const float *dval, const void *x, float *dw_enc, float *db_enc, int64_t T, int64_t d,
+                                       int64_t F, int64_t L, int dtype, void *stream) {
+  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (T <= 0 || F <= 0 || L <= 0 || L > 65535 || !list_ptr || !list_tok || !list_src || !dval || !x || !dw_enc) return CLT_ERR_ARG;
+  if (!bw_shape_ok(d)) return CLT_ERR_RANGE;
+  hipStream_t s = (hipStream_t)stream;
+  const int nc4 = (int)clt_ceil_div(d, 256);
+  const unsigned nb = 256 * 32;
+#define CLT_EW(ST, N) k_feature_outer<ST, float, N, false><<<nb, BW_THREADS, 0, s>>>(list_ptr, list_tok, list_src, dval, (const ST *)x, dw_enc, db_enc, T, d, F, L)
+#define CLT_EW_N(ST)                                                                       \
+  do {                                                                                     \
+    switch (nc4) {                                                                         \
+      case 1: CLT_EW(ST, 1); break; case 2: CLT_EW(ST, 2); break; case 3: CLT_EW(ST, 3); break; \
+      case 4: CLT_EW(ST, 4); break; case 5: CLT_EW(ST, 5); break; case 6: CLT_EW(ST, 6); break; \
+      case 7: CLT_EW(ST, 7); break; default: CLT_EW(ST, 8); break;                         \
+    }                                                                                      \
+  } while (0)
+  if (dtype == CLT_BF16) CLT_EW_N(bf16_t); else CLT_EW_N(float);
+#undef CLT_EW_N
+#undef CLT_EW
+  return clt_check_launch();
+}

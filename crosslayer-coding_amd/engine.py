@@ -302,6 +302,85 @@ def encode_threshold(x: torch.Tensor, w: torch.Tensor, b: Optional[torch.Tensor]
     return SurvivorList(row_ptr, col[:total], val[:total], T, F, L, x.dtype)
 
 
+# ---- backward pass (MSE reconstruction loss) ---------------------------------------------------------
+def mse_loss_grad(rec: torch.Tensor, target: torch.Tensor, ws: Optional[Workspace] = None):
+    """(loss per layer [L] fp32, g [L, T, d] fp32 = d loss / d rec, bias_grad [L, d] fp32) for
+    loss = sum over layers of mean((rec - target)^2) (losses.py:45-92)."""
+    nat.require_device(rec, "mse_loss_grad")
+    L, T, d = rec.shape
+    assert target.shape == rec.shape and target.dtype == rec.dtype and rec.is_contiguous() and target.is_contiguous()
+    dev = rec.device
+    loss = torch.empty(L, dtype=torch.float32, device=dev)
+    g = torch.empty((L, T, d), dtype=torch.float32, device=dev)
+    bias_grad = torch.empty((L, d), dtype=torch.float32, device=dev)
+    lib = nat.load()
+    wbuf = (ws or Workspace(dev)).get("mse", lib.clt_mse_workspace_bytes(T, d, L))
+    code = lib.clt_mse_loss_grad(nat.ptr(rec), nat.ptr(target), T, d, L, nat.dtype_code(rec.dtype), nat.ptr(loss),
+                                 nat.ptr(g), nat.ptr(bias_grad), nat.ptr(wbuf), wbuf.numel(), _stream(rec))
+    nat.check(code, "clt_mse_loss_grad")
+    return loss, g, bias_grad
+
+
+def decode_backward_values(surv: SurvivorList, w_packed: torch.Tensor, g: torch.Tensor, tying: str,
+                           src_mask: Optional[int] = None) -> torch.Tensor:
+    """d loss / d (kept activation) for every survivor, fp32 [nnz] (the straight-through gate hands
+    it to the pre-activation unchanged, activations.py:66-96)."""
+    L, T, F = surv.L, surv.T, surv.F
+    d = w_packed.shape[2]
+    assert g.shape == (L, T, d) and g.dtype == torch.float32 and g.is_contiguous()
+    assert w_packed.dtype == surv.dtype and w_packed.is_contiguous()
+    if src_mask is None:
+        src_mask = (1 << L) - 1
+    dval = torch.empty(max(surv.nnz, 1), dtype=torch.float32, device=g.device)
+    code = nat.load().clt_decode_backward_values(nat.ptr(surv.row_ptr), nat.ptr(surv.col), nat.ptr(w_packed), nat.ptr(g),
+                                                 T, d, F, L, nat.TYING[tying], src_mask & ((1 << 64) - 1),
+                                                 nat.dtype_code(surv.dtype), nat.ptr(dval), _stream(g))
+    nat.check(code, "clt_decode_backward_values")
+    return dval[:surv.nnz]
+
+
+def feature_lists(surv: SurvivorList, ws: Optional[Workspace] = None):
+    """The survivor list regrouped by (layer, feature): (ptr [L*F+1], token [nnz], source index [nnz])."""
+    L, T, F = surv.L, surv.T, surv.F
+    dev = surv.row_ptr.device
+    ptr = torch.empty(L * F + 1, dtype=torch.int32, device=dev)
+    tok = torch.empty(max(surv.nnz, 1), dtype=torch.int32, device=dev)
+    src = torch.empty(max(surv.nnz, 1), dtype=torch.int32, device=dev)
+    lib = nat.load()
+    wbuf = (ws or Workspace(dev)).get("feature_lists", lib.clt_feature_lists_workspace_bytes(F, L))
+    code = lib.clt_feature_lists(nat.ptr(surv.row_ptr), nat.ptr(surv.col), T, F, L, nat.ptr(ptr), nat.ptr(tok),
+                                 nat.ptr(src), nat.ptr(wbuf), wbuf.numel(), nat.current_stream(dev))
+    nat.check(code, "clt_feature_lists")
+    return ptr, tok, src
+
+
+def decoder_weight_grad(lists, surv: SurvivorList, g: torch.Tensor, tying: str) -> torch.Tensor:
+    """fp32 [n_dec, F, d] gradient of the packed (feature-major) untied decoder weights."""
+    ptr, tok, src = lists
+    L, T, F = surv.L, surv.T, surv.F
+    d = g.shape[2]
+    n_dec = L * (L + 1) // 2
+    out = torch.empty((n_dec, F, d), dtype=torch.float32, device=g.device)
+    code = nat.load().clt_decoder_weight_grad(nat.ptr(ptr), nat.ptr(tok), nat.ptr(src), nat.ptr(surv.val), nat.ptr(g),
+                                              nat.ptr(out), T, d, F, L, nat.TYING[tying], nat.dtype_code(surv.dtype),
+                                              _stream(g))
+    nat.check(code, "clt_decoder_weight_grad")
+    return out
+
+
+def encoder_weight_grad(lists, dval: torch.Tensor, x: torch.Tensor, F: int):
+    """(fp32 [L, F, d], fp32 [L, F]): gradients of the stacked encoder weights and biases."""
+    ptr, tok, src = lists
+    L, T, d = x.shape
+    assert x.is_contiguous() and dval.dtype == torch.float32
+    dw = torch.empty((L, F, d), dtype=torch.float32, device=x.device)
+    db = torch.empty((L, F), dtype=torch.float32, device=x.device)
+    code = nat.load().clt_encoder_weight_grad(nat.ptr(ptr), nat.ptr(tok), nat.ptr(src), nat.ptr(dval), nat.ptr(x),
+                                              nat.ptr(dw), nat.ptr(db), T, d, F, L, nat.dtype_code(x.dtype), _stream(x))
+    nat.check(code, "clt_encoder_weight_grad")
+    return dw, db
+
+
 def pack_decoder(w_ref: torch.Tensor, out: torch.Tensor) -> None:
     """[d, F] checkpoint layout -> [F, d] feature-major (one matrix)."""
     nat.require_device(w_ref, "pack_decoder")

@@ -31,6 +31,9 @@ How each function is pinned (see ``tests/test_oracle_*.py``):
   properties the reference's own test asserts (tests/unit/models/test_theta.py:110-175:
   thresholds finite and positive, higher for the features that were selected); the
   reference holds no golden numbers for them: PARITY UNPINNED beyond that.
+* ``mse_loss_and_gradients``  - torch autograd itself computes the gradients; a central
+  finite-difference check in float64 on a tiny model pins the loss / gradient pairing, and the
+  reference's backward tables (test_activations.py:114-152: grad * mask) pin the gate.
 * ``forward``  - composition of the above; the reference has no golden tensors
   for a full forward: PARITY UNPINNED beyond shape/keys and the pins of its parts.
 
@@ -490,6 +493,59 @@ def theta_convert(ssum: torch.Tensor, scnt: torch.Tensor, mus: torch.Tensor, sig
         theta_raw[l] = scalar * sigmas[l].clamp_min(1e-6) + mus[l]
     theta_raw.clamp_min_(1e-7)
     return torch.log(theta_raw)
+
+
+# ---------------------------------------------------------------------------
+# MSE reconstruction loss and its gradients (torch autograd, as the reference trains)
+# ---------------------------------------------------------------------------
+
+def mse_loss_and_gradients(inputs: Dict[int, torch.Tensor], targets: Dict[int, torch.Tensor], *,
+                           enc_w: List[torch.Tensor], enc_b: List[torch.Tensor],
+                           dec_w: Dict[str, torch.Tensor], dec_b: Dict[str, torch.Tensor],
+                           activation_fn: str, num_layers: int, k: Optional[float] = None,
+                           theta: Optional[torch.Tensor] = None,
+                           masks: Optional[Dict[int, torch.Tensor]] = None):
+    """loss = sum over layers of nn.MSELoss()(prediction, target) (losses.py:45-92, no
+    de-normalisation statistics) through the reference's forward with untied decoders, and
+    d loss / d parameter from torch autograd (trainer.py:751): F.linear backward for encoder
+    and decoders, the straight-through gate of BatchTopK (activations.py:66-96: grad * mask)
+    or the pass-through part of JumpReLU's backward (activations.py:183-220: grad * 1[x >= theta];
+    the threshold's own gradient is not part of this function).  Per-layer selection, fp32.
+    ``masks`` (bool [T, F] per layer) replaces the gate computed here, for comparisons in which
+    the other side selected on differently rounded pre-activations.
+    Returns (loss, {state-dict key: gradient})."""
+    L = num_layers
+    params: Dict[str, torch.Tensor] = {}
+    for l in range(L):
+        params[f"encoder_module.encoders.{l}.weight"] = enc_w[l].detach().float().clone().requires_grad_(True)
+        params[f"encoder_module.encoders.{l}.bias_param"] = enc_b[l].detach().float().clone().requires_grad_(True)
+    for name in dec_w:
+        params[f"decoder_module.decoders.{name}.weight"] = dec_w[name].detach().float().clone().requires_grad_(True)
+        params[f"decoder_module.decoders.{name}.bias_param"] = dec_b[name].detach().float().clone().requires_grad_(True)
+    acts = {}
+    for l in range(L):
+        pre = F.linear(inputs[l].float(), params[f"encoder_module.encoders.{l}.weight"],
+                       params[f"encoder_module.encoders.{l}.bias_param"])
+        if masks is not None:
+            mask = masks[l]
+        elif activation_fn == "batchtopk":
+            mask = batchtopk_mask(pre.detach(), int(k), pre.detach())
+        elif activation_fn == "jumprelu":
+            mask = pre.detach() >= theta[l].float()
+        elif activation_fn == "relu":
+            mask = pre.detach() > 0
+        else:
+            raise ValueError(activation_fn)
+        acts[l] = pre * mask.to(pre.dtype)
+    loss = torch.zeros((), dtype=torch.float32)
+    for t in range(L):
+        rec = torch.zeros_like(targets[t], dtype=torch.float32)
+        for s_ in range(t + 1):
+            rec = rec + F.linear(acts[s_], params[f"decoder_module.decoders.{s_}->{t}.weight"],
+                                 params[f"decoder_module.decoders.{s_}->{t}.bias_param"])
+        loss = loss + F.mse_loss(rec, targets[t].float())
+    loss.backward()
+    return loss.detach(), {name: p.grad for name, p in params.items()}
 
 
 # ---------------------------------------------------------------------------
