@@ -250,6 +250,40 @@ def run_theta(args):
     }
 
 
+def run_backward(args):
+    """Forward, MSE reconstruction loss and the gradients of every encoder / decoder parameter
+    (CrossLayerTranscoder.loss_and_gradients); one step = one batch.  No optimizer step."""
+    import crosslayer_coding_amd as cca
+    from crosslayer_coding_amd import synth
+
+    wl = synth.WORKLOADS[args.workload]
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    cca._native.load(build_if_missing=False)
+    model, inputs, _ = synth.build_model(wl, dev)
+    model.eval()
+    g = torch.Generator(device=dev).manual_seed(99)
+    targets = {l: torch.randn(wl.tokens, wl.d_model, generator=g, device=dev).to(model.dtype) for l in range(wl.num_layers)}
+    for _ in range(args.warmup):
+        loss, grads = model.loss_and_gradients(inputs, targets)
+    del grads
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        loss, grads = model.loss_and_gradients(inputs, targets)
+        del grads
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return {
+        "metric": "CLT forward + MSE loss + gradients tokens/sec (no optimizer step)",
+        "value": wl.tokens * args.steps / wall, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": wall / args.steps * 1e3, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16" if wl.dtype == "bfloat16" else "f32", "data": "synthetic",
+        "config": {"workload": f"{wl.name}: forward + backward, L={wl.num_layers} d_model={wl.d_model} "
+                               f"F={wl.num_features} T={wl.tokens} {wl.activation_fn} k={wl.k}", "loss": float(loss)},
+    }
+
+
 def cpu_baseline(wl, model, slab, tokens):
     """The reference's dense forward (F.linear encoder, torch.topk mask, one dense F.linear
     per decoder, sum in the model dtype) from ``oracle/``, on the first ``tokens`` tokens of
@@ -298,6 +332,8 @@ def main():
     ap.add_argument("--theta-estimation", action="store_true",
                     help="time batches of the post-hoc theta estimation (encoder, column statistics, global "
                          "selection, per-feature minimum) instead of the forward")
+    ap.add_argument("--backward", action="store_true",
+                    help="time forward + MSE loss + all gradients (loss_and_gradients) instead of the forward")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one 256 MiB elementwise copy (counter yardstick for profiled runs)")
     args = ap.parse_args()
@@ -308,7 +344,7 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a ROCm GPU", file=sys.stderr)
         sys.exit(2)
-    print(json.dumps(run_theta(args) if args.theta_estimation else run_gpu(args)))
+    print(json.dumps(run_theta(args) if args.theta_estimation else run_backward(args) if args.backward else run_gpu(args)))
 
 
 if __name__ == "__main__":

@@ -54,8 +54,9 @@ _SIGNATURES = {
     "clt_decode_sparse": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _i64, _i64, _u64, _int, _int, _vp, _sz, _vp]),
     "clt_densify": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp]),
     "clt_mse_workspace_bytes": (_sz, [_i64, _i64, _i64]),
-    "clt_mse_loss_grad": (_int, [_vp, _vp, _i64, _i64, _i64, _int, _vp, _vp, _vp, _vp, _sz, _vp]),
-    "clt_decode_backward_values": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _u64, _int, _vp, _vp]),
+    "clt_mse_loss_grad": (_int, [_vp, _vp, _i64, _i64, _i64, _int, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "clt_decode_backward_workspace_bytes": (_sz, [_i64, _i64, _i64]),
+    "clt_decode_backward_values": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _u64, _i64, _int, _vp, _vp, _sz, _vp]),
     "clt_feature_lists_workspace_bytes": (_sz, [_i64, _i64]),
     "clt_feature_lists": (_int, [_vp, _vp, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _sz, _vp]),
     "clt_decoder_weight_grad": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp]),

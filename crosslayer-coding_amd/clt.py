@@ -181,11 +181,11 @@ class CrossLayerTranscoder(BaseTranscoder):
         mask = (1 << L) - 1
         rec = self.decoder_module.decode_survivors(surv, mask, ws=ws)
         tgt = torch.stack([targets[l].to(device=self.device, dtype=self.dtype).reshape(-1, d) for l in range(L)])
-        loss_l, g, bias_grad = engine.mse_loss_grad(rec, tgt.contiguous(), ws)
+        loss_l, g, g_model, bias_grad = engine.mse_loss_grad(rec, tgt.contiguous(), ws)
         w_packed = self.decoder_module.packed()
-        dval = engine.decode_backward_values(surv, w_packed, g, cfg.decoder_tying, mask)
+        dval = engine.decode_backward_values(surv, w_packed, g, cfg.decoder_tying, mask, ws)
         lists = engine.feature_lists(surv, ws)
-        dw_dec = engine.decoder_weight_grad(lists, surv, g, cfg.decoder_tying)
+        dw_dec = engine.decoder_weight_grad(lists, surv, g_model, cfg.decoder_tying)
         _, x_slab, _, _ = self.encoder_module.prepare_slab(inputs)
         dw_enc, db_enc = engine.encoder_weight_grad(lists, dval, x_slab.contiguous(), F)
         grads: Dict[str, torch.Tensor] = {}

@@ -34,6 +34,23 @@ template <> __device__ __forceinline__ float4 load4<bf16_t>(const bf16_t *p) {
                      __uint_as_float(u.y & 0xFFFF0000u));
 }
 
+// 16 raw bytes of a row (EV = 8 bf16 or 4 fp32 elements) and their float values
+template <typename T> struct Piece;
+template <> struct Piece<float> {
+  static constexpr int EV = 4;
+  __device__ static __forceinline__ void unpack(const uint4 &w, float (&x)[4]) {
+    x[0] = __uint_as_float(w.x); x[1] = __uint_as_float(w.y); x[2] = __uint_as_float(w.z); x[3] = __uint_as_float(w.w);
+  }
+};
+template <> struct Piece<bf16_t> {
+  static constexpr int EV = 8;
+  __device__ static __forceinline__ void unpack(const uint4 &w, float (&x)[8]) {
+    const uint32_t u[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) { x[2 * j] = __uint_as_float(u[j] << 16); x[2 * j + 1] = __uint_as_float(u[j] & 0xFFFF0000u); }
+  }
+};
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
@@ -44,16 +61,19 @@ __device__ __forceinline__ float wave_sum(float v) {
 // loss_acc[l] += sum of squared differences (double); g[l][t][:] = 2 (rec - target) / (T d)
 template <typename T>
 __global__ __launch_bounds__(BW_THREADS) void k_mse_grad(const T *rec, const T *target, int64_t per_layer, float scale,
-                                                          float *g, double *loss_acc) {
+                                                          float *g, T *g_model, double *loss_acc) {
   __shared__ double red[BW_THREADS / 64];
   const int l = blockIdx.y;
   const T *r = rec + (int64_t)l * per_layer, *y = target + (int64_t)l * per_layer;
   float *gl = g + (int64_t)l * per_layer;
+  T *gm = g_model ? g_model + (int64_t)l * per_layer : nullptr;
   double acc = 0.0;
   for (int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4; i < per_layer; i += (int64_t)gridDim.x * blockDim.x * 4) {
     const float4 a = load4<T>(r + i), b = load4<T>(y + i);
     const float d0 = a.x - b.x, d1 = a.y - b.y, d2 = a.z - b.z, d3 = a.w - b.w;
     *reinterpret_cast<float4 *>(gl + i) = make_float4(scale * d0, scale * d1, scale * d2, scale * d3);
+    if (gm) { gm[i] = Elem<T>::from_f32(scale * d0); gm[i + 1] = Elem<T>::from_f32(scale * d1);
+              gm[i + 2] = Elem<T>::from_f32(scale * d2); gm[i + 3] = Elem<T>::from_f32(scale * d3); }
     acc += (double)d0 * d0 + (double)d1 * d1 + (double)d2 * d2 + (double)d3 * d3;
   }
 #pragma unroll
@@ -102,57 +122,145 @@ __global__ __launch_bounds__(BW_THREADS) void k_colsum_finish(const float *part,
 }
 
 // ---- gradient with respect to the survivor values ---------------------------------------------------
-// One wavefront per source row (s, token): its survivors sit one per lane; for every target the
-// row g[t][token] is held in registers and each survivor's decoder vector is fetched and dotted
-// with it (four survivors in flight).
-template <typename T, int NC4>
-__global__ __launch_bounds__(BW_THREADS) void k_decode_bwd_values(
-    const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ col, const T *__restrict__ wp,
-    const float *__restrict__ g, int64_t Tn, int64_t d, int64_t F, int64_t L, int tying, uint64_t src_mask,
-    float *__restrict__ dval) {
+// sptr[r][j] = first survivor of row r whose feature index is >= j * F / ns  (j = 0..ns)
+__global__ void k_bw_slice_ptr(const int32_t *row_ptr, const int32_t *col, int64_t R, int64_t F, int ns, int32_t *sptr) {
+  const int64_t total = R * (ns + 1);
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t r = i / (ns + 1);
+    const int j = (int)(i - r * (ns + 1));
+    const int32_t bound = (int32_t)(((int64_t)j * F) / ns);
+    int32_t lo = row_ptr[r], hi = row_ptr[r + 1];
+    while (lo < hi) {
+      const int32_t mid = lo + ((hi - lo) >> 1);
+      if (col[mid] < bound) lo = mid + 1; else hi = mid;
+    }
+    sptr[i] = lo;
+  }
+}
+
+constexpr int BWV_XCDS = 8;    // feature slices = XCDs; workgroup b runs on XCD b % 8
+constexpr int BWV_NTOK = 4;    // tokens per wavefront
+constexpr int BWV_NU = 8;      // survivors whose decoder vectors are in flight together
+
+// Sum of p[u] over the wavefront for BWV_NU values at once: three exchange steps that halve the
+// values a lane keeps, then three steps on the one value left.  Afterwards lane l holds the
+// total of value ((l >> 5) & 1) * 4 + ((l >> 4) & 1) * 2 + ((l >> 3) & 1).
+__device__ __forceinline__ float wave_sum8(const float (&p)[BWV_NU], int lane) {
+  float q4[4], q2[2], q1;
+  const bool hi32 = lane & 32, hi16 = lane & 16, hi8 = lane & 8;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float keep = hi32 ? p[4 + i] : p[i], give = hi32 ? p[i] : p[4 + i];
+    q4[i] = keep + __shfl_xor(give, 32);
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const float keep = hi16 ? q4[2 + i] : q4[i], give = hi16 ? q4[i] : q4[2 + i];
+    q2[i] = keep + __shfl_xor(give, 16);
+  }
+  {
+    const float keep = hi8 ? q2[1] : q2[0], give = hi8 ? q2[0] : q2[1];
+    q1 = keep + __shfl_xor(give, 8);
+  }
+  q1 += __shfl_xor(q1, 4);
+  q1 += __shfl_xor(q1, 2);
+  q1 += __shfl_xor(q1, 1);
+  return q1;
+}
+
+// One wavefront per (source s, target t >= s, feature slice, BWV_NTOK tokens): like the forward
+// gather, block b works on slice b % 8 and blocks are ordered (s, t)-pair-major, so an XCD gathers
+// from one slice of one decoder matrix at a time.  part[t][j] = g[t][token] . W[s->t][feature of j].
+// A row is read in 16-byte pieces (lane l: elements c * 64 EV + l EV ..., NCH pieces); the raw pieces
+// of up to BWV_NU rows are in flight together, and BWV_NU dot products are reduced across the
+// wavefront at once.
+template <typename T, int NCH>
+__global__ __launch_bounds__(BW_THREADS) void k_bwd_values_sliced(
+    const int32_t *__restrict__ sptr, const int32_t *__restrict__ col, const T *__restrict__ wp,
+    const float *__restrict__ g, int64_t Tn, int64_t d, int64_t F, int64_t L, int tying, int64_t nnz,
+    float *__restrict__ part) {
+  constexpr int EV = Piece<T>::EV;
+  const int lane = lane_id(), wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
+  const int slice = (int)(blockIdx.x % BWV_XCDS);
+  const int64_t bid = (int64_t)blockIdx.x / BWV_XCDS;
+  const int64_t groups = (Tn + (int64_t)nwv * BWV_NTOK - 1) / ((int64_t)nwv * BWV_NTOK);
+  const int64_t pair = bid / groups;
+  const int64_t tok0 = ((bid - pair * groups) * nwv + wv) * BWV_NTOK;
+  // pair -> (s, t): pairs are numbered like the untied decoder slots
+  int64_t s = 0, rem = pair;
+  while (rem >= L - s) { rem -= L - s; ++s; }
+  const int64_t t = s + rem;
+  const T *wbase = wp + bw_decoder_slot(tying, s, t, L) * F * d;
+  float *pt = part + t * nnz;
+  bool on[NCH];
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) on[c] = (int64_t)c * 64 * EV + lane * EV < d;
+  for (int i = 0; i < BWV_NTOK; ++i) {
+    const int64_t tok = tok0 + i;
+    if (tok >= Tn) break;
+    const int64_t r = s * Tn + tok;
+    const int32_t b = sptr[r * (BWV_XCDS + 1) + slice], e = sptr[r * (BWV_XCDS + 1) + slice + 1];
+    if (b == e) continue;
+    float gv[NCH][EV];
+#pragma unroll
+    for (int c = 0; c < NCH; ++c)
+#pragma unroll
+      for (int q = 0; q < EV; q += 4) {
+        const float4 v = on[c] ? *reinterpret_cast<const float4 *>(g + (t * Tn + tok) * d + (int64_t)c * 64 * EV + lane * EV + q)
+                               : make_float4(0.f, 0.f, 0.f, 0.f);
+        gv[c][q] = v.x; gv[c][q + 1] = v.y; gv[c][q + 2] = v.z; gv[c][q + 3] = v.w;
+      }
+    for (int32_t j0 = b; j0 < e; j0 += 64) {
+      const int n = (e - j0) < 64 ? (e - j0) : 64;
+      const int32_t my_col = lane < n ? col[j0 + lane] : 0;
+      constexpr int LB = NCH <= 2 ? BWV_NU : NCH <= 4 ? BWV_NU / 2 : BWV_NU / 4;   // rows fetched together
+      for (int i0 = 0; i0 < n; i0 += BWV_NU) {
+        float p[BWV_NU];
+#pragma unroll
+        for (int h = 0; h < BWV_NU; h += LB) {
+          uint4 w[LB][NCH];
+#pragma unroll
+          for (int u = 0; u < LB; ++u) {
+            const int idx = i0 + h + u < n ? i0 + h + u : n - 1;
+            const T *wrow = wbase + (int64_t)__builtin_amdgcn_readlane(my_col, idx) * d;
+#pragma unroll
+            for (int c = 0; c < NCH; ++c)
+              w[u][c] = on[c] ? *reinterpret_cast<const uint4 *>(wrow + (int64_t)c * 64 * EV + lane * EV) : make_uint4(0, 0, 0, 0);
+          }
+#pragma unroll
+          for (int u = 0; u < LB; ++u) {
+            float a = 0.0f;
+#pragma unroll
+            for (int c = 0; c < NCH; ++c) {
+              float x[EV];
+              Piece<T>::unpack(w[u][c], x);
+#pragma unroll
+              for (int q = 0; q < EV; ++q) a = fmaf(x[q], gv[c][q], a);
+            }
+            p[h + u] = a;
+          }
+        }
+        const float tot = wave_sum8(p, lane);
+        const int u = ((lane >> 5) & 1) * 4 + ((lane >> 4) & 1) * 2 + ((lane >> 3) & 1);
+        if ((lane & 7) == 0 && i0 + u < n) pt[j0 + i0 + u] = tot;
+      }
+    }
+  }
+}
+
+// dval[j] = sum over the targets t >= s of part[t][j], in target order; one wavefront per row
+__global__ __launch_bounds__(BW_THREADS) void k_bwd_values_sum(const int32_t *row_ptr, const float *part, int64_t Tn,
+                                                                int64_t L, int64_t nnz, uint64_t src_mask, float *dval) {
   const int lane = lane_id(), wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
   const int64_t R = L * Tn;
   for (int64_t r = (int64_t)blockIdx.x * nwv + wv; r < R; r += (int64_t)gridDim.x * nwv) {
-    const int64_t s = r / Tn, tok = r - s * Tn;
-    const bool src_on = (src_mask >> s) & 1ull;
-    for (int32_t j0 = row_ptr[r]; j0 < row_ptr[r + 1]; j0 += 64) {
-      const int n = (row_ptr[r + 1] - j0) < 64 ? (row_ptr[r + 1] - j0) : 64;
-      const int32_t my_col = lane < n ? col[j0 + lane] : 0;
+    const int64_t s = r / Tn;
+    const bool on = (src_mask >> s) & 1ull;
+    for (int32_t j = row_ptr[r] + lane; j < row_ptr[r + 1]; j += 64) {
       float acc = 0.0f;
-      if (src_on) {
-        for (int64_t t = s; t < L; ++t) {
-          float4 gv[NC4];
-#pragma unroll
-          for (int c = 0; c < NC4; ++c) {
-            const int64_t e = (int64_t)c * 256 + lane * 4;
-            gv[c] = e < d ? *reinterpret_cast<const float4 *>(g + (t * Tn + tok) * d + e) : make_float4(0.f, 0.f, 0.f, 0.f);
-          }
-          const T *wbase = wp + bw_decoder_slot(tying, s, t, L) * F * d;
-          for (int i0 = 0; i0 < n; i0 += 4) {
-            float4 w[4][NC4];
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-              const int idx = i0 + u < n ? i0 + u : n - 1;
-              const T *wrow = wbase + (int64_t)__builtin_amdgcn_readlane(my_col, idx) * d;
-#pragma unroll
-              for (int c = 0; c < NC4; ++c) {
-                const int64_t e = (int64_t)c * 256 + lane * 4;
-                w[u][c] = e < d ? load4<T>(wrow + e) : make_float4(0.f, 0.f, 0.f, 0.f);
-              }
-            }
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-              float p = 0.0f;
-#pragma unroll
-              for (int c = 0; c < NC4; ++c)
-                p = fmaf(w[u][c].x, gv[c].x, fmaf(w[u][c].y, gv[c].y, fmaf(w[u][c].z, gv[c].z, fmaf(w[u][c].w, gv[c].w, p))));
-              p = wave_sum(p);
-              if (i0 + u < n && lane == i0 + u) acc += p;
-            }
-          }
-        }
-      }
-      if (lane < n) dval[j0 + lane] = acc;
+      if (on)
+        for (int64_t t = s; t < L; ++t) acc += part[t * nnz + j];
+      dval[j] = acc;
     }
   }
 }
@@ -223,16 +331,23 @@ __global__ __launch_bounds__(BW_THREADS) void k_csc_order(const int32_t *ptr, in
 
 // ---- weight gradients: one wavefront per output row ---------------------------------------------------
 // out_row[:] = sum over the list of (layer, feature) of coef[entry] * src[token][:]
-//   DECODER: wavefront (s, f, t >= s): coef = survivor value, src = g[t], out = dW[slot(s,t)][f]
-//   encoder: wavefront (s, f):         coef = dval,           src = x[s], out = dW_enc[s][f], rowsum = db_enc[s][f]
-template <typename SrcT, typename CoefT, int NC4, bool DECODER>
+//   DECODER: wavefront (s, f, t >= s): coef = survivor value, src = g[t] (model dtype copy),
+//            out = dW[slot(s,t)][f]
+//   encoder: wavefront (s, f):         coef = dval, src = x[s], out = dW_enc[s][f], rowsum = db_enc[s][f]
+// Rows are read in raw 16-byte pieces, up to FO_NU rows in flight.
+constexpr int FO_NU = 8;
+template <typename T, typename CoefT, int NCH, bool DECODER>
 __global__ __launch_bounds__(BW_THREADS) void k_feature_outer(
     const int32_t *__restrict__ ptr, const int32_t *__restrict__ ltok, const int32_t *__restrict__ lsrc,
-    const CoefT *__restrict__ coef, const SrcT *__restrict__ src, float *__restrict__ out, float *__restrict__ rowsum,
+    const CoefT *__restrict__ coef, const T *__restrict__ src, float *__restrict__ out, float *__restrict__ rowsum,
     int64_t Tn, int64_t d, int64_t F, int64_t L) {
+  constexpr int EV = Piece<T>::EV;
   const int lane = lane_id(), wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
-  const int64_t per_layer_rows = DECODER ? F * L : F;   // upper bound used to enumerate (f, t) pairs of a layer
+  const int64_t per_layer_rows = DECODER ? F * L : F;   // (target, feature) pairs of a layer (targets < s are skipped)
   const int64_t total = L * per_layer_rows;
+  bool on[NCH];
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) on[c] = (int64_t)c * 64 * EV + lane * EV < d;
   for (int64_t w = (int64_t)blockIdx.x * nwv + wv; w < total; w += (int64_t)gridDim.x * nwv) {
     const int64_t s = w / per_layer_rows, rem = w - s * per_layer_rows;
     int64_t f, t;
@@ -240,50 +355,57 @@ __global__ __launch_bounds__(BW_THREADS) void k_feature_outer(
     else { f = rem; t = s; }
     const int64_t q = s * F + f;
     const int32_t b = ptr[q], e = ptr[q + 1];
-    const SrcT *sbase = src + (DECODER ? t : s) * Tn * d;
-    float4 acc[NC4];
+    const T *sbase = src + (DECODER ? t : s) * Tn * d;
+    float acc[NCH][EV];
 #pragma unroll
-    for (int c = 0; c < NC4; ++c) acc[c] = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int c = 0; c < NCH; ++c)
+#pragma unroll
+      for (int k = 0; k < EV; ++k) acc[c][k] = 0.0f;
     float csum = 0.0f;
     for (int32_t i0 = b; i0 < e; i0 += 64) {
       const int n = (e - i0) < 64 ? (e - i0) : 64;
       int32_t mt = 0; float mc = 0.0f;
       if (lane < n) { mt = ltok[i0 + lane]; mc = Elem<CoefT>::to_f32(coef[lsrc[i0 + lane]]); }
-      for (int i = 0; i < n; i += 2) {
-        float4 v[2][NC4]; float cf[2];
+      constexpr int NU = NCH <= 2 ? FO_NU : NCH <= 4 ? FO_NU / 2 : FO_NU / 4;   // rows in flight: about 16 pieces per lane
+      for (int i = 0; i < n; i += NU) {
+        uint4 v[NU][NCH];
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
+        for (int u = 0; u < NU; ++u) {
           const int idx = i + u < n ? i + u : n - 1;
-          const SrcT *row = sbase + (int64_t)__builtin_amdgcn_readlane(mt, idx) * d;
-          cf[u] = i + u < n ? __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(mc), idx)) : 0.0f;
+          const T *row = sbase + (int64_t)__builtin_amdgcn_readlane(mt, idx) * d;
 #pragma unroll
-          for (int c = 0; c < NC4; ++c) {
-            const int64_t el = (int64_t)c * 256 + lane * 4;
-            v[u][c] = el < d ? load4<SrcT>(row + el) : make_float4(0.f, 0.f, 0.f, 0.f);
-          }
+          for (int c = 0; c < NCH; ++c)
+            v[u][c] = on[c] ? *reinterpret_cast<const uint4 *>(row + (int64_t)c * 64 * EV + lane * EV) : make_uint4(0, 0, 0, 0);
         }
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
-          csum += cf[u];
+        for (int u = 0; u < NU; ++u) {
+          const int idx = i + u < n ? i + u : n - 1;
+          const float cf = i + u < n ? __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(mc), idx)) : 0.0f;
+          csum += cf;
 #pragma unroll
-          for (int c = 0; c < NC4; ++c) {
-            acc[c].x = fmaf(cf[u], v[u][c].x, acc[c].x); acc[c].y = fmaf(cf[u], v[u][c].y, acc[c].y);
-            acc[c].z = fmaf(cf[u], v[u][c].z, acc[c].z); acc[c].w = fmaf(cf[u], v[u][c].w, acc[c].w);
+          for (int c = 0; c < NCH; ++c) {
+            float x[EV];
+            Piece<T>::unpack(v[u][c], x);
+#pragma unroll
+            for (int k = 0; k < EV; ++k) acc[c][k] = fmaf(cf, x[k], acc[c][k]);
           }
         }
       }
     }
     float *orow = out + (DECODER ? (bw_decoder_slot(CLT_TYING_NONE, s, t, L) * F + f) : q) * d;
 #pragma unroll
-    for (int c = 0; c < NC4; ++c) {
-      const int64_t el = (int64_t)c * 256 + lane * 4;
-      if (el < d) *reinterpret_cast<float4 *>(orow + el) = acc[c];
-    }
+    for (int c = 0; c < NCH; ++c)
+      if (on[c]) {
+#pragma unroll
+        for (int k = 0; k < EV; k += 4)
+          *reinterpret_cast<float4 *>(orow + (int64_t)c * 64 * EV + lane * EV + k) =
+              make_float4(acc[c][k], acc[c][k + 1], acc[c][k + 2], acc[c][k + 3]);
+      }
     if (!DECODER && rowsum && lane == 0) rowsum[q] = csum;
   }
 }
 
-static bool bw_shape_ok(int64_t d) { return d > 0 && d % 4 == 0 && d <= 2048; }
+static bool bw_shape_ok(int64_t d, int dtype) { return d > 0 && d % (dtype == CLT_BF16 ? 8 : 4) == 0 && d <= 2048; }
 
 }  // namespace
 
@@ -294,7 +416,7 @@ extern "C" size_t clt_mse_workspace_bytes(int64_t T, int64_t d, int64_t L) {
 }
 
 extern "C" int clt_mse_loss_grad(const void *rec, const void *target, int64_t T, int64_t d, int64_t L, int dtype,
-                                 float *loss_per_layer, float *g, float *bias_grad, void *workspace,
+                                 float *loss_per_layer, float *g, void *g_model, float *bias_grad, void *workspace,
                                  size_t workspace_bytes, void *stream) {
   if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
   if (T <= 0 || d <= 0 || L <= 0 || L > 65535 || !rec || !target || !loss_per_layer || !g || !workspace) return CLT_ERR_ARG;
@@ -308,8 +430,8 @@ extern "C" int clt_mse_loss_grad(const void *rec, const void *target, int64_t T,
   const int64_t per_layer = T * d;
   const float scale = (float)(2.0 / (double)per_layer);
   dim3 grid(512, (unsigned)L);
-  if (dtype == CLT_BF16) k_mse_grad<bf16_t><<<grid, BW_THREADS, 0, s>>>((const bf16_t *)rec, (const bf16_t *)target, per_layer, scale, g, acc);
-  else k_mse_grad<float><<<grid, BW_THREADS, 0, s>>>((const float *)rec, (const float *)target, per_layer, scale, g, acc);
+  if (dtype == CLT_BF16) k_mse_grad<bf16_t><<<grid, BW_THREADS, 0, s>>>((const bf16_t *)rec, (const bf16_t *)target, per_layer, scale, g, (bf16_t *)g_model, acc);
+  else k_mse_grad<float><<<grid, BW_THREADS, 0, s>>>((const float *)rec, (const float *)target, per_layer, scale, g, (float *)g_model, acc);
   k_loss_finish<<<(unsigned)clt_ceil_div(L, 256), 256, 0, s>>>(acc, (int)L, 1.0 / (double)per_layer, loss_per_layer);
   if (bias_grad) {
     k_colsum_partial<<<dim3((unsigned)clt_ceil_div(d, BW_THREADS), (unsigned)L, CS_SPLIT), BW_THREADS, 0, s>>>(g, T, d, part);
@@ -318,17 +440,31 @@ extern "C" int clt_mse_loss_grad(const void *rec, const void *target, int64_t T,
   return clt_check_launch();
 }
 
+extern "C" size_t clt_decode_backward_workspace_bytes(int64_t T, int64_t L, int64_t nnz) {
+  if (T <= 0 || L <= 0 || nnz < 0) return 256;
+  return (((size_t)L * (size_t)T * (BWV_XCDS + 1) * 4 + 255) & ~(size_t)255) + (size_t)L * (size_t)(nnz > 0 ? nnz : 1) * 4;
+}
+
 extern "C" int clt_decode_backward_values(const int32_t *row_ptr, const int32_t *col, const void *w_packed, const float *g,
                                           int64_t T, int64_t d, int64_t F, int64_t L, int tying, uint64_t src_mask,
-                                          int dtype, float *dval, void *stream) {
+                                          int64_t nnz, int dtype, float *dval, void *workspace, size_t workspace_bytes,
+                                          void *stream) {
   if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
-  if (T <= 0 || F <= 0 || L <= 0 || L > 64 || tying < 0 || tying > 2) return CLT_ERR_ARG;
-  if (!row_ptr || !w_packed || !g || !dval) return CLT_ERR_ARG;
-  if (!bw_shape_ok(d)) return CLT_ERR_RANGE;
+  if (T <= 0 || F <= 0 || L <= 0 || L > 64 || tying < 0 || tying > 2 || nnz < 0) return CLT_ERR_ARG;
+  if (!row_ptr || !w_packed || !g || !dval || !workspace) return CLT_ERR_ARG;
+  if (!bw_shape_ok(d, dtype)) return CLT_ERR_RANGE;
+  if (nnz == 0) return CLT_OK;
+  if (workspace_bytes < clt_decode_backward_workspace_bytes(T, L, nnz)) return CLT_ERR_WORKSPACE;
+  if ((((uintptr_t)workspace) & 255u) != 0) return CLT_ERR_ALIGN;
   hipStream_t s = (hipStream_t)stream;
-  const int nc4 = (int)clt_ceil_div(d, 256);
-  const unsigned nb = 256 * 16;
-#define CLT_BWV(TT, N) k_decode_bwd_values<TT, N><<<nb, BW_THREADS, 0, s>>>(row_ptr, col, (const TT *)w_packed, g, T, d, F, L, tying, src_mask, dval)
+  int32_t *sptr = (int32_t *)workspace;
+  float *part = (float *)((char *)workspace + (((size_t)L * (size_t)T * (BWV_XCDS + 1) * 4 + 255) & ~(size_t)255));
+  k_bw_slice_ptr<<<1024, 256, 0, s>>>(row_ptr, col, L * T, F, BWV_XCDS, sptr);
+  const int nc4 = (int)clt_ceil_div(d, dtype == CLT_BF16 ? 512 : 256);   // 16-byte pieces per lane
+  const int64_t npair = L * (L + 1) / 2;
+  const int64_t nblk = npair * clt_ceil_div(T, (BW_THREADS / 64) * BWV_NTOK) * BWV_XCDS;
+  if (nblk > 2147483647LL) return CLT_ERR_RANGE;
+#define CLT_BWV(TT, N) k_bwd_values_sliced<TT, N><<<(unsigned)nblk, BW_THREADS, 0, s>>>(sptr, col, (const TT *)w_packed, g, T, d, F, L, tying, nnz, part)
 #define CLT_BWV_N(TT)                                                                       \
   do {                                                                                      \
     switch (nc4) {                                                                          \
@@ -340,6 +476,7 @@ extern "C" int clt_decode_backward_values(const int32_t *row_ptr, const int32_t 
   if (dtype == CLT_BF16) CLT_BWV_N(bf16_t); else CLT_BWV_N(float);
 #undef CLT_BWV_N
 #undef CLT_BWV
+  k_bwd_values_sum<<<256 * 8, BW_THREADS, 0, s>>>(row_ptr, part, T, L, nnz, src_mask, dval);
   return clt_check_launch();
 }
 
@@ -369,16 +506,16 @@ extern "C" int clt_feature_lists(const int32_t *row_ptr, const int32_t *col, int
 }
 
 extern "C" int clt_decoder_weight_grad(const int32_t *list_ptr, const int32_t *list_tok, const int32_t *list_src,
-                                       const void *val, const float *g, float *dw_packed, int64_t T, int64_t d, int64_t F,
-                                       int64_t L, int tying, int dtype, void *stream) {
+                                       const void *val, const void *g_model, float *dw_packed, int64_t T, int64_t d,
+                                       int64_t F, int64_t L, int tying, int dtype, void *stream) {
   if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
   if (tying != CLT_TYING_NONE) return CLT_ERR_ARG;   // tied decoders sum over several (source, target) pairs: not built
-  if (T <= 0 || F <= 0 || L <= 0 || L > 64 || !list_ptr || !list_tok || !list_src || !val || !g || !dw_packed) return CLT_ERR_ARG;
-  if (!bw_shape_ok(d)) return CLT_ERR_RANGE;
+  if (T <= 0 || F <= 0 || L <= 0 || L > 64 || !list_ptr || !list_tok || !list_src || !val || !g_model || !dw_packed) return CLT_ERR_ARG;
+  if (!bw_shape_ok(d, dtype)) return CLT_ERR_RANGE;
   hipStream_t s = (hipStream_t)stream;
-  const int nc4 = (int)clt_ceil_div(d, 256);
+  const int nc4 = (int)clt_ceil_div(d, dtype == CLT_BF16 ? 512 : 256);   // 16-byte pieces per lane
   const unsigned nb = 256 * 32;
-#define CLT_DW(CT, N) k_feature_outer<float, CT, N, true><<<nb, BW_THREADS, 0, s>>>(list_ptr, list_tok, list_src, (const CT *)val, g, dw_packed, nullptr, T, d, F, L)
+#define CLT_DW(CT, N) k_feature_outer<CT, CT, N, true><<<nb, BW_THREADS, 0, s>>>(list_ptr, list_tok, list_src, (const CT *)val, (const CT *)g_model, dw_packed, nullptr, T, d, F, L)
 #define CLT_DW_N(CT)                                                                       \
   do {                                                                                     \
     switch (nc4) {                                                                         \
@@ -398,9 +535,9 @@ extern "C" int clt_encoder_weight_grad(const int32_t *list_ptr, const int32_t *l
                                        int64_t F, int64_t L, int dtype, void *stream) {
   if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
   if (T <= 0 || F <= 0 || L <= 0 || L > 65535 || !list_ptr || !list_tok || !list_src || !dval || !x || !dw_enc) return CLT_ERR_ARG;
-  if (!bw_shape_ok(d)) return CLT_ERR_RANGE;
+  if (!bw_shape_ok(d, dtype)) return CLT_ERR_RANGE;
   hipStream_t s = (hipStream_t)stream;
-  const int nc4 = (int)clt_ceil_div(d, 256);
+  const int nc4 = (int)clt_ceil_div(d, dtype == CLT_BF16 ? 512 : 256);   // 16-byte pieces per lane
   const unsigned nb = 256 * 32;
 #define CLT_EW(ST, N) k_feature_outer<ST, float, N, false><<<nb, BW_THREADS, 0, s>>>(list_ptr, list_tok, list_src, dval, (const ST *)x, dw_enc, db_enc, T, d, F, L)
 #define CLT_EW_N(ST)                                                                       \

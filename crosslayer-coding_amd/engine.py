@@ -304,8 +304,8 @@ def encode_threshold(x: torch.Tensor, w: torch.Tensor, b: Optional[torch.Tensor]
 
 # ---- backward pass (MSE reconstruction loss) ---------------------------------------------------------
 def mse_loss_grad(rec: torch.Tensor, target: torch.Tensor, ws: Optional[Workspace] = None):
-    """(loss per layer [L] fp32, g [L, T, d] fp32 = d loss / d rec, bias_grad [L, d] fp32) for
-    loss = sum over layers of mean((rec - target)^2) (losses.py:45-92)."""
+    """(loss per layer [L] fp32, g [L, T, d] fp32 = d loss / d rec, the same in the model dtype,
+    bias_grad [L, d] fp32) for loss = sum over layers of mean((rec - target)^2) (losses.py:45-92)."""
     nat.require_device(rec, "mse_loss_grad")
     L, T, d = rec.shape
     assert target.shape == rec.shape and target.dtype == rec.dtype and rec.is_contiguous() and target.is_contiguous()
@@ -313,16 +313,18 @@ def mse_loss_grad(rec: torch.Tensor, target: torch.Tensor, ws: Optional[Workspac
     loss = torch.empty(L, dtype=torch.float32, device=dev)
     g = torch.empty((L, T, d), dtype=torch.float32, device=dev)
     bias_grad = torch.empty((L, d), dtype=torch.float32, device=dev)
+    g_model = g if rec.dtype == torch.float32 else torch.empty((L, T, d), dtype=rec.dtype, device=dev)
     lib = nat.load()
     wbuf = (ws or Workspace(dev)).get("mse", lib.clt_mse_workspace_bytes(T, d, L))
     code = lib.clt_mse_loss_grad(nat.ptr(rec), nat.ptr(target), T, d, L, nat.dtype_code(rec.dtype), nat.ptr(loss),
-                                 nat.ptr(g), nat.ptr(bias_grad), nat.ptr(wbuf), wbuf.numel(), _stream(rec))
+                                 nat.ptr(g), nat.ptr(g_model) if g_model is not g else None, nat.ptr(bias_grad),
+                                 nat.ptr(wbuf), wbuf.numel(), _stream(rec))
     nat.check(code, "clt_mse_loss_grad")
-    return loss, g, bias_grad
+    return loss, g, g_model, bias_grad
 
 
 def decode_backward_values(surv: SurvivorList, w_packed: torch.Tensor, g: torch.Tensor, tying: str,
-                           src_mask: Optional[int] = None) -> torch.Tensor:
+                           src_mask: Optional[int] = None, ws: Optional[Workspace] = None) -> torch.Tensor:
     """d loss / d (kept activation) for every survivor, fp32 [nnz] (the straight-through gate hands
     it to the pre-activation unchanged, activations.py:66-96)."""
     L, T, F = surv.L, surv.T, surv.F
@@ -332,9 +334,11 @@ def decode_backward_values(surv: SurvivorList, w_packed: torch.Tensor, g: torch.
     if src_mask is None:
         src_mask = (1 << L) - 1
     dval = torch.empty(max(surv.nnz, 1), dtype=torch.float32, device=g.device)
-    code = nat.load().clt_decode_backward_values(nat.ptr(surv.row_ptr), nat.ptr(surv.col), nat.ptr(w_packed), nat.ptr(g),
-                                                 T, d, F, L, nat.TYING[tying], src_mask & ((1 << 64) - 1),
-                                                 nat.dtype_code(surv.dtype), nat.ptr(dval), _stream(g))
+    lib = nat.load()
+    wbuf = (ws or Workspace(g.device)).get("decode_backward", lib.clt_decode_backward_workspace_bytes(T, L, surv.nnz))
+    code = lib.clt_decode_backward_values(nat.ptr(surv.row_ptr), nat.ptr(surv.col), nat.ptr(w_packed), nat.ptr(g),
+                                          T, d, F, L, nat.TYING[tying], src_mask & ((1 << 64) - 1), surv.nnz,
+                                          nat.dtype_code(surv.dtype), nat.ptr(dval), nat.ptr(wbuf), wbuf.numel(), _stream(g))
     nat.check(code, "clt_decode_backward_values")
     return dval[:surv.nnz]
 
@@ -355,7 +359,9 @@ def feature_lists(surv: SurvivorList, ws: Optional[Workspace] = None):
 
 
 def decoder_weight_grad(lists, surv: SurvivorList, g: torch.Tensor, tying: str) -> torch.Tensor:
-    """fp32 [n_dec, F, d] gradient of the packed (feature-major) untied decoder weights."""
+    """fp32 [n_dec, F, d] gradient of the packed (feature-major) untied decoder weights; ``g`` is
+    d loss / d rec in the model dtype."""
+    assert g.dtype == surv.dtype and g.is_contiguous()
     ptr, tok, src = lists
     L, T, F = surv.L, surv.T, surv.F
     d = g.shape[2]

@@ -309,35 +309,40 @@ int clt_decoder_norms(const void *w_packed, void *norms, int64_t d, int64_t F,
  *
  * clt_mse_loss_grad: loss_per_layer[l] = mean((rec[l] - target[l])^2) as nn.MSELoss gives per
  *   layer (clt/training/losses.py:45-92, summed over layers by the caller), g[l][t][:] =
- *   2 (rec - target) / (T d) in fp32, and (when bias_grad != NULL) bias_grad[l][:] = sum over
+ *   2 (rec - target) / (T d) in fp32 (and, when g_model != NULL, the same rounded to the model
+ *   dtype: what clt_decoder_weight_grad reads), and (when bias_grad != NULL) bias_grad[l][:] = sum over
  *   tokens of g[l] - the gradient of every decoder bias that feeds target l.
  *   rec / target [L][T][d] in the model dtype; workspace clt_mse_workspace_bytes().
  * clt_decode_backward_values: dval[j] = sum over targets t >= s of g[t][token] . w[slot(s,t)][f]
  *   for survivor j = (s, token, f): the gradient of the loss with respect to the kept
  *   activation, which the straight-through gate passes on to the pre-activation
- *   (clt/models/activations.py:66-96).  dval [nnz] fp32.
+ *   (clt/models/activations.py:66-96).  dval [nnz] fp32; nnz = row_ptr[L*T]; workspace
+ *   clt_decode_backward_workspace_bytes() (slice pointers and one partial per target and survivor,
+ *   summed in target order).
  * clt_feature_lists: the survivor list regrouped by (layer, feature): list_ptr [L*F+1],
  *   list_tok [nnz] token of each entry, list_src [nnz] its position in col / val.  Lists of up to
  *   64 entries are in token order.  Pass list_tok = list_src = NULL to get the counts only.
  * clt_decoder_weight_grad: dw_packed[slot(s,t)][f][:] = sum over the list of (s, f) of
- *   val * g[t][token][:] (fp32, feature-major like w_packed; untied decoders only).
+ *   val * g_model[t][token][:] (fp32 sums, feature-major like w_packed; untied decoders only).
  * clt_encoder_weight_grad: dw_enc[s][f][:] = sum over the list of dval * x[s][token][:],
  *   db_enc[s][f] = sum of dval (fp32; x [L][T][d] in the model dtype).
- * Limits: d % 4 == 0 and d <= 2048.
+ * Limits: d % 8 == 0 (bf16) / d % 4 == 0 (fp32) and d <= 2048.
  */
 size_t clt_mse_workspace_bytes(int64_t T, int64_t d, int64_t L);
 int clt_mse_loss_grad(const void *rec, const void *target, int64_t T, int64_t d, int64_t L,
-                      int dtype, float *loss_per_layer, float *g, float *bias_grad,
+                      int dtype, float *loss_per_layer, float *g, void *g_model, float *bias_grad,
                       void *workspace, size_t workspace_bytes, void *stream);
+size_t clt_decode_backward_workspace_bytes(int64_t T, int64_t L, int64_t nnz);
 int clt_decode_backward_values(const int32_t *row_ptr, const int32_t *col, const void *w_packed,
                                const float *g, int64_t T, int64_t d, int64_t F, int64_t L,
-                               int tying, uint64_t src_mask, int dtype, float *dval, void *stream);
+                               int tying, uint64_t src_mask, int64_t nnz, int dtype, float *dval,
+                               void *workspace, size_t workspace_bytes, void *stream);
 size_t clt_feature_lists_workspace_bytes(int64_t F, int64_t L);
 int clt_feature_lists(const int32_t *row_ptr, const int32_t *col, int64_t T, int64_t F, int64_t L,
                       int32_t *list_ptr, int32_t *list_tok, int32_t *list_src,
                       void *workspace, size_t workspace_bytes, void *stream);
 int clt_decoder_weight_grad(const int32_t *list_ptr, const int32_t *list_tok, const int32_t *list_src,
-                            const void *val, const float *g, float *dw_packed,
+                            const void *val, const void *g_model, float *dw_packed,
                             int64_t T, int64_t d, int64_t F, int64_t L, int tying, int dtype,
                             void *stream);
 int clt_encoder_weight_grad(const int32_t *list_ptr, const int32_t *list_tok, const int32_t *list_src,
