@@ -264,18 +264,26 @@ def run_backward(args):
     model.eval()
     g = torch.Generator(device=dev).manual_seed(99)
     targets = {l: torch.randn(wl.tokens, wl.d_model, generator=g, device=dev).to(model.dtype) for l in range(wl.num_layers)}
-    for _ in range(args.warmup):
+    opt = cca.CLTAdam(model, lr=1e-4) if args.train_step else None
+
+    def one():
+        if opt is not None:
+            return model.training_step(inputs, targets, opt)
         loss, grads = model.loss_and_gradients(inputs, targets)
-    del grads
+        del grads
+        return loss
+
+    for _ in range(args.warmup):
+        loss = one()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        loss, grads = model.loss_and_gradients(inputs, targets)
-        del grads
+        loss = one()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     return {
-        "metric": "CLT forward + MSE loss + gradients tokens/sec (no optimizer step)",
+        "metric": ("CLT training step tokens/sec (forward, MSE loss, gradients, Adam lr 1e-4 with fp32 moments)"
+                   if opt is not None else "CLT forward + MSE loss + gradients tokens/sec (no optimizer step)"),
         "value": wl.tokens * args.steps / wall, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": wall / args.steps * 1e3, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16" if wl.dtype == "bfloat16" else "f32", "data": "synthetic",
@@ -334,6 +342,8 @@ def main():
                          "selection, per-feature minimum) instead of the forward")
     ap.add_argument("--backward", action="store_true",
                     help="time forward + MSE loss + all gradients (loss_and_gradients) instead of the forward")
+    ap.add_argument("--train-step", action="store_true",
+                    help="time full optimisation steps: forward, MSE loss, gradients, Adam update")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one 256 MiB elementwise copy (counter yardstick for profiled runs)")
     args = ap.parse_args()
@@ -344,7 +354,7 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a ROCm GPU", file=sys.stderr)
         sys.exit(2)
-    print(json.dumps(run_theta(args) if args.theta_estimation else run_backward(args) if args.backward else run_gpu(args)))
+    print(json.dumps(run_theta(args) if args.theta_estimation else run_backward(args) if (args.backward or args.train_step) else run_gpu(args)))
 
 
 if __name__ == "__main__":

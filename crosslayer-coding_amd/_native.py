@@ -26,6 +26,7 @@ _vp = ctypes.c_void_p
 _int = ctypes.c_int
 _u64 = ctypes.c_uint64
 _sz = ctypes.c_size_t
+_f64 = ctypes.c_double
 
 # name -> (restype, argtypes); mirrors include/clt_hip.h one to one
 _SIGNATURES = {
@@ -61,6 +62,8 @@ _SIGNATURES = {
     "clt_feature_lists": (_int, [_vp, _vp, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _sz, _vp]),
     "clt_decoder_weight_grad": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp]),
     "clt_encoder_weight_grad": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
+    "clt_adam_step": (_int, [_vp, _vp, _vp, _vp, _i64, _f64, _f64, _f64, _f64, _i64, _int, _vp]),
+    "clt_adam_step_decoder": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _f64, _f64, _f64, _f64, _i64, _int, _vp]),
     "clt_decoder_norms": (_int, [_vp, _vp, _i64, _i64, _i64, _int, _int, _vp]),
 }
 

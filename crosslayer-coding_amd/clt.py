@@ -159,13 +159,10 @@ class CrossLayerTranscoder(BaseTranscoder):
         logger.info(f"Rank {self.rank}: CLT model config updated by ThetaManager. New activation_fn='{self.config.activation_fn}'.")
 
     # ---- loss and gradients --------------------------------------------------------------------
-    @torch.no_grad()
-    def loss_and_gradients(self, inputs: Dict[int, torch.Tensor], targets: Dict[int, torch.Tensor]):
-        """MSE reconstruction loss (sum over layers of the per-layer mean, losses.py:45-92) and the
-        gradients torch autograd gives the reference for it, computed from the survivor list:
-        returns (loss [fp32 scalar tensor], {state-dict key: fp32 gradient in the parameter's shape}).
-        Needs every layer present, equal token counts, untied decoders, a top-k or JumpReLU /
-        ReLU activation without skip connections or feature affine terms."""
+    def _loss_and_raw_gradients(self, inputs: Dict[int, torch.Tensor], targets: Dict[int, torch.Tensor]):
+        """(per-layer losses [L] fp32, raw gradients): ``enc_w`` [L, F, d], ``enc_b`` [L, F],
+        ``dec_w`` [n_dec, F, d] (feature-major, decoders in "s->t" order), ``dec_b`` [L, d] (row t is the
+        gradient of every decoder bias that feeds target t); all fp32."""
         cfg = self.config
         L, d, F = cfg.num_layers, cfg.d_model, cfg.num_features
         if cfg.decoder_tying != "none" or cfg.skip_connection or getattr(cfg, "enable_feature_offset", False) \
@@ -176,32 +173,50 @@ class CrossLayerTranscoder(BaseTranscoder):
         res = self._survivors(inputs)
         if res is None:
             raise ValueError("inputs do not form one [layers, tokens, d_model] batch")
-        layers, T, surv = res
+        _, T, surv = res
         ws = self._workspace()
         mask = (1 << L) - 1
         rec = self.decoder_module.decode_survivors(surv, mask, ws=ws)
         tgt = torch.stack([targets[l].to(device=self.device, dtype=self.dtype).reshape(-1, d) for l in range(L)])
         loss_l, g, g_model, bias_grad = engine.mse_loss_grad(rec, tgt.contiguous(), ws)
-        w_packed = self.decoder_module.packed()
-        dval = engine.decode_backward_values(surv, w_packed, g, cfg.decoder_tying, mask, ws)
+        dval = engine.decode_backward_values(surv, self.decoder_module.packed(), g, cfg.decoder_tying, mask, ws)
         lists = engine.feature_lists(surv, ws)
         dw_dec = engine.decoder_weight_grad(lists, surv, g_model, cfg.decoder_tying)
         _, x_slab, _, _ = self.encoder_module.prepare_slab(inputs)
         dw_enc, db_enc = engine.encoder_weight_grad(lists, dval, x_slab.contiguous(), F)
-        grads: Dict[str, torch.Tensor] = {}
+        return loss_l, {"enc_w": dw_enc, "enc_b": db_enc, "dec_w": dw_dec, "dec_b": bias_grad}
+
+    @torch.no_grad()
+    def loss_and_gradients(self, inputs: Dict[int, torch.Tensor], targets: Dict[int, torch.Tensor]):
+        """MSE reconstruction loss (sum over layers of the per-layer mean, losses.py:45-92) and the
+        gradients torch autograd gives the reference for it, computed from the survivor list:
+        returns (loss [fp32 scalar tensor], {state-dict key: fp32 gradient in the parameter's shape}).
+        Needs every layer present, equal token counts, untied decoders, a top-k or JumpReLU /
+        ReLU activation without skip connections or feature affine terms."""
+        L = self.config.num_layers
+        loss_l, raw = self._loss_and_raw_gradients(inputs, targets)
+        grads: Dict[str, Optional[torch.Tensor]] = {}
         for l in range(L):
-            grads[f"encoder_module.encoders.{l}.weight"] = dw_enc[l]
-            grads[f"encoder_module.encoders.{l}.bias_param"] = db_enc[l]
+            grads[f"encoder_module.encoders.{l}.weight"] = raw["enc_w"][l]
+            grads[f"encoder_module.encoders.{l}.bias_param"] = raw["enc_b"][l]
         slot = 0
         for s_ in range(L):
             for t in range(s_, L):
-                grads[f"decoder_module.decoders.{s_}->{t}.weight"] = dw_dec[slot].t()     # [d, F] view of the packed gradient
-                grads[f"decoder_module.decoders.{s_}->{t}.bias_param"] = bias_grad[t]
+                grads[f"decoder_module.decoders.{s_}->{t}.weight"] = raw["dec_w"][slot].t()   # [d, F] view
+                grads[f"decoder_module.decoders.{s_}->{t}.bias_param"] = raw["dec_b"][t]
                 slot += 1
-        if cfg.activation_fn == "jumprelu":
+        if self.config.activation_fn == "jumprelu":
             # the threshold's own gradient (activations.py:183-220) needs the dense neighbourhood of theta
             grads["theta_manager.log_threshold"] = None
         return loss_l.sum(), grads
+
+    @torch.no_grad()
+    def training_step(self, inputs: Dict[int, torch.Tensor], targets: Dict[int, torch.Tensor], optimizer) -> torch.Tensor:
+        """One optimisation step on the MSE reconstruction loss (trainer.py:663-778 without the
+        auxiliary losses): forward, gradients, ``optimizer.step``; returns the loss before the step."""
+        loss_l, raw = self._loss_and_raw_gradients(inputs, targets)
+        optimizer.step(raw)
+        return loss_l.sum()
 
     # ---- encode (per-layer activations) ---------------------------------------------------
     def encode(self, x: torch.Tensor, layer_idx: int) -> torch.Tensor:

@@ -1,0 +1,94 @@
+// Adam update (torch.optim.Adam semantics: bias-corrected first / second moments, no weight decay,
+// no amsgrad; the reference builds its optimizer in clt/training/trainer.py:290-312) with fp32
+// moments and fp32 gradients on parameters in the model dtype:
+//   m = b1 m + (1 - b1) g;  v = b2 v + (1 - b2) g^2
+//   p -= (lr / (1 - b1^step)) * m / (sqrt(v) / sqrt(1 - b2^step) + eps)
+// computed in fp32 and rounded once to the parameter dtype.
+#include "clt_common.h"
+
+namespace {
+
+struct AdamCoef { float b1, b2, step_size, inv_sqrt_bc2, eps; };
+
+__device__ __forceinline__ float adam_update(float p, float g, float &m, float &v, const AdamCoef &c) {
+  m = c.b1 * m + (1.0f - c.b1) * g;
+  v = c.b2 * v + (1.0f - c.b2) * g * g;
+  return p - c.step_size * m / (sqrtf(v) * c.inv_sqrt_bc2 + c.eps);
+}
+
+// parameter, gradient and moments in the same layout
+template <typename T>
+__global__ __launch_bounds__(256) void k_adam(T *p, const float *g, float *m, float *v, int64_t n, AdamCoef c) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+    float mi = m[i], vi = v[i];
+    const float np = adam_update(Elem<T>::to_f32(p[i]), g[i], mi, vi, c);
+    m[i] = mi; v[i] = vi; p[i] = Elem<T>::from_f32(np);
+  }
+}
+
+// Decoder matrix: the parameter lives in the checkpoint layout [d][F]; gradient, moments and the
+// feature-major working copy are [F][d].  A block takes a 64 x 64 tile: the update runs on the
+// feature-major side (all accesses contiguous), the new values go to the working copy directly and
+// to the parameter through an LDS transpose.
+template <typename T>
+__global__ __launch_bounds__(256) void k_adam_decoder(T *w_ref, T *w_packed, const float *g, float *m, float *v,
+                                                      int64_t d, int64_t F, AdamCoef c) {
+  __shared__ T tile[64][65];
+  const int64_t f0 = (int64_t)blockIdx.x * 64, d0 = (int64_t)blockIdx.y * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int i = ty; i < 64; i += 4) {
+    const int64_t f = f0 + i, dd = d0 + tx;
+    if (f < F && dd < d) {
+      const int64_t at = f * d + dd;
+      float mi = m[at], vi = v[at];
+      const T np = Elem<T>::from_f32(adam_update(Elem<T>::to_f32(w_packed[at]), g[at], mi, vi, c));
+      m[at] = mi; v[at] = vi; w_packed[at] = np;
+      tile[i][tx] = np;
+    }
+  }
+  __syncthreads();
+  for (int i = ty; i < 64; i += 4) {
+    const int64_t dd = d0 + i, f = f0 + tx;
+    if (dd < d && f < F) w_ref[dd * F + f] = tile[tx][i];
+  }
+}
+
+static AdamCoef adam_coef(double lr, double b1, double b2, double eps, int64_t step) {
+  AdamCoef c;
+  c.b1 = (float)b1; c.b2 = (float)b2; c.eps = (float)eps;
+  c.step_size = (float)(lr / (1.0 - pow(b1, (double)step)));
+  c.inv_sqrt_bc2 = (float)(1.0 / sqrt(1.0 - pow(b2, (double)step)));
+  return c;
+}
+
+}  // namespace
+
+extern "C" int clt_adam_step(void *param, const float *grad, float *m, float *v, int64_t n, double lr, double beta1,
+                             double beta2, double eps, int64_t step, int dtype, void *stream) {
+  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (n < 0 || step < 1 || !(beta1 >= 0 && beta1 < 1) || !(beta2 >= 0 && beta2 < 1)) return CLT_ERR_ARG;
+  if (n == 0) return CLT_OK;
+  if (!param || !grad || !m || !v) return CLT_ERR_ARG;
+  const AdamCoef c = adam_coef(lr, beta1, beta2, eps, step);
+  hipStream_t s = (hipStream_t)stream;
+  int64_t nb = clt_ceil_div(n, 256);
+  if (nb > 256 * 64) nb = 256 * 64;
+  if (dtype == CLT_BF16) k_adam<bf16_t><<<(unsigned)nb, 256, 0, s>>>((bf16_t *)param, grad, m, v, n, c);
+  else k_adam<float><<<(unsigned)nb, 256, 0, s>>>((float *)param, grad, m, v, n, c);
+  return clt_check_launch();
+}
+
+extern "C" int clt_adam_step_decoder(void *w_ref, void *w_packed, const float *grad_packed, float *m, float *v, int64_t d,
+                                     int64_t F, double lr, double beta1, double beta2, double eps, int64_t step, int dtype,
+                                     void *stream) {
+  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (d <= 0 || F <= 0 || step < 1 || !(beta1 >= 0 && beta1 < 1) || !(beta2 >= 0 && beta2 < 1)) return CLT_ERR_ARG;
+  if (!w_ref || !w_packed || !grad_packed || !m || !v) return CLT_ERR_ARG;
+  if (clt_ceil_div(d, 64) > 65535) return CLT_ERR_RANGE;
+  const AdamCoef c = adam_coef(lr, beta1, beta2, eps, step);
+  hipStream_t s = (hipStream_t)stream;
+  dim3 grid((unsigned)clt_ceil_div(F, 64), (unsigned)clt_ceil_div(d, 64));
+  if (dtype == CLT_BF16) k_adam_decoder<bf16_t><<<grid, 256, 0, s>>>((bf16_t *)w_ref, (bf16_t *)w_packed, grad_packed, m, v, d, F, c);
+  else k_adam_decoder<float><<<grid, 256, 0, s>>>((float *)w_ref, (float *)w_packed, grad_packed, m, v, d, F, c);
+  return clt_check_launch();
+}

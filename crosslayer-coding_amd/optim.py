@@ -1,0 +1,75 @@
+"""Adam for the transcoder's encoder / decoder parameters, driven by the sparse gradients of
+``CrossLayerTranscoder.loss_and_gradients``.
+
+The reference trains with ``torch.optim.Adam`` / ``AdamW`` over autograd gradients
+(clt/training/trainer.py:290-312, 751-778).  Here the moments are fp32 whatever the parameter dtype,
+the decoder moments live in the feature-major layout of the gradients, and one kernel per decoder
+matrix updates the checkpoint-layout parameter and its feature-major working copy together, so no
+repacking follows a step.  Semantics: torch.optim.Adam without weight decay or amsgrad.
+"""
+
+from __future__ import annotations
+
+from typing import Dict, Tuple
+
+import torch
+
+from . import _native as nat
+
+
+class CLTAdam:
+    def __init__(self, model, lr: float = 1e-4, betas: Tuple[float, float] = (0.9, 0.999), eps: float = 1e-8):
+        self.model = model
+        self.lr, self.betas, self.eps = float(lr), (float(betas[0]), float(betas[1])), float(eps)
+        self.step_count = 0
+        cfg = model.config
+        if cfg.decoder_tying != "none":
+            raise NotImplementedError("CLTAdam is built for untied decoders")
+        L, F, d = cfg.num_layers, cfg.num_features, cfg.d_model
+        dev = model.device
+        n_dec = L * (L + 1) // 2
+        z = lambda *shape: torch.zeros(shape, dtype=torch.float32, device=dev)   # noqa: E731
+        self.state: Dict[str, Tuple[torch.Tensor, torch.Tensor]] = {
+            "enc_w": (z(L, F, d), z(L, F, d)), "enc_b": (z(L, F), z(L, F)),
+            "dec_w": (z(n_dec, F, d), z(n_dec, F, d)), "dec_b": (z(n_dec, d), z(n_dec, d)),
+        }
+
+    def _adam(self, param: torch.Tensor, grad: torch.Tensor, m: torch.Tensor, v: torch.Tensor) -> None:
+        assert param.is_contiguous() and grad.is_contiguous() and grad.dtype == torch.float32 and grad.numel() == param.numel()
+        code = nat.load().clt_adam_step(nat.ptr(param), nat.ptr(grad), nat.ptr(m), nat.ptr(v), param.numel(), self.lr,
+                                        self.betas[0], self.betas[1], self.eps, self.step_count,
+                                        nat.dtype_code(param.dtype), nat.current_stream(param.device))
+        nat.check(code, "clt_adam_step")
+
+    @torch.no_grad()
+    def step(self, raw) -> None:
+        """``raw``: the gradient tensors of ``CrossLayerTranscoder._loss_and_raw_gradients``."""
+        model = self.model
+        self.step_count += 1
+        w_slab, b_slab = model.encoder_module.stacked()
+        self._adam(w_slab, raw["enc_w"], *self.state["enc_w"])
+        self._adam(b_slab, raw["enc_b"], *self.state["enc_b"])
+        dec = model.decoder_module
+        packed = dec.packed()
+        decs = dec._ordered()
+        L = model.config.num_layers
+        lib = nat.load()
+        m_w, v_w = self.state["dec_w"]
+        m_b, v_b = self.state["dec_b"]
+        slot = 0
+        for s in range(L):
+            for t in range(s, L):
+                lin = decs[slot]
+                w = lin.weight.data
+                assert w.is_contiguous()
+                d, F = w.shape
+                code = lib.clt_adam_step_decoder(nat.ptr(w), nat.ptr(packed[slot]), nat.ptr(raw["dec_w"][slot]),
+                                                 nat.ptr(m_w[slot]), nat.ptr(v_w[slot]), d, F, self.lr, self.betas[0],
+                                                 self.betas[1], self.eps, self.step_count, nat.dtype_code(w.dtype),
+                                                 nat.current_stream(w.device))
+                nat.check(code, "clt_adam_step_decoder")
+                self._adam(lin.bias_param.data, raw["dec_b"][t], m_b[slot], v_b[slot])
+                slot += 1
+        # the kernels wrote through .data: caches keyed on version counters would not notice
+        dec._bias_cache.clear()
+        dec._cached_decoder_norms = None

@@ -349,6 +349,22 @@ int clt_encoder_weight_grad(const int32_t *list_ptr, const int32_t *list_tok, co
                             const float *dval, const void *x, float *dw_enc, float *db_enc,
                             int64_t T, int64_t d, int64_t F, int64_t L, int dtype, void *stream);
 
+/*
+ * Adam update with fp32 moments and fp32 gradients on parameters in the model dtype
+ * (torch.optim.Adam semantics without weight decay / amsgrad; the reference builds its
+ * optimizer in clt/training/trainer.py:290-312).  `step` counts from 1.
+ * clt_adam_step: param, grad, m, v share one layout (n elements).
+ * clt_adam_step_decoder: one decoder matrix; w_ref is the parameter in the checkpoint layout
+ *   [d][F], w_packed its feature-major working copy [F][d]; grad_packed, m, v are [F][d].  Both
+ *   copies receive the same new values.
+ */
+int clt_adam_step(void *param, const float *grad, float *m, float *v, int64_t n,
+                  double lr, double beta1, double beta2, double eps, int64_t step,
+                  int dtype, void *stream);
+int clt_adam_step_decoder(void *w_ref, void *w_packed, const float *grad_packed, float *m, float *v,
+                          int64_t d, int64_t F, double lr, double beta1, double beta2, double eps,
+                          int64_t step, int dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -85,3 +85,103 @@ def test_feature_lists_are_a_permutation_grouped_by_feature(dev):
             assert torch.equal(rows[src[b:e]] % T, tok[b:e])
             if e - b <= 64:
                 assert bool((tok[b + 1:e] > tok[b:e - 1]).all())
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_training_steps_match_torch_adam_on_autograd_gradients(dev, dtype):
+    # two optimisation steps; reference: torch.optim.Adam over the oracle's autograd gradients, fp32
+    # parameters, the gate of each step taken from the model (so both sides differentiate the same
+    # function); bf16 parameters are compared after rounding the reference to bf16
+    import crosslayer_coding_amd as cca
+    wl = BASE.scaled("tr", dtype=dtype, num_layers=2, d_model=128, num_features=256, tokens=64, k=6)
+    tdt = getattr(torch, dtype)
+    model, sd, x, targets = build(wl, dev)
+    L = wl.num_layers
+    names = synth.decoder_names(wl)
+    ref = {k: v.detach().float().clone().requires_grad_(True) for k, v in sd.items()}
+    ropt = torch.optim.Adam(list(ref.values()), lr=1e-2, betas=(0.9, 0.999), eps=1e-8)
+    opt = cca.CLTAdam(model, lr=1e-2)
+    inputs = {l: x[l].to(dev) for l in range(L)}
+    tg = {l: t.to(dev) for l, t in targets.items()}
+    for step in range(2):
+        masks = {l: (a != 0).cpu() for l, a in model.get_feature_activations(inputs).items()}
+        loss = model.training_step(inputs, tg, opt)
+        # the bf16 model computes with bf16-rounded parameters: give the reference the same view
+        cur = {k: (v.detach().to(tdt).float() if tdt == torch.bfloat16 else v.detach()) for k, v in ref.items()}
+        ref_loss, grads = orc.mse_loss_and_gradients(
+            {l: x[l] for l in range(L)}, targets,
+            enc_w=[cur[f"encoder_module.encoders.{l}.weight"] for l in range(L)],
+            enc_b=[cur[f"encoder_module.encoders.{l}.bias_param"] for l in range(L)],
+            dec_w={n: cur[f"decoder_module.decoders.{n}.weight"] for n in names},
+            dec_b={n: cur[f"decoder_module.decoders.{n}.bias_param"] for n in names},
+            activation_fn="batchtopk", num_layers=L, k=wl.k, masks=masks)
+        assert abs(float(loss) - float(ref_loss)) <= (1e-4 if tdt == torch.float32 else 2e-2) * abs(float(ref_loss))
+        ropt.zero_grad()
+        for k, p in ref.items():
+            p.grad = grads[k].clone()
+        ropt.step()
+    new_sd = model.state_dict()
+    # Adam's first steps move a parameter by about lr * sign(gradient) whatever the gradient's size, so
+    # an element whose gradient is zero up to rounding may move either way: compare the displacement
+    # as a whole (rel-L2), and element by element where the reference gradient is not negligible
+    for k, p in ref.items():
+        got = new_sd[k].float().cpu()
+        moved = got - sd[k].float()
+        want = p.detach() - sd[k].float()
+        err = orc.rel_l2(moved, want)
+        print(k, "displacement rel-L2", err)
+        assert err <= (2e-2 if tdt == torch.float32 else 0.15), (k, err)
+        if tdt == torch.float32:
+            g = grads[k]
+            clear = g.abs() > 1e-3 * g.abs().max()
+            assert torch.allclose(got[clear], p.detach()[clear], rtol=1e-4, atol=1e-4), k
+    # the feature-major working copy was updated together with the parameters
+    packed = model.decoder_module.packed()
+    slot = 0
+    for s in range(L):
+        for t in range(s, L):
+            assert torch.equal(packed[slot], new_sd[f"decoder_module.decoders.{s}->{t}.weight"].t())
+            slot += 1
+    # and a forward after the steps runs on the new weights
+    rec = model(inputs)
+    assert all(torch.isfinite(r).all() for r in rec.values())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_adam_kernels_match_torch_adam_on_given_gradients(dev, dtype):
+    # same gradients on both sides (zeros and tiny values included): the update itself, three steps
+    from crosslayer_coding_amd import _native
+    lib = _native.load()
+    gen = torch.Generator().manual_seed(5)
+    d, F = 96, 200  # not multiples of the 64 x 64 tile
+    p0 = (torch.randn(d, F, generator=gen) * 0.1).to(dtype)
+    ref = p0.float().clone().requires_grad_(True)
+    ropt = torch.optim.Adam([ref], lr=3e-3, betas=(0.9, 0.999), eps=1e-8)
+    w_ref = p0.to(dev).contiguous()
+    w_packed = p0.t().contiguous().to(dev)
+    flat = p0.to(dev).clone().view(-1)
+    m = torch.zeros(F, d, device=dev); v = torch.zeros(F, d, device=dev)
+    m2 = torch.zeros(d * F, device=dev); v2 = torch.zeros(d * F, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    for step in range(1, 4):
+        g = torch.randn(d, F, generator=gen) * 10.0 ** float(torch.randint(-9, 0, (1,), generator=gen))
+        g[torch.rand(d, F, generator=gen) < 0.3] = 0.0
+        if dtype == torch.bfloat16:
+            # the reference keeps fp32 master values; the kernel rounds the parameter each step
+            with torch.no_grad():
+                ref.copy_(ref.to(dtype).float())
+        ropt.zero_grad(); ref.grad = g.clone(); ropt.step()
+        gp = g.t().contiguous().to(dev)
+        rc = lib.clt_adam_step_decoder(w_ref.data_ptr(), w_packed.data_ptr(), gp.data_ptr(), m.data_ptr(), v.data_ptr(),
+                                       d, F, 3e-3, 0.9, 0.999, 1e-8, step, _native.dtype_code(dtype), stream)
+        assert rc == 0
+        gf = g.contiguous().view(-1).to(dev)
+        rc = lib.clt_adam_step(flat.data_ptr(), gf.data_ptr(), m2.data_ptr(), v2.data_ptr(), d * F,
+                               3e-3, 0.9, 0.999, 1e-8, step, _native.dtype_code(dtype), stream)
+        assert rc == 0
+    torch.cuda.synchronize()
+    assert torch.equal(w_ref, w_packed.t())
+    assert torch.equal(w_ref.view(-1), flat)
+    want = ref.detach().to(dtype).float()
+    tol = dict(rtol=1e-5, atol=1e-6) if dtype == torch.float32 else dict(rtol=1e-2, atol=1e-3)
+    assert torch.allclose(w_ref.float().cpu(), want, **tol)
