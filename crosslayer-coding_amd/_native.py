@@ -65,6 +65,10 @@ _SIGNATURES = {
     "clt_adam_step": (_int, [_vp, _vp, _vp, _vp, _i64, _f64, _f64, _f64, _f64, _i64, _int, _vp]),
     "clt_adam_step_decoder": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _f64, _f64, _f64, _f64, _i64, _int, _vp]),
     "clt_decoder_norms": (_int, [_vp, _vp, _i64, _i64, _i64, _int, _int, _vp]),
+    "clt_survivor_metrics": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _int, ctypes.c_float, _vp, _vp, _vp]),
+    "clt_dead_feature_update": (_int, [_vp, _vp, _i64, _vp]),
+    "clt_reconstruction_stats_workspace_bytes": (_sz, [_i64, _i64]),
+    "clt_reconstruction_stats": (_int, [_vp, _vp, _i64, _i64, _i64, _int, _int, _vp, _vp, _f64, _vp, _vp, _sz, _vp]),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)

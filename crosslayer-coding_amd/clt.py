@@ -391,23 +391,35 @@ class CrossLayerTranscoder(BaseTranscoder):
         return {l: dense[i] for i, l in enumerate(layers)}
 
     # ---- forward ---------------------------------------------------------------------------
+    def forward_with_survivors(self, inputs: Dict[int, torch.Tensor]):
+        """(reconstructions, survivor list over all num_layers) from one pass, or None when the inputs
+        need the per-layer fallbacks.  The list is what get_feature_activations would densify; the
+        evaluator and the dead-feature counters read it directly."""
+        self._sync_device()
+        cfg = self.config
+        L = cfg.num_layers
+        res = self._survivors(inputs)
+        if res is None:
+            return None
+        layers, T, surv = res
+        full = self._expand_layers(layers, surv)
+        src_mask = 0
+        for l in layers:
+            src_mask |= 1 << l
+        skip = (self.decoder_module.skip_all_targets(inputs, src_mask, T) if cfg.skip_connection else None)
+        targets = [t for t in range(L) if t in inputs]
+        out = self.decoder_module.decode_survivors(full, src_mask, min(targets), max(targets) + 1, skip_add=skip,
+                                                   ws=self._workspace())
+        return {t: out[t] for t in targets}, full
+
     def forward(self, inputs: Dict[int, torch.Tensor]) -> Dict[int, torch.Tensor]:
         """Reconstruction of every layer present in ``inputs`` (clt.py:186-218)."""
         self._sync_device()
         cfg = self.config
         L, d = cfg.num_layers, cfg.d_model
-        res = self._survivors(inputs)
+        res = self.forward_with_survivors(inputs)
         if res is not None:
-            layers, T, surv = res
-            full = self._expand_layers(layers, surv)
-            src_mask = 0
-            for l in layers:
-                src_mask |= 1 << l
-            skip = (self.decoder_module.skip_all_targets(inputs, src_mask, T) if cfg.skip_connection else None)
-            targets = [t for t in range(L) if t in inputs]
-            out = self.decoder_module.decode_survivors(full, src_mask, min(targets), max(targets) + 1, skip_add=skip,
-                                                       ws=self._workspace())
-            return {t: out[t] for t in targets}
+            return res[0]
         # fallback wiring over dense activations
         acts = self.get_feature_activations(inputs)
         recs: Dict[int, torch.Tensor] = {}

@@ -302,6 +302,57 @@ def encode_threshold(x: torch.Tensor, w: torch.Tensor, b: Optional[torch.Tensor]
     return SurvivorList(row_ptr, col[:total], val[:total], T, F, L, x.dtype)
 
 
+# ---- evaluation reductions ------------------------------------------------------------------------------
+def survivor_metrics(surv: SurvivorList, fired_eps: float = 1e-6):
+    """(entries != 0 per layer, int64 [L]; tokens with value > fired_eps per (layer, feature),
+    int32 [L, F]) straight from the survivor list (evaluator.py:194-244, 350-405)."""
+    nat.require_device(surv.row_ptr, "survivor_metrics")
+    dev = surv.row_ptr.device
+    nonzero = torch.empty(surv.L, dtype=torch.int64, device=dev)
+    fired = torch.empty((surv.L, surv.F), dtype=torch.int32, device=dev)
+    empty = surv.nnz == 0
+    code = nat.load().clt_survivor_metrics(nat.ptr(surv.row_ptr), None if empty else nat.ptr(surv.col),
+                                           None if empty else nat.ptr(surv.val), surv.T, surv.F, surv.L,
+                                           nat.dtype_code(surv.dtype), fired_eps, nat.ptr(nonzero), nat.ptr(fired),
+                                           _stream(surv.row_ptr))
+    nat.check(code, "clt_survivor_metrics")
+    return nonzero, fired
+
+
+def dead_feature_update(fired: torch.Tensor, passes_since_fired: torch.Tensor) -> None:
+    """In place: counters of features that fired go to 0, the others go up by one (trainer.py:711-712)."""
+    nat.require_device(fired, "dead_feature_update")
+    assert fired.dtype == torch.int32 and passes_since_fired.dtype == torch.int64
+    assert fired.is_contiguous() and passes_since_fired.is_contiguous() and fired.numel() == passes_since_fired.numel()
+    code = nat.load().clt_dead_feature_update(nat.ptr(fired), nat.ptr(passes_since_fired), fired.numel(), _stream(fired))
+    nat.check(code, "clt_dead_feature_update")
+
+
+DENORM_MODES = {"none": 0, "mean_std": 1, "sqrt_d_model": 2}
+
+
+def reconstruction_stats(rec: torch.Tensor, target: torch.Tensor, mode: str = "none",
+                         mean: Optional[torch.Tensor] = None, std: Optional[torch.Tensor] = None,
+                         scale: float = 1.0, ws: Optional[Workspace] = None) -> torch.Tensor:
+    """float64 [L, 3]: MSE, mean column variance of the target, mean column variance of the error,
+    after de-normalising rec and target [L, T, d] in their dtype (evaluator.py:246-345)."""
+    nat.require_device(rec, "reconstruction_stats")
+    L, T, d = rec.shape
+    assert target.shape == rec.shape and target.dtype == rec.dtype and rec.is_contiguous() and target.is_contiguous()
+    if mode == "mean_std":
+        assert mean is not None and std is not None and mean.shape == (L, d) and std.shape == (L, d)
+        mean, std = mean.to(rec.dtype).contiguous(), std.to(rec.dtype).contiguous()
+    stats = torch.empty((L, 3), dtype=torch.float64, device=rec.device)
+    lib = nat.load()
+    wbuf = (ws or Workspace(rec.device)).get("recon_stats", lib.clt_reconstruction_stats_workspace_bytes(d, L))
+    code = lib.clt_reconstruction_stats(nat.ptr(rec), nat.ptr(target), T, d, L, nat.dtype_code(rec.dtype),
+                                        DENORM_MODES[mode], nat.ptr(mean) if mode == "mean_std" else None,
+                                        nat.ptr(std) if mode == "mean_std" else None, float(scale), nat.ptr(stats),
+                                        nat.ptr(wbuf), wbuf.numel(), _stream(rec))
+    nat.check(code, "clt_reconstruction_stats")
+    return stats
+
+
 # ---- backward pass (MSE reconstruction loss) ---------------------------------------------------------
 def mse_loss_grad(rec: torch.Tensor, target: torch.Tensor, ws: Optional[Workspace] = None):
     """(loss per layer [L] fp32, g [L, T, d] fp32 = d loss / d rec, the same in the model dtype,

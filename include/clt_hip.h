@@ -55,6 +55,11 @@ extern "C" {
 #define CLT_PRED_GT_ZERO 1  /* x > 0                        (ReLU)     */
 #define CLT_PRED_NONZERO 2  /* x != 0                       (compaction of a dense tensor) */
 
+/* de-normalisation applied by clt_reconstruction_stats (reference clt/training/evaluator.py:279-292) */
+#define CLT_DENORM_NONE 0
+#define CLT_DENORM_MEAN_STD 1 /* x * std[layer][column] + mean[layer][column] */
+#define CLT_DENORM_SCALE 2    /* x / scale   (scale = sqrt(d_model)) */
+
 /* Library version (major*10000 + minor*100 + patch). */
 int clt_version(void);
 
@@ -364,6 +369,36 @@ int clt_adam_step(void *param, const float *grad, float *m, float *v, int64_t n,
 int clt_adam_step_decoder(void *w_ref, void *w_packed, const float *grad_packed, float *m, float *v,
                           int64_t d, int64_t F, double lr, double beta1, double beta2, double eps,
                           int64_t step, int dtype, void *stream);
+
+/* ---- evaluation reductions ---------------------------------------------------
+ * clt_survivor_metrics: from a survivor list, per layer the number of entries whose value is
+ *   != 0 (nonzero_per_layer [L]; divided by T it is the layer's mean L0 of
+ *   CLTEvaluator._compute_sparsity, clt/training/evaluator.py:194-244) and per (layer, feature)
+ *   the number of tokens whose value is > fired_eps (fired_count [L][F]; the reference's
+ *   `act_bool.sum(dim=0)` of _compute_feature_density, evaluator.py:350-405, which uses 1e-6,
+ *   and the `fired_mask_per_token.any(dim=0)` of the trainer's dead-feature update,
+ *   clt/training/trainer.py:701-707).  Both outputs are cleared by the call.  col / val may be
+ *   NULL for an empty list.
+ * clt_dead_feature_update: passes_since_fired[i] = fired_count[i] ? 0 : passes_since_fired[i] + 1
+ *   over n = L*F counters (int64, the dtype of Trainer.n_forward_passes_since_fired,
+ *   trainer.py:342-347, 711-712).
+ * clt_reconstruction_stats: for rec, target [L][T][d] in the model dtype, per layer
+ *   stats[l] = { MSE, mean over columns of the population variance of the target, the same of
+ *   (target - rec) }, after de-normalising both in the model dtype (mean / std [L][d] in the model
+ *   dtype for CLT_DENORM_MEAN_STD); the quantities CLTEvaluator._compute_reconstruction_metrics
+ *   (evaluator.py:246-345) turns into explained variance and normalised MSE.
+ *   workspace: clt_reconstruction_stats_workspace_bytes(d, L), 8-byte aligned.
+ */
+int clt_survivor_metrics(const int32_t *row_ptr, const int32_t *col, const void *val, int64_t T,
+                         int64_t F, int64_t L, int dtype, float fired_eps,
+                         uint64_t *nonzero_per_layer, uint32_t *fired_count, void *stream);
+int clt_dead_feature_update(const uint32_t *fired_count, int64_t *passes_since_fired, int64_t n,
+                            void *stream);
+size_t clt_reconstruction_stats_workspace_bytes(int64_t d, int64_t L);
+int clt_reconstruction_stats(const void *rec, const void *target, int64_t T, int64_t d, int64_t L,
+                             int dtype, int denorm_mode, const void *mean, const void *stdv,
+                             double scale, double *stats, void *workspace, size_t workspace_bytes,
+                             void *stream);
 
 #ifdef __cplusplus
 }

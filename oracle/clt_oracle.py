@@ -34,6 +34,11 @@ How each function is pinned (see ``tests/test_oracle_*.py``):
 * ``mse_loss_and_gradients``  - torch autograd itself computes the gradients; a central
   finite-difference check in float64 on a tiny model pins the loss / gradient pairing, and the
   reference's backward tables (test_activations.py:114-152: grad * mask) pin the gate.
+* ``sparsity_metrics`` / ``feature_density_metrics`` / ``reconstruction_metrics`` /
+  ``dead_feature_update``  - hand-computed small cases, numpy's ``var`` in float64, and the
+  closed forms (a perfect reconstruction has explained variance 1 and NMSE 0; an all-zero
+  reconstruction of a zero-mean target has NMSE 1); the reference has no test of its evaluator:
+  PARITY UNPINNED beyond that.
 * ``forward``  - composition of the above; the reference has no golden tensors
   for a full forward: PARITY UNPINNED beyond shape/keys and the pins of its parts.
 
@@ -546,6 +551,94 @@ def mse_loss_and_gradients(inputs: Dict[int, torch.Tensor], targets: Dict[int, t
         loss = loss + F.mse_loss(rec, targets[t].float())
     loss.backward()
     return loss.detach(), {name: p.grad for name, p in params.items()}
+
+
+# ---------------------------------------------------------------------------
+# evaluation reductions
+# ---------------------------------------------------------------------------
+
+def sparsity_metrics(acts: Dict[int, torch.Tensor], num_features: int, num_layers: int) -> Dict[str, object]:
+    """L0 per layer and its aggregates (reference clt/training/evaluator.py:194-244)."""
+    if not acts or not any(v.numel() > 0 for v in acts.values()):
+        return {"sparsity/total_l0": 0.0, "sparsity/avg_l0": 0.0, "sparsity/sparsity_fraction": 1.0,
+                "layerwise/l0": {f"layer_{i}": 0.0 for i in range(num_layers)}}
+    per_layer, total, valid = {}, 0.0, 0
+    for l, a in acts.items():
+        if a.numel() == 0 or a.shape[0] == 0:
+            per_layer[f"layer_{l}"] = 0.0
+            continue
+        v = (a != 0).float().sum(dim=-1).mean().item()
+        per_layer[f"layer_{l}"] = v
+        total += v
+        valid += 1
+    avg = total / valid if valid > 0 else 0.0
+    frac = 1.0 - (avg / num_features) if num_features > 0 else 1.0
+    return {"sparsity/total_l0": total, "sparsity/avg_l0": avg, "sparsity/sparsity_fraction": max(0.0, min(1.0, frac)),
+            "layerwise/l0": per_layer}
+
+
+def feature_density_metrics(acts: Dict[int, torch.Tensor]) -> Dict[str, object]:
+    """log10 firing density and the activation-count heuristic per feature
+    (reference clt/training/evaluator.py:350-405, _log_density :71-74)."""
+    if not acts or not any(v.numel() > 0 for v in acts.values()):
+        return {"layerwise/log_feature_density": {}, "layerwise/consistent_activation_heuristic": {}}
+    dens, heur = {}, {}
+    for l, a in acts.items():
+        if a.numel() == 0 or a.shape[0] == 0:
+            continue
+        fired = (a > 1e-6).float()
+        dens[f"layer_{l}"] = torch.log10(fired.mean(dim=0) + 1e-10).tolist()
+        heur[f"layer_{l}"] = (fired.sum(dim=0) / (fired.any(dim=0).float() + 1e-9)).tolist()
+    return {"layerwise/log_feature_density": dens, "layerwise/consistent_activation_heuristic": heur}
+
+
+def dead_feature_update(passes_since_fired: torch.Tensor, acts: Dict[int, torch.Tensor]) -> torch.Tensor:
+    """New value of the per-feature counters after one batch (reference clt/training/trainer.py:693-712)."""
+    n = passes_since_fired.clone()
+    for l, a in acts.items():
+        if l < n.shape[0] and a.numel() > 0:
+            fired = (a > 1e-6).any(dim=0)
+            if fired.shape[0] == n.shape[1]:
+                n[l] += 1
+                n[l][fired] = 0
+    return n
+
+
+def reconstruction_metrics(targets: Dict[int, torch.Tensor], recs: Dict[int, torch.Tensor], *, method: str = "none",
+                           mean_tg: Optional[Dict[int, torch.Tensor]] = None,
+                           std_tg: Optional[Dict[int, torch.Tensor]] = None,
+                           d_model: Optional[int] = None) -> Dict[str, object]:
+    """Explained variance and normalised MSE (reference clt/training/evaluator.py:246-345)."""
+    mean_tg, std_tg = mean_tg or {}, std_tg or {}
+    tot_ev, tot_nmse, n = 0.0, 0.0, 0
+    lw_nmse, lw_ev = {}, {}
+    for l, tgt in targets.items():
+        if l not in recs:
+            continue
+        rec = recs[l]
+        if method == "mean_std" and l in mean_tg and l in std_tg:
+            mean, std = mean_tg[l].to(rec.dtype), std_tg[l].to(rec.dtype)
+            tgt, rec = tgt * std + mean, rec * std + mean
+        elif method == "sqrt_d_model" and d_model is not None:
+            tgt, rec = tgt / (d_model ** 0.5), rec / (d_model ** 0.5)
+        tf = tgt.reshape(-1, tgt.shape[-1]).float()
+        rf = rec.reshape(-1, rec.shape[-1]).float()
+        if tf.shape != rf.shape or tf.numel() == 0:
+            continue
+        mse = F.mse_loss(rf, tf, reduction="mean").item()
+        tvar = torch.var(tf, dim=0, unbiased=False).mean().item()
+        evar = torch.var(tf - rf, dim=0, unbiased=False).mean().item()
+        ev = (1.0 - evar / tvar) if tvar > 1e-9 else (1.0 if evar < 1e-9 else 0.0)
+        nmse = (mse / tvar) if tvar > 1e-9 else (0.0 if mse < 1e-9 else float("inf"))
+        tot_ev += ev
+        tot_nmse += nmse
+        lw_nmse[f"layer_{l}"] = nmse
+        lw_ev[f"layer_{l}"] = ev
+        n += 1
+    avg_ev = tot_ev / n if n > 0 else 0.0
+    return {"reconstruction/explained_variance": max(0.0, min(1.0, avg_ev)),
+            "reconstruction/normalized_mean_reconstruction_error": tot_nmse / n if n > 0 else 0.0,
+            "layerwise/normalized_mse": lw_nmse, "layerwise/explained_variance": lw_ev}
 
 
 # ---------------------------------------------------------------------------

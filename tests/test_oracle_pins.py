@@ -305,3 +305,69 @@ def test_mse_gradients_match_finite_differences():
         arr[idx] = old
         fd = (up - dn) / (2 * eps)
         assert abs(fd - float(grads[name][idx])) <= 1e-4 * max(1.0, abs(fd)), (name, fd, float(grads[name][idx]))
+
+
+def test_evaluator_reductions_hand_computed():
+    # layer 0: 3 tokens x 4 features; layer 1 the same shape, one feature never fires
+    a0 = torch.tensor([[0.0, 2.0, -1.0, 0.0], [1e-7, 0.0, 3.0, 0.0], [0.0, 0.0, 0.5, 0.0]])
+    a1 = torch.tensor([[1.0, 1.0, 0.0, 0.0], [1.0, 0.0, 0.0, 0.0], [1.0, 0.0, 0.0, 0.0]])
+    sp = orc.sparsity_metrics({0: a0, 1: a1}, num_features=4, num_layers=2)
+    # non-zeros per token: layer 0 -> 2, 2, 1 (the 1e-7 and the negative count); layer 1 -> 2, 1, 1
+    assert sp["layerwise/l0"]["layer_0"] == pytest.approx(5 / 3)
+    assert sp["layerwise/l0"]["layer_1"] == pytest.approx(4 / 3)
+    assert sp["sparsity/total_l0"] == pytest.approx(3.0)
+    assert sp["sparsity/avg_l0"] == pytest.approx(1.5)
+    assert sp["sparsity/sparsity_fraction"] == pytest.approx(1 - 1.5 / 4)
+    fd = orc.feature_density_metrics({0: a0, 1: a1})
+    # firing (> 1e-6): layer 0 feature counts 0, 1, 2, 0 (1e-7 and -1 do not fire)
+    want = [math.log10(c / 3 + 1e-10) for c in (0, 1, 2, 0)]
+    assert fd["layerwise/log_feature_density"]["layer_0"] == pytest.approx(want, rel=1e-6)
+    assert fd["layerwise/consistent_activation_heuristic"]["layer_0"] == pytest.approx([0, 1, 2, 0])
+    assert fd["layerwise/consistent_activation_heuristic"]["layer_1"] == pytest.approx([3, 1, 0, 0])
+    n = torch.tensor([[5, 5, 5, 5], [0, 2, 7, 1]])
+    got = orc.dead_feature_update(n, {0: a0, 1: a1})
+    assert got.tolist() == [[6, 0, 0, 6], [0, 0, 8, 2]]
+    # a layer that is absent keeps its counters
+    assert orc.dead_feature_update(n, {1: a1}).tolist() == [[5, 5, 5, 5], [0, 0, 8, 2]]
+    empty = orc.sparsity_metrics({}, 4, 2)
+    assert empty["sparsity/sparsity_fraction"] == 1.0 and empty["layerwise/l0"] == {"layer_0": 0.0, "layer_1": 0.0}
+
+
+def test_reconstruction_metrics_closed_forms_and_numpy():
+    g = torch.Generator().manual_seed(3)
+    tgt = {0: torch.randn(50, 6, generator=g) * 2 + 1, 1: torch.randn(50, 6, generator=g)}
+    rec = {l: t + 0.3 * torch.randn(50, 6, generator=g) for l, t in tgt.items()}
+    # perfect reconstruction: EV 1, NMSE 0
+    m = orc.reconstruction_metrics(tgt, tgt)
+    assert m["reconstruction/explained_variance"] == pytest.approx(1.0)
+    assert m["reconstruction/normalized_mean_reconstruction_error"] == pytest.approx(0.0)
+    # numpy float64: per-column population variances
+    m = orc.reconstruction_metrics(tgt, rec)
+    for l in (0, 1):
+        t, r = tgt[l].double().numpy(), rec[l].double().numpy()
+        tvar, evar = np.var(t, axis=0).mean(), np.var(t - r, axis=0).mean()
+        assert m["layerwise/explained_variance"][f"layer_{l}"] == pytest.approx(1 - evar / tvar, rel=1e-5)
+        assert m["layerwise/normalized_mse"][f"layer_{l}"] == pytest.approx(((t - r) ** 2).mean() / tvar, rel=1e-5)
+    # an all-zero reconstruction of a centred target: MSE equals the variance, NMSE 1, EV 0
+    c = {0: tgt[1] - tgt[1].mean(dim=0, keepdim=True)}
+    z = orc.reconstruction_metrics(c, {0: torch.zeros_like(c[0])})
+    assert z["layerwise/normalized_mse"]["layer_0"] == pytest.approx(1.0, rel=1e-5)
+    assert z["layerwise/explained_variance"]["layer_0"] == pytest.approx(0.0, abs=1e-6)
+    # de-normalisation with per-column std changes the weighting of the columns: numpy on x * std + mean
+    mean = {0: torch.arange(6.0), 1: torch.zeros(6)}
+    std = {0: torch.tensor([1.0, 2.0, 3.0, 0.5, 0.25, 4.0]), 1: torch.ones(6)}
+    m = orc.reconstruction_metrics(tgt, rec, method="mean_std", mean_tg=mean, std_tg=std)
+    t = (tgt[0] * std[0] + mean[0]).double().numpy()
+    r = (rec[0] * std[0] + mean[0]).double().numpy()
+    assert m["layerwise/explained_variance"]["layer_0"] == pytest.approx(
+        1 - np.var(t - r, axis=0).mean() / np.var(t, axis=0).mean(), rel=1e-5)
+    # sqrt(d_model) scaling leaves the ratios alone
+    s = orc.reconstruction_metrics(tgt, rec, method="sqrt_d_model", d_model=6)
+    base = orc.reconstruction_metrics(tgt, rec)
+    assert s["reconstruction/explained_variance"] == pytest.approx(base["reconstruction/explained_variance"], rel=1e-5)
+    # constant target, reconstruction off by a constant: both variances 0 -> EV 1, NMSE inf; an error
+    # that varies -> EV 0 (the reference's branches, evaluator.py:309-325)
+    k = orc.reconstruction_metrics({0: torch.ones(4, 2)}, {0: torch.zeros(4, 2)})
+    assert k["layerwise/explained_variance"]["layer_0"] == 1.0 and math.isinf(k["layerwise/normalized_mse"]["layer_0"])
+    k = orc.reconstruction_metrics({0: torch.ones(4, 2)}, {0: torch.arange(8.0).view(4, 2)})
+    assert k["layerwise/explained_variance"]["layer_0"] == 0.0 and math.isinf(k["layerwise/normalized_mse"]["layer_0"])
