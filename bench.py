@@ -250,6 +250,75 @@ def run_theta(args):
     }
 
 
+def run_evaluator(args):
+    """The evaluator's reductions (reference clt/training/evaluator.py:194-405, trainer.py:693-712) on one
+    batch whose forward has already run: L0 and per-feature firing counts from the survivor list, the
+    dead-feature counter update, reconstruction statistics.  One step = the reductions of one batch; the
+    same quantities from dense [T, F] activations with torch ops on the GPU are timed beside it."""
+    import crosslayer_coding_amd as cca
+    from crosslayer_coding_amd import engine, synth
+
+    wl = synth.WORKLOADS[args.workload]
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    cca._native.load(build_if_missing=False)
+    model, inputs, _ = synth.build_model(wl, dev)
+    model.eval()
+    g = torch.Generator(device=dev).manual_seed(99)
+    L, T, F, d = wl.num_layers, wl.tokens, wl.num_features, wl.d_model
+    tgt = torch.randn(L, T, d, generator=g, device=dev).to(model.dtype)
+    recs, surv = model.forward_with_survivors(inputs)
+    rec = torch.stack([recs[l] for l in range(L)]).contiguous()
+    tracker = cca.DeadFeatureTracker(L, F, 1000, dev)
+    ws = engine.Workspace(dev)
+
+    def one():
+        nonzero, fired = engine.survivor_metrics(surv)
+        tracker.update(surv, fired)
+        return nonzero, fired, engine.reconstruction_stats(rec, tgt, ws=ws)
+
+    def timed(fn, n):
+        for _ in range(args.warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / n
+
+    sec = timed(one, args.steps)
+    dense = model.get_feature_activations(inputs)
+    counter = torch.zeros(L, F, dtype=torch.long, device=dev)
+
+    def dense_scan():
+        for l, a in dense.items():
+            (a != 0).float().sum(dim=-1).mean()
+            fired = (a > 1e-6).float()
+            fired.mean(dim=0); fired.sum(dim=0)
+            hit = fired.any(dim=0)
+            counter[l] += 1
+            counter[l][hit] = 0
+            t, r = tgt[l].float(), rec[l].float()
+            torch.nn.functional.mse_loss(r, t); torch.var(t, dim=0, unbiased=False).mean()
+            torch.var(t - r, dim=0, unbiased=False).mean()
+
+    dense_sec = timed(dense_scan, max(1, args.steps // 4))
+    esz = 2 if wl.dtype == "bfloat16" else 4
+    list_bytes = surv.nnz * (4 + esz) + (L * T + 1) * 4 + L * F * (4 + 4 + 8 + 8) + 2 * L * T * d * esz
+    return {
+        "metric": "evaluator reductions tokens/sec (L0, firing counts, dead-feature counters, reconstruction statistics)",
+        "value": T / sec, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": sec * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if wl.dtype == "bfloat16" else "f32", "data": "synthetic",
+        "config": {"workload": f"{wl.name}: evaluator reductions, L={L} d_model={d} F={F} T={T} k={wl.k}"},
+        "roofline": {"bound": "hbm", "achieved": list_bytes / sec / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": list_bytes / sec / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                     "note": "bytes = survivor list + counters + reconstructions and targets, all launches of a step"},
+        "dense_torch_ms": dense_sec * 1e3,
+    }
+
+
 def run_backward(args):
     """Forward, MSE reconstruction loss and the gradients of every encoder / decoder parameter
     (CrossLayerTranscoder.loss_and_gradients); one step = one batch.  No optimizer step."""
@@ -342,6 +411,8 @@ def main():
                          "selection, per-feature minimum) instead of the forward")
     ap.add_argument("--backward", action="store_true",
                     help="time forward + MSE loss + all gradients (loss_and_gradients) instead of the forward")
+    ap.add_argument("--evaluator", action="store_true",
+                    help="time the evaluator's reductions on the survivor list of one batch")
     ap.add_argument("--train-step", action="store_true",
                     help="time full optimisation steps: forward, MSE loss, gradients, Adam update")
     ap.add_argument("--copy-probe", action="store_true",
@@ -354,7 +425,7 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a ROCm GPU", file=sys.stderr)
         sys.exit(2)
-    print(json.dumps(run_theta(args) if args.theta_estimation else run_backward(args) if (args.backward or args.train_step) else run_gpu(args)))
+    print(json.dumps(run_theta(args) if args.theta_estimation else run_evaluator(args) if args.evaluator else run_backward(args) if (args.backward or args.train_step) else run_gpu(args)))
 
 
 if __name__ == "__main__":

@@ -17,25 +17,34 @@ __global__ void k_metrics_zero(uint32_t *fired, int64_t n, unsigned long long *n
     for (int i = threadIdx.x; i < L; i += blockDim.x) nonzero[i] = 0ull;
 }
 
-// one wavefront per (layer, token) row of the survivor list
+// Each wavefront takes a run of consecutive (layer, token) rows, so its non-zero count goes to the
+// layer's counter once per run (a same-address atomic per row would serialise the whole grid).
 template <typename T>
 __global__ __launch_bounds__(MT_THREADS) void k_survivor_metrics(const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ col,
                                                                  const T *__restrict__ val, int64_t Tn, int64_t F, int64_t L,
                                                                  float eps, unsigned long long *nonzero, uint32_t *fired) {
-  const int lane = lane_id(), wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
-  const int64_t R = L * Tn;
-  for (int64_t r = (int64_t)blockIdx.x * nwv + wv; r < R; r += (int64_t)gridDim.x * nwv) {
+  const int lane = lane_id(), nwv = blockDim.x >> 6;
+  const int64_t R = L * Tn, nwave = (int64_t)gridDim.x * nwv, w = (int64_t)blockIdx.x * nwv + (threadIdx.x >> 6);
+  const int64_t per = (R + nwave - 1) / nwave, r0 = w * per, r1 = r0 + per < R ? r0 + per : R;
+  uint32_t nz = 0;
+  int64_t cur = r0 < R ? r0 / Tn : 0;
+  auto flush = [&](int64_t layer) {
+    uint32_t tot = nz;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) tot += __shfl_xor(tot, o);
+    if (lane == 0 && tot) atomicAdd(&nonzero[layer], (unsigned long long)tot);
+    nz = 0;
+  };
+  for (int64_t r = r0; r < r1; ++r) {
     const int64_t l = r / Tn;
-    uint32_t nz = 0;
+    if (l != cur) { flush(cur); cur = l; }
     for (int32_t j = row_ptr[r] + lane; j < row_ptr[r + 1]; j += 64) {
       const float v = Elem<T>::to_f32(val[j]);
       nz += v != 0.0f ? 1u : 0u;            // NaN counts, as `!= 0` does
       if (v > eps) atomicAdd(&fired[l * F + col[j]], 1u);
     }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) nz += __shfl_xor(nz, o);
-    if (lane == 0 && nz) atomicAdd(&nonzero[l], (unsigned long long)nz);
   }
+  if (r0 < r1) flush(cur);
 }
 
 __global__ void k_dead_update(const uint32_t *fired, int64_t *passes, int64_t n) {
