@@ -250,6 +250,67 @@ def run_theta(args):
     }
 
 
+def run_feed(args):
+    """Activation-store feed (reference clt/training/data/manifest_activation_store.py:776-958): one step =
+    one batch of T random rows drawn from 8 chunks of 8192 rows, gathered, normalised (mean / std) and cast
+    into the [L, T, d] input and target slabs.  Timed with the chunks resident in HBM (`value`), with the
+    chunks in pinned host memory read in place, and with slices arriving as wire-format bytes."""
+    import numpy as np
+    import crosslayer_coding_amd as cca
+    from crosslayer_coding_amd import synth
+
+    wl = synth.WORKLOADS[args.workload]
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    cca._native.load(build_if_missing=False)
+    L, T, d = wl.num_layers, wl.tokens, wl.d_model
+    dt = torch.bfloat16 if wl.dtype == "bfloat16" else torch.float32
+    n_chunks, rows = 8, 8192
+    g = torch.Generator().manual_seed(0)
+    stats = {str(l): {k: {"mean": torch.randn(d, generator=g).tolist(), "std": (torch.rand(d, generator=g) + 0.5).tolist()}
+                      for k in ("inputs", "targets")} for l in range(L)}
+    chunks = [torch.randn(L, 2, rows, d, generator=g).to(dt) for _ in range(n_chunks)]
+    rng = np.random.RandomState(1)
+    batches = [np.stack([rng.randint(0, n_chunks, T), rng.randint(0, rows, T)], axis=1).astype(np.uint32)
+               for _ in range(args.warmup + args.steps)]
+
+    def wire(chunk_id, sorted_rows):
+        return chunks[chunk_id][:, :, torch.as_tensor(sorted_rows.astype(np.int64)), :].contiguous().view(torch.uint8).numpy().tobytes()
+
+    def timed(where):
+        feed = cca.DeviceActivationFeed(L, d, dtype=dt, device=dev, normalization_method="mean_std", norm_stats=stats)
+        if where != "wire":
+            for c, t in enumerate(chunks):
+                feed.add_chunk(c, t, where=where)
+        fetch = wire if where == "wire" else None
+        for b in batches[:args.warmup]:
+            feed.parse_batch(b, fetch)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for b in batches[args.warmup:]:
+            feed.parse_batch(b, fetch)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / args.steps
+
+    sec = timed("device")
+    pinned = timed("pinned")
+    wire_sec = timed("wire")
+    esz = 2 if dt == torch.bfloat16 else 4
+    nbytes = 2 * L * T * d * (esz + esz)
+    return {
+        "metric": "activation-store feed tokens/sec (gather + mean/std normalisation + cast into the batch slabs)",
+        "value": T / sec, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": sec * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if dt == torch.bfloat16 else "f32", "data": "synthetic",
+        "config": {"workload": f"{wl.name}: store feed, L={L} d_model={d} T={T}, {n_chunks} resident chunks x {rows} rows"},
+        "roofline": {"bound": "hbm", "achieved": nbytes / sec / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": nbytes / sec / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                     "note": "bytes = rows read + rows written, inputs and targets of all layers; wall time of a step "
+                             "including the host-side grouping and 8 launches"},
+        "pinned_host_ms": pinned * 1e3, "wire_bytes_ms": wire_sec * 1e3,
+    }
+
+
 def run_evaluator(args):
     """The evaluator's reductions (reference clt/training/evaluator.py:194-405, trainer.py:693-712) on one
     batch whose forward has already run: L0 and per-feature firing counts from the survivor list, the
@@ -411,6 +472,8 @@ def main():
                          "selection, per-feature minimum) instead of the forward")
     ap.add_argument("--backward", action="store_true",
                     help="time forward + MSE loss + all gradients (loss_and_gradients) instead of the forward")
+    ap.add_argument("--feed", action="store_true",
+                    help="time the activation-store feed (gather + normalise + cast into the batch slabs)")
     ap.add_argument("--evaluator", action="store_true",
                     help="time the evaluator's reductions on the survivor list of one batch")
     ap.add_argument("--train-step", action="store_true",
@@ -425,7 +488,7 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a ROCm GPU", file=sys.stderr)
         sys.exit(2)
-    print(json.dumps(run_theta(args) if args.theta_estimation else run_evaluator(args) if args.evaluator else run_backward(args) if (args.backward or args.train_step) else run_gpu(args)))
+    print(json.dumps(run_theta(args) if args.theta_estimation else run_evaluator(args) if args.evaluator else run_feed(args) if args.feed else run_backward(args) if (args.backward or args.train_step) else run_gpu(args)))
 
 
 if __name__ == "__main__":

@@ -8,16 +8,17 @@ import it as ``crosslayer_coding_amd`` (the alias module next to this directory)
 """
 
 from . import _native, engine  # noqa: F401
-from . import activations, base, build, config, decoder, encoder, evaluator, optim, parallel, registry, synth, theta  # noqa: F401
+from . import activations, base, build, config, decoder, encoder, evaluator, feed, optim, parallel, registry, synth, theta  # noqa: F401
 from .activations import BatchTopK, JumpReLU, TokenTopK
 from .clt import CrossLayerTranscoder
 from .config import CLTConfig
 from .engine import SurvivorList
 from .optim import CLTAdam
 from .evaluator import CLTEvaluator, DeadFeatureTracker
+from .feed import DeviceActivationFeed
 from .registry import ACTIVATION_REGISTRY, get_activation_fn, register_activation_fn
 
 __all__ = [
-    "CrossLayerTranscoder", "CLTConfig", "CLTAdam", "CLTEvaluator", "DeadFeatureTracker", "BatchTopK", "TokenTopK", "JumpReLU", "SurvivorList",
+    "CrossLayerTranscoder", "CLTConfig", "CLTAdam", "CLTEvaluator", "DeadFeatureTracker", "DeviceActivationFeed", "BatchTopK", "TokenTopK", "JumpReLU", "SurvivorList",
     "ACTIVATION_REGISTRY", "get_activation_fn", "register_activation_fn",
 ]

@@ -16,7 +16,7 @@ import torch
 
 from . import build as _build
 
-CLT_F32, CLT_BF16 = 0, 1
+CLT_F32, CLT_BF16, CLT_F16 = 0, 1, 2
 TYING = {"none": 0, "per_source": 1, "per_target": 2}
 TOPK_PER_LAYER, TOPK_GLOBAL = 0, 1
 PRED_GE_THETA, PRED_GT_ZERO, PRED_NONZERO = 0, 1, 2
@@ -65,6 +65,8 @@ _SIGNATURES = {
     "clt_adam_step": (_int, [_vp, _vp, _vp, _vp, _i64, _f64, _f64, _f64, _f64, _i64, _int, _vp]),
     "clt_adam_step_decoder": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _f64, _f64, _f64, _f64, _i64, _int, _vp]),
     "clt_decoder_norms": (_int, [_vp, _vp, _i64, _i64, _i64, _int, _int, _vp]),
+    "clt_feed_gather": (_int, [_vp, _int, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _int, _vp, _vp, _vp, _vp, _f64, _vp, _vp,
+                              _i64, _i64, _int, _vp]),
     "clt_survivor_metrics": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _int, ctypes.c_float, _vp, _vp, _vp]),
     "clt_dead_feature_update": (_int, [_vp, _vp, _i64, _vp]),
     "clt_reconstruction_stats_workspace_bytes": (_sz, [_i64, _i64]),

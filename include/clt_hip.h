@@ -32,6 +32,7 @@ extern "C" {
 
 #define CLT_F32 0
 #define CLT_BF16 1
+#define CLT_F16 2 /* source dtype of clt_feed_gather only */
 
 #define CLT_OK 0
 #define CLT_ERR_ARG (-1)       /* null pointer, negative size, unsupported combination */
@@ -399,6 +400,32 @@ int clt_reconstruction_stats(const void *rec, const void *target, int64_t T, int
                              int dtype, int denorm_mode, const void *mean, const void *stdv,
                              double scale, double *stats, void *workspace, size_t workspace_bytes,
                              void *stream);
+
+/* ---- activation-store feed -----------------------------------------------------
+ * clt_feed_gather: rows of one stored chunk -> rows [out_row0, out_row0 + n) of the batch slabs
+ *   x_out, tgt_out [L][T][d] (out_dtype CLT_F32 / CLT_BF16), for all layers, inputs and targets.
+ *     out[l][out_row0 + j][:] = cast(norm(float(src_l[row_index[j]][:])))
+ *   src is the chunk (or a fetched slice of it) in the store's layout
+ *   Layer0_Inputs | Layer0_Targets | Layer1_Inputs | ... (ManifestActivationStore._fetch_slice,
+ *   clt/training/data/manifest_activation_store.py:555-560): [src_rows][d] elements of src_dtype
+ *   (CLT_F32 / CLT_BF16 / CLT_F16) per tensor, a layer's targets src_target_offset elements after
+ *   its inputs, layers src_layer_stride elements apart (the packed wire format has
+ *   src_target_offset = src_rows*d, src_layer_stride = 2*src_rows*d).  src may be device memory or
+ *   pinned (hipHostMalloc) host memory; anything else returns CLT_ERR_ARG.  row_index [n] int32
+ *   (device): for a fetched slice, the position of each batch row among the sorted rows that were
+ *   fetched (the `reorder_idx` of manifest_activation_store.py:868-872); for a resident chunk,
+ *   the row numbers themselves.  An index outside [0, src_rows) is not read: its row becomes NaN.
+ *   norm_mode: CLT_DENORM_NONE cast only; CLT_DENORM_MEAN_STD (x - mean) / std with mean / std
+ *   [L][d] fp32 per tensor kind (std already holds the store's + 1e-6; a NULL pair leaves that
+ *   kind as it is); CLT_DENORM_SCALE x * scale (scale = sqrt(d_model)).  fp32 arithmetic, one
+ *   rounding to out_dtype.  Replaces the parse / re-order / cat / normalise / cast tail of
+ *   ManifestActivationStore._fetch_and_parse_batch (manifest_activation_store.py:859-934).
+ */
+int clt_feed_gather(const void *src, int src_dtype, int64_t src_rows, int64_t src_layer_stride,
+                    int64_t src_target_offset, const int32_t *row_index, int64_t n, int64_t d,
+                    int64_t L, int norm_mode, const float *mean_in, const float *std_in,
+                    const float *mean_tg, const float *std_tg, double scale, void *x_out,
+                    void *tgt_out, int64_t out_row0, int64_t T, int out_dtype, void *stream);
 
 #ifdef __cplusplus
 }

@@ -39,6 +39,11 @@ How each function is pinned (see ``tests/test_oracle_*.py``):
   closed forms (a perfect reconstruction has explained variance 1 and NMSE 0; an all-zero
   reconstruction of a zero-mean target has NMSE 1); the reference has no test of its evaluator:
   PARITY UNPINNED beyond that.
+* ``store_parse_batch``  - a hand-written two-chunk case with every expected row spelled out, the
+  ordering property of the reference's own test (tests/unit/data/test_data_integrity.py:215-294:
+  every row once, identified by a value that encodes its position) and its normalisation test
+  (:137-213: statistics of the normalised batch, same generator and seed); the reference's store
+  tests need h5py files, which this image cannot write: PARITY UNPINNED beyond that.
 * ``forward``  - composition of the above; the reference has no golden tensors
   for a full forward: PARITY UNPINNED beyond shape/keys and the pins of its parts.
 
@@ -639,6 +644,52 @@ def reconstruction_metrics(targets: Dict[int, torch.Tensor], recs: Dict[int, tor
     return {"reconstruction/explained_variance": max(0.0, min(1.0, avg_ev)),
             "reconstruction/normalized_mean_reconstruction_error": tot_nmse / n if n > 0 else 0.0,
             "layerwise/normalized_mse": lw_nmse, "layerwise/explained_variance": lw_ev}
+
+
+# ---------------------------------------------------------------------------
+# activation-store batch assembly
+# ---------------------------------------------------------------------------
+
+def store_parse_batch(idxs: np.ndarray, fetch_slice, *, num_layers: int, d_model: int, dtype: torch.dtype,
+                      method: str = "none", mean_in=None, std_in=None, mean_tg=None, std_tg=None):
+    """Inputs and targets of one batch from (chunk, row) indices (reference
+    clt/training/data/manifest_activation_store.py:776-958, without the retry loop).
+    ``fetch_slice(chunk_id, sorted_rows)`` returns Layer0_Inputs | Layer0_Targets | Layer1_Inputs | ...
+    for the sorted rows; ``mean_*`` / ``std_*`` map layer -> fp32 [1, d] (std already + 1e-6)."""
+    mean_in, std_in, mean_tg, std_tg = mean_in or {}, std_in or {}, mean_tg or {}, std_tg or {}
+    itemsize = torch.finfo(dtype).bits // 8
+    bytes_per_row = d_model * itemsize
+    unique_chunks, inverse = np.unique(idxs[:, 0], return_inverse=True)
+    rows_by_chunk = {int(c): idxs[inverse == i, 1] for i, c in enumerate(unique_chunks)}
+    ins: Dict[int, List[torch.Tensor]] = {l: [] for l in range(num_layers)}
+    tgs: Dict[int, List[torch.Tensor]] = {l: [] for l in range(num_layers)}
+    for chunk_id, rows in rows_by_chunk.items():
+        sorted_rows = np.sort(rows)
+        raw = fetch_slice(chunk_id, sorted_rows)
+        assert len(raw) == len(sorted_rows) * bytes_per_row * 2 * num_layers
+        n = len(rows)
+        per_tensor = n * bytes_per_row
+        reorder = torch.as_tensor(np.searchsorted(sorted_rows, rows), dtype=torch.long)
+        for l in range(num_layers):
+            a = l * 2 * per_tensor
+            inp = torch.frombuffer(bytearray(raw[a:a + per_tensor]), dtype=dtype).reshape(n, d_model)
+            tgt = torch.frombuffer(bytearray(raw[a + per_tensor:a + 2 * per_tensor]), dtype=dtype).reshape(n, d_model)
+            ins[l].append(inp[reorder])
+            tgs[l].append(tgt[reorder])
+    inputs = {l: torch.cat(v) for l, v in ins.items()}
+    targets = {l: torch.cat(v) for l, v in tgs.items()}
+    if method in ("mean_std", "sqrt_d_model"):
+        for l in range(num_layers):
+            x, t = inputs[l].float(), targets[l].float()
+            if method == "mean_std":
+                if l in mean_in and l in std_in:
+                    x = (x - mean_in[l]) / std_in[l]
+                if l in mean_tg and l in std_tg:
+                    t = (t - mean_tg[l]) / std_tg[l]
+            else:
+                x, t = x * math.sqrt(d_model), t * math.sqrt(d_model)
+            inputs[l], targets[l] = x.to(dtype), t.to(dtype)
+    return inputs, targets
 
 
 # ---------------------------------------------------------------------------

@@ -5,6 +5,7 @@ import math
 
 import logging
 
+import numpy as np
 import pytest
 import torch
 
@@ -162,3 +163,59 @@ def test_convert_to_jumprelu_requires_estimation_first():
     tm = ThetaManager(cfg, None, torch.device("cpu"), torch.float32)
     with pytest.raises(RuntimeError, match="Required buffer .* not found"):
         tm.convert_to_jumprelu_inplace()
+
+
+def test_manifest_formats_and_fallback(tmp_path):
+    from crosslayer_coding_amd.feed import read_manifest
+    # legacy pairs (tests/unit/data/test_data_integrity.py:296-357 writes both formats)
+    legacy = np.array([(0, 0), (0, 1), (1, 0), (1, 1), (1, 2)], dtype=np.uint32)
+    p = tmp_path / "legacy.bin"
+    legacy.tofile(p)
+    assert np.array_equal(read_manifest(p), legacy)      # 40 bytes: not a multiple of 16
+    # 16-byte records expand to per-row entries, empty chunks are skipped
+    rec = np.array([(0, 2, 0), (1, 0, 2), (2, 3, 2)], dtype=[("chunk_id", np.int32), ("num_tokens", np.int32), ("offset", np.int64)])
+    p3 = tmp_path / "records.bin"
+    rec.tofile(p3)
+    want = np.array([(0, 0), (0, 1), (2, 0), (2, 1), (2, 2)], dtype=np.uint32)
+    assert np.array_equal(read_manifest(p3), want)
+    assert np.array_equal(read_manifest(p3, total_tokens=5), want)
+    # a legacy file whose size happens to be a multiple of 16: the token total tells the formats apart
+    even = np.array([(0, 0), (0, 1), (1, 0), (1, 1)], dtype=np.uint32)
+    pe = tmp_path / "even.bin"
+    even.tofile(pe)
+    assert np.array_equal(read_manifest(pe, total_tokens=4), even)
+    assert read_manifest(tmp_path / "absent.bin") is None
+    (tmp_path / "odd.bin").write_bytes(bytes(12))
+    assert read_manifest(tmp_path / "odd.bin") is None
+
+
+def test_normalisation_tables_follow_prep_norm():
+    from crosslayer_coding_amd.feed import prepare_normalization
+    good = {"0": {"inputs": {"mean": [1.0, 2.0], "std": [0.5, 0.0]}, "targets": {"mean": [0.0, 0.0], "std": [1.0, 1.0]}},
+            "1": {"inputs": {"mean": [3.0, 4.0], "std": [2.0, 2.0]}, "targets": {"mean": [1.0, 1.0], "std": [3.0, 3.0]}},
+            "7": {"inputs": {"mean": [0.0, 0.0], "std": [1.0, 1.0]}}}       # unknown layer: skipped
+    ok, mi, si, mt, st = prepare_normalization(good, [0, 1], 2)
+    assert ok and mi.tolist() == [[1.0, 2.0], [3.0, 4.0]]
+    assert torch.equal(si, torch.tensor([[0.5, 0.0], [2.0, 2.0]]) + 1e-6)
+    assert torch.equal(st, torch.tensor([[1.0, 1.0], [3.0, 3.0]]) + 1e-6) and mt.tolist() == [[0.0, 0.0], [1.0, 1.0]]
+    assert si[0, 1].item() == pytest.approx(1e-6)                           # std 0 survives thanks to the epsilon
+    for bad in (None, {}, {"0": good["0"]},                                  # nothing, or layer 1 missing
+                {"0": good["0"], "1": {"inputs": good["1"]["inputs"]}},      # no targets
+                {"0": good["0"], "1": {**good["1"], "targets": {"mean": [0.0, 0.0], "std": [-1.0, 1.0]}}}):
+        assert prepare_normalization(bad, [0, 1], 2)[0] is False
+
+
+def test_feed_rejects_bad_arguments_and_needs_a_gpu():
+    from crosslayer_coding_amd import DeviceActivationFeed
+    from crosslayer_coding_amd._native import CLTNativeError
+    with pytest.raises(ValueError):
+        DeviceActivationFeed(2, 8, normalization_method="bogus")
+    with pytest.raises(ValueError):
+        DeviceActivationFeed(2, 8, dtype="float64")
+    feed = DeviceActivationFeed(2, 8, dtype="float32", device="cpu", normalization_method="mean_std", norm_stats=None)
+    assert feed.apply_normalization is False
+    if not torch.cuda.is_available():
+        with pytest.raises(CLTNativeError):
+            feed.parse_batch(np.zeros((4, 2), dtype=np.uint32))
+    with pytest.raises(ValueError):
+        feed.add_chunk(0, torch.zeros(2, 2, 5, 7))

@@ -371,3 +371,86 @@ def test_reconstruction_metrics_closed_forms_and_numpy():
     assert k["layerwise/explained_variance"]["layer_0"] == 1.0 and math.isinf(k["layerwise/normalized_mse"]["layer_0"])
     k = orc.reconstruction_metrics({0: torch.ones(4, 2)}, {0: torch.arange(8.0).view(4, 2)})
     assert k["layerwise/explained_variance"]["layer_0"] == 0.0 and math.isinf(k["layerwise/normalized_mse"]["layer_0"])
+
+
+def _chunk_store(chunks, dtype):
+    """fetch_slice over in-memory chunks [L, 2, rows, d]: the wire bytes Layer0_Inputs | Layer0_Targets | ..."""
+    def fetch(chunk_id, sorted_rows):
+        sel = chunks[chunk_id][:, :, torch.as_tensor(np.asarray(sorted_rows, dtype=np.int64)), :].contiguous()
+        return sel.view(torch.uint8).numpy().tobytes() if dtype != torch.float32 else sel.numpy().tobytes()
+    return fetch
+
+
+def test_store_batch_assembly_hand_written():
+    # value = 1000*chunk + 100*layer + 50*is_target + row + col/4: every expected row can be written down
+    L, d, rows = 2, 2, 6
+    chunks = {}
+    for c in (0, 1):
+        t = torch.zeros(L, 2, rows, d)
+        for l in range(L):
+            for k in range(2):
+                for r in range(rows):
+                    for j in range(d):
+                        t[l, k, r, j] = 1000 * c + 100 * l + 50 * k + r + j / 4
+        chunks[c] = t
+    idxs = np.array([(1, 3), (0, 2), (1, 0), (0, 5)], dtype=np.uint32)
+    ins, tgs = orc.store_parse_batch(idxs, _chunk_store(chunks, torch.float32), num_layers=L, d_model=d, dtype=torch.float32)
+    # chunks in ascending order; inside a chunk the sampler's order: (0,2), (0,5), (1,3), (1,0)
+    assert ins[0].tolist() == [[2.0, 2.25], [5.0, 5.25], [1003.0, 1003.25], [1000.0, 1000.25]]
+    assert tgs[0].tolist() == [[52.0, 52.25], [55.0, 55.25], [1053.0, 1053.25], [1050.0, 1050.25]]
+    assert ins[1].tolist() == [[102.0, 102.25], [105.0, 105.25], [1103.0, 1103.25], [1100.0, 1100.25]]
+    assert tgs[1][:, 0].tolist() == [152.0, 155.0, 1153.0, 1150.0]
+    # normalisation by hand: (x - mean) / std in fp32, only where the layer has statistics; sqrt(d) scaling
+    mean_in, std_in = {0: torch.tensor([[1.0, 2.0]])}, {0: torch.tensor([[2.0, 4.0]])}
+    ins, tgs = orc.store_parse_batch(idxs, _chunk_store(chunks, torch.float32), num_layers=L, d_model=d, dtype=torch.float32,
+                                     method="mean_std", mean_in=mean_in, std_in=std_in)
+    assert ins[0][0].tolist() == [0.5, 0.0625]
+    assert ins[1][0].tolist() == [102.0, 102.25] and tgs[0][0].tolist() == [52.0, 52.25]
+    ins, _ = orc.store_parse_batch(idxs, _chunk_store(chunks, torch.float32), num_layers=L, d_model=d, dtype=torch.float32,
+                                   method="sqrt_d_model")
+    assert ins[0][1].tolist() == [float(np.float32(5.0) * np.float32(math.sqrt(2))), float(np.float32(5.25) * np.float32(math.sqrt(2)))]
+    # 16-bit store: arithmetic in fp32, one rounding at the end (here 3.0 / 7.0 -> nearest bfloat16)
+    c16 = {0: torch.full((1, 2, 2, 2), 3.0, dtype=torch.bfloat16)}
+    ins, _ = orc.store_parse_batch(np.array([(0, 1)], dtype=np.uint32), _chunk_store(c16, torch.bfloat16), num_layers=1, d_model=2,
+                                   dtype=torch.bfloat16, method="mean_std", mean_in={0: torch.zeros(1, 2)},
+                                   std_in={0: torch.full((1, 2), 7.0)})
+    assert ins[0].dtype == torch.bfloat16 and ins[0][0, 0].item() == torch.tensor(3.0 / 7.0).to(torch.bfloat16).item()
+
+
+def test_store_batch_properties_of_the_reference_tests():
+    # every row exactly once across sequential batches that span chunk boundaries
+    # (tests/unit/data/test_data_integrity.py:215-294: the first element encodes the global position)
+    L, d, per_chunk, n_chunks = 2, 4, 50, 3
+    chunks = {}
+    for c in range(n_chunks):
+        t = torch.zeros(L, 2, per_chunk, d)
+        for l in range(L):
+            t[l, 0, :, 0] = torch.arange(per_chunk) + c * per_chunk
+            t[l, 0, :, 1], t[l, 0, :, 2], t[l, 0, :, 3] = c, l, torch.arange(per_chunk)
+            t[l, 1] = t[l, 0] + 1000
+        chunks[c] = t
+    manifest = np.array([(c, i) for c in range(n_chunks) for i in range(per_chunk)], dtype=np.uint32)
+    seen = []
+    for b in range(0, len(manifest), 25):
+        ins, tgs = orc.store_parse_batch(manifest[b:b + 25], _chunk_store(chunks, torch.float32), num_layers=L, d_model=d,
+                                         dtype=torch.float32)
+        seen += ins[0][:, 0].tolist()
+        assert torch.equal(tgs[1], ins[1] + 1000) and bool((ins[1][:, 2] == 1).all())
+    assert seen == list(range(per_chunk * n_chunks))
+    # normalised batches have mean ~ 0 and std ~ 1 (test_data_integrity.py:137-213, same generator and seed)
+    d, n = 8, 1000
+    stats = {0: (10.0, 2.0), 1: (-5.0, 0.5)}
+    t = torch.zeros(2, 2, n, d)
+    for l, (mu, sd) in stats.items():
+        rng = np.random.RandomState(42)
+        t[l, 0] = torch.from_numpy(rng.normal(mu, sd, (n, d)).astype(np.float32))
+        t[l, 1] = torch.from_numpy(rng.normal(mu + 1, sd, (n, d)).astype(np.float32))
+    mean_in = {l: torch.full((1, d), mu) for l, (mu, sd) in stats.items()}
+    mean_tg = {l: torch.full((1, d), mu + 1) for l, (mu, sd) in stats.items()}
+    std = {l: torch.full((1, d), sd) + 1e-6 for l, (mu, sd) in stats.items()}
+    idxs = np.array([(0, i) for i in range(100)], dtype=np.uint32)
+    ins, tgs = orc.store_parse_batch(idxs, _chunk_store({0: t}, torch.float32), num_layers=2, d_model=d, dtype=torch.float32,
+                                     method="mean_std", mean_in=mean_in, std_in=std, mean_tg=mean_tg, std_tg=std)
+    for l in (0, 1):
+        for x in (ins[l], tgs[l]):
+            assert abs(x.mean().item()) < 0.1 and abs(x.std().item() - 1.0) < 0.1
