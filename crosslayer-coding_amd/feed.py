@@ -250,12 +250,11 @@ class DeviceActivationFeed:
         mode = NORM_MODES[self.normalization_method] if self.apply_normalization else 0
         tabs = [nat.ptr(t) if (t is not None and mode == 1) else None for t in self._tables]
         scale = math.sqrt(d) if mode == 2 else 1.0
+        # all row indices of the batch go up in one copy; each piece points into it
+        index_dev = torch.from_numpy(np.concatenate([p[1] for p in pieces])).to(self.device)
         out_row, at = 0, 0
-        keep = []
         for chunk, index, raw in pieces:
             n = int(index.shape[0])
-            index_dev = torch.from_numpy(index).to(self.device)
-            keep.append(index_dev)
             if chunk is not None:
                 src_ptr, src_rows = chunk.data.data_ptr(), chunk.rows
                 layer_stride, target_offset = chunk.layer_stride, chunk.target_offset
@@ -266,8 +265,8 @@ class DeviceActivationFeed:
                 layer_stride, target_offset = 2 * n * d, n * d
                 at += (len(raw) + 255) & ~255
             code = lib.clt_feed_gather(src_ptr, _SRC_CODES[self.dtype], src_rows, layer_stride, target_offset,
-                                       nat.ptr(index_dev), n, d, L, mode, *tabs, scale, nat.ptr(x), nat.ptr(tg),
-                                       out_row, N, nat.dtype_code(self.out_dtype), stream)
+                                       index_dev.data_ptr() + 4 * out_row, n, d, L, mode, *tabs, scale, nat.ptr(x),
+                                       nat.ptr(tg), out_row, N, nat.dtype_code(self.out_dtype), stream)
             nat.check(code, "clt_feed_gather")
             out_row += n
         if stage is not None:
