@@ -137,6 +137,18 @@ __device__ __forceinline__ void decode_chunk_pipelined(float *acc, const T *wbas
   }
 }
 
+// The partial rows are touched once per launch: streaming loads / stores keep them from pushing the
+// decoder slice out of the L2.
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float4 ldg_stream4(const float *p) {
+  const f32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const f32x4_t *>(p));
+  return make_float4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void stg_stream4(float *p, float4 v) {
+  f32x4_t q = {v.x, v.y, v.z, v.w};
+  __builtin_nontemporal_store(q, reinterpret_cast<f32x4_t *>(p));
+}
+
 constexpr int SLICED_NTOK = 4;   // tokens per wavefront in the sliced kernel
 
 // One wavefront per (target, token): walks all sources s <= t, accumulates in registers,
@@ -236,7 +248,7 @@ __global__ __launch_bounds__(256) void k_decode(
           const float *pp = prow + (int64_t)c * 64 * V + (int64_t)lane * V;
 #pragma unroll
           for (int j = 0; j < V; j += 4) {
-            float4 q = *reinterpret_cast<const float4 *>(pp + j);
+            float4 q = ldg_stream4(pp + j);
             old[c * V + j] = q.x; old[c * V + j + 1] = q.y; old[c * V + j + 2] = q.z; old[c * V + j + 3] = q.w;
           }
         }
@@ -267,8 +279,8 @@ __global__ __launch_bounds__(256) void k_decode(
         float *pp = prow + (int64_t)c * 64 * V + (int64_t)lane * V;
 #pragma unroll
         for (int j = 0; j < V; j += 4)
-          *reinterpret_cast<float4 *>(pp + j) = make_float4(old[c * V + j] + acc[c * V + j], old[c * V + j + 1] + acc[c * V + j + 1],
-                                                            old[c * V + j + 2] + acc[c * V + j + 2], old[c * V + j + 3] + acc[c * V + j + 3]);
+          stg_stream4(pp + j, make_float4(old[c * V + j] + acc[c * V + j], old[c * V + j + 1] + acc[c * V + j + 1],
+                                          old[c * V + j + 2] + acc[c * V + j + 2], old[c * V + j + 3] + acc[c * V + j + 3]));
       }
       if (TAIL == 1) {
 #pragma unroll

@@ -28,6 +28,8 @@ constexpr int BM = 256;   // tokens per block
 constexpr int BN = 256;   // features per block
 constexpr int ROWB = 128; // bytes of K per LDS row
 constexpr int STAGE = (BM + BN) * ROWB;  // bytes of one LDS stage
+constexpr int ENC_SN = 8;  // feature tiles x token tiles that one XCD works on at a time
+constexpr int ENC_SM = 4;
 
 
 template <typename T> struct Mma;
@@ -112,9 +114,8 @@ __device__ __forceinline__ uint32_t wave_inclusive_scan32(uint32_t v) {
 // computed twice and stored twice with identical values), so no load or store is predicated.
 //
 // Block -> tile map: workgroups go to the 8 XCDs round-robin, so block b runs on XCD b % 8.
-// When the feature tiles split evenly, XCD x takes the feature tiles n = x, x+8, ... and walks
-// all token tiles of one n before the next: a W tile is fetched by one XCD only and the x slab
-// of the layer stays in that XCD's L2.
+// When the feature tiles split evenly, XCD x takes the feature tiles n = x, x+8, ... in groups
+// (see the map below): a W tile is fetched by one XCD only.
 //
 // COLLECT 0 stores the tile.  COLLECT 1 / 2 store nothing: the epilogue compares every element
 // with the layer's cut value (1) or its feature's threshold (2) and appends the ones that reach
@@ -144,9 +145,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   if (COLLECT == 0 && gate && gate[layer].status != ST_RETRY) return;
   int tn, tm;
   if ((tiles_n & 7) == 0) {
-    const int xcd = bid & 7, idx = bid >> 3;
-    tm = idx % tiles_m;
-    tn = (idx / tiles_m) * 8 + xcd;
+    // XCD x owns the feature tiles n = x, x+8, ...  Its tiles run in groups of ENC_SN feature tiles
+    // x ENC_SM token tiles (about one tile per CU of the XCD): the group's W tiles stay in the L2
+    // while the token groups sweep past, so W is fetched once and the x slab once per ENC_SN tiles.
+    const int xcd = bid & 7, idx = bid >> 3, nloc = tiles_n >> 3;
+    const int g = idx / (ENC_SN * tiles_m), r = idx - g * ENC_SN * tiles_m;
+    const int cnt = (nloc - g * ENC_SN) < ENC_SN ? (nloc - g * ENC_SN) : ENC_SN;
+    const int mg = r / (cnt * ENC_SM), r2 = r - mg * cnt * ENC_SM;
+    tm = mg * ENC_SM + r2 / cnt;
+    tn = (g * ENC_SN + r2 % cnt) * 8 + xcd;
   } else {
     tn = bid / tiles_m; tm = bid - tn * tiles_m;
   }
