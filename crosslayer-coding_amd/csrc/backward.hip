@@ -335,24 +335,31 @@ __global__ __launch_bounds__(BW_THREADS) void k_csc_order(const int32_t *ptr, in
 //            out = dW[slot(s,t)][f]
 //   encoder: wavefront (s, f):         coef = dval, src = x[s], out = dW_enc[s][f], rowsum = db_enc[s][f]
 // Rows are read in raw 16-byte pieces, up to FO_NU rows in flight.
+// SPLIT 2: the source matrix of one layer ([T, d]) does not fit one XCD's L2, so the columns are
+// cut in two and the workgroups of even XCDs (block b runs on XCD b % 8) take the first half, those
+// of odd XCDs the second: each XCD then gathers from half a matrix, which does fit.
 constexpr int FO_NU = 8;
-template <typename T, typename CoefT, int NCH, bool DECODER>
+template <typename T, typename CoefT, int NCH, bool DECODER, int SPLIT>
 __global__ __launch_bounds__(BW_THREADS) void k_feature_outer(
     const int32_t *__restrict__ ptr, const int32_t *__restrict__ ltok, const int32_t *__restrict__ lsrc,
     const CoefT *__restrict__ coef, const T *__restrict__ src, float *__restrict__ out, float *__restrict__ rowsum,
-    int64_t Tn, int64_t d, int64_t F, int64_t L) {
+    int64_t Tn, int64_t d, int64_t F, int64_t L, int64_t target) {
   constexpr int EV = Piece<T>::EV;
   const int lane = lane_id(), wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
-  const int64_t per_layer_rows = DECODER ? F * L : F;   // (target, feature) pairs of a layer (targets < s are skipped)
-  const int64_t total = L * per_layer_rows;
+  // One launch per layer of the gathered matrix, so that every wavefront of a launch gathers from the
+  // same [T, d] matrix: DECODER launch `target` covers the (source <= target, feature) pairs and reads
+  // g[target]; the encoder launch `target` covers the features of that layer and reads x[target].
+  const int64_t total = DECODER ? (target + 1) * F : F;
+  const int half = SPLIT == 2 ? (int)(blockIdx.x & 1) : 0;
+  const int64_t vblock = SPLIT == 2 ? (int64_t)(blockIdx.x >> 3) * 4 + ((blockIdx.x & 7) >> 1) : (int64_t)blockIdx.x;
+  const int64_t nvblock = SPLIT == 2 ? (int64_t)gridDim.x / 2 : (int64_t)gridDim.x;
+  const int64_t pieces = d / EV, first_half = SPLIT == 2 ? (pieces + 1) / 2 : pieces;
+  const int64_t col0 = half ? first_half * EV : 0, my_pieces = half ? pieces - first_half : first_half;
   bool on[NCH];
 #pragma unroll
-  for (int c = 0; c < NCH; ++c) on[c] = (int64_t)c * 64 * EV + lane * EV < d;
-  for (int64_t w = (int64_t)blockIdx.x * nwv + wv; w < total; w += (int64_t)gridDim.x * nwv) {
-    const int64_t s = w / per_layer_rows, rem = w - s * per_layer_rows;
-    int64_t f, t;
-    if (DECODER) { t = rem / F; f = rem - t * F; if (t < s) continue; }
-    else { f = rem; t = s; }
+  for (int c = 0; c < NCH; ++c) on[c] = (int64_t)c * 64 + lane < my_pieces;
+  for (int64_t w = vblock * nwv + wv; w < total; w += nvblock * nwv) {
+    const int64_t s = DECODER ? w / F : target, f = DECODER ? w - s * F : w, t = target;
     const int64_t q = s * F + f;
     const int32_t b = ptr[q], e = ptr[q + 1];
     const T *sbase = src + (DECODER ? t : s) * Tn * d;
@@ -375,7 +382,7 @@ __global__ __launch_bounds__(BW_THREADS) void k_feature_outer(
           const T *row = sbase + (int64_t)__builtin_amdgcn_readlane(mt, idx) * d;
 #pragma unroll
           for (int c = 0; c < NCH; ++c)
-            v[u][c] = on[c] ? *reinterpret_cast<const uint4 *>(row + (int64_t)c * 64 * EV + lane * EV) : make_uint4(0, 0, 0, 0);
+            v[u][c] = on[c] ? *reinterpret_cast<const uint4 *>(row + col0 + (int64_t)c * 64 * EV + lane * EV) : make_uint4(0, 0, 0, 0);
         }
 #pragma unroll
         for (int u = 0; u < NU; ++u) {
@@ -398,11 +405,30 @@ __global__ __launch_bounds__(BW_THREADS) void k_feature_outer(
       if (on[c]) {
 #pragma unroll
         for (int k = 0; k < EV; k += 4)
-          *reinterpret_cast<float4 *>(orow + (int64_t)c * 64 * EV + lane * EV + k) =
+          *reinterpret_cast<float4 *>(orow + col0 + (int64_t)c * 64 * EV + lane * EV + k) =
               make_float4(acc[c][k], acc[c][k + 1], acc[c][k + 2], acc[c][k + 3]);
       }
-    if (!DECODER && rowsum && lane == 0) rowsum[q] = csum;
+    if (!DECODER && rowsum && lane == 0 && half == 0) rowsum[q] = csum;
   }
+}
+
+// one layer of the gathered matrix ([T, d]) against the 4 MB L2 of an XCD, with room for the other streams
+static bool bw_split_columns(int64_t T, int64_t d, int esz) { return T * d * esz > (3ll << 20) && d / (16 / esz) >= 2; }
+
+// Grid for the grid-stride weight-gradient kernels: exactly the workgroups that are resident at once,
+// so that all wavefronts walk the (source, target, feature) order together and the XCDs gather from
+// one layer of the source matrix at a time.  (With more workgroups than fit, the early ones run
+// through every layer before the late ones start and nothing stays in the L2.)
+template <typename K>
+static unsigned bw_resident_blocks(K kernel) {
+  int dev = 0, cus = 0, per_cu = 0;
+  if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+      hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, BW_THREADS, 0) != hipSuccess || cus <= 0 || per_cu <= 0) {
+    (void)hipGetLastError();
+    return 256 * 4;
+  }
+  unsigned nb = (unsigned)cus * (unsigned)per_cu;
+  return nb < 8 ? 8 : nb & ~7u;   // a multiple of the 8 XCDs
 }
 
 static bool bw_shape_ok(int64_t d, int dtype) { return d > 0 && d % (dtype == CLT_BF16 ? 8 : 4) == 0 && d <= 2048; }
@@ -513,9 +539,17 @@ extern "C" int clt_decoder_weight_grad(const int32_t *list_ptr, const int32_t *l
   if (T <= 0 || F <= 0 || L <= 0 || L > 64 || !list_ptr || !list_tok || !list_src || !val || !g_model || !dw_packed) return CLT_ERR_ARG;
   if (!bw_shape_ok(d, dtype)) return CLT_ERR_RANGE;
   hipStream_t s = (hipStream_t)stream;
-  const int nc4 = (int)clt_ceil_div(d, dtype == CLT_BF16 ? 512 : 256);   // 16-byte pieces per lane
-  const unsigned nb = 256 * 32;
-#define CLT_DW(CT, N) k_feature_outer<CT, CT, N, true><<<nb, BW_THREADS, 0, s>>>(list_ptr, list_tok, list_src, (const CT *)val, (const CT *)g_model, dw_packed, nullptr, T, d, F, L)
+  // split the columns over XCD pairs when one layer of g does not fit an XCD's L2
+  const int esz = dtype == CLT_BF16 ? 2 : 4, ev = 16 / esz;
+  const bool split = bw_split_columns(T, d, esz);
+  const int nc4 = (int)clt_ceil_div(split ? (d / ev + 1) / 2 : d / ev, 64);   // 16-byte pieces per lane
+#define CLT_DW(CT, N)                                                                                                      \
+  do {                                                                                                                     \
+    for (int64_t t = 0; t < L; ++t) {                                                                                      \
+      if (split) k_feature_outer<CT, CT, N, true, 2><<<bw_resident_blocks(k_feature_outer<CT, CT, N, true, 2>), BW_THREADS, 0, s>>>(list_ptr, list_tok, list_src, (const CT *)val, (const CT *)g_model, dw_packed, nullptr, T, d, F, L, t); \
+      else k_feature_outer<CT, CT, N, true, 1><<<bw_resident_blocks(k_feature_outer<CT, CT, N, true, 1>), BW_THREADS, 0, s>>>(list_ptr, list_tok, list_src, (const CT *)val, (const CT *)g_model, dw_packed, nullptr, T, d, F, L, t); \
+    }                                                                                                                      \
+  } while (0)
 #define CLT_DW_N(CT)                                                                       \
   do {                                                                                     \
     switch (nc4) {                                                                         \
@@ -537,9 +571,16 @@ extern "C" int clt_encoder_weight_grad(const int32_t *list_ptr, const int32_t *l
   if (T <= 0 || F <= 0 || L <= 0 || L > 65535 || !list_ptr || !list_tok || !list_src || !dval || !x || !dw_enc) return CLT_ERR_ARG;
   if (!bw_shape_ok(d, dtype)) return CLT_ERR_RANGE;
   hipStream_t s = (hipStream_t)stream;
-  const int nc4 = (int)clt_ceil_div(d, dtype == CLT_BF16 ? 512 : 256);   // 16-byte pieces per lane
-  const unsigned nb = 256 * 32;
-#define CLT_EW(ST, N) k_feature_outer<ST, float, N, false><<<nb, BW_THREADS, 0, s>>>(list_ptr, list_tok, list_src, dval, (const ST *)x, dw_enc, db_enc, T, d, F, L)
+  const int esz = dtype == CLT_BF16 ? 2 : 4, ev = 16 / esz;
+  const bool split = bw_split_columns(T, d, esz);
+  const int nc4 = (int)clt_ceil_div(split ? (d / ev + 1) / 2 : d / ev, 64);   // 16-byte pieces per lane
+#define CLT_EW(ST, N)                                                                                                      \
+  do {                                                                                                                     \
+    for (int64_t l = 0; l < L; ++l) {                                                                                      \
+      if (split) k_feature_outer<ST, float, N, false, 2><<<bw_resident_blocks(k_feature_outer<ST, float, N, false, 2>), BW_THREADS, 0, s>>>(list_ptr, list_tok, list_src, dval, (const ST *)x, dw_enc, db_enc, T, d, F, L, l); \
+      else k_feature_outer<ST, float, N, false, 1><<<bw_resident_blocks(k_feature_outer<ST, float, N, false, 1>), BW_THREADS, 0, s>>>(list_ptr, list_tok, list_src, dval, (const ST *)x, dw_enc, db_enc, T, d, F, L, l); \
+    }                                                                                                                      \
+  } while (0)
 #define CLT_EW_N(ST)                                                                       \
   do {                                                                                     \
     switch (nc4) {                                                                         \

@@ -10,10 +10,13 @@ namespace {
 
 struct AdamCoef { float b1, b2, step_size, inv_sqrt_bc2, eps; };
 
+// The sequence of roundings is spelled out with fmaf so that every kernel that inlines this produces
+// the same bits for the same inputs.
 __device__ __forceinline__ float adam_update(float p, float g, float &m, float &v, const AdamCoef &c) {
-  m = c.b1 * m + (1.0f - c.b1) * g;
-  v = c.b2 * v + (1.0f - c.b2) * g * g;
-  return p - c.step_size * m / (sqrtf(v) * c.inv_sqrt_bc2 + c.eps);
+  m = fmaf(c.b1, m, __fmul_rn(1.0f - c.b1, g));
+  v = fmaf(c.b2, v, __fmul_rn(__fmul_rn(1.0f - c.b2, g), g));
+  const float denom = fmaf(sqrtf(v), c.inv_sqrt_bc2, c.eps);
+  return fmaf(-c.step_size, __fdiv_rn(m, denom), p);
 }
 
 // parameter, gradient and moments in the same layout
@@ -53,6 +56,61 @@ __global__ __launch_bounds__(256) void k_adam_decoder(T *w_ref, T *w_packed, con
   }
 }
 
+// Vector version (d % 4 == 0, F % 4 == 0): a thread updates 4 consecutive elements of a feature row
+// (16-byte accesses to gradient and moments) and writes 4 consecutive features of a parameter row.
+template <typename T>
+__global__ __launch_bounds__(256) void k_adam_decoder_vec(T *w_ref, T *w_packed, const float *g, float *m, float *v,
+                                                          int64_t d, int64_t F, AdamCoef c) {
+  __shared__ T tile[64][68];
+  const int64_t f0 = (int64_t)blockIdx.x * 64, d0 = (int64_t)blockIdx.y * 64;
+  const int q = threadIdx.x & 15, r = threadIdx.x >> 4;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int fl = r + 16 * i;
+    const int64_t f = f0 + fl, dd = d0 + q * 4;
+    if (f < F && dd < d) {
+      const int64_t at = f * d + dd;
+      const float4 gv = *reinterpret_cast<const float4 *>(g + at);
+      float4 mv = *reinterpret_cast<const float4 *>(m + at), vv = *reinterpret_cast<const float4 *>(v + at);
+      float p[4];
+      if constexpr (sizeof(T) == 2) {
+        const uint2 raw = *reinterpret_cast<const uint2 *>(w_packed + at);
+        p[0] = bf16_bits_to_f32(raw.x & 0xFFFFu); p[1] = bf16_bits_to_f32(raw.x >> 16);
+        p[2] = bf16_bits_to_f32(raw.y & 0xFFFFu); p[3] = bf16_bits_to_f32(raw.y >> 16);
+      } else {
+        const float4 raw = *reinterpret_cast<const float4 *>(w_packed + at);
+        p[0] = raw.x; p[1] = raw.y; p[2] = raw.z; p[3] = raw.w;
+      }
+      p[0] = adam_update(p[0], gv.x, mv.x, vv.x, c); p[1] = adam_update(p[1], gv.y, mv.y, vv.y, c);
+      p[2] = adam_update(p[2], gv.z, mv.z, vv.z, c); p[3] = adam_update(p[3], gv.w, mv.w, vv.w, c);
+      *reinterpret_cast<float4 *>(m + at) = mv;
+      *reinterpret_cast<float4 *>(v + at) = vv;
+      T np[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) { np[k] = Elem<T>::from_f32(p[k]); tile[fl][q * 4 + k] = np[k]; }
+      if constexpr (sizeof(T) == 2)
+        *reinterpret_cast<uint2 *>(w_packed + at) = make_uint2((uint32_t)np[0] | ((uint32_t)np[1] << 16), (uint32_t)np[2] | ((uint32_t)np[3] << 16));
+      else
+        *reinterpret_cast<float4 *>(w_packed + at) = make_float4(np[0], np[1], np[2], np[3]);
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int dl = r + 16 * i;
+    const int64_t dd = d0 + dl, f = f0 + q * 4;
+    if (dd < d && f < F) {
+      T o[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) o[k] = tile[q * 4 + k][dl];
+      if constexpr (sizeof(T) == 2)
+        *reinterpret_cast<uint2 *>(w_ref + dd * F + f) = make_uint2((uint32_t)o[0] | ((uint32_t)o[1] << 16), (uint32_t)o[2] | ((uint32_t)o[3] << 16));
+      else
+        *reinterpret_cast<float4 *>(w_ref + dd * F + f) = make_float4(o[0], o[1], o[2], o[3]);
+    }
+  }
+}
+
 static AdamCoef adam_coef(double lr, double b1, double b2, double eps, int64_t step) {
   AdamCoef c;
   c.b1 = (float)b1; c.b2 = (float)b2; c.eps = (float)eps;
@@ -88,7 +146,14 @@ extern "C" int clt_adam_step_decoder(void *w_ref, void *w_packed, const float *g
   const AdamCoef c = adam_coef(lr, beta1, beta2, eps, step);
   hipStream_t s = (hipStream_t)stream;
   dim3 grid((unsigned)clt_ceil_div(F, 64), (unsigned)clt_ceil_div(d, 64));
-  if (dtype == CLT_BF16) k_adam_decoder<bf16_t><<<grid, 256, 0, s>>>((bf16_t *)w_ref, (bf16_t *)w_packed, grad_packed, m, v, d, F, c);
-  else k_adam_decoder<float><<<grid, 256, 0, s>>>((float *)w_ref, (float *)w_packed, grad_packed, m, v, d, F, c);
+  const bool vec = d % 4 == 0 && F % 4 == 0 && clt_aligned16(w_ref) && clt_aligned16(w_packed) && clt_aligned16(grad_packed) &&
+                   clt_aligned16(m) && clt_aligned16(v);
+  if (dtype == CLT_BF16) {
+    if (vec) k_adam_decoder_vec<bf16_t><<<grid, 256, 0, s>>>((bf16_t *)w_ref, (bf16_t *)w_packed, grad_packed, m, v, d, F, c);
+    else k_adam_decoder<bf16_t><<<grid, 256, 0, s>>>((bf16_t *)w_ref, (bf16_t *)w_packed, grad_packed, m, v, d, F, c);
+  } else {
+    if (vec) k_adam_decoder_vec<float><<<grid, 256, 0, s>>>((float *)w_ref, (float *)w_packed, grad_packed, m, v, d, F, c);
+    else k_adam_decoder<float><<<grid, 256, 0, s>>>((float *)w_ref, (float *)w_packed, grad_packed, m, v, d, F, c);
+  }
   return clt_check_launch();
 }

@@ -34,6 +34,9 @@ def build(wl, dev):
     BASE.scaled("bw-wide", num_layers=2, d_model=768, num_features=512, tokens=64, k=20),
     BASE.scaled("bw-jump", activation_fn="jumprelu", k=None),
     BASE.scaled("bw-fused", num_layers=2, d_model=128, num_features=512, tokens=256, k=10, dtype="bfloat16"),
+    # one layer of inputs / loss gradient larger than an XCD's L2: the weight-gradient kernels split the columns
+    BASE.scaled("bw-split", num_layers=2, d_model=768, num_features=512, tokens=4096, k=12, dtype="bfloat16"),
+    BASE.scaled("bw-split-f32", num_layers=2, d_model=200, num_features=256, tokens=4096, k=6),
 ], ids=lambda w: w.name)
 def test_loss_and_gradients_match_autograd(dev, wl):
     dtype = getattr(torch, wl.dtype)
@@ -147,13 +150,14 @@ def test_training_steps_match_torch_adam_on_autograd_gradients(dev, dtype):
     assert all(torch.isfinite(r).all() for r in rec.values())
 
 
+@pytest.mark.parametrize("shape", [(96, 200), (50, 77)], ids=["vector", "scalar"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_adam_kernels_match_torch_adam_on_given_gradients(dev, dtype):
+def test_adam_kernels_match_torch_adam_on_given_gradients(dev, dtype, shape):
     # same gradients on both sides (zeros and tiny values included): the update itself, three steps
     from crosslayer_coding_amd import _native
     lib = _native.load()
     gen = torch.Generator().manual_seed(5)
-    d, F = 96, 200  # not multiples of the 64 x 64 tile
+    d, F = shape  # not multiples of the 64 x 64 tile; (50, 77) is not a multiple of 4 either
     p0 = (torch.randn(d, F, generator=gen) * 0.1).to(dtype)
     ref = p0.float().clone().requires_grad_(True)
     ropt = torch.optim.Adam([ref], lr=3e-3, betas=(0.9, 0.999), eps=1e-8)
