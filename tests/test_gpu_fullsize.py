@@ -124,3 +124,107 @@ def test_c0_full_size_against_the_oracle_stage_by_stage(dev):
         ref = orc.decode(cpu_acts, t, tying="none", weights=dec_w, biases=dec_b, d_model=d, num_features=F,
                          dtype=torch.float32)
         assert orc.rel_l2(recs[t].cpu(), ref) <= 1e-5
+
+
+def test_c1_sized_gradients_against_exact_differences_of_the_quadratic_loss(dev):
+    # The loss is quadratic in the decoder weights and biases, so along any direction V
+    #     loss(W + V) - loss(W - V) = 2 <grad(W), V>
+    # holds exactly (no step-size limit), and the encoder / selection do not move.  fp32 so that W +- V
+    # is what the kernels read; C1's shape otherwise.
+    wl = synth.WORKLOADS["c1"].scaled("c1-f32", dtype="float32")
+    L, T, d, F = wl.num_layers, wl.tokens, wl.d_model, wl.num_features
+    model, inputs, _ = synth.build_model(wl, dev)
+    model.eval()
+    g = torch.Generator(device=dev).manual_seed(17)
+    targets = {l: torch.randn(T, d, generator=g, device=dev) for l in range(L)}
+    loss, grads = model.loss_and_gradients(inputs, targets)
+    params = dict(model.named_parameters())
+    names = ["decoder_module.decoders.0->0.weight", "decoder_module.decoders.3->7.weight",
+             "decoder_module.decoders.11->11.weight", "decoder_module.decoders.2->5.bias_param"]
+    # direction: the gradient itself, scaled to the size of the parameter (a random direction is almost
+    # orthogonal to the gradient and its effect drowns in the rounding of the loss)
+    predicted, dirs = 0.0, {}
+    for n in names:
+        p, gr = params[n], grads[n]
+        v = gr * (float(p.detach().norm().clamp_min(1.0)) / float(gr.norm()))
+        dirs[n] = v
+        predicted += 2.0 * float((gr.double() * v.double()).sum())
+    del grads
+    with torch.no_grad():
+        for n in names:
+            params[n].add_(dirs[n])
+        plus, _ = model.loss_and_gradients(inputs, targets)
+        for n in names:
+            params[n].sub_(2 * dirs[n])
+        minus, _ = model.loss_and_gradients(inputs, targets)
+    measured = float(plus.double() - minus.double())
+    assert abs(predicted) > 1e-2 * float(loss)              # the direction is not degenerate
+    assert abs(measured - predicted) <= 1e-4 * abs(predicted), (measured, predicted)
+    # the bias gradient of target t is the column sum of d loss / d rec[t] = 2 (rec - target) / (T d)
+    with torch.no_grad():
+        for n in names:
+            params[n].add_(dirs[n])
+    loss2, grads = model.loss_and_gradients(inputs, targets)
+    assert abs(float(loss2) - float(loss)) <= 1e-5 * float(loss)
+    rec = model(inputs)
+    for t in (0, 5, L - 1):
+        want = (2.0 * (rec[t].double() - targets[t].double()) / (T * d)).sum(dim=0)
+        assert orc.rel_l2(grads[f"decoder_module.decoders.{t}->{t}.bias_param"].double().cpu(), want.cpu()) <= 1e-4
+    del model, grads, params, dirs
+    torch.cuda.empty_cache()
+
+
+def test_c1_evaluator_counts_against_dense_scans(dev, c1):
+    # the reductions on the survivor list against the reference's own formulation (dense scans with torch
+    # ops) on the GPU, layer by layer, at full size
+    wl, model, inputs, _ = c1
+    L, T, F, k = wl.num_layers, wl.tokens, wl.num_features, wl.k
+    recs, surv = model.forward_with_survivors(inputs)
+    nonzero, fired = engine.survivor_metrics(surv)
+    dense = engine.densify(surv)
+    for l in range(L):
+        a = dense[l]
+        assert int(nonzero[l]) == int((a != 0).sum())
+        assert torch.equal(fired[l].long(), (a.float() > 1e-6).sum(dim=0))
+    assert int(nonzero.sum()) <= L * k * T        # a kept value can be an exact zero, never more than k*T entries
+    passes = torch.randint(0, 5, (L, F), device=dev)
+    want = torch.where(fired > 0, torch.zeros_like(passes), passes + 1)
+    engine.dead_feature_update(fired, passes)
+    assert torch.equal(passes, want)
+    # reconstruction statistics against torch's own variance / mse on the same tensors
+    tgt = torch.stack([inputs[l] for l in range(L)]).contiguous()        # any [L, T, d] tensor serves as target
+    rec = torch.stack([recs[l] for l in range(L)]).contiguous()
+    stats = engine.reconstruction_stats(rec, tgt)
+    for l in (0, L - 1):
+        t, r = tgt[l].float(), rec[l].float()
+        assert float(stats[l, 0]) == pytest.approx(float(torch.nn.functional.mse_loss(r, t)), rel=1e-4)
+        assert float(stats[l, 1]) == pytest.approx(float(torch.var(t, dim=0, unbiased=False).mean()), rel=1e-4)
+        assert float(stats[l, 2]) == pytest.approx(float(torch.var(t - r, dim=0, unbiased=False).mean()), rel=1e-4)
+
+
+def test_c1_sized_feed_round_trip(dev):
+    # rows gathered without normalisation are the stored rows, bit for bit; with sqrt(d) scaling they
+    # equal torch's own fp32 multiply and cast on the GPU
+    import numpy as np
+    import crosslayer_coding_amd as cca
+    L, T, d, rows = 12, 4096, 768, 8192
+    g = torch.Generator().manual_seed(3)
+    chunks = [torch.randn(L, 2, rows, d, generator=g).to(torch.bfloat16) for _ in range(2)]
+    rng = np.random.RandomState(4)
+    idxs = np.stack([rng.randint(0, 2, T), rng.randint(0, rows, T)], axis=1).astype(np.uint32)
+    order = np.concatenate([np.nonzero(idxs[:, 0] == c)[0] for c in (0, 1)])        # ascending chunk, sampler order inside
+    for method in ("none", "sqrt_d_model"):
+        feed = cca.DeviceActivationFeed(L, d, dtype="bfloat16", device=dev, normalization_method=method)
+        for c, t in enumerate(chunks):
+            feed.add_chunk(c, t)
+        ins, tgs = feed.parse_batch(idxs)
+        for kind, got in ((0, ins), (1, tgs)):
+            for l in (0, 7, L - 1):
+                want = torch.stack([chunks[int(idxs[i, 0])][l, kind, int(idxs[i, 1])] for i in order[:64]]).to(dev)
+                if method == "sqrt_d_model":
+                    want = (want.float() * (d ** 0.5)).to(torch.bfloat16)
+                assert torch.equal(got[l][:64].view(torch.int16), want.view(torch.int16))
+        full = torch.cat([chunks[c][5, 0, torch.as_tensor(idxs[idxs[:, 0] == c, 1].astype(np.int64))] for c in (0, 1)]).to(dev)
+        if method == "sqrt_d_model":
+            full = (full.float() * (d ** 0.5)).to(torch.bfloat16)
+        assert torch.equal(ins[5].view(torch.int16), full.view(torch.int16))
