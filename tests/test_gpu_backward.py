@@ -37,6 +37,11 @@ def build(wl, dev):
     # one layer of inputs / loss gradient larger than an XCD's L2: the weight-gradient kernels split the columns
     BASE.scaled("bw-split", num_layers=2, d_model=768, num_features=512, tokens=4096, k=12, dtype="bfloat16"),
     BASE.scaled("bw-split-f32", num_layers=2, d_model=200, num_features=256, tokens=4096, k=6),
+    # other gates: the survivor list is whatever the forward selected, the backward does not care how
+    BASE.scaled("bw-global", topk_mode="global"),
+    BASE.scaled("bw-tokentopk", activation_fn="topk", k=5),
+    BASE.scaled("bw-tokentopk-global", activation_fn="topk", k=5, topk_mode="global", dtype="bfloat16"),
+    BASE.scaled("bw-relu", activation_fn="relu", k=None),
 ], ids=lambda w: w.name)
 def test_loss_and_gradients_match_autograd(dev, wl):
     dtype = getattr(torch, wl.dtype)
@@ -47,7 +52,7 @@ def test_loss_and_gradients_match_autograd(dev, wl):
     # in bf16 the oracle's fp32 pre-activations would select a slightly different set at the
     # threshold; the comparison here is about gradients, so it gets the model's gate
     masks = None
-    if dtype == torch.bfloat16:
+    if dtype == torch.bfloat16 or wl.topk_mode == "global" or wl.activation_fn == "topk":
         masks = {l: (a != 0).cpu() for l, a in model.get_feature_activations(inputs).items()}
     names = synth.decoder_names(wl)
     theta = None
