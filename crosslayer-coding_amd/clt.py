@@ -161,13 +161,13 @@ class CrossLayerTranscoder(BaseTranscoder):
     # ---- loss and gradients --------------------------------------------------------------------
     def _loss_and_raw_gradients(self, inputs: Dict[int, torch.Tensor], targets: Dict[int, torch.Tensor]):
         """(per-layer losses [L] fp32, raw gradients): ``enc_w`` [L, F, d], ``enc_b`` [L, F],
-        ``dec_w`` [n_dec, F, d] (feature-major, decoders in "s->t" order), ``dec_b`` [L, d] (row t is the
-        gradient of every decoder bias that feeds target t); all fp32."""
+        ``dec_w`` [n_dec, F, d] (feature-major, decoders in slot order: "s->t" pairs, or one per source /
+        per target for tied decoders), ``dec_b`` [n_dec, d] (bias gradient of each decoder); all fp32."""
         cfg = self.config
         L, d, F = cfg.num_layers, cfg.d_model, cfg.num_features
-        if cfg.decoder_tying != "none" or cfg.skip_connection or getattr(cfg, "enable_feature_offset", False) \
+        if cfg.skip_connection or getattr(cfg, "enable_feature_offset", False) \
                 or getattr(cfg, "enable_feature_scale", False):
-            raise NotImplementedError("gradients are built for untied decoders without skip / feature affine terms")
+            raise NotImplementedError("gradients are built for decoders without skip / feature affine terms")
         if sorted(inputs) != list(range(L)) or sorted(targets) != list(range(L)):
             raise ValueError("loss_and_gradients needs inputs and targets for every layer")
         res = self._survivors(inputs)
@@ -184,27 +184,36 @@ class CrossLayerTranscoder(BaseTranscoder):
         dw_dec = engine.decoder_weight_grad(lists, surv, g_model, cfg.decoder_tying)
         _, x_slab, _, _ = self.encoder_module.prepare_slab(inputs)
         dw_enc, db_enc = engine.encoder_weight_grad(lists, dval, x_slab.contiguous(), F)
-        return loss_l, {"enc_w": dw_enc, "enc_b": db_enc, "dec_w": dw_dec, "dec_b": bias_grad}
+        # bias_grad[t] = column sums of d loss / d rec[t]; a decoder's bias takes the rows of the targets
+        # it is added to: its own pair's target, all targets >= its source, or its target (once)
+        if cfg.decoder_tying == "none":
+            dec_b = bias_grad[torch.tensor([t for s_ in range(L) for t in range(s_, L)], device=bias_grad.device)]
+        elif cfg.decoder_tying == "per_source":
+            dec_b = torch.flip(torch.cumsum(torch.flip(bias_grad, dims=[0]), dim=0), dims=[0])
+        else:
+            dec_b = bias_grad
+        return loss_l, {"enc_w": dw_enc, "enc_b": db_enc, "dec_w": dw_dec, "dec_b": dec_b.contiguous()}
 
     @torch.no_grad()
     def loss_and_gradients(self, inputs: Dict[int, torch.Tensor], targets: Dict[int, torch.Tensor]):
         """MSE reconstruction loss (sum over layers of the per-layer mean, losses.py:45-92) and the
         gradients torch autograd gives the reference for it, computed from the survivor list:
         returns (loss [fp32 scalar tensor], {state-dict key: fp32 gradient in the parameter's shape}).
-        Needs every layer present, equal token counts, untied decoders, a top-k or JumpReLU /
-        ReLU activation without skip connections or feature affine terms."""
+        Needs every layer present, equal token counts, a top-k or JumpReLU / ReLU activation,
+        no skip connections or feature affine terms; decoders untied or tied per source / per target."""
         L = self.config.num_layers
         loss_l, raw = self._loss_and_raw_gradients(inputs, targets)
         grads: Dict[str, Optional[torch.Tensor]] = {}
         for l in range(L):
             grads[f"encoder_module.encoders.{l}.weight"] = raw["enc_w"][l]
             grads[f"encoder_module.encoders.{l}.bias_param"] = raw["enc_b"][l]
-        slot = 0
-        for s_ in range(L):
-            for t in range(s_, L):
-                grads[f"decoder_module.decoders.{s_}->{t}.weight"] = raw["dec_w"][slot].t()   # [d, F] view
-                grads[f"decoder_module.decoders.{s_}->{t}.bias_param"] = raw["dec_b"][t]
-                slot += 1
+        if self.config.decoder_tying == "none":
+            keys = [f"{s_}->{t}" for s_ in range(L) for t in range(s_, L)]
+        else:
+            keys = [str(i) for i in range(L)]
+        for slot, key in enumerate(keys):
+            grads[f"decoder_module.decoders.{key}.weight"] = raw["dec_w"][slot].t()   # [d, F] view
+            grads[f"decoder_module.decoders.{key}.bias_param"] = raw["dec_b"][slot]
         if self.config.activation_fn == "jumprelu":
             # the threshold's own gradient (activations.py:183-220) needs the dense neighbourhood of theta
             grads["theta_manager.log_threshold"] = None

@@ -343,13 +343,18 @@ template <typename T, typename CoefT, int NCH, bool DECODER, int SPLIT>
 __global__ __launch_bounds__(BW_THREADS) void k_feature_outer(
     const int32_t *__restrict__ ptr, const int32_t *__restrict__ ltok, const int32_t *__restrict__ lsrc,
     const CoefT *__restrict__ coef, const T *__restrict__ src, float *__restrict__ out, float *__restrict__ rowsum,
-    int64_t Tn, int64_t d, int64_t F, int64_t L, int64_t target) {
+    int64_t Tn, int64_t d, int64_t F, int64_t L, int64_t target, int tying) {
   constexpr int EV = Piece<T>::EV;
   const int lane = lane_id(), wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
   // One launch per layer of the gathered matrix, so that every wavefront of a launch gathers from the
   // same [T, d] matrix: DECODER launch `target` covers the (source <= target, feature) pairs and reads
   // g[target]; the encoder launch `target` covers the features of that layer and reads x[target].
-  const int64_t total = DECODER ? (target + 1) * F : F;
+  // Tied decoders: one matrix per source collects its targets over the launches (the launch
+  // target == source writes the row, later launches add to it: launches must run in ascending
+  // target order on one stream); one matrix per target sums the lists of all sources <= target
+  // inside the wavefront.
+  const bool per_target = DECODER && tying == CLT_TYING_PER_TARGET;
+  const int64_t total = (DECODER && !per_target) ? (target + 1) * F : F;
   const int half = SPLIT == 2 ? (int)(blockIdx.x & 1) : 0;
   const int64_t vblock = SPLIT == 2 ? (int64_t)(blockIdx.x >> 3) * 4 + ((blockIdx.x & 7) >> 1) : (int64_t)blockIdx.x;
   const int64_t nvblock = SPLIT == 2 ? (int64_t)gridDim.x / 2 : (int64_t)gridDim.x;
@@ -359,9 +364,7 @@ __global__ __launch_bounds__(BW_THREADS) void k_feature_outer(
 #pragma unroll
   for (int c = 0; c < NCH; ++c) on[c] = (int64_t)c * 64 + lane < my_pieces;
   for (int64_t w = vblock * nwv + wv; w < total; w += nvblock * nwv) {
-    const int64_t s = DECODER ? w / F : target, f = DECODER ? w - s * F : w, t = target;
-    const int64_t q = s * F + f;
-    const int32_t b = ptr[q], e = ptr[q + 1];
+    const int64_t s = (DECODER && !per_target) ? w / F : target, f = (DECODER && !per_target) ? w - s * F : w, t = target;
     const T *sbase = src + (DECODER ? t : s) * Tn * d;
     float acc[NCH][EV];
 #pragma unroll
@@ -369,6 +372,9 @@ __global__ __launch_bounds__(BW_THREADS) void k_feature_outer(
 #pragma unroll
       for (int k = 0; k < EV; ++k) acc[c][k] = 0.0f;
     float csum = 0.0f;
+    for (int64_t ls = per_target ? 0 : s; ls <= s; ++ls) {
+    const int64_t q = ls * F + f;
+    const int32_t b = ptr[q], e = ptr[q + 1];
     for (int32_t i0 = b; i0 < e; i0 += 64) {
       const int n = (e - i0) < 64 ? (e - i0) : 64;
       int32_t mt = 0; float mc = 0.0f;
@@ -399,14 +405,20 @@ __global__ __launch_bounds__(BW_THREADS) void k_feature_outer(
         }
       }
     }
-    float *orow = out + (DECODER ? (bw_decoder_slot(CLT_TYING_NONE, s, t, L) * F + f) : q) * d;
+    }
+    const int64_t q = s * F + f;
+    float *orow = out + (DECODER ? (bw_decoder_slot(tying, s, t, L) * F + f) : q) * d;
+    const bool add = DECODER && tying == CLT_TYING_PER_SOURCE && t > s;
 #pragma unroll
     for (int c = 0; c < NCH; ++c)
       if (on[c]) {
 #pragma unroll
-        for (int k = 0; k < EV; k += 4)
-          *reinterpret_cast<float4 *>(orow + col0 + (int64_t)c * 64 * EV + lane * EV + k) =
-              make_float4(acc[c][k], acc[c][k + 1], acc[c][k + 2], acc[c][k + 3]);
+        for (int k = 0; k < EV; k += 4) {
+          float4 *dst = reinterpret_cast<float4 *>(orow + col0 + (int64_t)c * 64 * EV + lane * EV + k);
+          float4 r = make_float4(acc[c][k], acc[c][k + 1], acc[c][k + 2], acc[c][k + 3]);
+          if (add) { const float4 o = *dst; r.x += o.x; r.y += o.y; r.z += o.z; r.w += o.w; }
+          *dst = r;
+        }
       }
     if (!DECODER && rowsum && lane == 0 && half == 0) rowsum[q] = csum;
   }
@@ -535,7 +547,7 @@ extern "C" int clt_decoder_weight_grad(const int32_t *list_ptr, const int32_t *l
                                        const void *val, const void *g_model, float *dw_packed, int64_t T, int64_t d,
                                        int64_t F, int64_t L, int tying, int dtype, void *stream) {
   if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
-  if (tying != CLT_TYING_NONE) return CLT_ERR_ARG;   // tied decoders sum over several (source, target) pairs: not built
+  if (tying < 0 || tying > 2) return CLT_ERR_ARG;
   if (T <= 0 || F <= 0 || L <= 0 || L > 64 || !list_ptr || !list_tok || !list_src || !val || !g_model || !dw_packed) return CLT_ERR_ARG;
   if (!bw_shape_ok(d, dtype)) return CLT_ERR_RANGE;
   hipStream_t s = (hipStream_t)stream;
@@ -546,8 +558,8 @@ extern "C" int clt_decoder_weight_grad(const int32_t *list_ptr, const int32_t *l
 #define CLT_DW(CT, N)                                                                                                      \
   do {                                                                                                                     \
     for (int64_t t = 0; t < L; ++t) {                                                                                      \
-      if (split) k_feature_outer<CT, CT, N, true, 2><<<bw_resident_blocks(k_feature_outer<CT, CT, N, true, 2>), BW_THREADS, 0, s>>>(list_ptr, list_tok, list_src, (const CT *)val, (const CT *)g_model, dw_packed, nullptr, T, d, F, L, t); \
-      else k_feature_outer<CT, CT, N, true, 1><<<bw_resident_blocks(k_feature_outer<CT, CT, N, true, 1>), BW_THREADS, 0, s>>>(list_ptr, list_tok, list_src, (const CT *)val, (const CT *)g_model, dw_packed, nullptr, T, d, F, L, t); \
+      if (split) k_feature_outer<CT, CT, N, true, 2><<<bw_resident_blocks(k_feature_outer<CT, CT, N, true, 2>), BW_THREADS, 0, s>>>(list_ptr, list_tok, list_src, (const CT *)val, (const CT *)g_model, dw_packed, nullptr, T, d, F, L, t, tying); \
+      else k_feature_outer<CT, CT, N, true, 1><<<bw_resident_blocks(k_feature_outer<CT, CT, N, true, 1>), BW_THREADS, 0, s>>>(list_ptr, list_tok, list_src, (const CT *)val, (const CT *)g_model, dw_packed, nullptr, T, d, F, L, t, tying); \
     }                                                                                                                      \
   } while (0)
 #define CLT_DW_N(CT)                                                                       \
@@ -577,8 +589,8 @@ extern "C" int clt_encoder_weight_grad(const int32_t *list_ptr, const int32_t *l
 #define CLT_EW(ST, N)                                                                                                      \
   do {                                                                                                                     \
     for (int64_t l = 0; l < L; ++l) {                                                                                      \
-      if (split) k_feature_outer<ST, float, N, false, 2><<<bw_resident_blocks(k_feature_outer<ST, float, N, false, 2>), BW_THREADS, 0, s>>>(list_ptr, list_tok, list_src, dval, (const ST *)x, dw_enc, db_enc, T, d, F, L, l); \
-      else k_feature_outer<ST, float, N, false, 1><<<bw_resident_blocks(k_feature_outer<ST, float, N, false, 1>), BW_THREADS, 0, s>>>(list_ptr, list_tok, list_src, dval, (const ST *)x, dw_enc, db_enc, T, d, F, L, l); \
+      if (split) k_feature_outer<ST, float, N, false, 2><<<bw_resident_blocks(k_feature_outer<ST, float, N, false, 2>), BW_THREADS, 0, s>>>(list_ptr, list_tok, list_src, dval, (const ST *)x, dw_enc, db_enc, T, d, F, L, l, CLT_TYING_NONE); \
+      else k_feature_outer<ST, float, N, false, 1><<<bw_resident_blocks(k_feature_outer<ST, float, N, false, 1>), BW_THREADS, 0, s>>>(list_ptr, list_tok, list_src, dval, (const ST *)x, dw_enc, db_enc, T, d, F, L, l, CLT_TYING_NONE); \
     }                                                                                                                      \
   } while (0)
 #define CLT_EW_N(ST)                                                                       \

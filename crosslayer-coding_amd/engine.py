@@ -410,13 +410,14 @@ def feature_lists(surv: SurvivorList, ws: Optional[Workspace] = None):
 
 
 def decoder_weight_grad(lists, surv: SurvivorList, g: torch.Tensor, tying: str) -> torch.Tensor:
-    """fp32 [n_dec, F, d] gradient of the packed (feature-major) untied decoder weights; ``g`` is
-    d loss / d rec in the model dtype."""
+    """fp32 [n_dec, F, d] gradient of the packed (feature-major) decoder weights (one matrix per
+    (source, target) pair, per source or per target, as ``tying`` says); ``g`` is d loss / d rec in
+    the model dtype."""
     assert g.dtype == surv.dtype and g.is_contiguous()
     ptr, tok, src = lists
     L, T, F = surv.L, surv.T, surv.F
     d = g.shape[2]
-    n_dec = L * (L + 1) // 2
+    n_dec = L * (L + 1) // 2 if tying == "none" else L
     out = torch.empty((n_dec, F, d), dtype=torch.float32, device=g.device)
     code = nat.load().clt_decoder_weight_grad(nat.ptr(ptr), nat.ptr(tok), nat.ptr(src), nat.ptr(surv.val), nat.ptr(g),
                                               nat.ptr(out), T, d, F, L, nat.TYING[tying], nat.dtype_code(surv.dtype),

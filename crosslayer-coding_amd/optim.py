@@ -23,11 +23,9 @@ class CLTAdam:
         self.lr, self.betas, self.eps = float(lr), (float(betas[0]), float(betas[1])), float(eps)
         self.step_count = 0
         cfg = model.config
-        if cfg.decoder_tying != "none":
-            raise NotImplementedError("CLTAdam is built for untied decoders")
         L, F, d = cfg.num_layers, cfg.num_features, cfg.d_model
         dev = model.device
-        n_dec = L * (L + 1) // 2
+        n_dec = L * (L + 1) // 2 if cfg.decoder_tying == "none" else L
         z = lambda *shape: torch.zeros(shape, dtype=torch.float32, device=dev)   # noqa: E731
         self.state: Dict[str, Tuple[torch.Tensor, torch.Tensor]] = {
             "enc_w": (z(L, F, d), z(L, F, d)), "enc_b": (z(L, F), z(L, F)),
@@ -52,24 +50,19 @@ class CLTAdam:
         dec = model.decoder_module
         packed = dec.packed()
         decs = dec._ordered()
-        L = model.config.num_layers
         lib = nat.load()
         m_w, v_w = self.state["dec_w"]
         m_b, v_b = self.state["dec_b"]
-        slot = 0
-        for s in range(L):
-            for t in range(s, L):
-                lin = decs[slot]
-                w = lin.weight.data
-                assert w.is_contiguous()
-                d, F = w.shape
-                code = lib.clt_adam_step_decoder(nat.ptr(w), nat.ptr(packed[slot]), nat.ptr(raw["dec_w"][slot]),
-                                                 nat.ptr(m_w[slot]), nat.ptr(v_w[slot]), d, F, self.lr, self.betas[0],
-                                                 self.betas[1], self.eps, self.step_count, nat.dtype_code(w.dtype),
-                                                 nat.current_stream(w.device))
-                nat.check(code, "clt_adam_step_decoder")
-                self._adam(lin.bias_param.data, raw["dec_b"][t], m_b[slot], v_b[slot])
-                slot += 1
+        for slot, lin in enumerate(decs):
+            w = lin.weight.data
+            assert w.is_contiguous()
+            d, F = w.shape
+            code = lib.clt_adam_step_decoder(nat.ptr(w), nat.ptr(packed[slot]), nat.ptr(raw["dec_w"][slot]),
+                                             nat.ptr(m_w[slot]), nat.ptr(v_w[slot]), d, F, self.lr, self.betas[0],
+                                             self.betas[1], self.eps, self.step_count, nat.dtype_code(w.dtype),
+                                             nat.current_stream(w.device))
+            nat.check(code, "clt_adam_step_decoder")
+            self._adam(lin.bias_param.data, raw["dec_b"][slot], m_b[slot], v_b[slot])
         # the kernels wrote through .data: caches keyed on version counters would not notice
         dec._bias_cache.clear()
         dec._cached_decoder_norms = None

@@ -329,7 +329,10 @@ int clt_decoder_norms(const void *w_packed, void *norms, int64_t d, int64_t F,
  *   list_tok [nnz] token of each entry, list_src [nnz] its position in col / val.  Lists of up to
  *   64 entries are in token order.  Pass list_tok = list_src = NULL to get the counts only.
  * clt_decoder_weight_grad: dw_packed[slot(s,t)][f][:] = sum over the list of (s, f) of
- *   val * g_model[t][token][:] (fp32 sums, feature-major like w_packed; untied decoders only).
+ *   val * g_model[t][token][:] (fp32 sums, feature-major like w_packed); with tied decoders the
+ *   slot collects every pair that shares it (CLT_TYING_PER_SOURCE: all t >= s; CLT_TYING_PER_TARGET:
+ *   all s <= t), so dw_packed has L matrices instead of L(L+1)/2.  One launch per target layer,
+ *   in ascending order on `stream`.
  * clt_encoder_weight_grad: dw_enc[s][f][:] = sum over the list of dval * x[s][token][:],
  *   db_enc[s][f] = sum of dval (fp32; x [L][T][d] in the model dtype).
  * Limits: d % 8 == 0 (bf16) / d % 4 == 0 (fp32) and d <= 2048.

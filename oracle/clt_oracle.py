@@ -514,9 +514,10 @@ def mse_loss_and_gradients(inputs: Dict[int, torch.Tensor], targets: Dict[int, t
                            dec_w: Dict[str, torch.Tensor], dec_b: Dict[str, torch.Tensor],
                            activation_fn: str, num_layers: int, k: Optional[float] = None,
                            theta: Optional[torch.Tensor] = None,
-                           masks: Optional[Dict[int, torch.Tensor]] = None):
+                           masks: Optional[Dict[int, torch.Tensor]] = None, tying: str = "none"):
     """loss = sum over layers of nn.MSELoss()(prediction, target) (losses.py:45-92, no
-    de-normalisation statistics) through the reference's forward with untied decoders, and
+    de-normalisation statistics) through the reference's forward (decoders untied, keys "s->t", or
+    tied per source / per target, keys "i", decoder.py:176-340 without feature affine terms), and
     d loss / d parameter from torch autograd (trainer.py:751): F.linear backward for encoder
     and decoders, the straight-through gate of BatchTopK (activations.py:66-96: grad * mask)
     or the pass-through part of JumpReLU's backward (activations.py:183-220: grad * 1[x >= theta];
@@ -550,9 +551,15 @@ def mse_loss_and_gradients(inputs: Dict[int, torch.Tensor], targets: Dict[int, t
     loss = torch.zeros((), dtype=torch.float32)
     for t in range(L):
         rec = torch.zeros_like(targets[t], dtype=torch.float32)
-        for s_ in range(t + 1):
-            rec = rec + F.linear(acts[s_], params[f"decoder_module.decoders.{s_}->{t}.weight"],
-                                 params[f"decoder_module.decoders.{s_}->{t}.bias_param"])
+        if tying == "per_target":      # one decoder per target over the summed activations, bias once
+            summed = sum(acts[s_] for s_ in range(t + 1))
+            rec = F.linear(summed, params[f"decoder_module.decoders.{t}.weight"],
+                           params[f"decoder_module.decoders.{t}.bias_param"])
+        else:
+            for s_ in range(t + 1):
+                key = f"{s_}->{t}" if tying == "none" else str(s_)
+                rec = rec + F.linear(acts[s_], params[f"decoder_module.decoders.{key}.weight"],
+                                     params[f"decoder_module.decoders.{key}.bias_param"])
         loss = loss + F.mse_loss(rec, targets[t].float())
     loss.backward()
     return loss.detach(), {name: p.grad for name, p in params.items()}

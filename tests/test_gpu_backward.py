@@ -42,6 +42,11 @@ def build(wl, dev):
     BASE.scaled("bw-tokentopk", activation_fn="topk", k=5),
     BASE.scaled("bw-tokentopk-global", activation_fn="topk", k=5, topk_mode="global", dtype="bfloat16"),
     BASE.scaled("bw-relu", activation_fn="relu", k=None),
+    # tied decoders: one matrix per source (collects its targets) or per target (sums its sources)
+    BASE.scaled("bw-per-source", decoder_tying="per_source"),
+    BASE.scaled("bw-per-target", decoder_tying="per_target"),
+    BASE.scaled("bw-per-source-bf16", decoder_tying="per_source", dtype="bfloat16", num_layers=4),
+    BASE.scaled("bw-per-target-split", decoder_tying="per_target", num_layers=3, d_model=200, num_features=256, tokens=4096, k=6),
 ], ids=lambda w: w.name)
 def test_loss_and_gradients_match_autograd(dev, wl):
     dtype = getattr(torch, wl.dtype)
@@ -64,7 +69,7 @@ def test_loss_and_gradients_match_autograd(dev, wl):
         enc_b=[sd[f"encoder_module.encoders.{l}.bias_param"] for l in range(L)],
         dec_w={n: sd[f"decoder_module.decoders.{n}.weight"] for n in names},
         dec_b={n: sd[f"decoder_module.decoders.{n}.bias_param"] for n in names},
-        activation_fn=wl.activation_fn, num_layers=L, k=wl.k, theta=theta, masks=masks)
+        activation_fn=wl.activation_fn, num_layers=L, k=wl.k, theta=theta, masks=masks, tying=wl.decoder_tying)
     tol = TOL[dtype]
     assert abs(float(loss) - float(ref_loss)) <= max(tol, 1e-6) * abs(float(ref_loss)) * 10
     for name, gref in ref.items():
@@ -95,13 +100,14 @@ def test_feature_lists_are_a_permutation_grouped_by_feature(dev):
                 assert bool((tok[b + 1:e] > tok[b:e - 1]).all())
 
 
+@pytest.mark.parametrize("tying", ["none", "per_source", "per_target"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_training_steps_match_torch_adam_on_autograd_gradients(dev, dtype):
+def test_training_steps_match_torch_adam_on_autograd_gradients(dev, dtype, tying):
     # two optimisation steps; reference: torch.optim.Adam over the oracle's autograd gradients, fp32
     # parameters, the gate of each step taken from the model (so both sides differentiate the same
     # function); bf16 parameters are compared after rounding the reference to bf16
     import crosslayer_coding_amd as cca
-    wl = BASE.scaled("tr", dtype=dtype, num_layers=2, d_model=128, num_features=256, tokens=64, k=6)
+    wl = BASE.scaled("tr", dtype=dtype, num_layers=2, d_model=128, num_features=256, tokens=64, k=6, decoder_tying=tying)
     tdt = getattr(torch, dtype)
     model, sd, x, targets = build(wl, dev)
     L = wl.num_layers
@@ -122,7 +128,7 @@ def test_training_steps_match_torch_adam_on_autograd_gradients(dev, dtype):
             enc_b=[cur[f"encoder_module.encoders.{l}.bias_param"] for l in range(L)],
             dec_w={n: cur[f"decoder_module.decoders.{n}.weight"] for n in names},
             dec_b={n: cur[f"decoder_module.decoders.{n}.bias_param"] for n in names},
-            activation_fn="batchtopk", num_layers=L, k=wl.k, masks=masks)
+            activation_fn="batchtopk", num_layers=L, k=wl.k, masks=masks, tying=tying)
         assert abs(float(loss) - float(ref_loss)) <= (1e-4 if tdt == torch.float32 else 2e-2) * abs(float(ref_loss))
         ropt.zero_grad()
         for k, p in ref.items():
@@ -145,11 +151,8 @@ def test_training_steps_match_torch_adam_on_autograd_gradients(dev, dtype):
             assert torch.allclose(got[clear], p.detach()[clear], rtol=1e-4, atol=1e-4), k
     # the feature-major working copy was updated together with the parameters
     packed = model.decoder_module.packed()
-    slot = 0
-    for s in range(L):
-        for t in range(s, L):
-            assert torch.equal(packed[slot], new_sd[f"decoder_module.decoders.{s}->{t}.weight"].t())
-            slot += 1
+    for slot, n in enumerate(names):
+        assert torch.equal(packed[slot], new_sd[f"decoder_module.decoders.{n}.weight"].t())
     # and a forward after the steps runs on the new weights
     rec = model(inputs)
     assert all(torch.isfinite(r).all() for r in rec.values())

@@ -270,25 +270,31 @@ def test_theta_estimation_reference_test_properties():
 
 
 # ---- MSE loss gradients: finite differences in float64 on a tiny model ---------------------------
-def test_mse_gradients_match_finite_differences():
+@pytest.mark.parametrize("tying", ["none", "per_source", "per_target"])
+def test_mse_gradients_match_finite_differences(tying):
     g = torch.Generator().manual_seed(3)
     L, T, d, F_, k = 2, 6, 3, 5, 2
     x = {l: torch.randn(T, d, generator=g) for l in range(L)}
     tgt = {l: torch.randn(T, d, generator=g) for l in range(L)}
     enc_w = [torch.randn(F_, d, generator=g) for _ in range(L)]
     enc_b = [0.1 * torch.randn(F_, generator=g) for _ in range(L)]
-    names = ["0->0", "0->1", "1->1"]
+    names = ["0->0", "0->1", "1->1"] if tying == "none" else ["0", "1"]
     dec_w = {n: torch.randn(d, F_, generator=g) for n in names}
     dec_b = {n: 0.1 * torch.randn(d, generator=g) for n in names}
     loss, grads = orc.mse_loss_and_gradients(x, tgt, enc_w=enc_w, enc_b=enc_b, dec_w=dec_w, dec_b=dec_b,
-                                             activation_fn="batchtopk", num_layers=L, k=k)
+                                             activation_fn="batchtopk", num_layers=L, k=k, tying=tying)
     masks = {l: orc.batchtopk_mask(torch.nn.functional.linear(x[l], enc_w[l], enc_b[l]), k) for l in range(L)}
 
     def loss64(ew, eb, dw, db):     # independent float64 numpy forward with the gate held fixed
         acts = {l: (x[l].double().numpy() @ ew[l].T + eb[l]) * masks[l].numpy() for l in range(L)}
         total = 0.0
         for t in range(L):
-            rec = sum(acts[s] @ dw[f"{s}->{t}"].T + db[f"{s}->{t}"] for s in range(t + 1))
+            if tying == "none":
+                rec = sum(acts[s] @ dw[f"{s}->{t}"].T + db[f"{s}->{t}"] for s in range(t + 1))
+            elif tying == "per_source":      # the source's decoder and bias, once per contributing source
+                rec = sum(acts[s] @ dw[str(s)].T + db[str(s)] for s in range(t + 1))
+            else:                            # the target's decoder over the summed activations, bias once
+                rec = sum(acts[s] for s in range(t + 1)) @ dw[str(t)].T + db[str(t)]
             total += float(np.mean((rec - tgt[t].double().numpy()) ** 2))
         return total
 
@@ -296,8 +302,10 @@ def test_mse_gradients_match_finite_differences():
     dw = {n: w.double().numpy().copy() for n, w in dec_w.items()}; db = {n: b.double().numpy().copy() for n, b in dec_b.items()}
     assert abs(loss64(ew, eb, dw, db) - float(loss)) < 1e-5
     eps = 1e-6
+    wn, bn = (("0->1", "1->1") if tying == "none" else ("0", "1"))
     checks = [("encoder_module.encoders.0.weight", ew[0], (1, 2)), ("encoder_module.encoders.1.bias_param", eb[1], (3,)),
-              ("decoder_module.decoders.0->1.weight", dw["0->1"], (2, 4)), ("decoder_module.decoders.1->1.bias_param", db["1->1"], (0,))]
+              (f"decoder_module.decoders.{wn}.weight", dw[wn], (2, 4)), (f"decoder_module.decoders.{bn}.bias_param", db[bn], (0,)),
+              (f"decoder_module.decoders.{wn}.bias_param", db[wn], (1,))]
     for name, arr, idx in checks:
         old = arr[idx]
         arr[idx] = old + eps; up = loss64(ew, eb, dw, db)
