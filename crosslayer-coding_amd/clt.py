@@ -184,6 +184,9 @@ class CrossLayerTranscoder(BaseTranscoder):
         dw_dec = engine.decoder_weight_grad(lists, surv, g_model, cfg.decoder_tying)
         _, x_slab, _, _ = self.encoder_module.prepare_slab(inputs)
         dw_enc, db_enc = engine.encoder_weight_grad(lists, dval, x_slab.contiguous(), F)
+        theta_grad = None
+        if cfg.activation_fn == "jumprelu" and self.theta_manager.log_threshold is not None:
+            theta_grad = self._log_threshold_gradient(x_slab, g_model, ws)
         # bias_grad[t] = column sums of d loss / d rec[t]; a decoder's bias takes the rows of the targets
         # it is added to: its own pair's target, all targets >= its source, or its target (once)
         if cfg.decoder_tying == "none":
@@ -192,7 +195,36 @@ class CrossLayerTranscoder(BaseTranscoder):
             dec_b = torch.flip(torch.cumsum(torch.flip(bias_grad, dims=[0]), dim=0), dims=[0])
         else:
             dec_b = bias_grad
-        return loss_l, {"enc_w": dw_enc, "enc_b": db_enc, "dec_w": dw_dec, "dec_b": dec_b.contiguous()}
+        return loss_l, {"enc_w": dw_enc, "enc_b": db_enc, "dec_w": dw_dec, "dec_b": dec_b.contiguous(), "theta": theta_grad}
+
+    def _log_threshold_gradient(self, x_slab: torch.Tensor, g_model: torch.Tensor, ws) -> torch.Tensor:
+        """fp32 [L, F] gradient of ``log_threshold`` (JumpReLU.backward, activations.py:196-199, through
+        theta = exp(log_threshold), theta.py:70-79).  The band |x - theta| <= bandwidth / 2 holds elements
+        on both sides of the threshold, so this part is dense: per source layer, d loss / d activation
+        is one product of the stacked loss gradients [T, (L-s) d] with the stacked decoders [F, (L-s) d]
+        on the MFMA kernel, reduced over tokens together with the dense pre-activations."""
+        cfg = self.config
+        L, F = cfg.num_layers, cfg.num_features
+        tying = cfg.decoder_tying
+        w, b = self.encoder_module.stacked()
+        pre = engine.encode(x_slab.contiguous(), w, b, out=ws.typed("pre", tuple(x_slab.shape[:2]) + (F,), self.dtype))
+        theta = self.theta_manager.thresholds(self.dtype)
+        packed = self.decoder_module.packed()
+        out = torch.empty((L, F), dtype=torch.float32, device=pre.device)
+        for s_ in range(L):
+            targets = list(range(s_, L))
+            if tying == "none":
+                slots = [s_ * L - (s_ * (s_ - 1)) // 2 + (t - s_) for t in targets]
+            elif tying == "per_source":
+                slots = [s_] * len(targets)
+            else:
+                slots = targets
+            stacked_w = torch.cat([packed[i] for i in slots], dim=1).unsqueeze(0)          # [1, F, n d]
+            stacked_g = torch.cat([g_model[t] for t in targets], dim=1).unsqueeze(0)       # [1, T, n d]
+            dact = engine.encode(stacked_g.contiguous(), stacked_w.contiguous(), None)[0]  # [T, F]
+            engine.jumprelu_theta_grad(pre[s_], dact, theta[s_].contiguous(), self.theta_manager.bandwidth, out[s_], ws)
+        # theta = exp(log_threshold): the reference casts theta to the model dtype for the forward
+        return out * torch.exp(self.theta_manager.log_threshold.detach().float())
 
     @torch.no_grad()
     def loss_and_gradients(self, inputs: Dict[int, torch.Tensor], targets: Dict[int, torch.Tensor]):
@@ -214,9 +246,8 @@ class CrossLayerTranscoder(BaseTranscoder):
         for slot, key in enumerate(keys):
             grads[f"decoder_module.decoders.{key}.weight"] = raw["dec_w"][slot].t()   # [d, F] view
             grads[f"decoder_module.decoders.{key}.bias_param"] = raw["dec_b"][slot]
-        if self.config.activation_fn == "jumprelu":
-            # the threshold's own gradient (activations.py:183-220) needs the dense neighbourhood of theta
-            grads["theta_manager.log_threshold"] = None
+        if raw.get("theta") is not None:
+            grads["theta_manager.log_threshold"] = raw["theta"]
         return loss_l.sum(), grads
 
     @torch.no_grad()

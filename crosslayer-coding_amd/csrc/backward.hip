@@ -443,6 +443,37 @@ static unsigned bw_resident_blocks(K kernel) {
   return nb < 8 ? 8 : nb & ~7u;   // a multiple of the 8 XCDs
 }
 
+// ---- JumpReLU threshold gradient (reference clt/models/activations.py:196-199) -------------------
+//   grad_theta[f] = sum over tokens of grad_out * (-x / bandwidth)  where |x - theta[f]| <= bandwidth / 2
+// on dense [T, F] pre-activations x and dense d loss / d activation, every step rounded to the
+// model dtype as the reference's tensor arithmetic is; the sum itself is fp32, rows in a fixed order.
+constexpr int TG_SPLIT = 32;
+template <typename T>
+__global__ __launch_bounds__(BW_THREADS) void k_theta_grad_partial(const T *__restrict__ pre, const T *__restrict__ dact,
+                                                                    const T *__restrict__ theta, int64_t Tn, int64_t F,
+                                                                    float bw, float *__restrict__ part) {
+  const int64_t f = (int64_t)blockIdx.x * BW_THREADS + threadIdx.x;
+  if (f >= F) return;
+  const int64_t rows = (Tn + TG_SPLIT - 1) / TG_SPLIT, r0 = (int64_t)blockIdx.y * rows, r1 = r0 + rows < Tn ? r0 + rows : Tn;
+  const float th = Elem<T>::to_f32(theta[f]), half = 0.5f * bw;
+  float acc = 0.0f;
+  for (int64_t r = r0; r < r1; ++r) {
+    const float x = Elem<T>::to_f32(pre[r * F + f]);
+    if (fabsf(Elem<T>::round(x - th)) <= half) {
+      const float g = Elem<T>::to_f32(dact[r * F + f]);
+      acc += Elem<T>::round(g * Elem<T>::round(-x / bw));
+    }
+  }
+  part[(int64_t)blockIdx.y * F + f] = acc;
+}
+__global__ void k_theta_grad_finish(const float *part, int64_t F, float *out) {
+  for (int64_t f = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; f < F; f += (int64_t)gridDim.x * blockDim.x) {
+    float a = 0.0f;
+    for (int z = 0; z < TG_SPLIT; ++z) a += part[(int64_t)z * F + f];
+    out[f] = a;
+  }
+}
+
 static bool bw_shape_ok(int64_t d, int dtype) { return d > 0 && d % (dtype == CLT_BF16 ? 8 : 4) == 0 && d <= 2048; }
 
 }  // namespace
@@ -604,5 +635,25 @@ extern "C" int clt_encoder_weight_grad(const int32_t *list_ptr, const int32_t *l
   if (dtype == CLT_BF16) CLT_EW_N(bf16_t); else CLT_EW_N(float);
 #undef CLT_EW_N
 #undef CLT_EW
+  return clt_check_launch();
+}
+
+extern "C" size_t clt_jumprelu_theta_grad_workspace_bytes(int64_t F) { return F > 0 ? (size_t)TG_SPLIT * (size_t)F * 4 : 256; }
+
+extern "C" int clt_jumprelu_theta_grad(const void *pre, const void *dact, const void *theta, int64_t T, int64_t F,
+                                       double bandwidth, int dtype, float *grad_theta, void *workspace, size_t workspace_bytes,
+                                       void *stream) {
+  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (T <= 0 || F <= 0 || !(bandwidth > 0.0) || !pre || !dact || !theta || !grad_theta || !workspace) return CLT_ERR_ARG;
+  if (workspace_bytes < clt_jumprelu_theta_grad_workspace_bytes(F)) return CLT_ERR_WORKSPACE;
+  if ((((uintptr_t)workspace) & 3u) != 0) return CLT_ERR_ALIGN;
+  hipStream_t s = (hipStream_t)stream;
+  float *part = (float *)workspace;
+  dim3 grid((unsigned)clt_ceil_div(F, BW_THREADS), TG_SPLIT);
+  if (dtype == CLT_BF16)
+    k_theta_grad_partial<bf16_t><<<grid, BW_THREADS, 0, s>>>((const bf16_t *)pre, (const bf16_t *)dact, (const bf16_t *)theta, T, F, (float)bandwidth, part);
+  else
+    k_theta_grad_partial<float><<<grid, BW_THREADS, 0, s>>>((const float *)pre, (const float *)dact, (const float *)theta, T, F, (float)bandwidth, part);
+  k_theta_grad_finish<<<(unsigned)clt_ceil_div(F, 256), 256, 0, s>>>(part, F, grad_theta);
   return clt_check_launch();
 }

@@ -439,6 +439,22 @@ def encoder_weight_grad(lists, dval: torch.Tensor, x: torch.Tensor, F: int):
     return dw, db
 
 
+def jumprelu_theta_grad(pre: torch.Tensor, grad_out: torch.Tensor, theta: torch.Tensor, bandwidth: float,
+                        out: torch.Tensor, ws: Optional[Workspace] = None) -> None:
+    """out [F] fp32 = gradient of one layer's JumpReLU thresholds from dense pre-activations and dense
+    d loss / d activation, both [T, F] in the model dtype (activations.py:196-199)."""
+    nat.require_device(pre, "jumprelu_theta_grad")
+    T, F = pre.shape
+    assert grad_out.shape == pre.shape and grad_out.dtype == pre.dtype and theta.dtype == pre.dtype
+    assert pre.is_contiguous() and grad_out.is_contiguous() and theta.is_contiguous() and theta.numel() == F
+    assert out.dtype == torch.float32 and out.is_contiguous() and out.numel() == F
+    lib = nat.load()
+    wbuf = (ws or Workspace(pre.device)).get("theta_grad", lib.clt_jumprelu_theta_grad_workspace_bytes(F))
+    code = lib.clt_jumprelu_theta_grad(nat.ptr(pre), nat.ptr(grad_out), nat.ptr(theta), T, F, float(bandwidth),
+                                       nat.dtype_code(pre.dtype), nat.ptr(out), nat.ptr(wbuf), wbuf.numel(), _stream(pre))
+    nat.check(code, "clt_jumprelu_theta_grad")
+
+
 def pack_decoder(w_ref: torch.Tensor, out: torch.Tensor) -> None:
     """[d, F] checkpoint layout -> [F, d] feature-major (one matrix)."""
     nat.require_device(w_ref, "pack_decoder")

@@ -31,6 +31,8 @@ class CLTAdam:
             "enc_w": (z(L, F, d), z(L, F, d)), "enc_b": (z(L, F), z(L, F)),
             "dec_w": (z(n_dec, F, d), z(n_dec, F, d)), "dec_b": (z(n_dec, d), z(n_dec, d)),
         }
+        if cfg.activation_fn == "jumprelu" and model.theta_manager.log_threshold is not None:
+            self.state["theta"] = (z(L, F), z(L, F))
 
     def _adam(self, param: torch.Tensor, grad: torch.Tensor, m: torch.Tensor, v: torch.Tensor) -> None:
         assert param.is_contiguous() and grad.is_contiguous() and grad.dtype == torch.float32 and grad.numel() == param.numel()
@@ -63,6 +65,8 @@ class CLTAdam:
                                              nat.current_stream(w.device))
             nat.check(code, "clt_adam_step_decoder")
             self._adam(lin.bias_param.data, raw["dec_b"][slot], m_b[slot], v_b[slot])
+        if raw.get("theta") is not None and "theta" in self.state:
+            self._adam(model.theta_manager.log_threshold.data, raw["theta"].contiguous(), *self.state["theta"])
         # the kernels wrote through .data: caches keyed on version counters would not notice
         dec._bias_cache.clear()
         dec._cached_decoder_norms = None

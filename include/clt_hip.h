@@ -374,6 +374,21 @@ int clt_adam_step_decoder(void *w_ref, void *w_packed, const float *grad_packed,
                           int64_t d, int64_t F, double lr, double beta1, double beta2, double eps,
                           int64_t step, int dtype, void *stream);
 
+/* clt_jumprelu_theta_grad: gradient of the JumpReLU thresholds of one layer (JumpReLU.backward,
+ *   clt/models/activations.py:196-199; bandwidth is 1.0 in ThetaManager, clt/models/theta.py:41):
+ *     grad_theta[f] = sum over tokens of grad_out[tok][f] * (-pre[tok][f] / bandwidth)
+ *                     over the elements with |pre - theta[f]| <= bandwidth / 2
+ *   pre, grad_out [T][F] and theta [F] in the model dtype (each arithmetic step is rounded to it,
+ *   as the reference's tensor arithmetic is), grad_theta [F] fp32.  The band holds elements on
+ *   both sides of the threshold, so pre and grad_out are dense: the caller gets grad_out of a
+ *   source layer as one product of the stacked loss gradients with the stacked decoders (clt_encode
+ *   serves as that product).  workspace: clt_jumprelu_theta_grad_workspace_bytes(F).
+ */
+size_t clt_jumprelu_theta_grad_workspace_bytes(int64_t F);
+int clt_jumprelu_theta_grad(const void *pre, const void *grad_out, const void *theta, int64_t T,
+                            int64_t F, double bandwidth, int dtype, float *grad_theta,
+                            void *workspace, size_t workspace_bytes, void *stream);
+
 /* ---- evaluation reductions ---------------------------------------------------
  * clt_survivor_metrics: from a survivor list, per layer the number of entries whose value is
  *   != 0 (nonzero_per_layer [L]; divided by T it is the layer's mean L0 of

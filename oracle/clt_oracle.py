@@ -31,6 +31,8 @@ How each function is pinned (see ``tests/test_oracle_*.py``):
   properties the reference's own test asserts (tests/unit/models/test_theta.py:110-175:
   thresholds finite and positive, higher for the features that were selected); the
   reference holds no golden numbers for them: PARITY UNPINNED beyond that.
+* ``JumpReLUFunction``  - the reference's table of input / threshold gradients
+  (tests/unit/models/test_activations.py:318-381, 16 cases).
 * ``mse_loss_and_gradients``  - torch autograd itself computes the gradients; a central
   finite-difference check in float64 on a tiny model pins the loss / gradient pairing, and the
   reference's backward tables (test_activations.py:114-152: grad * mask) pin the gate.
@@ -186,6 +188,29 @@ def jumprelu_forward(x: torch.Tensor, threshold: torch.Tensor) -> torch.Tensor:
     The product is fp32 whatever the input dtype, as in the reference.
     """
     return (x >= threshold).float() * x
+
+
+class JumpReLUFunction(torch.autograd.Function):
+    """JumpReLU with the reference's backward (activations.py:175-220): the input gradient passes
+    where input >= threshold; the threshold gradient is grad_output * (-input / bandwidth) on the
+    elements with |input - threshold| <= bandwidth / 2, summed over the leading dimensions that the
+    threshold does not have."""
+
+    @staticmethod
+    def forward(ctx, x, threshold, bandwidth):
+        ctx.save_for_backward(x, threshold)
+        ctx.bandwidth = bandwidth
+        return (x >= threshold).to(x.dtype) * x
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        x, threshold = ctx.saved_tensors
+        grad_x = grad_output * (x >= threshold).type_as(grad_output)
+        near = torch.abs(x - threshold) <= (ctx.bandwidth / 2.0)
+        per_element = grad_output * ((-x / ctx.bandwidth) * near.type_as(x))
+        extra = per_element.dim() - threshold.dim()
+        grad_t = per_element.sum(dim=tuple(range(extra))) if extra > 0 else per_element
+        return grad_x, grad_t.reshape(threshold.shape), None
 
 
 def theta_from_log(log_threshold_row: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
@@ -514,7 +539,9 @@ def mse_loss_and_gradients(inputs: Dict[int, torch.Tensor], targets: Dict[int, t
                            dec_w: Dict[str, torch.Tensor], dec_b: Dict[str, torch.Tensor],
                            activation_fn: str, num_layers: int, k: Optional[float] = None,
                            theta: Optional[torch.Tensor] = None,
-                           masks: Optional[Dict[int, torch.Tensor]] = None, tying: str = "none"):
+                           masks: Optional[Dict[int, torch.Tensor]] = None, tying: str = "none",
+                           log_threshold: Optional[torch.Tensor] = None, bandwidth: float = 1.0,
+                           model_dtype: torch.dtype = torch.float32):
     """loss = sum over layers of nn.MSELoss()(prediction, target) (losses.py:45-92, no
     de-normalisation statistics) through the reference's forward (decoders untied, keys "s->t", or
     tied per source / per target, keys "i", decoder.py:176-340 without feature affine terms), and
@@ -524,9 +551,15 @@ def mse_loss_and_gradients(inputs: Dict[int, torch.Tensor], targets: Dict[int, t
     the threshold's own gradient is not part of this function).  Per-layer selection, fp32.
     ``masks`` (bool [T, F] per layer) replaces the gate computed here, for comparisons in which
     the other side selected on differently rounded pre-activations.
+    With ``log_threshold`` ([L, F], the parameter itself) the JumpReLU runs through
+    ``JumpReLUFunction`` with threshold = exp(log_threshold) cast to ``model_dtype`` and back
+    (theta.py:70-79, bandwidth 1.0 at theta.py:41) and the result holds the gradient of
+    "theta_manager.log_threshold" as well.
     Returns (loss, {state-dict key: gradient})."""
     L = num_layers
     params: Dict[str, torch.Tensor] = {}
+    if log_threshold is not None:
+        params["theta_manager.log_threshold"] = log_threshold.detach().float().clone().requires_grad_(True)
     for l in range(L):
         params[f"encoder_module.encoders.{l}.weight"] = enc_w[l].detach().float().clone().requires_grad_(True)
         params[f"encoder_module.encoders.{l}.bias_param"] = enc_b[l].detach().float().clone().requires_grad_(True)
@@ -537,6 +570,10 @@ def mse_loss_and_gradients(inputs: Dict[int, torch.Tensor], targets: Dict[int, t
     for l in range(L):
         pre = F.linear(inputs[l].float(), params[f"encoder_module.encoders.{l}.weight"],
                        params[f"encoder_module.encoders.{l}.bias_param"])
+        if log_threshold is not None and activation_fn == "jumprelu":
+            thr = torch.exp(params["theta_manager.log_threshold"][l]).to(model_dtype).float()
+            acts[l] = JumpReLUFunction.apply(pre, thr, bandwidth)
+            continue
         if masks is not None:
             mask = masks[l]
         elif activation_fn == "batchtopk":

@@ -33,3 +33,15 @@ def test_oracle_tokentopk(case):
 def test_oracle_jumprelu(case):
     out = orc.jumprelu_forward(torch.tensor(case["x"]), torch.tensor([case["threshold"]]))
     assert torch.equal(out, torch.tensor(case["expected_output"]))
+
+
+@pytest.mark.parametrize("case", GOLD["jumprelu_backward"], ids=lambda c: f"bw{c['bandwidth']}-x{c['input']}-t{c['threshold']}")
+def test_oracle_jumprelu_backward(case):
+    x = torch.tensor([case["input"]], dtype=torch.float64, requires_grad=True)
+    thr = torch.tensor([case["threshold"]], dtype=torch.float64, requires_grad=True)
+    out = orc.JumpReLUFunction.apply(x, thr, case["bandwidth"])
+    out.backward(torch.tensor([case["grad_output"]], dtype=torch.float64))
+    assert x.grad.item() == case["expected_grad_input"] * case["grad_output"]
+    near = abs(case["input"] - case["threshold"]) <= case["bandwidth"] / 2.0
+    want = (-case["input"] / case["bandwidth"]) * case["grad_output"] if near else 0.0
+    assert thr.grad.item() == pytest.approx(want, abs=1e-12)

@@ -33,6 +33,8 @@ def build(wl, dev):
     BASE.scaled("bw-bf16", dtype="bfloat16"),
     BASE.scaled("bw-wide", num_layers=2, d_model=768, num_features=512, tokens=64, k=20),
     BASE.scaled("bw-jump", activation_fn="jumprelu", k=None),
+    BASE.scaled("bw-jump-bf16", activation_fn="jumprelu", k=None, dtype="bfloat16", num_layers=2, d_model=128, num_features=512, tokens=256),
+    BASE.scaled("bw-jump-per-target", activation_fn="jumprelu", k=None, decoder_tying="per_target"),
     BASE.scaled("bw-fused", num_layers=2, d_model=128, num_features=512, tokens=256, k=10, dtype="bfloat16"),
     # one layer of inputs / loss gradient larger than an XCD's L2: the weight-gradient kernels split the columns
     BASE.scaled("bw-split", num_layers=2, d_model=768, num_features=512, tokens=4096, k=12, dtype="bfloat16"),
@@ -60,23 +62,32 @@ def test_loss_and_gradients_match_autograd(dev, wl):
     if dtype == torch.bfloat16 or wl.topk_mode == "global" or wl.activation_fn == "topk":
         masks = {l: (a != 0).cpu() for l, a in model.get_feature_activations(inputs).items()}
     names = synth.decoder_names(wl)
-    theta = None
+    theta, log_theta = None, None
     if wl.activation_fn == "jumprelu":
+        # the oracle then runs the reference's JumpReLU backward, threshold gradient included
         theta = torch.exp(sd["theta_manager.log_threshold"].float()).to(dtype)
+        log_theta = sd["theta_manager.log_threshold"]
+        masks = None
     ref_loss, ref = orc.mse_loss_and_gradients(
         {l: x[l] for l in range(L)}, targets,
         enc_w=[sd[f"encoder_module.encoders.{l}.weight"] for l in range(L)],
         enc_b=[sd[f"encoder_module.encoders.{l}.bias_param"] for l in range(L)],
         dec_w={n: sd[f"decoder_module.decoders.{n}.weight"] for n in names},
         dec_b={n: sd[f"decoder_module.decoders.{n}.bias_param"] for n in names},
-        activation_fn=wl.activation_fn, num_layers=L, k=wl.k, theta=theta, masks=masks, tying=wl.decoder_tying)
+        activation_fn=wl.activation_fn, num_layers=L, k=wl.k, theta=theta, masks=masks, tying=wl.decoder_tying,
+        log_threshold=log_theta, model_dtype=dtype)
     tol = TOL[dtype]
     assert abs(float(loss) - float(ref_loss)) <= max(tol, 1e-6) * abs(float(ref_loss)) * 10
     for name, gref in ref.items():
         got = grads[name]
         assert got is not None and tuple(got.shape) == tuple(gref.shape), name
         err = orc.rel_l2(got.float().cpu(), gref)
-        assert err <= tol * (5 if dtype == torch.bfloat16 else 1), (name, err)
+        bound = tol * (5 if dtype == torch.bfloat16 else 1)
+        if name.endswith("log_threshold"):
+            # band membership |x - theta| <= 1/2 is decided on pre-activations that differ in the last
+            # bits between the two sides; an element that changes side moves the sum by its whole term
+            bound = 1e-3 if dtype == torch.float32 else 1e-1
+        assert err <= bound, (name, err)
 
 
 def test_feature_lists_are_a_permutation_grouped_by_feature(dev):
@@ -100,14 +111,16 @@ def test_feature_lists_are_a_permutation_grouped_by_feature(dev):
                 assert bool((tok[b + 1:e] > tok[b:e - 1]).all())
 
 
-@pytest.mark.parametrize("tying", ["none", "per_source", "per_target"])
+@pytest.mark.parametrize("tying,fn", [("none", "batchtopk"), ("per_source", "batchtopk"), ("per_target", "batchtopk"),
+                                      ("none", "jumprelu")])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_training_steps_match_torch_adam_on_autograd_gradients(dev, dtype, tying):
+def test_training_steps_match_torch_adam_on_autograd_gradients(dev, dtype, tying, fn):
     # two optimisation steps; reference: torch.optim.Adam over the oracle's autograd gradients, fp32
     # parameters, the gate of each step taken from the model (so both sides differentiate the same
     # function); bf16 parameters are compared after rounding the reference to bf16
     import crosslayer_coding_amd as cca
-    wl = BASE.scaled("tr", dtype=dtype, num_layers=2, d_model=128, num_features=256, tokens=64, k=6, decoder_tying=tying)
+    wl = BASE.scaled("tr", dtype=dtype, num_layers=2, d_model=128, num_features=256, tokens=64, decoder_tying=tying,
+                     activation_fn=fn, k=6 if fn == "batchtopk" else None)
     tdt = getattr(torch, dtype)
     model, sd, x, targets = build(wl, dev)
     L = wl.num_layers
@@ -128,7 +141,8 @@ def test_training_steps_match_torch_adam_on_autograd_gradients(dev, dtype, tying
             enc_b=[cur[f"encoder_module.encoders.{l}.bias_param"] for l in range(L)],
             dec_w={n: cur[f"decoder_module.decoders.{n}.weight"] for n in names},
             dec_b={n: cur[f"decoder_module.decoders.{n}.bias_param"] for n in names},
-            activation_fn="batchtopk", num_layers=L, k=wl.k, masks=masks, tying=tying)
+            activation_fn=fn, num_layers=L, k=wl.k, masks=masks if fn == "batchtopk" else None, tying=tying,
+            log_threshold=cur.get("theta_manager.log_threshold"), model_dtype=tdt)
         assert abs(float(loss) - float(ref_loss)) <= (1e-4 if tdt == torch.float32 else 2e-2) * abs(float(ref_loss))
         ropt.zero_grad()
         for k, p in ref.items():
@@ -144,7 +158,10 @@ def test_training_steps_match_torch_adam_on_autograd_gradients(dev, dtype, tying
         want = p.detach() - sd[k].float()
         err = orc.rel_l2(moved, want)
         print(k, "displacement rel-L2", err)
-        assert err <= (2e-2 if tdt == torch.float32 else 0.15), (k, err)
+        bound = 2e-2 if tdt == torch.float32 else 0.15
+        if k.endswith("log_threshold") and tdt == torch.bfloat16:
+            bound = 0.3      # a threshold whose tiny gradient changes sign with the rounding moves the other way
+        assert err <= bound, (k, err)
         if tdt == torch.float32:
             g = grads[k]
             clear = g.abs() > 1e-3 * g.abs().max()
