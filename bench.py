@@ -392,8 +392,8 @@ def run_backward(args):
     cca._native.load(build_if_missing=False)
     model, inputs, _ = synth.build_model(wl, dev)
     model.eval()
-    g = torch.Generator(device=dev).manual_seed(99)
-    targets = {l: torch.randn(wl.tokens, wl.d_model, generator=g, device=dev).to(model.dtype) for l in range(wl.num_layers)}
+    slab = synth.make_targets(wl, dev)
+    targets = {l: slab[l] for l in range(wl.num_layers)}
     opt = cca.CLTAdam(model, lr=1e-4) if args.train_step else None
 
     def one():
@@ -411,7 +411,47 @@ def run_backward(args):
         loss = one()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
+
+    # one more step, stage by stage, with events on the stream the kernels run on
+    from crosslayer_coding_amd import engine
+    L, T, d, F = wl.num_layers, wl.tokens, wl.d_model, wl.num_features
+    stages = {}
+
+    def timed(name, fn):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        out = fn()
+        b.record()
+        b.synchronize()
+        stages[name] = a.elapsed_time(b)
+        return out
+
+    cfg, ws, mask = model.config, model._workspace(), (1 << L) - 1
+    _, _, surv = timed("forward: encode + select", lambda: model._survivors(inputs))
+    rec = timed("forward: decode", lambda: model.decoder_module.decode_survivors(surv, mask, ws=ws))
+    tgt = torch.stack([targets[l] for l in range(L)]).contiguous()
+    loss_l, g, g_model, bias_grad = timed("loss and its gradient", lambda: engine.mse_loss_grad(rec, tgt, ws))
+    dval = timed("gradient of the kept activations", lambda: engine.decode_backward_values(
+        surv, model.decoder_module.packed(), g, cfg.decoder_tying, mask, ws))
+    lists = timed("per-feature token lists", lambda: engine.feature_lists(surv, ws))
+    dw_dec = timed("decoder weight gradient", lambda: engine.decoder_weight_grad(lists, surv, g_model, cfg.decoder_tying))
+    _, x_slab, _, _ = model.encoder_module.prepare_slab(inputs)
+    dw_enc, db_enc = timed("encoder weight gradient", lambda: engine.encoder_weight_grad(lists, dval, x_slab.contiguous(), F))
+    if opt is not None:
+        dec_b = bias_grad[torch.tensor([t for s_ in range(L) for t in range(s_, L)], device=dev)].contiguous()
+        timed("Adam", lambda: opt.step({"enc_w": dw_enc, "enc_b": db_enc, "dec_w": dw_dec, "dec_b": dec_b, "theta": None}))
+    esz = 2 if wl.dtype == "bfloat16" else 4
+    pairs = L * (L + 1) // 2
+    gathered = surv.nnz / L * pairs * d * esz           # one row of g per (survivor, target >= its source)
+    dw_bytes = gathered + pairs * F * d * 4
+    dw_sec = stages["decoder weight gradient"] * 1e-3
+    roofline = {"kernel": f"k_feature_outer (decoder weight gradient, {L} launches per step)", "bound": "hbm",
+                "achieved": dw_bytes / dw_sec / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": dw_bytes / dw_sec / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                "note": "algorithmic bytes = rows of the loss gradient gathered per (survivor, target) + the fp32 gradient "
+                        "written once; above the HBM peak because the gathered rows are L2 hits"}
     return {
+        "stages_ms": stages, "roofline": roofline,
         "metric": ("CLT training step tokens/sec (forward, MSE loss, gradients, Adam lr 1e-4 with fp32 moments)"
                    if opt is not None else "CLT forward + MSE loss + gradients tokens/sec (no optimizer step)"),
         "value": wl.tokens * args.steps / wall, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,

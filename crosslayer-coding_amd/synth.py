@@ -95,6 +95,20 @@ def make_inputs(wl: Workload, device="cpu", seed: Optional[int] = None) -> torch
     return out
 
 
+def make_targets(wl: Workload, device="cpu", seed: Optional[int] = None) -> torch.Tensor:
+    """Reconstruction targets [L, T, d_model] of the training-step workload: N(0, 1) per coordinate
+    times a per-dimension scale ~ LogNormal(0, 0.5), standardised per layer."""
+    device = torch.device(device)
+    dtype = getattr(torch, wl.dtype)
+    g = _gen(device, 1090 + wl.index if seed is None else seed + 90)
+    L, T, d = wl.num_layers, wl.tokens, wl.d_model
+    out = torch.empty(L, T, d, dtype=dtype, device=device)
+    for l in range(L):
+        y = torch.randn(T, d, generator=g, device=device) * torch.exp(0.5 * torch.randn(d, generator=g, device=device))
+        out[l] = ((y - y.mean()) / y.std()).to(dtype)
+    return out
+
+
 def make_state_dict(wl: Workload, device="cpu", seed: Optional[int] = None,
                     inputs: Optional[torch.Tensor] = None) -> Dict[str, torch.Tensor]:
     """Checkpoint-layout parameters (the keys ``CrossLayerTranscoder.state_dict()`` has)."""
