@@ -24,30 +24,39 @@ How each function is pinned (see ``tests/test_oracle_*.py``):
 * ``decode``  - additivity over sources (tests/unit/models/test_decoder.py:62-81),
   zero weights give zero output (tests/unit/models/test_tied_decoders.py:138-166),
   and a float64 numpy per-element loop on tiny shapes.
-* ``global_batchtopk``  - closed form of the z-score on hand-computable columns;
-  the reference has no golden numbers for it: PARITY UNPINNED beyond that
-  closed form (its tests only check shapes, test_clt_encode_decode.py:70-116).
+* ``global_batchtopk`` / ``global_tokentopk``  - closed form of the z-score on hand-computable
+  columns, and the reference's own outputs on seeded tiny models (the forward cases of
+  tests/golden/reference_fixtures.json, written by tests/golden/make_reference_fixtures.py).
 * ``theta_estimate_posthoc`` / ``theta_convert``  - a hand-computed two-feature case and the
   properties the reference's own test asserts (tests/unit/models/test_theta.py:110-175:
   thresholds finite and positive, higher for the features that were selected); the
-  reference holds no golden numbers for them: PARITY UNPINNED beyond that.
+  reference holds no golden numbers for them; pinned by the reference's own run on seeded tiny
+  models (theta_estimation cases of tests/golden/reference_fixtures.json).
 * ``JumpReLUFunction``  - the reference's table of input / threshold gradients
   (tests/unit/models/test_activations.py:318-381, 16 cases).
 * ``mse_loss_and_gradients``  - torch autograd itself computes the gradients; a central
   finite-difference check in float64 on a tiny model pins the loss / gradient pairing, and the
-  reference's backward tables (test_activations.py:114-152: grad * mask) pin the gate.
+  reference's backward tables (test_activations.py:114-152: grad * mask) pin the gate; the
+  reference's own loss and autograd gradients on seeded tiny models (gradients cases of
+  tests/golden/reference_fixtures.json: global BatchTopK, JumpReLU with its threshold gradient,
+  decoders tied per source and per target) pin the whole function.
 * ``sparsity_metrics`` / ``feature_density_metrics`` / ``reconstruction_metrics`` /
   ``dead_feature_update``  - hand-computed small cases, numpy's ``var`` in float64, and the
   closed forms (a perfect reconstruction has explained variance 1 and NMSE 0; an all-zero
-  reconstruction of a zero-mean target has NMSE 1); the reference has no test of its evaluator:
-  PARITY UNPINNED beyond that.
+  reconstruction of a zero-mean target has NMSE 1); the reference has no test of its evaluator, so
+  ``sparsity_metrics`` / ``feature_density_metrics`` / ``reconstruction_metrics`` are also checked
+  against the reference's own methods run on a seeded case (evaluator section of
+  tests/golden/reference_fixtures.json); ``dead_feature_update`` restates trainer code that cannot be
+  imported here (it needs wandb): PARITY UNPINNED beyond the hand-computed case.
 * ``store_parse_batch``  - a hand-written two-chunk case with every expected row spelled out, the
   ordering property of the reference's own test (tests/unit/data/test_data_integrity.py:215-294:
   every row once, identified by a value that encodes its position) and its normalisation test
   (:137-213: statistics of the normalised batch, same generator and seed); the reference's store
   tests need h5py files, which this image cannot write: PARITY UNPINNED beyond that.
-* ``forward``  - composition of the above; the reference has no golden tensors
-  for a full forward: PARITY UNPINNED beyond shape/keys and the pins of its parts.
+* ``forward``  - composition of the above; pinned by the reference's own reconstructions and
+  activations on six seeded tiny models (global BatchTopK / TokenTopK, JumpReLU, ReLU; untied,
+  per-source and per-target decoders; skip connections; feature offset / scale) in
+  tests/golden/reference_fixtures.json.
 
 Tie rule.  ``torch.topk(sorted=False)`` leaves the choice among equal ranking
 values unspecified (reference activations.py:28).  This oracle fixes it the way

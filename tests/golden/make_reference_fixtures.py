@@ -1,0 +1,151 @@
+#!/usr/bin/env python3
+"""Writes tests/golden/reference_fixtures.json: inputs, parameters and outputs of tiny seeded runs of
+the reference's own code, for the functions that nothing else pins (full forward wiring, the global
+BatchTopK / TokenTopK helper, post-hoc theta estimation, gradients of the reconstruction loss, the
+evaluator's metric formulas).
+
+Runs only where the reference checkout is present (default /root/reference, or the path given as
+the first argument); it imports the reference on the CPU and nothing else.  The JSON it writes is
+data only and is what travels: the tests read the JSON, never the reference.
+
+    python tests/golden/make_reference_fixtures.py [/path/to/reference]
+"""
+import json
+import os
+import sys
+
+import torch
+
+sys.dont_write_bytecode = True     # the reference checkout is read-only for this build: no __pycache__ there
+REF = sys.argv[1] if len(sys.argv) > 1 else "/root/reference"
+sys.path.insert(0, REF)
+
+from clt.config import CLTConfig, TrainingConfig          # noqa: E402
+from clt.models.clt import CrossLayerTranscoder           # noqa: E402
+from clt.training.evaluator import CLTEvaluator           # noqa: E402
+from clt.training.losses import LossManager               # noqa: E402
+
+torch.set_num_threads(1)
+CPU = torch.device("cpu")
+
+
+def lists(obj):
+    if isinstance(obj, torch.Tensor):
+        return obj.detach().to(torch.float64).tolist()
+    if isinstance(obj, dict):
+        return {str(k): lists(v) for k, v in obj.items()}
+    if isinstance(obj, (list, tuple)):
+        return [lists(v) for v in obj]
+    return obj
+
+
+def build(cfg_kw, seed):
+    torch.manual_seed(seed)
+    cfg = CLTConfig(**cfg_kw)
+    model = CrossLayerTranscoder(cfg, process_group=None, device=CPU)
+    g = torch.Generator().manual_seed(seed + 1)
+    with torch.no_grad():
+        for name, p in model.named_parameters():
+            if name.endswith("log_threshold"):
+                p.copy_(torch.log(0.05 + 0.3 * torch.rand(p.shape, generator=g)))
+            elif "feature_scale" in name:
+                p.copy_(0.5 + torch.rand(p.shape, generator=g))
+            else:
+                p.copy_(torch.randn(p.shape, generator=g) * 0.4)
+    model.eval()
+    return cfg, model, g
+
+
+def forward_case(name, cfg_kw, seed, tokens=5):
+    cfg, model, g = build(cfg_kw, seed)
+    L, d = cfg.num_layers, cfg.d_model
+    inputs = {l: torch.randn(tokens, d, generator=g) for l in range(L)}
+    with torch.no_grad():
+        recs = model(inputs)
+        acts = model.get_feature_activations(inputs)
+    return {"name": name, "config": cfg_kw, "state_dict": lists(dict(model.state_dict())), "inputs": lists(inputs),
+            "reconstructions": lists(recs), "activations": lists(acts)}
+
+
+def theta_case(cfg_kw, seed, tokens=6, batches=3):
+    cfg, model, g = build(cfg_kw, seed)
+    L, d = cfg.num_layers, cfg.d_model
+    data = [({l: torch.randn(tokens, d, generator=g) for l in range(L)},
+             {l: torch.randn(tokens, d, generator=g) for l in range(L)}) for _ in range(batches)]
+    sd_before = lists(dict(model.state_dict()))
+    theta = model.estimate_theta_posthoc(iter(data), num_batches=batches, default_theta_value=1e6, device=CPU)
+    return {"config": cfg_kw, "state_dict": sd_before, "batches": [lists(b[0]) for b in data],
+            "theta": lists(theta), "log_threshold_after": lists(model.log_threshold),
+            "activation_fn_after": model.config.activation_fn}
+
+
+def gradient_case(name, cfg_kw, seed, tokens=6):
+    cfg, model, g = build(cfg_kw, seed)
+    model.train()
+    L, d = cfg.num_layers, cfg.d_model
+    inputs = {l: torch.randn(tokens, d, generator=g) for l in range(L)}
+    targets = {l: torch.randn(tokens, d, generator=g) for l in range(L)}
+    tc = TrainingConfig(learning_rate=1e-4, training_steps=10, activation_source="local_manifest",
+                        activation_path="unused", normalization_method="none")
+    lm = LossManager(tc, clt_config=cfg)
+    loss = lm.compute_reconstruction_loss(model(inputs), targets)
+    loss.backward()
+    grads = {n: p.grad for n, p in model.named_parameters() if p.grad is not None}
+    return {"name": name, "config": cfg_kw, "state_dict": lists(dict(model.state_dict())), "inputs": lists(inputs),
+            "targets": lists(targets), "loss": float(loss), "gradients": lists(grads)}
+
+
+def evaluator_case(seed):
+    cfg_kw = dict(num_features=12, num_layers=2, d_model=6, activation_fn="relu")
+    cfg, model, g = build(cfg_kw, seed)
+    acts = {l: torch.relu(torch.randn(7, 12, generator=g) - 0.3) for l in range(2)}
+    acts[1][:, 4] = 0.0
+    acts[0][2, 1] = 5e-7
+    targets = {l: torch.randn(7, 6, generator=g) * (1 + l) + 0.5 for l in range(2)}
+    recs = {l: targets[l] + 0.3 * torch.randn(7, 6, generator=g) for l in range(2)}
+    mean = {l: torch.randn(1, 6, generator=g) for l in range(2)}
+    std = {l: torch.rand(1, 6, generator=g) + 0.5 for l in range(2)}
+    out = {"activations": lists(acts), "targets": lists(targets), "reconstructions": lists(recs), "mean_tg": lists(mean),
+           "std_tg": lists(std), "num_features": 12, "num_layers": 2, "d_model": 6, "metrics": {}}
+    for method in ("none", "mean_std", "sqrt_d_model"):
+        ev = CLTEvaluator(model, CPU, mean_tg=mean, std_tg=std, normalization_method=method, d_model=6)
+        m = {}
+        m.update(ev._compute_sparsity(acts))
+        m.update(ev._compute_feature_density(acts))
+        m.update(ev._compute_reconstruction_metrics(targets, recs))
+        out["metrics"][method] = lists(m)
+    return out
+
+
+def main():
+    base = dict(num_features=16, num_layers=3, d_model=8)
+    fixtures = {"_about": "Produced by tests/golden/make_reference_fixtures.py from the reference's own code on the CPU "
+                          "(fp32, tiny shapes, fixed seeds).  Data only.",
+                "forward": [
+                    forward_case("batchtopk-global", dict(base, activation_fn="batchtopk", batchtopk_k=3), 11),
+                    forward_case("tokentopk-global", dict(base, activation_fn="topk", topk_k=4), 12),
+                    forward_case("jumprelu", dict(base, activation_fn="jumprelu"), 13),
+                    forward_case("relu-per-target-affine-skip", dict(base, activation_fn="relu", decoder_tying="per_target",
+                                                                     enable_feature_offset=True, enable_feature_scale=True,
+                                                                     skip_connection=True), 14),
+                    forward_case("batchtopk-global-per-source", dict(base, activation_fn="batchtopk", batchtopk_k=3,
+                                                                     decoder_tying="per_source"), 15),
+                    forward_case("relu-untied-skip", dict(base, activation_fn="relu", skip_connection=True), 16),
+                ],
+                "theta_estimation": [theta_case(dict(base, activation_fn="batchtopk", batchtopk_k=3), 21),
+                                     theta_case(dict(base, activation_fn="topk", topk_k=4), 22)],
+                "gradients": [
+                    gradient_case("batchtopk-global", dict(base, activation_fn="batchtopk", batchtopk_k=3), 31),
+                    gradient_case("jumprelu", dict(base, activation_fn="jumprelu"), 32),
+                    gradient_case("relu-per-source", dict(base, activation_fn="relu", decoder_tying="per_source"), 33),
+                    gradient_case("relu-per-target", dict(base, activation_fn="relu", decoder_tying="per_target"), 34),
+                ],
+                "evaluator": evaluator_case(41)}
+    out = os.path.join(os.path.dirname(os.path.abspath(__file__)), "reference_fixtures.json")
+    with open(out, "w") as f:
+        json.dump(fixtures, f)
+    print("wrote", out, os.path.getsize(out), "bytes")
+
+
+if __name__ == "__main__":
+    main()

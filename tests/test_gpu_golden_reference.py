@@ -1,0 +1,91 @@
+"""The HIP path against tests/golden/reference_fixtures.json (tiny seeded runs of the reference's own
+code, fp32): full forward for every tying / skip / affine variant, global BatchTopK / TokenTopK, post-hoc
+theta estimation, gradients of the reconstruction loss, evaluator metrics."""
+import json
+import math
+import os
+
+import pytest
+import torch
+
+import crosslayer_coding_amd as cca
+
+pytestmark = pytest.mark.gpu
+
+FIX = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_fixtures.json")))
+
+
+def T(x, dev=None):
+    return torch.tensor(x, dtype=torch.float32, device=dev)
+
+
+def load_model(case, dev):
+    model = cca.CrossLayerTranscoder(cca.CLTConfig(**case["config"]), None, dev)
+    model.load_state_dict({k: T(v) for k, v in case["state_dict"].items()})
+    return model
+
+
+@pytest.mark.parametrize("case", FIX["forward"], ids=lambda c: c["name"])
+def test_forward_matches_the_reference(dev, case):
+    model = load_model(case, dev)
+    model.eval()
+    inputs = {int(l): T(v, dev) for l, v in case["inputs"].items()}
+    recs = model(inputs)
+    acts = model.get_feature_activations(inputs)
+    for l in range(case["config"]["num_layers"]):
+        want_a, want_r = T(case["activations"][str(l)]), T(case["reconstructions"][str(l)])
+        assert torch.equal(acts[l].cpu() != 0, want_a != 0), f"selected set of layer {l}"
+        assert torch.allclose(acts[l].cpu(), want_a, rtol=1e-5, atol=1e-6)
+        assert torch.allclose(recs[l].cpu(), want_r, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("case", FIX["theta_estimation"], ids=lambda c: c["config"]["activation_fn"])
+def test_theta_estimation_matches_the_reference(dev, case):
+    model = load_model(case, dev)
+    data = [({int(l): T(v, dev) for l, v in b.items()}, None) for b in case["batches"]]
+    theta = model.estimate_theta_posthoc(iter(data), num_batches=len(data), default_theta_value=1e6)
+    assert model.config.activation_fn == case["activation_fn_after"]
+    assert torch.allclose(theta.cpu().float(), T(case["theta"]), rtol=1e-4, atol=1e-6)
+    assert torch.allclose(model.log_threshold.detach().cpu().float(), T(case["log_threshold_after"]), rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("case", FIX["gradients"], ids=lambda c: c["name"])
+def test_gradients_match_the_reference(dev, case):
+    model = load_model(case, dev)
+    inputs = {int(l): T(v, dev) for l, v in case["inputs"].items()}
+    targets = {int(l): T(v, dev) for l, v in case["targets"].items()}
+    loss, grads = model.loss_and_gradients(inputs, targets)
+    assert float(loss) == pytest.approx(case["loss"], rel=1e-5)
+    for name, want in case["gradients"].items():
+        assert grads.get(name) is not None, name
+        assert torch.allclose(grads[name].cpu(), T(want), rtol=1e-4, atol=1e-6), name
+
+
+@pytest.mark.parametrize("method", ["none", "mean_std", "sqrt_d_model"])
+def test_evaluator_metrics_match_the_reference(dev, method):
+    ev = FIX["evaluator"]
+    cfg = cca.CLTConfig(num_features=ev["num_features"], num_layers=ev["num_layers"], d_model=ev["d_model"], activation_fn="relu")
+    evaluator = cca.CLTEvaluator(cca.CrossLayerTranscoder(cfg, None, dev), dev,
+                                 mean_tg={int(l): T(v) for l, v in ev["mean_tg"].items()},
+                                 std_tg={int(l): T(v) for l, v in ev["std_tg"].items()},
+                                 normalization_method=method, d_model=ev["d_model"])
+    acts = {int(l): T(v, dev) for l, v in ev["activations"].items()}
+    got = {**evaluator._compute_sparsity(acts), **evaluator._compute_feature_density(acts),
+           **evaluator._compute_reconstruction_metrics({int(l): T(v, dev) for l, v in ev["targets"].items()},
+                                                       {int(l): T(v, dev) for l, v in ev["reconstructions"].items()})}
+    want = ev["metrics"][method]
+    assert got.keys() == want.keys()
+
+    def same(a, b, path):
+        if isinstance(b, dict):
+            assert a.keys() == b.keys(), path
+            for k in b:
+                same(a[k], b[k], f"{path}/{k}")
+        elif isinstance(b, list):
+            assert len(a) == len(b), path
+            for i, (x, y) in enumerate(zip(a, b)):
+                same(x, y, f"{path}[{i}]")
+        else:
+            assert a == pytest.approx(b, rel=1e-5, abs=1e-7) or (math.isinf(a) and math.isinf(b)), (path, a, b)
+
+    same(got, want, method)
