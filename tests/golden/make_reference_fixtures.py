@@ -21,6 +21,7 @@ REF = sys.argv[1] if len(sys.argv) > 1 else "/root/reference"
 sys.path.insert(0, REF)
 
 from clt.config import CLTConfig, TrainingConfig          # noqa: E402
+from clt.models.activations import _apply_batch_topk_helper, _apply_token_topk_helper   # noqa: E402
 from clt.models.clt import CrossLayerTranscoder           # noqa: E402
 from clt.training.evaluator import CLTEvaluator           # noqa: E402
 from clt.training.losses import LossManager               # noqa: E402
@@ -117,6 +118,28 @@ def evaluator_case(seed):
     return out
 
 
+def global_select_case(dtype, seed, L=3, tokens=16, F=32, k=5, kk=6):
+    """The global helpers fed pre-activations directly, in ``dtype``: pins the rounding sequence of the
+    ranking values.  Seeds whose k-th and (k+1)-th ranking values coincide are skipped, because
+    torch.topk's choice among equal values is unspecified."""
+    while True:
+        g = torch.Generator().manual_seed(seed)
+        pre = {l: (torch.randn(tokens, F, generator=g) * (0.5 + l) + 0.3 * l).to(dtype) for l in range(L)}
+        z = torch.cat([(p - p.mean(dim=0, keepdim=True)) / (p.std(dim=0, keepdim=True) + 1e-6) for p in pre.values()], dim=1)
+        flat = torch.sort(z.float().reshape(-1), descending=True).values
+        rows = torch.sort(z.float(), dim=1, descending=True).values
+        if flat[k * tokens - 1] != flat[k * tokens] and bool((rows[:, kk - 1] != rows[:, kk]).all()):
+            break
+        seed += 1000
+    name = str(dtype).split(".")[-1]
+    cfg_b = CLTConfig(num_features=F, num_layers=L, d_model=8, activation_fn="batchtopk", batchtopk_k=k, clt_dtype=name)
+    cfg_t = CLTConfig(num_features=F, num_layers=L, d_model=8, activation_fn="topk", topk_k=float(kk), clt_dtype=name)
+    out_b = _apply_batch_topk_helper(pre, cfg_b, CPU, dtype, 0, None)
+    out_t = _apply_token_topk_helper(pre, cfg_t, CPU, dtype, 0, None)
+    return {"dtype": name, "seed": seed, "batchtopk_k": k, "topk_k": kk, "preactivations": lists(pre),
+            "batchtopk": lists(out_b), "tokentopk": lists(out_t)}
+
+
 def main():
     base = dict(num_features=16, num_layers=3, d_model=8)
     fixtures = {"_about": "Produced by tests/golden/make_reference_fixtures.py from the reference's own code on the CPU "
@@ -140,6 +163,7 @@ def main():
                     gradient_case("relu-per-source", dict(base, activation_fn="relu", decoder_tying="per_source"), 33),
                     gradient_case("relu-per-target", dict(base, activation_fn="relu", decoder_tying="per_target"), 34),
                 ],
+                "global_select": [global_select_case(torch.float32, 51), global_select_case(torch.bfloat16, 52)],
                 "evaluator": evaluator_case(41)}
     out = os.path.join(os.path.dirname(os.path.abspath(__file__)), "reference_fixtures.json")
     with open(out, "w") as f:

@@ -120,3 +120,16 @@ def test_oracle_evaluator_metrics_match_the_reference(method):
             assert a == pytest.approx(b, rel=1e-6, abs=1e-9) or (math.isinf(a) and math.isinf(b)), (path, a, b)
 
     same(got, want, method)
+
+
+@pytest.mark.parametrize("case", FIX["global_select"], ids=lambda c: c["dtype"])
+def test_oracle_global_selection_matches_the_reference_in_each_dtype(case):
+    # pre-activations handed over as they are: the selected set must be the reference's, bit for bit
+    dtype = getattr(torch, case["dtype"])
+    pre = {int(l): T(v).to(dtype) for l, v in case["preactivations"].items()}
+    L = len(pre)
+    got_b = orc.global_batchtopk(pre, L, case["batchtopk_k"])
+    got_t = orc.global_tokentopk(pre, L, float(case["topk_k"]))
+    for l in range(L):
+        assert torch.equal(got_b[l].float(), T(case["batchtopk"][str(l)])), ("batchtopk", l)
+        assert torch.equal(got_t[l].float(), T(case["tokentopk"][str(l)])), ("tokentopk", l)

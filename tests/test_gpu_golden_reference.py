@@ -89,3 +89,18 @@ def test_evaluator_metrics_match_the_reference(dev, method):
             assert a == pytest.approx(b, rel=1e-5, abs=1e-7) or (math.isinf(a) and math.isinf(b)), (path, a, b)
 
     same(got, want, method)
+
+
+@pytest.mark.parametrize("case", FIX["global_select"], ids=lambda c: c["dtype"])
+def test_global_selection_matches_the_reference_in_each_dtype(dev, case):
+    # the reference's global helpers were fed these pre-activations directly; so are the kernels
+    # (column statistics + selection ranked on the z-score): same survivors, same values, bit for bit
+    from crosslayer_coding_amd import engine
+    dtype = getattr(torch, case["dtype"])
+    L = len(case["preactivations"])
+    pre = torch.stack([T(case["preactivations"][str(l)]).to(dtype) for l in range(L)]).to(dev).contiguous()
+    got_b = engine.densify(engine.batchtopk_select(pre, case["batchtopk_k"], True))
+    got_t = engine.densify(engine.tokentopk_select(pre, case["topk_k"], True))
+    for l in range(L):
+        assert torch.equal(got_b[l].float().cpu(), T(case["batchtopk"][str(l)])), ("batchtopk", l)
+        assert torch.equal(got_t[l].float().cpu(), T(case["tokentopk"][str(l)])), ("tokentopk", l)
