@@ -60,12 +60,16 @@ def build(cfg_kw, seed):
 def forward_case(name, cfg_kw, seed, tokens=5):
     cfg, model, g = build(cfg_kw, seed)
     L, d = cfg.num_layers, cfg.d_model
-    inputs = {l: torch.randn(tokens, d, generator=g) for l in range(L)}
+    dtype = next(model.parameters()).dtype
+    inputs = {l: torch.randn(tokens, d, generator=g).to(dtype) for l in range(L)}
     with torch.no_grad():
         recs = model(inputs)
         acts = model.get_feature_activations(inputs)
+        pre = {l: model.get_preactivations(inputs[l], l) for l in range(L)}
+        norms = model.get_decoder_norms()
     return {"name": name, "config": cfg_kw, "state_dict": lists(dict(model.state_dict())), "inputs": lists(inputs),
-            "reconstructions": lists(recs), "activations": lists(acts)}
+            "reconstructions": lists(recs), "activations": lists(acts), "preactivations": lists(pre),
+            "decoder_norms": lists(norms)}
 
 
 def theta_case(cfg_kw, seed, tokens=6, batches=3):
@@ -154,6 +158,13 @@ def main():
                     forward_case("batchtopk-global-per-source", dict(base, activation_fn="batchtopk", batchtopk_k=3,
                                                                      decoder_tying="per_source"), 15),
                     forward_case("relu-untied-skip", dict(base, activation_fn="relu", skip_connection=True), 16),
+                    # bf16 on the CPU: sums run in another order than on the GPU, so these are held to the
+                    # rel-L2 tolerance of the bf16 path, not to equality
+                    forward_case("jumprelu-bf16", dict(num_features=32, num_layers=3, d_model=16, activation_fn="jumprelu",
+                                                       clt_dtype="bfloat16"), 17, tokens=16),
+                    forward_case("batchtopk-global-bf16", dict(num_features=32, num_layers=3, d_model=16,
+                                                               activation_fn="batchtopk", batchtopk_k=4,
+                                                               clt_dtype="bfloat16"), 18, tokens=16),
                 ],
                 "theta_estimation": [theta_case(dict(base, activation_fn="batchtopk", batchtopk_k=3), 21),
                                      theta_case(dict(base, activation_fn="topk", topk_k=4), 22)],

@@ -50,14 +50,27 @@ def model_kwargs(cfg, sd, L, tying, names):
 @pytest.mark.parametrize("case", FIX["forward"], ids=lambda c: c["name"])
 def test_oracle_forward_matches_the_reference(case):
     cfg, sd, L, tying, names, kw = unpack(case)
-    inputs = {int(l): T(v) for l, v in case["inputs"].items()}
-    recs, acts = orc.forward(inputs, **kw, dtype=torch.float32, d_model=cfg["d_model"], num_features=cfg["num_features"],
-                             topk_mode="global", **model_kwargs(cfg, sd, L, tying, names))
+    dtype = getattr(torch, cfg.get("clt_dtype", "float32"))
+    if dtype != torch.float32:
+        kw = {k: ([w.to(dtype) for w in v] if isinstance(v, list) else {n: w.to(dtype) for n, w in v.items()}) for k, v in kw.items()}
+    inputs = {int(l): T(v).to(dtype) for l, v in case["inputs"].items()}
+    extra = model_kwargs(cfg, sd, L, tying, names)
+    recs, acts = orc.forward(inputs, **kw, dtype=dtype, d_model=cfg["d_model"], num_features=cfg["num_features"],
+                             topk_mode="global", **extra)
     for l in range(L):
         want_a, want_r = T(case["activations"][str(l)]), T(case["reconstructions"][str(l)])
-        assert torch.equal(acts[l] != 0, want_a != 0), f"selected set of layer {l}"
-        assert torch.allclose(acts[l], want_a, rtol=1e-5, atol=1e-6)
-        assert torch.allclose(recs[l], want_r, rtol=1e-5, atol=1e-5)
+        pre = orc.encoder_preactivations(inputs[l], kw["enc_w"][l], kw["enc_b"][l])
+        if dtype == torch.float32:
+            assert torch.allclose(pre, T(case["preactivations"][str(l)]), rtol=1e-5, atol=1e-6)
+            assert torch.equal(acts[l] != 0, want_a != 0), f"selected set of layer {l}"
+            assert torch.allclose(acts[l], want_a, rtol=1e-5, atol=1e-6)
+            assert torch.allclose(recs[l], want_r, rtol=1e-5, atol=1e-5)
+        else:   # the same torch-CPU ops on the same bf16 values: equal
+            assert torch.equal(pre.float(), T(case["preactivations"][str(l)]))
+            assert torch.equal(acts[l].float(), want_a)
+            assert orc.rel_l2(recs[l].float(), want_r) <= 1e-2
+    got_n = orc.decoder_norms(kw["dec_w"], L, cfg["num_features"], tying, dtype).float()
+    assert torch.allclose(got_n, T(case["decoder_norms"]), rtol=2e-2 if dtype != torch.float32 else 1e-5, atol=1e-6)
 
 
 @pytest.mark.parametrize("case", FIX["theta_estimation"], ids=lambda c: c["config"]["activation_fn"])
