@@ -276,27 +276,77 @@ __global__ __launch_bounds__(BW_THREADS) void k_csc_count(const int32_t *row_ptr
   }
 }
 
-// single block: ptr = exclusive scan of cnt (n entries), ptr[n] = total; cnt is reset to zero (it
-// serves as the fill cursor next)
-__global__ __launch_bounds__(1024) void k_csc_scan(uint32_t *cnt, int64_t n, int32_t *ptr) {
-  __shared__ unsigned long long ws[16];
-  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
-  const int64_t per = (n + 1023) / 1024, b = (int64_t)tid * per, e = b + per < n ? b + per : n;
+// ptr = exclusive scan of cnt (n entries), ptr[n] = total; cnt is reset to zero (it serves as the
+// fill cursor next).  Three steps over chunks of CSC_CHUNK counters: chunk sums, a scan of the
+// sums in one block, and the scan inside every chunk from its offset; all accesses coalesced.
+constexpr int CSC_CHUNK = 4096;
+__global__ __launch_bounds__(BW_THREADS) void k_csc_chunk_sum(const uint32_t *cnt, int64_t n, unsigned long long *sums) {
+  __shared__ unsigned long long red[BW_THREADS / 64];
+  const int64_t base = (int64_t)blockIdx.x * CSC_CHUNK;
   unsigned long long s = 0;
-  for (int64_t i = b; i < e; ++i) s += cnt[i];
-  unsigned long long inc = s;
+  for (int i = threadIdx.x; i < CSC_CHUNK; i += BW_THREADS)
+    if (base + i < n) s += cnt[base + i];
 #pragma unroll
-  for (int o = 1; o < 64; o <<= 1) {
-    unsigned long long y = __shfl_up(inc, o);
-    if (lane >= o) inc += y;
-  }
-  if (lane == 63) ws[wv] = inc;
+  for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
   __syncthreads();
-  unsigned long long base = 0, tot = 0;
-  for (int i = 0; i < 16; ++i) { if (i < wv) base += ws[i]; tot += ws[i]; }
-  unsigned long long run = base + inc - s;
-  for (int64_t i = b; i < e; ++i) { ptr[i] = (int32_t)run; run += cnt[i]; cnt[i] = 0; }
-  if (tid == 0) ptr[n] = (int32_t)tot;
+  if (threadIdx.x == 0) {
+    unsigned long long t = 0;
+    for (int i = 0; i < BW_THREADS / 64; ++i) t += red[i];
+    sums[blockIdx.x] = t;
+  }
+}
+// one block: sums -> exclusive offsets in place; ptr[n] = total
+__global__ __launch_bounds__(BW_THREADS) void k_csc_chunk_offsets(unsigned long long *sums, int64_t nchunk, int32_t *ptr, int64_t n) {
+  __shared__ unsigned long long wsum[BW_THREADS / 64];
+  __shared__ unsigned long long carry_s;
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  if (threadIdx.x == 0) carry_s = 0;
+  __syncthreads();
+  for (int64_t b0 = 0; b0 < nchunk; b0 += BW_THREADS) {
+    const int64_t i = b0 + threadIdx.x;
+    const unsigned long long v = i < nchunk ? sums[i] : 0;
+    unsigned long long inc = v;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const unsigned long long y = __shfl_up(inc, o);
+      if (lane >= o) inc += y;
+    }
+    if (lane == 63) wsum[wv] = inc;
+    __syncthreads();
+    unsigned long long before = carry_s, total = 0;
+    for (int k = 0; k < BW_THREADS / 64; ++k) { if (k < wv) before += wsum[k]; total += wsum[k]; }
+    if (i < nchunk) sums[i] = before + inc - v;
+    __syncthreads();
+    if (threadIdx.x == 0) carry_s += total;
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) ptr[n] = (int32_t)carry_s;
+}
+__global__ __launch_bounds__(BW_THREADS) void k_csc_chunk_scan(uint32_t *cnt, int64_t n, const unsigned long long *offsets,
+                                                                int32_t *ptr) {
+  __shared__ uint32_t wsum[BW_THREADS / 64];
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int64_t base = (int64_t)blockIdx.x * CSC_CHUNK;
+  unsigned long long carry = offsets[blockIdx.x];
+  for (int it = 0; it < CSC_CHUNK / BW_THREADS; ++it) {
+    const int64_t i = base + (int64_t)it * BW_THREADS + threadIdx.x;
+    const uint32_t v = i < n ? cnt[i] : 0u;
+    uint32_t inc = v;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const uint32_t y = __shfl_up(inc, o);
+      if (lane >= o) inc += y;
+    }
+    if (lane == 63) wsum[wv] = inc;
+    __syncthreads();
+    uint32_t before = 0, total = 0;
+#pragma unroll
+    for (int k = 0; k < BW_THREADS / 64; ++k) { if (k < wv) before += wsum[k]; total += wsum[k]; }
+    if (i < n) { ptr[i] = (int32_t)(carry + before + inc - v); cnt[i] = 0u; }
+    carry += total;
+    __syncthreads();
+  }
 }
 
 __global__ __launch_bounds__(BW_THREADS) void k_csc_fill(const int32_t *row_ptr, const int32_t *col, int64_t Tn, int64_t F,
@@ -551,7 +601,8 @@ extern "C" int clt_decode_backward_values(const int32_t *row_ptr, const int32_t 
 
 extern "C" size_t clt_feature_lists_workspace_bytes(int64_t F, int64_t L) {
   if (F <= 0 || L <= 0) return 256;
-  return (size_t)L * (size_t)F * 4;
+  const size_t n = (size_t)L * (size_t)F;
+  return ((n * 4 + 255) & ~(size_t)255) + ((n + CSC_CHUNK - 1) / CSC_CHUNK) * 8;   // counters + chunk sums
 }
 
 extern "C" int clt_feature_lists(const int32_t *row_ptr, const int32_t *col, int64_t T, int64_t F, int64_t L,
@@ -560,13 +611,18 @@ extern "C" int clt_feature_lists(const int32_t *row_ptr, const int32_t *col, int
   if (T <= 0 || F <= 0 || L <= 0 || L > 65535 || !row_ptr || !list_ptr || !workspace) return CLT_ERR_ARG;
   if ((double)L * (double)F >= 2147483647.0) return CLT_ERR_RANGE;
   if (workspace_bytes < clt_feature_lists_workspace_bytes(F, L)) return CLT_ERR_WORKSPACE;
+  if ((((uintptr_t)workspace) & 7u) != 0) return CLT_ERR_ALIGN;
   hipStream_t s = (hipStream_t)stream;
   uint32_t *cnt = (uint32_t *)workspace;
   const int64_t n = L * F;
   const unsigned nb = 256 * 8;
   k_zero_u32<<<nb, BW_THREADS, 0, s>>>(cnt, n);
   k_csc_count<<<nb, BW_THREADS, 0, s>>>(row_ptr, col, T, F, L, cnt);
-  k_csc_scan<<<1, 1024, 0, s>>>(cnt, n, list_ptr);
+  const int64_t nchunk = clt_ceil_div(n, CSC_CHUNK);
+  unsigned long long *sums = (unsigned long long *)((char *)workspace + (((size_t)n * 4 + 255) & ~(size_t)255));
+  k_csc_chunk_sum<<<(unsigned)nchunk, BW_THREADS, 0, s>>>(cnt, n, sums);
+  k_csc_chunk_offsets<<<1, BW_THREADS, 0, s>>>(sums, nchunk, list_ptr, n);
+  k_csc_chunk_scan<<<(unsigned)nchunk, BW_THREADS, 0, s>>>(cnt, n, sums, list_ptr);
   if (list_tok && list_src) {
     k_csc_fill<<<nb, BW_THREADS, 0, s>>>(row_ptr, col, T, F, L, list_ptr, cnt, list_tok, list_src);
     k_csc_order<<<nb, BW_THREADS, 0, s>>>(list_ptr, n, list_tok, list_src);
