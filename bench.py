@@ -250,6 +250,56 @@ def run_theta(args):
     }
 
 
+def run_probe(args):
+    """Calibration of the gather-bound stages: a bare gather of 1536-byte rows (the decoder row of C1)
+    from tables of growing size, timed with events.  Every XCD reads the whole table, so the table
+    size is each L2's working set: 2-3 MB fit the 4 MB L2, 4.7 MB is the decoder slice one XCD works on
+    at C1, 64 MB fits the memory-side cache, 4 GB neither."""
+    import crosslayer_coding_amd as cca
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    lib = cca._native.load(build_if_missing=False)
+    row_bytes, n_idx = 1536, 5_400_000                      # one decode launch at C1 gathers 5.3 M rows
+    stream = torch.cuda.current_stream().cuda_stream
+    g = torch.Generator(device=dev).manual_seed(0)
+    results = {}
+    for label, table_bytes in (("2 MB", 2 << 20), ("3 MB", 3 << 20), ("4 MB", 4 << 20), ("4.7 MB", 4928307), ("6 MB", 6 << 20),
+                               ("64 MB", 64 << 20), ("4 GB", 4 << 30)):
+        n_rows = table_bytes // row_bytes
+        table = torch.randint(0, 1 << 30, (n_rows * row_bytes // 4,), dtype=torch.int32, device=dev, generator=g)
+        idx = torch.randint(0, n_rows, (n_idx,), dtype=torch.int32, device=dev, generator=g)
+        best, best_lds = None, None
+        for to_lds in (0, 1):
+            moved = row_bytes if not to_lds else 2048
+            for blocks in (256 * 2, 256 * 4, 256 * 8, 256 * 16):
+                out = torch.empty(blocks * 256, dtype=torch.float32, device=dev)
+                for _ in range(2):
+                    rc = lib.clt_probe_gather(table.data_ptr(), n_rows, row_bytes, idx.data_ptr(), n_idx, blocks, to_lds,
+                                              out.data_ptr(), stream)
+                    assert rc == 0
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+                for _ in range(args.steps):
+                    lib.clt_probe_gather(table.data_ptr(), n_rows, row_bytes, idx.data_ptr(), n_idx, blocks, to_lds,
+                                         out.data_ptr(), stream)
+                b.record()
+                b.synchronize()
+                gbs = n_idx * moved * args.steps / (a.elapsed_time(b) * 1e-3) / 1e9
+                if to_lds:
+                    if best_lds is None or gbs > best_lds[0]:
+                        best_lds = (gbs, blocks)
+                elif best is None or gbs > best[0]:
+                    best = (gbs, blocks)
+        results[label] = {"GB/s": best[0], "blocks": best[1], "direct_to_lds_GB/s": best_lds[0], "direct_to_lds_blocks": best_lds[1]}
+        del table, idx
+    top = results["2 MB"]["GB/s"]
+    return {"metric": "bare gather of 1536-byte rows, best of three grid sizes", "value": top, "unit": "GB/s", "n_gpus": 1,
+            "steps": args.steps, "warmup": 2, "ms_per_step": n_idx * row_bytes / top / 1e6, "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+            "config": {"workload": "gather probe: 5.4 M random rows of 1536 bytes per launch"}, "tables": results}
+
+
 def run_feed(args):
     """Activation-store feed (reference clt/training/data/manifest_activation_store.py:776-958): one step =
     one batch of T random rows drawn from 8 chunks of 8192 rows, gathered, normalised (mean / std) and cast
@@ -512,6 +562,8 @@ def main():
                          "selection, per-feature minimum) instead of the forward")
     ap.add_argument("--backward", action="store_true",
                     help="time forward + MSE loss + all gradients (loss_and_gradients) instead of the forward")
+    ap.add_argument("--gather-probe", action="store_true",
+                    help="calibration: the rate a bare row gather reaches from L2-, cache- and HBM-sized tables")
     ap.add_argument("--feed", action="store_true",
                     help="time the activation-store feed (gather + normalise + cast into the batch slabs)")
     ap.add_argument("--evaluator", action="store_true",
@@ -528,7 +580,7 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a ROCm GPU", file=sys.stderr)
         sys.exit(2)
-    print(json.dumps(run_theta(args) if args.theta_estimation else run_evaluator(args) if args.evaluator else run_feed(args) if args.feed else run_backward(args) if (args.backward or args.train_step) else run_gpu(args)))
+    print(json.dumps(run_theta(args) if args.theta_estimation else run_evaluator(args) if args.evaluator else run_feed(args) if args.feed else run_probe(args) if args.gather_probe else run_backward(args) if (args.backward or args.train_step) else run_gpu(args)))
 
 
 if __name__ == "__main__":

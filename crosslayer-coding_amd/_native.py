@@ -67,6 +67,7 @@ _SIGNATURES = {
     "clt_decoder_norms": (_int, [_vp, _vp, _i64, _i64, _i64, _int, _int, _vp]),
     "clt_jumprelu_theta_grad_workspace_bytes": (_sz, [_i64]),
     "clt_jumprelu_theta_grad": (_int, [_vp, _vp, _vp, _i64, _i64, _f64, _int, _vp, _vp, _sz, _vp]),
+    "clt_probe_gather": (_int, [_vp, _i64, _i64, _vp, _i64, _i64, _int, _vp, _vp]),
     "clt_feed_gather": (_int, [_vp, _int, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _int, _vp, _vp, _vp, _vp, _f64, _vp, _vp,
                               _i64, _i64, _int, _vp]),
     "clt_survivor_metrics": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _int, ctypes.c_float, _vp, _vp, _vp]),

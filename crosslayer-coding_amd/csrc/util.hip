@@ -152,3 +152,70 @@ extern "C" int clt_colstats_full(const void *pre, float *mean, float *stdv, floa
   if (!stdv) return CLT_ERR_ARG;
   return run_colstats(pre, mean, denom, stdv, T, F, L, pre_layer_stride, dtype, stream);
 }
+
+// ---- calibration: what a row gather can reach on this GPU -------------------------------------------
+// Every wavefront sums the rows idx[...] of `table` ([n_rows][row_bytes], row_bytes a multiple of 16
+// and at most 2048), PROBE_U rows in flight, 16 bytes per lane and load - the access pattern of the
+// decode and backward gathers without any of their other work.  With a table that fits every XCD's L2
+// this measures the L2 -> CU rate of such a gather; with larger tables, the rate from the memory-side
+// cache and from HBM.  out [gridDim.x * 4 * 64] floats receives one value per lane so that the loads
+// cannot be dropped.
+namespace {
+constexpr int PROBE_U = 6;
+template <bool TO_LDS>
+__global__ __launch_bounds__(256) void k_probe_gather(const uint4 *__restrict__ table, int pieces, const int32_t *__restrict__ idx,
+                                                      int64_t n_idx, float *__restrict__ out) {
+  // TO_LDS: the same loads issued as direct-to-LDS loads (the encoder's way of bringing tiles in)
+  __shared__ __attribute__((aligned(16))) unsigned char lds[TO_LDS ? 4 * PROBE_U * 2 * 1024 : 16];
+  const int lane = lane_id(), wv = threadIdx.x >> 6;
+  const int64_t nwave = (int64_t)gridDim.x * 4, w = (int64_t)blockIdx.x * 4 + wv;
+  const int64_t per = (n_idx + nwave - 1) / nwave, b = w * per, e = b + per < n_idx ? b + per : n_idx;
+  const bool on1 = lane + 64 < pieces, on0 = lane < pieces;
+  uint32_t acc = 0;
+  for (int64_t i0 = b; i0 < e; i0 += 64) {
+    const int n = (e - i0) < 64 ? (int)(e - i0) : 64;
+    const int32_t mine = lane < n ? idx[i0 + lane] : 0;
+    for (int i = 0; i < n; i += PROBE_U) {
+      if constexpr (TO_LDS) {
+        unsigned char *mybuf = lds + wv * (PROBE_U * 2 * 1024);
+#pragma unroll
+        for (int u = 0; u < PROBE_U; ++u) {
+          const int k = i + u < n ? i + u : n - 1;
+          const uint4 *row = table + (int64_t)__builtin_amdgcn_readlane(mine, k) * pieces;
+          // whole 1-KB groups only: a row of 1536 bytes is fetched as 1 KB + the first 512 bytes again
+          __builtin_amdgcn_global_load_lds(row + lane, (__attribute__((address_space(3))) void *)(mybuf + u * 2048), 16, 0, 0);
+          __builtin_amdgcn_global_load_lds(row + (on1 ? lane + 64 : lane), (__attribute__((address_space(3))) void *)(mybuf + u * 2048 + 1024), 16, 0, 0);
+        }
+        __builtin_amdgcn_s_waitcnt(0);
+        acc += *reinterpret_cast<const uint32_t *>(mybuf + lane * 4);
+      } else {
+        uint4 v[PROBE_U][2];
+#pragma unroll
+        for (int u = 0; u < PROBE_U; ++u) {
+          const int k = i + u < n ? i + u : n - 1;
+          const uint4 *row = table + (int64_t)__builtin_amdgcn_readlane(mine, k) * pieces;
+          v[u][0] = on0 ? row[lane] : make_uint4(0, 0, 0, 0);
+          v[u][1] = on1 ? row[lane + 64] : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int u = 0; u < PROBE_U; ++u)
+          acc += v[u][0].x ^ v[u][0].y ^ v[u][0].z ^ v[u][0].w ^ v[u][1].x ^ v[u][1].y ^ v[u][1].z ^ v[u][1].w;
+      }
+    }
+  }
+  out[w * 64 + lane] = __uint_as_float(acc & 0x3FFFFFFFu);
+}
+}  // namespace
+
+extern "C" int clt_probe_gather(const void *table, int64_t n_rows, int64_t row_bytes, const int32_t *idx, int64_t n_idx,
+                                int64_t blocks, int to_lds, float *out, void *stream) {
+  if (!table || !idx || !out || n_rows <= 0 || n_idx <= 0 || blocks <= 0 || blocks > 1048576) return CLT_ERR_ARG;
+  if (row_bytes <= 0 || row_bytes % 16 != 0 || row_bytes > 2048 || !clt_aligned16(table)) return CLT_ERR_ARG;
+  if (to_lds) {
+    if (row_bytes < 1024) return CLT_ERR_ARG;   // the direct-to-LDS variant moves whole 1-KB groups
+    k_probe_gather<true><<<(unsigned)blocks, 256, 0, (hipStream_t)stream>>>((const uint4 *)table, (int)(row_bytes / 16), idx, n_idx, out);
+  } else {
+    k_probe_gather<false><<<(unsigned)blocks, 256, 0, (hipStream_t)stream>>>((const uint4 *)table, (int)(row_bytes / 16), idx, n_idx, out);
+  }
+  return clt_check_launch();
+}

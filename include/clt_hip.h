@@ -419,6 +419,20 @@ int clt_reconstruction_stats(const void *rec, const void *target, int64_t T, int
                              double scale, double *stats, void *workspace, size_t workspace_bytes,
                              void *stream);
 
+/* ---- calibration ------------------------------------------------------------------
+ * clt_probe_gather: no counterpart in the reference.  A bare row gather with the access pattern of
+ *   clt_decode_sparse (16 bytes per lane, six rows in flight per wavefront): every wavefront of
+ *   `blocks` workgroups (4 wavefronts each) sums its share of the rows idx[0..n_idx) of table
+ *   [n_rows][row_bytes] (row_bytes % 16 == 0, <= 2048; idx values must be in [0, n_rows)).
+ *   to_lds != 0 issues the same loads as direct-to-LDS loads (the encoder's way of bringing its
+ *   tiles in; row_bytes >= 1024, the bytes moved are then 2 KB per row).
+ *   out: blocks * 256 floats.  Timed with a table that fits an L2, the memory-side cache, or neither,
+ *   it gives the rate such a gather can reach on the GPU at hand - the yardstick bench.py prints
+ *   next to the decode stage.
+ */
+int clt_probe_gather(const void *table, int64_t n_rows, int64_t row_bytes, const int32_t *idx,
+                     int64_t n_idx, int64_t blocks, int to_lds, float *out, void *stream);
+
 /* ---- activation-store feed -----------------------------------------------------
  * clt_feed_gather: rows of one stored chunk -> rows [out_row0, out_row0 + n) of the batch slabs
  *   x_out, tgt_out [L][T][d] (out_dtype CLT_F32 / CLT_BF16), for all layers, inputs and targets.
