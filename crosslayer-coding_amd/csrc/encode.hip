@@ -203,6 +203,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   // the barrier the next stage may be read (its first fragments are fetched under the last
   // k-step's matrix ops) and the current one may be overwritten by the stage after next.
   const int nk = K / BK;
+  // K is walked from a tile-dependent starting stage, wrapping around: the CUs of an XCD that share an
+  // x tile or a W tile then ask for different lines of it at any one time, so one of them takes the
+  // L2 miss and the others find the line there later, instead of all of them queueing behind the miss.
+  const int rot = ((tiles_n & 7) == 0 ? 3 * tm + (tn >> 3) : tm + tn) % nk;
+  auto stage_k0 = [&](int kt) { int q = kt + rot; if (q >= nk) q -= nk; return q * BK; };
   uint4 fa[8], fb[8];   // [0..3] x fragments, [4..7] W fragments
   auto load_frags = [&](uint4 (&f)[8], const unsigned char *sb, int kk) {
 #pragma unroll
@@ -234,7 +239,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     __syncthreads();
     // past the end of K the last stage is fetched again (never read)
     const int kn = kt + 2 < nk ? kt + 2 : nk - 1;
-    issue_stage(cur, kn * BK);
+    issue_stage(cur, stage_k0(kn));
     load_frags(fa, nxt, 0);
     mma16(fb);
 #pragma unroll
@@ -244,10 +249,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
     }
   };
-  issue_stage(stage0, 0);
+  issue_stage(stage0, stage_k0(0));
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
-  issue_stage(stage1, BK);
+  issue_stage(stage1, stage_k0(1));
   load_frags(fa, stage0, 0);
   // nk is even (checked by the launcher).  The last two bodies fetch the final stage again and
   // read fragments that are never used: cheaper than a differently shaped last iteration.
