@@ -164,7 +164,7 @@ namespace {
 constexpr int PROBE_U = 6;
 template <bool TO_LDS>
 __global__ __launch_bounds__(256) void k_probe_gather(const uint4 *__restrict__ table, int pieces, const int32_t *__restrict__ idx,
-                                                      int64_t n_idx, float *__restrict__ out) {
+                                                      int64_t n_idx, float *__restrict__ out, int32_t n_rows) {
   // TO_LDS: the same loads issued as direct-to-LDS loads (the encoder's way of bringing tiles in)
   __shared__ __attribute__((aligned(16))) unsigned char lds[TO_LDS ? 4 * PROBE_U * 2 * 1024 : 16];
   const int lane = lane_id(), wv = threadIdx.x >> 6;
@@ -174,7 +174,8 @@ __global__ __launch_bounds__(256) void k_probe_gather(const uint4 *__restrict__ 
   uint32_t acc = 0;
   for (int64_t i0 = b; i0 < e; i0 += 64) {
     const int n = (e - i0) < 64 ? (int)(e - i0) : 64;
-    const int32_t mine = lane < n ? idx[i0 + lane] : 0;
+    int32_t mine = lane < n ? idx[i0 + lane] : 0;
+    mine = mine < 0 ? 0 : (mine >= n_rows ? n_rows - 1 : mine);   // an index outside the table is clamped, never followed
     for (int i = 0; i < n; i += PROBE_U) {
       if constexpr (TO_LDS) {
         unsigned char *mybuf = lds + wv * (PROBE_U * 2 * 1024);
@@ -209,13 +210,13 @@ __global__ __launch_bounds__(256) void k_probe_gather(const uint4 *__restrict__ 
 
 extern "C" int clt_probe_gather(const void *table, int64_t n_rows, int64_t row_bytes, const int32_t *idx, int64_t n_idx,
                                 int64_t blocks, int to_lds, float *out, void *stream) {
-  if (!table || !idx || !out || n_rows <= 0 || n_idx <= 0 || blocks <= 0 || blocks > 1048576) return CLT_ERR_ARG;
+  if (!table || !idx || !out || n_rows <= 0 || n_rows > 2147483647LL || n_idx <= 0 || blocks <= 0 || blocks > 1048576) return CLT_ERR_ARG;
   if (row_bytes <= 0 || row_bytes % 16 != 0 || row_bytes > 2048 || !clt_aligned16(table)) return CLT_ERR_ARG;
   if (to_lds) {
     if (row_bytes < 1024) return CLT_ERR_ARG;   // the direct-to-LDS variant moves whole 1-KB groups
-    k_probe_gather<true><<<(unsigned)blocks, 256, 0, (hipStream_t)stream>>>((const uint4 *)table, (int)(row_bytes / 16), idx, n_idx, out);
+    k_probe_gather<true><<<(unsigned)blocks, 256, 0, (hipStream_t)stream>>>((const uint4 *)table, (int)(row_bytes / 16), idx, n_idx, out, (int32_t)n_rows);
   } else {
-    k_probe_gather<false><<<(unsigned)blocks, 256, 0, (hipStream_t)stream>>>((const uint4 *)table, (int)(row_bytes / 16), idx, n_idx, out);
+    k_probe_gather<false><<<(unsigned)blocks, 256, 0, (hipStream_t)stream>>>((const uint4 *)table, (int)(row_bytes / 16), idx, n_idx, out, (int32_t)n_rows);
   }
   return clt_check_launch();
 }

@@ -423,7 +423,7 @@ int clt_reconstruction_stats(const void *rec, const void *target, int64_t T, int
  * clt_probe_gather: no counterpart in the reference.  A bare row gather with the access pattern of
  *   clt_decode_sparse (16 bytes per lane, six rows in flight per wavefront): every wavefront of
  *   `blocks` workgroups (4 wavefronts each) sums its share of the rows idx[0..n_idx) of table
- *   [n_rows][row_bytes] (row_bytes % 16 == 0, <= 2048; idx values must be in [0, n_rows)).
+ *   [n_rows][row_bytes] (row_bytes % 16 == 0, <= 2048; idx values outside [0, n_rows) are clamped).
  *   to_lds != 0 issues the same loads as direct-to-LDS loads (the encoder's way of bringing its
  *   tiles in; row_bytes >= 1024, the bytes moved are then 2 KB per row).
  *   out: blocks * 256 floats.  Timed with a table that fits an L2, the memory-side cache, or neither,

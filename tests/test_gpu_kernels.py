@@ -554,3 +554,20 @@ def test_decoder_norms(dev, dtype, tying):
     got = engine.decoder_norms(slab, L, tying).cpu()
     ref = orc.decoder_norms(w, L, F, tying, dtype)
     assert orc.rel_l2(got, ref) <= TOL[dtype]
+
+
+def test_gather_probe_runs_and_rejects_bad_arguments(dev):
+    # calibration entry point: results are not meaningful numbers, the call must just be safe
+    from crosslayer_coding_amd import _native as nat
+    lib = nat.load()
+    table = torch.arange(64 * 1536 // 4, dtype=torch.int32, device=dev)
+    idx = torch.tensor([0, 63, 5, 1 << 20, -3], dtype=torch.int32, device=dev)     # two indices outside the table: clamped
+    out = torch.empty(8 * 256, dtype=torch.float32, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    for to_lds in (0, 1):
+        assert lib.clt_probe_gather(table.data_ptr(), 64, 1536, idx.data_ptr(), 5, 8, to_lds, out.data_ptr(), stream) == 0
+    torch.cuda.synchronize()
+    assert torch.isfinite(out).all()
+    assert lib.clt_probe_gather(table.data_ptr(), 64, 1530, idx.data_ptr(), 5, 8, 0, out.data_ptr(), stream) != 0   # not 16-byte rows
+    assert lib.clt_probe_gather(table.data_ptr(), 64, 512, idx.data_ptr(), 5, 8, 1, out.data_ptr(), stream) != 0    # LDS variant needs >= 1 KB
+    assert lib.clt_probe_gather(None, 64, 1536, idx.data_ptr(), 5, 8, 0, out.data_ptr(), stream) != 0
