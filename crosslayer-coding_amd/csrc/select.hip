@@ -645,17 +645,20 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_select_allot(
   if (!GLOBAL && tid == 0 && p == (int)gridDim.x - 1) row_ptr[(int64_t)gridDim.x * Tn] = (int32_t)((unsigned long long)gridDim.x * K);
 }
 
-// Single block: row_ptr = exclusive scan of keep[] in storage order (row = layer*T + token).
+// Single block: row_ptr = exclusive scan of keep[] in storage order (row = layer*T + token), one
+// coalesced sweep of SCAN_THREADS rows at a time with a running carry.
 __global__ __launch_bounds__(SCAN_THREADS) void k_rowptr_scan(const uint32_t *keep, int64_t R, int32_t *row_ptr) {
   const int tid = threadIdx.x;
-  const int64_t per = (R + SCAN_THREADS - 1) / SCAN_THREADS;
-  const int64_t b = (int64_t)tid * per, e = b + per < R ? b + per : R;
-  unsigned long long s = 0;
-  for (int64_t i = b; i < e; ++i) s += keep[i];
-  unsigned long long tot;
-  unsigned long long run = block_excl_scan_u64(s, tot);
-  for (int64_t i = b; i < e; ++i) { row_ptr[i] = (int32_t)run; run += keep[i]; }
-  if (tid == 0) row_ptr[R] = (int32_t)tot;
+  unsigned long long carry = 0;
+  for (int64_t i0 = 0; i0 < R; i0 += SCAN_THREADS) {
+    const int64_t i = i0 + tid;
+    const unsigned long long v = i < R ? keep[i] : 0;
+    unsigned long long tot;
+    const unsigned long long before = carry + block_excl_scan_u64(v, tot);
+    if (i < R) row_ptr[i] = (int32_t)before;
+    carry += tot;
+  }
+  if (tid == 0) row_ptr[R] = (int32_t)carry;
 }
 
 // Ordered write of the survivors of each row.
