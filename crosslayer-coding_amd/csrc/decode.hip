@@ -215,6 +215,49 @@ __global__ __launch_bounds__(256) void k_decode(
     // next token is requested before the current token's rows are gathered.
     const int64_t tok0 = tok * SLICED_NTOK;
     if (tok0 >= Tn) return;
+    if (src < 0) {
+      // All sources in one launch (decoders tied per target: every source <= t gathers from the same
+      // matrix W[t], so the slice an XCD works on stays the same while the sources go by): the
+      // accumulators stay in registers over the sources and the partial row is written once.
+      const T *wb = wp + decoder_slot(tying, 0, t, L) * F * d;
+      for (int i = 0; i < SLICED_NTOK; ++i) {
+        if (tok0 + i >= Tn) break;
+#pragma unroll
+        for (int j = 0; j < NACC; ++j) acc[j] = 0.0f;
+        for (int64_t s = 0; s <= t; ++s) {
+          if (!((src_mask >> s) & 1ull)) continue;
+          const int64_t r = s * Tn + tok0 + i;
+          const int32_t b = sptr[r * (ns + 1) + slice], e = sptr[r * (ns + 1) + slice + 1];
+          for (int32_t j0 = b; j0 < e; j0 += 64) {
+            const int n = (e - j0) < 64 ? (e - j0) : 64;
+            int32_t my_col = 0; float my_val = 0.0f;
+            if (lane < n) { my_col = col[j0 + lane]; my_val = Elem<T>::to_f32(val[j0 + lane]); }
+            if (AFFINE && my_val != 0.0f) {
+              if (foff) my_val = Elem<T>::round(my_val + Elem<T>::to_f32(foff[t * F + my_col]));
+              if (fscale) my_val = Elem<T>::round(my_val * Elem<T>::to_f32(fscale[t * F + my_col]));
+            }
+            decode_chunk_pipelined<T, NF, TAIL, (U > 6 ? 6 : U)>(acc, wb, d, my_col, my_val, n, lane, tail_off, tail_on);
+          }
+        }
+        float *prow = partial + (((int64_t)slice * L + t) * Tn + tok0 + i) * d;
+#pragma unroll
+        for (int c = 0; c < NF; ++c) {
+          float *pp = prow + (int64_t)c * 64 * V + (int64_t)lane * V;
+#pragma unroll
+          for (int j = 0; j < V; j += 4)
+            stg_stream4(pp + j, make_float4(acc[c * V + j], acc[c * V + j + 1], acc[c * V + j + 2], acc[c * V + j + 3]));
+        }
+        if (TAIL == 1) {
+#pragma unroll
+          for (int j = 0; j < HV; ++j) prow[tail_off + j] = acc[NF * V + j];
+        }
+        if (TAIL == 2 && tail_on) {
+#pragma unroll
+          for (int j = 0; j < V; ++j) prow[tail_off + j] = acc[NF * V + j];
+        }
+      }
+      return;
+    }
     const uint64_t below = src_mask & ((1ull << src) - 1ull);
     const bool first = below == 0;   // the first source initialises the partial rows
     int32_t mb = 0, me = 0;
@@ -524,10 +567,16 @@ static int launch_decode(const int32_t *row_ptr, const int32_t *col, const void 
   } while (0)
   if (fast) {
     // sliced: one launch per source layer, targets max(src, t_begin) .. t_end-1
-    const int n_launch = can_slice ? (int)t_end : 1;
-    for (int src = 0; src < n_launch; ++src) {
+    // decoders tied per target: one launch, sources walked inside the wavefront (src = -1)
+    const bool all_src = can_slice && tying == CLT_TYING_PER_TARGET;
+    const int n_launch = all_src ? 1 : (can_slice ? (int)t_end : 1);
+    for (int src0 = 0; src0 < n_launch; ++src0) {
+      const int src = all_src ? -1 : src0;
       int64_t tb = t_begin;
-      if (can_slice) {
+      if (all_src) {
+        nblk = clt_ceil_div(Tn, nwv * SLICED_NTOK) * (t_end - tb) * ns;
+        if (nblk > 2147483647LL) return CLT_ERR_RANGE;
+      } else if (can_slice) {
         if (!((src_mask >> src) & 1ull)) continue;
         if (src > tb) tb = src;
         nblk = clt_ceil_div(Tn, nwv * SLICED_NTOK) * (t_end - tb) * ns;
