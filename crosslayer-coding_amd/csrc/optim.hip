@@ -21,7 +21,8 @@ __device__ __forceinline__ float adam_update(float p, float g, float &m, float &
 
 // parameter, gradient and moments in the same layout
 template <typename T>
-__global__ __launch_bounds__(256) void k_adam(T *p, const float *g, float *m, float *v, int64_t n, AdamCoef c) {
+__global__ __launch_bounds__(256) void k_adam(T *__restrict__ p, const float *__restrict__ g, float *__restrict__ m, float *__restrict__ v,
+                                              int64_t n, AdamCoef c) {
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
     float mi = m[i], vi = v[i];
     const float np = adam_update(Elem<T>::to_f32(p[i]), g[i], mi, vi, c);
@@ -59,7 +60,8 @@ __global__ __launch_bounds__(256) void k_adam_decoder(T *w_ref, T *w_packed, con
 // Vector version (d % 4 == 0, F % 4 == 0): a thread updates 4 consecutive elements of a feature row
 // (16-byte accesses to gradient and moments) and writes 4 consecutive features of a parameter row.
 template <typename T>
-__global__ __launch_bounds__(256) void k_adam_decoder_vec(T *w_ref, T *w_packed, const float *g, float *m, float *v,
+__global__ __launch_bounds__(256) void k_adam_decoder_vec(T *__restrict__ w_ref, T *__restrict__ w_packed, const float *__restrict__ g,
+                                                          float *__restrict__ m, float *__restrict__ v,
                                                           int64_t d, int64_t F, AdamCoef c) {
   __shared__ T tile[64][68];
   const int64_t f0 = (int64_t)blockIdx.x * 64, d0 = (int64_t)blockIdx.y * 64;
