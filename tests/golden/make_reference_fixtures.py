@@ -67,9 +67,13 @@ def forward_case(name, cfg_kw, seed, tokens=5):
         acts = model.get_feature_activations(inputs)
         pre = {l: model.get_preactivations(inputs[l], l) for l in range(L)}
         norms = model.get_decoder_norms()
+        # the per-layer entry points: encode(x, layer) and decode(activations up to a layer, layer)
+        encoded = {l: model.encode(inputs[l], l) for l in range(L)}
+        mid = L // 2
+        decoded_mid = model.decode({l: acts[l] for l in range(mid + 1)}, mid)
     return {"name": name, "config": cfg_kw, "state_dict": lists(dict(model.state_dict())), "inputs": lists(inputs),
             "reconstructions": lists(recs), "activations": lists(acts), "preactivations": lists(pre),
-            "decoder_norms": lists(norms)}
+            "decoder_norms": lists(norms), "encode": lists(encoded), "decode_layer": mid, "decode": lists(decoded_mid)}
 
 
 def theta_case(cfg_kw, seed, tokens=6, batches=3):

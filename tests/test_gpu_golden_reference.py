@@ -48,6 +48,19 @@ def test_forward_matches_the_reference(dev, case):
             assert orc.rel_l2(pre, T(case["preactivations"][str(l)])) <= 1e-2
             assert orc.rel_l2(recs[l].float().cpu(), want_r) <= (1e-2 if case["config"]["activation_fn"] == "jumprelu" else 5e-2)
             assert ((acts[l].float().cpu() != 0) != (want_a != 0)).float().mean() <= 0.01
+    # the per-layer entry points (clt.py:112-184): encode() serves relu / jumprelu and returns zeros (with an
+    # error log) for the top-k activations; decode() of the activations up to a layer
+    tol = dict(rtol=1e-5, atol=1e-5) if fp32 else dict(rtol=5e-2, atol=5e-2)
+    for l in range(case["config"]["num_layers"]):
+        got_e = model.encode(inputs[l], l).float().cpu()
+        want_e = T(case["encode"][str(l)])
+        assert got_e.shape == want_e.shape
+        if fp32:
+            assert torch.equal(got_e != 0, want_e != 0), ("encode", l)
+        assert torch.allclose(got_e, want_e, **tol) or not fp32, ("encode", l)
+    mid = case["decode_layer"]
+    got_d = model.decode({l: acts[l] for l in range(mid + 1)}, mid).float().cpu()
+    assert torch.allclose(got_d, T(case["decode"]), **tol) or orc.rel_l2(got_d, T(case["decode"])) <= 5e-2
     want_n = T(case["decoder_norms"])
     got_n = model.get_decoder_norms().float().cpu()
     assert got_n.shape == want_n.shape
