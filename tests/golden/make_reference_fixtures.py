@@ -76,6 +76,35 @@ def forward_case(name, cfg_kw, seed, tokens=5):
             "decoder_norms": lists(norms), "encode": lists(encoded), "decode_layer": mid, "decode": lists(decoded_mid)}
 
 
+def irregular_cases(seed):
+    """Inputs the reference answers with its fallbacks: a missing layer, 3-D inputs, a layer whose width
+    is wrong, a layer with another token count."""
+    out = {"models": {}, "cases": []}
+    for fn_kw in (dict(activation_fn="relu"), dict(activation_fn="batchtopk", batchtopk_k=3)):
+        cfg_kw = dict(num_features=16, num_layers=3, d_model=8, **fn_kw)
+        cfg, model, g = build(cfg_kw, seed)
+        out["models"][fn_kw["activation_fn"]] = {"config": cfg_kw, "state_dict": lists(dict(model.state_dict()))}
+        variants = {
+            "missing-layer-1": {0: torch.randn(5, 8, generator=g), 2: torch.randn(5, 8, generator=g)},
+            "three-dimensional": {l: torch.randn(2, 3, 8, generator=g) for l in range(3)},
+            "wrong-width-layer-1": {0: torch.randn(5, 8, generator=g), 1: torch.randn(5, 7, generator=g),
+                                    2: torch.randn(5, 8, generator=g)},
+            "other-token-count-layer-2": {0: torch.randn(5, 8, generator=g), 1: torch.randn(5, 8, generator=g),
+                                          2: torch.randn(4, 8, generator=g)},
+        }
+        for vname, inputs in variants.items():
+            with torch.no_grad():
+                try:
+                    recs = lists(model(inputs))
+                    acts = lists(model.get_feature_activations(inputs))
+                    err = None
+                except Exception as e:      # the reference itself fails on this input: recorded as such
+                    recs, acts, err = None, None, type(e).__name__
+            out["cases"].append({"name": f"{fn_kw['activation_fn']}-{vname}", "model": fn_kw["activation_fn"],
+                                 "inputs": lists(inputs), "reconstructions": recs, "activations": acts, "raises": err})
+    return out
+
+
 def theta_case(cfg_kw, seed, tokens=6, batches=3):
     cfg, model, g = build(cfg_kw, seed)
     L, d = cfg.num_layers, cfg.d_model
@@ -170,6 +199,7 @@ def main():
                                                                activation_fn="batchtopk", batchtopk_k=4,
                                                                clt_dtype="bfloat16"), 18, tokens=16),
                 ],
+                "forward_irregular": irregular_cases(19),
                 "theta_estimation": [theta_case(dict(base, activation_fn="batchtopk", batchtopk_k=3), 21),
                                      theta_case(dict(base, activation_fn="topk", topk_k=4), 22)],
                 "gradients": [

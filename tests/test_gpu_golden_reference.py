@@ -132,3 +132,31 @@ def test_global_selection_matches_the_reference_in_each_dtype(dev, case):
     for l in range(L):
         assert torch.equal(got_b[l].float().cpu(), T(case["batchtopk"][str(l)])), ("batchtopk", l)
         assert torch.equal(got_t[l].float().cpu(), T(case["tokentopk"][str(l)])), ("tokentopk", l)
+
+
+@pytest.mark.parametrize("case", [dict(c, **FIX["forward_irregular"]["models"][c["model"]]) for c in FIX["forward_irregular"]["cases"]],
+                         ids=lambda c: c["name"])
+def test_irregular_inputs_are_answered_like_the_reference(dev, case):
+    # a missing layer, 3-D inputs, a layer of the wrong width, a layer with another token count: same keys,
+    # shapes and values as the reference's fallbacks give (or an exception where the reference raises one)
+    model = load_model(case, dev)
+    model.eval()
+    inputs = {int(l): T(v, dev) for l, v in case["inputs"].items()}
+    if case["raises"]:
+        with pytest.raises(Exception):
+            model(inputs)
+        return
+    recs = model(inputs)
+    acts = model.get_feature_activations(inputs)
+    assert sorted(recs) == sorted(int(k) for k in case["reconstructions"])
+    assert sorted(acts) == sorted(int(k) for k in case["activations"])
+    for l, want in case["activations"].items():
+        want = T(want)
+        got = acts[int(l)].float().cpu()
+        assert got.shape == want.shape, ("activations", l)
+        assert torch.equal(got != 0, want != 0) and torch.allclose(got, want, rtol=1e-5, atol=1e-6), ("activations", l)
+    for l, want in case["reconstructions"].items():
+        want = T(want)
+        got = recs[int(l)].float().cpu()
+        assert got.shape == want.shape, ("reconstructions", l)
+        assert torch.allclose(got, want, rtol=1e-5, atol=1e-5), ("reconstructions", l)
