@@ -105,6 +105,24 @@ def irregular_cases(seed):
     return out
 
 
+def config_json_cases():
+    """cfg.json as the reference writes it, for two configurations."""
+    import tempfile
+    out = []
+    for kw in (dict(num_features=16, num_layers=3, d_model=8, activation_fn="batchtopk", batchtopk_k=3),
+               dict(num_features=32, num_layers=2, d_model=4, activation_fn="jumprelu", decoder_tying="per_target",
+                    enable_feature_offset=True, enable_feature_scale=True, skip_connection=True, clt_dtype="bfloat16",
+                    model_name="gpt2", jumprelu_threshold=0.05)):
+        cfg = CLTConfig(**kw)
+        with tempfile.TemporaryDirectory() as tmp:
+            path = os.path.join(tmp, "cfg.json")
+            cfg.to_json(path)
+            written = json.load(open(path))
+            back = CLTConfig.from_json(path)
+        out.append({"kwargs": kw, "json": written, "fields_after_reload": {k: getattr(back, k) for k in written}})
+    return out
+
+
 def theta_case(cfg_kw, seed, tokens=6, batches=3):
     cfg, model, g = build(cfg_kw, seed)
     L, d = cfg.num_layers, cfg.d_model
@@ -200,6 +218,7 @@ def main():
                                                                clt_dtype="bfloat16"), 18, tokens=16),
                 ],
                 "forward_irregular": irregular_cases(19),
+                "config_json": config_json_cases(),
                 "theta_estimation": [theta_case(dict(base, activation_fn="batchtopk", batchtopk_k=3), 21),
                                      theta_case(dict(base, activation_fn="topk", topk_k=4), 22)],
                 "gradients": [

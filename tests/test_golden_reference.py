@@ -146,3 +146,19 @@ def test_oracle_global_selection_matches_the_reference_in_each_dtype(case):
     for l in range(L):
         assert torch.equal(got_b[l].float(), T(case["batchtopk"][str(l)])), ("batchtopk", l)
         assert torch.equal(got_t[l].float(), T(case["tokentopk"][str(l)])), ("tokentopk", l)
+
+
+@pytest.mark.parametrize("case", FIX["config_json"], ids=lambda c: c["kwargs"]["activation_fn"])
+def test_config_json_round_trip_matches_the_reference(case, tmp_path):
+    # cfg.json as the reference writes it: this build reads it to the same field values, and writes the
+    # same file for the same constructor arguments
+    import json as _json
+    from crosslayer_coding_amd import CLTConfig
+    path = tmp_path / "cfg.json"
+    path.write_text(_json.dumps(case["json"]))
+    cfg = CLTConfig.from_json(str(path))
+    for key, want in case["fields_after_reload"].items():
+        assert getattr(cfg, key) == want, key
+    out = tmp_path / "mine.json"
+    CLTConfig(**case["kwargs"]).to_json(str(out))
+    assert _json.loads(out.read_text()) == case["json"]
