@@ -57,8 +57,10 @@ def build(cfg_kw, seed):
     return cfg, model, g
 
 
-def forward_case(name, cfg_kw, seed, tokens=5):
+def forward_case(name, cfg_kw, seed, tokens=5, save_as=None):
     cfg, model, g = build(cfg_kw, seed)
+    if save_as:      # the reference's own checkpoint format (BaseTranscoder.save): one torch file
+        model.save(os.path.join(os.path.dirname(os.path.abspath(__file__)), save_as))
     L, d = cfg.num_layers, cfg.d_model
     dtype = next(model.parameters()).dtype
     inputs = {l: torch.randn(tokens, d, generator=g).to(dtype) for l in range(L)}
@@ -205,7 +207,8 @@ def main():
                     forward_case("jumprelu", dict(base, activation_fn="jumprelu"), 13),
                     forward_case("relu-per-target-affine-skip", dict(base, activation_fn="relu", decoder_tying="per_target",
                                                                      enable_feature_offset=True, enable_feature_scale=True,
-                                                                     skip_connection=True), 14),
+                                                                     skip_connection=True), 14,
+                                 save_as="reference_checkpoint.pt"),
                     forward_case("batchtopk-global-per-source", dict(base, activation_fn="batchtopk", batchtopk_k=3,
                                                                      decoder_tying="per_source"), 15),
                     forward_case("relu-untied-skip", dict(base, activation_fn="relu", skip_connection=True), 16),

@@ -160,3 +160,23 @@ def test_irregular_inputs_are_answered_like_the_reference(dev, case):
         got = recs[int(l)].float().cpu()
         assert got.shape == want.shape, ("reconstructions", l)
         assert torch.allclose(got, want, rtol=1e-5, atol=1e-5), ("reconstructions", l)
+
+
+def test_checkpoint_written_by_the_reference_loads_and_reproduces_its_forward(dev):
+    # tests/golden/reference_checkpoint.pt was written by the reference's own BaseTranscoder.save for the
+    # "relu-per-target-affine-skip" model of the forward fixtures; it is read with weights_only=True
+    case = next(c for c in FIX["forward"] if c["name"] == "relu-per-target-affine-skip")
+    path = os.path.join(os.path.dirname(__file__), "golden", "reference_checkpoint.pt")
+    model = cca.CrossLayerTranscoder.load(path, dev)
+    model.eval()
+    assert model.config.decoder_tying == "per_target" and model.config.skip_connection
+    inputs = {int(l): T(v, dev) for l, v in case["inputs"].items()}
+    recs = model(inputs)
+    for l, want in case["reconstructions"].items():
+        assert torch.allclose(recs[int(l)].cpu(), T(want), rtol=1e-5, atol=1e-5)
+    # and a checkpoint written here has the same keys and values as the reference's
+    import torch as _t
+    ref = _t.load(path, weights_only=True)
+    assert ref["state_dict"].keys() == model.state_dict().keys()
+    for k, v in ref["state_dict"].items():
+        assert torch.equal(v, model.state_dict()[k].cpu()), k
