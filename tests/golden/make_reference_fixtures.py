@@ -125,6 +125,26 @@ def config_json_cases():
     return out
 
 
+def migration_case(seed):
+    """An untied checkpoint, with its feature affine parameters under the old encoder_module names, loaded
+    into a per-source model by the reference's load_state_dict (clt.py:347-432)."""
+    base = dict(num_features=16, num_layers=3, d_model=8, activation_fn="relu")
+    _, untied, g = build(base, seed)
+    tied_kw = dict(base, decoder_tying="per_source", enable_feature_offset=True, enable_feature_scale=True)
+    _, tied, _ = build(tied_kw, seed + 5)
+    old = {k: v.clone() for k, v in untied.state_dict().items()}
+    for i in range(3):
+        old[f"encoder_module.feature_offset.{i}"] = torch.randn(16, generator=g) * 0.1
+        old[f"encoder_module.feature_scale.{i}"] = 0.5 + torch.rand(16, generator=g)
+    tied.load_state_dict(dict(old))
+    tied.eval()
+    inputs = {l: torch.randn(5, 8, generator=g) for l in range(3)}
+    with torch.no_grad():
+        recs = tied(inputs)
+    return {"config": tied_kw, "old_state_dict": lists(old), "state_dict_after": lists(dict(tied.state_dict())),
+            "inputs": lists(inputs), "reconstructions": lists(recs)}
+
+
 def theta_case(cfg_kw, seed, tokens=6, batches=3):
     cfg, model, g = build(cfg_kw, seed)
     L, d = cfg.num_layers, cfg.d_model
@@ -222,6 +242,7 @@ def main():
                 ],
                 "forward_irregular": irregular_cases(19),
                 "config_json": config_json_cases(),
+                "checkpoint_migration": migration_case(61),
                 "theta_estimation": [theta_case(dict(base, activation_fn="batchtopk", batchtopk_k=3), 21),
                                      theta_case(dict(base, activation_fn="topk", topk_k=4), 22)],
                 "gradients": [

@@ -180,3 +180,19 @@ def test_checkpoint_written_by_the_reference_loads_and_reproduces_its_forward(de
     assert ref["state_dict"].keys() == model.state_dict().keys()
     for k, v in ref["state_dict"].items():
         assert torch.equal(v, model.state_dict()[k].cpu()), k
+
+
+def test_old_checkpoint_migration_matches_the_reference(dev):
+    # an untied checkpoint with feature affine parameters under their old encoder_module names, loaded into
+    # a per-source model: same parameters afterwards, same forward
+    case = FIX["checkpoint_migration"]
+    model = cca.CrossLayerTranscoder(cca.CLTConfig(**case["config"]), None, dev)
+    model.load_state_dict({k: T(v) for k, v in case["old_state_dict"].items()})
+    model.eval()
+    after = model.state_dict()
+    assert after.keys() == case["state_dict_after"].keys()
+    for k, v in case["state_dict_after"].items():
+        assert torch.equal(after[k].cpu(), T(v)), k
+    recs = model({int(l): T(v, dev) for l, v in case["inputs"].items()})
+    for l, want in case["reconstructions"].items():
+        assert torch.allclose(recs[int(l)].cpu(), T(want), rtol=1e-5, atol=1e-5)
