@@ -22,6 +22,7 @@ sys.path.insert(0, REF)
 
 from clt.config import CLTConfig, TrainingConfig          # noqa: E402
 from clt.models.activations import _apply_batch_topk_helper, _apply_token_topk_helper   # noqa: E402
+from clt.activations.registry import get_activation_fn    # noqa: E402
 from clt.models.clt import CrossLayerTranscoder           # noqa: E402
 from clt.training.evaluator import CLTEvaluator           # noqa: E402
 from clt.training.losses import LossManager               # noqa: E402
@@ -145,6 +146,39 @@ def migration_case(seed):
             "inputs": lists(inputs), "reconstructions": lists(recs)}
 
 
+def per_layer_case(name, cfg_kw, seed, tokens=16):
+    """The per-layer scope of BatchTopK / TokenTopK, assembled from the reference's own pieces: the registry's
+    per-layer activation (clt/activations/registry.py:43-98) on the model's pre-activations, then
+    Decoder.decode per target.  (The model's own forward does not reach the registry function for this scope in
+    this snapshot.)  Seeds with a tie at the threshold are skipped."""
+    while True:
+        cfg, model, g = build(cfg_kw, seed)
+        dtype = next(model.parameters()).dtype
+        L, d = cfg.num_layers, cfg.d_model
+        inputs = {l: torch.randn(tokens, d, generator=g).to(dtype) for l in range(L)}
+        fn = get_activation_fn(cfg.activation_fn)
+        with torch.no_grad():
+            pre = {l: model.get_preactivations(inputs[l], l) for l in range(L)}
+            ok = True
+            for l in range(L):
+                if cfg.activation_fn == "batchtopk":
+                    flat = torch.sort(pre[l].float().reshape(-1), descending=True).values
+                    K = int(cfg.batchtopk_k) * tokens
+                    ok = ok and bool(flat[K - 1] != flat[K])
+                else:
+                    rows = torch.sort(pre[l].float(), dim=1, descending=True).values
+                    kk = int(cfg.topk_k)
+                    ok = ok and bool((rows[:, kk - 1] != rows[:, kk]).all())
+            if not ok:
+                seed += 1000
+                continue
+            acts = {l: fn(model, pre[l], l) for l in range(L)}
+            recs = {t: model.decode({s_: acts[s_] for s_ in range(t + 1)}, t) for t in range(L)}
+        return {"name": name, "config": dict(cfg_kw, topk_mode="per_layer"), "seed": seed,
+                "state_dict": lists(dict(model.state_dict())), "inputs": lists(inputs), "preactivations": lists(pre),
+                "activations": lists(acts), "reconstructions": lists(recs)}
+
+
 def theta_case(cfg_kw, seed, tokens=6, batches=3):
     cfg, model, g = build(cfg_kw, seed)
     L, d = cfg.num_layers, cfg.d_model
@@ -239,6 +273,14 @@ def main():
                     forward_case("batchtopk-global-bf16", dict(num_features=32, num_layers=3, d_model=16,
                                                                activation_fn="batchtopk", batchtopk_k=4,
                                                                clt_dtype="bfloat16"), 18, tokens=16),
+                ],
+                "per_layer": [
+                    per_layer_case("batchtopk", dict(num_features=32, num_layers=3, d_model=8, activation_fn="batchtopk",
+                                                     batchtopk_k=4), 71),
+                    per_layer_case("batchtopk-bf16", dict(num_features=32, num_layers=3, d_model=8, activation_fn="batchtopk",
+                                                          batchtopk_k=4, clt_dtype="bfloat16"), 72),
+                    per_layer_case("tokentopk", dict(num_features=32, num_layers=3, d_model=8, activation_fn="topk",
+                                                     topk_k=5.0), 73),
                 ],
                 "forward_irregular": irregular_cases(19),
                 "config_json": config_json_cases(),

@@ -162,3 +162,17 @@ def test_config_json_round_trip_matches_the_reference(case, tmp_path):
     out = tmp_path / "mine.json"
     CLTConfig(**case["kwargs"]).to_json(str(out))
     assert _json.loads(out.read_text()) == case["json"]
+
+
+@pytest.mark.parametrize("case", FIX["per_layer"], ids=lambda c: c["name"])
+def test_oracle_per_layer_scope_matches_the_reference_registry(case):
+    # the registry's per-layer BatchTopK / TokenTopK on given pre-activations: bit for bit, in the model dtype
+    cfg = case["config"]
+    dtype = getattr(torch, cfg.get("clt_dtype", "float32"))
+    for l, pre in case["preactivations"].items():
+        pre = T(pre).to(dtype)
+        if cfg["activation_fn"] == "batchtopk":
+            got = orc.batchtopk_forward(pre, float(cfg["batchtopk_k"]), pre)
+        else:
+            got = orc.tokentopk_forward(pre, float(cfg["topk_k"]), pre)
+        assert torch.equal(got.float(), T(case["activations"][l])), l

@@ -196,3 +196,35 @@ def test_old_checkpoint_migration_matches_the_reference(dev):
     recs = model({int(l): T(v, dev) for l, v in case["inputs"].items()})
     for l, want in case["reconstructions"].items():
         assert torch.allclose(recs[int(l)].cpu(), T(want), rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("case", FIX["per_layer"], ids=lambda c: c["name"])
+def test_per_layer_scope_matches_the_reference_pieces(dev, case):
+    # the headline scope: the reference's registry function on the pre-activations, then its decode per
+    # target.  Selection on the fixture's own pre-activations is bit-exact; the model's forward (its own
+    # encoder in front) is held to the tolerance of the dtype.
+    from crosslayer_coding_amd import engine
+    from oracle import clt_oracle as orc
+    cfg = case["config"]
+    model = load_model(case, dev)
+    model.eval()
+    fp32 = model.dtype == torch.float32
+    L = cfg["num_layers"]
+    pre = torch.stack([T(case["preactivations"][str(l)]).to(model.dtype) for l in range(L)]).to(dev).contiguous()
+    if cfg["activation_fn"] == "batchtopk":
+        dense = engine.densify(engine.batchtopk_select(pre, cfg["batchtopk_k"], False))
+    else:
+        dense = engine.densify(engine.tokentopk_select(pre, int(cfg["topk_k"]), False))
+    for l in range(L):
+        assert torch.equal(dense[l].float().cpu(), T(case["activations"][str(l)])), ("selection", l)
+    inputs = {int(l): T(v, dev).to(model.dtype) for l, v in case["inputs"].items()}
+    recs = model(inputs)
+    acts = model.get_feature_activations(inputs)
+    for l in range(L):
+        want_a, want_r = T(case["activations"][str(l)]), T(case["reconstructions"][str(l)])
+        if fp32:
+            assert torch.equal(acts[l].cpu() != 0, want_a != 0), l
+            assert torch.allclose(acts[l].cpu(), want_a, rtol=1e-5, atol=1e-6)
+            assert torch.allclose(recs[l].cpu(), want_r, rtol=1e-5, atol=1e-5)
+        else:
+            assert orc.rel_l2(recs[l].float().cpu(), want_r) <= 5e-2
