@@ -251,6 +251,21 @@ def global_select_case(dtype, seed, L=3, tokens=16, F=32, k=5, kk=6):
             "batchtopk": lists(out_b), "tokentopk": lists(out_t)}
 
 
+def compute_metrics_case(seed):
+    """CLTEvaluator.compute_metrics end to end on a seeded model (global BatchTopK)."""
+    cfg_kw = dict(num_features=16, num_layers=3, d_model=8, activation_fn="batchtopk", batchtopk_k=3)
+    cfg, model, g = build(cfg_kw, seed)
+    inputs = {l: torch.randn(12, 8, generator=g) for l in range(3)}
+    targets = {l: torch.randn(12, 8, generator=g) for l in range(3)}
+    mask = torch.zeros(3, 16, dtype=torch.bool)
+    mask[0, :3] = True
+    mask[2, 5] = True
+    ev = CLTEvaluator(model, CPU)
+    metrics = ev.compute_metrics(inputs, targets, dead_neuron_mask=mask)
+    return {"config": cfg_kw, "state_dict": lists(dict(model.state_dict())), "inputs": lists(inputs), "targets": lists(targets),
+            "dead_neuron_mask": mask.int().tolist(), "metrics": lists(metrics)}
+
+
 def main():
     base = dict(num_features=16, num_layers=3, d_model=8)
     fixtures = {"_about": "Produced by tests/golden/make_reference_fixtures.py from the reference's own code on the CPU "
@@ -294,7 +309,8 @@ def main():
                     gradient_case("relu-per-target", dict(base, activation_fn="relu", decoder_tying="per_target"), 34),
                 ],
                 "global_select": [global_select_case(torch.float32, 51), global_select_case(torch.bfloat16, 52)],
-                "evaluator": evaluator_case(41)}
+                "evaluator": evaluator_case(41),
+                "compute_metrics": compute_metrics_case(42)}
     out = os.path.join(os.path.dirname(os.path.abspath(__file__)), "reference_fixtures.json")
     with open(out, "w") as f:
         json.dump(fixtures, f)

@@ -228,3 +228,28 @@ def test_per_layer_scope_matches_the_reference_pieces(dev, case):
             assert torch.allclose(recs[l].cpu(), want_r, rtol=1e-5, atol=1e-5)
         else:
             assert orc.rel_l2(recs[l].float().cpu(), want_r) <= 5e-2
+
+
+def test_compute_metrics_end_to_end_matches_the_reference(dev):
+    case = FIX["compute_metrics"]
+    model = load_model(case, dev)
+    model.eval()
+    ev = cca.CLTEvaluator(model, dev)
+    got = ev.compute_metrics({int(l): T(v) for l, v in case["inputs"].items()}, {int(l): T(v) for l, v in case["targets"].items()},
+                             dead_neuron_mask=torch.tensor(case["dead_neuron_mask"], dtype=torch.bool))
+    want = case["metrics"]
+    assert got.keys() == want.keys(), (sorted(got), sorted(want))
+
+    def same(a, b, path):
+        if isinstance(b, dict):
+            assert a.keys() == b.keys(), path
+            for k in b:
+                same(a[k], b[k], f"{path}/{k}")
+        elif isinstance(b, list):
+            assert len(a) == len(b), path
+            for i, (x, y) in enumerate(zip(a, b)):
+                same(x, y, f"{path}[{i}]")
+        else:
+            assert a == pytest.approx(b, rel=1e-4, abs=1e-6) or (math.isinf(a) and math.isinf(b)), (path, a, b)
+
+    same(got, want, "metrics")
