@@ -266,6 +266,42 @@ def compute_metrics_case(seed):
             "dead_neuron_mask": mask.int().tolist(), "metrics": lists(metrics)}
 
 
+def c0_summary():
+    """The full-size fp32 configuration (12 layers, d_model 768, 6144 features, 1024 tokens, k = 200) through the
+    reference, on the weights and inputs of this build's own generator drawn on the CPU (so the test can
+    rebuild them anywhere).  Too large to store: kept are, per layer, the sum and sum of squares of the
+    reconstruction, the number of non-zero activations, and four token rows of three layers in full; for the
+    global scope (the model's own forward) and for the per-layer scope (registry function + decode)."""
+    sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__)))))
+    from crosslayer_coding_amd import synth
+    wl = synth.WORKLOADS["c0"]
+    sd = synth.make_state_dict(wl, "cpu")
+    x = synth.make_inputs(wl, "cpu")
+    L = wl.num_layers
+    rows = [0, 333, 700, 1023]
+    out = {"workload": "c0", "rows": rows, "layers_in_full": [0, 6, 11]}
+    for scope in ("global", "per_layer"):
+        cfg = CLTConfig(num_features=wl.num_features, num_layers=L, d_model=wl.d_model, activation_fn="batchtopk",
+                        batchtopk_k=wl.k)
+        model = CrossLayerTranscoder(cfg, process_group=None, device=CPU)
+        model.load_state_dict(sd)
+        model.eval()
+        inputs = {l: x[l] for l in range(L)}
+        with torch.no_grad():
+            if scope == "global":
+                recs = model(inputs)
+                acts = model.get_feature_activations(inputs)
+            else:
+                fn = get_activation_fn("batchtopk")
+                acts = {l: fn(model, model.get_preactivations(inputs[l], l), l) for l in range(L)}
+                recs = {t: model.decode({s_: acts[s_] for s_ in range(t + 1)}, t) for t in range(L)}
+        out[scope] = {"sum": [float(recs[l].double().sum()) for l in range(L)],
+                      "sumsq": [float((recs[l].double() ** 2).sum()) for l in range(L)],
+                      "nonzero": [int((acts[l] != 0).sum()) for l in range(L)],
+                      "rows": {str(l): lists(recs[l][rows]) for l in out["layers_in_full"]}}
+    return out
+
+
 def main():
     base = dict(num_features=16, num_layers=3, d_model=8)
     fixtures = {"_about": "Produced by tests/golden/make_reference_fixtures.py from the reference's own code on the CPU "
@@ -310,7 +346,8 @@ def main():
                 ],
                 "global_select": [global_select_case(torch.float32, 51), global_select_case(torch.bfloat16, 52)],
                 "evaluator": evaluator_case(41),
-                "compute_metrics": compute_metrics_case(42)}
+                "compute_metrics": compute_metrics_case(42),
+                "c0_summary": c0_summary()}
     out = os.path.join(os.path.dirname(os.path.abspath(__file__)), "reference_fixtures.json")
     with open(out, "w") as f:
         json.dump(fixtures, f)

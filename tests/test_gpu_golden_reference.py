@@ -253,3 +253,39 @@ def test_compute_metrics_end_to_end_matches_the_reference(dev):
             assert a == pytest.approx(b, rel=1e-4, abs=1e-6) or (math.isinf(a) and math.isinf(b)), (path, a, b)
 
     same(got, want, "metrics")
+
+
+@pytest.mark.parametrize("scope", ["global", "per_layer"])
+def test_full_size_c0_against_the_reference_summary(dev, scope):
+    # C0 (fp32, 12 x 768 x 6144, 1024 tokens, k = 200) went through the reference once, on the weights and
+    # inputs this build's generator draws on the CPU; the fixture keeps sums, counts and a few rows in full
+    from crosslayer_coding_amd import synth
+    from oracle import clt_oracle as orc
+    fx = FIX["c0_summary"]
+    wl = synth.WORKLOADS["c0"].scaled("c0-" + scope, topk_mode=scope)
+    sd = synth.make_state_dict(synth.WORKLOADS["c0"], "cpu")
+    x = synth.make_inputs(synth.WORKLOADS["c0"], "cpu")
+    model = cca.CrossLayerTranscoder(wl.config(), None, dev)
+    model.load_state_dict(sd)
+    model.eval()
+    L = wl.num_layers
+    inputs = {l: x[l].to(dev) for l in range(L)}
+    recs = model(inputs)
+    acts = model.get_feature_activations(inputs)
+    want = fx[scope]
+    for l in range(L):
+        r = recs[l].double()
+        ss = float((r ** 2).sum())
+        assert ss == pytest.approx(want["sumsq"][l], rel=1e-4), ("sumsq", l)
+        assert abs(float(r.sum()) - want["sum"][l]) <= 1e-4 * (ss * r.numel()) ** 0.5, ("sum", l)
+        nz = int((acts[l] != 0).sum())
+        # the two encoders sum in different orders: a pre-activation at the threshold can land on either side,
+        # which moves a survivor between layers in the global scope and nowhere in the per-layer scope
+        assert abs(nz - want["nonzero"][l]) <= (8 if scope == "global" else 0), ("nonzero", l, nz)
+    # rows kept in full: equal to 1e-5 unless one of the row's survivors sits at the threshold and fell on the
+    # other side there (then one feature's decoder vector differs: ~1e-2); at most one such row per layer
+    for l in fx["layers_in_full"]:
+        got = recs[l][fx["rows"]].float().cpu()
+        ref = T(want["rows"][str(l)])
+        errs = sorted(orc.rel_l2(got[i], ref[i]) for i in range(len(fx["rows"])))
+        assert errs[-2] <= 1e-5 and errs[-1] <= 5e-2, ("rows", l, errs)
