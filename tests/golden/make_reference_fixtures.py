@@ -302,6 +302,35 @@ def c0_summary():
     return out
 
 
+def c1_summary():
+    """The headline configuration (bf16, 12 layers, d_model 768, 24576 features, 4096 tokens, k = 200, per-layer
+    scope) through the reference's registry function and decode, on this build's CPU-drawn weights and inputs.
+    Kept: per layer the sum of squares of the reconstruction and the number of non-zero activations, and four
+    token rows of three layers in full.  Takes a few minutes."""
+    sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__)))))
+    from crosslayer_coding_amd import synth
+    torch.set_num_threads(8)
+    wl = synth.WORKLOADS["c1"]
+    sd = synth.make_state_dict(wl, "cpu")
+    x = synth.make_inputs(wl, "cpu")
+    L = wl.num_layers
+    rows = [0, 1333, 2700, 4095]
+    cfg = CLTConfig(num_features=wl.num_features, num_layers=L, d_model=wl.d_model, activation_fn="batchtopk",
+                    batchtopk_k=wl.k, clt_dtype="bfloat16")
+    model = CrossLayerTranscoder(cfg, process_group=None, device=CPU)
+    model.load_state_dict(sd)
+    model.eval()
+    fn = get_activation_fn("batchtopk")
+    with torch.no_grad():
+        acts = {l: fn(model, model.get_preactivations(x[l], l), l) for l in range(L)}
+        recs = {t: model.decode({s_: acts[s_] for s_ in range(t + 1)}, t) for t in range(L)}
+    torch.set_num_threads(1)
+    return {"workload": "c1", "rows": rows, "layers_in_full": [0, 6, 11],
+            "sumsq": [float((recs[l].double() ** 2).sum()) for l in range(L)],
+            "nonzero": [int((acts[l] != 0).sum()) for l in range(L)],
+            "rows_full": {str(l): lists(recs[l][rows]) for l in (0, 6, 11)}}
+
+
 def main():
     base = dict(num_features=16, num_layers=3, d_model=8)
     fixtures = {"_about": "Produced by tests/golden/make_reference_fixtures.py from the reference's own code on the CPU "
@@ -347,7 +376,8 @@ def main():
                 "global_select": [global_select_case(torch.float32, 51), global_select_case(torch.bfloat16, 52)],
                 "evaluator": evaluator_case(41),
                 "compute_metrics": compute_metrics_case(42),
-                "c0_summary": c0_summary()}
+                "c0_summary": c0_summary(),
+                "c1_summary": c1_summary()}
     out = os.path.join(os.path.dirname(os.path.abspath(__file__)), "reference_fixtures.json")
     with open(out, "w") as f:
         json.dump(fixtures, f)

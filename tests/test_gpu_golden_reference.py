@@ -289,3 +289,37 @@ def test_full_size_c0_against_the_reference_summary(dev, scope):
         ref = T(want["rows"][str(l)])
         errs = sorted(orc.rel_l2(got[i], ref[i]) for i in range(len(fx["rows"])))
         assert errs[-2] <= 1e-5 and errs[-1] <= 5e-2, ("rows", l, errs)
+
+
+def test_headline_c1_against_the_reference_summary(dev):
+    # C1 (bf16, 12 x 768 x 24576, 4096 tokens, k = 200, per-layer scope) went through the reference's registry
+    # function and decode once on the CPU; same CPU-drawn weights and inputs here.  In bf16 tens of thousands
+    # of a layer's 100 M pre-activations share the threshold's value, and which of them survive is torch.topk's
+    # unspecified choice there and the lowest flat index here: a few per cent of the survivors differ, every
+    # layer still keeps exactly k*T, the energy of each reconstruction agrees to 1 %, and a token row agrees
+    # either to bf16 rounding or up to the decoder vectors of the features that were swapped.
+    from crosslayer_coding_amd import synth
+    from oracle import clt_oracle as orc
+    fx = FIX["c1_summary"]
+    wl = synth.WORKLOADS["c1"]
+    sd = synth.make_state_dict(wl, "cpu")
+    x = synth.make_inputs(wl, "cpu")
+    model = cca.CrossLayerTranscoder(wl.config(), None, dev)
+    model.load_state_dict(sd)
+    model.eval()
+    L = wl.num_layers
+    inputs = {l: x[l].to(dev) for l in range(L)}
+    recs, surv = model.forward_with_survivors(inputs)
+    rp = surv.row_ptr.long()
+    per_layer = (rp[wl.tokens::wl.tokens] - rp[:-1:wl.tokens]).tolist()
+    assert per_layer == fx["nonzero"]
+    for l in range(L):
+        ss = float((recs[l].double() ** 2).sum())
+        assert ss == pytest.approx(fx["sumsq"][l], rel=1e-2), ("sumsq", l)
+    for l in fx["layers_in_full"]:
+        got = recs[l][fx["rows"]].float().cpu()
+        ref = T(fx["rows_full"][str(l)])
+        errs = sorted(orc.rel_l2(got[i], ref[i]) for i in range(len(fx["rows"])))
+        assert errs[0] <= 1e-2 and errs[-1] <= 0.3, ("rows", l, errs)
+    del model, recs, surv
+    torch.cuda.empty_cache()
