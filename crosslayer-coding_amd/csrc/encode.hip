@@ -13,10 +13,12 @@
 //               all banks
 //   math        the matrix-core "A" operand is the W tile and "B" the x tile, so a lane ends
 //               up with 4 consecutive features of one token per accumulator group
-//   epilogue    bias add, rounding, then the tile goes through LDS so that the stores are
-//               16 bytes per lane and 256 contiguous bytes per token
+//   bias        the accumulators start from the bias, so it is added in fp32 before the one rounding
+//   epilogue    rounding, then the tile goes through LDS so that the stores are 16 bytes per lane
+//               and 256 contiguous bytes per token
 //   bf16        v_mfma_f32_32x32x16_bf16, fp32 accumulate, one rounding (v_cvt_pk_bf16_f32)
 //   fp32        v_mfma_f32_32x32x2_f32
+#include <type_traits>
 #include "select_state.h"
 
 namespace {
@@ -28,6 +30,7 @@ constexpr int BM = 256;   // tokens per block
 constexpr int BN = 256;   // features per block
 constexpr int ROWB = 128; // bytes of K per LDS row
 constexpr int STAGE = (BM + BN) * ROWB;  // bytes of one LDS stage
+constexpr int CAND_LIST = 2048;          // candidates of one wave tile the collecting epilogue lists in LDS
 constexpr int ENC_SN = 8;  // feature tiles x token tiles that one XCD works on at a time
 constexpr int ENC_SM = 4;
 
@@ -134,6 +137,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   // other, and does not wait for them.
   __shared__ __attribute__((aligned(16))) unsigned char stage0[STAGE];
   __shared__ __attribute__((aligned(16))) unsigned char stage1[STAGE];
+  __shared__ uint16_t cand_list[COLLECT ? 4 : 1][COLLECT ? CAND_LIST : 1];   // per wavefront, see the emission
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -188,13 +192,40 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #pragma unroll
   for (int kk = 0; kk < 4; ++kk) koff[kk] = ((kk * 2 + lh) ^ ((l31 >> 1) & 7)) << 4;
 
+  // The accumulators start from the bias (the matrix core adds its products onto them in fp32), so
+  // the epilogue has no bias loads or adds: accumulator (j, rg*4+q) of a lane belongs to feature
+  // j*32 + rg*8 + (lane>>5)*4 + q of the wave tile, whatever the token group i.  The bias is asked
+  // for here, ahead of the first stage, and lands in the accumulators while the second stage loads.
   f32x16_t acc[4][4];
+  typedef typename std::conditional<sizeof(T) == 4, float4, uint2>::type bias4_t;
+  bias4_t braw[16];
+  {
+    const T *bl = bias ? bias + (int64_t)layer * bs + n0 + wn * 128 + (lane >> 5) * 4 : nullptr;
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+    for (int g = 0; g < 16; ++g) {
+      if (bl) braw[g] = *reinterpret_cast<const bias4_t *>(bl + g * 8);
+      else if constexpr (sizeof(T) == 4) braw[g] = make_float4(0.f, 0.f, 0.f, 0.f);
+      else braw[g] = make_uint2(0u, 0u);
+    }
+  }
+  auto init_acc = [&]() {
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+      for (int rg = 0; rg < 4; ++rg) {
+        float bv[4];
+        if constexpr (sizeof(T) == 4) {
+          bv[0] = braw[j * 4 + rg].x; bv[1] = braw[j * 4 + rg].y; bv[2] = braw[j * 4 + rg].z; bv[3] = braw[j * 4 + rg].w;
+        } else {
+          bv[0] = __uint_as_float(braw[j * 4 + rg].x << 16); bv[1] = __uint_as_float(braw[j * 4 + rg].x & 0xFFFF0000u);
+          bv[2] = __uint_as_float(braw[j * 4 + rg].y << 16); bv[3] = __uint_as_float(braw[j * 4 + rg].y & 0xFFFF0000u);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) acc[i][j][rg * 4 + q] = bv[q];
+      }
+  };
 
   // Software pipeline over the K stages.  Fragments are double-buffered in registers (fa/fb)
   // and read one k-step ahead of the matrix ops that use them.  There is one barrier per
@@ -210,10 +241,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   auto stage_k0 = [&](int kt) { int q = kt + rot; if (q >= nk) q -= nk; return q * BK; };
   uint4 fa[8], fb[8];   // [0..3] x fragments, [4..7] W fragments
   auto load_frags = [&](uint4 (&f)[8], const unsigned char *sb, int kk) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) f[i] = *reinterpret_cast<const uint4 *>(sb + xrow + i * 32 * ROWB + koff[kk]);
+    // in the order the matrix ops of the next k-step want them: x0 and all of W first
+    f[0] = *reinterpret_cast<const uint4 *>(sb + xrow + koff[kk]);
 #pragma unroll
     for (int j = 0; j < 4; ++j) f[4 + j] = *reinterpret_cast<const uint4 *>(sb + wrow + j * 32 * ROWB + koff[kk]);
+#pragma unroll
+    for (int i = 1; i < 4; ++i) f[i] = *reinterpret_cast<const uint4 *>(sb + xrow + i * 32 * ROWB + koff[kk]);
   };
   auto mma16 = [&](const uint4 (&f)[8]) {
 #pragma unroll
@@ -221,13 +254,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #pragma unroll
       for (int j = 0; j < 4; ++j) Mma<T>::run(acc[i][j], f[4 + j], f[i]);
   };
-  // interleave hint: pairs of matrix ops with one LDS read between them
+  // interleave hint: the eight LDS reads go out behind the first matrix ops of the k-step, one
+  // apiece, so that the last of them has half a k-step to arrive before the next k-step waits for it
   auto mix_ds = [&]() {
 #pragma unroll
     for (int g = 0; g < 8; ++g) {
-      __builtin_amdgcn_sched_group_barrier(0x008, sizeof(T) == 2 ? 2 : 8, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, sizeof(T) == 2 ? 1 : 4, 0);
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
     }
+    __builtin_amdgcn_sched_group_barrier(0x008, sizeof(T) == 2 ? 8 : 32, 0);
   };
   // one stage except its last k-step, the barrier, then the last k-step overlapped with the
   // loads of the stage after next (into `cur`) and the first fragments of `nxt`
@@ -245,14 +280,23 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #pragma unroll
     for (int g = 0; g < 16; ++g) {
       __builtin_amdgcn_sched_group_barrier(0x008, sizeof(T) == 2 ? 1 : 4, 0);
+      if (g < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
     }
   };
+  // both stage buffers are free at this point: the second stage is asked for right behind the first,
+  // and only the first (this wavefront's 16 older loads, and the bias before them) is waited for
   issue_stage(stage0, stage_k0(0));
-  __builtin_amdgcn_s_waitcnt(0);
-  __syncthreads();
   issue_stage(stage1, stage_k0(1));
+  __builtin_amdgcn_sched_barrier(0);
+  __builtin_amdgcn_s_waitcnt(0x4F70);   // vmcnt(16): at most the 16 loads of the second stage outstanding
+  // a bare barrier between two compiler-only fences: the fences of __syncthreads() would wait for the
+  // second stage too
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);    // nothing that reads the bias may move above the wait
+  init_acc();
   load_frags(fa, stage0, 0);
   // nk is even (checked by the launcher).  The last two bodies fetch the final stage again and
   // read fragments that are never used: cheaper than a differently shaped last iteration.
@@ -266,7 +310,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   // 16 bytes per lane, 256 contiguous bytes per token.
   __syncthreads();   // every wavefront is done with the last stage
   T *pl = pre + (int64_t)layer * ps;
-  const T *bl = bias ? bias + (int64_t)layer * bs : nullptr;
   unsigned char *park = (wave < 2 ? stage0 : stage1) + (wave & 1) * (STAGE / 2);
   constexpr int NPASS = sizeof(T) == 2 ? 1 : 2;           // feature halves per pass
   constexpr int JP = 4 / NPASS;                            // 32-feature groups per pass
@@ -279,24 +322,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #pragma unroll
       for (int rg = 0; rg < 4; ++rg) {
         const int nl = jj * 32 + rg * 8 + lh * 4;          // feature inside this pass
-        const int n = n0 + wn * 128 + j * 32 + rg * 8 + lh * 4;
-        float bv[4] = {0.f, 0.f, 0.f, 0.f};
-        if (bl) {
-          if (sizeof(T) == 4) {
-            float4 b4 = *reinterpret_cast<const float4 *>(bl + n);
-            bv[0] = b4.x; bv[1] = b4.y; bv[2] = b4.z; bv[3] = b4.w;
-          } else {
-            uint2 b2 = *reinterpret_cast<const uint2 *>(bl + n);
-            bv[0] = __uint_as_float(b2.x << 16); bv[1] = __uint_as_float(b2.x & 0xFFFF0000u);
-            bv[2] = __uint_as_float(b2.y << 16); bv[3] = __uint_as_float(b2.y & 0xFFFF0000u);
-          }
-        }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int ml = i * 32 + l31;                     // token inside the wave tile
           float y[4];
 #pragma unroll
-          for (int q = 0; q < 4; ++q) y[q] = acc[i][j][rg * 4 + q] + bv[q];
+          for (int q = 0; q < 4; ++q) y[q] = acc[i][j][rg * 4 + q];
           if (sizeof(T) == 4) {
             const int slot = (nl >> 2) ^ (ml & 15);
             *reinterpret_cast<float4 *>(park + ml * 256 + slot * 16) = make_float4(y[0], y[1], y[2], y[3]);
@@ -449,17 +480,47 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
       uint2 *mypool = ca.pool + (unsigned long long)layer * ca.pool_cap;
       if (lane == 0) ca.tile_meta[(int64_t)layer * nseg * nrb + tile] = make_uint2(off, ok ? total : 0u);
       uint2 *meta = ca.seg_meta + ((int64_t)layer * nseg + seg) * M + m0 + wm * 128;
+      // Emission.  Each lane first drops a 16-bit code (row, column) for every candidate of its two
+      // rows into the wavefront's list, at the candidate's ordered position inside the tile; then the
+      // lanes take one candidate each: 64 consecutive pool entries per store instruction, and the
+      // number of rounds is the tile's count / 64 instead of the fullest row's count.
+      const uint32_t rel[2] = {incl0 - cnt[0], tot0 + incl1 - cnt[1]};
 #pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        const int ml = h * 64 + lane;
-        uint32_t pos = off + (h ? tot0 + incl1 - cnt[1] : incl0 - cnt[0]);
-        meta[ml] = ok ? make_uint2(pos, cnt[h]) : make_uint2(0u, 0u);
-        if (!ok) continue;
+      for (int h = 0; h < 2; ++h) meta[h * 64 + lane] = ok ? make_uint2(off + rel[h], cnt[h]) : make_uint2(0u, 0u);
+      if (ok && total <= (uint32_t)CAND_LIST) {
+        uint16_t *lst = cand_list[wave];
 #pragma unroll
-        for (int i = 0; i < NW; ++i) {
-          uint32_t w = W[h][i];
-          while (__ballot(w != 0)) {
-            if (w) {
+        for (int h = 0; h < 2; ++h) {
+          const uint32_t rowcode = (uint32_t)(h * 64 + lane) << 8;
+          uint32_t p = rel[h];
+#pragma unroll
+          for (int i = 0; i < NW; ++i) {
+            uint32_t w = W[h][i];
+            while (w) {
+              lst[p++] = (uint16_t)(rowcode | (uint32_t)(i * 32 + (__ffs(w) - 1)));
+              w &= w - 1u;
+            }
+          }
+        }
+        uint2 *dst = mypool + off;
+#pragma unroll 2
+        for (uint32_t idx = lane; idx < total; idx += 64) {
+          const uint32_t code = lst[idx];
+          const int ml = (int)(code >> 8), c = (int)(code & 255u);
+          const int sl = c / EPS, j = c % EPS;
+          const T rawv = *reinterpret_cast<const T *>(park + ml * 256 + ((sl ^ (ml & 15)) * 16) + j * (int)sizeof(T));
+          dst[idx] = make_uint2((uint32_t)(ncol0 + c), Elem<T>::raw(rawv));
+        }
+      } else if (ok) {
+        // a tile with more candidates than the list holds: every lane walks its own rows
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const int ml = h * 64 + lane;
+          uint32_t pos = off + rel[h];
+#pragma unroll
+          for (int i = 0; i < NW; ++i) {
+            uint32_t w = W[h][i];
+            while (w) {
               const int c = i * 32 + (__ffs(w) - 1);       // column inside the segment
               w &= w - 1u;
               const int sl = c / EPS, j = c % EPS;
@@ -552,3 +613,4 @@ extern "C" int clt_encode(const void *x, const void *w, const void *b, void *pre
   return clt_launch_encode(x, w, b, pre, T, d, F, L, x_layer_stride, w_layer_stride, b_layer_stride,
                            pre_layer_stride, dtype, 0, nullptr, nullptr, (hipStream_t)stream);
 }
+
