@@ -47,7 +47,7 @@ def algorithmic_work(wl, nnz_rows_pairs: int, nnz_total: int):
 # HBM bytes per k_decode launch (FETCH_SIZE + WRITE_SIZE of `rocprofv3 --pmc`, each scaled by
 # what the same counter reads for the known-size copy at the end of this script), keyed by
 # (workload, launches per step).  Filled from the counter runs kept under profiles/.
-MEASURED_TRAFFIC = {("c1", 12): (1580583.0 + 586658.0) * 1024.0}
+MEASURED_TRAFFIC = {("c1", 12): (1583907.0 + 608867.0) * 1024.0}
 
 
 def copy_probe(dev):

@@ -175,14 +175,16 @@ def test_training_steps_match_torch_adam_on_autograd_gradients(dev, dtype, tying
     assert all(torch.isfinite(r).all() for r in rec.values())
 
 
-@pytest.mark.parametrize("shape", [(96, 200), (50, 77)], ids=["vector", "scalar"])
+@pytest.mark.parametrize("shape", [(96, 200), (50, 77), (96, 192), (1028, 128)],
+                         ids=["vector", "scalar", "whole-tiles", "tall"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_adam_kernels_match_torch_adam_on_given_gradients(dev, dtype, shape):
     # same gradients on both sides (zeros and tiny values included): the update itself, three steps
     from crosslayer_coding_amd import _native
     lib = _native.load()
     gen = torch.Generator().manual_seed(5)
-    d, F = shape  # not multiples of the 64 x 64 tile; (50, 77) is not a multiple of 4 either
+    # the first two are not multiples of the 64 x 64 tile, (50, 77) is not a multiple of 4 either
+    d, F = shape
     p0 = (torch.randn(d, F, generator=gen) * 0.1).to(dtype)
     ref = p0.float().clone().requires_grad_(True)
     ropt = torch.optim.Adam([ref], lr=3e-3, betas=(0.9, 0.999), eps=1e-8)
