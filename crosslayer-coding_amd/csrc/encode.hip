@@ -220,6 +220,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
           bv[0] = __uint_as_float(braw[j * 4 + rg].x << 16); bv[1] = __uint_as_float(braw[j * 4 + rg].x & 0xFFFF0000u);
           bv[2] = __uint_as_float(braw[j * 4 + rg].y << 16); bv[3] = __uint_as_float(braw[j * 4 + rg].y & 0xFFFF0000u);
         }
+        // pins the copies into the accumulators here, behind the wait, instead of at the loads
+#pragma unroll
+        for (int q = 0; q < 4; ++q) asm volatile("" : "+v"(bv[q]));
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
