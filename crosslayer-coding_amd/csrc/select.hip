@@ -399,11 +399,22 @@ __global__ __launch_bounds__(256) void k_select_pass(
       const uint32_t total = t0 + t1 + t2 + t3;
       if (n_buf + total > (uint32_t)WBUF) flush();
       const bool fits = total <= (uint32_t)WBUF;
-      if (!fits) dense = true;   // a step denser than the buffer: leave this row to the dense readers
       // start of each vector's candidates in the buffer, plus this lane's exclusive prefix
       const uint32_t sA = (iA - cA) + (n_buf | ((n_buf + t0) << 16));
       const uint32_t sB = (iB - cB) + ((n_buf + t0 + t1) | ((n_buf + t0 + t1 + t2) << 16));
       const uint32_t c0u = (uint32_t)c0;
+      // the lanes finish `cnt` new entries (step-relative columns at wbuf[n_buf ..]) in parallel
+      auto finish = [&](uint32_t cnt) {
+        for (uint32_t i = lane; i < cnt; i += 64) {
+          const uint32_t rel = wbuf[n_buf + i].x;
+          const T rawv = stage[rel];
+          const uint32_t col = c0u + rel;
+          const uint32_t key = rank_key<KB>(rk(Elem<T>::to_f32(rawv), (int64_t)col));
+          atomicAdd(&lh[bin_level0<KB>(key - cut_key)], 1u);
+          wbuf[n_buf + i] = make_uint2(col, Elem<T>::raw(rawv));
+        }
+        n_buf += cnt;
+      };
       if (fits) {
         // each lane drops the step-relative column of its candidates at their ordered slots
         uint32_t mm = m;
@@ -418,26 +429,26 @@ __global__ __launch_bounds__(256) void k_select_pass(
             wbuf[start + below].x = (uint32_t)(q * 64 * V + lane * V + (bit % V));
           }
         }
-        // the lanes finish the new entries in parallel
-        for (uint32_t i = lane; i < total; i += 64) {
-          const uint32_t rel = wbuf[n_buf + i].x;
-          const T rawv = stage[rel];
-          const uint32_t col = c0u + rel;
-          const uint32_t key = rank_key<KB>(rk(Elem<T>::to_f32(rawv), (int64_t)col));
-          atomicAdd(&lh[bin_level0<KB>(key - cut_key)], 1u);
-          wbuf[n_buf + i] = make_uint2(col, Elem<T>::raw(rawv));
-        }
-        n_buf += total;
+        finish(total);
       } else {
-        uint32_t mm = m;   // histogram only
-        while (ballot64(mm != 0)) {
-          if (mm) {
+        // A step with more candidates than the buffer holds (a token whose activations stand out from
+        // the batch): one vector at a time - 64 * V elements always fit - with a flush in between, so
+        // the row keeps its extents and is not left to the slow dense readers.
+        static_assert(64 * V <= WBUF, "one vector of candidates must fit the buffer");
+        const uint32_t exA = iA - cA, exB = iB - cB;
+        const uint32_t tq[PASS_NV] = {t0, t1, t2, t3};
+        const uint32_t exq[PASS_NV] = {exA & 0xFFFFu, exA >> 16, exB & 0xFFFFu, exB >> 16};
+#pragma unroll
+        for (int q = 0; q < PASS_NV; ++q) {
+          if (tq[q] == 0) continue;
+          if (n_buf + tq[q] > (uint32_t)WBUF) flush();
+          uint32_t mm = (m >> (q * V)) & FM, slot = n_buf + exq[q];
+          while (mm) {
             const int bit = __ffs(mm) - 1;
             mm &= mm - 1u;
-            const uint32_t rel = (uint32_t)((bit / V) * 64 * V + lane * V + (bit % V));
-            const uint32_t key = rank_key<KB>(rk(Elem<T>::to_f32(stage[rel]), (int64_t)(c0u + rel)));
-            atomicAdd(&lh[bin_level0<KB>(key - cut_key)], 1u);
+            wbuf[slot++].x = (uint32_t)(q * 64 * V + lane * V + bit);
           }
+          finish(tq[q]);
         }
       }
     }
@@ -512,35 +523,65 @@ __device__ __forceinline__ void visit_candidates(
   const int64_t r = (int64_t)l * Tn + t;
   uint32_t off = row_first[r];
   if (off != ROW_DENSE) {
+    // Up to four steps of 64 entries are fetched together and their keys computed before the first
+    // callback, and the header of the next extent is requested before this extent's entries are used: a
+    // row with thousands of candidates (a token with outlying activations under a batch-wide cut) is
+    // walked by one wavefront, so every serial round trip here is multiplied by its extent count.
+    constexpr int NS = 4;
+    uint2 hdr = make_uint2(ROW_NONE, 0u);
+    if (off != ROW_NONE) hdr = mypool[off];
     while (off != ROW_NONE) {
-      const uint2 hdr = mypool[off];
       const uint2 *sg = mypool + off + 1u;
-      for (uint32_t i0 = 0; i0 < hdr.y; i0 += 64) {
-        uint32_t i = i0 + lane;
-        bool act = i < hdr.y;
-        uint2 e = act ? sg[i] : make_uint2(0, 0);
-        uint32_t key = 0;
-        if (act) key = rank_key<KB>(rk(Elem<T>::to_f32(Elem<T>::from_raw(e.y)), (int64_t)e.x));
-        f(act, e.x, e.y, key);
+      const uint32_t cnt = hdr.y, next = hdr.x;
+      if (next != ROW_NONE) hdr = mypool[next];
+      for (uint32_t i0 = 0; i0 < cnt; i0 += 64 * NS) {
+        bool act[NS]; uint2 e[NS]; uint32_t key[NS];
+#pragma unroll
+        for (int u = 0; u < NS; ++u) {
+          const uint32_t i = i0 + u * 64 + lane;
+          act[u] = i < cnt;
+          e[u] = act[u] ? sg[i] : make_uint2(0, 0);
+        }
+#pragma unroll
+        for (int u = 0; u < NS; ++u) {
+          key[u] = 0;
+          if (act[u]) key[u] = rank_key<KB>(rk(Elem<T>::to_f32(Elem<T>::from_raw(e[u].y)), (int64_t)e[u].x));
+        }
+#pragma unroll
+        for (int u = 0; u < NS; ++u)
+          if (i0 + u * 64 < cnt) f(act[u], e[u].x, e[u].y, key[u]);
       }
-      off = hdr.x;
+      off = next;
     }
   } else {
-    constexpr int NQ = 8;  // independent loads in flight; each covers 64 consecutive columns
+    // The dense row, 64 consecutive columns per load.  The values of the next block of NQ loads are
+    // requested before the current block is ranked, and all keys of a block are computed (the
+    // statistics they need fetched) before its first callback: such a row keeps one wavefront busy for
+    // F / 64 steps, and anything serial per step would make it the tail of the whole launch.
+    constexpr int NQ = 16;
     const T *row = pre + l * lstride + t * F;
-    for (int64_t c0 = 0; c0 < F; c0 += 64 * NQ) {
-      T v[NQ];
+    T v[NQ], vn[NQ];
 #pragma unroll
-      for (int q = 0; q < NQ; ++q) { int64_t col = c0 + q * 64 + lane; v[q] = col < F ? row[col] : T(0); }
+    for (int q = 0; q < NQ; ++q) { const int64_t col = (int64_t)q * 64 + lane; v[q] = col < F ? row[col] : T(0); }
+    for (int64_t c0 = 0; c0 < F; c0 += 64 * NQ) {
+      const int64_t cn = c0 + 64 * NQ;
+#pragma unroll
+      for (int q = 0; q < NQ; ++q) { const int64_t col = cn + q * 64 + lane; vn[q] = col < F ? row[col] : T(0); }
+      uint32_t key[NQ];
+#pragma unroll
+      for (int q = 0; q < NQ; ++q) {
+        const int64_t col = c0 + q * 64 + lane;
+        key[q] = col < F ? rank_key<KB>(rk(Elem<T>::to_f32(v[q]), col)) : 0u;
+      }
 #pragma unroll
       for (int q = 0; q < NQ; ++q) {
         const int64_t col = c0 + q * 64 + lane;
         if (c0 + q * 64 >= F) break;
-        bool act = col < F;
-        uint32_t raw = Elem<T>::raw(v[q]), key = 0;
-        if (act) { key = rank_key<KB>(rk(Elem<T>::to_f32(v[q]), col)); act = key >= cut_key; }
-        f(act, (uint32_t)col, raw, key);
+        const bool act = col < F && key[q] >= cut_key;
+        f(act, (uint32_t)col, (uint32_t)Elem<T>::raw(v[q]), key[q]);
       }
+#pragma unroll
+      for (int q = 0; q < NQ; ++q) v[q] = vn[q];
     }
   }
 }

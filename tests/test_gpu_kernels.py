@@ -332,6 +332,33 @@ def test_batchtopk_global(dev, dtype, L, T, F, k):
         assert torch.equal(got, ref)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_batchtopk_global_outlier_tokens(dev, dtype):
+    # two tokens stand far out of the batch in every feature: under the batch-wide cut nearly all of
+    # their values are candidates, more per step of the streaming pass than its buffer holds
+    g = torch.Generator().manual_seed(21)
+    L, T, F, k = 2, 256, 4096, 24
+    pre = torch.randn(L, T, F, generator=g)
+    pre[:, 7] += 9.0
+    pre[1, 130] += 12.0
+    pre = pre.to(dtype)
+    surv = run_select(pre, k, dev, global_mode=True)
+    check_rows_sorted(surv)
+    assert surv.nnz == k * T
+    got = dense_from(surv)
+    ref = orc.global_batchtopk({l: pre[l] for l in range(L)}, L, k)
+    ref = torch.stack([ref[l] for l in range(L)])
+    z = torch.cat([orc.zscore_for_ranking(pre[l]) for l in range(L)], dim=1).double()
+    kth = torch.topk(z.reshape(-1), k * T).values[-1]
+    band = (2.0 ** -6 if dtype == torch.bfloat16 else 1e-5) * max(abs(float(kth)), 1e-3)
+    zl = torch.stack([z[:, l * F:(l + 1) * F] for l in range(L)])
+    sure = (zl - kth).abs() > band
+    assert torch.equal((got != 0) & sure, (ref != 0) & sure)
+    assert torch.equal(got[got != 0], pre[got != 0])
+    # the outlying tokens do hold most of the survivors
+    assert int((got[:, 7] != 0).sum()) + int((got[1, 130] != 0).sum()) > k * T // 2
+
+
 def test_batchtopk_global_closed_form(dev):
     # hand-computed case of tests/test_oracle_pins.py::test_zscore_closed_form_and_global_selection
     pre = torch.tensor([[[0.0, 5.0], [2.0, 5.0]], [[10.0, -1.0], [10.0, 3.0]]])
