@@ -657,7 +657,10 @@ __device__ __forceinline__ unsigned long long block_excl_scan_u64(unsigned long 
 }
 
 // One block per problem: hand the tie budget out in flat-index order; in per-layer mode
-// also write this layer's part of row_ptr (every layer keeps exactly K rows' worth).
+// also write this layer's part of row_ptr (every layer keeps exactly K rows' worth).  A thread takes
+// SCAN_ITEMS consecutive rows per sweep, so a sweep's round trip to memory and its two block-wide
+// scans are paid once per SCAN_THREADS * SCAN_ITEMS rows.
+constexpr int SCAN_ITEMS = 4;
 template <bool GLOBAL>
 __global__ __launch_bounds__(SCAN_THREADS) void k_select_allot(
     const SelState *st, int64_t Tn, int64_t L, const uint32_t *row_gt, const uint32_t *row_eq,
@@ -666,37 +669,57 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_select_allot(
   const unsigned long long budget = st[p].tie_budget;
   const int64_t nrows = GLOBAL ? Tn * L : Tn;
   unsigned long long eq_run = 0, keep_run = 0;
-  for (int64_t i0 = 0; i0 < nrows; i0 += SCAN_THREADS) {
-    int64_t i = i0 + tid;
-    int64_t r = -1;
-    if (i < nrows) r = GLOBAL ? ((i % L) * Tn + i / L) : ((int64_t)p * Tn + i);
-    unsigned long long eq = r >= 0 ? row_eq[r] : 0, gt = r >= 0 ? row_gt[r] : 0, tot;
-    unsigned long long before = eq_run + block_excl_scan_u64(eq, tot);
+  for (int64_t i0 = 0; i0 < nrows; i0 += (int64_t)SCAN_THREADS * SCAN_ITEMS) {
+    int64_t r[SCAN_ITEMS];
+    unsigned long long eq[SCAN_ITEMS], gt[SCAN_ITEMS], kp[SCAN_ITEMS], eq_sum = 0, kp_sum = 0, tot;
+#pragma unroll
+    for (int j = 0; j < SCAN_ITEMS; ++j) {
+      const int64_t i = i0 + (int64_t)tid * SCAN_ITEMS + j;
+      r[j] = i < nrows ? (GLOBAL ? ((i % L) * Tn + i / L) : ((int64_t)p * Tn + i)) : -1;
+      eq[j] = r[j] >= 0 ? row_eq[r[j]] : 0;
+      gt[j] = r[j] >= 0 ? row_gt[r[j]] : 0;
+      eq_sum += eq[j];
+    }
+    unsigned long long before = eq_run + block_excl_scan_u64(eq_sum, tot);
     eq_run += tot;
-    unsigned long long a = before >= budget ? 0 : (budget - before < eq ? budget - before : eq);
-    unsigned long long kp = gt + a;
-    if (r >= 0) { allot[r] = (uint32_t)a; keep[r] = (uint32_t)kp; }
+#pragma unroll
+    for (int j = 0; j < SCAN_ITEMS; ++j) {
+      const unsigned long long a = before >= budget ? 0 : (budget - before < eq[j] ? budget - before : eq[j]);
+      before += eq[j];
+      kp[j] = gt[j] + a;
+      kp_sum += kp[j];
+      if (r[j] >= 0) { allot[r[j]] = (uint32_t)a; keep[r[j]] = (uint32_t)kp[j]; }
+    }
     if (!GLOBAL) {
       unsigned long long kt;
-      unsigned long long kbefore = keep_run + block_excl_scan_u64(kp, kt);
+      unsigned long long kbefore = keep_run + block_excl_scan_u64(kp_sum, kt);
       keep_run += kt;
-      if (r >= 0) row_ptr[r] = (int32_t)((unsigned long long)p * K + kbefore);
+#pragma unroll
+      for (int j = 0; j < SCAN_ITEMS; ++j) {
+        if (r[j] >= 0) row_ptr[r[j]] = (int32_t)((unsigned long long)p * K + kbefore);
+        kbefore += kp[j];
+      }
     }
   }
   if (!GLOBAL && tid == 0 && p == (int)gridDim.x - 1) row_ptr[(int64_t)gridDim.x * Tn] = (int32_t)((unsigned long long)gridDim.x * K);
 }
 
 // Single block: row_ptr = exclusive scan of keep[] in storage order (row = layer*T + token), one
-// coalesced sweep of SCAN_THREADS rows at a time with a running carry.
+// coalesced sweep of SCAN_THREADS * SCAN_ITEMS rows at a time with a running carry.
 __global__ __launch_bounds__(SCAN_THREADS) void k_rowptr_scan(const uint32_t *keep, int64_t R, int32_t *row_ptr) {
   const int tid = threadIdx.x;
   unsigned long long carry = 0;
-  for (int64_t i0 = 0; i0 < R; i0 += SCAN_THREADS) {
-    const int64_t i = i0 + tid;
-    const unsigned long long v = i < R ? keep[i] : 0;
-    unsigned long long tot;
-    const unsigned long long before = carry + block_excl_scan_u64(v, tot);
-    if (i < R) row_ptr[i] = (int32_t)before;
+  for (int64_t i0 = 0; i0 < R; i0 += (int64_t)SCAN_THREADS * SCAN_ITEMS) {
+    const int64_t i = i0 + (int64_t)tid * SCAN_ITEMS;
+    unsigned long long v[SCAN_ITEMS], sum = 0, tot;
+#pragma unroll
+    for (int j = 0; j < SCAN_ITEMS; ++j) { v[j] = i + j < R ? keep[i + j] : 0; sum += v[j]; }
+    unsigned long long before = carry + block_excl_scan_u64(sum, tot);
+#pragma unroll
+    for (int j = 0; j < SCAN_ITEMS; ++j) {
+      if (i + j < R) row_ptr[i + j] = (int32_t)before;
+      before += v[j];
+    }
     carry += tot;
   }
   if (tid == 0) row_ptr[R] = (int32_t)carry;
