@@ -346,41 +346,41 @@ __global__ __launch_bounds__(256) void k_select_pass(
       }
       n_buf = 0;
     };
+    // global ranking, first pass: the z-score is monotone in x, so "z reaches the cut" is
+    // "x reaches the column's own bound" (k_col_cut), one compare instead of a division
+    const bool by_column = GLOBAL && V > 1 && phase == 0 && xcut != nullptr;
     for (int64_t c0 = 0; c0 < F; c0 += STEP) {
-      uint4 w[PASS_NV];
+      // all loads of the step - values and, when ranking by column, the bounds - go out together,
+      // unpredicated (a vector past the end of the row reads the row's start and is masked below)
+      uint4 w[PASS_NV], xc[PASS_NV];
       bool on[PASS_NV];
 #pragma unroll
       for (int q = 0; q < PASS_NV; ++q) {
         const int64_t col = c0 + (int64_t)q * 64 * V + (int64_t)lane * V;
         on[q] = col < F;
-        w[q] = make_uint4(0, 0, 0, 0);
-        if (on[q]) {
-          if (V > 1) w[q] = *reinterpret_cast<const uint4 *>(row + col);
-          else w[q].x = sizeof(T) == 2 ? ((uint32_t)Elem<T>::raw(row[col]) << 16) : (uint32_t)Elem<T>::raw(row[col]);
-        }
+        const int64_t cl = on[q] ? col : 0;
+        if (V > 1) w[q] = *reinterpret_cast<const uint4 *>(row + cl);
+        else w[q] = make_uint4(sizeof(T) == 2 ? ((uint32_t)Elem<T>::raw(row[cl]) << 16) : (uint32_t)Elem<T>::raw(row[cl]), 0, 0, 0);
+        xc[q] = make_uint4(0, 0, 0, 0);
+        if (V > 1 && by_column) xc[q] = *reinterpret_cast<const uint4 *>(xcut + (int64_t)l * F + cl);
       }
       uint32_t m = 0;  // bit q*V + j: element j of vector q reaches the cut
-      // global ranking, first pass: the z-score is monotone in x, so "z reaches the cut" is
-      // "x reaches the column's own bound" (k_col_cut), one compare instead of a division
-      const bool by_column = GLOBAL && V > 1 && phase == 0 && xcut != nullptr;
 #pragma unroll
       for (int q = 0; q < PASS_NV; ++q) {
         const int64_t col = c0 + (int64_t)q * 64 * V + (int64_t)lane * V;
-        if (on[q]) {
-          uint4 xc = make_uint4(0, 0, 0, 0);
-          if (by_column) xc = *reinterpret_cast<const uint4 *>(xcut + (int64_t)l * F + col);
+        uint32_t mq = 0;
 #pragma unroll
-          for (int j = 0; j < V; ++j) {
-            const float xv = V > 1 ? vec_elem<T>(w[q], j) : __uint_as_float(w[q].x);
-            bool c;
-            if (by_column) c = xv >= vec_elem<T>(xc, j) || xv != xv;
-            else {
-              const float rv = rk(xv, col + j);
-              c = cut_nan ? (rv != rv) : !(rv < cutf);
-            }
-            m |= (c ? 1u : 0u) << (q * V + j);
+        for (int j = 0; j < V; ++j) {
+          const float xv = V > 1 ? vec_elem<T>(w[q], j) : __uint_as_float(w[q].x);
+          bool c;
+          if (by_column) c = xv >= vec_elem<T>(xc[q], j) || xv != xv;
+          else {
+            const float rv = rk(xv, col + j);
+            c = cut_nan ? (rv != rv) : !(rv < cutf);
           }
+          mq |= (c ? 1u : 0u) << j;
         }
+        if (on[q]) m |= mq << (q * V);
       }
       if (ballot64(m != 0) == 0) continue;
       // stage the step in column order: stage[col - c0]
