@@ -149,6 +149,12 @@ __device__ __forceinline__ void stg_stream4(float *p, float4 v) {
   __builtin_nontemporal_store(q, reinterpret_cast<f32x4_t *>(p));
 }
 
+template <typename T, int NF, int TAIL, bool SLICED> constexpr int decode_min_waves() {
+  constexpr int V = 16 / (int)sizeof(T);
+  constexpr int nacc = NF * V + (TAIL == 1 ? V / 2 : TAIL == 2 ? V : 0);
+  return (SLICED && sizeof(T) == 2 && nacc <= 12) ? 4 : 1;
+}
+
 constexpr int SLICED_NTOK = 4;   // tokens per wavefront in the sliced kernel
 
 // One wavefront per (target, token): walks all sources s <= t, accumulates in registers,
@@ -165,7 +171,11 @@ constexpr int SLICED_NTOK = 4;   // tokens per wavefront in the sliced kernel
 // reads, updates and writes back (skipped when the token has no survivor in the slice).
 // k_decode_reduce finally adds the slices in a fixed order and applies bias / skip / rounding.
 template <typename T, int NF, int TAIL, int U, bool AFFINE, bool SLICED>
-__global__ __launch_bounds__(256) void k_decode(
+// The sliced variant with up to 12 accumulators per lane (d <= 768 in bf16) needs 129 registers when left
+// alone, one more than four wavefronts per SIMD allow; held to 128 it spills nothing and runs 4 % faster.
+// Wider rows would spill at that limit and keep the compiler's own choice.
+__global__ __launch_bounds__(256)
+__attribute__((amdgpu_waves_per_eu(decode_min_waves<T, NF, TAIL, SLICED>(), 8))) void k_decode(
     const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ col, const T *__restrict__ val,
     const T *__restrict__ wp, const float *__restrict__ bias_sum, const T *__restrict__ foff,
     const T *__restrict__ fscale, const float *__restrict__ skip_add, void *__restrict__ out,
@@ -359,6 +369,185 @@ __global__ __launch_bounds__(256) void k_decode(
   if (TAIL == 2) emit(tail_off, acc + NF * V, V, tail_on);
 }
 
+// ---- half-row schedule ----------------------------------------------------------------------------
+// Large batches, untied or per-source decoders, d a multiple of 256: the feature axis is cut into 4
+// slices and the columns into 2 halves; workgroup b works on part b % 8 = (slice, half), so an XCD still
+// gathers from one 1/8 of one decoder matrix at a time (F/4 rows x d/2 columns) but a (target, token)
+// has 4 partial rows instead of 8: half the fp32 read-modify-write traffic between source launches.
+// So that a half row (768 bytes at d = 768) costs no more instructions than its share of a whole one,
+// a wavefront fetches TWO rows per load: lanes 0-31 take one survivor's half row, lanes 32-63 the next
+// survivor's, 16 (+8) bytes per lane; each half of the wavefront accumulates its own rows and the two
+// halves are added once per token.
+template <typename T, int HQ, int HTAIL, int UU> struct HalfBatch {
+  uint4 wq[UU][HQ > 0 ? HQ : 1];
+  uint2 wt8[UU];
+  float v[UU];
+  // slots i0 .. i0 + 2*UU - 1 of the (up to 64) survivors held one per lane: slot 2u goes to lanes 0-31,
+  // slot 2u+1 to lanes 32-63
+  __device__ __forceinline__ void load(const T *wbase, int64_t d, int32_t my_col, float my_val, int i0, int n, int ll, bool hi) {
+    constexpr int V = WVec<T>::V;
+#pragma unroll
+    for (int u = 0; u < UU; ++u) {
+      const int ia = i0 + 2 * u, ib = ia + 1;
+      const int ca = ia < n ? ia : n - 1, cb = ib < n ? ib : n - 1;   // clamp: a repeated fetch, weight 0
+      const int32_t fa = __builtin_amdgcn_readlane(my_col, ca), fb = __builtin_amdgcn_readlane(my_col, cb);
+      const float va = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(my_val), ca));
+      const float vb = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(my_val), cb));
+      const int32_t f = hi ? fb : fa;
+      v[u] = hi ? (ib < n ? vb : 0.0f) : (ia < n ? va : 0.0f);
+      const T *wrow = wbase + (int64_t)f * d;
+#pragma unroll
+      for (int c = 0; c < HQ; ++c) wq[u][c] = *reinterpret_cast<const uint4 *>(wrow + c * 32 * V + ll * V);
+      if (HTAIL) wt8[u] = *reinterpret_cast<const uint2 *>(wrow + HQ * 32 * V + ll * (V / 2));
+    }
+  }
+  __device__ __forceinline__ void consume(float *acc) const {
+    constexpr int V = WVec<T>::V;
+    if constexpr (sizeof(T) == 2 && (UU % 2) == 0) {
+#pragma unroll
+      for (int u = 0; u < UU; u += 2) {
+        const uint32_t vb = (__float_as_uint(v[u]) >> 16) | (__float_as_uint(v[u + 1]) & 0xFFFF0000u);
+        const bf16x2_t vv = __builtin_bit_cast(bf16x2_t, vb);
+#pragma unroll
+        for (int c = 0; c < HQ; ++c) WVec<T>::dot16(acc + c * V, wq[u][c], wq[u + 1][c], vv);
+        if (HTAIL) WVec<T>::dot8(acc + HQ * V, wt8[u], wt8[u + 1], vv);
+      }
+    } else {
+#pragma unroll
+      for (int u = 0; u < UU; ++u) {
+#pragma unroll
+        for (int c = 0; c < HQ; ++c) WVec<T>::fma16(acc + c * V, wq[u][c], v[u]);
+        if (HTAIL) WVec<T>::fma8(acc + HQ * V, wt8[u], v[u]);
+      }
+    }
+  }
+};
+
+constexpr int HALF_SLICES = 4;
+constexpr int HALF_NTOK = 2;     // tokens per wavefront
+// 12 accumulators per lane (d = 768): 65 registers, seven wavefronts per SIMD; wider rows are left alone
+template <typename T, int HQ, int HTAIL> constexpr int half_min_waves() {
+  constexpr int V = 16 / (int)sizeof(T);
+  return (sizeof(T) == 2 && HQ * V + (HTAIL ? V / 2 : 0) <= 12) ? 7 : 1;   // fp32 at 7 would spill
+}
+
+template <typename T, int HQ, int HTAIL, int UU, bool AFFINE>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(half_min_waves<T, HQ, HTAIL>(), 8))) void k_decode_half(
+    const int32_t *__restrict__ col, const T *__restrict__ val, const T *__restrict__ wp, const T *__restrict__ foff,
+    const T *__restrict__ fscale, int64_t Tn, int64_t d, int64_t F, int64_t L, int tying, int64_t t_begin, uint64_t src_mask,
+    const int32_t *__restrict__ sptr, float *__restrict__ partial, int src) {
+  constexpr int V = WVec<T>::V;
+  constexpr int NACC = HQ * V + (HTAIL ? V / 2 : 0);      // columns per lane: d / 64
+  constexpr int ns = HALF_SLICES;
+  const int lane = lane_id(), wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
+  const int ll = lane & 31;
+  const bool hi = lane >= 32;
+  const int part = (int)(blockIdx.x % 8), slice = part & 3, half = part >> 2;
+  const int64_t bid = (int64_t)blockIdx.x / 8;
+  const int64_t blocks_per_t = (Tn + (int64_t)nwv * HALF_NTOK - 1) / ((int64_t)nwv * HALF_NTOK);
+  const int64_t t = t_begin + bid / blocks_per_t;
+  const int64_t tok0 = ((bid % blocks_per_t) * nwv + wv) * HALF_NTOK;
+  if (tok0 >= Tn) return;
+  const uint64_t below = src_mask & ((1ull << src) - 1ull);
+  const bool first = below == 0;   // the first source initialises the partial rows
+  int32_t mb = 0, me = 0;
+  if (lane < HALF_NTOK && tok0 + lane < Tn) {
+    const int64_t r = (int64_t)src * Tn + tok0 + lane;
+    mb = sptr[r * (ns + 1) + slice];
+    me = sptr[r * (ns + 1) + slice + 1];
+  }
+  const T *wbase = wp + decoder_slot(tying, src, t, L) * F * d + (int64_t)half * (d / 2);
+  int32_t nb = __builtin_amdgcn_readlane(mb, 0), ne = __builtin_amdgcn_readlane(me, 0);
+  int32_t nxt_col = 0; T nxt_val = T(0);
+  if (lane < ne - nb) { nxt_col = col[nb + lane]; nxt_val = val[nb + lane]; }
+#pragma unroll
+  for (int i = 0; i < HALF_NTOK; ++i) {
+    const int32_t b = nb, e = ne;
+    const int32_t cur_col = nxt_col; const T cur_val = nxt_val;
+    if (i + 1 < HALF_NTOK) {
+      nb = __builtin_amdgcn_readlane(mb, i + 1); ne = __builtin_amdgcn_readlane(me, i + 1);
+      nxt_col = 0; nxt_val = T(0);
+      if (lane < ne - nb) { nxt_col = col[nb + lane]; nxt_val = val[nb + lane]; }
+    }
+    if (tok0 + i >= Tn) break;
+    if (b == e && !first) continue;
+    // this lane's columns of the partial row (lanes 0-31 write it): pieces of V, then the tail
+    float *prow = partial + (((int64_t)slice * L + t) * Tn + tok0 + i) * d + (int64_t)half * (d / 2);
+    float old[NACC], acc[NACC];
+#pragma unroll
+    for (int j = 0; j < NACC; ++j) { old[j] = 0.0f; acc[j] = 0.0f; }
+    for (int32_t j0 = b; j0 < e; j0 += 64) {
+      const int n = (e - j0) < 64 ? (e - j0) : 64;
+      int32_t my_col = cur_col; float my_val = Elem<T>::to_f32(cur_val);
+      if (j0 > b) {   // more than 64 survivors in this slice: fetch the next 64
+        my_col = 0; my_val = 0.0f;
+        if (lane < n) { my_col = col[j0 + lane]; my_val = Elem<T>::to_f32(val[j0 + lane]); }
+      }
+      if (AFFINE && my_val != 0.0f) {
+        if (foff) my_val = Elem<T>::round(my_val + Elem<T>::to_f32(foff[t * F + my_col]));
+        if (fscale) my_val = Elem<T>::round(my_val * Elem<T>::to_f32(fscale[t * F + my_col]));
+      }
+      // two batches of UU row pairs in flight
+      HalfBatch<T, HQ, HTAIL, UU> ra, rb;
+      ra.load(wbase, d, my_col, my_val, 0, n, ll, hi);
+      for (int i0 = 0; i0 < n; i0 += 4 * UU) {
+        if (i0 + 2 * UU < n) rb.load(wbase, d, my_col, my_val, i0 + 2 * UU, n, ll, hi);
+        ra.consume(acc);
+        if (i0 + 2 * UU < n) {
+          if (i0 + 4 * UU < n) ra.load(wbase, d, my_col, my_val, i0 + 4 * UU, n, ll, hi);
+          rb.consume(acc);
+        }
+      }
+    }
+    // The old partial row is asked for only now: held across the gathers it would cost 12 registers and
+    // one wavefront per SIMD, and the other wavefronts cover its latency better than an early request.
+    if (!first && !hi) {
+#pragma unroll
+      for (int c = 0; c < HQ; ++c) {
+#pragma unroll
+        for (int j = 0; j < V; j += 4) {
+          const float4 q = ldg_stream4(prow + c * 32 * V + ll * V + j);
+          old[c * V + j] = q.x; old[c * V + j + 1] = q.y; old[c * V + j + 2] = q.z; old[c * V + j + 3] = q.w;
+        }
+      }
+      if (HTAIL) {
+        if constexpr (V / 2 == 4) {
+          const float4 q = ldg_stream4(prow + HQ * 32 * V + ll * 4);
+          old[HQ * V] = q.x; old[HQ * V + 1] = q.y; old[HQ * V + 2] = q.z; old[HQ * V + 3] = q.w;
+        } else {
+#pragma unroll
+          for (int j = 0; j < V / 2; ++j) old[HQ * V + j] = prow[HQ * 32 * V + ll * (V / 2) + j];
+        }
+      }
+    }
+    // the two halves of the wavefront hold sums over different survivors: add them, in a fixed order
+#pragma unroll
+    for (int j = 0; j < NACC; ++j) {
+      const float other = __shfl_xor(acc[j], 32);
+      acc[j] = hi ? other + acc[j] : acc[j] + other;
+    }
+    if (!hi) {
+#pragma unroll
+      for (int c = 0; c < HQ; ++c) {
+#pragma unroll
+        for (int j = 0; j < V; j += 4)
+          stg_stream4(prow + c * 32 * V + ll * V + j,
+                      make_float4(old[c * V + j] + acc[c * V + j], old[c * V + j + 1] + acc[c * V + j + 1],
+                                  old[c * V + j + 2] + acc[c * V + j + 2], old[c * V + j + 3] + acc[c * V + j + 3]));
+      }
+      if (HTAIL) {
+        if constexpr (V / 2 == 4) {
+          stg_stream4(prow + HQ * 32 * V + ll * 4, make_float4(old[HQ * V] + acc[HQ * V], old[HQ * V + 1] + acc[HQ * V + 1],
+                                                               old[HQ * V + 2] + acc[HQ * V + 2], old[HQ * V + 3] + acc[HQ * V + 3]));
+        } else {
+#pragma unroll
+          for (int j = 0; j < V / 2; ++j) prow[HQ * 32 * V + ll * (V / 2) + j] = old[HQ * V + j] + acc[HQ * V + j];
+        }
+      }
+    }
+  }
+}
+
 // sptr[r][j] = first survivor of row r whose feature index is >= j * F / ns  (j = 0..ns)
 __global__ void k_slice_ptr(const int32_t *row_ptr, const int32_t *col, int64_t R, int64_t F, int ns, int32_t *sptr) {
   const int64_t total = R * (ns + 1);
@@ -544,7 +733,6 @@ static int launch_decode(const int32_t *row_ptr, const int32_t *col, const void 
   const bool fast = (d % V == 0) && clt_aligned16(wp) && nf <= 4 && (nf > 0 || rem > 0);
   if (can_slice && !fast) return launch_decode<T>(row_ptr, col, val, wp, bias_sum, foff, fscale, skip_add, out, Tn, d, F,
                                                   L, tying, t_begin, t_end, src_mask, out_f32, nullptr, 0, stream);
-  if (can_slice) k_slice_ptr<<<1024, 256, 0, stream>>>(row_ptr, col, L * Tn, F, ns, sptr);
 #define CLT_DEC_ARGS(FO, FS)                                                                                    \
   row_ptr, col, (const T *)val, (const T *)wp, bias_sum, FO, FS, skip_add, out, Tn, d, F, L, tying, tb,         \
       t_end, src_mask, out_f32, sptr, partial, ns, src
@@ -565,6 +753,45 @@ static int launch_decode(const int32_t *row_ptr, const int32_t *col, const void 
     else if (rem * 2 == chunk) CLT_DEC(NFN, 1, UN);        \
     else CLT_DEC(NFN, 2, UN);                              \
   } while (0)
+  // half-row schedule: 4 feature slices x 2 column halves (see k_decode_half)
+  bool halved = false;
+  if (fast && can_slice && tying != CLT_TYING_PER_TARGET && d % 256 == 0 && F >= 64 * HALF_SLICES) {
+    const int per_lane = (int)(d / 64);                    // columns per lane
+    const int hq = per_lane / V, htail = (per_lane % V) != 0;
+    const int64_t hblk_per_t = clt_ceil_div(Tn, nwv * HALF_NTOK);
+#define CLT_DECH(HQN, HTN, UN)                                                                                       \
+  do {                                                                                                               \
+    k_slice_ptr<<<1024, 256, 0, stream>>>(row_ptr, col, L * Tn, F, HALF_SLICES, sptr);                               \
+    for (int src = 0; src < (int)t_end; ++src) {                                                                     \
+      if (!((src_mask >> src) & 1ull)) continue;                                                                     \
+      const int64_t tb = src > t_begin ? src : t_begin;                                                              \
+      const int64_t hb = hblk_per_t * (t_end - tb) * 8;                                                              \
+      if (hb <= 0) continue;                                                                                         \
+      if (hb > 2147483647LL) return CLT_ERR_RANGE;                                                                   \
+      if (affine) k_decode_half<T, HQN, HTN, UN, true><<<(unsigned)hb, 256, 0, stream>>>(col, (const T *)val, (const T *)wp, \
+          (const T *)foff, (const T *)fscale, Tn, d, F, L, tying, tb, src_mask, sptr, partial, src);                 \
+      else k_decode_half<T, HQN, HTN, UN, false><<<(unsigned)hb, 256, 0, stream>>>(col, (const T *)val, (const T *)wp, \
+          nullptr, nullptr, Tn, d, F, L, tying, tb, src_mask, sptr, partial, src);                                   \
+    }                                                                                                                \
+    halved = true;                                                                                                   \
+  } while (0)
+    if constexpr (sizeof(T) == 2) {
+      if (hq == 1 && !htail) CLT_DECH(1, 0, 2);
+      else if (hq == 1 && htail) CLT_DECH(1, 1, 2);
+      else if (hq == 2 && !htail) CLT_DECH(2, 0, 2);
+      else if (hq == 4 && !htail) CLT_DECH(4, 0, 2);
+    } else {
+      if (hq == 2 && !htail) CLT_DECH(2, 0, 2);
+      else if (hq == 3 && !htail) CLT_DECH(3, 0, 2);
+      else if (hq == 4 && !htail) CLT_DECH(4, 0, 2);
+    }
+#undef CLT_DECH
+  }
+  if (halved) {
+    k_decode_reduce<T><<<2048, 256, 0, stream>>>(partial, bias_sum, skip_add, out, Tn, d, L, t_begin, t_end, HALF_SLICES, out_f32, src_mask);
+    return clt_check_launch();
+  }
+  if (can_slice) k_slice_ptr<<<1024, 256, 0, stream>>>(row_ptr, col, L * Tn, F, ns, sptr);
   if (fast) {
     // sliced: one launch per source layer, targets max(src, t_begin) .. t_end-1
     // decoders tied per target: one launch, sources walked inside the wavefront (src = -1)

@@ -519,11 +519,14 @@ def test_decode_sparse_parity(dev, dtype, tying, L, T, d, F):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("tying", ["none", "per_target"])
-def test_decode_sliced_matches_single_pass(dev, dtype, tying):
-    # the XCD-sliced kernel (workspace given) against the one-wavefront-per-row kernel and the oracle
+@pytest.mark.parametrize("tying,d", [("none", 768), ("per_source", 768), ("none", 1024), ("none", 640), ("per_source", 320),
+                                     ("per_target", 768)])
+def test_decode_sliced_matches_single_pass(dev, dtype, tying, d):
+    # the XCD-sliced schedules (workspace given) against the one-wavefront-per-row kernel and the oracle:
+    # d a multiple of 256 takes the half-row kernel (4 feature slices x 2 column halves) unless the decoders
+    # are tied per target; other widths and per-target tying take the 8-slice kernel
     g = torch.Generator().manual_seed(21)
-    L, T, d, F = 3, 160, 768, 1024
+    L, T, F = 3, 161, 1024
     names, w, b = make_decoder(L, d, F, tying, dtype, g)
     acts = (torch.randn(L, T, F, generator=g) * (torch.rand(L, T, F, generator=g) < 0.05)).to(dtype)
     acts[0, 5] = 0                                     # an empty row
