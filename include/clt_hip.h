@@ -274,11 +274,12 @@ int clt_pack_decoder(const void *w_ref, void *w_packed, int64_t d, int64_t F,
  * (clt/models/clt.py:192-199).
  * Limits: L <= 64; d % 8 == 0 (bf16) / d % 4 == 0 (fp32) on the fast path.
  * workspace: NULL runs one wavefront per (target, token) over all features and sources.
- * With a workspace of clt_decode_workspace_bytes() the feature axis is cut into 8 slices,
- * one per XCD, and there is one launch per source layer, so that each slice of a decoder
- * matrix stays in one L2 while all tokens pass; partial sums live as fp32 rows per (slice,
- * target, token) in the workspace and are added in a fixed order at the end.  Both give the
- * same result up to fp32 summation order.
+ * With a workspace of clt_decode_workspace_bytes() each of the 8 XCDs works on one eighth of a
+ * decoder matrix at a time - 4 feature slices x 2 column halves when d is a multiple of 256 and
+ * the decoders are not tied per target, 8 feature slices of whole rows otherwise - with one
+ * launch per source layer, so that the eighth stays in one L2 while all tokens pass; partial
+ * sums live as fp32 rows per (slice, target, token) in the workspace and are added in a fixed
+ * order at the end.  All routes give the same result up to fp32 summation order.
  */
 size_t clt_decode_workspace_bytes(int64_t T, int64_t d, int64_t F, int64_t L);
 int clt_decode_sparse(const int32_t *row_ptr, const int32_t *col, const void *val,
