@@ -47,7 +47,7 @@ def algorithmic_work(wl, nnz_rows_pairs: int, nnz_total: int):
 # HBM bytes per decode launch (FETCH_SIZE + WRITE_SIZE of `rocprofv3 --pmc`, each scaled by
 # what the same counter reads for the known-size copy at the end of this script), keyed by
 # (workload, launches per step).  Filled from the counter runs kept under profiles/.
-MEASURED_TRAFFIC = {("c1", 12): (1617609.0 + 303514.0) * 1024.0}
+MEASURED_TRAFFIC = {("c1", 12): (1756599.0 + 152273.0) * 1024.0}
 
 
 def copy_probe(dev):
@@ -152,9 +152,9 @@ def run_gpu(args):
     # slice-pointer kernel before and one reduce kernel after, timed with them); a small batch
     # is a single launch
     n_dec_launch = L if T * L >= engine.SLICED_DECODE_MIN_ROWS else 1
-    # widths that are a multiple of 256 take the half-row kernel unless the decoders are tied per target
-    half_rows = n_dec_launch > 1 and wl.d_model % 256 == 0 and wl.decoder_tying != "per_target"
-    dec_kernel_desc = (f"{'k_decode_half' if half_rows else 'k_decode'} (sparse cross-layer decode; {n_dec_launch} "
+    # widths that are a multiple of 256 take the quarter-row kernel unless the decoders are tied per target
+    quarter_rows = n_dec_launch > 1 and wl.d_model % 256 == 0 and wl.decoder_tying != "per_target"
+    dec_kernel_desc = (f"{'k_decode_quarter' if quarter_rows else 'k_decode'} (sparse cross-layer decode; {n_dec_launch} "
                        "launch(es) per step; the per-launch figures are the step's decode stage divided by that count)")
     traffic = MEASURED_TRAFFIC.get((wl.name, n_dec_launch))
     mfma_peak = MFMA_BF16_PEAK_TF if wl.dtype == "bfloat16" else MFMA_FP32_PEAK_TF

@@ -369,36 +369,37 @@ __attribute__((amdgpu_waves_per_eu(decode_min_waves<T, NF, TAIL, SLICED>(), 8)))
   if (TAIL == 2) emit(tail_off, acc + NF * V, V, tail_on);
 }
 
-// ---- half-row schedule ----------------------------------------------------------------------------
-// Large batches, untied or per-source decoders, d a multiple of 256: the feature axis is cut into 4
-// slices and the columns into 2 halves; workgroup b works on part b % 8 = (slice, half), so an XCD still
-// gathers from one 1/8 of one decoder matrix at a time (F/4 rows x d/2 columns) but a (target, token)
-// has 4 partial rows instead of 8: half the fp32 read-modify-write traffic between source launches.
-// So that a half row (768 bytes at d = 768) costs no more instructions than its share of a whole one,
-// a wavefront fetches TWO rows per load: lanes 0-31 take one survivor's half row, lanes 32-63 the next
-// survivor's, 16 (+8) bytes per lane; each half of the wavefront accumulates its own rows and the two
-// halves are added once per token.
-template <typename T, int HQ, int HTAIL, int UU> struct HalfBatch {
+// ---- quarter-row schedule -------------------------------------------------------------------------
+// Large batches, untied or per-source decoders, d a multiple of 256: the feature axis is cut into 2
+// slices and the columns into 4 quarters; workgroup b works on part b % 8 = (slice, quarter), so an XCD
+// still gathers from one 1/8 of one decoder matrix at a time (F/2 rows x d/4 columns) but a (target,
+// token) has 2 partial rows instead of 8: a quarter of the fp32 read-modify-write traffic between source
+// launches.  So that a quarter row (384 bytes at d = 768, three whole cache lines) costs no more
+// instructions than its share of a whole one, a wavefront fetches FOUR rows per load: each group of
+// QLANES = 16 lanes takes one survivor's quarter row, 16 (+8) bytes per lane; every group accumulates
+// its own rows and the four groups are added once per token.
+constexpr int QLANES = 16;              // lanes per quarter row
+constexpr int QROWS = 64 / QLANES;      // rows per load
+constexpr int QUARTER_SLICES = 2;       // feature slices; 8 / QUARTER_SLICES column parts
+constexpr int QUARTER_PARTS = 8 / QUARTER_SLICES;
+template <typename T, int HQ, int HTAIL, int UU> struct PartBatch {
   uint4 wq[UU][HQ > 0 ? HQ : 1];
   uint2 wt8[UU];
   float v[UU];
-  // slots i0 .. i0 + 2*UU - 1 of the (up to 64) survivors held one per lane: slot 2u goes to lanes 0-31,
-  // slot 2u+1 to lanes 32-63
-  __device__ __forceinline__ void load(const T *wbase, int64_t d, int32_t my_col, float my_val, int i0, int n, int ll, bool hi) {
+  // slot QROWS * u + g of the (up to 64) survivors held one per lane goes to lane group g
+  __device__ __forceinline__ void load(const T *wbase, int64_t d, int32_t my_col, float my_val, int i0, int n, int ll, int grp) {
     constexpr int V = WVec<T>::V;
 #pragma unroll
     for (int u = 0; u < UU; ++u) {
-      const int ia = i0 + 2 * u, ib = ia + 1;
-      const int ca = ia < n ? ia : n - 1, cb = ib < n ? ib : n - 1;   // clamp: a repeated fetch, weight 0
-      const int32_t fa = __builtin_amdgcn_readlane(my_col, ca), fb = __builtin_amdgcn_readlane(my_col, cb);
-      const float va = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(my_val), ca));
-      const float vb = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(my_val), cb));
-      const int32_t f = hi ? fb : fa;
-      v[u] = hi ? (ib < n ? vb : 0.0f) : (ia < n ? va : 0.0f);
+      const int idx = i0 + QROWS * u + grp;
+      const int ci = idx < n ? idx : n - 1;                 // clamp: a repeated fetch, weight 0
+      const int32_t f = __shfl(my_col, ci);
+      const float vv = __shfl(my_val, ci);
+      v[u] = idx < n ? vv : 0.0f;
       const T *wrow = wbase + (int64_t)f * d;
 #pragma unroll
-      for (int c = 0; c < HQ; ++c) wq[u][c] = *reinterpret_cast<const uint4 *>(wrow + c * 32 * V + ll * V);
-      if (HTAIL) wt8[u] = *reinterpret_cast<const uint2 *>(wrow + HQ * 32 * V + ll * (V / 2));
+      for (int c = 0; c < HQ; ++c) wq[u][c] = *reinterpret_cast<const uint4 *>(wrow + c * QLANES * V + ll * V);
+      if (HTAIL) wt8[u] = *reinterpret_cast<const uint2 *>(wrow + HQ * QLANES * V + ll * (V / 2));
     }
   }
   __device__ __forceinline__ void consume(float *acc) const {
@@ -423,56 +424,55 @@ template <typename T, int HQ, int HTAIL, int UU> struct HalfBatch {
   }
 };
 
-constexpr int HALF_SLICES = 4;
-constexpr int HALF_NTOK = 2;     // tokens per wavefront
-// 12 accumulators per lane (d = 768): 65 registers, seven wavefronts per SIMD; wider rows are left alone
-template <typename T, int HQ, int HTAIL> constexpr int half_min_waves() {
+constexpr int QUARTER_NTOK = 2;     // tokens per wavefront
+// 12 accumulators per lane (d = 768): 72 registers, seven wavefronts per SIMD; wider rows are left alone
+template <typename T, int HQ, int HTAIL> constexpr int quarter_min_waves() {
   constexpr int V = 16 / (int)sizeof(T);
   return (sizeof(T) == 2 && HQ * V + (HTAIL ? V / 2 : 0) <= 12) ? 7 : 1;   // fp32 at 7 would spill
 }
 
 template <typename T, int HQ, int HTAIL, int UU, bool AFFINE>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(half_min_waves<T, HQ, HTAIL>(), 8))) void k_decode_half(
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(quarter_min_waves<T, HQ, HTAIL>(), 8))) void k_decode_quarter(
     const int32_t *__restrict__ col, const T *__restrict__ val, const T *__restrict__ wp, const T *__restrict__ foff,
     const T *__restrict__ fscale, int64_t Tn, int64_t d, int64_t F, int64_t L, int tying, int64_t t_begin, uint64_t src_mask,
     const int32_t *__restrict__ sptr, float *__restrict__ partial, int src) {
   constexpr int V = WVec<T>::V;
   constexpr int NACC = HQ * V + (HTAIL ? V / 2 : 0);      // columns per lane: d / 64
-  constexpr int ns = HALF_SLICES;
+  constexpr int ns = QUARTER_SLICES, NCP = QUARTER_PARTS;
   const int lane = lane_id(), wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
-  const int ll = lane & 31;
-  const bool hi = lane >= 32;
-  const int part = (int)(blockIdx.x % 8), slice = part & 3, half = part >> 2;
+  const int ll = lane & (QLANES - 1), grp = lane / QLANES;
+  const bool hi = grp != 0;                    // only the first lane group touches the partial row
+  const int part = (int)(blockIdx.x % 8), slice = part % ns, cpart = part / ns;
   const int64_t bid = (int64_t)blockIdx.x / 8;
-  const int64_t blocks_per_t = (Tn + (int64_t)nwv * HALF_NTOK - 1) / ((int64_t)nwv * HALF_NTOK);
+  const int64_t blocks_per_t = (Tn + (int64_t)nwv * QUARTER_NTOK - 1) / ((int64_t)nwv * QUARTER_NTOK);
   const int64_t t = t_begin + bid / blocks_per_t;
-  const int64_t tok0 = ((bid % blocks_per_t) * nwv + wv) * HALF_NTOK;
+  const int64_t tok0 = ((bid % blocks_per_t) * nwv + wv) * QUARTER_NTOK;
   if (tok0 >= Tn) return;
   const uint64_t below = src_mask & ((1ull << src) - 1ull);
   const bool first = below == 0;   // the first source initialises the partial rows
   int32_t mb = 0, me = 0;
-  if (lane < HALF_NTOK && tok0 + lane < Tn) {
+  if (lane < QUARTER_NTOK && tok0 + lane < Tn) {
     const int64_t r = (int64_t)src * Tn + tok0 + lane;
     mb = sptr[r * (ns + 1) + slice];
     me = sptr[r * (ns + 1) + slice + 1];
   }
-  const T *wbase = wp + decoder_slot(tying, src, t, L) * F * d + (int64_t)half * (d / 2);
+  const T *wbase = wp + decoder_slot(tying, src, t, L) * F * d + (int64_t)cpart * (d / NCP);
   int32_t nb = __builtin_amdgcn_readlane(mb, 0), ne = __builtin_amdgcn_readlane(me, 0);
   int32_t nxt_col = 0; T nxt_val = T(0);
   if (lane < ne - nb) { nxt_col = col[nb + lane]; nxt_val = val[nb + lane]; }
 #pragma unroll
-  for (int i = 0; i < HALF_NTOK; ++i) {
+  for (int i = 0; i < QUARTER_NTOK; ++i) {
     const int32_t b = nb, e = ne;
     const int32_t cur_col = nxt_col; const T cur_val = nxt_val;
-    if (i + 1 < HALF_NTOK) {
+    if (i + 1 < QUARTER_NTOK) {
       nb = __builtin_amdgcn_readlane(mb, i + 1); ne = __builtin_amdgcn_readlane(me, i + 1);
       nxt_col = 0; nxt_val = T(0);
       if (lane < ne - nb) { nxt_col = col[nb + lane]; nxt_val = val[nb + lane]; }
     }
     if (tok0 + i >= Tn) break;
     if (b == e && !first) continue;
-    // this lane's columns of the partial row (lanes 0-31 write it): pieces of V, then the tail
-    float *prow = partial + (((int64_t)slice * L + t) * Tn + tok0 + i) * d + (int64_t)half * (d / 2);
+    // this lane's columns of the partial row (the first lane group writes it): pieces of V, then the tail
+    float *prow = partial + (((int64_t)slice * L + t) * Tn + tok0 + i) * d + (int64_t)cpart * (d / NCP);
     float old[NACC], acc[NACC];
 #pragma unroll
     for (int j = 0; j < NACC; ++j) { old[j] = 0.0f; acc[j] = 0.0f; }
@@ -488,13 +488,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(half_min_wa
         if (fscale) my_val = Elem<T>::round(my_val * Elem<T>::to_f32(fscale[t * F + my_col]));
       }
       // two batches of UU row pairs in flight
-      HalfBatch<T, HQ, HTAIL, UU> ra, rb;
-      ra.load(wbase, d, my_col, my_val, 0, n, ll, hi);
-      for (int i0 = 0; i0 < n; i0 += 4 * UU) {
-        if (i0 + 2 * UU < n) rb.load(wbase, d, my_col, my_val, i0 + 2 * UU, n, ll, hi);
+      PartBatch<T, HQ, HTAIL, UU> ra, rb;
+      constexpr int R = QROWS;
+      ra.load(wbase, d, my_col, my_val, 0, n, ll, grp);
+      for (int i0 = 0; i0 < n; i0 += 2 * R * UU) {
+        if (i0 + R * UU < n) rb.load(wbase, d, my_col, my_val, i0 + R * UU, n, ll, grp);
         ra.consume(acc);
-        if (i0 + 2 * UU < n) {
-          if (i0 + 4 * UU < n) ra.load(wbase, d, my_col, my_val, i0 + 4 * UU, n, ll, hi);
+        if (i0 + R * UU < n) {
+          if (i0 + 2 * R * UU < n) ra.load(wbase, d, my_col, my_val, i0 + 2 * R * UU, n, ll, grp);
           rb.consume(acc);
         }
       }
@@ -506,42 +507,45 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(half_min_wa
       for (int c = 0; c < HQ; ++c) {
 #pragma unroll
         for (int j = 0; j < V; j += 4) {
-          const float4 q = ldg_stream4(prow + c * 32 * V + ll * V + j);
+          const float4 q = ldg_stream4(prow + c * QLANES * V + ll * V + j);
           old[c * V + j] = q.x; old[c * V + j + 1] = q.y; old[c * V + j + 2] = q.z; old[c * V + j + 3] = q.w;
         }
       }
       if (HTAIL) {
         if constexpr (V / 2 == 4) {
-          const float4 q = ldg_stream4(prow + HQ * 32 * V + ll * 4);
+          const float4 q = ldg_stream4(prow + HQ * QLANES * V + ll * 4);
           old[HQ * V] = q.x; old[HQ * V + 1] = q.y; old[HQ * V + 2] = q.z; old[HQ * V + 3] = q.w;
         } else {
 #pragma unroll
-          for (int j = 0; j < V / 2; ++j) old[HQ * V + j] = prow[HQ * 32 * V + ll * (V / 2) + j];
+          for (int j = 0; j < V / 2; ++j) old[HQ * V + j] = prow[HQ * QLANES * V + ll * (V / 2) + j];
         }
       }
     }
-    // the two halves of the wavefront hold sums over different survivors: add them, in a fixed order
+    // the lane groups hold sums over different survivors: add them, in a fixed order (group 0 ends up
+    // with ((g0 + g1) + (g2 + g3)))
 #pragma unroll
     for (int j = 0; j < NACC; ++j) {
-      const float other = __shfl_xor(acc[j], 32);
-      acc[j] = hi ? other + acc[j] : acc[j] + other;
+      const float o16 = __shfl_xor(acc[j], 16);
+      acc[j] = (lane & 16) ? o16 + acc[j] : acc[j] + o16;
+      const float o32 = __shfl_xor(acc[j], 32);
+      acc[j] = (lane & 32) ? o32 + acc[j] : acc[j] + o32;
     }
     if (!hi) {
 #pragma unroll
       for (int c = 0; c < HQ; ++c) {
 #pragma unroll
         for (int j = 0; j < V; j += 4)
-          stg_stream4(prow + c * 32 * V + ll * V + j,
+          stg_stream4(prow + c * QLANES * V + ll * V + j,
                       make_float4(old[c * V + j] + acc[c * V + j], old[c * V + j + 1] + acc[c * V + j + 1],
                                   old[c * V + j + 2] + acc[c * V + j + 2], old[c * V + j + 3] + acc[c * V + j + 3]));
       }
       if (HTAIL) {
         if constexpr (V / 2 == 4) {
-          stg_stream4(prow + HQ * 32 * V + ll * 4, make_float4(old[HQ * V] + acc[HQ * V], old[HQ * V + 1] + acc[HQ * V + 1],
+          stg_stream4(prow + HQ * QLANES * V + ll * 4, make_float4(old[HQ * V] + acc[HQ * V], old[HQ * V + 1] + acc[HQ * V + 1],
                                                                old[HQ * V + 2] + acc[HQ * V + 2], old[HQ * V + 3] + acc[HQ * V + 3]));
         } else {
 #pragma unroll
-          for (int j = 0; j < V / 2; ++j) prow[HQ * 32 * V + ll * (V / 2) + j] = old[HQ * V + j] + acc[HQ * V + j];
+          for (int j = 0; j < V / 2; ++j) prow[HQ * QLANES * V + ll * (V / 2) + j] = old[HQ * V + j] + acc[HQ * V + j];
         }
       }
     }
@@ -753,42 +757,42 @@ static int launch_decode(const int32_t *row_ptr, const int32_t *col, const void 
     else if (rem * 2 == chunk) CLT_DEC(NFN, 1, UN);        \
     else CLT_DEC(NFN, 2, UN);                              \
   } while (0)
-  // half-row schedule: 4 feature slices x 2 column halves (see k_decode_half)
-  bool halved = false;
-  if (fast && can_slice && tying != CLT_TYING_PER_TARGET && d % 256 == 0 && F >= 64 * HALF_SLICES) {
+  // quarter-row schedule: 2 feature slices x 4 column quarters (see k_decode_quarter)
+  bool quartered = false;
+  if (fast && can_slice && tying != CLT_TYING_PER_TARGET && d % 256 == 0 && F >= 64 * QUARTER_SLICES) {
     const int per_lane = (int)(d / 64);                    // columns per lane
     const int hq = per_lane / V, htail = (per_lane % V) != 0;
-    const int64_t hblk_per_t = clt_ceil_div(Tn, nwv * HALF_NTOK);
-#define CLT_DECH(HQN, HTN, UN)                                                                                       \
+    const int64_t qblk_per_t = clt_ceil_div(Tn, nwv * QUARTER_NTOK);
+#define CLT_DECQ(HQN, HTN, UN)                                                                                       \
   do {                                                                                                               \
-    k_slice_ptr<<<1024, 256, 0, stream>>>(row_ptr, col, L * Tn, F, HALF_SLICES, sptr);                               \
+    k_slice_ptr<<<1024, 256, 0, stream>>>(row_ptr, col, L * Tn, F, QUARTER_SLICES, sptr);                            \
     for (int src = 0; src < (int)t_end; ++src) {                                                                     \
       if (!((src_mask >> src) & 1ull)) continue;                                                                     \
       const int64_t tb = src > t_begin ? src : t_begin;                                                              \
-      const int64_t hb = hblk_per_t * (t_end - tb) * 8;                                                              \
-      if (hb <= 0) continue;                                                                                         \
-      if (hb > 2147483647LL) return CLT_ERR_RANGE;                                                                   \
-      if (affine) k_decode_half<T, HQN, HTN, UN, true><<<(unsigned)hb, 256, 0, stream>>>(col, (const T *)val, (const T *)wp, \
+      const int64_t qb = qblk_per_t * (t_end - tb) * 8;                                                              \
+      if (qb <= 0) continue;                                                                                         \
+      if (qb > 2147483647LL) return CLT_ERR_RANGE;                                                                   \
+      if (affine) k_decode_quarter<T, HQN, HTN, UN, true><<<(unsigned)qb, 256, 0, stream>>>(col, (const T *)val, (const T *)wp, \
           (const T *)foff, (const T *)fscale, Tn, d, F, L, tying, tb, src_mask, sptr, partial, src);                 \
-      else k_decode_half<T, HQN, HTN, UN, false><<<(unsigned)hb, 256, 0, stream>>>(col, (const T *)val, (const T *)wp, \
+      else k_decode_quarter<T, HQN, HTN, UN, false><<<(unsigned)qb, 256, 0, stream>>>(col, (const T *)val, (const T *)wp, \
           nullptr, nullptr, Tn, d, F, L, tying, tb, src_mask, sptr, partial, src);                                   \
     }                                                                                                                \
-    halved = true;                                                                                                   \
+    quartered = true;                                                                                                \
   } while (0)
     if constexpr (sizeof(T) == 2) {
-      if (hq == 1 && !htail) CLT_DECH(1, 0, 2);
-      else if (hq == 1 && htail) CLT_DECH(1, 1, 2);
-      else if (hq == 2 && !htail) CLT_DECH(2, 0, 2);
-      else if (hq == 4 && !htail) CLT_DECH(4, 0, 2);
+      if (hq == 1 && !htail) CLT_DECQ(1, 0, 2);
+      else if (hq == 1 && htail) CLT_DECQ(1, 1, 2);
+      else if (hq == 2 && !htail) CLT_DECQ(2, 0, 2);
+      else if (hq == 4 && !htail) CLT_DECQ(4, 0, 2);
     } else {
-      if (hq == 2 && !htail) CLT_DECH(2, 0, 2);
-      else if (hq == 3 && !htail) CLT_DECH(3, 0, 2);
-      else if (hq == 4 && !htail) CLT_DECH(4, 0, 2);
+      if (hq == 2 && !htail) CLT_DECQ(2, 0, 2);
+      else if (hq == 3 && !htail) CLT_DECQ(3, 0, 2);
+      else if (hq == 4 && !htail) CLT_DECQ(4, 0, 2);
     }
-#undef CLT_DECH
+#undef CLT_DECQ
   }
-  if (halved) {
-    k_decode_reduce<T><<<2048, 256, 0, stream>>>(partial, bias_sum, skip_add, out, Tn, d, L, t_begin, t_end, HALF_SLICES, out_f32, src_mask);
+  if (quartered) {
+    k_decode_reduce<T><<<2048, 256, 0, stream>>>(partial, bias_sum, skip_add, out, Tn, d, L, t_begin, t_end, QUARTER_SLICES, out_f32, src_mask);
     return clt_check_launch();
   }
   if (can_slice) k_slice_ptr<<<1024, 256, 0, stream>>>(row_ptr, col, L * Tn, F, ns, sptr);

@@ -275,7 +275,7 @@ int clt_pack_decoder(const void *w_ref, void *w_packed, int64_t d, int64_t F,
  * Limits: L <= 64; d % 8 == 0 (bf16) / d % 4 == 0 (fp32) on the fast path.
  * workspace: NULL runs one wavefront per (target, token) over all features and sources.
  * With a workspace of clt_decode_workspace_bytes() each of the 8 XCDs works on one eighth of a
- * decoder matrix at a time - 4 feature slices x 2 column halves when d is a multiple of 256 and
+ * decoder matrix at a time - 2 feature slices x 4 column quarters when d is a multiple of 256 and
  * the decoders are not tied per target, 8 feature slices of whole rows otherwise - with one
  * launch per source layer, so that the eighth stays in one L2 while all tokens pass; partial
  * sums live as fp32 rows per (slice, target, token) in the workspace and are added in a fixed

@@ -523,8 +523,8 @@ def test_decode_sparse_parity(dev, dtype, tying, L, T, d, F):
                                      ("per_target", 768)])
 def test_decode_sliced_matches_single_pass(dev, dtype, tying, d):
     # the XCD-sliced schedules (workspace given) against the one-wavefront-per-row kernel and the oracle:
-    # d a multiple of 256 takes the half-row kernel (4 feature slices x 2 column halves) unless the decoders
-    # are tied per target; other widths and per-target tying take the 8-slice kernel
+    # d a multiple of 256 takes the quarter-row kernel (2 feature slices x 4 column quarters) unless the
+    # decoders are tied per target; other widths and per-target tying take the 8-slice kernel
     g = torch.Generator().manual_seed(21)
     L, T, F = 3, 161, 1024
     names, w, b = make_decoder(L, d, F, tying, dtype, g)
