@@ -168,6 +168,39 @@ __device__ __forceinline__ float wave_sum8(const float (&p)[BWV_NU], int lane) {
   return q1;
 }
 
+// The same for four values: lane l ends up with the total of value ((l >> 5) & 1) * 2 + ((l >> 4) & 1).
+__device__ __forceinline__ float wave_sum4(const float (&p)[4], int lane) {
+  float q2[2], q1;
+  const bool hi32 = lane & 32, hi16 = lane & 16;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const float keep = hi32 ? p[2 + i] : p[i], give = hi32 ? p[i] : p[2 + i];
+    q2[i] = keep + __shfl_xor(give, 32);
+  }
+  {
+    const float keep = hi16 ? q2[1] : q2[0], give = hi16 ? q2[0] : q2[1];
+    q1 = keep + __shfl_xor(give, 16);
+  }
+  q1 += __shfl_xor(q1, 8);
+  q1 += __shfl_xor(q1, 4);
+  q1 += __shfl_xor(q1, 2);
+  q1 += __shfl_xor(q1, 1);
+  return q1;
+}
+
+// ... and for two: lane l ends up with the total of value (l >> 5) & 1.
+__device__ __forceinline__ float wave_sum2(const float (&p)[2], int lane) {
+  const bool hi32 = lane & 32;
+  const float keep = hi32 ? p[1] : p[0], give = hi32 ? p[0] : p[1];
+  float q1 = keep + __shfl_xor(give, 32);
+  q1 += __shfl_xor(q1, 16);
+  q1 += __shfl_xor(q1, 8);
+  q1 += __shfl_xor(q1, 4);
+  q1 += __shfl_xor(q1, 2);
+  q1 += __shfl_xor(q1, 1);
+  return q1;
+}
+
 // One wavefront per (source s, target t >= s, feature slice, BWV_NTOK tokens): like the forward
 // gather, block b works on slice b % 8 and blocks are ordered (s, t)-pair-major, so an XCD gathers
 // from one slice of one decoder matrix at a time.  part[t][j] = g[t][token] . W[s->t][feature of j].
@@ -213,11 +246,14 @@ __global__ __launch_bounds__(BW_THREADS) void k_bwd_values_sliced(
     for (int32_t j0 = b; j0 < e; j0 += 64) {
       const int n = (e - j0) < 64 ? (e - j0) : 64;
       const int32_t my_col = lane < n ? col[j0 + lane] : 0;
-      constexpr int LB = NCH <= 2 ? BWV_NU : NCH <= 4 ? BWV_NU / 2 : BWV_NU / 4;   // rows fetched together
-      for (int i0 = 0; i0 < n; i0 += BWV_NU) {
-        float p[BWV_NU];
+      // dot products reduced together.  Narrow rows (d <= 1024 in bf16) run best with four: 79 registers, six
+      // wavefronts per SIMD (eight: 105 registers, four wavefronts, 10 % slower; two: 6 % slower than four)
+      constexpr int NUV = NCH <= 2 ? 4 : BWV_NU;
+      constexpr int LB = NCH <= 2 ? NUV : NCH <= 4 ? BWV_NU / 2 : BWV_NU / 4;     // rows fetched together
+      for (int i0 = 0; i0 < n; i0 += NUV) {
+        float p[NUV];
 #pragma unroll
-        for (int h = 0; h < BWV_NU; h += LB) {
+        for (int h = 0; h < NUV; h += LB) {
           uint4 w[LB][NCH];
 #pragma unroll
           for (int u = 0; u < LB; ++u) {
@@ -240,9 +276,19 @@ __global__ __launch_bounds__(BW_THREADS) void k_bwd_values_sliced(
             p[h + u] = a;
           }
         }
-        const float tot = wave_sum8(p, lane);
-        const int u = ((lane >> 5) & 1) * 4 + ((lane >> 4) & 1) * 2 + ((lane >> 3) & 1);
-        if ((lane & 7) == 0 && i0 + u < n) pt[j0 + i0 + u] = tot;
+        if constexpr (NUV == 8) {
+          const float tot = wave_sum8(p, lane);
+          const int u = ((lane >> 5) & 1) * 4 + ((lane >> 4) & 1) * 2 + ((lane >> 3) & 1);
+          if ((lane & 7) == 0 && i0 + u < n) pt[j0 + i0 + u] = tot;
+        } else if constexpr (NUV == 4) {
+          const float tot = wave_sum4(p, lane);
+          const int u = ((lane >> 5) & 1) * 2 + ((lane >> 4) & 1);
+          if ((lane & 15) == 0 && i0 + u < n) pt[j0 + i0 + u] = tot;
+        } else {
+          const float tot = wave_sum2(p, lane);
+          const int u = (lane >> 5) & 1;
+          if ((lane & 31) == 0 && i0 + u < n) pt[j0 + i0 + u] = tot;
+        }
       }
     }
   }
@@ -429,7 +475,9 @@ __global__ __launch_bounds__(BW_THREADS) void k_feature_outer(
       const int n = (e - i0) < 64 ? (e - i0) : 64;
       int32_t mt = 0; float mc = 0.0f;
       if (lane < n) { mt = ltok[i0 + lane]; mc = Elem<CoefT>::to_f32(coef[lsrc[i0 + lane]]); }
-      constexpr int NU = NCH <= 2 ? FO_NU : NCH <= 4 ? FO_NU / 2 : FO_NU / 4;   // rows in flight: about 16 pieces per lane
+      // rows in flight.  Narrow rows (d <= 1024 in bf16) run best with four: 55 registers, eight wavefronts per
+      // SIMD (eight in flight, six wavefronts: 11 % slower); wide rows keep about 16 pieces per lane
+      constexpr int NU = NCH <= 4 ? FO_NU / 2 : FO_NU / 4;
       for (int i = 0; i < n; i += NU) {
         uint4 v[NU][NCH];
 #pragma unroll
