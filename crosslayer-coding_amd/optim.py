@@ -10,6 +10,7 @@ repacking follows a step.  Semantics: torch.optim.Adam without weight decay or a
 
 from __future__ import annotations
 
+import ctypes
 from typing import Dict, Tuple
 
 import torch
@@ -27,6 +28,7 @@ class CLTAdam:
         dev = model.device
         n_dec = L * (L + 1) // 2 if cfg.decoder_tying == "none" else L
         z = lambda *shape: torch.zeros(shape, dtype=torch.float32, device=dev)   # noqa: E731
+        self._tables: Dict[str, tuple] = {}
         self.state: Dict[str, Tuple[torch.Tensor, torch.Tensor]] = {
             "enc_w": (z(L, F, d), z(L, F, d)), "enc_b": (z(L, F), z(L, F)),
             "dec_w": (z(n_dec, F, d), z(n_dec, F, d)), "dec_b": (z(n_dec, d), z(n_dec, d)),
@@ -40,6 +42,17 @@ class CLTAdam:
                                         self.betas[0], self.betas[1], self.eps, self.step_count,
                                         nat.dtype_code(param.dtype), nat.current_stream(param.device))
         nat.check(code, "clt_adam_step")
+
+    def _pointer_table(self, key: str, tensors):
+        """(device int64 tensor, host ctypes array) holding the data pointers of ``tensors``."""
+        ptrs = tuple(t.data_ptr() for t in tensors)
+        ent = self._tables.get(key)
+        if ent is None or ent[0] != ptrs:
+            host = (ctypes.c_void_p * len(ptrs))(*ptrs)
+            dev = torch.tensor(ptrs, dtype=torch.int64, device=tensors[0].device)
+            ent = (ptrs, dev, host)
+            self._tables[key] = ent
+        return ent[1], ent[2]
 
     @torch.no_grad()
     def step(self, raw) -> None:
@@ -55,16 +68,27 @@ class CLTAdam:
         lib = nat.load()
         m_w, v_w = self.state["dec_w"]
         m_b, v_b = self.state["dec_b"]
-        for slot, lin in enumerate(decs):
-            w = lin.weight.data
-            assert w.is_contiguous()
-            d, F = w.shape
-            code = lib.clt_adam_step_decoder(nat.ptr(w), nat.ptr(packed[slot]), nat.ptr(raw["dec_w"][slot]),
-                                             nat.ptr(m_w[slot]), nat.ptr(v_w[slot]), d, F, self.lr, self.betas[0],
-                                             self.betas[1], self.eps, self.step_count, nat.dtype_code(w.dtype),
-                                             nat.current_stream(w.device))
-            nat.check(code, "clt_adam_step_decoder")
-            self._adam(lin.bias_param.data, raw["dec_b"][slot], m_b[slot], v_b[slot])
+        # all decoder matrices in one launch, all decoder biases in another: the parameters are separate
+        # tensors, so the kernels get their addresses as a device array (rebuilt only when one has moved)
+        ws = [lin.weight.data for lin in decs]
+        bs = [lin.bias_param.data for lin in decs]
+        assert all(w.is_contiguous() and w.shape == ws[0].shape and w.dtype == ws[0].dtype for w in ws)
+        assert all(b.is_contiguous() and b.numel() == bs[0].numel() and b.dtype == bs[0].dtype for b in bs)
+        d, F = ws[0].shape
+        assert packed.is_contiguous() and raw["dec_w"].is_contiguous() and raw["dec_w"].dtype == torch.float32
+        assert tuple(packed.shape) == (len(ws), F, d) == tuple(raw["dec_w"].shape)
+        w_dev, w_host = self._pointer_table("w", ws)
+        code = lib.clt_adam_step_decoders(nat.ptr(w_dev), ctypes.addressof(w_host), len(ws), nat.ptr(packed),
+                                          nat.ptr(raw["dec_w"]), nat.ptr(m_w), nat.ptr(v_w), d, F, self.lr,
+                                          self.betas[0], self.betas[1], self.eps, self.step_count,
+                                          nat.dtype_code(ws[0].dtype), nat.current_stream(ws[0].device))
+        nat.check(code, "clt_adam_step_decoders")
+        b_dev, _ = self._pointer_table("b", bs)
+        assert raw["dec_b"].is_contiguous() and raw["dec_b"].dtype == torch.float32
+        code = lib.clt_adam_step_many(nat.ptr(b_dev), nat.ptr(raw["dec_b"]), nat.ptr(m_b), nat.ptr(v_b), len(bs),
+                                      bs[0].numel(), self.lr, self.betas[0], self.betas[1], self.eps, self.step_count,
+                                      nat.dtype_code(bs[0].dtype), nat.current_stream(bs[0].device))
+        nat.check(code, "clt_adam_step_many")
         if raw.get("theta") is not None and "theta" in self.state:
             self._adam(model.theta_manager.log_threshold.data, raw["theta"].contiguous(), *self.state["theta"])
         # the kernels wrote through .data: caches keyed on version counters would not notice

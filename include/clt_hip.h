@@ -367,6 +367,12 @@ int clt_encoder_weight_grad(const int32_t *list_ptr, const int32_t *list_tok, co
  * clt_adam_step_decoder: one decoder matrix; w_ref is the parameter in the checkpoint layout
  *   [d][F], w_packed its feature-major working copy [F][d]; grad_packed, m, v are [F][d].  Both
  *   copies receive the same new values.
+ * clt_adam_step_decoders: n_dec decoder matrices in one launch.  w_packed, grad_packed, m, v are
+ *   [n_dec][F][d] slabs; the parameters are separate tensors (one per nn.Linear of the reference's
+ *   Decoder.decoders, clt/models/decoder.py:57-99), given as a device array of pointers for the kernel and
+ *   the same pointers in a host array for checking.
+ * clt_adam_step_many: `count` small parameters of n elements each (the decoder biases), gradient and
+ *   moments as [count][n] slabs, parameters as a device array of pointers.
  */
 int clt_adam_step(void *param, const float *grad, float *m, float *v, int64_t n,
                   double lr, double beta1, double beta2, double eps, int64_t step,
@@ -374,6 +380,13 @@ int clt_adam_step(void *param, const float *grad, float *m, float *v, int64_t n,
 int clt_adam_step_decoder(void *w_ref, void *w_packed, const float *grad_packed, float *m, float *v,
                           int64_t d, int64_t F, double lr, double beta1, double beta2, double eps,
                           int64_t step, int dtype, void *stream);
+int clt_adam_step_decoders(void *const *w_refs_dev, void *const *w_refs_host, int64_t n_dec,
+                           void *w_packed, const float *grad_packed, float *m, float *v,
+                           int64_t d, int64_t F, double lr, double beta1, double beta2, double eps,
+                           int64_t step, int dtype, void *stream);
+int clt_adam_step_many(void *const *params_dev, const float *grad, float *m, float *v, int64_t count,
+                       int64_t n, double lr, double beta1, double beta2, double eps, int64_t step,
+                       int dtype, void *stream);
 
 /* clt_jumprelu_theta_grad: gradient of the JumpReLU thresholds of one layer (JumpReLU.backward,
  *   clt/models/activations.py:196-199; bandwidth is 1.0 in ThetaManager, clt/models/theta.py:41):

@@ -216,3 +216,50 @@ def test_adam_kernels_match_torch_adam_on_given_gradients(dev, dtype, shape):
     want = ref.detach().to(dtype).float()
     tol = dict(rtol=1e-5, atol=1e-6) if dtype == torch.float32 else dict(rtol=1e-2, atol=1e-3)
     assert torch.allclose(w_ref.float().cpu(), want, **tol)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_adam_batched_entry_points_equal_the_single_ones(dev, dtype):
+    # three decoder matrices and their biases in one launch each against one call per tensor: same bits
+    import ctypes
+    from crosslayer_coding_amd import _native
+    lib = _native.load()
+    gen = torch.Generator().manual_seed(11)
+    n, d, F = 3, 96, 200
+    stream = torch.cuda.current_stream().cuda_stream
+    code = _native.dtype_code(dtype)
+    w0 = [(torch.randn(d, F, generator=gen) * 0.1).to(dtype) for _ in range(n)]
+    b0 = [(torch.randn(d, generator=gen) * 0.1).to(dtype) for _ in range(n)]
+    g = (torch.randn(n, F, d, generator=gen) * 1e-2).to(dev)
+    gb = (torch.randn(n, d, generator=gen) * 1e-2).to(dev)
+    out = []
+    for batched in (False, True):
+        ws = [w.to(dev).contiguous() for w in w0]
+        bs = [b.to(dev).contiguous() for b in b0]
+        packed = torch.stack([w.t().contiguous() for w in ws]).contiguous()
+        m = torch.zeros(n, F, d, device=dev); v = torch.zeros(n, F, d, device=dev)
+        mb = torch.zeros(n, d, device=dev); vb = torch.zeros(n, d, device=dev)
+        for step in (1, 2):
+            if batched:
+                ptrs = [w.data_ptr() for w in ws]
+                host = (ctypes.c_void_p * n)(*ptrs)
+                devp = torch.tensor(ptrs, dtype=torch.int64, device=dev)
+                assert lib.clt_adam_step_decoders(devp.data_ptr(), ctypes.addressof(host), n, packed.data_ptr(), g.data_ptr(),
+                                                  m.data_ptr(), v.data_ptr(), d, F, 3e-3, 0.9, 0.999, 1e-8, step, code, stream) == 0
+                bp = torch.tensor([b.data_ptr() for b in bs], dtype=torch.int64, device=dev)
+                assert lib.clt_adam_step_many(bp.data_ptr(), gb.data_ptr(), mb.data_ptr(), vb.data_ptr(), n, d,
+                                              3e-3, 0.9, 0.999, 1e-8, step, code, stream) == 0
+            else:
+                for i in range(n):
+                    assert lib.clt_adam_step_decoder(ws[i].data_ptr(), packed[i].data_ptr(), g[i].data_ptr(), m[i].data_ptr(),
+                                                     v[i].data_ptr(), d, F, 3e-3, 0.9, 0.999, 1e-8, step, code, stream) == 0
+                    assert lib.clt_adam_step(bs[i].data_ptr(), gb[i].data_ptr(), mb[i].data_ptr(), vb[i].data_ptr(), d,
+                                             3e-3, 0.9, 0.999, 1e-8, step, code, stream) == 0
+        torch.cuda.synchronize()
+        out.append((torch.stack(ws).cpu(), packed.cpu(), torch.stack(bs).cpu(), m.cpu(), vb.cpu()))
+    for a, b in zip(*out):
+        assert torch.equal(a, b)
+    assert torch.equal(out[1][0], out[1][1].transpose(1, 2))
+    # bad arguments are refused before anything is launched
+    assert lib.clt_adam_step_decoders(None, None, 1, None, None, None, None, d, F, 3e-3, 0.9, 0.999, 1e-8, 1, code, stream) != 0
+    assert lib.clt_adam_step_many(None, None, None, None, 2, d, 3e-3, 0.9, 0.999, 1e-8, 1, code, stream) != 0
