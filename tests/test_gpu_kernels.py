@@ -519,8 +519,8 @@ def test_decode_sparse_parity(dev, dtype, tying, L, T, d, F):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("tying,d", [("none", 768), ("per_source", 768), ("none", 1024), ("none", 640), ("per_source", 320),
-                                     ("per_target", 768)])
+@pytest.mark.parametrize("tying,d", [("none", 768), ("per_source", 768), ("none", 1024), ("none", 512), ("per_source", 2048),
+                                     ("none", 640), ("per_source", 320), ("per_target", 768)])
 def test_decode_sliced_matches_single_pass(dev, dtype, tying, d):
     # the XCD-sliced schedules (workspace given) against the one-wavefront-per-row kernel and the oracle:
     # d a multiple of 256 takes the quarter-row kernel (2 feature slices x 4 column quarters) unless the
