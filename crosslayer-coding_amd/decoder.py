@@ -148,16 +148,20 @@ class Decoder(nn.Module):
         if hit is not None and hit[0] == key:
             return hit[1]
         L, d = self.config.num_layers, self.config.d_model
-        B = torch.stack([dec.bias_param.detach().float() for dec in decs])
+        B = torch.stack([dec.bias_param.detach() for dec in decs]).float()
         tying = self.config.decoder_tying
         if tying == "per_target":
             out = B.contiguous()
         else:
             out = torch.zeros(L, d, dtype=torch.float32, device=B.device)
             if tying == "none":
-                for i, (s, t) in enumerate(self._slots()):
+                # the decoders of source s are the slots of the targets s .. L-1, in a row: one addition per
+                # source, so every target still adds its sources in ascending order
+                first = 0
+                for s in range(L):
                     if (src_mask >> s) & 1:
-                        out[t] += B[i]
+                        out[s:] += B[first:first + L - s]
+                    first += L - s
             else:
                 run = torch.zeros(d, dtype=torch.float32, device=B.device)
                 for t in range(L):
