@@ -207,7 +207,10 @@ __device__ __forceinline__ float wave_sum2(const float (&p)[2], int lane) {
 // A row is read in 16-byte pieces (lane l: elements c * 64 EV + l EV ..., NCH pieces); the raw pieces
 // of up to BWV_NU rows are in flight together, and BWV_NU dot products are reduced across the
 // wavefront at once.
-template <typename T, int NCH>
+// T8: d = (NCH - 1) * 64 EV + 32 EV (768 in bf16): the last piece of a lane is 8 bytes wide and all 64 lanes
+// take one, instead of a 16-byte piece that only the first 32 lanes have - no idle lanes in the loads and
+// in the multiply-adds of the last piece.
+template <typename T, int NCH, bool T8>
 __global__ __launch_bounds__(BW_THREADS) void k_bwd_values_sliced(
     const int32_t *__restrict__ sptr, const int32_t *__restrict__ col, const T *__restrict__ wp,
     const float *__restrict__ g, int64_t Tn, int64_t d, int64_t F, int64_t L, int tying, int64_t nnz,
@@ -225,6 +228,8 @@ __global__ __launch_bounds__(BW_THREADS) void k_bwd_values_sliced(
   const int64_t t = s + rem;
   const T *wbase = wp + bw_decoder_slot(tying, s, t, L) * F * d;
   float *pt = part + t * nnz;
+  constexpr int NFULL = T8 ? NCH - 1 : NCH, HV = EV / 2;
+  const int64_t tail_at = (int64_t)NFULL * 64 * EV + lane * HV;
   bool on[NCH];
 #pragma unroll
   for (int c = 0; c < NCH; ++c) on[c] = (int64_t)c * 64 * EV + lane * EV < d;
@@ -235,8 +240,12 @@ __global__ __launch_bounds__(BW_THREADS) void k_bwd_values_sliced(
     const int32_t b = sptr[r * (BWV_XCDS + 1) + slice], e = sptr[r * (BWV_XCDS + 1) + slice + 1];
     if (b == e) continue;
     float gv[NCH][EV];
+    if constexpr (T8) {
+      const float4 v = *reinterpret_cast<const float4 *>(g + (t * Tn + tok) * d + tail_at);
+      gv[NFULL][0] = v.x; gv[NFULL][1] = v.y; gv[NFULL][2] = v.z; gv[NFULL][3] = v.w;
+    }
 #pragma unroll
-    for (int c = 0; c < NCH; ++c)
+    for (int c = 0; c < NFULL; ++c)
 #pragma unroll
       for (int q = 0; q < EV; q += 4) {
         const float4 v = on[c] ? *reinterpret_cast<const float4 *>(g + (t * Tn + tok) * d + (int64_t)c * 64 * EV + lane * EV + q)
@@ -255,23 +264,31 @@ __global__ __launch_bounds__(BW_THREADS) void k_bwd_values_sliced(
 #pragma unroll
         for (int h = 0; h < NUV; h += LB) {
           uint4 w[LB][NCH];
+          uint2 wt[LB];
 #pragma unroll
           for (int u = 0; u < LB; ++u) {
             const int idx = i0 + h + u < n ? i0 + h + u : n - 1;
             const T *wrow = wbase + (int64_t)__builtin_amdgcn_readlane(my_col, idx) * d;
 #pragma unroll
-            for (int c = 0; c < NCH; ++c)
+            for (int c = 0; c < NFULL; ++c)
               w[u][c] = on[c] ? *reinterpret_cast<const uint4 *>(wrow + (int64_t)c * 64 * EV + lane * EV) : make_uint4(0, 0, 0, 0);
+            if constexpr (T8) wt[u] = *reinterpret_cast<const uint2 *>(wrow + tail_at);
           }
 #pragma unroll
           for (int u = 0; u < LB; ++u) {
             float a = 0.0f;
 #pragma unroll
-            for (int c = 0; c < NCH; ++c) {
+            for (int c = 0; c < NFULL; ++c) {
               float x[EV];
               Piece<T>::unpack(w[u][c], x);
 #pragma unroll
               for (int q = 0; q < EV; ++q) a = fmaf(x[q], gv[c][q], a);
+            }
+            if constexpr (T8 && sizeof(T) == 2) {
+              a = fmaf(__uint_as_float(wt[u].x << 16), gv[NFULL][0], a);
+              a = fmaf(__uint_as_float(wt[u].x & 0xFFFF0000u), gv[NFULL][1], a);
+              a = fmaf(__uint_as_float(wt[u].y << 16), gv[NFULL][2], a);
+              a = fmaf(__uint_as_float(wt[u].y & 0xFFFF0000u), gv[NFULL][3], a);
             }
             p[h + u] = a;
           }
@@ -625,7 +642,7 @@ extern "C" int clt_decode_backward_values(const int32_t *row_ptr, const int32_t 
   const int64_t npair = L * (L + 1) / 2;
   const int64_t nblk = npair * clt_ceil_div(T, (BW_THREADS / 64) * BWV_NTOK) * BWV_XCDS;
   if (nblk > 2147483647LL) return CLT_ERR_RANGE;
-#define CLT_BWV(TT, N) k_bwd_values_sliced<TT, N><<<(unsigned)nblk, BW_THREADS, 0, s>>>(sptr, col, (const TT *)w_packed, g, T, d, F, L, tying, nnz, part)
+#define CLT_BWV(TT, N) k_bwd_values_sliced<TT, N, false><<<(unsigned)nblk, BW_THREADS, 0, s>>>(sptr, col, (const TT *)w_packed, g, T, d, F, L, tying, nnz, part)
 #define CLT_BWV_N(TT)                                                                       \
   do {                                                                                      \
     switch (nc4) {                                                                          \
@@ -634,7 +651,9 @@ extern "C" int clt_decode_backward_values(const int32_t *row_ptr, const int32_t 
       case 7: CLT_BWV(TT, 7); break; default: CLT_BWV(TT, 8); break;                        \
     }                                                                                       \
   } while (0)
-  if (dtype == CLT_BF16) CLT_BWV_N(bf16_t); else CLT_BWV_N(float);
+  if (dtype == CLT_BF16 && d == 768)
+    k_bwd_values_sliced<bf16_t, 2, true><<<(unsigned)nblk, BW_THREADS, 0, s>>>(sptr, col, (const bf16_t *)w_packed, g, T, d, F, L, tying, nnz, part);
+  else if (dtype == CLT_BF16) CLT_BWV_N(bf16_t); else CLT_BWV_N(float);
 #undef CLT_BWV_N
 #undef CLT_BWV
   k_bwd_values_sum<<<256 * 8, BW_THREADS, 0, s>>>(row_ptr, part, T, L, nnz, src_mask, dval);
