@@ -451,7 +451,8 @@ __global__ __launch_bounds__(BW_THREADS) void k_csc_order(const int32_t *ptr, in
 // (Cutting the columns in two over XCD pairs, so that each XCD gathers from half a [T, d] matrix that
 // fits its L2, was measured and dropped: with four rows in flight per wavefront whole rows are 8 % faster.)
 constexpr int FO_NU = 8;
-template <typename T, typename CoefT, int NCH, bool DECODER>
+// T8: as in k_bwd_values_sliced, the last piece of a lane is 8 bytes wide and every lane has one.
+template <typename T, typename CoefT, int NCH, bool DECODER, bool T8 = false>
 __global__ __launch_bounds__(BW_THREADS) void k_feature_outer(
     const int32_t *__restrict__ ptr, const int32_t *__restrict__ ltok, const int32_t *__restrict__ lsrc,
     const CoefT *__restrict__ coef, const T *__restrict__ src, float *__restrict__ out, float *__restrict__ rowsum,
@@ -469,6 +470,8 @@ __global__ __launch_bounds__(BW_THREADS) void k_feature_outer(
   const int64_t total = (DECODER && !per_target) ? (target + 1) * F : F;
   const int64_t vblock = (int64_t)blockIdx.x, nvblock = (int64_t)gridDim.x;
   const int64_t my_pieces = d / EV;
+  constexpr int NFULL = T8 ? NCH - 1 : NCH, HV = EV / 2;
+  const int64_t tail_at = (int64_t)NFULL * 64 * EV + lane * HV;
   bool on[NCH];
 #pragma unroll
   for (int c = 0; c < NCH; ++c) on[c] = (int64_t)c * 64 + lane < my_pieces;
@@ -493,13 +496,15 @@ __global__ __launch_bounds__(BW_THREADS) void k_feature_outer(
       constexpr int NU = NCH <= 4 ? FO_NU / 2 : FO_NU / 4;
       for (int i = 0; i < n; i += NU) {
         uint4 v[NU][NCH];
+        uint2 vt[NU];
 #pragma unroll
         for (int u = 0; u < NU; ++u) {
           const int idx = i + u < n ? i + u : n - 1;
           const T *row = sbase + (int64_t)__builtin_amdgcn_readlane(mt, idx) * d;
 #pragma unroll
-          for (int c = 0; c < NCH; ++c)
+          for (int c = 0; c < NFULL; ++c)
             v[u][c] = on[c] ? *reinterpret_cast<const uint4 *>(row + (int64_t)c * 64 * EV + lane * EV) : make_uint4(0, 0, 0, 0);
+          if constexpr (T8) vt[u] = *reinterpret_cast<const uint2 *>(row + tail_at);
         }
 #pragma unroll
         for (int u = 0; u < NU; ++u) {
@@ -507,11 +512,17 @@ __global__ __launch_bounds__(BW_THREADS) void k_feature_outer(
           const float cf = i + u < n ? __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(mc), idx)) : 0.0f;
           csum += cf;
 #pragma unroll
-          for (int c = 0; c < NCH; ++c) {
+          for (int c = 0; c < NFULL; ++c) {
             float x[EV];
             Piece<T>::unpack(v[u][c], x);
 #pragma unroll
             for (int k = 0; k < EV; ++k) acc[c][k] = fmaf(cf, x[k], acc[c][k]);
+          }
+          if constexpr (T8 && sizeof(T) == 2) {
+            acc[NFULL][0] = fmaf(cf, __uint_as_float(vt[u].x << 16), acc[NFULL][0]);
+            acc[NFULL][1] = fmaf(cf, __uint_as_float(vt[u].x & 0xFFFF0000u), acc[NFULL][1]);
+            acc[NFULL][2] = fmaf(cf, __uint_as_float(vt[u].y << 16), acc[NFULL][2]);
+            acc[NFULL][3] = fmaf(cf, __uint_as_float(vt[u].y & 0xFFFF0000u), acc[NFULL][3]);
           }
         }
       }
@@ -520,8 +531,14 @@ __global__ __launch_bounds__(BW_THREADS) void k_feature_outer(
     const int64_t q = s * F + f;
     float *orow = out + (DECODER ? (bw_decoder_slot(tying, s, t, L) * F + f) : q) * d;
     const bool add = DECODER && tying == CLT_TYING_PER_SOURCE && t > s;
+    if constexpr (T8) {
+      float4 *dst = reinterpret_cast<float4 *>(orow + tail_at);
+      float4 r = make_float4(acc[NFULL][0], acc[NFULL][1], acc[NFULL][2], acc[NFULL][3]);
+      if (add) { const float4 o = *dst; r.x += o.x; r.y += o.y; r.z += o.z; r.w += o.w; }
+      *dst = r;
+    }
 #pragma unroll
-    for (int c = 0; c < NCH; ++c)
+    for (int c = 0; c < NFULL; ++c)
       if (on[c]) {
 #pragma unroll
         for (int k = 0; k < EV; k += 4) {
@@ -715,7 +732,11 @@ extern "C" int clt_decoder_weight_grad(const int32_t *list_ptr, const int32_t *l
       case 7: CLT_DW(CT, 7); break; default: CLT_DW(CT, 8); break;                         \
     }                                                                                      \
   } while (0)
-  if (dtype == CLT_BF16) CLT_DW_N(bf16_t); else CLT_DW_N(float);
+  if (dtype == CLT_BF16 && d == 768) {
+    for (int64_t t = 0; t < L; ++t)
+      k_feature_outer<bf16_t, bf16_t, 2, true, true><<<bw_resident_blocks(k_feature_outer<bf16_t, bf16_t, 2, true, true>), BW_THREADS, 0, s>>>(
+          list_ptr, list_tok, list_src, (const bf16_t *)val, (const bf16_t *)g_model, dw_packed, nullptr, T, d, F, L, t, tying);
+  } else if (dtype == CLT_BF16) CLT_DW_N(bf16_t); else CLT_DW_N(float);
 #undef CLT_DW_N
 #undef CLT_DW
   return clt_check_launch();
@@ -744,7 +765,11 @@ extern "C" int clt_encoder_weight_grad(const int32_t *list_ptr, const int32_t *l
       case 7: CLT_EW(ST, 7); break; default: CLT_EW(ST, 8); break;                         \
     }                                                                                      \
   } while (0)
-  if (dtype == CLT_BF16) CLT_EW_N(bf16_t); else CLT_EW_N(float);
+  if (dtype == CLT_BF16 && d == 768) {
+    for (int64_t l = 0; l < L; ++l)
+      k_feature_outer<bf16_t, float, 2, false, true><<<bw_resident_blocks(k_feature_outer<bf16_t, float, 2, false, true>), BW_THREADS, 0, s>>>(
+          list_ptr, list_tok, list_src, dval, (const bf16_t *)x, dw_enc, db_enc, T, d, F, L, l, CLT_TYING_NONE);
+  } else if (dtype == CLT_BF16) CLT_EW_N(bf16_t); else CLT_EW_N(float);
 #undef CLT_EW_N
 #undef CLT_EW
   return clt_check_launch();
