@@ -321,8 +321,15 @@ __global__ __launch_bounds__(BW_THREADS) void k_bwd_values_sum(const int32_t *ro
     const bool on = (src_mask >> s) & 1ull;
     for (int32_t j = row_ptr[r] + lane; j < row_ptr[r + 1]; j += 64) {
       float acc = 0.0f;
-      if (on)
-        for (int64_t t = s; t < L; ++t) acc += part[t * nnz + j];
+      if (on) {
+        // four loads in flight; the additions keep the target order
+        int64_t t = s;
+        for (; t + 4 <= L; t += 4) {
+          const float p0 = part[t * nnz + j], p1 = part[(t + 1) * nnz + j], p2 = part[(t + 2) * nnz + j], p3 = part[(t + 3) * nnz + j];
+          acc += p0; acc += p1; acc += p2; acc += p3;
+        }
+        for (; t < L; ++t) acc += part[t * nnz + j];
+      }
       dval[j] = acc;
     }
   }
