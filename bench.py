@@ -262,7 +262,8 @@ def run_probe(args):
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     lib = cca._native.load(build_if_missing=False)
-    row_bytes, n_idx = 1536, 5_400_000                      # one decode launch at C1 gathers 5.3 M rows
+    row_bytes = int(args.probe_row_bytes)
+    n_idx = 5_400_000 * 1536 // row_bytes                   # one decode launch at C1 gathers 5.3 M rows of 1536 bytes
     stream = torch.cuda.current_stream().cuda_stream
     g = torch.Generator(device=dev).manual_seed(0)
     results = {}
@@ -272,7 +273,7 @@ def run_probe(args):
         table = torch.randint(0, 1 << 30, (n_rows * row_bytes // 4,), dtype=torch.int32, device=dev, generator=g)
         idx = torch.randint(0, n_rows, (n_idx,), dtype=torch.int32, device=dev, generator=g)
         best, best_lds = None, None
-        for to_lds in (0, 1):
+        for to_lds in ((0, 1) if row_bytes >= 1024 else (0,)):
             moved = row_bytes if not to_lds else 2048
             for blocks in (256 * 2, 256 * 4, 256 * 8, 256 * 16):
                 out = torch.empty(blocks * 256, dtype=torch.float32, device=dev)
@@ -293,13 +294,15 @@ def run_probe(args):
                         best_lds = (gbs, blocks)
                 elif best is None or gbs > best[0]:
                     best = (gbs, blocks)
-        results[label] = {"GB/s": best[0], "blocks": best[1], "direct_to_lds_GB/s": best_lds[0], "direct_to_lds_blocks": best_lds[1]}
+        results[label] = {"GB/s": best[0], "blocks": best[1]}
+        if best_lds is not None:
+            results[label].update({"direct_to_lds_GB/s": best_lds[0], "direct_to_lds_blocks": best_lds[1]})
         del table, idx
     top = results["2 MB"]["GB/s"]
-    return {"metric": "bare gather of 1536-byte rows, best of three grid sizes", "value": top, "unit": "GB/s", "n_gpus": 1,
+    return {"metric": f"bare gather of {row_bytes}-byte rows, best of four grid sizes", "value": top, "unit": "GB/s", "n_gpus": 1,
             "steps": args.steps, "warmup": 2, "ms_per_step": n_idx * row_bytes / top / 1e6, "higher_is_better": True,
             "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
-            "config": {"workload": "gather probe: 5.4 M random rows of 1536 bytes per launch"}, "tables": results}
+            "config": {"workload": f"gather probe: {n_idx / 1e6:.1f} M random rows of {row_bytes} bytes per launch"}, "tables": results}
 
 
 def run_feed(args):
@@ -564,6 +567,8 @@ def main():
                          "selection, per-feature minimum) instead of the forward")
     ap.add_argument("--backward", action="store_true",
                     help="time forward + MSE loss + all gradients (loss_and_gradients) instead of the forward")
+    ap.add_argument("--probe-row-bytes", type=int, default=1536,
+                    help="row size of --gather-probe (a multiple of 16 up to 2048; 1536 is a whole C1 decoder row, 384 a quarter)")
     ap.add_argument("--gather-probe", action="store_true",
                     help="calibration: the rate a bare row gather reaches from L2-, cache- and HBM-sized tables")
     ap.add_argument("--feed", action="store_true",
