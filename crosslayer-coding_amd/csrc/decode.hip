@@ -61,6 +61,12 @@ __device__ __forceinline__ int64_t decoder_slot(int tying, int64_t s, int64_t t,
   return s * L - (s * (s - 1)) / 2 + (t - s);
 }
 
+static inline int64_t decoder_slot_host(int tying, int64_t s, int64_t t, int64_t L) {
+  if (tying == CLT_TYING_PER_SOURCE) return s;
+  if (tying == CLT_TYING_PER_TARGET) return t;
+  return s * L - (s * (s - 1)) / 2 + (t - s);
+}
+
 // UU decoder vectors in flight: the row pieces of one lane plus the (wave-uniform) weights.
 template <typename T, int NF, int TAIL, int UU> struct RowBatch {
   uint4 wq[UU][NF > 0 ? NF : 1];
@@ -703,12 +709,60 @@ __global__ __launch_bounds__(256) void k_norms(const T *wp, T *norms, int64_t d,
   }
 }
 
+// acc[tok][f] = round(acc[tok][f] + v') over the survivors (f, v) of one layer: the running sum of
+// activations that decoders tied per target consume (reference clt/models/decoder.py:208-246), every
+// addition rounded to the model dtype as the reference's `summed_activation += activation_tensor` is.
+// One wavefront per token row; a row's columns are distinct, so no two lanes touch one element.
+template <typename T>
+__global__ __launch_bounds__(256) void k_accumulate_dense(const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ col,
+                                                          const T *__restrict__ val, const T *__restrict__ foff,
+                                                          const T *__restrict__ fscale, T *__restrict__ acc, int64_t Tn,
+                                                          int64_t F, int64_t layer, int init) {
+  const int lane = lane_id(), wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
+  for (int64_t tok = (int64_t)blockIdx.x * nwv + wv; tok < Tn; tok += (int64_t)gridDim.x * nwv) {
+    const int64_t r = layer * Tn + tok;
+    T *arow = acc + tok * F;
+    for (int32_t j = row_ptr[r] + lane; j < row_ptr[r + 1]; j += 64) {
+      const int32_t f = col[j];
+      float v = Elem<T>::to_f32(val[j]);
+      if (v != 0.0f) {   // the affine terms apply to the selected (non-zero) entries only
+        if (foff) v = Elem<T>::round(v + Elem<T>::to_f32(foff[f]));
+        if (fscale) v = Elem<T>::round(v * Elem<T>::to_f32(fscale[f]));
+      }
+      const float old = init ? 0.0f : Elem<T>::to_f32(arow[f]);
+      arow[f] = Elem<T>::from_f32(old + v);
+    }
+  }
+}
+
 constexpr int DEC_SLICES = 8;  // one feature slice per XCD of an MI355X
 
 static size_t decode_ws_bytes(int64_t Tn, int64_t d, int64_t L) {
   size_t part = ((size_t)DEC_SLICES * L * Tn * d * 4 + 255) & ~(size_t)255;
   size_t sp = ((size_t)L * Tn * (DEC_SLICES + 1) * 4 + 255) & ~(size_t)255;
   return part + sp;
+}
+
+static bool quarter_shape_ok(int64_t d, int elem_bytes) {
+  const int V = 16 / elem_bytes;
+  const int per_lane = (int)(d / 64), hq = per_lane / V;
+  const bool htail = (per_lane % V) != 0;
+  if (elem_bytes == 2) return (hq == 1) || (hq == 2 && !htail) || (hq == 4 && !htail);
+  return (hq == 2 || hq == 3 || hq == 4) && !htail;
+}
+
+// Which schedule launch_decode takes; `ws_ok`: a workspace of decode_ws_bytes(), 256-byte aligned;
+// `wp_ok`: the packed decoders are 16-byte aligned.
+static int plan_route(int64_t d, int64_t F, int tying, int elem_bytes, bool ws_ok, bool wp_ok) {
+  const int V = 16 / elem_bytes;
+  const int64_t chunk = 64 * V, nf = d / chunk, rem = d % chunk;
+  const bool can_slice = ws_ok && (d % 4 == 0) && F >= 64 * DEC_SLICES;
+  const bool fast = (d % V == 0) && wp_ok && nf <= 4 && (nf > 0 || rem > 0);
+  if (!fast) return CLT_ROUTE_GENERIC;
+  if (!can_slice) return CLT_ROUTE_SINGLE;
+  if (tying != CLT_TYING_PER_TARGET && d % 256 == 0 && F >= 64 * QUARTER_SLICES && quarter_shape_ok(d, elem_bytes))
+    return CLT_ROUTE_QUARTER;
+  return tying == CLT_TYING_PER_TARGET ? CLT_ROUTE_SLICED_ALL_SOURCES : CLT_ROUTE_SLICED;
 }
 
 template <typename T>
@@ -759,7 +813,8 @@ static int launch_decode(const int32_t *row_ptr, const int32_t *col, const void 
   } while (0)
   // quarter-row schedule: 2 feature slices x 4 column quarters (see k_decode_quarter)
   bool quartered = false;
-  if (fast && can_slice && tying != CLT_TYING_PER_TARGET && d % 256 == 0 && F >= 64 * QUARTER_SLICES) {
+  const int route = plan_route(d, F, tying, (int)sizeof(T), can_slice, clt_aligned16(wp));
+  if (route == CLT_ROUTE_QUARTER) {
     const int per_lane = (int)(d / 64);                    // columns per lane
     const int hq = per_lane / V, htail = (per_lane % V) != 0;
     const int64_t qblk_per_t = clt_ceil_div(Tn, nwv * QUARTER_NTOK);
@@ -896,5 +951,43 @@ extern "C" int clt_decoder_norms(const void *w_packed, void *norms, int64_t d, i
   hipStream_t s = (hipStream_t)stream;
   if (dtype == CLT_BF16) k_norms<bf16_t><<<256 * 8, 256, 0, s>>>((const bf16_t *)w_packed, (bf16_t *)norms, d, F, L, tying);
   else k_norms<float><<<256 * 8, 256, 0, s>>>((const float *)w_packed, (float *)norms, d, F, L, tying);
+  return clt_check_launch();
+}
+
+extern "C" int clt_decode_route(int64_t T, int64_t d, int64_t F, int64_t L, int tying, int dtype,
+                                size_t workspace_bytes) {
+  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (T <= 0 || d <= 0 || F <= 0 || L <= 0 || L > 64 || tying < 0 || tying > 2) return CLT_ERR_ARG;
+  return plan_route(d, F, tying, dtype == CLT_BF16 ? 2 : 4, workspace_bytes >= decode_ws_bytes(T, d, L), true);
+}
+
+extern "C" int64_t clt_decoder_slab_elems(int64_t d, int64_t F, int64_t L, int tying) {
+  if (d <= 0 || F <= 0 || L <= 0 || tying < 0 || tying > 2) return -1;
+  const int64_t n_dec = tying == CLT_TYING_NONE ? L * (L + 1) / 2 : L;
+  // the last element any schedule can touch: row F-1 of slot n_dec-1, formed like the kernels form it
+  const int64_t last = decoder_slot_host(tying, L - 1, L - 1, L) * F * d + (F - 1) * d + (d - 1);
+  return last + 1 == n_dec * F * d ? n_dec * F * d : -1;
+}
+
+extern "C" int clt_accumulate_dense(const int32_t *row_ptr, const int32_t *col, const void *val,
+                                    const void *feat_offset, const void *feat_scale, void *acc, int64_t T,
+                                    int64_t F, int64_t layer, int init, int dtype, void *stream) {
+  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (T < 0 || F <= 0 || (layer < 0 && !init)) return CLT_ERR_ARG;
+  if (T == 0) return CLT_OK;
+  if (!acc || (layer >= 0 && !row_ptr)) return CLT_ERR_ARG;
+  hipStream_t s = (hipStream_t)stream;
+  const unsigned nb = (unsigned)(clt_ceil_div(T, 4) < 8192 ? clt_ceil_div(T, 4) : 8192);
+  if (init) {
+    if (dtype == CLT_BF16) k_zero_rows<bf16_t><<<2048, 256, 0, s>>>((bf16_t *)acc, T, F, 1, T * F);
+    else k_zero_rows<float><<<2048, 256, 0, s>>>((float *)acc, T, F, 1, T * F);
+  }
+  if (layer < 0) return clt_check_launch();   // clear only
+  if (dtype == CLT_BF16)
+    k_accumulate_dense<bf16_t><<<nb, 256, 0, s>>>(row_ptr, col, (const bf16_t *)val, (const bf16_t *)feat_offset,
+                                                 (const bf16_t *)feat_scale, (bf16_t *)acc, T, F, layer, init);
+  else
+    k_accumulate_dense<float><<<nb, 256, 0, s>>>(row_ptr, col, (const float *)val, (const float *)feat_offset,
+                                                (const float *)feat_scale, (float *)acc, T, F, layer, init);
   return clt_check_launch();
 }

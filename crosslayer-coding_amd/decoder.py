@@ -97,6 +97,10 @@ class Decoder(nn.Module):
         self._norm_key = None
         self._bias_cache: Dict[int, Tuple[tuple, torch.Tensor]] = {}
         self._compact_cache: Dict[int, tuple] = {}
+        # decoders tied per target: targets whose summed activations are dense enough go through the
+        # matrix cores (see dense_split); False keeps every target on the row gather
+        self.dense_route = True
+        self.last_route: Dict[str, Tuple[int, int]] = {}
 
     # ---- decoder bookkeeping -------------------------------------------------------
     def _ordered(self) -> List[RowParallelLinear]:
@@ -186,13 +190,92 @@ class Decoder(nn.Module):
         return engine.encode(x, w_skip.detach().unsqueeze(0).contiguous(), None)[0].float()
 
     # ---- fused path ------------------------------------------------------------------
+    # Rates behind the choice between the two decode routes, measured on an MI355X: the row gather of
+    # clt_decode_sparse delivers about 14.5 TB/s of decoder rows whatever the shape; the MFMA kernel
+    # sustains about 1.0 PFLOP/s in bf16 (0.1 in fp32) on [T, F] x [F, d] products with F >= 16384.
+    GATHER_BYTES_PER_S = 14.5e12
+    MFMA_FLOPS_PER_S = {torch.bfloat16: 1.0e15, torch.float32: 1.0e14}
+
+    def dense_split(self, surv: SurvivorList, src_mask: int, t_begin: int, t_end: int,
+                    skip_add: Optional[torch.Tensor]) -> int:
+        """First target of [t_begin, t_end) that is decoded as a dense product (``t_end``: none is).
+
+        Decoders tied per target multiply the SUM of the activations of all sources <= t
+        (decoder.py:208-251), so target t gathers (t + 1) k T decoder rows of d elements from one matrix:
+        with every further source the gather grows and the dense product ``summed [T, F] @ W[t].T`` does
+        not.  The dense route is taken from the first target on for which
+        ``2 T F d / MFMA rate < rows gathered x d x element size / gather rate``.  Untied and per-source
+        decoders never qualify: each (source, target) pair has its own operand or its own matrix, so the
+        dense cost is the reference's full 2 T F d per pair against k T rows per pair."""
+        cfg = self.config
+        if cfg.decoder_tying != "per_target" or not self.dense_route or skip_add is not None:
+            return t_end
+        T, F, d = surv.T, surv.F, cfg.d_model
+        esize = 2 if surv.dtype == torch.bfloat16 else 4
+        rate = self.MFMA_FLOPS_PER_S.get(surv.dtype)
+        # shapes the MFMA kernel of clt_encode takes (K = F in whole pairs of 128-byte stages, 256 x 256 tiles)
+        if rate is None or T < 256 or d < 256 or d % 4 or F % (256 // esize):
+            return t_end
+        dense_s = 2.0 * T * F * d / rate
+        per_layer = surv.col.numel() / max(1, surv.L)            # survivors of one source layer (host-side size)
+        n_src = 0
+        for t in range(t_end):
+            n_src += (src_mask >> t) & 1
+            if t >= t_begin and n_src * per_layer * d * esize / self.GATHER_BYTES_PER_S > dense_s:
+                return t
+        return t_end
+
+    def _decode_dense(self, surv: SurvivorList, src_mask: int, t_first: int, t_end: int, out: torch.Tensor, ws) -> None:
+        """Targets [t_first, t_end) of decoders tied per target as dense products: the reference's own
+        formulation (decoder.py:208-251) - activations summed over the sources in the model dtype, one
+        ``F.linear`` with the target's decoder in its checkpoint layout - with the sum built by scattering
+        the survivor lists and the product on the MFMA kernel."""
+        T, F = surv.T, surv.F
+        acc = (ws.typed("dense_sum", (T, F), surv.dtype) if ws is not None
+               else torch.empty((T, F), dtype=surv.dtype, device=out.device))
+        off, sc = self._affine()
+        affine = off is not None or sc is not None
+        started = False
+        for t in range(t_end):
+            if affine:
+                # the affine terms are the TARGET's: the sum is rebuilt for every target
+                if t < t_first:
+                    continue
+                engine.accumulate_dense(surv, -1, acc, True)
+                for s in range(t + 1):
+                    if (src_mask >> s) & 1:
+                        engine.accumulate_dense(surv, s, acc, False, off[t] if off is not None else None,
+                                                sc[t] if sc is not None else None)
+            else:
+                if (src_mask >> t) & 1:
+                    engine.accumulate_dense(surv, t, acc, not started)
+                    started = True
+                if t < t_first:
+                    continue
+                if not started:
+                    engine.accumulate_dense(surv, -1, acc, True)
+                    started = True
+            lin = self.decoders[t]
+            engine.encode(acc.unsqueeze(0), lin.weight.detach().unsqueeze(0), lin.bias_param.detach().unsqueeze(0),
+                          out=out[t].unsqueeze(0))
+
     def decode_survivors(self, surv: SurvivorList, src_mask: int, t_begin: int = 0, t_end: Optional[int] = None,
                          skip_add: Optional[torch.Tensor] = None, ws=None) -> torch.Tensor:
         """Reconstructions [L, T, d] (rows outside [t_begin, t_end) are not written)."""
+        cfg = self.config
+        t_end = cfg.num_layers if t_end is None else t_end
+        split = self.dense_split(surv, src_mask, t_begin, t_end, skip_add)
+        self.last_route = {"sparse_targets": (t_begin, split), "dense_targets": (split, t_end)}
+        out = None
+        if split < t_end:
+            out = torch.empty((surv.L, surv.T, cfg.d_model), dtype=surv.dtype, device=surv.row_ptr.device)
+            self._decode_dense(surv, src_mask, split, t_end, out, ws)
+            if split == t_begin:
+                return out
         off, sc = self._affine()
-        return engine.decode_sparse(surv, self.packed(), self.config.decoder_tying, self.config.d_model,
+        return engine.decode_sparse(surv, self.packed(), cfg.decoder_tying, cfg.d_model,
                                     bias_sum=self.bias_sum(src_mask), feat_offset=off, feat_scale=sc,
-                                    skip_add=skip_add, t_begin=t_begin, t_end=t_end, src_mask=src_mask, ws=ws)
+                                    skip_add=skip_add, t_begin=t_begin, t_end=split, src_mask=src_mask, out=out, ws=ws)
 
     def skip_all_targets(self, inputs: Dict[int, torch.Tensor], src_mask: int, T: int) -> Optional[torch.Tensor]:
         """[L, T, d] fp32 skip-connection terms for every target present in ``inputs``."""

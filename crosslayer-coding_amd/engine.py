@@ -490,6 +490,11 @@ def decode_sparse(surv: SurvivorList, w_packed: torch.Tensor, tying: str, d: int
     for a in (feat_offset, feat_scale):
         assert a is None or (a.dtype == surv.dtype and a.is_contiguous() and a.shape == (L, F))
     lib = nat.load()
+    # the largest offset the kernels form, slot * F * d + f * d + column, is a 64-bit quantity (1.0e10
+    # elements for 300 decoders of 32768 x 1024); it must lie inside the slab that was handed in
+    need = lib.clt_decoder_slab_elems(d, F, L, nat.TYING[tying])
+    if need < 0 or w_packed.numel() < need:
+        raise nat.CLTNativeError(f"decode_sparse: packed decoders hold {w_packed.numel()} elements, the kernels index {need}")
     wbuf, wbytes = None, 0
     if ws is not None and T * (t_end - t_begin) >= SLICED_DECODE_MIN_ROWS:
         wbytes = lib.clt_decode_workspace_bytes(T, d, F, L)
@@ -501,6 +506,33 @@ def decode_sparse(surv: SurvivorList, w_packed: torch.Tensor, tying: str, d: int
         1 if out_f32 else 0, nat.ptr(wbuf), wbytes, _stream(w_packed))
     nat.check(code, "clt_decode_sparse")
     return out
+
+
+def decode_route(T: int, d: int, F: int, L: int, tying: str, dtype: torch.dtype, rows: Optional[int] = None) -> int:
+    """The schedule (``nat.ROUTE_*``) decode_sparse takes for these shapes when it is given a workspace
+    and ``rows`` = tokens x targets of the call (default: all L targets)."""
+    lib = nat.load()
+    rows = T * L if rows is None else rows
+    wbytes = lib.clt_decode_workspace_bytes(T, d, F, L) if rows >= SLICED_DECODE_MIN_ROWS else 0
+    code = lib.clt_decode_route(T, d, F, L, nat.TYING[tying], nat.dtype_code(dtype), wbytes)
+    if code < 0:
+        nat.check(code, "clt_decode_route")
+    return code
+
+
+def accumulate_dense(surv: SurvivorList, layer: int, acc: torch.Tensor, init: bool,
+                     feat_offset: Optional[torch.Tensor] = None, feat_scale: Optional[torch.Tensor] = None) -> None:
+    """acc [T, F] (model dtype) += the survivors of ``layer``, each addition rounded to the model dtype:
+    the ``summed_activation`` a decoder tied per target multiplies (decoder.py:208-246).  ``feat_offset``
+    / ``feat_scale`` [F]: the target layer's affine terms, applied to the non-zero entries."""
+    nat.require_device(acc, "accumulate_dense")
+    assert acc.shape == (surv.T, surv.F) and acc.is_contiguous() and acc.dtype == surv.dtype
+    for a in (feat_offset, feat_scale):
+        assert a is None or (a.dtype == surv.dtype and a.is_contiguous() and a.numel() == surv.F)
+    code = nat.load().clt_accumulate_dense(nat.ptr(surv.row_ptr), nat.ptr(surv.col), nat.ptr(surv.val),
+                                           nat.ptr(feat_offset), nat.ptr(feat_scale), nat.ptr(acc), surv.T, surv.F,
+                                           int(layer), 1 if init else 0, nat.dtype_code(surv.dtype), _stream(acc))
+    nat.check(code, "clt_accumulate_dense")
 
 
 def densify(surv: SurvivorList, out_f32: bool = False, out: Optional[torch.Tensor] = None) -> torch.Tensor:

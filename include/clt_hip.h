@@ -292,6 +292,43 @@ int clt_decode_sparse(const int32_t *row_ptr, const int32_t *col, const void *va
                       void *stream);
 
 /*
+ * Which schedule clt_decode_sparse takes for these shapes when it is given a workspace of
+ * `workspace_bytes` (16-byte aligned weights assumed): one of CLT_ROUTE_*, or a negative error code.
+ * A query for callers and tests; it launches nothing.
+ */
+#define CLT_ROUTE_GENERIC 0            /* any d: lanes stride over the output row */
+#define CLT_ROUTE_SINGLE 1             /* one wavefront per (target, token), all sources */
+#define CLT_ROUTE_SLICED 2             /* 8 feature slices, one launch per source layer */
+#define CLT_ROUTE_SLICED_ALL_SOURCES 3 /* 8 feature slices, decoders tied per target: one launch */
+#define CLT_ROUTE_QUARTER 4            /* 2 feature slices x 4 column quarters, one launch per source */
+int clt_decode_route(int64_t T, int64_t d, int64_t F, int64_t L, int tying, int dtype,
+                     size_t workspace_bytes);
+
+/*
+ * Number of elements of the packed decoder slab that clt_decode_sparse (and the backward entry
+ * points) may index: n_dec * F * d with n_dec = L(L+1)/2 untied, L tied - formed in 64 bits, as every
+ * kernel forms slot * F * d + f * d (the Pythia-410m shape has 1.0e10 elements).  Callers check their
+ * allocation against it.  Returns -1 on bad arguments.
+ */
+int64_t clt_decoder_slab_elems(int64_t d, int64_t F, int64_t L, int tying);
+
+/*
+ * Running dense sum of activations over source layers, the operand of a decoder tied per target
+ * (`summed_activation += activation_tensor`, clt/models/decoder.py:208-246):
+ *   acc[tok][f] = round(acc[tok][f] + v')   for the survivors (f, v) of rows layer*T .. layer*T+T-1
+ *   v' = v, or round(round(v + feat_offset[f]) * feat_scale[f]) on non-zero v when those rows
+ *   ([F], the target layer's, model dtype) are given (decoder.py:228-244).
+ * acc [T][F] in the model dtype, every addition rounded to it as the reference's tensor is; init != 0
+ * clears acc first (layer < 0 with init != 0: clear only).  The decode of target t is then one dense product of acc with the target's
+ * decoder in its checkpoint layout [d][F], which clt_encode computes (x = acc, w = decoder weight,
+ * b = decoder bias): the route for targets whose summed activations are dense enough that the matrix
+ * cores beat the row gather of clt_decode_sparse.
+ */
+int clt_accumulate_dense(const int32_t *row_ptr, const int32_t *col, const void *val,
+                         const void *feat_offset, const void *feat_scale, void *acc,
+                         int64_t T, int64_t F, int64_t layer, int init, int dtype, void *stream);
+
+/*
  * Dense materialisation of a survivor list: out[l][t][f] = value or 0.
  * out_f32 selects fp32 output (JumpReLU returns fp32, activations.py:180).
  * Replaces `x * mask.to(x.dtype)` (clt/models/activations.py:65, 347).

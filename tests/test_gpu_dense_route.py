@@ -1,0 +1,100 @@
+"""Decoders tied per target: the dense route (survivors scattered into the summed activation, then one
+product on the MFMA kernel - the reference's own formulation, clt/models/decoder.py:208-251) against the
+oracle and against the row-gather route, through the host mirror and through the C ABI."""
+import math
+
+import pytest
+import torch
+
+import crosslayer_coding_amd as cca
+from crosslayer_coding_amd import _native as nat
+from crosslayer_coding_amd import engine, synth
+from oracle import clt_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float32: 1e-5, torch.bfloat16: 1e-2}
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_accumulate_dense_is_the_running_sum_in_the_model_dtype(dev, dtype):
+    g = torch.Generator().manual_seed(3)
+    L, T, F = 3, 70, 200
+    acts = (torch.randn(L, T, F, generator=g) * (torch.rand(L, T, F, generator=g) < 0.3)).to(dtype)
+    acts[1, 4] = 0
+    off = torch.randn(F, generator=g).to(dtype)
+    sc = torch.randn(F, generator=g).to(dtype)
+    surv = engine.threshold_select(acts.to(dev), None, nat.PRED_NONZERO)
+    acc = torch.full((T, F), 7.0, dtype=dtype, device=dev)
+    want = torch.zeros(T, F, dtype=dtype)
+    for s in range(L):
+        engine.accumulate_dense(surv, s, acc, init=(s == 0))
+        want = want + acts[s]                       # the reference's `summed_activation += activation_tensor`
+        assert torch.equal(acc.cpu(), want)
+    # the target's affine terms touch the non-zero entries only (decoder.py:228-244)
+    engine.accumulate_dense(surv, -1, acc, init=True)
+    assert float(acc.abs().max()) == 0.0
+    want = torch.zeros(T, F, dtype=dtype)
+    for s in range(L):
+        engine.accumulate_dense(surv, s, acc, False, off.to(dev), sc.to(dev))
+        a = acts[s].clone()
+        nz = a != 0
+        a[nz] = ((a + off)[nz].to(dtype) * sc.expand(T, F)[nz]).to(dtype)
+        want = want + a
+    assert torch.equal(acc.cpu(), want)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("affine", [False, True])
+def test_dense_route_matches_the_oracle_and_the_gather_route(dev, dtype, affine):
+    tdt = getattr(torch, dtype)
+    wl = synth.Workload("dense-route", 7, 4, 256, 512, 512, dtype, k=24, decoder_tying="per_target")
+    cfg = wl.config()
+    cfg.enable_feature_offset = cfg.enable_feature_scale = affine
+    x = synth.make_inputs(wl, "cpu")
+    sd = synth.make_state_dict(wl, "cpu")
+    g = torch.Generator().manual_seed(9)
+    L, F, d = wl.num_layers, wl.num_features, wl.d_model
+    for i in range(L):
+        sd[f"decoder_module.decoders.{i}.bias_param"] = (torch.randn(d, generator=g) * 0.1).to(tdt)
+        if affine:
+            sd[f"decoder_module.feature_offset.{i}"] = (torch.randn(F, generator=g) * 0.2).to(tdt)
+            sd[f"decoder_module.feature_scale.{i}"] = (1 + 0.3 * torch.randn(F, generator=g)).to(tdt)
+    model = cca.CrossLayerTranscoder(cfg, None, dev)
+    model.load_state_dict(sd)
+    inputs = {l: x[l].to(dev) for l in range(L)}
+    dense = model(inputs)
+    route = dict(model.decoder_module.last_route)
+    assert route["dense_targets"][0] < route["dense_targets"][1] == L      # the dense route was taken
+    model.decoder_module.dense_route = False
+    sparse = model(inputs)
+    assert model.decoder_module.last_route["dense_targets"] == (L, L)
+    acts = {l: a.cpu() for l, a in model.get_feature_activations(inputs).items()}
+    names = synth.decoder_names(wl)
+    for t in range(L):
+        ref = orc.decode(acts, t, tying="per_target", weights={n: sd[f"decoder_module.decoders.{n}.weight"] for n in names},
+                         biases={n: sd[f"decoder_module.decoders.{n}.bias_param"] for n in names}, d_model=d,
+                         num_features=F, dtype=tdt,
+                         feature_offset=[sd[f"decoder_module.feature_offset.{i}"] for i in range(L)] if affine else None,
+                         feature_scale=[sd[f"decoder_module.feature_scale.{i}"] for i in range(L)] if affine else None)
+        assert orc.rel_l2(dense[t].cpu(), ref) <= TOL[tdt], (t, "dense")
+        assert orc.rel_l2(sparse[t].cpu(), ref) <= TOL[tdt], (t, "gather")
+    # a subset of layers: the missing source contributes nothing, the missing target is not produced
+    model.decoder_module.dense_route = True
+    part = model({l: inputs[l] for l in (0, 2, 3)})
+    assert sorted(part) == [0, 2, 3]
+    model.decoder_module.dense_route = False
+    want = model({l: inputs[l] for l in (0, 2, 3)})
+    for t in part:
+        assert orc.rel_l2(part[t].float().cpu(), want[t].float().cpu()) <= TOL[tdt]
+
+
+def test_route_query_names_the_schedules(dev):
+    big = 12 * 4096
+    assert engine.decode_route(4096, 768, 24576, 12, "none", torch.bfloat16) == nat.ROUTE_QUARTER
+    assert engine.decode_route(4096, 1024, 32768, 24, "none", torch.bfloat16) == nat.ROUTE_QUARTER
+    assert engine.decode_route(8192, 2048, 16384, 16, "per_target", torch.bfloat16) == nat.ROUTE_SLICED_ALL_SOURCES
+    assert engine.decode_route(4096, 640, 24576, 12, "per_source", torch.bfloat16) == nat.ROUTE_SLICED
+    assert engine.decode_route(4096, 768, 24576, 12, "none", torch.float32) == nat.ROUTE_QUARTER
+    assert engine.decode_route(16, 768, 24576, 12, "none", torch.bfloat16, rows=16) == nat.ROUTE_SINGLE
+    assert engine.decode_route(4096, 100, 24576, 12, "none", torch.bfloat16, rows=big) == nat.ROUTE_GENERIC
