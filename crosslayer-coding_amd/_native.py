@@ -46,6 +46,7 @@ _SIGNATURES = {
     "clt_tokentopk_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64, _int, _int]),
     "clt_tokentopk_select": (_int, [_vp, _i64, _i64, _i64, _i64, _i64, _int, _vp, _vp, _int, _vp, _vp, _vp, _vp, _sz, _vp]),
     "clt_threshold_count": (_int, [_vp, _i64, _i64, _i64, _i64, _vp, _int, _int, _vp, _vp, _sz, _vp]),
+    "clt_threshold_count_static": (_int, [_vp, _i64, _i64, _i64, _i64, _vp, _int, _int, _vp, _vp]),
     "clt_threshold_emit": (_int, [_vp, _i64, _i64, _i64, _i64, _vp, _int, _int, _vp, _vp, _vp, _vp]),
     "clt_encode_threshold_supported": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _int]),
     "clt_encode_threshold_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64, _i64, _int]),

@@ -24,6 +24,7 @@
 // again with the lowest cut, so the result is exact for any input; only the speed depends
 // on the sample being representative.
 #include "select_state.h"
+#include <mutex>
 
 namespace {
 
@@ -1733,6 +1734,43 @@ extern "C" int clt_threshold_count(const void *pre, int64_t T, int64_t F, int64_
   uint32_t *cnt = (uint32_t *)workspace;
   if (dtype == CLT_BF16) return dispatch_threshold<bf16_t>(false, pre, T, F, L, pre_layer_stride, theta, pred, cnt, row_ptr, nullptr, nullptr, s);
   return dispatch_threshold<float>(false, pre, T, F, L, pre_layer_stride, theta, pred, cnt, row_ptr, nullptr, nullptr, s);
+}
+
+// ---- clt_threshold_count for callers that cannot allocate ---------------------------------------
+// The per-row counters of clt_threshold_count live in a file-scope device array instead of a caller
+// workspace.  In host code `scratch` is only a handle for the symbol: the address a kernel can use is
+// looked up once per device with hipGetSymbolAddress (every GPU holds its own copy of the array at
+// its own address) and that pointer is what the launches get.
+constexpr int64_t STATIC_ROWS_MAX = 1 << 20;          // L*T rows: 4 MiB of counters per GPU
+constexpr int STATIC_MAX_DEVICES = 64;
+static __device__ __align__(256) uint32_t scratch[STATIC_ROWS_MAX];
+static uint32_t *g_scratch_ptr[STATIC_MAX_DEVICES];   // device address of `scratch`, per device
+static std::mutex g_scratch_mutex;
+
+static int scratch_of_current_device(uint32_t **out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= STATIC_MAX_DEVICES) return CLT_ERR_ARG;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void *p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return CLT_ERR_LAUNCH;
+    g_scratch_ptr[dev] = (uint32_t *)p;
+  }
+  *out = g_scratch_ptr[dev];
+  return CLT_OK;
+}
+
+extern "C" int clt_threshold_count_static(const void *pre, int64_t T, int64_t F, int64_t L, int64_t pre_layer_stride,
+                                          const void *theta, int pred, int dtype, int32_t *row_ptr, void *stream) {
+  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (T < 0 || F < 0 || L <= 0 || L > 65535 || !row_ptr) return CLT_ERR_ARG;
+  if (L * T > STATIC_ROWS_MAX) return CLT_ERR_RANGE;
+  uint32_t *cnt = nullptr;
+  const int rc = scratch_of_current_device(&cnt);
+  if (rc != CLT_OK) return rc;
+  // every counter of the L*T rows in use is written before it is read, so nothing has to be cleared
+  return clt_threshold_count(pre, T, F, L, pre_layer_stride, theta, pred, dtype, row_ptr, cnt,
+                             (size_t)STATIC_ROWS_MAX * 4, stream);
 }
 
 extern "C" int clt_threshold_emit(const void *pre, int64_t T, int64_t F, int64_t L, int64_t pre_layer_stride,

@@ -213,6 +213,20 @@ int clt_threshold_emit(const void *pre, int64_t T, int64_t F, int64_t L,
                        void *stream);
 
 /*
+ * clt_threshold_count for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * Same arguments and result as clt_threshold_count without the workspace: the per-row counters live
+ * in a device array inside the library (4 MiB per GPU, held until the process ends), so the call
+ * allocates and frees nothing.  Limit: L*T <= 1048576 rows, else CLT_ERR_RANGE.  The device that
+ * owns `stream` must be current.  All calls on one GPU share the array: calls that overlap on one
+ * GPU (different streams or threads) race; calls on one stream are ordered and safe.  The first call
+ * on a device looks the array's address up (hipGetSymbolAddress); make that call outside a capture.
+ */
+int clt_threshold_count_static(const void *pre, int64_t T, int64_t F, int64_t L,
+                               int64_t pre_layer_stride, const void *theta, int pred,
+                               int dtype, int32_t *row_ptr, void *stream);
+
+/*
  * Encoder projection and JumpReLU in one path, without writing the dense pre-activations:
  * the encoder's epilogue compares every value with its feature's threshold and appends the
  * survivors to a pool; the survivor list is then laid out from the pool.  Same result as
