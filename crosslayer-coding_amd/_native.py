@@ -20,7 +20,7 @@ CLT_F32, CLT_BF16, CLT_F16 = 0, 1, 2
 TYING = {"none": 0, "per_source": 1, "per_target": 2}
 TOPK_PER_LAYER, TOPK_GLOBAL = 0, 1
 PRED_GE_THETA, PRED_GT_ZERO, PRED_NONZERO = 0, 1, 2
-ROUTE_GENERIC, ROUTE_SINGLE, ROUTE_SLICED, ROUTE_SLICED_ALL_SOURCES, ROUTE_QUARTER = 0, 1, 2, 3, 4
+ROUTE_GENERIC, ROUTE_SINGLE, ROUTE_SLICED, ROUTE_SLICED_ALL_SOURCES, ROUTE_QUARTER, ROUTE_LINE = 0, 1, 2, 3, 4, 5
 
 _i64 = ctypes.c_int64
 _vp = ctypes.c_void_p
@@ -56,7 +56,8 @@ _SIGNATURES = {
     "clt_decode_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64]),
     "clt_decode_sparse": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _i64, _i64, _u64, _int, _int, _vp, _sz, _vp]),
     "clt_decode_route": (_int, [_i64, _i64, _i64, _i64, _int, _int, _sz]),
-    "clt_decoder_slab_elems": (_i64, [_i64, _i64, _i64, _int]),
+    "clt_decoder_pitch": (_i64, [_i64, _int]),
+    "clt_decoder_slab_elems": (_i64, [_i64, _i64, _i64, _int, _int]),
     "clt_accumulate_dense": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _int, _vp]),
     "clt_densify": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp]),
     "clt_mse_workspace_bytes": (_sz, [_i64, _i64, _i64]),

@@ -219,7 +219,7 @@ class CrossLayerTranscoder(BaseTranscoder):
                 slots = [s_] * len(targets)
             else:
                 slots = targets
-            stacked_w = torch.cat([packed[i] for i in slots], dim=1).unsqueeze(0)          # [1, F, n d]
+            stacked_w = torch.cat([packed[i][:, :cfg.d_model] for i in slots], dim=1).unsqueeze(0)   # [1, F, n d]
             stacked_g = torch.cat([g_model[t] for t in targets], dim=1).unsqueeze(0)       # [1, T, n d]
             dact = engine.encode(stacked_g.contiguous(), stacked_w.contiguous(), None)[0]  # [T, F]
             engine.jumprelu_theta_grad(pre[s_], dact, theta[s_].contiguous(), self.theta_manager.bandwidth, out[s_], ws)

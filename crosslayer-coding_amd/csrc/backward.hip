@@ -226,7 +226,8 @@ __global__ __launch_bounds__(BW_THREADS) void k_bwd_values_sliced(
   int64_t s = 0, rem = pair;
   while (rem >= L - s) { rem -= L - s; ++s; }
   const int64_t t = s + rem;
-  const T *wbase = wp + bw_decoder_slot(tying, s, t, L) * F * d;
+  const int64_t pitch = clt_pitch(d, (int)sizeof(T));
+  const T *wbase = wp + bw_decoder_slot(tying, s, t, L) * F * pitch;
   float *pt = part + t * nnz;
   constexpr int NFULL = T8 ? NCH - 1 : NCH, HV = EV / 2;
   const int64_t tail_at = (int64_t)NFULL * 64 * EV + lane * HV;
@@ -268,7 +269,7 @@ __global__ __launch_bounds__(BW_THREADS) void k_bwd_values_sliced(
 #pragma unroll
           for (int u = 0; u < LB; ++u) {
             const int idx = i0 + h + u < n ? i0 + h + u : n - 1;
-            const T *wrow = wbase + (int64_t)__builtin_amdgcn_readlane(my_col, idx) * d;
+            const T *wrow = wbase + (int64_t)__builtin_amdgcn_readlane(my_col, idx) * pitch;
 #pragma unroll
             for (int c = 0; c < NFULL; ++c)
               w[u][c] = on[c] ? *reinterpret_cast<const uint4 *>(wrow + (int64_t)c * 64 * EV + lane * EV) : make_uint4(0, 0, 0, 0);

@@ -75,6 +75,18 @@ __device__ __forceinline__ uint32_t mbcnt64(uint64_t mask) {
 
 __device__ __forceinline__ uint64_t ballot64(bool p) { return __ballot(p); }
 
+// ---------------------------------------------------------------- packed decoder rows
+// Row pitch (elements) of the feature-major decoder slab [n_dec][F][pitch].  A row that is a whole,
+// EVEN number of 128-byte cache lines is padded by one line: with an even line pitch the same column part
+// of every row falls on a fraction of the 16 L2 channels (pitch 16 lines: on ONE channel), so a kernel
+// that gathers one column part per XCD would use only that fraction of its L2; an odd pitch spreads any
+// column part over all channels and sets.  Other widths are stored densely.
+__host__ __device__ static inline int64_t clt_pitch(int64_t d, int elem_bytes) {
+  const int64_t row_bytes = d * elem_bytes;
+  if (row_bytes % 128 != 0 || (row_bytes / 128) % 2 != 0) return d;
+  return d + 128 / elem_bytes;
+}
+
 // ---------------------------------------------------------------- host helpers
 static inline int clt_check_launch() {
   hipError_t e = hipGetLastError();

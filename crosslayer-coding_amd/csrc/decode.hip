@@ -187,7 +187,7 @@ __attribute__((amdgpu_waves_per_eu(decode_min_waves<T, NF, TAIL, SLICED>(), 8)))
     const T *__restrict__ fscale, const float *__restrict__ skip_add, void *__restrict__ out,
     int64_t Tn, int64_t d, int64_t F, int64_t L, int tying, int64_t t_begin, int64_t t_end,
     uint64_t src_mask, int out_f32, const int32_t *__restrict__ sptr, float *__restrict__ partial, int ns,
-    int src) {
+    int src, int64_t pitch) {
   constexpr int V = WVec<T>::V;
   constexpr int HV = V / 2;                       // elements per 8 bytes
   constexpr int NACC = NF * V + (TAIL == 1 ? HV : TAIL == 2 ? V : 0);
@@ -207,7 +207,7 @@ __attribute__((amdgpu_waves_per_eu(decode_min_waves<T, NF, TAIL, SLICED>(), 8)))
   const bool tail_on = TAIL == 1 ? true : (TAIL == 2 ? tail_off < d : false);
 
   auto gather_rows = [&](int64_t s, int32_t b, int32_t e) {
-    const T *wbase = wp + decoder_slot(tying, s, t, L) * F * d;
+    const T *wbase = wp + decoder_slot(tying, s, t, L) * F * pitch;
     for (int32_t j0 = b; j0 < e; j0 += 64) {
       const int n = (e - j0) < 64 ? (e - j0) : 64;
       int32_t my_col = 0; float my_val = 0.0f;
@@ -220,8 +220,8 @@ __attribute__((amdgpu_waves_per_eu(decode_min_waves<T, NF, TAIL, SLICED>(), 8)))
         }
       }
       int i0 = 0;
-      for (; i0 + U <= n; i0 += U) decode_batch<T, NF, TAIL, U>(acc, wbase, d, my_col, my_val, i0, n, lane, tail_off, tail_on);
-      for (; i0 < n; i0 += 2) decode_batch<T, NF, TAIL, 2>(acc, wbase, d, my_col, my_val, i0, n, lane, tail_off, tail_on);
+      for (; i0 + U <= n; i0 += U) decode_batch<T, NF, TAIL, U>(acc, wbase, pitch, my_col, my_val, i0, n, lane, tail_off, tail_on);
+      for (; i0 < n; i0 += 2) decode_batch<T, NF, TAIL, 2>(acc, wbase, pitch, my_col, my_val, i0, n, lane, tail_off, tail_on);
     }
   };
 
@@ -235,7 +235,7 @@ __attribute__((amdgpu_waves_per_eu(decode_min_waves<T, NF, TAIL, SLICED>(), 8)))
       // All sources in one launch (decoders tied per target: every source <= t gathers from the same
       // matrix W[t], so the slice an XCD works on stays the same while the sources go by): the
       // accumulators stay in registers over the sources and the partial row is written once.
-      const T *wb = wp + decoder_slot(tying, 0, t, L) * F * d;
+      const T *wb = wp + decoder_slot(tying, 0, t, L) * F * pitch;
       for (int i = 0; i < SLICED_NTOK; ++i) {
         if (tok0 + i >= Tn) break;
 #pragma unroll
@@ -252,7 +252,7 @@ __attribute__((amdgpu_waves_per_eu(decode_min_waves<T, NF, TAIL, SLICED>(), 8)))
               if (foff) my_val = Elem<T>::round(my_val + Elem<T>::to_f32(foff[t * F + my_col]));
               if (fscale) my_val = Elem<T>::round(my_val * Elem<T>::to_f32(fscale[t * F + my_col]));
             }
-            decode_chunk_pipelined<T, NF, TAIL, (U > 6 ? 6 : U)>(acc, wb, d, my_col, my_val, n, lane, tail_off, tail_on);
+            decode_chunk_pipelined<T, NF, TAIL, (U > 6 ? 6 : U)>(acc, wb, pitch, my_col, my_val, n, lane, tail_off, tail_on);
           }
         }
         float *prow = partial + (((int64_t)slice * L + t) * Tn + tok0 + i) * d;
@@ -282,7 +282,7 @@ __attribute__((amdgpu_waves_per_eu(decode_min_waves<T, NF, TAIL, SLICED>(), 8)))
       mb = sptr[r * (ns + 1) + slice];
       me = sptr[r * (ns + 1) + slice + 1];
     }
-    const T *wbase = wp + decoder_slot(tying, src, t, L) * F * d;
+    const T *wbase = wp + decoder_slot(tying, src, t, L) * F * pitch;
     int32_t nb = __builtin_amdgcn_readlane(mb, 0), ne = __builtin_amdgcn_readlane(me, 0);
     int32_t nxt_col = 0; T nxt_val = T(0);
     if (lane < ne - nb) { nxt_col = col[nb + lane]; nxt_val = val[nb + lane]; }
@@ -331,7 +331,7 @@ __attribute__((amdgpu_waves_per_eu(decode_min_waves<T, NF, TAIL, SLICED>(), 8)))
           if (foff) my_val = Elem<T>::round(my_val + Elem<T>::to_f32(foff[t * F + my_col]));
           if (fscale) my_val = Elem<T>::round(my_val * Elem<T>::to_f32(fscale[t * F + my_col]));
         }
-        decode_chunk_pipelined<T, NF, TAIL, (U > 6 ? 6 : U)>(acc, wbase, d, my_col, my_val, n, lane, tail_off, tail_on);
+        decode_chunk_pipelined<T, NF, TAIL, (U > 6 ? 6 : U)>(acc, wbase, pitch, my_col, my_val, n, lane, tail_off, tail_on);
       }
 #pragma unroll
       for (int c = 0; c < NF; ++c) {
@@ -375,6 +375,58 @@ __attribute__((amdgpu_waves_per_eu(decode_min_waves<T, NF, TAIL, SLICED>(), 8)))
   if (TAIL == 2) emit(tail_off, acc + NF * V, V, tail_on);
 }
 
+// How the units (slice, column part) of one target are dealt to the 8 XCDs: `full` rounds in which XCD x
+// takes unit round * 8 + x over all tokens, then the `rem` units that are left over, with the tokens of each
+// split between q XCDs so that all eight stay busy (rem divides 8: one round, q = 8 / rem; otherwise `rem`
+// rounds in which all XCDs share one unit, q = 8).  Blocks go to the XCDs round-robin, so block b runs on
+// XCD b % 8; within an XCD the blocks are ordered target, round, token block: an XCD finishes one part of
+// one decoder matrix before it touches the next.
+struct UnitPlan {
+  int ns, ncp, full, rem, q;
+  int bf, br;            // blocks per XCD in a full round / in a remainder round
+  int64_t tpp;           // tokens per XCD in a remainder round
+  int bpx;               // blocks per XCD and target
+};
+
+static UnitPlan make_unit_plan(int ns, int ncp, int64_t Tn, int tok_per_block) {
+  UnitPlan up;
+  up.ns = ns; up.ncp = ncp;
+  const int units = ns * ncp;
+  up.full = units / 8; up.rem = units % 8;
+  up.q = up.rem == 0 ? 1 : (8 % up.rem == 0 ? 8 / up.rem : 8);
+  const int rem_rounds = up.rem == 0 ? 0 : (8 % up.rem == 0 ? 1 : up.rem);
+  up.tpp = clt_ceil_div(Tn, up.q);
+  up.bf = (int)clt_ceil_div(Tn, tok_per_block);
+  up.br = (int)clt_ceil_div(up.tpp, tok_per_block);
+  up.bpx = up.full * up.bf + rem_rounds * up.br;
+  return up;
+}
+
+// this block's work: target index (relative), unit -> (slice, column part), its token range and its token block
+struct UnitWork { int64_t target; int slice, cpart; int64_t tok_begin, tok_end; int tb; };
+__device__ __forceinline__ UnitWork unit_work(const UnitPlan &up, int64_t Tn) {
+  UnitWork w;
+  const int xcd = (int)(blockIdx.x & 7);
+  const int64_t i = (int64_t)(blockIdx.x >> 3);
+  w.target = i / up.bpx;
+  const int j = (int)(i % up.bpx);
+  int unit;
+  w.tok_begin = 0; w.tok_end = Tn;
+  if (j < up.full * up.bf) {
+    unit = (j / up.bf) * 8 + xcd; w.tb = j % up.bf;
+  } else {
+    const int jr = j - up.full * up.bf, rr = jr / up.br;
+    w.tb = jr % up.br;
+    int tpart;
+    if (up.q * up.rem == 8) { unit = up.full * 8 + xcd / up.q; tpart = xcd % up.q; }
+    else { unit = up.full * 8 + rr; tpart = xcd; }
+    w.tok_begin = (int64_t)tpart * up.tpp;
+    w.tok_end = w.tok_begin + up.tpp < Tn ? w.tok_begin + up.tpp : Tn;
+  }
+  w.cpart = unit % up.ncp; w.slice = unit / up.ncp;
+  return w;
+}
+
 // ---- quarter-row schedule -------------------------------------------------------------------------
 // Large batches, untied or per-source decoders, d a multiple of 256: the feature axis is cut into 2
 // slices and the columns into 4 quarters; workgroup b works on part b % 8 = (slice, quarter), so an XCD
@@ -388,33 +440,49 @@ constexpr int QLANES = 16;              // lanes per quarter row
 constexpr int QROWS = 64 / QLANES;      // rows per load
 constexpr int QUARTER_SLICES = 2;       // feature slices; 8 / QUARTER_SLICES column parts
 constexpr int QUARTER_PARTS = 8 / QUARTER_SLICES;
-template <typename T, int HQ, int HTAIL, int UU> struct PartBatch {
+template <typename T, int HQ, int HTAIL, int UU, bool PACK> struct PartBatch {
   uint4 wq[UU][HQ > 0 ? HQ : 1];
   uint2 wt8[UU];
-  float v[UU];
-  // slot QROWS * u + g of the (up to 64) survivors held one per lane goes to lane group g
-  __device__ __forceinline__ void load(const T *wbase, int64_t d, int32_t my_col, float my_val, int i0, int n, int ll, int grp) {
+  float v[UU];          // !PACK: the activation values
+  uint32_t pk[UU];      // PACK: feature index | bf16 value << 16
+  // slot QROWS * u + g of the (up to 64) survivors held one per lane goes to lane group g.  Lanes past the
+  // end of the list hold feature 0 with value 0: a repeated fetch with weight 0, so nothing is clamped.
+  // PACK (bf16, F <= 65536): one cross-lane move per row, and the row offset is a 24-bit multiply-add.
+  __device__ __forceinline__ void load(const T *wbase, int64_t d, uint32_t my_pk, int32_t my_col, float my_val, int i0, int n,
+                                       int ll, int grp) {
     constexpr int V = WVec<T>::V;
 #pragma unroll
     for (int u = 0; u < UU; ++u) {
       const int idx = i0 + QROWS * u + grp;
-      const int ci = idx < n ? idx : n - 1;                 // clamp: a repeated fetch, weight 0
-      const int32_t f = __shfl(my_col, ci);
-      const float vv = __shfl(my_val, ci);
-      v[u] = idx < n ? vv : 0.0f;
-      const T *wrow = wbase + (int64_t)f * d;
+      if constexpr (PACK) {
+        pk[u] = (uint32_t)__builtin_amdgcn_ds_bpermute(idx << 2, (int)my_pk);
+        const uint32_t off = __umul24(pk[u] & 0xFFFFu, (uint32_t)d * (uint32_t)sizeof(T)) + (uint32_t)(ll * 16);
+        const char *wrow = reinterpret_cast<const char *>(wbase) + off;
 #pragma unroll
-      for (int c = 0; c < HQ; ++c) wq[u][c] = *reinterpret_cast<const uint4 *>(wrow + c * QLANES * V + ll * V);
-      if (HTAIL) wt8[u] = *reinterpret_cast<const uint2 *>(wrow + HQ * QLANES * V + ll * (V / 2));
+        for (int c = 0; c < HQ; ++c) wq[u][c] = *reinterpret_cast<const uint4 *>(wrow + c * QLANES * 16);
+        if (HTAIL) wt8[u] = *reinterpret_cast<const uint2 *>(wrow + HQ * QLANES * 16 - ll * 8);
+      } else {
+        const int ci = idx < n ? idx : n - 1;                 // clamp: a repeated fetch, weight 0
+        const int32_t f = __shfl(my_col, ci);
+        const float vv = __shfl(my_val, ci);
+        v[u] = idx < n ? vv : 0.0f;
+        const T *wrow = wbase + (int64_t)f * d;
+#pragma unroll
+        for (int c = 0; c < HQ; ++c) wq[u][c] = *reinterpret_cast<const uint4 *>(wrow + c * QLANES * V + ll * V);
+        if (HTAIL) wt8[u] = *reinterpret_cast<const uint2 *>(wrow + HQ * QLANES * V + ll * (V / 2));
+      }
     }
+  }
+  __device__ __forceinline__ uint32_t value_pair(int u) const {
+    if constexpr (PACK) return __builtin_amdgcn_perm(pk[u + 1], pk[u], 0x07060302u);   // (value u, value u + 1)
+    else return (__float_as_uint(v[u]) >> 16) | (__float_as_uint(v[u + 1]) & 0xFFFF0000u);
   }
   __device__ __forceinline__ void consume(float *acc) const {
     constexpr int V = WVec<T>::V;
     if constexpr (sizeof(T) == 2 && (UU % 2) == 0) {
 #pragma unroll
       for (int u = 0; u < UU; u += 2) {
-        const uint32_t vb = (__float_as_uint(v[u]) >> 16) | (__float_as_uint(v[u + 1]) & 0xFFFF0000u);
-        const bf16x2_t vv = __builtin_bit_cast(bf16x2_t, vb);
+        const bf16x2_t vv = __builtin_bit_cast(bf16x2_t, value_pair(u));
 #pragma unroll
         for (int c = 0; c < HQ; ++c) WVec<T>::dot16(acc + c * V, wq[u][c], wq[u + 1][c], vv);
         if (HTAIL) WVec<T>::dot8(acc + HQ * V, wt8[u], wt8[u + 1], vv);
@@ -437,32 +505,33 @@ template <typename T, int HQ, int HTAIL> constexpr int quarter_min_waves() {
   return (sizeof(T) == 2 && HQ * V + (HTAIL ? V / 2 : 0) <= 12) ? 7 : 1;   // fp32 at 7 would spill
 }
 
-template <typename T, int HQ, int HTAIL, int UU, bool AFFINE>
+template <typename T, int HQ, int HTAIL, int UU, bool AFFINE, bool PACK>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(quarter_min_waves<T, HQ, HTAIL>(), 8))) void k_decode_quarter(
     const int32_t *__restrict__ col, const T *__restrict__ val, const T *__restrict__ wp, const T *__restrict__ foff,
     const T *__restrict__ fscale, int64_t Tn, int64_t d, int64_t F, int64_t L, int tying, int64_t t_begin, uint64_t src_mask,
-    const int32_t *__restrict__ sptr, float *__restrict__ partial, int src) {
+    const int32_t *__restrict__ sptr, float *__restrict__ partial, int src, int64_t pitch, UnitPlan up) {
   constexpr int V = WVec<T>::V;
   constexpr int NACC = HQ * V + (HTAIL ? V / 2 : 0);      // columns per lane: d / 64
-  constexpr int ns = QUARTER_SLICES, NCP = QUARTER_PARTS;
+  constexpr int NCP = QUARTER_PARTS;
+  const int ns = up.ns;
   const int lane = lane_id(), wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
   const int ll = lane & (QLANES - 1), grp = lane / QLANES;
   const bool hi = grp != 0;                    // only the first lane group touches the partial row
-  const int part = (int)(blockIdx.x % 8), slice = part % ns, cpart = part / ns;
-  const int64_t bid = (int64_t)blockIdx.x / 8;
-  const int64_t blocks_per_t = (Tn + (int64_t)nwv * QUARTER_NTOK - 1) / ((int64_t)nwv * QUARTER_NTOK);
-  const int64_t t = t_begin + bid / blocks_per_t;
-  const int64_t tok0 = ((bid % blocks_per_t) * nwv + wv) * QUARTER_NTOK;
-  if (tok0 >= Tn) return;
+  const UnitWork uw = unit_work(up, Tn);
+  const int slice = uw.slice, cpart = uw.cpart;
+  const int64_t t = t_begin + uw.target;
+  const int64_t tok_end = uw.tok_end;
+  const int64_t tok0 = uw.tok_begin + ((int64_t)uw.tb * nwv + wv) * QUARTER_NTOK;
+  if (tok0 >= tok_end) return;
   const uint64_t below = src_mask & ((1ull << src) - 1ull);
   const bool first = below == 0;   // the first source initialises the partial rows
   int32_t mb = 0, me = 0;
-  if (lane < QUARTER_NTOK && tok0 + lane < Tn) {
+  if (lane < QUARTER_NTOK && tok0 + lane < tok_end) {
     const int64_t r = (int64_t)src * Tn + tok0 + lane;
     mb = sptr[r * (ns + 1) + slice];
     me = sptr[r * (ns + 1) + slice + 1];
   }
-  const T *wbase = wp + decoder_slot(tying, src, t, L) * F * d + (int64_t)cpart * (d / NCP);
+  const T *wbase = wp + decoder_slot(tying, src, t, L) * F * pitch + (int64_t)cpart * (d / NCP);
   int32_t nb = __builtin_amdgcn_readlane(mb, 0), ne = __builtin_amdgcn_readlane(me, 0);
   int32_t nxt_col = 0; T nxt_val = T(0);
   if (lane < ne - nb) { nxt_col = col[nb + lane]; nxt_val = val[nb + lane]; }
@@ -475,7 +544,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(quarter_min
       nxt_col = 0; nxt_val = T(0);
       if (lane < ne - nb) { nxt_col = col[nb + lane]; nxt_val = val[nb + lane]; }
     }
-    if (tok0 + i >= Tn) break;
+    if (tok0 + i >= tok_end) break;
     if (b == e && !first) continue;
     // this lane's columns of the partial row (the first lane group writes it): pieces of V, then the tail
     float *prow = partial + (((int64_t)slice * L + t) * Tn + tok0 + i) * d + (int64_t)cpart * (d / NCP);
@@ -494,14 +563,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(quarter_min
         if (fscale) my_val = Elem<T>::round(my_val * Elem<T>::to_f32(fscale[t * F + my_col]));
       }
       // two batches of UU row pairs in flight
-      PartBatch<T, HQ, HTAIL, UU> ra, rb;
+      const uint32_t my_pk = PACK ? ((uint32_t)my_col | (__float_as_uint(my_val) & 0xFFFF0000u)) : 0u;
+      PartBatch<T, HQ, HTAIL, UU, PACK> ra, rb;
       constexpr int R = QROWS;
-      ra.load(wbase, d, my_col, my_val, 0, n, ll, grp);
+      ra.load(wbase, pitch, my_pk, my_col, my_val, 0, n, ll, grp);
       for (int i0 = 0; i0 < n; i0 += 2 * R * UU) {
-        if (i0 + R * UU < n) rb.load(wbase, d, my_col, my_val, i0 + R * UU, n, ll, grp);
+        if (i0 + R * UU < n) rb.load(wbase, pitch, my_pk, my_col, my_val, i0 + R * UU, n, ll, grp);
         ra.consume(acc);
         if (i0 + R * UU < n) {
-          if (i0 + 2 * R * UU < n) ra.load(wbase, d, my_col, my_val, i0 + 2 * R * UU, n, ll, grp);
+          if (i0 + 2 * R * UU < n) ra.load(wbase, pitch, my_pk, my_col, my_val, i0 + 2 * R * UU, n, ll, grp);
           rb.consume(acc);
         }
       }
@@ -558,6 +628,169 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(quarter_min
   }
 }
 
+// ---- line schedule ---------------------------------------------------------------------------------
+// Large batches, untied or per-source decoders, rows that are whole 128-byte cache lines: the COLUMNS are
+// cut into parts of exactly one cache line (64 bf16 / 32 fp32), so the piece of a decoder matrix that an
+// XCD gathers from while all tokens stream past is F x 128 bytes (3.0 MiB at F = 24576, inside its 4 MiB
+// L2; wider feature axes are cut into `ns` slices to stay there).  The units of work (slice, column part,
+// token part) are dealt to the XCDs in rounds - unit u runs on XCD u % 8 in round u / 8 - and the token
+// axis is cut into `ntp` parts only to make their number a multiple of 8.  A load instruction fetches the
+// line of EIGHT survivors (8 lanes x 16 bytes each); every lane group accumulates its own survivors and a
+// butterfly that halves the accumulators at every step (reduce-scatter: 7 shuffles for 8 accumulators)
+// leaves each lane with the finished sum of one column.  With ns = 1 a (target, token) has one fp32
+// partial row, read and written once per source layer.
+constexpr int LINE_UU = 2;                // loads per batch (two batches in flight)
+constexpr int64_t LINE_L2_BYTES = 3407872;   // 3.25 MiB: the part of a matrix one XCD works on stays below this
+
+template <typename T, int UU, bool PACK> struct LineBatch {
+  uint4 wq[UU];
+  float v[UU];          // !PACK: the activation values
+  uint32_t pk[UU];      // PACK: feature index | bf16 value << 16
+  // entry 8 * u + grp of the (up to 64) survivors held one per lane goes to lane group grp; lanes past the
+  // end of the list hold feature 0 with value 0 (a repeated fetch, weight 0)
+  __device__ __forceinline__ void load(const T *wbase, int64_t rstride, uint32_t my_pk, int32_t my_col, float my_val, int i0,
+                                       int n, int ll, int grp) {
+    constexpr int V = WVec<T>::V;
+#pragma unroll
+    for (int u = 0; u < UU; ++u) {
+      const int idx = i0 + 8 * u + grp;
+      if constexpr (PACK) {
+        pk[u] = (uint32_t)__builtin_amdgcn_ds_bpermute(idx << 2, (int)my_pk);
+        const uint32_t off = __umul24(pk[u] & 0xFFFFu, (uint32_t)rstride * (uint32_t)sizeof(T)) + (uint32_t)(ll * 16);
+        wq[u] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const char *>(wbase) + off);
+      } else {
+        const int ci = idx < n ? idx : n - 1;
+        const int32_t f = __shfl(my_col, ci);
+        const float vv = __shfl(my_val, ci);
+        v[u] = idx < n ? vv : 0.0f;
+        wq[u] = *reinterpret_cast<const uint4 *>(wbase + (int64_t)f * rstride + ll * V);
+      }
+    }
+  }
+  __device__ __forceinline__ void consume(float *acc) const {
+    if constexpr (sizeof(T) == 2 && (UU % 2) == 0) {
+#pragma unroll
+      for (int u = 0; u < UU; u += 2) {
+        uint32_t vb;
+        if constexpr (PACK) vb = __builtin_amdgcn_perm(pk[u + 1], pk[u], 0x07060302u);
+        else vb = (__float_as_uint(v[u]) >> 16) | (__float_as_uint(v[u + 1]) & 0xFFFF0000u);
+        WVec<T>::dot16(acc, wq[u], wq[u + 1], __builtin_bit_cast(bf16x2_t, vb));
+      }
+    } else {
+#pragma unroll
+      for (int u = 0; u < UU; ++u) WVec<T>::fma16(acc, wq[u], v[u]);
+    }
+  }
+};
+
+template <typename T, bool AFFINE, bool PACK, int NTOK>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))) void k_decode_line(
+    const int32_t *__restrict__ col, const T *__restrict__ val, const T *__restrict__ wp, const T *__restrict__ foff,
+    const T *__restrict__ fscale, int64_t Tn, int64_t d, int64_t F, int64_t L, int tying, int64_t t_begin, uint64_t src_mask,
+    const int32_t *__restrict__ sptr, float *__restrict__ partial, int src, UnitPlan lp, int64_t pitch) {
+  constexpr int V = WVec<T>::V;                     // elements per lane: 16 bytes
+  constexpr int LW = 8 * V;                         // columns per part: one 128-byte line
+  constexpr int LINE_NTOK = NTOK;
+  const int lane = lane_id(), wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
+  const int ll = lane & 7, grp = lane >> 3;
+  const int ns = lp.ns;
+  const UnitWork uw = unit_work(lp, Tn);
+  const int64_t t = t_begin + uw.target;
+  const int cpart = uw.cpart, slice = uw.slice;
+  const int64_t part_end = uw.tok_end;
+  const int64_t tok0 = uw.tok_begin + ((int64_t)uw.tb * nwv + wv) * LINE_NTOK;
+  if (tok0 >= part_end) return;
+  const uint64_t below = src_mask & ((1ull << src) - 1ull);
+  const bool first = below == 0;   // the first source initialises the partial rows
+  int32_t mb = 0, me = 0;
+  if (lane < LINE_NTOK && tok0 + lane < part_end) {
+    const int64_t r = (int64_t)src * Tn + tok0 + lane;
+    mb = sptr[r * (ns + 1) + slice];
+    me = sptr[r * (ns + 1) + slice + 1];
+  }
+  const T *wbase = wp + decoder_slot(tying, src, t, L) * F * pitch + (int64_t)cpart * LW;
+  int32_t nb = __builtin_amdgcn_readlane(mb, 0), ne = __builtin_amdgcn_readlane(me, 0);
+  int32_t nxt_col = 0; T nxt_val = T(0);
+  if (lane < ne - nb) { nxt_col = col[nb + lane]; nxt_val = val[nb + lane]; }
+#pragma unroll
+  for (int it = 0; it < LINE_NTOK; ++it) {
+    const int32_t b = nb, e = ne;
+    const int32_t cur_col = nxt_col; const T cur_val = nxt_val;
+    if (it + 1 < LINE_NTOK) {
+      nb = __builtin_amdgcn_readlane(mb, it + 1); ne = __builtin_amdgcn_readlane(me, it + 1);
+      nxt_col = 0; nxt_val = T(0);
+      if (lane < ne - nb) { nxt_col = col[nb + lane]; nxt_val = val[nb + lane]; }
+    }
+    if (tok0 + it >= part_end) break;
+    if (b == e && !first) continue;
+    float acc[V];
+#pragma unroll
+    for (int j = 0; j < V; ++j) acc[j] = 0.0f;
+    LineBatch<T, LINE_UU, PACK> ra, rb;
+    for (int32_t j0 = b; j0 < e; j0 += 64) {
+      const int n = (e - j0) < 64 ? (e - j0) : 64;
+      int32_t my_col = cur_col; float my_val = Elem<T>::to_f32(cur_val);
+      if (j0 > b) {   // more than 64 survivors in this slice: fetch the next 64
+        my_col = 0; my_val = 0.0f;
+        if (lane < n) { my_col = col[j0 + lane]; my_val = Elem<T>::to_f32(val[j0 + lane]); }
+      }
+      if (AFFINE && my_val != 0.0f) {
+        if (foff) my_val = Elem<T>::round(my_val + Elem<T>::to_f32(foff[t * F + my_col]));
+        if (fscale) my_val = Elem<T>::round(my_val * Elem<T>::to_f32(fscale[t * F + my_col]));
+      }
+      // bf16: feature index (< 65536) and value travel to their lane group in one 32-bit word
+      const uint32_t my_pk = PACK ? ((uint32_t)my_col | (__float_as_uint(my_val) & 0xFFFF0000u)) : 0u;
+      constexpr int R = 8 * LINE_UU;                 // survivors per batch
+      ra.load(wbase, pitch, my_pk, my_col, my_val, 0, n, ll, grp);
+      for (int i0 = 0; i0 < n; i0 += 2 * R) {
+        if (i0 + R < n) rb.load(wbase, pitch, my_pk, my_col, my_val, i0 + R, n, ll, grp);
+        ra.consume(acc);
+        if (i0 + R < n) {
+          if (i0 + 2 * R < n) ra.load(wbase, pitch, my_pk, my_col, my_val, i0 + 2 * R, n, ll, grp);
+          rb.consume(acc);
+        }
+      }
+    }
+    // reduce-scatter over the eight lane groups (fixed order): every step hands half of the accumulators to
+    // the partner group and adds the half that comes back, so a lane ends with the sum of ONE column
+    float r; int csel; bool writer = true;
+    if constexpr (V == 8) {
+      float a4[4], a2[2];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float keep = (grp & 4) ? acc[j + 4] : acc[j], send = (grp & 4) ? acc[j] : acc[j + 4];
+        a4[j] = keep + __shfl_xor(send, 32);
+      }
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const float keep = (grp & 2) ? a4[j + 2] : a4[j], send = (grp & 2) ? a4[j] : a4[j + 2];
+        a2[j] = keep + __shfl_xor(send, 16);
+      }
+      const float keep = (grp & 1) ? a2[1] : a2[0], send = (grp & 1) ? a2[0] : a2[1];
+      r = keep + __shfl_xor(send, 8);
+      csel = ll * 8 + grp;
+    } else {
+      float a2[2];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const float keep = (grp & 4) ? acc[j + 2] : acc[j], send = (grp & 4) ? acc[j] : acc[j + 2];
+        a2[j] = keep + __shfl_xor(send, 32);
+      }
+      const float keep = (grp & 2) ? a2[1] : a2[0], send = (grp & 2) ? a2[0] : a2[1];
+      const float a1 = keep + __shfl_xor(send, 16);
+      const float o = __shfl_xor(a1, 8);
+      r = (grp & 1) ? o + a1 : a1 + o;             // both lanes of a pair form the same sum
+      csel = ll * 4 + ((grp >> 2) & 1) * 2 + ((grp >> 1) & 1);
+      writer = (grp & 1) == 0;
+    }
+    float *pp = partial + (((int64_t)slice * L + t) * Tn + tok0 + it) * d + (int64_t)cpart * LW + csel;
+    if (writer) {
+      const float old = first ? 0.0f : __builtin_nontemporal_load(pp);
+      __builtin_nontemporal_store(old + r, pp);
+    }
+  }
+}
+
 // sptr[r][j] = first survivor of row r whose feature index is >= j * F / ns  (j = 0..ns)
 __global__ void k_slice_ptr(const int32_t *row_ptr, const int32_t *col, int64_t R, int64_t F, int ns, int32_t *sptr) {
   const int64_t total = R * (ns + 1);
@@ -609,7 +842,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void k_decode_generic(
     const int32_t *row_ptr, const int32_t *col, const T *val, const T *wp, const float *bias_sum,
     const T *foff, const T *fscale, const float *skip_add, void *out, int64_t Tn, int64_t d,
-    int64_t F, int64_t L, int tying, int64_t t_begin, int64_t t_end, uint64_t src_mask, int out_f32) {
+    int64_t F, int64_t L, int tying, int64_t t_begin, int64_t t_end, uint64_t src_mask, int out_f32, int64_t pitch) {
   const int lane = lane_id(), wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
   const int64_t blocks_per_t = (Tn + nwv - 1) / nwv;
   const int64_t t = t_end - 1 - (int64_t)blockIdx.x / blocks_per_t;
@@ -621,7 +854,7 @@ __global__ __launch_bounds__(256) void k_decode_generic(
     for (int64_t s = 0; s <= t; ++s) {
       if (!((src_mask >> s) & 1ull)) continue;
       const int64_t r = s * Tn + tok;
-      const T *wbase = wp + decoder_slot(tying, s, t, L) * F * d;
+      const T *wbase = wp + decoder_slot(tying, s, t, L) * F * pitch;
       for (int32_t j = row_ptr[r]; j < row_ptr[r + 1]; ++j) {
         const int32_t f = col[j];
         float v = Elem<T>::to_f32(val[j]);
@@ -629,7 +862,7 @@ __global__ __launch_bounds__(256) void k_decode_generic(
           if (foff) v = Elem<T>::round(v + Elem<T>::to_f32(foff[t * F + f]));
           if (fscale) v = Elem<T>::round(v * Elem<T>::to_f32(fscale[t * F + f]));
         }
-        if (o < d) acc = fmaf(v, Elem<T>::to_f32(wbase[(int64_t)f * d + o]), acc);
+        if (o < d) acc = fmaf(v, Elem<T>::to_f32(wbase[(int64_t)f * pitch + o]), acc);
       }
     }
     if (o < d) {
@@ -644,7 +877,7 @@ __global__ __launch_bounds__(256) void k_decode_generic(
 // [d][F] -> [F][d] through a 64x64 LDS tile (coalesced on both sides).
 template <typename T>
 __global__ __launch_bounds__(256) void k_pack(const T *src, T *dst, int64_t d, int64_t F,
-                                              int64_t in_stride, int64_t out_stride) {
+                                              int64_t in_stride, int64_t out_stride, int64_t pitch) {
   __shared__ T tile[64][65];
   const T *s = src + (int64_t)blockIdx.z * in_stride;
   T *o = dst + (int64_t)blockIdx.z * out_stride;
@@ -657,7 +890,7 @@ __global__ __launch_bounds__(256) void k_pack(const T *src, T *dst, int64_t d, i
   __syncthreads();
   for (int i = ty; i < 64; i += 4) {
     int64_t ff = f0 + i, dd = d0 + tx;
-    if (ff < F && dd < d) o[ff * d + dd] = tile[tx][i];
+    if (ff < F && dd < d) o[ff * pitch + dd] = tile[tx][i];
   }
 }
 
@@ -688,7 +921,7 @@ __global__ void k_zero_rows(OT *out, int64_t Tn, int64_t F, int64_t L, int64_t o
 
 // norms[s][f]: one wavefront per (s, f), summing over the decoders fed by s.
 template <typename T>
-__global__ __launch_bounds__(256) void k_norms(const T *wp, T *norms, int64_t d, int64_t F, int64_t L, int tying) {
+__global__ __launch_bounds__(256) void k_norms(const T *wp, T *norms, int64_t d, int64_t F, int64_t L, int tying, int64_t pitch) {
   const int lane = lane_id(), wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
   const int64_t total = L * F;
   for (int64_t i = (int64_t)blockIdx.x * nwv + wv; i < total; i += (int64_t)gridDim.x * nwv) {
@@ -696,7 +929,7 @@ __global__ __launch_bounds__(256) void k_norms(const T *wp, T *norms, int64_t d,
     float acc = 0.0f;
     const int64_t t0 = s, t1 = tying == CLT_TYING_PER_SOURCE ? s + 1 : L;
     for (int64_t t = t0; t < t1; ++t) {
-      const T *row = wp + (decoder_slot(tying, s, t, L) * F + f) * d;
+      const T *row = wp + (decoder_slot(tying, s, t, L) * F + f) * pitch;
       float part = 0.0f;
       for (int64_t o = lane; o < d; o += 64) { float w = Elem<T>::to_f32(row[o]); part = fmaf(w, w, part); }
 #pragma unroll
@@ -743,6 +976,16 @@ static size_t decode_ws_bytes(int64_t Tn, int64_t d, int64_t L) {
   return part + sp;
 }
 
+// feature slices of the line schedule: F x 128 bytes per slice must stay inside an L2
+static int line_slices(int64_t F) { return (int)clt_ceil_div(F * 128, LINE_L2_BYTES); }
+// The quarter schedule keeps F / QUARTER_SLICES rows x a quarter of the columns per XCD: it is taken while
+// that stays near one 4 MiB L2 (measured: 4.7 MiB at F = 24576, d = 768 bf16 is still 2 % ahead of the line
+// schedule, 8.4 MiB at F = 32768, d = 1024 is 25 % behind it)
+constexpr int64_t QUARTER_L2_BYTES = 5 << 20;
+static bool quarter_fits(int64_t F, int64_t d, int elem_bytes) {
+  return (F / QUARTER_SLICES) * (d / QUARTER_PARTS) * elem_bytes <= QUARTER_L2_BYTES;
+}
+
 static bool quarter_shape_ok(int64_t d, int elem_bytes) {
   const int V = 16 / elem_bytes;
   const int per_lane = (int)(d / 64), hq = per_lane / V;
@@ -758,10 +1001,14 @@ static int plan_route(int64_t d, int64_t F, int tying, int elem_bytes, bool ws_o
   const int64_t chunk = 64 * V, nf = d / chunk, rem = d % chunk;
   const bool can_slice = ws_ok && (d % 4 == 0) && F >= 64 * DEC_SLICES;
   const bool fast = (d % V == 0) && wp_ok && nf <= 4 && (nf > 0 || rem > 0);
+  if (fast && can_slice && tying != CLT_TYING_PER_TARGET && d % 256 == 0 && F >= 64 * QUARTER_SLICES &&
+      quarter_shape_ok(d, elem_bytes) && quarter_fits(F, d, elem_bytes))
+    return CLT_ROUTE_QUARTER;
+  // the line schedule takes any width that is a whole number of cache lines
+  if (can_slice && wp_ok && tying != CLT_TYING_PER_TARGET && (d * elem_bytes) % 128 == 0 && line_slices(F) <= DEC_SLICES)
+    return CLT_ROUTE_LINE;
   if (!fast) return CLT_ROUTE_GENERIC;
   if (!can_slice) return CLT_ROUTE_SINGLE;
-  if (tying != CLT_TYING_PER_TARGET && d % 256 == 0 && F >= 64 * QUARTER_SLICES && quarter_shape_ok(d, elem_bytes))
-    return CLT_ROUTE_QUARTER;
   return tying == CLT_TYING_PER_TARGET ? CLT_ROUTE_SLICED_ALL_SOURCES : CLT_ROUTE_SLICED;
 }
 
@@ -773,6 +1020,7 @@ static int launch_decode(const int32_t *row_ptr, const int32_t *col, const void 
                          hipStream_t stream) {
   constexpr int V = WVec<T>::V;
   const int nwv = 4;
+  const int64_t pitch = clt_pitch(d, (int)sizeof(T));
   const int64_t blocks_per_t = clt_ceil_div(Tn, nwv);
   const bool can_slice = workspace && workspace_bytes >= decode_ws_bytes(Tn, d, L) && (d % 4 == 0) &&
                          F >= 64 * DEC_SLICES && ((((uintptr_t)workspace) & 255u) == 0);
@@ -789,11 +1037,13 @@ static int launch_decode(const int32_t *row_ptr, const int32_t *col, const void 
   const int64_t chunk = 64 * V;
   const int64_t nf = d / chunk, rem = d % chunk;
   const bool fast = (d % V == 0) && clt_aligned16(wp) && nf <= 4 && (nf > 0 || rem > 0);
-  if (can_slice && !fast) return launch_decode<T>(row_ptr, col, val, wp, bias_sum, foff, fscale, skip_add, out, Tn, d, F,
-                                                  L, tying, t_begin, t_end, src_mask, out_f32, nullptr, 0, stream);
+  const int route = plan_route(d, F, tying, (int)sizeof(T), can_slice, clt_aligned16(wp));
+  if (can_slice && !fast && route != CLT_ROUTE_LINE)
+    return launch_decode<T>(row_ptr, col, val, wp, bias_sum, foff, fscale, skip_add, out, Tn, d, F,
+                            L, tying, t_begin, t_end, src_mask, out_f32, nullptr, 0, stream);
 #define CLT_DEC_ARGS(FO, FS)                                                                                    \
   row_ptr, col, (const T *)val, (const T *)wp, bias_sum, FO, FS, skip_add, out, Tn, d, F, L, tying, tb,         \
-      t_end, src_mask, out_f32, sptr, partial, ns, src
+      t_end, src_mask, out_f32, sptr, partial, ns, src, pitch
 #define CLT_DEC(NFN, TL, UN)                                                                                    \
   do {                                                                                                          \
     if (affine && can_slice)                                                                                    \
@@ -812,27 +1062,56 @@ static int launch_decode(const int32_t *row_ptr, const int32_t *col, const void 
     else CLT_DEC(NFN, 2, UN);                              \
   } while (0)
   // quarter-row schedule: 2 feature slices x 4 column quarters (see k_decode_quarter)
-  bool quartered = false;
-  const int route = plan_route(d, F, tying, (int)sizeof(T), can_slice, clt_aligned16(wp));
+  bool quartered = false; int quarter_ns = QUARTER_SLICES;
+  if (route == CLT_ROUTE_LINE) {
+    constexpr int ntok = 2;                               // tokens per wavefront
+    const UnitPlan lp = make_unit_plan(line_slices(F), (int)(d * (int64_t)sizeof(T) / 128), Tn, nwv * ntok);
+    // one 32-bit word per survivor and 32-bit row offsets: feature index below 2^16, matrix below 4 GiB
+    const bool pack = sizeof(T) == 2 && F <= 65536 && F * pitch * (int64_t)sizeof(T) < (1ll << 32);
+    k_slice_ptr<<<1024, 256, 0, stream>>>(row_ptr, col, L * Tn, F, lp.ns, sptr);
+    for (int src = 0; src < (int)t_end; ++src) {
+      if (!((src_mask >> src) & 1ull)) continue;
+      const int64_t tb = src > t_begin ? src : t_begin;
+      const int64_t lb = 8 * (int64_t)lp.bpx * (t_end - tb);
+      if (lb <= 0) continue;
+      if (lb > 2147483647LL) return CLT_ERR_RANGE;
+#define CLT_DECL(AF, PK, NT)                                                                                          \
+  k_decode_line<T, AF, PK, NT><<<(unsigned)lb, 256, 0, stream>>>(col, (const T *)val, (const T *)wp, (const T *)foff, \
+      (const T *)fscale, Tn, d, F, L, tying, tb, src_mask, sptr, partial, src, lp, pitch)
+#define CLT_DECL2(AF, PK) CLT_DECL(AF, PK, ntok)
+      if (affine) { if (pack) CLT_DECL2(true, true); else CLT_DECL2(true, false); }
+      else { if (pack) CLT_DECL2(false, true); else CLT_DECL2(false, false); }
+#undef CLT_DECL2
+#undef CLT_DECL
+    }
+    k_decode_reduce<T><<<2048, 256, 0, stream>>>(partial, bias_sum, skip_add, out, Tn, d, L, t_begin, t_end, lp.ns, out_f32, src_mask);
+    return clt_check_launch();
+  }
   if (route == CLT_ROUTE_QUARTER) {
     const int per_lane = (int)(d / 64);                    // columns per lane
     const int hq = per_lane / V, htail = (per_lane % V) != 0;
-    const int64_t qblk_per_t = clt_ceil_div(Tn, nwv * QUARTER_NTOK);
+    // feature slices: F / qs rows x a quarter of the columns per XCD at a time, about one L2
+    const int qs = QUARTER_SLICES;
+    const UnitPlan up = make_unit_plan(qs, QUARTER_PARTS, Tn, nwv * QUARTER_NTOK);
+    // one 32-bit word per survivor and 32-bit row offsets: feature index below 2^16, matrix below 4 GiB
+    const bool qpack = sizeof(T) == 2 && F <= 65536 && F * pitch * (int64_t)sizeof(T) < (1ll << 32);
 #define CLT_DECQ(HQN, HTN, UN)                                                                                       \
   do {                                                                                                               \
-    k_slice_ptr<<<1024, 256, 0, stream>>>(row_ptr, col, L * Tn, F, QUARTER_SLICES, sptr);                            \
+    k_slice_ptr<<<1024, 256, 0, stream>>>(row_ptr, col, L * Tn, F, qs, sptr);                                        \
     for (int src = 0; src < (int)t_end; ++src) {                                                                     \
       if (!((src_mask >> src) & 1ull)) continue;                                                                     \
       const int64_t tb = src > t_begin ? src : t_begin;                                                              \
-      const int64_t qb = qblk_per_t * (t_end - tb) * 8;                                                              \
+      const int64_t qb = 8 * (int64_t)up.bpx * (t_end - tb);                                                         \
       if (qb <= 0) continue;                                                                                         \
       if (qb > 2147483647LL) return CLT_ERR_RANGE;                                                                   \
-      if (affine) k_decode_quarter<T, HQN, HTN, UN, true><<<(unsigned)qb, 256, 0, stream>>>(col, (const T *)val, (const T *)wp, \
-          (const T *)foff, (const T *)fscale, Tn, d, F, L, tying, tb, src_mask, sptr, partial, src);                 \
-      else k_decode_quarter<T, HQN, HTN, UN, false><<<(unsigned)qb, 256, 0, stream>>>(col, (const T *)val, (const T *)wp, \
-          nullptr, nullptr, Tn, d, F, L, tying, tb, src_mask, sptr, partial, src);                                   \
+      if (affine) k_decode_quarter<T, HQN, HTN, UN, true, false><<<(unsigned)qb, 256, 0, stream>>>(col, (const T *)val, (const T *)wp, \
+          (const T *)foff, (const T *)fscale, Tn, d, F, L, tying, tb, src_mask, sptr, partial, src, pitch, up);      \
+      else if (qpack) k_decode_quarter<T, HQN, HTN, UN, false, sizeof(T) == 2><<<(unsigned)qb, 256, 0, stream>>>(col, (const T *)val, (const T *)wp, \
+          nullptr, nullptr, Tn, d, F, L, tying, tb, src_mask, sptr, partial, src, pitch, up);                        \
+      else k_decode_quarter<T, HQN, HTN, UN, false, false><<<(unsigned)qb, 256, 0, stream>>>(col, (const T *)val, (const T *)wp, \
+          nullptr, nullptr, Tn, d, F, L, tying, tb, src_mask, sptr, partial, src, pitch, up);                        \
     }                                                                                                                \
-    quartered = true;                                                                                                \
+    quartered = true; quarter_ns = qs;                                                                               \
   } while (0)
     if constexpr (sizeof(T) == 2) {
       if (hq == 1 && !htail) CLT_DECQ(1, 0, 2);
@@ -847,7 +1126,7 @@ static int launch_decode(const int32_t *row_ptr, const int32_t *col, const void 
 #undef CLT_DECQ
   }
   if (quartered) {
-    k_decode_reduce<T><<<2048, 256, 0, stream>>>(partial, bias_sum, skip_add, out, Tn, d, L, t_begin, t_end, QUARTER_SLICES, out_f32, src_mask);
+    k_decode_reduce<T><<<2048, 256, 0, stream>>>(partial, bias_sum, skip_add, out, Tn, d, L, t_begin, t_end, quarter_ns, out_f32, src_mask);
     return clt_check_launch();
   }
   if (can_slice) k_slice_ptr<<<1024, 256, 0, stream>>>(row_ptr, col, L * Tn, F, ns, sptr);
@@ -879,7 +1158,7 @@ static int launch_decode(const int32_t *row_ptr, const int32_t *col, const void 
   } else {
     const int64_t tb = t_begin; const int src = 0; (void)tb; (void)src;
     k_decode_generic<T><<<(unsigned)nblk, 256, 0, stream>>>(row_ptr, col, (const T *)val, (const T *)wp, bias_sum,
-        (const T *)foff, (const T *)fscale, skip_add, out, Tn, d, F, L, tying, t_begin, t_end, src_mask, out_f32);
+        (const T *)foff, (const T *)fscale, skip_add, out, Tn, d, F, L, tying, t_begin, t_end, src_mask, out_f32, pitch);
   }
 #undef CLT_DEC_TAIL
 #undef CLT_DEC
@@ -923,8 +1202,8 @@ extern "C" int clt_pack_decoder(const void *w_ref, void *w_packed, int64_t d, in
   dim3 grid((unsigned)clt_ceil_div(F, 64), (unsigned)clt_ceil_div(d, 64), (unsigned)n_dec);
   if (clt_ceil_div(d, 64) > 65535) return CLT_ERR_RANGE;
   hipStream_t s = (hipStream_t)stream;
-  if (dtype == CLT_BF16) k_pack<bf16_t><<<grid, 256, 0, s>>>((const bf16_t *)w_ref, (bf16_t *)w_packed, d, F, in_stride, out_stride);
-  else k_pack<float><<<grid, 256, 0, s>>>((const float *)w_ref, (float *)w_packed, d, F, in_stride, out_stride);
+  if (dtype == CLT_BF16) k_pack<bf16_t><<<grid, 256, 0, s>>>((const bf16_t *)w_ref, (bf16_t *)w_packed, d, F, in_stride, out_stride, clt_pitch(d, 2));
+  else k_pack<float><<<grid, 256, 0, s>>>((const float *)w_ref, (float *)w_packed, d, F, in_stride, out_stride, clt_pitch(d, 4));
   return clt_check_launch();
 }
 
@@ -949,8 +1228,8 @@ extern "C" int clt_decoder_norms(const void *w_packed, void *norms, int64_t d, i
   if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
   if (d <= 0 || F <= 0 || L <= 0 || tying < 0 || tying > 2 || !w_packed || !norms) return CLT_ERR_ARG;
   hipStream_t s = (hipStream_t)stream;
-  if (dtype == CLT_BF16) k_norms<bf16_t><<<256 * 8, 256, 0, s>>>((const bf16_t *)w_packed, (bf16_t *)norms, d, F, L, tying);
-  else k_norms<float><<<256 * 8, 256, 0, s>>>((const float *)w_packed, (float *)norms, d, F, L, tying);
+  if (dtype == CLT_BF16) k_norms<bf16_t><<<256 * 8, 256, 0, s>>>((const bf16_t *)w_packed, (bf16_t *)norms, d, F, L, tying, clt_pitch(d, 2));
+  else k_norms<float><<<256 * 8, 256, 0, s>>>((const float *)w_packed, (float *)norms, d, F, L, tying, clt_pitch(d, 4));
   return clt_check_launch();
 }
 
@@ -961,12 +1240,18 @@ extern "C" int clt_decode_route(int64_t T, int64_t d, int64_t F, int64_t L, int 
   return plan_route(d, F, tying, dtype == CLT_BF16 ? 2 : 4, workspace_bytes >= decode_ws_bytes(T, d, L), true);
 }
 
-extern "C" int64_t clt_decoder_slab_elems(int64_t d, int64_t F, int64_t L, int tying) {
-  if (d <= 0 || F <= 0 || L <= 0 || tying < 0 || tying > 2) return -1;
+extern "C" int64_t clt_decoder_pitch(int64_t d, int dtype) {
+  if (d <= 0 || (dtype != CLT_F32 && dtype != CLT_BF16)) return -1;
+  return clt_pitch(d, dtype == CLT_BF16 ? 2 : 4);
+}
+
+extern "C" int64_t clt_decoder_slab_elems(int64_t d, int64_t F, int64_t L, int tying, int dtype) {
+  if (d <= 0 || F <= 0 || L <= 0 || tying < 0 || tying > 2 || (dtype != CLT_F32 && dtype != CLT_BF16)) return -1;
+  const int64_t pitch = clt_pitch(d, dtype == CLT_BF16 ? 2 : 4);
   const int64_t n_dec = tying == CLT_TYING_NONE ? L * (L + 1) / 2 : L;
   // the last element any schedule can touch: row F-1 of slot n_dec-1, formed like the kernels form it
-  const int64_t last = decoder_slot_host(tying, L - 1, L - 1, L) * F * d + (F - 1) * d + (d - 1);
-  return last + 1 == n_dec * F * d ? n_dec * F * d : -1;
+  const int64_t last = decoder_slot_host(tying, L - 1, L - 1, L) * F * pitch + (F - 1) * pitch + (d - 1);
+  return last + 1 == n_dec * F * pitch - (pitch - d) ? n_dec * F * pitch : -1;
 }
 
 extern "C" int clt_accumulate_dense(const int32_t *row_ptr, const int32_t *col, const void *val,

@@ -53,16 +53,17 @@ __global__ __launch_bounds__(256) void k_adam_decoder(T *w_ref, T *const *w_refs
                                                       int64_t d, int64_t F, AdamCoef c) {
   __shared__ T tile[64][65];
   // blockIdx.z: decoder of a batch (w_refs holds one parameter pointer per decoder; the other arrays are slabs)
-  if (w_refs) { w_ref = w_refs[blockIdx.z]; const int64_t o = (int64_t)blockIdx.z * F * d; w_packed += o; g += o; m += o; v += o; }
+  const int64_t pitch = clt_pitch(d, (int)sizeof(T));   // row pitch of the working copy; gradient and moments are dense
+  if (w_refs) { w_ref = w_refs[blockIdx.z]; const int64_t o = (int64_t)blockIdx.z * F * d; w_packed += (int64_t)blockIdx.z * F * pitch; g += o; m += o; v += o; }
   const int64_t f0 = (int64_t)blockIdx.x * 64, d0 = (int64_t)blockIdx.y * 64;
   const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
   for (int i = ty; i < 64; i += 4) {
     const int64_t f = f0 + i, dd = d0 + tx;
     if (f < F && dd < d) {
-      const int64_t at = f * d + dd;
+      const int64_t at = f * d + dd, wat = f * pitch + dd;
       float mi = m[at], vi = v[at];
-      const T np = Elem<T>::from_f32(adam_update(Elem<T>::to_f32(w_packed[at]), g[at], mi, vi, c));
-      m[at] = mi; v[at] = vi; w_packed[at] = np;
+      const T np = Elem<T>::from_f32(adam_update(Elem<T>::to_f32(w_packed[wat]), g[at], mi, vi, c));
+      m[at] = mi; v[at] = vi; w_packed[wat] = np;
       tile[i][tx] = np;
     }
   }
@@ -80,7 +81,8 @@ __global__ __launch_bounds__(256) void k_adam_decoder_vec(T *__restrict__ w_ref,
                                                           const float *__restrict__ g, float *__restrict__ m, float *__restrict__ v,
                                                           int64_t d, int64_t F, AdamCoef c) {
   __shared__ T tile[64][68];
-  if (w_refs) { w_ref = w_refs[blockIdx.z]; const int64_t o = (int64_t)blockIdx.z * F * d; w_packed += o; g += o; m += o; v += o; }
+  const int64_t pitch = clt_pitch(d, (int)sizeof(T));   // row pitch of the working copy; gradient and moments are dense
+  if (w_refs) { w_ref = w_refs[blockIdx.z]; const int64_t o = (int64_t)blockIdx.z * F * d; w_packed += (int64_t)blockIdx.z * F * pitch; g += o; m += o; v += o; }
   const int64_t f0 = (int64_t)blockIdx.x * 64, d0 = (int64_t)blockIdx.y * 64;
   const int q = threadIdx.x & 15, r = threadIdx.x >> 4;
 #pragma unroll
@@ -88,16 +90,16 @@ __global__ __launch_bounds__(256) void k_adam_decoder_vec(T *__restrict__ w_ref,
     const int fl = r + 16 * i;
     const int64_t f = f0 + fl, dd = d0 + q * 4;
     if (f < F && dd < d) {
-      const int64_t at = f * d + dd;
+      const int64_t at = f * d + dd, wat = f * pitch + dd;
       const float4 gv = *reinterpret_cast<const float4 *>(g + at);
       float4 mv = *reinterpret_cast<const float4 *>(m + at), vv = *reinterpret_cast<const float4 *>(v + at);
       float p[4];
       if constexpr (sizeof(T) == 2) {
-        const uint2 raw = *reinterpret_cast<const uint2 *>(w_packed + at);
+        const uint2 raw = *reinterpret_cast<const uint2 *>(w_packed + wat);
         p[0] = bf16_bits_to_f32(raw.x & 0xFFFFu); p[1] = bf16_bits_to_f32(raw.x >> 16);
         p[2] = bf16_bits_to_f32(raw.y & 0xFFFFu); p[3] = bf16_bits_to_f32(raw.y >> 16);
       } else {
-        const float4 raw = *reinterpret_cast<const float4 *>(w_packed + at);
+        const float4 raw = *reinterpret_cast<const float4 *>(w_packed + wat);
         p[0] = raw.x; p[1] = raw.y; p[2] = raw.z; p[3] = raw.w;
       }
       p[0] = adam_update(p[0], gv.x, mv.x, vv.x, c); p[1] = adam_update(p[1], gv.y, mv.y, vv.y, c);
@@ -108,9 +110,9 @@ __global__ __launch_bounds__(256) void k_adam_decoder_vec(T *__restrict__ w_ref,
 #pragma unroll
       for (int k = 0; k < 4; ++k) { np[k] = Elem<T>::from_f32(p[k]); tile[fl][q * 4 + k] = np[k]; }
       if constexpr (sizeof(T) == 2)
-        *reinterpret_cast<uint2 *>(w_packed + at) = make_uint2((uint32_t)np[0] | ((uint32_t)np[1] << 16), (uint32_t)np[2] | ((uint32_t)np[3] << 16));
+        *reinterpret_cast<uint2 *>(w_packed + wat) = make_uint2((uint32_t)np[0] | ((uint32_t)np[1] << 16), (uint32_t)np[2] | ((uint32_t)np[3] << 16));
       else
-        *reinterpret_cast<float4 *>(w_packed + at) = make_float4(np[0], np[1], np[2], np[3]);
+        *reinterpret_cast<float4 *>(w_packed + wat) = make_float4(np[0], np[1], np[2], np[3]);
     }
   }
   __syncthreads();

@@ -118,13 +118,14 @@ class Decoder(nn.Module):
         return [(i, i) for i in range(L)]
 
     def packed(self) -> torch.Tensor:
-        """[n_dec, F, d] feature-major slab; matrices whose parameter changed are repacked."""
+        """[n_dec, F, pitch] feature-major slab (``engine.decoder_pitch``); matrices whose parameter changed
+        are repacked."""
         decs = self._ordered()
         w0 = decs[0].weight
         F, d = self.config.num_features, self.config.d_model
         if (self._slab is None or self._slab.device != w0.device or self._slab.dtype != w0.dtype
                 or self._slab.shape[0] != len(decs)):
-            self._slab = torch.empty(len(decs), F, d, device=w0.device, dtype=w0.dtype)
+            self._slab = engine.alloc_packed(len(decs), F, d, w0.dtype, w0.device)
             self._slab_keys = [None] * len(decs)
             self.device, self.dtype = w0.device, w0.dtype
         for i, dec in enumerate(decs):
@@ -367,7 +368,8 @@ class Decoder(nn.Module):
         key = tuple((dec.weight.data_ptr(), dec.weight._version) for dec in decs)
         if self._cached_decoder_norms is not None and self._norm_key == key:
             return self._cached_decoder_norms
-        norms = engine.decoder_norms(self.packed(), self.config.num_layers, self.config.decoder_tying)
+        norms = engine.decoder_norms(self.packed(), self.config.num_layers, self.config.decoder_tying,
+                                     self.config.d_model)
         self._cached_decoder_norms = norms
         self._norm_key = key
         return norms

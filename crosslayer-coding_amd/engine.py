@@ -7,7 +7,7 @@ Layouts
     w_enc      [L, F, d]      encoder weights (nn.Linear layout)
     pre        [L, T, F]      pre-activations
     survivors  SurvivorList   rows r = layer * T + token; (col, val) sorted by col in a row
-    w_packed   [n_dec, F, d]  decoder weights, feature-major
+    w_packed   [n_dec, F, pitch]  decoder weights, feature-major; pitch = decoder_pitch(d, dtype) >= d
     out        [L, T, d]      reconstructions
 """
 
@@ -375,13 +375,14 @@ def mse_loss_grad(rec: torch.Tensor, target: torch.Tensor, ws: Optional[Workspac
 
 
 def decode_backward_values(surv: SurvivorList, w_packed: torch.Tensor, g: torch.Tensor, tying: str,
-                           src_mask: Optional[int] = None, ws: Optional[Workspace] = None) -> torch.Tensor:
+                           src_mask: Optional[int] = None, ws: Optional[Workspace] = None) -> torch.Tensor:  # noqa: E501
     """d loss / d (kept activation) for every survivor, fp32 [nnz] (the straight-through gate hands
     it to the pre-activation unchanged, activations.py:66-96)."""
     L, T, F = surv.L, surv.T, surv.F
-    d = w_packed.shape[2]
+    d = g.shape[2]
     assert g.shape == (L, T, d) and g.dtype == torch.float32 and g.is_contiguous()
     assert w_packed.dtype == surv.dtype and w_packed.is_contiguous()
+    assert tuple(w_packed.shape[1:]) == (F, decoder_pitch(d, surv.dtype))
     if src_mask is None:
         src_mask = (1 << L) - 1
     dval = torch.empty(max(surv.nnz, 1), dtype=torch.float32, device=g.device)
@@ -455,12 +456,24 @@ def jumprelu_theta_grad(pre: torch.Tensor, grad_out: torch.Tensor, theta: torch.
     nat.check(code, "clt_jumprelu_theta_grad")
 
 
+def decoder_pitch(d: int, dtype: torch.dtype) -> int:
+    """Row pitch (elements) of the feature-major decoder slab: d, plus one 128-byte line when a row is an
+    even number of lines (so that a column part of all rows spreads over every L2 channel)."""
+    return int(nat.load().clt_decoder_pitch(int(d), nat.dtype_code(dtype)))
+
+
+def alloc_packed(n_dec: int, F: int, d: int, dtype: torch.dtype, device) -> torch.Tensor:
+    """Zeroed slab [n_dec, F, pitch] for feature-major decoders; ``slab[i, :, :d]`` is matrix i."""
+    return torch.zeros((n_dec, F, decoder_pitch(d, dtype)), dtype=dtype, device=device)
+
+
 def pack_decoder(w_ref: torch.Tensor, out: torch.Tensor) -> None:
-    """[d, F] checkpoint layout -> [F, d] feature-major (one matrix)."""
+    """[d, F] checkpoint layout -> feature-major rows of one matrix of the slab, out [F, pitch]."""
     nat.require_device(w_ref, "pack_decoder")
     d, F = w_ref.shape
-    assert w_ref.is_contiguous() and out.shape == (F, d) and out.is_contiguous() and out.dtype == w_ref.dtype
-    code = nat.load().clt_pack_decoder(nat.ptr(w_ref), nat.ptr(out), d, F, 1, d * F, d * F,
+    pitch = decoder_pitch(d, w_ref.dtype)
+    assert w_ref.is_contiguous() and out.shape == (F, pitch) and out.is_contiguous() and out.dtype == w_ref.dtype
+    code = nat.load().clt_pack_decoder(nat.ptr(w_ref), nat.ptr(out), d, F, 1, d * F, F * pitch,
                                        nat.dtype_code(w_ref.dtype), _stream(w_ref))
     nat.check(code, "clt_pack_decoder")
 
@@ -484,7 +497,8 @@ def decode_sparse(surv: SurvivorList, w_packed: torch.Tensor, tying: str, d: int
     if out is None:
         out = torch.empty((L, T, d), dtype=odt, device=dev)
     assert out.shape == (L, T, d) and out.is_contiguous() and out.dtype == odt
-    assert w_packed.is_contiguous() and w_packed.dtype == surv.dtype and w_packed.shape[1:] == (F, d)
+    assert w_packed.is_contiguous() and w_packed.dtype == surv.dtype
+    assert tuple(w_packed.shape[1:]) == (F, decoder_pitch(d, surv.dtype))
     for a in (bias_sum, skip_add):
         assert a is None or (a.dtype == torch.float32 and a.is_contiguous())
     for a in (feat_offset, feat_scale):
@@ -492,7 +506,7 @@ def decode_sparse(surv: SurvivorList, w_packed: torch.Tensor, tying: str, d: int
     lib = nat.load()
     # the largest offset the kernels form, slot * F * d + f * d + column, is a 64-bit quantity (1.0e10
     # elements for 300 decoders of 32768 x 1024); it must lie inside the slab that was handed in
-    need = lib.clt_decoder_slab_elems(d, F, L, nat.TYING[tying])
+    need = lib.clt_decoder_slab_elems(d, F, L, nat.TYING[tying], nat.dtype_code(surv.dtype))
     if need < 0 or w_packed.numel() < need:
         raise nat.CLTNativeError(f"decode_sparse: packed decoders hold {w_packed.numel()} elements, the kernels index {need}")
     wbuf, wbytes = None, 0
@@ -549,10 +563,11 @@ def densify(surv: SurvivorList, out_f32: bool = False, out: Optional[torch.Tenso
     return out
 
 
-def decoder_norms(w_packed: torch.Tensor, L: int, tying: str) -> torch.Tensor:
+def decoder_norms(w_packed: torch.Tensor, L: int, tying: str, d: int) -> torch.Tensor:
     """[L, F] per-feature decoder norms in the model dtype (decoder.py:374-485)."""
     nat.require_device(w_packed, "decoder_norms")
-    _, F, d = w_packed.shape
+    F = w_packed.shape[1]
+    assert w_packed.is_contiguous() and w_packed.shape[2] == decoder_pitch(d, w_packed.dtype)
     out = torch.empty((L, F), dtype=w_packed.dtype, device=w_packed.device)
     code = nat.load().clt_decoder_norms(nat.ptr(w_packed), nat.ptr(out), d, F, L, nat.TYING[tying],
                                         nat.dtype_code(w_packed.dtype), _stream(w_packed))

@@ -76,7 +76,9 @@ class CLTAdam:
         assert all(b.is_contiguous() and b.numel() == bs[0].numel() and b.dtype == bs[0].dtype for b in bs)
         d, F = ws[0].shape
         assert packed.is_contiguous() and raw["dec_w"].is_contiguous() and raw["dec_w"].dtype == torch.float32
-        assert tuple(packed.shape) == (len(ws), F, d) == tuple(raw["dec_w"].shape)
+        from . import engine
+        assert tuple(raw["dec_w"].shape) == (len(ws), F, d)
+        assert tuple(packed.shape) == (len(ws), F, engine.decoder_pitch(d, ws[0].dtype))
         w_dev, w_host = self._pointer_table("w", ws)
         code = lib.clt_adam_step_decoders(nat.ptr(w_dev), ctypes.addressof(w_host), len(ws), nat.ptr(packed),
                                           nat.ptr(raw["dec_w"]), nat.ptr(m_w), nat.ptr(v_w), d, F, self.lr,

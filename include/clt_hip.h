@@ -261,8 +261,10 @@ int clt_encode_threshold_emit(int64_t T, int64_t F, int64_t L, int64_t density_p
 
 /*
  * Repack decoder weights from the checkpoint layout [d][F] (nn.Linear weight of
- * RowParallelLinear, clt/models/parallel.py:66-70) to feature-major [F][d], so a
- * feature's decoder vector is one contiguous run.  n_dec matrices, element strides.
+ * RowParallelLinear, clt/models/parallel.py:66-70) to feature-major [F][pitch] (pitch =
+ * clt_decoder_pitch(d, dtype); the padding columns are not written), so a feature's decoder vector is
+ * one contiguous run.  n_dec matrices; in_stride / out_stride are the element strides between matrices
+ * (out_stride = F * pitch for a slab).
  */
 int clt_pack_decoder(const void *w_ref, void *w_packed, int64_t d, int64_t F,
                      int64_t n_dec, int64_t in_stride, int64_t out_stride,
@@ -315,16 +317,25 @@ int clt_decode_sparse(const int32_t *row_ptr, const int32_t *col, const void *va
 #define CLT_ROUTE_SLICED 2             /* 8 feature slices, one launch per source layer */
 #define CLT_ROUTE_SLICED_ALL_SOURCES 3 /* 8 feature slices, decoders tied per target: one launch */
 #define CLT_ROUTE_QUARTER 4            /* 2 feature slices x 4 column quarters, one launch per source */
+#define CLT_ROUTE_LINE 5               /* column parts of one cache line, one launch per source */
 int clt_decode_route(int64_t T, int64_t d, int64_t F, int64_t L, int tying, int dtype,
                      size_t workspace_bytes);
 
 /*
- * Number of elements of the packed decoder slab that clt_decode_sparse (and the backward entry
- * points) may index: n_dec * F * d with n_dec = L(L+1)/2 untied, L tied - formed in 64 bits, as every
- * kernel forms slot * F * d + f * d (the Pythia-410m shape has 1.0e10 elements).  Callers check their
- * allocation against it.  Returns -1 on bad arguments.
+ * Layout of the packed (feature-major) decoder slab that every entry point taking `w_packed` assumes:
+ *   w_packed[slot][f][c],  0 <= c < d,  rows clt_decoder_pitch(d, dtype) elements apart,
+ *   matrices F * pitch elements apart.
+ * pitch = d, except that a row of a whole, EVEN number of 128-byte cache lines gets one line more
+ * (d + 64 in bf16, d + 32 in fp32): with an even line pitch one column part of all rows falls on a
+ * fraction of the 16 L2 channels, and the schedules of clt_decode_sparse that give each XCD one column
+ * part would use only that fraction of its L2.  clt_pack_decoder writes this layout.
+ * clt_decoder_slab_elems: the number of elements such a slab has, n_dec * F * pitch with n_dec =
+ * L(L+1)/2 untied and L tied, formed in 64 bits as every kernel forms slot * F * pitch + f * pitch + c
+ * (the Pythia-410m shape has 1.1e10 elements); callers check their allocation against it.  Both return
+ * -1 on bad arguments.
  */
-int64_t clt_decoder_slab_elems(int64_t d, int64_t F, int64_t L, int tying);
+int64_t clt_decoder_pitch(int64_t d, int dtype);
+int64_t clt_decoder_slab_elems(int64_t d, int64_t F, int64_t L, int tying, int dtype);
 
 /*
  * Running dense sum of activations over source layers, the operand of a decoder tied per target
@@ -381,7 +392,7 @@ int clt_decoder_norms(const void *w_packed, void *norms, int64_t d, int64_t F,
  *   list_tok [nnz] token of each entry, list_src [nnz] its position in col / val.  Lists of up to
  *   64 entries are in token order.  Pass list_tok = list_src = NULL to get the counts only.
  * clt_decoder_weight_grad: dw_packed[slot(s,t)][f][:] = sum over the list of (s, f) of
- *   val * g_model[t][token][:] (fp32 sums, feature-major like w_packed); with tied decoders the
+ *   val * g_model[t][token][:] (fp32 sums, feature-major, dense rows of d elements); with tied decoders the
  *   slot collects every pair that shares it (CLT_TYING_PER_SOURCE: all t >= s; CLT_TYING_PER_TARGET:
  *   all s <= t), so dw_packed has L matrices instead of L(L+1)/2.  One launch per target layer,
  *   in ascending order on `stream`.
@@ -416,10 +427,10 @@ int clt_encoder_weight_grad(const int32_t *list_ptr, const int32_t *list_tok, co
  * optimizer in clt/training/trainer.py:290-312).  `step` counts from 1.
  * clt_adam_step: param, grad, m, v share one layout (n elements).
  * clt_adam_step_decoder: one decoder matrix; w_ref is the parameter in the checkpoint layout
- *   [d][F], w_packed its feature-major working copy [F][d]; grad_packed, m, v are [F][d].  Both
+ *   [d][F], w_packed its feature-major working copy [F][pitch]; grad_packed, m, v are dense [F][d].  Both
  *   copies receive the same new values.
- * clt_adam_step_decoders: n_dec decoder matrices in one launch.  w_packed, grad_packed, m, v are
- *   [n_dec][F][d] slabs; the parameters are separate tensors (one per nn.Linear of the reference's
+ * clt_adam_step_decoders: n_dec decoder matrices in one launch.  w_packed is the [n_dec][F][pitch] slab,
+ *   grad_packed, m, v are [n_dec][F][d] slabs; the parameters are separate tensors (one per nn.Linear of the reference's
  *   Decoder.decoders, clt/models/decoder.py:57-99), given as a device array of pointers for the kernel and
  *   the same pointers in a host array for checking.
  * clt_adam_step_many: `count` small parameters of n elements each (the decoder biases), gradient and

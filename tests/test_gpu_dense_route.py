@@ -91,10 +91,15 @@ def test_dense_route_matches_the_oracle_and_the_gather_route(dev, dtype, affine)
 
 def test_route_query_names_the_schedules(dev):
     big = 12 * 4096
+    # GPT-2-small x32: a quarter of the columns of half the rows is 4.7 MiB, about one L2: quarter-row schedule
     assert engine.decode_route(4096, 768, 24576, 12, "none", torch.bfloat16) == nat.ROUTE_QUARTER
-    assert engine.decode_route(4096, 1024, 32768, 24, "none", torch.bfloat16) == nat.ROUTE_QUARTER
+    assert engine.decode_route(4096, 768, 24576, 12, "none", torch.float32) == nat.ROUTE_LINE      # 9.4 MiB in fp32
+    assert engine.decode_route(1024, 768, 6144, 12, "none", torch.float32) == nat.ROUTE_QUARTER
+    # Pythia-410m shape: the same piece would be 8.4 MiB: one cache line of columns per XCD instead
+    assert engine.decode_route(4096, 1024, 32768, 24, "none", torch.bfloat16) == nat.ROUTE_LINE
     assert engine.decode_route(8192, 2048, 16384, 16, "per_target", torch.bfloat16) == nat.ROUTE_SLICED_ALL_SOURCES
-    assert engine.decode_route(4096, 640, 24576, 12, "per_source", torch.bfloat16) == nat.ROUTE_SLICED
-    assert engine.decode_route(4096, 768, 24576, 12, "none", torch.float32) == nat.ROUTE_QUARTER
+    assert engine.decode_route(4096, 640, 24576, 12, "per_source", torch.bfloat16) == nat.ROUTE_LINE
+    assert engine.decode_route(4096, 4096, 24576, 12, "none", torch.bfloat16) == nat.ROUTE_LINE     # wider than a wavefront's registers hold
+    assert engine.decode_route(4096, 200, 24576, 12, "per_source", torch.bfloat16) == nat.ROUTE_SLICED
     assert engine.decode_route(16, 768, 24576, 12, "none", torch.bfloat16, rows=16) == nat.ROUTE_SINGLE
     assert engine.decode_route(4096, 100, 24576, 12, "none", torch.bfloat16, rows=big) == nat.ROUTE_GENERIC

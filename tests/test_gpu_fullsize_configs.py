@@ -32,9 +32,11 @@ def test_c2_jumprelu_forward_at_full_size(dev):
     model.eval()
     dec = model.decoder_module
     # the packed decoders: 300 * 32768 * 1024 = 1.0e10 elements, past 32-bit offsets
-    n_elems = nat.load().clt_decoder_slab_elems(d, F, L, nat.TYING["none"])
-    assert n_elems == 300 * F * d > 2 ** 32 and dec.packed().numel() == n_elems
-    assert engine.decode_route(T, d, F, L, "none", torch.bfloat16) == nat.ROUTE_QUARTER
+    n_elems = nat.load().clt_decoder_slab_elems(d, F, L, nat.TYING["none"], nat.CLT_BF16)
+    pitch = engine.decoder_pitch(d, torch.bfloat16)
+    assert pitch == d + 64                              # 16 cache lines per row: padded to 17
+    assert n_elems == 300 * F * pitch > 2 ** 32 and dec.packed().numel() == n_elems
+    assert engine.decode_route(T, d, F, L, "none", torch.bfloat16) == nat.ROUTE_LINE
 
     # thresholds in the encoder epilogue == dense pre-activations + threshold pass, bit for bit
     _, x, w, b = model.encoder_module.prepare_slab(inputs)
@@ -240,6 +242,6 @@ def test_c4_training_step_at_full_size_in_bf16(dev):
         moved = (got.float() != before[key]).float().mean()
         assert float(moved) > 0.0                                     # the step did change bf16 values
     # the feature-major working copy of the decoder follows its parameter
-    assert torch.equal(model.decoder_module.packed()[slot], after["dec"].t())
+    assert torch.equal(model.decoder_module.packed()[slot][:, :d], after["dec"].t())
     del model, inputs, raw, opt
     _free()

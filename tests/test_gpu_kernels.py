@@ -461,9 +461,15 @@ def test_jumprelu_reference_known_answer(dev):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_pack_is_transpose(dev, dtype):
     w = torch.randn(70, 130).to(dtype)
-    out = torch.empty(130, 70, dtype=dtype, device=dev)
+    out = engine.alloc_packed(1, 130, 70, dtype, dev)[0]
     engine.pack_decoder(w.to(dev), out)
-    assert torch.equal(out.cpu(), w.T.contiguous())
+    assert torch.equal(out.cpu()[:, :70], w.T.contiguous())
+    # a row of whole, evenly many cache lines gets one more line of pitch; the matrix sits in the leading columns
+    w2 = torch.randn(128, 40).to(dtype)
+    out2 = engine.alloc_packed(1, 40, 128, dtype, dev)[0]
+    assert out2.shape[1] == 128 + 128 // w2.element_size()
+    engine.pack_decoder(w2.to(dev), out2)
+    assert torch.equal(out2.cpu()[:, :128], w2.T.contiguous()) and float(out2[:, 128:].abs().max()) == 0.0
 
 
 # ---- sparse decode -------------------------------------------------------------------------------
@@ -486,7 +492,7 @@ def test_decode_sparse_parity(dev, dtype, tying, L, T, d, F):
     off = torch.randn(L, F, generator=g).to(dtype) if tied else None
     sc = torch.randn(L, F, generator=g).to(dtype) if tied else None
     surv = engine.threshold_select(acts.to(dev), None, nat.PRED_NONZERO)
-    slab = torch.empty(len(names), F, d, dtype=dtype, device=dev)
+    slab = engine.alloc_packed(len(names), F, d, dtype, dev)
     for i, n in enumerate(names):
         engine.pack_decoder(w[n].to(dev), slab[i])
     B = torch.stack([b[n].float() for n in names])
@@ -520,11 +526,14 @@ def test_decode_sparse_parity(dev, dtype, tying, L, T, d, F):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("tying,d", [("none", 768), ("per_source", 768), ("none", 1024), ("none", 512), ("per_source", 2048),
-                                     ("none", 640), ("per_source", 320), ("per_target", 768)])
+                                     ("none", 640), ("per_source", 320), ("per_target", 768), ("none", 192),
+                                     ("per_source", 4096), ("none", 200)])
 def test_decode_sliced_matches_single_pass(dev, dtype, tying, d):
     # the XCD-sliced schedules (workspace given) against the one-wavefront-per-row kernel and the oracle:
-    # d a multiple of 256 takes the quarter-row kernel (2 feature slices x 4 column quarters) unless the
-    # decoders are tied per target; other widths and per-target tying take the 8-slice kernel
+    # d a multiple of 256 takes the quarter-row kernel (2 feature slices x 4 column quarters); other widths
+    # that are whole cache lines take the line kernel (640 and 320: 10 / 5 column parts in bf16, dealt to the
+    # XCDs in rounds with a remainder; 192: 3 parts, all XCDs share each; 4096: more columns than the
+    # whole-row kernels hold); per-target tying and the remaining widths take the 8-slice kernel
     g = torch.Generator().manual_seed(21)
     L, T, F = 3, 161, 1024
     names, w, b = make_decoder(L, d, F, tying, dtype, g)
@@ -532,7 +541,7 @@ def test_decode_sliced_matches_single_pass(dev, dtype, tying, d):
     acts[0, 5] = 0                                     # an empty row
     acts[1, 7, :] = torch.randn(F, generator=g).to(dtype)   # a full row (more than 64 per slice)
     surv = engine.threshold_select(acts.to(dev), None, nat.PRED_NONZERO)
-    slab = torch.empty(len(names), F, d, dtype=dtype, device=dev)
+    slab = engine.alloc_packed(len(names), F, d, dtype, dev)
     for i, n in enumerate(names):
         engine.pack_decoder(w[n].to(dev), slab[i])
     bias = torch.randn(L, d, generator=g)
@@ -556,13 +565,47 @@ def test_decode_sliced_matches_single_pass(dev, dtype, tying, d):
         assert orc.rel_l2(sliced[t], ref) <= TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_decode_line_schedule_with_feature_slices(dev, dtype):
+    # F x 128 bytes above 3.25 MiB: the line kernel cuts the feature axis in two and keeps two partial rows
+    g = torch.Generator().manual_seed(4)
+    L, T, F, d = 2, 300, 28672, 192
+    assert engine.decode_route(T, d, F, L, "none", dtype, rows=10 ** 6) == nat.ROUTE_LINE
+    names, w, b = make_decoder(L, d, F, "none", dtype, g)
+    acts = torch.zeros(L, T, F)
+    for l in range(L):
+        for t in range(T):
+            idx = torch.randint(0, F, (40,), generator=g)
+            acts[l, t, idx] = torch.randn(40, generator=g)
+    acts[1, 3] = 0
+    acts = acts.to(dtype)
+    surv = engine.threshold_select(acts.to(dev), None, nat.PRED_NONZERO)
+    slab = engine.alloc_packed(len(names), F, d, dtype, dev)
+    for i, n in enumerate(names):
+        engine.pack_decoder(w[n].to(dev), slab[i])
+    ws = engine.Workspace(dev)
+    old = engine.SLICED_DECODE_MIN_ROWS
+    try:
+        engine.SLICED_DECODE_MIN_ROWS = 1
+        sliced = engine.decode_sparse(surv, slab, "none", d, out_f32=True, ws=ws)
+    finally:
+        engine.SLICED_DECODE_MIN_ROWS = old
+    single = engine.decode_sparse(surv, slab, "none", d, out_f32=True)
+    assert orc.rel_l2(sliced, single) <= 1e-6
+    zero_b = {n: torch.zeros(d, dtype=dtype) for n in names}
+    for t in range(L):
+        ref = orc.decode({s: acts[s] for s in range(L)}, t, tying="none", weights=w, biases=zero_b, d_model=d,
+                         num_features=F, dtype=dtype).float()
+        assert orc.rel_l2(sliced[t].cpu(), ref) <= TOL[dtype]
+
+
 def test_decode_linearity_property(dev):
     # decode(2 * a) - bias == 2 * (decode(a) - bias), exact in fp32 for power-of-two scaling
     g = torch.Generator().manual_seed(2)
     L, T, d, F = 3, 64, 768, 512
     names, w, b = make_decoder(L, d, F, "none", torch.float32, g)
     acts = torch.randn(L, T, F, generator=g) * (torch.rand(L, T, F, generator=g) < 0.05)
-    slab = torch.empty(len(names), F, d, device=dev)
+    slab = engine.alloc_packed(len(names), F, d, torch.float32, dev)
     for i, n in enumerate(names):
         engine.pack_decoder(w[n].to(dev), slab[i])
     s1 = engine.threshold_select(acts.to(dev), None, nat.PRED_NONZERO)
@@ -578,10 +621,10 @@ def test_decoder_norms(dev, dtype, tying):
     g = torch.Generator().manual_seed(8)
     L, d, F = 3, 40, 50
     names, w, _ = make_decoder(L, d, F, tying, dtype, g)
-    slab = torch.empty(len(names), F, d, dtype=dtype, device=dev)
+    slab = engine.alloc_packed(len(names), F, d, dtype, dev)
     for i, n in enumerate(names):
         engine.pack_decoder(w[n].to(dev), slab[i])
-    got = engine.decoder_norms(slab, L, tying).cpu()
+    got = engine.decoder_norms(slab, L, tying, d).cpu()
     ref = orc.decoder_norms(w, L, F, tying, dtype)
     assert orc.rel_l2(got, ref) <= TOL[dtype]
 
