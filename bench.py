@@ -44,10 +44,49 @@ def algorithmic_work(wl, nnz_rows_pairs: int, nnz_total: int):
     }
 
 
-# HBM bytes per decode launch (FETCH_SIZE + WRITE_SIZE of `rocprofv3 --pmc`, each scaled by
-# what the same counter reads for the known-size copy at the end of this script), keyed by
-# (workload, launches per step).  Filled from the counter runs kept under profiles/.
-MEASURED_TRAFFIC = {("c1", 12): (1756599.0 + 152273.0) * 1024.0}
+def profiled_traffic(workload: str):
+    """({kernel name: (dispatches, HBM bytes per launch)}, forwards profiled) from the counter summary kept
+    under profiles/ for this workload: FETCH_SIZE and WRITE_SIZE of `rocprofv3 --pmc`, each scaled by what
+    the same counter reads for the known-size copy of ``--copy-probe``.  ({}, 0) when there is no such file:
+    the traffic figures are then left out rather than guessed."""
+    path = os.path.join(ROOT, "profiles", f"forward_{workload}_hbm_traffic.txt")
+    table, forwards = {}, 0
+    try:
+        for line in open(path):
+            if line.startswith("forwards profiled:"):
+                forwards = int(line.split(":")[1])
+            elif line.startswith("k_"):
+                f = line.split()
+                name = " ".join(f[:-6])
+                table[name] = (int(f[-6]), float(f[-1]) * 1e6)
+    except (OSError, ValueError, IndexError):
+        return {}, 0
+    return table, forwards
+
+
+def gather_yardstick(lib, dev, table_bytes: int, row_bytes: int, steps: int = 3):
+    """GB/s of a bare gather of ``row_bytes`` rows from a table of ``table_bytes`` (the piece of a decoder
+    matrix one XCD works on), best of four grid sizes: what the L2 -> CU path delivers to this access
+    pattern on the GPU at hand, with no survivor lists, partial rows or arithmetic around it."""
+    n_rows = max(1, table_bytes // row_bytes)
+    n_idx = 4_000_000 * 1536 // row_bytes
+    g = torch.Generator(device=dev).manual_seed(0)
+    table = torch.randint(0, 1 << 30, (n_rows * row_bytes // 4,), dtype=torch.int32, device=dev, generator=g)
+    idx = torch.randint(0, n_rows, (n_idx,), dtype=torch.int32, device=dev, generator=g)
+    stream = torch.cuda.current_stream().cuda_stream
+    best = 0.0
+    for blocks in (256 * 2, 256 * 4, 256 * 8, 256 * 16):
+        out = torch.empty(blocks * 256, dtype=torch.float32, device=dev)
+        if lib.clt_probe_gather(table.data_ptr(), n_rows, row_bytes, idx.data_ptr(), n_idx, blocks, 0, out.data_ptr(), stream):
+            return None
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(steps):
+            lib.clt_probe_gather(table.data_ptr(), n_rows, row_bytes, idx.data_ptr(), n_idx, blocks, 0, out.data_ptr(), stream)
+        b.record()
+        b.synchronize()
+        best = max(best, n_idx * row_bytes * steps / (a.elapsed_time(b) * 1e-3) / 1e9)
+    return best
 
 
 def copy_probe(dev):
@@ -148,16 +187,79 @@ def run_gpu(args):
     sel_gbs = work["select_bytes"] / (st["select"] * 1e-3) / 1e9
     dec_gbs = work["decode_gathered_bytes"] / (st["decode"] * 1e-3) / 1e9
     dec_c_gbs = work["decode_compulsory_bytes"] / (st["decode"] * 1e-3) / 1e9
-    # the decode of a large batch is one k_decode launch per source layer (plus one small
-    # slice-pointer kernel before and one reduce kernel after, timed with them); a small batch
-    # is a single launch
-    n_dec_launch = L if T * L >= engine.SLICED_DECODE_MIN_ROWS else 1
-    # widths that are a multiple of 256 take the quarter-row kernel unless the decoders are tied per target
-    quarter_rows = n_dec_launch > 1 and wl.d_model % 256 == 0 and wl.decoder_tying != "per_target"
-    dec_kernel_desc = (f"{'k_decode_quarter' if quarter_rows else 'k_decode'} (sparse cross-layer decode; {n_dec_launch} "
-                       "launch(es) per step; the per-launch figures are the step's decode stage divided by that count)")
-    traffic = MEASURED_TRAFFIC.get((wl.name, n_dec_launch))
+    # ---- the dominant kernel: the decode ----------------------------------------------------------------
+    nat = cca._native
+    e = 2 if wl.dtype == "bfloat16" else 4
+    F, d = wl.num_features, wl.d_model
     mfma_peak = MFMA_BF16_PEAK_TF if wl.dtype == "bfloat16" else MFMA_FP32_PEAK_TF
+    route = engine.decode_route(T, d, F, L, wl.decoder_tying, model.dtype)
+    dense_first, dense_end = dec.last_route.get("dense_targets", (L, L))
+    n_dense = dense_end - dense_first
+    table, forwards = profiled_traffic(wl.name)
+    if n_dense > 0:
+        # decoders tied per target: targets [dense_first, L) are dense products on the MFMA kernel
+        flop = 2.0 * T * F * d * n_dense
+        tf = flop / (st["decode"] * 1e-3) / 1e12
+        roofline = {
+            "kernel": (f"k_encode_mfma as the decoder product summed[T,F] @ W[t].T of targets {dense_first}..{dense_end - 1} "
+                       f"({n_dense} launches per step, with the scatter of the summed activations before each)"),
+            "bound": "mfma", "achieved": tf, "peak": mfma_peak, "unit": "TFLOP/s", "frac": tf / mfma_peak, "traffic": None,
+            "algorithmic_flop_per_launch": flop / n_dense, "avg_launch_ms": st["decode"] / n_dense,
+            "launches_per_step": n_dense,
+            "note": "achieved = 2 T F d per dense target / the whole decode stage (scatter kernels and any gathered targets included)",
+        }
+        decode_stage = {"ms": st["decode"], "bound": "mfma", "achieved": tf, "peak": mfma_peak, "unit": "TFLOP/s",
+                        "frac": tf / mfma_peak}
+    else:
+        sliced = route in (nat.ROUTE_QUARTER, nat.ROUTE_LINE, nat.ROUTE_SLICED)
+        n_dec_launch = L if sliced else 1
+        kname = {nat.ROUTE_QUARTER: "k_decode_quarter", nat.ROUTE_LINE: "k_decode_line"}.get(route, "k_decode")
+        # the piece of one decoder matrix that an XCD gathers from while the tokens stream past
+        if route == nat.ROUTE_QUARTER:
+            part_bytes = (F // 2) * (d // 4) * e
+        elif route == nat.ROUTE_LINE:
+            part_bytes = F * 128 // max(1, -(-F * 128 // 3407872))
+        elif route in (nat.ROUTE_SLICED, nat.ROUTE_SLICED_ALL_SOURCES):
+            part_bytes = (F // 8) * d * e
+        else:
+            part_bytes = F * d * e
+        row_bytes = min(d * e, 2048) // 16 * 16
+        yard = gather_yardstick(nat.load(), dev, part_bytes, row_bytes) if row_bytes >= 16 else None
+        per_launch_s = st["decode"] / n_dec_launch * 1e-3
+        hit = [v for k, v in table.items() if k.startswith(kname + "<")]
+        traffic = hit[0][1] if hit else None
+        comp = work["decode_compulsory_bytes"] / n_dec_launch
+        roofline = {
+            "kernel": (f"{kname} (sparse cross-layer decode; {n_dec_launch} launch(es) per step; the per-launch figures are "
+                       "the step's decode stage divided by that count)"),
+            "bound": "l2_gather (measured)",
+            "achieved": dec_gbs,
+            "peak": yard,
+            "unit": "GB/s",
+            "frac": (dec_gbs / yard) if yard else None,
+            "traffic": traffic,
+            "hbm": {"peak": HBM_PEAK_GBS, "compulsory_bytes_per_launch": comp, "compulsory_GBps": dec_c_gbs,
+                    "compulsory_frac": dec_c_gbs / HBM_PEAK_GBS,
+                    "traffic_GBps": (traffic / per_launch_s / 1e9) if traffic else None,
+                    "traffic_frac": (traffic / per_launch_s / 1e9 / HBM_PEAK_GBS) if traffic else None},
+            "note": ("achieved = gathered bytes (every active (token, feature, source->target) fetches one decoder row) per "
+                     "launch / launch time.  The rows come from the L2s, not from HBM, so the bound is what a bare gather of "
+                     f"{row_bytes}-byte rows reaches from a table the size of the piece an XCD works on ({part_bytes / 1e6:.1f} MB), "
+                     "measured in this run with clt_probe_gather (best of four grid sizes).  hbm: the same launch against the "
+                     "HBM peak, on the compulsory bytes (each decoder row once) and on the profiled traffic (FETCH_SIZE + "
+                     "WRITE_SIZE of the counter run kept under profiles/, null when there is none)"),
+            "algorithmic_bytes_per_launch": work["decode_gathered_bytes"] / n_dec_launch,
+            "avg_launch_ms": st["decode"] / n_dec_launch,
+            "launches_per_step": n_dec_launch,
+        }
+        decode_stage = {"ms": st["decode"], "bound": "l2_gather (measured)", "achieved": dec_gbs, "peak": yard,
+                        "unit": "GB/s", "frac": (dec_gbs / yard) if yard else None,
+                        "compulsory_GBps": dec_c_gbs, "compulsory_frac": dec_c_gbs / HBM_PEAK_GBS}
+    # what the selection stage really moves, from the same counter run (it never reads the ranking values in the
+    # fused path: they are compared in the encoder epilogue)
+    sel_kernels = ("k_tile_emit", "k_tile_count", "k_pool_hist", "k_row_prefix", "k_select_allot", "k_select_scan",
+                   "k_select_pass", "k_select_emit", "k_select_count", "k_select_level", "k_rowptr_scan")
+    sel_real = sum(n * b for k, (n, b) in table.items() if k.split("<")[0] in sel_kernels) / forwards if forwards else None
     result = {
         "metric": "CLT forward tokens/sec at GPT-2-small x32 BatchTopK k=200; % of roofline per stage",
         "value": T * args.steps / wall,
@@ -180,22 +282,7 @@ def run_gpu(args):
                               "fused (thresholds applied in the encoder epilogue; the select stage is empty)"
                               if fused_thr else "separate kernels"),
         },
-        "roofline": {
-            "kernel": dec_kernel_desc,
-            "bound": "hbm",
-            "achieved": dec_gbs,
-            "peak": HBM_PEAK_GBS,
-            "unit": "GB/s",
-            "frac": dec_gbs / HBM_PEAK_GBS,
-            "traffic": traffic,
-            "traffic_GBps": (traffic / (st["decode"] / n_dec_launch * 1e-3) / 1e9) if traffic else None,
-            "note": ("achieved = gathered bytes (every active (token, feature, source->target) fetches one decoder row) per "
-                     "launch / launch time; it exceeds the HBM peak because most rows are served by the L2s; traffic = "
-                     "HBM bytes per launch from FETCH_SIZE + WRITE_SIZE"),
-            "algorithmic_bytes_per_launch": work["decode_gathered_bytes"] / n_dec_launch,
-            "avg_launch_ms": st["decode"] / n_dec_launch,
-            "launches_per_step": n_dec_launch,
-        },
+        "roofline": roofline,
         "stages": {
             "encoder": {"ms": st["encode"], "bound": "mfma", "achieved": enc_tf, "peak": mfma_peak,
                         "unit": "TFLOP/s", "frac": enc_tf / mfma_peak,
@@ -203,14 +290,16 @@ def run_gpu(args):
                                  if fused else "projection only")},
             "select": {"ms": st["select"], "bound": "hbm", "achieved": None if fused_thr else sel_gbs,
                        "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": None if fused_thr else sel_gbs / HBM_PEAK_GBS,
-                       "note": ("algorithmic bytes = one read of the ranking values + the survivor write; in the fused "
-                                "path the ranking values are compared in the encoder epilogue and never reach HBM, so "
-                                "this stage only touches the candidates") if fused else
+                       "moved_bytes": sel_real,
+                       "moved_GBps": (sel_real / (st["select"] * 1e-3) / 1e9) if sel_real and st["select"] > 0 else None,
+                       "moved_frac": (sel_real / (st["select"] * 1e-3) / 1e9 / HBM_PEAK_GBS) if sel_real and st["select"] > 0 else None,
+                       "note": ("achieved / frac: algorithmic bytes = one read of the ranking values + the survivor write. "
+                                "In the fused path the ranking values are compared in the encoder epilogue and never reach "
+                                "HBM, so this stage only touches the candidates: moved_* are the HBM bytes its kernels "
+                                "really move (profiled counters, null without a counter run)") if fused else
                                "empty: the survivor list is written by the encoder stage" if fused_thr else
                                "separate streaming pass"},
-            "decode": {"ms": st["decode"], "bound": "hbm", "achieved": dec_gbs, "peak": HBM_PEAK_GBS,
-                       "unit": "GB/s", "frac": dec_gbs / HBM_PEAK_GBS,
-                       "compulsory_GBps": dec_c_gbs, "compulsory_frac": dec_c_gbs / HBM_PEAK_GBS},
+            "decode": decode_stage,
         },
     }
     if args.copy_probe:
