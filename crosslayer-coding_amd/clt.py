@@ -69,6 +69,9 @@ class CrossLayerTranscoder(BaseTranscoder):
         self.decoder_module = Decoder(config, process_group, self.device, self.dtype)
         self.theta_manager = ThetaManager(config, process_group, self.device, self.dtype)
         self._ws: Optional[Workspace] = None
+        # threshold activations: survivor-array size per (activation, layers, tokens) and totals on their way back
+        self._thr_key, self._thr_capacity, self._thr_elems = None, None, 0
+        self._thr_pending: List[tuple] = []
 
     # ---- small helpers ---------------------------------------------------------------
     def _resolve_dtype(self, dtype_input: Optional[Union[str, torch.dtype]]) -> torch.dtype:
@@ -341,30 +344,78 @@ class CrossLayerTranscoder(BaseTranscoder):
                     surv = engine.collect_select(engine.encode_collect(x_slab, w_slab, b_slab, k, pre_buf, ws))
                 self._record("batchtopk_activation", tm)
                 return layers, T, surv
-        if fn == "jumprelu" and self.fuse_encode_select:
-            # thresholds applied in the encoder epilogue; the pool is sized from the density seen last
-            theta = self.theta_manager.thresholds(self.dtype)
-            if layers != list(range(cfg.num_layers)):
-                theta = theta.index_select(0, torch.tensor(layers, device=theta.device)).contiguous()
-            surv = engine.encode_threshold(x_slab, w_slab, b_slab, theta, ws, self._density_ppm)
-            if surv is not None:
-                seen = int(1e6 * surv.nnz / max(1, n * T * cfg.num_features))
-                self._density_ppm = max(2000, 2 * seen)
-                return layers, T, surv
-            self._density_ppm = min(1000000, 4 * self._density_ppm)
+        if fn in ("jumprelu", "relu"):
+            return layers, T, self._threshold_survivors(fn, layers, T, x_slab, w_slab, b_slab, pre_buf, ws)
         pre = engine.encode(x_slab, w_slab, b_slab, out=pre_buf)
         if fn in ("batchtopk", "topk"):
             surv = self._select(pre)
-        elif fn == "jumprelu":
-            theta = self.theta_manager.thresholds(self.dtype)
-            if layers != list(range(cfg.num_layers)):
-                theta = theta.index_select(0, torch.tensor(layers, device=theta.device)).contiguous()
-            surv = engine.threshold_select(pre, theta, nat.PRED_GE_THETA, ws)
-        elif fn == "relu":
-            surv = engine.threshold_select(pre, None, nat.PRED_GT_ZERO, ws)
         else:
             return None
         return layers, T, surv
+
+    # ---- threshold activations: survivor arrays sized without a read-back ---------------------------
+    def _poll_threshold_runs(self) -> None:
+        """Look at the totals of earlier forwards whose copies have arrived (no waiting): a list that did
+        not fit drops the estimate, so the next forward measures again; a larger total raises it."""
+        keep = []
+        for host, ev, key in self._thr_pending:
+            if not ev.query():
+                keep.append((host, ev, key))
+                continue
+            total, status = int(host[0]), int(host[1])
+            if key != self._thr_key:
+                continue
+            if status != 0:
+                logger.error(
+                    f"Rank {self.rank}: a forward found more active features than its survivor arrays held "
+                    f"({self._thr_capacity} entries); that batch was decoded as if nothing fired. Measuring again.")
+                self._thr_capacity = None
+            elif self._thr_capacity is not None and 2 * total > self._thr_capacity:
+                self._thr_capacity = 2 * total + 4096
+                self._density_ppm = max(self._density_ppm, int(2e6 * total / max(1, self._thr_elems)))
+        self._thr_pending = keep
+
+    def _threshold_survivors(self, fn: str, layers: List[int], T: int, x_slab, w_slab, b_slab, pre_buf, ws) -> SurvivorList:
+        """JumpReLU / ReLU survivors.  The number of survivors depends on the data.  The first forward of a
+        shape reads it back once and sizes the arrays exactly; later forwards give col / val twice the
+        largest total seen, check on the device that the list fits (clt_survivors_fit) and read nothing
+        back, so the forward is a pure sequence of launches on the current stream."""
+        cfg = self.config
+        n, F = len(layers), cfg.num_features
+        key = (fn, tuple(layers), T, self.dtype)
+        if key != self._thr_key:
+            self._thr_key, self._thr_capacity, self._thr_pending = key, None, []
+        self._thr_elems = n * T * F
+        self._poll_threshold_runs()
+        theta = None
+        if fn == "jumprelu":
+            theta = self.theta_manager.thresholds(self.dtype)
+            if layers != list(range(cfg.num_layers)):
+                theta = theta.index_select(0, torch.tensor(layers, device=theta.device)).contiguous()
+        cap = self._thr_capacity
+        surv = None
+        if fn == "jumprelu" and self.fuse_encode_select:
+            # thresholds applied in the encoder epilogue; the pool is sized from the density seen so far
+            surv = engine.encode_threshold(x_slab, w_slab, b_slab, theta, ws, self._density_ppm, capacity=cap)
+            if surv is None and cap is None:
+                self._density_ppm = min(1000000, 4 * self._density_ppm)
+        if surv is None:
+            pre = engine.encode(x_slab, w_slab, b_slab, out=pre_buf)
+            surv = engine.threshold_select(pre, theta, nat.PRED_GE_THETA if fn == "jumprelu" else nat.PRED_GT_ZERO, ws,
+                                           capacity=cap)
+        if cap is None:
+            total = surv.nnz                       # the one read-back: first forward of this shape
+            self._thr_capacity = 2 * total + 4096
+            self._density_ppm = max(2000, int(2e6 * total / max(1, self._thr_elems)))
+        else:
+            # total and fit flag travel to pinned memory behind the kernels; a later forward looks at them
+            host = torch.empty(2, dtype=torch.int32, pin_memory=True)
+            host[0:1].copy_(surv.row_ptr[-1:], non_blocking=True)
+            host[1:2].copy_(surv.status, non_blocking=True)
+            ev = torch.cuda.Event()
+            ev.record()
+            self._thr_pending.append((host, ev, key))
+        return surv
 
     def _expand_layers(self, layers: List[int], surv: SurvivorList) -> SurvivorList:
         """Re-index a list over the present layers to all num_layers (absent layers: empty rows)."""

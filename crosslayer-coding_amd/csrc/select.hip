@@ -1026,7 +1026,8 @@ __global__ void k_thresh_finish(const SelState *st, int L, int32_t *row_ptr, int
 template <typename T>
 __global__ __launch_bounds__(256) void k_tile_emit_all(
     int Tn, const uint2 *seg_meta, int nseg, const uint2 *pool, unsigned long long pool_cap, const uint32_t *pfx,
-    const int32_t *row_ptr, int32_t *col_out, T *val_out) {
+    const int32_t *row_ptr, int32_t *col_out, T *val_out, const int32_t *skip) {
+  if (skip && *skip != 0) return;             // the list did not fit the caller's arrays: it was emptied
   const int l = blockIdx.z, seg = blockIdx.y;
   const uint2 *mypool = pool + (unsigned long long)l * pool_cap;
   const int row = blockIdx.x * 256 + threadIdx.x;
@@ -1057,7 +1058,8 @@ template <typename T, int PRED> __device__ __forceinline__ bool pred_keep(float 
 template <typename T, int V, int PRED, bool EMIT>
 __global__ __launch_bounds__(256) void k_threshold(
     const T *pre, int64_t Tn, int64_t F, int64_t L, int64_t lstride, const T *theta,
-    uint32_t *row_cnt, const int32_t *row_ptr, int32_t *col_out, T *val_out) {
+    uint32_t *row_cnt, const int32_t *row_ptr, int32_t *col_out, T *val_out, const int32_t *skip) {
+  if (EMIT && skip && *skip != 0) return;     // the list did not fit the caller's arrays: it was emptied
   const int l = blockIdx.y;
   const int lane = lane_id(), wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
   const T *th_row = PRED == CLT_PRED_GE_THETA ? theta + (int64_t)l * F : nullptr;
@@ -1368,17 +1370,17 @@ static int run_batchtopk_v(const T *pre, int64_t Tn, int64_t F, int64_t L, int64
 template <typename T, int V, int PRED>
 static int run_threshold(bool emit, const T *pre, int64_t Tn, int64_t F, int64_t L, int64_t lstride,
                          const T *theta, uint32_t *row_cnt, int32_t *row_ptr, int32_t *col, T *val,
-                         hipStream_t stream) {
+                         const int32_t *skip, hipStream_t stream) {
   int gx = (int)clt_ceil_div(Tn, 4);
   int maxgx = (int)clt_ceil_div(256 * 8, L);
   if (maxgx < 1) maxgx = 1;
   if (gx > maxgx) gx = maxgx;
   dim3 grid(gx, (unsigned)L);
   if (!emit) {
-    k_threshold<T, V, PRED, false><<<grid, 256, 0, stream>>>(pre, Tn, F, L, lstride, theta, row_cnt, nullptr, nullptr, nullptr);
+    k_threshold<T, V, PRED, false><<<grid, 256, 0, stream>>>(pre, Tn, F, L, lstride, theta, row_cnt, nullptr, nullptr, nullptr, nullptr);
     k_rowptr_scan<<<1, SCAN_THREADS, 0, stream>>>(row_cnt, L * Tn, row_ptr);
   } else {
-    k_threshold<T, V, PRED, true><<<grid, 256, 0, stream>>>(pre, Tn, F, L, lstride, theta, nullptr, row_ptr, col, val);
+    k_threshold<T, V, PRED, true><<<grid, 256, 0, stream>>>(pre, Tn, F, L, lstride, theta, nullptr, row_ptr, col, val, skip);
   }
   return clt_check_launch();
 }
@@ -1386,14 +1388,14 @@ static int run_threshold(bool emit, const T *pre, int64_t Tn, int64_t F, int64_t
 template <typename T>
 static int dispatch_threshold(bool emit, const void *pre, int64_t Tn, int64_t F, int64_t L, int64_t lstride,
                               const void *theta, int pred, uint32_t *row_cnt, int32_t *row_ptr,
-                              int32_t *col, void *val, hipStream_t stream) {
+                              int32_t *col, void *val, const int32_t *skip, hipStream_t stream) {
   constexpr int VV = Elem<T>::VEC;
   bool vec = (F % VV == 0) && clt_aligned16(pre) && ((lstride * (int64_t)sizeof(T)) % 16 == 0) &&
              (pred != CLT_PRED_GE_THETA || clt_aligned16(theta));
   const T *p = (const T *)pre; const T *th = (const T *)theta; T *v = (T *)val;
 #define CLT_TH(PR)                                                                                       \
-  return vec ? run_threshold<T, VV, PR>(emit, p, Tn, F, L, lstride, th, row_cnt, row_ptr, col, v, stream) \
-             : run_threshold<T, 1, PR>(emit, p, Tn, F, L, lstride, th, row_cnt, row_ptr, col, v, stream)
+  return vec ? run_threshold<T, VV, PR>(emit, p, Tn, F, L, lstride, th, row_cnt, row_ptr, col, v, skip, stream) \
+             : run_threshold<T, 1, PR>(emit, p, Tn, F, L, lstride, th, row_cnt, row_ptr, col, v, skip, stream)
   if (pred == CLT_PRED_GE_THETA) { CLT_TH(CLT_PRED_GE_THETA); }
   if (pred == CLT_PRED_GT_ZERO) { CLT_TH(CLT_PRED_GT_ZERO); }
   CLT_TH(CLT_PRED_NONZERO);
@@ -1613,8 +1615,8 @@ extern "C" int clt_encode_threshold_count(const void *x, const void *w, const vo
 }
 
 extern "C" int clt_encode_threshold_emit(int64_t T, int64_t F, int64_t L, int64_t density_ppm, int dtype,
-                                         const int32_t *row_ptr, int32_t *col, void *val, void *workspace,
-                                         size_t workspace_bytes, void *stream) {
+                                         const int32_t *row_ptr, int32_t *col, void *val, const int32_t *skip,
+                                         void *workspace, size_t workspace_bytes, void *stream) {
   if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
   if (T <= 0 || F <= 0 || L <= 0 || L > 65535 || !row_ptr || !col || !val || !workspace) return CLT_ERR_ARG;
   const ThreshLayout tl = thresh_layout(T, F, L, density_ppm, dtype);
@@ -1624,10 +1626,10 @@ extern "C" int clt_encode_threshold_emit(int64_t T, int64_t F, int64_t L, int64_
   dim3 grid((unsigned)clt_ceil_div(T, 256), (unsigned)tl.nseg, (unsigned)L);
   if (dtype == CLT_BF16)
     k_tile_emit_all<bf16_t><<<grid, 256, 0, s>>>((int)T, (const uint2 *)(ws + tl.off_meta), tl.nseg, (const uint2 *)(ws + tl.off_tpool),
-                                                  tl.tpool_cap, (const uint32_t *)(ws + tl.off_pfx), row_ptr, col, (bf16_t *)val);
+                                                  tl.tpool_cap, (const uint32_t *)(ws + tl.off_pfx), row_ptr, col, (bf16_t *)val, skip);
   else
     k_tile_emit_all<float><<<grid, 256, 0, s>>>((int)T, (const uint2 *)(ws + tl.off_meta), tl.nseg, (const uint2 *)(ws + tl.off_tpool),
-                                                 tl.tpool_cap, (const uint32_t *)(ws + tl.off_pfx), row_ptr, col, (float *)val);
+                                                 tl.tpool_cap, (const uint32_t *)(ws + tl.off_pfx), row_ptr, col, (float *)val, skip);
   return clt_check_launch();
 }
 
@@ -1732,8 +1734,28 @@ extern "C" int clt_threshold_count(const void *pre, int64_t T, int64_t F, int64_
   if (F >= 2147483648LL || R >= 2147483647LL) return CLT_ERR_RANGE;   // the survivor total must also stay below 2^31
   if (workspace_bytes < (size_t)R * 4) return CLT_ERR_WORKSPACE;
   uint32_t *cnt = (uint32_t *)workspace;
-  if (dtype == CLT_BF16) return dispatch_threshold<bf16_t>(false, pre, T, F, L, pre_layer_stride, theta, pred, cnt, row_ptr, nullptr, nullptr, s);
-  return dispatch_threshold<float>(false, pre, T, F, L, pre_layer_stride, theta, pred, cnt, row_ptr, nullptr, nullptr, s);
+  if (dtype == CLT_BF16) return dispatch_threshold<bf16_t>(false, pre, T, F, L, pre_layer_stride, theta, pred, cnt, row_ptr, nullptr, nullptr, nullptr, s);
+  return dispatch_threshold<float>(false, pre, T, F, L, pre_layer_stride, theta, pred, cnt, row_ptr, nullptr, nullptr, nullptr, s);
+}
+
+// ---- sizing col / val without reading the total back -------------------------------------------------
+__global__ void k_survivors_fit_flag(const int32_t *row_ptr, int64_t R, int64_t capacity, int32_t *status) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) {
+    const int32_t tot = row_ptr[R];
+    *status = (tot < 0 || (int64_t)tot > capacity) ? 1 : 0;
+  }
+}
+__global__ void k_survivors_fit_clear(int32_t *row_ptr, int64_t n, const int32_t *status) {
+  if (*status == 0) return;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) row_ptr[i] = 0;
+}
+
+extern "C" int clt_survivors_fit(int32_t *row_ptr, int64_t R, int64_t capacity, int32_t *status, void *stream) {
+  if (!row_ptr || !status || R < 0 || capacity < 0) return CLT_ERR_ARG;
+  hipStream_t s = (hipStream_t)stream;
+  k_survivors_fit_flag<<<1, 64, 0, s>>>(row_ptr, R, capacity, status);
+  k_survivors_fit_clear<<<256, 256, 0, s>>>(row_ptr, R + 1, status);
+  return clt_check_launch();
 }
 
 // ---- clt_threshold_count for callers that cannot allocate ---------------------------------------
@@ -1775,15 +1797,15 @@ extern "C" int clt_threshold_count_static(const void *pre, int64_t T, int64_t F,
 
 extern "C" int clt_threshold_emit(const void *pre, int64_t T, int64_t F, int64_t L, int64_t pre_layer_stride,
                                   const void *theta, int pred, int dtype, const int32_t *row_ptr, int32_t *col,
-                                  void *val, void *stream) {
+                                  void *val, const int32_t *skip, void *stream) {
   if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
   if (T < 0 || F < 0 || L <= 0 || L > 65535 || !row_ptr) return CLT_ERR_ARG;
   if (pred < 0 || pred > 2 || (pred == CLT_PRED_GE_THETA && !theta)) return CLT_ERR_ARG;
   if (T == 0 || F == 0) return CLT_OK;
   if (!pre || !col || !val) return CLT_ERR_ARG;
   hipStream_t s = (hipStream_t)stream;
-  if (dtype == CLT_BF16) return dispatch_threshold<bf16_t>(true, pre, T, F, L, pre_layer_stride, theta, pred, nullptr, (int32_t *)row_ptr, col, val, s);
-  return dispatch_threshold<float>(true, pre, T, F, L, pre_layer_stride, theta, pred, nullptr, (int32_t *)row_ptr, col, val, s);
+  if (dtype == CLT_BF16) return dispatch_threshold<bf16_t>(true, pre, T, F, L, pre_layer_stride, theta, pred, nullptr, (int32_t *)row_ptr, col, val, skip, s);
+  return dispatch_threshold<float>(true, pre, T, F, L, pre_layer_stride, theta, pred, nullptr, (int32_t *)row_ptr, col, val, skip, s);
 }
 
 extern "C" int clt_selected_min_accumulate(const int32_t *row_ptr, const int32_t *col, const void *val, const float *mean,

@@ -23,19 +23,31 @@ from . import _native as nat
 
 @dataclass
 class SurvivorList:
-    """Compact activations of L layers x T tokens (CSR by row = layer*T + token)."""
+    """Compact activations of L layers x T tokens (CSR by row = layer*T + token).
+
+    ``col`` / ``val`` may be longer than the list (sized from an estimate, see ``status``); every
+    kernel walks the rows through ``row_ptr``, so the tail is never read."""
 
     row_ptr: torch.Tensor  # int32 [L*T + 1]
-    col: torch.Tensor      # int32 [nnz]   feature index
-    val: torch.Tensor      # model dtype [nnz]   raw pre-activation
+    col: torch.Tensor      # int32 [capacity >= nnz]   feature index
+    val: torch.Tensor      # model dtype [capacity >= nnz]   raw pre-activation
     T: int
     F: int
     L: int
     dtype: torch.dtype
+    # int32 [1] on the device when col / val were sized without reading the total back: 1 = the list did
+    # not fit and was emptied (clt_survivors_fit); None = sized from the exact total
+    status: Optional[torch.Tensor] = None
 
     @property
     def nnz(self) -> int:
+        """Survivor total; reads one int back from the device (synchronises)."""
         return int(self.row_ptr[-1].item())
+
+    @property
+    def capacity(self) -> int:
+        """Entries col / val hold: what buffers indexed by survivor are sized from, without a read-back."""
+        return int(self.col.numel())
 
 
 class Workspace:
@@ -242,12 +254,23 @@ def tokentopk_select(pre: torch.Tensor, kk: int, global_mode: bool, ws: Optional
     return SurvivorList(row_ptr, col[:total], val[:total], T, F, L, pre.dtype)
 
 
+def _fit(row_ptr: torch.Tensor, capacity: int) -> torch.Tensor:
+    """Device-side check that the survivor total fits ``capacity`` (else the list is emptied): the int32
+    [1] status the emit call is gated on."""
+    status = torch.empty(1, dtype=torch.int32, device=row_ptr.device)
+    code = nat.load().clt_survivors_fit(nat.ptr(row_ptr), row_ptr.numel() - 1, int(capacity), nat.ptr(status),
+                                        nat.current_stream(row_ptr.device))
+    nat.check(code, "clt_survivors_fit")
+    return status
+
+
 def threshold_select(pre: torch.Tensor, theta: Optional[torch.Tensor], pred: int,
-                     ws: Optional[Workspace] = None) -> SurvivorList:
+                     ws: Optional[Workspace] = None, capacity: Optional[int] = None) -> SurvivorList:
     """JumpReLU (x >= theta), ReLU (x > 0) or non-zero compaction of pre [L, T, F].
 
-    Two kernels with one 4-byte read-back in between: the survivor total sizes col/val.
-    """
+    Two kernels.  ``capacity`` None: one 4-byte read-back in between sizes col / val exactly.  With a
+    ``capacity`` nothing is read back: col / val get that many entries and the returned ``status`` says
+    on the device whether the list fitted (if not, it is empty)."""
     L, T, F = _check_pre(pre)
     dev = pre.device
     lib = nat.load()
@@ -259,21 +282,27 @@ def threshold_select(pre: torch.Tensor, theta: Optional[torch.Tensor], pred: int
     code = lib.clt_threshold_count(nat.ptr(pre), T, F, L, pre.stride(0), nat.ptr(theta), pred, code_dt,
                                    nat.ptr(row_ptr), nat.ptr(wbuf), wbuf.numel(), _stream(pre))
     nat.check(code, "clt_threshold_count")
-    total = int(row_ptr[-1].item())
+    status = None
+    if capacity is None:
+        total = int(row_ptr[-1].item())
+    else:
+        total = int(capacity)
+        status = _fit(row_ptr, total)
     col = torch.empty(max(total, 1), dtype=torch.int32, device=dev)
     val = torch.empty(max(total, 1), dtype=pre.dtype, device=dev)
     code = lib.clt_threshold_emit(nat.ptr(pre), T, F, L, pre.stride(0), nat.ptr(theta), pred, code_dt,
-                                  nat.ptr(row_ptr), nat.ptr(col), nat.ptr(val), _stream(pre))
+                                  nat.ptr(row_ptr), nat.ptr(col), nat.ptr(val), nat.ptr(status), _stream(pre))
     nat.check(code, "clt_threshold_emit")
-    return SurvivorList(row_ptr, col[:total], val[:total], T, F, L, pre.dtype)
+    return SurvivorList(row_ptr, col[:total], val[:total], T, F, L, pre.dtype, status)
 
 
 def encode_threshold(x: torch.Tensor, w: torch.Tensor, b: Optional[torch.Tensor], theta: torch.Tensor,
-                     ws: Workspace, density_ppm: int = 20000) -> Optional[SurvivorList]:
+                     ws: Workspace, density_ppm: int = 20000, capacity: Optional[int] = None) -> Optional[SurvivorList]:
     """Encoder projection + JumpReLU (x >= theta) without dense pre-activations
-    (parallel.py:286 + theta.py:70-79).  Returns None when the shapes do not qualify or the
-    survivors exceeded what ``density_ppm`` provides for: the caller then runs ``encode`` and
-    ``threshold_select``."""
+    (parallel.py:286 + theta.py:70-79).  Returns None when the shapes do not qualify or (``capacity``
+    None) the survivors exceeded what ``density_ppm`` provides for: the caller then runs ``encode`` and
+    ``threshold_select``.  With a ``capacity`` nothing is read back from the device: col / val get that
+    many entries and ``status`` tells, on the device, whether pool and arrays were large enough."""
     nat.require_device(x, "encode_threshold")
     L, T, d = x.shape
     F = w.shape[1]
@@ -291,15 +320,20 @@ def encode_threshold(x: torch.Tensor, w: torch.Tensor, b: Optional[torch.Tensor]
     code = lib.clt_encode_threshold_count(nat.ptr(x), nat.ptr(w), nat.ptr(b), nat.ptr(theta), T, d, F, L, *strides,
                                           int(density_ppm), dt, nat.ptr(row_ptr), nat.ptr(wbuf), wbuf.numel(), _stream(x))
     nat.check(code, "clt_encode_threshold_count")
-    total = int(row_ptr[-1].item())
-    if total < 0:
-        return None
+    status = None
+    if capacity is None:
+        total = int(row_ptr[-1].item())
+        if total < 0:
+            return None
+    else:
+        total = int(capacity)
+        status = _fit(row_ptr, total)
     col = torch.empty(max(total, 1), dtype=torch.int32, device=x.device)
     val = torch.empty(max(total, 1), dtype=x.dtype, device=x.device)
     code = lib.clt_encode_threshold_emit(T, F, L, int(density_ppm), dt, nat.ptr(row_ptr), nat.ptr(col), nat.ptr(val),
-                                         nat.ptr(wbuf), wbuf.numel(), _stream(x))
+                                         nat.ptr(status), nat.ptr(wbuf), wbuf.numel(), _stream(x))
     nat.check(code, "clt_encode_threshold_emit")
-    return SurvivorList(row_ptr, col[:total], val[:total], T, F, L, x.dtype)
+    return SurvivorList(row_ptr, col[:total], val[:total], T, F, L, x.dtype, status)
 
 
 # ---- evaluation reductions ------------------------------------------------------------------------------
@@ -310,7 +344,7 @@ def survivor_metrics(surv: SurvivorList, fired_eps: float = 1e-6):
     dev = surv.row_ptr.device
     nonzero = torch.empty(surv.L, dtype=torch.int64, device=dev)
     fired = torch.empty((surv.L, surv.F), dtype=torch.int32, device=dev)
-    empty = surv.nnz == 0
+    empty = surv.capacity == 0
     code = nat.load().clt_survivor_metrics(nat.ptr(surv.row_ptr), None if empty else nat.ptr(surv.col),
                                            None if empty else nat.ptr(surv.val), surv.T, surv.F, surv.L,
                                            nat.dtype_code(surv.dtype), fired_eps, nat.ptr(nonzero), nat.ptr(fired),
@@ -385,14 +419,15 @@ def decode_backward_values(surv: SurvivorList, w_packed: torch.Tensor, g: torch.
     assert tuple(w_packed.shape[1:]) == (F, decoder_pitch(d, surv.dtype))
     if src_mask is None:
         src_mask = (1 << L) - 1
-    dval = torch.empty(max(surv.nnz, 1), dtype=torch.float32, device=g.device)
+    cap = surv.capacity          # survivor-indexed buffers are sized from the arrays, not from a read-back
+    dval = torch.empty(max(cap, 1), dtype=torch.float32, device=g.device)
     lib = nat.load()
-    wbuf = (ws or Workspace(g.device)).get("decode_backward", lib.clt_decode_backward_workspace_bytes(T, L, surv.nnz))
+    wbuf = (ws or Workspace(g.device)).get("decode_backward", lib.clt_decode_backward_workspace_bytes(T, L, cap))
     code = lib.clt_decode_backward_values(nat.ptr(surv.row_ptr), nat.ptr(surv.col), nat.ptr(w_packed), nat.ptr(g),
-                                          T, d, F, L, nat.TYING[tying], src_mask & ((1 << 64) - 1), surv.nnz,
+                                          T, d, F, L, nat.TYING[tying], src_mask & ((1 << 64) - 1), cap,
                                           nat.dtype_code(surv.dtype), nat.ptr(dval), nat.ptr(wbuf), wbuf.numel(), _stream(g))
     nat.check(code, "clt_decode_backward_values")
-    return dval[:surv.nnz]
+    return dval[:cap]
 
 
 def feature_lists(surv: SurvivorList, ws: Optional[Workspace] = None):
@@ -400,8 +435,8 @@ def feature_lists(surv: SurvivorList, ws: Optional[Workspace] = None):
     L, T, F = surv.L, surv.T, surv.F
     dev = surv.row_ptr.device
     ptr = torch.empty(L * F + 1, dtype=torch.int32, device=dev)
-    tok = torch.empty(max(surv.nnz, 1), dtype=torch.int32, device=dev)
-    src = torch.empty(max(surv.nnz, 1), dtype=torch.int32, device=dev)
+    tok = torch.empty(max(surv.capacity, 1), dtype=torch.int32, device=dev)
+    src = torch.empty(max(surv.capacity, 1), dtype=torch.int32, device=dev)
     lib = nat.load()
     wbuf = (ws or Workspace(dev)).get("feature_lists", lib.clt_feature_lists_workspace_bytes(F, L))
     code = lib.clt_feature_lists(nat.ptr(surv.row_ptr), nat.ptr(surv.col), T, F, L, nat.ptr(ptr), nat.ptr(tok),

@@ -210,7 +210,20 @@ int clt_threshold_count(const void *pre, int64_t T, int64_t F, int64_t L,
 int clt_threshold_emit(const void *pre, int64_t T, int64_t F, int64_t L,
                        int64_t pre_layer_stride, const void *theta, int pred,
                        int dtype, const int32_t *row_ptr, int32_t *col, void *val,
-                       void *stream);
+                       const int32_t *skip, void *stream);
+
+/*
+ * For callers that do not read the survivor total back between a count call and its emit call (no
+ * host synchronisation in the forward): col / val are sized from an estimate, `capacity` entries, and
+ * this check runs on the device in between.  If the total row_ptr[R] (R = L*T) is negative (the pool of
+ * clt_encode_threshold_count overflowed) or exceeds `capacity`, *status = 1 and the list is emptied
+ * (row_ptr := 0 everywhere, so every later kernel sees rows without survivors); otherwise *status = 0.
+ * The emit calls take `status` as their `skip` argument and write nothing when it is set (NULL: no
+ * check).  The caller looks at *status whenever it next touches the host anyway, and repeats the batch
+ * with a larger capacity if it was set.  No counterpart in the reference, where the dense mask has a
+ * fixed size.
+ */
+int clt_survivors_fit(int32_t *row_ptr, int64_t R, int64_t capacity, int32_t *status, void *stream);
 
 /*
  * clt_threshold_count for callers that cannot allocate device memory (code under HIP graph capture,
@@ -256,7 +269,7 @@ int clt_encode_threshold_count(const void *x, const void *w, const void *b, cons
                                int64_t density_ppm, int dtype, int32_t *row_ptr,
                                void *workspace, size_t workspace_bytes, void *stream);
 int clt_encode_threshold_emit(int64_t T, int64_t F, int64_t L, int64_t density_ppm, int dtype,
-                              const int32_t *row_ptr, int32_t *col, void *val,
+                              const int32_t *row_ptr, int32_t *col, void *val, const int32_t *skip,
                               void *workspace, size_t workspace_bytes, void *stream);
 
 /*

@@ -72,6 +72,13 @@ def test_c2_jumprelu_forward_at_full_size(dev):
     _, _, surv = res
     assert torch.equal(surv.row_ptr, fused.row_ptr) and torch.equal(surv.col, fused.col)
     recs = model(inputs)
+    # from the second forward of a shape on, nothing is read back from the device
+    torch.cuda.synchronize()
+    torch.cuda.set_sync_debug_mode("error")
+    try:
+        recs = model(inputs)
+    finally:
+        torch.cuda.set_sync_debug_mode("default")
     dense = engine.densify(surv)                         # [L, T, F] in the model dtype
     for t in (0, 12, L - 1):
         want = torch.zeros(T, d, dtype=torch.float32, device=dev)

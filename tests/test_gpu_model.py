@@ -223,3 +223,55 @@ def test_model_to_device_keeps_results(dev):
     ref, _ = oracle_forward(wl, sd, x)
     for t in recs:
         assert orc.rel_l2(recs[t], ref[t]) <= 1e-5
+
+
+@pytest.mark.parametrize("name", ["fused-topk-bf16", "fused-jump-bf16", "tiny-jump", "tiny-relu", "tiny-global", "tiny-per-target"])
+def test_forward_reads_nothing_back_from_the_device(dev, name):
+    # The forward is a sequence of launches on the current stream.  The survivor count of a threshold
+    # activation depends on the data: the first forward of a shape reads it back once to size the arrays,
+    # every later one sizes them from what was seen and checks the fit on the device.
+    wl = next(c for c in CASES if c.name == name)
+    model, sd, x = build(wl, dev)
+    inputs = {l: x[l].to(dev) for l in range(wl.num_layers)}
+    first = model(inputs)
+    torch.cuda.synchronize()
+    torch.cuda.set_sync_debug_mode("error")
+    try:
+        second = model(inputs)
+        third = model({l: (1.05 * v).to(v.dtype) for l, v in inputs.items()})      # other data, same shape
+    finally:
+        torch.cuda.set_sync_debug_mode("default")
+    torch.cuda.synchronize()
+    for t in first:
+        assert torch.equal(first[t], second[t])
+        assert torch.isfinite(third[t]).all()
+    if wl.activation_fn in ("jumprelu", "relu"):
+        model(inputs)                                   # polls the totals of the two forwards above
+        assert model._thr_capacity is not None and not model._thr_pending[:-1]
+
+
+def test_threshold_forward_recovers_when_the_survivors_outgrow_the_arrays(dev, caplog):
+    # a batch with many more active features than any seen before: its list does not fit, it is decoded as
+    # empty (bias only), the next forward reports it and measures again
+    wl = next(c for c in CASES if c.name == "fused-jump-bf16")
+    model, sd, x = build(wl, dev)
+    L = wl.num_layers
+    inputs = {l: x[l].to(dev) for l in range(L)}
+    want_small = {t: v.clone() for t, v in model(inputs).items()}
+    big = {l: (40.0 * v).to(v.dtype) for l, v in inputs.items()}        # scales every pre-activation: far more survivors
+    overflowed = model(big)
+    torch.cuda.synchronize()
+    bias_only = model.decoder_module.bias_sum((1 << L) - 1)
+    for t in range(L):
+        assert torch.equal(overflowed[t].float(), bias_only[t].to(overflowed[t].dtype).float().expand_as(overflowed[t]))
+    with caplog.at_level(logging.ERROR):
+        again = model(big)                                             # sees the flag, measures, sizes exactly
+    assert any("more active features than its survivor arrays held" in r.message for r in caplog.records)
+    torch.cuda.synchronize()
+    acts = model.get_feature_activations(big)
+    assert int((acts[0] != 0).sum()) > 4 * int((model.get_feature_activations(inputs)[0] != 0).sum())
+    ref = model.decoder_module.decode({l: acts[l] for l in range(L)}, L - 1)
+    assert orc.rel_l2(again[L - 1].float().cpu(), ref.float().cpu()) <= 1e-2
+    back = model(inputs)
+    for t in range(L):
+        assert torch.equal(back[t], want_small[t])
