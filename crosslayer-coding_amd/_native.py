@@ -62,12 +62,14 @@ _SIGNATURES = {
     "clt_accumulate_dense": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _int, _vp]),
     "clt_densify": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp]),
     "clt_mse_workspace_bytes": (_sz, [_i64, _i64, _i64]),
-    "clt_mse_loss_grad": (_int, [_vp, _vp, _i64, _i64, _i64, _int, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "clt_mse_loss_grad": (_int, [_vp, _vp, _i64, _i64, _i64, _int, _int, _vp, _vp, _f64, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "clt_decode_backward_workspace_bytes": (_sz, [_i64, _i64, _i64]),
-    "clt_decode_backward_values": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _u64, _i64, _int, _vp, _vp, _sz, _vp]),
+    "clt_decode_backward_values": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _u64, _i64, _int, _vp, _vp, _sz, _vp]),
+    "clt_feature_affine_grad": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _u64, _i64, _int, _vp, _vp, _vp, _sz, _vp]),
+    "clt_skip_weight_grad": (_int, [_vp, _vp, _vp, _i64, _i64, _int, _int, _vp]),
     "clt_feature_lists_workspace_bytes": (_sz, [_i64, _i64]),
     "clt_feature_lists": (_int, [_vp, _vp, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _sz, _vp]),
-    "clt_decoder_weight_grad": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp]),
+    "clt_decoder_weight_grad": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp]),
     "clt_encoder_weight_grad": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
     "clt_adam_step": (_int, [_vp, _vp, _vp, _vp, _i64, _f64, _f64, _f64, _f64, _i64, _int, _vp]),
     "clt_adam_step_decoder": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _f64, _f64, _f64, _f64, _i64, _int, _vp]),

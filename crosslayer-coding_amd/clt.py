@@ -162,15 +162,33 @@ class CrossLayerTranscoder(BaseTranscoder):
         logger.info(f"Rank {self.rank}: CLT model config updated by ThetaManager. New activation_fn='{self.config.activation_fn}'.")
 
     # ---- loss and gradients --------------------------------------------------------------------
-    def _loss_and_raw_gradients(self, inputs: Dict[int, torch.Tensor], targets: Dict[int, torch.Tensor]):
+    def _denorm_args(self, normalization_method, mean_tg, std_tg):
+        """(mode, mean [L, d], std [L, d], scale) of the de-normalisation the reference's LossManager applies
+        before the loss (losses.py:70-86): "mean_std" needs the target statistics of EVERY layer (the
+        reference skips a layer that has none; a mixture is not supported here and raises)."""
+        cfg = self.config
+        method = cfg.normalization_method if normalization_method is None else normalization_method
+        L, d = cfg.num_layers, cfg.d_model
+        if method == "mean_std":
+            have = [l for l in range(L) if mean_tg and std_tg and l in mean_tg and l in std_tg]
+            if not have:
+                return "none", None, None, 1.0          # no statistics given: the reference leaves the tensors alone
+            if len(have) != L:
+                raise ValueError("mean_std de-normalisation needs mean_tg / std_tg for every layer")
+            stack = lambda dct: torch.stack([dct[l].to(device=self.device, dtype=self.dtype).reshape(-1)[-d:]  # noqa: E731
+                                             for l in range(L)]).contiguous()
+            return "mean_std", stack(mean_tg), stack(std_tg), 1.0
+        if method == "sqrt_d_model":
+            return "sqrt_d_model", None, None, float(d) ** 0.5
+        return "none", None, None, 1.0
+
+    def _loss_and_raw_gradients(self, inputs: Dict[int, torch.Tensor], targets: Dict[int, torch.Tensor],
+                                normalization_method: Optional[str] = None, mean_tg=None, std_tg=None):
         """(per-layer losses [L] fp32, raw gradients): ``enc_w`` [L, F, d], ``enc_b`` [L, F],
         ``dec_w`` [n_dec, F, d] (feature-major, decoders in slot order: "s->t" pairs, or one per source /
         per target for tied decoders), ``dec_b`` [n_dec, d] (bias gradient of each decoder); all fp32."""
         cfg = self.config
         L, d, F = cfg.num_layers, cfg.d_model, cfg.num_features
-        if cfg.skip_connection or getattr(cfg, "enable_feature_offset", False) \
-                or getattr(cfg, "enable_feature_scale", False):
-            raise NotImplementedError("gradients are built for decoders without skip / feature affine terms")
         if sorted(inputs) != list(range(L)) or sorted(targets) != list(range(L)):
             raise ValueError("loss_and_gradients needs inputs and targets for every layer")
         res = self._survivors(inputs)
@@ -179,14 +197,30 @@ class CrossLayerTranscoder(BaseTranscoder):
         _, T, surv = res
         ws = self._workspace()
         mask = (1 << L) - 1
-        rec = self.decoder_module.decode_survivors(surv, mask, ws=ws)
+        dec = self.decoder_module
+        skip = dec.skip_all_targets(inputs, mask, T) if cfg.skip_connection else None
+        rec = dec.decode_survivors(surv, mask, skip_add=skip, ws=ws)
         tgt = torch.stack([targets[l].to(device=self.device, dtype=self.dtype).reshape(-1, d) for l in range(L)])
-        loss_l, g, g_model, bias_grad = engine.mse_loss_grad(rec, tgt.contiguous(), ws)
-        dval = engine.decode_backward_values(surv, self.decoder_module.packed(), g, cfg.decoder_tying, mask, ws)
+        mode, mean, std, scale = self._denorm_args(normalization_method, mean_tg, std_tg)
+        loss_l, g, g_model, bias_grad = engine.mse_loss_grad(rec, tgt.contiguous(), ws, mode, mean, std, scale)
+        off, sc = dec._affine()                     # per-target feature offset / scale of tied decoders, or None
+        if cfg.activation_fn == "jumprelu" and (off is not None or sc is not None):
+            raise NotImplementedError("the JumpReLU threshold gradient is not built for decoders with feature offset / scale")
+        dval = engine.decode_backward_values(surv, dec.packed(), g, cfg.decoder_tying, mask, ws, feat_scale=sc)
         lists = engine.feature_lists(surv, ws)
-        dw_dec = engine.decoder_weight_grad(lists, surv, g_model, cfg.decoder_tying)
+        d_off, d_sc = (engine.feature_affine_grad(lists, surv, ws, off, sc, mask) if (off is not None or sc is not None)
+                       else (None, None))
+        dw_dec = engine.decoder_weight_grad(lists, surv, g_model, cfg.decoder_tying, off, sc)
         _, x_slab, _, _ = self.encoder_module.prepare_slab(inputs)
-        dw_enc, db_enc = engine.encoder_weight_grad(lists, dval, x_slab.contiguous(), F)
+        x_slab = x_slab.contiguous()
+        dw_enc, db_enc = engine.encoder_weight_grad(lists, dval, x_slab, F)
+        d_skip = None
+        if dec.skip_weights is not None:
+            # rec[t] += x[s] @ W_skip[s->t].T (untied, every pair) or x[t] @ W_skip[t].T (tied): dW = g[t].T @ x
+            pairs = [(s_, t) for s_ in range(L) for t in range(s_, L)] if cfg.decoder_tying == "none" else [(t, t) for t in range(L)]
+            d_skip = torch.empty((len(pairs), d, d), dtype=torch.float32, device=g.device)
+            for i, (s_, t) in enumerate(pairs):
+                engine.skip_weight_grad(g[t], x_slab[s_], d_skip[i])
         theta_grad = None
         if cfg.activation_fn == "jumprelu" and self.theta_manager.log_threshold is not None:
             theta_grad = self._log_threshold_gradient(x_slab, g_model, ws)
@@ -198,7 +232,8 @@ class CrossLayerTranscoder(BaseTranscoder):
             dec_b = torch.flip(torch.cumsum(torch.flip(bias_grad, dims=[0]), dim=0), dims=[0])
         else:
             dec_b = bias_grad
-        return loss_l, {"enc_w": dw_enc, "enc_b": db_enc, "dec_w": dw_dec, "dec_b": dec_b.contiguous(), "theta": theta_grad}
+        return loss_l, {"enc_w": dw_enc, "enc_b": db_enc, "dec_w": dw_dec, "dec_b": dec_b.contiguous(), "theta": theta_grad,
+                        "skip": d_skip, "feat_offset": d_off, "feat_scale": d_sc}
 
     def _log_threshold_gradient(self, x_slab: torch.Tensor, g_model: torch.Tensor, ws) -> torch.Tensor:
         """fp32 [L, F] gradient of ``log_threshold`` (JumpReLU.backward, activations.py:196-199, through
@@ -230,14 +265,19 @@ class CrossLayerTranscoder(BaseTranscoder):
         return out * torch.exp(self.theta_manager.log_threshold.detach().float())
 
     @torch.no_grad()
-    def loss_and_gradients(self, inputs: Dict[int, torch.Tensor], targets: Dict[int, torch.Tensor]):
+    def loss_and_gradients(self, inputs: Dict[int, torch.Tensor], targets: Dict[int, torch.Tensor],
+                           normalization_method: Optional[str] = None, mean_tg=None, std_tg=None):
         """MSE reconstruction loss (sum over layers of the per-layer mean, losses.py:45-92) and the
         gradients torch autograd gives the reference for it, computed from the survivor list:
         returns (loss [fp32 scalar tensor], {state-dict key: fp32 gradient in the parameter's shape}).
-        Needs every layer present, equal token counts, a top-k or JumpReLU / ReLU activation,
-        no skip connections or feature affine terms; decoders untied or tied per source / per target."""
+        Like the reference's LossManager, the loss is measured on de-normalised tensors:
+        ``normalization_method`` (default: the config's) "mean_std" with the activation store's target
+        statistics ``mean_tg`` / ``std_tg`` ({layer: tensor [d_model]}), "sqrt_d_model", or "none".
+        Needs every layer present, equal token counts and a top-k or JumpReLU / ReLU activation; decoders
+        untied or tied per source / per target, with or without skip connections and the per-target feature
+        offset / scale (decoder.py:228-338)."""
         L = self.config.num_layers
-        loss_l, raw = self._loss_and_raw_gradients(inputs, targets)
+        loss_l, raw = self._loss_and_raw_gradients(inputs, targets, normalization_method, mean_tg, std_tg)
         grads: Dict[str, Optional[torch.Tensor]] = {}
         for l in range(L):
             grads[f"encoder_module.encoders.{l}.weight"] = raw["enc_w"][l]
@@ -251,13 +291,22 @@ class CrossLayerTranscoder(BaseTranscoder):
             grads[f"decoder_module.decoders.{key}.bias_param"] = raw["dec_b"][slot]
         if raw.get("theta") is not None:
             grads["theta_manager.log_threshold"] = raw["theta"]
+        if raw.get("skip") is not None:
+            for slot, key in enumerate(keys):
+                grads[f"decoder_module.skip_weights.{key}"] = raw["skip"][slot]
+        for name in ("feat_offset", "feat_scale"):
+            if raw.get(name) is not None:
+                for t in range(L):
+                    grads[f"decoder_module.feature_{name[5:]}.{t}"] = raw[name][t]
         return loss_l.sum(), grads
 
     @torch.no_grad()
-    def training_step(self, inputs: Dict[int, torch.Tensor], targets: Dict[int, torch.Tensor], optimizer) -> torch.Tensor:
+    def training_step(self, inputs: Dict[int, torch.Tensor], targets: Dict[int, torch.Tensor], optimizer,
+                      normalization_method: Optional[str] = None, mean_tg=None, std_tg=None) -> torch.Tensor:
         """One optimisation step on the MSE reconstruction loss (trainer.py:663-778 without the
-        auxiliary losses): forward, gradients, ``optimizer.step``; returns the loss before the step."""
-        loss_l, raw = self._loss_and_raw_gradients(inputs, targets)
+        auxiliary losses): forward, gradients, ``optimizer.step``; returns the loss before the step.
+        De-normalisation arguments as in ``loss_and_gradients``."""
+        loss_l, raw = self._loss_and_raw_gradients(inputs, targets, normalization_method, mean_tg, std_tg)
         optimizer.step(raw)
         return loss_l.sum()
 

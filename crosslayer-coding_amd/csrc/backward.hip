@@ -58,9 +58,20 @@ __device__ __forceinline__ float wave_sum(float v) {
 }
 
 // ---- loss and its gradient -------------------------------------------------------------------
-// loss_acc[l] += sum of squared differences (double); g[l][t][:] = 2 (rec - target) / (T d)
+// loss_acc[l] += sum of squared differences (double); g[l][t][:] = d loss / d rec.
+// The reference measures the loss on de-normalised tensors (clt/training/losses.py:70-86): with
+// CLT_DENORM_MEAN_STD both sides become x * std + mean, with CLT_DENORM_SCALE x / scale, every step rounded
+// to the model dtype as its tensor arithmetic is; the chain rule then puts a factor std (or 1 / scale) on
+// the gradient: g = 2 (rec' - target') / (T d) * std.
+template <typename T> __device__ __forceinline__ float bw_denorm(float x, int mode, float mean, float stdv, float scale) {
+  if (mode == CLT_DENORM_MEAN_STD) return Elem<T>::round(Elem<T>::round(x * stdv) + mean);
+  if (mode == CLT_DENORM_SCALE) return Elem<T>::round(x / scale);
+  return x;
+}
+
 template <typename T>
-__global__ __launch_bounds__(BW_THREADS) void k_mse_grad(const T *rec, const T *target, int64_t per_layer, float scale,
+__global__ __launch_bounds__(BW_THREADS) void k_mse_grad(const T *rec, const T *target, int64_t per_layer, int64_t d, float scale,
+                                                          int mode, const T *mean, const T *stdv, float dscale,
                                                           float *g, T *g_model, double *loss_acc) {
   __shared__ double red[BW_THREADS / 64];
   const int l = blockIdx.y;
@@ -70,11 +81,25 @@ __global__ __launch_bounds__(BW_THREADS) void k_mse_grad(const T *rec, const T *
   double acc = 0.0;
   for (int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4; i < per_layer; i += (int64_t)gridDim.x * blockDim.x * 4) {
     const float4 a = load4<T>(r + i), b = load4<T>(y + i);
-    const float d0 = a.x - b.x, d1 = a.y - b.y, d2 = a.z - b.z, d3 = a.w - b.w;
-    *reinterpret_cast<float4 *>(gl + i) = make_float4(scale * d0, scale * d1, scale * d2, scale * d3);
-    if (gm) { gm[i] = Elem<T>::from_f32(scale * d0); gm[i + 1] = Elem<T>::from_f32(scale * d1);
-              gm[i + 2] = Elem<T>::from_f32(scale * d2); gm[i + 3] = Elem<T>::from_f32(scale * d3); }
-    acc += (double)d0 * d0 + (double)d1 * d1 + (double)d2 * d2 + (double)d3 * d3;
+    const float av[4] = {a.x, a.y, a.z, a.w}, bv[4] = {b.x, b.y, b.z, b.w};
+    float dv[4], gv[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      if (mode == CLT_DENORM_NONE) {
+        dv[k] = av[k] - bv[k];
+        gv[k] = scale * dv[k];
+      } else {
+        const int64_t c = (i + k) % d;
+        const float mu = mode == CLT_DENORM_MEAN_STD ? Elem<T>::to_f32(mean[(int64_t)l * d + c]) : 0.0f;
+        const float sd = mode == CLT_DENORM_MEAN_STD ? Elem<T>::to_f32(stdv[(int64_t)l * d + c]) : 1.0f;
+        dv[k] = bw_denorm<T>(av[k], mode, mu, sd, dscale) - bw_denorm<T>(bv[k], mode, mu, sd, dscale);
+        gv[k] = scale * dv[k] * (mode == CLT_DENORM_MEAN_STD ? sd : 1.0f / dscale);
+      }
+    }
+    *reinterpret_cast<float4 *>(gl + i) = make_float4(gv[0], gv[1], gv[2], gv[3]);
+    if (gm) { gm[i] = Elem<T>::from_f32(gv[0]); gm[i + 1] = Elem<T>::from_f32(gv[1]);
+              gm[i + 2] = Elem<T>::from_f32(gv[2]); gm[i + 3] = Elem<T>::from_f32(gv[3]); }
+    acc += (double)dv[0] * dv[0] + (double)dv[1] * dv[1] + (double)dv[2] * dv[2] + (double)dv[3] * dv[3];
   }
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o);
@@ -312,9 +337,13 @@ __global__ __launch_bounds__(BW_THREADS) void k_bwd_values_sliced(
   }
 }
 
-// dval[j] = sum over the targets t >= s of part[t][j], in target order; one wavefront per row
+// dval[j] = sum over the targets t >= s of part[t][j], in target order; one wavefront per row.
+// With a feature scale (tied decoders, decoder.py:228-285) target t saw the activation times
+// fscale[t][feature] (non-zero activations only), so its share of the gradient carries that factor.
+template <typename T>
 __global__ __launch_bounds__(BW_THREADS) void k_bwd_values_sum(const int32_t *row_ptr, const float *part, int64_t Tn,
-                                                                int64_t L, int64_t nnz, uint64_t src_mask, float *dval) {
+                                                                int64_t L, int64_t nnz, uint64_t src_mask, float *dval,
+                                                                const int32_t *col, const T *val, const T *fscale, int64_t F) {
   const int lane = lane_id(), wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
   const int64_t R = L * Tn;
   for (int64_t r = (int64_t)blockIdx.x * nwv + wv; r < R; r += (int64_t)gridDim.x * nwv) {
@@ -322,7 +351,11 @@ __global__ __launch_bounds__(BW_THREADS) void k_bwd_values_sum(const int32_t *ro
     const bool on = (src_mask >> s) & 1ull;
     for (int32_t j = row_ptr[r] + lane; j < row_ptr[r + 1]; j += 64) {
       float acc = 0.0f;
-      if (on) {
+      if (on && fscale) {
+        const int64_t f = col[j];
+        const bool nz = Elem<T>::to_f32(val[j]) != 0.0f;
+        for (int64_t t = s; t < L; ++t) acc += part[t * nnz + j] * (nz ? Elem<T>::to_f32(fscale[t * F + f]) : 1.0f);
+      } else if (on) {
         // four loads in flight; the additions keep the target order
         int64_t t = s;
         for (; t + 4 <= L; t += 4) {
@@ -334,6 +367,89 @@ __global__ __launch_bounds__(BW_THREADS) void k_bwd_values_sum(const int32_t *ro
       dval[j] = acc;
     }
   }
+}
+
+// Gradients of the per-target feature offset / scale of tied decoders (decoder.py:228-245, 268-285).  Target t
+// sees a' = (a + off[t][f]) * scale[t][f] for the non-zero activations a of feature f in the sources s <= t; with
+// h = d loss / d a' (= part[t][j], the dot product of the loss gradient with the decoder row):
+//   d off[t][f]   = scale[t][f] * sum h          d scale[t][f] = sum h * (a + off[t][f])
+// One wavefront per (target, feature) walks the token-ordered lists of (s, f), s <= t: fixed summation order.
+template <typename T>
+__global__ __launch_bounds__(BW_THREADS) void k_affine_grad(const int32_t *__restrict__ ptr, const int32_t *__restrict__ lsrc,
+                                                             const T *__restrict__ val, const float *__restrict__ part,
+                                                             const T *__restrict__ foff, const T *__restrict__ fscale,
+                                                             int64_t F, int64_t L, int64_t nnz, uint64_t src_mask,
+                                                             float *__restrict__ doff, float *__restrict__ dscale) {
+  const int lane = lane_id(), wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
+  const int64_t total = L * F;
+  for (int64_t w = (int64_t)blockIdx.x * nwv + wv; w < total; w += (int64_t)gridDim.x * nwv) {
+    const int64_t t = w / F, f = w - t * F;
+    const float off = foff ? Elem<T>::to_f32(foff[w]) : 0.0f, sc = fscale ? Elem<T>::to_f32(fscale[w]) : 1.0f;
+    float a_sum = 0.0f, b_sum = 0.0f;
+    for (int64_t s = 0; s <= t; ++s) {
+      if (!((src_mask >> s) & 1ull)) continue;
+      const int32_t b = ptr[s * F + f], e = ptr[s * F + f + 1];
+      for (int32_t i = b + lane; i < e; i += 64) {
+        const int32_t j = lsrc[i];
+        const float a = Elem<T>::to_f32(val[j]);
+        if (a != 0.0f) {
+          const float h = part[t * nnz + j];
+          a_sum += h;
+          b_sum += h * (foff ? Elem<T>::round(a + off) : a);
+        }
+      }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) { a_sum += __shfl_xor(a_sum, o); b_sum += __shfl_xor(b_sum, o); }
+    if (lane == 0) {
+      if (doff) doff[w] = sc * a_sum;
+      if (dscale) dscale[w] = b_sum;
+    }
+  }
+}
+
+// Skip-connection weight gradient (decoder.py:297-338: rec += x @ W_skip.T): out[i][j] (+)= sum over tokens of
+// g[tok][i] * x[tok][j].  A block owns a 64 x 64 tile of the [d, d] result and walks all tokens, 16 at a time
+// through LDS; a thread owns a 4 x 4 piece.  Tokens in order: the same bits every run.
+constexpr int SK_TOK = 16;
+template <typename T>
+__global__ __launch_bounds__(256) void k_skip_grad(const float *__restrict__ g, const T *__restrict__ x, float *__restrict__ out,
+                                                   int64_t Tn, int64_t d, int accumulate) {
+  __shared__ float gs[SK_TOK][64], xs[SK_TOK][64];
+  const int i0 = blockIdx.y * 64, j0 = blockIdx.x * 64;
+  const int ti = (threadIdx.x >> 4) * 4, tj = (threadIdx.x & 15) * 4;
+  float acc[4][4];
+#pragma unroll
+  for (int a = 0; a < 4; ++a)
+#pragma unroll
+    for (int b = 0; b < 4; ++b) acc[a][b] = 0.0f;
+  for (int64_t t0 = 0; t0 < Tn; t0 += SK_TOK) {
+    for (int e = threadIdx.x; e < SK_TOK * 64; e += 256) {
+      const int tt = e >> 6, c = e & 63;
+      const int64_t tok = t0 + tt;
+      gs[tt][c] = (tok < Tn && i0 + c < d) ? g[tok * d + i0 + c] : 0.0f;
+      xs[tt][c] = (tok < Tn && j0 + c < d) ? Elem<T>::to_f32(x[tok * d + j0 + c]) : 0.0f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int tt = 0; tt < SK_TOK; ++tt) {
+      float gv[4], xv[4];
+#pragma unroll
+      for (int a = 0; a < 4; ++a) { gv[a] = gs[tt][ti + a]; xv[a] = xs[tt][tj + a]; }
+#pragma unroll
+      for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) acc[a][b] = fmaf(gv[a], xv[b], acc[a][b]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int a = 0; a < 4; ++a)
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const int64_t i = i0 + ti + a, j = j0 + tj + b;
+      if (i < d && j < d) out[i * d + j] = accumulate ? out[i * d + j] + acc[a][b] : acc[a][b];
+    }
 }
 
 // ---- feature lists: the survivor list regrouped by (layer, feature) ----------------------------------
@@ -436,17 +552,70 @@ __global__ __launch_bounds__(BW_THREADS) void k_csc_fill(const int32_t *row_ptr,
   }
 }
 
-// Lists of up to 64 entries are put in token order (the fill order depends on scheduling), so
-// that the sums over a list always run in the same order; longer lists stay as filled.
-__global__ __launch_bounds__(BW_THREADS) void k_csc_order(const int32_t *ptr, int64_t nlist, int32_t *tok, int32_t *src) {
+// Every list is put in token order (the fill order depends on scheduling), so that the sums over a list
+// always run in the same order and the weight gradients are the same bits from run to run.
+//   up to 64 entries: one entry per lane, rank = number of smaller tokens;
+//   longer lists: the tokens of a list are distinct, so the list is a set of tokens: the wavefront marks them in
+//   a bitmap in LDS (T bits), takes prefix popcounts over its words, and then walks the WORDS, not the entries:
+//   the i-th set bit is the i-th token.  The position of the survivor in col / val is looked up again in its row
+//   (the columns of a row ascend), so nothing is read from the arrays that are being rewritten.
+// LDS per wavefront: 2 * ceil(T / 32) words (dynamic shared memory, bm_words = ceil(T / 32)).
+__global__ __launch_bounds__(BW_THREADS) void k_csc_order(const int32_t *ptr, int64_t nlist, int32_t *tok, int32_t *src,
+                                                           const int32_t *row_ptr, const int32_t *col, int64_t Tn, int64_t F,
+                                                           int bm_words) {
+  extern __shared__ uint32_t order_lds[];
   const int lane = lane_id(), wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
+  uint32_t *bm = order_lds + (size_t)wv * 2 * bm_words, *pfx = bm + bm_words;
   for (int64_t q = (int64_t)blockIdx.x * nwv + wv; q < nlist; q += (int64_t)gridDim.x * nwv) {
     const int32_t b = ptr[q], n = ptr[q + 1] - b;
-    if (n < 2 || n > 64) continue;
-    const int32_t mt = lane < n ? tok[b + lane] : 0x7FFFFFFF, ms = lane < n ? src[b + lane] : 0;
-    int rank = 0;
-    for (int i = 0; i < n; ++i) rank += __builtin_amdgcn_readlane(mt, i) < mt ? 1 : 0;   // tokens of one list are distinct
-    if (lane < n) { tok[b + rank] = mt; src[b + rank] = ms; }
+    if (n < 2) continue;
+    if (n <= 64) {
+      const int32_t mt = lane < n ? tok[b + lane] : 0x7FFFFFFF, ms = lane < n ? src[b + lane] : 0;
+      int rank = 0;
+      for (int i = 0; i < n; ++i) rank += __builtin_amdgcn_readlane(mt, i) < mt ? 1 : 0;   // tokens of one list are distinct
+      if (lane < n) { tok[b + rank] = mt; src[b + rank] = ms; }
+      continue;
+    }
+    const int64_t l = q / F, f = q - l * F;
+    for (int w = lane; w < bm_words; w += 64) bm[w] = 0u;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    for (int32_t i = lane; i < n; i += 64) {
+      const int32_t tk = tok[b + i];
+      atomicOr(&bm[tk >> 5], 1u << (tk & 31));
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    // exclusive prefix popcounts over the words, 64 words at a time
+    uint32_t carry = 0;
+    for (int w0 = 0; w0 < bm_words; w0 += 64) {
+      const int w = w0 + lane;
+      const uint32_t c = w < bm_words ? (uint32_t)__popc(bm[w]) : 0u;
+      uint32_t inc = c;
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {
+        const uint32_t y = __shfl_up(inc, o);
+        if (lane >= o) inc += y;
+      }
+      if (w < bm_words) pfx[w] = carry + inc - c;
+      carry += __shfl(inc, 63);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    for (int w = lane; w < bm_words; w += 64) {
+      uint32_t bits = bm[w];
+      int32_t pos = b + (int32_t)pfx[w];
+      while (bits) {
+        const int32_t tk = w * 32 + (__ffs(bits) - 1);
+        bits &= bits - 1u;
+        // the survivor (layer l, token tk, feature f): its place in the row's ascending columns
+        const int64_t r = l * Tn + tk;
+        int32_t lo = row_ptr[r], hi = row_ptr[r + 1];
+        while (lo < hi) {
+          const int32_t mid = lo + ((hi - lo) >> 1);
+          if (col[mid] < (int32_t)f) lo = mid + 1; else hi = mid;
+        }
+        tok[pos] = tk; src[pos] = lo;
+        ++pos;
+      }
+    }
   }
 }
 
@@ -464,7 +633,8 @@ template <typename T, typename CoefT, int NCH, bool DECODER, bool T8 = false>
 __global__ __launch_bounds__(BW_THREADS) void k_feature_outer(
     const int32_t *__restrict__ ptr, const int32_t *__restrict__ ltok, const int32_t *__restrict__ lsrc,
     const CoefT *__restrict__ coef, const T *__restrict__ src, float *__restrict__ out, float *__restrict__ rowsum,
-    int64_t Tn, int64_t d, int64_t F, int64_t L, int64_t target, int tying) {
+    int64_t Tn, int64_t d, int64_t F, int64_t L, int64_t target, int tying, const T *__restrict__ foff = nullptr,
+    const T *__restrict__ fscale = nullptr) {
   constexpr int EV = Piece<T>::EV;
   const int lane = lane_id(), wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
   // One launch per layer of the gathered matrix, so that every wavefront of a launch gathers from the
@@ -499,6 +669,11 @@ __global__ __launch_bounds__(BW_THREADS) void k_feature_outer(
       const int n = (e - i0) < 64 ? (e - i0) : 64;
       int32_t mt = 0; float mc = 0.0f;
       if (lane < n) { mt = ltok[i0 + lane]; mc = Elem<CoefT>::to_f32(coef[lsrc[i0 + lane]]); }
+      if (DECODER && (foff || fscale) && mc != 0.0f) {
+        // the target's feature offset / scale: what this decoder was multiplied with (decoder.py:228-245)
+        if (foff) mc = Elem<T>::round(mc + Elem<T>::to_f32(foff[t * F + f]));
+        if (fscale) mc = Elem<T>::round(mc * Elem<T>::to_f32(fscale[t * F + f]));
+      }
       // rows in flight.  Narrow rows (d <= 1024 in bf16) run best with four: 55 registers, eight wavefronts per
       // SIMD (eight in flight, six wavefronts: 11 % slower); wide rows keep about 16 pieces per lane
       constexpr int NU = NCH <= 4 ? FO_NU / 2 : FO_NU / 4;
@@ -619,10 +794,14 @@ extern "C" size_t clt_mse_workspace_bytes(int64_t T, int64_t d, int64_t L) {
 }
 
 extern "C" int clt_mse_loss_grad(const void *rec, const void *target, int64_t T, int64_t d, int64_t L, int dtype,
+                                 int denorm_mode, const void *mean, const void *stdv, double denorm_scale,
                                  float *loss_per_layer, float *g, void *g_model, float *bias_grad, void *workspace,
                                  size_t workspace_bytes, void *stream) {
   if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
   if (T <= 0 || d <= 0 || L <= 0 || L > 65535 || !rec || !target || !loss_per_layer || !g || !workspace) return CLT_ERR_ARG;
+  if (denorm_mode < CLT_DENORM_NONE || denorm_mode > CLT_DENORM_SCALE) return CLT_ERR_ARG;
+  if (denorm_mode == CLT_DENORM_MEAN_STD && (!mean || !stdv)) return CLT_ERR_ARG;
+  if (denorm_mode == CLT_DENORM_SCALE && !(denorm_scale != 0.0)) return CLT_ERR_ARG;
   if ((T * d) % 4 != 0) return CLT_ERR_ARG;
   if (workspace_bytes < clt_mse_workspace_bytes(T, d, L)) return CLT_ERR_WORKSPACE;
   if ((((uintptr_t)workspace) & 255u) != 0) return CLT_ERR_ALIGN;
@@ -633,8 +812,8 @@ extern "C" int clt_mse_loss_grad(const void *rec, const void *target, int64_t T,
   const int64_t per_layer = T * d;
   const float scale = (float)(2.0 / (double)per_layer);
   dim3 grid(512, (unsigned)L);
-  if (dtype == CLT_BF16) k_mse_grad<bf16_t><<<grid, BW_THREADS, 0, s>>>((const bf16_t *)rec, (const bf16_t *)target, per_layer, scale, g, (bf16_t *)g_model, acc);
-  else k_mse_grad<float><<<grid, BW_THREADS, 0, s>>>((const float *)rec, (const float *)target, per_layer, scale, g, (float *)g_model, acc);
+  if (dtype == CLT_BF16) k_mse_grad<bf16_t><<<grid, BW_THREADS, 0, s>>>((const bf16_t *)rec, (const bf16_t *)target, per_layer, d, scale, denorm_mode, (const bf16_t *)mean, (const bf16_t *)stdv, (float)denorm_scale, g, (bf16_t *)g_model, acc);
+  else k_mse_grad<float><<<grid, BW_THREADS, 0, s>>>((const float *)rec, (const float *)target, per_layer, d, scale, denorm_mode, (const float *)mean, (const float *)stdv, (float)denorm_scale, g, (float *)g_model, acc);
   k_loss_finish<<<(unsigned)clt_ceil_div(L, 256), 256, 0, s>>>(acc, (int)L, 1.0 / (double)per_layer, loss_per_layer);
   if (bias_grad) {
     k_colsum_partial<<<dim3((unsigned)clt_ceil_div(d, BW_THREADS), (unsigned)L, CS_SPLIT), BW_THREADS, 0, s>>>(g, T, d, part);
@@ -648,10 +827,10 @@ extern "C" size_t clt_decode_backward_workspace_bytes(int64_t T, int64_t L, int6
   return (((size_t)L * (size_t)T * (BWV_XCDS + 1) * 4 + 255) & ~(size_t)255) + (size_t)L * (size_t)(nnz > 0 ? nnz : 1) * 4;
 }
 
-extern "C" int clt_decode_backward_values(const int32_t *row_ptr, const int32_t *col, const void *w_packed, const float *g,
-                                          int64_t T, int64_t d, int64_t F, int64_t L, int tying, uint64_t src_mask,
-                                          int64_t nnz, int dtype, float *dval, void *workspace, size_t workspace_bytes,
-                                          void *stream) {
+extern "C" int clt_decode_backward_values(const int32_t *row_ptr, const int32_t *col, const void *val, const void *w_packed,
+                                          const void *feat_scale, const float *g, int64_t T, int64_t d, int64_t F, int64_t L,
+                                          int tying, uint64_t src_mask, int64_t nnz, int dtype, float *dval, void *workspace,
+                                          size_t workspace_bytes, void *stream) {
   if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
   if (T <= 0 || F <= 0 || L <= 0 || L > 64 || tying < 0 || tying > 2 || nnz < 0) return CLT_ERR_ARG;
   if (!row_ptr || !w_packed || !g || !dval || !workspace) return CLT_ERR_ARG;
@@ -681,7 +860,45 @@ extern "C" int clt_decode_backward_values(const int32_t *row_ptr, const int32_t 
   else if (dtype == CLT_BF16) CLT_BWV_N(bf16_t); else CLT_BWV_N(float);
 #undef CLT_BWV_N
 #undef CLT_BWV
-  k_bwd_values_sum<<<256 * 8, BW_THREADS, 0, s>>>(row_ptr, part, T, L, nnz, src_mask, dval);
+  if (feat_scale && !val) return CLT_ERR_ARG;
+  if (dtype == CLT_BF16)
+    k_bwd_values_sum<bf16_t><<<256 * 8, BW_THREADS, 0, s>>>(row_ptr, part, T, L, nnz, src_mask, dval, col, (const bf16_t *)val,
+                                                            (const bf16_t *)feat_scale, F);
+  else
+    k_bwd_values_sum<float><<<256 * 8, BW_THREADS, 0, s>>>(row_ptr, part, T, L, nnz, src_mask, dval, col, (const float *)val,
+                                                           (const float *)feat_scale, F);
+  return clt_check_launch();
+}
+
+extern "C" int clt_feature_affine_grad(const int32_t *list_ptr, const int32_t *list_src, const void *val,
+                                       const void *feat_offset, const void *feat_scale, int64_t T, int64_t F, int64_t L,
+                                       uint64_t src_mask, int64_t nnz, int dtype, float *d_offset, float *d_scale,
+                                       const void *workspace, size_t workspace_bytes, void *stream) {
+  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (T <= 0 || F <= 0 || L <= 0 || L > 64 || nnz < 0 || !list_ptr || !list_src || !val || !workspace) return CLT_ERR_ARG;
+  if (!d_offset && !d_scale) return CLT_OK;
+  if (workspace_bytes < clt_decode_backward_workspace_bytes(T, L, nnz)) return CLT_ERR_WORKSPACE;
+  hipStream_t s = (hipStream_t)stream;
+  // the per-target dot products clt_decode_backward_values left behind the slice pointers
+  const float *part = (const float *)((const char *)workspace + (((size_t)L * (size_t)T * (BWV_XCDS + 1) * 4 + 255) & ~(size_t)255));
+  if (dtype == CLT_BF16)
+    k_affine_grad<bf16_t><<<256 * 8, BW_THREADS, 0, s>>>(list_ptr, list_src, (const bf16_t *)val, part, (const bf16_t *)feat_offset,
+                                                         (const bf16_t *)feat_scale, F, L, nnz, src_mask, d_offset, d_scale);
+  else
+    k_affine_grad<float><<<256 * 8, BW_THREADS, 0, s>>>(list_ptr, list_src, (const float *)val, part, (const float *)feat_offset,
+                                                        (const float *)feat_scale, F, L, nnz, src_mask, d_offset, d_scale);
+  return clt_check_launch();
+}
+
+extern "C" int clt_skip_weight_grad(const float *g, const void *x, float *out, int64_t T, int64_t d, int accumulate, int dtype,
+                                    void *stream) {
+  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (T <= 0 || d <= 0 || !g || !x || !out) return CLT_ERR_ARG;
+  if (clt_ceil_div(d, 64) > 65535) return CLT_ERR_RANGE;
+  dim3 grid((unsigned)clt_ceil_div(d, 64), (unsigned)clt_ceil_div(d, 64));
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == CLT_BF16) k_skip_grad<bf16_t><<<grid, 256, 0, s>>>(g, (const bf16_t *)x, out, T, d, accumulate);
+  else k_skip_grad<float><<<grid, 256, 0, s>>>(g, (const float *)x, out, T, d, accumulate);
   return clt_check_launch();
 }
 
@@ -696,6 +913,7 @@ extern "C" int clt_feature_lists(const int32_t *row_ptr, const int32_t *col, int
                                  size_t workspace_bytes, void *stream) {
   if (T <= 0 || F <= 0 || L <= 0 || L > 65535 || !row_ptr || !list_ptr || !workspace) return CLT_ERR_ARG;
   if ((double)L * (double)F >= 2147483647.0) return CLT_ERR_RANGE;
+  if (T > 65536) return CLT_ERR_RANGE;    // the token bitmaps of a workgroup's four wavefronts take T bytes of LDS
   if (workspace_bytes < clt_feature_lists_workspace_bytes(F, L)) return CLT_ERR_WORKSPACE;
   if ((((uintptr_t)workspace) & 7u) != 0) return CLT_ERR_ALIGN;
   hipStream_t s = (hipStream_t)stream;
@@ -711,14 +929,17 @@ extern "C" int clt_feature_lists(const int32_t *row_ptr, const int32_t *col, int
   k_csc_chunk_scan<<<(unsigned)nchunk, BW_THREADS, 0, s>>>(cnt, n, sums, list_ptr);
   if (list_tok && list_src) {
     k_csc_fill<<<nb, BW_THREADS, 0, s>>>(row_ptr, col, T, F, L, list_ptr, cnt, list_tok, list_src);
-    k_csc_order<<<nb, BW_THREADS, 0, s>>>(list_ptr, n, list_tok, list_src);
+    const int bm_words = (int)clt_ceil_div(T, 32);
+    k_csc_order<<<nb, BW_THREADS, (size_t)(BW_THREADS / 64) * 2 * bm_words * 4, s>>>(list_ptr, n, list_tok, list_src, row_ptr, col,
+                                                                                   T, F, bm_words);
   }
   return clt_check_launch();
 }
 
 extern "C" int clt_decoder_weight_grad(const int32_t *list_ptr, const int32_t *list_tok, const int32_t *list_src,
-                                       const void *val, const void *g_model, float *dw_packed, int64_t T, int64_t d,
-                                       int64_t F, int64_t L, int tying, int dtype, void *stream) {
+                                       const void *val, const void *g_model, const void *feat_offset, const void *feat_scale,
+                                       float *dw_packed, int64_t T, int64_t d, int64_t F, int64_t L, int tying, int dtype,
+                                       void *stream) {
   if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
   if (tying < 0 || tying > 2) return CLT_ERR_ARG;
   if (T <= 0 || F <= 0 || L <= 0 || L > 64 || !list_ptr || !list_tok || !list_src || !val || !g_model || !dw_packed) return CLT_ERR_ARG;
@@ -729,7 +950,7 @@ extern "C" int clt_decoder_weight_grad(const int32_t *list_ptr, const int32_t *l
 #define CLT_DW(CT, N)                                                                                                      \
   do {                                                                                                                     \
     for (int64_t t = 0; t < L; ++t) {                                                                                      \
-      k_feature_outer<CT, CT, N, true><<<bw_resident_blocks(k_feature_outer<CT, CT, N, true>), BW_THREADS, 0, s>>>(list_ptr, list_tok, list_src, (const CT *)val, (const CT *)g_model, dw_packed, nullptr, T, d, F, L, t, tying); \
+      k_feature_outer<CT, CT, N, true><<<bw_resident_blocks(k_feature_outer<CT, CT, N, true>), BW_THREADS, 0, s>>>(list_ptr, list_tok, list_src, (const CT *)val, (const CT *)g_model, dw_packed, nullptr, T, d, F, L, t, tying, (const CT *)feat_offset, (const CT *)feat_scale); \
     }                                                                                                                      \
   } while (0)
 #define CLT_DW_N(CT)                                                                       \
@@ -743,7 +964,8 @@ extern "C" int clt_decoder_weight_grad(const int32_t *list_ptr, const int32_t *l
   if (dtype == CLT_BF16 && d == 768) {
     for (int64_t t = 0; t < L; ++t)
       k_feature_outer<bf16_t, bf16_t, 2, true, true><<<bw_resident_blocks(k_feature_outer<bf16_t, bf16_t, 2, true, true>), BW_THREADS, 0, s>>>(
-          list_ptr, list_tok, list_src, (const bf16_t *)val, (const bf16_t *)g_model, dw_packed, nullptr, T, d, F, L, t, tying);
+          list_ptr, list_tok, list_src, (const bf16_t *)val, (const bf16_t *)g_model, dw_packed, nullptr, T, d, F, L, t, tying,
+          (const bf16_t *)feat_offset, (const bf16_t *)feat_scale);
   } else if (dtype == CLT_BF16) CLT_DW_N(bf16_t); else CLT_DW_N(float);
 #undef CLT_DW_N
 #undef CLT_DW

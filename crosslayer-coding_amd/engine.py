@@ -388,12 +388,18 @@ def reconstruction_stats(rec: torch.Tensor, target: torch.Tensor, mode: str = "n
 
 
 # ---- backward pass (MSE reconstruction loss) ---------------------------------------------------------
-def mse_loss_grad(rec: torch.Tensor, target: torch.Tensor, ws: Optional[Workspace] = None):
+def mse_loss_grad(rec: torch.Tensor, target: torch.Tensor, ws: Optional[Workspace] = None, mode: str = "none",
+                  mean: Optional[torch.Tensor] = None, std: Optional[torch.Tensor] = None, scale: float = 1.0):
     """(loss per layer [L] fp32, g [L, T, d] fp32 = d loss / d rec, the same in the model dtype,
-    bias_grad [L, d] fp32) for loss = sum over layers of mean((rec - target)^2) (losses.py:45-92)."""
+    bias_grad [L, d] fp32) for loss = sum over layers of mean((rec' - target')^2), ' being the reference's
+    de-normalisation (losses.py:45-92): ``mode`` "mean_std" with the target statistics ``mean`` / ``std``
+    [L, d], "sqrt_d_model" with ``scale`` = sqrt(d_model), or "none"."""
     nat.require_device(rec, "mse_loss_grad")
     L, T, d = rec.shape
     assert target.shape == rec.shape and target.dtype == rec.dtype and rec.is_contiguous() and target.is_contiguous()
+    if mode == "mean_std":
+        assert mean is not None and std is not None and mean.shape == (L, d) and std.shape == (L, d)
+        mean, std = mean.to(rec.dtype).contiguous(), std.to(rec.dtype).contiguous()
     dev = rec.device
     loss = torch.empty(L, dtype=torch.float32, device=dev)
     g = torch.empty((L, T, d), dtype=torch.float32, device=dev)
@@ -401,33 +407,72 @@ def mse_loss_grad(rec: torch.Tensor, target: torch.Tensor, ws: Optional[Workspac
     g_model = g if rec.dtype == torch.float32 else torch.empty((L, T, d), dtype=rec.dtype, device=dev)
     lib = nat.load()
     wbuf = (ws or Workspace(dev)).get("mse", lib.clt_mse_workspace_bytes(T, d, L))
-    code = lib.clt_mse_loss_grad(nat.ptr(rec), nat.ptr(target), T, d, L, nat.dtype_code(rec.dtype), nat.ptr(loss),
-                                 nat.ptr(g), nat.ptr(g_model) if g_model is not g else None, nat.ptr(bias_grad),
-                                 nat.ptr(wbuf), wbuf.numel(), _stream(rec))
+    code = lib.clt_mse_loss_grad(nat.ptr(rec), nat.ptr(target), T, d, L, nat.dtype_code(rec.dtype), DENORM_MODES[mode],
+                                 nat.ptr(mean) if mode == "mean_std" else None, nat.ptr(std) if mode == "mean_std" else None,
+                                 float(scale), nat.ptr(loss), nat.ptr(g), nat.ptr(g_model) if g_model is not g else None,
+                                 nat.ptr(bias_grad), nat.ptr(wbuf), wbuf.numel(), _stream(rec))
     nat.check(code, "clt_mse_loss_grad")
     return loss, g, g_model, bias_grad
 
 
 def decode_backward_values(surv: SurvivorList, w_packed: torch.Tensor, g: torch.Tensor, tying: str,
-                           src_mask: Optional[int] = None, ws: Optional[Workspace] = None) -> torch.Tensor:  # noqa: E501
-    """d loss / d (kept activation) for every survivor, fp32 [nnz] (the straight-through gate hands
-    it to the pre-activation unchanged, activations.py:66-96)."""
+                           src_mask: Optional[int] = None, ws: Optional[Workspace] = None,
+                           feat_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """d loss / d (kept activation) for every survivor, fp32 [capacity] (the straight-through gate hands
+    it to the pre-activation unchanged, activations.py:66-96).  ``feat_scale`` [L, F]: the per-target
+    feature scale of tied decoders, a factor on each target's share (decoder.py:228-285).  The per-target
+    dot products stay in the "decode_backward" buffer of ``ws`` for ``feature_affine_grad``."""
     L, T, F = surv.L, surv.T, surv.F
     d = g.shape[2]
     assert g.shape == (L, T, d) and g.dtype == torch.float32 and g.is_contiguous()
     assert w_packed.dtype == surv.dtype and w_packed.is_contiguous()
     assert tuple(w_packed.shape[1:]) == (F, decoder_pitch(d, surv.dtype))
+    assert feat_scale is None or (feat_scale.shape == (L, F) and feat_scale.dtype == surv.dtype and feat_scale.is_contiguous())
     if src_mask is None:
         src_mask = (1 << L) - 1
     cap = surv.capacity          # survivor-indexed buffers are sized from the arrays, not from a read-back
     dval = torch.empty(max(cap, 1), dtype=torch.float32, device=g.device)
     lib = nat.load()
     wbuf = (ws or Workspace(g.device)).get("decode_backward", lib.clt_decode_backward_workspace_bytes(T, L, cap))
-    code = lib.clt_decode_backward_values(nat.ptr(surv.row_ptr), nat.ptr(surv.col), nat.ptr(w_packed), nat.ptr(g),
-                                          T, d, F, L, nat.TYING[tying], src_mask & ((1 << 64) - 1), cap,
-                                          nat.dtype_code(surv.dtype), nat.ptr(dval), nat.ptr(wbuf), wbuf.numel(), _stream(g))
+    code = lib.clt_decode_backward_values(nat.ptr(surv.row_ptr), nat.ptr(surv.col), nat.ptr(surv.val), nat.ptr(w_packed),
+                                          nat.ptr(feat_scale), nat.ptr(g), T, d, F, L, nat.TYING[tying],
+                                          src_mask & ((1 << 64) - 1), cap, nat.dtype_code(surv.dtype), nat.ptr(dval),
+                                          nat.ptr(wbuf), wbuf.numel(), _stream(g))
     nat.check(code, "clt_decode_backward_values")
     return dval[:cap]
+
+
+def feature_affine_grad(lists, surv: SurvivorList, ws: Workspace, feat_offset: Optional[torch.Tensor],
+                        feat_scale: Optional[torch.Tensor], src_mask: Optional[int] = None):
+    """(d offset [L, F] or None, d scale [L, F] or None), fp32: gradients of the per-target feature offset /
+    scale of tied decoders (decoder.py:228-285).  Must follow ``decode_backward_values`` on the same ``ws``."""
+    L, T, F = surv.L, surv.T, surv.F
+    ptr, _, src = lists
+    dev = surv.row_ptr.device
+    if src_mask is None:
+        src_mask = (1 << L) - 1
+    doff = torch.empty((L, F), dtype=torch.float32, device=dev) if feat_offset is not None else None
+    dsc = torch.empty((L, F), dtype=torch.float32, device=dev) if feat_scale is not None else None
+    lib = nat.load()
+    cap = surv.capacity
+    wbuf = ws.get("decode_backward", lib.clt_decode_backward_workspace_bytes(T, L, cap))
+    code = lib.clt_feature_affine_grad(nat.ptr(ptr), nat.ptr(src), nat.ptr(surv.val), nat.ptr(feat_offset), nat.ptr(feat_scale),
+                                       T, F, L, src_mask & ((1 << 64) - 1), cap, nat.dtype_code(surv.dtype), nat.ptr(doff),
+                                       nat.ptr(dsc), nat.ptr(wbuf), wbuf.numel(), nat.current_stream(dev))
+    nat.check(code, "clt_feature_affine_grad")
+    return doff, dsc
+
+
+def skip_weight_grad(g_t: torch.Tensor, x_s: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
+    """out [d, d] fp32 (+)= g_t.T @ x_s: gradient of one skip matrix (rec[t] += x[s] @ W_skip.T,
+    decoder.py:297-338); g_t [T, d] fp32, x_s [T, d] in the model dtype."""
+    nat.require_device(g_t, "skip_weight_grad")
+    T, d = g_t.shape
+    assert x_s.shape == (T, d) and g_t.dtype == torch.float32 and g_t.is_contiguous() and x_s.is_contiguous()
+    assert out.shape == (d, d) and out.dtype == torch.float32 and out.is_contiguous()
+    code = nat.load().clt_skip_weight_grad(nat.ptr(g_t), nat.ptr(x_s), nat.ptr(out), T, d, 1 if accumulate else 0,
+                                           nat.dtype_code(x_s.dtype), _stream(g_t))
+    nat.check(code, "clt_skip_weight_grad")
 
 
 def feature_lists(surv: SurvivorList, ws: Optional[Workspace] = None):
@@ -445,10 +490,11 @@ def feature_lists(surv: SurvivorList, ws: Optional[Workspace] = None):
     return ptr, tok, src
 
 
-def decoder_weight_grad(lists, surv: SurvivorList, g: torch.Tensor, tying: str) -> torch.Tensor:
+def decoder_weight_grad(lists, surv: SurvivorList, g: torch.Tensor, tying: str,
+                        feat_offset: Optional[torch.Tensor] = None, feat_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
     """fp32 [n_dec, F, d] gradient of the packed (feature-major) decoder weights (one matrix per
     (source, target) pair, per source or per target, as ``tying`` says); ``g`` is d loss / d rec in
-    the model dtype."""
+    the model dtype; ``feat_offset`` / ``feat_scale`` [L, F]: the per-target affine terms the forward applied."""
     assert g.dtype == surv.dtype and g.is_contiguous()
     ptr, tok, src = lists
     L, T, F = surv.L, surv.T, surv.F
@@ -456,8 +502,8 @@ def decoder_weight_grad(lists, surv: SurvivorList, g: torch.Tensor, tying: str) 
     n_dec = L * (L + 1) // 2 if tying == "none" else L
     out = torch.empty((n_dec, F, d), dtype=torch.float32, device=g.device)
     code = nat.load().clt_decoder_weight_grad(nat.ptr(ptr), nat.ptr(tok), nat.ptr(src), nat.ptr(surv.val), nat.ptr(g),
-                                              nat.ptr(out), T, d, F, L, nat.TYING[tying], nat.dtype_code(surv.dtype),
-                                              _stream(g))
+                                              nat.ptr(feat_offset), nat.ptr(feat_scale), nat.ptr(out), T, d, F, L,
+                                              nat.TYING[tying], nat.dtype_code(surv.dtype), _stream(g))
     nat.check(code, "clt_decoder_weight_grad")
     return out
 

@@ -35,6 +35,13 @@ class CLTAdam:
         }
         if cfg.activation_fn == "jumprelu" and model.theta_manager.log_threshold is not None:
             self.state["theta"] = (z(L, F), z(L, F))
+        dec = model.decoder_module
+        if dec.skip_weights is not None:
+            self.state["skip"] = (z(len(dec.skip_weights), d, d), z(len(dec.skip_weights), d, d))
+        if dec.feature_offset is not None:
+            self.state["feat_offset"] = (z(L, F), z(L, F))
+        if dec.feature_scale is not None:
+            self.state["feat_scale"] = (z(L, F), z(L, F))
 
     def _adam(self, param: torch.Tensor, grad: torch.Tensor, m: torch.Tensor, v: torch.Tensor) -> None:
         assert param.is_contiguous() and grad.is_contiguous() and grad.dtype == torch.float32 and grad.numel() == param.numel()
@@ -93,6 +100,26 @@ class CLTAdam:
         nat.check(code, "clt_adam_step_many")
         if raw.get("theta") is not None and "theta" in self.state:
             self._adam(model.theta_manager.log_threshold.data, raw["theta"].contiguous(), *self.state["theta"])
+        # skip matrices and per-target feature offset / scale: separate small tensors, one launch per family
+        if dec.skip_weights is not None:
+            skips = list(dec.skip_weights.values()) if hasattr(dec.skip_weights, "values") else list(dec.skip_weights)
+        else:
+            skips = None
+        for key, params in (("skip", skips),
+                            ("feat_offset", list(dec.feature_offset) if dec.feature_offset is not None else None),
+                            ("feat_scale", list(dec.feature_scale) if dec.feature_scale is not None else None)):
+            if params is None or raw.get(key) is None or key not in self.state:
+                continue
+            ps = [p.data for p in params]
+            assert all(p.is_contiguous() and p.numel() == ps[0].numel() and p.dtype == ps[0].dtype for p in ps)
+            grad = raw[key].contiguous()
+            assert grad.dtype == torch.float32 and grad.numel() == len(ps) * ps[0].numel()
+            p_dev, _ = self._pointer_table(key, ps)
+            m_p, v_p = self.state[key]
+            code = lib.clt_adam_step_many(nat.ptr(p_dev), nat.ptr(grad), nat.ptr(m_p), nat.ptr(v_p), len(ps), ps[0].numel(),
+                                          self.lr, self.betas[0], self.betas[1], self.eps, self.step_count,
+                                          nat.dtype_code(ps[0].dtype), nat.current_stream(ps[0].device))
+            nat.check(code, "clt_adam_step_many")
         # the kernels wrote through .data: caches keyed on version counters would not notice
         dec._bias_cache.clear()
         dec._cached_decoder_norms = None

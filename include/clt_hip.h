@@ -389,45 +389,73 @@ int clt_decoder_norms(const void *w_packed, void *norms, int64_t d, int64_t F,
  * The reference trains through torch autograd (clt/training/trainer.py:663-751); these entry
  * points compute the same gradients from the survivor list, without dense activations.
  *
- * clt_mse_loss_grad: loss_per_layer[l] = mean((rec[l] - target[l])^2) as nn.MSELoss gives per
- *   layer (clt/training/losses.py:45-92, summed over layers by the caller), g[l][t][:] =
- *   2 (rec - target) / (T d) in fp32 (and, when g_model != NULL, the same rounded to the model
- *   dtype: what clt_decoder_weight_grad reads), and (when bias_grad != NULL) bias_grad[l][:] = sum over
- *   tokens of g[l] - the gradient of every decoder bias that feeds target l.
+ * clt_mse_loss_grad: loss_per_layer[l] = mean((rec'[l] - target'[l])^2) as nn.MSELoss gives per
+ *   layer (clt/training/losses.py:45-92, summed over layers by the caller), where ' is the
+ *   de-normalisation LossManager applies first (losses.py:70-86): CLT_DENORM_NONE nothing,
+ *   CLT_DENORM_MEAN_STD x * std[l][c] + mean[l][c] (the store's target statistics, [L][d] in the model
+ *   dtype), CLT_DENORM_SCALE x / denorm_scale (sqrt(d_model)), each step rounded to the model dtype.
+ *   g[l][t][:] = d loss / d rec = 2 (rec' - target') / (T d) * std (or / denorm_scale) in fp32 (and,
+ *   when g_model != NULL, the same rounded to the model dtype: what clt_decoder_weight_grad reads), and
+ *   (when bias_grad != NULL) bias_grad[l][:] = sum over tokens of g[l] - the gradient of every decoder
+ *   bias that feeds target l.
  *   rec / target [L][T][d] in the model dtype; workspace clt_mse_workspace_bytes().
  * clt_decode_backward_values: dval[j] = sum over targets t >= s of g[t][token] . w[slot(s,t)][f]
  *   for survivor j = (s, token, f): the gradient of the loss with respect to the kept
  *   activation, which the straight-through gate passes on to the pre-activation
- *   (clt/models/activations.py:66-96).  dval [nnz] fp32; nnz = row_ptr[L*T]; workspace
+ *   (clt/models/activations.py:66-96).  With feat_scale ([L][F] model dtype, tied decoders,
+ *   clt/models/decoder.py:228-285) target t's share carries the factor feat_scale[t][f] for a non-zero
+ *   activation (val is needed then; both may be NULL otherwise).  dval [nnz] fp32; nnz = row_ptr[L*T]; workspace
  *   clt_decode_backward_workspace_bytes() (slice pointers and one partial per target and survivor,
- *   summed in target order).
+ *   summed in target order); `nnz` is the stride of those partials: any value >= row_ptr[L*T], e.g. the
+ *   number of entries col holds, so that no total has to be read back.
  * clt_feature_lists: the survivor list regrouped by (layer, feature): list_ptr [L*F+1],
- *   list_tok [nnz] token of each entry, list_src [nnz] its position in col / val.  Lists of up to
- *   64 entries are in token order.  Pass list_tok = list_src = NULL to get the counts only.
+ *   list_tok [nnz] token of each entry, list_src [nnz] its position in col / val.  Every
+ *   list is in ascending token order, so sums over a list always run in the same order (T <= 65536).
+ *   Pass list_tok = list_src = NULL to get the counts only.
  * clt_decoder_weight_grad: dw_packed[slot(s,t)][f][:] = sum over the list of (s, f) of
  *   val * g_model[t][token][:] (fp32 sums, feature-major, dense rows of d elements); with tied decoders the
  *   slot collects every pair that shares it (CLT_TYING_PER_SOURCE: all t >= s; CLT_TYING_PER_TARGET:
  *   all s <= t), so dw_packed has L matrices instead of L(L+1)/2.  One launch per target layer,
  *   in ascending order on `stream`.
+ *   With feat_offset / feat_scale ([L][F] model dtype or NULL) the values are first transformed as the
+ *   forward transforms them for target t: (val + feat_offset[t][f]) * feat_scale[t][f] on non-zero val.
+ * clt_feature_affine_grad: gradients of feat_offset / feat_scale, fp32 [L][F] (either may be NULL):
+ *   d_offset[t][f] = feat_scale[t][f] * sum h, d_scale[t][f] = sum h * (val + feat_offset[t][f]), over the
+ *   non-zero survivors of feature f in the sources s <= t, h = g[t][token] . w[slot(s,t)][f].  Call it after
+ *   clt_decode_backward_values with the SAME workspace and nnz: it reads the per-target dot products that
+ *   call left there.
+ * clt_skip_weight_grad: gradient of one skip-connection matrix (rec[t] += x[s] @ W_skip.T,
+ *   clt/models/decoder.py:297-338): out[i][j] (+)= sum over tokens of g[token][i] * x[token][j];
+ *   g [T][d] fp32 (the loss gradient of the target), x [T][d] model dtype (the source's input),
+ *   out [d][d] fp32, accumulate != 0 adds to out.
  * clt_encoder_weight_grad: dw_enc[s][f][:] = sum over the list of dval * x[s][token][:],
  *   db_enc[s][f] = sum of dval (fp32; x [L][T][d] in the model dtype).
  * Limits: d % 8 == 0 (bf16) / d % 4 == 0 (fp32) and d <= 2048.
  */
 size_t clt_mse_workspace_bytes(int64_t T, int64_t d, int64_t L);
 int clt_mse_loss_grad(const void *rec, const void *target, int64_t T, int64_t d, int64_t L,
-                      int dtype, float *loss_per_layer, float *g, void *g_model, float *bias_grad,
-                      void *workspace, size_t workspace_bytes, void *stream);
+                      int dtype, int denorm_mode, const void *mean, const void *stdv,
+                      double denorm_scale, float *loss_per_layer, float *g, void *g_model,
+                      float *bias_grad, void *workspace, size_t workspace_bytes, void *stream);
 size_t clt_decode_backward_workspace_bytes(int64_t T, int64_t L, int64_t nnz);
-int clt_decode_backward_values(const int32_t *row_ptr, const int32_t *col, const void *w_packed,
-                               const float *g, int64_t T, int64_t d, int64_t F, int64_t L,
-                               int tying, uint64_t src_mask, int64_t nnz, int dtype, float *dval,
+int clt_decode_backward_values(const int32_t *row_ptr, const int32_t *col, const void *val,
+                               const void *w_packed, const void *feat_scale, const float *g,
+                               int64_t T, int64_t d, int64_t F, int64_t L, int tying,
+                               uint64_t src_mask, int64_t nnz, int dtype, float *dval,
                                void *workspace, size_t workspace_bytes, void *stream);
+int clt_feature_affine_grad(const int32_t *list_ptr, const int32_t *list_src, const void *val,
+                            const void *feat_offset, const void *feat_scale, int64_t T, int64_t F,
+                            int64_t L, uint64_t src_mask, int64_t nnz, int dtype, float *d_offset,
+                            float *d_scale, const void *workspace, size_t workspace_bytes, void *stream);
+int clt_skip_weight_grad(const float *g, const void *x, float *out, int64_t T, int64_t d,
+                         int accumulate, int dtype, void *stream);
 size_t clt_feature_lists_workspace_bytes(int64_t F, int64_t L);
 int clt_feature_lists(const int32_t *row_ptr, const int32_t *col, int64_t T, int64_t F, int64_t L,
                       int32_t *list_ptr, int32_t *list_tok, int32_t *list_src,
                       void *workspace, size_t workspace_bytes, void *stream);
 int clt_decoder_weight_grad(const int32_t *list_ptr, const int32_t *list_tok, const int32_t *list_src,
-                            const void *val, const void *g_model, float *dw_packed,
+                            const void *val, const void *g_model, const void *feat_offset,
+                            const void *feat_scale, float *dw_packed,
                             int64_t T, int64_t d, int64_t F, int64_t L, int tying, int dtype,
                             void *stream);
 int clt_encoder_weight_grad(const int32_t *list_ptr, const int32_t *list_tok, const int32_t *list_src,

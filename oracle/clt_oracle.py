@@ -550,14 +550,21 @@ def mse_loss_and_gradients(inputs: Dict[int, torch.Tensor], targets: Dict[int, t
                            theta: Optional[torch.Tensor] = None,
                            masks: Optional[Dict[int, torch.Tensor]] = None, tying: str = "none",
                            log_threshold: Optional[torch.Tensor] = None, bandwidth: float = 1.0,
-                           model_dtype: torch.dtype = torch.float32):
-    """loss = sum over layers of nn.MSELoss()(prediction, target) (losses.py:45-92, no
-    de-normalisation statistics) through the reference's forward (decoders untied, keys "s->t", or
-    tied per source / per target, keys "i", decoder.py:176-340 without feature affine terms), and
-    d loss / d parameter from torch autograd (trainer.py:751): F.linear backward for encoder
-    and decoders, the straight-through gate of BatchTopK (activations.py:66-96: grad * mask)
-    or the pass-through part of JumpReLU's backward (activations.py:183-220: grad * 1[x >= theta];
-    the threshold's own gradient is not part of this function).  Per-layer selection, fp32.
+                           model_dtype: torch.dtype = torch.float32,
+                           normalization_method: str = "none", mean_tg: Optional[Dict[int, torch.Tensor]] = None,
+                           std_tg: Optional[Dict[int, torch.Tensor]] = None,
+                           skip_w: Optional[Dict[str, torch.Tensor]] = None,
+                           feature_offset: Optional[List[torch.Tensor]] = None,
+                           feature_scale: Optional[List[torch.Tensor]] = None):
+    """loss = sum over layers of nn.MSELoss()(prediction', target') (losses.py:45-92; ' = the
+    de-normalisation of losses.py:70-86: ``x * std + mean`` for "mean_std" with the target statistics,
+    ``x / sqrt(d_model)`` for "sqrt_d_model") through the reference's forward (decoders untied, keys
+    "s->t", or tied per source / per target, keys "i", decoder.py:176-340; skip connections
+    ``skip_w`` with the same keys, decoder.py:297-338; the target's feature offset / scale on the
+    non-zero activations of tied decoders, decoder.py:228-245, 268-285), and d loss / d parameter from
+    torch autograd (trainer.py:751): F.linear backward for encoder and decoders, the straight-through
+    gate of BatchTopK (activations.py:66-96: grad * mask) or the pass-through part of JumpReLU's backward
+    (activations.py:183-220: grad * 1[x >= theta]).  Per-layer selection, fp32.
     ``masks`` (bool [T, F] per layer) replaces the gate computed here, for comparisons in which
     the other side selected on differently rounded pre-activations.
     With ``log_threshold`` ([L, F], the parameter itself) the JumpReLU runs through
@@ -567,14 +574,25 @@ def mse_loss_and_gradients(inputs: Dict[int, torch.Tensor], targets: Dict[int, t
     Returns (loss, {state-dict key: gradient})."""
     L = num_layers
     params: Dict[str, torch.Tensor] = {}
+
+    def param(name, t):
+        params[name] = t.detach().float().clone().requires_grad_(True)
+        return params[name]
+
     if log_threshold is not None:
-        params["theta_manager.log_threshold"] = log_threshold.detach().float().clone().requires_grad_(True)
+        param("theta_manager.log_threshold", log_threshold)
     for l in range(L):
-        params[f"encoder_module.encoders.{l}.weight"] = enc_w[l].detach().float().clone().requires_grad_(True)
-        params[f"encoder_module.encoders.{l}.bias_param"] = enc_b[l].detach().float().clone().requires_grad_(True)
+        param(f"encoder_module.encoders.{l}.weight", enc_w[l])
+        param(f"encoder_module.encoders.{l}.bias_param", enc_b[l])
     for name in dec_w:
-        params[f"decoder_module.decoders.{name}.weight"] = dec_w[name].detach().float().clone().requires_grad_(True)
-        params[f"decoder_module.decoders.{name}.bias_param"] = dec_b[name].detach().float().clone().requires_grad_(True)
+        param(f"decoder_module.decoders.{name}.weight", dec_w[name])
+        param(f"decoder_module.decoders.{name}.bias_param", dec_b[name])
+    for name, w in (skip_w or {}).items():
+        param(f"decoder_module.skip_weights.{name}", w)
+    for i, v in enumerate(feature_offset or []):
+        param(f"decoder_module.feature_offset.{i}", v)
+    for i, v in enumerate(feature_scale or []):
+        param(f"decoder_module.feature_scale.{i}", v)
     acts = {}
     for l in range(L):
         pre = F.linear(inputs[l].float(), params[f"encoder_module.encoders.{l}.weight"],
@@ -594,19 +612,43 @@ def mse_loss_and_gradients(inputs: Dict[int, torch.Tensor], targets: Dict[int, t
         else:
             raise ValueError(activation_fn)
         acts[l] = pre * mask.to(pre.dtype)
+
+    def affine(a, t):
+        # the target's offset and scale act on the selected (non-zero) entries only (decoder.py:228-245)
+        if feature_offset is None and feature_scale is None:
+            return a
+        nz = (a.detach() != 0).to(a.dtype)
+        if feature_offset is not None:
+            a = a + params[f"decoder_module.feature_offset.{t}"] * nz
+        if feature_scale is not None:
+            a = a * (params[f"decoder_module.feature_scale.{t}"] * nz + (1 - nz))
+        return a
+
     loss = torch.zeros((), dtype=torch.float32)
     for t in range(L):
         rec = torch.zeros_like(targets[t], dtype=torch.float32)
         if tying == "per_target":      # one decoder per target over the summed activations, bias once
-            summed = sum(acts[s_] for s_ in range(t + 1))
+            summed = sum(affine(acts[s_], t) for s_ in range(t + 1))
             rec = F.linear(summed, params[f"decoder_module.decoders.{t}.weight"],
                            params[f"decoder_module.decoders.{t}.bias_param"])
         else:
             for s_ in range(t + 1):
                 key = f"{s_}->{t}" if tying == "none" else str(s_)
-                rec = rec + F.linear(acts[s_], params[f"decoder_module.decoders.{key}.weight"],
+                a = affine(acts[s_], t) if tying == "per_source" else acts[s_]
+                rec = rec + F.linear(a, params[f"decoder_module.decoders.{key}.weight"],
                                      params[f"decoder_module.decoders.{key}.bias_param"])
-        loss = loss + F.mse_loss(rec, targets[t].float())
+                if skip_w is not None and tying == "none":
+                    rec = rec + inputs[s_].float() @ params[f"decoder_module.skip_weights.{key}"].T
+        if skip_w is not None and tying != "none":
+            rec = rec + inputs[t].float() @ params[f"decoder_module.skip_weights.{t}"].T
+        tgt = targets[t].float()
+        if normalization_method == "mean_std" and mean_tg is not None and std_tg is not None and t in mean_tg and t in std_tg:
+            rec = rec * std_tg[t].float() + mean_tg[t].float()
+            tgt = tgt * std_tg[t].float() + mean_tg[t].float()
+        elif normalization_method == "sqrt_d_model":
+            rec = rec / (rec.shape[-1] ** 0.5)
+            tgt = tgt / (tgt.shape[-1] ** 0.5)
+        loss = loss + F.mse_loss(rec, tgt)
     loss.backward()
     return loss.detach(), {name: p.grad for name, p in params.items()}
 

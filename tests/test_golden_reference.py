@@ -88,7 +88,8 @@ def test_oracle_theta_estimation_matches_the_reference(case):
     assert torch.allclose(torch.exp(log_theta), T(case["theta"]), rtol=1e-4, atol=1e-6)     # the method's return value
 
 
-@pytest.mark.parametrize("case", FIX["gradients"], ids=lambda c: c["name"])
+@pytest.mark.parametrize("case", FIX["gradients"] + FIX["gradients_normalized"] + FIX["gradients_skip_affine"],
+                         ids=lambda c: c["name"])
 def test_oracle_gradients_match_the_reference(case):
     cfg, sd, L, tying, names, kw = unpack(case)
     fn = cfg["activation_fn"]
@@ -98,8 +99,19 @@ def test_oracle_gradients_match_the_reference(case):
     if fn == "batchtopk":      # the reference's default scope is global: the gate comes from the global helper
         pre = {l: orc.encoder_preactivations(inputs[l], kw["enc_w"][l], kw["enc_b"][l]) for l in range(L)}
         masks = {l: a != 0 for l, a in orc.global_batchtopk(pre, L, cfg["batchtopk_k"]).items()}
+    extra = {}
+    if "normalization_method" in case:      # the loss on de-normalised tensors (losses.py:70-86)
+        extra = dict(normalization_method=case["normalization_method"],
+                     mean_tg={int(l): T(v) for l, v in case["mean_tg"].items()},
+                     std_tg={int(l): T(v) for l, v in case["std_tg"].items()})
+    if cfg.get("skip_connection"):
+        extra["skip_w"] = {n: sd[f"decoder_module.skip_weights.{n}"] for n in names}
+    if cfg.get("enable_feature_offset"):
+        extra["feature_offset"] = [sd[f"decoder_module.feature_offset.{i}"] for i in range(L)]
+    if cfg.get("enable_feature_scale"):
+        extra["feature_scale"] = [sd[f"decoder_module.feature_scale.{i}"] for i in range(L)]
     loss, grads = orc.mse_loss_and_gradients(inputs, targets, **kw, activation_fn=fn, num_layers=L, k=cfg.get("batchtopk_k"),
-                                             masks=masks, tying=tying,
+                                             masks=masks, tying=tying, **extra,
                                              log_threshold=sd.get("theta_manager.log_threshold") if fn == "jumprelu" else None)
     assert float(loss) == pytest.approx(case["loss"], rel=1e-5)
     assert set(case["gradients"]) <= set(grads), set(case["gradients"]) - set(grads)

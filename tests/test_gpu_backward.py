@@ -107,8 +107,41 @@ def test_feature_lists_are_a_permutation_grouped_by_feature(dev):
             l, f = divmod(q, F)
             assert bool((col[src[b:e]] == f).all()) and bool((rows[src[b:e]] // T == l).all())
             assert torch.equal(rows[src[b:e]] % T, tok[b:e])
-            if e - b <= 64:
-                assert bool((tok[b + 1:e] > tok[b:e - 1]).all())
+            assert bool((tok[b + 1:e] > tok[b:e - 1]).all())      # token order, whatever the length
+
+
+def test_long_feature_lists_are_in_token_order_and_gradients_repeat_bit_for_bit(dev):
+    # a few features fire on most tokens: their lists are far longer than a wavefront; every list must come
+    # out in token order, and two runs of the whole backward must give the same bits
+    g = torch.Generator().manual_seed(12)
+    L, T, F = 2, 1500, 64
+    pre = torch.randn(L, T, F, generator=g)
+    pre[:, :, 5] += 6.0
+    pre[0, ::3, 17] += 6.0
+    surv = engine.batchtopk_select(pre.to(dev), 4, False)
+    ptr, tok, src = (t.cpu().long() for t in engine.feature_lists(surv))
+    lens = ptr[1:] - ptr[:-1]
+    assert int(lens.max()) > 1000 and int((lens > 64).sum()) >= 3
+    rows = engine.survivor_rows(surv).cpu().long()
+    col = surv.col.cpu().long()
+    for q in range(L * F):
+        b, e = int(ptr[q]), int(ptr[q + 1])
+        if e > b:
+            l, f = divmod(q, F)
+            assert bool((tok[b + 1:e] > tok[b:e - 1]).all())
+            assert bool((col[src[b:e]] == f).all()) and torch.equal(rows[src[b:e]], l * T + tok[b:e])
+    wl = BASE.scaled("bw-repeat", num_layers=2, d_model=128, num_features=256, tokens=2048, k=16, dtype="bfloat16")
+    model, sd, x, targets = build(wl, dev)
+    with torch.no_grad():       # two features that fire on nearly every token
+        for l in range(2):
+            model.encoder_module.encoders[l].bias_param[:2] += 8.0
+    inputs = {l: x[l].to(dev) for l in range(2)}
+    tg = {l: t.to(dev) for l, t in targets.items()}
+    _, g1 = model.loss_and_gradients(inputs, tg)
+    g1 = {k: v.clone() for k, v in g1.items()}
+    _, g2 = model.loss_and_gradients(inputs, tg)
+    for k in g1:
+        assert torch.equal(g1[k], g2[k]), k
 
 
 @pytest.mark.parametrize("tying,fn", [("none", "batchtopk"), ("per_source", "batchtopk"), ("per_target", "batchtopk"),

