@@ -352,7 +352,10 @@ class CrossLayerTranscoder(BaseTranscoder):
         glob = cfg.topk_mode != "per_layer"
         if fn == "batchtopk":
             with self._timed("batchtopk_activation") as tm:
-                surv = engine.batchtopk_select(pre, int(cfg.batchtopk_k), glob, ws)
+                # the reference times the mask computation inside its helper separately (activations.py:335-341)
+                with self._timed("batchtopk_compute_mask") as tm_mask:
+                    surv = engine.batchtopk_select(pre, int(cfg.batchtopk_k), glob, ws)
+                self._record("batchtopk_compute_mask", tm_mask)
             self._record("batchtopk_activation", tm)
             return surv
         if fn == "topk":

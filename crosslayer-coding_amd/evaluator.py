@@ -103,12 +103,19 @@ class CLTEvaluator:
         nat.require_device(dense, "CLTEvaluator")
         return layers, engine.threshold_select(dense, None, nat.PRED_NONZERO)
 
-    def _counts(self, activations):
+    def _counts(self, activations, present: Optional[List[int]] = None):
+        """(layers, tokens, entries != 0 per layer, firing tokens per (layer, feature)).  ``present``: the
+        layers the batch really held, when ``activations`` is a survivor list over all num_layers with
+        empty rows for the others: the reference's metrics run over the layers get_feature_activations
+        returned (evaluator.py:194-244, 350-405), so the absent ones must not enter the averages."""
         got = self._as_survivors(activations)
         if got is None:
             return None
         layers, surv = got
         nonzero, fired = engine.survivor_metrics(surv, FIRED_EPS)
+        if present is not None and list(present) != layers:
+            idx = torch.tensor([layers.index(l) for l in present], device=nonzero.device)
+            layers, nonzero, fired = list(present), nonzero[idx], fired[idx]
         return layers, surv.T, nonzero, fired
 
     # ---- metrics (evaluator.py:194-244) ----
@@ -211,7 +218,8 @@ class CLTEvaluator:
         else:
             reconstructions = self.model(inputs)
             activations = self.model.get_feature_activations(inputs)
-        counts = self._counts(activations) if _has_data(activations) else None
+        present = sorted(inputs) if res is not None else None
+        counts = self._counts(activations, present) if _has_data(activations) else None
         sparsity = self._compute_sparsity(activations, counts)
         reconstruction = self._compute_reconstruction_metrics(targets, reconstructions)
         density = self._compute_feature_density(activations, counts)

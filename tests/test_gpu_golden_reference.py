@@ -274,6 +274,31 @@ def test_compute_metrics_end_to_end_matches_the_reference(dev):
     same(got, want, "metrics")
 
 
+def test_compute_metrics_on_a_subset_of_layers_matches_the_reference(dev):
+    # a batch that holds only layers 0 and 2 of 4: averages, per-layer entries and histograms run over those two
+    case = FIX["compute_metrics_subset"]
+    model = load_model(case, dev)
+    model.eval()
+    ev = cca.CLTEvaluator(model, dev)
+    got = ev.compute_metrics({int(l): T(v) for l, v in case["inputs"].items()}, {int(l): T(v) for l, v in case["targets"].items()})
+    want = case["metrics"]
+    assert got.keys() == want.keys(), (sorted(got), sorted(want))
+
+    def same(a, b, path):
+        if isinstance(b, dict):
+            assert a.keys() == b.keys(), (path, sorted(a), sorted(b))
+            for k in b:
+                same(a[k], b[k], f"{path}/{k}")
+        elif isinstance(b, list):
+            assert len(a) == len(b), path
+            for i, (x, y) in enumerate(zip(a, b)):
+                same(x, y, f"{path}[{i}]")
+        else:
+            assert a == pytest.approx(b, rel=1e-4, abs=1e-6) or (math.isinf(a) and math.isinf(b)), (path, a, b)
+
+    same(got, want, "metrics")
+
+
 @pytest.mark.parametrize("scope", ["global", "per_layer"])
 def test_full_size_c0_against_the_reference_summary(dev, scope):
     # C0 (fp32, 12 x 768 x 6144, 1024 tokens, k = 200) went through the reference once, on the weights and

@@ -333,6 +333,31 @@ def test_batchtopk_global(dev, dtype, L, T, F, k):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("L,T,F,k", [(4, 200, 520, 12), (3, 512, 2048, 20)])
+def test_batchtopk_global_is_bit_exact_given_the_column_statistics(dev, dtype, L, T, F, k):
+    # The only thing that can differ between two correct implementations of the global helper is the last
+    # bit of the per-feature mean / std reductions.  Given the statistics the kernel itself used, the ranking
+    # values are fixed (each step rounded to the model dtype, activations.py:283) and the selection must be
+    # exactly the k*T largest of them over the [T, L*F] block, ties to the lowest flat index.
+    g = torch.Generator().manual_seed(L * 7 + F)
+    pre = (torch.randn(L, T, F, generator=g) * (1 + torch.arange(L).view(L, 1, 1))).to(dtype)
+    if dtype == torch.bfloat16:
+        pre[1, :, 5] = pre[0, :, 5]                 # equal columns: equal z-scores, ties across layers
+    pre_dev = pre.to(dev)
+    mean, denom = engine.colstats(pre_dev)
+    surv = engine.batchtopk_select(pre_dev, k, True, stats=(mean, denom))
+    check_rows_sorted(surv)
+    got = dense_from(surv) != 0
+    mean, denom = mean.cpu(), denom.cpu()
+    z = torch.cat([((pre[l].float() - mean[l]).to(dtype).float() / denom[l]).to(dtype).float() for l in range(L)], dim=1)
+    order = torch.sort(z.reshape(-1), descending=True, stable=True).indices[:k * T]
+    want = torch.zeros(T * L * F, dtype=torch.bool)
+    want[order] = True
+    want = torch.stack([want.view(T, L * F)[:, l * F:(l + 1) * F] for l in range(L)])
+    assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_batchtopk_global_outlier_tokens(dev, dtype):
     # two tokens stand far out of the batch in every feature: under the batch-wide cut nearly all of
     # their values are candidates, more per step of the streaming pass than its buffer holds

@@ -275,3 +275,37 @@ def test_threshold_forward_recovers_when_the_survivors_outgrow_the_arrays(dev, c
     back = model(inputs)
     for t in range(L):
         assert torch.equal(back[t], want_small[t])
+
+
+def test_profiler_hook_receives_the_reference_timer_names(dev):
+    # the `profiler=` argument of the constructor (clt.py:30-36): timers "batchtopk_activation" (clt.py:254-257)
+    # and, inside the global helper, "batchtopk_compute_mask" (activations.py:335-341)
+    class Timer:
+        def __init__(self):
+            self.elapsed = 0.0
+
+        def __enter__(self):
+            return self
+
+        def __exit__(self, *exc):
+            self.elapsed = 1.0
+            return False
+
+    class Profiler:
+        def __init__(self):
+            self.records = []
+
+        def timer(self, name):
+            return Timer()
+
+        def record(self, name, elapsed):
+            self.records.append(name)
+
+    wl = next(c for c in CASES if c.name == "tiny-global")
+    x = synth.make_inputs(wl, "cpu")
+    sd = synth.make_state_dict(wl, "cpu", inputs=x)
+    prof = Profiler()
+    model = cca.CrossLayerTranscoder(wl.config(), None, dev, profiler=prof)
+    model.load_state_dict(sd)
+    model({l: x[l].to(dev) for l in range(wl.num_layers)})
+    assert "batchtopk_activation" in prof.records and "batchtopk_compute_mask" in prof.records
