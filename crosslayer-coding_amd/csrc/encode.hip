@@ -19,6 +19,7 @@
 //   bf16        v_mfma_f32_32x32x16_bf16, fp32 accumulate, one rounding (v_cvt_pk_bf16_f32)
 //   fp32        v_mfma_f32_32x32x2_f32
 #include <type_traits>
+#include <cstdlib>
 #include "select_state.h"
 
 namespace {
@@ -30,7 +31,9 @@ constexpr int BM = 256;   // tokens per block
 constexpr int BN = 256;   // features per block
 constexpr int ROWB = 128; // bytes of K per LDS row
 constexpr int STAGE = (BM + BN) * ROWB;  // bytes of one LDS stage
-constexpr int CAND_LIST = 2048;          // candidates of one wave tile the collecting epilogue lists in LDS
+constexpr int NWAVES = 8;                // wavefronts per block (4 x 2, wave tile 64 tokens x 128 features): two per SIMD
+constexpr int NTHREADS = NWAVES * 64;
+constexpr int CAND_LIST = 512;           // candidates of one 32-token piece the collecting epilogue lists in LDS
 constexpr int ENC_SN = 8;  // feature tiles x token tiles that one XCD works on at a time
 constexpr int ENC_SM = 4;
 
@@ -126,58 +129,82 @@ __device__ __forceinline__ uint32_t wave_inclusive_scan32(uint32_t v) {
 // candidate pool per wavefront and feature segment (see CollectArgs).  These modes need
 // M % BM == 0 and N % BN == 0 (a shifted tile would report its overlap twice).
 template <typename T, int COLLECT>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void k_encode_mfma(
+__global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void k_encode_mfma(
     const T *__restrict__ x, const T *__restrict__ w, const T *__restrict__ bias, T *__restrict__ pre,
-    int M, int K, int N, int tiles_m, int tiles_n, int64_t xs, int64_t wstr, int64_t bs, int64_t ps,
-    const SelState *__restrict__ gate, CollectArgs ca) {
+    int M, int K, int N, int tiles_m, int tiles_n, int total_tiles, int64_t xs, int64_t wstr, int64_t bs,
+    int64_t ps, const SelState *__restrict__ gate, CollectArgs ca) {
   constexpr int CE = 16 / (int)sizeof(T);  // elements per 16-byte chunk
   constexpr int BK = ROWB / (int)sizeof(T);
+  // The collecting modes run as persistent workgroups (the grid is one block per CU, block b takes the
+  // tiles b, b + gridDim.x, ...) and overlap the start of the next tile with the end of this one: their
+  // epilogue parks only in the second stage buffer, 32 tokens of a wave tile at a time, so the first
+  // stage of the next tile is asked for two stages before this tile's K loop ends and has landed when
+  // the epilogue is over.  The storing mode parks whole wave tiles in both buffers, one tile per block.
+  constexpr bool OVERLAP = COLLECT != 0;
   // Two separate stage buffers (not one array with an offset): the compiler can then tell that
   // a fragment read of one stage does not depend on the direct-to-LDS loads in flight into the
   // other, and does not wait for them.
   __shared__ __attribute__((aligned(16))) unsigned char stage0[STAGE];
   __shared__ __attribute__((aligned(16))) unsigned char stage1[STAGE];
-  __shared__ uint16_t cand_list[COLLECT ? 4 : 1][COLLECT ? CAND_LIST : 1];   // per wavefront, see the emission
+  __shared__ uint16_t cand_list[COLLECT ? NWAVES : 1][COLLECT ? CAND_LIST : 1];   // per wavefront, see the emission
+  __shared__ __attribute__((aligned(16))) T bias_lds[NWAVES][128];                // per wavefront: the bias of its features
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave & 1, wn = wave >> 1;
-  int bid = blockIdx.x;
+  const int wm = wave & 3, wn = wave >> 2;   // wave tile: tokens [64 wm, +64) x features [128 wn, +128)
   const int per_layer = tiles_m * tiles_n;
-  const int layer = bid / per_layer;
-  bid -= layer * per_layer;
-  if (COLLECT == 0 && gate && gate[layer].status != ST_RETRY) return;
-  int tn, tm;
-  if ((tiles_n & 7) == 0) {
-    // XCD x owns the feature tiles n = x, x+8, ...  Its tiles run in groups of ENC_SN feature tiles
-    // x ENC_SM token tiles (about one tile per CU of the XCD): the group's W tiles stay in the L2
-    // while the token groups sweep past, so W is fetched once and the x slab once per ENC_SN tiles.
-    const int xcd = bid & 7, idx = bid >> 3, nloc = tiles_n >> 3;
-    const int g = idx / (ENC_SN * tiles_m), r = idx - g * ENC_SN * tiles_m;
-    const int cnt = (nloc - g * ENC_SN) < ENC_SN ? (nloc - g * ENC_SN) : ENC_SN;
-    const int mg = r / (cnt * ENC_SM), r2 = r - mg * cnt * ENC_SM;
-    tm = mg * ENC_SM + r2 / cnt;
-    tn = (g * ENC_SN + r2 % cnt) * 8 + xcd;
-  } else {
-    tn = bid / tiles_m; tm = bid - tn * tiles_m;
-  }
-  int m0 = tm * BM, n0 = tn * BN;
-  if (m0 + BM > M) m0 = M - BM;
-  if (n0 + BN > N) n0 = N - BN;
+  const int nk = K / BK;
 
-  // ---- loader: wave `wave` brings in rows [64*wave, 64*wave+64) of both tiles, 8 rows (1 KB)
+  struct TileAt { int layer, tm, tn, m0, n0, rot; };
+  auto locate = [&](int bid) {
+    TileAt t;
+    t.layer = bid / per_layer;
+    bid -= t.layer * per_layer;
+    if ((tiles_n & 7) == 0) {
+      // XCD x owns the feature tiles n = x, x+8, ...  Its tiles run in groups of ENC_SN feature tiles
+      // x ENC_SM token tiles (about one tile per CU of the XCD): the group's W tiles stay in the L2
+      // while the token groups sweep past, so W is fetched once and the x slab once per ENC_SN tiles.
+      const int xcd = bid & 7, idx = bid >> 3, nloc = tiles_n >> 3;
+      const int g = idx / (ENC_SN * tiles_m), r = idx - g * ENC_SN * tiles_m;
+      const int cnt = (nloc - g * ENC_SN) < ENC_SN ? (nloc - g * ENC_SN) : ENC_SN;
+      const int mg = r / (cnt * ENC_SM), r2 = r - mg * cnt * ENC_SM;
+      t.tm = mg * ENC_SM + r2 / cnt;
+      t.tn = (g * ENC_SN + r2 % cnt) * 8 + xcd;
+    } else {
+      t.tn = bid / tiles_m; t.tm = bid - t.tn * tiles_m;
+    }
+    t.m0 = t.tm * BM; t.n0 = t.tn * BN;
+    if (t.m0 + BM > M) t.m0 = M - BM;
+    if (t.n0 + BN > N) t.n0 = N - BN;
+    // K is walked from a tile-dependent starting stage, wrapping around: the CUs of an XCD that share an
+    // x tile or a W tile then ask for different lines of it at any one time, so one of them takes the
+    // L2 miss and the others find the line there later, instead of all of them queueing behind the miss.
+    t.rot = ((tiles_n & 7) == 0 ? 3 * t.tm + (t.tn >> 3) : t.tm + t.tn) % nk;
+    return t;
+  };
+  // the storing mode computes only the layers that asked for it when a gate is given
+  auto wanted = [&](int bid) {
+    if (COLLECT != 0 || !gate) return true;
+    return gate[bid / per_layer].status == ST_RETRY;
+  };
+  int bid = blockIdx.x;
+  while (bid < total_tiles && !wanted(bid)) bid += gridDim.x;
+  if (bid >= total_tiles) return;
+
+  // ---- loader: wave `wave` brings in rows [32*wave, 32*wave+32) of both tiles, 8 rows (1 KB)
   // per instruction.  Lane l lands at row l>>3, chunk position l&7 of its 8-row group and
   // therefore fetches global chunk (l&7) ^ ((row >> 1) & 7).
   const int lr = lane >> 3, lp = lane & 7;
   const int offE = lr * K + ((lp ^ (lane >> 4)) * CE);          // 8-row groups starting at a multiple of 16
   const int offO = lr * K + ((lp ^ ((lane >> 4) | 4)) * CE);    // ... at 8 mod 16
-  const T *xt = x + (int64_t)layer * xs + (int64_t)(m0 + wave * 64) * K;
-  const T *wt = w + (int64_t)layer * wstr + (int64_t)(n0 + wave * 64) * K;
-  auto issue_stage = [&](unsigned char *stage, int k0) {
-    unsigned char *xs_l = stage + wave * 64 * ROWB;
+  auto x_rows = [&](const TileAt &t) { return x + (int64_t)t.layer * xs + (int64_t)(t.m0 + wave * 32) * K; };
+  auto w_rows = [&](const TileAt &t) { return w + (int64_t)t.layer * wstr + (int64_t)(t.n0 + wave * 32) * K; };
+  auto stage_k0 = [&](const TileAt &t, int kt) { int q = kt + t.rot; if (q >= nk) q -= nk; return q * BK; };
+  auto issue_stage = [&](unsigned char *stage, const T *xt, const T *wt, int k0) {
+    unsigned char *xs_l = stage + wave * 32 * ROWB;
     unsigned char *ws_l = xs_l + BM * ROWB;
 #pragma unroll
-    for (int t = 0; t < 8; ++t) {
+    for (int t = 0; t < 4; ++t) {
       const int off = (t & 1) ? offO : offE;
       load16_to_lds(xt + (int64_t)t * 8 * K + k0 + off, xs_l + t * 8 * ROWB);
       load16_to_lds(wt + (int64_t)t * 8 * K + k0 + off, ws_l + t * 8 * ROWB);
@@ -186,7 +213,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 
   // ---- fragment reader: row l31 of each 32-row group; chunk (kk*2 + lh) at its swizzled position
   const int l31 = lane & 31, lh = lane >> 5;
-  const int xrow = (wm * 128 + l31) * ROWB;             // + i * 32 * ROWB
+  const int xrow = (wm * 64 + l31) * ROWB;              // + i * 32 * ROWB
   const int wrow = BM * ROWB + (wn * 128 + l31) * ROWB; // + j * 32 * ROWB
   int koff[4];
 #pragma unroll
@@ -194,37 +221,38 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 
   // The accumulators start from the bias (the matrix core adds its products onto them in fp32), so
   // the epilogue has no bias loads or adds: accumulator (j, rg*4+q) of a lane belongs to feature
-  // j*32 + rg*8 + (lane>>5)*4 + q of the wave tile, whatever the token group i.  The bias is asked
-  // for here, ahead of the first stage, and lands in the accumulators while the second stage loads.
-  f32x16_t acc[4][4];
-  typedef typename std::conditional<sizeof(T) == 4, float4, uint2>::type bias4_t;
-  bias4_t braw[16];
-  {
-    const T *bl = bias ? bias + (int64_t)layer * bs + n0 + wn * 128 + (lane >> 5) * 4 : nullptr;
-#pragma unroll
-    for (int g = 0; g < 16; ++g) {
-      if (bl) braw[g] = *reinterpret_cast<const bias4_t *>(bl + g * 8);
-      else if constexpr (sizeof(T) == 4) braw[g] = make_float4(0.f, 0.f, 0.f, 0.f);
-      else braw[g] = make_uint2(0u, 0u);
-    }
-  }
+  // j*32 + rg*8 + (lane>>5)*4 + q of the wave tile, whatever the token group i.  Each wavefront brings
+  // the bias of its 128 features into LDS with one direct load ahead of the tile's stages - no register
+  // holds it while the previous tile's epilogue runs - and reads it from there when the first stage has
+  // landed.
+  f32x16_t acc[2][4];
+  constexpr int BIAS_LANES = 128 * (int)sizeof(T) / 16;   // lanes of the one 16-byte-per-lane load
+  auto load_bias = [&](const TileAt &t) {
+    if (bias && lane < BIAS_LANES)
+      load16_to_lds(bias + (int64_t)t.layer * bs + t.n0 + wn * 128 + lane * CE, bias_lds[wave]);
+  };
+  if (!bias && lane < BIAS_LANES)   // no bias: the slot holds zeros for good
+    *reinterpret_cast<uint4 *>(reinterpret_cast<unsigned char *>(bias_lds[wave]) + lane * 16) = make_uint4(0u, 0u, 0u, 0u);
   auto init_acc = [&]() {
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
       for (int rg = 0; rg < 4; ++rg) {
         float bv[4];
+        const T *bp = bias_lds[wave] + j * 32 + rg * 8 + (lane >> 5) * 4;
         if constexpr (sizeof(T) == 4) {
-          bv[0] = braw[j * 4 + rg].x; bv[1] = braw[j * 4 + rg].y; bv[2] = braw[j * 4 + rg].z; bv[3] = braw[j * 4 + rg].w;
+          const float4 r = *reinterpret_cast<const float4 *>(bp);
+          bv[0] = r.x; bv[1] = r.y; bv[2] = r.z; bv[3] = r.w;
         } else {
-          bv[0] = __uint_as_float(braw[j * 4 + rg].x << 16); bv[1] = __uint_as_float(braw[j * 4 + rg].x & 0xFFFF0000u);
-          bv[2] = __uint_as_float(braw[j * 4 + rg].y << 16); bv[3] = __uint_as_float(braw[j * 4 + rg].y & 0xFFFF0000u);
+          const uint2 r = *reinterpret_cast<const uint2 *>(bp);
+          bv[0] = __uint_as_float(r.x << 16); bv[1] = __uint_as_float(r.x & 0xFFFF0000u);
+          bv[2] = __uint_as_float(r.y << 16); bv[3] = __uint_as_float(r.y & 0xFFFF0000u);
         }
-        // pins the copies into the accumulators here, behind the wait, instead of at the loads
+        // pins the copies into the accumulators here instead of at the reads
 #pragma unroll
         for (int q = 0; q < 4; ++q) asm volatile("" : "+v"(bv[q]));
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < 2; ++i)
 #pragma unroll
           for (int q = 0; q < 4; ++q) acc[i][j][rg * 4 + q] = bv[q];
       }
@@ -236,148 +264,173 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   // the next stage have landed and its LDS reads of the current stage are complete, so after
   // the barrier the next stage may be read (its first fragments are fetched under the last
   // k-step's matrix ops) and the current one may be overwritten by the stage after next.
-  const int nk = K / BK;
-  // K is walked from a tile-dependent starting stage, wrapping around: the CUs of an XCD that share an
-  // x tile or a W tile then ask for different lines of it at any one time, so one of them takes the
-  // L2 miss and the others find the line there later, instead of all of them queueing behind the miss.
-  const int rot = ((tiles_n & 7) == 0 ? 3 * tm + (tn >> 3) : tm + tn) % nk;
-  auto stage_k0 = [&](int kt) { int q = kt + rot; if (q >= nk) q -= nk; return q * BK; };
-  uint4 fa[8], fb[8];   // [0..3] x fragments, [4..7] W fragments
-  auto load_frags = [&](uint4 (&f)[8], const unsigned char *sb, int kk) {
+  uint4 fa[6], fb[6];   // [0..1] x fragments, [2..5] W fragments
+  auto load_frags = [&](uint4 (&f)[6], const unsigned char *sb, int kk) {
     // in the order the matrix ops of the next k-step want them: x0 and all of W first
     f[0] = *reinterpret_cast<const uint4 *>(sb + xrow + koff[kk]);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) f[4 + j] = *reinterpret_cast<const uint4 *>(sb + wrow + j * 32 * ROWB + koff[kk]);
-#pragma unroll
-    for (int i = 1; i < 4; ++i) f[i] = *reinterpret_cast<const uint4 *>(sb + xrow + i * 32 * ROWB + koff[kk]);
+    for (int j = 0; j < 4; ++j) f[2 + j] = *reinterpret_cast<const uint4 *>(sb + wrow + j * 32 * ROWB + koff[kk]);
+    f[1] = *reinterpret_cast<const uint4 *>(sb + xrow + 32 * ROWB + koff[kk]);
   };
-  auto mma16 = [&](const uint4 (&f)[8]) {
+  auto mma8 = [&](const uint4 (&f)[6]) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < 2; ++i)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) Mma<T>::run(acc[i][j], f[4 + j], f[i]);
+      for (int j = 0; j < 4; ++j) Mma<T>::run(acc[i][j], f[2 + j], f[i]);
   };
-  // interleave hint: the eight LDS reads go out behind the first matrix ops of the k-step, one
-  // apiece, so that the last of them has half a k-step to arrive before the next k-step waits for it
+  constexpr int MPI = sizeof(T) == 2 ? 1 : 4;   // matrix instructions per Mma::run
+  // interleave hint: the six LDS reads go out behind the first matrix ops of the k-step, one apiece
   auto mix_ds = [&]() {
 #pragma unroll
-    for (int g = 0; g < 8; ++g) {
-      __builtin_amdgcn_sched_group_barrier(0x008, sizeof(T) == 2 ? 1 : 4, 0);
+    for (int g = 0; g < 6; ++g) {
+      __builtin_amdgcn_sched_group_barrier(0x008, MPI, 0);
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
     }
-    __builtin_amdgcn_sched_group_barrier(0x008, sizeof(T) == 2 ? 8 : 32, 0);
+    __builtin_amdgcn_sched_group_barrier(0x008, 2 * MPI, 0);
   };
-  // one stage except its last k-step, the barrier, then the last k-step overlapped with the
-  // loads of the stage after next (into `cur`) and the first fragments of `nxt`
-  auto body = [&](unsigned char *cur, unsigned char *nxt, int kt) {
-    load_frags(fb, cur, 1); mma16(fa); mix_ds();
-    load_frags(fa, cur, 2); mma16(fb); mix_ds();
-    load_frags(fb, cur, 3); mma16(fa); mix_ds();
+  // one stage except its last k-step, the barrier, then the last k-step overlapped with the loads that
+  // `refill` asks for (the stage after next, into `cur`) and, unless this is the tile's last stage,
+  // the first fragments of `nxt`
+  auto body = [&](unsigned char *cur, unsigned char *nxt, bool last, auto refill) {
+    load_frags(fb, cur, 1); mma8(fa); mix_ds();
+    load_frags(fa, cur, 2); mma8(fb); mix_ds();
+    load_frags(fb, cur, 3); mma8(fa); mix_ds();
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
-    // past the end of K the last stage is fetched again (never read)
-    const int kn = kt + 2 < nk ? kt + 2 : nk - 1;
-    issue_stage(cur, stage_k0(kn));
-    load_frags(fa, nxt, 0);
-    mma16(fb);
+    refill();
+    if (!last) load_frags(fa, nxt, 0);
+    mma8(fb);
 #pragma unroll
-    for (int g = 0; g < 16; ++g) {
-      __builtin_amdgcn_sched_group_barrier(0x008, sizeof(T) == 2 ? 1 : 4, 0);
-      if (g < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    for (int g = 0; g < 8; ++g) {
+      __builtin_amdgcn_sched_group_barrier(0x008, MPI, 0);
+      if (g < 6) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
     }
   };
-  // both stage buffers are free at this point: the second stage is asked for right behind the first,
-  // and only the first (this wavefront's 16 older loads, and the bias before them) is waited for
-  issue_stage(stage0, stage_k0(0));
-  issue_stage(stage1, stage_k0(1));
-  __builtin_amdgcn_sched_barrier(0);
-  __builtin_amdgcn_s_waitcnt(0x4F70);   // vmcnt(16): at most the 16 loads of the second stage outstanding
-  // a bare barrier between two compiler-only fences: the fences of __syncthreads() would wait for the
-  // second stage too
-  asm volatile("" ::: "memory");
-  __builtin_amdgcn_s_barrier();
-  asm volatile("" ::: "memory");
-  __builtin_amdgcn_sched_barrier(0);    // nothing that reads the bias may move above the wait
-  init_acc();
-  load_frags(fa, stage0, 0);
-  // nk is even (checked by the launcher).  The last two bodies fetch the final stage again and
-  // read fragments that are never used: cheaper than a differently shaped last iteration.
-  for (int kt = 0; kt < nk; kt += 2) { body(stage0, stage1, kt); body(stage1, stage0, kt + 1); }
-  __builtin_amdgcn_s_waitcnt(0);   // no direct-to-LDS load may be in flight when the block retires
 
-  // ---- epilogue.  The accumulator layout gives a lane 4 consecutive features of one token,
-  // i.e. 8-byte pieces scattered over 32 rows per store - slow to write.  Each wavefront
-  // therefore parks its 128 x 128 tile in LDS (the stage buffers are free now; 32 KB per
-  // wavefront for bf16, two passes of 64 features for fp32) and writes it out row by row,
-  // 16 bytes per lane, 256 contiguous bytes per token.
-  __syncthreads();   // every wavefront is done with the last stage
-  T *pl = pre + (int64_t)layer * ps;
-  unsigned char *park = (wave < 2 ? stage0 : stage1) + (wave & 1) * (STAGE / 2);
-  constexpr int NPASS = sizeof(T) == 2 ? 1 : 2;           // feature halves per pass
-  constexpr int JP = 4 / NPASS;                            // 32-feature groups per pass
+  TileAt cur = locate(bid);
+  // both stage buffers are free at this point: the bias, then the first stage, then the second
+  load_bias(cur);
+  __builtin_amdgcn_sched_barrier(0);
+  issue_stage(stage0, x_rows(cur), w_rows(cur), stage_k0(cur, 0));
+  issue_stage(stage1, x_rows(cur), w_rows(cur), stage_k0(cur, 1));
+
+  for (;;) {
+    int nbid = bid + (int)gridDim.x;
+    while (nbid < total_tiles && !wanted(nbid)) nbid += gridDim.x;
+    const bool has_next = nbid < total_tiles;
+    const TileAt nxt_tile = locate(has_next ? nbid : bid);
+    const T *xt = x_rows(cur), *wt = w_rows(cur);
+    const int m0 = cur.m0, n0 = cur.n0, layer = cur.layer;
+
+    // only the first stage (this wavefront's 8 older loads, and the bias load before them) is waited for:
+    // at most the 8 loads of the second stage stay outstanding
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_waitcnt(0x0F78);   // vmcnt(8)
+    // a bare barrier between two compiler-only fences: the fences of __syncthreads() would wait for the
+    // second stage too
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);    // nothing that reads the bias may move above the wait
+    init_acc();
+    load_frags(fa, stage0, 0);
+    // nk is even (checked by the launcher)
+    for (int kt = 0; kt < nk - 2; kt += 2) {
+      body(stage0, stage1, false, [&]() { issue_stage(stage0, xt, wt, stage_k0(cur, kt + 2)); });
+      body(stage1, stage0, false, [&]() { issue_stage(stage1, xt, wt, stage_k0(cur, kt + 3)); });
+    }
+    // the last two stages: the first buffer is free after the first of them and takes the next tile's
+    // first stage (overlapping modes); nothing may be in flight into the second one, which is parked in
+    body(stage0, stage1, false, [&]() {
+      if (OVERLAP && has_next) issue_stage(stage0, x_rows(nxt_tile), w_rows(nxt_tile), stage_k0(nxt_tile, 0));
+    });
+    body(stage1, stage0, true, [&]() {});
+    // past the barrier of the last stage no wavefront reads either buffer any more
+
+    // ---- epilogue.  The accumulator layout gives a lane 4 consecutive features of one token,
+    // i.e. 8-byte pieces scattered over 32 rows per store - slow to write.  Each wavefront
+    // therefore parks its tile in LDS and works on it row by row from there: the storing mode the
+    // whole 64 x 128 tile (16 KB per wavefront for bf16, two passes of 64 features for fp32) in its
+    // eighth of the two stage buffers, the collecting modes 32 tokens at a time (8 KB) in its eighth
+    // of the second buffer.
+    T *pl = pre + (int64_t)layer * ps;
+    // The epilogue's addresses are rebuilt from the lane number for every tile.  Left visible as loop
+    // invariants they would be computed once ahead of the tile loop and live across the K loop.
+    int lane_e = lane;
+    asm volatile("" : "+v"(lane_e));
+    const int l31 = lane_e & 31, lh = lane_e >> 5;
+    unsigned char *park = OVERLAP ? stage1 + wave * (STAGE / 8) : (wave < 4 ? stage0 : stage1) + (wave & 3) * (STAGE / 4);
+    constexpr int NPASS = sizeof(T) == 2 ? 1 : 2;           // feature halves per pass
+    constexpr int JP = 4 / NPASS;                            // 32-feature groups per pass
+    // token groups [i0, i0 + ni) of feature pass `pass` -> rows (i - i0) * 32 + l31 of 256 bytes
+    // (128 bf16 / 64 fp32), 16-byte slots XOR-swizzled with the row
+    auto park_rows = [&](int pass, int i0, int ni) {
 #pragma unroll
-  for (int pass = 0; pass < NPASS; ++pass) {
-    // rows of 256 bytes (128 bf16 / 64 fp32), 16-byte slots XOR-swizzled with the token
+      for (int jj = 0; jj < JP; ++jj) {
+        const int j = pass * JP + jj;
 #pragma unroll
-    for (int jj = 0; jj < JP; ++jj) {
-      const int j = pass * JP + jj;
+        for (int rg = 0; rg < 4; ++rg) {
+          const int nl = jj * 32 + rg * 8 + lh * 4;          // feature inside this pass
 #pragma unroll
-      for (int rg = 0; rg < 4; ++rg) {
-        const int nl = jj * 32 + rg * 8 + lh * 4;          // feature inside this pass
+          for (int ii = 0; ii < ni; ++ii) {
+            const int i = i0 + ii;
+            const int ml = ii * 32 + l31;                    // row inside the parked piece
+            float y[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int ml = i * 32 + l31;                     // token inside the wave tile
-          float y[4];
-#pragma unroll
-          for (int q = 0; q < 4; ++q) y[q] = acc[i][j][rg * 4 + q];
-          if (sizeof(T) == 4) {
-            const int slot = (nl >> 2) ^ (ml & 15);
-            *reinterpret_cast<float4 *>(park + ml * 256 + slot * 16) = make_float4(y[0], y[1], y[2], y[3]);
-          } else {
-            const int slot = (nl >> 3) ^ (ml & 15);
-            uint2 o;
-            o.x = pack_bf16x2(y[0], y[1]);
-            o.y = pack_bf16x2(y[2], y[3]);
-            *reinterpret_cast<uint2 *>(park + ml * 256 + slot * 16 + (nl & 4) * 2) = o;
+            for (int q = 0; q < 4; ++q) y[q] = acc[i][j][rg * 4 + q];
+            if (sizeof(T) == 4) {
+              const int slot = (nl >> 2) ^ (ml & 15);
+              *reinterpret_cast<float4 *>(park + ml * 256 + slot * 16) = make_float4(y[0], y[1], y[2], y[3]);
+            } else {
+              const int slot = (nl >> 3) ^ (ml & 15);
+              uint2 o;
+              o.x = pack_bf16x2(y[0], y[1]);
+              o.y = pack_bf16x2(y[2], y[3]);
+              *reinterpret_cast<uint2 *>(park + ml * 256 + slot * 16 + (nl & 4) * 2) = o;
+            }
           }
         }
       }
-    }
-    // the wavefront reads its own tile back: lane -> (row = it*4 + lane/16, slot = lane%16)
+    };
     constexpr int EPS = 16 / (int)sizeof(T);               // elements per 16-byte slot
-    if constexpr (COLLECT == 0) {
+#pragma unroll
+    for (int pass = 0; pass < NPASS; ++pass) {
+      if constexpr (COLLECT == 0) {
+        park_rows(pass, 0, 2);
+        // the wavefront reads its own tile back: lane -> (row = it*4 + lane/16, slot = lane%16)
 #pragma unroll 4
-      for (int it = 0; it < 32; ++it) {
-        const int ml = it * 4 + (lane >> 4), sl = lane & 15;
-        const uint4 v = *reinterpret_cast<const uint4 *>(park + ml * 256 + ((sl ^ (ml & 15)) * 16));
-        const int m = m0 + wm * 128 + ml;
-        const int n = n0 + wn * 128 + pass * (128 / NPASS) + sl * EPS;
-        *reinterpret_cast<uint4 *>(pl + (int64_t)m * N + n) = v;
-      }
-    } else {
-      // lane -> token row (two rows per lane, 64 apart): counting and ordering inside a row
-      // need no cross-lane work, and the per-row bookkeeping is written 64 rows at a time
-      constexpr int KB = Elem<T>::KEYBITS;
-      constexpr int SEGW = 128 / NPASS;                    // features per segment (16 slots)
-      constexpr int NW = SEGW / 32;                        // 32-bit mask words per row
-      const int ncol0 = n0 + wn * 128 + pass * SEGW;       // first feature of the segment
-      uint32_t cut_bits = 0;
-      if constexpr (COLLECT == 1) cut_bits = key_to_f32_bits<KB>(ca.st[layer].cut_key);
-      const bool cut_nan = (cut_bits & 0x7FFFFFFFu) > 0x7F800000u;   // only NaNs reach such a cut
-      const float cutf = __uint_as_float(cut_bits);
-      uint32_t W[2][NW];
-      uint32_t cnt[2];
-      // generic: float compares, element by element; bit c of a row's mask = column c
-      auto scan_generic = [&]() {
+        for (int it = 0; it < 16; ++it) {
+          const int ml = it * 4 + (lane_e >> 4), sl = lane_e & 15;
+          const uint4 v = *reinterpret_cast<const uint4 *>(park + ml * 256 + ((sl ^ (ml & 15)) * 16));
+          const int m = m0 + wm * 64 + ml;
+          const int n = n0 + wn * 128 + pass * (128 / NPASS) + sl * EPS;
+          *reinterpret_cast<uint4 *>(pl + (int64_t)m * N + n) = v;
+        }
+      } else {
+        // Two lanes per token row of the parked piece: lane -> row lane % 32, slots [8 hs, 8 hs + 8) with
+        // hs = lane / 32.  Counting and ordering inside a half row need no cross-lane work; the two halves
+        // of a row meet through one lane exchange.
+        constexpr int KB = Elem<T>::KEYBITS;
+        constexpr int SEGW = 128 / NPASS;                    // features per segment (16 slots)
+        constexpr int NWL = SEGW / 64;                       // 32-bit mask words per lane (half a row)
+        const int ncol0 = n0 + wn * 128 + pass * SEGW;       // first feature of the segment
+        uint32_t cut_bits = 0;
+        if constexpr (COLLECT == 1) cut_bits = key_to_f32_bits<KB>(ca.st[layer].cut_key);
+        const bool cut_nan = (cut_bits & 0x7FFFFFFFu) > 0x7F800000u;   // only NaNs reach such a cut
+        const float cutf = __uint_as_float(cut_bits);
+        const int hs = lh, rsw = l31 & 15;
+        const unsigned char *myrow = park + l31 * 256;
+        uint32_t W[2][NWL];
+        uint32_t cnt[2], part[2], incl[2], tot[2];           // own half row, the other half, rows up to this one
+        // generic: float compares, element by element; bit c of a lane's mask = column 64 hs + c
+        auto scan_generic = [&](uint32_t (&Wh)[NWL]) {
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          const int ml = h * 64 + lane;
+          for (int i = 0; i < NWL; ++i) Wh[i] = 0;
 #pragma unroll
-          for (int i = 0; i < NW; ++i) W[h][i] = 0;
-#pragma unroll
-          for (int sl = 0; sl < 16; ++sl) {
-            const uint4 v = *reinterpret_cast<const uint4 *>(park + ml * 256 + ((sl ^ (ml & 15)) * 16));
+          for (int s8 = 0; s8 < 8; ++s8) {
+            const int sl = hs * 8 + s8;
+            const uint4 v = *reinterpret_cast<const uint4 *>(myrow + ((sl ^ rsw) * 16));
             uint4 tv = make_uint4(0, 0, 0, 0);
             if constexpr (COLLECT == 2)
               tv = *reinterpret_cast<const uint4 *>((const T *)ca.theta + (int64_t)layer * ca.theta_stride + ncol0 + sl * EPS);
@@ -390,151 +443,185 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
               else c = xv >= slot_elem<T>(tv, j);
               m |= (c ? 1u : 0u) << j;
             }
-            W[h][(sl * EPS) >> 5] |= m << ((sl * EPS) & 31);
+            Wh[(s8 * EPS) >> 5] |= m << ((s8 * EPS) & 31);
           }
-        }
-      };
-      bool done = false;
-      if constexpr (sizeof(T) == 2) {
+        };
         // bf16 and a positive cut / threshold: x >= c  <=>  bits(x) >= bits(c) as signed 16-bit
         // integers (negative values have the sign bit), two elements per operation: the sign of
         // the saturated difference (c - 1) - x marks a candidate.  NaNs would be treated wrongly
         // (a top-k cut must take them all, also those with the sign bit set; a threshold must take
-        // none), so the unsigned maximum of the raw values is tracked and the tile is redone with
+        // none), so the unsigned maximum of the raw values is tracked and the piece is redone with
         // float compares if it shows one.
-        bool fast_ok;
+        bool fast_ok = false;
         uint32_t cm1 = 0;
         const T *theta_seg = nullptr;
-        if constexpr (COLLECT == 1) {
-          const uint32_t cb = cut_bits >> 16;
-          fast_ok = cb >= 1u && cb <= 0x7F80u;
-          cm1 = (cb - 1u) | ((cb - 1u) << 16);
-        } else {
-          theta_seg = (const T *)ca.theta + (int64_t)layer * ca.theta_stride + ncol0;
-          bool bad = false;
-          if (lane < 16) {   // every threshold of the segment must be a positive number
-            const uint4 tv = *reinterpret_cast<const uint4 *>(theta_seg + lane * 8);
-            const uint32_t t4[4] = {tv.x, tv.y, tv.z, tv.w};
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-              const uint32_t lo = t4[k] & 0xFFFFu, hi = t4[k] >> 16;
-              bad = bad || lo < 1u || lo > 0x7F80u || hi < 1u || hi > 0x7F80u;
-            }
-          }
-          fast_ok = __ballot(bad) == 0;
-        }
-        if (fast_ok) {
-          uint32_t mx = 0;
-#pragma unroll
-          for (int h = 0; h < 2; ++h) {
-            const int ml = h * 64 + lane;
-#pragma unroll
-            for (int i = 0; i < NW; ++i) W[h][i] = 0;
-#pragma unroll
-            for (int sl = 0; sl < 16; ++sl) {
-              const uint4 v = *reinterpret_cast<const uint4 *>(park + ml * 256 + ((sl ^ (ml & 15)) * 16));
-              const uint32_t w4[4] = {v.x, v.y, v.z, v.w};
-              uint32_t c4[4] = {cm1, cm1, cm1, cm1};
-              if constexpr (COLLECT == 2) {
-                const uint4 tv = *reinterpret_cast<const uint4 *>(theta_seg + sl * 8);   // same address in all lanes
-                c4[0] = tv.x - 0x00010001u; c4[1] = tv.y - 0x00010001u; c4[2] = tv.z - 0x00010001u; c4[3] = tv.w - 0x00010001u;
-              }
-              uint32_t a = 0;
+        if constexpr (sizeof(T) == 2) {
+          if constexpr (COLLECT == 1) {
+            const uint32_t cb = cut_bits >> 16;
+            fast_ok = cb >= 1u && cb <= 0x7F80u;
+            cm1 = (cb - 1u) | ((cb - 1u) << 16);
+          } else {
+            theta_seg = (const T *)ca.theta + (int64_t)layer * ca.theta_stride + ncol0;
+            bool bad = false;
+            if (lane_e < 16) {   // every threshold of the segment must be a positive number
+              const uint4 tv = *reinterpret_cast<const uint4 *>(theta_seg + lane_e * 8);
+              const uint32_t t4[4] = {tv.x, tv.y, tv.z, tv.w};
 #pragma unroll
               for (int k = 0; k < 4; ++k) {
-                const uint32_t sg = pk_sign16(pk_sub_sat16(c4[k], w4[k]));   // 0xFFFF per candidate half
-                a |= sg & ((1u << (2 * k)) | (0x20000u << (2 * k)));         // element 2k -> bit 2k, 2k+1 -> bit 16+2k+1
-                mx = pk_max_u16(mx, COLLECT == 1 ? w4[k] : (w4[k] & 0x7FFF7FFFu));
+                const uint32_t lo = t4[k] & 0xFFFFu, hi = t4[k] >> 16;
+                bad = bad || lo < 1u || lo > 0x7F80u || hi < 1u || hi > 0x7F80u;
               }
-              const uint32_t m = (a | (a >> 16)) & 0xFFu;
-              W[h][sl >> 2] |= m << ((sl & 3) * 8);
             }
-          }
-          const uint32_t nan_above = COLLECT == 1 ? 0xFF80u : 0x7F80u;
-          const bool nan_seen = (mx & 0xFFFFu) > nan_above || (mx >> 16) > nan_above;
-          done = __ballot(nan_seen) == 0;
-        }
-      }
-      if (!done) scan_generic();
-#pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        cnt[h] = 0;
-#pragma unroll
-        for (int i = 0; i < NW; ++i) cnt[h] += __popc(W[h][i]);
-      }
-      const uint32_t incl0 = wave_inclusive_scan32(cnt[0]), incl1 = wave_inclusive_scan32(cnt[1]);
-      const uint32_t tot0 = __builtin_amdgcn_readlane(incl0, 63), tot1 = __builtin_amdgcn_readlane(incl1, 63);
-      const uint32_t total = tot0 + tot1;
-      const int nseg = N / SEGW;
-      const int seg = ncol0 / SEGW;
-      const int nrb = M >> 7, rowblk = (m0 + wm * 128) >> 7;
-      const uint32_t tile = (uint32_t)seg * (uint32_t)nrb + (uint32_t)rowblk;
-      uint32_t off = tile * ca.caps;                       // the tile's fixed slot
-      bool ok = true;
-      if (total > ca.caps) {                               // rare: an extent behind the slots
-        const unsigned long long fixed = (unsigned long long)nseg * nrb * ca.caps;
-        uint32_t a = 0;
-        if (lane == 0) a = atomicAdd(&ca.pool_count[layer], total);
-        a = __builtin_amdgcn_readfirstlane(a);
-        ok = fixed + a + total <= ca.pool_cap;
-        off = (uint32_t)(fixed + a);
-        if (!ok && lane == 0) atomicOr(&ca.st[layer].overflow, 1u);
-      }
-      uint2 *mypool = ca.pool + (unsigned long long)layer * ca.pool_cap;
-      if (lane == 0) ca.tile_meta[(int64_t)layer * nseg * nrb + tile] = make_uint2(off, ok ? total : 0u);
-      uint2 *meta = ca.seg_meta + ((int64_t)layer * nseg + seg) * M + m0 + wm * 128;
-      // Emission.  Each lane first drops a 16-bit code (row, column) for every candidate of its two
-      // rows into the wavefront's list, at the candidate's ordered position inside the tile; then the
-      // lanes take one candidate each: 64 consecutive pool entries per store instruction, and the
-      // number of rounds is the tile's count / 64 instead of the fullest row's count.
-      const uint32_t rel[2] = {incl0 - cnt[0], tot0 + incl1 - cnt[1]};
-#pragma unroll
-      for (int h = 0; h < 2; ++h) meta[h * 64 + lane] = ok ? make_uint2(off + rel[h], cnt[h]) : make_uint2(0u, 0u);
-      if (ok && total <= (uint32_t)CAND_LIST) {
-        uint16_t *lst = cand_list[wave];
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          const uint32_t rowcode = (uint32_t)(h * 64 + lane) << 8;
-          uint32_t p = rel[h];
-#pragma unroll
-          for (int i = 0; i < NW; ++i) {
-            uint32_t w = W[h][i];
-            while (w) {
-              lst[p++] = (uint16_t)(rowcode | (uint32_t)(i * 32 + (__ffs(w) - 1)));
-              w &= w - 1u;
-            }
+            fast_ok = __ballot(bad) == 0;
           }
         }
-        uint2 *dst = mypool + off;
+        auto scan_piece = [&](uint32_t (&Wh)[NWL]) {
+          bool done = false;
+          if constexpr (sizeof(T) == 2) {
+            if (fast_ok) {
+              uint32_t mx = 0;
+#pragma unroll
+              for (int i = 0; i < NWL; ++i) Wh[i] = 0;
+#pragma unroll
+              for (int s8 = 0; s8 < 8; ++s8) {
+                const int sl = hs * 8 + s8;
+                const uint4 v = *reinterpret_cast<const uint4 *>(myrow + ((sl ^ rsw) * 16));
+                const uint32_t w4[4] = {v.x, v.y, v.z, v.w};
+                uint32_t c4[4] = {cm1, cm1, cm1, cm1};
+                if constexpr (COLLECT == 2) {
+                  const uint4 tv = *reinterpret_cast<const uint4 *>(theta_seg + sl * 8);   // one address per half wave
+                  c4[0] = tv.x - 0x00010001u; c4[1] = tv.y - 0x00010001u; c4[2] = tv.z - 0x00010001u; c4[3] = tv.w - 0x00010001u;
+                }
+                uint32_t a = 0;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                  const uint32_t sg = pk_sign16(pk_sub_sat16(c4[k], w4[k]));   // 0xFFFF per candidate half
+                  a |= sg & ((1u << (2 * k)) | (0x20000u << (2 * k)));         // element 2k -> bit 2k, 2k+1 -> bit 16+2k+1
+                  mx = pk_max_u16(mx, COLLECT == 1 ? w4[k] : (w4[k] & 0x7FFF7FFFu));
+                }
+                const uint32_t m = (a | (a >> 16)) & 0xFFu;
+                Wh[s8 >> 2] |= m << ((s8 & 3) * 8);
+              }
+              const uint32_t nan_above = COLLECT == 1 ? 0xFF80u : 0x7F80u;
+              const bool nan_seen = (mx & 0xFFFFu) > nan_above || (mx >> 16) > nan_above;
+              done = __ballot(nan_seen) == 0;
+            }
+          }
+          if (!done) scan_generic(Wh);
+        };
+        uint2 *mypool = ca.pool + (unsigned long long)layer * ca.pool_cap;
+        // Emission of the parked piece: `n` candidates, this lane's starting at position `first` of
+        // the piece, to dst[0 .. n).  Each lane first drops a 16-bit code (row, column) for every
+        // candidate of its half row into the wavefront's list, at the candidate's ordered position; then
+        // the lanes take one candidate each: 64 consecutive pool entries per store instruction, and the
+        // number of rounds is the piece's count / 64 instead of the fullest row's count.
+        auto emit_piece = [&](const uint32_t (&Wh)[NWL], uint32_t first, uint32_t n, uint2 *dst) {
+          if (n <= (uint32_t)CAND_LIST) {
+            uint16_t *lst = cand_list[wave];
+            const uint32_t rowcode = ((uint32_t)l31 << 8) | (uint32_t)(hs * (SEGW / 2));
+            uint32_t p = first;
+#pragma unroll
+            for (int i = 0; i < NWL; ++i) {
+              uint32_t wd = Wh[i];
+              while (wd) {
+                lst[p++] = (uint16_t)(rowcode + (uint32_t)(i * 32 + (__ffs(wd) - 1)));
+                wd &= wd - 1u;
+              }
+            }
 #pragma unroll 2
-        for (uint32_t idx = lane; idx < total; idx += 64) {
-          const uint32_t code = lst[idx];
-          const int ml = (int)(code >> 8), c = (int)(code & 255u);
-          const int sl = c / EPS, j = c % EPS;
-          const T rawv = *reinterpret_cast<const T *>(park + ml * 256 + ((sl ^ (ml & 15)) * 16) + j * (int)sizeof(T));
-          dst[idx] = make_uint2((uint32_t)(ncol0 + c), Elem<T>::raw(rawv));
-        }
-      } else if (ok) {
-        // a tile with more candidates than the list holds: every lane walks its own rows
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          const int ml = h * 64 + lane;
-          uint32_t pos = off + rel[h];
-#pragma unroll
-          for (int i = 0; i < NW; ++i) {
-            uint32_t w = W[h][i];
-            while (w) {
-              const int c = i * 32 + (__ffs(w) - 1);       // column inside the segment
-              w &= w - 1u;
+            for (uint32_t idx = lane_e; idx < n; idx += 64) {
+              const uint32_t code = lst[idx];
+              const int ml = (int)(code >> 8), c = (int)(code & 255u);
               const int sl = c / EPS, j = c % EPS;
               const T rawv = *reinterpret_cast<const T *>(park + ml * 256 + ((sl ^ (ml & 15)) * 16) + j * (int)sizeof(T));
-              mypool[pos++] = make_uint2((uint32_t)(ncol0 + c), Elem<T>::raw(rawv));
+              dst[idx] = make_uint2((uint32_t)(ncol0 + c), Elem<T>::raw(rawv));
             }
+          } else {
+            // more candidates than the list holds: every lane walks its own half row
+            uint32_t pos = first;
+#pragma unroll
+            for (int i = 0; i < NWL; ++i) {
+              uint32_t wd = Wh[i];
+              while (wd) {
+                const int c = hs * (SEGW / 2) + i * 32 + (__ffs(wd) - 1);   // column inside the segment
+                wd &= wd - 1u;
+                const int sl = c / EPS, j = c % EPS;
+                const T rawv = *reinterpret_cast<const T *>(myrow + ((sl ^ rsw) * 16) + j * (int)sizeof(T));
+                dst[pos++] = make_uint2((uint32_t)(ncol0 + c), Elem<T>::raw(rawv));
+              }
+            }
+          }
+        };
+        const int nseg = N / SEGW;
+        const int seg = ncol0 / SEGW;
+        const int nrb = M / COLLECT_ROWS, rowblk = (m0 + wm * 64) / COLLECT_ROWS;
+        const uint32_t tile = (uint32_t)seg * (uint32_t)nrb + (uint32_t)rowblk;
+        uint32_t off = tile * ca.caps;                       // the tile's fixed slot
+        // Each piece of 32 tokens is emitted into the fixed slot as soon as it is scanned, while it is
+        // parked; the rare tile whose two pieces do not fit the slot takes an extent behind the slots (one
+        // atomic) and parks and emits both again.
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          park_rows(pass, h, 1);
+          scan_piece(W[h]);
+          cnt[h] = 0;
+#pragma unroll
+          for (int i = 0; i < NWL; ++i) cnt[h] += __popc(W[h][i]);
+          part[h] = (uint32_t)__shfl_xor((int)cnt[h], 32);
+          // rows up to and including this one, inside each half of the wavefront
+          uint32_t v = row16_inclusive_scan(cnt[h] + part[h]);
+          v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x142, 0xa, 0xf, false);  // row_bcast:15
+          incl[h] = v;
+          tot[h] = __builtin_amdgcn_readlane(v, 31);
+          const uint32_t before = h ? tot[0] : 0u;
+          const uint32_t first = incl[h] - cnt[h] - (hs ? 0u : part[h]);
+          if (before + tot[h] <= ca.caps) emit_piece(W[h], first, tot[h], mypool + off + before);
+        }
+        const uint32_t total = tot[0] + tot[1];
+        bool ok = true;
+        if (total > ca.caps) {
+          const unsigned long long fixed = (unsigned long long)nseg * nrb * ca.caps;
+          uint32_t a = 0;
+          if (lane_e == 0) a = atomicAdd(&ca.pool_count[layer], total);
+          a = __builtin_amdgcn_readfirstlane(a);
+          ok = fixed + a + total <= ca.pool_cap;
+          off = (uint32_t)(fixed + a);
+          if (!ok && lane_e == 0) atomicOr(&ca.st[layer].overflow, 1u);
+          if (ok) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+              park_rows(pass, h, 1);
+              emit_piece(W[h], incl[h] - cnt[h] - (hs ? 0u : part[h]), tot[h], mypool + off + (h ? tot[0] : 0u));
+            }
+          }
+        }
+        if (lane_e == 0) ca.tile_meta[(int64_t)layer * nseg * nrb + tile] = make_uint2(off, ok ? total : 0u);
+        uint2 *meta = ca.seg_meta + ((int64_t)layer * nseg + seg) * M + m0 + wm * 64;
+        if (hs == 0) {
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            const uint32_t rowtot = cnt[h] + part[h];
+            const uint32_t rel = (h ? tot[0] : 0u) + incl[h] - rowtot;
+            meta[h * 32 + l31] = ok ? make_uint2(off + rel, rowtot) : make_uint2(0u, 0u);
           }
         }
       }
     }
+    if (!has_next) break;
+    // Every wavefront is done with its parked rows before the next tile's loads overwrite them.  The wait
+    // is for this wavefront's LDS reads only: the first stage of the next tile may still be on its way.
+    __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0)
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    bid = nbid;
+    cur = nxt_tile;
+    load_bias(cur);
+    __builtin_amdgcn_sched_barrier(0);   // the bias stays ahead of the stage loads: the wait above counts on it
+    if (!OVERLAP) issue_stage(stage0, x_rows(cur), w_rows(cur), stage_k0(cur, 0));
+    issue_stage(stage1, x_rows(cur), w_rows(cur), stage_k0(cur, 1));
   }
+  __builtin_amdgcn_s_waitcnt(0);   // no direct-to-LDS load may be in flight when the block retires
 }
 
 // Any shape: one thread per output, fp32 accumulation.
@@ -574,10 +661,21 @@ static int launch_encode(const void *x, const void *w, const void *b, void *pre,
     if (nblk > 2147483647LL) return CLT_ERR_RANGE;
     CollectArgs none = {};
     const CollectArgs a = ca ? *ca : none;
+    // the collecting modes run one persistent workgroup per CU (a whole number of rounds over the 8 XCDs,
+    // so that block b stays on XCD b % 8 for all of its tiles); the storing mode one tile per workgroup
+    int64_t grid = nblk;
+    if (collect) {
+      int dev = 0, cus = 0;
+      if (hipGetDevice(&dev) != hipSuccess ||
+          hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 8)
+        return CLT_ERR_LAUNCH;
+      cus -= cus % 8;
+      if (grid > cus && !getenv("CLT_EXP_GRID")) grid = cus;
+    }
 #define CLT_ENC(C)                                                                                               \
-  k_encode_mfma<T, C><<<(unsigned)nblk, 256, 0, stream>>>((const T *)x, (const T *)w, (const T *)b, (T *)pre,    \
-                                                          (int)T_, (int)d, (int)F, (int)tm, (int)tn, xs, wstr,   \
-                                                          bs, ps, gate, a)
+  k_encode_mfma<T, C><<<(unsigned)grid, NTHREADS, 0, stream>>>((const T *)x, (const T *)w, (const T *)b, (T *)pre,    \
+                                                          (int)T_, (int)d, (int)F, (int)tm, (int)tn, (int)nblk,  \
+                                                          xs, wstr, bs, ps, gate, a)
     if (collect == 0) CLT_ENC(0);
     else if (collect == 1) CLT_ENC(1);
     else CLT_ENC(2);

@@ -1416,11 +1416,11 @@ static TileLayout tile_layout(int64_t T, int64_t F, int64_t L, int64_t k, int dt
   tl.sel = sel_layout(T, F, L, k, CLT_TOPK_PER_LAYER);
   const int segw = dtype == CLT_BF16 ? 128 : 64;
   tl.nseg = (int)(F / segw);
-  tl.ntile = tl.nseg * (int)(T / 128);
+  tl.ntile = tl.nseg * (int)(T / COLLECT_ROWS);
   // about 2.3x K candidates are expected, i.e. 2.3 * k / F of a tile's 128 * segw elements; a
   // slot holds three times that (at least 64, at most the whole tile)
-  unsigned long long caps = (unsigned long long)(3.0 * 2.3 * (double)k / (double)F * 128.0 * segw) + 64ull;
-  if (caps > 128ull * segw) caps = 128ull * segw;
+  unsigned long long caps = (unsigned long long)(3.0 * 2.3 * (double)k / (double)F * (double)COLLECT_ROWS * segw) + 64ull;
+  if (caps > (unsigned long long)COLLECT_ROWS * segw) caps = (unsigned long long)COLLECT_ROWS * segw;
   tl.caps = (uint32_t)caps;
   const unsigned long long N = (unsigned long long)T * F;
   unsigned long long K = (unsigned long long)k * T;
@@ -1537,11 +1537,11 @@ static ThreshLayout thresh_layout(int64_t T, int64_t F, int64_t L, int64_t densi
   ThreshLayout tl;
   const int segw = dtype == CLT_BF16 ? 128 : 64;
   tl.nseg = (int)(F / segw);
-  tl.ntile = tl.nseg * (int)(T / 128);
+  tl.ntile = tl.nseg * (int)(T / COLLECT_ROWS);
   const double dens = (double)(density_ppm < 1 ? 1 : density_ppm) * 1e-6;
   // a fixed slot holds three times the expected entries of a tile (at least 64, at most the tile)
-  unsigned long long caps = (unsigned long long)(3.0 * dens * 128.0 * segw) + 64ull;
-  if (caps > 128ull * segw) caps = 128ull * segw;
+  unsigned long long caps = (unsigned long long)(3.0 * dens * (double)COLLECT_ROWS * segw) + 64ull;
+  if (caps > (unsigned long long)COLLECT_ROWS * segw) caps = (unsigned long long)COLLECT_ROWS * segw;
   tl.caps = (uint32_t)caps;
   const unsigned long long N = (unsigned long long)T * F;
   unsigned long long dyn = (unsigned long long)(2.0 * dens * (double)N) + 4096ull;

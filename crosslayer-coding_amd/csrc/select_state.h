@@ -25,9 +25,12 @@ struct SelState {
   uint32_t overflow;  // the encoder epilogue ran out of pool space (set with atomicOr)
 };
 
-// What the collecting encoder epilogue writes.  A wavefront's 128-token tile of one feature
+// tokens of one wave tile of the collecting encoder epilogue
+constexpr int COLLECT_ROWS = 64;
+
+// What the collecting encoder epilogue writes.  A wavefront's 64-token tile of one feature
 // segment (128 features for 16-bit elements, 64 for 32-bit) becomes ONE extent of the layer's
-// pool, ordered by (token, feature).  Tile number i = segment * (T / 128) + token block owns
+// pool, ordered by (token, feature).  Tile number i = segment * (T / 64) + token block owns
 // the fixed slot [i * caps, (i + 1) * caps) of the pool; only a tile with more than `caps`
 // candidates takes an extent behind the slots instead, handed out by an atomic counter (one
 // same-address atomic per tile from every CU at once would cost more than the whole epilogue).
