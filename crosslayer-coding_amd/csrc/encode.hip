@@ -19,7 +19,6 @@
 //   bf16        v_mfma_f32_32x32x16_bf16, fp32 accumulate, one rounding (v_cvt_pk_bf16_f32)
 //   fp32        v_mfma_f32_32x32x2_f32
 #include <type_traits>
-#include <cstdlib>
 #include "select_state.h"
 
 namespace {
@@ -182,11 +181,18 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
     t.rot = ((tiles_n & 7) == 0 ? 3 * t.tm + (t.tn >> 3) : t.tm + t.tn) % nk;
     return t;
   };
-  // the storing mode computes only the layers that asked for it when a gate is given
+  // the storing mode computes only the layers that asked for it when a gate is given; the states of up to
+  // 64 layers are fetched with one load
+  const int nlayer = total_tiles / per_layer;
+  unsigned long long want_mask = ~0ull;
+  if (COLLECT == 0 && gate && nlayer <= 64)
+    want_mask = __ballot(lane < nlayer && gate[lane < nlayer ? lane : 0].status == ST_RETRY);
   auto wanted = [&](int bid) {
     if (COLLECT != 0 || !gate) return true;
-    return gate[bid / per_layer].status == ST_RETRY;
+    const int l = bid / per_layer;
+    return nlayer <= 64 ? ((want_mask >> l) & 1ull) != 0ull : gate[l].status == ST_RETRY;
   };
+  if (COLLECT == 0 && gate && nlayer <= 64 && want_mask == 0ull) return;
   int bid = blockIdx.x;
   while (bid < total_tiles && !wanted(bid)) bid += gridDim.x;
   if (bid >= total_tiles) return;
@@ -662,15 +668,16 @@ static int launch_encode(const void *x, const void *w, const void *b, void *pre,
     CollectArgs none = {};
     const CollectArgs a = ca ? *ca : none;
     // the collecting modes run one persistent workgroup per CU (a whole number of rounds over the 8 XCDs,
-    // so that block b stays on XCD b % 8 for all of its tiles); the storing mode one tile per workgroup
+    // so that block b stays on XCD b % 8 for all of its tiles); the storing mode one tile per workgroup,
+    // unless it is gated: that launch usually finds nothing to do, which a small grid finds out sooner
     int64_t grid = nblk;
-    if (collect) {
+    if (collect || gate) {
       int dev = 0, cus = 0;
       if (hipGetDevice(&dev) != hipSuccess ||
           hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 8)
         return CLT_ERR_LAUNCH;
       cus -= cus % 8;
-      if (grid > cus && !getenv("CLT_EXP_GRID")) grid = cus;
+      if (grid > cus) grid = cus;
     }
 #define CLT_ENC(C)                                                                                               \
   k_encode_mfma<T, C><<<(unsigned)grid, NTHREADS, 0, stream>>>((const T *)x, (const T *)w, (const T *)b, (T *)pre,    \
