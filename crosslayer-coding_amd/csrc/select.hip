@@ -31,7 +31,8 @@ namespace {
 constexpr int NBINS = 2048;
 constexpr uint32_t FINE16 = 1984;  // 16-bit keys: bins [0,FINE16) are one key wide
 constexpr int SAMPLE_N = 16384;
-constexpr int SAMPLE_TOK = 64;           // tokens of the sample taken before the pre-activations exist
+constexpr int SAMPLE_WAVES = 64;         // sample taken before the pre-activations exist: wavefronts per layer,
+constexpr int SAMPLE_PRE_N = SAMPLE_WAVES * 1024;   // each 32 hashed tokens x 32 hashed features
 constexpr int SAMPLE_BLOCKS = 16;        // blocks per problem that gather the sample
 constexpr int SCAN_THREADS = 1024;
 constexpr int WBUF = 512;                // candidate entries buffered in LDS per wavefront
@@ -190,14 +191,14 @@ __global__ __launch_bounds__(256) void k_sample_keys(
 // One block per problem: the cut key = the r-th largest sample key, r chosen so that the
 // expected number of elements above the cut is about 1.25 K plus six standard deviations.
 // Also resets the problem's histogram, pool counter and state.
-template <int KB>
+template <int KB, int SN>
 __global__ __launch_bounds__(SCAN_THREADS) void k_sample_cut(
     const uint32_t *sample, unsigned long long N, unsigned long long K, SelState *st, uint32_t *hist,
     uint32_t *pool_count, uint32_t *aux_count, uint32_t path) {
-  constexpr int PER = SAMPLE_N / SCAN_THREADS;
+  constexpr int PER = SN / SCAN_THREADS;
   __shared__ uint32_t lh[NBINS];
   const int p = blockIdx.x, tid = threadIdx.x;
-  const unsigned long long ns = N < (unsigned long long)SAMPLE_N ? N : (unsigned long long)SAMPLE_N;
+  const unsigned long long ns = N < (unsigned long long)SN ? N : (unsigned long long)SN;
   for (int i = tid; i < NBINS; i += SCAN_THREADS) hist[(int64_t)p * NBINS + i] = 0;
   if (tid == 0) { pool_count[p] = 0; if (aux_count) aux_count[p] = 0; }
   uint32_t keys[PER];
@@ -206,15 +207,15 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_sample_cut(
   for (int i = 0; i < PER; ++i) {
     unsigned long long si = (unsigned long long)tid + (unsigned long long)i * SCAN_THREADS;
     valid[i] = si < ns;
-    keys[i] = valid[i] ? sample[(int64_t)p * SAMPLE_N + si] : 0u;
+    keys[i] = valid[i] ? sample[(int64_t)p * SN + si] : 0u;
   }
   unsigned long long r;
-  if (ns == N) r = K;
+  if (ns == N && path != PATH_TILES) r = K;   // the sample is the whole problem
   else {
     double e = (double)K / (double)N * (double)ns;
-    // the sample taken from a token x feature grid (PATH_TILES) is less even than a hashed
-    // one: leave it more room
-    r = path == PATH_TILES ? (unsigned long long)(1.5 * e + 8.0 * sqrt(e) + 16.0) + 1
+    // the sample taken ahead of the projection (PATH_TILES) is four times larger and made of 32 x 32
+    // blocks of tokens x features: a smaller relative margin, the same six standard deviations
+    r = path == PATH_TILES ? (unsigned long long)(1.2 * e + 6.0 * sqrt(e) + 16.0) + 1
                            : (unsigned long long)(1.25 * e + 6.0 * sqrt(e) + 16.0) + 1;
   }
   uint32_t cut = min_key<KB>();
@@ -760,56 +761,57 @@ __global__ __launch_bounds__(256) void k_select_emit(
 }
 
 // ---- candidates collected by the encoder epilogue (PATH_TILES) -------------------------
-// Ranking keys of a sample taken BEFORE the pre-activations exist: SAMPLE_TOK hashed tokens x
-// SAMPLE_N / SAMPLE_TOK hashed features per layer, each value computed as a plain dot product
-// (fp32 accumulation, rounded to the model dtype).  It only has to give a cut of the right
-// size; the selection stays exact whatever the cut is.
+// Ranking keys of a sample taken BEFORE the pre-activations exist.  Per layer SAMPLE_WAVES wavefronts
+// each compute a 32 x 32 block of pre-activations with the matrix core, for 32 hashed tokens and 32
+// hashed features of their own (so a layer's sample covers 2048 tokens and 2048 features): a lane reads
+// 16 bytes of "its" x row and W row per step straight from global memory - the K order inside a step is
+// the same permutation for both operands, which a dot product does not mind - fp32 accumulation, bias,
+// one rounding to the model dtype.  The sample only has to give a cut of the right size; the selection
+// stays exact whatever the cut is.
+typedef __attribute__((ext_vector_type(8))) __bf16 smp_bf16x8_t;
+typedef __attribute__((ext_vector_type(16))) float smp_f32x16_t;
 template <typename T>
-__global__ __launch_bounds__(256) void k_sample_dot(
+__global__ __launch_bounds__(256) void k_sample_mfma(
     const T *__restrict__ x, const T *__restrict__ w, const T *__restrict__ b, int64_t Tn, int64_t d, int64_t F,
     int64_t xs, int64_t wstr, int64_t bs, uint32_t *sample) {
   constexpr int KB = Elem<T>::KEYBITS;
-  constexpr int V = Elem<T>::VEC;
-  constexpr int NFEAT = SAMPLE_N / SAMPLE_TOK;
-  constexpr int NJ = 4;   // features in flight per wavefront
-  const int l = blockIdx.y, ti = blockIdx.x;
-  const int lane = lane_id(), wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
-  const int64_t tok = (int64_t)hash_index((uint64_t)ti * 131u + (uint64_t)l * 7919u, (uint64_t)Tn);
-  const T *xr = x + (int64_t)l * xs + tok * d;
-  const int64_t nch = d / V;   // 16-byte chunks per row (the collecting encoder needs d % V == 0)
-  // blockIdx.z cuts the features of this token into gridDim.z groups
-  const int jper = NFEAT / (int)gridDim.z, jb = (int)blockIdx.z * jper;
-  for (int j0 = jb + wv * NJ; j0 < jb + jper; j0 += nwv * NJ) {
-    const T *wr[NJ];
-    int64_t f[NJ];
-    float acc[NJ];
+  constexpr int V = 16 / (int)sizeof(T);   // elements of one 16-byte piece
+  const int l = blockIdx.y, lane = lane_id();
+  const int g = (int)blockIdx.x * (int)(blockDim.x >> 6) + (int)(threadIdx.x >> 6);   // block of the sample
+  const int l31 = lane & 31, lh = lane >> 5;
+  const uint64_t salt = (uint64_t)l * 7919u + (uint64_t)g * 104729u;
+  const int64_t tok = (int64_t)hash_index(salt * 64u + (uint64_t)l31, (uint64_t)Tn);
+  const int64_t f = (int64_t)hash_index(salt * 64u + 32u + (uint64_t)l31, (uint64_t)F);
+  const T *xr = x + (int64_t)l * xs + tok * d + lh * V;
+  const T *wr = w + (int64_t)l * wstr + f * d + lh * V;
+  smp_f32x16_t acc;
 #pragma unroll
-    for (int q = 0; q < NJ; ++q) {
-      f[q] = (int64_t)hash_index((uint64_t)(j0 + q) * 257u + (uint64_t)ti * 65537u + (uint64_t)l * 104729u + 1u, (uint64_t)F);
-      wr[q] = w + (int64_t)l * wstr + f[q] * d;
-      acc[q] = 0.0f;
-    }
-    for (int64_t c = lane; c < nch; c += 64) {
-      const uint4 xv = *reinterpret_cast<const uint4 *>(xr + c * V);
-      uint4 wq[NJ];
-#pragma unroll
-      for (int q = 0; q < NJ; ++q) wq[q] = *reinterpret_cast<const uint4 *>(wr[q] + c * V);
-#pragma unroll
-      for (int q = 0; q < NJ; ++q)
-#pragma unroll
-        for (int e = 0; e < V; ++e) acc[q] = fmaf(vec_elem<T>(xv, e), vec_elem<T>(wq[q], e), acc[q]);
-    }
-#pragma unroll
-    for (int q = 0; q < NJ; ++q) {
-      float a = acc[q];
-#pragma unroll
-      for (int o = 32; o > 0; o >>= 1) a += __shfl_xor(a, o);
-      if (lane == 0) {
-        if (b) a += Elem<T>::to_f32(b[(int64_t)l * bs + f[q]]);
-        sample[(int64_t)l * SAMPLE_N + (int64_t)ti * NFEAT + j0 + q] = rank_key<KB>(Elem<T>::round(a));
-      }
+  for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+  const int64_t nstep = d / (2 * V);       // the collecting encoder needs d to be a multiple of 2 V
+#pragma unroll 4
+  for (int64_t st = 0; st < nstep; ++st) {
+    const uint4 a = *reinterpret_cast<const uint4 *>(wr + st * 2 * V);
+    const uint4 q = *reinterpret_cast<const uint4 *>(xr + st * 2 * V);
+    if constexpr (sizeof(T) == 2) {
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(smp_bf16x8_t, a), __builtin_bit_cast(smp_bf16x8_t, q), acc, 0, 0, 0);
+    } else {
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.x), __uint_as_float(q.x), acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.y), __uint_as_float(q.y), acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.z), __uint_as_float(q.z), acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.w), __uint_as_float(q.w), acc, 0, 0, 0);
     }
   }
+  // accumulator rg*4+q of a lane: feature row rg*8 + lh*4 + q of the block, token column l31
+  const float bown = b ? Elem<T>::to_f32(b[(int64_t)l * bs + f]) : 0.0f;   // bias of feature row l31
+  uint32_t *out = sample + (int64_t)l * SAMPLE_PRE_N + (int64_t)g * 1024;
+#pragma unroll
+  for (int rg = 0; rg < 4; ++rg)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int m = rg * 8 + lh * 4 + q;
+      const float bv = __shfl(bown, m);
+      out[m * 32 + l31] = rank_key<KB>(Elem<T>::round(acc[rg * 4 + q] + bv));
+    }
 }
 
 // Histogram of the collected candidates of every layer that is at `level`: one wavefront per
@@ -1293,7 +1295,7 @@ static SelLayout sel_layout(int64_t T, int64_t F, int64_t L, int64_t k, int mode
   lo.off_state = take(sizeof(SelState) * (size_t)lo.nprob);
   lo.off_hist = take(sizeof(uint32_t) * NBINS * (size_t)lo.nprob);
   lo.off_poolcnt = take(4 * (size_t)lo.nprob);
-  lo.off_sample = take(4 * (size_t)SAMPLE_N * (size_t)lo.nprob);
+  lo.off_sample = take(4 * (size_t)(SAMPLE_PRE_N > SAMPLE_N ? SAMPLE_PRE_N : SAMPLE_N) * (size_t)lo.nprob);
   lo.off_first = take(4 * R);
   lo.off_gt = take(4 * R);
   lo.off_eq = take(4 * R);
@@ -1325,7 +1327,7 @@ static int run_batchtopk(const T *pre, int64_t Tn, int64_t F, int64_t L, int64_t
   if (K > N) K = N;
   const int nprob = lo.nprob;
   k_sample_keys<T, GLOBAL><<<dim3(SAMPLE_BLOCKS, nprob), 256, 0, stream>>>(pre, Tn, F, L, lstride, mean, denom, N, sample);
-  k_sample_cut<KB><<<nprob, SCAN_THREADS, 0, stream>>>(sample, N, K, st, hist, poolcnt, nullptr, PATH_ROWS);
+  k_sample_cut<KB, SAMPLE_N><<<nprob, SCAN_THREADS, 0, stream>>>(sample, N, K, st, hist, poolcnt, nullptr, PATH_ROWS);
   // two rows per wavefront: many more blocks than fit at once, so rows of very different
   // candidate counts balance out over the CUs
   int gx = (int)clt_ceil_div(Tn, 8);
@@ -1417,9 +1419,9 @@ static TileLayout tile_layout(int64_t T, int64_t F, int64_t L, int64_t k, int dt
   const int segw = dtype == CLT_BF16 ? 128 : 64;
   tl.nseg = (int)(F / segw);
   tl.ntile = tl.nseg * (int)(T / COLLECT_ROWS);
-  // about 2.3x K candidates are expected, i.e. 2.3 * k / F of a tile's 128 * segw elements; a
+  // about 1.5x K candidates are expected, i.e. 1.5 * k / F of a tile's 64 * segw elements; a
   // slot holds three times that (at least 64, at most the whole tile)
-  unsigned long long caps = (unsigned long long)(3.0 * 2.3 * (double)k / (double)F * (double)COLLECT_ROWS * segw) + 64ull;
+  unsigned long long caps = (unsigned long long)(3.0 * 1.5 * (double)k / (double)F * (double)COLLECT_ROWS * segw) + 64ull;
   if (caps > (unsigned long long)COLLECT_ROWS * segw) caps = (unsigned long long)COLLECT_ROWS * segw;
   tl.caps = (uint32_t)caps;
   const unsigned long long N = (unsigned long long)T * F;
@@ -1457,9 +1459,9 @@ static int run_encode_collect(const void *x, const void *w, const void *b, void 
   const unsigned long long N = (unsigned long long)Tn * (unsigned long long)F;
   unsigned long long K = (unsigned long long)k * (unsigned long long)Tn;
   if (K > N) K = N;
-  k_sample_dot<T><<<dim3(SAMPLE_TOK, (unsigned)L, 8), 256, 0, stream>>>((const T *)x, (const T *)w, (const T *)b, Tn, d, F,
-                                                                      xs, wstr, bs, sample);
-  k_sample_cut<KB><<<(unsigned)L, SCAN_THREADS, 0, stream>>>(sample, N, K, st, hist, poolcnt,
+  k_sample_mfma<T><<<dim3(SAMPLE_WAVES / 4, (unsigned)L), 256, 0, stream>>>((const T *)x, (const T *)w, (const T *)b, Tn, d,
+                                                                          F, xs, wstr, bs, sample);
+  k_sample_cut<KB, SAMPLE_PRE_N><<<(unsigned)L, SCAN_THREADS, 0, stream>>>(sample, N, K, st, hist, poolcnt,
                                                               (uint32_t *)(ws + tl.off_tcount), PATH_TILES);
   uint2 *tpool = (uint2 *)(ws + tl.off_tpool);
   CollectArgs ca;
