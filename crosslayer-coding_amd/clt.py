@@ -249,17 +249,28 @@ class CrossLayerTranscoder(BaseTranscoder):
         theta = self.theta_manager.thresholds(self.dtype)
         packed = self.decoder_module.packed()
         out = torch.empty((L, F), dtype=torch.float32, device=pre.device)
+        T, d, pitch = g_model.shape[1], cfg.d_model, packed.shape[2]
+        g_model = g_model.contiguous()
+        piece = 64 if self.dtype == torch.bfloat16 else 32      # elements of K the matrix-core kernel takes at a time
+        dact_buf = ws.typed("theta_dact", (T, F), self.dtype)
         for s_ in range(L):
             targets = list(range(s_, L))
+            n = len(targets)
             if tying == "none":
                 slots = [s_ * L - (s_ * (s_ - 1)) // 2 + (t - s_) for t in targets]
             elif tying == "per_source":
-                slots = [s_] * len(targets)
+                slots = [s_] * n
             else:
                 slots = targets
-            stacked_w = torch.cat([packed[i][:, :cfg.d_model] for i in slots], dim=1).unsqueeze(0)   # [1, F, n d]
-            stacked_g = torch.cat([g_model[t] for t in targets], dim=1).unsqueeze(0)       # [1, T, n d]
-            dact = engine.encode(stacked_g.contiguous(), stacked_w.contiguous(), None)[0]  # [T, F]
+            if T >= 256 and F >= 256 and F % 4 == 0 and d % piece == 0 and (n * d // piece) % 2 == 0:
+                # both operands where they lie: segment q = target s + q, in the gradient slab [L, T, d] and
+                # in the packed decoders [n_dec, F, pitch] (one matrix for all targets when tied per source)
+                dact = engine.encode_segmented(g_model[s_:], packed[slots[0]:], n, d, T * d, d,
+                                               0 if tying == "per_source" else F * pitch, pitch, T, F, out=dact_buf)
+            else:
+                stacked_w = torch.cat([packed[i][:, :d] for i in slots], dim=1).unsqueeze(0)   # [1, F, n d]
+                stacked_g = torch.cat([g_model[t] for t in targets], dim=1).unsqueeze(0)       # [1, T, n d]
+                dact = engine.encode(stacked_g.contiguous(), stacked_w.contiguous(), None)[0]  # [T, F]
             engine.jumprelu_theta_grad(pre[s_], dact, theta[s_].contiguous(), self.theta_manager.bandwidth, out[s_], ws)
         # theta = exp(log_threshold): the reference casts theta to the model dtype for the forward
         return out * torch.exp(self.theta_manager.log_threshold.detach().float())

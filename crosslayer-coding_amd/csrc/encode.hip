@@ -116,7 +116,7 @@ __device__ __forceinline__ uint32_t wave_inclusive_scan32(uint32_t v) {
 
 // Requires K % (256 / sizeof(T)) == 0 (an even number of LDS stages), M >= BM and N >= BN.  A tile that
 // would stick out of the matrix is shifted back inside (its overlap with the neighbour is
-// computed twice and stored twice with identical values), so no load or store is predicated.
+// computed twice and stored by the neighbour only), so no load is predicated.
 //
 // Block -> tile map: workgroups go to the 8 XCDs round-robin, so block b runs on XCD b % 8.
 // When the feature tiles split evenly, XCD x takes the feature tiles n = x, x+8, ... in groups
@@ -127,11 +127,22 @@ __device__ __forceinline__ uint32_t wave_inclusive_scan32(uint32_t v) {
 // it, as (feature, raw value) entries ordered by (token, feature), to one extent of the layer's
 // candidate pool per wavefront and feature segment (see CollectArgs).  These modes need
 // M % BM == 0 and N % BN == 0 (a shifted tile would report its overlap twice).
-template <typename T, int COLLECT>
+// SEG (storing mode only): K is made of segments of `sps` stages each; segment q of a row starts
+// q * xss (x) / q * wss (W) elements after the row's first segment and rows are xrs / wrs elements apart,
+// so both operands may be gathered from several matrices side by side (see clt_encode_segmented).
+struct SegArgs {
+  int sps;           // stages per segment
+  uint32_t magic;    // ceil(2^32 / sps): segment of stage i = (i * magic) >> 32 for i < 2^16
+  int64_t xss, wss;  // segment strides, elements
+  int xrs, wrs;      // row strides, elements
+};
+
+template <typename T, int COLLECT, bool SEG>
 __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void k_encode_mfma(
     const T *__restrict__ x, const T *__restrict__ w, const T *__restrict__ bias, T *__restrict__ pre,
     int M, int K, int N, int tiles_m, int tiles_n, int total_tiles, int64_t xs, int64_t wstr, int64_t bs,
-    int64_t ps, const SelState *__restrict__ gate, CollectArgs ca) {
+    int64_t ps, const SelState *__restrict__ gate, CollectArgs ca, SegArgs sg) {
+  static_assert(!SEG || COLLECT == 0, "segmented operands only in the storing mode");
   constexpr int CE = 16 / (int)sizeof(T);  // elements per 16-byte chunk
   constexpr int BK = ROWB / (int)sizeof(T);
   // The collecting modes run as persistent workgroups (the grid is one block per CU, block b takes the
@@ -154,7 +165,7 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
   const int per_layer = tiles_m * tiles_n;
   const int nk = K / BK;
 
-  struct TileAt { int layer, tm, tn, m0, n0, rot; };
+  struct TileAt { int layer, tm, tn, m0, n0, om0, on0, rot; };
   auto locate = [&](int bid) {
     TileAt t;
     t.layer = bid / per_layer;
@@ -173,6 +184,7 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
       t.tn = bid / tiles_m; t.tm = bid - t.tn * tiles_m;
     }
     t.m0 = t.tm * BM; t.n0 = t.tn * BN;
+    t.om0 = t.m0; t.on0 = t.n0;       // what the tile owns: it stores nothing before these
     if (t.m0 + BM > M) t.m0 = M - BM;
     if (t.n0 + BN > N) t.n0 = N - BN;
     // K is walked from a tile-dependent starting stage, wrapping around: the CUs of an XCD that share an
@@ -201,19 +213,29 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
   // per instruction.  Lane l lands at row l>>3, chunk position l&7 of its 8-row group and
   // therefore fetches global chunk (l&7) ^ ((row >> 1) & 7).
   const int lr = lane >> 3, lp = lane & 7;
-  const int offE = lr * K + ((lp ^ (lane >> 4)) * CE);          // 8-row groups starting at a multiple of 16
-  const int offO = lr * K + ((lp ^ ((lane >> 4) | 4)) * CE);    // ... at 8 mod 16
-  auto x_rows = [&](const TileAt &t) { return x + (int64_t)t.layer * xs + (int64_t)(t.m0 + wave * 32) * K; };
-  auto w_rows = [&](const TileAt &t) { return w + (int64_t)t.layer * wstr + (int64_t)(t.n0 + wave * 32) * K; };
-  auto stage_k0 = [&](const TileAt &t, int kt) { int q = kt + t.rot; if (q >= nk) q -= nk; return q * BK; };
-  auto issue_stage = [&](unsigned char *stage, const T *xt, const T *wt, int k0) {
+  const int xrs = SEG ? sg.xrs : K, wrs = SEG ? sg.wrs : K;     // row strides
+  const int chE = (lp ^ (lane >> 4)) * CE;                      // 8-row groups starting at a multiple of 16
+  const int chO = (lp ^ ((lane >> 4) | 4)) * CE;                // ... at 8 mod 16
+  const int offE = lr * xrs + chE, offO = lr * xrs + chO;
+  const int woffE = SEG ? lr * wrs + chE : offE, woffO = SEG ? lr * wrs + chO : offO;
+  auto x_rows = [&](const TileAt &t) { return x + (int64_t)t.layer * xs + (int64_t)(t.m0 + wave * 32) * xrs; };
+  auto w_rows = [&](const TileAt &t) { return w + (int64_t)t.layer * wstr + (int64_t)(t.n0 + wave * 32) * wrs; };
+  // the stage walked kt-th by a tile (an index into K / BK)
+  auto stage_k0 = [&](const TileAt &t, int kt) { int q = kt + t.rot; if (q >= nk) q -= nk; return q; };
+  auto issue_stage = [&](unsigned char *stage, const T *xt, const T *wt, int kst) {
     unsigned char *xs_l = stage + wave * 32 * ROWB;
     unsigned char *ws_l = xs_l + BM * ROWB;
+    int64_t xk = (int64_t)kst * BK, wk = xk;
+    if constexpr (SEG) {
+      const int q = sg.sps == 1 ? kst : (int)__umulhi((uint32_t)kst, sg.magic);
+      const int kin = (kst - q * sg.sps) * BK;
+      xk = q * sg.xss + kin;
+      wk = q * sg.wss + kin;
+    }
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-      const int off = (t & 1) ? offO : offE;
-      load16_to_lds(xt + (int64_t)t * 8 * K + k0 + off, xs_l + t * 8 * ROWB);
-      load16_to_lds(wt + (int64_t)t * 8 * K + k0 + off, ws_l + t * 8 * ROWB);
+      load16_to_lds(xt + (int64_t)t * 8 * xrs + xk + ((t & 1) ? offO : offE), xs_l + t * 8 * ROWB);
+      load16_to_lds(wt + (int64_t)t * 8 * wrs + wk + ((t & 1) ? woffO : woffE), ws_l + t * 8 * ROWB);
     }
   };
 
@@ -411,7 +433,13 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
           const uint4 v = *reinterpret_cast<const uint4 *>(park + ml * 256 + ((sl ^ (ml & 15)) * 16));
           const int m = m0 + wm * 64 + ml;
           const int n = n0 + wn * 128 + pass * (128 / NPASS) + sl * EPS;
-          *reinterpret_cast<uint4 *>(pl + (int64_t)m * N + n) = v;
+          // the part of a shifted tile that its neighbour owns is left to the neighbour: the two walk K
+          // from different stages, so their sums may differ in the last bit
+          // (N is a multiple of 4, so a 16-byte piece of bf16 may straddle the line by half)
+          if (m >= cur.om0) {
+            if (n >= cur.on0) *reinterpret_cast<uint4 *>(pl + (int64_t)m * N + n) = v;
+            else if (sizeof(T) == 2 && n + 4 >= cur.on0) *reinterpret_cast<uint2 *>(pl + (int64_t)m * N + n + 4) = make_uint2(v.z, v.w);
+          }
         }
       } else {
         // Two lanes per token row of the parked piece: lane -> row lane % 32, slots [8 hs, 8 hs + 8) with
@@ -679,10 +707,12 @@ static int launch_encode(const void *x, const void *w, const void *b, void *pre,
       cus -= cus % 8;
       if (grid > cus) grid = cus;
     }
-#define CLT_ENC(C)                                                                                               \
-  k_encode_mfma<T, C><<<(unsigned)grid, NTHREADS, 0, stream>>>((const T *)x, (const T *)w, (const T *)b, (T *)pre,    \
-                                                          (int)T_, (int)d, (int)F, (int)tm, (int)tn, (int)nblk,  \
-                                                          xs, wstr, bs, ps, gate, a)
+    const SegArgs noseg = {};
+#define CLT_ENC(C)                                                                                                  \
+  k_encode_mfma<T, C, false><<<(unsigned)grid, NTHREADS, 0, stream>>>((const T *)x, (const T *)w, (const T *)b,     \
+                                                                     (T *)pre, (int)T_, (int)d, (int)F, (int)tm,  \
+                                                                     (int)tn, (int)nblk, xs, wstr, bs, ps, gate,  \
+                                                                     a, noseg)
     if (collect == 0) CLT_ENC(0);
     else if (collect == 1) CLT_ENC(1);
     else CLT_ENC(2);
@@ -695,7 +725,48 @@ static int launch_encode(const void *x, const void *w, const void *b, void *pre,
   return clt_check_launch();
 }
 
+// pre[T][F] = sum over segments q of x_q[T][dseg] . w_q[F][dseg]^T on the matrix-core kernel
+template <typename T>
+static int launch_encode_segmented(const void *x, const void *w, void *pre, int64_t T_, int64_t dseg, int64_t nseg,
+                                   int64_t F, int64_t xss, int64_t xrs, int64_t wss, int64_t wrs, hipStream_t stream) {
+  constexpr int CE = 16 / (int)sizeof(T);
+  constexpr int BK = ROWB / (int)sizeof(T);
+  const int64_t K = dseg * nseg;
+  const bool ok = dseg % BK == 0 && (K / BK) % 2 == 0 && K / BK < 65536 && T_ >= BM && F >= BN && F % 4 == 0 &&
+                  clt_aligned16(x) && clt_aligned16(w) && clt_aligned16(pre) && xss % CE == 0 && wss % CE == 0 &&
+                  xrs % CE == 0 && wrs % CE == 0 && xrs < (1 << 24) && wrs < (1 << 24) && T_ < (1 << 30) &&
+                  F < (1 << 30) && (F * (int64_t)sizeof(T)) % 8 == 0;
+  if (!ok) return CLT_ERR_ARG;
+  const int64_t tm = clt_ceil_div(T_, BM), tn = clt_ceil_div(F, BN), nblk = tm * tn;
+  if (nblk > 2147483647LL) return CLT_ERR_RANGE;
+  SegArgs sg;
+  sg.sps = (int)(dseg / BK);
+  sg.magic = (uint32_t)((0x100000000ull + (uint64_t)sg.sps - 1ull) / (uint64_t)sg.sps);
+  sg.xss = xss; sg.wss = wss; sg.xrs = (int)xrs; sg.wrs = (int)wrs;
+  const CollectArgs none = {};
+  k_encode_mfma<T, 0, true><<<(unsigned)nblk, NTHREADS, 0, stream>>>((const T *)x, (const T *)w, nullptr, (T *)pre, (int)T_,
+                                                                    (int)K, (int)F, (int)tm, (int)tn, (int)nblk, 0, 0, 0,
+                                                                    0, nullptr, none, sg);
+  return clt_check_launch();
+}
+
 }  // namespace
+
+extern "C" int clt_encode_segmented(const void *x, const void *w, void *pre, int64_t T, int64_t d_seg, int64_t n_seg,
+                                    int64_t F, int64_t x_seg_stride, int64_t x_row_stride, int64_t w_seg_stride,
+                                    int64_t w_row_stride, int dtype, void *stream) {
+  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (T < 0 || d_seg <= 0 || n_seg <= 0 || F <= 0 || x_row_stride < d_seg || w_row_stride < d_seg || x_seg_stride < 0 ||
+      w_seg_stride < 0)
+    return CLT_ERR_ARG;
+  if (T == 0) return CLT_OK;
+  if (!x || !w || !pre) return CLT_ERR_ARG;
+  if (dtype == CLT_BF16)
+    return launch_encode_segmented<bf16_t>(x, w, pre, T, d_seg, n_seg, F, x_seg_stride, x_row_stride, w_seg_stride,
+                                           w_row_stride, (hipStream_t)stream);
+  return launch_encode_segmented<float>(x, w, pre, T, d_seg, n_seg, F, x_seg_stride, x_row_stride, w_seg_stride,
+                                        w_row_stride, (hipStream_t)stream);
+}
 
 int clt_launch_encode(const void *x, const void *w, const void *b, void *pre, int64_t T, int64_t d, int64_t F,
                       int64_t L, int64_t xs, int64_t wstr, int64_t bs, int64_t ps, int dtype, int collect,

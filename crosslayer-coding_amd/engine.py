@@ -106,6 +106,26 @@ def encode(x: torch.Tensor, w: torch.Tensor, b: Optional[torch.Tensor],
     return out
 
 
+def encode_segmented(x: torch.Tensor, w: torch.Tensor, n_seg: int, d_seg: int, x_seg_stride: int, x_row_stride: int,
+                     w_seg_stride: int, w_row_stride: int, T: int, F: int,
+                     out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[T, F] = sum over segments q of x_q[T, d_seg] @ w_q[F, d_seg].T, where segment q of either operand
+    starts q * seg_stride elements after the tensor's first element and its rows are row_stride apart: the
+    per-source product behind the JumpReLU threshold gradient (activations.py:183-220) taken from the
+    gradient slab and the packed decoder slab in place."""
+    nat.require_device(x, "encode_segmented")
+    assert x.dtype == w.dtype and x.is_contiguous() and w.is_contiguous()
+    assert (n_seg - 1) * x_seg_stride + (T - 1) * x_row_stride + d_seg <= x.numel()
+    assert (n_seg - 1) * w_seg_stride + (F - 1) * w_row_stride + d_seg <= w.numel()
+    if out is None:
+        out = torch.empty((T, F), dtype=x.dtype, device=x.device)
+    assert out.shape == (T, F) and out.is_contiguous()
+    code = nat.load().clt_encode_segmented(nat.ptr(x), nat.ptr(w), nat.ptr(out), T, d_seg, n_seg, F, x_seg_stride,
+                                           x_row_stride, w_seg_stride, w_row_stride, nat.dtype_code(x.dtype), _stream(x))
+    nat.check(code, "clt_encode_segmented")
+    return out
+
+
 def colstats(pre: torch.Tensor):
     """(mean, denom) fp32 [L, F] of the global ranking z-score (activations.py:281-283)."""
     nat.require_device(pre, "colstats")

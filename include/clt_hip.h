@@ -83,6 +83,24 @@ int clt_encode(const void *x, const void *w, const void *b, void *pre,
                int dtype, void *stream);
 
 /*
+ * The same product with both operands cut into n_seg segments of d_seg along K, each segment
+ * in a matrix of its own:
+ *   pre[t][f] = sum_q sum_k x[q * x_seg_stride + t * x_row_stride + k] * w[q * w_seg_stride + f * w_row_stride + k]
+ * (k < d_seg; strides in elements, a segment stride of 0 repeats the matrix).  No bias, one layer.
+ * It is the product of the stacked loss gradients [T][(L-s) d] with the stacked decoders
+ * [F][(L-s) d] that autograd forms per source layer behind JumpReLU.backward
+ * (clt/models/activations.py:183-220 reached through Decoder.decode, clt/models/decoder.py:176-340),
+ * taken from the gradient slab and the packed decoder slab where they lie, without copying them
+ * side by side.  Needs T >= 256, F >= 256, d_seg a multiple of 64 (bf16) / 32 (fp32) elements with an
+ * even number of such pieces over all segments, 16-byte aligned rows; CLT_ERR_ARG otherwise.
+ */
+int clt_encode_segmented(const void *x, const void *w, void *pre,
+                         int64_t T, int64_t d_seg, int64_t n_seg, int64_t F,
+                         int64_t x_seg_stride, int64_t x_row_stride,
+                         int64_t w_seg_stride, int64_t w_row_stride,
+                         int dtype, void *stream);
+
+/*
  * Per-feature ranking statistics of the global BatchTopK / TokenTopK helper:
  *   mean[l][f]  = mean over tokens of pre[l][:, f]
  *   denom[l][f] = unbiased std over tokens + 1e-6

@@ -62,6 +62,37 @@ def oracle_per_layer(pre, k):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("T,F,d,n,pitch,tied", [(512, 512, 128, 3, 192, False), (256, 768, 256, 4, 320, True),
+                                                 (300, 260, 64, 2, 64, False), (512, 256, 768, 5, 832, False)])
+def test_encode_segmented_equals_product_of_stacked_operands(dev, dtype, T, F, d, n, pitch, tied):
+    """K cut into n segments that live in separate matrices (a gradient slab [n, T, d] and padded
+    feature-major decoders [n, F, pitch]; `tied`: one decoder for all segments): bit for bit the product
+    of the operands copied side by side, and within the encoder tolerance of an fp64 matmul."""
+    g = torch.Generator().manual_seed(T + F + d + n)
+    x = torch.randn(n, T, d, generator=g).to(dtype).to(dev)
+    w = (torch.randn(1 if tied else n, F, pitch, generator=g) / math.sqrt(n * d)).to(dtype).to(dev)
+    got = engine.encode_segmented(x, w, n, d, T * d, d, 0 if tied else F * pitch, pitch, T, F)
+    xs = torch.cat([x[q] for q in range(n)], dim=1).unsqueeze(0).contiguous()                       # [1, T, n d]
+    wsd = torch.cat([w[0 if tied else q][:, :d] for q in range(n)], dim=1).unsqueeze(0).contiguous()  # [1, F, n d]
+    side_by_side = engine.encode(xs, wsd, None)[0]
+    assert torch.equal(got, side_by_side)
+    ref = xs[0].double().cpu() @ wsd[0].double().cpu().T
+    rel = (got.double().cpu() - ref).norm() / ref.norm()
+    assert rel <= TOL[dtype], rel
+
+
+def test_encode_segmented_rejects_shapes_the_matrix_kernel_cannot_take(dev):
+    x = torch.zeros(2, 100, 64, device=dev)
+    w = torch.zeros(2, 256, 64, device=dev)
+    with pytest.raises(nat.CLTNativeError):
+        engine.encode_segmented(x, w, 2, 64, 100 * 64, 64, 256 * 64, 64, 100, 256)   # fewer than 256 tokens
+    x = torch.zeros(3, 256, 32, device=dev)
+    w = torch.zeros(3, 256, 32, device=dev)
+    with pytest.raises(nat.CLTNativeError):
+        engine.encode_segmented(x, w, 3, 32, 256 * 32, 32, 256 * 32, 32, 256, 256)   # an odd number of K pieces
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("L,T,F,k", [(1, 2, 4, 2), (2, 64, 256, 8), (3, 100, 1000, 17), (1, 33, 77, 5),
                                      (2, 16, 64, 64), (2, 16, 64, 100), (1, 1, 8, 3), (2, 512, 2048, 40)])
 def test_batchtopk_per_layer_bit_exact(dev, dtype, L, T, F, k):
