@@ -144,6 +144,31 @@ def test_long_feature_lists_are_in_token_order_and_gradients_repeat_bit_for_bit(
         assert torch.equal(g1[k], g2[k]), k
 
 
+@pytest.mark.parametrize("fn", ["batchtopk", "jumprelu"])
+def test_three_training_steps_repeat_bit_for_bit(dev, fn):
+    # two models built from the same state take three optimisation steps on the same batches: every
+    # parameter and both Adam moments must agree bit for bit (features that fire on nearly every token
+    # give lists far longer than a wavefront, the case whose order used to depend on atomics)
+    import crosslayer_coding_amd as cca
+    wl = BASE.scaled("bw-det", num_layers=2, d_model=128, num_features=256, tokens=1024, dtype="bfloat16",
+                     activation_fn=fn, k=12 if fn == "batchtopk" else None)
+    runs = []
+    for rep in range(2):
+        model, sd, x, targets = build(wl, dev)
+        with torch.no_grad():
+            for l in range(2):
+                model.encoder_module.encoders[l].bias_param[:2] += 8.0
+        opt = cca.CLTAdam(model, lr=1e-2)
+        inputs = {l: x[l].to(dev) for l in range(2)}
+        tg = {l: t.to(dev) for l, t in targets.items()}
+        losses = [float(model.training_step(inputs, tg, opt)) for _ in range(3)]
+        runs.append((losses, {k: v.detach().clone() for k, v in model.state_dict().items()}))
+    assert runs[0][0] == runs[1][0]
+    assert runs[0][0][2] < runs[0][0][0]          # and the steps do reduce the loss
+    for k, v in runs[0][1].items():
+        assert torch.equal(v, runs[1][1][k]), k
+
+
 @pytest.mark.parametrize("tying,fn", [("none", "batchtopk"), ("per_source", "batchtopk"), ("per_target", "batchtopk"),
                                       ("none", "jumprelu")])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
