@@ -589,11 +589,28 @@ def run_backward(args):
     gathered = surv.nnz / L * pairs * d * esz           # one row of g per (survivor, target >= its source)
     dw_bytes = gathered + pairs * F * d * 4
     dw_sec = stages["decoder weight gradient"] * 1e-3
-    roofline = {"kernel": f"k_feature_outer (decoder weight gradient, {L} launches per step)", "bound": "hbm",
-                "achieved": dw_bytes / dw_sec / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": dw_bytes / dw_sec / 1e9 / HBM_PEAK_GBS, "traffic": None,
-                "note": "algorithmic bytes = rows of the loss gradient gathered per (survivor, target) + the fp32 gradient "
-                        "written once; above the HBM peak because the gathered rows are L2 hits"}
+    # The weight-gradient gather reads rows of one layer's loss gradient (every XCD all of it), nearly all of
+    # them from the L2: it is priced against what a bare gather of such rows from such a table reaches on
+    # this GPU, measured now; what has to cross the HBM interface (the fp32 gradient written once, the
+    # gradient slab and the lists read once) is the second figure.
+    yard = gather_yardstick(cca._native.load(build_if_missing=False), dev, wl.tokens * d * esz, d * esz)
+    hbm_bytes = pairs * F * d * 4 + L * wl.tokens * d * esz + surv.nnz * (8 + esz)
+    roofline = {"kernel": f"k_feature_outer (decoder weight gradient, {L} launches per step)",
+                "bound": "l2_gather (measured)", "achieved": gathered / dw_sec / 1e9, "peak": yard, "unit": "GB/s",
+                "frac": (gathered / dw_sec / 1e9 / yard) if yard else None, "traffic": None,
+                "hbm": {"compulsory_bytes": hbm_bytes, "compulsory_GBps": hbm_bytes / dw_sec / 1e9,
+                        "compulsory_frac": hbm_bytes / dw_sec / 1e9 / HBM_PEAK_GBS},
+                "note": "achieved = rows of the loss gradient gathered per (survivor, target) / the stage's time; peak = "
+                        "clt_probe_gather on rows of this length from a table the size of one layer's gradient"}
+    if opt is not None:
+        # Adam is the one stage that streams: per decoder element the fp32 gradient (4), both moments read and
+        # written (16), the feature-major copy read and written (2 e) and the checkpoint-layout parameter (e);
+        # per encoder element gradient, moments and the parameter read and written
+        n_dec, n_enc = pairs * F * d, L * F * d
+        adam_bytes = n_dec * (20 + 3 * esz) + n_enc * (20 + 2 * esz)
+        adam_sec = stages["Adam"] * 1e-3
+        roofline["adam"] = {"bound": "hbm", "bytes": adam_bytes, "achieved": adam_bytes / adam_sec / 1e9,
+                            "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": adam_bytes / adam_sec / 1e9 / HBM_PEAK_GBS}
     return {
         "stages_ms": stages, "roofline": roofline,
         "metric": ("CLT training step tokens/sec (forward, MSE loss, gradients, Adam lr 1e-4 with fp32 moments)"
