@@ -578,24 +578,34 @@ def run_backward(args):
     dval = timed("gradient of the kept activations", lambda: engine.decode_backward_values(
         surv, model.decoder_module.packed(), g, cfg.decoder_tying, mask, ws))
     lists = timed("per-feature token lists", lambda: engine.feature_lists(surv, ws))
-    dw_dec = timed("decoder weight gradient", lambda: engine.decoder_weight_grad(lists, surv, g_model, cfg.decoder_tying))
+    fused = opt is not None and opt.fuses_decoder_step()
+    dw_name = "decoder weight gradient + its Adam step in place" if fused else "decoder weight gradient"
+    if fused:
+        # what training_step does for untied decoders: the gradient rows go from registers into the update of the
+        # moments and of the packed copy, then the checkpoint-layout parameters are rewritten from that copy
+        dw_dec = None
+        timed(dw_name, lambda: opt.decoder_weight_step(lists, surv, g_model))
+    else:
+        dw_dec = timed(dw_name, lambda: engine.decoder_weight_grad(lists, surv, g_model, cfg.decoder_tying))
     _, x_slab, _, _ = model.encoder_module.prepare_slab(inputs)
     dw_enc, db_enc = timed("encoder weight gradient", lambda: engine.encoder_weight_grad(lists, dval, x_slab.contiguous(), F))
     if opt is not None:
         dec_b = bias_grad[torch.tensor([t for s_ in range(L) for t in range(s_, L)], device=dev)].contiguous()
-        timed("Adam", lambda: opt.step({"enc_w": dw_enc, "enc_b": db_enc, "dec_w": dw_dec, "dec_b": dec_b, "theta": None}))
+        timed("Adam (other parameters)" if fused else "Adam",
+              lambda: opt.step({"enc_w": dw_enc, "enc_b": db_enc, "dec_w": dw_dec, "dec_b": dec_b, "theta": None}))
     esz = 2 if wl.dtype == "bfloat16" else 4
     pairs = L * (L + 1) // 2
     gathered = surv.nnz / L * pairs * d * esz           # one row of g per (survivor, target >= its source)
-    dw_bytes = gathered + pairs * F * d * 4
-    dw_sec = stages["decoder weight gradient"] * 1e-3
+    dw_sec = stages[dw_name] * 1e-3
     # The weight-gradient gather reads rows of one layer's loss gradient (every XCD all of it), nearly all of
     # them from the L2: it is priced against what a bare gather of such rows from such a table reaches on
     # this GPU, measured now; what has to cross the HBM interface (the fp32 gradient written once, the
     # gradient slab and the lists read once) is the second figure.
     yard = gather_yardstick(cca._native.load(build_if_missing=False), dev, wl.tokens * d * esz, d * esz)
-    hbm_bytes = pairs * F * d * 4 + L * wl.tokens * d * esz + surv.nnz * (8 + esz)
-    roofline = {"kernel": f"k_feature_outer (decoder weight gradient, {L} launches per step)",
+    # per decoder element the fp32 gradient written once - or, with the step in place, both moments and the packed
+    # copy read and written and the parameter rewritten from the copy
+    hbm_bytes = pairs * F * d * ((16 + 4 * esz) if fused else 4) + L * wl.tokens * d * esz + surv.nnz * (8 + esz)
+    roofline = {"kernel": f"k_feature_outer ({dw_name}, {L} launches per step)",
                 "bound": "l2_gather (measured)", "achieved": gathered / dw_sec / 1e9, "peak": yard, "unit": "GB/s",
                 "frac": (gathered / dw_sec / 1e9 / yard) if yard else None, "traffic": None,
                 "hbm": {"compulsory_bytes": hbm_bytes, "compulsory_GBps": hbm_bytes / dw_sec / 1e9,
@@ -607,8 +617,8 @@ def run_backward(args):
         # written (16), the feature-major copy read and written (2 e) and the checkpoint-layout parameter (e);
         # per encoder element gradient, moments and the parameter read and written
         n_dec, n_enc = pairs * F * d, L * F * d
-        adam_bytes = n_dec * (20 + 3 * esz) + n_enc * (20 + 2 * esz)
-        adam_sec = stages["Adam"] * 1e-3
+        adam_bytes = (0 if fused else n_dec * (20 + 3 * esz)) + n_enc * (20 + 2 * esz)
+        adam_sec = stages["Adam (other parameters)" if fused else "Adam"] * 1e-3
         roofline["adam"] = {"bound": "hbm", "bytes": adam_bytes, "achieved": adam_bytes / adam_sec / 1e9,
                             "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": adam_bytes / adam_sec / 1e9 / HBM_PEAK_GBS}
     return {

@@ -73,6 +73,8 @@ _SIGNATURES = {
     "clt_decoder_weight_grad": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp]),
     "clt_encoder_weight_grad": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
     "clt_adam_step": (_int, [_vp, _vp, _vp, _vp, _i64, _f64, _f64, _f64, _f64, _i64, _int, _vp]),
+    "clt_decoder_weight_grad_adam": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _f64, _f64, _f64, _f64, _i64, _int, _vp]),
+    "clt_unpack_decoders": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
     "clt_adam_step_decoder": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _f64, _f64, _f64, _f64, _i64, _int, _vp]),
     "clt_adam_step_decoders": (_int, [_vp, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _f64, _f64, _f64, _f64, _i64, _int, _vp]),
     "clt_adam_step_many": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _f64, _f64, _f64, _f64, _i64, _int, _vp]),

@@ -183,7 +183,8 @@ class CrossLayerTranscoder(BaseTranscoder):
         return "none", None, None, 1.0
 
     def _loss_and_raw_gradients(self, inputs: Dict[int, torch.Tensor], targets: Dict[int, torch.Tensor],
-                                normalization_method: Optional[str] = None, mean_tg=None, std_tg=None):
+                                normalization_method: Optional[str] = None, mean_tg=None, std_tg=None,
+                                decoder_step=None):
         """(per-layer losses [L] fp32, raw gradients): ``enc_w`` [L, F, d], ``enc_b`` [L, F],
         ``dec_w`` [n_dec, F, d] (feature-major, decoders in slot order: "s->t" pairs, or one per source /
         per target for tied decoders), ``dec_b`` [n_dec, d] (bias gradient of each decoder); all fp32."""
@@ -210,7 +211,9 @@ class CrossLayerTranscoder(BaseTranscoder):
         lists = engine.feature_lists(surv, ws)
         d_off, d_sc = (engine.feature_affine_grad(lists, surv, ws, off, sc, mask) if (off is not None or sc is not None)
                        else (None, None))
-        dw_dec = engine.decoder_weight_grad(lists, surv, g_model, cfg.decoder_tying, off, sc)
+        # ``decoder_step`` (an optimiser whose ``fuses_decoder_step()`` holds): the decoder weights take their
+        # step inside the weight-gradient kernel, after everything that reads the old decoders (below)
+        dw_dec = None if decoder_step is not None else engine.decoder_weight_grad(lists, surv, g_model, cfg.decoder_tying, off, sc)
         _, x_slab, _, _ = self.encoder_module.prepare_slab(inputs)
         x_slab = x_slab.contiguous()
         dw_enc, db_enc = engine.encoder_weight_grad(lists, dval, x_slab, F)
@@ -224,6 +227,8 @@ class CrossLayerTranscoder(BaseTranscoder):
         theta_grad = None
         if cfg.activation_fn == "jumprelu" and self.theta_manager.log_threshold is not None:
             theta_grad = self._log_threshold_gradient(x_slab, g_model, ws)
+        if decoder_step is not None:
+            decoder_step.decoder_weight_step(lists, surv, g_model)
         # bias_grad[t] = column sums of d loss / d rec[t]; a decoder's bias takes the rows of the targets
         # it is added to: its own pair's target, all targets >= its source, or its target (once)
         if cfg.decoder_tying == "none":
@@ -317,7 +322,8 @@ class CrossLayerTranscoder(BaseTranscoder):
         """One optimisation step on the MSE reconstruction loss (trainer.py:663-778 without the
         auxiliary losses): forward, gradients, ``optimizer.step``; returns the loss before the step.
         De-normalisation arguments as in ``loss_and_gradients``."""
-        loss_l, raw = self._loss_and_raw_gradients(inputs, targets, normalization_method, mean_tg, std_tg)
+        fuse = optimizer if getattr(optimizer, "fuses_decoder_step", lambda: False)() else None
+        loss_l, raw = self._loss_and_raw_gradients(inputs, targets, normalization_method, mean_tg, std_tg, decoder_step=fuse)
         optimizer.step(raw)
         return loss_l.sum()
 

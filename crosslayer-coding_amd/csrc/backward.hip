@@ -14,7 +14,8 @@
 //
 // Row vectors are spread over a wavefront in groups of four elements: lane l holds elements
 // c * 256 + 4 l .. + 3 of chunk c (NC4 chunks cover d <= 2048; d % 4 == 0).
-#include "clt_common.h"
+#include <type_traits>
+#include "adam.h"
 
 namespace {
 
@@ -629,12 +630,21 @@ __global__ __launch_bounds__(BW_THREADS) void k_csc_order(const int32_t *ptr, in
 // fits its L2, was measured and dropped: with four rows in flight per wavefront whole rows are 8 % faster.)
 constexpr int FO_NU = 8;
 // T8: as in k_bwd_values_sliced, the last piece of a lane is 8 bytes wide and every lane has one.
-template <typename T, typename CoefT, int NCH, bool DECODER, bool T8 = false>
+// ADAM (untied decoders only): the row is not written; it is the gradient of an Adam step applied on the
+// spot to the moments [n_dec][F][d] and to the feature-major working copy [n_dec][F][pitch] of the decoder.
+struct AdamInPlace {
+  float *m, *v;      // moments, dense like the gradient would be
+  void *w_packed;    // the decoders' working copy
+  int64_t pitch;
+  AdamCoef c;
+};
+template <typename T, typename CoefT, int NCH, bool DECODER, bool T8 = false, bool ADAM = false>
 __global__ __launch_bounds__(BW_THREADS) void k_feature_outer(
     const int32_t *__restrict__ ptr, const int32_t *__restrict__ ltok, const int32_t *__restrict__ lsrc,
     const CoefT *__restrict__ coef, const T *__restrict__ src, float *__restrict__ out, float *__restrict__ rowsum,
     int64_t Tn, int64_t d, int64_t F, int64_t L, int64_t target, int tying, const T *__restrict__ foff = nullptr,
-    const T *__restrict__ fscale = nullptr) {
+    const T *__restrict__ fscale = nullptr, AdamInPlace ad = AdamInPlace()) {
+  static_assert(!ADAM || DECODER, "the in-place step is for decoder rows");
   constexpr int EV = Piece<T>::EV;
   const int lane = lane_id(), wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
   // One launch per layer of the gathered matrix, so that every wavefront of a launch gathers from the
@@ -662,6 +672,35 @@ __global__ __launch_bounds__(BW_THREADS) void k_feature_outer(
 #pragma unroll
       for (int k = 0; k < EV; ++k) acc[c][k] = 0.0f;
     float csum = 0.0f;
+    // ADAM: the row's moments and parameters are asked for now (streaming: they pass through once and must
+    // not push the gathered rows out of the L2) and arrive while the row's gradient is being summed
+    typedef float bw_f4 __attribute__((ext_vector_type(4)));
+    typedef uint32_t bw_u2 __attribute__((ext_vector_type(2)));
+    typedef uint32_t bw_u4 __attribute__((ext_vector_type(4)));
+    constexpr int NG = ADAM ? NFULL * (EV / 4) + (T8 ? 1 : 0) : 1;
+    bw_f4 am[NG], av[NG];
+    typename std::conditional<sizeof(T) == 2, bw_u2, bw_u4>::type aw[NG];
+    float *mrow = nullptr, *vrow = nullptr;
+    T *wrow = nullptr;
+    if constexpr (ADAM) {
+      const int64_t rowi = bw_decoder_slot(tying, s, t, L) * F + f;
+      mrow = ad.m + rowi * d; vrow = ad.v + rowi * d;
+      wrow = reinterpret_cast<T *>(ad.w_packed) + rowi * ad.pitch;
+      auto ask4 = [&](int gi, int64_t at) {
+        am[gi] = __builtin_nontemporal_load(reinterpret_cast<const bw_f4 *>(mrow + at));
+        av[gi] = __builtin_nontemporal_load(reinterpret_cast<const bw_f4 *>(vrow + at));
+        aw[gi] = __builtin_nontemporal_load(reinterpret_cast<const decltype(aw[0] + aw[0]) *>(wrow + at));
+      };
+      int gi = 0;
+      if constexpr (T8) ask4(gi++, tail_at);
+#pragma unroll
+      for (int c = 0; c < NFULL; ++c)
+#pragma unroll
+        for (int k = 0; k < EV; k += 4) {
+          if (on[c]) ask4(gi, (int64_t)c * 64 * EV + lane * EV + k);
+          ++gi;
+        }
+    }
     for (int64_t ls = per_target ? 0 : s; ls <= s; ++ls) {
     const int64_t q = ls * F + f;
     const int32_t b = ptr[q], e = ptr[q + 1];
@@ -712,6 +751,43 @@ __global__ __launch_bounds__(BW_THREADS) void k_feature_outer(
     }
     }
     const int64_t q = s * F + f;
+    if constexpr (ADAM) {
+      // groups of four elements, as they were asked for ahead of the gather
+      auto step4 = [&](int gi, int64_t at, const float *gk) {
+        float mm[4] = {am[gi].x, am[gi].y, am[gi].z, am[gi].w}, vv[4] = {av[gi].x, av[gi].y, av[gi].z, av[gi].w}, pp[4];
+        if constexpr (sizeof(T) == 2) {
+          pp[0] = __uint_as_float(aw[gi].x << 16); pp[1] = __uint_as_float(aw[gi].x & 0xFFFF0000u);
+          pp[2] = __uint_as_float(aw[gi].y << 16); pp[3] = __uint_as_float(aw[gi].y & 0xFFFF0000u);
+        } else {
+          pp[0] = __uint_as_float(aw[gi].x); pp[1] = __uint_as_float(aw[gi].y);
+          pp[2] = __uint_as_float(aw[gi].z); pp[3] = __uint_as_float(aw[gi].w);
+        }
+        T np[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) np[k] = Elem<T>::from_f32(adam_update(pp[k], gk[k], mm[k], vv[k], ad.c));
+        bw_f4 mo = {mm[0], mm[1], mm[2], mm[3]}, vo = {vv[0], vv[1], vv[2], vv[3]};
+        __builtin_nontemporal_store(mo, reinterpret_cast<bw_f4 *>(mrow + at));
+        __builtin_nontemporal_store(vo, reinterpret_cast<bw_f4 *>(vrow + at));
+        if constexpr (sizeof(T) == 2) {
+          bw_u2 wo = {(uint32_t)Elem<T>::raw(np[0]) | ((uint32_t)Elem<T>::raw(np[1]) << 16),
+                      (uint32_t)Elem<T>::raw(np[2]) | ((uint32_t)Elem<T>::raw(np[3]) << 16)};
+          __builtin_nontemporal_store(wo, reinterpret_cast<bw_u2 *>(wrow + at));
+        } else {
+          bw_f4 wo = {(float)np[0], (float)np[1], (float)np[2], (float)np[3]};
+          __builtin_nontemporal_store(wo, reinterpret_cast<bw_f4 *>(wrow + at));
+        }
+      };
+      int gi = 0;
+      if constexpr (T8) step4(gi++, tail_at, acc[NFULL]);
+#pragma unroll
+      for (int c = 0; c < NFULL; ++c)
+#pragma unroll
+        for (int k = 0; k < EV; k += 4) {
+          if (on[c]) step4(gi, (int64_t)c * 64 * EV + lane * EV + k, &acc[c][k]);
+          ++gi;
+        }
+      continue;
+    }
     float *orow = out + (DECODER ? (bw_decoder_slot(tying, s, t, L) * F + f) : q) * d;
     const bool add = DECODER && tying == CLT_TYING_PER_SOURCE && t > s;
     if constexpr (T8) {
@@ -969,6 +1045,42 @@ extern "C" int clt_decoder_weight_grad(const int32_t *list_ptr, const int32_t *l
   } else if (dtype == CLT_BF16) CLT_DW_N(bf16_t); else CLT_DW_N(float);
 #undef CLT_DW_N
 #undef CLT_DW
+  return clt_check_launch();
+}
+
+extern "C" int clt_decoder_weight_grad_adam(const int32_t *list_ptr, const int32_t *list_tok, const int32_t *list_src,
+                                            const void *val, const void *g_model, void *w_packed, float *m, float *v,
+                                            int64_t T, int64_t d, int64_t F, int64_t L, double lr, double beta1, double beta2,
+                                            double eps, int64_t step, int dtype, void *stream) {
+  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (T <= 0 || F <= 0 || L <= 0 || L > 64 || step < 1 || !(beta1 >= 0 && beta1 < 1) || !(beta2 >= 0 && beta2 < 1) ||
+      !list_ptr || !list_tok || !list_src || !val || !g_model || !w_packed || !m || !v)
+    return CLT_ERR_ARG;
+  if (!bw_shape_ok(d, dtype)) return CLT_ERR_RANGE;
+  hipStream_t s = (hipStream_t)stream;
+  const int esz = dtype == CLT_BF16 ? 2 : 4, ev = 16 / esz;
+  const int nc4 = (int)clt_ceil_div(d / ev, 64);   // 16-byte pieces per lane
+  AdamInPlace ad;
+  ad.m = m; ad.v = v; ad.w_packed = w_packed; ad.pitch = clt_pitch(d, esz); ad.c = adam_coef(lr, beta1, beta2, eps, step);
+#define CLT_DWA(CT, N, T8)                                                                                                 \
+  do {                                                                                                                     \
+    for (int64_t t = 0; t < L; ++t) {                                                                                      \
+      k_feature_outer<CT, CT, N, true, T8, true><<<bw_resident_blocks(k_feature_outer<CT, CT, N, true, T8, true>), BW_THREADS, 0, s>>>(list_ptr, list_tok, list_src, (const CT *)val, (const CT *)g_model, nullptr, nullptr, T, d, F, L, t, CLT_TYING_NONE, nullptr, nullptr, ad); \
+    }                                                                                                                      \
+  } while (0)
+#define CLT_DWA_N(CT)                                                                                \
+  do {                                                                                               \
+    switch (nc4) {                                                                                   \
+      case 1: CLT_DWA(CT, 1, false); break; case 2: CLT_DWA(CT, 2, false); break; case 3: CLT_DWA(CT, 3, false); break; \
+      case 4: CLT_DWA(CT, 4, false); break; case 5: CLT_DWA(CT, 5, false); break; case 6: CLT_DWA(CT, 6, false); break; \
+      case 7: CLT_DWA(CT, 7, false); break; default: CLT_DWA(CT, 8, false); break;                     \
+    }                                                                                                \
+  } while (0)
+  if (dtype == CLT_BF16 && d == 768) CLT_DWA(bf16_t, 2, true);
+  else if (dtype == CLT_BF16) CLT_DWA_N(bf16_t);
+  else CLT_DWA_N(float);
+#undef CLT_DWA_N
+#undef CLT_DWA
   return clt_check_launch();
 }
 

@@ -6,6 +6,7 @@
 // decoder vector of every active feature (feature-major packing: one contiguous
 // d-element run, 16 bytes per lane per load) and accumulates in fp32 registers; the
 // output row is written once.
+#include <type_traits>
 #include "clt_common.h"
 
 namespace {
@@ -894,6 +895,55 @@ __global__ __launch_bounds__(256) void k_pack(const T *src, T *dst, int64_t d, i
   }
 }
 
+// [F][pitch] -> [d][F], the way back: decoder z of the slab into the parameter whose address is w_refs[z].
+template <typename T>
+__global__ __launch_bounds__(256) void k_unpack(const T *src, T *const *w_refs, int64_t d, int64_t F, int64_t pitch) {
+  __shared__ T tile[64][65];
+  const T *s = src + (int64_t)blockIdx.z * F * pitch;
+  T *o = w_refs[blockIdx.z];
+  const int64_t f0 = (int64_t)blockIdx.x * 64, d0 = (int64_t)blockIdx.y * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int i = ty; i < 64; i += 4) {
+    int64_t ff = f0 + i, dd = d0 + tx;
+    if (ff < F && dd < d) tile[i][tx] = s[ff * pitch + dd];
+  }
+  __syncthreads();
+  for (int i = ty; i < 64; i += 4) {
+    int64_t dd = d0 + i, ff = f0 + tx;
+    if (dd < d && ff < F) o[dd * F + ff] = tile[tx][i];
+  }
+}
+
+// the same with 4 consecutive elements per access on both sides (d % 4 == 0, F % 4 == 0, 16-byte aligned parameters)
+template <typename T>
+__global__ __launch_bounds__(256) void k_unpack_vec(const T *__restrict__ src, T *const *__restrict__ w_refs, int64_t d, int64_t F,
+                                                    int64_t pitch) {
+  __shared__ T tile[64][68];
+  const T *s = src + (int64_t)blockIdx.z * F * pitch;
+  T *o = w_refs[blockIdx.z];
+  const int64_t f0 = (int64_t)blockIdx.x * 64, d0 = (int64_t)blockIdx.y * 64;
+  const int q = threadIdx.x & 15, r = threadIdx.x >> 4;
+  typedef typename std::conditional<sizeof(T) == 2, uint2, uint4>::type quad_t;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int fl = r + 16 * i;
+    const int64_t f = f0 + fl, dd = d0 + q * 4;
+    if (f < F && dd < d) *reinterpret_cast<quad_t *>(&tile[fl][q * 4]) = *reinterpret_cast<const quad_t *>(s + f * pitch + dd);
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int dl = r + 16 * i;
+    const int64_t dd = d0 + dl, f = f0 + q * 4;
+    if (dd < d && f < F) {
+      T t4[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) t4[k] = tile[q * 4 + k][dl];
+      *reinterpret_cast<quad_t *>(o + dd * F + f) = *reinterpret_cast<const quad_t *>(t4);
+    }
+  }
+}
+
 template <typename T, typename OT>
 __global__ void k_densify_scatter(const int32_t *row_ptr, const int32_t *col, const T *val, OT *out,
                                   int64_t Tn, int64_t F, int64_t L, int64_t out_layer_stride) {
@@ -1204,6 +1254,28 @@ extern "C" int clt_pack_decoder(const void *w_ref, void *w_packed, int64_t d, in
   hipStream_t s = (hipStream_t)stream;
   if (dtype == CLT_BF16) k_pack<bf16_t><<<grid, 256, 0, s>>>((const bf16_t *)w_ref, (bf16_t *)w_packed, d, F, in_stride, out_stride, clt_pitch(d, 2));
   else k_pack<float><<<grid, 256, 0, s>>>((const float *)w_ref, (float *)w_packed, d, F, in_stride, out_stride, clt_pitch(d, 4));
+  return clt_check_launch();
+}
+
+extern "C" int clt_unpack_decoders(const void *w_packed, void *const *w_refs_dev, void *const *w_refs_host, int64_t n_dec,
+                                   int64_t d, int64_t F, int dtype, void *stream) {
+  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (d <= 0 || F <= 0 || n_dec < 0 || n_dec > 65535) return CLT_ERR_ARG;
+  if (n_dec == 0) return CLT_OK;
+  if (!w_packed || !w_refs_dev) return CLT_ERR_ARG;
+  if (clt_ceil_div(d, 64) > 65535) return CLT_ERR_RANGE;
+  dim3 grid((unsigned)clt_ceil_div(F, 64), (unsigned)clt_ceil_div(d, 64), (unsigned)n_dec);
+  hipStream_t s = (hipStream_t)stream;
+  // w_refs_host (optional): the same addresses on the host, to see whether the 4-element kernel may be used
+  bool vec = w_refs_host != nullptr && d % 4 == 0 && F % 4 == 0;
+  for (int64_t i = 0; vec && i < n_dec; ++i) vec = clt_aligned16(w_refs_host[i]);
+  if (vec) {
+    if (dtype == CLT_BF16) k_unpack_vec<bf16_t><<<grid, 256, 0, s>>>((const bf16_t *)w_packed, (bf16_t *const *)w_refs_dev, d, F, clt_pitch(d, 2));
+    else k_unpack_vec<float><<<grid, 256, 0, s>>>((const float *)w_packed, (float *const *)w_refs_dev, d, F, clt_pitch(d, 4));
+  } else {
+    if (dtype == CLT_BF16) k_unpack<bf16_t><<<grid, 256, 0, s>>>((const bf16_t *)w_packed, (bf16_t *const *)w_refs_dev, d, F, clt_pitch(d, 2));
+    else k_unpack<float><<<grid, 256, 0, s>>>((const float *)w_packed, (float *const *)w_refs_dev, d, F, clt_pitch(d, 4));
+  }
   return clt_check_launch();
 }
 

@@ -528,6 +528,37 @@ def decoder_weight_grad(lists, surv: SurvivorList, g: torch.Tensor, tying: str,
     return out
 
 
+def decoder_weight_grad_adam(lists, surv: SurvivorList, g: torch.Tensor, w_packed: torch.Tensor, m: torch.Tensor,
+                             v: torch.Tensor, lr: float, betas, eps: float, step: int) -> None:
+    """``decoder_weight_grad`` and the Adam step of the untied decoder weights in one pass: the moments
+    [n_dec, F, d] and the packed working copy [n_dec, F, pitch] are updated in place, the gradient is never
+    written (trainer.py:663-778 for the decoder weights).  The checkpoint-layout parameters follow with
+    ``unpack_decoders``."""
+    assert g.dtype == surv.dtype and g.is_contiguous() and w_packed.dtype == surv.dtype and w_packed.is_contiguous()
+    ptr, tok, src = lists
+    L, T, F = surv.L, surv.T, surv.F
+    d = g.shape[2]
+    n_dec = L * (L + 1) // 2
+    assert tuple(w_packed.shape) == (n_dec, F, decoder_pitch(d, surv.dtype))
+    assert m.shape == (n_dec, F, d) and v.shape == m.shape and m.dtype == torch.float32 and v.dtype == torch.float32
+    assert m.is_contiguous() and v.is_contiguous()
+    code = nat.load().clt_decoder_weight_grad_adam(nat.ptr(ptr), nat.ptr(tok), nat.ptr(src), nat.ptr(surv.val), nat.ptr(g),
+                                                   nat.ptr(w_packed), nat.ptr(m), nat.ptr(v), T, d, F, L, lr, betas[0],
+                                                   betas[1], eps, step, nat.dtype_code(surv.dtype), _stream(g))
+    nat.check(code, "clt_decoder_weight_grad_adam")
+
+
+def unpack_decoders(w_packed: torch.Tensor, w_refs_dev: torch.Tensor, w_refs_host, d: int, F: int) -> None:
+    """Checkpoint-layout parameters [d, F] (their addresses in the device int64 tensor ``w_refs_dev`` and in the
+    host ctypes array ``w_refs_host``) from the packed working copy [n_dec, F, pitch]."""
+    import ctypes
+    n_dec = w_packed.shape[0]
+    assert w_refs_dev.dtype == torch.int64 and w_refs_dev.numel() == n_dec and w_packed.is_contiguous()
+    code = nat.load().clt_unpack_decoders(nat.ptr(w_packed), nat.ptr(w_refs_dev), ctypes.addressof(w_refs_host), n_dec, d, F,
+                                          nat.dtype_code(w_packed.dtype), _stream(w_packed))
+    nat.check(code, "clt_unpack_decoders")
+
+
 def encoder_weight_grad(lists, dval: torch.Tensor, x: torch.Tensor, F: int):
     """(fp32 [L, F, d], fp32 [L, F]): gradients of the stacked encoder weights and biases."""
     ptr, tok, src = lists

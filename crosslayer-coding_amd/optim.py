@@ -23,6 +23,7 @@ class CLTAdam:
         self.model = model
         self.lr, self.betas, self.eps = float(lr), (float(betas[0]), float(betas[1])), float(eps)
         self.step_count = 0
+        self.fuse_decoder_step = True    # untied decoders: Adam inside the weight-gradient kernel (training_step)
         cfg = model.config
         L, F, d = cfg.num_layers, cfg.num_features, cfg.d_model
         dev = model.device
@@ -61,9 +62,34 @@ class CLTAdam:
             self._tables[key] = ent
         return ent[1], ent[2]
 
+    def fuses_decoder_step(self) -> bool:
+        """Whether the decoder weights can take their Adam step inside the weight-gradient kernel: untied
+        decoders without the per-target feature offset / scale (``fuse_decoder_step = False`` switches it off)."""
+        dec = self.model.decoder_module
+        return (self.fuse_decoder_step and self.model.config.decoder_tying == "none"
+                and dec.feature_offset is None and dec.feature_scale is None)
+
+    @torch.no_grad()
+    def decoder_weight_step(self, lists, surv, g_model) -> None:
+        """The decoder weights' part of the NEXT ``step`` (which must follow with ``raw["dec_w"] = None``), taken
+        straight from the survivor lists: gradient rows go from registers into the update of the moments and
+        of the packed copy; the checkpoint-layout parameters are then rewritten from the packed copy."""
+        from . import engine
+        dec = self.model.decoder_module
+        packed = dec.packed()
+        ws = [lin.weight.data for lin in dec._ordered()]
+        assert all(w.is_contiguous() and w.shape == ws[0].shape and w.dtype == ws[0].dtype for w in ws)
+        d, F = ws[0].shape
+        m_w, v_w = self.state["dec_w"]
+        engine.decoder_weight_grad_adam(lists, surv, g_model, packed, m_w, v_w, self.lr, self.betas, self.eps,
+                                        self.step_count + 1)
+        w_dev, w_host = self._pointer_table("w", ws)
+        engine.unpack_decoders(packed, w_dev, w_host, d, F)
+
     @torch.no_grad()
     def step(self, raw) -> None:
-        """``raw``: the gradient tensors of ``CrossLayerTranscoder._loss_and_raw_gradients``."""
+        """``raw``: the gradient tensors of ``CrossLayerTranscoder._loss_and_raw_gradients``; ``dec_w`` is None
+        when ``decoder_weight_step`` has already applied it."""
         model = self.model
         self.step_count += 1
         w_slab, b_slab = model.encoder_module.stacked()
@@ -82,16 +108,17 @@ class CLTAdam:
         assert all(w.is_contiguous() and w.shape == ws[0].shape and w.dtype == ws[0].dtype for w in ws)
         assert all(b.is_contiguous() and b.numel() == bs[0].numel() and b.dtype == bs[0].dtype for b in bs)
         d, F = ws[0].shape
-        assert packed.is_contiguous() and raw["dec_w"].is_contiguous() and raw["dec_w"].dtype == torch.float32
-        from . import engine
-        assert tuple(raw["dec_w"].shape) == (len(ws), F, d)
-        assert tuple(packed.shape) == (len(ws), F, engine.decoder_pitch(d, ws[0].dtype))
-        w_dev, w_host = self._pointer_table("w", ws)
-        code = lib.clt_adam_step_decoders(nat.ptr(w_dev), ctypes.addressof(w_host), len(ws), nat.ptr(packed),
-                                          nat.ptr(raw["dec_w"]), nat.ptr(m_w), nat.ptr(v_w), d, F, self.lr,
-                                          self.betas[0], self.betas[1], self.eps, self.step_count,
-                                          nat.dtype_code(ws[0].dtype), nat.current_stream(ws[0].device))
-        nat.check(code, "clt_adam_step_decoders")
+        if raw["dec_w"] is not None:
+            assert packed.is_contiguous() and raw["dec_w"].is_contiguous() and raw["dec_w"].dtype == torch.float32
+            from . import engine
+            assert tuple(raw["dec_w"].shape) == (len(ws), F, d)
+            assert tuple(packed.shape) == (len(ws), F, engine.decoder_pitch(d, ws[0].dtype))
+            w_dev, w_host = self._pointer_table("w", ws)
+            code = lib.clt_adam_step_decoders(nat.ptr(w_dev), ctypes.addressof(w_host), len(ws), nat.ptr(packed),
+                                              nat.ptr(raw["dec_w"]), nat.ptr(m_w), nat.ptr(v_w), d, F, self.lr,
+                                              self.betas[0], self.betas[1], self.eps, self.step_count,
+                                              nat.dtype_code(ws[0].dtype), nat.current_stream(ws[0].device))
+            nat.check(code, "clt_adam_step_decoders")
         b_dev, _ = self._pointer_table("b", bs)
         assert raw["dec_b"].is_contiguous() and raw["dec_b"].dtype == torch.float32
         code = lib.clt_adam_step_many(nat.ptr(b_dev), nat.ptr(raw["dec_b"]), nat.ptr(m_b), nat.ptr(v_b), len(bs),

@@ -498,6 +498,28 @@ int clt_encoder_weight_grad(const int32_t *list_ptr, const int32_t *list_tok, co
 int clt_adam_step(void *param, const float *grad, float *m, float *v, int64_t n,
                   double lr, double beta1, double beta2, double eps, int64_t step,
                   int dtype, void *stream);
+
+/*
+ * Decoder weight gradient and its Adam step in one pass, for untied decoders: what
+ * clt_decoder_weight_grad followed by clt_adam_step_decoders computes (loss.backward() and
+ * optimizer.step() of clt/training/trainer.py:663-778 for the decoder weights), without the fp32
+ * gradient [n_dec][F][d] ever reaching memory: every gradient row goes from the registers that
+ * summed it straight into the update of the moments m, v [n_dec][F][d] and of the feature-major
+ * working copy w_packed [n_dec][F][pitch].  Bit-identical to the two-call sequence.  The
+ * checkpoint-layout parameters [d][F] are NOT written: clt_unpack_decoders brings them up to date
+ * from the working copy (w_refs_dev: device array of n_dec parameter addresses, w_refs_host: the
+ * same addresses in host memory or NULL, as for clt_adam_step_decoders).  Everything that reads the decoders of the step being differentiated
+ * (clt_decode_backward_values, clt_feature_affine_grad, the threshold-gradient product) must have
+ * run before.
+ */
+int clt_decoder_weight_grad_adam(const int32_t *list_ptr, const int32_t *list_tok,
+                                 const int32_t *list_src, const void *val, const void *g_model,
+                                 void *w_packed, float *m, float *v,
+                                 int64_t T, int64_t d, int64_t F, int64_t L,
+                                 double lr, double beta1, double beta2, double eps, int64_t step,
+                                 int dtype, void *stream);
+int clt_unpack_decoders(const void *w_packed, void *const *w_refs_dev, void *const *w_refs_host,
+                        int64_t n_dec, int64_t d, int64_t F, int dtype, void *stream);
 int clt_adam_step_decoder(void *w_ref, void *w_packed, const float *grad_packed, float *m, float *v,
                           int64_t d, int64_t F, double lr, double beta1, double beta2, double eps,
                           int64_t step, int dtype, void *stream);

@@ -144,6 +144,45 @@ def test_long_feature_lists_are_in_token_order_and_gradients_repeat_bit_for_bit(
         assert torch.equal(g1[k], g2[k]), k
 
 
+@pytest.mark.parametrize("dtype,d_model,fn", [("bfloat16", 128, "batchtopk"), ("bfloat16", 768, "batchtopk"),
+                                              ("float32", 64, "batchtopk"), ("bfloat16", 128, "jumprelu")])
+def test_adam_inside_the_weight_gradient_kernel_equals_the_two_step_sequence(dev, dtype, d_model, fn):
+    # untied decoders: training_step lets the decoder weights take their Adam step inside the weight-gradient
+    # kernel (no fp32 gradient in memory, parameters rewritten from the packed copy); three steps must leave
+    # every parameter, the packed copy and both moments bit-identical to gradient-then-Adam
+    import crosslayer_coding_amd as cca
+    wl = BASE.scaled("bw-fuse", num_layers=3, d_model=d_model, num_features=256, tokens=256, dtype=dtype,
+                     activation_fn=fn, k=10 if fn == "batchtopk" else None)
+    runs = []
+    for fuse in (True, False):
+        model, sd, x, targets = build(wl, dev)
+        opt = cca.CLTAdam(model, lr=1e-2)
+        opt.fuse_decoder_step = fuse
+        assert opt.fuses_decoder_step() == fuse
+        inputs = {l: x[l].to(dev) for l in range(3)}
+        tg = {l: t.to(dev) for l, t in targets.items()}
+        losses = [float(model.training_step(inputs, tg, opt)) for _ in range(3)]
+        runs.append((losses, {k: v.detach().clone() for k, v in model.state_dict().items()},
+                     model.decoder_module.packed().clone(), [t.clone() for t in opt.state["dec_w"]]))
+    assert runs[0][0] == runs[1][0]
+    for k, v in runs[0][1].items():
+        assert torch.equal(v, runs[1][1][k]), k
+    assert torch.equal(runs[0][2], runs[1][2])
+    for a, b in zip(runs[0][3], runs[1][3]):
+        assert torch.equal(a, b)
+    # the parameters are what the packed copy holds
+    model_keys = [k for k in runs[0][1] if k.startswith("decoder_module.decoders.") and k.endswith(".weight")]
+    for i, k in enumerate(sorted(model_keys, key=lambda n: [int(p) for p in n.split(".")[2].split("->")])):
+        assert torch.equal(runs[0][1][k].t(), runs[0][2][i][:, :d_model]), k
+
+
+def test_tied_decoders_do_not_fuse_the_step(dev):
+    import crosslayer_coding_amd as cca
+    wl = BASE.scaled("bw-nofuse", num_layers=2, d_model=64, num_features=128, tokens=64, decoder_tying="per_source")
+    model, sd, x, targets = build(wl, dev)
+    assert not cca.CLTAdam(model).fuses_decoder_step()
+
+
 @pytest.mark.parametrize("fn", ["batchtopk", "jumprelu"])
 def test_three_training_steps_repeat_bit_for_bit(dev, fn):
     # two models built from the same state take three optimisation steps on the same batches: every
