@@ -105,6 +105,73 @@ def test_c2_jumprelu_forward_at_full_size(dev):
     _free()
 
 
+def test_c2_training_step_at_full_size(dev):
+    """One optimisation step of the JumpReLU configuration at its own size: the backward kernels index a
+    decoder slab and moment slabs of 1.0e10 elements, the threshold gradient takes its dense product from
+    24 K-segments of the gradient slab and of the packed decoders, and the untied decoder weights take their
+    Adam step inside the weight-gradient kernel (no 40 GB fp32 gradient).  The weight gradients of the first,
+    a middle and the LAST decoder pair are checked against dense torch formulations, the in-place step against
+    torch.optim.Adam on those gradients, and the step as a whole through the loss."""
+    wl = synth.WORKLOADS["c2"]
+    L, T, F, d = wl.num_layers, wl.tokens, wl.num_features, wl.d_model
+    model, inputs, _ = synth.build_model(wl, dev)
+    model.eval()
+    tgt = synth.make_targets(wl, dev)
+    targets = {l: tgt[l] for l in range(L)}
+    lr = 1e-3
+    opt = cca.CLTAdam(model, lr=lr)
+    assert opt.fuses_decoder_step()
+    pairs = [(0, 0), (7, 19), (L - 1, L - 1)]                    # slots 0, a middle one, 299
+    slot_of = lambda s, t: s * L - (s * (s - 1)) // 2 + (t - s)  # noqa: E731
+    # the gradients as separate tensors first (the two-step route: 40 GB of fp32 decoder gradients)
+    recs, surv = model.forward_with_survivors(inputs)
+    diff = torch.stack([recs[l] for l in range(L)]).float() - tgt.float()
+    want_loss = float((diff.double() ** 2).mean(dim=(1, 2)).sum())
+    g32 = 2.0 * diff / (T * d)                                   # d loss / d rec, [L, T, d]
+    del recs, diff
+    dense = engine.densify(surv)                                 # kept activations, [L, T, F] bf16 (6.4 GB)
+    loss_l, raw = model._loss_and_raw_gradients(inputs, targets)
+    assert abs(float(loss_l.sum()) - want_loss) <= 1e-4 * want_loss
+    kept = {}
+    for s, t in pairs:
+        got = raw["dec_w"][slot_of(s, t)]                        # [F, d]
+        want = dense[s].float().t() @ g32[t]                     # dW[s->t] = a[s]^T g[t]
+        err = orc.rel_l2(got.cpu(), want.cpu())
+        assert err <= 2e-2, (s, t, err)                          # the kernel reads g rounded to bf16
+        kept[(s, t)] = got.t().contiguous().clone()              # checkpoint layout [d, F]
+    assert raw["theta"] is not None and bool(torch.isfinite(raw["theta"]).all())
+    del dense, g32, raw, surv, want, got
+    _free()
+    before = {k: model.decoder_module.decoders[f"{k[0]}->{k[1]}"].weight.detach().float().clone() for k in pairs}
+    theta_before = model.theta_manager.log_threshold.detach().float().clone()
+    # the step itself, with the decoder weights updated inside the weight-gradient kernel
+    loss0 = float(model.training_step(inputs, targets, opt))
+    assert abs(loss0 - want_loss) <= 1e-4 * want_loss
+    for (s, t) in pairs:
+        p = torch.nn.Parameter(before[(s, t)].clone())
+        p.grad = kept[(s, t)]
+        torch.optim.Adam([p], lr=lr, betas=(0.9, 0.999), eps=1e-8).step()
+        want = p.detach().to(torch.bfloat16)
+        got = model.decoder_module.decoders[f"{s}->{t}"].weight.detach()
+        same = (got.view(torch.int16) == want.view(torch.int16)).float().mean()
+        # fp32 rounding differences can move a value that sits on a bf16 rounding boundary by one ulp (the
+        # gradients here are of the order of eps, so the step is not simply lr * sign(g))
+        assert float(same) >= 0.99, (s, t, float(same))
+        assert orc.rel_l2(got.float().cpu(), want.float().cpu()) <= 1e-3
+        assert float((got.float() != before[(s, t)]).float().mean()) > 0.1     # the step did change bf16 values
+        assert torch.equal(model.decoder_module.packed()[slot_of(s, t)][:, :d], got.t())
+    del before, kept
+    _free()
+    theta_after = model.theta_manager.log_threshold.detach().float()
+    # (log_threshold is a bf16 parameter near -1: a step of lr = 1e-3 is below half an ulp for most elements)
+    assert bool(torch.isfinite(theta_after).all()) and float((theta_after != theta_before).float().mean()) > 0.01
+    loss1, _ = model._loss_and_raw_gradients(inputs, targets)
+    assert float(loss1.sum()) < loss0, (float(loss1.sum()), loss0)
+    print(f"c2 training step: loss {loss0:.5f} -> {float(loss1.sum()):.5f}")
+    del model, inputs, opt
+    _free()
+
+
 # ---- C3: decoders tied per target, 8192 tokens, d_model 2048 -------------------------------------------
 def test_c3_per_target_forward_at_full_size(dev):
     wl = synth.WORKLOADS["c3"]
