@@ -206,6 +206,72 @@ def test_c3_per_target_forward_at_full_size(dev):
     _free()
 
 
+def test_c3_training_step_at_full_size(dev):
+    """Gradients and one optimisation step with decoders tied per target at the configuration's own size
+    (d_model 2048 is the widest row the backward kernels take, 8192 tokens): a decoder matrix sums the token
+    lists of all its sources, the value gradients walk all sources of a target.  Against dense torch
+    formulations of the reference's computation (decoder.py:208-251 differentiated)."""
+    wl = synth.WORKLOADS["c3"]
+    L, T, F, d, k = wl.num_layers, wl.tokens, wl.num_features, wl.d_model, wl.k
+    model, inputs, _ = synth.build_model(wl, dev)
+    model.eval()
+    tgt = synth.make_targets(wl, dev)
+    targets = {l: tgt[l] for l in range(L)}
+    loss, grads = model.loss_and_gradients(inputs, targets)
+    recs, surv = model.forward_with_survivors(inputs)
+    diff = torch.stack([recs[l] for l in range(L)]).float() - tgt.float()
+    want_loss = float((diff.double() ** 2).mean(dim=(1, 2)).sum())
+    assert abs(float(loss) - want_loss) <= 1e-4 * want_loss
+    g32 = 2.0 * diff / (T * d)
+    del recs, diff
+    dense = engine.densify(surv)                                  # [L, T, F] bf16, 4.3 GB
+    # decoder t: rec[t] = (sum over s <= t of a[s]) W[t]^T + b[t]   =>   dW[t] = g[t]^T sum_s a[s]
+    for t in (0, 8, L - 1):
+        summed = torch.zeros(T, F, dtype=torch.float32, device=dev)
+        for s_ in range(t + 1):
+            summed += dense[s_].float()
+        want = g32[t].t() @ summed
+        err = orc.rel_l2(grads[f"decoder_module.decoders.{t}.weight"].float().cpu(), want.cpu())
+        assert err <= 2e-2, (t, err)
+        err_b = orc.rel_l2(grads[f"decoder_module.decoders.{t}.bias_param"].cpu(), g32[t].sum(dim=0).cpu())
+        assert err_b <= 1e-3, (t, err_b)
+    del summed, want
+    # encoder s: d loss / d a[s] = sum over t >= s of g[t] W[t], through the straight-through gate
+    for s_ in (0, L - 1, 9):
+        dact = None
+        for t in range(s_, L):
+            term = g32[t] @ model.decoder_module.decoders[t].weight.float()
+            dact = term if dact is None else dact + term
+        dpre = dact * (dense[s_] != 0)
+        err_w = orc.rel_l2(grads[f"encoder_module.encoders.{s_}.weight"].cpu(), (dpre.t() @ inputs[s_].float()).cpu())
+        err_b = orc.rel_l2(grads[f"encoder_module.encoders.{s_}.bias_param"].cpu(), dpre.sum(dim=0).cpu())
+        assert err_w <= 2e-2 and err_b <= 2e-2, (s_, err_w, err_b)
+    names = ["decoder_module.decoders.8.weight", f"decoder_module.decoders.{L - 1}.weight", "encoder_module.encoders.9.weight"]
+    params = dict(model.named_parameters())
+    g_ref = {n: grads[n].float().contiguous().clone() for n in names}
+    before = {n: params[n].detach().float().clone() for n in names}
+    del dense, dact, dpre, term, g32, grads, surv
+    _free()
+    # one optimisation step (two-step route: a tied matrix collects its gradient over several launches)
+    opt = cca.CLTAdam(model, lr=1e-4)
+    assert not opt.fuses_decoder_step()
+    loss0 = float(model.training_step(inputs, targets, opt))
+    assert abs(loss0 - want_loss) <= 1e-4 * want_loss
+    for n in names:
+        p = torch.nn.Parameter(before[n].clone())
+        p.grad = g_ref[n]
+        torch.optim.Adam([p], lr=1e-4, betas=(0.9, 0.999), eps=1e-8).step()
+        want = p.detach().to(torch.bfloat16)
+        got = params[n].detach()
+        same = (got.view(torch.int16) == want.view(torch.int16)).float().mean()
+        assert float(same) >= 0.99, (n, float(same))
+        assert orc.rel_l2(got.float().cpu(), want.float().cpu()) <= 1e-3
+        assert float((got.float() != before[n]).float().mean()) > 0.05    # the step did change bf16 values
+    print(f"c3 training step: loss {loss0:.5f}")
+    del model, inputs, opt, params, before, g_ref
+    _free()
+
+
 # ---- C4: training step at the GPT-2-small x32 shape, bf16 parameters, fp32 Adam moments ------------------
 def _dense_dact(model, g32, s, L):
     """d loss / d activation of source layer s as the reference's autograd forms it: sum over the targets
