@@ -145,12 +145,10 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
   static_assert(!SEG || COLLECT == 0, "segmented operands only in the storing mode");
   constexpr int CE = 16 / (int)sizeof(T);  // elements per 16-byte chunk
   constexpr int BK = ROWB / (int)sizeof(T);
-  // The collecting modes run as persistent workgroups (the grid is one block per CU, block b takes the
-  // tiles b, b + gridDim.x, ...) and overlap the start of the next tile with the end of this one: their
-  // epilogue parks only in the second stage buffer, 32 tokens of a wave tile at a time, so the first
-  // stage of the next tile is asked for two stages before this tile's K loop ends and has landed when
-  // the epilogue is over.  The storing mode parks whole wave tiles in both buffers, one tile per block.
-  constexpr bool OVERLAP = COLLECT != 0;
+  // Persistent workgroups (the grid is one block per CU, block b takes the tiles b, b + gridDim.x, ...)
+  // that overlap the start of the next tile with the end of this one: the epilogue parks only in the
+  // second stage buffer, 32 tokens of a wave tile at a time, so the first stage of the next tile is asked
+  // for two stages before this tile's K loop ends and has landed when the epilogue is over.
   // Two separate stage buffers (not one array with an offset): the compiler can then tell that
   // a fragment read of one stage does not depend on the direct-to-LDS loads in flight into the
   // other, and does not wait for them.
@@ -369,26 +367,24 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
       body(stage1, stage0, false, [&]() { issue_stage(stage1, xt, wt, stage_k0(cur, kt + 3)); });
     }
     // the last two stages: the first buffer is free after the first of them and takes the next tile's
-    // first stage (overlapping modes); nothing may be in flight into the second one, which is parked in
+    // first stage; nothing may be in flight into the second one, which is parked in
     body(stage0, stage1, false, [&]() {
-      if (OVERLAP && has_next) issue_stage(stage0, x_rows(nxt_tile), w_rows(nxt_tile), stage_k0(nxt_tile, 0));
+      if (has_next) issue_stage(stage0, x_rows(nxt_tile), w_rows(nxt_tile), stage_k0(nxt_tile, 0));
     });
     body(stage1, stage0, true, [&]() {});
     // past the barrier of the last stage no wavefront reads either buffer any more
 
     // ---- epilogue.  The accumulator layout gives a lane 4 consecutive features of one token,
     // i.e. 8-byte pieces scattered over 32 rows per store - slow to write.  Each wavefront
-    // therefore parks its tile in LDS and works on it row by row from there: the storing mode the
-    // whole 64 x 128 tile (16 KB per wavefront for bf16, two passes of 64 features for fp32) in its
-    // eighth of the two stage buffers, the collecting modes 32 tokens at a time (8 KB) in its eighth
-    // of the second buffer.
+    // therefore parks its tile in LDS, 32 tokens at a time (8 KB; two passes of 64 features for fp32) in its
+    // eighth of the second stage buffer, and works on it row by row from there.
     T *pl = pre + (int64_t)layer * ps;
     // The epilogue's addresses are rebuilt from the lane number for every tile.  Left visible as loop
     // invariants they would be computed once ahead of the tile loop and live across the K loop.
     int lane_e = lane;
     asm volatile("" : "+v"(lane_e));
     const int l31 = lane_e & 31, lh = lane_e >> 5;
-    unsigned char *park = OVERLAP ? stage1 + wave * (STAGE / 8) : (wave < 4 ? stage0 : stage1) + (wave & 3) * (STAGE / 4);
+    unsigned char *park = stage1 + wave * (STAGE / 8);
     constexpr int NPASS = sizeof(T) == 2 ? 1 : 2;           // feature halves per pass
     constexpr int JP = 4 / NPASS;                            // 32-feature groups per pass
     // token groups [i0, i0 + ni) of feature pass `pass` -> rows (i - i0) * 32 + l31 of 256 bytes
@@ -425,13 +421,15 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
 #pragma unroll
     for (int pass = 0; pass < NPASS; ++pass) {
       if constexpr (COLLECT == 0) {
-        park_rows(pass, 0, 2);
-        // the wavefront reads its own tile back: lane -> (row = it*4 + lane/16, slot = lane%16)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+        park_rows(pass, h, 1);
+        // the wavefront reads its own piece back: lane -> (row = it*4 + lane/16, slot = lane%16)
 #pragma unroll 4
-        for (int it = 0; it < 16; ++it) {
+        for (int it = 0; it < 8; ++it) {
           const int ml = it * 4 + (lane_e >> 4), sl = lane_e & 15;
           const uint4 v = *reinterpret_cast<const uint4 *>(park + ml * 256 + ((sl ^ (ml & 15)) * 16));
-          const int m = m0 + wm * 64 + ml;
+          const int m = m0 + wm * 64 + h * 32 + ml;
           const int n = n0 + wn * 128 + pass * (128 / NPASS) + sl * EPS;
           // the part of a shifted tile that its neighbour owns is left to the neighbour: the two walk K
           // from different stages, so their sums may differ in the last bit
@@ -440,6 +438,7 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
             if (n >= cur.on0) *reinterpret_cast<uint4 *>(pl + (int64_t)m * N + n) = v;
             else if (sizeof(T) == 2 && n + 4 >= cur.on0) *reinterpret_cast<uint2 *>(pl + (int64_t)m * N + n + 4) = make_uint2(v.z, v.w);
           }
+        }
         }
       } else {
         // Two lanes per token row of the parked piece: lane -> row lane % 32, slots [8 hs, 8 hs + 8) with
@@ -652,7 +651,6 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
     cur = nxt_tile;
     load_bias(cur);
     __builtin_amdgcn_sched_barrier(0);   // the bias stays ahead of the stage loads: the wait above counts on it
-    if (!OVERLAP) issue_stage(stage0, x_rows(cur), w_rows(cur), stage_k0(cur, 0));
     issue_stage(stage1, x_rows(cur), w_rows(cur), stage_k0(cur, 1));
   }
   __builtin_amdgcn_s_waitcnt(0);   // no direct-to-LDS load may be in flight when the block retires
@@ -683,6 +681,17 @@ static bool encode_fast_ok(const void *x, const void *w, const void *b, const vo
          F < (1 << 30) && d < (1 << 30) && (!b || (((uintptr_t)b) % 16 == 0 && bs % 8 == 0));
 }
 
+// One persistent workgroup per CU (a whole number of rounds over the 8 XCDs, so that block b stays on XCD
+// b % 8 for all of its tiles), or one per tile when there are fewer tiles; 0 when the device cannot be asked.
+static int64_t persistent_grid(int64_t tiles) {
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess ||
+      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 8)
+    return 0;
+  cus -= cus % 8;
+  return tiles < cus ? tiles : cus;
+}
+
 template <typename T>
 static int launch_encode(const void *x, const void *w, const void *b, void *pre, int64_t T_, int64_t d, int64_t F,
                          int64_t L, int64_t xs, int64_t wstr, int64_t bs, int64_t ps, int collect,
@@ -695,18 +704,8 @@ static int launch_encode(const void *x, const void *w, const void *b, void *pre,
     if (nblk > 2147483647LL) return CLT_ERR_RANGE;
     CollectArgs none = {};
     const CollectArgs a = ca ? *ca : none;
-    // the collecting modes run one persistent workgroup per CU (a whole number of rounds over the 8 XCDs,
-    // so that block b stays on XCD b % 8 for all of its tiles); the storing mode one tile per workgroup,
-    // unless it is gated: that launch usually finds nothing to do, which a small grid finds out sooner
-    int64_t grid = nblk;
-    if (collect || gate) {
-      int dev = 0, cus = 0;
-      if (hipGetDevice(&dev) != hipSuccess ||
-          hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 8)
-        return CLT_ERR_LAUNCH;
-      cus -= cus % 8;
-      if (grid > cus) grid = cus;
-    }
+    const int64_t grid = persistent_grid(nblk);
+    if (grid <= 0) return CLT_ERR_LAUNCH;
     const SegArgs noseg = {};
 #define CLT_ENC(C)                                                                                                  \
   k_encode_mfma<T, C, false><<<(unsigned)grid, NTHREADS, 0, stream>>>((const T *)x, (const T *)w, (const T *)b,     \
@@ -744,7 +743,9 @@ static int launch_encode_segmented(const void *x, const void *w, void *pre, int6
   sg.magic = (uint32_t)((0x100000000ull + (uint64_t)sg.sps - 1ull) / (uint64_t)sg.sps);
   sg.xss = xss; sg.wss = wss; sg.xrs = (int)xrs; sg.wrs = (int)wrs;
   const CollectArgs none = {};
-  k_encode_mfma<T, 0, true><<<(unsigned)nblk, NTHREADS, 0, stream>>>((const T *)x, (const T *)w, nullptr, (T *)pre, (int)T_,
+  const int64_t grid = persistent_grid(nblk);
+  if (grid <= 0) return CLT_ERR_LAUNCH;
+  k_encode_mfma<T, 0, true><<<(unsigned)grid, NTHREADS, 0, stream>>>((const T *)x, (const T *)w, nullptr, (T *)pre, (int)T_,
                                                                     (int)K, (int)F, (int)tm, (int)tn, (int)nblk, 0, 0, 0,
                                                                     0, nullptr, none, sg);
   return clt_check_launch();
