@@ -105,6 +105,59 @@ class CrossLayerTranscoder(BaseTranscoder):
             for m in (self.encoder_module, self.decoder_module, self.theta_manager):
                 m.device, m.dtype = w.device, w.dtype
 
+    # ---- float16 models ----------------------------------------------------------------------------------
+    # The kernels implement float32 and bfloat16.  A model whose parameters are float16 (config.clt_dtype, or
+    # module.half()) keeps them in float16 - state dict, checkpoints and outputs are float16 as the reference's
+    # are - and computes its forward on the float32 kernels from a float32 copy of them, with every dense
+    # product and the thresholds rounded to float16 where the reference's float16 tensors would round
+    # (engine.emulate_dtype); sums across features and sources are therefore the more exact float32 ones.
+    # Forward-path methods only: gradients, the optimiser step and theta estimation raise NotImplementedError.
+    def _is_half(self) -> bool:
+        self._sync_device()
+        return self.dtype == torch.float16
+
+    def _half_twin(self) -> "CrossLayerTranscoder":
+        import copy
+        sd = self.state_dict()
+        key = tuple((k, v.data_ptr(), v._version) for k, v in sd.items())
+        if getattr(self, "_twin", None) is None or self._twin_key[0] != (self.config.activation_fn, self.device):
+            cfg = copy.deepcopy(self.config)
+            cfg.clt_dtype = "float32"
+            twin = CrossLayerTranscoder(cfg, None, self.device, profiler=self.profiler)
+            twin.fuse_encode_select = False      # the pre-activations must exist to be rounded
+            object.__setattr__(self, "_twin", twin)
+            self._twin_key = ((self.config.activation_fn, self.device), None)
+        if self._twin_key[1] != key:
+            self._twin.load_state_dict({k: v.detach().float() for k, v in sd.items()}, strict=False)
+            self._twin.decoder_module.invalidate_packed()
+            self._twin_key = (self._twin_key[0], key)
+        return self._twin
+
+    def _via_twin(self, name: str, *args):
+        def cast_in(a):
+            if isinstance(a, torch.Tensor):
+                return a.to(device=self.device, dtype=torch.float32) if a.is_floating_point() else a
+            if isinstance(a, dict):
+                return {k: cast_in(v) for k, v in a.items()}
+            return a
+
+        def cast_out(a):
+            if isinstance(a, torch.Tensor):
+                return a.to(torch.float16) if a.is_floating_point() else a
+            if isinstance(a, dict):
+                return {k: cast_out(v) for k, v in a.items()}
+            if isinstance(a, tuple):
+                return tuple(cast_out(v) for v in a)
+            return a
+
+        twin = self._half_twin()
+        with engine.emulate_dtype(torch.float16):
+            return cast_out(getattr(twin, name)(*[cast_in(a) for a in args]))
+
+    def _no_half(self, what: str) -> None:
+        if self._is_half():
+            raise NotImplementedError(f"{what} is not built for float16 models (the kernels implement float32 and bfloat16)")
+
     def release_workspace(self) -> None:
         """Free the cached scratch buffers (pre-activations, selection workspace)."""
         if self._ws is not None:
@@ -112,10 +165,13 @@ class CrossLayerTranscoder(BaseTranscoder):
 
     # ---- reference API: thin delegations ------------------------------------------------
     def jumprelu(self, x: torch.Tensor, layer_idx: int) -> torch.Tensor:
+        if self._is_half():
+            return self._via_twin("jumprelu", x, layer_idx)
         return self.theta_manager.jumprelu(x, layer_idx)
 
     def get_preactivations(self, x: torch.Tensor, layer_idx: int) -> torch.Tensor:
-        self._sync_device()
+        if self._is_half():
+            return self._via_twin("get_preactivations", x, layer_idx)
         return self.encoder_module.get_preactivations(x, layer_idx)
 
     def _encode_all_layers(self, inputs: Dict[int, torch.Tensor]
@@ -125,11 +181,13 @@ class CrossLayerTranscoder(BaseTranscoder):
 
     def decode(self, a: Dict[int, torch.Tensor], layer_idx: int,
                source_inputs: Optional[Dict[int, torch.Tensor]] = None) -> torch.Tensor:
-        self._sync_device()
+        if self._is_half():
+            return self._via_twin("decode", a, layer_idx, source_inputs)
         return self.decoder_module.decode(a, layer_idx, source_inputs)
 
     def get_decoder_norms(self) -> torch.Tensor:
-        self._sync_device()
+        if self._is_half():
+            return self._via_twin("get_decoder_norms")
         return self.decoder_module.get_decoder_norms()
 
     @property
@@ -148,6 +206,7 @@ class CrossLayerTranscoder(BaseTranscoder):
                                device: Optional[torch.device] = None) -> torch.Tensor:
         """Estimate theta post-hoc using a specified number of batches (clt.py:282-307).  The
         estimation runs where the model lives; ``device`` is accepted for signature parity."""
+        self._no_half("estimate_theta_posthoc")
         if device is not None and torch.device(device) != self.theta_manager.device:
             logger.info(f"Rank {self.rank}: theta estimation stays on {self.theta_manager.device} (asked for {device}).")
         return self.theta_manager.estimate_theta_posthoc(
@@ -158,6 +217,7 @@ class CrossLayerTranscoder(BaseTranscoder):
     def convert_to_jumprelu_inplace(self, default_theta_value: float = 1e6) -> None:
         """BatchTopK / TokenTopK -> JumpReLU from the estimated statistics (clt.py:309-318); the
         ThetaManager updates the config object it shares with the model."""
+        self._no_half("convert_to_jumprelu_inplace")
         self.theta_manager.convert_to_jumprelu_inplace(default_theta_value=default_theta_value)
         logger.info(f"Rank {self.rank}: CLT model config updated by ThetaManager. New activation_fn='{self.config.activation_fn}'.")
 
@@ -292,6 +352,7 @@ class CrossLayerTranscoder(BaseTranscoder):
         Needs every layer present, equal token counts and a top-k or JumpReLU / ReLU activation; decoders
         untied or tied per source / per target, with or without skip connections and the per-target feature
         offset / scale (decoder.py:228-338)."""
+        self._no_half("loss_and_gradients")
         L = self.config.num_layers
         loss_l, raw = self._loss_and_raw_gradients(inputs, targets, normalization_method, mean_tg, std_tg)
         grads: Dict[str, Optional[torch.Tensor]] = {}
@@ -322,6 +383,7 @@ class CrossLayerTranscoder(BaseTranscoder):
         """One optimisation step on the MSE reconstruction loss (trainer.py:663-778 without the
         auxiliary losses): forward, gradients, ``optimizer.step``; returns the loss before the step.
         De-normalisation arguments as in ``loss_and_gradients``."""
+        self._no_half("training_step")
         fuse = optimizer if getattr(optimizer, "fuses_decoder_step", lambda: False)() else None
         loss_l, raw = self._loss_and_raw_gradients(inputs, targets, normalization_method, mean_tg, std_tg, decoder_step=fuse)
         optimizer.step(raw)
@@ -331,7 +393,8 @@ class CrossLayerTranscoder(BaseTranscoder):
     def encode(self, x: torch.Tensor, layer_idx: int) -> torch.Tensor:
         """Activations [tokens, F] of one layer for relu / jumprelu; for the top-k family the
         reference logs an error and returns zeros here (clt.py:135-149), and so does this."""
-        self._sync_device()
+        if self._is_half():
+            return self._via_twin("encode", x, layer_idx)
         x = x.to(device=self.device, dtype=self.dtype)
         preact = self.get_preactivations(x, layer_idx)
         F = self.config.num_features
@@ -502,7 +565,8 @@ class CrossLayerTranscoder(BaseTranscoder):
     # ---- get_feature_activations -------------------------------------------------------------
     def get_feature_activations(self, inputs: Dict[int, torch.Tensor]) -> Dict[int, torch.Tensor]:
         """Dense activations per layer (clt.py:220-277)."""
-        self._sync_device()
+        if self._is_half():
+            return self._via_twin("get_feature_activations", inputs)
         cfg = self.config
         topk_family = cfg.activation_fn in ("batchtopk", "topk")
         res = self._survivors(inputs)
@@ -555,7 +619,7 @@ class CrossLayerTranscoder(BaseTranscoder):
         """(reconstructions, survivor list over all num_layers) from one pass, or None when the inputs
         need the per-layer fallbacks.  The list is what get_feature_activations would densify; the
         evaluator and the dead-feature counters read it directly."""
-        self._sync_device()
+        self._no_half("forward_with_survivors")
         cfg = self.config
         L = cfg.num_layers
         res = self._survivors(inputs)
@@ -574,7 +638,8 @@ class CrossLayerTranscoder(BaseTranscoder):
 
     def forward(self, inputs: Dict[int, torch.Tensor]) -> Dict[int, torch.Tensor]:
         """Reconstruction of every layer present in ``inputs`` (clt.py:186-218)."""
-        self._sync_device()
+        if self._is_half():
+            return self._via_twin("forward", inputs)
         cfg = self.config
         L, d = cfg.num_layers, cfg.d_model
         res = self.forward_with_survivors(inputs)

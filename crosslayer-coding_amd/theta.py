@@ -56,7 +56,10 @@ class ThetaManager(nn.Module):
     def thresholds(self, dtype: torch.dtype) -> torch.Tensor:
         """exp(log_threshold) for all layers, rounded to ``dtype``: [L, F], contiguous."""
         assert self.log_threshold is not None
-        return torch.exp(self.log_threshold.detach()).to(dtype).contiguous()
+        th = torch.exp(self.log_threshold.detach())
+        if engine.emulated_dtype() is not None:        # a float16 model on the float32 kernels: theta as it would round
+            th = th.to(engine.emulated_dtype())
+        return th.to(dtype).contiguous()
 
     def jumprelu(self, x: torch.Tensor, layer_idx: int) -> torch.Tensor:
         if self.log_threshold is None:
@@ -65,7 +68,10 @@ class ThetaManager(nn.Module):
         if layer_idx >= self.log_threshold.shape[0]:
             logger.error(f"Rank {self.rank}: Invalid layer_idx {layer_idx} for log_threshold. Returning input.")
             return x.to(device=self.device, dtype=self.dtype)
-        theta = torch.exp(self.log_threshold[layer_idx]).to(device=self.device, dtype=self.dtype)
+        theta = torch.exp(self.log_threshold[layer_idx])
+        if engine.emulated_dtype() is not None:
+            theta = theta.to(engine.emulated_dtype())
+        theta = theta.to(device=self.device, dtype=self.dtype)
         return cast(torch.Tensor, JumpReLU.apply(x, theta, self.bandwidth))
 
     # ---- post-hoc estimation ----------------------------------------------------------------

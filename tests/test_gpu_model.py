@@ -103,6 +103,61 @@ def test_forward_matches_oracle(dev, wl):
                                                               sd[f"encoder_module.encoders.{l}.bias_param"])) <= TOL[dtype]
 
 
+HALF_CASES = [
+    BASE.scaled("half-topk", dtype="float16"),
+    BASE.scaled("half-global", dtype="float16", topk_mode="global"),
+    BASE.scaled("half-jump", dtype="float16", activation_fn="jumprelu", k=None),
+    BASE.scaled("half-per-target", dtype="float16", decoder_tying="per_target"),
+    BASE.scaled("half-fused-shape", dtype="float16", num_layers=3, d_model=128, num_features=512, tokens=256, k=12),
+]
+
+
+@pytest.mark.parametrize("wl", HALF_CASES, ids=lambda w: w.name)
+def test_float16_model_forward_matches_oracle(dev, wl):
+    # float16 parameters and outputs, computed on the float32 kernels with the dense products and thresholds
+    # rounded to float16 where the reference's tensors round; the oracle runs the reference's algorithm in
+    # float16 on the CPU
+    model, sd, x = build(wl, dev)
+    assert model.dtype == torch.float16 and all(v.dtype == torch.float16 for v in model.state_dict().values()
+                                                if v.is_floating_point())
+    inputs = {l: x[l].to(dev) for l in range(wl.num_layers)}
+    recs = model(inputs)
+    ref_recs, ref_acts = oracle_forward(wl, sd, x)
+    for t in recs:
+        assert recs[t].dtype == torch.float16 and recs[t].shape == ref_recs[t].shape
+        err = orc.rel_l2(recs[t], ref_recs[t])
+        assert err <= 5e-3, (t, err)
+    acts = model.get_feature_activations(inputs)
+    pre_cpu = {l: model.get_preactivations(inputs[l], l).cpu() for l in range(wl.num_layers)}
+    for l in acts:
+        assert acts[l].dtype == torch.float16 and pre_cpu[l].dtype == torch.float16
+        # pre-activations: the float32 sum rounded once to float16
+        want_pre = orc.encoder_preactivations(x[l], sd[f"encoder_module.encoders.{l}.weight"],
+                                              sd[f"encoder_module.encoders.{l}.bias_param"])
+        assert orc.rel_l2(pre_cpu[l], want_pre) <= 2e-3
+        if wl.activation_fn == "batchtopk" and wl.topk_mode == "per_layer":
+            assert torch.equal(acts[l].cpu(), orc.batchtopk_forward(pre_cpu[l], float(wl.k), pre_cpu[l]))
+        elif wl.activation_fn == "jumprelu":
+            lt = sd["theta_manager.log_threshold"]
+            assert torch.equal(acts[l].cpu(), orc.jumprelu_forward(pre_cpu[l], orc.theta_from_log(lt[l], torch.float16)))
+    norms = model.get_decoder_norms()
+    assert norms.dtype == torch.float16 and bool(torch.isfinite(norms).all())
+    # parameters changed in place are picked up by the next forward
+    with torch.no_grad():
+        model.decoder_module._ordered()[0].bias_param.add_(1.0)
+    recs2 = model(inputs)
+    assert not torch.equal(recs2[0], recs[0])
+    # module.half() on a float32 model takes the same route
+    wl32 = wl.scaled(wl.name + "-32", dtype="float32")
+    m32, _, _ = build(wl32, dev)
+    m32.half()
+    out = m32(inputs)
+    assert m32.dtype == torch.float16 and all(v.dtype == torch.float16 for v in out.values())
+    # what is not built for float16 says so
+    with pytest.raises(NotImplementedError):
+        model.loss_and_gradients(inputs, inputs)
+
+
 @pytest.mark.parametrize("fn", ["batchtopk", "jumprelu"])
 def test_fused_routes_equal_separate_kernels_in_the_model(dev, fn):
     # same model, same inputs: with and without the encoder-epilogue routes, all layers and a subset
