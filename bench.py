@@ -605,7 +605,22 @@ def run_backward(args):
     # per decoder element the fp32 gradient written once - or, with the step in place, both moments and the packed
     # copy read and written and the parameter rewritten from the copy
     hbm_bytes = pairs * F * d * ((16 + 4 * esz) if fused else 4) + L * wl.tokens * d * esz + surv.nnz * (8 + esz)
-    roofline = {"kernel": f"k_feature_outer ({dw_name}, {L} launches per step)",
+    tiled = fused and opt._dec_layout == "tiles"
+    if tiled:
+        # Column-tile route: the gather of the loss gradient is LDS traffic; through the HBM interface go both
+        # moments (read and written: 16 bytes per decoder element), the tiled weight copy (read and written) and
+        # the conversion that follows (tiles read, feature-major slab and checkpoint layout written): 5 elements.
+        hbm_bytes = pairs * F * d * (16 + 5 * esz) + L * wl.tokens * d * esz + surv.nnz * (8 + esz)
+        roofline = {"kernel": f"k_tile_outer_adam + k_tile_convert ({dw_name}, one launch each per step)",
+                    "bound": "hbm", "achieved": hbm_bytes / dw_sec / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": hbm_bytes / dw_sec / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                    "lds_gather_GBps": gathered / dw_sec / 1e9,
+                    "note": "achieved = compulsory HBM bytes of the stage (moments, tiled weights, converted layouts, "
+                            "loss gradient, lists) / the stage's time; the kernel itself is bound by vector-instruction "
+                            "issue (see the profile summary), not by this interface"}
+    else:
+        roofline = None
+    roofline = roofline or {"kernel": f"k_feature_outer ({dw_name}, {L} launches per step)",
                 "bound": "l2_gather (measured)", "achieved": gathered / dw_sec / 1e9, "peak": yard, "unit": "GB/s",
                 "frac": (gathered / dw_sec / 1e9 / yard) if yard else None, "traffic": None,
                 "hbm": {"compulsory_bytes": hbm_bytes, "compulsory_GBps": hbm_bytes / dw_sec / 1e9,

@@ -75,6 +75,12 @@ _SIGNATURES = {
     "clt_adam_step": (_int, [_vp, _vp, _vp, _vp, _i64, _f64, _f64, _f64, _f64, _i64, _int, _vp]),
     "clt_decoder_weight_grad_adam": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _f64, _f64, _f64, _f64, _i64, _int, _vp]),
     "clt_unpack_decoders": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
+    "clt_decoder_tile_width": (_int, [_i64, _i64, _i64, _int]),
+    "clt_decoder_tiles_workspace_bytes": (_sz, [_i64, _int]),
+    "clt_tile_decoders": (_int, [_vp, _vp, _i64, _i64, _i64, _int, _vp]),
+    "clt_untile_decoders": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
+    "clt_decoder_weight_grad_adam_tiled": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _f64, _f64, _f64,
+                                                  _f64, _i64, _int, _vp, _sz, _vp]),
     "clt_adam_step_decoder": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _f64, _f64, _f64, _f64, _i64, _int, _vp]),
     "clt_adam_step_decoders": (_int, [_vp, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _f64, _f64, _f64, _f64, _i64, _int, _vp]),
     "clt_adam_step_many": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _f64, _f64, _f64, _f64, _i64, _int, _vp]),

@@ -134,7 +134,13 @@ class Decoder(nn.Module):
             if self._slab_keys[i] != key:
                 engine.pack_decoder(w.detach().contiguous(), self._slab[i])
                 self._slab_keys[i] = key
+                self._repacks = getattr(self, "_repacks", 0) + 1
         return self._slab
+
+    def packed_generation(self):
+        """Changes whenever ``packed()`` has rebuilt any matrix from its parameter: other copies derived from the
+        slab (the optimiser's tiled weights) are stale then."""
+        return (None if self._slab is None else self._slab.data_ptr(), getattr(self, "_repacks", 0))
 
     def invalidate_packed(self) -> None:
         """Force a repack on next use (needed only after writes that bypass autograd

@@ -592,6 +592,70 @@ def unpack_decoders(w_packed: torch.Tensor, w_refs_dev: torch.Tensor, w_refs_hos
     nat.check(code, "clt_unpack_decoders")
 
 
+def decoder_tile_width(T: int, d: int, F: int, dtype: torch.dtype) -> int:
+    """Columns per tile of the tiled decoder layout [n_dec, d // CS, F, CS] when the column-tile weight-gradient
+    kernel takes this shape, else 0."""
+    return int(nat.load().clt_decoder_tile_width(int(T), int(d), int(F), nat.dtype_code(dtype)))
+
+
+def tile_decoders(w_packed: torch.Tensor, d: int, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Tiled copy [n_dec, d // CS, F, CS] of the feature-major slab [n_dec, F, pitch]."""
+    n_dec, F, _ = w_packed.shape
+    cs = 32 // w_packed.element_size()
+    assert d % cs == 0 and w_packed.is_contiguous()
+    if out is None:
+        out = torch.empty((n_dec, d // cs, F, cs), dtype=w_packed.dtype, device=w_packed.device)
+    assert out.is_contiguous() and tuple(out.shape) == (n_dec, d // cs, F, cs) and out.dtype == w_packed.dtype
+    code = nat.load().clt_tile_decoders(nat.ptr(w_packed), nat.ptr(out), n_dec, d, F, nat.dtype_code(w_packed.dtype),
+                                        _stream(w_packed))
+    nat.check(code, "clt_tile_decoders")
+    return out
+
+
+def untile_decoders(w_tiles: torch.Tensor, w_packed: torch.Tensor, w_refs_dev: Optional[torch.Tensor] = None,
+                    w_refs_host=None) -> None:
+    """The feature-major slab [n_dec, F, pitch] and (when their addresses are given, as for ``unpack_decoders``)
+    the checkpoint-layout parameters [d, F], rewritten from the tiled weights."""
+    import ctypes
+    n_dec, ns, F, cs = w_tiles.shape
+    d = ns * cs
+    assert w_tiles.is_contiguous() and w_packed.is_contiguous() and w_packed.dtype == w_tiles.dtype
+    assert tuple(w_packed.shape) == (n_dec, F, decoder_pitch(d, w_tiles.dtype))
+    assert (w_refs_dev is None) == (w_refs_host is None)
+    if w_refs_dev is not None:
+        assert w_refs_dev.dtype == torch.int64 and w_refs_dev.numel() == n_dec
+    code = nat.load().clt_untile_decoders(nat.ptr(w_tiles), nat.ptr(w_packed), nat.ptr(w_refs_dev),
+                                          ctypes.addressof(w_refs_host) if w_refs_host is not None else None, n_dec, d, F,
+                                          nat.dtype_code(w_tiles.dtype), _stream(w_tiles))
+    nat.check(code, "clt_untile_decoders")
+
+
+def decoder_weight_grad_adam_tiled(lists, surv: SurvivorList, g: torch.Tensor, w_tiles: torch.Tensor, m_tiles: torch.Tensor,
+                                   v_tiles: torch.Tensor, lr: float, betas, eps: float, step: int,
+                                   ws: Optional[Workspace] = None) -> None:
+    """``decoder_weight_grad_adam`` over column tiles: weights and moments [n_dec, d // CS, F, CS] are updated in
+    place (equal to the row route up to the fp32 association of some gradient sums, repeatable bit for bit);
+    ``untile_decoders`` brings the slab and the checkpoint-layout parameters up to date."""
+    assert g.dtype == surv.dtype and g.is_contiguous() and w_tiles.dtype == surv.dtype and w_tiles.is_contiguous()
+    ptr, tok, src = lists
+    L, T, F = surv.L, surv.T, surv.F
+    d = g.shape[2]
+    n_dec = L * (L + 1) // 2
+    cs = decoder_tile_width(T, d, F, surv.dtype)
+    assert cs > 0, "shape not taken by the column-tile kernel"
+    assert tuple(w_tiles.shape) == (n_dec, d // cs, F, cs)
+    assert m_tiles.shape == w_tiles.shape and v_tiles.shape == w_tiles.shape and m_tiles.dtype == torch.float32
+    assert v_tiles.dtype == torch.float32 and m_tiles.is_contiguous() and v_tiles.is_contiguous()
+    lib = nat.load()
+    cap = int(tok.numel())
+    wbuf = (ws or Workspace(g.device)).get("decoder_tiles", lib.clt_decoder_tiles_workspace_bytes(cap, nat.dtype_code(surv.dtype)))
+    code = lib.clt_decoder_weight_grad_adam_tiled(nat.ptr(ptr), nat.ptr(tok), nat.ptr(src), nat.ptr(surv.val), nat.ptr(g),
+                                                  nat.ptr(w_tiles), nat.ptr(m_tiles), nat.ptr(v_tiles), T, d, F, L, cap, lr,
+                                                  betas[0], betas[1], eps, step, nat.dtype_code(surv.dtype), nat.ptr(wbuf),
+                                                  wbuf.numel(), _stream(g))
+    nat.check(code, "clt_decoder_weight_grad_adam_tiled")
+
+
 def encoder_weight_grad(lists, dval: torch.Tensor, x: torch.Tensor, F: int):
     """(fp32 [L, F, d], fp32 [L, F]): gradients of the stacked encoder weights and biases."""
     ptr, tok, src = lists

@@ -24,6 +24,10 @@ class CLTAdam:
         self.lr, self.betas, self.eps = float(lr), (float(betas[0]), float(betas[1])), float(eps)
         self.step_count = 0
         self.fuse_decoder_step = True    # untied decoders: Adam inside the weight-gradient kernel (training_step)
+        self.tile_decoder_step = True    # ... over column tiles, when the shape allows (moments and a weight copy tiled)
+        self._dec_layout = "rows"        # layout of state["dec_w"]: "rows" [n_dec, F, d] or "tiles" [n_dec, d // CS, F, CS]
+        self._w_tiles = None             # tiled copy of the decoder weights, valid while _w_tiles_gen matches the slab
+        self._w_tiles_gen = None
         cfg = model.config
         L, F, d = cfg.num_layers, cfg.num_features, cfg.d_model
         dev = model.device
@@ -69,21 +73,65 @@ class CLTAdam:
         return (self.fuse_decoder_step and self.model.config.decoder_tying == "none"
                 and dec.feature_offset is None and dec.feature_scale is None)
 
+    def _decoder_moments_to(self, layout: str) -> None:
+        """Regroup both decoder moments: "rows" [n_dec, F, d] <-> "tiles" [n_dec, d // CS, F, CS] (CS = 32 bytes of
+        the model dtype).  Happens when the route of the decoder step changes, normally once."""
+        if layout == self._dec_layout:
+            return
+        cfg = self.model.config
+        F, d = cfg.num_features, cfg.d_model
+        cs = 32 // self.model.decoder_module._ordered()[0].weight.element_size()
+        out = []
+        for t in self.state["dec_w"]:
+            n_dec = t.shape[0]
+            if layout == "tiles":
+                out.append(t.view(n_dec, F, d // cs, cs).permute(0, 2, 1, 3).contiguous())
+            else:
+                out.append(t.permute(0, 2, 1, 3).contiguous().view(n_dec, F, d))
+            del t
+        self.state["dec_w"] = tuple(out)
+        self._dec_layout = layout
+
+    def decoder_moments(self):
+        """(m, v) of the decoder weights as [n_dec, F, d] whatever layout the optimiser keeps them in."""
+        m, v = self.state["dec_w"]
+        if self._dec_layout == "rows":
+            return m, v
+        n_dec, ns, F, cs = m.shape
+        return tuple(t.permute(0, 2, 1, 3).contiguous().view(n_dec, F, ns * cs) for t in (m, v))
+
     @torch.no_grad()
     def decoder_weight_step(self, lists, surv, g_model) -> None:
         """The decoder weights' part of the NEXT ``step`` (which must follow with ``raw["dec_w"] = None``), taken
         straight from the survivor lists: gradient rows go from registers into the update of the moments and
-        of the packed copy; the checkpoint-layout parameters are then rewritten from the packed copy."""
+        of the working copy of the weights; the checkpoint-layout parameters are then rewritten from that copy.
+        Two routes: over column tiles (tiled moments and a tiled weight copy, the gather of d loss /
+        d reconstruction served from LDS) when ``engine.decoder_tile_width`` takes the shape, else row by row on
+        the feature-major slab.  The row route is bit-identical to gradient-then-Adam; the tile route sums the
+        lists it cuts between lanes in another fixed association (equal to fp32 rounding, repeatable)."""
         from . import engine
         dec = self.model.decoder_module
         packed = dec.packed()
         ws = [lin.weight.data for lin in dec._ordered()]
         assert all(w.is_contiguous() and w.shape == ws[0].shape and w.dtype == ws[0].dtype for w in ws)
         d, F = ws[0].shape
+        w_dev, w_host = self._pointer_table("w", ws)
+        cs = engine.decoder_tile_width(surv.T, d, F, ws[0].dtype) if self.tile_decoder_step else 0
+        if cs and all(w.data_ptr() % 16 == 0 for w in ws):
+            self._decoder_moments_to("tiles")
+            if self._w_tiles is None or self._w_tiles_gen != dec.packed_generation():
+                self._w_tiles = engine.tile_decoders(packed, d, out=self._w_tiles)
+                self._w_tiles_gen = dec.packed_generation()
+            m_w, v_w = self.state["dec_w"]
+            engine.decoder_weight_grad_adam_tiled(lists, surv, g_model, self._w_tiles, m_w, v_w, self.lr, self.betas,
+                                                  self.eps, self.step_count + 1, ws=self.model._workspace())
+            engine.untile_decoders(self._w_tiles, packed, w_dev, w_host)
+            return
+        self._decoder_moments_to("rows")
+        self._w_tiles_gen = None
         m_w, v_w = self.state["dec_w"]
         engine.decoder_weight_grad_adam(lists, surv, g_model, packed, m_w, v_w, self.lr, self.betas, self.eps,
                                         self.step_count + 1)
-        w_dev, w_host = self._pointer_table("w", ws)
         engine.unpack_decoders(packed, w_dev, w_host, d, F)
 
     @torch.no_grad()
@@ -109,6 +157,9 @@ class CLTAdam:
         assert all(b.is_contiguous() and b.numel() == bs[0].numel() and b.dtype == bs[0].dtype for b in bs)
         d, F = ws[0].shape
         if raw["dec_w"] is not None:
+            self._decoder_moments_to("rows")
+            self._w_tiles_gen = None      # the slab is about to change under the tiled copy
+            m_w, v_w = self.state["dec_w"]
             assert packed.is_contiguous() and raw["dec_w"].is_contiguous() and raw["dec_w"].dtype == torch.float32
             from . import engine
             assert tuple(raw["dec_w"].shape) == (len(ws), F, d)

@@ -520,6 +520,39 @@ int clt_decoder_weight_grad_adam(const int32_t *list_ptr, const int32_t *list_to
                                  int dtype, void *stream);
 int clt_unpack_decoders(const void *w_packed, void *const *w_refs_dev, void *const *w_refs_host,
                         int64_t n_dec, int64_t d, int64_t F, int dtype, void *stream);
+/*
+ * The same step over COLUMN TILES (same reference lines; the gradient sums of lists that the kernel
+ * cuts between two lane pairs are associated differently, so results agree with the call above to
+ * fp32 rounding of the gradient and repeat bit for bit from run to run).
+ * clt_decoder_weight_grad_adam gathers one row of d loss / d reconstruction per list entry through
+ * the L2; here a workgroup parks one 32-byte column slice of one target's g_model [T][d] in its LDS
+ * and runs over every (source <= target, feature) row of that slice, so that only the lists, the
+ * moments and the parameters pass through the vector memory path.  For that the decoder weights and
+ * both moments are kept tiled,
+ *     [n_dec][d / CS][F][CS],   CS = clt_decoder_tile_width(...) = 16 bf16 / 8 fp32 columns,
+ * so that one slice of consecutive features is contiguous.  clt_decoder_tile_width returns 0 when
+ * the shape cannot take this route (d % CS != 0, F % 4 != 0, or T * 32 bytes beyond the LDS of a
+ * compute unit, T <= 4350): callers then use clt_decoder_weight_grad_adam with feature-major moments.
+ * clt_tile_decoders fills the tiled weights from the feature-major slab [n_dec][F][pitch];
+ * clt_untile_decoders writes the slab back from the tiles and, when w_refs_dev / w_refs_host (both
+ * or neither) are given, the checkpoint-layout parameters [d][F] too.
+ * workspace: clt_decoder_tiles_workspace_bytes(capacity of the lists, dtype) bytes, 256-byte
+ * aligned (the list entries regrouped as token|coefficient pairs, and a work counter).
+ */
+int clt_decoder_tile_width(int64_t T, int64_t d, int64_t F, int dtype);
+size_t clt_decoder_tiles_workspace_bytes(int64_t capacity, int dtype);
+int clt_tile_decoders(const void *w_packed, void *w_tiles, int64_t n_dec, int64_t d, int64_t F,
+                      int dtype, void *stream);
+int clt_untile_decoders(const void *w_tiles, void *w_packed, void *const *w_refs_dev,
+                        void *const *w_refs_host, int64_t n_dec, int64_t d, int64_t F, int dtype,
+                        void *stream);
+int clt_decoder_weight_grad_adam_tiled(const int32_t *list_ptr, const int32_t *list_tok,
+                                       const int32_t *list_src, const void *val, const void *g_model,
+                                       void *w_tiles, float *m_tiles, float *v_tiles,
+                                       int64_t T, int64_t d, int64_t F, int64_t L, int64_t capacity,
+                                       double lr, double beta1, double beta2, double eps,
+                                       int64_t step, int dtype, void *workspace,
+                                       size_t workspace_bytes, void *stream);
 int clt_adam_step_decoder(void *w_ref, void *w_packed, const float *grad_packed, float *m, float *v,
                           int64_t d, int64_t F, double lr, double beta1, double beta2, double eps,
                           int64_t step, int dtype, void *stream);

@@ -144,36 +144,133 @@ def test_long_feature_lists_are_in_token_order_and_gradients_repeat_bit_for_bit(
         assert torch.equal(g1[k], g2[k]), k
 
 
-@pytest.mark.parametrize("dtype,d_model,fn", [("bfloat16", 128, "batchtopk"), ("bfloat16", 768, "batchtopk"),
-                                              ("float32", 64, "batchtopk"), ("bfloat16", 128, "jumprelu")])
-def test_adam_inside_the_weight_gradient_kernel_equals_the_two_step_sequence(dev, dtype, d_model, fn):
+def _assert_same_training(a, b, dtype, steps):
+    """(losses, state dict, packed slab, moments) of two runs that differ only in the association of some fp32
+    sums of the decoder weight gradient.  After ONE step from the same state everything agrees to rounding; later
+    steps start from states that differ in last places, where an element at the selection threshold or a
+    gradient near zero can move a parameter by a whole Adam step, so then nearly all elements must agree."""
+    ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -20
+    # (even after one step: where a gradient sum cancels to nearly nothing, below Adam's eps, its last places
+    # decide the step; fp32 parameters show that, bf16 ones round it away.  The moments below are the strict check.)
+    allowed = (1e-4 if dtype == torch.bfloat16 else 2e-2) if steps == 1 else 2e-2
+
+    def close(x, y, what):
+        # one unit in the last place of the larger of the value and the size of an Adam step (lr 1e-2 here)
+        x, y = x.float(), y.float()
+        bad = (x - y).abs() > ulp * torch.maximum(x.abs(), y.abs()).clamp_min(0.05)
+        assert float(bad.float().mean()) <= allowed, what
+        if dtype == torch.bfloat16:
+            assert float((x != y).float().mean()) <= 2e-3 * steps, what
+    if a[0] is not None:
+        assert a[0] == pytest.approx(b[0], rel=1e-3)
+    for k, v in a[1].items():
+        close(v, b[1][k], k)
+    if a[2] is not None:
+        close(a[2], b[2], "slab")
+    for x, y in zip(a[3], b[3]):
+        # moments: rounding of the gradient sums, measured against the size of the terms
+        assert float((x - y).abs().max()) <= (1e-5 if steps == 1 else 1e-2) * float(x.abs().max())
+
+
+@pytest.mark.parametrize("dtype,d_model,fn,tokens", [
+    ("bfloat16", 128, "batchtopk", 256), ("bfloat16", 768, "batchtopk", 256), ("float32", 64, "batchtopk", 256),
+    ("bfloat16", 128, "jumprelu", 256),
+    ("bfloat16", 136, "batchtopk", 256),    # d not a multiple of the tile width: the tile route declines
+    ("bfloat16", 80, "batchtopk", 300),     # d a multiple of the tile width, not of the 64-column conversion block
+    ("float32", 72, "batchtopk", 4100)])    # the slice of one target fills nearly all the LDS it may take
+def test_adam_inside_the_weight_gradient_kernel_equals_the_two_step_sequence(dev, dtype, d_model, fn, tokens):
     # untied decoders: training_step lets the decoder weights take their Adam step inside the weight-gradient
-    # kernel (no fp32 gradient in memory, parameters rewritten from the packed copy); three steps must leave
-    # every parameter, the packed copy and both moments bit-identical to gradient-then-Adam
+    # kernel (no fp32 gradient in memory, parameters rewritten from the working copy), over column tiles where
+    # the shape allows and row by row otherwise; three steps must leave every parameter, the packed copy and
+    # both moments bit-identical to gradient-then-Adam
     import crosslayer_coding_amd as cca
-    wl = BASE.scaled("bw-fuse", num_layers=3, d_model=d_model, num_features=256, tokens=256, dtype=dtype,
+    wl = BASE.scaled("bw-fuse", num_layers=3, d_model=d_model, num_features=256, tokens=tokens, dtype=dtype,
                      activation_fn=fn, k=10 if fn == "batchtopk" else None)
-    runs = []
-    for fuse in (True, False):
+    runs, first = [], []
+    for fuse, tiles in ((True, True), (True, False), (False, False)):
         model, sd, x, targets = build(wl, dev)
         opt = cca.CLTAdam(model, lr=1e-2)
         opt.fuse_decoder_step = fuse
+        opt.tile_decoder_step = tiles
         assert opt.fuses_decoder_step() == fuse
         inputs = {l: x[l].to(dev) for l in range(3)}
         tg = {l: t.to(dev) for l, t in targets.items()}
-        losses = [float(model.training_step(inputs, tg, opt)) for _ in range(3)]
-        runs.append((losses, {k: v.detach().clone() for k, v in model.state_dict().items()},
-                     model.decoder_module.packed().clone(), [t.clone() for t in opt.state["dec_w"]]))
-    assert runs[0][0] == runs[1][0]
-    for k, v in runs[0][1].items():
-        assert torch.equal(v, runs[1][1][k]), k
-    assert torch.equal(runs[0][2], runs[1][2])
-    for a, b in zip(runs[0][3], runs[1][3]):
+        def snapshot(losses):
+            return (list(losses), {k: v.detach().clone() for k, v in model.state_dict().items()},
+                    model.decoder_module.packed().clone(), [t.clone() for t in opt.decoder_moments()])
+        losses = [float(model.training_step(inputs, tg, opt))]
+        first.append(snapshot(losses))
+        losses += [float(model.training_step(inputs, tg, opt)) for _ in range(2)]
+        if fuse:
+            took = engine.decoder_tile_width(tokens, d_model, 256, getattr(torch, dtype)) > 0
+            assert (opt._dec_layout == "tiles") == (tiles and took)
+            assert took == (d_model != 136)
+        runs.append(snapshot(losses))
+    # row by row inside the kernel == gradient-then-Adam, bit for bit
+    assert runs[1][0] == runs[2][0]
+    for k, v in runs[1][1].items():
+        assert torch.equal(v, runs[2][1][k]), k
+    assert torch.equal(runs[1][2], runs[2][2])
+    for a, b in zip(runs[1][3], runs[2][3]):
         assert torch.equal(a, b)
+    # over column tiles: a list cut between two lane pairs is summed in another association, so the gradient
+    # agrees to fp32 rounding; parameters may differ where that moves a rounding decision
+    _assert_same_training(first[0], first[1], getattr(torch, dtype), 1)
+    _assert_same_training(runs[0], runs[1], getattr(torch, dtype), 3)
     # the parameters are what the packed copy holds
     model_keys = [k for k in runs[0][1] if k.startswith("decoder_module.decoders.") and k.endswith(".weight")]
     for i, k in enumerate(sorted(model_keys, key=lambda n: [int(p) for p in n.split(".")[2].split("->")])):
         assert torch.equal(runs[0][1][k].t(), runs[0][2][i][:, :d_model]), k
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_tiled_decoder_layout_round_trip(dev, dtype):
+    # slab -> tiles -> slab + checkpoint layout, on a shape with ragged 64 x 64 conversion blocks
+    import ctypes
+    n_dec, F, d = 3, 200, 80 if dtype == torch.bfloat16 else 72
+    g = torch.Generator().manual_seed(3)
+    slab = engine.alloc_packed(n_dec, F, d, dtype, dev)
+    w = torch.randn(n_dec, F, d, generator=g).to(dtype).to(dev)
+    slab[:, :, :d] = w
+    tiles = engine.tile_decoders(slab, d)
+    cs = 32 // slab.element_size()
+    assert tuple(tiles.shape) == (n_dec, d // cs, F, cs)
+    assert torch.equal(tiles.permute(0, 2, 1, 3).reshape(n_dec, F, d), w)
+    slab2 = engine.alloc_packed(n_dec, F, d, dtype, dev)
+    refs = [torch.zeros(d, F, dtype=dtype, device=dev) for _ in range(n_dec)]
+    host = (ctypes.c_void_p * n_dec)(*[r.data_ptr() for r in refs])
+    table = torch.tensor([r.data_ptr() for r in refs], dtype=torch.int64, device=dev)
+    engine.untile_decoders(tiles, slab2, table, host)
+    assert torch.equal(slab2[:, :, :d], w) and not bool(slab2[:, :, d:].any())
+    for i in range(n_dec):
+        assert torch.equal(refs[i], w[i].t())
+    slab3 = engine.alloc_packed(n_dec, F, d, dtype, dev)
+    engine.untile_decoders(tiles, slab3)
+    assert torch.equal(slab3, slab2)
+
+
+def test_optimiser_moves_between_the_tiled_and_the_row_route(dev):
+    # one optimiser, steps taken in turn through the tiled kernel, the row kernel and gradient-then-Adam: the
+    # moments change layout under way and the tiled weight copy is rebuilt when the slab changed behind it;
+    # the result must be the one of three plain steps
+    import crosslayer_coding_amd as cca
+    wl = BASE.scaled("bw-mixed", num_layers=3, d_model=128, num_features=256, tokens=256, dtype="bfloat16", k=10)
+    runs = []
+    for mixed in (True, False):
+        model, sd, x, targets = build(wl, dev)
+        opt = cca.CLTAdam(model, lr=1e-2)
+        inputs = {l: x[l].to(dev) for l in range(3)}
+        tg = {l: t.to(dev) for l, t in targets.items()}
+        for step in range(4):
+            if mixed:
+                opt.fuse_decoder_step = step != 2
+                opt.tile_decoder_step = step != 1
+            else:
+                opt.fuse_decoder_step = False
+            model.training_step(inputs, tg, opt)
+        runs.append(({k: v.detach().clone() for k, v in model.state_dict().items()},
+                     [t.clone() for t in opt.decoder_moments()]))
+    _assert_same_training((None, runs[0][0], None, runs[0][1]), (None, runs[1][0], None, runs[1][1]), torch.bfloat16, 4)
 
 
 def test_tied_decoders_do_not_fuse_the_step(dev):
