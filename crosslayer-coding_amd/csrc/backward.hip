@@ -620,6 +620,137 @@ __global__ __launch_bounds__(BW_THREADS) void k_csc_order(const int32_t *ptr, in
   }
 }
 
+// ---- the same lists without device-scope atomics and without the sort -----------------------------------
+// The tokens of a layer are cut into NB blocks; workgroup (layer, block) keeps one counter per feature in LDS.
+//   k_fl_count: histogram of the block's entries (LDS atomics: only counts, the order does not matter);
+//   k_fl_total: list length = sum over the blocks (the counts become running sums over the blocks), then the
+//               chunked scan above gives list_ptr;
+//   k_fl_fill:  LDS counter f starts where the block's part of list (layer, f) starts (list_ptr plus the entries
+//               in earlier blocks) and the block's tokens are taken ONE AFTER THE OTHER: the columns of a
+//               row are distinct, so within one token no two threads touch the same counter and a plain read /
+//               increment gives every entry its place -- in token order by construction.
+// Needs F counters of LDS (F <= 35 K); longer feature axes take the atomic route above.
+constexpr int FL_THREADS = 512, FL_MAX_BLOCKS = 64, FL_MIN_BLOCK_TOKENS = 64, FL_MIN_CAP = 1024, FL_MAX_CAP = 16384;
+constexpr int64_t FL_LDS_MAX = 150 * 1024;
+__global__ __launch_bounds__(FL_THREADS) void k_fl_count(const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ col,
+                                                          int64_t Tn, int64_t F, int TB, int NB, uint16_t *__restrict__ counts,
+                                                          int64_t n) {
+  extern __shared__ uint32_t fl_lds[];
+  const int64_t l = blockIdx.x / NB, b = blockIdx.x % NB;
+  for (int64_t f = threadIdx.x; f < F; f += FL_THREADS) fl_lds[f] = 0u;
+  __syncthreads();
+  const int64_t t0 = b * TB, t1 = t0 + TB < Tn ? t0 + TB : Tn;
+  if (t0 < t1) {
+    const int32_t e0 = row_ptr[l * Tn + t0], e1 = row_ptr[l * Tn + t1];
+    for (int32_t j0 = e0 + (int32_t)threadIdx.x; j0 < e1; j0 += 8 * FL_THREADS) {
+      int32_t c[8];       // eight loads in flight per thread
+#pragma unroll
+      for (int u = 0; u < 8; ++u) c[u] = j0 + u * FL_THREADS < e1 ? col[j0 + u * FL_THREADS] : -1;
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (c[u] >= 0) atomicAdd(&fl_lds[c[u]], 1u);
+    }
+  }
+  __syncthreads();
+  uint16_t *out = counts + b * n + l * F;
+  for (int64_t f = threadIdx.x; f < F; f += FL_THREADS) out[f] = (uint16_t)fl_lds[f];    // <= TB <= 1024
+}
+// counts[b][q] -> number of entries of list q in the blocks before b (at most T <= 65535), cnt[q] = list length
+__global__ __launch_bounds__(BW_THREADS) void k_fl_total(uint16_t *counts, int NB, int64_t n, uint32_t *__restrict__ cnt) {
+  for (int64_t q = (int64_t)blockIdx.x * BW_THREADS + threadIdx.x; q < n; q += (int64_t)gridDim.x * BW_THREADS) {
+    uint32_t a = 0;
+    for (int b0 = 0; b0 < NB; b0 += 16) {
+      uint16_t c[16];       // sixteen independent loads, then the stores over them
+#pragma unroll
+      for (int u = 0; u < 16; ++u) c[u] = b0 + u < NB ? counts[(int64_t)(b0 + u) * n + q] : (uint16_t)0;
+#pragma unroll
+      for (int u = 0; u < 16; ++u)
+        if (b0 + u < NB) { counts[(int64_t)(b0 + u) * n + q] = (uint16_t)a; a += c[u]; }
+    }
+    cnt[q] = a;
+  }
+}
+__global__ __launch_bounds__(FL_THREADS) void k_fl_fill(const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ col,
+                                                         int64_t Tn, int64_t F, int TB, int NB,
+                                                         const uint16_t *__restrict__ counts, int64_t n,
+                                                         const int32_t *__restrict__ ptr, int32_t *__restrict__ tok_out,
+                                                         int32_t *__restrict__ src_out, int cap) {
+  extern __shared__ uint32_t fl_lds[];
+  uint32_t *pos = fl_lds;
+  uint32_t *buf = fl_lds + F;                               // cap staged entries: column index, then place
+  uint16_t *tk = reinterpret_cast<uint16_t *>(buf + cap);   // their tokens, counted from the batch's first
+  int32_t *rp = reinterpret_cast<int32_t *>(buf + cap + cap / 2);   // the block's row pointers, TB + 1 of them
+  const int64_t l = blockIdx.x / NB, b = blockIdx.x % NB;
+  const int64_t t0 = b * TB, t1 = t0 + TB < Tn ? t0 + TB : Tn;
+  if (t0 >= t1) return;
+  const int ntok = (int)(t1 - t0), tid = (int)threadIdx.x;
+  for (int64_t f0 = tid; f0 < F; f0 += 8 * FL_THREADS) {
+    uint32_t base[8];     // start of the list + its entries in earlier blocks; eight pairs of loads in flight
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int64_t f = f0 + u * FL_THREADS, q = l * F + f;
+      base[u] = f < F ? (uint32_t)ptr[q] + counts[b * n + q] : 0u;
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (f0 + u * FL_THREADS < F) pos[f0 + u * FL_THREADS] = base[u];
+  }
+  for (int i = tid; i <= ntok; i += FL_THREADS) rp[i] = row_ptr[l * Tn + t0 + i];
+  __syncthreads();
+  // Batches of whole tokens whose entries fit the staging buffer (a row longer than the buffer goes in pieces).
+  //   A: the batch's column indices come into LDS (one wait for memory per batch);
+  //   B: token after token, every entry swaps its column index for its place in the output -- LDS traffic
+  //      only, with a barrier that waits for LDS alone between two tokens;
+  //   C: the entries are scattered to their places (no order to keep any more).
+  auto lds_barrier = [] {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0xC07F);      // lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+  };
+  int tb = 0;
+  while (tb < ntok) {
+    const int32_t eb = rp[tb];
+    int te = tb + 1;
+    while (te < ntok && rp[te + 1] - eb <= cap) ++te;
+    int32_t ee = rp[te];
+    const bool cut = ee - eb > cap;      // one row longer than the buffer: its first cap entries now
+    if (cut) ee = eb + cap;
+    const int nb_e = ee - eb;
+    for (int i0 = tid; i0 < nb_e; i0 += 8 * FL_THREADS) {
+      uint32_t c[8];      // eight loads in flight per thread
+#pragma unroll
+      for (int u = 0; u < 8; ++u) c[u] = i0 + u * FL_THREADS < nb_e ? (uint32_t)col[eb + i0 + u * FL_THREADS] : 0u;
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (i0 + u * FL_THREADS < nb_e) buf[i0 + u * FL_THREADS] = c[u];
+    }
+    __syncthreads();
+    for (int t = tb; t < te; ++t) {
+      const int a0 = rp[t] - eb, a1 = (rp[t + 1] < ee ? rp[t + 1] : ee) - eb;
+      for (int i = a0 + tid; i < a1; i += FL_THREADS) {
+        const uint32_t f = buf[i], p = pos[f];
+        pos[f] = p + 1u;
+        buf[i] = p;
+        tk[i] = (uint16_t)(t - tb);
+      }
+      lds_barrier();      // the next token may meet the same features
+    }
+    for (int i = tid; i < nb_e; i += FL_THREADS) {
+      const uint32_t p = buf[i];
+      tok_out[p] = (int32_t)(t0 + tb + tk[i]);
+      src_out[p] = eb + i;
+    }
+    __syncthreads();      // buf, tk and rp[tb] are free again
+    if (cut) {
+      if (tid == 0) rp[tb] = ee;
+      __syncthreads();
+    } else {
+      tb = te;
+    }
+  }
+}
+
 // ---- weight gradients: one wavefront per output row ---------------------------------------------------
 // out_row[:] = sum over the list of (layer, feature) of coef[entry] * src[token][:]
 //   DECODER: wavefront (s, f, t >= s): coef = survivor value, src = g[t] (model dtype copy),
@@ -978,10 +1109,26 @@ extern "C" int clt_skip_weight_grad(const float *g, const void *x, float *out, i
   return clt_check_launch();
 }
 
+// More than 64 KB of dynamic LDS has to be granted per kernel; false when the device does not have it.
+static bool fl_lds_granted(size_t bytes) {
+  if (bytes <= 64 * 1024) return true;
+  int dev = 0, lds_max = 0;
+  if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&lds_max, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess ||
+      (size_t)lds_max < bytes ||
+      hipFuncSetAttribute((const void *)k_fl_count, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) != hipSuccess ||
+      hipFuncSetAttribute((const void *)k_fl_fill, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  return true;
+}
+
 extern "C" size_t clt_feature_lists_workspace_bytes(int64_t F, int64_t L) {
   if (F <= 0 || L <= 0) return 256;
   const size_t n = (size_t)L * (size_t)F;
-  return ((n * 4 + 255) & ~(size_t)255) + ((n + CSC_CHUNK - 1) / CSC_CHUNK) * 8;   // counters + chunk sums
+  // counters + chunk sums + the per-block counts of the blocked route
+  return ((n * 4 + 255) & ~(size_t)255) + ((((n + CSC_CHUNK - 1) / CSC_CHUNK) * 8 + 255) & ~(size_t)255) +
+         n * FL_MAX_BLOCKS * sizeof(uint16_t);
 }
 
 extern "C" int clt_feature_lists(const int32_t *row_ptr, const int32_t *col, int64_t T, int64_t F, int64_t L,
@@ -996,10 +1143,37 @@ extern "C" int clt_feature_lists(const int32_t *row_ptr, const int32_t *col, int
   uint32_t *cnt = (uint32_t *)workspace;
   const int64_t n = L * F;
   const unsigned nb = 256 * 8;
-  k_zero_u32<<<nb, BW_THREADS, 0, s>>>(cnt, n);
-  k_csc_count<<<nb, BW_THREADS, 0, s>>>(row_ptr, col, T, F, L, cnt);
   const int64_t nchunk = clt_ceil_div(n, CSC_CHUNK);
   unsigned long long *sums = (unsigned long long *)((char *)workspace + (((size_t)n * 4 + 255) & ~(size_t)255));
+  // blocked route: F counters in LDS, lists in token order by construction
+  // one workgroup per (layer, block of tokens) and per CU (the counters fill its LDS): as many blocks as
+  // give every CU one workgroup, at least FL_MIN_BLOCK_TOKENS tokens each
+  int cus = 0, dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) {
+    (void)hipGetLastError();
+    cus = 256;
+  }
+  int64_t NB64 = cus / L > 0 ? cus / L : 1;
+  if (NB64 > clt_ceil_div(T, FL_MIN_BLOCK_TOKENS)) NB64 = clt_ceil_div(T, FL_MIN_BLOCK_TOKENS);
+  if (NB64 > FL_MAX_BLOCKS) NB64 = FL_MAX_BLOCKS;
+  if (clt_ceil_div(T, NB64) > 1024) NB64 = clt_ceil_div(T, 1024);     // the staged token offsets and the counts are 16-bit
+  const int NB = (int)NB64, TB = (int)clt_ceil_div(T, NB);
+  // the staging buffer takes what the counters leave (6 bytes per entry)
+  int64_t cap = ((int64_t)FL_LDS_MAX - ((int64_t)F + TB + 1) * 4) / 6;
+  cap = cap > FL_MAX_CAP ? FL_MAX_CAP : cap & ~(int64_t)511;
+  const size_t fl_lds = ((size_t)F + (size_t)(cap > 0 ? cap : 0) * 3 / 2 + (size_t)TB + 1) * 4;
+  if (list_tok && list_src && NB <= FL_MAX_BLOCKS && cap >= FL_MIN_CAP && L * NB < 2147483647LL && fl_lds_granted(fl_lds)) {
+    uint16_t *counts = (uint16_t *)((char *)sums + ((((size_t)nchunk * 8) + 255) & ~(size_t)255));
+    k_fl_count<<<(unsigned)(L * NB), FL_THREADS, (size_t)F * 4, s>>>(row_ptr, col, T, F, TB, NB, counts, n);
+    k_fl_total<<<nb, BW_THREADS, 0, s>>>(counts, NB, n, cnt);
+    k_csc_chunk_sum<<<(unsigned)nchunk, BW_THREADS, 0, s>>>(cnt, n, sums);
+    k_csc_chunk_offsets<<<1, BW_THREADS, 0, s>>>(sums, nchunk, list_ptr, n);
+    k_csc_chunk_scan<<<(unsigned)nchunk, BW_THREADS, 0, s>>>(cnt, n, sums, list_ptr);
+    k_fl_fill<<<(unsigned)(L * NB), FL_THREADS, fl_lds, s>>>(row_ptr, col, T, F, TB, NB, counts, n, list_ptr, list_tok, list_src, (int)cap);
+    return clt_check_launch();
+  }
+  k_zero_u32<<<nb, BW_THREADS, 0, s>>>(cnt, n);
+  k_csc_count<<<nb, BW_THREADS, 0, s>>>(row_ptr, col, T, F, L, cnt);
   k_csc_chunk_sum<<<(unsigned)nchunk, BW_THREADS, 0, s>>>(cnt, n, sums);
   k_csc_chunk_offsets<<<1, BW_THREADS, 0, s>>>(sums, nchunk, list_ptr, n);
   k_csc_chunk_scan<<<(unsigned)nchunk, BW_THREADS, 0, s>>>(cnt, n, sums, list_ptr);

@@ -90,11 +90,16 @@ def test_loss_and_gradients_match_autograd(dev, wl):
         assert err <= bound, (name, err)
 
 
-def test_feature_lists_are_a_permutation_grouped_by_feature(dev):
+@pytest.mark.parametrize("T,F,k", [(300, 128, 9), (4100, 96, 9), (70, 40960, 9), (40, 2048, 800)],
+                         ids=["blocks-of-tokens", "ragged-last-block", "feature-axis-beyond-lds", "rows-longer-than-a-workgroup"])
+def test_feature_lists_are_a_permutation_grouped_by_feature(dev, T, F, k):
+    # the blocked construction (counters of a token block in LDS, token order by construction; 4100 tokens = 33
+    # blocks, the last one ragged; rows of ~800 survivors against 512 threads), and for a feature axis whose
+    # counters do not fit the LDS the atomic construction followed by the sort
     g = torch.Generator().manual_seed(2)
-    L, T, F = 2, 300, 128
+    L = 2
     pre = torch.randn(L, T, F, generator=g).to(dev)
-    surv = engine.batchtopk_select(pre, 9, False)
+    surv = engine.batchtopk_select(pre, k, False)
     ptr, tok, src = engine.feature_lists(surv)
     ptr, tok, src = ptr.cpu().long(), tok.cpu().long(), src.cpu().long()
     assert ptr[0] == 0 and ptr[-1] == surv.nnz and bool((ptr[1:] >= ptr[:-1]).all())
