@@ -182,7 +182,8 @@ def _assert_same_training(a, b, dtype, steps):
     ("bfloat16", 128, "jumprelu", 256),
     ("bfloat16", 136, "batchtopk", 256),    # d not a multiple of the tile width: the tile route declines
     ("bfloat16", 80, "batchtopk", 300),     # d a multiple of the tile width, not of the 64-column conversion block
-    ("float32", 72, "batchtopk", 4100)])    # the slice of one target fills nearly all the LDS it may take
+    ("float32", 72, "batchtopk", 4100),     # the slice of one target fills nearly all the LDS it may take
+    ("bfloat16", 128, "batchtopk", 1501)])  # two features fire on nearly every token: lists cut over many lanes
 def test_adam_inside_the_weight_gradient_kernel_equals_the_two_step_sequence(dev, dtype, d_model, fn, tokens):
     # untied decoders: training_step lets the decoder weights take their Adam step inside the weight-gradient
     # kernel (no fp32 gradient in memory, parameters rewritten from the working copy), over column tiles where
@@ -194,6 +195,10 @@ def test_adam_inside_the_weight_gradient_kernel_equals_the_two_step_sequence(dev
     runs, first = [], []
     for fuse, tiles in ((True, True), (True, False), (False, False)):
         model, sd, x, targets = build(wl, dev)
+        if tokens == 1501:
+            with torch.no_grad():
+                for l in range(3):
+                    model.encoder_module.encoders[l].bias_param[5:7] += 8.0
         opt = cca.CLTAdam(model, lr=1e-2)
         opt.fuse_decoder_step = fuse
         opt.tile_decoder_step = tiles
