@@ -90,8 +90,9 @@ def test_loss_and_gradients_match_autograd(dev, wl):
         assert err <= bound, (name, err)
 
 
-@pytest.mark.parametrize("T,F,k", [(300, 128, 9), (4100, 96, 9), (70, 40960, 9), (40, 2048, 800)],
-                         ids=["blocks-of-tokens", "ragged-last-block", "feature-axis-beyond-lds", "rows-longer-than-a-workgroup"])
+@pytest.mark.parametrize("T,F,k", [(300, 128, 9), (4100, 96, 9), (70, 40960, 9), (40, 2048, 800), (8, 32768, 5000)],
+                         ids=["blocks-of-tokens", "ragged-last-block", "feature-axis-beyond-lds", "rows-longer-than-a-workgroup",
+                              "rows-longer-than-the-staging-buffer"])
 def test_feature_lists_are_a_permutation_grouped_by_feature(dev, T, F, k):
     # the blocked construction (counters of a token block in LDS, token order by construction; 4100 tokens = 33
     # blocks, the last one ragged; rows of ~800 survivors against 512 threads), and for a feature axis whose
@@ -257,6 +258,50 @@ def test_tiled_decoder_layout_round_trip(dev, dtype):
     slab3 = engine.alloc_packed(n_dec, F, d, dtype, dev)
     engine.untile_decoders(tiles, slab3)
     assert torch.equal(slab3, slab2)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("T,F", [(300, 200), (257, 2248)], ids=["ragged-row-block", "two-feature-chunks"])
+def test_tiled_decoder_step_kernel_against_the_row_kernel(dev, dtype, T, F):
+    # the two fused kernels on the same lists, loss gradient, weights and (non-zero) moments: feature counts that
+    # leave the last block of 32 rows ragged and that cross the 2048-feature work units; one feature with a long list
+    g = torch.Generator().manual_seed(21)
+    L, d = 3, 64
+    n_dec = L * (L + 1) // 2
+    pre = torch.randn(L, T, F, generator=g)
+    pre[:, :, 3] += 5.0
+    surv = engine.batchtopk_select(pre.to(dtype).to(dev), 11, False)
+    lists = engine.feature_lists(surv)
+    g_model = (torch.randn(L, T, d, generator=g) * 1e-3).to(dtype).to(dev)
+    w = (torch.randn(n_dec, F, d, generator=g) * 0.1).to(dtype).to(dev)
+    m0 = (torch.randn(n_dec, F, d, generator=g) * 1e-4).to(dev)
+    v0 = (torch.rand(n_dec, F, d, generator=g) * 1e-7).to(dev)
+    slab = engine.alloc_packed(n_dec, F, d, dtype, dev)
+    slab[:, :, :d] = w
+    cs = engine.decoder_tile_width(T, d, F, dtype)
+    assert cs == 32 // slab.element_size()
+    # row kernel
+    slab_r, m_r, v_r = slab.clone(), m0.clone(), v0.clone()
+    engine.decoder_weight_grad_adam(lists, surv, g_model, slab_r, m_r, v_r, 1e-3, (0.9, 0.999), 1e-8, 3)
+    # tile kernel on the tiled copies
+    tiles = engine.tile_decoders(slab, d)
+    to_tiles = lambda t: t.view(n_dec, F, d // cs, cs).permute(0, 2, 1, 3).contiguous()      # noqa: E731
+    from_tiles = lambda t: t.permute(0, 2, 1, 3).contiguous().view(n_dec, F, d)               # noqa: E731
+    m_t, v_t = to_tiles(m0), to_tiles(v0)
+    engine.decoder_weight_grad_adam_tiled(lists, surv, g_model, tiles, m_t, v_t, 1e-3, (0.9, 0.999), 1e-8, 3)
+    slab_t = engine.alloc_packed(n_dec, F, d, dtype, dev)
+    engine.untile_decoders(tiles, slab_t)
+    # the gradient enters m linearly: (m - 0.9 m0) / 0.1 is the gradient each kernel summed
+    g_r, g_t = (m_r - 0.9 * m0) / 0.1, (from_tiles(m_t) - 0.9 * m0) / 0.1
+    assert float((g_r - g_t).abs().max()) <= 2e-5 * float(g_r.abs().max())
+    assert torch.allclose(from_tiles(v_t), v_r, rtol=1e-4, atol=1e-14)
+    x, y = slab_t[:, :, :d].float(), slab_r[:, :, :d].float()
+    ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -20
+    # (fp32: the step is lr * m / sqrt(v) with lr 1e-3, so gradient rounding shows at the 1e-7 level whatever |w|)
+    floor = 1e-3 if dtype == torch.bfloat16 else 0.1
+    assert bool(((x - y).abs() <= ulp * torch.maximum(x.abs(), y.abs()).clamp_min(floor)).all())
+    assert float((x != y).float().mean()) <= (1e-3 if dtype == torch.bfloat16 else 0.5)
+    assert float((y - w.float()).abs().max()) > 0          # and the step did move the weights
 
 
 def test_optimiser_moves_between_the_tiled_and_the_row_route(dev):
