@@ -67,9 +67,25 @@ __global__ __launch_bounds__(256) void k_tile_pairs(const int32_t *__restrict__ 
   for (int64_t q = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 3; q < nlist; q += ((int64_t)gridDim.x * blockDim.x) >> 3) {
     const int32_t b = ptr[q], e = ptr[q + 1];
     const uint8_t place = (uint8_t)((q % F) & (TL_ROWS - 1));
-    for (int32_t i = b + sub; i < e; i += 8) {
-      pairs[i] = TlPair<T>::make(tok[i], val[src[i]]);
-      rowb[i] = place | (i == e - 1 ? 0x80 : 0);
+    for (int32_t i0 = b + sub; i0 < e; i0 += 32) {
+      // four entries per lane with their loads in flight together (token and position, then the value)
+      int32_t tk[4], sr[4];
+      T vl[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int32_t i = i0 + 8 * u < e ? i0 + 8 * u : e - 1;
+        tk[u] = tok[i]; sr[u] = src[i];
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) vl[u] = val[sr[u]];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int32_t i = i0 + 8 * u;
+        if (i < e) {
+          pairs[i] = TlPair<T>::make(tk[u], vl[u]);
+          rowb[i] = place | (i == e - 1 ? 0x80 : 0);
+        }
+      }
     }
   }
 }
@@ -132,8 +148,10 @@ __global__ __launch_bounds__(TL_THREADS) void k_tile_outer_adam(
       for (int64_t base = threadIdx.x >> 1; base < Tn; base += FB * STEP) {
         uint4 tmp[FB];
 #pragma unroll
-        for (int u2 = 0; u2 < FB; ++u2)
-          if (base + u2 * STEP < Tn) tmp[u2] = *reinterpret_cast<const uint4 *>(gt + (base + u2 * STEP) * d);
+        for (int u2 = 0; u2 < FB; ++u2) {      // (past the end: the last token again, not stored)
+          const int64_t tk = base + u2 * STEP < Tn ? base + u2 * STEP : Tn - 1;
+          tmp[u2] = *reinterpret_cast<const uint4 *>(gt + tk * d);
+        }
 #pragma unroll
         for (int u2 = 0; u2 < FB; ++u2)
           if (base + u2 * STEP < Tn) slice[(base + u2 * STEP) * 2 + (threadIdx.x & 1)] = tmp[u2];
