@@ -126,7 +126,7 @@ __global__ __launch_bounds__(TL_THREADS) void k_tile_outer_adam(
   __shared__ uint32_t unit_sh;
   constexpr int EL = 16 / (int)sizeof(T), CS = 2 * EL, NQ = EL / 4;   // NQ: 16-byte pieces of a lane's fp32 values
   typedef typename TlPair<T>::type pair_t;
-  const int lane = lane_id(), wv = threadIdx.x >> 6, h = lane & 1, rl = lane >> 1;
+  const int lane = lane_id(), wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), h = lane & 1, rl = lane >> 1;
   uint4 *slice = tl_lds;
   const char *slice_h = reinterpret_cast<const char *>(tl_lds) + h * 16;    // this lane's half of every token
   // staging: [32 rows][2 halves][NQ pieces]; a bf16 half is 8 fp32 = 2 pieces, an fp32 half 4 fp32 = 1 piece
@@ -160,8 +160,13 @@ __global__ __launch_bounds__(TL_THREADS) void k_tile_outer_adam(
     __syncthreads();
     const int64_t f_begin = k * TL_CHUNK, f_end = f_begin + TL_CHUNK < F ? f_begin + TL_CHUNK : F;
     const int64_t nblk = (f_end - f_begin + TL_ROWS - 1) / TL_ROWS;
-    for (int64_t rb = wv; rb < (t + 1) * nblk; rb += TL_WAVES) {
-      const int64_t s = rb / nblk, f0 = f_begin + (rb - s * nblk) * TL_ROWS, f = f0 + rl;
+    // row blocks wv, wv + 12, ... of the (t + 1) * nblk blocks of the unit, as (source, block) without a division;
+    // everything derived from them is the same for the whole wavefront and stays in scalar registers
+    int sb = 0, blk = wv;
+    for (;; blk += TL_WAVES) {
+      while (blk >= (int)nblk) { blk -= (int)nblk; ++sb; }
+      if (sb > (int)t) break;
+      const int64_t s = sb, f0 = f_begin + (int64_t)blk * TL_ROWS, f = f0 + rl;
       const int nrows = (int)(f_end - f0 < TL_ROWS ? f_end - f0 : TL_ROWS);
       const int64_t q0 = s * F + f0;
       // this lane pair's row as a list: [p_lo, p_hi) (empty beyond the chunk)
@@ -237,16 +242,20 @@ __global__ __launch_bounds__(TL_THREADS) void k_tile_outer_adam(
           }
         }
       };
-      // a group of four: lanes whose group lies wholly inside [B, E) skip the per-entry bounds test (only the
-      // groups at the two ends of the run take the other branch)
+      // a group of four: normally every lane's group lies wholly inside [B, E) or wholly outside, and the
+      // wavefront takes the branch without per-entry bounds tests (a uniform branch: one of the two bodies
+      // runs); only the groups at the two ends of the run have lanes with part of a group inside
       auto group = [&](const pair_t *pr, uint32_t rw, int32_t i) {
         const int32_t i0 = (int32_t)start + i;
-        if (i0 >= B && i0 + 4 <= E) {
-          uint4 pc[4];      // the four LDS reads go out together: their latency is paid once per group
+        const bool whole = i0 >= B && i0 + 4 <= E, some = i0 + 4 > B && i0 < E;
+        if (__builtin_amdgcn_ballot_w64(some && !whole) == 0) {
+          if (whole) {
+            uint4 pc[4];      // the four LDS reads go out together: their latency is paid once per group
 #pragma unroll
-          for (int j = 0; j < 4; ++j) pc[j] = fetch(pr[j]);
+            for (int j = 0; j < 4; ++j) pc[j] = fetch(pr[j]);
 #pragma unroll
-          for (int j = 0; j < 4; ++j) entry(pr[j], pc[j], (rw >> (8 * j)) & 0xFFu);
+            for (int j = 0; j < 4; ++j) entry(pr[j], pc[j], (rw >> (8 * j)) & 0xFFu);
+          }
         } else {
 #pragma unroll
           for (int j = 0; j < 4; ++j)
