@@ -4,6 +4,7 @@ bf16 weights / inputs and accumulate in fp32; the oracle runs in fp32 on the sam
 import pytest
 import torch
 
+from crosslayer_coding_amd import _native as nat
 from crosslayer_coding_amd import engine, synth
 from oracle import clt_oracle as orc
 
@@ -114,6 +115,14 @@ def test_feature_lists_are_a_permutation_grouped_by_feature(dev, T, F, k):
             assert bool((col[src[b:e]] == f).all()) and bool((rows[src[b:e]] // T == l).all())
             assert torch.equal(rows[src[b:e]] % T, tok[b:e])
             assert bool((tok[b + 1:e] > tok[b:e - 1]).all())      # token order, whatever the length
+
+
+def test_feature_lists_of_an_empty_survivor_list(dev):
+    L, T, F = 2, 100, 256
+    surv = engine.threshold_select(torch.zeros(L, T, F, device=dev), None, nat.PRED_NONZERO)
+    assert surv.nnz == 0
+    ptr, tok, src = engine.feature_lists(surv)
+    assert ptr.numel() == L * F + 1 and not bool(ptr.any())
 
 
 def test_long_feature_lists_are_in_token_order_and_gradients_repeat_bit_for_bit(dev):
@@ -270,8 +279,11 @@ def test_tiled_decoder_step_kernel_against_the_row_kernel(dev, dtype, T, F):
     n_dec = L * (L + 1) // 2
     pre = torch.randn(L, T, F, generator=g)
     pre[:, :, 3] += 5.0
+    pre[:, :, 64:128] -= 100.0          # two whole blocks of 32 rows whose lists are empty
     surv = engine.batchtopk_select(pre.to(dtype).to(dev), 11, False)
     lists = engine.feature_lists(surv)
+    ptr = lists[0].cpu()
+    assert int(ptr[128] - ptr[64]) == 0 and int(ptr[4] - ptr[3]) > 64
     g_model = (torch.randn(L, T, d, generator=g) * 1e-3).to(dtype).to(dev)
     w = (torch.randn(n_dec, F, d, generator=g) * 0.1).to(dtype).to(dev)
     m0 = (torch.randn(n_dec, F, d, generator=g) * 1e-4).to(dev)
