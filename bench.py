@@ -638,6 +638,7 @@ def run_backward(args):
                             "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": adam_bytes / adam_sec / 1e9 / HBM_PEAK_GBS}
     return {
         "stages_ms": stages, "roofline": roofline,
+        "decoder_step_route": (("column tiles" if tiled else "rows") if fused else "gradient then Adam") if opt is not None else None,
         "metric": ("CLT training step tokens/sec (forward, MSE loss, gradients, Adam lr 1e-4 with fp32 moments)"
                    if opt is not None else "CLT forward + MSE loss + gradients tokens/sec (no optimizer step)"),
         "value": wl.tokens * args.steps / wall, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,

@@ -147,6 +147,9 @@ def test_c2_training_step_at_full_size(dev):
     # the step itself, with the decoder weights updated inside the weight-gradient kernel
     loss0 = float(model.training_step(inputs, targets, opt))
     assert abs(loss0 - want_loss) <= 1e-4 * want_loss
+    # ... over column tiles where the batch's slice fits the LDS (4096 tokens do), else row by row
+    assert (opt._dec_layout == "tiles") == (engine.decoder_tile_width(T, d, F, torch.bfloat16) > 0)
+    assert opt._dec_layout == ("tiles" if T <= 4096 else "rows")
     for (s, t) in pairs:
         p = torch.nn.Parameter(before[(s, t)].clone())
         p.grad = kept[(s, t)]
