@@ -54,6 +54,9 @@ _SIGNATURES = {
     "clt_encode_threshold_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64, _i64, _int]),
     "clt_encode_threshold_count": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _int, _vp, _vp, _sz, _vp]),
     "clt_encode_threshold_emit": (_int, [_i64, _i64, _i64, _i64, _int, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "clt_encode_threshold_recover": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _int,
+                                            _vp, _i64, _vp, _vp, _sz, _vp]),
+    "clt_poison_if": (_int, [_vp, _i64, _vp, _vp]),
     "clt_pack_decoder": (_int, [_vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _vp]),
     "clt_decode_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64]),
     "clt_decode_sparse": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _i64, _i64, _u64, _int, _int, _vp, _sz, _vp]),

@@ -69,8 +69,12 @@ class CrossLayerTranscoder(BaseTranscoder):
         self.decoder_module = Decoder(config, process_group, self.device, self.dtype)
         self.theta_manager = ThetaManager(config, process_group, self.device, self.dtype)
         self._ws: Optional[Workspace] = None
-        # threshold activations: survivor-array size per (activation, layers, tokens) and totals on their way back
-        self._thr_key, self._thr_capacity, self._thr_elems = None, None, 0
+        # threshold activations (JumpReLU, ReLU): a forward reads nothing back when survivor arrays that hold ANY
+        # batch of the shape fit this many bytes (None: an eighth of the device memory); beyond that it reads
+        # the survivor total back once per forward and sizes the arrays exactly
+        self.threshold_list_budget_bytes: Optional[int] = None
+        # survivor totals on their way back to the host (they tune the candidate pool, nothing depends on them)
+        self._thr_key, self._thr_elems, self._thr_last_total = None, 0, None
         self._thr_pending: List[tuple] = []
 
     # ---- small helpers ---------------------------------------------------------------
@@ -256,6 +260,7 @@ class CrossLayerTranscoder(BaseTranscoder):
         if res is None:
             raise ValueError("inputs do not form one [layers, tokens, d_model] batch")
         _, T, surv = res
+        surv = surv.trimmed()      # buffers indexed by survivor are sized from the list: exact arrays (one read-back)
         ws = self._workspace()
         mask = (1 << L) - 1
         dec = self.decoder_module
@@ -485,38 +490,47 @@ class CrossLayerTranscoder(BaseTranscoder):
             return None
         return layers, T, surv
 
-    # ---- threshold activations: survivor arrays sized without a read-back ---------------------------
+    # ---- threshold activations: exact survivor lists without a read-back ---------------------------------
+    def _note_threshold_total(self, total: int, first: bool) -> None:
+        """The candidate pool of the fused route follows the density seen: set from the first total of a
+        shape, raised by a later one that comes close to it.  Only speed depends on it."""
+        self._thr_last_total = total
+        want = int(2e6 * total / max(1, self._thr_elems))
+        if first:
+            self._density_ppm = min(1000000, max(2000, want))
+        elif want > self._density_ppm:
+            self._density_ppm = min(1000000, want)
+
     def _poll_threshold_runs(self) -> None:
-        """Look at the totals of earlier forwards whose copies have arrived (no waiting): a list that did
-        not fit drops the estimate, so the next forward measures again; a larger total raises it."""
+        """Look at the totals of earlier forwards whose copies have arrived (no waiting)."""
         keep = []
         for host, ev, key in self._thr_pending:
             if not ev.query():
                 keep.append((host, ev, key))
                 continue
-            total, status = int(host[0]), int(host[1])
-            if key != self._thr_key:
-                continue
-            if status != 0:
-                logger.error(
-                    f"Rank {self.rank}: a forward found more active features than its survivor arrays held "
-                    f"({self._thr_capacity} entries); that batch was decoded as if nothing fired. Measuring again.")
-                self._thr_capacity = None
-            elif self._thr_capacity is not None and 2 * total > self._thr_capacity:
-                self._thr_capacity = 2 * total + 4096
-                self._density_ppm = max(self._density_ppm, int(2e6 * total / max(1, self._thr_elems)))
+            if key == self._thr_key and int(host[0]) >= 0:
+                self._note_threshold_total(int(host[0]), self._thr_last_total is None)
         self._thr_pending = keep
 
+    def _threshold_reads_back(self, n: int, T: int, F: int) -> bool:
+        budget = self.threshold_list_budget_bytes
+        if budget is None:
+            budget = torch.cuda.get_device_properties(self.device).total_memory // 8
+        item = torch.empty((), dtype=self.dtype).element_size()
+        return engine.max_list_entries(n, T, F) * (4 + item) > budget
+
     def _threshold_survivors(self, fn: str, layers: List[int], T: int, x_slab, w_slab, b_slab, pre_buf, ws) -> SurvivorList:
-        """JumpReLU / ReLU survivors.  The number of survivors depends on the data.  The first forward of a
-        shape reads it back once and sizes the arrays exactly; later forwards give col / val twice the
-        largest total seen, check on the device that the list fits (clt_survivors_fit) and read nothing
-        back, so the forward is a pure sequence of launches on the current stream."""
+        """JumpReLU / ReLU survivors (clt.py:271-277, theta.py:70-79).  The number of survivors depends on the
+        data.  When arrays for the largest list the shape can produce are affordable, col / val get that size
+        and the forward is a pure sequence of launches on the current stream: the fused route collects into a
+        pool sized from the density seen so far, and a batch that outgrows the pool is redone by the device
+        itself on the dense route (engine.encode_threshold), so the list is exact for any batch.  Otherwise
+        the total is read back once per forward and the arrays are sized exactly."""
         cfg = self.config
         n, F = len(layers), cfg.num_features
         key = (fn, tuple(layers), T, self.dtype)
         if key != self._thr_key:
-            self._thr_key, self._thr_capacity, self._thr_pending = key, None, []
+            self._thr_key, self._thr_pending, self._thr_last_total = key, [], None
         self._thr_elems = n * T * F
         self._poll_threshold_runs()
         theta = None
@@ -524,26 +538,25 @@ class CrossLayerTranscoder(BaseTranscoder):
             theta = self.theta_manager.thresholds(self.dtype)
             if layers != list(range(cfg.num_layers)):
                 theta = theta.index_select(0, torch.tensor(layers, device=theta.device)).contiguous()
-        cap = self._thr_capacity
+        read_back = pre_buf is None or self._threshold_reads_back(n, T, F)
         surv = None
         if fn == "jumprelu" and self.fuse_encode_select:
             # thresholds applied in the encoder epilogue; the pool is sized from the density seen so far
-            surv = engine.encode_threshold(x_slab, w_slab, b_slab, theta, ws, self._density_ppm, capacity=cap)
-            if surv is None and cap is None:
+            surv = engine.encode_threshold(x_slab, w_slab, b_slab, theta, ws, self._density_ppm,
+                                           pre_scratch=None if read_back else pre_buf)
+            if surv is None and read_back:
                 self._density_ppm = min(1000000, 4 * self._density_ppm)
         if surv is None:
             pre = engine.encode(x_slab, w_slab, b_slab, out=pre_buf)
             surv = engine.threshold_select(pre, theta, nat.PRED_GE_THETA if fn == "jumprelu" else nat.PRED_GT_ZERO, ws,
-                                           capacity=cap)
-        if cap is None:
-            total = surv.nnz                       # the one read-back: first forward of this shape
-            self._thr_capacity = 2 * total + 4096
-            self._density_ppm = max(2000, int(2e6 * total / max(1, self._thr_elems)))
+                                           read_back=read_back)
+        if surv.status is None:
+            self._note_threshold_total(int(surv.nnz_hint), self._thr_last_total is None)
         else:
-            # total and fit flag travel to pinned memory behind the kernels; a later forward looks at them
-            host = torch.empty(2, dtype=torch.int32, pin_memory=True)
-            host[0:1].copy_(surv.row_ptr[-1:], non_blocking=True)
-            host[1:2].copy_(surv.status, non_blocking=True)
+            # the total travels to pinned memory behind the kernels; a later forward looks at it
+            surv.nnz_hint = self._thr_last_total
+            host = torch.empty(1, dtype=torch.int32, pin_memory=True)
+            host.copy_(surv.row_ptr[-1:], non_blocking=True)
             ev = torch.cuda.Event()
             ev.record()
             self._thr_pending.append((host, ev, key))
@@ -560,7 +573,7 @@ class CrossLayerTranscoder(BaseTranscoder):
             counts[l * T:(l + 1) * T] = per_row[i * T:(i + 1) * T]
         row_ptr = torch.zeros(L * T + 1, dtype=torch.int32, device=counts.device)
         row_ptr[1:] = torch.cumsum(counts, 0).to(torch.int32)
-        return SurvivorList(row_ptr, surv.col, surv.val, T, surv.F, L, surv.dtype)
+        return SurvivorList(row_ptr, surv.col, surv.val, T, surv.F, L, surv.dtype, surv.status, surv.nnz_hint)
 
     # ---- get_feature_activations -------------------------------------------------------------
     def get_feature_activations(self, inputs: Dict[int, torch.Tensor]) -> Dict[int, torch.Tensor]:
@@ -573,6 +586,8 @@ class CrossLayerTranscoder(BaseTranscoder):
         if res is not None:
             layers, T, surv = res
             dense = engine.densify(surv, out_f32=(cfg.activation_fn == "jumprelu"))
+            if surv.status is not None:
+                engine.poison_if(dense, surv.status)      # a batch no list can hold: NaN, never zeros
             return {l: dense[i] for i, l in enumerate(layers)}
         # inputs that need the per-layer fallbacks
         proc = {l: x.to(device=self.device, dtype=self.dtype) for l, x in inputs.items()}
@@ -634,6 +649,10 @@ class CrossLayerTranscoder(BaseTranscoder):
         targets = [t for t in range(L) if t in inputs]
         out = self.decoder_module.decode_survivors(full, src_mask, min(targets), max(targets) + 1, skip_add=skip,
                                                    ws=self._workspace())
+        if full.status is not None:
+            # a threshold batch with more survivors than a list can hold has no reconstruction here: the
+            # device overwrites the output with NaN rather than leave what an empty list decodes to
+            engine.poison_if(out, full.status)
         return {t: out[t] for t in targets}, full
 
     def forward(self, inputs: Dict[int, torch.Tensor]) -> Dict[int, torch.Tensor]:

@@ -708,7 +708,11 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_select_allot(
 
 // Single block: row_ptr = exclusive scan of keep[] in storage order (row = layer*T + token), one
 // coalesced sweep of SCAN_THREADS * SCAN_ITEMS rows at a time with a running carry.
-__global__ __launch_bounds__(SCAN_THREADS) void k_rowptr_scan(const uint32_t *keep, int64_t R, int32_t *row_ptr) {
+// A total beyond what an int32 row pointer can hold is written as -2 (the prefixes before it are then
+// meaningless); `skip` (may be NULL) gates the whole launch on a device flag.
+__global__ __launch_bounds__(SCAN_THREADS) void k_rowptr_scan(const uint32_t *keep, int64_t R, int32_t *row_ptr,
+                                                              const int32_t *skip = nullptr) {
+  if (skip && *skip != 0) return;
   const int tid = threadIdx.x;
   unsigned long long carry = 0;
   for (int64_t i0 = 0; i0 < R; i0 += (int64_t)SCAN_THREADS * SCAN_ITEMS) {
@@ -724,7 +728,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_rowptr_scan(const uint32_t *ke
     }
     carry += tot;
   }
-  if (tid == 0) row_ptr[R] = (int32_t)carry;
+  if (tid == 0) row_ptr[R] = carry > 0x7FFFFFFFull ? -2 : (int32_t)carry;
 }
 
 // Ordered write of the survivors of each row.
@@ -1061,7 +1065,7 @@ template <typename T, int V, int PRED, bool EMIT>
 __global__ __launch_bounds__(256) void k_threshold(
     const T *pre, int64_t Tn, int64_t F, int64_t L, int64_t lstride, const T *theta,
     uint32_t *row_cnt, const int32_t *row_ptr, int32_t *col_out, T *val_out, const int32_t *skip) {
-  if (EMIT && skip && *skip != 0) return;     // the list did not fit the caller's arrays: it was emptied
+  if (skip && *skip != 0) return;             // gated off by a device flag (another route holds the list, or it was emptied)
   const int l = blockIdx.y;
   const int lane = lane_id(), wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
   const T *th_row = PRED == CLT_PRED_GE_THETA ? theta + (int64_t)l * F : nullptr;
@@ -1379,8 +1383,8 @@ static int run_threshold(bool emit, const T *pre, int64_t Tn, int64_t F, int64_t
   if (gx > maxgx) gx = maxgx;
   dim3 grid(gx, (unsigned)L);
   if (!emit) {
-    k_threshold<T, V, PRED, false><<<grid, 256, 0, stream>>>(pre, Tn, F, L, lstride, theta, row_cnt, nullptr, nullptr, nullptr, nullptr);
-    k_rowptr_scan<<<1, SCAN_THREADS, 0, stream>>>(row_cnt, L * Tn, row_ptr);
+    k_threshold<T, V, PRED, false><<<grid, 256, 0, stream>>>(pre, Tn, F, L, lstride, theta, row_cnt, nullptr, nullptr, nullptr, skip);
+    k_rowptr_scan<<<1, SCAN_THREADS, 0, stream>>>(row_cnt, L * Tn, row_ptr, skip);
   } else {
     k_threshold<T, V, PRED, true><<<grid, 256, 0, stream>>>(pre, Tn, F, L, lstride, theta, nullptr, row_ptr, col, val, skip);
   }
@@ -1613,6 +1617,61 @@ extern "C" int clt_encode_threshold_count(const void *x, const void *w, const vo
                                                                                     (uint32_t *)(ws + tl.off_pfx), rowcnt);
   k_rowptr_scan<<<1, SCAN_THREADS, 0, s>>>(rowcnt, L * T, row_ptr);
   k_thresh_finish<<<1, 64, 0, s>>>(st, (int)L, row_ptr, L * T);
+  return clt_check_launch();
+}
+
+__global__ void k_survivors_fit_clear(int32_t *row_ptr, int64_t n, const int32_t *status);
+
+// ---- the fused threshold route's fallback, decided and run on the device ---------------------------------
+// status[0] != 0: the pool list is not the one to emit (the dense route holds the list, or there is none)
+// status[1] != 0: the dense route is not the one to emit
+// status[2] != 0: the batch has no survivor list (more entries than `capacity`); the list was emptied
+__global__ void k_recover_flag(SelState *st, int L, const int32_t *row_ptr, int64_t R, int32_t *status) {
+  const bool over = row_ptr[R] == -1;
+  for (int l = threadIdx.x; l < L; l += blockDim.x) st[l].status = over ? ST_RETRY : ST_RUN;
+  if (threadIdx.x == 0) { status[0] = over ? 1 : 0; status[1] = over ? 0 : 1; status[2] = 0; }
+}
+__global__ void k_recover_guard(const int32_t *row_ptr, int64_t R, int64_t capacity, int32_t *status) {
+  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+  const int32_t tot = row_ptr[R];
+  if (tot < 0 || (int64_t)tot > capacity) { status[0] = 1; status[1] = 1; status[2] = 1; }
+}
+
+extern "C" int clt_encode_threshold_recover(const void *x, const void *w, const void *b, const void *theta, void *pre,
+                                            int64_t T, int64_t d, int64_t F, int64_t L, int64_t x_layer_stride,
+                                            int64_t w_layer_stride, int64_t b_layer_stride, int64_t theta_layer_stride,
+                                            int64_t pre_layer_stride, int64_t density_ppm, int dtype, int32_t *row_ptr,
+                                            int64_t capacity, int32_t *status, void *workspace, size_t workspace_bytes,
+                                            void *stream) {
+  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (!row_ptr || !workspace || !status || !pre || capacity < 0) return CLT_ERR_ARG;
+  if (!clt_encode_threshold_supported(x, w, b, theta, T, d, F, L, x_layer_stride, w_layer_stride, b_layer_stride,
+                                      theta_layer_stride, density_ppm, dtype))
+    return CLT_ERR_ARG;
+  if (theta_layer_stride != F) return CLT_ERR_ARG;       // the dense compare walks theta as [L][F]
+  const ThreshLayout tl = thresh_layout(T, F, L, density_ppm, dtype);
+  if (workspace_bytes < tl.total) return CLT_ERR_WORKSPACE;
+  if ((((uintptr_t)workspace) & 255u) != 0) return CLT_ERR_ALIGN;
+  hipStream_t s = (hipStream_t)stream;
+  char *ws = (char *)workspace;
+  SelState *st = (SelState *)(ws + tl.off_state);
+  const int64_t R = L * T;
+  k_recover_flag<<<1, 64, 0, s>>>(st, (int)L, row_ptr, R, status);
+  // every launch below returns at once unless the pool overflowed: the projection is stored densely (all
+  // layers carry ST_RETRY then), counted against the thresholds, and the row pointers are rebuilt
+  int rc = clt_launch_encode(x, w, b, pre, T, d, F, L, x_layer_stride, w_layer_stride, b_layer_stride,
+                             pre_layer_stride, dtype, 0, st, nullptr, s);
+  if (rc != CLT_OK) return rc;
+  uint32_t *rowcnt = (uint32_t *)(ws + tl.off_rowcnt);
+  if (dtype == CLT_BF16)
+    rc = dispatch_threshold<bf16_t>(false, pre, T, F, L, pre_layer_stride, theta, CLT_PRED_GE_THETA, rowcnt, row_ptr, nullptr,
+                                    nullptr, status + 1, s);
+  else
+    rc = dispatch_threshold<float>(false, pre, T, F, L, pre_layer_stride, theta, CLT_PRED_GE_THETA, rowcnt, row_ptr, nullptr,
+                                   nullptr, status + 1, s);
+  if (rc != CLT_OK) return rc;
+  k_recover_guard<<<1, 64, 0, s>>>(row_ptr, R, capacity, status);
+  k_survivors_fit_clear<<<256, 256, 0, s>>>(row_ptr, R + 1, status + 2);
   return clt_check_launch();
 }
 

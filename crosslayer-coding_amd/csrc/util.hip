@@ -107,9 +107,26 @@ __global__ __launch_bounds__(256) void k_colstats_vec(const T *pre, float *mean,
   }
 }
 
+// NaN (all-ones bit pattern) over a buffer when a device flag is set
+__global__ void k_poison_if(uint32_t *buf, int64_t bytes, const int32_t *flag) {
+  if (*flag == 0) return;
+  const int64_t words = bytes / 4;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < words; i += (int64_t)gridDim.x * blockDim.x)
+    buf[i] = 0xFFFFFFFFu;
+  if (blockIdx.x == 0 && threadIdx.x < (unsigned)(bytes - words * 4)) ((uint8_t *)buf)[words * 4 + threadIdx.x] = 0xFFu;
+}
+
 }  // namespace
 
-extern "C" int clt_version(void) { return 100; }
+extern "C" int clt_version(void) { return 101; }
+
+extern "C" int clt_poison_if(void *buf, int64_t bytes, const int32_t *flag, void *stream) {
+  if (bytes < 0 || !flag || (bytes > 0 && !buf)) return CLT_ERR_ARG;
+  if ((((uintptr_t)buf) & 3u) != 0) return CLT_ERR_ALIGN;
+  if (bytes == 0) return CLT_OK;
+  k_poison_if<<<1024, 256, 0, (hipStream_t)stream>>>((uint32_t *)buf, bytes, flag);
+  return clt_check_launch();
+}
 
 extern "C" const char *clt_error_string(int code) {
   switch (code) {

@@ -224,7 +224,13 @@ class Decoder(nn.Module):
         if rate is None or T < 256 or d < 256 or d % 4 or F % (256 // esize):
             return t_end
         dense_s = 2.0 * T * F * d / rate
-        per_layer = surv.col.numel() / max(1, surv.L)            # survivors of one source layer (host-side size)
+        # survivors of one source layer, from a host-side figure: the exact total where the list was sized from
+        # it, else the last total seen for the shape; a threshold list whose total is not known yet is priced
+        # at 2 % density (its arrays are sized for the largest list, which says nothing about the batch)
+        total = surv.nnz_hint
+        if total is None:
+            total = surv.col.numel() if surv.status is None else min(surv.col.numel(), surv.L * T * F // 50)
+        per_layer = total / max(1, surv.L)
         n_src = 0
         for t in range(t_end):
             n_src += (src_mask >> t) & 1

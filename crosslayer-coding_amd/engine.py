@@ -25,8 +25,8 @@ from . import _native as nat
 class SurvivorList:
     """Compact activations of L layers x T tokens (CSR by row = layer*T + token).
 
-    ``col`` / ``val`` may be longer than the list (sized from an estimate, see ``status``); every
-    kernel walks the rows through ``row_ptr``, so the tail is never read."""
+    ``col`` / ``val`` may be longer than the list (threshold activations size them for any batch, see
+    ``threshold_select``); every kernel walks the rows through ``row_ptr``, so the tail is never read."""
 
     row_ptr: torch.Tensor  # int32 [L*T + 1]
     col: torch.Tensor      # int32 [capacity >= nnz]   feature index
@@ -35,9 +35,12 @@ class SurvivorList:
     F: int
     L: int
     dtype: torch.dtype
-    # int32 [1] on the device when col / val were sized without reading the total back: 1 = the list did
-    # not fit and was emptied (clt_survivors_fit); None = sized from the exact total
+    # int32 [1] on the device when col / val were sized without reading the total back: 1 = the batch has more
+    # survivors than a list can hold (2^31 - 1) and the list was emptied - whatever is computed from it must
+    # be poisoned (``poison_if``) or refused (``trimmed``); None = sized from the exact total
     status: Optional[torch.Tensor] = None
+    # host-side estimate of the survivor total where one is known without a read-back (cost models only)
+    nnz_hint: Optional[int] = None
 
     @property
     def nnz(self) -> int:
@@ -48,6 +51,32 @@ class SurvivorList:
     def capacity(self) -> int:
         """Entries col / val hold: what buffers indexed by survivor are sized from, without a read-back."""
         return int(self.col.numel())
+
+    def trimmed(self) -> "SurvivorList":
+        """The same list with col / val cut to the exact total (one read-back): for consumers that size
+        survivor-indexed buffers from ``capacity``.  Raises when the batch had no representable list."""
+        if self.status is None:
+            return self
+        total, bad = int(self.row_ptr[-1].item()), int(self.status.item())
+        if bad:
+            raise nat.CLTNativeError("the batch has more active features than a survivor list can hold (2^31 - 1)")
+        return SurvivorList(self.row_ptr, self.col[:total], self.val[:total], self.T, self.F, self.L, self.dtype,
+                            None, total)
+
+
+def max_list_entries(L: int, T: int, F: int) -> int:
+    """Entries no survivor list of this shape exceeds: every element, or what an int32 row pointer addresses."""
+    return min(int(L) * int(T) * int(F), 2 ** 31 - 1)
+
+
+def poison_if(buf: torch.Tensor, flag: torch.Tensor) -> None:
+    """NaN over ``buf`` when the device flag is set (decided on the device, nothing is read back)."""
+    if buf.numel() == 0:
+        return
+    assert buf.is_contiguous()
+    code = nat.load().clt_poison_if(nat.ptr(buf), buf.numel() * buf.element_size(), nat.ptr(flag),
+                                    nat.current_stream(buf.device))
+    nat.check(code, "clt_poison_if")
 
 
 class Workspace:
@@ -317,13 +346,20 @@ def _fit(row_ptr: torch.Tensor, capacity: int) -> torch.Tensor:
     return status
 
 
+def _read_total(row_ptr: torch.Tensor) -> int:
+    total = int(row_ptr[-1].item())
+    if total == -2:
+        raise nat.CLTNativeError("the batch has more active features than a survivor list can hold (2^31 - 1)")
+    return total
+
+
 def threshold_select(pre: torch.Tensor, theta: Optional[torch.Tensor], pred: int,
-                     ws: Optional[Workspace] = None, capacity: Optional[int] = None) -> SurvivorList:
+                     ws: Optional[Workspace] = None, read_back: bool = True) -> SurvivorList:
     """JumpReLU (x >= theta), ReLU (x > 0) or non-zero compaction of pre [L, T, F].
 
-    Two kernels.  ``capacity`` None: one 4-byte read-back in between sizes col / val exactly.  With a
-    ``capacity`` nothing is read back: col / val get that many entries and the returned ``status`` says
-    on the device whether the list fitted (if not, it is empty)."""
+    Two kernels.  ``read_back``: one 4-byte read-back in between sizes col / val exactly.  Without it nothing
+    is read back: col / val get ``max_list_entries`` entries, which every batch fits that a list can
+    represent at all, and ``status`` says on the device whether this one could be (else it is empty)."""
     L, T, F = _check_pre(pre)
     dev = pre.device
     lib = nat.load()
@@ -336,26 +372,31 @@ def threshold_select(pre: torch.Tensor, theta: Optional[torch.Tensor], pred: int
                                    nat.ptr(row_ptr), nat.ptr(wbuf), wbuf.numel(), _stream(pre))
     nat.check(code, "clt_threshold_count")
     status = None
-    if capacity is None:
-        total = int(row_ptr[-1].item())
+    if read_back:
+        total = _read_total(row_ptr)
     else:
-        total = int(capacity)
+        total = max_list_entries(L, T, F)
         status = _fit(row_ptr, total)
     col = torch.empty(max(total, 1), dtype=torch.int32, device=dev)
     val = torch.empty(max(total, 1), dtype=pre.dtype, device=dev)
     code = lib.clt_threshold_emit(nat.ptr(pre), T, F, L, pre.stride(0), nat.ptr(theta), pred, code_dt,
                                   nat.ptr(row_ptr), nat.ptr(col), nat.ptr(val), nat.ptr(status), _stream(pre))
     nat.check(code, "clt_threshold_emit")
-    return SurvivorList(row_ptr, col[:total], val[:total], T, F, L, pre.dtype, status)
+    return SurvivorList(row_ptr, col[:total], val[:total], T, F, L, pre.dtype, status, total if read_back else None)
 
 
 def encode_threshold(x: torch.Tensor, w: torch.Tensor, b: Optional[torch.Tensor], theta: torch.Tensor,
-                     ws: Workspace, density_ppm: int = 20000, capacity: Optional[int] = None) -> Optional[SurvivorList]:
+                     ws: Workspace, density_ppm: int = 20000,
+                     pre_scratch: Optional[torch.Tensor] = None) -> Optional[SurvivorList]:
     """Encoder projection + JumpReLU (x >= theta) without dense pre-activations
-    (parallel.py:286 + theta.py:70-79).  Returns None when the shapes do not qualify or (``capacity``
-    None) the survivors exceeded what ``density_ppm`` provides for: the caller then runs ``encode`` and
-    ``threshold_select``.  With a ``capacity`` nothing is read back from the device: col / val get that
-    many entries and ``status`` tells, on the device, whether pool and arrays were large enough."""
+    (parallel.py:286 + theta.py:70-79).  Returns None when the shapes do not qualify.
+
+    ``pre_scratch`` None: the total is read back once and col / val are sized exactly; None is returned when
+    the survivors exceeded the pool ``density_ppm`` provides for (the caller then runs ``encode`` and
+    ``threshold_select``).  With ``pre_scratch`` [L, T, F] nothing is read back: col / val get
+    ``max_list_entries`` entries, and a pool that turns out too small makes the device itself take the
+    dense route through ``pre_scratch`` (clt_encode_threshold_recover), so the list is exact whatever the
+    density; ``status`` is set only for a batch no list can represent."""
     nat.require_device(x, "encode_threshold")
     L, T, d = x.shape
     F = w.shape[1]
@@ -367,26 +408,40 @@ def encode_threshold(x: torch.Tensor, w: torch.Tensor, b: Optional[torch.Tensor]
     if not lib.clt_encode_threshold_supported(nat.ptr(x), nat.ptr(w), nat.ptr(b), nat.ptr(theta), T, d, F, L,
                                               *strides, int(density_ppm), dt):
         return None
+    if pre_scratch is not None and theta.stride(0) != F:
+        return None
     nbytes = lib.clt_encode_threshold_workspace_bytes(T, d, F, L, int(density_ppm), dt)
     wbuf = ws.get("collect_threshold", nbytes)
     row_ptr = torch.empty(L * T + 1, dtype=torch.int32, device=x.device)
     code = lib.clt_encode_threshold_count(nat.ptr(x), nat.ptr(w), nat.ptr(b), nat.ptr(theta), T, d, F, L, *strides,
                                           int(density_ppm), dt, nat.ptr(row_ptr), nat.ptr(wbuf), wbuf.numel(), _stream(x))
     nat.check(code, "clt_encode_threshold_count")
-    status = None
-    if capacity is None:
-        total = int(row_ptr[-1].item())
+    flags = None
+    if pre_scratch is None:
+        total = _read_total(row_ptr)
         if total < 0:
             return None
     else:
-        total = int(capacity)
-        status = _fit(row_ptr, total)
+        assert pre_scratch.shape == (L, T, F) and pre_scratch.dtype == x.dtype
+        assert pre_scratch.stride(2) == 1 and pre_scratch.stride(1) == F
+        total = max_list_entries(L, T, F)
+        flags = torch.empty(3, dtype=torch.int32, device=x.device)
+        code = lib.clt_encode_threshold_recover(nat.ptr(x), nat.ptr(w), nat.ptr(b), nat.ptr(theta), nat.ptr(pre_scratch),
+                                                T, d, F, L, *strides, pre_scratch.stride(0), int(density_ppm), dt,
+                                                nat.ptr(row_ptr), total, nat.ptr(flags), nat.ptr(wbuf), wbuf.numel(),
+                                                _stream(x))
+        nat.check(code, "clt_encode_threshold_recover")
     col = torch.empty(max(total, 1), dtype=torch.int32, device=x.device)
     val = torch.empty(max(total, 1), dtype=x.dtype, device=x.device)
     code = lib.clt_encode_threshold_emit(T, F, L, int(density_ppm), dt, nat.ptr(row_ptr), nat.ptr(col), nat.ptr(val),
-                                         nat.ptr(status), nat.ptr(wbuf), wbuf.numel(), _stream(x))
+                                         nat.ptr(flags), nat.ptr(wbuf), wbuf.numel(), _stream(x))
     nat.check(code, "clt_encode_threshold_emit")
-    return SurvivorList(row_ptr, col[:total], val[:total], T, F, L, x.dtype, status)
+    if flags is None:
+        return SurvivorList(row_ptr, col[:total], val[:total], T, F, L, x.dtype, None, total)
+    code = lib.clt_threshold_emit(nat.ptr(pre_scratch), T, F, L, pre_scratch.stride(0), nat.ptr(theta), nat.PRED_GE_THETA,
+                                  dt, nat.ptr(row_ptr), nat.ptr(col), nat.ptr(val), flags[1:].data_ptr(), _stream(x))
+    nat.check(code, "clt_threshold_emit")
+    return SurvivorList(row_ptr, col[:total], val[:total], T, F, L, x.dtype, flags[2:3])
 
 
 # ---- evaluation reductions ------------------------------------------------------------------------------

@@ -45,7 +45,7 @@ class DeadFeatureTracker:
                            f"Counter: {tuple(n.shape)}. Skipping dead neuron update.")
             return
         if fired is None:
-            _, fired = engine.survivor_metrics(survivors, FIRED_EPS)
+            _, fired = engine.survivor_metrics(survivors.trimmed(), FIRED_EPS)
         engine.dead_feature_update(fired, n)
 
     @property
@@ -95,7 +95,7 @@ class CLTEvaluator:
         """A survivor list plus the layers it covers.  Accepts the list itself (all layers) or the
         reference's ``{layer: dense [T, F]}``, which is compacted on the device."""
         if isinstance(activations, SurvivorList):
-            return list(range(activations.L)), activations
+            return list(range(activations.L)), activations.trimmed()   # raises for a batch without a valid list
         layers = sorted(l for l, a in activations.items() if a.numel() > 0 and a.shape[0] > 0)
         if not layers:
             return None

@@ -232,16 +232,25 @@ int clt_threshold_emit(const void *pre, int64_t T, int64_t F, int64_t L,
 
 /*
  * For callers that do not read the survivor total back between a count call and its emit call (no
- * host synchronisation in the forward): col / val are sized from an estimate, `capacity` entries, and
- * this check runs on the device in between.  If the total row_ptr[R] (R = L*T) is negative (the pool of
- * clt_encode_threshold_count overflowed) or exceeds `capacity`, *status = 1 and the list is emptied
- * (row_ptr := 0 everywhere, so every later kernel sees rows without survivors); otherwise *status = 0.
- * The emit calls take `status` as their `skip` argument and write nothing when it is set (NULL: no
- * check).  The caller looks at *status whenever it next touches the host anyway, and repeats the batch
- * with a larger capacity if it was set.  No counterpart in the reference, where the dense mask has a
- * fixed size.
+ * host synchronisation in the forward).  Such a caller gives col / val a capacity that no batch it can
+ * represent exceeds - min(L*T*F, 2^31 - 1) entries, the most an int32 row pointer addresses - and runs
+ * this check on the device in between.  If the total row_ptr[R] (R = L*T) is negative (a count beyond
+ * 2^31 - 1 is stored as -2) or exceeds `capacity`, *status = 1 and the list is emptied (row_ptr := 0
+ * everywhere, so every later kernel sees rows without survivors); otherwise *status = 0.  The emit
+ * calls take `status` as their `skip` argument and write nothing when it is set (NULL: no check).  A
+ * batch with *status = 1 has NO valid survivor list: the caller must not hand results computed from it
+ * on (see clt_poison_if).  No counterpart in the reference, where the dense mask has a fixed size.
  */
 int clt_survivors_fit(int32_t *row_ptr, int64_t R, int64_t capacity, int32_t *status, void *stream);
+
+/*
+ * Fills `buf` (`bytes` of it, 4-byte aligned) with NaN bit patterns (all bits set:
+ * NaN as float32, bfloat16 and float16 alike) when *flag != 0, and does nothing otherwise; the decision
+ * is taken on the device.  For results computed from a survivor list that clt_survivors_fit or
+ * clt_encode_threshold_recover had to give up on: they become unmistakably invalid instead of looking
+ * like reconstructions without active features.  No counterpart in the reference.
+ */
+int clt_poison_if(void *buf, int64_t bytes, const int32_t *flag, void *stream);
 
 /*
  * clt_threshold_count for callers that cannot allocate device memory (code under HIP graph capture,
@@ -289,6 +298,32 @@ int clt_encode_threshold_count(const void *x, const void *w, const void *b, cons
 int clt_encode_threshold_emit(int64_t T, int64_t F, int64_t L, int64_t density_ppm, int dtype,
                               const int32_t *row_ptr, int32_t *col, void *val, const int32_t *skip,
                               void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * The fused route's fallback, decided and run on the device: call it between
+ * clt_encode_threshold_count and the emit calls, on the same stream, with the same workspace and
+ * density_ppm.  If the pool of clt_encode_threshold_count was too small (row_ptr[L*T] == -1), the
+ * projection is repeated with the dense store into `pre` [L][T][F] (scratch, written only then),
+ * compared with the thresholds and row_ptr is rebuilt from the dense counts - the route of
+ * clt_encode + clt_threshold_count, launched behind a device flag so that the host never has to
+ * look.  status is int32[3] on the device:
+ *   status[0]  pass as `skip` to clt_encode_threshold_emit (set when the pool list is not the one to emit)
+ *   status[1]  pass as `skip` to clt_threshold_emit on `pre` with CLT_PRED_GE_THETA (set when the dense
+ *              route was not needed)
+ *   status[2]  set when the batch has more than `capacity` survivors (or more than 2^31 - 1): the list
+ *              was emptied as by clt_survivors_fit, both emits skip; cannot happen with
+ *              capacity = min(L*T*F, 2^31 - 1) unless the total exceeds 2^31 - 1
+ * After both emit calls the list in row_ptr / col / val is the exact one whichever route produced it.
+ * theta_layer_stride must be F.  Replaces the same reference calls as clt_encode_threshold_count
+ * (clt/models/parallel.py:286, clt/models/theta.py:70-79), for a batch of any density.
+ */
+int clt_encode_threshold_recover(const void *x, const void *w, const void *b, const void *theta, void *pre,
+                                 int64_t T, int64_t d, int64_t F, int64_t L,
+                                 int64_t x_layer_stride, int64_t w_layer_stride,
+                                 int64_t b_layer_stride, int64_t theta_layer_stride,
+                                 int64_t pre_layer_stride, int64_t density_ppm, int dtype,
+                                 int32_t *row_ptr, int64_t capacity, int32_t *status,
+                                 void *workspace, size_t workspace_bytes, void *stream);
 
 /*
  * Repack decoder weights from the checkpoint layout [d][F] (nn.Linear weight of

@@ -5,7 +5,8 @@ import pytest
 import torch
 
 import crosslayer_coding_amd as cca
-from crosslayer_coding_amd import synth
+from crosslayer_coding_amd import _native as nat
+from crosslayer_coding_amd import engine, synth
 from oracle import clt_oracle as orc
 
 pytestmark = pytest.mark.gpu
@@ -282,18 +283,19 @@ def test_model_to_device_keeps_results(dev):
 
 @pytest.mark.parametrize("name", ["fused-topk-bf16", "fused-jump-bf16", "tiny-jump", "tiny-relu", "tiny-global", "tiny-per-target"])
 def test_forward_reads_nothing_back_from_the_device(dev, name):
-    # The forward is a sequence of launches on the current stream.  The survivor count of a threshold
-    # activation depends on the data: the first forward of a shape reads it back once to size the arrays,
-    # every later one sizes them from what was seen and checks the fit on the device.
+    # The forward is a sequence of launches on the current stream - from the first one on.  The survivor count
+    # of a threshold activation depends on the data: its arrays are sized for any batch of the shape.
     wl = next(c for c in CASES if c.name == name)
     model, sd, x = build(wl, dev)
     inputs = {l: x[l].to(dev) for l in range(wl.num_layers)}
-    first = model(inputs)
+    other = {l: (1.05 * v).to(v.dtype) for l, v in inputs.items()}                 # other data, same shape
+    model.decoder_module.packed()                      # the one-off repack of the decoders is not the forward
     torch.cuda.synchronize()
     torch.cuda.set_sync_debug_mode("error")
     try:
+        first = model(inputs)
         second = model(inputs)
-        third = model({l: (1.05 * v).to(v.dtype) for l, v in inputs.items()})      # other data, same shape
+        third = model(other)
     finally:
         torch.cuda.set_sync_debug_mode("default")
     torch.cuda.synchronize()
@@ -301,35 +303,101 @@ def test_forward_reads_nothing_back_from_the_device(dev, name):
         assert torch.equal(first[t], second[t])
         assert torch.isfinite(third[t]).all()
     if wl.activation_fn in ("jumprelu", "relu"):
-        model(inputs)                                   # polls the totals of the two forwards above
-        assert model._thr_capacity is not None and not model._thr_pending[:-1]
+        model(inputs)                                   # polls the totals of the forwards above
+        assert model._thr_last_total is not None and not model._thr_pending[:-1]
+        # with a budget that the arrays of the shape exceed, every forward reads the total back: same result
+        model.threshold_list_budget_bytes = 1024
+        exact = model(inputs)
+        for t in first:
+            assert torch.equal(first[t], exact[t])
 
 
-def test_threshold_forward_recovers_when_the_survivors_outgrow_the_arrays(dev, caplog):
-    # a batch with many more active features than any seen before: its list does not fit, it is decoded as
-    # empty (bias only), the next forward reports it and measures again
+def dense_compare_forward(model, inputs, L):
+    """The reference's formulation on the device: dense pre-activations, compare, decode of the dense result."""
+    pre = {l: model.get_preactivations(inputs[l], l) for l in range(L)}
+    theta = model.theta_manager.thresholds(model.dtype)
+    acts = {l: torch.where(pre[l] >= theta[l], pre[l], torch.zeros_like(pre[l])) for l in range(L)}
+    return acts, {t: model.decoder_module.decode({l: acts[l] for l in range(t + 1)}, t) for t in range(L)}
+
+
+def test_threshold_forward_is_exact_when_the_survivors_outgrow_the_pool(dev):
+    # A batch with many times the active features of any seen before (clt.py:271-277, theta.py:70-79: exact
+    # for any batch).  The fused route's candidate pool, sized from the density seen so far, overflows; the
+    # device itself redoes the batch on the dense route.  The forward reads nothing back and is exact.
     wl = next(c for c in CASES if c.name == "fused-jump-bf16")
     model, sd, x = build(wl, dev)
     L = wl.num_layers
     inputs = {l: x[l].to(dev) for l in range(L)}
     want_small = {t: v.clone() for t, v in model(inputs).items()}
+    model(inputs)
+    torch.cuda.synchronize()
+    model(inputs)                                                       # the pool now follows the density seen
+    small_total = model._thr_last_total
+    ppm = model._density_ppm
     big = {l: (40.0 * v).to(v.dtype) for l, v in inputs.items()}        # scales every pre-activation: far more survivors
-    overflowed = model(big)
+    acts_ref, rec_ref = dense_compare_forward(model, big, L)
     torch.cuda.synchronize()
-    bias_only = model.decoder_module.bias_sum((1 << L) - 1)
+    torch.cuda.set_sync_debug_mode("error")
+    try:
+        res = model.forward_with_survivors(big)
+    finally:
+        torch.cuda.set_sync_debug_mode("default")
+    assert res is not None
+    overflowed, surv = res
+    torch.cuda.synchronize()
+    assert model._density_ppm == ppm                                    # the pool was the small one
+    total = surv.nnz
+    assert total > 8 * small_total
+    assert int(surv.status.item()) == 0
+    dense = engine.densify(surv)
+    for l in range(L):
+        assert torch.equal(dense[l], acts_ref[l])                       # the survivor set and values, bit for bit
     for t in range(L):
-        assert torch.equal(overflowed[t].float(), bias_only[t].to(overflowed[t].dtype).float().expand_as(overflowed[t]))
-    with caplog.at_level(logging.ERROR):
-        again = model(big)                                             # sees the flag, measures, sizes exactly
-    assert any("more active features than its survivor arrays held" in r.message for r in caplog.records)
+        assert orc.rel_l2(overflowed[t].float().cpu(), rec_ref[t].float().cpu()) <= 1e-2
+    # the same batch again: the pool has grown, the fused route holds it, the result is the same list
+    again, surv2 = model.forward_with_survivors(big)
     torch.cuda.synchronize()
+    assert model._density_ppm > ppm
+    assert torch.equal(surv2.row_ptr, surv.row_ptr)
+    assert torch.equal(surv2.col[:total], surv.col[:total])
+    assert torch.equal(surv2.val[:total].view(torch.int16), surv.val[:total].view(torch.int16))
+    for t in range(L):
+        assert torch.equal(again[t], overflowed[t])
     acts = model.get_feature_activations(big)
-    assert int((acts[0] != 0).sum()) > 4 * int((model.get_feature_activations(inputs)[0] != 0).sum())
-    ref = model.decoder_module.decode({l: acts[l] for l in range(L)}, L - 1)
-    assert orc.rel_l2(again[L - 1].float().cpu(), ref.float().cpu()) <= 1e-2
+    for l in range(L):
+        assert torch.equal(acts[l].to(acts_ref[l].dtype), acts_ref[l])
     back = model(inputs)
     for t in range(L):
         assert torch.equal(back[t], want_small[t])
+
+
+def test_threshold_batch_beyond_any_list_is_poisoned_not_returned(dev):
+    # clt_survivors_fit / clt_poison_if: a list that cannot be represented must not decode as "nothing fired".
+    # Forced here through a tiny capacity on a real count; the model uses the largest list of the shape.
+    g = torch.Generator().manual_seed(3)
+    pre = torch.randn(2, 64, 256, generator=g).to(dev)
+    lib = nat.load()
+    row_ptr = torch.empty(2 * 64 + 1, dtype=torch.int32, device=dev)
+    wbuf = torch.empty(2 * 64 * 4, dtype=torch.uint8, device=dev)
+    s = torch.cuda.current_stream().cuda_stream
+    nat.check(lib.clt_threshold_count(pre.data_ptr(), 64, 256, 2, 64 * 256, None, nat.PRED_GT_ZERO, nat.CLT_F32,
+                                      row_ptr.data_ptr(), wbuf.data_ptr(), wbuf.numel(), s), "count")
+    total = int(row_ptr[-1].item())
+    status = engine._fit(row_ptr, total - 1)
+    out = torch.ones(5, 7, device=dev, dtype=torch.bfloat16)
+    engine.poison_if(out, status)
+    assert int(status.item()) == 1 and int(row_ptr.abs().sum()) == 0 and torch.isnan(out).all()
+    surv = engine.SurvivorList(row_ptr, torch.empty(1, dtype=torch.int32, device=dev), torch.empty(1, device=dev), 64, 256, 2,
+                               torch.float32, status)
+    with pytest.raises(nat.CLTNativeError):
+        surv.trimmed()
+    # a list that fits: flag clear, nothing touched
+    nat.check(lib.clt_threshold_count(pre.data_ptr(), 64, 256, 2, 64 * 256, None, nat.PRED_GT_ZERO, nat.CLT_F32,
+                                      row_ptr.data_ptr(), wbuf.data_ptr(), wbuf.numel(), s), "count")
+    status = engine._fit(row_ptr, total)
+    out = torch.ones(5, 7, device=dev, dtype=torch.bfloat16)
+    engine.poison_if(out, status)
+    assert int(status.item()) == 0 and int(row_ptr[-1].item()) == total and bool((out == 1).all())
 
 
 def test_profiler_hook_receives_the_reference_timer_names(dev):
