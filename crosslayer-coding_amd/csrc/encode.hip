@@ -156,6 +156,7 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
   __shared__ __attribute__((aligned(16))) unsigned char stage1[STAGE];
   __shared__ uint16_t cand_list[COLLECT ? NWAVES : 1][COLLECT ? CAND_LIST : 1];   // per wavefront, see the emission
   __shared__ __attribute__((aligned(16))) T bias_lds[NWAVES][128];                // per wavefront: the bias of its features
+  __shared__ __attribute__((aligned(16))) T theta_lds[COLLECT == 2 ? NWAVES : 1][COLLECT == 2 ? 128 : 8];   // and their thresholds
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -256,27 +257,45 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
   auto load_bias = [&](const TileAt &t) {
     if (bias && lane < BIAS_LANES)
       load16_to_lds(bias + (int64_t)t.layer * bs + t.n0 + wn * 128 + lane * CE, bias_lds[wave]);
+    if constexpr (COLLECT == 2) {
+      if (lane < BIAS_LANES)
+        load16_to_lds((const T *)ca.theta + (int64_t)t.layer * ca.theta_stride + t.n0 + wn * 128 + lane * CE, theta_lds[wave]);
+    }
   };
   if (!bias && lane < BIAS_LANES)   // no bias: the slot holds zeros for good
     *reinterpret_cast<uint4 *>(reinterpret_cast<unsigned char *>(bias_lds[wave]) + lane * 16) = make_uint4(0u, 0u, 0u, 0u);
+  // The bias is read with hand-written LDS loads and a hand-placed wait: the compiler, which cannot tell how
+  // many of the outstanding direct loads are older than the one into the bias slot, would otherwise wait for
+  // all of them (the stage just asked for included) before the first read.
+  const uint32_t bias_at = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)
+                               reinterpret_cast<unsigned char *>(bias_lds[wave]) + (uint32_t)(lane >> 5) * 4u * (uint32_t)sizeof(T);
   auto init_acc = [&]() {
+    typedef typename std::conditional<sizeof(T) == 4, uint4, uint2>::type braw_t;
+    braw_t raw[16];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg) {
+        if constexpr (sizeof(T) == 4)
+          asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(raw[j * 4 + rg]) : "v"(bias_at), "n"((j * 32 + rg * 8) * 4));
+        else
+          asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(raw[j * 4 + rg]) : "v"(bias_at), "n"((j * 32 + rg * 8) * 2));
+      }
+    __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0)
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
       for (int rg = 0; rg < 4; ++rg) {
         float bv[4];
-        const T *bp = bias_lds[wave] + j * 32 + rg * 8 + (lane >> 5) * 4;
         if constexpr (sizeof(T) == 4) {
-          const float4 r = *reinterpret_cast<const float4 *>(bp);
-          bv[0] = r.x; bv[1] = r.y; bv[2] = r.z; bv[3] = r.w;
+          const uint4 r = raw[j * 4 + rg];
+          bv[0] = __uint_as_float(r.x); bv[1] = __uint_as_float(r.y); bv[2] = __uint_as_float(r.z); bv[3] = __uint_as_float(r.w);
         } else {
-          const uint2 r = *reinterpret_cast<const uint2 *>(bp);
+          const uint2 r = raw[j * 4 + rg];
           bv[0] = __uint_as_float(r.x << 16); bv[1] = __uint_as_float(r.x & 0xFFFF0000u);
           bv[2] = __uint_as_float(r.y << 16); bv[3] = __uint_as_float(r.y & 0xFFFF0000u);
         }
-        // pins the copies into the accumulators here instead of at the reads
-#pragma unroll
-        for (int q = 0; q < 4; ++q) asm volatile("" : "+v"(bv[q]));
 #pragma unroll
         for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -360,6 +379,14 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
     asm volatile("" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);    // nothing that reads the bias may move above the wait
     init_acc();
+    // The layer's cut is asked for here and used in the epilogue.  A hand-written load: the compiler does not
+    // know that it is outstanding and waits for nothing; it is older than the loads of the first refill below,
+    // so the wait of the stage after that one guarantees that it has arrived.
+    uint32_t cut_key_v = 0;
+    if constexpr (COLLECT == 1) {
+      const uint32_t *cut_at = &ca.st[layer].cut_key;
+      asm volatile("global_load_dword %0, %1, off" : "=v"(cut_key_v) : "v"(cut_at));
+    }
     load_frags(fa, stage0, 0);
     // nk is even (checked by the launcher)
     for (int kt = 0; kt < nk - 2; kt += 2) {
@@ -449,7 +476,10 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
         constexpr int NWL = SEGW / 64;                       // 32-bit mask words per lane (half a row)
         const int ncol0 = n0 + wn * 128 + pass * SEGW;       // first feature of the segment
         uint32_t cut_bits = 0;
-        if constexpr (COLLECT == 1) cut_bits = key_to_f32_bits<KB>(ca.st[layer].cut_key);
+        if constexpr (COLLECT == 1) {
+          asm volatile("" : "+v"(cut_key_v));      // nothing that reads the cut may move above this point
+          cut_bits = key_to_f32_bits<KB>((uint32_t)__builtin_amdgcn_readfirstlane((int)cut_key_v));
+        }
         const bool cut_nan = (cut_bits & 0x7FFFFFFFu) > 0x7F800000u;   // only NaNs reach such a cut
         const float cutf = __uint_as_float(cut_bits);
         const int hs = lh, rsw = l31 & 15;
@@ -466,7 +496,7 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
             const uint4 v = *reinterpret_cast<const uint4 *>(myrow + ((sl ^ rsw) * 16));
             uint4 tv = make_uint4(0, 0, 0, 0);
             if constexpr (COLLECT == 2)
-              tv = *reinterpret_cast<const uint4 *>((const T *)ca.theta + (int64_t)layer * ca.theta_stride + ncol0 + sl * EPS);
+              tv = *reinterpret_cast<const uint4 *>(theta_lds[wave] + pass * SEGW + sl * EPS);
             uint32_t m = 0;
 #pragma unroll
             for (int j = 0; j < EPS; ++j) {
@@ -494,7 +524,7 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
             fast_ok = cb >= 1u && cb <= 0x7F80u;
             cm1 = (cb - 1u) | ((cb - 1u) << 16);
           } else {
-            theta_seg = (const T *)ca.theta + (int64_t)layer * ca.theta_stride + ncol0;
+            theta_seg = theta_lds[wave] + pass * SEGW;
             bool bad = false;
             if (lane_e < 16) {   // every threshold of the segment must be a positive number
               const uint4 tv = *reinterpret_cast<const uint4 *>(theta_seg + lane_e * 8);
@@ -642,8 +672,9 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
     }
     if (!has_next) break;
     // Every wavefront is done with its parked rows before the next tile's loads overwrite them.  The wait
-    // is for this wavefront's LDS reads only: the first stage of the next tile may still be on its way.
-    __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0)
+    // covers the epilogue's stores as well (and the next tile's first stage, long since landed): with only
+    // loads outstanding afterwards, the counted wait at the top of the tile is exact.
+    __builtin_amdgcn_s_waitcnt(0);
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
