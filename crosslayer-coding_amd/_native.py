@@ -88,6 +88,7 @@ _SIGNATURES = {
     "clt_adam_step_decoders": (_int, [_vp, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _f64, _f64, _f64, _f64, _i64, _int, _vp]),
     "clt_adam_step_many": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _f64, _f64, _f64, _f64, _i64, _int, _vp]),
     "clt_decoder_norms": (_int, [_vp, _vp, _i64, _i64, _i64, _int, _int, _vp]),
+    "clt_scatter_survivor_values": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp, _vp]),
     "clt_jumprelu_theta_grad_workspace_bytes": (_sz, [_i64]),
     "clt_jumprelu_theta_grad": (_int, [_vp, _vp, _vp, _i64, _i64, _f64, _int, _vp, _vp, _sz, _vp]),
     "clt_probe_gather": (_int, [_vp, _i64, _i64, _vp, _i64, _i64, _int, _vp, _vp]),

@@ -228,8 +228,10 @@ class CrossLayerTranscoder(BaseTranscoder):
     # ---- loss and gradients --------------------------------------------------------------------
     def _denorm_args(self, normalization_method, mean_tg, std_tg):
         """(mode, mean [L, d], std [L, d], scale) of the de-normalisation the reference's LossManager applies
-        before the loss (losses.py:70-86): "mean_std" needs the target statistics of EVERY layer (the
-        reference skips a layer that has none; a mixture is not supported here and raises)."""
+        before the loss (losses.py:70-86): "mean_std" uses the target statistics of the layers that have them
+        and leaves the others alone, as the reference does.  The method defaults to CLTConfig.normalization_method;
+        the reference's LossManager reads TrainingConfig.normalization_method, which its trainer sets to the same
+        value - pass ``normalization_method`` when the two differ."""
         cfg = self.config
         method = cfg.normalization_method if normalization_method is None else normalization_method
         L, d = cfg.num_layers, cfg.d_model
@@ -237,11 +239,14 @@ class CrossLayerTranscoder(BaseTranscoder):
             have = [l for l in range(L) if mean_tg and std_tg and l in mean_tg and l in std_tg]
             if not have:
                 return "none", None, None, 1.0          # no statistics given: the reference leaves the tensors alone
-            if len(have) != L:
-                raise ValueError("mean_std de-normalisation needs mean_tg / std_tg for every layer")
-            stack = lambda dct: torch.stack([dct[l].to(device=self.device, dtype=self.dtype).reshape(-1)[-d:]  # noqa: E731
-                                             for l in range(L)]).contiguous()
-            return "mean_std", stack(mean_tg), stack(std_tg), 1.0
+            # a layer without statistics is left alone by the reference: mean 0 and std 1 do exactly that
+            # (x * 1 + 0 is x in any dtype, and the gradient's factor is 1)
+            mean = torch.zeros((L, d), device=self.device, dtype=self.dtype)
+            std = torch.ones((L, d), device=self.device, dtype=self.dtype)
+            for l in have:
+                mean[l] = mean_tg[l].to(device=self.device, dtype=self.dtype).reshape(-1)[-d:]
+                std[l] = std_tg[l].to(device=self.device, dtype=self.dtype).reshape(-1)[-d:]
+            return "mean_std", mean, std, 1.0
         if method == "sqrt_d_model":
             return "sqrt_d_model", None, None, float(d) ** 0.5
         return "none", None, None, 1.0
@@ -270,8 +275,6 @@ class CrossLayerTranscoder(BaseTranscoder):
         mode, mean, std, scale = self._denorm_args(normalization_method, mean_tg, std_tg)
         loss_l, g, g_model, bias_grad = engine.mse_loss_grad(rec, tgt.contiguous(), ws, mode, mean, std, scale)
         off, sc = dec._affine()                     # per-target feature offset / scale of tied decoders, or None
-        if cfg.activation_fn == "jumprelu" and (off is not None or sc is not None):
-            raise NotImplementedError("the JumpReLU threshold gradient is not built for decoders with feature offset / scale")
         dval = engine.decode_backward_values(surv, dec.packed(), g, cfg.decoder_tying, mask, ws, feat_scale=sc)
         lists = engine.feature_lists(surv, ws)
         d_off, d_sc = (engine.feature_affine_grad(lists, surv, ws, off, sc, mask) if (off is not None or sc is not None)
@@ -291,7 +294,7 @@ class CrossLayerTranscoder(BaseTranscoder):
                 engine.skip_weight_grad(g[t], x_slab[s_], d_skip[i])
         theta_grad = None
         if cfg.activation_fn == "jumprelu" and self.theta_manager.log_threshold is not None:
-            theta_grad = self._log_threshold_gradient(x_slab, g_model, ws)
+            theta_grad = self._log_threshold_gradient(x_slab, g_model, ws, surv, dval if sc is not None else None)
         if decoder_step is not None:
             decoder_step.decoder_weight_step(lists, surv, g_model)
         # bias_grad[t] = column sums of d loss / d rec[t]; a decoder's bias takes the rows of the targets
@@ -305,12 +308,15 @@ class CrossLayerTranscoder(BaseTranscoder):
         return loss_l, {"enc_w": dw_enc, "enc_b": db_enc, "dec_w": dw_dec, "dec_b": dec_b.contiguous(), "theta": theta_grad,
                         "skip": d_skip, "feat_offset": d_off, "feat_scale": d_sc}
 
-    def _log_threshold_gradient(self, x_slab: torch.Tensor, g_model: torch.Tensor, ws) -> torch.Tensor:
+    def _log_threshold_gradient(self, x_slab: torch.Tensor, g_model: torch.Tensor, ws, surv=None, dval=None) -> torch.Tensor:
         """fp32 [L, F] gradient of ``log_threshold`` (JumpReLU.backward, activations.py:196-199, through
         theta = exp(log_threshold), theta.py:70-79).  The band |x - theta| <= bandwidth / 2 holds elements
         on both sides of the threshold, so this part is dense: per source layer, d loss / d activation
         is one product of the stacked loss gradients [T, (L-s) d] with the stacked decoders [F, (L-s) d]
-        on the MFMA kernel, reduced over tokens together with the dense pre-activations."""
+        on the MFMA kernel, reduced over tokens together with the dense pre-activations.  Behind a per-target
+        feature scale (decoder.py:228-285: applied to the non-zero activations only) the kept elements of the
+        band carry every target's scale: their entries of the product are replaced by ``dval``, the scaled
+        value gradients of the survivor list; the elements below the threshold keep the plain product."""
         cfg = self.config
         L, F = cfg.num_layers, cfg.num_features
         tying = cfg.decoder_tying
@@ -341,6 +347,8 @@ class CrossLayerTranscoder(BaseTranscoder):
                 stacked_w = torch.cat([packed[i][:, :d] for i in slots], dim=1).unsqueeze(0)   # [1, F, n d]
                 stacked_g = torch.cat([g_model[t] for t in targets], dim=1).unsqueeze(0)       # [1, T, n d]
                 dact = engine.encode(stacked_g.contiguous(), stacked_w.contiguous(), None)[0]  # [T, F]
+            if dval is not None:
+                engine.scatter_survivor_values(surv, dval, s_, dact)
             engine.jumprelu_theta_grad(pre[s_], dact, theta[s_].contiguous(), self.theta_manager.bandwidth, out[s_], ws)
         # theta = exp(log_threshold): the reference casts theta to the model dtype for the forward
         return out * torch.exp(self.theta_manager.log_threshold.detach().float())

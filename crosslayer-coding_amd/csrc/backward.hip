@@ -13,7 +13,7 @@
 //   decoder db    db[t][:] = sum over tokens of g[t][token][:]
 //
 // Row vectors are spread over a wavefront in groups of four elements: lane l holds elements
-// c * 256 + 4 l .. + 3 of chunk c (NC4 chunks cover d <= 2048; d % 4 == 0).
+// c * 256 + 4 l .. + 3 of chunk c (NC4 chunks cover d <= 4096; d % 4 == 0).
 #include <type_traits>
 #include "adam.h"
 
@@ -990,7 +990,20 @@ __global__ void k_theta_grad_finish(const float *part, int64_t F, float *out) {
   }
 }
 
-static bool bw_shape_ok(int64_t d, int dtype) { return d > 0 && d % (dtype == CLT_BF16 ? 8 : 4) == 0 && d <= 2048; }
+// dense[tok][col[j]] = src[j] (rounded to the model dtype) for the survivors j of one layer's rows
+template <typename T>
+__global__ __launch_bounds__(BW_THREADS) void k_scatter_layer(const int32_t *row_ptr, const int32_t *col, const float *src,
+                                                               int64_t layer, int64_t Tn, int64_t F, T *dense) {
+  const int lane = lane_id(), wv = threadIdx.x >> 6, nwv = blockDim.x >> 6;
+  for (int64_t t = (int64_t)blockIdx.x * nwv + wv; t < Tn; t += (int64_t)gridDim.x * nwv) {
+    const int64_t r = layer * Tn + t;
+    T *row = dense + t * F;
+    for (int32_t j = row_ptr[r] + lane; j < row_ptr[r + 1]; j += 64) row[col[j]] = Elem<T>::from_f32(src[j]);
+  }
+}
+
+// rows of up to 4096 elements: 8 16-byte pieces per lane in bf16, up to 16 in fp32
+static bool bw_shape_ok(int64_t d, int dtype) { return d > 0 && d % (dtype == CLT_BF16 ? 8 : 4) == 0 && d <= 4096; }
 
 }  // namespace
 
@@ -1064,7 +1077,12 @@ extern "C" int clt_decode_backward_values(const int32_t *row_ptr, const int32_t 
   } while (0)
   if (dtype == CLT_BF16 && d == 768)
     k_bwd_values_sliced<bf16_t, 2, true><<<(unsigned)nblk, BW_THREADS, 0, s>>>(sptr, col, (const bf16_t *)w_packed, g, T, d, F, L, tying, nnz, part);
-  else if (dtype == CLT_BF16) CLT_BWV_N(bf16_t); else CLT_BWV_N(float);
+  else if (dtype == CLT_BF16) CLT_BWV_N(bf16_t);
+  else if (nc4 <= 8) CLT_BWV_N(float);
+  else if (nc4 <= 10) CLT_BWV(float, 10);      // fp32 rows beyond 2048 elements: a piece count that covers them
+  else if (nc4 <= 12) CLT_BWV(float, 12);
+  else if (nc4 <= 14) CLT_BWV(float, 14);
+  else CLT_BWV(float, 16);
 #undef CLT_BWV_N
 #undef CLT_BWV
   if (feat_scale && !val) return CLT_ERR_ARG;
@@ -1216,7 +1234,12 @@ extern "C" int clt_decoder_weight_grad(const int32_t *list_ptr, const int32_t *l
       k_feature_outer<bf16_t, bf16_t, 2, true, true><<<bw_resident_blocks(k_feature_outer<bf16_t, bf16_t, 2, true, true>), BW_THREADS, 0, s>>>(
           list_ptr, list_tok, list_src, (const bf16_t *)val, (const bf16_t *)g_model, dw_packed, nullptr, T, d, F, L, t, tying,
           (const bf16_t *)feat_offset, (const bf16_t *)feat_scale);
-  } else if (dtype == CLT_BF16) CLT_DW_N(bf16_t); else CLT_DW_N(float);
+  } else if (dtype == CLT_BF16) CLT_DW_N(bf16_t);
+  else if (nc4 <= 8) CLT_DW_N(float);
+  else if (nc4 <= 10) CLT_DW(float, 10);
+  else if (nc4 <= 12) CLT_DW(float, 12);
+  else if (nc4 <= 14) CLT_DW(float, 14);
+  else CLT_DW(float, 16);
 #undef CLT_DW_N
 #undef CLT_DW
   return clt_check_launch();
@@ -1252,7 +1275,11 @@ extern "C" int clt_decoder_weight_grad_adam(const int32_t *list_ptr, const int32
   } while (0)
   if (dtype == CLT_BF16 && d == 768) CLT_DWA(bf16_t, 2, true);
   else if (dtype == CLT_BF16) CLT_DWA_N(bf16_t);
-  else CLT_DWA_N(float);
+  else if (nc4 <= 8) CLT_DWA_N(float);
+  else if (nc4 <= 10) CLT_DWA(float, 10, false);
+  else if (nc4 <= 12) CLT_DWA(float, 12, false);
+  else if (nc4 <= 14) CLT_DWA(float, 14, false);
+  else CLT_DWA(float, 16, false);
 #undef CLT_DWA_N
 #undef CLT_DWA
   return clt_check_launch();
@@ -1285,9 +1312,26 @@ extern "C" int clt_encoder_weight_grad(const int32_t *list_ptr, const int32_t *l
     for (int64_t l = 0; l < L; ++l)
       k_feature_outer<bf16_t, float, 2, false, true><<<bw_resident_blocks(k_feature_outer<bf16_t, float, 2, false, true>), BW_THREADS, 0, s>>>(
           list_ptr, list_tok, list_src, dval, (const bf16_t *)x, dw_enc, db_enc, T, d, F, L, l, CLT_TYING_NONE);
-  } else if (dtype == CLT_BF16) CLT_EW_N(bf16_t); else CLT_EW_N(float);
+  } else if (dtype == CLT_BF16) CLT_EW_N(bf16_t);
+  else if (nc4 <= 8) CLT_EW_N(float);
+  else if (nc4 <= 10) CLT_EW(float, 10);
+  else if (nc4 <= 12) CLT_EW(float, 12);
+  else if (nc4 <= 14) CLT_EW(float, 14);
+  else CLT_EW(float, 16);
 #undef CLT_EW_N
 #undef CLT_EW
+  return clt_check_launch();
+}
+
+extern "C" int clt_scatter_survivor_values(const int32_t *row_ptr, const int32_t *col, const float *src, int64_t layer,
+                                           int64_t T, int64_t F, int64_t L, int dtype, void *dense, void *stream) {
+  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (T < 0 || F <= 0 || L <= 0 || layer < 0 || layer >= L) return CLT_ERR_ARG;
+  if (T == 0) return CLT_OK;
+  if (!row_ptr || !col || !src || !dense) return CLT_ERR_ARG;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == CLT_BF16) k_scatter_layer<bf16_t><<<256 * 8, BW_THREADS, 0, s>>>(row_ptr, col, src, layer, T, F, (bf16_t *)dense);
+  else k_scatter_layer<float><<<256 * 8, BW_THREADS, 0, s>>>(row_ptr, col, src, layer, T, F, (float *)dense);
   return clt_check_launch();
 }
 

@@ -724,6 +724,16 @@ def encoder_weight_grad(lists, dval: torch.Tensor, x: torch.Tensor, F: int):
     return dw, db
 
 
+def scatter_survivor_values(surv: SurvivorList, src: torch.Tensor, layer: int, dense: torch.Tensor) -> None:
+    """dense[tok, col] = src[j] for the survivors j of ``layer`` (decoder.py:228-285 with activations.py:183-220: the
+    kept activations' share of d loss / d activation behind a per-target feature scale)."""
+    assert dense.shape == (surv.T, surv.F) and dense.dtype == surv.dtype and dense.is_contiguous()
+    assert src.dtype == torch.float32 and src.numel() >= surv.col.numel()
+    code = nat.load().clt_scatter_survivor_values(nat.ptr(surv.row_ptr), nat.ptr(surv.col), nat.ptr(src), int(layer), surv.T,
+                                                  surv.F, surv.L, nat.dtype_code(surv.dtype), nat.ptr(dense), _stream(dense))
+    nat.check(code, "clt_scatter_survivor_values")
+
+
 def jumprelu_theta_grad(pre: torch.Tensor, grad_out: torch.Tensor, theta: torch.Tensor, bandwidth: float,
                         out: torch.Tensor, ws: Optional[Workspace] = None) -> None:
     """out [F] fp32 = gradient of one layer's JumpReLU thresholds from dense pre-activations and dense

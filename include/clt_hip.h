@@ -483,7 +483,7 @@ int clt_decoder_norms(const void *w_packed, void *norms, int64_t d, int64_t F,
  *   out [d][d] fp32, accumulate != 0 adds to out.
  * clt_encoder_weight_grad: dw_enc[s][f][:] = sum over the list of dval * x[s][token][:],
  *   db_enc[s][f] = sum of dval (fp32; x [L][T][d] in the model dtype).
- * Limits: d % 8 == 0 (bf16) / d % 4 == 0 (fp32) and d <= 2048.
+ * Limits: d % 8 == 0 (bf16) / d % 4 == 0 (fp32) and d <= 4096.
  */
 size_t clt_mse_workspace_bytes(int64_t T, int64_t d, int64_t L);
 int clt_mse_loss_grad(const void *rec, const void *target, int64_t T, int64_t d, int64_t L,
@@ -598,6 +598,18 @@ int clt_adam_step_decoders(void *const *w_refs_dev, void *const *w_refs_host, in
 int clt_adam_step_many(void *const *params_dev, const float *grad, float *m, float *v, int64_t count,
                        int64_t n, double lr, double beta1, double beta2, double eps, int64_t step,
                        int dtype, void *stream);
+
+/*
+ * dense[tok][col[j]] = src[j], rounded to the model dtype, for every survivor j of layer `layer`
+ * (rows layer*T .. layer*T + T - 1 of the list); the other elements of dense [T][F] are left as they
+ * are.  Used for the JumpReLU threshold gradient behind a per-target feature scale: at the kept
+ * activations d loss / d activation carries the scale of every target (the values of
+ * clt_decode_backward_values), elsewhere it is the plain product (clt/models/decoder.py:228-245,
+ * 268-285: the scale is applied to the non-zero activations only; clt/models/activations.py:183-220).
+ */
+int clt_scatter_survivor_values(const int32_t *row_ptr, const int32_t *col, const float *src,
+                                int64_t layer, int64_t T, int64_t F, int64_t L, int dtype,
+                                void *dense, void *stream);
 
 /* clt_jumprelu_theta_grad: gradient of the JumpReLU thresholds of one layer (JumpReLU.backward,
  *   clt/models/activations.py:196-199; bandwidth is 1.0 in ThetaManager, clt/models/theta.py:41):

@@ -211,10 +211,11 @@ def gradient_case(name, cfg_kw, seed, tokens=6):
             "targets": lists(targets), "loss": float(loss), "gradients": lists(grads)}
 
 
-def gradient_case_normalized(name, cfg_kw, seed, method, tokens=6):
+def gradient_case_normalized(name, cfg_kw, seed, method, tokens=6, stat_layers=None):
     """Loss and gradients with the de-normalisation of LossManager.compute_reconstruction_loss
     (clt/training/losses.py:70-86): target statistics as the trainer takes them from the activation store
-    ([1, d_model] per layer), or the 1 / sqrt(d_model) scaling."""
+    ([1, d_model] per layer), or the 1 / sqrt(d_model) scaling.  ``stat_layers``: only these layers have
+    statistics (the reference de-normalises those and leaves the others alone)."""
     cfg, model, g = build(cfg_kw, seed)
     model.train()
     L, d = cfg.num_layers, cfg.d_model
@@ -222,6 +223,9 @@ def gradient_case_normalized(name, cfg_kw, seed, method, tokens=6):
     targets = {l: torch.randn(tokens, d, generator=g) for l in range(L)}
     mean = {l: torch.randn(1, d, generator=g) * 0.5 for l in range(L)}
     std = {l: torch.rand(1, d, generator=g) + 0.5 for l in range(L)}
+    if stat_layers is not None:
+        mean = {l: v for l, v in mean.items() if l in stat_layers}
+        std = {l: v for l, v in std.items() if l in stat_layers}
     tc = TrainingConfig(learning_rate=1e-4, training_steps=10, activation_source="local_manifest",
                         activation_path="unused", normalization_method=method)
     lm = LossManager(tc, mean_tg=mean, std_tg=std, clt_config=cfg)
@@ -434,6 +438,15 @@ def sections():
         "gradients_normalized": lambda: [
             gradient_case_normalized("mean-std", dict(base, activation_fn="relu"), 35, "mean_std"),
             gradient_case_normalized("sqrt-d-model", dict(base, activation_fn="batchtopk", batchtopk_k=3), 36, "sqrt_d_model"),
+            gradient_case_normalized("mean-std-some-layers", dict(base, activation_fn="relu"), 44, "mean_std", stat_layers=(0, 2)),
+        ],
+        # the JumpReLU threshold gradient (activations.py:183-220) behind the per-target feature offset / scale
+        "gradients_jumprelu_affine": lambda: [
+            gradient_case("jumprelu-per-target-affine", dict(tied_affine, activation_fn="jumprelu", decoder_tying="per_target"), 45),
+            gradient_case("jumprelu-per-source-scale", dict(base, activation_fn="jumprelu", decoder_tying="per_source",
+                                                            enable_feature_scale=True), 46),
+            gradient_case("jumprelu-per-target-offset-skip", dict(base, activation_fn="jumprelu", decoder_tying="per_target",
+                                                                  enable_feature_offset=True, skip_connection=True), 47),
         ],
         # gradients through skip connections and the per-target feature offset / scale (decoder.py:228-338)
         "gradients_skip_affine": lambda: [

@@ -88,7 +88,7 @@ def test_oracle_theta_estimation_matches_the_reference(case):
     assert torch.allclose(torch.exp(log_theta), T(case["theta"]), rtol=1e-4, atol=1e-6)     # the method's return value
 
 
-@pytest.mark.parametrize("case", FIX["gradients"] + FIX["gradients_normalized"] + FIX["gradients_skip_affine"],
+@pytest.mark.parametrize("case", FIX["gradients"] + FIX["gradients_normalized"] + FIX["gradients_skip_affine"] + FIX["gradients_jumprelu_affine"],
                          ids=lambda c: c["name"])
 def test_oracle_gradients_match_the_reference(case):
     cfg, sd, L, tying, names, kw = unpack(case)

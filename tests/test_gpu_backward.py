@@ -50,6 +50,11 @@ def build(wl, dev):
     BASE.scaled("bw-per-target", decoder_tying="per_target"),
     BASE.scaled("bw-per-source-bf16", decoder_tying="per_source", dtype="bfloat16", num_layers=4),
     BASE.scaled("bw-per-target-split", decoder_tying="per_target", num_layers=3, d_model=200, num_features=256, tokens=4096, k=6),
+    # rows beyond 2048 elements (up to 4096: eight 16-byte pieces per lane in bf16, up to sixteen in fp32)
+    BASE.scaled("bw-d4096-bf16", num_layers=2, d_model=4096, num_features=256, tokens=96, k=8, dtype="bfloat16"),
+    BASE.scaled("bw-d2304-f32", num_layers=2, d_model=2304, num_features=256, tokens=64, k=8),
+    BASE.scaled("bw-d4096-f32-jump", num_layers=2, d_model=4096, num_features=256, tokens=64, activation_fn="jumprelu", k=None),
+    BASE.scaled("bw-d3072-f32-per-source", num_layers=2, d_model=3072, num_features=128, tokens=64, k=6, decoder_tying="per_source"),
 ], ids=lambda w: w.name)
 def test_loss_and_gradients_match_autograd(dev, wl):
     dtype = getattr(torch, wl.dtype)

@@ -90,7 +90,7 @@ def test_theta_estimation_matches_the_reference(dev, case):
     assert torch.allclose(model.log_threshold.detach().cpu().float(), T(case["log_threshold_after"]), rtol=1e-4, atol=1e-5)
 
 
-@pytest.mark.parametrize("case", FIX["gradients"] + FIX["gradients_normalized"] + FIX["gradients_skip_affine"],
+@pytest.mark.parametrize("case", FIX["gradients"] + FIX["gradients_normalized"] + FIX["gradients_skip_affine"] + FIX["gradients_jumprelu_affine"],
                          ids=lambda c: c["name"])
 def test_gradients_match_the_reference(dev, case):
     model = load_model(case, dev)
