@@ -692,6 +692,15 @@ class CrossLayerTranscoder(BaseTranscoder):
                 recs[t] = torch.zeros((rows, d), device=self.device, dtype=self.dtype)
         return recs
 
+    # ---- parameters that an optimiser step may have left behind the kernels' working copy ------------------
+    def named_parameters(self, *args, **kwargs):
+        self.decoder_module.sync_parameters()
+        return super().named_parameters(*args, **kwargs)
+
+    def _apply(self, fn, *args, **kwargs):
+        self.decoder_module.sync_parameters()
+        return super()._apply(fn, *args, **kwargs)
+
     # ---- checkpoints -----------------------------------------------------------------------
     def load_state_dict(self, state_dict: Dict[str, torch.Tensor], strict: bool = True):
         """nn.Module.load_state_dict plus the reference's migrations (clt.py:347-425): an untied

@@ -45,6 +45,49 @@ def merge_layer_lists(parts: List[Tuple[int, SurvivorList]], L: int, T: int, F: 
     return SurvivorList(row_ptr, col, val, T, F, L, dtype)
 
 
+class _SyncedModuleDict(nn.ModuleDict):
+    """The decoders by key.  Reading an entry first brings the checkpoint-layout parameters up to date when an
+    optimiser step has left them behind the feature-major working copy (``Decoder.sync_parameters``)."""
+
+    def _sync(self):
+        owner = self.__dict__.get("_owner")
+        if owner is not None and owner() is not None:
+            owner().sync_parameters()
+
+    def __getitem__(self, key):
+        self._sync()
+        return super().__getitem__(key)
+
+    def __iter__(self):
+        self._sync()
+        return super().__iter__()
+
+    def values(self):
+        self._sync()
+        return super().values()
+
+    def items(self):
+        self._sync()
+        return super().items()
+
+
+class _SyncedModuleList(nn.ModuleList):
+    """Same for tied decoders (a list)."""
+
+    def _sync(self):
+        owner = self.__dict__.get("_owner")
+        if owner is not None and owner() is not None:
+            owner().sync_parameters()
+
+    def __getitem__(self, idx):
+        self._sync()
+        return super().__getitem__(idx)
+
+    def __iter__(self):
+        self._sync()
+        return super().__iter__()
+
+
 class Decoder(nn.Module):
     def __init__(self, config, process_group, device: torch.device, dtype: torch.dtype):
         super().__init__()
@@ -61,13 +104,20 @@ class Decoder(nn.Module):
             return RowParallelLinear(F, d, bias=True, process_group=process_group, d_model_for_init=d,
                                      num_layers_for_init=L, device=device, dtype=dtype)
 
+        # the optimiser's in-kernel decoder step updates the feature-major working copy only and leaves the
+        # checkpoint-layout parameters behind until something reads them (sync_parameters)
+        self._params_behind = False
+        self._sync_table = None
         if tied:
-            self.decoders = nn.ModuleList(make() for _ in range(L))
+            self.decoders = _SyncedModuleList(make() for _ in range(L))
             for dec in self.decoders:  # tied decoders start at zero (decoder.py:80-86)
                 nn.init.zeros_(dec.weight)
                 nn.init.zeros_(dec.bias_param)
         else:
-            self.decoders = nn.ModuleDict({f"{s}->{t}": make() for s in range(L) for t in range(s, L)})
+            self.decoders = _SyncedModuleDict({f"{s}->{t}": make() for s in range(L) for t in range(s, L)})
+        import weakref
+        self.decoders.__dict__["_owner"] = weakref.ref(self)
+        self.register_state_dict_pre_hook(lambda module, prefix, keep_vars: module.sync_parameters())
 
         def square():
             return nn.Parameter(torch.zeros(d, d, device=device, dtype=dtype))
@@ -105,10 +155,40 @@ class Decoder(nn.Module):
     # ---- decoder bookkeeping -------------------------------------------------------
     def _ordered(self) -> List[RowParallelLinear]:
         """Decoder layers in slot order (untied: "0->0", "0->1", ..., as created)."""
+        mods = self.decoders._modules      # straight to the registry: no parameter sync for internal walks
         if isinstance(self.decoders, nn.ModuleDict):
             L = self.config.num_layers
-            return [self.decoders[f"{s}->{t}"] for s in range(L) for t in range(s, L)]
-        return list(self.decoders)
+            return [mods[f"{s}->{t}"] for s in range(L) for t in range(s, L)]
+        return list(mods.values())
+
+    # ---- parameters behind the working copy -------------------------------------------
+    def mark_parameters_behind(self) -> None:
+        """The feature-major slab now holds newer decoder weights than the checkpoint-layout parameters."""
+        self._params_behind = True
+
+    def sync_parameters(self) -> None:
+        """Rewrite the checkpoint-layout decoder weights [d, F] from the feature-major slab when a step has left
+        them behind.  Runs by itself before anything hands the parameters out: ``state_dict``,
+        ``parameters`` / ``named_parameters``, ``decoders[key]``, ``.to(...)``."""
+        if not self._params_behind:
+            return
+        self._params_behind = False
+        import ctypes
+        ws = [lin.weight.data for lin in self._ordered()]
+        ptrs = tuple(w.data_ptr() for w in ws)
+        if self._sync_table is None or self._sync_table[0] != ptrs:
+            self._sync_table = (ptrs, torch.tensor(ptrs, dtype=torch.int64, device=ws[0].device),
+                                (ctypes.c_void_p * len(ptrs))(*ptrs))
+        d, F = ws[0].shape
+        engine.unpack_decoders(self._slab, self._sync_table[1], self._sync_table[2], d, F)
+
+    def named_parameters(self, *args, **kwargs):
+        self.sync_parameters()
+        return super().named_parameters(*args, **kwargs)
+
+    def _apply(self, fn, *args, **kwargs):
+        self.sync_parameters()
+        return super()._apply(fn, *args, **kwargs)
 
     def _slots(self) -> List[Tuple[int, int]]:
         """(source, target) fed by each slot; tied decoders report (i, i)."""
@@ -145,6 +225,7 @@ class Decoder(nn.Module):
     def invalidate_packed(self) -> None:
         """Force a repack on next use (needed only after writes that bypass autograd
         version counting, e.g. through ``.data``)."""
+        self._params_behind = False        # the parameters are what counts from here on
         self._slab_keys = [None] * len(self._slab_keys)
         self._bias_cache.clear()
         self._cached_decoder_norms = None
@@ -268,7 +349,7 @@ class Decoder(nn.Module):
                 if not started:
                     engine.accumulate_dense(surv, -1, acc, True)
                     started = True
-            lin = self.decoders[t]
+            lin = self.decoders[t]          # (brings the parameters up to date if a step left them behind)
             engine.encode(acc.unsqueeze(0), lin.weight.detach().unsqueeze(0), lin.bias_param.detach().unsqueeze(0),
                           out=out[t].unsqueeze(0))
 

@@ -25,6 +25,9 @@ class CLTAdam:
         self.step_count = 0
         self.fuse_decoder_step = True    # untied decoders: Adam inside the weight-gradient kernel (training_step)
         self.tile_decoder_step = True    # ... over column tiles, when the shape allows (moments and a weight copy tiled)
+        # the in-kernel decoder step rewrites the feature-major slab only; the checkpoint-layout parameters follow
+        # when something reads them (Decoder.sync_parameters).  False: rewrite them in every step
+        self.defer_parameter_sync = True
         self._dec_layout = "rows"        # layout of state["dec_w"]: "rows" [n_dec, F, d] or "tiles" [n_dec, d // CS, F, CS]
         self._w_tiles = None             # tiled copy of the decoder weights, valid while _w_tiles_gen matches the slab
         self._w_tiles_gen = None
@@ -125,14 +128,21 @@ class CLTAdam:
             m_w, v_w = self.state["dec_w"]
             engine.decoder_weight_grad_adam_tiled(lists, surv, g_model, self._w_tiles, m_w, v_w, self.lr, self.betas,
                                                   self.eps, self.step_count + 1, ws=self.model._workspace())
-            engine.untile_decoders(self._w_tiles, packed, w_dev, w_host)
+            if self.defer_parameter_sync:
+                engine.untile_decoders(self._w_tiles, packed)
+                dec.mark_parameters_behind()
+            else:
+                engine.untile_decoders(self._w_tiles, packed, w_dev, w_host)
             return
         self._decoder_moments_to("rows")
         self._w_tiles_gen = None
         m_w, v_w = self.state["dec_w"]
         engine.decoder_weight_grad_adam(lists, surv, g_model, packed, m_w, v_w, self.lr, self.betas, self.eps,
                                         self.step_count + 1)
-        engine.unpack_decoders(packed, w_dev, w_host, d, F)
+        if self.defer_parameter_sync:
+            dec.mark_parameters_behind()
+        else:
+            engine.unpack_decoders(packed, w_dev, w_host, d, F)
 
     @torch.no_grad()
     def step(self, raw) -> None:
@@ -157,6 +167,7 @@ class CLTAdam:
         assert all(b.is_contiguous() and b.numel() == bs[0].numel() and b.dtype == bs[0].dtype for b in bs)
         d, F = ws[0].shape
         if raw["dec_w"] is not None:
+            dec.sync_parameters()         # the two-copy kernel below reads neither copy's old value from the other
             self._decoder_moments_to("rows")
             self._w_tiles_gen = None      # the slab is about to change under the tiled copy
             m_w, v_w = self.state["dec_w"]

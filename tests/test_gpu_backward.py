@@ -345,6 +345,53 @@ def test_optimiser_moves_between_the_tiled_and_the_row_route(dev):
     _assert_same_training((None, runs[0][0], None, runs[0][1]), (None, runs[1][0], None, runs[1][1]), torch.bfloat16, 4)
 
 
+@pytest.mark.parametrize("tiled", [True, False], ids=["tile-route", "row-route"])
+def test_parameters_left_behind_by_the_decoder_step_are_current_whenever_they_are_read(dev, tiled):
+    # The in-kernel decoder step rewrites the feature-major slab only; the checkpoint-layout parameters [d, F]
+    # follow when something reads them.  Against an optimiser that rewrites them in every step
+    # (trainer.py:751-778: the reference's parameters are always current): state_dict(), named_parameters(),
+    # decoders[key] and the forward must all see the same bits.
+    import crosslayer_coding_amd as cca
+    wl = BASE.scaled("bw-lazy", num_layers=3, d_model=128, num_features=256, tokens=256, dtype="bfloat16", k=10)
+    models, opts = [], []
+    for defer in (True, False):
+        model, sd, x, targets = build(wl, dev)
+        opt = cca.CLTAdam(model, lr=1e-2)
+        opt.defer_parameter_sync, opt.tile_decoder_step = defer, tiled
+        models.append(model); opts.append(opt)
+    inputs = {l: x[l].to(dev) for l in range(3)}
+    tg = {l: t.to(dev) for l, t in targets.items()}
+    lazy, eager = models
+    for step in range(3):
+        for m, o in zip(models, opts):
+            m.training_step(inputs, tg, o)
+        assert opts[0]._dec_layout == ("tiles" if tiled else "rows")
+        dec = lazy.decoder_module
+        assert dec._params_behind and not eager.decoder_module._params_behind
+        raw = dec.decoders._modules["0->1"].weight.detach().clone()      # the registry itself: no sync
+        want = eager.decoder_module.decoders["0->1"].weight.detach()
+        assert not torch.equal(raw, want)                                 # really behind ...
+        if step == 0:
+            got = dec.decoders["0->1"].weight.detach()                    # ... until an entry is read
+        elif step == 1:
+            got = dict(lazy.named_parameters())["decoder_module.decoders.0->1.weight"].detach()
+        else:
+            got = lazy.state_dict()["decoder_module.decoders.0->1.weight"]
+        assert not dec._params_behind and torch.equal(got, want)
+        # the forward never depended on them
+        a, b = lazy(inputs), eager(inputs)
+        assert all(torch.equal(a[t], b[t]) for t in a)
+    sa, sb = lazy.state_dict(), eager.state_dict()
+    assert set(sa) == set(sb) and all(torch.equal(sa[k], sb[k]) for k in sa)
+    # loading a checkpoint makes the parameters the truth again
+    lazy.training_step(inputs, tg, opts[0])
+    assert lazy.decoder_module._params_behind
+    lazy.load_state_dict(sb)
+    assert not lazy.decoder_module._params_behind
+    a, b = lazy(inputs), eager(inputs)
+    assert all(torch.equal(a[t], b[t]) for t in a)
+
+
 def test_tied_decoders_do_not_fuse_the_step(dev):
     import crosslayer_coding_amd as cca
     wl = BASE.scaled("bw-nofuse", num_layers=2, d_model=64, num_features=128, tokens=64, decoder_tying="per_source")

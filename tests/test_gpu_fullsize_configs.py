@@ -389,5 +389,38 @@ def test_c4_training_step_at_full_size_in_bf16(dev):
         assert float(moved) > 0.0                                     # the step did change bf16 values
     # the feature-major working copy of the decoder follows its parameter
     assert torch.equal(model.decoder_module.packed()[slot][:, :d], after["dec"].t())
-    del model, inputs, raw, opt
+    del raw, opt, before, after, g_ref
+    _free()
+
+    # The route training_step takes at this size (what `bench.py --train-step` times): the untied decoder weights
+    # take their Adam step inside the column-tile weight-gradient kernel (d = 768: 48 column slices, T * 32 B =
+    # 128 KB filling the LDS).  Three decoder pairs against torch.optim.Adam on separately computed gradients.
+    pairs = [(0, 0), (3, 7), (L - 1, L - 1)]
+    slot_of = lambda s_, t_: s_ * L - (s_ * (s_ - 1)) // 2 + (t_ - s_)  # noqa: E731
+    loss_l, raw = model._loss_and_raw_gradients(inputs, targets)
+    want_loss = float(loss_l.sum())
+    kept = {k_: raw["dec_w"][slot_of(*k_)].t().contiguous().clone() for k_ in pairs}
+    del raw
+    _free()
+    before = {k_: model.decoder_module.decoders[f"{k_[0]}->{k_[1]}"].weight.detach().float().clone() for k_ in pairs}
+    opt = cca.CLTAdam(model, lr=1e-4, betas=(0.9, 0.999))
+    assert opt.fuses_decoder_step() and engine.decoder_tile_width(T, d, F, torch.bfloat16) > 0
+    loss0 = float(model.training_step(inputs, targets, opt))
+    assert abs(loss0 - want_loss) <= 1e-5 * want_loss
+    assert opt._dec_layout == "tiles"
+    assert model.decoder_module._params_behind            # the parameters follow when they are read (below)
+    for (s_, t_) in pairs:
+        p = torch.nn.Parameter(before[(s_, t_)].clone())
+        p.grad = kept[(s_, t_)]
+        torch.optim.Adam([p], lr=1e-4, betas=(0.9, 0.999), eps=1e-8).step()
+        want = p.detach().to(torch.bfloat16)
+        got = model.decoder_module.decoders[f"{s_}->{t_}"].weight.detach()
+        same = (got.view(torch.int16) == want.view(torch.int16)).float().mean()
+        assert float(same) >= 0.99, (s_, t_, float(same))
+        assert orc.rel_l2(got.float().cpu(), want.float().cpu()) <= 1e-3
+        assert float((got.float() != before[(s_, t_)]).float().mean()) > 0.1
+        assert torch.equal(model.decoder_module.packed()[slot_of(s_, t_)][:, :d], got.t())
+    loss1, _ = model._loss_and_raw_gradients(inputs, targets)
+    assert float(loss1.sum()) < loss0
+    del model, inputs, opt, before, kept
     _free()
