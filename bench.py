@@ -64,29 +64,35 @@ def profiled_traffic(workload: str):
     return table, forwards
 
 
-def gather_yardstick(lib, dev, table_bytes: int, row_bytes: int, steps: int = 3):
-    """GB/s of a bare gather of ``row_bytes`` rows from a table of ``table_bytes`` (the piece of a decoder
-    matrix one XCD works on), best of four grid sizes: what the L2 -> CU path delivers to this access
-    pattern on the GPU at hand, with no survivor lists, partial rows or arithmetic around it."""
+def gather_yardstick(lib, dev, table_bytes: int, row_bytes: int, steps: int = 5, reps: int = 4):
+    """(GB/s, spread) of a bare gather of ``row_bytes`` rows from a table of ``table_bytes`` (the piece of a
+    decoder matrix one XCD works on): what the L2 -> CU path delivers to this access pattern on the GPU at
+    hand, with no survivor lists, partial rows or arithmetic around it.  Four grid sizes, each timed ``reps``
+    times over ``steps`` launches after a warm-up; the figure is the best run of the best grid size, and
+    ``spread`` = (lowest, highest) of that grid size's runs - how far the yardstick itself moves."""
     n_rows = max(1, table_bytes // row_bytes)
     n_idx = 4_000_000 * 1536 // row_bytes
     g = torch.Generator(device=dev).manual_seed(0)
     table = torch.randint(0, 1 << 30, (n_rows * row_bytes // 4,), dtype=torch.int32, device=dev, generator=g)
     idx = torch.randint(0, n_rows, (n_idx,), dtype=torch.int32, device=dev, generator=g)
     stream = torch.cuda.current_stream().cuda_stream
-    best = 0.0
+    best, spread = 0.0, (0.0, 0.0)
     for blocks in (256 * 2, 256 * 4, 256 * 8, 256 * 16):
         out = torch.empty(blocks * 256, dtype=torch.float32, device=dev)
         if lib.clt_probe_gather(table.data_ptr(), n_rows, row_bytes, idx.data_ptr(), n_idx, blocks, 0, out.data_ptr(), stream):
-            return None
-        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        a.record()
-        for _ in range(steps):
-            lib.clt_probe_gather(table.data_ptr(), n_rows, row_bytes, idx.data_ptr(), n_idx, blocks, 0, out.data_ptr(), stream)
-        b.record()
-        b.synchronize()
-        best = max(best, n_idx * row_bytes * steps / (a.elapsed_time(b) * 1e-3) / 1e9)
-    return best
+            return None, None
+        runs = []
+        for _ in range(reps):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(steps):
+                lib.clt_probe_gather(table.data_ptr(), n_rows, row_bytes, idx.data_ptr(), n_idx, blocks, 0, out.data_ptr(), stream)
+            b.record()
+            b.synchronize()
+            runs.append(n_idx * row_bytes * steps / (a.elapsed_time(b) * 1e-3) / 1e9)
+        if max(runs) > best:
+            best, spread = max(runs), (min(runs), max(runs))
+    return best, spread
 
 
 def copy_probe(dev):
@@ -224,7 +230,7 @@ def run_gpu(args):
         else:
             part_bytes = F * d * e
         row_bytes = min(d * e, 2048) // 16 * 16
-        yard = gather_yardstick(nat.load(), dev, part_bytes, row_bytes) if row_bytes >= 16 else None
+        yard, yard_spread = gather_yardstick(nat.load(), dev, part_bytes, row_bytes) if row_bytes >= 16 else (None, None)
         per_launch_s = st["decode"] / n_dec_launch * 1e-3
         hit = [v for k, v in table.items() if k.startswith(kname + "<")]
         traffic = hit[0][1] if hit else None
@@ -235,9 +241,14 @@ def run_gpu(args):
             "bound": "l2_gather (measured)",
             "achieved": dec_gbs,
             "peak": yard,
+            "peak_spread": yard_spread,
             "unit": "GB/s",
             "frac": (dec_gbs / yard) if yard else None,
             "traffic": traffic,
+            # the same launch against the published HBM peak (8 TB/s): on the bytes that must come from HBM at
+            # least once, and on the HBM traffic the counters measured
+            "hbm_compulsory_frac": dec_c_gbs / HBM_PEAK_GBS,
+            "hbm_traffic_frac": (traffic / per_launch_s / 1e9 / HBM_PEAK_GBS) if traffic else None,
             "hbm": {"peak": HBM_PEAK_GBS, "compulsory_bytes_per_launch": comp, "compulsory_GBps": dec_c_gbs,
                     "compulsory_frac": dec_c_gbs / HBM_PEAK_GBS,
                     "traffic_GBps": (traffic / per_launch_s / 1e9) if traffic else None,
@@ -601,7 +612,7 @@ def run_backward(args):
     # them from the L2: it is priced against what a bare gather of such rows from such a table reaches on
     # this GPU, measured now; what has to cross the HBM interface (the fp32 gradient written once, the
     # gradient slab and the lists read once) is the second figure.
-    yard = gather_yardstick(cca._native.load(build_if_missing=False), dev, wl.tokens * d * esz, d * esz)
+    yard, _ = gather_yardstick(cca._native.load(build_if_missing=False), dev, wl.tokens * d * esz, d * esz)
     # per decoder element the fp32 gradient written once - or, with the step in place, both moments and the packed
     # copy read and written and the parameter rewritten from the copy
     hbm_bytes = pairs * F * d * ((16 + 4 * esz) if fused else 4) + L * wl.tokens * d * esz + surv.nnz * (8 + esz)

@@ -115,7 +115,6 @@ class Decoder(nn.Module):
                 nn.init.zeros_(dec.bias_param)
         else:
             self.decoders = _SyncedModuleDict({f"{s}->{t}": make() for s in range(L) for t in range(s, L)})
-        import weakref
         self.decoders.__dict__["_owner"] = weakref.ref(self)
         self.register_state_dict_pre_hook(lambda module, prefix, keep_vars: module.sync_parameters())
 
@@ -278,11 +277,60 @@ class Decoder(nn.Module):
         return engine.encode(x, w_skip.detach().unsqueeze(0).contiguous(), None)[0].float()
 
     # ---- fused path ------------------------------------------------------------------
-    # Rates behind the choice between the two decode routes, measured on an MI355X: the row gather of
-    # clt_decode_sparse delivers about 14.5 TB/s of decoder rows whatever the shape; the MFMA kernel
-    # sustains about 1.0 PFLOP/s in bf16 (0.1 in fp32) on [T, F] x [F, d] products with F >= 16384.
-    GATHER_BYTES_PER_S = 14.5e12
-    MFMA_FLOPS_PER_S = {torch.bfloat16: 1.0e15, torch.float32: 1.0e14}
+    # Rates behind the choice between the two decode routes.  Both are measured on the GPU at hand, once per
+    # process and shape (``route_rates``): the matrix-core kernel on the very product the dense route would
+    # run, and a bare gather of decoder rows from a table the size of one L2 (clt_probe_gather), of which the
+    # sparse decode - survivor lists, partial rows and arithmetic around the same loads - delivers a fraction.
+    GATHER_EFFICIENCY = 0.62          # sparse decode / bare gather, see bench.py's roofline.frac (0.60 - 0.67)
+    _rate_cache: Dict[tuple, Tuple[float, float]] = {}
+    rate_override: Optional[Tuple[float, float]] = None     # (gather bytes / s, MFMA flop / s): tests and experiments
+
+    def route_rates(self, T: int, F: int, d: int, dtype: torch.dtype) -> Tuple[float, float]:
+        """(bytes / s of decoder rows the row gather delivers, flop / s of the dense product [T, F] x [F, d])."""
+        if self.rate_override is not None:
+            return self.rate_override
+        dev = self._ordered()[0].weight.device
+        key = (dev.index, T, F, d, dtype)
+        hit = Decoder._rate_cache.get(key)
+        if hit is not None:
+            return hit
+
+        def best_of(fn, reps=3):
+            fn()
+            best = float("inf")
+            for _ in range(reps):
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+                fn()
+                b.record()
+                b.synchronize()
+                best = min(best, a.elapsed_time(b) * 1e-3)
+            return best
+
+        esize = 2 if dtype == torch.bfloat16 else 4
+        # the dense product itself, on scratch operands of the real shape
+        x = torch.zeros((1, T, F), dtype=dtype, device=dev)
+        w = torch.zeros((1, d, F), dtype=dtype, device=dev)
+        out = torch.empty((1, T, d), dtype=dtype, device=dev)
+        mfma = 2.0 * T * F * d / best_of(lambda: engine.encode(x, w, None, out=out))
+        del x, w, out
+        # a bare gather of rows of this width from 4 MB (what an XCD's L2 holds of a decoder matrix)
+        row_bytes = max(16, min(d * esize, 2048) // 16 * 16)
+        n_rows = max(1, (4 << 20) // row_bytes)
+        n_idx = max(1, (1 << 30) // row_bytes)
+        g = torch.Generator(device=dev).manual_seed(0)
+        table = torch.randint(0, 1 << 30, (n_rows * row_bytes // 4,), dtype=torch.int32, device=dev, generator=g)
+        idx = torch.randint(0, n_rows, (n_idx,), dtype=torch.int32, device=dev, generator=g)
+        sink = torch.empty(256 * 8 * 256, dtype=torch.float32, device=dev)
+        lib, stream = nat.load(), nat.current_stream(dev)
+
+        def probe():
+            nat.check(lib.clt_probe_gather(table.data_ptr(), n_rows, row_bytes, idx.data_ptr(), n_idx, 256 * 8, 0,
+                                           sink.data_ptr(), stream), "clt_probe_gather")
+
+        gather = self.GATHER_EFFICIENCY * n_idx * row_bytes / best_of(probe)
+        Decoder._rate_cache[key] = (gather, mfma)
+        return gather, mfma
 
     def dense_split(self, surv: SurvivorList, src_mask: int, t_begin: int, t_end: int,
                     skip_add: Optional[torch.Tensor]) -> int:
@@ -292,7 +340,7 @@ class Decoder(nn.Module):
         (decoder.py:208-251), so target t gathers (t + 1) k T decoder rows of d elements from one matrix:
         with every further source the gather grows and the dense product ``summed [T, F] @ W[t].T`` does
         not.  The dense route is taken from the first target on for which
-        ``2 T F d / MFMA rate < rows gathered x d x element size / gather rate``.  Untied and per-source
+        ``2 T F d / MFMA rate < rows gathered x d x element size / gather rate`` (``route_rates``).  Untied and per-source
         decoders never qualify: each (source, target) pair has its own operand or its own matrix, so the
         dense cost is the reference's full 2 T F d per pair against k T rows per pair."""
         cfg = self.config
@@ -300,11 +348,11 @@ class Decoder(nn.Module):
             return t_end
         T, F, d = surv.T, surv.F, cfg.d_model
         esize = 2 if surv.dtype == torch.bfloat16 else 4
-        rate = self.MFMA_FLOPS_PER_S.get(surv.dtype)
         # shapes the MFMA kernel of clt_encode takes (K = F in whole pairs of 128-byte stages, 256 x 256 tiles)
-        if rate is None or T < 256 or d < 256 or d % 4 or F % (256 // esize):
+        if surv.dtype not in (torch.bfloat16, torch.float32) or T < 256 or d < 256 or d % 4 or F % (256 // esize):
             return t_end
-        dense_s = 2.0 * T * F * d / rate
+        gather_rate, mfma_rate = self.route_rates(T, F, d, surv.dtype)
+        dense_s = 2.0 * T * F * d / mfma_rate
         # survivors of one source layer, from a host-side figure: the exact total where the list was sized from
         # it, else the last total seen for the shape; a threshold list whose total is not known yet is priced
         # at 2 % density (its arrays are sized for the largest list, which says nothing about the batch)
@@ -315,7 +363,7 @@ class Decoder(nn.Module):
         n_src = 0
         for t in range(t_end):
             n_src += (src_mask >> t) & 1
-            if t >= t_begin and n_src * per_layer * d * esize / self.GATHER_BYTES_PER_S > dense_s:
+            if t >= t_begin and n_src * per_layer * d * esize / gather_rate > dense_s:
                 return t
         return t_end
 

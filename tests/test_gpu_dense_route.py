@@ -63,6 +63,8 @@ def test_dense_route_matches_the_oracle_and_the_gather_route(dev, dtype, affine)
     model = cca.CrossLayerTranscoder(cfg, None, dev)
     model.load_state_dict(sd)
     inputs = {l: x[l].to(dev) for l in range(L)}
+    # rates of a large shape: at this size the measured ones would (rightly) keep every target on the gather
+    model.decoder_module.rate_override = (14.5e12, 1.0e15 if tdt == torch.bfloat16 else 1.0e14)
     dense = model(inputs)
     route = dict(model.decoder_module.last_route)
     assert route["dense_targets"][0] < route["dense_targets"][1] == L      # the dense route was taken
@@ -87,6 +89,43 @@ def test_dense_route_matches_the_oracle_and_the_gather_route(dev, dtype, affine)
     want = model({l: inputs[l] for l in (0, 2, 3)})
     for t in part:
         assert orc.rel_l2(part[t].float().cpu(), want[t].float().cpu()) <= TOL[tdt]
+
+
+def test_dense_split_follows_the_measured_rates(dev):
+    # The split between the row gather and the dense product is decided from rates measured on this GPU
+    # (Decoder.route_rates: the product itself on the matrix cores, a bare row gather), cached per shape;
+    # with the two rates swapped the decision flips.
+    wl = synth.Workload("dense-split", 7, 6, 512, 4096, 1024, "bfloat16", k=64, decoder_tying="per_target")
+    model = cca.CrossLayerTranscoder(wl.config(), None, dev)
+    dec = model.decoder_module
+    L, T, F, d = wl.num_layers, wl.tokens, wl.num_features, wl.d_model
+    gather, mfma = dec.route_rates(T, F, d, torch.bfloat16)
+    assert 1e12 < gather < 4e13 and 5e13 < mfma < 2.5e15, (gather, mfma)        # plausible for one MI355X
+    assert dec.route_rates(T, F, d, torch.bfloat16) == (gather, mfma)           # cached: measured once
+    total = L * wl.k * T
+    surv = engine.SurvivorList(torch.zeros(L * T + 1, dtype=torch.int32, device=dev),
+                               torch.zeros(total, dtype=torch.int32, device=dev),
+                               torch.zeros(total, dtype=torch.bfloat16, device=dev), T, F, L, torch.bfloat16, None, total)
+    mask = (1 << L) - 1
+
+    def first_dense(rates):
+        dec.rate_override = rates
+        return dec.dense_split(surv, mask, 0, L, None)
+
+    # target t gathers (t + 1) k T rows of d elements; the product costs 2 T F d whatever t is
+    def expected(g_rate, m_rate):
+        for t in range(L):
+            if (t + 1) * wl.k * T * d * 2 / g_rate > 2.0 * T * F * d / m_rate:
+                return t
+        return L
+
+    for rates in ((gather, mfma), (1e12, 1e15), (1e15, 1e12), (mfma, gather)):
+        assert first_dense(rates) == expected(*rates), rates
+    assert first_dense((1e12, 1e15)) == 0 and first_dense((1e15, 1e12)) == L      # the decision flips with the rates
+    dec.rate_override = None
+    assert dec.dense_split(surv, mask, 0, L, None) == expected(gather, mfma)
+    dec.dense_route = False
+    assert dec.dense_split(surv, mask, 0, L, None) == L
 
 
 def test_route_query_names_the_schedules(dev):
