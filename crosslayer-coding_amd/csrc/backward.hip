@@ -1154,7 +1154,7 @@ extern "C" int clt_feature_lists(const int32_t *row_ptr, const int32_t *col, int
                                  size_t workspace_bytes, void *stream) {
   if (T <= 0 || F <= 0 || L <= 0 || L > 65535 || !row_ptr || !list_ptr || !workspace) return CLT_ERR_ARG;
   if ((double)L * (double)F >= 2147483647.0) return CLT_ERR_RANGE;
-  if (T > 65536) return CLT_ERR_RANGE;    // the token bitmaps of a workgroup's four wavefronts take T bytes of LDS
+  if (T > 262144) return CLT_ERR_RANGE;   // a wavefront's two token bitmaps take T / 4 bytes of LDS (64 KB here)
   if (workspace_bytes < clt_feature_lists_workspace_bytes(F, L)) return CLT_ERR_WORKSPACE;
   if ((((uintptr_t)workspace) & 7u) != 0) return CLT_ERR_ALIGN;
   hipStream_t s = (hipStream_t)stream;
@@ -1198,8 +1198,10 @@ extern "C" int clt_feature_lists(const int32_t *row_ptr, const int32_t *col, int
   if (list_tok && list_src) {
     k_csc_fill<<<nb, BW_THREADS, 0, s>>>(row_ptr, col, T, F, L, list_ptr, cnt, list_tok, list_src);
     const int bm_words = (int)clt_ceil_div(T, 32);
-    k_csc_order<<<nb, BW_THREADS, (size_t)(BW_THREADS / 64) * 2 * bm_words * 4, s>>>(list_ptr, n, list_tok, list_src, row_ptr, col,
-                                                                                   T, F, bm_words);
+    // as many wavefronts per workgroup as have room for their bitmaps in 64 KB: four up to 65536 tokens
+    const int order_waves = T <= 65536 ? 4 : T <= 131072 ? 2 : 1;
+    k_csc_order<<<nb, order_waves * 64, (size_t)order_waves * 2 * bm_words * 4, s>>>(list_ptr, n, list_tok, list_src, row_ptr, col,
+                                                                                     T, F, bm_words);
   }
   return clt_check_launch();
 }

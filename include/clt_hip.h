@@ -463,7 +463,7 @@ int clt_decoder_norms(const void *w_packed, void *norms, int64_t d, int64_t F,
  *   number of entries col holds, so that no total has to be read back.
  * clt_feature_lists: the survivor list regrouped by (layer, feature): list_ptr [L*F+1],
  *   list_tok [nnz] token of each entry, list_src [nnz] its position in col / val.  Every
- *   list is in ascending token order, so sums over a list always run in the same order (T <= 65536).
+ *   list is in ascending token order, so sums over a list always run in the same order (T <= 262144).
  *   Pass list_tok = list_src = NULL to get the counts only.
  * clt_decoder_weight_grad: dw_packed[slot(s,t)][f][:] = sum over the list of (s, f) of
  *   val * g_model[t][token][:] (fp32 sums, feature-major, dense rows of d elements); with tied decoders the

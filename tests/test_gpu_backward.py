@@ -55,6 +55,8 @@ def build(wl, dev):
     BASE.scaled("bw-d2304-f32", num_layers=2, d_model=2304, num_features=256, tokens=64, k=8),
     BASE.scaled("bw-d4096-f32-jump", num_layers=2, d_model=4096, num_features=256, tokens=64, activation_fn="jumprelu", k=None),
     BASE.scaled("bw-d3072-f32-per-source", num_layers=2, d_model=3072, num_features=128, tokens=64, k=6, decoder_tying="per_source"),
+    # a batch beyond 65536 tokens (the per-feature lists are ordered with fewer wavefronts per workgroup)
+    BASE.scaled("bw-66000-tokens", num_layers=2, d_model=64, num_features=128, tokens=66000, k=4),
 ], ids=lambda w: w.name)
 def test_loss_and_gradients_match_autograd(dev, wl):
     dtype = getattr(torch, wl.dtype)
@@ -96,9 +98,10 @@ def test_loss_and_gradients_match_autograd(dev, wl):
         assert err <= bound, (name, err)
 
 
-@pytest.mark.parametrize("T,F,k", [(300, 128, 9), (4100, 96, 9), (70, 40960, 9), (40, 2048, 800), (8, 32768, 5000)],
+@pytest.mark.parametrize("T,F,k", [(300, 128, 9), (4100, 96, 9), (70, 40960, 9), (40, 2048, 800), (8, 32768, 5000),
+                                   (70000, 32, 2), (140000, 16, 1)],
                          ids=["blocks-of-tokens", "ragged-last-block", "feature-axis-beyond-lds", "rows-longer-than-a-workgroup",
-                              "rows-longer-than-the-staging-buffer"])
+                              "rows-longer-than-the-staging-buffer", "tokens-beyond-65536", "tokens-beyond-131072"])
 def test_feature_lists_are_a_permutation_grouped_by_feature(dev, T, F, k):
     # the blocked construction (counters of a token block in LDS, token order by construction; 4100 tokens = 33
     # blocks, the last one ragged; rows of ~800 survivors against 512 threads), and for a feature axis whose
