@@ -141,7 +141,7 @@ template <typename T, int COLLECT, bool SEG>
 __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void k_encode_mfma(
     const T *__restrict__ x, const T *__restrict__ w, const T *__restrict__ bias, T *__restrict__ pre,
     int M, int K, int N, int tiles_m, int tiles_n, int total_tiles, int64_t xs, int64_t wstr, int64_t bs,
-    int64_t ps, const SelState *__restrict__ gate, CollectArgs ca, SegArgs sg) {
+    int64_t ps, const SelState *__restrict__ gate, CollectArgs ca, SegArgs sg, int by_tokens) {
   static_assert(!SEG || COLLECT == 0, "segmented operands only in the storing mode");
   constexpr int CE = 16 / (int)sizeof(T);  // elements per 16-byte chunk
   constexpr int BK = ROWB / (int)sizeof(T);
@@ -169,7 +169,17 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
     TileAt t;
     t.layer = bid / per_layer;
     bid -= t.layer * per_layer;
-    if ((tiles_n & 7) == 0) {
+    if (by_tokens) {
+      // The mirror image, for products whose token operand is the larger one (the dense decoder product
+      // summed [T, F] x W[t] [d, F]: few feature tiles, many token tiles): XCD x owns the TOKEN tiles
+      // m = x, x+8, ..., so the large operand is fetched by one XCD only and the small one by all.
+      const int xcd = bid & 7, idx = bid >> 3, mloc = tiles_m >> 3;
+      const int g = idx / (ENC_SN * tiles_n), r = idx - g * ENC_SN * tiles_n;
+      const int cnt = (mloc - g * ENC_SN) < ENC_SN ? (mloc - g * ENC_SN) : ENC_SN;
+      const int ng = r / (cnt * ENC_SM), r2 = r - ng * cnt * ENC_SM;
+      t.tn = ng * ENC_SM + r2 / cnt;
+      t.tm = (g * ENC_SN + r2 % cnt) * 8 + xcd;
+    } else if ((tiles_n & 7) == 0) {
       // XCD x owns the feature tiles n = x, x+8, ...  Its tiles run in groups of ENC_SN feature tiles
       // x ENC_SM token tiles (about one tile per CU of the XCD): the group's W tiles stay in the L2
       // while the token groups sweep past, so W is fetched once and the x slab once per ENC_SN tiles.
@@ -189,7 +199,7 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
     // K is walked from a tile-dependent starting stage, wrapping around: the CUs of an XCD that share an
     // x tile or a W tile then ask for different lines of it at any one time, so one of them takes the
     // L2 miss and the others find the line there later, instead of all of them queueing behind the miss.
-    t.rot = ((tiles_n & 7) == 0 ? 3 * t.tm + (t.tn >> 3) : t.tm + t.tn) % nk;
+    t.rot = (by_tokens ? 3 * t.tn + (t.tm >> 3) : (tiles_n & 7) == 0 ? 3 * t.tm + (t.tn >> 3) : t.tm + t.tn) % nk;
     return t;
   };
   // the storing mode computes only the layers that asked for it when a gate is given; the states of up to
@@ -738,11 +748,14 @@ static int launch_encode(const void *x, const void *w, const void *b, void *pre,
     const int64_t grid = persistent_grid(nblk);
     if (grid <= 0) return CLT_ERR_LAUNCH;
     const SegArgs noseg = {};
+    // which operand an XCD keeps to itself: the feature tiles (W, the larger one in the encoder), or the token
+    // tiles when there are more of those and they split evenly over the XCDs
+    const int by_tokens = (tm % 8 == 0 && tm > tn) ? 1 : 0;
 #define CLT_ENC(C)                                                                                                  \
   k_encode_mfma<T, C, false><<<(unsigned)grid, NTHREADS, 0, stream>>>((const T *)x, (const T *)w, (const T *)b,     \
                                                                      (T *)pre, (int)T_, (int)d, (int)F, (int)tm,  \
                                                                      (int)tn, (int)nblk, xs, wstr, bs, ps, gate,  \
-                                                                     a, noseg)
+                                                                     a, noseg, by_tokens)
     if (collect == 0) CLT_ENC(0);
     else if (collect == 1) CLT_ENC(1);
     else CLT_ENC(2);
@@ -778,7 +791,7 @@ static int launch_encode_segmented(const void *x, const void *w, void *pre, int6
   if (grid <= 0) return CLT_ERR_LAUNCH;
   k_encode_mfma<T, 0, true><<<(unsigned)grid, NTHREADS, 0, stream>>>((const T *)x, (const T *)w, nullptr, (T *)pre, (int)T_,
                                                                     (int)K, (int)F, (int)tm, (int)tn, (int)nblk, 0, 0, 0,
-                                                                    0, nullptr, none, sg);
+                                                                    0, nullptr, none, sg, (tm % 8 == 0 && tm > tn) ? 1 : 0);
   return clt_check_launch();
 }
 
