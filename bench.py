@@ -30,9 +30,17 @@ MFMA_BF16_PEAK_TF = 2500.0  # dense bf16, TFLOP/s
 MFMA_FP32_PEAK_TF = 157.3
 
 
+def _esize(dtype_name: str) -> int:
+    return 4 if dtype_name == "float32" else 2
+
+
+def _dtname(dtype_name: str) -> str:
+    return {"float32": "f32", "bfloat16": "bf16", "float16": "f16"}[dtype_name]
+
+
 def algorithmic_work(wl, nnz_rows_pairs: int, nnz_total: int):
     """Algorithmic flops / bytes per forward, by stage (e = bytes per element)."""
-    e = 2 if wl.dtype == "bfloat16" else 4
+    e = _esize(wl.dtype)
     L, T, d, F = wl.num_layers, wl.tokens, wl.d_model, wl.num_features
     P = nnz_rows_pairs  # (token, feature, source->target) triples that fetch a decoder vector
     n_dec = L * (L + 1) // 2 if wl.decoder_tying == "none" else L
@@ -117,6 +125,8 @@ def run_gpu(args):
     wl = synth.WORKLOADS[args.workload]
     if args.topk_mode and args.topk_mode != wl.topk_mode:
         wl = wl.scaled(f"{wl.name}-{args.topk_mode}", topk_mode=args.topk_mode)
+    if args.dtype and args.dtype != wl.dtype:
+        wl = wl.scaled(f"{wl.name}-{_dtname(args.dtype)}", dtype=args.dtype)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     cca._native.load(build_if_missing=False)
@@ -195,9 +205,9 @@ def run_gpu(args):
     dec_c_gbs = work["decode_compulsory_bytes"] / (st["decode"] * 1e-3) / 1e9
     # ---- the dominant kernel: the decode ----------------------------------------------------------------
     nat = cca._native
-    e = 2 if wl.dtype == "bfloat16" else 4
+    e = _esize(wl.dtype)
     F, d = wl.num_features, wl.d_model
-    mfma_peak = MFMA_BF16_PEAK_TF if wl.dtype == "bfloat16" else MFMA_FP32_PEAK_TF
+    mfma_peak = MFMA_FP32_PEAK_TF if wl.dtype == "float32" else MFMA_BF16_PEAK_TF   # fp16 and bf16: the same dense peak
     route = engine.decode_route(T, d, F, L, wl.decoder_tying, model.dtype)
     dense_first, dense_end = dec.last_route.get("dense_targets", (L, L))
     n_dense = dense_end - dense_first
@@ -282,7 +292,7 @@ def run_gpu(args):
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16" if wl.dtype == "bfloat16" else "f32",
+        "dtype": _dtname(wl.dtype),
         "data": "synthetic",
         "config": {
             "workload": f"{wl.name}: CLT forward, L={L} d_model={wl.d_model} F={wl.num_features} T={T} "
@@ -346,7 +356,7 @@ def run_theta(args):
         "metric": "post-hoc theta estimation tokens/sec (encoder + statistics + global BatchTopK + selected minimum)",
         "value": wl.tokens * args.steps / wall, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": wall / args.steps * 1e3, "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "bf16" if wl.dtype == "bfloat16" else "f32", "data": "synthetic",
+        "vs_baseline": None, "dtype": _dtname(wl.dtype), "data": "synthetic",
         "config": {"workload": f"{wl.name}: theta estimation, L={wl.num_layers} d_model={wl.d_model} "
                                f"F={wl.num_features} T={wl.tokens} batchtopk k={wl.k} (global)"},
     }
@@ -520,13 +530,13 @@ def run_evaluator(args):
             torch.var(t - r, dim=0, unbiased=False).mean()
 
     dense_sec = timed(dense_scan, max(1, args.steps // 4))
-    esz = 2 if wl.dtype == "bfloat16" else 4
+    esz = _esize(wl.dtype)
     list_bytes = surv.nnz * (4 + esz) + (L * T + 1) * 4 + L * F * (4 + 4 + 8 + 8) + 2 * L * T * d * esz
     return {
         "metric": "evaluator reductions tokens/sec (L0, firing counts, dead-feature counters, reconstruction statistics)",
         "value": T / sec, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": sec * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16" if wl.dtype == "bfloat16" else "f32", "data": "synthetic",
+        "dtype": _dtname(wl.dtype), "data": "synthetic",
         "config": {"workload": f"{wl.name}: evaluator reductions, L={L} d_model={d} F={F} T={T} k={wl.k}"},
         "roofline": {"bound": "hbm", "achieved": list_bytes / sec / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": list_bytes / sec / 1e9 / HBM_PEAK_GBS, "traffic": None,
@@ -604,7 +614,7 @@ def run_backward(args):
         dec_b = bias_grad[torch.tensor([t for s_ in range(L) for t in range(s_, L)], device=dev)].contiguous()
         timed("Adam (other parameters)" if fused else "Adam",
               lambda: opt.step({"enc_w": dw_enc, "enc_b": db_enc, "dec_w": dw_dec, "dec_b": dec_b, "theta": None}))
-    esz = 2 if wl.dtype == "bfloat16" else 4
+    esz = _esize(wl.dtype)
     pairs = L * (L + 1) // 2
     gathered = surv.nnz / L * pairs * d * esz           # one row of g per (survivor, target >= its source)
     dw_sec = stages[dw_name] * 1e-3
@@ -654,7 +664,7 @@ def run_backward(args):
                    if opt is not None else "CLT forward + MSE loss + gradients tokens/sec (no optimizer step)"),
         "value": wl.tokens * args.steps / wall, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": wall / args.steps * 1e3, "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "bf16" if wl.dtype == "bfloat16" else "f32", "data": "synthetic",
+        "vs_baseline": None, "dtype": _dtname(wl.dtype), "data": "synthetic",
         "config": {"workload": f"{wl.name}: forward + backward, L={wl.num_layers} d_model={wl.d_model} "
                                f"F={wl.num_features} T={wl.tokens} {wl.activation_fn} k={wl.k}", "loss": float(loss)},
     }
@@ -700,6 +710,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c1")
+    ap.add_argument("--dtype", choices=["float32", "bfloat16", "float16"], default=None,
+                    help="forward bench only: run the workload in another element type than its own")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-tokens", type=int, default=4096)
     ap.add_argument("--no-fuse", action="store_true", help="separate encoder and selection kernels")

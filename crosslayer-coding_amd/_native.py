@@ -143,7 +143,9 @@ def dtype_code(dtype: torch.dtype) -> int:
         return CLT_F32
     if dtype == torch.bfloat16:
         return CLT_BF16
-    raise CLTNativeError(f"unsupported CLT dtype {dtype}; the HIP kernels implement float32 and bfloat16")
+    if dtype == torch.float16:
+        return CLT_F16      # forward-path entry points; the backward and optimiser kernels return CLT_ERR_DTYPE
+    raise CLTNativeError(f"unsupported CLT dtype {dtype}; the HIP kernels implement float32, bfloat16 and float16")
 
 
 def ptr(t: Optional[torch.Tensor]) -> Optional[int]:

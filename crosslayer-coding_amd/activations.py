@@ -27,7 +27,7 @@ def _mask_from_survivors(surv: engine.SurvivorList, shape) -> torch.Tensor:
 
 def _as_block(t: torch.Tensor) -> torch.Tensor:
     """[B, F] tensor as a one-layer [1, B, F] slab the kernels accept."""
-    if t.dtype not in (torch.float32, torch.bfloat16):
+    if t.dtype not in (torch.float32, torch.bfloat16, torch.float16):
         t = t.to(torch.float32)
     return t.detach().contiguous().unsqueeze(0)
 
@@ -116,7 +116,7 @@ class JumpReLU(torch.autograd.Function):
         nat.require_device(input, "JumpReLU")
         feat = input.shape[-1] if input.dim() > 0 else 1
         x2 = input.detach().reshape(-1, feat)
-        if x2.dtype not in (torch.float32, torch.bfloat16):
+        if x2.dtype not in (torch.float32, torch.bfloat16, torch.float16):
             x2 = x2.to(torch.float32)
         theta = threshold.detach().to(device=x2.device, dtype=x2.dtype)
         theta = torch.broadcast_to(theta.reshape(-1) if theta.dim() > 0 else theta, (feat,)).contiguous()

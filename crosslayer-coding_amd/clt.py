@@ -110,57 +110,15 @@ class CrossLayerTranscoder(BaseTranscoder):
                 m.device, m.dtype = w.device, w.dtype
 
     # ---- float16 models ----------------------------------------------------------------------------------
-    # The kernels implement float32 and bfloat16.  A model whose parameters are float16 (config.clt_dtype, or
-    # module.half()) keeps them in float16 - state dict, checkpoints and outputs are float16 as the reference's
-    # are - and computes its forward on the float32 kernels from a float32 copy of them, with every dense
-    # product and the thresholds rounded to float16 where the reference's float16 tensors would round
-    # (engine.emulate_dtype); sums across features and sources are therefore the more exact float32 ones.
-    # Forward-path methods only: gradients, the optimiser step and theta estimation raise NotImplementedError.
+    # The forward path (encoder, selection, decode, evaluator reductions) has float16 kernels of its own; the
+    # backward, the optimiser step and theta estimation are built for float32 and bfloat16 only.
     def _is_half(self) -> bool:
         self._sync_device()
         return self.dtype == torch.float16
 
-    def _half_twin(self) -> "CrossLayerTranscoder":
-        import copy
-        sd = self.state_dict()
-        key = tuple((k, v.data_ptr(), v._version) for k, v in sd.items())
-        if getattr(self, "_twin", None) is None or self._twin_key[0] != (self.config.activation_fn, self.device):
-            cfg = copy.deepcopy(self.config)
-            cfg.clt_dtype = "float32"
-            twin = CrossLayerTranscoder(cfg, None, self.device, profiler=self.profiler)
-            twin.fuse_encode_select = False      # the pre-activations must exist to be rounded
-            object.__setattr__(self, "_twin", twin)
-            self._twin_key = ((self.config.activation_fn, self.device), None)
-        if self._twin_key[1] != key:
-            self._twin.load_state_dict({k: v.detach().float() for k, v in sd.items()}, strict=False)
-            self._twin.decoder_module.invalidate_packed()
-            self._twin_key = (self._twin_key[0], key)
-        return self._twin
-
-    def _via_twin(self, name: str, *args):
-        def cast_in(a):
-            if isinstance(a, torch.Tensor):
-                return a.to(device=self.device, dtype=torch.float32) if a.is_floating_point() else a
-            if isinstance(a, dict):
-                return {k: cast_in(v) for k, v in a.items()}
-            return a
-
-        def cast_out(a):
-            if isinstance(a, torch.Tensor):
-                return a.to(torch.float16) if a.is_floating_point() else a
-            if isinstance(a, dict):
-                return {k: cast_out(v) for k, v in a.items()}
-            if isinstance(a, tuple):
-                return tuple(cast_out(v) for v in a)
-            return a
-
-        twin = self._half_twin()
-        with engine.emulate_dtype(torch.float16):
-            return cast_out(getattr(twin, name)(*[cast_in(a) for a in args]))
-
     def _no_half(self, what: str) -> None:
         if self._is_half():
-            raise NotImplementedError(f"{what} is not built for float16 models (the kernels implement float32 and bfloat16)")
+            raise NotImplementedError(f"{what} is not built for float16 models (float32 and bfloat16 only)")
 
     def release_workspace(self) -> None:
         """Free the cached scratch buffers (pre-activations, selection workspace)."""
@@ -169,13 +127,11 @@ class CrossLayerTranscoder(BaseTranscoder):
 
     # ---- reference API: thin delegations ------------------------------------------------
     def jumprelu(self, x: torch.Tensor, layer_idx: int) -> torch.Tensor:
-        if self._is_half():
-            return self._via_twin("jumprelu", x, layer_idx)
+        self._sync_device()
         return self.theta_manager.jumprelu(x, layer_idx)
 
     def get_preactivations(self, x: torch.Tensor, layer_idx: int) -> torch.Tensor:
-        if self._is_half():
-            return self._via_twin("get_preactivations", x, layer_idx)
+        self._sync_device()
         return self.encoder_module.get_preactivations(x, layer_idx)
 
     def _encode_all_layers(self, inputs: Dict[int, torch.Tensor]
@@ -185,13 +141,11 @@ class CrossLayerTranscoder(BaseTranscoder):
 
     def decode(self, a: Dict[int, torch.Tensor], layer_idx: int,
                source_inputs: Optional[Dict[int, torch.Tensor]] = None) -> torch.Tensor:
-        if self._is_half():
-            return self._via_twin("decode", a, layer_idx, source_inputs)
+        self._sync_device()
         return self.decoder_module.decode(a, layer_idx, source_inputs)
 
     def get_decoder_norms(self) -> torch.Tensor:
-        if self._is_half():
-            return self._via_twin("get_decoder_norms")
+        self._sync_device()
         return self.decoder_module.get_decoder_norms()
 
     @property
@@ -406,8 +360,7 @@ class CrossLayerTranscoder(BaseTranscoder):
     def encode(self, x: torch.Tensor, layer_idx: int) -> torch.Tensor:
         """Activations [tokens, F] of one layer for relu / jumprelu; for the top-k family the
         reference logs an error and returns zeros here (clt.py:135-149), and so does this."""
-        if self._is_half():
-            return self._via_twin("encode", x, layer_idx)
+        self._sync_device()
         x = x.to(device=self.device, dtype=self.dtype)
         preact = self.get_preactivations(x, layer_idx)
         F = self.config.num_features
@@ -586,8 +539,7 @@ class CrossLayerTranscoder(BaseTranscoder):
     # ---- get_feature_activations -------------------------------------------------------------
     def get_feature_activations(self, inputs: Dict[int, torch.Tensor]) -> Dict[int, torch.Tensor]:
         """Dense activations per layer (clt.py:220-277)."""
-        if self._is_half():
-            return self._via_twin("get_feature_activations", inputs)
+        self._sync_device()
         cfg = self.config
         topk_family = cfg.activation_fn in ("batchtopk", "topk")
         res = self._survivors(inputs)
@@ -642,7 +594,6 @@ class CrossLayerTranscoder(BaseTranscoder):
         """(reconstructions, survivor list over all num_layers) from one pass, or None when the inputs
         need the per-layer fallbacks.  The list is what get_feature_activations would densify; the
         evaluator and the dead-feature counters read it directly."""
-        self._no_half("forward_with_survivors")
         cfg = self.config
         L = cfg.num_layers
         res = self._survivors(inputs)
@@ -665,8 +616,7 @@ class CrossLayerTranscoder(BaseTranscoder):
 
     def forward(self, inputs: Dict[int, torch.Tensor]) -> Dict[int, torch.Tensor]:
         """Reconstruction of every layer present in ``inputs`` (clt.py:186-218)."""
-        if self._is_half():
-            return self._via_twin("forward", inputs)
+        self._sync_device()
         cfg = self.config
         L, d = cfg.num_layers, cfg.d_model
         res = self.forward_with_survivors(inputs)

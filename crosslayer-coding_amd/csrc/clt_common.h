@@ -25,7 +25,44 @@ __device__ __forceinline__ float round_to_bf16(float f) {
   return bf16_bits_to_f32(f32_to_bf16_bits(f));
 }
 
-// Element traits: T is float or bf16_t (raw bits).
+// IEEE half as raw bits, a type of its own so that templates tell it from bf16_t
+struct f16_t { uint16_t bits; };
+
+__host__ __device__ static inline float f16_bits_to_f32(uint32_t h) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  const uint16_t b = (uint16_t)h;
+  _Float16 v;
+  __builtin_memcpy(&v, &b, 2);
+  return (float)v;
+#else
+  const uint32_t sign = (h & 0x8000u) << 16, ex = (h >> 10) & 0x1Fu, man = h & 0x3FFu;
+  uint32_t u;
+  if (ex == 0x1Fu) u = sign | 0x7F800000u | (man << 13);
+  else if (ex != 0u) u = sign | ((ex + 112u) << 23) | (man << 13);
+  else if (man == 0u) u = sign;
+  else {
+    int e = -1;
+    uint32_t m = man;
+    do { m <<= 1; ++e; } while ((m & 0x400u) == 0u);
+    u = sign | ((uint32_t)(112 - e) << 23) | ((m & 0x3FFu) << 13);
+  }
+  float f;
+  __builtin_memcpy(&f, &u, 4);
+  return f;
+#endif
+}
+
+// round-to-nearest-even (v_cvt_f16_f32 under the default rounding mode), NaN stays NaN
+__device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
+  const _Float16 v = (_Float16)f;
+  uint16_t b;
+  __builtin_memcpy(&b, &v, 2);
+  return b;
+}
+
+// Element traits: T is float, bf16_t (raw bits) or f16_t (raw bits).
+//   IS16   16-bit element (eight per 16-byte vector, 16-bit ranking keys)
+//   INF16  raw bits of +infinity of a 16-bit type
 template <typename T> struct Elem;
 template <> struct Elem<float> {
   static constexpr int VEC = 4;       // elements per 16-byte vector
@@ -39,12 +76,49 @@ template <> struct Elem<float> {
 template <> struct Elem<bf16_t> {
   static constexpr int VEC = 8;
   static constexpr int KEYBITS = 16;
+  static constexpr uint32_t INF16 = 0x7F80u;
   __device__ static __forceinline__ float to_f32(bf16_t v) { return bf16_bits_to_f32(v); }
   __device__ static __forceinline__ bf16_t from_f32(float v) { return (bf16_t)f32_to_bf16_bits(v); }
   __device__ static __forceinline__ float round(float v) { return round_to_bf16(v); }
   __device__ static __forceinline__ uint32_t raw(bf16_t v) { return v; }
   __device__ static __forceinline__ bf16_t from_raw(uint32_t r) { return (bf16_t)r; }
 };
+
+template <> struct Elem<f16_t> {
+  static constexpr int VEC = 8;
+  static constexpr int KEYBITS = 16;
+  static constexpr uint32_t INF16 = 0x7C00u;
+  __device__ static __forceinline__ float to_f32(f16_t v) { return f16_bits_to_f32(v.bits); }
+  __device__ static __forceinline__ f16_t from_f32(float v) { return f16_t{(uint16_t)f32_to_f16_bits(v)}; }
+  __device__ static __forceinline__ float round(float v) { return f16_bits_to_f32(f32_to_f16_bits(v)); }
+  __device__ static __forceinline__ uint32_t raw(f16_t v) { return v.bits; }
+  __device__ static __forceinline__ f16_t from_raw(uint32_t r) { return f16_t{(uint16_t)r}; }
+};
+template <typename T> struct IsHalf { static constexpr bool value = false; };
+template <> struct IsHalf<f16_t> { static constexpr bool value = true; };
+
+// Two 16-bit elements of one 32-bit word (low half first) as floats, and back (round to nearest even).
+template <typename T> __device__ __forceinline__ void unpack_pair(uint32_t w, float &lo, float &hi) {
+  if constexpr (IsHalf<T>::value) {
+    lo = f16_bits_to_f32(w & 0xFFFFu);
+    hi = f16_bits_to_f32(w >> 16);
+  } else {
+    lo = __uint_as_float(w << 16);
+    hi = __uint_as_float(w & 0xFFFF0000u);
+  }
+}
+template <typename T> __device__ __forceinline__ uint32_t pack_pair(float lo, float hi) {
+  if constexpr (IsHalf<T>::value) return f32_to_f16_bits(lo) | (f32_to_f16_bits(hi) << 16);
+  else return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+}
+// raw 16 bits of a float that is a value of the 16-bit type T (exact)
+template <typename T> __device__ __forceinline__ uint32_t raw16_of(float v) {
+  if constexpr (IsHalf<T>::value) return f32_to_f16_bits(v);
+  else return __float_as_uint(v) >> 16;
+}
+// dtype code -> element size in bytes (0: not a model dtype)
+static inline int clt_elem_bytes(int dtype) { return dtype == CLT_F32 ? 4 : (dtype == CLT_BF16 || dtype == CLT_F16) ? 2 : 0; }
+static inline bool clt_model_dtype(int dtype) { return dtype == CLT_F32 || dtype == CLT_BF16 || dtype == CLT_F16; }
 
 // ---------------------------------------------------------------- ranking keys
 // Order-preserving unsigned key: ascending float order, -0.0 == +0.0, NaN on top.
@@ -62,6 +136,29 @@ template <int KB> __device__ __forceinline__ uint32_t rank_key(float x) {
 template <int KB> __device__ __host__ __forceinline__ uint32_t key_to_f32_bits(uint32_t key) {
   uint32_t k32 = KB == 32 ? key : ((key << 16) | ((key & 0x8000u) ? 0u : 0xFFFFu));
   return (k32 & 0x80000000u) ? (k32 & 0x7FFFFFFFu) : ~k32;
+}
+
+// The same by element type.  `x` must be a value of T (the key of a 16-bit type is taken from its own bits).
+template <typename T> __device__ __forceinline__ uint32_t rank_key_of(float x) {
+  if constexpr (IsHalf<T>::value) {
+    if (x != x) return 0xFFFFu;
+    uint32_t h = f32_to_f16_bits(x);
+    if (h == 0x8000u) h = 0u;
+    return (h & 0x8000u) ? (~h & 0xFFFFu) : (h | 0x8000u);
+  } else {
+    return rank_key<Elem<T>::KEYBITS>(x);
+  }
+}
+template <typename T> __device__ __host__ __forceinline__ uint32_t key_value_bits(uint32_t key) {
+  if constexpr (IsHalf<T>::value) {
+    const uint32_t h = (key & 0x8000u) ? (key & 0x7FFFu) : (~key & 0xFFFFu);
+    const float f = f16_bits_to_f32(h);
+    uint32_t u;
+    __builtin_memcpy(&u, &f, 4);
+    return u;
+  } else {
+    return key_to_f32_bits<Elem<T>::KEYBITS>(key);
+  }
 }
 
 // ---------------------------------------------------------------- wave helpers

@@ -32,21 +32,54 @@ template <> struct WVec<bf16_t> {
   // Two survivors at once: for each pair of bf16 weights in a 32-bit word, a byte permute puts
   // the same element of both rows side by side and v_dot2c_f32_bf16 multiplies them with the two
   // activation values (bf16 pair `vv`) and accumulates in fp32 - one op per element instead of two.
-  __device__ static __forceinline__ void dot32(float *acc, uint32_t a, uint32_t b, bf16x2_t vv) {
+  // `vp`: the two activation values as raw 16-bit elements, (first | second << 16)
+  __device__ static __forceinline__ void dot32(float *acc, uint32_t a, uint32_t b, uint32_t vp) {
+    const bf16x2_t vv = __builtin_bit_cast(bf16x2_t, vp);
     const uint32_t lo = __builtin_amdgcn_perm(b, a, 0x05040100u);   // (a.lo16, b.lo16)
     const uint32_t hi = __builtin_amdgcn_perm(b, a, 0x07060302u);   // (a.hi16, b.hi16)
     acc[0] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, lo), vv, acc[0], false);
     acc[1] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, hi), vv, acc[1], false);
   }
-  __device__ static __forceinline__ void dot16(float *acc, const uint4 &a, const uint4 &b, bf16x2_t vv) {
-    dot32(acc, a.x, b.x, vv); dot32(acc + 2, a.y, b.y, vv); dot32(acc + 4, a.z, b.z, vv); dot32(acc + 6, a.w, b.w, vv);
+  __device__ static __forceinline__ void dot16(float *acc, const uint4 &a, const uint4 &b, uint32_t vp) {
+    dot32(acc, a.x, b.x, vp); dot32(acc + 2, a.y, b.y, vp); dot32(acc + 4, a.z, b.z, vp); dot32(acc + 6, a.w, b.w, vp);
   }
-  __device__ static __forceinline__ void dot8(float *acc, const uint2 &a, const uint2 &b, bf16x2_t vv) {
-    dot32(acc, a.x, b.x, vv); dot32(acc + 2, a.y, b.y, vv);
+  __device__ static __forceinline__ void dot8(float *acc, const uint2 &a, const uint2 &b, uint32_t vp) {
+    dot32(acc, a.x, b.x, vp); dot32(acc + 2, a.y, b.y, vp);
   }
   __device__ static __forceinline__ void fma32(float *acc, uint32_t u, float v) {
     acc[0] = fmaf(v, __uint_as_float(u << 16), acc[0]);
     acc[1] = fmaf(v, __uint_as_float(u & 0xFFFF0000u), acc[1]);
+  }
+  __device__ static __forceinline__ void fma16(float *acc, const uint4 &w, float v) {
+    fma32(acc, w.x, v); fma32(acc + 2, w.y, v); fma32(acc + 4, w.z, v); fma32(acc + 6, w.w, v);
+  }
+  __device__ static __forceinline__ void fma8(float *acc, const uint2 &w, float v) {
+    fma32(acc, w.x, v); fma32(acc + 2, w.y, v);
+  }
+};
+
+// IEEE half: the same scheme with v_dot2_f32_f16 (exact products, fp32 accumulation)
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2_t;
+template <> struct WVec<f16_t> {
+  static constexpr int V = 8;
+  __device__ static __forceinline__ void dot32(float *acc, uint32_t a, uint32_t b, uint32_t vp) {
+    const f16x2_t vv = __builtin_bit_cast(f16x2_t, vp);
+    const uint32_t lo = __builtin_amdgcn_perm(b, a, 0x05040100u);
+    const uint32_t hi = __builtin_amdgcn_perm(b, a, 0x07060302u);
+    acc[0] = __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, lo), vv, acc[0], false);
+    acc[1] = __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, hi), vv, acc[1], false);
+  }
+  __device__ static __forceinline__ void dot16(float *acc, const uint4 &a, const uint4 &b, uint32_t vp) {
+    dot32(acc, a.x, b.x, vp); dot32(acc + 2, a.y, b.y, vp); dot32(acc + 4, a.z, b.z, vp); dot32(acc + 6, a.w, b.w, vp);
+  }
+  __device__ static __forceinline__ void dot8(float *acc, const uint2 &a, const uint2 &b, uint32_t vp) {
+    dot32(acc, a.x, b.x, vp); dot32(acc + 2, a.y, b.y, vp);
+  }
+  __device__ static __forceinline__ void fma32(float *acc, uint32_t u, float v) {
+    float lo, hi;
+    unpack_pair<f16_t>(u, lo, hi);
+    acc[0] = fmaf(v, lo, acc[0]);
+    acc[1] = fmaf(v, hi, acc[1]);
   }
   __device__ static __forceinline__ void fma16(float *acc, const uint4 &w, float v) {
     fma32(acc, w.x, v); fma32(acc + 2, w.y, v); fma32(acc + 4, w.z, v); fma32(acc + 6, w.w, v);
@@ -99,8 +132,7 @@ template <typename T, int NF, int TAIL, int UU> struct RowBatch {
       // bf16: the activation values are exact bf16 numbers, so two of them fit one dot2 operand
 #pragma unroll
       for (int u = 0; u < UU; u += 2) {
-        const uint32_t vb = (__float_as_uint(v[u]) >> 16) | (__float_as_uint(v[u + 1]) & 0xFFFF0000u);
-        const bf16x2_t vv = __builtin_bit_cast(bf16x2_t, vb);
+        const uint32_t vv = raw16_of<T>(v[u]) | (raw16_of<T>(v[u + 1]) << 16);
 #pragma unroll
         for (int c = 0; c < NF; ++c) WVec<T>::dot16(acc + c * V, wq[u][c], wq[u + 1][c], vv);
         if (TAIL == 1) WVec<T>::dot8(acc + NF * V, wt8[u], wt8[u + 1], vv);
@@ -285,7 +317,7 @@ __attribute__((amdgpu_waves_per_eu(decode_min_waves<T, NF, TAIL, SLICED>(), 8)))
     }
     const T *wbase = wp + decoder_slot(tying, src, t, L) * F * pitch;
     int32_t nb = __builtin_amdgcn_readlane(mb, 0), ne = __builtin_amdgcn_readlane(me, 0);
-    int32_t nxt_col = 0; T nxt_val = T(0);
+    int32_t nxt_col = 0; T nxt_val = Elem<T>::from_raw(0u);
     if (lane < ne - nb) { nxt_col = col[nb + lane]; nxt_val = val[nb + lane]; }
 #pragma unroll
     for (int i = 0; i < SLICED_NTOK; ++i) {
@@ -293,7 +325,7 @@ __attribute__((amdgpu_waves_per_eu(decode_min_waves<T, NF, TAIL, SLICED>(), 8)))
       const int32_t cur_col = nxt_col; const T cur_val = nxt_val;
       if (i + 1 < SLICED_NTOK) {
         nb = __builtin_amdgcn_readlane(mb, i + 1); ne = __builtin_amdgcn_readlane(me, i + 1);
-        nxt_col = 0; nxt_val = T(0);
+        nxt_col = 0; nxt_val = Elem<T>::from_raw(0u);
         if (lane < ne - nb) { nxt_col = col[nb + lane]; nxt_val = val[nb + lane]; }
       }
       if (tok0 + i >= Tn) break;
@@ -476,14 +508,14 @@ template <typename T, int HQ, int HTAIL, int UU, bool PACK> struct PartBatch {
   }
   __device__ __forceinline__ uint32_t value_pair(int u) const {
     if constexpr (PACK) return __builtin_amdgcn_perm(pk[u + 1], pk[u], 0x07060302u);   // (value u, value u + 1)
-    else return (__float_as_uint(v[u]) >> 16) | (__float_as_uint(v[u + 1]) & 0xFFFF0000u);
+    else return raw16_of<T>(v[u]) | (raw16_of<T>(v[u + 1]) << 16);
   }
   __device__ __forceinline__ void consume(float *acc) const {
     constexpr int V = WVec<T>::V;
     if constexpr (sizeof(T) == 2 && (UU % 2) == 0) {
 #pragma unroll
       for (int u = 0; u < UU; u += 2) {
-        const bf16x2_t vv = __builtin_bit_cast(bf16x2_t, value_pair(u));
+        const uint32_t vv = value_pair(u);
 #pragma unroll
         for (int c = 0; c < HQ; ++c) WVec<T>::dot16(acc + c * V, wq[u][c], wq[u + 1][c], vv);
         if (HTAIL) WVec<T>::dot8(acc + HQ * V, wt8[u], wt8[u + 1], vv);
@@ -534,7 +566,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(quarter_min
   }
   const T *wbase = wp + decoder_slot(tying, src, t, L) * F * pitch + (int64_t)cpart * (d / NCP);
   int32_t nb = __builtin_amdgcn_readlane(mb, 0), ne = __builtin_amdgcn_readlane(me, 0);
-  int32_t nxt_col = 0; T nxt_val = T(0);
+  int32_t nxt_col = 0; T nxt_val = Elem<T>::from_raw(0u);
   if (lane < ne - nb) { nxt_col = col[nb + lane]; nxt_val = val[nb + lane]; }
 #pragma unroll
   for (int i = 0; i < QUARTER_NTOK; ++i) {
@@ -542,7 +574,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(quarter_min
     const int32_t cur_col = nxt_col; const T cur_val = nxt_val;
     if (i + 1 < QUARTER_NTOK) {
       nb = __builtin_amdgcn_readlane(mb, i + 1); ne = __builtin_amdgcn_readlane(me, i + 1);
-      nxt_col = 0; nxt_val = T(0);
+      nxt_col = 0; nxt_val = Elem<T>::from_raw(0u);
       if (lane < ne - nb) { nxt_col = col[nb + lane]; nxt_val = val[nb + lane]; }
     }
     if (tok0 + i >= tok_end) break;
@@ -564,7 +596,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(quarter_min
         if (fscale) my_val = Elem<T>::round(my_val * Elem<T>::to_f32(fscale[t * F + my_col]));
       }
       // two batches of UU row pairs in flight
-      const uint32_t my_pk = PACK ? ((uint32_t)my_col | (__float_as_uint(my_val) & 0xFFFF0000u)) : 0u;
+      const uint32_t my_pk = PACK ? ((uint32_t)my_col | (raw16_of<T>(my_val) << 16)) : 0u;
       PartBatch<T, HQ, HTAIL, UU, PACK> ra, rb;
       constexpr int R = QROWS;
       ra.load(wbase, pitch, my_pk, my_col, my_val, 0, n, ll, grp);
@@ -674,8 +706,8 @@ template <typename T, int UU, bool PACK> struct LineBatch {
       for (int u = 0; u < UU; u += 2) {
         uint32_t vb;
         if constexpr (PACK) vb = __builtin_amdgcn_perm(pk[u + 1], pk[u], 0x07060302u);
-        else vb = (__float_as_uint(v[u]) >> 16) | (__float_as_uint(v[u + 1]) & 0xFFFF0000u);
-        WVec<T>::dot16(acc, wq[u], wq[u + 1], __builtin_bit_cast(bf16x2_t, vb));
+        else vb = raw16_of<T>(v[u]) | (raw16_of<T>(v[u + 1]) << 16);
+        WVec<T>::dot16(acc, wq[u], wq[u + 1], vb);
       }
     } else {
 #pragma unroll
@@ -711,7 +743,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))) voi
   }
   const T *wbase = wp + decoder_slot(tying, src, t, L) * F * pitch + (int64_t)cpart * LW;
   int32_t nb = __builtin_amdgcn_readlane(mb, 0), ne = __builtin_amdgcn_readlane(me, 0);
-  int32_t nxt_col = 0; T nxt_val = T(0);
+  int32_t nxt_col = 0; T nxt_val = Elem<T>::from_raw(0u);
   if (lane < ne - nb) { nxt_col = col[nb + lane]; nxt_val = val[nb + lane]; }
 #pragma unroll
   for (int it = 0; it < LINE_NTOK; ++it) {
@@ -719,7 +751,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))) voi
     const int32_t cur_col = nxt_col; const T cur_val = nxt_val;
     if (it + 1 < LINE_NTOK) {
       nb = __builtin_amdgcn_readlane(mb, it + 1); ne = __builtin_amdgcn_readlane(me, it + 1);
-      nxt_col = 0; nxt_val = T(0);
+      nxt_col = 0; nxt_val = Elem<T>::from_raw(0u);
       if (lane < ne - nb) { nxt_col = col[nb + lane]; nxt_val = val[nb + lane]; }
     }
     if (tok0 + it >= part_end) break;
@@ -740,7 +772,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))) voi
         if (fscale) my_val = Elem<T>::round(my_val * Elem<T>::to_f32(fscale[t * F + my_col]));
       }
       // bf16: feature index (< 65536) and value travel to their lane group in one 32-bit word
-      const uint32_t my_pk = PACK ? ((uint32_t)my_col | (__float_as_uint(my_val) & 0xFFFF0000u)) : 0u;
+      const uint32_t my_pk = PACK ? ((uint32_t)my_col | (raw16_of<T>(my_val) << 16)) : 0u;
       constexpr int R = 8 * LINE_UU;                 // survivors per batch
       ra.load(wbase, pitch, my_pk, my_col, my_val, 0, n, ll, grp);
       for (int i0 = 0; i0 < n; i0 += 2 * R) {
@@ -831,8 +863,8 @@ __global__ void k_decode_reduce(const float *__restrict__ partial, const float *
     else if (sizeof(T) == 4) *reinterpret_cast<float4 *>((float *)out + g) = a;
     else {
       uint2 o2;
-      o2.x = f32_to_bf16_bits(a.x) | (f32_to_bf16_bits(a.y) << 16);
-      o2.y = f32_to_bf16_bits(a.z) | (f32_to_bf16_bits(a.w) << 16);
+      o2.x = pack_pair<T>(a.x, a.y);
+      o2.y = pack_pair<T>(a.z, a.w);
       *reinterpret_cast<uint2 *>((bf16_t *)out + g) = o2;
     }
   }
@@ -953,8 +985,8 @@ __global__ void k_densify_scatter(const int32_t *row_ptr, const int32_t *col, co
     const int64_t l = r / Tn, t = r - l * Tn;
     OT *orow = out + l * out_layer_stride + t * F;
     for (int32_t j = row_ptr[r] + lane; j < row_ptr[r + 1]; j += 64) {
-      float v = Elem<T>::to_f32(val[j]);
-      orow[col[j]] = sizeof(OT) == 4 ? (OT)v : (OT)val[j];
+      if constexpr (std::is_same<T, OT>::value) orow[col[j]] = val[j];
+      else orow[col[j]] = (OT)Elem<T>::to_f32(val[j]);
     }
   }
 }
@@ -1231,7 +1263,7 @@ extern "C" int clt_decode_sparse(const int32_t *row_ptr, const int32_t *col, con
                                  const float *skip_add, void *out, int64_t T, int64_t d, int64_t F, int64_t L,
                                  int tying, int64_t t_begin, int64_t t_end, uint64_t src_mask, int dtype,
                                  int out_f32, void *workspace, size_t workspace_bytes, void *stream) {
-  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (!clt_model_dtype(dtype)) return CLT_ERR_DTYPE;
   if (T < 0 || d <= 0 || F <= 0 || L <= 0 || L > 64) return CLT_ERR_ARG;
   if (t_begin < 0 || t_end > L || t_begin > t_end) return CLT_ERR_ARG;
   if (tying < 0 || tying > 2) return CLT_ERR_ARG;
@@ -1240,26 +1272,28 @@ extern "C" int clt_decode_sparse(const int32_t *row_ptr, const int32_t *col, con
   hipStream_t s = (hipStream_t)stream;
   if (dtype == CLT_BF16)
     return launch_decode<bf16_t>(row_ptr, col, val, w_packed, bias_sum, feat_offset, feat_scale, skip_add, out, T, d, F, L, tying, t_begin, t_end, src_mask, out_f32, workspace, workspace_bytes, s);
+  if (dtype == CLT_F16)
+    return launch_decode<f16_t>(row_ptr, col, val, w_packed, bias_sum, feat_offset, feat_scale, skip_add, out, T, d, F, L, tying, t_begin, t_end, src_mask, out_f32, workspace, workspace_bytes, s);
   return launch_decode<float>(row_ptr, col, val, w_packed, bias_sum, feat_offset, feat_scale, skip_add, out, T, d, F, L, tying, t_begin, t_end, src_mask, out_f32, workspace, workspace_bytes, s);
 }
 
 extern "C" int clt_pack_decoder(const void *w_ref, void *w_packed, int64_t d, int64_t F, int64_t n_dec,
                                 int64_t in_stride, int64_t out_stride, int dtype, void *stream) {
-  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (!clt_model_dtype(dtype)) return CLT_ERR_DTYPE;
   if (d <= 0 || F <= 0 || n_dec < 0 || n_dec > 65535) return CLT_ERR_ARG;
   if (n_dec == 0) return CLT_OK;
   if (!w_ref || !w_packed) return CLT_ERR_ARG;
   dim3 grid((unsigned)clt_ceil_div(F, 64), (unsigned)clt_ceil_div(d, 64), (unsigned)n_dec);
   if (clt_ceil_div(d, 64) > 65535) return CLT_ERR_RANGE;
   hipStream_t s = (hipStream_t)stream;
-  if (dtype == CLT_BF16) k_pack<bf16_t><<<grid, 256, 0, s>>>((const bf16_t *)w_ref, (bf16_t *)w_packed, d, F, in_stride, out_stride, clt_pitch(d, 2));
+  if (dtype != CLT_F32) k_pack<bf16_t><<<grid, 256, 0, s>>>((const bf16_t *)w_ref, (bf16_t *)w_packed, d, F, in_stride, out_stride, clt_pitch(d, 2));
   else k_pack<float><<<grid, 256, 0, s>>>((const float *)w_ref, (float *)w_packed, d, F, in_stride, out_stride, clt_pitch(d, 4));
   return clt_check_launch();
 }
 
 extern "C" int clt_unpack_decoders(const void *w_packed, void *const *w_refs_dev, void *const *w_refs_host, int64_t n_dec,
                                    int64_t d, int64_t F, int dtype, void *stream) {
-  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (!clt_model_dtype(dtype)) return CLT_ERR_DTYPE;
   if (d <= 0 || F <= 0 || n_dec < 0 || n_dec > 65535) return CLT_ERR_ARG;
   if (n_dec == 0) return CLT_OK;
   if (!w_packed || !w_refs_dev) return CLT_ERR_ARG;
@@ -1270,10 +1304,10 @@ extern "C" int clt_unpack_decoders(const void *w_packed, void *const *w_refs_dev
   bool vec = w_refs_host != nullptr && d % 4 == 0 && F % 4 == 0;
   for (int64_t i = 0; vec && i < n_dec; ++i) vec = clt_aligned16(w_refs_host[i]);
   if (vec) {
-    if (dtype == CLT_BF16) k_unpack_vec<bf16_t><<<grid, 256, 0, s>>>((const bf16_t *)w_packed, (bf16_t *const *)w_refs_dev, d, F, clt_pitch(d, 2));
+    if (dtype != CLT_F32) k_unpack_vec<bf16_t><<<grid, 256, 0, s>>>((const bf16_t *)w_packed, (bf16_t *const *)w_refs_dev, d, F, clt_pitch(d, 2));
     else k_unpack_vec<float><<<grid, 256, 0, s>>>((const float *)w_packed, (float *const *)w_refs_dev, d, F, clt_pitch(d, 4));
   } else {
-    if (dtype == CLT_BF16) k_unpack<bf16_t><<<grid, 256, 0, s>>>((const bf16_t *)w_packed, (bf16_t *const *)w_refs_dev, d, F, clt_pitch(d, 2));
+    if (dtype != CLT_F32) k_unpack<bf16_t><<<grid, 256, 0, s>>>((const bf16_t *)w_packed, (bf16_t *const *)w_refs_dev, d, F, clt_pitch(d, 2));
     else k_unpack<float><<<grid, 256, 0, s>>>((const float *)w_packed, (float *const *)w_refs_dev, d, F, clt_pitch(d, 4));
   }
   return clt_check_launch();
@@ -1281,7 +1315,7 @@ extern "C" int clt_unpack_decoders(const void *w_packed, void *const *w_refs_dev
 
 extern "C" int clt_densify(const int32_t *row_ptr, const int32_t *col, const void *val, void *out, int64_t T,
                            int64_t F, int64_t L, int64_t out_layer_stride, int dtype, int out_f32, void *stream) {
-  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (!clt_model_dtype(dtype)) return CLT_ERR_DTYPE;
   if (T < 0 || F < 0 || L <= 0) return CLT_ERR_ARG;
   if (T == 0 || F == 0) return CLT_OK;
   if (!row_ptr || !out) return CLT_ERR_ARG;
@@ -1290,6 +1324,7 @@ extern "C" int clt_densify(const int32_t *row_ptr, const int32_t *col, const voi
   if (dtype == CLT_F32 || out_f32) k_zero_rows<float><<<nb, 256, 0, s>>>((float *)out, T, F, L, out_layer_stride);
   else k_zero_rows<bf16_t><<<nb, 256, 0, s>>>((bf16_t *)out, T, F, L, out_layer_stride);
   if (dtype == CLT_F32) k_densify_scatter<float, float><<<nb, 256, 0, s>>>(row_ptr, col, (const float *)val, (float *)out, T, F, L, out_layer_stride);
+  else if (out_f32 && dtype == CLT_F16) k_densify_scatter<f16_t, float><<<nb, 256, 0, s>>>(row_ptr, col, (const f16_t *)val, (float *)out, T, F, L, out_layer_stride);
   else if (out_f32) k_densify_scatter<bf16_t, float><<<nb, 256, 0, s>>>(row_ptr, col, (const bf16_t *)val, (float *)out, T, F, L, out_layer_stride);
   else k_densify_scatter<bf16_t, bf16_t><<<nb, 256, 0, s>>>(row_ptr, col, (const bf16_t *)val, (bf16_t *)out, T, F, L, out_layer_stride);
   return clt_check_launch();
@@ -1297,29 +1332,30 @@ extern "C" int clt_densify(const int32_t *row_ptr, const int32_t *col, const voi
 
 extern "C" int clt_decoder_norms(const void *w_packed, void *norms, int64_t d, int64_t F, int64_t L, int tying,
                                  int dtype, void *stream) {
-  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (!clt_model_dtype(dtype)) return CLT_ERR_DTYPE;
   if (d <= 0 || F <= 0 || L <= 0 || tying < 0 || tying > 2 || !w_packed || !norms) return CLT_ERR_ARG;
   hipStream_t s = (hipStream_t)stream;
   if (dtype == CLT_BF16) k_norms<bf16_t><<<256 * 8, 256, 0, s>>>((const bf16_t *)w_packed, (bf16_t *)norms, d, F, L, tying, clt_pitch(d, 2));
+  else if (dtype == CLT_F16) k_norms<f16_t><<<256 * 8, 256, 0, s>>>((const f16_t *)w_packed, (f16_t *)norms, d, F, L, tying, clt_pitch(d, 2));
   else k_norms<float><<<256 * 8, 256, 0, s>>>((const float *)w_packed, (float *)norms, d, F, L, tying, clt_pitch(d, 4));
   return clt_check_launch();
 }
 
 extern "C" int clt_decode_route(int64_t T, int64_t d, int64_t F, int64_t L, int tying, int dtype,
                                 size_t workspace_bytes) {
-  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (!clt_model_dtype(dtype)) return CLT_ERR_DTYPE;
   if (T <= 0 || d <= 0 || F <= 0 || L <= 0 || L > 64 || tying < 0 || tying > 2) return CLT_ERR_ARG;
-  return plan_route(d, F, tying, dtype == CLT_BF16 ? 2 : 4, workspace_bytes >= decode_ws_bytes(T, d, L), true);
+  return plan_route(d, F, tying, clt_elem_bytes(dtype), workspace_bytes >= decode_ws_bytes(T, d, L), true);
 }
 
 extern "C" int64_t clt_decoder_pitch(int64_t d, int dtype) {
-  if (d <= 0 || (dtype != CLT_F32 && dtype != CLT_BF16)) return -1;
-  return clt_pitch(d, dtype == CLT_BF16 ? 2 : 4);
+  if (d <= 0 || !clt_model_dtype(dtype)) return -1;
+  return clt_pitch(d, clt_elem_bytes(dtype));
 }
 
 extern "C" int64_t clt_decoder_slab_elems(int64_t d, int64_t F, int64_t L, int tying, int dtype) {
-  if (d <= 0 || F <= 0 || L <= 0 || tying < 0 || tying > 2 || (dtype != CLT_F32 && dtype != CLT_BF16)) return -1;
-  const int64_t pitch = clt_pitch(d, dtype == CLT_BF16 ? 2 : 4);
+  if (d <= 0 || F <= 0 || L <= 0 || tying < 0 || tying > 2 || !clt_model_dtype(dtype)) return -1;
+  const int64_t pitch = clt_pitch(d, clt_elem_bytes(dtype));
   const int64_t n_dec = tying == CLT_TYING_NONE ? L * (L + 1) / 2 : L;
   // the last element any schedule can touch: row F-1 of slot n_dec-1, formed like the kernels form it
   const int64_t last = decoder_slot_host(tying, L - 1, L - 1, L) * F * pitch + (F - 1) * pitch + (d - 1);
@@ -1329,20 +1365,23 @@ extern "C" int64_t clt_decoder_slab_elems(int64_t d, int64_t F, int64_t L, int t
 extern "C" int clt_accumulate_dense(const int32_t *row_ptr, const int32_t *col, const void *val,
                                     const void *feat_offset, const void *feat_scale, void *acc, int64_t T,
                                     int64_t F, int64_t layer, int init, int dtype, void *stream) {
-  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (!clt_model_dtype(dtype)) return CLT_ERR_DTYPE;
   if (T < 0 || F <= 0 || (layer < 0 && !init)) return CLT_ERR_ARG;
   if (T == 0) return CLT_OK;
   if (!acc || (layer >= 0 && !row_ptr)) return CLT_ERR_ARG;
   hipStream_t s = (hipStream_t)stream;
   const unsigned nb = (unsigned)(clt_ceil_div(T, 4) < 8192 ? clt_ceil_div(T, 4) : 8192);
   if (init) {
-    if (dtype == CLT_BF16) k_zero_rows<bf16_t><<<2048, 256, 0, s>>>((bf16_t *)acc, T, F, 1, T * F);
+    if (dtype != CLT_F32) k_zero_rows<bf16_t><<<2048, 256, 0, s>>>((bf16_t *)acc, T, F, 1, T * F);
     else k_zero_rows<float><<<2048, 256, 0, s>>>((float *)acc, T, F, 1, T * F);
   }
   if (layer < 0) return clt_check_launch();   // clear only
   if (dtype == CLT_BF16)
     k_accumulate_dense<bf16_t><<<nb, 256, 0, s>>>(row_ptr, col, (const bf16_t *)val, (const bf16_t *)feat_offset,
                                                  (const bf16_t *)feat_scale, (bf16_t *)acc, T, F, layer, init);
+  else if (dtype == CLT_F16)
+    k_accumulate_dense<f16_t><<<nb, 256, 0, s>>>(row_ptr, col, (const f16_t *)val, (const f16_t *)feat_offset,
+                                                 (const f16_t *)feat_scale, (f16_t *)acc, T, F, layer, init);
   else
     k_accumulate_dense<float><<<nb, 256, 0, s>>>(row_ptr, col, (const float *)val, (const float *)feat_offset,
                                                 (const float *)feat_scale, (float *)acc, T, F, layer, init);

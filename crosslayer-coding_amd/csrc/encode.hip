@@ -44,6 +44,13 @@ template <> struct Mma<bf16_t> {
     acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, bv, acc, 0, 0, 0);
   }
 };
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
+template <> struct Mma<f16_t> {
+  __device__ static __forceinline__ void run(f32x16_t &acc, const uint4 &a, const uint4 &b) {
+    f16x8_t av = __builtin_bit_cast(f16x8_t, a), bv = __builtin_bit_cast(f16x8_t, b);
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(av, bv, acc, 0, 0, 0);
+  }
+};
 template <> struct Mma<float> {
   __device__ static __forceinline__ void run(f32x16_t &acc, const uint4 &a, const uint4 &b) {
     acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.x), __uint_as_float(b.x), acc, 0, 0, 0);
@@ -62,10 +69,12 @@ __device__ __forceinline__ void load16_to_lds(const void *gsrc, void *lds_base) 
 typedef __attribute__((ext_vector_type(2))) float f32x2_t;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
 
-// two fp32 -> packed bf16 (round to nearest even; one v_cvt_pk_bf16_f32)
-__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+// two fp32 -> packed 16-bit elements (round to nearest even; bf16: one v_cvt_pk_bf16_f32)
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2_t;
+template <typename T> __device__ __forceinline__ uint32_t pack16x2(float a, float b) {
   f32x2_t v = {a, b};
-  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+  if constexpr (IsHalf<T>::value) return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2_t));
+  else return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
 
 // element j of a 16-byte slot as a float / as raw bits
@@ -77,6 +86,10 @@ template <> __device__ __forceinline__ float slot_elem<bf16_t>(const uint4 &w, i
   const uint32_t u = (j >> 1) == 0 ? w.x : (j >> 1) == 1 ? w.y : (j >> 1) == 2 ? w.z : w.w;
   return __uint_as_float((j & 1) ? (u & 0xFFFF0000u) : (u << 16));
 }
+template <> __device__ __forceinline__ float slot_elem<f16_t>(const uint4 &w, int j) {
+  const uint32_t u = (j >> 1) == 0 ? w.x : (j >> 1) == 1 ? w.y : (j >> 1) == 2 ? w.z : w.w;
+  return f16_bits_to_f32((j & 1) ? (u >> 16) : (u & 0xFFFFu));
+}
 template <typename T> __device__ __forceinline__ uint32_t slot_raw(const uint4 &w, int j);
 template <> __device__ __forceinline__ uint32_t slot_raw<float>(const uint4 &w, int j) {
   return j == 0 ? w.x : j == 1 ? w.y : j == 2 ? w.z : w.w;
@@ -85,6 +98,8 @@ template <> __device__ __forceinline__ uint32_t slot_raw<bf16_t>(const uint4 &w,
   const uint32_t u = (j >> 1) == 0 ? w.x : (j >> 1) == 1 ? w.y : (j >> 1) == 2 ? w.z : w.w;
   return (j & 1) ? (u >> 16) : (u & 0xFFFFu);
 }
+
+template <> __device__ __forceinline__ uint32_t slot_raw<f16_t>(const uint4 &w, int j) { return slot_raw<bf16_t>(w, j); }
 
 // packed 16-bit helpers (two elements per 32-bit word)
 typedef short i16x2_t __attribute__((ext_vector_type(2)));
@@ -303,8 +318,8 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
           bv[0] = __uint_as_float(r.x); bv[1] = __uint_as_float(r.y); bv[2] = __uint_as_float(r.z); bv[3] = __uint_as_float(r.w);
         } else {
           const uint2 r = raw[j * 4 + rg];
-          bv[0] = __uint_as_float(r.x << 16); bv[1] = __uint_as_float(r.x & 0xFFFF0000u);
-          bv[2] = __uint_as_float(r.y << 16); bv[3] = __uint_as_float(r.y & 0xFFFF0000u);
+          unpack_pair<T>(r.x, bv[0], bv[1]);
+          unpack_pair<T>(r.y, bv[2], bv[3]);
         }
 #pragma unroll
         for (int i = 0; i < 2; ++i)
@@ -446,8 +461,8 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
             } else {
               const int slot = (nl >> 3) ^ (ml & 15);
               uint2 o;
-              o.x = pack_bf16x2(y[0], y[1]);
-              o.y = pack_bf16x2(y[2], y[3]);
+              o.x = pack16x2<T>(y[0], y[1]);
+              o.y = pack16x2<T>(y[2], y[3]);
               *reinterpret_cast<uint2 *>(park + ml * 256 + slot * 16 + (nl & 4) * 2) = o;
             }
           }
@@ -488,7 +503,7 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
         uint32_t cut_bits = 0;
         if constexpr (COLLECT == 1) {
           asm volatile("" : "+v"(cut_key_v));      // nothing that reads the cut may move above this point
-          cut_bits = key_to_f32_bits<KB>((uint32_t)__builtin_amdgcn_readfirstlane((int)cut_key_v));
+          cut_bits = key_value_bits<T>((uint32_t)__builtin_amdgcn_readfirstlane((int)cut_key_v));
         }
         const bool cut_nan = (cut_bits & 0x7FFFFFFFu) > 0x7F800000u;   // only NaNs reach such a cut
         const float cutf = __uint_as_float(cut_bits);
@@ -530,8 +545,8 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
         const T *theta_seg = nullptr;
         if constexpr (sizeof(T) == 2) {
           if constexpr (COLLECT == 1) {
-            const uint32_t cb = cut_bits >> 16;
-            fast_ok = cb >= 1u && cb <= 0x7F80u;
+            const uint32_t cb = Elem<T>::raw(Elem<T>::from_f32(cutf));   // the cut is a value of T
+            fast_ok = cb >= 1u && cb <= Elem<T>::INF16;
             cm1 = (cb - 1u) | ((cb - 1u) << 16);
           } else {
             theta_seg = theta_lds[wave] + pass * SEGW;
@@ -542,7 +557,7 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
 #pragma unroll
               for (int k = 0; k < 4; ++k) {
                 const uint32_t lo = t4[k] & 0xFFFFu, hi = t4[k] >> 16;
-                bad = bad || lo < 1u || lo > 0x7F80u || hi < 1u || hi > 0x7F80u;
+                bad = bad || lo < 1u || lo > Elem<T>::INF16 || hi < 1u || hi > Elem<T>::INF16;
               }
             }
             fast_ok = __ballot(bad) == 0;
@@ -575,7 +590,7 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
                 const uint32_t m = (a | (a >> 16)) & 0xFFu;
                 Wh[s8 >> 2] |= m << ((s8 & 3) * 8);
               }
-              const uint32_t nan_above = COLLECT == 1 ? 0xFF80u : 0x7F80u;
+              const uint32_t nan_above = COLLECT == 1 ? (0x8000u | Elem<T>::INF16) : Elem<T>::INF16;
               const bool nan_seen = (mx & 0xFFFFu) > nan_above || (mx >> 16) > nan_above;
               done = __ballot(nan_seen) == 0;
             }
@@ -817,20 +832,21 @@ int clt_launch_encode(const void *x, const void *w, const void *b, void *pre, in
                       int64_t L, int64_t xs, int64_t wstr, int64_t bs, int64_t ps, int dtype, int collect,
                       const SelState *gate, const CollectArgs *ca, hipStream_t stream) {
   if (dtype == CLT_BF16) return launch_encode<bf16_t>(x, w, b, pre, T, d, F, L, xs, wstr, bs, ps, collect, gate, ca, stream);
+  if (dtype == CLT_F16) return launch_encode<f16_t>(x, w, b, pre, T, d, F, L, xs, wstr, bs, ps, collect, gate, ca, stream);
   return launch_encode<float>(x, w, b, pre, T, d, F, L, xs, wstr, bs, ps, collect, gate, ca, stream);
 }
 
 bool clt_encode_can_collect(const void *x, const void *w, const void *b, int64_t T, int64_t d, int64_t F,
                             int64_t xs, int64_t wstr, int64_t bs, int dtype) {
-  const bool fast = dtype == CLT_BF16 ? encode_fast_ok<bf16_t>(x, w, b, nullptr, T, d, F, xs, wstr, bs, 16)
-                                      : encode_fast_ok<float>(x, w, b, nullptr, T, d, F, xs, wstr, bs, 16);
+  const bool fast = dtype != CLT_F32 ? encode_fast_ok<bf16_t>(x, w, b, nullptr, T, d, F, xs, wstr, bs, 16)   // any 16-bit type
+                                     : encode_fast_ok<float>(x, w, b, nullptr, T, d, F, xs, wstr, bs, 16);
   return fast && T % BM == 0 && F % BN == 0;
 }
 
 extern "C" int clt_encode(const void *x, const void *w, const void *b, void *pre, int64_t T, int64_t d, int64_t F,
                           int64_t L, int64_t x_layer_stride, int64_t w_layer_stride, int64_t b_layer_stride,
                           int64_t pre_layer_stride, int dtype, void *stream) {
-  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (!clt_model_dtype(dtype)) return CLT_ERR_DTYPE;
   if (T < 0 || d <= 0 || F <= 0 || L <= 0) return CLT_ERR_ARG;
   if (T == 0) return CLT_OK;
   if (!x || !w || !pre) return CLT_ERR_ARG;

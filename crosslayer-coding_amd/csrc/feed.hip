@@ -82,7 +82,7 @@ __global__ __launch_bounds__(FD_THREADS) void k_feed_gather(const typename Src<S
     if constexpr (sizeof(OutT) == 2) {
       uint32_t p[4];
 #pragma unroll
-      for (int k = 0; k < 4; ++k) p[k] = f32_to_bf16_bits(x[2 * k]) | (f32_to_bf16_bits(x[2 * k + 1]) << 16);
+      for (int k = 0; k < 4; ++k) p[k] = pack_pair<OutT>(x[2 * k], x[2 * k + 1]);
       *reinterpret_cast<uint4 *>(op) = make_uint4(p[0], p[1], p[2], p[3]);
     } else {
       *reinterpret_cast<float4 *>(op) = make_float4(x[0], x[1], x[2], x[3]);
@@ -146,7 +146,7 @@ extern "C" int clt_feed_gather(const void *src, int src_dtype, int64_t src_rows,
                                int norm_mode, const float *mean_in, const float *std_in, const float *mean_tg,
                                const float *std_tg, double scale, void *x_out, void *tgt_out, int64_t out_row0, int64_t T,
                                int out_dtype, void *stream) {
-  if (out_dtype != CLT_F32 && out_dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (!clt_model_dtype(out_dtype)) return CLT_ERR_DTYPE;
   if (src_dtype != CLT_F32 && src_dtype != CLT_BF16 && src_dtype != CLT_F16) return CLT_ERR_DTYPE;
   if (n < 0 || d <= 0 || L <= 0 || L > 32767 || T <= 0 || out_row0 < 0 || out_row0 + n > T || src_rows < 0) return CLT_ERR_ARG;
   if (norm_mode < CLT_DENORM_NONE || norm_mode > CLT_DENORM_SCALE) return CLT_ERR_ARG;
@@ -168,6 +168,8 @@ extern "C" int clt_feed_gather(const void *src, int src_dtype, int64_t src_rows,
 #define CLT_FEED(S)                                                                                                         \
   (out_dtype == CLT_BF16                                                                                                    \
        ? launch_feed<S, bf16_t>(src, src_rows, src_layer_stride, src_target_offset, row_index, n, d, L, nm, x_out, tgt_out, out_row0, T, s) \
+   : out_dtype == CLT_F16                                                                                                   \
+       ? launch_feed<S, f16_t>(src, src_rows, src_layer_stride, src_target_offset, row_index, n, d, L, nm, x_out, tgt_out, out_row0, T, s) \
        : launch_feed<S, float>(src, src_rows, src_layer_stride, src_target_offset, row_index, n, d, L, nm, x_out, tgt_out, out_row0, T, s))
   if (src_dtype == CLT_F32) return CLT_FEED(CLT_F32);
   if (src_dtype == CLT_BF16) return CLT_FEED(CLT_BF16);

@@ -135,7 +135,7 @@ __global__ __launch_bounds__(MT_THREADS) void k_recon_finish(const double *part,
 extern "C" int clt_survivor_metrics(const int32_t *row_ptr, const int32_t *col, const void *val, int64_t T, int64_t F,
                                     int64_t L, int dtype, float fired_eps, uint64_t *nonzero_per_layer,
                                     uint32_t *fired_count, void *stream) {
-  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (!clt_model_dtype(dtype)) return CLT_ERR_DTYPE;
   if (T <= 0 || F <= 0 || L <= 0 || L > 65535 || !row_ptr || !nonzero_per_layer || !fired_count) return CLT_ERR_ARG;
   hipStream_t s = (hipStream_t)stream;
   k_metrics_zero<<<1024, MT_THREADS, 0, s>>>(fired_count, L * F, (unsigned long long *)nonzero_per_layer, (int)L);
@@ -143,6 +143,9 @@ extern "C" int clt_survivor_metrics(const int32_t *row_ptr, const int32_t *col, 
     const unsigned nb = 256 * 8;
     if (dtype == CLT_BF16)
       k_survivor_metrics<bf16_t><<<nb, MT_THREADS, 0, s>>>(row_ptr, col, (const bf16_t *)val, T, F, L, fired_eps,
+                                                           (unsigned long long *)nonzero_per_layer, fired_count);
+    else if (dtype == CLT_F16)
+      k_survivor_metrics<f16_t><<<nb, MT_THREADS, 0, s>>>(row_ptr, col, (const f16_t *)val, T, F, L, fired_eps,
                                                            (unsigned long long *)nonzero_per_layer, fired_count);
     else
       k_survivor_metrics<float><<<nb, MT_THREADS, 0, s>>>(row_ptr, col, (const float *)val, T, F, L, fired_eps,
@@ -168,7 +171,7 @@ extern "C" size_t clt_reconstruction_stats_workspace_bytes(int64_t d, int64_t L)
 extern "C" int clt_reconstruction_stats(const void *rec, const void *target, int64_t T, int64_t d, int64_t L, int dtype,
                                         int denorm_mode, const void *mean, const void *stdv, double scale, double *stats,
                                         void *workspace, size_t workspace_bytes, void *stream) {
-  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (!clt_model_dtype(dtype)) return CLT_ERR_DTYPE;
   if (T <= 0 || d <= 0 || L <= 0 || L > 65535 || !rec || !target || !stats || !workspace) return CLT_ERR_ARG;
   if (denorm_mode < CLT_DENORM_NONE || denorm_mode > CLT_DENORM_SCALE) return CLT_ERR_ARG;
   if (denorm_mode == CLT_DENORM_MEAN_STD && (!mean || !stdv)) return CLT_ERR_ARG;
@@ -181,6 +184,9 @@ extern "C" int clt_reconstruction_stats(const void *rec, const void *target, int
   if (dtype == CLT_BF16)
     k_recon_partial<bf16_t><<<grid, MT_THREADS, 0, s>>>((const bf16_t *)rec, (const bf16_t *)target, T, d, denorm_mode,
                                                         (const bf16_t *)mean, (const bf16_t *)stdv, (float)scale, part);
+  else if (dtype == CLT_F16)
+    k_recon_partial<f16_t><<<grid, MT_THREADS, 0, s>>>((const f16_t *)rec, (const f16_t *)target, T, d, denorm_mode,
+                                                        (const f16_t *)mean, (const f16_t *)stdv, (float)scale, part);
   else
     k_recon_partial<float><<<grid, MT_THREADS, 0, s>>>((const float *)rec, (const float *)target, T, d, denorm_mode,
                                                        (const float *)mean, (const float *)stdv, (float)scale, part);

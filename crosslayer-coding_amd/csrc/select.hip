@@ -43,6 +43,10 @@ constexpr uint32_t ROW_DENSE = 0xFFFFFFFEu;  // row did not fit the pool: read i
 template <int KB> __device__ __forceinline__ uint32_t min_key() {
   return KB == 32 ? 0x007FFFFFu : 0x007Fu;  // key(-inf); nothing ranks below it
 }
+// key(-inf) of the element type
+template <typename T> __device__ __forceinline__ uint32_t min_key_of() {
+  return IsHalf<T>::value ? 0x03FFu : min_key<Elem<T>::KEYBITS>();
+}
 template <int KB> __device__ __forceinline__ uint32_t bin_level0(uint32_t diff) {
   if (KB == 16) return diff < FINE16 ? diff : FINE16 + (diff >> 10);
   return diff >> 21;
@@ -96,6 +100,22 @@ template <> struct VecLoad<bf16_t, 8> {
       raw[2 * j] = w[j] & 0xFFFFu; raw[2 * j + 1] = w[j] >> 16;
       x[2 * j] = __uint_as_float(w[j] << 16); x[2 * j + 1] = __uint_as_float(w[j] & 0xFFFF0000u);
     }
+  }
+};
+template <> struct VecLoad<f16_t, 8> {
+  __device__ static __forceinline__ void load(const f16_t *p, float (&x)[8], uint32_t (&raw)[8]) {
+    uint4 v = *reinterpret_cast<const uint4 *>(p);
+    uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      raw[2 * j] = w[j] & 0xFFFFu; raw[2 * j + 1] = w[j] >> 16;
+      unpack_pair<f16_t>(w[j], x[2 * j], x[2 * j + 1]);
+    }
+  }
+};
+template <> struct VecLoad<f16_t, 1> {
+  __device__ static __forceinline__ void load(const f16_t *p, float (&x)[1], uint32_t (&raw)[1]) {
+    raw[0] = p->bits; x[0] = f16_bits_to_f32(raw[0]);
   }
 };
 template <> struct VecLoad<bf16_t, 1> {
@@ -184,7 +204,7 @@ __global__ __launch_bounds__(256) void k_sample_keys(
     else { l = p; t = idx / F; f = idx - t * F; }
     float x = Elem<T>::to_f32(pre[l * lstride + t * F + f]);
     typename RankOf<T, GLOBAL>::type rk = RankOf<T, GLOBAL>::make(mean, denom, l, F);
-    sample[(int64_t)p * SAMPLE_N + si] = rank_key<KB>(rk(x, f));
+    sample[(int64_t)p * SAMPLE_N + si] = rank_key_of<T>(rk(x, f));
   }
 }
 
@@ -273,6 +293,11 @@ template <> __device__ __forceinline__ float vec_elem<bf16_t>(const uint4 &w, in
   return __uint_as_float((j & 1) ? (u & 0xFFFF0000u) : (u << 16));
 }
 
+template <> __device__ __forceinline__ float vec_elem<f16_t>(const uint4 &w, int j) {
+  const uint32_t u = (j >> 1) == 0 ? w.x : (j >> 1) == 1 ? w.y : (j >> 1) == 2 ? w.z : w.w;
+  return f16_bits_to_f32((j & 1) ? (u >> 16) : (u & 0xFFFFu));
+}
+
 // Global ranking: for every (layer, feature) the lowest value x whose z-score reaches the cut
 // key (binary search over the ordered keys of the element type; the z-score with its two
 // roundings is monotone in x).  NaN when only a NaN reaches the cut.
@@ -284,14 +309,14 @@ __global__ __launch_bounds__(256) void k_col_cut(const float *mean, const float 
   if (i >= L * F) return;
   const uint32_t cut_key = st[0].cut_key;
   RankZ<T> rk; rk.mean = mean; rk.denom = denom;   // indexed with the flat (layer, feature) position
-  uint32_t lo = min_key<KB>(), hi = KB == 32 ? 0xFFFFFFFFu : 0xFFFFu;
+  uint32_t lo = min_key_of<T>(), hi = KB == 32 ? 0xFFFFFFFFu : 0xFFFFu;
   while (lo < hi) {
     const uint32_t mid = lo + ((hi - lo) >> 1);
-    const float xv = __uint_as_float(key_to_f32_bits<KB>(mid));
-    if (rank_key<KB>(rk(xv, i)) >= cut_key) hi = mid; else lo = mid + 1u;
+    const float xv = __uint_as_float(key_value_bits<T>(mid));
+    if (rank_key_of<T>(rk(xv, i)) >= cut_key) hi = mid; else lo = mid + 1u;
   }
-  const uint32_t bits = key_to_f32_bits<KB>(lo);
-  xcut[i] = Elem<T>::from_raw(sizeof(T) == 2 ? (bits >> 16) : bits);
+  const uint32_t bits = key_value_bits<T>(lo);
+  xcut[i] = Elem<T>::from_f32(__uint_as_float(bits));   // exact: the value is one of T
 }
 
 // The streaming pass: one wavefront per row.  A step covers PASS_NV vectors of 64 lanes x 16
@@ -314,7 +339,7 @@ __global__ __launch_bounds__(256) void k_select_pass(
   const uint32_t status = st[p].status;
   if (phase == 0 ? status != ST_RUN : status != ST_RETRY) return;
   const uint32_t cut_key = st[p].cut_key;
-  const uint32_t cut_bits = key_to_f32_bits<KB>(cut_key);
+  const uint32_t cut_bits = key_value_bits<T>(cut_key);
   const float cutf = __uint_as_float(cut_bits);
   const bool cut_nan = (cut_bits & 0x7FFFFFFFu) > 0x7F800000u;  // only NaNs reach such a cut
   for (int i = threadIdx.x; i < NBINS; i += blockDim.x) lh[i] = 0;
@@ -373,7 +398,7 @@ __global__ __launch_bounds__(256) void k_select_pass(
         uint32_t mq = 0;
 #pragma unroll
         for (int j = 0; j < V; ++j) {
-          const float xv = V > 1 ? vec_elem<T>(w[q], j) : __uint_as_float(w[q].x);
+          const float xv = V > 1 ? vec_elem<T>(w[q], j) : Elem<T>::to_f32(Elem<T>::from_raw(sizeof(T) == 2 ? (w[q].x >> 16) : w[q].x));
           bool c;
           if (by_column) c = xv >= vec_elem<T>(xc[q], j) || xv != xv;
           else {
@@ -411,7 +436,7 @@ __global__ __launch_bounds__(256) void k_select_pass(
           const uint32_t rel = wbuf[n_buf + i].x;
           const T rawv = stage[rel];
           const uint32_t col = c0u + rel;
-          const uint32_t key = rank_key<KB>(rk(Elem<T>::to_f32(rawv), (int64_t)col));
+          const uint32_t key = rank_key_of<T>(rk(Elem<T>::to_f32(rawv), (int64_t)col));
           atomicAdd(&lh[bin_level0<KB>(key - cut_key)], 1u);
           wbuf[n_buf + i] = make_uint2(col, Elem<T>::raw(rawv));
         }
@@ -547,7 +572,7 @@ __device__ __forceinline__ void visit_candidates(
 #pragma unroll
         for (int u = 0; u < NS; ++u) {
           key[u] = 0;
-          if (act[u]) key[u] = rank_key<KB>(rk(Elem<T>::to_f32(Elem<T>::from_raw(e[u].y)), (int64_t)e[u].x));
+          if (act[u]) key[u] = rank_key_of<T>(rk(Elem<T>::to_f32(Elem<T>::from_raw(e[u].y)), (int64_t)e[u].x));
         }
 #pragma unroll
         for (int u = 0; u < NS; ++u)
@@ -564,16 +589,16 @@ __device__ __forceinline__ void visit_candidates(
     const T *row = pre + l * lstride + t * F;
     T v[NQ], vn[NQ];
 #pragma unroll
-    for (int q = 0; q < NQ; ++q) { const int64_t col = (int64_t)q * 64 + lane; v[q] = col < F ? row[col] : T(0); }
+    for (int q = 0; q < NQ; ++q) { const int64_t col = (int64_t)q * 64 + lane; v[q] = col < F ? row[col] : Elem<T>::from_raw(0u); }
     for (int64_t c0 = 0; c0 < F; c0 += 64 * NQ) {
       const int64_t cn = c0 + 64 * NQ;
 #pragma unroll
-      for (int q = 0; q < NQ; ++q) { const int64_t col = cn + q * 64 + lane; vn[q] = col < F ? row[col] : T(0); }
+      for (int q = 0; q < NQ; ++q) { const int64_t col = cn + q * 64 + lane; vn[q] = col < F ? row[col] : Elem<T>::from_raw(0u); }
       uint32_t key[NQ];
 #pragma unroll
       for (int q = 0; q < NQ; ++q) {
         const int64_t col = c0 + q * 64 + lane;
-        key[q] = col < F ? rank_key<KB>(rk(Elem<T>::to_f32(v[q]), col)) : 0u;
+        key[q] = col < F ? rank_key_of<T>(rk(Elem<T>::to_f32(v[q]), col)) : 0u;
       }
 #pragma unroll
       for (int q = 0; q < NQ; ++q) {
@@ -773,6 +798,7 @@ __global__ __launch_bounds__(256) void k_select_emit(
 // one rounding to the model dtype.  The sample only has to give a cut of the right size; the selection
 // stays exact whatever the cut is.
 typedef __attribute__((ext_vector_type(8))) __bf16 smp_bf16x8_t;
+typedef __attribute__((ext_vector_type(8))) _Float16 smp_f16x8_t;
 typedef __attribute__((ext_vector_type(16))) float smp_f32x16_t;
 template <typename T>
 __global__ __launch_bounds__(256) void k_sample_mfma(
@@ -796,7 +822,9 @@ __global__ __launch_bounds__(256) void k_sample_mfma(
   for (int64_t st = 0; st < nstep; ++st) {
     const uint4 a = *reinterpret_cast<const uint4 *>(wr + st * 2 * V);
     const uint4 q = *reinterpret_cast<const uint4 *>(xr + st * 2 * V);
-    if constexpr (sizeof(T) == 2) {
+    if constexpr (IsHalf<T>::value) {
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(smp_f16x8_t, a), __builtin_bit_cast(smp_f16x8_t, q), acc, 0, 0, 0);
+    } else if constexpr (sizeof(T) == 2) {
       acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(smp_bf16x8_t, a), __builtin_bit_cast(smp_bf16x8_t, q), acc, 0, 0, 0);
     } else {
       acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.x), __uint_as_float(q.x), acc, 0, 0, 0);
@@ -814,7 +842,7 @@ __global__ __launch_bounds__(256) void k_sample_mfma(
     for (int q = 0; q < 4; ++q) {
       const int m = rg * 8 + lh * 4 + q;
       const float bv = __shfl(bown, m);
-      out[m * 32 + l31] = rank_key<KB>(Elem<T>::round(acc[rg * 4 + q] + bv));
+      out[m * 32 + l31] = rank_key_of<T>(Elem<T>::round(acc[rg * 4 + q] + bv));
     }
 }
 
@@ -842,7 +870,7 @@ __global__ __launch_bounds__(256) void k_pool_hist(const SelState *st, const uin
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         if (e0 + q * 64 + lane >= tm.y) continue;
-        const uint32_t diff = rank_key<KB>(Elem<T>::to_f32(Elem<T>::from_raw(raw[q]))) - s.cut_key;
+        const uint32_t diff = rank_key_of<T>(Elem<T>::to_f32(Elem<T>::from_raw(raw[q]))) - s.cut_key;
         if (level == 0) atomicAdd(&lh[bin_level0<KB>(diff)], 1u);
         else if (diff >= s.flo && diff <= s.fhi) atomicAdd(&lh[(diff - s.bbase) >> s.shift], 1u);
       }
@@ -883,12 +911,12 @@ __global__ __launch_bounds__(256) void k_tile_count(
 #pragma unroll
   for (int e = 0; e < TILE_NE; ++e)
     if ((uint32_t)e < m.y) {
-      const uint32_t key = rank_key<KB>(Elem<T>::to_f32(Elem<T>::from_raw(raw[e])));
+      const uint32_t key = rank_key_of<T>(Elem<T>::to_f32(Elem<T>::from_raw(raw[e])));
       ngt += key > s.thr_key ? 1u : 0u;
       neq += key == s.thr_key ? 1u : 0u;
     }
   for (uint32_t e = TILE_NE; e < m.y; ++e) {
-    const uint32_t key = rank_key<KB>(Elem<T>::to_f32(Elem<T>::from_raw(mypool[m.x + e].y)));
+    const uint32_t key = rank_key_of<T>(Elem<T>::to_f32(Elem<T>::from_raw(mypool[m.x + e].y)));
     ngt += key > s.thr_key ? 1u : 0u;
     neq += key == s.thr_key ? 1u : 0u;
   }
@@ -951,7 +979,7 @@ __global__ __launch_bounds__(256) void k_tile_emit(
   uint32_t tie = peq[at];
   int64_t pos = (int64_t)row_ptr[r] + pgt[at] + (tie < al ? tie : al);
   auto put = [&](const uint2 &e2) {
-    const uint32_t key = rank_key<KB>(Elem<T>::to_f32(Elem<T>::from_raw(e2.y)));
+    const uint32_t key = rank_key_of<T>(Elem<T>::to_f32(Elem<T>::from_raw(e2.y)));
     bool keepit = key > s.thr_key;
     if (key == s.thr_key) { keepit = tie < al; ++tie; }
     if (keepit) { col_out[pos] = (int32_t)e2.x; val_out[pos] = Elem<T>::from_raw(e2.y); ++pos; }
@@ -1142,7 +1170,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_token_threshold(
       const T *row = pre + l * lstride + t * F;
       typename RankOf<T, GLOBAL>::type rk = RankOf<T, GLOBAL>::make(mean, denom, l, F);
       for (int64_t f = tid; f < F; f += SCAN_THREADS) {
-        const uint32_t key = rank_key<KB>(rk(Elem<T>::to_f32(row[f]), f));
+        const uint32_t key = rank_key_of<T>(rk(Elem<T>::to_f32(row[f]), f));
         if ((key & prefix_mask) == prefix) atomicAdd(&lh[(key >> sh) & dm], 1u);
       }
     }
@@ -1163,7 +1191,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_token_threshold(
     typename RankOf<T, GLOBAL>::type rk = RankOf<T, GLOBAL>::make(mean, denom, l, F);
     uint32_t g = 0, e = 0;
     for (int64_t f = tid; f < F; f += SCAN_THREADS) {
-      const uint32_t key = rank_key<KB>(rk(Elem<T>::to_f32(row[f]), f));
+      const uint32_t key = rank_key_of<T>(rk(Elem<T>::to_f32(row[f]), f));
       g += key > thr; e += key == thr;
     }
 #pragma unroll
@@ -1209,7 +1237,7 @@ __global__ __launch_bounds__(256) void k_token_emit(
         VecLoad<T, V>::load(row + col, x, raw);
 #pragma unroll
         for (int j = 0; j < V; ++j) {
-          const uint32_t key = rank_key<KB>(rk(x[j], col + j));
+          const uint32_t key = rank_key_of<T>(rk(x[j], col + j));
           if (key > thr) mg |= 1u << j;
           if (key == thr) me |= 1u << j;
         }
@@ -1420,7 +1448,7 @@ struct TileLayout {
 static TileLayout tile_layout(int64_t T, int64_t F, int64_t L, int64_t k, int dtype) {
   TileLayout tl;
   tl.sel = sel_layout(T, F, L, k, CLT_TOPK_PER_LAYER);
-  const int segw = dtype == CLT_BF16 ? 128 : 64;
+  const int segw = dtype != CLT_F32 ? 128 : 64;
   tl.nseg = (int)(F / segw);
   tl.ntile = tl.nseg * (int)(T / COLLECT_ROWS);
   // about 1.5x K candidates are expected, i.e. 1.5 * k / F of a tile's 64 * segw elements; a
@@ -1541,7 +1569,7 @@ struct ThreshLayout {
 
 static ThreshLayout thresh_layout(int64_t T, int64_t F, int64_t L, int64_t density_ppm, int dtype) {
   ThreshLayout tl;
-  const int segw = dtype == CLT_BF16 ? 128 : 64;
+  const int segw = dtype != CLT_F32 ? 128 : 64;
   tl.nseg = (int)(F / segw);
   tl.ntile = tl.nseg * (int)(T / COLLECT_ROWS);
   const double dens = (double)(density_ppm < 1 ? 1 : density_ppm) * 1e-6;
@@ -1572,10 +1600,10 @@ extern "C" int clt_encode_threshold_supported(const void *x, const void *w, cons
                                               int64_t T, int64_t d, int64_t F, int64_t L, int64_t x_layer_stride,
                                               int64_t w_layer_stride, int64_t b_layer_stride,
                                               int64_t theta_layer_stride, int64_t density_ppm, int dtype) {
-  if (dtype != CLT_F32 && dtype != CLT_BF16) return 0;
+  if (!clt_model_dtype(dtype)) return 0;
   if (T <= 0 || d <= 0 || F <= 0 || L <= 0 || L > 65535 || !x || !w || !theta) return 0;
   if ((double)T * (double)F >= 4294967296.0 || (double)T * (double)L >= 2147483647.0) return 0;
-  if (!clt_aligned16(theta) || (theta_layer_stride * (dtype == CLT_BF16 ? 2 : 4)) % 16 != 0) return 0;
+  if (!clt_aligned16(theta) || (theta_layer_stride * clt_elem_bytes(dtype)) % 16 != 0) return 0;
   if (thresh_layout(T, F, L, density_ppm, dtype).tpool_cap >= 0xFFF00000ull) return 0;
   return clt_encode_can_collect(x, w, b, T, d, F, x_layer_stride, w_layer_stride, b_layer_stride, dtype) ? 1 : 0;
 }
@@ -1592,7 +1620,7 @@ extern "C" int clt_encode_threshold_count(const void *x, const void *w, const vo
                                           int64_t w_layer_stride, int64_t b_layer_stride,
                                           int64_t theta_layer_stride, int64_t density_ppm, int dtype,
                                           int32_t *row_ptr, void *workspace, size_t workspace_bytes, void *stream) {
-  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (!clt_model_dtype(dtype)) return CLT_ERR_DTYPE;
   if (!row_ptr || !workspace) return CLT_ERR_ARG;
   if (!clt_encode_threshold_supported(x, w, b, theta, T, d, F, L, x_layer_stride, w_layer_stride, b_layer_stride,
                                       theta_layer_stride, density_ppm, dtype))
@@ -1643,7 +1671,7 @@ extern "C" int clt_encode_threshold_recover(const void *x, const void *w, const 
                                             int64_t pre_layer_stride, int64_t density_ppm, int dtype, int32_t *row_ptr,
                                             int64_t capacity, int32_t *status, void *workspace, size_t workspace_bytes,
                                             void *stream) {
-  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (!clt_model_dtype(dtype)) return CLT_ERR_DTYPE;
   if (!row_ptr || !workspace || !status || !pre || capacity < 0) return CLT_ERR_ARG;
   if (!clt_encode_threshold_supported(x, w, b, theta, T, d, F, L, x_layer_stride, w_layer_stride, b_layer_stride,
                                       theta_layer_stride, density_ppm, dtype))
@@ -1666,6 +1694,9 @@ extern "C" int clt_encode_threshold_recover(const void *x, const void *w, const 
   if (dtype == CLT_BF16)
     rc = dispatch_threshold<bf16_t>(false, pre, T, F, L, pre_layer_stride, theta, CLT_PRED_GE_THETA, rowcnt, row_ptr, nullptr,
                                     nullptr, status + 1, s);
+  else if (dtype == CLT_F16)
+    rc = dispatch_threshold<f16_t>(false, pre, T, F, L, pre_layer_stride, theta, CLT_PRED_GE_THETA, rowcnt, row_ptr, nullptr,
+                                    nullptr, status + 1, s);
   else
     rc = dispatch_threshold<float>(false, pre, T, F, L, pre_layer_stride, theta, CLT_PRED_GE_THETA, rowcnt, row_ptr, nullptr,
                                    nullptr, status + 1, s);
@@ -1678,7 +1709,7 @@ extern "C" int clt_encode_threshold_recover(const void *x, const void *w, const 
 extern "C" int clt_encode_threshold_emit(int64_t T, int64_t F, int64_t L, int64_t density_ppm, int dtype,
                                          const int32_t *row_ptr, int32_t *col, void *val, const int32_t *skip,
                                          void *workspace, size_t workspace_bytes, void *stream) {
-  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (!clt_model_dtype(dtype)) return CLT_ERR_DTYPE;
   if (T <= 0 || F <= 0 || L <= 0 || L > 65535 || !row_ptr || !col || !val || !workspace) return CLT_ERR_ARG;
   const ThreshLayout tl = thresh_layout(T, F, L, density_ppm, dtype);
   if (workspace_bytes < tl.total) return CLT_ERR_WORKSPACE;
@@ -1688,6 +1719,9 @@ extern "C" int clt_encode_threshold_emit(int64_t T, int64_t F, int64_t L, int64_
   if (dtype == CLT_BF16)
     k_tile_emit_all<bf16_t><<<grid, 256, 0, s>>>((int)T, (const uint2 *)(ws + tl.off_meta), tl.nseg, (const uint2 *)(ws + tl.off_tpool),
                                                   tl.tpool_cap, (const uint32_t *)(ws + tl.off_pfx), row_ptr, col, (bf16_t *)val, skip);
+  else if (dtype == CLT_F16)
+    k_tile_emit_all<f16_t><<<grid, 256, 0, s>>>((int)T, (const uint2 *)(ws + tl.off_meta), tl.nseg, (const uint2 *)(ws + tl.off_tpool),
+                                                  tl.tpool_cap, (const uint32_t *)(ws + tl.off_pfx), row_ptr, col, (f16_t *)val, skip);
   else
     k_tile_emit_all<float><<<grid, 256, 0, s>>>((int)T, (const uint2 *)(ws + tl.off_meta), tl.nseg, (const uint2 *)(ws + tl.off_tpool),
                                                  tl.tpool_cap, (const uint32_t *)(ws + tl.off_pfx), row_ptr, col, (float *)val, skip);
@@ -1697,7 +1731,7 @@ extern "C" int clt_encode_threshold_emit(int64_t T, int64_t F, int64_t L, int64_
 extern "C" int clt_encode_collect_supported(const void *x, const void *w, const void *b, int64_t T, int64_t d,
                                             int64_t F, int64_t L, int64_t x_layer_stride, int64_t w_layer_stride,
                                             int64_t b_layer_stride, int64_t k, int dtype) {
-  if (dtype != CLT_F32 && dtype != CLT_BF16) return 0;
+  if (!clt_model_dtype(dtype)) return 0;
   if (T <= 0 || d <= 0 || F <= 0 || L <= 0 || L > 65535 || k <= 0 || !x || !w) return 0;
   if ((double)T * (double)F >= 4294967296.0) return 0;
   if (tile_layout(T, F, L, k, dtype).tpool_cap >= 0xFFF00000ull) return 0;
@@ -1715,7 +1749,7 @@ extern "C" int clt_encode_collect(const void *x, const void *w, const void *b, v
                                   int64_t F, int64_t L, int64_t x_layer_stride, int64_t w_layer_stride,
                                   int64_t b_layer_stride, int64_t pre_layer_stride, int64_t k, int dtype,
                                   void *workspace, size_t workspace_bytes, void *stream) {
-  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (!clt_model_dtype(dtype)) return CLT_ERR_DTYPE;
   if (!pre || !workspace) return CLT_ERR_ARG;
   if (!clt_encode_collect_supported(x, w, b, T, d, F, L, x_layer_stride, w_layer_stride, b_layer_stride, k, dtype))
     return CLT_ERR_ARG;
@@ -1725,6 +1759,9 @@ extern "C" int clt_encode_collect(const void *x, const void *w, const void *b, v
   if (dtype == CLT_BF16)
     return run_encode_collect<bf16_t>(x, w, b, pre, T, d, F, L, x_layer_stride, w_layer_stride, b_layer_stride,
                                       pre_layer_stride, k, dtype, (char *)workspace, s);
+  if (dtype == CLT_F16)
+    return run_encode_collect<f16_t>(x, w, b, pre, T, d, F, L, x_layer_stride, w_layer_stride, b_layer_stride,
+                                      pre_layer_stride, k, dtype, (char *)workspace, s);
   return run_encode_collect<float>(x, w, b, pre, T, d, F, L, x_layer_stride, w_layer_stride, b_layer_stride,
                                    pre_layer_stride, k, dtype, (char *)workspace, s);
 }
@@ -1732,7 +1769,7 @@ extern "C" int clt_encode_collect(const void *x, const void *w, const void *b, v
 extern "C" int clt_collect_select(const void *pre, int64_t T, int64_t F, int64_t L, int64_t pre_layer_stride, int64_t k,
                                   int dtype, int32_t *row_ptr, int32_t *col, void *val, void *workspace,
                                   size_t workspace_bytes, void *stream) {
-  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (!clt_model_dtype(dtype)) return CLT_ERR_DTYPE;
   if (T <= 0 || F <= 0 || L <= 0 || L > 65535 || k <= 0) return CLT_ERR_ARG;
   if (!pre || !row_ptr || !col || !val || !workspace) return CLT_ERR_ARG;
   if (workspace_bytes < clt_encode_collect_workspace_bytes(T, 0, F, L, k, dtype)) return CLT_ERR_WORKSPACE;
@@ -1740,6 +1777,8 @@ extern "C" int clt_collect_select(const void *pre, int64_t T, int64_t F, int64_t
   hipStream_t s = (hipStream_t)stream;
   if (dtype == CLT_BF16)
     return run_collect_select<bf16_t>((const bf16_t *)pre, T, F, L, pre_layer_stride, k, dtype, row_ptr, col, (bf16_t *)val, (char *)workspace, s);
+  if (dtype == CLT_F16)
+    return run_collect_select<f16_t>((const f16_t *)pre, T, F, L, pre_layer_stride, k, dtype, row_ptr, col, (f16_t *)val, (char *)workspace, s);
   return run_collect_select<float>((const float *)pre, T, F, L, pre_layer_stride, k, dtype, row_ptr, col, (float *)val, (char *)workspace, s);
 }
 
@@ -1754,7 +1793,7 @@ extern "C" int clt_batchtopk_select(const void *pre, int64_t T, int64_t F, int64
                                     int64_t k, int mode, const float *mean, const float *denom, int dtype,
                                     int32_t *row_ptr, int32_t *col, void *val, void *workspace,
                                     size_t workspace_bytes, void *stream) {
-  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (!clt_model_dtype(dtype)) return CLT_ERR_DTYPE;
   if (T < 0 || F < 0 || L <= 0 || L > 65535 || !row_ptr) return CLT_ERR_ARG;
   if (mode != CLT_TOPK_PER_LAYER && mode != CLT_TOPK_GLOBAL) return CLT_ERR_ARG;
   hipStream_t s = (hipStream_t)stream;
@@ -1774,6 +1813,11 @@ extern "C" int clt_batchtopk_select(const void *pre, int64_t T, int64_t F, int64
       return run_batchtopk_v<bf16_t, true>((const bf16_t *)pre, T, F, L, pre_layer_stride, k, mean, denom, row_ptr, col, (bf16_t *)val, ws, s);
     return run_batchtopk_v<bf16_t, false>((const bf16_t *)pre, T, F, L, pre_layer_stride, k, mean, denom, row_ptr, col, (bf16_t *)val, ws, s);
   }
+  if (dtype == CLT_F16) {
+    if (mode == CLT_TOPK_GLOBAL)
+      return run_batchtopk_v<f16_t, true>((const f16_t *)pre, T, F, L, pre_layer_stride, k, mean, denom, row_ptr, col, (f16_t *)val, ws, s);
+    return run_batchtopk_v<f16_t, false>((const f16_t *)pre, T, F, L, pre_layer_stride, k, mean, denom, row_ptr, col, (f16_t *)val, ws, s);
+  }
   if (mode == CLT_TOPK_GLOBAL)
     return run_batchtopk_v<float, true>((const float *)pre, T, F, L, pre_layer_stride, k, mean, denom, row_ptr, col, (float *)val, ws, s);
   return run_batchtopk_v<float, false>((const float *)pre, T, F, L, pre_layer_stride, k, mean, denom, row_ptr, col, (float *)val, ws, s);
@@ -1782,7 +1826,7 @@ extern "C" int clt_batchtopk_select(const void *pre, int64_t T, int64_t F, int64
 extern "C" int clt_threshold_count(const void *pre, int64_t T, int64_t F, int64_t L, int64_t pre_layer_stride,
                                    const void *theta, int pred, int dtype, int32_t *row_ptr, void *workspace,
                                    size_t workspace_bytes, void *stream) {
-  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (!clt_model_dtype(dtype)) return CLT_ERR_DTYPE;
   if (T < 0 || F < 0 || L <= 0 || L > 65535 || !row_ptr) return CLT_ERR_ARG;
   if (pred < 0 || pred > 2 || (pred == CLT_PRED_GE_THETA && !theta)) return CLT_ERR_ARG;
   hipStream_t s = (hipStream_t)stream;
@@ -1796,6 +1840,7 @@ extern "C" int clt_threshold_count(const void *pre, int64_t T, int64_t F, int64_
   if (workspace_bytes < (size_t)R * 4) return CLT_ERR_WORKSPACE;
   uint32_t *cnt = (uint32_t *)workspace;
   if (dtype == CLT_BF16) return dispatch_threshold<bf16_t>(false, pre, T, F, L, pre_layer_stride, theta, pred, cnt, row_ptr, nullptr, nullptr, nullptr, s);
+  if (dtype == CLT_F16) return dispatch_threshold<f16_t>(false, pre, T, F, L, pre_layer_stride, theta, pred, cnt, row_ptr, nullptr, nullptr, nullptr, s);
   return dispatch_threshold<float>(false, pre, T, F, L, pre_layer_stride, theta, pred, cnt, row_ptr, nullptr, nullptr, nullptr, s);
 }
 
@@ -1845,7 +1890,7 @@ static int scratch_of_current_device(uint32_t **out) {
 
 extern "C" int clt_threshold_count_static(const void *pre, int64_t T, int64_t F, int64_t L, int64_t pre_layer_stride,
                                           const void *theta, int pred, int dtype, int32_t *row_ptr, void *stream) {
-  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (!clt_model_dtype(dtype)) return CLT_ERR_DTYPE;
   if (T < 0 || F < 0 || L <= 0 || L > 65535 || !row_ptr) return CLT_ERR_ARG;
   if (L * T > STATIC_ROWS_MAX) return CLT_ERR_RANGE;
   uint32_t *cnt = nullptr;
@@ -1859,20 +1904,21 @@ extern "C" int clt_threshold_count_static(const void *pre, int64_t T, int64_t F,
 extern "C" int clt_threshold_emit(const void *pre, int64_t T, int64_t F, int64_t L, int64_t pre_layer_stride,
                                   const void *theta, int pred, int dtype, const int32_t *row_ptr, int32_t *col,
                                   void *val, const int32_t *skip, void *stream) {
-  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (!clt_model_dtype(dtype)) return CLT_ERR_DTYPE;
   if (T < 0 || F < 0 || L <= 0 || L > 65535 || !row_ptr) return CLT_ERR_ARG;
   if (pred < 0 || pred > 2 || (pred == CLT_PRED_GE_THETA && !theta)) return CLT_ERR_ARG;
   if (T == 0 || F == 0) return CLT_OK;
   if (!pre || !col || !val) return CLT_ERR_ARG;
   hipStream_t s = (hipStream_t)stream;
   if (dtype == CLT_BF16) return dispatch_threshold<bf16_t>(true, pre, T, F, L, pre_layer_stride, theta, pred, nullptr, (int32_t *)row_ptr, col, val, skip, s);
+  if (dtype == CLT_F16) return dispatch_threshold<f16_t>(true, pre, T, F, L, pre_layer_stride, theta, pred, nullptr, (int32_t *)row_ptr, col, val, skip, s);
   return dispatch_threshold<float>(true, pre, T, F, L, pre_layer_stride, theta, pred, nullptr, (int32_t *)row_ptr, col, val, skip, s);
 }
 
 extern "C" int clt_selected_min_accumulate(const int32_t *row_ptr, const int32_t *col, const void *val, const float *mean,
                                            const float *denom, int64_t T, int64_t F, int64_t L, int dtype, void *sum,
                                            void *count, void *workspace, size_t workspace_bytes, void *stream) {
-  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (!clt_model_dtype(dtype)) return CLT_ERR_DTYPE;
   if (T <= 0 || F <= 0 || L <= 0 || !row_ptr || !mean || !denom || !sum || !count || !workspace) return CLT_ERR_ARG;
   if (workspace_bytes < (size_t)L * (size_t)F * 4) return CLT_ERR_WORKSPACE;
   hipStream_t s = (hipStream_t)stream;
@@ -1882,6 +1928,9 @@ extern "C" int clt_selected_min_accumulate(const int32_t *row_ptr, const int32_t
   if (dtype == CLT_BF16) {
     k_selected_min<bf16_t><<<2048, 256, 0, s>>>(row_ptr, col, (const bf16_t *)val, mean, denom, T, F, L, keys);
     k_selected_min_accumulate<bf16_t><<<256, 256, 0, s>>>(keys, n, (bf16_t *)sum, (bf16_t *)count);
+  } else if (dtype == CLT_F16) {
+    k_selected_min<f16_t><<<2048, 256, 0, s>>>(row_ptr, col, (const f16_t *)val, mean, denom, T, F, L, keys);
+    k_selected_min_accumulate<f16_t><<<256, 256, 0, s>>>(keys, n, (f16_t *)sum, (f16_t *)count);
   } else {
     k_selected_min<float><<<2048, 256, 0, s>>>(row_ptr, col, (const float *)val, mean, denom, T, F, L, keys);
     k_selected_min_accumulate<float><<<256, 256, 0, s>>>(keys, n, (float *)sum, (float *)count);
@@ -1899,7 +1948,7 @@ extern "C" int clt_tokentopk_select(const void *pre, int64_t T, int64_t F, int64
                                     int64_t kk, int mode, const float *mean, const float *denom, int dtype,
                                     int32_t *row_ptr, int32_t *col, void *val, void *workspace,
                                     size_t workspace_bytes, void *stream) {
-  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (!clt_model_dtype(dtype)) return CLT_ERR_DTYPE;
   if (T < 0 || F < 0 || L <= 0 || L > 64 || !row_ptr) return CLT_ERR_ARG;
   if (mode != CLT_TOPK_PER_LAYER && mode != CLT_TOPK_GLOBAL) return CLT_ERR_ARG;
   hipStream_t s = (hipStream_t)stream;
@@ -1919,6 +1968,11 @@ extern "C" int clt_tokentopk_select(const void *pre, int64_t T, int64_t F, int64
     if (mode == CLT_TOPK_GLOBAL)
       return run_tokentopk<bf16_t, true>((const bf16_t *)pre, T, F, L, pre_layer_stride, kk, mean, denom, row_ptr, col, (bf16_t *)val, ws, s);
     return run_tokentopk<bf16_t, false>((const bf16_t *)pre, T, F, L, pre_layer_stride, kk, mean, denom, row_ptr, col, (bf16_t *)val, ws, s);
+  }
+  if (dtype == CLT_F16) {
+    if (mode == CLT_TOPK_GLOBAL)
+      return run_tokentopk<f16_t, true>((const f16_t *)pre, T, F, L, pre_layer_stride, kk, mean, denom, row_ptr, col, (f16_t *)val, ws, s);
+    return run_tokentopk<f16_t, false>((const f16_t *)pre, T, F, L, pre_layer_stride, kk, mean, denom, row_ptr, col, (f16_t *)val, ws, s);
   }
   if (mode == CLT_TOPK_GLOBAL)
     return run_tokentopk<float, true>((const float *)pre, T, F, L, pre_layer_stride, kk, mean, denom, row_ptr, col, (float *)val, ws, s);

@@ -59,7 +59,7 @@ __global__ __launch_bounds__(256) void k_colstats_vec(const T *pre, float *mean,
     if constexpr (sizeof(T) == 2) {
       const uint32_t u[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
-      for (int j = 0; j < 4; ++j) { x[2 * j] = __uint_as_float(u[j] << 16); x[2 * j + 1] = __uint_as_float(u[j] & 0xFFFF0000u); }
+      for (int j = 0; j < 4; ++j) unpack_pair<T>(u[j], x[2 * j], x[2 * j + 1]);
     } else {
       x[0] = __uint_as_float(w.x); x[1] = __uint_as_float(w.y); x[2] = __uint_as_float(w.z); x[3] = __uint_as_float(w.w);
     }
@@ -132,7 +132,7 @@ extern "C" const char *clt_error_string(int code) {
   switch (code) {
     case CLT_OK: return "ok";
     case CLT_ERR_ARG: return "bad argument (null pointer, negative size or unsupported combination)";
-    case CLT_ERR_DTYPE: return "dtype must be CLT_F32 or CLT_BF16";
+    case CLT_ERR_DTYPE: return "dtype must be CLT_F32, CLT_BF16 or CLT_F16 (CLT_F16: forward-path entry points only)";
     case CLT_ERR_WORKSPACE: return "workspace too small";
     case CLT_ERR_LAUNCH: return "HIP reported an error at kernel launch";
     case CLT_ERR_ALIGN: return "pointer or row pitch not aligned as required";
@@ -143,18 +143,20 @@ extern "C" const char *clt_error_string(int code) {
 
 static int run_colstats(const void *pre, float *mean, float *denom, float *stdv, int64_t T, int64_t F, int64_t L,
                         int64_t pre_layer_stride, int dtype, void *stream) {
-  if (dtype != CLT_F32 && dtype != CLT_BF16) return CLT_ERR_DTYPE;
+  if (!clt_model_dtype(dtype)) return CLT_ERR_DTYPE;
   if (T <= 0 || F <= 0 || L <= 0 || L > 65535 || !pre || !mean || !denom) return CLT_ERR_ARG;
   hipStream_t s = (hipStream_t)stream;
-  const int V = dtype == CLT_BF16 ? 8 : 4;
+  const int V = 16 / clt_elem_bytes(dtype);
   if (F % V == 0 && clt_aligned16(pre) && (pre_layer_stride % V) == 0) {
     dim3 gridv((unsigned)clt_ceil_div(F, 32 * V), (unsigned)L);
     if (dtype == CLT_BF16) k_colstats_vec<bf16_t><<<gridv, 256, 0, s>>>((const bf16_t *)pre, mean, denom, stdv, T, F, pre_layer_stride);
+    else if (dtype == CLT_F16) k_colstats_vec<f16_t><<<gridv, 256, 0, s>>>((const f16_t *)pre, mean, denom, stdv, T, F, pre_layer_stride);
     else k_colstats_vec<float><<<gridv, 256, 0, s>>>((const float *)pre, mean, denom, stdv, T, F, pre_layer_stride);
     return clt_check_launch();
   }
   dim3 grid((unsigned)clt_ceil_div(F, 64), (unsigned)L);
   if (dtype == CLT_BF16) k_colstats<bf16_t><<<grid, 256, 0, s>>>((const bf16_t *)pre, mean, denom, stdv, T, F, pre_layer_stride);
+  else if (dtype == CLT_F16) k_colstats<f16_t><<<grid, 256, 0, s>>>((const f16_t *)pre, mean, denom, stdv, T, F, pre_layer_stride);
   else k_colstats<float><<<grid, 256, 0, s>>>((const float *)pre, mean, denom, stdv, T, F, pre_layer_stride);
   return clt_check_launch();
 }

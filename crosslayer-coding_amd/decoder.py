@@ -307,7 +307,7 @@ class Decoder(nn.Module):
                 best = min(best, a.elapsed_time(b) * 1e-3)
             return best
 
-        esize = 2 if dtype == torch.bfloat16 else 4
+        esize = torch.finfo(dtype).bits // 8
         # the dense product itself, on scratch operands of the real shape
         x = torch.zeros((1, T, F), dtype=dtype, device=dev)
         w = torch.zeros((1, d, F), dtype=dtype, device=dev)
@@ -347,9 +347,9 @@ class Decoder(nn.Module):
         if cfg.decoder_tying != "per_target" or not self.dense_route or skip_add is not None:
             return t_end
         T, F, d = surv.T, surv.F, cfg.d_model
-        esize = 2 if surv.dtype == torch.bfloat16 else 4
+        esize = torch.finfo(surv.dtype).bits // 8
         # shapes the MFMA kernel of clt_encode takes (K = F in whole pairs of 128-byte stages, 256 x 256 tiles)
-        if surv.dtype not in (torch.bfloat16, torch.float32) or T < 256 or d < 256 or d % 4 or F % (256 // esize):
+        if surv.dtype not in (torch.bfloat16, torch.float16, torch.float32) or T < 256 or d < 256 or d % 4 or F % (256 // esize):
             return t_end
         gather_rate, mfma_rate = self.route_rates(T, F, d, surv.dtype)
         dense_s = 2.0 * T * F * d / mfma_rate

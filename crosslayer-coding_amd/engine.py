@@ -114,39 +114,6 @@ def _stream(t: torch.Tensor) -> int:
     return nat.current_stream(t.device)
 
 
-# A float16 model (config.clt_dtype = "float16") computes on the float32 kernels from float16 parameters;
-# while it does, the results of dense products are rounded to float16 as the reference's tensors would be.
-_EMULATED_DTYPE: Optional[torch.dtype] = None
-
-
-class emulate_dtype:
-    """Context: dense products and thresholds are rounded to ``dtype`` (values stay in the kernels' dtype)."""
-
-    def __init__(self, dtype: Optional[torch.dtype]):
-        self.dtype, self.prev = dtype, None
-
-    def __enter__(self):
-        global _EMULATED_DTYPE
-        self.prev, _EMULATED_DTYPE = _EMULATED_DTYPE, self.dtype
-        return self
-
-    def __exit__(self, *exc):
-        global _EMULATED_DTYPE
-        _EMULATED_DTYPE = self.prev
-        return False
-
-
-def emulated_dtype() -> Optional[torch.dtype]:
-    return _EMULATED_DTYPE
-
-
-def round_emulated(t: torch.Tensor) -> torch.Tensor:
-    """``t`` rounded in place to the emulated dtype, if one is set."""
-    if _EMULATED_DTYPE is not None and t.numel() > 0:
-        t.copy_(t.to(_EMULATED_DTYPE))
-    return t
-
-
 def encode(x: torch.Tensor, w: torch.Tensor, b: Optional[torch.Tensor],
            out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """pre[l] = x[l] @ w[l].T + b[l] for stacked layers (parallel.py:286 per layer)."""
@@ -165,7 +132,7 @@ def encode(x: torch.Tensor, w: torch.Tensor, b: Optional[torch.Tensor],
                           x.stride(0), w.stride(0), b.stride(0) if b is not None else 0, out.stride(0),
                           nat.dtype_code(x.dtype), _stream(x))
     nat.check(code, "clt_encode")
-    return round_emulated(out)
+    return out
 
 
 def encode_segmented(x: torch.Tensor, w: torch.Tensor, n_seg: int, d_seg: int, x_seg_stride: int, x_row_stride: int,

@@ -127,7 +127,7 @@ class DeviceActivationFeed:
 
     ``dtype`` is both the stored element type the bytes are read as and the type of the batch,
     as in the reference (manifest_activation_store.py:881-886); ``out_dtype`` may name a
-    different batch type (float32 or bfloat16)."""
+    different batch type (float32, bfloat16 or float16)."""
 
     def __init__(self, num_layers: int, d_model: int, dtype: Union[str, torch.dtype] = "bfloat16",
                  device: Union[str, torch.device] = "cuda:0", normalization_method: str = "none",
@@ -142,8 +142,8 @@ class DeviceActivationFeed:
         if self.dtype not in _SRC_CODES:
             raise ValueError(f"Unsupported store dtype {self.dtype}")
         self.out_dtype = out_dtype or self.dtype
-        if self.out_dtype not in (torch.float32, torch.bfloat16):
-            raise ValueError(f"Unsupported batch dtype {self.out_dtype}: the kernels take float32 or bfloat16")
+        if self.out_dtype not in _SRC_CODES:
+            raise ValueError(f"Unsupported batch dtype {self.out_dtype}: the kernels take float32, bfloat16 or float16")
         self.bytes_per_element = torch.finfo(self.dtype).bits // 8
         self.bytes_per_row = d_model * self.bytes_per_element
         self.normalization_method = normalization_method

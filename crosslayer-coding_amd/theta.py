@@ -57,8 +57,6 @@ class ThetaManager(nn.Module):
         """exp(log_threshold) for all layers, rounded to ``dtype``: [L, F], contiguous."""
         assert self.log_threshold is not None
         th = torch.exp(self.log_threshold.detach())
-        if engine.emulated_dtype() is not None:        # a float16 model on the float32 kernels: theta as it would round
-            th = th.to(engine.emulated_dtype())
         return th.to(dtype).contiguous()
 
     def jumprelu(self, x: torch.Tensor, layer_idx: int) -> torch.Tensor:
@@ -69,8 +67,6 @@ class ThetaManager(nn.Module):
             logger.error(f"Rank {self.rank}: Invalid layer_idx {layer_idx} for log_threshold. Returning input.")
             return x.to(device=self.device, dtype=self.dtype)
         theta = torch.exp(self.log_threshold[layer_idx])
-        if engine.emulated_dtype() is not None:
-            theta = theta.to(engine.emulated_dtype())
         theta = theta.to(device=self.device, dtype=self.dtype)
         return cast(torch.Tensor, JumpReLU.apply(x, theta, self.bandwidth))
 

@@ -11,8 +11,13 @@
  * Conventions
  *   - every pointer is a DEVICE pointer unless its name ends in _host;
  *   - sizes and strides are int64 element counts (strides between layers);
- *   - `dtype` is CLT_F32 or CLT_BF16 and names the model dtype (inputs, weights,
- *     pre-activations, survivor values, outputs unless said otherwise);
+ *   - `dtype` is CLT_F32, CLT_BF16 or CLT_F16 and names the model dtype (inputs, weights,
+ *     pre-activations, survivor values, outputs unless said otherwise).  CLT_F16 (IEEE half,
+ *     fp32 accumulation, one rounding per product) is taken by the forward-path entry points -
+ *     encoder, column statistics, selection, thresholds, packing, decode, densify, decoder norms,
+ *     the dense accumulation of per-target tying, the evaluator reductions and the store feed;
+ *     the gradient, optimiser and tile entry points (and clt_encode_segmented, which serves the
+ *     threshold gradient) return CLT_ERR_DTYPE for it;
  *   - `stream` is a hipStream_t passed as void* (NULL = the null stream);
  *   - functions launch asynchronously on `stream` and return CLT_OK or a negative
  *     error code; nothing is allocated or freed inside;
@@ -32,11 +37,11 @@ extern "C" {
 
 #define CLT_F32 0
 #define CLT_BF16 1
-#define CLT_F16 2 /* source dtype of clt_feed_gather only */
+#define CLT_F16 2 /* forward-path entry points only, see above */
 
 #define CLT_OK 0
 #define CLT_ERR_ARG (-1)       /* null pointer, negative size, unsupported combination */
-#define CLT_ERR_DTYPE (-2)     /* dtype is not CLT_F32 / CLT_BF16 */
+#define CLT_ERR_DTYPE (-2)     /* dtype is not one this entry point takes */
 #define CLT_ERR_WORKSPACE (-3) /* workspace smaller than clt_*_workspace_bytes() says */
 #define CLT_ERR_LAUNCH (-4)    /* HIP reported an error when launching */
 #define CLT_ERR_ALIGN (-5)     /* a pointer or row pitch is not 16-byte aligned */
@@ -672,7 +677,7 @@ int clt_probe_gather(const void *table, int64_t n_rows, int64_t row_bytes, const
 
 /* ---- activation-store feed -----------------------------------------------------
  * clt_feed_gather: rows of one stored chunk -> rows [out_row0, out_row0 + n) of the batch slabs
- *   x_out, tgt_out [L][T][d] (out_dtype CLT_F32 / CLT_BF16), for all layers, inputs and targets.
+ *   x_out, tgt_out [L][T][d] (out_dtype CLT_F32 / CLT_BF16 / CLT_F16), for all layers, inputs and targets.
  *     out[l][out_row0 + j][:] = cast(norm(float(src_l[row_index[j]][:])))
  *   src is the chunk (or a fetched slice of it) in the store's layout
  *   Layer0_Inputs | Layer0_Targets | Layer1_Inputs | ... (ManifestActivationStore._fetch_slice,

@@ -13,10 +13,10 @@ from oracle import clt_oracle as orc
 
 pytestmark = pytest.mark.gpu
 
-TOL = {torch.float32: 1e-5, torch.bfloat16: 1e-2}
+TOL = {torch.float32: 1e-5, torch.bfloat16: 1e-2, torch.float16: 2e-3}
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 def test_accumulate_dense_is_the_running_sum_in_the_model_dtype(dev, dtype):
     g = torch.Generator().manual_seed(3)
     L, T, F = 3, 70, 200
@@ -44,7 +44,7 @@ def test_accumulate_dense_is_the_running_sum_in_the_model_dtype(dev, dtype):
     assert torch.equal(acc.cpu(), want)
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16", "float16"])
 @pytest.mark.parametrize("affine", [False, True])
 def test_dense_route_matches_the_oracle_and_the_gather_route(dev, dtype, affine):
     tdt = getattr(torch, dtype)
@@ -64,7 +64,7 @@ def test_dense_route_matches_the_oracle_and_the_gather_route(dev, dtype, affine)
     model.load_state_dict(sd)
     inputs = {l: x[l].to(dev) for l in range(L)}
     # rates of a large shape: at this size the measured ones would (rightly) keep every target on the gather
-    model.decoder_module.rate_override = (14.5e12, 1.0e15 if tdt == torch.bfloat16 else 1.0e14)
+    model.decoder_module.rate_override = (14.5e12, 1.0e14 if tdt == torch.float32 else 1.0e15)
     dense = model(inputs)
     route = dict(model.decoder_module.last_route)
     assert route["dense_targets"][0] < route["dense_targets"][1] == L      # the dense route was taken

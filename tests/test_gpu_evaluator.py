@@ -31,13 +31,13 @@ def dense_cases(dtype):
     return a.to(dtype)
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 def test_sparsity_density_and_dead_counters_from_dense_activations(dev, dtype):
     a = dense_cases(dtype)
     L, T, F = a.shape
     acts = {l: a[l] for l in range(L)}
     cfg = cca.CLTConfig(num_layers=L, d_model=8, num_features=F, activation_fn="relu",
-                        clt_dtype="float32" if dtype == torch.float32 else "bfloat16")
+                        clt_dtype=str(dtype).split(".")[1])
     model = cca.CrossLayerTranscoder(cfg, None, dev)
     ev = cca.CLTEvaluator(model, dev)
     dev_acts = {l: v.to(dev) for l, v in acts.items()}
@@ -81,7 +81,7 @@ def test_empty_inputs_follow_the_reference_branches(dev):
         cca.CLTEvaluator(ev.model, dev, normalization_method="bogus")
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("method", ["none", "mean_std", "sqrt_d_model"])
 def test_reconstruction_metrics_match_the_oracle(dev, dtype, method):
     g = torch.Generator().manual_seed(8)
@@ -117,7 +117,7 @@ def test_reconstruction_metric_branches_for_constant_targets(dev):
     assert m["layerwise/explained_variance"]["layer_0"] == 1.0 and m["layerwise/normalized_mse"]["layer_0"] == 0.0
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16", "float16"])
 def test_compute_metrics_on_a_model_matches_the_oracle_end_to_end(dev, dtype):
     wl = BASE.scaled("ev", dtype=dtype, num_layers=3, d_model=128, num_features=512, tokens=256, k=12)
     model, inputs, _ = synth.build_model(wl, dev)

@@ -59,7 +59,7 @@ def same_bits(a, b):
 def test_batches_equal_the_oracle_bit_for_bit(dev, dtype, method, source):
     L, d = 3, 72
     tdt = DT[dtype]
-    out_dt = torch.bfloat16 if dtype == "float16" else tdt     # the kernels downstream take float32 / bfloat16
+    out_dt = tdt
     chunks = make_chunks(L, d, [40, 17, 64], tdt, seed=3)
     js = stats_json(L, d, seed=4) if method == "mean_std" else None
     feed = cca.DeviceActivationFeed(L, d, dtype=dtype, device=dev, normalization_method=method, norm_stats=js, out_dtype=out_dt)
@@ -72,15 +72,8 @@ def test_batches_equal_the_oracle_bit_for_bit(dev, dtype, method, source):
         idxs = manifest[rng.permutation(len(manifest))[:50]]
         ins, tgs = feed.parse_batch(idxs, wire(chunks) if source == "wire" else None)
         tabs = oracle_tables(js, L) if js else {}
-        # the oracle works in the store dtype as the reference does; a float16 store is compared after the
-        # same fp32 arithmetic rounded to the batch dtype instead
-        if dtype == "float16":
-            want_in, want_tg = orc.store_parse_batch(idxs, wire({c: t.float() for c, t in chunks.items()}), num_layers=L,
-                                                     d_model=d, dtype=torch.float32, method=method, **tabs)
-            want_in = {l: v.to(out_dt) for l, v in want_in.items()}
-            want_tg = {l: v.to(out_dt) for l, v in want_tg.items()}
-        else:
-            want_in, want_tg = orc.store_parse_batch(idxs, wire(chunks), num_layers=L, d_model=d, dtype=tdt, method=method, **tabs)
+        # the oracle works in the store dtype, as the reference does
+        want_in, want_tg = orc.store_parse_batch(idxs, wire(chunks), num_layers=L, d_model=d, dtype=tdt, method=method, **tabs)
         for l in range(L):
             assert same_bits(ins[l], want_in[l]), (batch, l)
             assert same_bits(tgs[l], want_tg[l]), (batch, l)

@@ -16,7 +16,10 @@ from oracle import clt_oracle as orc
 
 pytestmark = pytest.mark.gpu
 
-TOL = {torch.float32: 1e-5, torch.bfloat16: 1e-2}
+TOL = {torch.float32: 1e-5, torch.bfloat16: 1e-2, torch.float16: 2e-3}
+DTYPES = [torch.float32, torch.bfloat16, torch.float16]
+# relative width of the band around a ranking threshold inside which two correct implementations may differ
+BAND = {torch.float32: 1e-5, torch.bfloat16: 2.0 ** -6, torch.float16: 2.0 ** -9}
 
 
 def dense_from(surv):
@@ -33,7 +36,7 @@ def check_rows_sorted(surv):
 
 
 # ---- encoder --------------------------------------------------------------------------------
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("L,T,d,F", [(1, 30, 8, 16), (2, 300, 64, 136), (3, 257, 96, 260), (1, 5, 7, 9), (2, 512, 768, 512)])
 def test_encode_parity(dev, dtype, L, T, d, F):
     g = torch.Generator().manual_seed(L * 1000 + T)
@@ -92,7 +95,7 @@ def test_encode_segmented_rejects_shapes_the_matrix_kernel_cannot_take(dev):
         engine.encode_segmented(x, w, 3, 32, 256 * 32, 32, 256 * 32, 32, 256, 256)   # an odd number of K pieces
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("L,T,F,k", [(1, 2, 4, 2), (2, 64, 256, 8), (3, 100, 1000, 17), (1, 33, 77, 5),
                                      (2, 16, 64, 64), (2, 16, 64, 100), (1, 1, 8, 3), (2, 512, 2048, 40)])
 def test_batchtopk_per_layer_bit_exact(dev, dtype, L, T, F, k):
@@ -115,7 +118,7 @@ def test_batchtopk_reference_known_answer(dev):
     assert torch.equal(dense_from(surv)[0], torch.tensor([[0.0, 0.0, 3.0, 4.0], [5.0, 0.0, 0.0, 3.5]]))
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_batchtopk_heavy_ties_lowest_index(dev, dtype):
     g = torch.Generator().manual_seed(11)
     pre = (torch.randint(-4, 5, (2, 96, 520), generator=g).float() * 0.25).to(dtype)
@@ -132,7 +135,7 @@ def test_batchtopk_heavy_ties_lowest_index(dev, dtype):
             assert torch.equal(torch.sort(flat).values, m.view(-1).nonzero().view(-1))
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_batchtopk_special_values(dev, dtype):
     g = torch.Generator().manual_seed(5)
     pre = torch.randn(1, 40, 128, generator=g).to(dtype)
@@ -157,7 +160,7 @@ def test_batchtopk_all_equal_and_constant_rows(dev):
     assert torch.equal(got, ref) and int((got != 0).sum()) == 2 * 500
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_batchtopk_outlier_rows_overflow_segments(dev, dtype):
     # a few rows hold nearly all survivors: their candidate segments overflow and are re-read
     g = torch.Generator().manual_seed(9)
@@ -171,7 +174,7 @@ def test_batchtopk_outlier_rows_overflow_segments(dev, dtype):
     assert torch.equal(dense_from(surv), oracle_per_layer(pre, k))
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_batchtopk_candidate_pool_overflow_falls_back_to_dense_rows(dev, dtype):
     # half of all values tie at the top: the sampled cut admits ~500x more candidates than the
     # pool holds, so most rows are re-read from the matrix; the result must not change
@@ -210,13 +213,13 @@ def threshold_fused_vs_separate(x, w, b, theta, dev, density_ppm=200000):
 
 
 def assert_same_list(got, ref, dtype):
-    iv = torch.int16 if dtype == torch.bfloat16 else torch.int32
+    iv = torch.int32 if dtype == torch.float32 else torch.int16
     assert torch.equal(got.row_ptr.cpu(), ref.row_ptr.cpu())
     assert torch.equal(got.col.cpu(), ref.col.cpu())
     assert torch.equal(got.val.cpu().view(iv), ref.val.cpu().view(iv))
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("L,T,d,F", [(1, 256, 128, 256), (2, 512, 256, 1024), (3, 256, 768, 512)])
 def test_encode_threshold_matches_separate_and_oracle(dev, dtype, L, T, d, F):
     g = torch.Generator().manual_seed(L * 17 + T + F)
@@ -233,7 +236,7 @@ def test_encode_threshold_matches_separate_and_oracle(dev, dtype, L, T, d, F):
         assert torch.equal(dense[l], orc.jumprelu_forward(pre[l], theta[l]))
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_encode_threshold_special_thresholds_and_values(dev, dtype):
     # zero / huge / infinite thresholds and NaN, +-inf, -0.0 pre-activations (reached through
     # crafted inputs: one-hot weights copy input values into the pre-activations)
@@ -278,12 +281,12 @@ def fused_vs_separate(x, w, b, k, dev):
     torch.cuda.synchronize()
     assert torch.equal(got.row_ptr.cpu(), ref.row_ptr.cpu())
     assert torch.equal(got.col.cpu(), ref.col.cpu())
-    assert torch.equal(got.val.cpu().view(torch.int16 if x.dtype == torch.bfloat16 else torch.int32),
-                       ref.val.cpu().view(torch.int16 if x.dtype == torch.bfloat16 else torch.int32))
+    assert torch.equal(got.val.cpu().view(torch.int32 if x.dtype == torch.float32 else torch.int16),
+                       ref.val.cpu().view(torch.int32 if x.dtype == torch.float32 else torch.int16))
     return pre.cpu(), got
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("L,T,d,F,k", [(1, 256, 128, 256, 3), (2, 512, 256, 1024, 20), (3, 256, 768, 512, 64),
                                        (2, 768, 128, 2048, 200)])
 def test_encode_collect_matches_separate_and_oracle(dev, dtype, L, T, d, F, k):
@@ -297,7 +300,7 @@ def test_encode_collect_matches_separate_and_oracle(dev, dtype, L, T, d, F, k):
     assert torch.equal(dense_from(got), oracle_per_layer(pre, k))
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_encode_collect_heavy_ties(dev, dtype):
     # small-integer inputs and weights: the pre-activations are exact small integers, so
     # thousands of them tie at the threshold and the lowest flat indices must win
@@ -309,7 +312,7 @@ def test_encode_collect_heavy_ties(dev, dtype):
     assert torch.equal(dense_from(got), oracle_per_layer(pre, k))
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_encode_collect_unusable_cut_takes_streaming_route(dev, dtype):
     # almost every pre-activation is exactly 0 and K reaches into the zeros: every element
     # reaches the sampled cut, the candidate pool overflows, and the layer must be redone from
@@ -337,7 +340,7 @@ def test_encode_collect_all_selected_and_shape_gate(dev):
     assert not engine.encode_collect_supported(x.to(dev), w.to(dev), None, 0)
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("L,T,F,k", [(2, 2, 2, 1), (3, 64, 128, 6), (4, 200, 520, 12)])
 def test_batchtopk_global(dev, dtype, L, T, F, k):
     g = torch.Generator().manual_seed(L + T + F)
@@ -354,7 +357,7 @@ def test_batchtopk_global(dev, dtype, L, T, F, k):
     z = torch.cat([orc.zscore_for_ranking(pre[l]) for l in range(L)], dim=1).double()
     flat = z.reshape(-1)
     kth = torch.topk(flat, min(k * T, flat.numel())).values[-1]
-    band = (2.0 ** -6 if dtype == torch.bfloat16 else 1e-5) * max(abs(float(kth)), 1e-3)
+    band = BAND[dtype] * max(abs(float(kth)), 1e-3)
     zl = torch.stack([z[:, l * F:(l + 1) * F] for l in range(L)])
     sure = (zl - kth).abs() > band
     assert torch.equal((got != 0) & sure, (ref != 0) & sure)
@@ -363,7 +366,7 @@ def test_batchtopk_global(dev, dtype, L, T, F, k):
         assert torch.equal(got, ref)
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("L,T,F,k", [(4, 200, 520, 12), (3, 512, 2048, 20)])
 def test_batchtopk_global_is_bit_exact_given_the_column_statistics(dev, dtype, L, T, F, k):
     # The only thing that can differ between two correct implementations of the global helper is the last
@@ -372,7 +375,7 @@ def test_batchtopk_global_is_bit_exact_given_the_column_statistics(dev, dtype, L
     # exactly the k*T largest of them over the [T, L*F] block, ties to the lowest flat index.
     g = torch.Generator().manual_seed(L * 7 + F)
     pre = (torch.randn(L, T, F, generator=g) * (1 + torch.arange(L).view(L, 1, 1))).to(dtype)
-    if dtype == torch.bfloat16:
+    if dtype != torch.float32:
         pre[1, :, 5] = pre[0, :, 5]                 # equal columns: equal z-scores, ties across layers
     pre_dev = pre.to(dev)
     mean, denom = engine.colstats(pre_dev)
@@ -388,7 +391,7 @@ def test_batchtopk_global_is_bit_exact_given_the_column_statistics(dev, dtype, L
     assert torch.equal(got, want)
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_batchtopk_global_outlier_tokens(dev, dtype):
     # two tokens stand far out of the batch in every feature: under the batch-wide cut nearly all of
     # their values are candidates, more per step of the streaming pass than its buffer holds
@@ -406,7 +409,7 @@ def test_batchtopk_global_outlier_tokens(dev, dtype):
     ref = torch.stack([ref[l] for l in range(L)])
     z = torch.cat([orc.zscore_for_ranking(pre[l]) for l in range(L)], dim=1).double()
     kth = torch.topk(z.reshape(-1), k * T).values[-1]
-    band = (2.0 ** -6 if dtype == torch.bfloat16 else 1e-5) * max(abs(float(kth)), 1e-3)
+    band = BAND[dtype] * max(abs(float(kth)), 1e-3)
     zl = torch.stack([z[:, l * F:(l + 1) * F] for l in range(L)])
     sure = (zl - kth).abs() > band
     assert torch.equal((got != 0) & sure, (ref != 0) & sure)
@@ -424,7 +427,7 @@ def test_batchtopk_global_closed_form(dev):
 
 
 # ---- TokenTopK -----------------------------------------------------------------------------------
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("L,T,F,kk", [(1, 2, 4, 2), (2, 40, 256, 7), (3, 33, 1000, 50), (1, 5, 77, 77), (2, 9, 64, 100)])
 def test_tokentopk_per_layer_bit_exact(dev, dtype, L, T, F, kk):
     g = torch.Generator().manual_seed(T * 3 + F)
@@ -464,7 +467,7 @@ def test_tokentopk_reference_known_answers(dev):
     assert torch.equal(xb.grad.cpu(), torch.tensor([[0.0, 0.0, 1.0, 1.0], [1.0, 0.0, 0.0, 1.0]]))
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_tokentopk_global(dev, dtype):
     g = torch.Generator().manual_seed(4)
     L, T, F, kk = 3, 50, 128, 9
@@ -480,13 +483,13 @@ def test_tokentopk_global(dev, dtype):
     z = torch.stack([orc.zscore_for_ranking(pre[l]) for l in range(L)]).double()       # [L, T, F]
     zt = z.permute(1, 0, 2).reshape(T, L * F)
     kth = torch.topk(zt, kk, dim=1).values[:, -1]                                        # per token
-    band = (2.0 ** -6 if dtype == torch.bfloat16 else 1e-5) * kth.abs().clamp(min=1e-3)
+    band = BAND[dtype] * kth.abs().clamp(min=1e-3)
     sure = (z - kth.view(1, T, 1)).abs() > band.view(1, T, 1)
     assert torch.equal((got != 0) & sure, (ref != 0) & sure)
 
 
 # ---- threshold activations ---------------------------------------------------------------------
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("L,T,F", [(1, 7, 7), (2, 100, 264), (3, 64, 1000)])
 def test_jumprelu_and_relu_exact(dev, dtype, L, T, F):
     g = torch.Generator().manual_seed(T + F)
@@ -514,7 +517,7 @@ def test_jumprelu_reference_known_answer(dev):
 
 
 # ---- pack / densify / norms -------------------------------------------------------------------
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_pack_is_transpose(dev, dtype):
     w = torch.randn(70, 130).to(dtype)
     out = engine.alloc_packed(1, 130, 70, dtype, dev)[0]
@@ -536,7 +539,7 @@ def make_decoder(L, d, F, tying, dtype, g):
     return names, w, b
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("tying", ["none", "per_source", "per_target"])
 @pytest.mark.parametrize("L,T,d,F", [(2, 30, 8, 16), (3, 70, 768, 256), (4, 33, 100, 72), (3, 20, 2048, 64)])
 def test_decode_sparse_parity(dev, dtype, tying, L, T, d, F):
@@ -580,7 +583,7 @@ def test_decode_sparse_parity(dev, dtype, tying, L, T, d, F):
         assert sub.dtype == torch.float32 and orc.rel_l2(sub[t], ref) <= TOL[dtype]
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("tying,d", [("none", 768), ("per_source", 768), ("none", 1024), ("none", 512), ("per_source", 2048),
                                      ("none", 640), ("per_source", 320), ("per_target", 768), ("none", 192),
                                      ("per_source", 4096), ("none", 200)])
@@ -621,7 +624,7 @@ def test_decode_sliced_matches_single_pass(dev, dtype, tying, d):
         assert orc.rel_l2(sliced[t], ref) <= TOL[dtype]
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_decode_line_schedule_with_feature_slices(dev, dtype):
     # F x 128 bytes above 3.25 MiB: the line kernel cuts the feature axis in two and keeps two partial rows
     g = torch.Generator().manual_seed(4)
@@ -671,7 +674,7 @@ def test_decode_linearity_property(dev):
     assert torch.equal(o2, 2 * o1)
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("tying", ["none", "per_source", "per_target"])
 def test_decoder_norms(dev, dtype, tying):
     g = torch.Generator().manual_seed(8)

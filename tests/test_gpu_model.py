@@ -110,14 +110,21 @@ HALF_CASES = [
     BASE.scaled("half-jump", dtype="float16", activation_fn="jumprelu", k=None),
     BASE.scaled("half-per-target", dtype="float16", decoder_tying="per_target"),
     BASE.scaled("half-fused-shape", dtype="float16", num_layers=3, d_model=128, num_features=512, tokens=256, k=12),
+    # large-batch schedules: quarter rows (d = 768), line parts (d = 640), the dense per-target route, fused thresholds
+    BASE.scaled("half-quarter", dtype="float16", num_layers=4, d_model=768, num_features=1024, tokens=2304, k=16),
+    BASE.scaled("half-line", dtype="float16", num_layers=4, d_model=640, num_features=1024, tokens=2304, k=16,
+                decoder_tying="per_source"),
+    BASE.scaled("half-dense-route", dtype="float16", num_layers=3, d_model=256, num_features=1024, tokens=512, k=24,
+                decoder_tying="per_target"),
+    BASE.scaled("half-fused-jump", dtype="float16", num_layers=3, d_model=256, num_features=1024, tokens=512,
+                activation_fn="jumprelu", k=None),
 ]
 
 
 @pytest.mark.parametrize("wl", HALF_CASES, ids=lambda w: w.name)
 def test_float16_model_forward_matches_oracle(dev, wl):
-    # float16 parameters and outputs, computed on the float32 kernels with the dense products and thresholds
-    # rounded to float16 where the reference's tensors round; the oracle runs the reference's algorithm in
-    # float16 on the CPU
+    # float16 parameters and outputs on the float16 kernels (fp32 accumulation, one rounding per product, like
+    # bfloat16); the oracle runs the reference's algorithm in float16 on the CPU
     model, sd, x = build(wl, dev)
     assert model.dtype == torch.float16 and all(v.dtype == torch.float16 for v in model.state_dict().values()
                                                 if v.is_floating_point())
@@ -131,7 +138,9 @@ def test_float16_model_forward_matches_oracle(dev, wl):
     acts = model.get_feature_activations(inputs)
     pre_cpu = {l: model.get_preactivations(inputs[l], l).cpu() for l in range(wl.num_layers)}
     for l in acts:
-        assert acts[l].dtype == torch.float16 and pre_cpu[l].dtype == torch.float16
+        # JumpReLU's `(input >= threshold).float() * input` promotes to float32 (activations.py:177-180)
+        assert acts[l].dtype == (torch.float32 if wl.activation_fn == "jumprelu" else torch.float16)
+        assert pre_cpu[l].dtype == torch.float16
         # pre-activations: the float32 sum rounded once to float16
         want_pre = orc.encoder_preactivations(x[l], sd[f"encoder_module.encoders.{l}.weight"],
                                               sd[f"encoder_module.encoders.{l}.bias_param"])
