@@ -110,8 +110,8 @@ class CrossLayerTranscoder(BaseTranscoder):
                 m.device, m.dtype = w.device, w.dtype
 
     # ---- float16 models ----------------------------------------------------------------------------------
-    # The forward path (encoder, selection, decode, evaluator reductions) has float16 kernels of its own; the
-    # backward, the optimiser step and theta estimation are built for float32 and bfloat16 only.
+    # The forward path (encoder, selection, decode, evaluator reductions) and theta estimation have float16
+    # kernels of their own; the backward and the optimiser step are built for float32 and bfloat16 only.
     def _is_half(self) -> bool:
         self._sync_device()
         return self.dtype == torch.float16
@@ -164,7 +164,6 @@ class CrossLayerTranscoder(BaseTranscoder):
                                device: Optional[torch.device] = None) -> torch.Tensor:
         """Estimate theta post-hoc using a specified number of batches (clt.py:282-307).  The
         estimation runs where the model lives; ``device`` is accepted for signature parity."""
-        self._no_half("estimate_theta_posthoc")
         if device is not None and torch.device(device) != self.theta_manager.device:
             logger.info(f"Rank {self.rank}: theta estimation stays on {self.theta_manager.device} (asked for {device}).")
         return self.theta_manager.estimate_theta_posthoc(
@@ -175,7 +174,6 @@ class CrossLayerTranscoder(BaseTranscoder):
     def convert_to_jumprelu_inplace(self, default_theta_value: float = 1e6) -> None:
         """BatchTopK / TokenTopK -> JumpReLU from the estimated statistics (clt.py:309-318); the
         ThetaManager updates the config object it shares with the model."""
-        self._no_half("convert_to_jumprelu_inplace")
         self.theta_manager.convert_to_jumprelu_inplace(default_theta_value=default_theta_value)
         logger.info(f"Rank {self.rank}: CLT model config updated by ThetaManager. New activation_fn='{self.config.activation_fn}'.")
 

@@ -14,8 +14,9 @@
  *   - `dtype` is CLT_F32, CLT_BF16 or CLT_F16 and names the model dtype (inputs, weights,
  *     pre-activations, survivor values, outputs unless said otherwise).  CLT_F16 (IEEE half,
  *     fp32 accumulation, one rounding per product) is taken by the forward-path entry points -
- *     encoder, column statistics, selection, thresholds, packing, decode, densify, decoder norms,
- *     the dense accumulation of per-target tying, the evaluator reductions and the store feed;
+ *     encoder, column statistics, selection, thresholds, the theta-estimation minimum, packing,
+ *     decode, densify, decoder norms, the dense accumulation of per-target tying, the evaluator
+ *     reductions and the store feed;
  *     the gradient, optimiser and tile entry points (and clt_encode_segmented, which serves the
  *     threshold gradient) return CLT_ERR_DTYPE for it;
  *   - `stream` is a hipStream_t passed as void* (NULL = the null stream);
