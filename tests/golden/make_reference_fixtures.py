@@ -414,6 +414,12 @@ def sections():
             forward_case("batchtopk-global-bf16", dict(num_features=32, num_layers=3, d_model=16,
                                                        activation_fn="batchtopk", batchtopk_k=4,
                                                        clt_dtype="bfloat16"), 18, tokens=16),
+            # float16 likewise
+            forward_case("jumprelu-f16", dict(num_features=32, num_layers=3, d_model=16, activation_fn="jumprelu",
+                                              clt_dtype="float16"), 23, tokens=16),
+            forward_case("batchtopk-global-f16", dict(num_features=32, num_layers=3, d_model=16,
+                                                      activation_fn="batchtopk", batchtopk_k=4,
+                                                      clt_dtype="float16"), 24, tokens=16),
         ],
         "per_layer": lambda: [
             per_layer_case("batchtopk", dict(num_features=32, num_layers=3, d_model=8, activation_fn="batchtopk",
@@ -422,6 +428,8 @@ def sections():
                                                   batchtopk_k=4, clt_dtype="bfloat16"), 72),
             per_layer_case("tokentopk", dict(num_features=32, num_layers=3, d_model=8, activation_fn="topk",
                                              topk_k=5.0), 73),
+            per_layer_case("batchtopk-f16", dict(num_features=32, num_layers=3, d_model=8, activation_fn="batchtopk",
+                                                 batchtopk_k=4, clt_dtype="float16"), 74),
         ],
         "forward_irregular": lambda: irregular_cases(19),
         "config_json": config_json_cases,
@@ -456,7 +464,8 @@ def sections():
             gradient_case("per-target-offset-only", dict(base, activation_fn="batchtopk", batchtopk_k=3, decoder_tying="per_target",
                                                          enable_feature_offset=True), 40),
         ],
-        "global_select": lambda: [global_select_case(torch.float32, 51), global_select_case(torch.bfloat16, 52)],
+        "global_select": lambda: [global_select_case(torch.float32, 51), global_select_case(torch.bfloat16, 52),
+                                  global_select_case(torch.float16, 53)],
         "evaluator": lambda: evaluator_case(41),
         "compute_metrics": lambda: compute_metrics_case(42),
         "compute_metrics_subset": lambda: evaluator_subset_case(43),

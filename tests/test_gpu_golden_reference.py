@@ -32,6 +32,7 @@ def test_forward_matches_the_reference(dev, case):
     model = load_model(case, dev)
     model.eval()
     fp32 = model.dtype == torch.float32
+    tol16 = 2e-3 if model.dtype == torch.float16 else 1e-2       # rel-L2 tolerance of the float16 / bfloat16 path
     inputs = {int(l): T(v, dev).to(model.dtype) for l, v in case["inputs"].items()}
     recs = model(inputs)
     acts = model.get_feature_activations(inputs)
@@ -48,13 +49,13 @@ def test_forward_matches_the_reference(dev, case):
             # pre-activation can round to the other side of the gate; a token is compared at the stated
             # tolerance of the path (rel-L2 <= 1e-2) when its selected sets agree with the reference's in
             # every source layer up to l, and most tokens must be of that kind
-            assert orc.rel_l2(pre, T(case["preactivations"][str(l)])) <= 1e-2
+            assert orc.rel_l2(pre, T(case["preactivations"][str(l)])) <= tol16
             assert ((acts[l].float().cpu() != 0) != (want_a != 0)).float().mean() <= 0.01
             same = torch.ones(want_a.shape[0], dtype=torch.bool)
             for s_ in range(l + 1):
                 same &= ((acts[s_].float().cpu() != 0) == (T(case["activations"][str(s_)]) != 0)).all(dim=1)
             assert int(same.sum()) >= want_a.shape[0] // 2, (l, int(same.sum()))
-            assert orc.rel_l2(recs[l].float().cpu()[same], want_r[same]) <= 1e-2
+            assert orc.rel_l2(recs[l].float().cpu()[same], want_r[same]) <= tol16
     # the per-layer entry points (clt.py:112-184): encode() serves relu / jumprelu and returns zeros (with an
     # error log) for the top-k activations; decode() of the activations up to a layer
     tol = dict(rtol=1e-5, atol=1e-5) if fp32 else dict(rtol=5e-2, atol=5e-2)
@@ -252,7 +253,7 @@ def test_per_layer_scope_matches_the_reference_pieces(dev, case):
             for s_ in range(l + 1):
                 same &= ((acts[s_].float().cpu() != 0) == (T(case["activations"][str(s_)]) != 0)).all(dim=1)
             assert int(same.sum()) >= want_a.shape[0] // 2, (l, int(same.sum()))
-            assert orc.rel_l2(recs[l].float().cpu()[same], want_r[same]) <= 1e-2
+            assert orc.rel_l2(recs[l].float().cpu()[same], want_r[same]) <= (2e-3 if model.dtype == torch.float16 else 1e-2)
 
 
 def test_compute_metrics_end_to_end_matches_the_reference(dev):
