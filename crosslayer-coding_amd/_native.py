@@ -78,6 +78,9 @@ _SIGNATURES = {
     "clt_adam_step": (_int, [_vp, _vp, _vp, _vp, _i64, _f64, _f64, _f64, _f64, _i64, _int, _vp]),
     "clt_decoder_weight_grad_adam": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _f64, _f64, _f64, _f64, _i64, _int, _vp]),
     "clt_unpack_decoders": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
+    "clt_decoder_fingerprint": (_int, [_vp, _i64, _i64, _i64, _int, _vp, _vp, _int, _vp]),
+    "clt_pack_decoders_if": (_int, [_vp, _vp, _i64, _i64, _i64, _int, _vp, _vp]),
+    "clt_bias_sum": (_int, [_vp, _i64, _i64, _i64, _int, _u64, _int, _vp, _vp]),
     "clt_decoder_tile_width": (_int, [_i64, _i64, _i64, _int]),
     "clt_decoder_tiles_workspace_bytes": (_sz, [_i64, _int]),
     "clt_tile_decoders": (_int, [_vp, _vp, _i64, _i64, _i64, _int, _vp]),

@@ -927,6 +927,123 @@ __global__ __launch_bounds__(256) void k_pack(const T *src, T *dst, int64_t d, i
   }
 }
 
+// The same for the matrices whose flag is set, addressed through a table of parameter pointers: FP_PACK_BLOCKS
+// workgroups per matrix walk its 64 x 64 tiles; a matrix whose flag is clear costs its workgroups one load.
+constexpr int FP_PACK_BLOCKS = 64;
+template <typename T>
+__global__ __launch_bounds__(256) void k_pack_if(T *const *w_refs, T *dst, int64_t d, int64_t F, int64_t pitch,
+                                                 const int32_t *changed) {
+  __shared__ T tile[64][65];
+  const int z = blockIdx.y;
+  if (changed[z] == 0) return;
+  const T *s = w_refs[z];
+  T *o = dst + (int64_t)z * F * pitch;
+  const int64_t tf = (F + 63) / 64, td = (d + 63) / 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int64_t tile_i = blockIdx.x; tile_i < tf * td; tile_i += gridDim.x) {
+    const int64_t f0 = (tile_i % tf) * 64, d0 = (tile_i / tf) * 64;
+    __syncthreads();
+    for (int i = ty; i < 64; i += 4) {
+      int64_t dd = d0 + i, ff = f0 + tx;
+      if (dd < d && ff < F) tile[i][tx] = s[dd * F + ff];
+    }
+    __syncthreads();
+    for (int i = ty; i < 64; i += 4) {
+      int64_t ff = f0 + i, dd = d0 + tx;
+      if (ff < F && dd < d) o[ff * pitch + dd] = tile[tx][i];
+    }
+  }
+}
+
+// Fingerprint of every decoder parameter [d][F]: a sum (order-free, so the workgroups of a matrix add to it with
+// atomics) of mixed 32-bit words from sampled runs of 64 words.  A matrix of up to FP_CHUNKS runs is taken whole.
+// A larger one gives one run per row, on a diagonal: row r gives run (61 r + r / runs_per_row) mod runs_per_row, so
+// every row is looked at and every column in d / runs_per_row rows - a write to a whole row, a whole column or the
+// whole matrix cannot be missed, and the sample is d x 256 bytes (0.5 % of a 768 x 24576 matrix).  Rows that are not
+// a whole number of words fall back to FP_CHUNKS evenly spread runs.
+// state = [store | running sum | arrival counter] per matrix; the last workgroup of a matrix to arrive compares
+// the sum with the stored fingerprint, stores it, reports the difference and leaves sum and counter at zero.
+constexpr int FP_BLOCKS = 16;
+constexpr int FP_CHUNKS = 4096;
+__device__ __forceinline__ unsigned long long fp_mix(uint32_t word, uint32_t index) {
+  unsigned long long h = ((unsigned long long)word << 32) | (unsigned long long)(index * 0x9E3779B1u + 0x7F4A7C15u);
+  h ^= h >> 29; h *= 0xBF58476D1CE4E5B9ull; h ^= h >> 32; h *= 0x94D049BB133111EBull; h ^= h >> 29;
+  return h;
+}
+__global__ __launch_bounds__(256) void k_fingerprint(const uint32_t *const *w_refs, int64_t words, int64_t rows,
+                                                     int64_t words_per_row, int64_t n_dec, unsigned long long *state,
+                                                     int32_t *changed, int store_only) {
+  __shared__ unsigned long long red[4];
+  __shared__ unsigned int last;
+  const int z = blockIdx.y, lane = lane_id(), wv = threadIdx.x >> 6;
+  const uint32_t *w = w_refs[z];
+  const int64_t n_chunks = (words + 63) / 64;
+  const int64_t rpr = words_per_row > 0 ? (words_per_row + 63) / 64 : 0;      // runs per row
+  const bool whole = n_chunks <= FP_CHUNKS, diagonal = !whole && rpr > 0;
+  const int64_t take = whole ? n_chunks : diagonal ? rows : FP_CHUNKS;
+  unsigned long long h = 0;
+  // eight runs per wavefront in flight: the kernel is a handful of independent loads per lane, all latency
+  constexpr int FP_UNROLL = 8;
+  const int64_t step = (int64_t)gridDim.x * 4;
+  for (int64_t j0 = (int64_t)blockIdx.x * 4 + wv; j0 < take; j0 += step * FP_UNROLL) {
+    uint32_t v[FP_UNROLL];
+    int64_t at[FP_UNROLL];
+#pragma unroll
+    for (int u = 0; u < FP_UNROLL; ++u) {
+      const int64_t j = j0 + u * step;
+      int64_t i = -1;
+      if (j < take) {
+        if (whole) i = j * 64 + lane;
+        else if (diagonal) {
+          const int64_t in_row = ((j * 61 + j / rpr) % rpr) * 64 + lane;
+          i = in_row < words_per_row ? j * words_per_row + in_row : -1;
+        } else i = ((j * n_chunks) / take) * 64 + lane;
+        if (i >= words) i = -1;
+      }
+      at[u] = i;
+      v[u] = i >= 0 ? w[i] : 0u;
+    }
+#pragma unroll
+    for (int u = 0; u < FP_UNROLL; ++u)
+      if (at[u] >= 0) h += fp_mix(v[u], (uint32_t)at[u]);
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) h += __shfl_xor(h, o);
+  if (lane == 0) red[wv] = h;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    unsigned long long *store = state + z, *sum = state + n_dec + z, *count = state + 2 * n_dec + z;
+    atomicAdd(sum, red[0] + red[1] + red[2] + red[3]);
+    __threadfence();
+    last = atomicAdd(count, 1ull) == (unsigned long long)(gridDim.x - 1) ? 1u : 0u;
+    if (last) {
+      __threadfence();
+      const unsigned long long now = atomicAdd(sum, 0ull);
+      changed[z] = (!store_only && now != *store) ? 1 : 0;
+      *store = now;
+      *sum = 0ull;
+      *count = 0ull;
+    }
+  }
+}
+
+// out[t][c] = sum of the biases of the decoders that run for target t, sources in ascending order, fp32
+template <typename T>
+__global__ __launch_bounds__(256) void k_bias_sum(const T *const *b_refs, int64_t d, int64_t L, int tying, uint64_t src_mask,
+                                                  float *out) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= L * d) return;
+  const int64_t t = i / d, c = i - t * d;
+  float acc = 0.0f;
+  if (tying == CLT_TYING_PER_TARGET) {
+    acc = Elem<T>::to_f32(b_refs[t][c]);
+  } else {
+    for (int64_t s = 0; s <= t; ++s)
+      if ((src_mask >> s) & 1ull) acc += Elem<T>::to_f32(b_refs[decoder_slot(tying, s, t, L)][c]);
+  }
+  out[i] = acc;
+}
+
 // [F][pitch] -> [d][F], the way back: decoder z of the slab into the parameter whose address is w_refs[z].
 template <typename T>
 __global__ __launch_bounds__(256) void k_unpack(const T *src, T *const *w_refs, int64_t d, int64_t F, int64_t pitch) {
@@ -1288,6 +1405,47 @@ extern "C" int clt_pack_decoder(const void *w_ref, void *w_packed, int64_t d, in
   hipStream_t s = (hipStream_t)stream;
   if (dtype != CLT_F32) k_pack<bf16_t><<<grid, 256, 0, s>>>((const bf16_t *)w_ref, (bf16_t *)w_packed, d, F, in_stride, out_stride, clt_pitch(d, 2));
   else k_pack<float><<<grid, 256, 0, s>>>((const float *)w_ref, (float *)w_packed, d, F, in_stride, out_stride, clt_pitch(d, 4));
+  return clt_check_launch();
+}
+
+extern "C" int clt_decoder_fingerprint(void *const *w_refs_dev, int64_t n_dec, int64_t d, int64_t F, int dtype,
+                                       uint64_t *state, int32_t *changed, int store_only, void *stream) {
+  if (!clt_model_dtype(dtype)) return CLT_ERR_DTYPE;
+  if (d <= 0 || F <= 0 || n_dec < 0 || n_dec > 65535) return CLT_ERR_ARG;
+  if (n_dec == 0) return CLT_OK;
+  if (!w_refs_dev || !state || !changed) return CLT_ERR_ARG;
+  const int64_t words = d * F * clt_elem_bytes(dtype) / 4;     // a last odd 16-bit element is not looked at
+  if (words <= 0) return CLT_ERR_ARG;
+  const int64_t row_bytes = F * clt_elem_bytes(dtype);
+  k_fingerprint<<<dim3(FP_BLOCKS, (unsigned)n_dec), 256, 0, (hipStream_t)stream>>>(
+      (const uint32_t *const *)w_refs_dev, words, d, row_bytes % 4 == 0 ? row_bytes / 4 : 0, n_dec,
+      (unsigned long long *)state, changed, store_only);
+  return clt_check_launch();
+}
+
+extern "C" int clt_pack_decoders_if(void *const *w_refs_dev, void *w_packed, int64_t n_dec, int64_t d, int64_t F,
+                                    int dtype, const int32_t *changed, void *stream) {
+  if (!clt_model_dtype(dtype)) return CLT_ERR_DTYPE;
+  if (d <= 0 || F <= 0 || n_dec < 0 || n_dec > 65535) return CLT_ERR_ARG;
+  if (n_dec == 0) return CLT_OK;
+  if (!w_refs_dev || !w_packed || !changed) return CLT_ERR_ARG;
+  const dim3 grid(FP_PACK_BLOCKS, (unsigned)n_dec);
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype != CLT_F32) k_pack_if<bf16_t><<<grid, 256, 0, s>>>((bf16_t *const *)w_refs_dev, (bf16_t *)w_packed, d, F, clt_pitch(d, 2), changed);
+  else k_pack_if<float><<<grid, 256, 0, s>>>((float *const *)w_refs_dev, (float *)w_packed, d, F, clt_pitch(d, 4), changed);
+  return clt_check_launch();
+}
+
+extern "C" int clt_bias_sum(void *const *b_refs_dev, int64_t n_dec, int64_t d, int64_t L, int tying, uint64_t src_mask,
+                            int dtype, float *out, void *stream) {
+  if (!clt_model_dtype(dtype)) return CLT_ERR_DTYPE;
+  if (d <= 0 || L <= 0 || L > 64 || tying < 0 || tying > 2 || !b_refs_dev || !out) return CLT_ERR_ARG;
+  if (n_dec != (tying == CLT_TYING_NONE ? L * (L + 1) / 2 : L)) return CLT_ERR_ARG;
+  const unsigned nb = (unsigned)clt_ceil_div(L * d, 256);
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == CLT_BF16) k_bias_sum<bf16_t><<<nb, 256, 0, s>>>((const bf16_t *const *)b_refs_dev, d, L, tying, src_mask, out);
+  else if (dtype == CLT_F16) k_bias_sum<f16_t><<<nb, 256, 0, s>>>((const f16_t *const *)b_refs_dev, d, L, tying, src_mask, out);
+  else k_bias_sum<float><<<nb, 256, 0, s>>>((const float *const *)b_refs_dev, d, L, tying, src_mask, out);
   return clt_check_launch();
 }
 

@@ -144,7 +144,14 @@ class Decoder(nn.Module):
         self._slab: Optional[torch.Tensor] = None
         self._slab_keys: List[Optional[tuple]] = []
         self._norm_key = None
-        self._bias_cache: Dict[int, Tuple[tuple, torch.Tensor]] = {}
+        self._bias_cache: Dict[int, Tuple[tuple, torch.Tensor]] = {}     # kept for callers that clear it; unused
+        # writes to the parameters that no version counter shows (``weight.data.copy_(...)``): every use of the
+        # packed copy checks a sampled fingerprint of the parameters on the device and repacks there what changed
+        self.watch_parameter_data = True
+        self._fp_state: Optional[torch.Tensor] = None
+        self._fp_changed: Optional[torch.Tensor] = None
+        self._fp_fresh = False
+        self._tables: Dict[str, tuple] = {}
         self._compact_cache: Dict[int, tuple] = {}
         # decoders tied per target: targets whose summed activations are dense enough go through the
         # matrix cores (see dense_split); False keeps every target on the row gather
@@ -155,10 +162,17 @@ class Decoder(nn.Module):
     def _ordered(self) -> List[RowParallelLinear]:
         """Decoder layers in slot order (untied: "0->0", "0->1", ..., as created)."""
         mods = self.decoders._modules      # straight to the registry: no parameter sync for internal walks
+        cached = self.__dict__.get("_ordered_cache")
+        if cached is not None and cached[0] is mods and cached[1] == len(mods) and all(
+                a is b for a, b in zip(cached[3], mods.values())):
+            return cached[2]
         if isinstance(self.decoders, nn.ModuleDict):
             L = self.config.num_layers
-            return [mods[f"{s}->{t}"] for s in range(L) for t in range(s, L)]
-        return list(mods.values())
+            out = [mods[f"{s}->{t}"] for s in range(L) for t in range(s, L)]
+        else:
+            out = list(mods.values())
+        self.__dict__["_ordered_cache"] = (mods, len(mods), out, list(mods.values()))
+        return out
 
     # ---- parameters behind the working copy -------------------------------------------
     def mark_parameters_behind(self) -> None:
@@ -180,6 +194,7 @@ class Decoder(nn.Module):
                                 (ctypes.c_void_p * len(ptrs))(*ptrs))
         d, F = ws[0].shape
         engine.unpack_decoders(self._slab, self._sync_table[1], self._sync_table[2], d, F)
+        self._fp_fresh = False             # the parameters hold new values: record them before comparing again
 
     def named_parameters(self, *args, **kwargs):
         self.sync_parameters()
@@ -196,9 +211,26 @@ class Decoder(nn.Module):
             return [(s, t) for s in range(L) for t in range(s, L)]
         return [(i, i) for i in range(L)]
 
+    def _pointer_table(self, name: str, tensors) -> torch.Tensor:
+        """Device int64 tensor with the addresses of ``tensors``, rebuilt only when one has moved."""
+        ptrs = tuple(t.data_ptr() for t in tensors)
+        ent = self._tables.get(name)
+        if ent is None or ent[0] != ptrs or ent[1].device != tensors[0].device:
+            # through pinned memory and an asynchronous copy: building the table must not synchronise a forward
+            host = torch.tensor(ptrs, dtype=torch.int64).pin_memory()
+            ent = (ptrs, host.to(tensors[0].device, non_blocking=True), host)
+            self._tables[name] = ent
+        return ent[1]
+
+    def note_parameters_written(self) -> None:
+        """A kernel of this library has just written the decoder parameters and the packed copy alike: the stored
+        fingerprints are of the old values and are taken again before they are next compared."""
+        self._fp_fresh = False
+
     def packed(self) -> torch.Tensor:
-        """[n_dec, F, pitch] feature-major slab (``engine.decoder_pitch``); matrices whose parameter changed
-        are repacked."""
+        """[n_dec, F, pitch] feature-major slab (``engine.decoder_pitch``), true to the parameters: matrices
+        whose parameter changed are repacked - by the host where the parameter's version counter shows it, by the
+        device itself where only the data does (``weight.data.fill_(...)``; ``watch_parameter_data``)."""
         decs = self._ordered()
         w0 = decs[0].weight
         F, d = self.config.num_features, self.config.d_model
@@ -207,6 +239,7 @@ class Decoder(nn.Module):
             self._slab = engine.alloc_packed(len(decs), F, d, w0.dtype, w0.device)
             self._slab_keys = [None] * len(decs)
             self.device, self.dtype = w0.device, w0.dtype
+            self._fp_state = None
         for i, dec in enumerate(decs):
             w = dec.weight
             key = (w.data_ptr(), w._version)
@@ -214,6 +247,24 @@ class Decoder(nn.Module):
                 engine.pack_decoder(w.detach().contiguous(), self._slab[i])
                 self._slab_keys[i] = key
                 self._repacks = getattr(self, "_repacks", 0) + 1
+                self._fp_fresh = False
+        if self.watch_parameter_data and not getattr(self, "_params_behind", False) \
+                and all(dec.weight.is_contiguous() for dec in decs):
+            if self._fp_state is None or self._fp_state.device != w0.device:
+                self._fp_state = torch.zeros(3 * len(decs), dtype=torch.int64, device=w0.device)
+                self._fp_changed = torch.zeros(len(decs), dtype=torch.int32, device=w0.device)
+                self._fp_fresh = False
+            table = self._pointer_table("w", [dec.weight for dec in decs])
+            if not self._fp_fresh:
+                # the slab has just been made from these values (or written together with them): record them
+                engine.decoder_fingerprint(table, d, F, w0.dtype, self._fp_state, self._fp_changed, True)
+                self._fp_fresh = True
+            else:
+                engine.decoder_fingerprint(table, d, F, w0.dtype, self._fp_state, self._fp_changed, False)
+                engine.pack_decoders_if(table, self._slab, d, F, self._fp_changed)
+                # copies derived from the slab (the optimiser's tiles) cannot know whether the device repacked
+                if getattr(self, "_derived_copies", False):
+                    self._repacks = getattr(self, "_repacks", 0) + 1
         return self._slab
 
     def packed_generation(self):
@@ -228,40 +279,36 @@ class Decoder(nn.Module):
         self._slab_keys = [None] * len(self._slab_keys)
         self._bias_cache.clear()
         self._cached_decoder_norms = None
+        self._fp_fresh = False
 
     def bias_sum(self, src_mask: int) -> torch.Tensor:
         """[L, d] fp32: for every target the sum of the biases of the decoders that run for
         it - one per contributing source (decoder.py:294-295 / parallel.py:380-381), or the
         target's own decoder for per_target tying (decoder.py:250-251)."""
         decs = self._ordered()
-        key = tuple((dec.bias_param.data_ptr(), dec.bias_param._version) for dec in decs)
-        hit = self._bias_cache.get(src_mask)
-        if hit is not None and hit[0] == key:
-            return hit[1]
+        bs = [dec.bias_param for dec in decs]
+        if all(b is not None and b.is_contiguous() and b.is_cuda for b in bs):
+            # computed anew on every call (one small launch): a write to a bias shows whichever way it was made
+            return engine.bias_sum(self._pointer_table("b", bs), self.config.d_model, self.config.num_layers,
+                                   self.config.decoder_tying, src_mask, bs[0].dtype)
         L, d = self.config.num_layers, self.config.d_model
         B = torch.stack([dec.bias_param.detach() for dec in decs]).float()
         tying = self.config.decoder_tying
         if tying == "per_target":
-            out = B.contiguous()
+            return B.contiguous()
+        out = torch.zeros(L, d, dtype=torch.float32, device=B.device)
+        if tying == "none":
+            first = 0
+            for s in range(L):
+                if (src_mask >> s) & 1:
+                    out[s:] += B[first:first + L - s]
+                first += L - s
         else:
-            out = torch.zeros(L, d, dtype=torch.float32, device=B.device)
-            if tying == "none":
-                # the decoders of source s are the slots of the targets s .. L-1, in a row: one addition per
-                # source, so every target still adds its sources in ascending order
-                first = 0
-                for s in range(L):
-                    if (src_mask >> s) & 1:
-                        out[s:] += B[first:first + L - s]
-                    first += L - s
-            else:
-                run = torch.zeros(d, dtype=torch.float32, device=B.device)
-                for t in range(L):
-                    if (src_mask >> t) & 1:
-                        run = run + B[t]
-                    out[t] = run
-        if len(self._bias_cache) > 64:
-            self._bias_cache.clear()
-        self._bias_cache[src_mask] = (key, out)
+            run = torch.zeros(d, dtype=torch.float32, device=B.device)
+            for t in range(L):
+                if (src_mask >> t) & 1:
+                    run = run + B[t]
+                out[t] = run
         return out
 
     def _affine(self):

@@ -614,6 +614,38 @@ def unpack_decoders(w_packed: torch.Tensor, w_refs_dev: torch.Tensor, w_refs_hos
     nat.check(code, "clt_unpack_decoders")
 
 
+def decoder_fingerprint(w_refs_dev: torch.Tensor, d: int, F: int, dtype: torch.dtype, state: torch.Tensor,
+                        changed: torch.Tensor, store_only: bool) -> None:
+    """Hash a sample of every decoder parameter ([d, F] each, addresses in the device int64 tensor ``w_refs_dev``):
+    ``changed[i]`` = 1 where it differs from the hash kept in ``state`` (int64 [3 n_dec], zeros before the first
+    call), which is brought up to date; ``store_only`` records without comparing."""
+    n_dec = w_refs_dev.numel()
+    assert w_refs_dev.dtype == torch.int64 and state.dtype == torch.int64 and state.numel() == 3 * n_dec
+    assert changed.dtype == torch.int32 and changed.numel() == n_dec and state.is_contiguous()
+    code = nat.load().clt_decoder_fingerprint(nat.ptr(w_refs_dev), n_dec, d, F, nat.dtype_code(dtype), nat.ptr(state),
+                                              nat.ptr(changed), 1 if store_only else 0, _stream(state))
+    nat.check(code, "clt_decoder_fingerprint")
+
+
+def pack_decoders_if(w_refs_dev: torch.Tensor, w_packed: torch.Tensor, d: int, F: int, changed: torch.Tensor) -> None:
+    """Repack, on the device's own decision, the matrices of the slab [n_dec, F, pitch] whose ``changed`` flag is set."""
+    n_dec = w_packed.shape[0]
+    assert w_refs_dev.numel() == n_dec and changed.numel() == n_dec and w_packed.is_contiguous()
+    code = nat.load().clt_pack_decoders_if(nat.ptr(w_refs_dev), nat.ptr(w_packed), n_dec, d, F,
+                                           nat.dtype_code(w_packed.dtype), nat.ptr(changed), _stream(w_packed))
+    nat.check(code, "clt_pack_decoders_if")
+
+
+def bias_sum(b_refs_dev: torch.Tensor, d: int, L: int, tying: str, src_mask: int, dtype: torch.dtype) -> torch.Tensor:
+    """fp32 [L, d]: per target the sum of the biases of the decoders that run for it (addresses of the n_dec bias
+    vectors in the device int64 tensor ``b_refs_dev``), sources of ``src_mask`` in ascending order."""
+    out = torch.empty((L, d), dtype=torch.float32, device=b_refs_dev.device)
+    code = nat.load().clt_bias_sum(nat.ptr(b_refs_dev), b_refs_dev.numel(), d, L, nat.TYING[tying], int(src_mask),
+                                   nat.dtype_code(dtype), nat.ptr(out), _stream(out))
+    nat.check(code, "clt_bias_sum")
+    return out
+
+
 def decoder_tile_width(T: int, d: int, F: int, dtype: torch.dtype) -> int:
     """Columns per tile of the tiled decoder layout [n_dec, d // CS, F, CS] when the column-tile weight-gradient
     kernel takes this shape, else 0."""

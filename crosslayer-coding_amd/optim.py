@@ -122,6 +122,7 @@ class CLTAdam:
         cs = engine.decoder_tile_width(surv.T, d, F, ws[0].dtype) if self.tile_decoder_step else 0
         if cs and all(w.data_ptr() % 16 == 0 for w in ws):
             self._decoder_moments_to("tiles")
+            dec._derived_copies = True      # the packed copy tells when the device may have repacked it
             if self._w_tiles is None or self._w_tiles_gen != dec.packed_generation():
                 self._w_tiles = engine.tile_decoders(packed, d, out=self._w_tiles)
                 self._w_tiles_gen = dec.packed_generation()
@@ -133,6 +134,7 @@ class CLTAdam:
                 dec.mark_parameters_behind()
             else:
                 engine.untile_decoders(self._w_tiles, packed, w_dev, w_host)
+                dec.note_parameters_written()
             return
         self._decoder_moments_to("rows")
         self._w_tiles_gen = None
@@ -143,6 +145,7 @@ class CLTAdam:
             dec.mark_parameters_behind()
         else:
             engine.unpack_decoders(packed, w_dev, w_host, d, F)
+            dec.note_parameters_written()
 
     @torch.no_grad()
     def step(self, raw) -> None:
@@ -212,3 +215,4 @@ class CLTAdam:
         # the kernels wrote through .data: caches keyed on version counters would not notice
         dec._bias_cache.clear()
         dec._cached_decoder_norms = None
+        dec.note_parameters_written()

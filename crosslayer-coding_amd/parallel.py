@@ -112,13 +112,13 @@ class RowParallelLinear(_Linear):
         self._packed_key = None
 
     def packed_weight(self) -> torch.Tensor:
-        """Feature-major [F, d] copy of ``weight``, refreshed when the parameter changes."""
+        """Feature-major [F, d] copy of ``weight``, made anew on every call: a layer used on its own is not a
+        hot path, and a write through ``weight.data`` leaves no trace a cache could be keyed on."""
         w = self.weight
-        key = (w.data_ptr(), w._version, w.device, w.dtype)
-        if self._packed is None or self._packed_key != key:
-            self._packed = torch.empty(self.full_in_features, self.full_out_features, device=w.device, dtype=w.dtype)
-            engine.pack_decoder(w.detach().contiguous(), self._packed)
-            self._packed_key = key
+        if self._packed is None or self._packed.device != w.device or self._packed.dtype != w.dtype:
+            self._packed = torch.empty(self.full_in_features, engine.decoder_pitch(self.full_out_features, w.dtype),
+                                       device=w.device, dtype=w.dtype)
+        engine.pack_decoder(w.detach().contiguous(), self._packed)
         return self._packed
 
     def forward(self, input_: torch.Tensor) -> torch.Tensor:

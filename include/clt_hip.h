@@ -394,6 +394,35 @@ int clt_decode_route(int64_t T, int64_t d, int64_t F, int64_t L, int tying, int 
                      size_t workspace_bytes);
 
 /*
+ * Keeping the packed copy true to its parameters without the host looking at them.  The reference reads
+ * its decoder parameters in place in every forward (clt/models/parallel.py:335-383), so any write to
+ * them - also one that bypasses autograd's version counters, like `weight.data.copy_(...)` - shows in the
+ * next result.  clt_decoder_fingerprint hashes a sample of every decoder parameter (w_refs_dev[i] = address
+ * of matrix i, [d][F]; all of a matrix up to 1 MiB, of a larger one a 256-byte run per row on a diagonal, so
+ * that every row is looked at and every column in several rows):
+ * changed[i] = 1 where the hash differs from the one kept in state, and state is brought up to date.
+ * store_only != 0 only records (after the caller itself wrote the parameters).  `state` holds 3 * n_dec
+ * 64-bit words, zeroed by the caller before the first call and left alone afterwards.
+ * clt_pack_decoders_if repacks the matrices whose flag is set (clt_pack_decoder otherwise) - a launch that
+ * costs microseconds when no flag is set.  Both run on the stream; nothing is read back.  A write to the
+ * whole matrix, a whole row or a whole column of it is always seen; one that touches a few scattered elements
+ * of a large matrix may miss the sample.
+ */
+int clt_decoder_fingerprint(void *const *w_refs_dev, int64_t n_dec, int64_t d, int64_t F, int dtype,
+                            uint64_t *state, int32_t *changed, int store_only, void *stream);
+int clt_pack_decoders_if(void *const *w_refs_dev, void *w_packed, int64_t n_dec, int64_t d, int64_t F,
+                         int dtype, const int32_t *changed, void *stream);
+
+/*
+ * bias_sum[t][c] (fp32 [L][d]) = sum of the biases of the decoders that run for target t: one per source
+ * s <= t whose bit is set in src_mask, in ascending order (clt/models/decoder.py:294-295 through
+ * parallel.py:380-381), or the target's own decoder for per-target tying (decoder.py:250-251).
+ * b_refs_dev[slot] = address of the bias of decoder `slot` (n_dec of them, d elements each).
+ */
+int clt_bias_sum(void *const *b_refs_dev, int64_t n_dec, int64_t d, int64_t L, int tying, uint64_t src_mask,
+                 int dtype, float *out, void *stream);
+
+/*
  * Layout of the packed (feature-major) decoder slab that every entry point taking `w_packed` assumes:
  *   w_packed[slot][f][c],  0 <= c < d,  rows clt_decoder_pitch(d, dtype) elements apart,
  *   matrices F * pitch elements apart.
