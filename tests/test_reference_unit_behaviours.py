@@ -319,3 +319,63 @@ def test_writes_through_data_show_in_the_next_forward(dev, dtype):
     want = reference()
     for t in range(3):
         assert orc.rel_l2(again[t].float().cpu(), want[t].float()) <= tol, t
+
+
+# ---- the autograd Functions (unit/models/test_activations.py) ----------------------------------------------------
+@pytest.mark.gpu
+def test_masks_of_empty_inputs_are_empty(dev):
+    # test_activations.py:53-63, :243-253
+    for fn, k in ((cca.BatchTopK, 2), (cca.TokenTopK, 2.0)):
+        for shape in ((0, 4), (2, 0)):
+            x = torch.empty(*shape, device=dev)
+            m = fn._compute_mask(x, k)
+            assert m.shape == x.shape and m.dtype == torch.bool and int(m.sum()) == 0
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("straight_through", [True, False])
+def test_top_k_backward_passes_the_gradient_where_the_gate_kept(dev, straight_through):
+    # test_activations.py:114-152 (BatchTopK; the non-straight-through flag behaves the same), :286-301 (TokenTopK)
+    g = torch.Generator().manual_seed(3)
+    for fn, k in ((cca.BatchTopK, 2.0), (cca.TokenTopK, 2.0)):
+        x = torch.randn(2, 4, generator=g).to(dev).requires_grad_(True)
+        out = fn.apply(x, k, straight_through, None)
+        gout = torch.randn(2, 4, generator=g).to(dev)
+        out.backward(gout)
+        mask = fn._compute_mask(x.detach(), int(k) if fn is cca.BatchTopK else k, None)
+        assert x.grad is not None and torch.allclose(x.grad, gout * mask.to(x.dtype))
+        assert int(mask.sum()) == 4
+
+
+@pytest.mark.gpu
+def test_jumprelu_backward_table_and_grad_flags(dev):
+    # test_activations.py:318-381 (the table, quoted in tests/golden/reference_known_answers.json), :384-420 (flags)
+    import json
+    import os
+    table = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_known_answers.json")))["jumprelu_backward"]
+    for case in table:
+        x = torch.tensor([case["input"]], device=dev, requires_grad=True)
+        thr = torch.tensor([case["threshold"]], device=dev, requires_grad=True)
+        out = cca.JumpReLU.apply(x, thr, case["bandwidth"])
+        out.backward(torch.tensor([case["grad_output"]], device=dev))
+        assert x.grad.item() == pytest.approx(case["expected_grad_input"] * case["grad_output"])
+        near = abs(case["input"] - case["threshold"]) <= case["bandwidth"] / 2.0
+        want = (-case["input"] / case["bandwidth"]) * case["grad_output"] if near else 0.0
+        assert thr.grad.item() == pytest.approx(want, abs=1e-6), case
+    one = torch.tensor([1.0], device=dev)
+    x = torch.tensor([1.5], device=dev, requires_grad=True)
+    thr = torch.tensor([0.5], device=dev)
+    cca.JumpReLU.apply(x, thr, 1.0).backward(one)
+    assert x.grad is not None and thr.grad is None
+    x = torch.tensor([1.5], device=dev)
+    thr = torch.tensor([0.5], device=dev, requires_grad=True)
+    cca.JumpReLU.apply(x, thr, 1.0).backward(one)
+    assert x.grad is None and thr.grad is not None
+
+    class Ctx:            # neither input asked for its gradient, the threshold did: backward called by hand
+        needs_input_grad = [False, True, False]
+        saved_tensors = (torch.tensor([1.5], device=dev), torch.tensor([0.5], device=dev))
+        bandwidth = 1.0
+
+    gx, gthr, _ = cca.JumpReLU.backward(Ctx(), one)
+    assert gx is None and gthr is not None
