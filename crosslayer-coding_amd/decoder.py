@@ -194,7 +194,7 @@ class Decoder(nn.Module):
                                 (ctypes.c_void_p * len(ptrs))(*ptrs))
         d, F = ws[0].shape
         engine.unpack_decoders(self._slab, self._sync_table[1], self._sync_table[2], d, F)
-        self._fp_fresh = False             # the parameters hold new values: record them before comparing again
+        self.note_parameters_written()     # the parameters hold new values: record them before a caller writes more
 
     def named_parameters(self, *args, **kwargs):
         self.sync_parameters()
@@ -224,8 +224,15 @@ class Decoder(nn.Module):
 
     def note_parameters_written(self) -> None:
         """A kernel of this library has just written the decoder parameters and the packed copy alike: the stored
-        fingerprints are of the old values and are taken again before they are next compared."""
+        fingerprints are of the old values.  They are taken again right here, behind that kernel on the stream, so
+        that a write the caller makes afterwards through ``.data`` still differs from what is stored."""
         self._fp_fresh = False
+        decs = self._ordered()
+        if (self.watch_parameter_data and self._fp_state is not None and self._slab is not None
+                and self._fp_state.device == decs[0].weight.device and all(dec.weight.is_contiguous() for dec in decs)):
+            engine.decoder_fingerprint(self._pointer_table("w", [dec.weight for dec in decs]), self.config.d_model,
+                                       self.config.num_features, decs[0].weight.dtype, self._fp_state, self._fp_changed, True)
+            self._fp_fresh = True
 
     def packed(self) -> torch.Tensor:
         """[n_dec, F, pitch] feature-major slab (``engine.decoder_pitch``), true to the parameters: matrices
@@ -247,7 +254,6 @@ class Decoder(nn.Module):
                 engine.pack_decoder(w.detach().contiguous(), self._slab[i])
                 self._slab_keys[i] = key
                 self._repacks = getattr(self, "_repacks", 0) + 1
-                self._fp_fresh = False
         if self.watch_parameter_data and not getattr(self, "_params_behind", False) \
                 and all(dec.weight.is_contiguous() for dec in decs):
             if self._fp_state is None or self._fp_state.device != w0.device:
@@ -256,7 +262,7 @@ class Decoder(nn.Module):
                 self._fp_fresh = False
             table = self._pointer_table("w", [dec.weight for dec in decs])
             if not self._fp_fresh:
-                # the slab has just been made from these values (or written together with them): record them
+                # first use (or after invalidate_packed): the slab has just been made from these values: record them
                 engine.decoder_fingerprint(table, d, F, w0.dtype, self._fp_state, self._fp_changed, True)
                 self._fp_fresh = True
             else:

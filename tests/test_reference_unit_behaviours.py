@@ -379,3 +379,41 @@ def test_jumprelu_backward_table_and_grad_flags(dev):
 
     gx, gthr, _ = cca.JumpReLU.backward(Ctx(), one)
     assert gx is None and gthr is not None
+
+
+@pytest.mark.gpu
+def test_data_writes_are_seen_next_to_other_kinds_of_writes_and_between_training_steps(dev):
+    # a versioned in-place write to one matrix and a .data write to another before the same forward; a .data write
+    # after an optimiser step (whose kernels write the parameters themselves)
+    from crosslayer_coding_amd import synth
+    wl = synth.WORKLOADS["c0"].scaled("data-writes-2", dtype="bfloat16", num_layers=3, d_model=128, num_features=256, tokens=256, k=8)
+    model, inputs, _ = synth.build_model(wl, dev)
+    twin, _, _ = synth.build_model(wl, dev)
+    dec, dec2 = model.decoder_module, twin.decoder_module
+    model(inputs)
+    with torch.no_grad():
+        dec.decoders["0->0"].weight.mul_(0.5)                   # bumps the version counter
+    dec.decoders["1->2"].weight.data.mul_(-2.0)                 # does not
+    out = model(inputs)
+    with torch.no_grad():
+        dec2.decoders["0->0"].weight.mul_(0.5)
+        dec2.decoders["1->2"].weight.mul_(-2.0)
+    want = twin(inputs)
+    for t in range(3):
+        assert torch.equal(out[t], want[t]), t
+    # training: each route's own kernels write the parameters; a .data write after the step must still count
+    targets = {l: torch.randn_like(x) for l, x in inputs.items()}
+    for fused in (False, True):
+        opts = []
+        for m in (model, twin):
+            opt = cca.CLTAdam(m, lr=1e-3)
+            opt.fuse_decoder_step = fused
+            m.training_step(inputs, targets, opt)
+            opts.append(opt)
+        w = dec.decoders["0->1"].weight          # (a fused step left the parameters behind: this access refreshes them)
+        w.data.add_(0.125)
+        with torch.no_grad():
+            dec2.decoders["0->1"].weight.add_(0.125)
+        out, want = model(inputs), twin(inputs)
+        for t in range(3):
+            assert torch.equal(out[t], want[t]), (fused, t)
