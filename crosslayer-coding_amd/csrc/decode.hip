@@ -961,9 +961,12 @@ __global__ __launch_bounds__(256) void k_pack_if(T *const *w_refs, T *dst, int64
 // every row is looked at and every column in d / runs_per_row rows - a write to a whole row, a whole column or the
 // whole matrix cannot be missed, and the sample is d x 256 bytes (0.5 % of a 768 x 24576 matrix).  Rows that are not
 // a whole number of words fall back to FP_CHUNKS evenly spread runs.
-// state = [store | running sum | arrival counter] per matrix; the last workgroup of a matrix to arrive compares
-// the sum with the stored fingerprint, stores it, reports the difference and leaves sum and counter at zero.
-constexpr int FP_BLOCKS = 16;
+// FP_BLOCKS workgroups per matrix (a CU keeps only ~64 line requests in flight, so a matrix's rows are spread over
+// several CUs).  state holds one 128-byte line per matrix - FP_BLOCKS partial sums, the stored fingerprint and an
+// arrival counter - so that the workgroups of different matrices never meet on a cache line; the last workgroup of
+// a matrix to arrive adds the partial sums, compares, stores and leaves the counter at zero.
+constexpr int FP_BLOCKS = 8;
+constexpr int FP_STATE_WORDS = 16;
 constexpr int FP_CHUNKS = 4096;
 __device__ __forceinline__ unsigned long long fp_mix(uint32_t word, uint32_t index) {
   unsigned long long h = ((unsigned long long)word << 32) | (unsigned long long)(index * 0x9E3779B1u + 0x7F4A7C15u);
@@ -971,10 +974,9 @@ __device__ __forceinline__ unsigned long long fp_mix(uint32_t word, uint32_t ind
   return h;
 }
 __global__ __launch_bounds__(256) void k_fingerprint(const uint32_t *const *w_refs, int64_t words, int64_t rows,
-                                                     int64_t words_per_row, int64_t n_dec, unsigned long long *state,
+                                                     int64_t words_per_row, unsigned long long *state,
                                                      int32_t *changed, int store_only) {
   __shared__ unsigned long long red[4];
-  __shared__ unsigned int last;
   const int z = blockIdx.y, lane = lane_id(), wv = threadIdx.x >> 6;
   const uint32_t *w = w_refs[z];
   const int64_t n_chunks = (words + 63) / 64;
@@ -984,7 +986,7 @@ __global__ __launch_bounds__(256) void k_fingerprint(const uint32_t *const *w_re
   unsigned long long h = 0;
   // eight runs per wavefront in flight: the kernel is a handful of independent loads per lane, all latency
   constexpr int FP_UNROLL = 8;
-  const int64_t step = (int64_t)gridDim.x * 4;
+  const int64_t step = (int64_t)FP_BLOCKS * 4;
   for (int64_t j0 = (int64_t)blockIdx.x * 4 + wv; j0 < take; j0 += step * FP_UNROLL) {
     uint32_t v[FP_UNROLL];
     int64_t at[FP_UNROLL];
@@ -995,9 +997,10 @@ __global__ __launch_bounds__(256) void k_fingerprint(const uint32_t *const *w_re
       if (j < take) {
         if (whole) i = j * 64 + lane;
         else if (diagonal) {
-          const int64_t in_row = ((j * 61 + j / rpr) % rpr) * 64 + lane;
+          const uint32_t r32 = (uint32_t)rpr, j32 = (uint32_t)j;        // rows and runs per row are far below 2^31
+          const int64_t in_row = (int64_t)((j32 * 61u + j32 / r32) % r32) * 64 + lane;
           i = in_row < words_per_row ? j * words_per_row + in_row : -1;
-        } else i = ((j * n_chunks) / take) * 64 + lane;
+        } else i = (int64_t)(((unsigned long long)j * (unsigned long long)n_chunks) / (unsigned long long)take) * 64 + lane;
         if (i >= words) i = -1;
       }
       at[u] = i;
@@ -1012,17 +1015,16 @@ __global__ __launch_bounds__(256) void k_fingerprint(const uint32_t *const *w_re
   if (lane == 0) red[wv] = h;
   __syncthreads();
   if (threadIdx.x == 0) {
-    unsigned long long *store = state + z, *sum = state + n_dec + z, *count = state + 2 * n_dec + z;
-    atomicAdd(sum, red[0] + red[1] + red[2] + red[3]);
+    unsigned long long *line = state + (int64_t)z * FP_STATE_WORDS;
+    __hip_atomic_store(line + blockIdx.x, red[0] + red[1] + red[2] + red[3], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __threadfence();
-    last = atomicAdd(count, 1ull) == (unsigned long long)(gridDim.x - 1) ? 1u : 0u;
-    if (last) {
+    if (atomicAdd(line + FP_BLOCKS + 1, 1ull) == (unsigned long long)(FP_BLOCKS - 1)) {
       __threadfence();
-      const unsigned long long now = atomicAdd(sum, 0ull);
-      changed[z] = (!store_only && now != *store) ? 1 : 0;
-      *store = now;
-      *sum = 0ull;
-      *count = 0ull;
+      unsigned long long now = 0;
+      for (int i = 0; i < FP_BLOCKS; ++i) now += __hip_atomic_load(line + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      changed[z] = (!store_only && now != line[FP_BLOCKS]) ? 1 : 0;
+      line[FP_BLOCKS] = now;
+      line[FP_BLOCKS + 1] = 0ull;
     }
   }
 }
@@ -1417,8 +1419,9 @@ extern "C" int clt_decoder_fingerprint(void *const *w_refs_dev, int64_t n_dec, i
   const int64_t words = d * F * clt_elem_bytes(dtype) / 4;     // a last odd 16-bit element is not looked at
   if (words <= 0) return CLT_ERR_ARG;
   const int64_t row_bytes = F * clt_elem_bytes(dtype);
+  if ((((uintptr_t)state) & 127u) != 0) return CLT_ERR_ALIGN;
   k_fingerprint<<<dim3(FP_BLOCKS, (unsigned)n_dec), 256, 0, (hipStream_t)stream>>>(
-      (const uint32_t *const *)w_refs_dev, words, d, row_bytes % 4 == 0 ? row_bytes / 4 : 0, n_dec,
+      (const uint32_t *const *)w_refs_dev, words, d, row_bytes % 4 == 0 ? row_bytes / 4 : 0,
       (unsigned long long *)state, changed, store_only);
   return clt_check_launch();
 }

@@ -257,7 +257,7 @@ class Decoder(nn.Module):
         if self.watch_parameter_data and not getattr(self, "_params_behind", False) \
                 and all(dec.weight.is_contiguous() for dec in decs):
             if self._fp_state is None or self._fp_state.device != w0.device:
-                self._fp_state = torch.zeros(3 * len(decs), dtype=torch.int64, device=w0.device)
+                self._fp_state = torch.zeros(16 * len(decs), dtype=torch.int64, device=w0.device)
                 self._fp_changed = torch.zeros(len(decs), dtype=torch.int32, device=w0.device)
                 self._fp_fresh = False
             table = self._pointer_table("w", [dec.weight for dec in decs])

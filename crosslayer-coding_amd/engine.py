@@ -617,10 +617,10 @@ def unpack_decoders(w_packed: torch.Tensor, w_refs_dev: torch.Tensor, w_refs_hos
 def decoder_fingerprint(w_refs_dev: torch.Tensor, d: int, F: int, dtype: torch.dtype, state: torch.Tensor,
                         changed: torch.Tensor, store_only: bool) -> None:
     """Hash a sample of every decoder parameter ([d, F] each, addresses in the device int64 tensor ``w_refs_dev``):
-    ``changed[i]`` = 1 where it differs from the hash kept in ``state`` (int64 [3 n_dec], zeros before the first
+    ``changed[i]`` = 1 where it differs from the hash kept in ``state`` (int64 [16 n_dec], zeros before the first
     call), which is brought up to date; ``store_only`` records without comparing."""
     n_dec = w_refs_dev.numel()
-    assert w_refs_dev.dtype == torch.int64 and state.dtype == torch.int64 and state.numel() == 3 * n_dec
+    assert w_refs_dev.dtype == torch.int64 and state.dtype == torch.int64 and state.numel() == 16 * n_dec
     assert changed.dtype == torch.int32 and changed.numel() == n_dec and state.is_contiguous()
     code = nat.load().clt_decoder_fingerprint(nat.ptr(w_refs_dev), n_dec, d, F, nat.dtype_code(dtype), nat.ptr(state),
                                               nat.ptr(changed), 1 if store_only else 0, _stream(state))

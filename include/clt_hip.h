@@ -401,8 +401,9 @@ int clt_decode_route(int64_t T, int64_t d, int64_t F, int64_t L, int tying, int 
  * of matrix i, [d][F]; all of a matrix up to 1 MiB, of a larger one a 256-byte run per row on a diagonal, so
  * that every row is looked at and every column in several rows):
  * changed[i] = 1 where the hash differs from the one kept in state, and state is brought up to date.
- * store_only != 0 only records (after the caller itself wrote the parameters).  `state` holds 3 * n_dec
- * 64-bit words, zeroed by the caller before the first call and left alone afterwards.
+ * store_only != 0 only records (after the caller itself wrote the parameters).  `state` holds 16 * n_dec
+ * 64-bit words (one 128-byte line per matrix, 128-byte aligned), zeroed by the caller before the first
+ * call - made with store_only - and left alone afterwards.
  * clt_pack_decoders_if repacks the matrices whose flag is set (clt_pack_decoder otherwise) - a launch that
  * costs microseconds when no flag is set.  Both run on the stream; nothing is read back.  A write to the
  * whole matrix, a whole row or a whole column of it is always seen; one that touches a few scattered elements
