@@ -705,6 +705,7 @@ def cpu_baseline(wl, model, slab, tokens):
 
 
 def main():
+    torch.set_grad_enabled(False)      # the forward is measured as inference; the training modes compute their own gradients
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)

@@ -44,6 +44,49 @@ class _NullTimer:
         return False
 
 
+class _ReconstructionsWithGraph(torch.autograd.Function):
+    """``forward`` as one node of an autograd graph: the reconstructions of all layers as functions of every
+    parameter.  The forward is the fused HIP path; the backward hands d loss / d reconstruction to the same
+    kernels ``loss_and_gradients`` uses (activations.py:66-96, 183-220 for the gates; the products are the
+    reference's linear layers, parallel.py:282-294, 335-383).  The inputs get no gradient."""
+
+    @staticmethod
+    def forward(ctx, model, inputs, names, *params):
+        with torch.no_grad():
+            recs, surv = model.forward_with_survivors(inputs)
+            surv = surv.trimmed()
+            # the list lives in the model's workspace, which the next forward overwrites: keep a copy
+            ctx.surv = SurvivorList(surv.row_ptr.clone(), surv.col.clone(), surv.val.clone(), surv.T, surv.F, surv.L,
+                                    surv.dtype, None, surv.nnz_hint)
+        ctx.model, ctx.inputs, ctx.names = model, inputs, names
+        ctx.versions = [p._version for p in params]
+        ctx.params = params
+        L = model.config.num_layers
+        return tuple(recs[l] for l in range(L))
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, *grad_outs):
+        model = ctx.model
+        if any(p._version != v for p, v in zip(ctx.params, ctx.versions)):
+            raise RuntimeError("a parameter of the CrossLayerTranscoder was modified in place between forward and "
+                               "backward: the gradient would be taken at other weights than the output was")
+        surv = ctx.surv
+        L, T, d = surv.L, surv.T, model.config.d_model
+        g = torch.zeros((L, T, d), dtype=torch.float32, device=surv.row_ptr.device)
+        for l, go in enumerate(grad_outs):
+            if go is not None:
+                g[l] = go.reshape(T, d)
+        g_model = g.to(model.dtype)
+        raw = model._raw_gradients_from(ctx.inputs, surv, g, g_model, g.sum(dim=1))
+        named = model._named_gradients(raw)
+        grads = []
+        for name, p in zip(ctx.names, ctx.params):
+            gp = named.get(name)
+            grads.append(None if gp is None or not p.requires_grad else gp.to(p.dtype).reshape(p.shape))
+        return (None, None, None, *grads)
+
+
 class CrossLayerTranscoder(BaseTranscoder):
     device: torch.device
     dtype: torch.dtype
@@ -226,6 +269,18 @@ class CrossLayerTranscoder(BaseTranscoder):
         tgt = torch.stack([targets[l].to(device=self.device, dtype=self.dtype).reshape(-1, d) for l in range(L)])
         mode, mean, std, scale = self._denorm_args(normalization_method, mean_tg, std_tg)
         loss_l, g, g_model, bias_grad = engine.mse_loss_grad(rec, tgt.contiguous(), ws, mode, mean, std, scale)
+        return loss_l, self._raw_gradients_from(inputs, surv, g, g_model, bias_grad, decoder_step)
+
+    def _raw_gradients_from(self, inputs: Dict[int, torch.Tensor], surv, g: torch.Tensor, g_model: torch.Tensor,
+                            bias_grad: torch.Tensor, decoder_step=None):
+        """The raw parameter gradients (see ``_loss_and_raw_gradients``) of any loss, given d loss / d reconstruction:
+        ``g`` fp32 [L, T, d], ``g_model`` the same in the model dtype, ``bias_grad`` [L, d] its sums over tokens.
+        ``surv`` is the (trimmed) survivor list of the forward on ``inputs``."""
+        cfg = self.config
+        L, d, F = cfg.num_layers, cfg.d_model, cfg.num_features
+        ws = self._workspace()
+        mask = (1 << L) - 1
+        dec = self.decoder_module
         off, sc = dec._affine()                     # per-target feature offset / scale of tied decoders, or None
         dval = engine.decode_backward_values(surv, dec.packed(), g, cfg.decoder_tying, mask, ws, feat_scale=sc)
         lists = engine.feature_lists(surv, ws)
@@ -257,8 +312,8 @@ class CrossLayerTranscoder(BaseTranscoder):
             dec_b = torch.flip(torch.cumsum(torch.flip(bias_grad, dims=[0]), dim=0), dims=[0])
         else:
             dec_b = bias_grad
-        return loss_l, {"enc_w": dw_enc, "enc_b": db_enc, "dec_w": dw_dec, "dec_b": dec_b.contiguous(), "theta": theta_grad,
-                        "skip": d_skip, "feat_offset": d_off, "feat_scale": d_sc}
+        return {"enc_w": dw_enc, "enc_b": db_enc, "dec_w": dw_dec, "dec_b": dec_b.contiguous(), "theta": theta_grad,
+                "skip": d_skip, "feat_offset": d_off, "feat_scale": d_sc}
 
     def _log_threshold_gradient(self, x_slab: torch.Tensor, g_model: torch.Tensor, ws, surv=None, dval=None) -> torch.Tensor:
         """fp32 [L, F] gradient of ``log_threshold`` (JumpReLU.backward, activations.py:196-199, through
@@ -320,6 +375,11 @@ class CrossLayerTranscoder(BaseTranscoder):
         self._no_half("loss_and_gradients")
         L = self.config.num_layers
         loss_l, raw = self._loss_and_raw_gradients(inputs, targets, normalization_method, mean_tg, std_tg)
+        return loss_l.sum(), self._named_gradients(raw)
+
+    def _named_gradients(self, raw) -> Dict[str, Optional[torch.Tensor]]:
+        """{state-dict key: fp32 gradient in the parameter's shape} from the raw gradient tensors."""
+        L = self.config.num_layers
         grads: Dict[str, Optional[torch.Tensor]] = {}
         for l in range(L):
             grads[f"encoder_module.encoders.{l}.weight"] = raw["enc_w"][l]
@@ -340,7 +400,7 @@ class CrossLayerTranscoder(BaseTranscoder):
             if raw.get(name) is not None:
                 for t in range(L):
                     grads[f"decoder_module.feature_{name[5:]}.{t}"] = raw[name][t]
-        return loss_l.sum(), grads
+        return grads
 
     @torch.no_grad()
     def training_step(self, inputs: Dict[int, torch.Tensor], targets: Dict[int, torch.Tensor], optimizer,
@@ -612,11 +672,36 @@ class CrossLayerTranscoder(BaseTranscoder):
             engine.poison_if(out, full.status)
         return {t: out[t] for t in targets}, full
 
+    def _graph_route_ok(self, inputs: Dict[int, torch.Tensor]) -> bool:
+        """Whether the gradient kernels take this batch: every layer present, one token count, right width."""
+        cfg = self.config
+        if sorted(inputs) != list(range(cfg.num_layers)):
+            return False
+        counts = set()
+        for x in inputs.values():
+            if not isinstance(x, torch.Tensor) or x.dim() not in (2, 3) or x.shape[-1] != cfg.d_model or x.numel() == 0:
+                return False
+            counts.add(x.numel() // cfg.d_model)
+        return len(counts) == 1 and cfg.activation_fn in ("batchtopk", "topk", "jumprelu", "relu")
+
     def forward(self, inputs: Dict[int, torch.Tensor]) -> Dict[int, torch.Tensor]:
-        """Reconstruction of every layer present in ``inputs`` (clt.py:186-218)."""
+        """Reconstruction of every layer present in ``inputs`` (clt.py:186-218).  With gradients enabled and
+        parameters that ask for them the result carries an autograd graph, as the reference's does: ``loss.backward()``
+        on any function of the reconstructions fills ``param.grad`` (inputs of every layer with equal token counts;
+        float32 / bfloat16)."""
         self._sync_device()
         cfg = self.config
         L, d = cfg.num_layers, cfg.d_model
+        if torch.is_grad_enabled() and self.dtype != torch.float16:
+            named = list(self.named_parameters())
+            if any(p.requires_grad for _, p in named):
+                if self._graph_route_ok(inputs):
+                    outs = _ReconstructionsWithGraph.apply(self, inputs, [n for n, _ in named], *[p for _, p in named])
+                    return {l: outs[l] for l in range(L)}
+                if not getattr(self, "_warned_no_graph", False):
+                    self._warned_no_graph = True
+                    logger.warning(f"Rank {self.rank}: forward builds no autograd graph for these inputs (it needs one "
+                                   f"2-D or 3-D tensor per layer with equal token counts); gradients will not flow.")
         res = self.forward_with_survivors(inputs)
         if res is not None:
             return res[0]

@@ -108,6 +108,30 @@ def test_gradients_match_the_reference(dev, case):
         assert torch.allclose(grads[name].cpu(), T(want), rtol=1e-4, atol=1e-6), name
 
 
+@pytest.mark.parametrize("case", FIX["gradients"] + FIX["gradients_skip_affine"] + FIX["gradients_jumprelu_affine"],
+                         ids=lambda c: c["name"])
+def test_backward_through_forward_matches_the_reference(dev, case):
+    # the reference's own idiom: reconstructions = model(inputs); loss = f(reconstructions); loss.backward().
+    # The forward carries an autograd graph whose backward runs the survivor-list kernels; the loss is written
+    # out in torch here (sum over layers of the mean squared error, losses.py:45-92 without normalisation)
+    model = load_model(case, dev)
+    for p in model.parameters():
+        p.requires_grad_(True)
+    inputs = {int(l): T(v, dev) for l, v in case["inputs"].items()}
+    targets = {int(l): T(v, dev) for l, v in case["targets"].items()}
+    recs = model(inputs)
+    loss = sum(((recs[l] - targets[l]) ** 2).mean() for l in sorted(recs))
+    assert float(loss) == pytest.approx(case["loss"], rel=1e-5)
+    loss.backward()
+    params = dict(model.named_parameters())
+    for name, want in case["gradients"].items():
+        assert params[name].grad is not None, name
+        assert torch.allclose(params[name].grad.cpu(), T(want), rtol=1e-4, atol=1e-6), name
+    # a forward under no_grad builds no graph
+    with torch.no_grad():
+        assert all(not r.requires_grad for r in model(inputs).values())
+
+
 @pytest.mark.parametrize("method", ["none", "mean_std", "sqrt_d_model"])
 def test_evaluator_metrics_match_the_reference(dev, method):
     ev = FIX["evaluator"]

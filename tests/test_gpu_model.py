@@ -302,9 +302,10 @@ def test_forward_reads_nothing_back_from_the_device(dev, name):
     torch.cuda.synchronize()
     torch.cuda.set_sync_debug_mode("error")
     try:
-        first = model(inputs)
-        second = model(inputs)
-        third = model(other)
+        with torch.no_grad():        # inference: with gradients enabled the forward keeps its survivor list for the backward
+            first = model(inputs)
+            second = model(inputs)
+            third = model(other)
     finally:
         torch.cuda.set_sync_debug_mode("default")
     torch.cuda.synchronize()

@@ -417,3 +417,58 @@ def test_data_writes_are_seen_next_to_other_kinds_of_writes_and_between_training
         out, want = model(inputs), twin(inputs)
         for t in range(3):
             assert torch.equal(out[t], want[t]), (fused, t)
+
+
+@pytest.mark.gpu
+def test_forward_then_backward_fills_the_gradients(dev):
+    # integration/test_clt_end_to_end.py:63-101: a ReLU model, the mean squared error of every reconstruction
+    # against its own input, loss.backward(), gradients on encoder weights, decoder weights and decoder biases
+    cfg = cca.CLTConfig(num_layers=2, d_model=8, num_features=16, activation_fn="relu")
+    model = cca.CrossLayerTranscoder(cfg, process_group=None, device=dev)
+    for p in model.parameters():
+        p.requires_grad = True
+    model = model.to(dev)
+    g = torch.Generator().manual_seed(9)
+    inputs = {0: torch.randn(20, 8, generator=g).to(dev), 1: torch.randn(20, 8, generator=g).to(dev)}
+    recs = model.forward(inputs)
+    loss = torch.tensor(0.0, device=dev, dtype=torch.float32)
+    for l, r in recs.items():
+        loss = loss + torch.mean((r - inputs[l]) ** 2)
+    loss.backward()
+    w_enc = model.encoder_module.encoders[0].weight
+    assert w_enc.grad is not None and bool(torch.isfinite(w_enc.grad).all())
+    # the reference initialises untied decoders to small random values, so the encoder sees a gradient
+    assert not bool((w_enc.grad == 0).all())
+    w_dec = model.decoder_module.decoders["0->1"].weight
+    assert w_dec.grad is not None and bool(torch.isfinite(w_dec.grad).all()) and not bool((w_dec.grad == 0).all())
+    b_dec = model.decoder_module.decoders["1->1"].bias_param
+    assert b_dec.grad is not None and bool(torch.isfinite(b_dec.grad).all())
+    # a parameter changed in place between forward and backward is reported, as autograd does for saved tensors
+    recs = model(inputs)
+    with torch.no_grad():
+        w_dec.mul_(2.0)
+    with pytest.raises(RuntimeError, match="modified in place"):
+        sum(r.sum() for r in recs.values()).backward()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_autograd_route_equals_loss_and_gradients(dev, dtype):
+    from crosslayer_coding_amd import synth
+    wl = synth.WORKLOADS["c0"].scaled("graph", dtype=dtype, num_layers=3, d_model=128, num_features=512, tokens=256, k=12)
+    model, inputs, _ = synth.build_model(wl, dev)
+    g = torch.Generator().manual_seed(2)
+    targets = {l: torch.randn(256, 128, generator=g).to(dev).to(model.dtype) for l in range(3)}
+    _, want = model.loss_and_gradients(inputs, targets)
+    recs = model(inputs)
+    assert all(r.requires_grad for r in recs.values())
+    loss = sum(((recs[l].float() - targets[l].float()) ** 2).mean() for l in range(3))
+    loss.backward()
+    for name, p in model.named_parameters():
+        if want.get(name) is None:
+            continue
+        assert p.grad is not None and p.grad.dtype == p.dtype, name
+        ref = want[name].float()
+        err = float((p.grad.float() - ref).norm() / ref.norm().clamp_min(1e-20))
+        # bfloat16: d loss / d reconstruction reaches the kernels rounded to bfloat16, as it does in the reference
+        assert err <= (1e-4 if dtype == "float32" else 2e-2), (name, err)
