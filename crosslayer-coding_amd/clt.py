@@ -175,6 +175,7 @@ class CrossLayerTranscoder(BaseTranscoder):
 
     def get_preactivations(self, x: torch.Tensor, layer_idx: int) -> torch.Tensor:
         self._sync_device()
+        self._note_no_graph("get_preactivations")
         return self.encoder_module.get_preactivations(x, layer_idx)
 
     def _encode_all_layers(self, inputs: Dict[int, torch.Tensor]
@@ -598,6 +599,7 @@ class CrossLayerTranscoder(BaseTranscoder):
     def get_feature_activations(self, inputs: Dict[int, torch.Tensor]) -> Dict[int, torch.Tensor]:
         """Dense activations per layer (clt.py:220-277)."""
         self._sync_device()
+        self._note_no_graph("get_feature_activations")
         cfg = self.config
         topk_family = cfg.activation_fn in ("batchtopk", "topk")
         res = self._survivors(inputs)
@@ -671,6 +673,16 @@ class CrossLayerTranscoder(BaseTranscoder):
             # device overwrites the output with NaN rather than leave what an empty list decodes to
             engine.poison_if(out, full.status)
         return {t: out[t] for t in targets}, full
+
+    def _note_no_graph(self, what: str) -> None:
+        """Say once per model that ``what`` returns tensors outside the autograd graph although gradients are on:
+        a loss term built on them (the reference's sparsity / pre-activation penalties, losses.py:94-328) would
+        silently contribute nothing to ``param.grad``."""
+        if torch.is_grad_enabled() and not self.__dict__.get("_told_no_graph", {}).get(what):
+            if any(p.requires_grad for p in self.encoder_module.parameters()):
+                self.__dict__.setdefault("_told_no_graph", {})[what] = True
+                logger.warning(f"Rank {self.rank}: {what} returns tensors without an autograd graph; only forward() is "
+                               f"differentiable here. Loss terms built on {what} add nothing to the gradients.")
 
     def _graph_route_ok(self, inputs: Dict[int, torch.Tensor]) -> bool:
         """Whether the gradient kernels take this batch: every layer present, one token count, right width."""
