@@ -121,7 +121,7 @@ def test_backward_through_forward_matches_the_reference(dev, case):
     targets = {int(l): T(v, dev) for l, v in case["targets"].items()}
     recs = model(inputs)
     loss = sum(((recs[l] - targets[l]) ** 2).mean() for l in sorted(recs))
-    assert float(loss) == pytest.approx(case["loss"], rel=1e-5)
+    assert float(loss.detach()) == pytest.approx(case["loss"], rel=1e-5)
     loss.backward()
     params = dict(model.named_parameters())
     for name, want in case["gradients"].items():
