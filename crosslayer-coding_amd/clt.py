@@ -552,7 +552,11 @@ class CrossLayerTranscoder(BaseTranscoder):
         if key != self._thr_key:
             self._thr_key, self._thr_pending, self._thr_last_total = key, [], None
         self._thr_elems = n * T * F
-        self._poll_threshold_runs()
+        # under stream capture (a HIP graph of the forward) nothing may be asked of events or copied for the host:
+        # the pool keeps the size it has, which only speed depends on
+        capturing = torch.cuda.is_current_stream_capturing()
+        if not capturing:
+            self._poll_threshold_runs()
         theta = None
         if fn == "jumprelu":
             theta = self.theta_manager.thresholds(self.dtype)
@@ -572,6 +576,8 @@ class CrossLayerTranscoder(BaseTranscoder):
                                            read_back=read_back)
         if surv.status is None:
             self._note_threshold_total(int(surv.nnz_hint), self._thr_last_total is None)
+        elif capturing:
+            surv.nnz_hint = self._thr_last_total
         else:
             # the total travels to pinned memory behind the kernels; a later forward looks at it
             surv.nnz_hint = self._thr_last_total

@@ -442,3 +442,39 @@ def test_profiler_hook_receives_the_reference_timer_names(dev):
     model.load_state_dict(sd)
     model({l: x[l].to(dev) for l in range(wl.num_layers)})
     assert "batchtopk_activation" in prof.records and "batchtopk_compute_mask" in prof.records
+
+
+@pytest.mark.parametrize("kw", [dict(), dict(activation_fn="jumprelu", k=None), dict(topk_mode="global"),
+                                dict(decoder_tying="per_target")], ids=["topk", "jumprelu", "global", "per-target"])
+def test_inference_forward_replays_from_a_graph(dev, kw):
+    # The inference forward is launches on the current stream and nothing else (no allocation inside the library,
+    # no memset, nothing read back), so it can be captured once and replayed.  Every replay - on new inputs, with
+    # eager forwards and synchronisations in between - must equal the eager result bit for bit.
+    wl = BASE.scaled("graph", dtype="bfloat16", num_layers=3, d_model=256, num_features=1024, tokens=512,
+                     **({"k": 16} if "k" not in kw else {}), **kw)
+    model, sd, x = build(wl, dev)
+    model.eval()
+    inputs = {l: x[l].to(dev) for l in range(wl.num_layers)}
+    static_in = {l: v.clone() for l, v in inputs.items()}
+    with torch.no_grad():
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                model(static_in)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            out = model(static_in)
+        for rep in range(4):
+            new = {l: (v * (1.0 + 0.1 * rep)).to(v.dtype) for l, v in inputs.items()}
+            for l in new:
+                static_in[l].copy_(new[l])
+            graph.replay()
+            torch.cuda.synchronize()
+            got = {l: o.clone() for l, o in out.items()}
+            want = model(new)
+            torch.cuda.synchronize()
+            for l in want:
+                assert torch.equal(got[l], want[l]), (rep, l)
