@@ -108,6 +108,18 @@ class Workspace:
 
 # below this many (token, target) rows one wavefront per row already underfills the GPU
 SLICED_DECODE_MIN_ROWS = 8192
+# ... or, whatever the batch, when the decoders are far larger than the caches: a short batch then spends its time
+# fetching decoder rows from HBM, and the schedules that give each XCD its own part of a matrix fetch every row once
+# instead of once per XCD that happens to need it (C1 with 64 tokens: 1.64 -> 1.29 ms, C0 with 256: 2.79 -> 1.87 ms)
+SLICED_DECODE_MIN_SLAB_BYTES = 128 << 20
+
+
+def _wants_sliced_decode(rows: int, slab_bytes: int) -> bool:
+    return rows >= SLICED_DECODE_MIN_ROWS or slab_bytes >= SLICED_DECODE_MIN_SLAB_BYTES
+
+
+# token rows of one tile of the matrix-core encoder: shorter batches are padded to it (see ``encode``)
+ENCODE_MIN_TOKENS = 256
 
 
 def _stream(t: torch.Tensor) -> int:
@@ -128,6 +140,20 @@ def encode(x: torch.Tensor, w: torch.Tensor, b: Optional[torch.Tensor],
     if b is not None:
         assert b.shape == (L, F) and b.stride(1) == 1 and b.dtype == x.dtype
     lib = nat.load()
+    stage = 256 // x.element_size()          # elements of K in two 128-byte stages of the matrix-core kernel
+    if 0 < T < ENCODE_MIN_TOKENS and F >= 256 and F % 4 == 0 and d % stage == 0:
+        # The matrix-core kernel works on whole 256-token tiles; a shorter batch (a short prompt) would fall to
+        # the one-thread-per-output kernel, which is 30x slower than the padded product.  Rows past T are zeros
+        # going in and are dropped coming out.
+        xp = torch.zeros((L, ENCODE_MIN_TOKENS, d), dtype=x.dtype, device=x.device)
+        xp[:, :T] = x
+        outp = torch.empty((L, ENCODE_MIN_TOKENS, F), dtype=x.dtype, device=x.device)
+        code = lib.clt_encode(nat.ptr(xp), nat.ptr(w), nat.ptr(b), nat.ptr(outp), ENCODE_MIN_TOKENS, d, F, L,
+                              xp.stride(0), w.stride(0), b.stride(0) if b is not None else 0, outp.stride(0),
+                              nat.dtype_code(x.dtype), _stream(x))
+        nat.check(code, "clt_encode")
+        out.copy_(outp[:, :T])
+        return out
     code = lib.clt_encode(nat.ptr(x), nat.ptr(w), nat.ptr(b), nat.ptr(out), T, d, F, L,
                           x.stride(0), w.stride(0), b.stride(0) if b is not None else 0, out.stride(0),
                           nat.dtype_code(x.dtype), _stream(x))
@@ -803,7 +829,7 @@ def decode_sparse(surv: SurvivorList, w_packed: torch.Tensor, tying: str, d: int
     if need < 0 or w_packed.numel() < need:
         raise nat.CLTNativeError(f"decode_sparse: packed decoders hold {w_packed.numel()} elements, the kernels index {need}")
     wbuf, wbytes = None, 0
-    if ws is not None and T * (t_end - t_begin) >= SLICED_DECODE_MIN_ROWS:
+    if ws is not None and _wants_sliced_decode(T * (t_end - t_begin), w_packed.numel() * w_packed.element_size()):
         wbytes = lib.clt_decode_workspace_bytes(T, d, F, L)
         wbuf = ws.get("decode", wbytes)
     code = lib.clt_decode_sparse(
@@ -820,7 +846,9 @@ def decode_route(T: int, d: int, F: int, L: int, tying: str, dtype: torch.dtype,
     and ``rows`` = tokens x targets of the call (default: all L targets)."""
     lib = nat.load()
     rows = T * L if rows is None else rows
-    wbytes = lib.clt_decode_workspace_bytes(T, d, F, L) if rows >= SLICED_DECODE_MIN_ROWS else 0
+    n_dec = L * (L + 1) // 2 if tying == "none" else L
+    slab_bytes = n_dec * F * decoder_pitch(d, dtype) * torch.empty((), dtype=dtype).element_size()
+    wbytes = lib.clt_decode_workspace_bytes(T, d, F, L) if _wants_sliced_decode(rows, slab_bytes) else 0
     code = lib.clt_decode_route(T, d, F, L, nat.TYING[tying], nat.dtype_code(dtype), wbytes)
     if code < 0:
         nat.check(code, "clt_decode_route")

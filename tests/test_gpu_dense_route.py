@@ -140,5 +140,8 @@ def test_route_query_names_the_schedules(dev):
     assert engine.decode_route(4096, 640, 24576, 12, "per_source", torch.bfloat16) == nat.ROUTE_LINE
     assert engine.decode_route(4096, 4096, 24576, 12, "none", torch.bfloat16) == nat.ROUTE_LINE     # wider than a wavefront's registers hold
     assert engine.decode_route(4096, 200, 24576, 12, "per_source", torch.bfloat16) == nat.ROUTE_SLICED
-    assert engine.decode_route(16, 768, 24576, 12, "none", torch.bfloat16, rows=16) == nat.ROUTE_SINGLE
+    # a short batch keeps the XCD-partitioned schedule when the decoders are far larger than the caches (3.2 GB
+    # here) and takes the one-pass kernel when they are small
+    assert engine.decode_route(16, 768, 24576, 12, "none", torch.bfloat16, rows=16) == nat.ROUTE_QUARTER
+    assert engine.decode_route(16, 768, 2048, 4, "none", torch.bfloat16, rows=16) == nat.ROUTE_SINGLE
     assert engine.decode_route(4096, 100, 24576, 12, "none", torch.bfloat16, rows=big) == nat.ROUTE_GENERIC

@@ -37,7 +37,8 @@ def check_rows_sorted(surv):
 
 # ---- encoder --------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("L,T,d,F", [(1, 30, 8, 16), (2, 300, 64, 136), (3, 257, 96, 260), (1, 5, 7, 9), (2, 512, 768, 512)])
+@pytest.mark.parametrize("L,T,d,F", [(1, 30, 8, 16), (2, 300, 64, 136), (3, 257, 96, 260), (1, 5, 7, 9), (2, 512, 768, 512),
+                                     (2, 40, 256, 512), (1, 1, 128, 256), (3, 255, 128, 260)])   # short batches: padded to a tile
 def test_encode_parity(dev, dtype, L, T, d, F):
     g = torch.Generator().manual_seed(L * 1000 + T)
     x = torch.randn(L, T, d, generator=g).to(dtype)

@@ -58,6 +58,9 @@ CASES = [
     # shapes that take the routes fused into the encoder epilogue (T % 256 == 0, F % 256 == 0)
     BASE.scaled("fused-topk", num_layers=3, d_model=128, num_features=512, tokens=256, k=12),
     BASE.scaled("fused-topk-bf16", num_layers=3, d_model=256, num_features=1024, tokens=512, k=24, dtype="bfloat16"),
+    # a short prompt on a model whose shapes take the matrix-core encoder: the batch is padded to one tile
+    BASE.scaled("short-prompt-bf16", num_layers=3, d_model=256, num_features=1024, tokens=40, k=8, dtype="bfloat16"),
+    BASE.scaled("short-prompt-jump", num_layers=3, d_model=256, num_features=1024, tokens=7, activation_fn="jumprelu", k=None),
     BASE.scaled("fused-jump", num_layers=3, d_model=128, num_features=512, tokens=256, activation_fn="jumprelu", k=None),
     BASE.scaled("fused-jump-bf16", num_layers=3, d_model=256, num_features=1024, tokens=512, activation_fn="jumprelu",
                 k=None, dtype="bfloat16"),
