@@ -211,10 +211,11 @@ __global__ __launch_bounds__(256) void k_sample_keys(
 // One block per problem: the cut key = the r-th largest sample key, r chosen so that the
 // expected number of elements above the cut is about 1.25 K plus six standard deviations.
 // Also resets the problem's histogram, pool counter and state.
-template <int KB, int SN>
+template <typename T, int SN>
 __global__ __launch_bounds__(SCAN_THREADS) void k_sample_cut(
     const uint32_t *sample, unsigned long long N, unsigned long long K, SelState *st, uint32_t *hist,
     uint32_t *pool_count, uint32_t *aux_count, uint32_t path) {
+  constexpr int KB = Elem<T>::KEYBITS;
   constexpr int PER = SN / SCAN_THREADS;
   __shared__ uint32_t lh[NBINS];
   const int p = blockIdx.x, tid = threadIdx.x;
@@ -238,7 +239,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_sample_cut(
     r = path == PATH_TILES ? (unsigned long long)(1.2 * e + 6.0 * sqrt(e) + 16.0) + 1
                            : (unsigned long long)(1.25 * e + 6.0 * sqrt(e) + 16.0) + 1;
   }
-  uint32_t cut = min_key<KB>();
+  uint32_t cut = min_key_of<T>();
   if (r <= ns && r > 0) {
     constexpr int NLEV = KB == 32 ? 3 : 2;
     const int shifts[3] = {KB == 32 ? 21 : 5, KB == 32 ? 10 : 0, 0};
@@ -262,7 +263,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_sample_cut(
       prefix_mask |= dm << sh;
     }
     cut = prefix;
-    if (cut < min_key<KB>()) cut = min_key<KB>();
+    if (cut < min_key_of<T>()) cut = min_key_of<T>();
   }
   if (tid == 0) {
     SelState s;
@@ -490,8 +491,9 @@ __global__ __launch_bounds__(256) void k_select_pass(
 }
 
 // One block per problem: consume the histogram of the current level.
-template <int KB>
+template <typename T>
 __global__ __launch_bounds__(SCAN_THREADS) void k_select_scan(SelState *st, uint32_t *hist, uint32_t *pool_count, int phase, int level) {
+  constexpr int KB = Elem<T>::KEYBITS;
   __shared__ uint32_t lh[NBINS];
   const int p = blockIdx.x, tid = threadIdx.x;
   SelState s = st[p];
@@ -508,7 +510,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_select_scan(SelState *st, uint
   if (s.overflow) found = false;   // the collecting encoder dropped candidates: start over from the matrix
   if (!found) {
     // fewer candidates than K: the sampled cut was too high -> run the pass again from the bottom
-    s.status = ST_RETRY; s.cut_key = min_key<KB>(); s.level = 0; s.path = PATH_ROWS; s.overflow = 0;
+    s.status = ST_RETRY; s.cut_key = min_key_of<T>(); s.level = 0; s.path = PATH_ROWS; s.overflow = 0;
     pool_count[p] = 0;  // the retry pass refills the pool from scratch
     st[p] = s;
     return;
@@ -893,7 +895,7 @@ __global__ __launch_bounds__(256) void k_pool_hist(const SelState *st, const uin
 constexpr int TILE_NE = 4;   // entries of a run fetched in one batch
 template <typename T>
 __global__ __launch_bounds__(256) void k_tile_count(
-    int Tn, const SelState *st, const uint2 *seg_meta, int nseg, const uint2 *pool, unsigned long long pool_cap,
+    int Tn, int Tp, const SelState *st, const uint2 *seg_meta, int nseg, const uint2 *pool, unsigned long long pool_cap,
     uint8_t *cgt, uint8_t *ceq) {
   constexpr int KB = Elem<T>::KEYBITS;
   const int l = blockIdx.z, seg = blockIdx.y;
@@ -902,7 +904,7 @@ __global__ __launch_bounds__(256) void k_tile_count(
   const uint2 *mypool = pool + (unsigned long long)l * pool_cap;
   const int row = blockIdx.x * 256 + threadIdx.x;
   if (row >= Tn) return;
-  const int64_t at = ((int64_t)l * nseg + seg) * Tn + row;
+  const int64_t at = ((int64_t)l * nseg + seg) * Tp + collect_grid_row(row, Tn, Tp);
   const uint2 m = seg_meta[at];
   uint32_t raw[TILE_NE];
 #pragma unroll
@@ -925,29 +927,29 @@ __global__ __launch_bounds__(256) void k_tile_count(
 
 // k_row_prefix: per row, exclusive prefix of those counts over the segments, and the row totals.
 __global__ __launch_bounds__(256) void k_row_prefix(
-    int64_t Tn, const SelState *st, int nseg, const uint8_t *cgt, const uint8_t *ceq, uint32_t *pgt, uint32_t *peq,
-    uint32_t *row_gt, uint32_t *row_eq) {
+    int64_t Tn, int64_t Tp, const SelState *st, int nseg, const uint8_t *cgt, const uint8_t *ceq, uint32_t *pgt,
+    uint32_t *peq, uint32_t *row_gt, uint32_t *row_eq) {
   const int l = blockIdx.y;
   const SelState s = st[l];
   if (s.path != PATH_TILES || s.status != ST_DONE) return;
   const int64_t row = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (row >= Tn) return;
   uint32_t g = 0, q = 0;
-  const int64_t base = (int64_t)l * nseg * Tn + row;
+  const int64_t base = (int64_t)l * nseg * Tp + collect_grid_row(row, Tn, Tp);
   int seg = 0;
   for (; seg + 8 <= nseg; seg += 8) {
     uint32_t a[8], b[8];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) { a[i] = cgt[base + (int64_t)(seg + i) * Tn]; b[i] = ceq[base + (int64_t)(seg + i) * Tn]; }
+    for (int i = 0; i < 8; ++i) { a[i] = cgt[base + (int64_t)(seg + i) * Tp]; b[i] = ceq[base + (int64_t)(seg + i) * Tp]; }
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      pgt[base + (int64_t)(seg + i) * Tn] = g; peq[base + (int64_t)(seg + i) * Tn] = q;
+      pgt[base + (int64_t)(seg + i) * Tp] = g; peq[base + (int64_t)(seg + i) * Tp] = q;
       g += a[i]; q += b[i];
     }
   }
   for (; seg < nseg; ++seg) {
-    const uint32_t a = cgt[base + (int64_t)seg * Tn], b = ceq[base + (int64_t)seg * Tn];
-    pgt[base + (int64_t)seg * Tn] = g; peq[base + (int64_t)seg * Tn] = q;
+    const uint32_t a = cgt[base + (int64_t)seg * Tp], b = ceq[base + (int64_t)seg * Tp];
+    pgt[base + (int64_t)seg * Tp] = g; peq[base + (int64_t)seg * Tp] = q;
     g += a; q += b;
   }
   row_gt[(int64_t)l * Tn + row] = g; row_eq[(int64_t)l * Tn + row] = q;
@@ -958,7 +960,7 @@ __global__ __launch_bounds__(256) void k_row_prefix(
 // the entries kept before it in its own run.
 template <typename T>
 __global__ __launch_bounds__(256) void k_tile_emit(
-    int Tn, const SelState *st, const uint2 *seg_meta, int nseg, const uint2 *pool, unsigned long long pool_cap,
+    int Tn, int Tp, const SelState *st, const uint2 *seg_meta, int nseg, const uint2 *pool, unsigned long long pool_cap,
     const uint32_t *pgt, const uint32_t *peq, const uint32_t *allot, const int32_t *row_ptr, int32_t *col_out,
     T *val_out) {
   constexpr int KB = Elem<T>::KEYBITS;
@@ -968,7 +970,7 @@ __global__ __launch_bounds__(256) void k_tile_emit(
   const uint2 *mypool = pool + (unsigned long long)l * pool_cap;
   const int row = blockIdx.x * 256 + threadIdx.x;
   if (row >= Tn) return;
-  const int64_t at = ((int64_t)l * nseg + seg) * Tn + row;
+  const int64_t at = ((int64_t)l * nseg + seg) * Tp + collect_grid_row(row, Tn, Tp);
   const uint2 m = seg_meta[at];
   if (m.y == 0) return;
   const int64_t r = (int64_t)l * Tn + row;
@@ -1026,24 +1028,24 @@ __global__ void k_selected_min_accumulate(const uint32_t *keys, int64_t n, T *su
 
 // ---- threshold activation on encoder-collected entries (every entry is a survivor) ----------
 // Per row: exclusive prefix of the run lengths over the segments, and the row total.
-__global__ __launch_bounds__(256) void k_row_prefix_meta(int64_t Tn, int nseg, const uint2 *seg_meta, uint32_t *pfx,
-                                                         uint32_t *row_cnt) {
+__global__ __launch_bounds__(256) void k_row_prefix_meta(int64_t Tn, int64_t Tp, int nseg, const uint2 *seg_meta,
+                                                         uint32_t *pfx, uint32_t *row_cnt) {
   const int l = blockIdx.y;
   const int64_t row = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (row >= Tn) return;
   uint32_t g = 0;
-  const int64_t base = (int64_t)l * nseg * Tn + row;
+  const int64_t base = (int64_t)l * nseg * Tp + collect_grid_row(row, Tn, Tp);
   int seg = 0;
   for (; seg + 8 <= nseg; seg += 8) {
     uint32_t a[8];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) a[i] = seg_meta[base + (int64_t)(seg + i) * Tn].y;
+    for (int i = 0; i < 8; ++i) a[i] = seg_meta[base + (int64_t)(seg + i) * Tp].y;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) { pfx[base + (int64_t)(seg + i) * Tn] = g; g += a[i]; }
+    for (int i = 0; i < 8; ++i) { pfx[base + (int64_t)(seg + i) * Tp] = g; g += a[i]; }
   }
   for (; seg < nseg; ++seg) {
-    const uint32_t a = seg_meta[base + (int64_t)seg * Tn].y;
-    pfx[base + (int64_t)seg * Tn] = g; g += a;
+    const uint32_t a = seg_meta[base + (int64_t)seg * Tp].y;
+    pfx[base + (int64_t)seg * Tp] = g; g += a;
   }
   row_cnt[(int64_t)l * Tn + row] = g;
 }
@@ -1059,14 +1061,14 @@ __global__ void k_thresh_finish(const SelState *st, int L, int32_t *row_ptr, int
 // Grid: x = blocks of 256 rows, y = segment, z = layer.
 template <typename T>
 __global__ __launch_bounds__(256) void k_tile_emit_all(
-    int Tn, const uint2 *seg_meta, int nseg, const uint2 *pool, unsigned long long pool_cap, const uint32_t *pfx,
+    int Tn, int Tp, const uint2 *seg_meta, int nseg, const uint2 *pool, unsigned long long pool_cap, const uint32_t *pfx,
     const int32_t *row_ptr, int32_t *col_out, T *val_out, const int32_t *skip) {
   if (skip && *skip != 0) return;             // the list did not fit the caller's arrays: it was emptied
   const int l = blockIdx.z, seg = blockIdx.y;
   const uint2 *mypool = pool + (unsigned long long)l * pool_cap;
   const int row = blockIdx.x * 256 + threadIdx.x;
   if (row >= Tn) return;
-  const int64_t at = ((int64_t)l * nseg + seg) * Tn + row;
+  const int64_t at = ((int64_t)l * nseg + seg) * Tp + collect_grid_row(row, Tn, Tp);
   const uint2 m = seg_meta[at];
   if (m.y == 0) return;
   uint2 en[TILE_NE];
@@ -1359,7 +1361,7 @@ static int run_batchtopk(const T *pre, int64_t Tn, int64_t F, int64_t L, int64_t
   if (K > N) K = N;
   const int nprob = lo.nprob;
   k_sample_keys<T, GLOBAL><<<dim3(SAMPLE_BLOCKS, nprob), 256, 0, stream>>>(pre, Tn, F, L, lstride, mean, denom, N, sample);
-  k_sample_cut<KB, SAMPLE_N><<<nprob, SCAN_THREADS, 0, stream>>>(sample, N, K, st, hist, poolcnt, nullptr, PATH_ROWS);
+  k_sample_cut<T, SAMPLE_N><<<nprob, SCAN_THREADS, 0, stream>>>(sample, N, K, st, hist, poolcnt, nullptr, PATH_ROWS);
   // two rows per wavefront: many more blocks than fit at once, so rows of very different
   // candidate counts balance out over the CUs
   int gx = (int)clt_ceil_div(Tn, 8);
@@ -1372,7 +1374,7 @@ static int run_batchtopk(const T *pre, int64_t Tn, int64_t F, int64_t L, int64_t
   }
   for (int phase = 0; phase < 2; ++phase) {
     k_select_pass<T, V, GLOBAL><<<grid, 256, 0, stream>>>(pre, Tn, F, L, lstride, mean, denom, st, hist, poolcnt, pool, lo.pool_cap, first, phase, xcut);
-    k_select_scan<KB><<<nprob, SCAN_THREADS, 0, stream>>>(st, hist, poolcnt, phase, 0);
+    k_select_scan<T><<<nprob, SCAN_THREADS, 0, stream>>>(st, hist, poolcnt, phase, 0);
   }
   int gx2 = (int)clt_ceil_div(Tn, 4);
   int maxgx2 = (int)clt_ceil_div(256 * 8, L);
@@ -1382,7 +1384,7 @@ static int run_batchtopk(const T *pre, int64_t Tn, int64_t F, int64_t L, int64_t
   const int nlev = KB == 32 ? 3 : 2;
   for (int level = 1; level < nlev; ++level) {
     k_select_level<T, GLOBAL><<<grid2, 256, 0, stream>>>(pre, Tn, F, L, lstride, mean, denom, st, hist, first, pool, lo.pool_cap, level);
-    k_select_scan<KB><<<nprob, SCAN_THREADS, 0, stream>>>(st, hist, poolcnt, 2, level);
+    k_select_scan<T><<<nprob, SCAN_THREADS, 0, stream>>>(st, hist, poolcnt, 2, level);
   }
   k_select_count<T, GLOBAL><<<grid2, 256, 0, stream>>>(pre, Tn, F, L, lstride, mean, denom, st, first, pool, lo.pool_cap, rgt, req);
   k_select_allot<GLOBAL><<<nprob, SCAN_THREADS, 0, stream>>>(st, Tn, L, rgt, req, allot, keep, row_ptr, K);
@@ -1450,7 +1452,8 @@ static TileLayout tile_layout(int64_t T, int64_t F, int64_t L, int64_t k, int dt
   tl.sel = sel_layout(T, F, L, k, CLT_TOPK_PER_LAYER);
   const int segw = dtype != CLT_F32 ? 128 : 64;
   tl.nseg = (int)(F / segw);
-  tl.ntile = tl.nseg * (int)(T / COLLECT_ROWS);
+  const int64_t Tp = collect_grid_rows(T);   // the epilogue's books cover whole token tiles
+  tl.ntile = tl.nseg * (int)(Tp / COLLECT_ROWS);
   // about 1.5x K candidates are expected, i.e. 1.5 * k / F of a tile's 64 * segw elements; a
   // slot holds three times that (at least 64, at most the whole tile)
   unsigned long long caps = (unsigned long long)(3.0 * 1.5 * (double)k / (double)F * (double)COLLECT_ROWS * segw) + 64ull;
@@ -1465,9 +1468,9 @@ static TileLayout tile_layout(int64_t T, int64_t F, int64_t L, int64_t k, int dt
   size_t o = tl.sel.total;
   auto take = [&](size_t bytes) { size_t at = o; o += (bytes + 255) & ~(size_t)255; return at; };
   tl.off_tmeta = take(8 * (size_t)tl.ntile * (size_t)L);
-  tl.off_meta = take(8 * (size_t)tl.nseg * (size_t)T * (size_t)L);
+  tl.off_meta = take(8 * (size_t)tl.nseg * (size_t)Tp * (size_t)L);
   tl.off_tpool = take(8 * (size_t)tl.tpool_cap * (size_t)L);
-  const size_t cells = (size_t)tl.nseg * (size_t)T * (size_t)L;   // (row, segment) pairs
+  const size_t cells = (size_t)tl.nseg * (size_t)Tp * (size_t)L;   // (row, segment) pairs
   tl.off_cgt = take(cells);
   tl.off_ceq = take(cells);
   tl.off_pgt = take(4 * cells);
@@ -1493,7 +1496,7 @@ static int run_encode_collect(const void *x, const void *w, const void *b, void 
   if (K > N) K = N;
   k_sample_mfma<T><<<dim3(SAMPLE_WAVES / 4, (unsigned)L), 256, 0, stream>>>((const T *)x, (const T *)w, (const T *)b, Tn, d,
                                                                           F, xs, wstr, bs, sample);
-  k_sample_cut<KB, SAMPLE_PRE_N><<<(unsigned)L, SCAN_THREADS, 0, stream>>>(sample, N, K, st, hist, poolcnt,
+  k_sample_cut<T, SAMPLE_PRE_N><<<(unsigned)L, SCAN_THREADS, 0, stream>>>(sample, N, K, st, hist, poolcnt,
                                                               (uint32_t *)(ws + tl.off_tcount), PATH_TILES);
   uint2 *tpool = (uint2 *)(ws + tl.off_tpool);
   CollectArgs ca;
@@ -1503,7 +1506,7 @@ static int run_encode_collect(const void *x, const void *w, const void *b, void 
   int rc = clt_launch_encode(x, w, b, nullptr, Tn, d, F, L, xs, wstr, bs, ps, dtype, 1, nullptr, &ca, stream);
   if (rc != CLT_OK) return rc;
   k_pool_hist<T><<<dim3(256, (unsigned)L), 256, 0, stream>>>(st, ca.tile_meta, tl.ntile, tpool, tl.tpool_cap, hist, 0);
-  k_select_scan<KB><<<(unsigned)L, SCAN_THREADS, 0, stream>>>(st, hist, poolcnt, 0, 0);
+  k_select_scan<T><<<(unsigned)L, SCAN_THREADS, 0, stream>>>(st, hist, poolcnt, 0, 0);
   // layers whose cut failed (too few candidates, or no pool space left) get their pre-activations
   // written out and go through the streaming pass; the launch does nothing for the others
   return clt_launch_encode(x, w, b, pre, Tn, d, F, L, xs, wstr, bs, ps, dtype, 0, st, nullptr, stream);
@@ -1534,7 +1537,7 @@ static int run_collect_select(const T *pre, int64_t Tn, int64_t F, int64_t L, in
   // retry of the layers whose cut failed: streaming pass from the bottom key over `pre`
   k_select_pass<T, VV, false><<<dim3(gx, (unsigned)L), 256, 0, stream>>>(pre, Tn, F, L, lstride, nullptr, nullptr, st, hist,
                                                                         poolcnt, pool, lo.pool_cap, first, 1, nullptr);
-  k_select_scan<KB><<<(unsigned)L, SCAN_THREADS, 0, stream>>>(st, hist, poolcnt, 1, 0);
+  k_select_scan<T><<<(unsigned)L, SCAN_THREADS, 0, stream>>>(st, hist, poolcnt, 1, 0);
   int gx2 = (int)clt_ceil_div(Tn, 4);
   int maxgx2 = (int)clt_ceil_div(256 * 8, L);
   if (maxgx2 < 1) maxgx2 = 1;
@@ -1544,16 +1547,17 @@ static int run_collect_select(const T *pre, int64_t Tn, int64_t F, int64_t L, in
   for (int level = 1; level < nlev; ++level) {
     k_pool_hist<T><<<dim3(256, (unsigned)L), 256, 0, stream>>>(st, tmeta, tl.ntile, tpool, tl.tpool_cap, hist, level);
     k_select_level<T, false><<<grid2, 256, 0, stream>>>(pre, Tn, F, L, lstride, nullptr, nullptr, st, hist, first, pool, lo.pool_cap, level);
-    k_select_scan<KB><<<(unsigned)L, SCAN_THREADS, 0, stream>>>(st, hist, poolcnt, 2, level);
+    k_select_scan<T><<<(unsigned)L, SCAN_THREADS, 0, stream>>>(st, hist, poolcnt, 2, level);
   }
   dim3 grid3((unsigned)clt_ceil_div(Tn, 256), (unsigned)tl.nseg, (unsigned)L);
   uint8_t *cgt = (uint8_t *)(ws + tl.off_cgt), *ceq = (uint8_t *)(ws + tl.off_ceq);
   uint32_t *pgt = (uint32_t *)(ws + tl.off_pgt), *peq = (uint32_t *)(ws + tl.off_peq);
-  k_tile_count<T><<<grid3, 256, 0, stream>>>((int)Tn, st, meta, tl.nseg, tpool, tl.tpool_cap, cgt, ceq);
-  k_row_prefix<<<dim3((unsigned)clt_ceil_div(Tn, 64), (unsigned)L), 64, 0, stream>>>(Tn, st, tl.nseg, cgt, ceq, pgt, peq, rgt, req);
+  const int64_t Tp = collect_grid_rows(Tn);
+  k_tile_count<T><<<grid3, 256, 0, stream>>>((int)Tn, (int)Tp, st, meta, tl.nseg, tpool, tl.tpool_cap, cgt, ceq);
+  k_row_prefix<<<dim3((unsigned)clt_ceil_div(Tn, 64), (unsigned)L), 64, 0, stream>>>(Tn, Tp, st, tl.nseg, cgt, ceq, pgt, peq, rgt, req);
   k_select_count<T, false><<<grid2, 256, 0, stream>>>(pre, Tn, F, L, lstride, nullptr, nullptr, st, first, pool, lo.pool_cap, rgt, req);
   k_select_allot<false><<<(unsigned)L, SCAN_THREADS, 0, stream>>>(st, Tn, L, rgt, req, allot, keep, row_ptr, K);
-  k_tile_emit<T><<<grid3, 256, 0, stream>>>((int)Tn, st, meta, tl.nseg, tpool, tl.tpool_cap, pgt, peq, allot, row_ptr, col, val);
+  k_tile_emit<T><<<grid3, 256, 0, stream>>>((int)Tn, (int)Tp, st, meta, tl.nseg, tpool, tl.tpool_cap, pgt, peq, allot, row_ptr, col, val);
   k_select_emit<T, false><<<grid2, 256, 0, stream>>>(pre, Tn, F, L, lstride, nullptr, nullptr, st, first, pool, lo.pool_cap, allot,
                                                      row_ptr, col, val);
   return clt_check_launch();
@@ -1571,7 +1575,8 @@ static ThreshLayout thresh_layout(int64_t T, int64_t F, int64_t L, int64_t densi
   ThreshLayout tl;
   const int segw = dtype != CLT_F32 ? 128 : 64;
   tl.nseg = (int)(F / segw);
-  tl.ntile = tl.nseg * (int)(T / COLLECT_ROWS);
+  const int64_t Tp = collect_grid_rows(T);   // the epilogue's books cover whole token tiles
+  tl.ntile = tl.nseg * (int)(Tp / COLLECT_ROWS);
   const double dens = (double)(density_ppm < 1 ? 1 : density_ppm) * 1e-6;
   // a fixed slot holds three times the expected entries of a tile (at least 64, at most the tile)
   unsigned long long caps = (unsigned long long)(3.0 * dens * (double)COLLECT_ROWS * segw) + 64ull;
@@ -1586,9 +1591,9 @@ static ThreshLayout thresh_layout(int64_t T, int64_t F, int64_t L, int64_t densi
   tl.off_state = take(sizeof(SelState) * (size_t)L);
   tl.off_tcount = take(4 * (size_t)L);
   tl.off_tmeta = take(8 * (size_t)tl.ntile * (size_t)L);
-  tl.off_meta = take(8 * (size_t)tl.nseg * (size_t)T * (size_t)L);
+  tl.off_meta = take(8 * (size_t)tl.nseg * (size_t)Tp * (size_t)L);
   tl.off_tpool = take(8 * (size_t)tl.tpool_cap * (size_t)L);
-  tl.off_pfx = take(4 * (size_t)tl.nseg * (size_t)T * (size_t)L);
+  tl.off_pfx = take(4 * (size_t)tl.nseg * (size_t)Tp * (size_t)L);
   tl.off_rowcnt = take(4 * (size_t)T * (size_t)L);
   tl.total = o;
   return tl;
@@ -1641,7 +1646,7 @@ extern "C" int clt_encode_threshold_count(const void *x, const void *w, const vo
                              nullptr, &ca, s);
   if (rc != CLT_OK) return rc;
   uint32_t *rowcnt = (uint32_t *)(ws + tl.off_rowcnt);
-  k_row_prefix_meta<<<dim3((unsigned)clt_ceil_div(T, 64), (unsigned)L), 64, 0, s>>>(T, tl.nseg, ca.seg_meta,
+  k_row_prefix_meta<<<dim3((unsigned)clt_ceil_div(T, 64), (unsigned)L), 64, 0, s>>>(T, collect_grid_rows(T), tl.nseg, ca.seg_meta,
                                                                                     (uint32_t *)(ws + tl.off_pfx), rowcnt);
   k_rowptr_scan<<<1, SCAN_THREADS, 0, s>>>(rowcnt, L * T, row_ptr);
   k_thresh_finish<<<1, 64, 0, s>>>(st, (int)L, row_ptr, L * T);
@@ -1717,13 +1722,13 @@ extern "C" int clt_encode_threshold_emit(int64_t T, int64_t F, int64_t L, int64_
   char *ws = (char *)workspace;
   dim3 grid((unsigned)clt_ceil_div(T, 256), (unsigned)tl.nseg, (unsigned)L);
   if (dtype == CLT_BF16)
-    k_tile_emit_all<bf16_t><<<grid, 256, 0, s>>>((int)T, (const uint2 *)(ws + tl.off_meta), tl.nseg, (const uint2 *)(ws + tl.off_tpool),
+    k_tile_emit_all<bf16_t><<<grid, 256, 0, s>>>((int)T, (int)collect_grid_rows(T), (const uint2 *)(ws + tl.off_meta), tl.nseg, (const uint2 *)(ws + tl.off_tpool),
                                                   tl.tpool_cap, (const uint32_t *)(ws + tl.off_pfx), row_ptr, col, (bf16_t *)val, skip);
   else if (dtype == CLT_F16)
-    k_tile_emit_all<f16_t><<<grid, 256, 0, s>>>((int)T, (const uint2 *)(ws + tl.off_meta), tl.nseg, (const uint2 *)(ws + tl.off_tpool),
+    k_tile_emit_all<f16_t><<<grid, 256, 0, s>>>((int)T, (int)collect_grid_rows(T), (const uint2 *)(ws + tl.off_meta), tl.nseg, (const uint2 *)(ws + tl.off_tpool),
                                                   tl.tpool_cap, (const uint32_t *)(ws + tl.off_pfx), row_ptr, col, (f16_t *)val, skip);
   else
-    k_tile_emit_all<float><<<grid, 256, 0, s>>>((int)T, (const uint2 *)(ws + tl.off_meta), tl.nseg, (const uint2 *)(ws + tl.off_tpool),
+    k_tile_emit_all<float><<<grid, 256, 0, s>>>((int)T, (int)collect_grid_rows(T), (const uint2 *)(ws + tl.off_meta), tl.nseg, (const uint2 *)(ws + tl.off_tpool),
                                                  tl.tpool_cap, (const uint32_t *)(ws + tl.off_pfx), row_ptr, col, (float *)val, skip);
   return clt_check_launch();
 }

@@ -27,22 +27,36 @@ struct SelState {
 
 // tokens of one wave tile of the collecting encoder epilogue
 constexpr int COLLECT_ROWS = 64;
+// tokens of one workgroup tile of the encoder kernel
+constexpr int COLLECT_TILE_ROWS = 256;
+
+// The collecting epilogue keeps its books on a grid of whole workgroup tiles: Tp = T rounded up to a multiple
+// of COLLECT_TILE_ROWS token rows.  When T is not such a multiple the last token tile is shifted back inside
+// the matrix (it covers the tokens [T - 256, T)), reports only the tokens its neighbour does not own, and
+// files them where it computed them: token t of the last tile sits at row t + (Tp - T) of the grid, the
+// Tp - T rows in front of them are empty.
+__host__ __device__ inline int64_t collect_grid_rows(int64_t T) {
+  return (T + COLLECT_TILE_ROWS - 1) / COLLECT_TILE_ROWS * COLLECT_TILE_ROWS;
+}
+__device__ __forceinline__ int64_t collect_grid_row(int64_t token, int64_t T, int64_t Tp) {
+  return token + (token >= Tp - COLLECT_TILE_ROWS ? Tp - T : 0);
+}
 
 // What the collecting encoder epilogue writes.  A wavefront's 64-token tile of one feature
 // segment (128 features for 16-bit elements, 64 for 32-bit) becomes ONE extent of the layer's
-// pool, ordered by (token, feature).  Tile number i = segment * (T / 64) + token block owns
+// pool, ordered by (token, feature).  Tile number i = segment * (Tp / 64) + token block owns
 // the fixed slot [i * caps, (i + 1) * caps) of the pool; only a tile with more than `caps`
 // candidates takes an extent behind the slots instead, handed out by an atomic counter (one
 // same-address atomic per tile from every CU at once would cost more than the whole epilogue).
 //   tile_meta[layer * ntile + i]                           = (offset of the extent, entries)
-//   seg_meta[(layer * nseg + segment) * T + token]         = (offset of the token's run, length)
+//   seg_meta[(layer * nseg + segment) * Tp + grid row]     = (offset of the token's run, length)
 struct CollectArgs {
   SelState *st;              // [L]
   uint32_t *pool_count;      // [L] entries handed out behind the fixed slots
   uint2 *pool;               // [L][pool_cap] entries (feature, raw value bits)
   unsigned long long pool_cap;
   uint2 *tile_meta;          // [L][ntile]
-  uint2 *seg_meta;           // [L][nseg][T]
+  uint2 *seg_meta;           // [L][nseg][Tp]
   uint32_t caps;             // entries per fixed slot
   const void *theta;         // COLLECT == 2: [L][F] thresholds in the model dtype
   int64_t theta_stride;

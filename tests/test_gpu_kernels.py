@@ -221,7 +221,9 @@ def assert_same_list(got, ref, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("L,T,d,F", [(1, 256, 128, 256), (2, 512, 256, 1024), (3, 256, 768, 512)])
+@pytest.mark.parametrize("L,T,d,F", [(1, 256, 128, 256), (2, 512, 256, 1024), (3, 256, 768, 512),
+                                     # token counts that are not whole tiles: the last tile is shifted back
+                                     (2, 257, 128, 256), (3, 300, 256, 512), (1, 511, 128, 1024), (2, 1000, 128, 256)])
 def test_encode_threshold_matches_separate_and_oracle(dev, dtype, L, T, d, F):
     g = torch.Generator().manual_seed(L * 17 + T + F)
     x = torch.randn(L, T, d, generator=g).to(dtype)
@@ -268,6 +270,27 @@ def test_encode_threshold_pool_too_small_reports_it(dev):
     assert_same_list(got, ref, torch.bfloat16)
 
 
+@pytest.mark.parametrize("T", [300, 700])
+def test_encode_threshold_ragged_batch_overflow_is_redone_densely(dev, T):
+    # the device-side fallback (pool overflow -> dense route) on a token count that is not a whole number of tiles
+    g = torch.Generator().manual_seed(T)
+    L, d, F = 2, 128, 512
+    x = torch.randn(L, T, d, generator=g).to(torch.bfloat16).to(dev)
+    w = (torch.randn(L, F, d, generator=g) / math.sqrt(d)).to(torch.bfloat16).to(dev)
+    theta = torch.full((L, F), 1e-3).to(torch.bfloat16).to(dev)
+    pre = engine.encode(x, w, None)
+    ref = engine.threshold_select(pre, theta, nat.PRED_GE_THETA)
+    for ppm in (1, 600000):        # 1: overflows and is redone from the dense scratch; 600000: fits
+        scratch = torch.full_like(pre, float("nan"))
+        got = engine.encode_threshold(x, w, None, theta, engine.Workspace(dev), ppm, pre_scratch=scratch)
+        torch.cuda.synchronize()
+        n = int(got.row_ptr[-1])
+        assert n == ref.nnz
+        assert torch.equal(got.row_ptr.cpu(), ref.row_ptr.cpu())
+        assert torch.equal(got.col[:n].cpu(), ref.col.cpu())
+        assert torch.equal(got.val[:n].cpu().view(torch.int16), ref.val.cpu().view(torch.int16))
+
+
 # ---- BatchTopK global ------------------------------------------------------------------------
 # ---- encoder with the collecting epilogue + BatchTopK on the candidates --------------------
 def fused_vs_separate(x, w, b, k, dev):
@@ -289,7 +312,10 @@ def fused_vs_separate(x, w, b, k, dev):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("L,T,d,F,k", [(1, 256, 128, 256, 3), (2, 512, 256, 1024, 20), (3, 256, 768, 512, 64),
-                                       (2, 768, 128, 2048, 200)])
+                                       (2, 768, 128, 2048, 200),
+                                       # token counts that are not whole tiles: the last tile is shifted back
+                                       (2, 257, 128, 256, 5), (3, 300, 256, 512, 20), (1, 511, 128, 1024, 64),
+                                       (2, 1000, 128, 256, 7), (1, 833, 256, 2048, 300)])
 def test_encode_collect_matches_separate_and_oracle(dev, dtype, L, T, d, F, k):
     g = torch.Generator().manual_seed(L * 31 + T + F + k)
     x = torch.randn(L, T, d, generator=g).to(dtype)
@@ -302,11 +328,12 @@ def test_encode_collect_matches_separate_and_oracle(dev, dtype, L, T, d, F, k):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_encode_collect_heavy_ties(dev, dtype):
+@pytest.mark.parametrize("T", [512, 333])
+def test_encode_collect_heavy_ties(dev, dtype, T):
     # small-integer inputs and weights: the pre-activations are exact small integers, so
     # thousands of them tie at the threshold and the lowest flat indices must win
     g = torch.Generator().manual_seed(5)
-    L, T, d, F, k = 2, 512, 128, 1024, 30
+    L, d, F, k = 2, 128, 1024, 30
     x = torch.randint(-1, 2, (L, T, d), generator=g).to(dtype)
     w = torch.randint(-1, 2, (L, F, d), generator=g).to(dtype)
     pre, got = fused_vs_separate(x, w, None, k, dev)
@@ -314,14 +341,15 @@ def test_encode_collect_heavy_ties(dev, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_encode_collect_unusable_cut_takes_streaming_route(dev, dtype):
+@pytest.mark.parametrize("T", [512, 450])
+def test_encode_collect_unusable_cut_takes_streaming_route(dev, dtype, T):
     # almost every pre-activation is exactly 0 and K reaches into the zeros: every element
     # reaches the sampled cut, the candidate pool overflows, and the layer must be redone from
     # the dense pre-activations (written to the scratch buffer for that purpose)
     g = torch.Generator().manual_seed(9)
-    L, T, d, F, k = 2, 512, 128, 2048, 8
+    L, d, F, k = 2, 128, 2048, 8
     x = torch.zeros(L, T, d)
-    x[:, ::64] = torch.randn(L, T // 64, d, generator=g)
+    x[:, ::64] = torch.randn(L, (T + 63) // 64, d, generator=g)
     w = (torch.randn(L, F, d, generator=g) / math.sqrt(d))
     pre, got = fused_vs_separate(x.to(dtype), w.to(dtype), None, k, dev)
     assert got.nnz == L * k * T
@@ -336,7 +364,7 @@ def test_encode_collect_all_selected_and_shape_gate(dev):
     pre, got = fused_vs_separate(x, w, None, F + 5, dev)          # k >= F: everything survives
     assert got.nnz == T * F
     # shapes the collecting epilogue does not take
-    assert not engine.encode_collect_supported(x[:, :200].contiguous().to(dev), w.to(dev), None, 4)
+    assert not engine.encode_collect_supported(x[:, :200].contiguous().to(dev), w.to(dev), None, 4)   # less than a tile
     assert not engine.encode_collect_supported(x.to(dev), w[:, :136].contiguous().to(dev), None, 4)
     assert not engine.encode_collect_supported(x.to(dev), w.to(dev), None, 0)
 

@@ -171,15 +171,19 @@ def test_float16_model_forward_matches_oracle(dev, wl):
         model.loss_and_gradients(inputs, inputs)
 
 
+@pytest.mark.parametrize("tokens", [512, 600])
 @pytest.mark.parametrize("fn", ["batchtopk", "jumprelu"])
-def test_fused_routes_equal_separate_kernels_in_the_model(dev, fn):
-    # same model, same inputs: with and without the encoder-epilogue routes, all layers and a subset
-    wl = BASE.scaled("f", num_layers=3, d_model=256, num_features=1024, tokens=512, k=24 if fn == "batchtopk" else None,
+def test_fused_routes_equal_separate_kernels_in_the_model(dev, fn, tokens):
+    # same model, same inputs: with and without the encoder-epilogue routes, all layers and a subset; a whole
+    # number of encoder token tiles, and a batch whose last tile is partial
+    wl = BASE.scaled("f", num_layers=3, d_model=256, num_features=1024, tokens=tokens, k=24 if fn == "batchtopk" else None,
                      activation_fn=fn, dtype="bfloat16")
     model, sd, x = build(wl, dev)
     for layers in ([0, 1, 2], [0, 2]):
         inputs = {l: x[l].to(dev) for l in layers}
         model.fuse_encode_select = True
+        if fn == "batchtopk":
+            assert engine.encode_collect_supported(*model.encoder_module.prepare_slab(inputs)[1:], int(wl.k))
         a1 = model.get_feature_activations(inputs)
         r1 = model(inputs)
         model.fuse_encode_select = False
