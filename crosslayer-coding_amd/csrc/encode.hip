@@ -129,7 +129,7 @@ __device__ __forceinline__ uint32_t wave_inclusive_scan32(uint32_t v) {
   return v;
 }
 
-// Requires K % (256 / sizeof(T)) == 0 (an even number of LDS stages), M >= BM and N >= BN.  A tile that
+// Requires K % (128 / sizeof(T)) == 0 (whole LDS stages), M >= BM and N >= BN.  A tile that
 // would stick out of the matrix is shifted back inside (its overlap with the neighbour is
 // computed twice and stored by the neighbour only), so no load is predicated.
 //
@@ -152,12 +152,13 @@ struct SegArgs {
   int xrs, wrs;      // row strides, elements
 };
 
-template <typename T, int COLLECT, bool SEG>
+template <typename T, int COLLECT, bool SEG, bool ODD>
 __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void k_encode_mfma(
     const T *__restrict__ x, const T *__restrict__ w, const T *__restrict__ bias, T *__restrict__ pre,
     int M, int K, int N, int tiles_m, int tiles_n, int total_tiles, int64_t xs, int64_t wstr, int64_t bs,
     int64_t ps, const SelState *__restrict__ gate, CollectArgs ca, SegArgs sg, int by_tokens) {
   static_assert(!SEG || COLLECT == 0, "segmented operands only in the storing mode");
+  static_assert(!SEG || !ODD, "segmented operands come in an even number of stages");
   constexpr int CE = 16 / (int)sizeof(T);  // elements per 16-byte chunk
   constexpr int BK = ROWB / (int)sizeof(T);
   // Persistent workgroups (the grid is one block per CU, block b takes the tiles b, b + gridDim.x, ...)
@@ -177,7 +178,12 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave & 3, wn = wave >> 2;   // wave tile: tokens [64 wm, +64) x features [128 wn, +128)
   const int per_layer = tiles_m * tiles_n;
-  const int nk = K / BK;
+  // The K loop walks its stages in pairs.  An odd number of stages (ODD, a separate instantiation so that the
+  // even case pays nothing for it) gets a repeat of the last one appended, which is loaded like any other (every
+  // count the pipeline's waits rely on stays the same) and multiplied by nothing.
+  const int nk_real = K / BK;
+  constexpr bool odd = ODD;
+  const int nk = nk_real + (odd ? 1 : 0);
 
   struct TileAt { int layer, tm, tn, m0, n0, om0, on0, rot; };
   auto locate = [&](int bid) {
@@ -214,7 +220,8 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
     // K is walked from a tile-dependent starting stage, wrapping around: the CUs of an XCD that share an
     // x tile or a W tile then ask for different lines of it at any one time, so one of them takes the
     // L2 miss and the others find the line there later, instead of all of them queueing behind the miss.
-    t.rot = (by_tokens ? 3 * t.tn + (t.tm >> 3) : (tiles_n & 7) == 0 ? 3 * t.tm + (t.tn >> 3) : t.tm + t.tn) % nk;
+    // (no rotation with an appended stage: that one must come last)
+    t.rot = odd ? 0 : (by_tokens ? 3 * t.tn + (t.tm >> 3) : (tiles_n & 7) == 0 ? 3 * t.tm + (t.tn >> 3) : t.tm + t.tn) % nk;
     return t;
   };
   // the storing mode computes only the layers that asked for it when a gate is given; the states of up to
@@ -245,7 +252,12 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
   auto x_rows = [&](const TileAt &t) { return x + (int64_t)t.layer * xs + (int64_t)(t.m0 + wave * 32) * xrs; };
   auto w_rows = [&](const TileAt &t) { return w + (int64_t)t.layer * wstr + (int64_t)(t.n0 + wave * 32) * wrs; };
   // the stage walked kt-th by a tile (an index into K / BK)
-  auto stage_k0 = [&](const TileAt &t, int kt) { int q = kt + t.rot; if (q >= nk) q -= nk; return q; };
+  auto stage_k0 = [&](const TileAt &t, int kt) {
+    int q = kt + t.rot;
+    if (q >= nk) q -= nk;
+    if constexpr (ODD) return q < nk_real ? q : nk_real - 1;
+    return q;
+  };
   auto issue_stage = [&](unsigned char *stage, const T *xt, const T *wt, int kst) {
     unsigned char *xs_l = stage + wave * 32 * ROWB;
     unsigned char *ws_l = xs_l + BM * ROWB;
@@ -361,14 +373,21 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
   // one stage except its last k-step, the barrier, then the last k-step overlapped with the loads that
   // `refill` asks for (the stage after next, into `cur`) and, unless this is the tile's last stage,
   // the first fragments of `nxt`
-  auto body = [&](unsigned char *cur, unsigned char *nxt, bool last, auto refill) {
-    load_frags(fb, cur, 1); mma8(fa); mix_ds();
-    load_frags(fa, cur, 2); mma8(fb); mix_ds();
-    load_frags(fb, cur, 3); mma8(fa); mix_ds();
+  // `cm` / `nm`: AND masks for the fragments read from `cur` / `nxt` (all ones, or zero for the appended stage,
+  // whose products must add nothing: both operands are cleared, so that an infinity in the repeated data cannot
+  // turn into a NaN)
+  auto mask_frags = [&](uint4 (&f)[6], uint32_t m) {
+#pragma unroll
+    for (int i = 0; i < 6; ++i) { f[i].x &= m; f[i].y &= m; f[i].z &= m; f[i].w &= m; }
+  };
+  auto body = [&](unsigned char *cur, unsigned char *nxt, bool last, auto refill, uint32_t cm, uint32_t nm) {
+    load_frags(fb, cur, 1); mask_frags(fb, cm); mma8(fa); mix_ds();
+    load_frags(fa, cur, 2); mask_frags(fa, cm); mma8(fb); mix_ds();
+    load_frags(fb, cur, 3); mask_frags(fb, cm); mma8(fa); mix_ds();
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
     refill();
-    if (!last) load_frags(fa, nxt, 0);
+    if (!last) { load_frags(fa, nxt, 0); mask_frags(fa, nm); }
     mma8(fb);
 #pragma unroll
     for (int g = 0; g < 8; ++g) {
@@ -413,17 +432,18 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
       asm volatile("global_load_dword %0, %1, off" : "=v"(cut_key_v) : "v"(cut_at));
     }
     load_frags(fa, stage0, 0);
-    // nk is even (checked by the launcher)
+    // nk is even
     for (int kt = 0; kt < nk - 2; kt += 2) {
-      body(stage0, stage1, false, [&]() { issue_stage(stage0, xt, wt, stage_k0(cur, kt + 2)); });
-      body(stage1, stage0, false, [&]() { issue_stage(stage1, xt, wt, stage_k0(cur, kt + 3)); });
+      body(stage0, stage1, false, [&]() { issue_stage(stage0, xt, wt, stage_k0(cur, kt + 2)); }, ~0u, ~0u);
+      body(stage1, stage0, false, [&]() { issue_stage(stage1, xt, wt, stage_k0(cur, kt + 3)); }, ~0u, ~0u);
     }
     // the last two stages: the first buffer is free after the first of them and takes the next tile's
     // first stage; nothing may be in flight into the second one, which is parked in
+    constexpr uint32_t last_mask = odd ? 0u : ~0u;
     body(stage0, stage1, false, [&]() {
       if (has_next) issue_stage(stage0, x_rows(nxt_tile), w_rows(nxt_tile), stage_k0(nxt_tile, 0));
-    });
-    body(stage1, stage0, true, [&]() {});
+    }, ~0u, last_mask);
+    body(stage1, stage0, true, [&]() {}, last_mask, ~0u);
     // past the barrier of the last stage no wavefront reads either buffer any more
 
     // ---- epilogue.  The accumulator layout gives a lane 4 consecutive features of one token,
@@ -739,7 +759,7 @@ template <typename T>
 static bool encode_fast_ok(const void *x, const void *w, const void *b, const void *pre, int64_t T_, int64_t d,
                            int64_t F, int64_t xs, int64_t wstr, int64_t bs, int64_t ps) {
   constexpr int CE = 16 / (int)sizeof(T);
-  return (d % (2 * ROWB / (int)sizeof(T)) == 0) && (F % 4 == 0) && T_ >= BM && F >= BN && clt_aligned16(x) &&
+  return (d % (ROWB / (int)sizeof(T)) == 0) && (F % 4 == 0) && T_ >= BM && F >= BN && clt_aligned16(x) &&
          clt_aligned16(w) && clt_aligned16(pre) && (xs % CE == 0) && (wstr % CE == 0) && (ps % 4 == 0) &&
          (ps * (int64_t)sizeof(T)) % 16 == 0 && (F * (int64_t)sizeof(T)) % 8 == 0 && T_ < (1 << 30) &&
          F < (1 << 30) && d < (1 << 30) && (!b || (((uintptr_t)b) % 16 == 0 && bs % 8 == 0));
@@ -774,14 +794,21 @@ static int launch_encode(const void *x, const void *w, const void *b, void *pre,
     // which operand an XCD keeps to itself: the feature tiles (W, the larger one in the encoder), or the token
     // tiles when there are more of those and they split evenly over the XCDs
     const int by_tokens = (tm % 8 == 0 && tm > tn) ? 1 : 0;
-#define CLT_ENC(C)                                                                                                  \
-  k_encode_mfma<T, C, false><<<(unsigned)grid, NTHREADS, 0, stream>>>((const T *)x, (const T *)w, (const T *)b,     \
+#define CLT_ENC(C, O)                                                                                               \
+  k_encode_mfma<T, C, false, O><<<(unsigned)grid, NTHREADS, 0, stream>>>((const T *)x, (const T *)w, (const T *)b,  \
                                                                      (T *)pre, (int)T_, (int)d, (int)F, (int)tm,  \
                                                                      (int)tn, (int)nblk, xs, wstr, bs, ps, gate,  \
                                                                      a, noseg, by_tokens)
-    if (collect == 0) CLT_ENC(0);
-    else if (collect == 1) CLT_ENC(1);
-    else CLT_ENC(2);
+    const bool odd_stages = ((d / (ROWB / (int64_t)sizeof(T))) & 1) != 0;
+    if (odd_stages) {
+      if (collect == 0) CLT_ENC(0, true);
+      else if (collect == 1) CLT_ENC(1, true);
+      else CLT_ENC(2, true);
+    } else {
+      if (collect == 0) CLT_ENC(0, false);
+      else if (collect == 1) CLT_ENC(1, false);
+      else CLT_ENC(2, false);
+    }
 #undef CLT_ENC
   } else {
     // the gate is ignored here: recomputing a layer that did not ask for it is harmless
@@ -812,7 +839,7 @@ static int launch_encode_segmented(const void *x, const void *w, void *pre, int6
   const CollectArgs none = {};
   const int64_t grid = persistent_grid(nblk);
   if (grid <= 0) return CLT_ERR_LAUNCH;
-  k_encode_mfma<T, 0, true><<<(unsigned)grid, NTHREADS, 0, stream>>>((const T *)x, (const T *)w, nullptr, (T *)pre, (int)T_,
+  k_encode_mfma<T, 0, true, false><<<(unsigned)grid, NTHREADS, 0, stream>>>((const T *)x, (const T *)w, nullptr, (T *)pre, (int)T_,
                                                                     (int)K, (int)F, (int)tm, (int)tn, (int)nblk, 0, 0, 0,
                                                                     0, nullptr, none, sg, (tm % 8 == 0 && tm > tn) ? 1 : 0);
   return clt_check_launch();

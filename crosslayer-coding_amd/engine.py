@@ -140,7 +140,7 @@ def encode(x: torch.Tensor, w: torch.Tensor, b: Optional[torch.Tensor],
     if b is not None:
         assert b.shape == (L, F) and b.stride(1) == 1 and b.dtype == x.dtype
     lib = nat.load()
-    stage = 256 // x.element_size()          # elements of K in two 128-byte stages of the matrix-core kernel
+    stage = 128 // x.element_size()          # elements of K in one 128-byte stage of the matrix-core kernel
     if 0 < T < ENCODE_MIN_TOKENS and F >= 256 and F % 4 == 0 and d % stage == 0:
         # The matrix-core kernel works on whole 256-token tiles; a shorter batch (a short prompt) would fall to
         # the one-thread-per-output kernel, which is 30x slower than the padded product.  Rows past T are zeros

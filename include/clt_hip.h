@@ -178,7 +178,7 @@ int clt_batchtopk_select(const void *pre, int64_t T, int64_t F, int64_t L,
  * (fewer than k*T candidates, or no pool space left), which then takes the streaming route.
  * clt_encode_collect_supported returns 1 when the shapes qualify (T >= 256, any remainder:
  * the last token tile is shifted back inside the matrix and reports only the tokens its
- * neighbour does not own; F % 256 == 0, d % 128 == 0 for 16-bit elements / d % 64 == 0 for
+ * neighbour does not own; F % 256 == 0, d % 64 == 0 for 16-bit elements / d % 32 == 0 for
  * fp32, 16-byte aligned rows, k > 0), else 0; callers then use clt_encode +
  * clt_batchtopk_select.
  * Replaces the same reference calls as clt_encode and clt_batchtopk_select

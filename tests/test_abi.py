@@ -53,3 +53,36 @@ def test_no_cpu_fallback():
         cca.engine.encode(torch.zeros(1, 2, 8), torch.zeros(1, 4, 8), None)
     with pytest.raises(nat.CLTNativeError):
         cca.BatchTopK._compute_mask(torch.randn(2, 4), 2)
+
+
+def test_encoder_kernels_spill_nothing(tmp_path):
+    """Every instantiation of the matrix-core encoder kernel must fit the register file.  A spill would cost the
+    K loop, and worse: the collecting epilogue fetches the layer's cut with a hand-written load that the
+    compiler does not know to be outstanding, so a spill of its destination register right behind the load would
+    store the register before the value has arrived.  Checked on the assembly the compiler reports for gfx950."""
+    import shutil
+    import subprocess
+
+    import pytest
+    from crosslayer_coding_amd import build as clt_build
+
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(hipcc):
+        pytest.skip("hipcc not found")
+    out = tmp_path / "encode.s"
+    flags = [f for f in clt_build.HIP_FLAGS if f != "-fPIC"]
+    proc = subprocess.run([hipcc, *flags, "--cuda-device-only", "-S", "-o", str(out),
+                           os.path.join(clt_build.CSRC, "encode.hip")], stdout=subprocess.PIPE, stderr=subprocess.STDOUT,
+                          text=True)
+    assert proc.returncode == 0, proc.stdout[-2000:]
+    current, scratch = None, {}
+    for line in open(out):
+        m = re.match(r"^(_Z\w+):", line)
+        if m:
+            current = m.group(1)
+        m = re.match(r"^; ScratchSize: (\d+)", line)
+        if m and current:
+            scratch[current] = int(m.group(1))
+    kernels = {k: v for k, v in scratch.items() if "k_encode_mfma" in k}
+    assert len(kernels) >= 18, sorted(kernels)      # 3 element types x 3 epilogues x even / odd stage counts, + segmented
+    assert all(v == 0 for v in kernels.values()), {k: v for k, v in kernels.items() if v}

@@ -38,7 +38,10 @@ def check_rows_sorted(surv):
 # ---- encoder --------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("L,T,d,F", [(1, 30, 8, 16), (2, 300, 64, 136), (3, 257, 96, 260), (1, 5, 7, 9), (2, 512, 768, 512),
-                                     (2, 40, 256, 512), (1, 1, 128, 256), (3, 255, 128, 260)])   # short batches: padded to a tile
+                                     (2, 40, 256, 512), (1, 1, 128, 256), (3, 255, 128, 260),     # short batches: padded to a tile
+                                     # an odd number of 128-byte stages along d (1, 3, 5 for 16-bit elements)
+                                     (1, 256, 64, 256), (2, 512, 192, 512), (2, 300, 320, 520), (1, 256, 32, 256),
+                                     (1, 700, 1600, 768)])
 def test_encode_parity(dev, dtype, L, T, d, F):
     g = torch.Generator().manual_seed(L * 1000 + T)
     x = torch.randn(L, T, d, generator=g).to(dtype)
@@ -223,7 +226,9 @@ def assert_same_list(got, ref, dtype):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("L,T,d,F", [(1, 256, 128, 256), (2, 512, 256, 1024), (3, 256, 768, 512),
                                      # token counts that are not whole tiles: the last tile is shifted back
-                                     (2, 257, 128, 256), (3, 300, 256, 512), (1, 511, 128, 1024), (2, 1000, 128, 256)])
+                                     (2, 257, 128, 256), (3, 300, 256, 512), (1, 511, 128, 1024), (2, 1000, 128, 256),
+                                     # an odd number of stages along d
+                                     (2, 512, 320, 512), (1, 300, 64, 256)])
 def test_encode_threshold_matches_separate_and_oracle(dev, dtype, L, T, d, F):
     g = torch.Generator().manual_seed(L * 17 + T + F)
     x = torch.randn(L, T, d, generator=g).to(dtype)
@@ -315,7 +320,9 @@ def fused_vs_separate(x, w, b, k, dev):
                                        (2, 768, 128, 2048, 200),
                                        # token counts that are not whole tiles: the last tile is shifted back
                                        (2, 257, 128, 256, 5), (3, 300, 256, 512, 20), (1, 511, 128, 1024, 64),
-                                       (2, 1000, 128, 256, 7), (1, 833, 256, 2048, 300)])
+                                       (2, 1000, 128, 256, 7), (1, 833, 256, 2048, 300),
+                                       # an odd number of stages along d
+                                       (2, 512, 192, 512, 20), (1, 300, 64, 256, 5), (1, 512, 1600, 512, 16)])
 def test_encode_collect_matches_separate_and_oracle(dev, dtype, L, T, d, F, k):
     g = torch.Generator().manual_seed(L * 31 + T + F + k)
     x = torch.randn(L, T, d, generator=g).to(dtype)

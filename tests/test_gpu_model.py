@@ -175,8 +175,8 @@ def test_float16_model_forward_matches_oracle(dev, wl):
 @pytest.mark.parametrize("fn", ["batchtopk", "jumprelu"])
 def test_fused_routes_equal_separate_kernels_in_the_model(dev, fn, tokens):
     # same model, same inputs: with and without the encoder-epilogue routes, all layers and a subset; a whole
-    # number of encoder token tiles, and a batch whose last tile is partial
-    wl = BASE.scaled("f", num_layers=3, d_model=256, num_features=1024, tokens=tokens, k=24 if fn == "batchtopk" else None,
+    # number of encoder token tiles, and a batch whose last tile is partial (with a d_model of five 128-byte stages)
+    wl = BASE.scaled("f", num_layers=3, d_model=256 if tokens == 512 else 320, num_features=1024, tokens=tokens, k=24 if fn == "batchtopk" else None,
                      activation_fn=fn, dtype="bfloat16")
     model, sd, x = build(wl, dev)
     for layers in ([0, 1, 2], [0, 2]):
