@@ -173,6 +173,7 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
   __shared__ uint16_t cand_list[COLLECT ? NWAVES : 1][COLLECT ? CAND_LIST : 1];   // per wavefront, see the emission
   __shared__ __attribute__((aligned(16))) T bias_lds[NWAVES][128];                // per wavefront: the bias of its features
   __shared__ __attribute__((aligned(16))) T theta_lds[COLLECT == 2 ? NWAVES : 1][COLLECT == 2 ? 128 : 8];   // and their thresholds
+  __shared__ __attribute__((aligned(16))) uint32_t cut_lds[COLLECT == 1 ? NWAVES : 1][4];                   // the layer's cut key
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -297,6 +298,11 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
     if constexpr (COLLECT == 2) {
       if (lane < BIAS_LANES)
         load16_to_lds((const T *)ca.theta + (int64_t)t.layer * ca.theta_stride + t.n0 + wn * 128 + lane * CE, theta_lds[wave]);
+    }
+    // the layer's cut travels the same way: four bytes into the wavefront's slot, read in the epilogue
+    if constexpr (COLLECT == 1) {
+      if (lane == 0)
+        __builtin_amdgcn_global_load_lds(&ca.st[t.layer].cut_key, (__attribute__((address_space(3))) void *)cut_lds[wave], 4, 0, 0);
     }
   };
   if (!bias && lane < BIAS_LANES)   // no bias: the slot holds zeros for good
@@ -423,14 +429,6 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
     asm volatile("" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);    // nothing that reads the bias may move above the wait
     init_acc();
-    // The layer's cut is asked for here and used in the epilogue.  A hand-written load: the compiler does not
-    // know that it is outstanding and waits for nothing; it is older than the loads of the first refill below,
-    // so the wait of the stage after that one guarantees that it has arrived.
-    uint32_t cut_key_v = 0;
-    if constexpr (COLLECT == 1) {
-      const uint32_t *cut_at = &ca.st[layer].cut_key;
-      asm volatile("global_load_dword %0, %1, off" : "=v"(cut_key_v) : "v"(cut_at));
-    }
     load_frags(fa, stage0, 0);
     // nk is even
     for (int kt = 0; kt < nk - 2; kt += 2) {
@@ -522,7 +520,12 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
         const int ncol0 = n0 + wn * 128 + pass * SEGW;       // first feature of the segment
         uint32_t cut_bits = 0;
         if constexpr (COLLECT == 1) {
-          asm volatile("" : "+v"(cut_key_v));      // nothing that reads the cut may move above this point
+          // The cut came in with the bias, ahead of the tile's stages, and has long landed.  Read by hand, with
+          // its own wait inside the statement: the compiler, which cannot tell the direct-to-LDS loads in flight
+          // (the next tile's first stage) from the one into this slot, would wait for all of them first.
+          uint32_t cut_key_v;
+          const uint32_t cut_at = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint32_t *)cut_lds[wave];
+          asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(cut_key_v) : "v"(cut_at) : "memory");
           cut_bits = key_value_bits<T>((uint32_t)__builtin_amdgcn_readfirstlane((int)cut_key_v));
         }
         const bool cut_nan = (cut_bits & 0x7FFFFFFFu) > 0x7F800000u;   // only NaNs reach such a cut

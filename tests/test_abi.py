@@ -56,10 +56,10 @@ def test_no_cpu_fallback():
 
 
 def test_encoder_kernels_spill_nothing(tmp_path):
-    """Every instantiation of the matrix-core encoder kernel must fit the register file.  A spill would cost the
-    K loop, and worse: the collecting epilogue fetches the layer's cut with a hand-written load that the
-    compiler does not know to be outstanding, so a spill of its destination register right behind the load would
-    store the register before the value has arrived.  Checked on the assembly the compiler reports for gfx950."""
+    """Every instantiation of the matrix-core encoder kernel must fit the register file: the kernel runs two
+    wavefronts per SIMD on 256 registers each, with 128 of them accumulators that live across the K loop, so a
+    change that tips it into spilling costs the loop dearly while every result stays right.  Checked on the
+    assembly the compiler reports for gfx950."""
     import shutil
     import subprocess
 
