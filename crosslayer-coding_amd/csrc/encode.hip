@@ -315,16 +315,51 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
   auto init_acc = [&]() {
     typedef typename std::conditional<sizeof(T) == 4, uint4, uint2>::type braw_t;
     braw_t raw[16];
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int rg = 0; rg < 4; ++rg) {
-        if constexpr (sizeof(T) == 4)
-          asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(raw[j * 4 + rg]) : "v"(bias_at), "n"((j * 32 + rg * 8) * 4));
-        else
-          asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(raw[j * 4 + rg]) : "v"(bias_at), "n"((j * 32 + rg * 8) * 2));
-      }
-    __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0)
+    // raw[4 j + rg] = the 4 values at feature j * 32 + rg * 8 of this lane's half.  All sixteen reads and their
+    // wait are one statement, so no register is looked at before its value has arrived.
+    if constexpr (sizeof(T) == 4) {
+        asm volatile(
+                     "ds_read_b128 %0, %16\n\t"
+                     "ds_read_b128 %1, %16 offset:32\n\t"
+                     "ds_read_b128 %2, %16 offset:64\n\t"
+                     "ds_read_b128 %3, %16 offset:96\n\t"
+                     "ds_read_b128 %4, %16 offset:128\n\t"
+                     "ds_read_b128 %5, %16 offset:160\n\t"
+                     "ds_read_b128 %6, %16 offset:192\n\t"
+                     "ds_read_b128 %7, %16 offset:224\n\t"
+                     "ds_read_b128 %8, %16 offset:256\n\t"
+                     "ds_read_b128 %9, %16 offset:288\n\t"
+                     "ds_read_b128 %10, %16 offset:320\n\t"
+                     "ds_read_b128 %11, %16 offset:352\n\t"
+                     "ds_read_b128 %12, %16 offset:384\n\t"
+                     "ds_read_b128 %13, %16 offset:416\n\t"
+                     "ds_read_b128 %14, %16 offset:448\n\t"
+                     "ds_read_b128 %15, %16 offset:480\n\t"
+                     "s_waitcnt lgkmcnt(0)"
+                     : "=&v"(raw[0]), "=&v"(raw[1]), "=&v"(raw[2]), "=&v"(raw[3]), "=&v"(raw[4]), "=&v"(raw[5]), "=&v"(raw[6]), "=&v"(raw[7]), "=&v"(raw[8]), "=&v"(raw[9]), "=&v"(raw[10]), "=&v"(raw[11]), "=&v"(raw[12]), "=&v"(raw[13]), "=&v"(raw[14]), "=&v"(raw[15])
+                     : "v"(bias_at));
+    } else {
+        asm volatile(
+                     "ds_read_b64 %0, %16\n\t"
+                     "ds_read_b64 %1, %16 offset:16\n\t"
+                     "ds_read_b64 %2, %16 offset:32\n\t"
+                     "ds_read_b64 %3, %16 offset:48\n\t"
+                     "ds_read_b64 %4, %16 offset:64\n\t"
+                     "ds_read_b64 %5, %16 offset:80\n\t"
+                     "ds_read_b64 %6, %16 offset:96\n\t"
+                     "ds_read_b64 %7, %16 offset:112\n\t"
+                     "ds_read_b64 %8, %16 offset:128\n\t"
+                     "ds_read_b64 %9, %16 offset:144\n\t"
+                     "ds_read_b64 %10, %16 offset:160\n\t"
+                     "ds_read_b64 %11, %16 offset:176\n\t"
+                     "ds_read_b64 %12, %16 offset:192\n\t"
+                     "ds_read_b64 %13, %16 offset:208\n\t"
+                     "ds_read_b64 %14, %16 offset:224\n\t"
+                     "ds_read_b64 %15, %16 offset:240\n\t"
+                     "s_waitcnt lgkmcnt(0)"
+                     : "=&v"(raw[0]), "=&v"(raw[1]), "=&v"(raw[2]), "=&v"(raw[3]), "=&v"(raw[4]), "=&v"(raw[5]), "=&v"(raw[6]), "=&v"(raw[7]), "=&v"(raw[8]), "=&v"(raw[9]), "=&v"(raw[10]), "=&v"(raw[11]), "=&v"(raw[12]), "=&v"(raw[13]), "=&v"(raw[14]), "=&v"(raw[15])
+                     : "v"(bias_at));
+    }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int j = 0; j < 4; ++j)
