@@ -140,8 +140,8 @@ __device__ __forceinline__ uint32_t wave_inclusive_scan32(uint32_t v) {
 // COLLECT 0 stores the tile.  COLLECT 1 / 2 store nothing: the epilogue compares every element
 // with the layer's cut value (1) or its feature's threshold (2) and appends the ones that reach
 // it, as (feature, raw value) entries ordered by (token, feature), to one extent of the layer's
-// candidate pool per wavefront and feature segment (see CollectArgs).  These modes need
-// N % BN == 0; a token tile that was shifted back reports only the tokens its neighbour does not own.
+// candidate pool per wavefront and feature segment (see CollectArgs).  A tile that was shifted
+// back, in either direction, reports only the tokens and features its neighbour does not own.
 // SEG (storing mode only): K is made of segments of `sps` stages each; segment q of a row starts
 // q * xss (x) / q * wss (W) elements after the row's first segment and rows are xrs / wrs elements apart,
 // so both operands may be gathered from several matrices side by side (see clt_encode_segmented).
@@ -698,12 +698,14 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
             }
           }
         };
-        const int nseg = N / SEGW;
-        const int seg = ncol0 / SEGW;
-        // the books are kept on the grid of whole tiles: this wave tile's rows start at grid row om0 + 64 wm
+        // the books are kept on the grid of whole tiles, in both directions: this wave tile's rows start at grid
+        // row om0 + 64 wm, its segment is the one at feature on0 + 128 wn (+ the pass's half) of the grid
+        const int nseg = tiles_n * BN / SEGW;
+        const int seg = (cur.on0 + wn * 128 + pass * SEGW) / SEGW;
         const int Mp = tiles_m * BM, grow0 = cur.om0 + wm * 64;
         const int nrb = Mp / COLLECT_ROWS, rowblk = grow0 / COLLECT_ROWS;
         const int shift = cur.om0 - m0;                      // > 0: the tile was shifted back inside the matrix
+        const int cshift = cur.on0 - ncol0;                  // > 0: the segment's first cshift features are the neighbour's
         const uint32_t tile = (uint32_t)seg * (uint32_t)nrb + (uint32_t)rowblk;
         uint32_t off = tile * ca.caps;                       // the tile's fixed slot
         // Each piece of 32 tokens is emitted into the fixed slot as soon as it is scanned, while it is
@@ -713,10 +715,18 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))
         for (int h = 0; h < 2; ++h) {
           park_rows(pass, h, 1);
           scan_piece(W[h]);
-          // the first `shift` tokens of a shifted tile belong to its neighbour, which reports them
+          // the first `shift` tokens of a shifted tile belong to its neighbour, which reports them, and so do the
+          // features in front of on0 (bit b of word i of a lane = feature hs * SEGW / 2 + 32 i + b of the segment)
           if (shift > 0 && wm * 64 + h * 32 + l31 < shift) {
 #pragma unroll
             for (int i = 0; i < NWL; ++i) W[h][i] = 0;
+          }
+          if (cshift > 0) {
+#pragma unroll
+            for (int i = 0; i < NWL; ++i) {
+              const int low = cshift - hs * (SEGW / 2) - i * 32;     // bits below `low` go
+              W[h][i] &= low <= 0 ? ~0u : low >= 32 ? 0u : ~0u << low;
+            }
           }
           cnt[h] = 0;
 #pragma unroll
@@ -819,7 +829,7 @@ static int launch_encode(const void *x, const void *w, const void *b, void *pre,
                          int64_t L, int64_t xs, int64_t wstr, int64_t bs, int64_t ps, int collect,
                          const SelState *gate, const CollectArgs *ca, hipStream_t stream) {
   const bool fast = encode_fast_ok<T>(x, w, b, collect ? nullptr : pre, T_, d, F, xs, wstr, bs, collect ? 16 : ps);
-  if (collect && !(fast && F % BN == 0)) return CLT_ERR_ARG;
+  if (collect && !fast) return CLT_ERR_ARG;
   if (fast) {
     const int64_t tm = clt_ceil_div(T_, BM), tn = clt_ceil_div(F, BN);
     const int64_t nblk = tm * tn * L;
@@ -913,7 +923,7 @@ bool clt_encode_can_collect(const void *x, const void *w, const void *b, int64_t
                             int64_t xs, int64_t wstr, int64_t bs, int dtype) {
   const bool fast = dtype != CLT_F32 ? encode_fast_ok<bf16_t>(x, w, b, nullptr, T, d, F, xs, wstr, bs, 16)   // any 16-bit type
                                      : encode_fast_ok<float>(x, w, b, nullptr, T, d, F, xs, wstr, bs, 16);
-  return fast && F % BN == 0;
+  return fast;
 }
 
 extern "C" int clt_encode(const void *x, const void *w, const void *b, void *pre, int64_t T, int64_t d, int64_t F,

@@ -1451,7 +1451,7 @@ static TileLayout tile_layout(int64_t T, int64_t F, int64_t L, int64_t k, int dt
   TileLayout tl;
   tl.sel = sel_layout(T, F, L, k, CLT_TOPK_PER_LAYER);
   const int segw = dtype != CLT_F32 ? 128 : 64;
-  tl.nseg = (int)(F / segw);
+  tl.nseg = (int)(collect_grid_rows(F) / segw);   // whole feature tiles too (COLLECT_TILE_ROWS is the tile's side)
   const int64_t Tp = collect_grid_rows(T);   // the epilogue's books cover whole token tiles
   tl.ntile = tl.nseg * (int)(Tp / COLLECT_ROWS);
   // about 1.5x K candidates are expected, i.e. 1.5 * k / F of a tile's 64 * segw elements; a
@@ -1574,7 +1574,7 @@ struct ThreshLayout {
 static ThreshLayout thresh_layout(int64_t T, int64_t F, int64_t L, int64_t density_ppm, int dtype) {
   ThreshLayout tl;
   const int segw = dtype != CLT_F32 ? 128 : 64;
-  tl.nseg = (int)(F / segw);
+  tl.nseg = (int)(collect_grid_rows(F) / segw);   // whole feature tiles too (COLLECT_TILE_ROWS is the tile's side)
   const int64_t Tp = collect_grid_rows(T);   // the epilogue's books cover whole token tiles
   tl.ntile = tl.nseg * (int)(Tp / COLLECT_ROWS);
   const double dens = (double)(density_ppm < 1 ? 1 : density_ppm) * 1e-6;

@@ -401,8 +401,8 @@ class Decoder(nn.Module):
             return t_end
         T, F, d = surv.T, surv.F, cfg.d_model
         esize = torch.finfo(surv.dtype).bits // 8
-        # shapes the MFMA kernel of clt_encode takes (K = F in whole pairs of 128-byte stages, 256 x 256 tiles)
-        if surv.dtype not in (torch.bfloat16, torch.float16, torch.float32) or T < 256 or d < 256 or d % 4 or F % (256 // esize):
+        # shapes the MFMA kernel of clt_encode takes (K = F in whole 128-byte stages, 256 x 256 tiles)
+        if surv.dtype not in (torch.bfloat16, torch.float16, torch.float32) or T < 256 or d < 256 or d % 4 or F % (128 // esize):
             return t_end
         gather_rate, mfma_rate = self.route_rates(T, F, d, surv.dtype)
         dense_s = 2.0 * T * F * d / mfma_rate

@@ -176,10 +176,10 @@ int clt_batchtopk_select(const void *pre, int64_t T, int64_t F, int64_t L,
  * the same stream, clt_collect_select after clt_encode_collect.
  * `pre` [L][T][F] is scratch: it is written only for a layer whose cut turned out unusable
  * (fewer than k*T candidates, or no pool space left), which then takes the streaming route.
- * clt_encode_collect_supported returns 1 when the shapes qualify (T >= 256, any remainder:
- * the last token tile is shifted back inside the matrix and reports only the tokens its
- * neighbour does not own; F % 256 == 0, d % 64 == 0 for 16-bit elements / d % 32 == 0 for
- * fp32, 16-byte aligned rows, k > 0), else 0; callers then use clt_encode +
+ * clt_encode_collect_supported returns 1 when the shapes qualify (T >= 256 and F >= 256 with
+ * any remainder: a last tile is shifted back inside the matrix and reports only the tokens
+ * and features its neighbour does not own; F % 8 == 0, d % 64 == 0 for 16-bit elements /
+ * d % 32 == 0 for fp32, 16-byte aligned rows, k > 0), else 0; callers then use clt_encode +
  * clt_batchtopk_select.
  * Replaces the same reference calls as clt_encode and clt_batchtopk_select
  * (clt/models/encoder.py:151-162, clt/activations/registry.py:43-72,

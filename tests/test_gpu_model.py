@@ -55,7 +55,7 @@ CASES = [
     BASE.scaled("tiny-topk-global", activation_fn="topk", k=6, topk_mode="global", dtype="bfloat16"),
     BASE.scaled("ref-shape", num_layers=2, d_model=8, num_features=16, tokens=30, k=3),   # the reference's own test shape
     BASE.scaled("mid", num_layers=4, d_model=768, num_features=2048, tokens=300, k=20, dtype="bfloat16"),
-    # shapes that take the routes fused into the encoder epilogue (T % 256 == 0, F % 256 == 0)
+    # shapes that take the routes fused into the encoder epilogue (at least one 256 x 256 tile)
     BASE.scaled("fused-topk", num_layers=3, d_model=128, num_features=512, tokens=256, k=12),
     BASE.scaled("fused-topk-bf16", num_layers=3, d_model=256, num_features=1024, tokens=512, k=24, dtype="bfloat16"),
     # a short prompt on a model whose shapes take the matrix-core encoder: the batch is padded to one tile
