@@ -46,9 +46,10 @@ def test_accumulate_dense_is_the_running_sum_in_the_model_dtype(dev, dtype):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16", "float16"])
 @pytest.mark.parametrize("affine", [False, True])
-def test_dense_route_matches_the_oracle_and_the_gather_route(dev, dtype, affine):
+@pytest.mark.parametrize("features", [512, 576])      # 576: an odd number of 128-byte stages along the product's K
+def test_dense_route_matches_the_oracle_and_the_gather_route(dev, dtype, affine, features):
     tdt = getattr(torch, dtype)
-    wl = synth.Workload("dense-route", 7, 4, 256, 512, 512, dtype, k=24, decoder_tying="per_target")
+    wl = synth.Workload("dense-route", 7, 4, 256, features, 512, dtype, k=24, decoder_tying="per_target")
     cfg = wl.config()
     cfg.enable_feature_offset = cfg.enable_feature_scale = affine
     x = synth.make_inputs(wl, "cpu")
