@@ -34,6 +34,7 @@ _SIGNATURES = {
     "clt_version": (_int, []),
     "clt_error_string": (ctypes.c_char_p, [_int]),
     "clt_encode": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _int, _vp]),
+    "clt_encode_fast_path": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _int]),
     "clt_encode_segmented": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _int, _vp]),
     "clt_colstats": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
     "clt_colstats_full": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),

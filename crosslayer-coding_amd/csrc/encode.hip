@@ -926,6 +926,17 @@ bool clt_encode_can_collect(const void *x, const void *w, const void *b, int64_t
   return fast;
 }
 
+extern "C" int clt_encode_fast_path(const void *x, const void *w, const void *b, const void *pre, int64_t T, int64_t d,
+                                    int64_t F, int64_t L, int64_t x_layer_stride, int64_t w_layer_stride,
+                                    int64_t b_layer_stride, int64_t pre_layer_stride, int dtype) {
+  if (!clt_model_dtype(dtype) || T <= 0 || d <= 0 || F <= 0 || L <= 0 || !x || !w || !pre) return 0;
+  if (clt_ceil_div(T, BM) * clt_ceil_div(F, BN) * L > 2147483647LL) return 0;
+  const bool fast = dtype != CLT_F32
+                        ? encode_fast_ok<bf16_t>(x, w, b, pre, T, d, F, x_layer_stride, w_layer_stride, b_layer_stride, pre_layer_stride)
+                        : encode_fast_ok<float>(x, w, b, pre, T, d, F, x_layer_stride, w_layer_stride, b_layer_stride, pre_layer_stride);
+  return fast ? 1 : 0;
+}
+
 extern "C" int clt_encode(const void *x, const void *w, const void *b, void *pre, int64_t T, int64_t d, int64_t F,
                           int64_t L, int64_t x_layer_stride, int64_t w_layer_stride, int64_t b_layer_stride,
                           int64_t pre_layer_stride, int dtype, void *stream) {

@@ -120,6 +120,9 @@ def _wants_sliced_decode(rows: int, slab_bytes: int) -> bool:
 
 # token rows of one tile of the matrix-core encoder: shorter batches are padded to it (see ``encode``)
 ENCODE_MIN_TOKENS = 256
+# below this many multiply-adds a shape the matrix-core encoder does not take stays on the generic kernel (about
+# 0.2 ms there); above it the operands are zero-padded to a shape it takes (see ``encode``)
+ENCODE_PAD_MIN_MACS = 5e7
 
 
 def _stream(t: torch.Tensor) -> int:
@@ -140,24 +143,49 @@ def encode(x: torch.Tensor, w: torch.Tensor, b: Optional[torch.Tensor],
     if b is not None:
         assert b.shape == (L, F) and b.stride(1) == 1 and b.dtype == x.dtype
     lib = nat.load()
-    stage = 128 // x.element_size()          # elements of K in one 128-byte stage of the matrix-core kernel
-    if 0 < T < ENCODE_MIN_TOKENS and F >= 256 and F % 4 == 0 and d % stage == 0:
-        # The matrix-core kernel works on whole 256-token tiles; a shorter batch (a short prompt) would fall to
-        # the one-thread-per-output kernel, which is 30x slower than the padded product.  Rows past T are zeros
-        # going in and are dropped coming out.
-        xp = torch.zeros((L, ENCODE_MIN_TOKENS, d), dtype=x.dtype, device=x.device)
-        xp[:, :T] = x
-        outp = torch.empty((L, ENCODE_MIN_TOKENS, F), dtype=x.dtype, device=x.device)
-        code = lib.clt_encode(nat.ptr(xp), nat.ptr(w), nat.ptr(b), nat.ptr(outp), ENCODE_MIN_TOKENS, d, F, L,
-                              xp.stride(0), w.stride(0), b.stride(0) if b is not None else 0, outp.stride(0),
-                              nat.dtype_code(x.dtype), _stream(x))
+    dt = nat.dtype_code(x.dtype)
+
+    def query(x_, w_, b_, out_):
+        return bool(lib.clt_encode_fast_path(nat.ptr(x_), nat.ptr(w_), nat.ptr(b_), nat.ptr(out_), x_.shape[1], x_.shape[2],
+                                             w_.shape[1], L, x_.stride(0), w_.stride(0),
+                                             b_.stride(0) if b_ is not None else 0, out_.stride(0), dt))
+
+    def run(x_, w_, b_, out_):
+        code = lib.clt_encode(nat.ptr(x_), nat.ptr(w_), nat.ptr(b_), nat.ptr(out_), x_.shape[1], x_.shape[2], w_.shape[1], L,
+                              x_.stride(0), w_.stride(0), b_.stride(0) if b_ is not None else 0, out_.stride(0),
+                              dt, _stream(x))
         nat.check(code, "clt_encode")
-        out.copy_(outp[:, :T])
+
+    if T == 0 or query(x, w, b, out):
+        run(x, w, b, out)
         return out
-    code = lib.clt_encode(nat.ptr(x), nat.ptr(w), nat.ptr(b), nat.ptr(out), T, d, F, L,
-                          x.stride(0), w.stride(0), b.stride(0) if b is not None else 0, out.stride(0),
-                          nat.dtype_code(x.dtype), _stream(x))
-    nat.check(code, "clt_encode")
+    # The matrix-core kernel works on whole 256 x 256 tiles and whole 128-byte stages along d; anything else falls
+    # to the one-thread-per-output kernel, which is 30x slower on a short prompt and hundreds of times on a large
+    # odd shape.  Such operands are handed over as zero-padded copies instead (zeros add nothing to the sums;
+    # rows and columns past the real ones are dropped coming out): only the tokens of a short batch when nothing
+    # else is in the way, the weights too (two passes over them, still far cheaper) when d or F is.
+    stage = 128 // x.element_size()
+    Tp, dp, Fp = max(T, ENCODE_MIN_TOKENS), -(-d // stage) * stage, max(256, -(-F // 8) * 8)
+    if (dp != d or Fp != F) and L * T * F * d < ENCODE_PAD_MIN_MACS:
+        run(x, w, b, out)
+        return out
+    xp, wp, bp = x, w, b
+    if Tp != T or dp != d:
+        xp = torch.zeros((L, Tp, dp), dtype=x.dtype, device=x.device)
+        xp[:, :T, :d] = x
+    if dp != d or Fp != F:
+        wp = torch.zeros((L, Fp, dp), dtype=x.dtype, device=x.device)
+        wp[:, :F, :d] = w
+    if b is not None and Fp != F:
+        bp = torch.zeros((L, Fp), dtype=x.dtype, device=x.device)
+        bp[:, :F] = b
+    outp = out if (Tp == T and Fp == F) else torch.empty((L, Tp, Fp), dtype=x.dtype, device=x.device)
+    if not query(xp, wp, bp, outp):       # something else is in the way (an unaligned view, say)
+        run(x, w, b, out)
+        return out
+    run(xp, wp, bp, outp)
+    if outp is not out:
+        out.copy_(outp[:, :T, :F])
     return out
 
 

@@ -89,6 +89,20 @@ int clt_encode(const void *x, const void *w, const void *b, void *pre,
                int dtype, void *stream);
 
 /*
+ * 1 when clt_encode runs these operands on the matrix cores: T >= 256, F >= 256, F % 4 == 0,
+ * d a whole number of 128-byte stages (64 elements of 16 bits, 32 of fp32), 16-byte aligned
+ * pointers, layer strides that keep every layer 16-byte aligned (the bias stride a multiple
+ * of 8 elements).  0: the call is served by a generic kernel with one thread per output,
+ * two to three orders of magnitude slower on large shapes; a caller with such a shape does
+ * better to hand over zero-padded copies (the host mirror does, crosslayer_coding_amd.engine.encode).
+ * No counterpart in the reference (its F.linear takes any shape at one speed).
+ */
+int clt_encode_fast_path(const void *x, const void *w, const void *b, const void *pre,
+                         int64_t T, int64_t d, int64_t F, int64_t L,
+                         int64_t x_layer_stride, int64_t w_layer_stride,
+                         int64_t b_layer_stride, int64_t pre_layer_stride, int dtype);
+
+/*
  * The same product with both operands cut into n_seg segments of d_seg along K, each segment
  * in a matrix of its own:
  *   pre[t][f] = sum_q sum_k x[q * x_seg_stride + t * x_row_stride + k] * w[q * w_seg_stride + f * w_row_stride + k]

@@ -41,7 +41,9 @@ def check_rows_sorted(surv):
                                      (2, 40, 256, 512), (1, 1, 128, 256), (3, 255, 128, 260),     # short batches: padded to a tile
                                      # an odd number of 128-byte stages along d (1, 3, 5 for 16-bit elements)
                                      (1, 256, 64, 256), (2, 512, 192, 512), (2, 300, 320, 520), (1, 256, 32, 256),
-                                     (1, 700, 1600, 768)])
+                                     (1, 700, 1600, 768),
+                                     # shapes the matrix kernel takes only as zero-padded copies (d, F, T or all three)
+                                     (2, 300, 200, 1092), (1, 100, 72, 7000), (3, 512, 100, 516), (1, 260, 1000, 250)])
 def test_encode_parity(dev, dtype, L, T, d, F):
     g = torch.Generator().manual_seed(L * 1000 + T)
     x = torch.randn(L, T, d, generator=g).to(dtype)
