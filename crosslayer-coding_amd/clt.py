@@ -87,6 +87,9 @@ class _ReconstructionsWithGraph(torch.autograd.Function):
         return (None, None, None, *grads)
 
 
+MAX_LAYERS = 64     # layers of one model (the kernels' source-layer masks are 64 bits wide)
+
+
 class CrossLayerTranscoder(BaseTranscoder):
     device: torch.device
     dtype: torch.dtype
@@ -95,6 +98,11 @@ class CrossLayerTranscoder(BaseTranscoder):
                  profiler: Optional[Any] = None):
         super().__init__(config)
         require_single_rank(process_group)
+        if config.num_layers > MAX_LAYERS:
+            # said here, not by the first forward: the decode and gradient kernels keep the set of layers a batch
+            # has inputs for in one 64-bit word
+            raise NotImplementedError(f"num_layers = {config.num_layers}: the HIP kernels of this build take at most "
+                                      f"{MAX_LAYERS} layers")
         self.process_group = process_group
         self.world_size, self.rank = 1, 0
         self.profiler = profiler

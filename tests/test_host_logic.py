@@ -219,3 +219,11 @@ def test_feed_rejects_bad_arguments_and_needs_a_gpu():
             feed.parse_batch(np.zeros((4, 2), dtype=np.uint32))
     with pytest.raises(ValueError):
         feed.add_chunk(0, torch.zeros(2, 2, 5, 7))
+
+
+def test_more_than_64_layers_are_refused_at_construction():
+    import pytest
+    with pytest.raises(NotImplementedError, match="at most 64 layers"):
+        cca.CrossLayerTranscoder(cfg(num_layers=65, decoder_tying="per_source"), None, torch.device("cpu"))
+    m = cca.CrossLayerTranscoder(cfg(num_layers=64, decoder_tying="per_source"), None, torch.device("cpu"))
+    assert len(m.decoder_module.decoders) == 64
