@@ -963,7 +963,7 @@ static unsigned bw_resident_blocks(K kernel) {
 //   grad_theta[f] = sum over tokens of grad_out * (-x / bandwidth)  where |x - theta[f]| <= bandwidth / 2
 // on dense [T, F] pre-activations x and dense d loss / d activation, every step rounded to the
 // model dtype as the reference's tensor arithmetic is; the sum itself is fp32, rows in a fixed order.
-constexpr int TG_SPLIT = 32;
+constexpr int TG_SPLIT = 128;   // row slices per column: enough wavefronts in flight to cover the memory latency
 template <typename T>
 __global__ __launch_bounds__(BW_THREADS) void k_theta_grad_partial(const T *__restrict__ pre, const T *__restrict__ dact,
                                                                     const T *__restrict__ theta, int64_t Tn, int64_t F,
@@ -971,7 +971,8 @@ __global__ __launch_bounds__(BW_THREADS) void k_theta_grad_partial(const T *__re
   const int64_t f = (int64_t)blockIdx.x * BW_THREADS + threadIdx.x;
   if (f >= F) return;
   const int64_t rows = (Tn + TG_SPLIT - 1) / TG_SPLIT, r0 = (int64_t)blockIdx.y * rows, r1 = r0 + rows < Tn ? r0 + rows : Tn;
-  const float th = Elem<T>::to_f32(theta[f]), half = 0.5f * bw;
+  // (the reference compares with the scalar bandwidth / 2 in the tensors' dtype: the scalar is rounded to it)
+  const float th = Elem<T>::to_f32(theta[f]), half = Elem<T>::round(0.5f * bw);
   float acc = 0.0f;
   for (int64_t r = r0; r < r1; ++r) {
     const float x = Elem<T>::to_f32(pre[r * F + f]);
@@ -981,6 +982,54 @@ __global__ __launch_bounds__(BW_THREADS) void k_theta_grad_partial(const T *__re
     }
   }
   part[(int64_t)blockIdx.y * F + f] = acc;
+}
+// The same sums with 16 bytes of a row per thread (8 bf16 / 4 fp32 columns) and four rows of both operands asked
+// for at a time: each column is still summed by one thread, over the same rows in the same order.  POW2: the
+// bandwidth is a power of two, so -x / bandwidth is the exact product with its reciprocal.
+template <typename T, bool POW2>
+__global__ __launch_bounds__(BW_THREADS) void k_theta_grad_partial_vec(const T *__restrict__ pre, const T *__restrict__ dact,
+                                                                        const T *__restrict__ theta, int64_t Tn, int64_t F,
+                                                                        float bw, float inv_bw, float *__restrict__ part) {
+  constexpr int V = 16 / (int)sizeof(T), NR = 4;
+  const int64_t f0 = ((int64_t)blockIdx.x * BW_THREADS + threadIdx.x) * V;
+  if (f0 >= F) return;
+  const int64_t rows = (Tn + TG_SPLIT - 1) / TG_SPLIT, r0 = (int64_t)blockIdx.y * rows, r1 = r0 + rows < Tn ? r0 + rows : Tn;
+  auto unpack = [](const uint4 &v, float (&x)[V]) {
+    if constexpr (sizeof(T) == 2) {
+      const uint32_t w4[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int k = 0; k < 4; ++k) { x[2 * k] = __uint_as_float(w4[k] << 16); x[2 * k + 1] = __uint_as_float(w4[k] & 0xFFFF0000u); }
+    } else {
+      x[0] = __uint_as_float(v.x); x[1] = __uint_as_float(v.y); x[2] = __uint_as_float(v.z); x[3] = __uint_as_float(v.w);
+    }
+  };
+  float th[V], acc[V];
+  unpack(*reinterpret_cast<const uint4 *>(theta + f0), th);
+#pragma unroll
+  for (int j = 0; j < V; ++j) acc[j] = 0.0f;
+  const float half = Elem<T>::round(0.5f * bw);    // the scalar of the comparison, in the tensors' dtype as torch has it
+  for (int64_t r = r0; r < r1; r += NR) {
+    uint4 xv[NR], gv[NR];
+#pragma unroll
+    for (int u = 0; u < NR; ++u) {      // (past the slice: its last row again, not used)
+      const int64_t rr = r + u < r1 ? r + u : r1 - 1;
+      xv[u] = *reinterpret_cast<const uint4 *>(pre + rr * F + f0);
+      gv[u] = *reinterpret_cast<const uint4 *>(dact + rr * F + f0);
+    }
+#pragma unroll
+    for (int u = 0; u < NR; ++u) {
+      if (r + u >= r1) break;
+      float x[V], g[V];
+      unpack(xv[u], x);
+      unpack(gv[u], g);
+#pragma unroll
+      for (int j = 0; j < V; ++j)
+        if (fabsf(Elem<T>::round(x[j] - th[j])) <= half)
+          acc[j] += Elem<T>::round(g[j] * Elem<T>::round(POW2 ? -x[j] * inv_bw : -x[j] / bw));
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < V; ++j) part[(int64_t)blockIdx.y * F + f0 + j] = acc[j];
 }
 __global__ void k_theta_grad_finish(const float *part, int64_t F, float *out) {
   for (int64_t f = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; f < F; f += (int64_t)gridDim.x * blockDim.x) {
@@ -1348,11 +1397,24 @@ extern "C" int clt_jumprelu_theta_grad(const void *pre, const void *dact, const 
   if ((((uintptr_t)workspace) & 3u) != 0) return CLT_ERR_ALIGN;
   hipStream_t s = (hipStream_t)stream;
   float *part = (float *)workspace;
-  dim3 grid((unsigned)clt_ceil_div(F, BW_THREADS), TG_SPLIT);
-  if (dtype == CLT_BF16)
-    k_theta_grad_partial<bf16_t><<<grid, BW_THREADS, 0, s>>>((const bf16_t *)pre, (const bf16_t *)dact, (const bf16_t *)theta, T, F, (float)bandwidth, part);
-  else
-    k_theta_grad_partial<float><<<grid, BW_THREADS, 0, s>>>((const float *)pre, (const float *)dact, (const float *)theta, T, F, (float)bandwidth, part);
+  const float bwf = (float)bandwidth;
+  const int esz = dtype == CLT_BF16 ? 2 : 4, vec = 16 / esz;
+  // whole 16-byte pieces per row and aligned rows: the vector kernel; anything else one column per thread
+  if (F % vec == 0 && clt_aligned16(pre) && clt_aligned16(dact) && clt_aligned16(theta)) {
+    int ex = 0;
+    const bool pow2 = frexpf(bwf, &ex) == 0.5f && ex > -100 && ex < 100;    // 1 / bandwidth is exact and normal
+    dim3 gridv((unsigned)clt_ceil_div(F / vec, BW_THREADS), TG_SPLIT);
+#define CLT_TG(CT, P2) k_theta_grad_partial_vec<CT, P2><<<gridv, BW_THREADS, 0, s>>>((const CT *)pre, (const CT *)dact, (const CT *)theta, T, F, bwf, 1.0f / bwf, part)
+    if (dtype == CLT_BF16) { if (pow2) CLT_TG(bf16_t, true); else CLT_TG(bf16_t, false); }
+    else { if (pow2) CLT_TG(float, true); else CLT_TG(float, false); }
+#undef CLT_TG
+  } else {
+    dim3 grid((unsigned)clt_ceil_div(F, BW_THREADS), TG_SPLIT);
+    if (dtype == CLT_BF16)
+      k_theta_grad_partial<bf16_t><<<grid, BW_THREADS, 0, s>>>((const bf16_t *)pre, (const bf16_t *)dact, (const bf16_t *)theta, T, F, bwf, part);
+    else
+      k_theta_grad_partial<float><<<grid, BW_THREADS, 0, s>>>((const float *)pre, (const float *)dact, (const float *)theta, T, F, bwf, part);
+  }
   k_theta_grad_finish<<<(unsigned)clt_ceil_div(F, 256), 256, 0, s>>>(part, F, grad_theta);
   return clt_check_launch();
 }

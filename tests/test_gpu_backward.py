@@ -581,3 +581,25 @@ def test_adam_batched_entry_points_equal_the_single_ones(dev, dtype):
     # bad arguments are refused before anything is launched
     assert lib.clt_adam_step_decoders(None, None, 1, None, None, None, None, d, F, 3e-3, 0.9, 0.999, 1e-8, 1, code, stream) != 0
     assert lib.clt_adam_step_many(None, None, None, None, 2, d, 3e-3, 0.9, 0.999, 1e-8, 1, code, stream) != 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("T,F", [(300, 520), (1000, 256), (77, 250), (4100, 1032)],
+                         ids=["vector", "vector-whole", "one-column-per-thread", "long-slices"])
+@pytest.mark.parametrize("bandwidth", [1.0, 0.3, 0.25])
+def test_threshold_gradient_reduction(dev, dtype, T, F, bandwidth):
+    """clt_jumprelu_theta_grad against the reference's tensor arithmetic (clt/models/activations.py:196-199): every
+    elementwise step in the model dtype, the column sums in fp32.  Both kernels behind the entry point (16 bytes of
+    a row per thread, or one column per thread when a row is not whole 16-byte pieces), power-of-two and other
+    bandwidths."""
+    g = torch.Generator().manual_seed(T + F)
+    x = (torch.randn(T, F, generator=g) * 0.7).to(dtype)
+    go = torch.randn(T, F, generator=g).to(dtype)
+    theta = torch.exp(0.4 * torch.randn(F, generator=g) - 0.5).to(dtype)
+    near = torch.abs(x - theta) <= (bandwidth / 2.0)
+    want = (go * ((-x / bandwidth) * near.type_as(x))).float().sum(0)
+    got = torch.empty(F, dtype=torch.float32, device=dev)
+    engine.jumprelu_theta_grad(x.to(dev), go.to(dev), theta.to(dev), bandwidth, got)
+    scale = float(want.abs().max())
+    assert float((got.cpu() - want).abs().max()) <= 2e-5 * scale + (1e-6 if dtype == torch.float32 else 0.0)
+    assert int(near.sum()) > 0
