@@ -232,7 +232,9 @@ def assert_same_list(got, ref, dtype):
                                      # an odd number of stages along d
                                      (2, 512, 320, 512), (1, 300, 64, 256),
                                      # feature counts that are not whole tiles: the last feature tile is shifted back
-                                     (2, 256, 128, 384), (1, 300, 128, 520), (2, 512, 64, 1096), (1, 257, 128, 264)])
+                                     (2, 256, 128, 384), (1, 300, 128, 520), (2, 512, 64, 1096), (1, 257, 128, 264),
+                                     # more token tiles than feature tiles, in eights: the token-major tile map
+                                     (1, 2000, 128, 256), (1, 4000, 64, 520)])
 def test_encode_threshold_matches_separate_and_oracle(dev, dtype, L, T, d, F):
     g = torch.Generator().manual_seed(L * 17 + T + F)
     x = torch.randn(L, T, d, generator=g).to(dtype)
@@ -329,7 +331,9 @@ def fused_vs_separate(x, w, b, k, dev):
                                        (2, 512, 192, 512, 20), (1, 300, 64, 256, 5), (1, 512, 1600, 512, 16),
                                        # feature counts that are not whole tiles: the last feature tile is shifted back
                                        (2, 256, 128, 384, 9), (1, 300, 128, 520, 30), (2, 512, 64, 1096, 17), (1, 257, 128, 264, 4),
-                                       (1, 600, 128, 448, 100), (2, 256, 128, 320, 3)])
+                                       (1, 600, 128, 448, 100), (2, 256, 128, 320, 3),
+                                       # more token tiles than feature tiles, in eights: the token-major tile map
+                                       (1, 2000, 128, 256, 6), (1, 4000, 64, 520, 11), (2, 2048, 128, 512, 9)])
 def test_encode_collect_matches_separate_and_oracle(dev, dtype, L, T, d, F, k):
     g = torch.Generator().manual_seed(L * 31 + T + F + k)
     x = torch.randn(L, T, d, generator=g).to(dtype)
