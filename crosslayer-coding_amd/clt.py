@@ -290,6 +290,10 @@ class CrossLayerTranscoder(BaseTranscoder):
         ws = self._workspace()
         mask = (1 << L) - 1
         dec = self.decoder_module
+        if dec.skip_weights is None and dec.dense_pairs_wanted(surv, None):
+            # so many survivors that the reference's dense products are the cheaper formulation (the decoder step is
+            # then not fused: ``dec_w`` is returned and the optimiser applies it)
+            return self._raw_gradients_dense(inputs, surv, g, g_model, bias_grad)
         off, sc = dec._affine()                     # per-target feature offset / scale of tied decoders, or None
         dval = engine.decode_backward_values(surv, dec.packed(), g, cfg.decoder_tying, mask, ws, feat_scale=sc)
         lists = engine.feature_lists(surv, ws)
@@ -341,33 +345,111 @@ class CrossLayerTranscoder(BaseTranscoder):
         theta = self.theta_manager.thresholds(self.dtype)
         packed = self.decoder_module.packed()
         out = torch.empty((L, F), dtype=torch.float32, device=pre.device)
-        T, d, pitch = g_model.shape[1], cfg.d_model, packed.shape[2]
+        T = g_model.shape[1]
         g_model = g_model.contiguous()
-        piece = 64 if self.dtype == torch.bfloat16 else 32      # elements of K the matrix-core kernel takes at a time
         dact_buf = ws.typed("theta_dact", (T, F), self.dtype)
         for s_ in range(L):
-            targets = list(range(s_, L))
-            n = len(targets)
-            if tying == "none":
-                slots = [s_ * L - (s_ * (s_ - 1)) // 2 + (t - s_) for t in targets]
-            elif tying == "per_source":
-                slots = [s_] * n
-            else:
-                slots = targets
-            if T >= 256 and F >= 256 and F % 4 == 0 and d % piece == 0 and (n * d // piece) % 2 == 0:
-                # both operands where they lie: segment q = target s + q, in the gradient slab [L, T, d] and
-                # in the packed decoders [n_dec, F, pitch] (one matrix for all targets when tied per source)
-                dact = engine.encode_segmented(g_model[s_:], packed[slots[0]:], n, d, T * d, d,
-                                               0 if tying == "per_source" else F * pitch, pitch, T, F, out=dact_buf)
-            else:
-                stacked_w = torch.cat([packed[i][:, :d] for i in slots], dim=1).unsqueeze(0)   # [1, F, n d]
-                stacked_g = torch.cat([g_model[t] for t in targets], dim=1).unsqueeze(0)       # [1, T, n d]
-                dact = engine.encode(stacked_g.contiguous(), stacked_w.contiguous(), None)[0]  # [T, F]
+            dact = self._dense_activation_gradient(s_, g_model, packed, dact_buf)
             if dval is not None:
                 engine.scatter_survivor_values(surv, dval, s_, dact)
             engine.jumprelu_theta_grad(pre[s_], dact, theta[s_].contiguous(), self.theta_manager.bandwidth, out[s_], ws)
         # theta = exp(log_threshold): the reference casts theta to the model dtype for the forward
         return out * torch.exp(self.theta_manager.log_threshold.detach().float())
+
+    def _dense_activation_gradient(self, s_: int, g_model: torch.Tensor, packed: torch.Tensor,
+                                   out: torch.Tensor) -> torch.Tensor:
+        """d loss / d activation of source layer ``s_`` for every element, [T, F] in the model dtype: the product of
+        the stacked loss gradients [T, (L-s) d] with the stacked decoders [F, (L-s) d] on the MFMA kernel (what
+        autograd forms behind the reference's dense decode, decoder.py:253-338)."""
+        cfg = self.config
+        L, F, d, tying = cfg.num_layers, cfg.num_features, cfg.d_model, cfg.decoder_tying
+        T, pitch = g_model.shape[1], packed.shape[2]
+        piece = 64 if self.dtype == torch.bfloat16 else 32      # elements of K the matrix-core kernel takes at a time
+        targets = list(range(s_, L))
+        n = len(targets)
+        if tying == "none":
+            slots = [s_ * L - (s_ * (s_ - 1)) // 2 + (t - s_) for t in targets]
+        elif tying == "per_source":
+            slots = [s_] * n
+        else:
+            slots = targets
+        if T >= 256 and F >= 256 and F % 4 == 0 and d % piece == 0 and (n * d // piece) % 2 == 0:
+            # both operands where they lie: segment q = target s + q, in the gradient slab [L, T, d] and
+            # in the packed decoders [n_dec, F, pitch] (one matrix for all targets when tied per source)
+            return engine.encode_segmented(g_model[s_:], packed[slots[0]:], n, d, T * d, d,
+                                           0 if tying == "per_source" else F * pitch, pitch, T, F, out=out)
+        stacked_w = torch.cat([packed[i][:, :d] for i in slots], dim=1).unsqueeze(0)   # [1, F, n d]
+        stacked_g = torch.cat([g_model[t] for t in targets], dim=1).unsqueeze(0)       # [1, T, n d]
+        return engine.encode(stacked_g.contiguous(), stacked_w.contiguous(), None)[0]  # [T, F]
+
+    def _raw_gradients_dense(self, inputs: Dict[int, torch.Tensor], surv, g: torch.Tensor, g_model: torch.Tensor,
+                             bias_grad: torch.Tensor):
+        """The raw gradients of ``_raw_gradients_from`` at densities the survivor-list kernels were not made for
+        (``Decoder.dense_pairs_wanted``: untied or per-source decoders, no skip, no feature affine): autograd's own
+        dense formulation behind the reference's dense forward, every product on the MFMA kernel -
+        d loss / d activation per source (``_dense_activation_gradient``), gated by list membership (the
+        straight-through rule of BatchTopK / TokenTopK, ``input >= threshold`` of JumpReLU, activations.py:68-96,
+        192-194), ``dW_enc = dpre.T @ x``, ``dW_dec[s->t] = a[s].T @ g[t]``.  Products are rounded to the model
+        dtype like the reference's autograd results, then kept in fp32."""
+        cfg = self.config
+        L, d, F, tying = cfg.num_layers, cfg.d_model, cfg.num_features, cfg.decoder_tying
+        T = surv.T
+        ws = self._workspace()
+        dec = self.decoder_module
+        packed = dec.packed()
+        dev = g.device
+        _, x_slab, _, _ = self.encoder_module.prepare_slab(inputs)
+        x_slab = x_slab.contiguous()
+        g_model = g_model.contiguous()
+        n_dec = len(dec._ordered())
+        dw_dec = torch.empty((n_dec, F, d), dtype=torch.float32, device=dev)
+        dw_enc = torch.empty((L, F, d), dtype=torch.float32, device=dev)
+        db_enc = torch.empty((L, F), dtype=torch.float32, device=dev)
+        if tying == "per_source":
+            # one decoder per source serves every target >= s: its gradient takes the sum of their loss gradients
+            g_t = torch.flip(torch.cumsum(torch.flip(g, dims=[0]), dim=0), dims=[0]).to(self.dtype)
+        else:
+            g_t = g_model
+        g_t = g_t.transpose(1, 2).contiguous()                                 # [L, d, T]: K = tokens
+        member = SurvivorList(surv.row_ptr, surv.col, torch.ones_like(surv.val), surv.T, surv.F, surv.L, surv.dtype,
+                              surv.status, surv.nnz_hint)
+        theta = pre = theta_out = None
+        if cfg.activation_fn == "jumprelu" and self.theta_manager.log_threshold is not None:
+            w, b = self.encoder_module.stacked()
+            pre = engine.encode(x_slab, w, b, out=ws.typed("pre", (L, T, F), self.dtype))
+            theta = self.theta_manager.thresholds(self.dtype)
+            theta_out = torch.empty((L, F), dtype=torch.float32, device=dev)
+        dact_buf = ws.typed("theta_dact", (T, F), self.dtype)
+        a_buf = ws.typed("dense_sum", (T, F), self.dtype)
+        m_buf = ws.typed("dense_member", (T, F), self.dtype)
+        row0 = 0
+        for s_ in range(L):
+            dact = self._dense_activation_gradient(s_, g_model, packed, dact_buf)
+            if theta_out is not None:
+                engine.jumprelu_theta_grad(pre[s_], dact, theta[s_].contiguous(), self.theta_manager.bandwidth, theta_out[s_], ws)
+            engine.accumulate_dense(member, s_, m_buf, True)
+            dpre = dact * m_buf
+            db_enc[s_] = dpre.sum(0, dtype=torch.float32)
+            dw_enc[s_] = engine.encode(dpre.t().contiguous().unsqueeze(0), x_slab[s_].t().contiguous().unsqueeze(0), None)[0]
+            del dpre
+            engine.accumulate_dense(surv, s_, a_buf, True)
+            a_t = a_buf.t().contiguous()                                       # [F, T]
+            if tying == "none":
+                n = L - s_
+                dw_dec[row0:row0 + n] = engine.encode(a_t.unsqueeze(0).expand(n, F, T), g_t[s_:], None)
+                row0 += n
+            else:
+                dw_dec[s_] = engine.encode(a_t.unsqueeze(0), g_t[s_:s_ + 1], None)[0]
+            del a_t
+        theta_grad = None
+        if theta_out is not None:
+            theta_grad = theta_out * torch.exp(self.theta_manager.log_threshold.detach().float())
+        if tying == "none":
+            dec_b = bias_grad[torch.tensor([t for s_ in range(L) for t in range(s_, L)], device=bias_grad.device)]
+        else:
+            dec_b = torch.flip(torch.cumsum(torch.flip(bias_grad, dims=[0]), dim=0), dims=[0])
+        return {"enc_w": dw_enc, "enc_b": db_enc, "dec_w": dw_dec, "dec_b": dec_b.contiguous(), "theta": theta_grad,
+                "skip": None, "feat_offset": None, "feat_scale": None}
 
     @torch.no_grad()
     def loss_and_gradients(self, inputs: Dict[int, torch.Tensor], targets: Dict[int, torch.Tensor],

@@ -394,8 +394,8 @@ class Decoder(nn.Module):
         with every further source the gather grows and the dense product ``summed [T, F] @ W[t].T`` does
         not.  The dense route is taken from the first target on for which
         ``2 T F d / MFMA rate < rows gathered x d x element size / gather rate`` (``route_rates``).  Untied and per-source
-        decoders never qualify: each (source, target) pair has its own operand or its own matrix, so the
-        dense cost is the reference's full 2 T F d per pair against k T rows per pair."""
+        decoders have no such sum - each (source, target) pair has its own operand or its own matrix - and go dense
+        only at high densities (``dense_pairs_wanted``)."""
         cfg = self.config
         if cfg.decoder_tying != "per_target" or not self.dense_route or skip_add is not None:
             return t_end
@@ -406,13 +406,7 @@ class Decoder(nn.Module):
             return t_end
         gather_rate, mfma_rate = self.route_rates(T, F, d, surv.dtype)
         dense_s = 2.0 * T * F * d / mfma_rate
-        # survivors of one source layer, from a host-side figure: the exact total where the list was sized from
-        # it, else the last total seen for the shape; a threshold list whose total is not known yet is priced
-        # at 2 % density (its arrays are sized for the largest list, which says nothing about the batch)
-        total = surv.nnz_hint
-        if total is None:
-            total = surv.col.numel() if surv.status is None else min(surv.col.numel(), surv.L * T * F // 50)
-        per_layer = total / max(1, surv.L)
+        per_layer = self._survivors_per_layer(surv)
         n_src = 0
         for t in range(t_end):
             n_src += (src_mask >> t) & 1
@@ -420,7 +414,83 @@ class Decoder(nn.Module):
                 return t
         return t_end
 
+    @staticmethod
+    def _survivors_per_layer(surv: SurvivorList) -> float:
+        """Survivors of one source layer, from a host-side figure: the exact total where the list was sized from
+        it, else the last total seen for the shape; a threshold list whose total is not known yet is priced at
+        2 % density (its arrays are sized for the largest list, which says nothing about the batch)."""
+        total = surv.nnz_hint
+        if total is None:
+            total = surv.col.numel() if surv.status is None else min(surv.col.numel(), surv.L * surv.T * surv.F // 50)
+        return total / max(1, surv.L)
+
+    # a (source, target) pair goes to the dense product when its gather is priced this many times dearer
+    DENSE_PAIR_MARGIN = 1.25
+
+    def dense_pairs_wanted(self, surv: SurvivorList, skip_add: Optional[torch.Tensor]) -> bool:
+        """Untied and per-source decoders at densities the survivor gather was not made for (a ReLU model, JumpReLU
+        thresholds at the start of a training run, a very large k): every active (token, feature) of a source
+        fetches a decoder row per target, k T rows of d elements, while the reference's dense product
+        ``a[s] @ W[s->t].T`` (decoder.py:253-316) costs 2 T F d whatever the density.  With the measured rates of
+        ``route_rates`` the product wins above roughly 1.5 - 2 % of the features active per token."""
+        cfg = self.config
+        if cfg.decoder_tying == "per_target" or not self.dense_route or skip_add is not None:
+            return False
+        if self.feature_offset is not None or self.feature_scale is not None:
+            return False
+        if surv.nnz_hint is None and surv.status is not None:
+            return False                # a threshold list of unknown size (first forward of a shape): the gather
+        T, F, d = surv.T, surv.F, cfg.d_model
+        esize = torch.finfo(surv.dtype).bits // 8
+        if surv.dtype not in (torch.bfloat16, torch.float16, torch.float32) or T < 256 or d < 256 or d % 4 or F % (128 // esize):
+            return False
+        per_layer = self._survivors_per_layer(surv)
+        if per_layer < 0.004 * T * F:
+            return False                # no plausible pair of rates sends so sparse a batch to the product
+        if self.rate_override is None and torch.cuda.is_current_stream_capturing():
+            return False                # (the rates are measured with events on first use: not under a capture)
+        gather_rate, mfma_rate = self.route_rates(T, F, d, surv.dtype)
+        gather_s = per_layer * d * esize / gather_rate
+        return gather_s > self.DENSE_PAIR_MARGIN * 2.0 * T * F * d / mfma_rate
+
+    def _decode_dense_pairs(self, surv: SurvivorList, src_mask: int, t_begin: int, t_end: int, ws) -> torch.Tensor:
+        """Targets [t_begin, t_end) of untied or per-source decoders as the reference's dense products: per source
+        layer the survivors are scattered into a dense [T, F] operand, one launch of the matrix-core kernel
+        multiplies it with the decoders of all its targets (checkpoint layout [d, F], bias included, one rounding
+        per product as ``F.linear`` has), and the products are added per target in source order in the model dtype
+        (decoder.py:283-316: ``reconstruction += decoded``)."""
+        cfg = self.config
+        L, T, F, d = cfg.num_layers, surv.T, surv.F, cfg.d_model
+        dev = surv.row_ptr.device
+        out = torch.zeros((surv.L, T, d), dtype=surv.dtype, device=dev)
+        acc = (ws.typed("dense_sum", (T, F), surv.dtype) if ws is not None
+               else torch.empty((T, F), dtype=surv.dtype, device=dev))
+        decs = self._ordered()
+        first = 0                       # slot of (s, s) in the untied order (s, t) = (0, 0), (0, 1), ..
+        for s in range(min(t_end, L)):
+            row0 = first
+            first += L - s
+            if not (src_mask >> s) & 1:
+                continue
+            lo = max(s, t_begin)
+            if lo >= t_end:
+                continue
+            engine.accumulate_dense(surv, s, acc, True)
+            if cfg.decoder_tying == "none":
+                lins = [decs[row0 + (t - s)] for t in range(lo, t_end)]
+            else:                       # one decoder per source: the same product goes to every target >= s
+                lins = [decs[s]]
+            w = torch.stack([lin.weight.detach() for lin in lins])
+            b = torch.stack([lin.bias_param.detach() for lin in lins])
+            prod = engine.encode(acc.unsqueeze(0).expand(len(lins), T, F), w, b)
+            if cfg.decoder_tying == "none":
+                out[lo:t_end] += prod
+            else:
+                out[lo:t_end] += prod[0]
+        return out
+
     def _decode_dense(self, surv: SurvivorList, src_mask: int, t_first: int, t_end: int, out: torch.Tensor, ws) -> None:
+
         """Targets [t_first, t_end) of decoders tied per target as dense products: the reference's own
         formulation (decoder.py:208-251) - activations summed over the sources in the model dtype, one
         ``F.linear`` with the target's decoder in its checkpoint layout - with the sum built by scattering
@@ -459,6 +529,9 @@ class Decoder(nn.Module):
         """Reconstructions [L, T, d] (rows outside [t_begin, t_end) are not written)."""
         cfg = self.config
         t_end = cfg.num_layers if t_end is None else t_end
+        if self.dense_pairs_wanted(surv, skip_add):
+            self.last_route = {"sparse_targets": (t_begin, t_begin), "dense_targets": (t_begin, t_end)}
+            return self._decode_dense_pairs(surv, src_mask, t_begin, t_end, ws)
         split = self.dense_split(surv, src_mask, t_begin, t_end, skip_add)
         self.last_route = {"sparse_targets": (t_begin, split), "dense_targets": (split, t_end)}
         out = None

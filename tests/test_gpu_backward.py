@@ -603,3 +603,77 @@ def test_threshold_gradient_reduction(dev, dtype, T, F, bandwidth):
     scale = float(want.abs().max())
     assert float((got.cpu() - want).abs().max()) <= 2e-5 * scale + (1e-6 if dtype == torch.float32 else 0.0)
     assert int(near.sum()) > 0
+
+
+@pytest.mark.parametrize("tying", ["none", "per_source"])
+@pytest.mark.parametrize("case", ["relu", "jumprelu-low-thresholds", "batchtopk-large-k"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_gradients_on_the_dense_route_at_high_density(dev, dtype, case, tying):
+    """Far above the densities the survivor-list kernels are made for, forward and gradients take the reference's
+    dense formulation on the matrix-core kernel (Decoder.dense_pairs_wanted).  Loss and every gradient against
+    autograd through the oracle; one optimisation step equal to the step taken from the same gradients."""
+    tdt = getattr(torch, dtype)
+    fn = {"relu": "relu", "jumprelu-low-thresholds": "jumprelu", "batchtopk-large-k": "batchtopk"}[case]
+    wl = BASE.scaled("dense-bw", num_layers=3, d_model=256, num_features=512, tokens=320, dtype=dtype, activation_fn=fn,
+                     k=200 if fn == "batchtopk" else None, decoder_tying=tying)
+    import crosslayer_coding_amd as cca
+    x = synth.make_inputs(wl, "cpu")
+    sd = synth.make_state_dict(wl, "cpu", inputs=x)
+    g = torch.Generator().manual_seed(5)
+    for k in list(sd):
+        if k.endswith("bias_param"):
+            sd[k] = (torch.randn(sd[k].shape, generator=g) * 0.05).to(sd[k].dtype)
+            if case == "jumprelu-low-thresholds" and "encoder" in k:
+                sd[k] = sd[k] + 2.0
+    L = wl.num_layers
+    tg = torch.Generator().manual_seed(6)
+    targets = {l: torch.randn(wl.tokens, wl.d_model, generator=tg).to(tdt) for l in range(L)}
+
+    def fresh():
+        m = cca.CrossLayerTranscoder(wl.config(), None, dev)
+        m.load_state_dict(sd)
+        m.decoder_module.rate_override = (14.5e12, 1.0e14 if tdt == torch.float32 else 1.0e15)
+        return m
+
+    model = fresh()
+    inputs = {l: x[l].to(dev) for l in range(L)}
+    tdev = {l: t.to(dev) for l, t in targets.items()}
+    loss, grads = model.loss_and_gradients(inputs, tdev)
+    assert model.decoder_module.last_route["dense_targets"] == (0, L)
+    acts = model.get_feature_activations(inputs)
+    assert float((acts[0] != 0).float().mean()) > 0.2
+    masks, theta, log_theta = None, None, None
+    if fn == "jumprelu":
+        theta = torch.exp(sd["theta_manager.log_threshold"].float()).to(tdt)
+        log_theta = sd["theta_manager.log_threshold"]
+    else:
+        masks = {l: (a != 0).cpu() for l, a in acts.items()}
+    names = synth.decoder_names(wl)
+    ref_loss, ref = orc.mse_loss_and_gradients(
+        {l: x[l] for l in range(L)}, targets,
+        enc_w=[sd[f"encoder_module.encoders.{l}.weight"] for l in range(L)],
+        enc_b=[sd[f"encoder_module.encoders.{l}.bias_param"] for l in range(L)],
+        dec_w={n: sd[f"decoder_module.decoders.{n}.weight"] for n in names},
+        dec_b={n: sd[f"decoder_module.decoders.{n}.bias_param"] for n in names},
+        activation_fn=fn, num_layers=L, k=wl.k, theta=theta, masks=masks, tying=tying, log_threshold=log_theta,
+        model_dtype=tdt)
+    tol = TOL[tdt]
+    assert abs(float(loss) - float(ref_loss)) <= max(tol, 1e-6) * abs(float(ref_loss)) * 10
+    for name, gref in ref.items():
+        err = orc.rel_l2(grads[name].float().cpu(), gref)
+        bound = tol * (5 if tdt == torch.bfloat16 else 1)
+        if name.endswith("log_threshold"):
+            bound = 1e-3 if tdt == torch.float32 else 1e-1
+        assert err <= bound, (name, err)
+    # the same route under training_step (an optimiser that would otherwise fuse the decoder step) == stepping on
+    # the gradients just checked
+    a, b = fresh(), fresh()
+    oa, ob = cca.CLTAdam(a, lr=1e-3), cca.CLTAdam(b, lr=1e-3)
+    ob.fuse_decoder_step = False
+    la = a.training_step(inputs, tdev, oa)
+    lb = b.training_step(inputs, tdev, ob)
+    assert float(la) == float(lb)
+    sa, sb = a.state_dict(), b.state_dict()
+    for k in sa:
+        assert torch.equal(sa[k], sb[k]), k
+    assert not torch.equal(sa["encoder_module.encoders.0.weight"].cpu(), sd["encoder_module.encoders.0.weight"])

@@ -146,3 +146,57 @@ def test_route_query_names_the_schedules(dev):
     assert engine.decode_route(16, 768, 24576, 12, "none", torch.bfloat16, rows=16) == nat.ROUTE_QUARTER
     assert engine.decode_route(16, 768, 2048, 4, "none", torch.bfloat16, rows=16) == nat.ROUTE_SINGLE
     assert engine.decode_route(4096, 100, 24576, 12, "none", torch.bfloat16, rows=big) == nat.ROUTE_GENERIC
+
+
+@pytest.mark.parametrize("tying", ["none", "per_source"])
+@pytest.mark.parametrize("case", ["relu", "jumprelu-low-thresholds", "batchtopk-large-k"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_dense_pair_route_at_high_density(dev, dtype, case, tying):
+    """Untied and per-source decoders at densities far above what the gather is made for: the decode takes the
+    reference's dense products (clt/models/decoder.py:253-338) on the matrix-core kernel; result against the oracle
+    and against the gather route of the same model."""
+    tdt = getattr(torch, dtype)
+    fn = {"relu": "relu", "jumprelu-low-thresholds": "jumprelu", "batchtopk-large-k": "batchtopk"}[case]
+    wl = synth.Workload("dense-pairs", 8, 3, 256, 512, 600, dtype, activation_fn=fn, k=200 if fn == "batchtopk" else None,
+                        decoder_tying=tying)
+    x = synth.make_inputs(wl, "cpu")
+    sd = synth.make_state_dict(wl, "cpu", inputs=x)
+    g = torch.Generator().manual_seed(3)
+    for key in list(sd):
+        if key.endswith("bias_param") and "decoder" in key:
+            sd[key] = (torch.randn(sd[key].shape, generator=g) * 0.1).to(tdt)
+        if case == "jumprelu-low-thresholds" and key.endswith("bias_param") and "encoder" in key:
+            sd[key] = sd[key] + 2.0            # most pre-activations pass their thresholds
+    model = cca.CrossLayerTranscoder(wl.config(), None, dev)
+    model.load_state_dict(sd)
+    L, F, d = wl.num_layers, wl.num_features, wl.d_model
+    inputs = {l: x[l].to(dev) for l in range(L)}
+    # rates of a large shape: at this size the measured ones may keep the gather
+    model.decoder_module.rate_override = (14.5e12, 1.0e14 if tdt == torch.float32 else 1.0e15)
+    with torch.no_grad():
+        model(inputs)                            # threshold activations: the density is known from the second forward on
+        torch.cuda.synchronize()
+        model(inputs)
+        torch.cuda.synchronize()
+        dense = model(inputs)
+        assert model.decoder_module.last_route["dense_targets"] == (0, L), model.decoder_module.last_route
+        model.decoder_module.dense_route = False
+        sparse = model(inputs)
+        assert model.decoder_module.last_route["dense_targets"] == (L, L)
+        acts = {l: a.cpu() for l, a in model.get_feature_activations(inputs).items()}
+        assert float((acts[0] != 0).float().mean()) > 0.2
+        # a subset of layers
+        model.decoder_module.dense_route = True
+        part = model({l: inputs[l] for l in (0, 2)})
+        model.decoder_module.dense_route = False
+        want = model({l: inputs[l] for l in (0, 2)})
+    names = synth.decoder_names(wl)
+    for t in range(L):
+        ref = orc.decode(acts, t, tying=tying, weights={n: sd[f"decoder_module.decoders.{n}.weight"] for n in names},
+                         biases={n: sd[f"decoder_module.decoders.{n}.bias_param"] for n in names}, d_model=d,
+                         num_features=F, dtype=tdt)
+        assert orc.rel_l2(dense[t].cpu(), ref) <= TOL[tdt], (t, "dense")
+        assert orc.rel_l2(sparse[t].cpu(), ref) <= TOL[tdt], (t, "gather")
+    assert sorted(part) == [0, 2]
+    for t in part:
+        assert orc.rel_l2(part[t].float().cpu(), want[t].float().cpu()) <= TOL[tdt]

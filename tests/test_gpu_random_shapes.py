@@ -60,9 +60,10 @@ def test_random_shapes_stage_by_stage(dev, seed):
             model.fuse_encode_select = False
             r2, a2 = model(inputs), model.get_feature_activations(inputs)
             pre, _ = model._encode_all_layers(inputs)
-        # a decoder tied per target moves between the gather and the dense product with the density seen so far,
-        # so two calls may differ in the last bit there
-        route_may_move = wl.decoder_tying == "per_target" and wl.activation_fn in ("relu", "jumprelu")
+        # under a threshold activation the decode moves between the gather and dense products with the density seen
+        # so far (always possible for decoders tied per target, at high densities for the others), so two calls
+        # may differ in the last bits there
+        route_may_move = wl.activation_fn in ("relu", "jumprelu")
         for l in layers:
             assert torch.equal(a1[l], a2[l]), tag
         for t in r1:
