@@ -50,6 +50,7 @@ _SIGNATURES = {
     "clt_threshold_count": (_int, [_vp, _i64, _i64, _i64, _i64, _vp, _int, _int, _vp, _vp, _sz, _vp]),
     "clt_threshold_count_static": (_int, [_vp, _i64, _i64, _i64, _i64, _vp, _int, _int, _vp, _vp]),
     "clt_threshold_emit": (_int, [_vp, _i64, _i64, _i64, _i64, _vp, _int, _int, _vp, _vp, _vp, _vp, _vp]),
+    "clt_threshold_dense": (_int, [_vp, _i64, _i64, _i64, _i64, _vp, _int, _int, _vp, _vp]),
     "clt_survivors_fit": (_int, [_vp, _i64, _i64, _vp, _vp]),
     "clt_encode_threshold_supported": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _int]),
     "clt_encode_threshold_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64, _i64, _int]),

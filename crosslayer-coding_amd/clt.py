@@ -770,6 +770,52 @@ class CrossLayerTranscoder(BaseTranscoder):
             engine.poison_if(out, full.status)
         return {t: out[t] for t in targets}, full
 
+    def _forward_dense_thresholds(self, inputs: Dict[int, torch.Tensor]) -> Optional[Dict[int, torch.Tensor]]:
+        """The forward of a JumpReLU / ReLU model whose recent batches were dense enough for the decode to run as
+        dense products (``Decoder.dense_pairs_wanted_for`` on the survivor total last seen for this shape): no
+        survivor list is made at all - the pre-activations are stored, gated in place (``clt_threshold_dense``) and
+        multiplied as they are; the number kept travels to the host behind the kernels like the list totals do,
+        so the route follows the density back down.  None: the list route is the one to take."""
+        cfg = self.config
+        fn = cfg.activation_fn
+        if fn not in ("jumprelu", "relu") or cfg.skip_connection or torch.cuda.is_current_stream_capturing():
+            return None
+        if self._thr_last_total is None or not inputs:
+            return None
+        prep = self.encoder_module.prepare_slab(inputs)
+        if prep is None:
+            return None
+        layers, x_slab, w_slab, b_slab = prep
+        n, T, F = len(layers), x_slab.shape[1], cfg.num_features
+        key = (fn, tuple(layers), T, self.dtype)
+        if key != self._thr_key:
+            return None
+        self._poll_threshold_runs()
+        dec = self.decoder_module
+        if not dec.dense_pairs_wanted_for(self._thr_last_total / n, T, self.dtype, None):
+            return None
+        ws = self._workspace()
+        pre = engine.encode(x_slab, w_slab, b_slab, out=ws.typed("pre", (n, T, F), self.dtype))
+        theta = None
+        if fn == "jumprelu":
+            theta = self.theta_manager.thresholds(self.dtype)
+            if layers != list(range(cfg.num_layers)):
+                theta = theta.index_select(0, torch.tensor(layers, device=theta.device)).contiguous()
+        total = engine.threshold_dense(pre, theta, nat.PRED_GE_THETA if fn == "jumprelu" else nat.PRED_GT_ZERO)
+        host = torch.empty(1, dtype=torch.int64, pin_memory=True)
+        host.copy_(total, non_blocking=True)
+        ev = torch.cuda.Event()
+        ev.record()
+        self._thr_pending.append((host, ev, key))
+        src_mask = 0
+        for l in layers:
+            src_mask |= 1 << l
+        out = dec._decode_dense_pairs(None, src_mask, min(layers), max(layers) + 1, ws,
+                                      dense={l: pre[i] for i, l in enumerate(layers)})
+        dec.last_route = {"sparse_targets": (min(layers), min(layers)), "dense_targets": (min(layers), max(layers) + 1),
+                          "survivor_list": False}
+        return {t: out[t] for t in layers}
+
     def _note_no_graph(self, what: str) -> None:
         """Say once per model that ``what`` returns tensors outside the autograd graph although gradients are on:
         a loss term built on them (the reference's sparsity / pre-activation penalties, losses.py:94-328) would
@@ -810,6 +856,9 @@ class CrossLayerTranscoder(BaseTranscoder):
                     self._warned_no_graph = True
                     logger.warning(f"Rank {self.rank}: forward builds no autograd graph for these inputs (it needs one "
                                    f"2-D or 3-D tensor per layer with equal token counts); gradients will not flow.")
+        dense = self._forward_dense_thresholds(inputs)
+        if dense is not None:
+            return dense
         res = self.forward_with_survivors(inputs)
         if res is not None:
             return res[0]

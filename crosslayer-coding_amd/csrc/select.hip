@@ -1849,6 +1849,82 @@ extern "C" int clt_threshold_count(const void *pre, int64_t T, int64_t F, int64_
   return dispatch_threshold<float>(false, pre, T, F, L, pre_layer_stride, theta, pred, cnt, row_ptr, nullptr, nullptr, nullptr, s);
 }
 
+// ---- threshold activation kept dense ----------------------------------------------------------------------
+// x[l][t][f] <- x if the predicate holds, else 0, in place; total += the number kept.  One 16-byte piece per
+// thread and step where rows are whole pieces, else element by element.
+template <typename T, int PRED, bool VEC>
+__global__ __launch_bounds__(256) void k_threshold_dense(T *__restrict__ x, const T *__restrict__ theta, int64_t Tn, int64_t F,
+                                                         int64_t lstride, unsigned long long *__restrict__ total) {
+  constexpr int V = VEC ? 16 / (int)sizeof(T) : 1;
+  const int l = blockIdx.y;
+  T *xl = x + (int64_t)l * lstride;
+  const T *th = PRED == CLT_PRED_GE_THETA ? theta + (int64_t)l * F : nullptr;
+  const int64_t per_row = F / V, n = Tn * per_row;
+  uint32_t kept = 0;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t r = i / per_row, c = (i - r * per_row) * V;
+    T *p = xl + r * F + c;
+    if constexpr (VEC) {
+      uint4 v = *reinterpret_cast<const uint4 *>(p), t4 = make_uint4(0, 0, 0, 0);
+      if (PRED == CLT_PRED_GE_THETA) t4 = *reinterpret_cast<const uint4 *>(th + c);
+      uint32_t w[4] = {v.x, v.y, v.z, v.w};
+      const uint32_t tw[4] = {t4.x, t4.y, t4.z, t4.w};
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        if constexpr (sizeof(T) == 4) {
+          const bool keep = pred_keep<T, PRED>(__uint_as_float(w[k]), __uint_as_float(tw[k]));
+          kept += keep ? 1u : 0u;
+          w[k] = keep ? w[k] : 0u;
+        } else {
+          float xa, xb, ta, tb;
+          unpack_pair<T>(w[k], xa, xb);
+          unpack_pair<T>(tw[k], ta, tb);
+          const bool ka = pred_keep<T, PRED>(xa, ta), kb = pred_keep<T, PRED>(xb, tb);
+          kept += (ka ? 1u : 0u) + (kb ? 1u : 0u);
+          w[k] &= (ka ? 0x0000FFFFu : 0u) | (kb ? 0xFFFF0000u : 0u);
+        }
+      }
+      *reinterpret_cast<uint4 *>(p) = make_uint4(w[0], w[1], w[2], w[3]);
+    } else {
+      const float xv = Elem<T>::to_f32(*p);
+      const bool keep = pred_keep<T, PRED>(xv, PRED == CLT_PRED_GE_THETA ? Elem<T>::to_f32(th[c]) : 0.0f);
+      kept += keep ? 1u : 0u;
+      if (!keep) *p = Elem<T>::from_raw(0u);
+    }
+  }
+  __shared__ uint32_t red[4];
+  for (int o = 32; o > 0; o >>= 1) kept += __shfl_xor(kept, o);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = kept;
+  __syncthreads();
+  if (threadIdx.x == 0) atomicAdd(total, (unsigned long long)red[0] + red[1] + red[2] + red[3]);
+}
+
+extern "C" int clt_threshold_dense(void *x, int64_t T, int64_t F, int64_t L, int64_t layer_stride, const void *theta,
+                                   int pred, int dtype, uint64_t *total, void *stream) {
+  if (!clt_model_dtype(dtype)) return CLT_ERR_DTYPE;
+  if (T < 0 || F < 0 || L <= 0 || L > 65535 || !total) return CLT_ERR_ARG;
+  if ((pred != CLT_PRED_GE_THETA && pred != CLT_PRED_GT_ZERO) || (pred == CLT_PRED_GE_THETA && !theta)) return CLT_ERR_ARG;
+  hipStream_t s = (hipStream_t)stream;
+  k_fill_u32<<<1, 64, 0, s>>>((uint32_t *)total, 0u, 2);
+  if (T == 0 || F == 0) return clt_check_launch();
+  if (!x) return CLT_ERR_ARG;
+  const int esz = clt_elem_bytes(dtype), vec = 16 / esz;
+  const bool vecok = F % vec == 0 && clt_aligned16(x) && (layer_stride * esz) % 16 == 0 && (!theta || clt_aligned16(theta));
+  dim3 grid(2048, (unsigned)L);
+#define CLT_TD(CT, P, VK) k_threshold_dense<CT, P, VK><<<grid, 256, 0, s>>>((CT *)x, (const CT *)theta, T, F, layer_stride, (unsigned long long *)total)
+#define CLT_TD_T(CT)                                                                            \
+  do {                                                                                          \
+    if (pred == CLT_PRED_GE_THETA) { if (vecok) CLT_TD(CT, CLT_PRED_GE_THETA, true); else CLT_TD(CT, CLT_PRED_GE_THETA, false); } \
+    else { if (vecok) CLT_TD(CT, CLT_PRED_GT_ZERO, true); else CLT_TD(CT, CLT_PRED_GT_ZERO, false); }                             \
+  } while (0)
+  if (dtype == CLT_BF16) CLT_TD_T(bf16_t);
+  else if (dtype == CLT_F16) CLT_TD_T(f16_t);
+  else CLT_TD_T(float);
+#undef CLT_TD_T
+#undef CLT_TD
+  return clt_check_launch();
+}
+
 // ---- sizing col / val without reading the total back -------------------------------------------------
 __global__ void k_survivors_fit_flag(const int32_t *row_ptr, int64_t R, int64_t capacity, int32_t *status) {
   if (threadIdx.x == 0 && blockIdx.x == 0) {

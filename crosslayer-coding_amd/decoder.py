@@ -338,12 +338,14 @@ class Decoder(nn.Module):
     _rate_cache: Dict[tuple, Tuple[float, float]] = {}
     rate_override: Optional[Tuple[float, float]] = None     # (gather bytes / s, MFMA flop / s): tests and experiments
 
-    def route_rates(self, T: int, F: int, d: int, dtype: torch.dtype) -> Tuple[float, float]:
-        """(bytes / s of decoder rows the row gather delivers, flop / s of the dense product [T, F] x [F, d])."""
+    def route_rates(self, T: int, F: int, d: int, dtype: torch.dtype, batch: int = 1) -> Tuple[float, float]:
+        """(bytes / s of decoder rows the row gather delivers, flop / s of the dense product [T, F] x [F, d]);
+        ``batch``: that many products with one left operand in one launch, as the dense route of untied decoders
+        runs them (a single product of few tiles leaves most compute units idle)."""
         if self.rate_override is not None:
             return self.rate_override
         dev = self._ordered()[0].weight.device
-        key = (dev.index, T, F, d, dtype)
+        key = (dev.index, T, F, d, dtype, batch)
         hit = Decoder._rate_cache.get(key)
         if hit is not None:
             return hit
@@ -362,10 +364,10 @@ class Decoder(nn.Module):
 
         esize = torch.finfo(dtype).bits // 8
         # the dense product itself, on scratch operands of the real shape
-        x = torch.zeros((1, T, F), dtype=dtype, device=dev)
-        w = torch.zeros((1, d, F), dtype=dtype, device=dev)
-        out = torch.empty((1, T, d), dtype=dtype, device=dev)
-        mfma = 2.0 * T * F * d / best_of(lambda: engine.encode(x, w, None, out=out))
+        x = torch.zeros((1, T, F), dtype=dtype, device=dev).expand(batch, T, F)
+        w = torch.zeros((batch, d, F), dtype=dtype, device=dev)
+        out = torch.empty((batch, T, d), dtype=dtype, device=dev)
+        mfma = 2.0 * T * F * d * batch / best_of(lambda: engine.encode(x, w, None, out=out))
         del x, w, out
         # a bare gather of rows of this width from 4 MB (what an XCD's L2 holds of a decoder matrix)
         row_bytes = max(16, min(d * esize, 2048) // 16 * 16)
@@ -433,38 +435,50 @@ class Decoder(nn.Module):
         fetches a decoder row per target, k T rows of d elements, while the reference's dense product
         ``a[s] @ W[s->t].T`` (decoder.py:253-316) costs 2 T F d whatever the density.  With the measured rates of
         ``route_rates`` the product wins above roughly 1.5 - 2 % of the features active per token."""
+        if surv.nnz_hint is None and surv.status is not None:
+            return False                # a threshold list of unknown size (first forward of a shape): the gather
+        return self.dense_pairs_wanted_for(self._survivors_per_layer(surv), surv.T, surv.dtype, skip_add)
+
+    def dense_pairs_wanted_for(self, per_layer: float, T: int, dtype: torch.dtype, skip_add: Optional[torch.Tensor]) -> bool:
+        """``dense_pairs_wanted`` for ``per_layer`` survivors per source layer in a batch of ``T`` tokens."""
         cfg = self.config
         if cfg.decoder_tying == "per_target" or not self.dense_route or skip_add is not None:
             return False
         if self.feature_offset is not None or self.feature_scale is not None:
             return False
-        if surv.nnz_hint is None and surv.status is not None:
-            return False                # a threshold list of unknown size (first forward of a shape): the gather
-        T, F, d = surv.T, surv.F, cfg.d_model
-        esize = torch.finfo(surv.dtype).bits // 8
-        if surv.dtype not in (torch.bfloat16, torch.float16, torch.float32) or T < 256 or d < 256 or d % 4 or F % (128 // esize):
+        F, d = cfg.num_features, cfg.d_model
+        esize = torch.finfo(dtype).bits // 8
+        if dtype not in (torch.bfloat16, torch.float16, torch.float32) or T < 256 or d < 256 or d % 4 or F % (128 // esize):
             return False
-        per_layer = self._survivors_per_layer(surv)
         if per_layer < 0.004 * T * F:
             return False                # no plausible pair of rates sends so sparse a batch to the product
         if self.rate_override is None and torch.cuda.is_current_stream_capturing():
             return False                # (the rates are measured with events on first use: not under a capture)
-        gather_rate, mfma_rate = self.route_rates(T, F, d, surv.dtype)
+        # a launch of the dense route multiplies a source with all its targets, (L + 1) / 2 of them on average
+        batch = max(1, (cfg.num_layers + 1) // 2) if cfg.decoder_tying == "none" else 1
+        gather_rate, mfma_rate = self.route_rates(T, F, d, dtype, batch)
         gather_s = per_layer * d * esize / gather_rate
         return gather_s > self.DENSE_PAIR_MARGIN * 2.0 * T * F * d / mfma_rate
 
-    def _decode_dense_pairs(self, surv: SurvivorList, src_mask: int, t_begin: int, t_end: int, ws) -> torch.Tensor:
+    def _decode_dense_pairs(self, surv: Optional[SurvivorList], src_mask: int, t_begin: int, t_end: int, ws,
+                            dense: Optional[Dict[int, torch.Tensor]] = None) -> torch.Tensor:
         """Targets [t_begin, t_end) of untied or per-source decoders as the reference's dense products: per source
         layer the survivors are scattered into a dense [T, F] operand, one launch of the matrix-core kernel
         multiplies it with the decoders of all its targets (checkpoint layout [d, F], bias included, one rounding
         per product as ``F.linear`` has), and the products are added per target in source order in the model dtype
-        (decoder.py:283-316: ``reconstruction += decoded``)."""
+        (decoder.py:283-316: ``reconstruction += decoded``).  ``dense`` {source layer: [T, F] activations}: operands
+        that are dense already (``clt_threshold_dense``) instead of a survivor list."""
         cfg = self.config
-        L, T, F, d = cfg.num_layers, surv.T, surv.F, cfg.d_model
-        dev = surv.row_ptr.device
-        out = torch.zeros((surv.L, T, d), dtype=surv.dtype, device=dev)
-        acc = (ws.typed("dense_sum", (T, F), surv.dtype) if ws is not None
-               else torch.empty((T, F), dtype=surv.dtype, device=dev))
+        L, F, d = cfg.num_layers, cfg.num_features, cfg.d_model
+        if dense is not None:
+            some = next(iter(dense.values()))
+            T, dtype, dev = some.shape[0], some.dtype, some.device
+            acc = None
+        else:
+            T, dtype, dev = surv.T, surv.dtype, surv.row_ptr.device
+            acc = (ws.typed("dense_sum", (T, F), dtype) if ws is not None
+                   else torch.empty((T, F), dtype=dtype, device=dev))
+        out = torch.zeros((L, T, d), dtype=dtype, device=dev)
         decs = self._ordered()
         first = 0                       # slot of (s, s) in the untied order (s, t) = (0, 0), (0, 1), ..
         for s in range(min(t_end, L)):
@@ -475,7 +489,10 @@ class Decoder(nn.Module):
             lo = max(s, t_begin)
             if lo >= t_end:
                 continue
-            engine.accumulate_dense(surv, s, acc, True)
+            if dense is not None:
+                acc = dense[s]
+            else:
+                engine.accumulate_dense(surv, s, acc, True)
             if cfg.decoder_tying == "none":
                 lins = [decs[row0 + (t - s)] for t in range(lo, t_end)]
             else:                       # one decoder per source: the same product goes to every target >= s

@@ -374,6 +374,20 @@ def _read_total(row_ptr: torch.Tensor) -> int:
     return total
 
 
+def threshold_dense(pre: torch.Tensor, theta: Optional[torch.Tensor], pred: int) -> torch.Tensor:
+    """``pre`` [L, T, F] gated in place - x where the predicate holds, else 0 (activations.py:177-180,
+    registry.py:30-33) - and the number of elements kept, as a one-element int64 tensor on the device."""
+    L, T, F = _check_pre(pre)
+    nat.require_device(pre, "threshold_dense")
+    if theta is not None:
+        assert theta.shape == (L, F) and theta.dtype == pre.dtype and theta.is_contiguous()
+    total = torch.empty(1, dtype=torch.int64, device=pre.device)
+    code = nat.load().clt_threshold_dense(nat.ptr(pre), T, F, L, pre.stride(0), nat.ptr(theta), int(pred),
+                                          nat.dtype_code(pre.dtype), nat.ptr(total), _stream(pre))
+    nat.check(code, "clt_threshold_dense")
+    return total
+
+
 def threshold_select(pre: torch.Tensor, theta: Optional[torch.Tensor], pred: int,
                      ws: Optional[Workspace] = None, read_back: bool = True) -> SurvivorList:
     """JumpReLU (x >= theta), ReLU (x > 0) or non-zero compaction of pre [L, T, F].

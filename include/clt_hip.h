@@ -253,6 +253,18 @@ int clt_threshold_emit(const void *pre, int64_t T, int64_t F, int64_t L,
                        const int32_t *skip, void *stream);
 
 /*
+ * The same activations kept dense, for densities at which a survivor list is the larger object
+ * (a ReLU model, JumpReLU thresholds at the start of a training run): x [L][T][F] is gated in
+ * place - x where the predicate holds (CLT_PRED_GE_THETA or CLT_PRED_GT_ZERO), else 0 - and
+ * *total (device memory) receives the number of elements kept.  The result is the dense
+ * activation tensor the reference itself works on (clt/models/activations.py:177-180,
+ * clt/activations/registry.py:30-33 as called from clt/models/clt.py:271-277), ready for the
+ * dense decode products.
+ */
+int clt_threshold_dense(void *x, int64_t T, int64_t F, int64_t L, int64_t layer_stride,
+                        const void *theta, int pred, int dtype, uint64_t *total, void *stream);
+
+/*
  * For callers that do not read the survivor total back between a count call and its emit call (no
  * host synchronisation in the forward).  Such a caller gives col / val a capacity that no batch it can
  * represent exceeds - min(L*T*F, 2^31 - 1) entries, the most an int32 row pointer addresses - and runs

@@ -180,6 +180,8 @@ def test_dense_pair_route_at_high_density(dev, dtype, case, tying):
         torch.cuda.synchronize()
         dense = model(inputs)
         assert model.decoder_module.last_route["dense_targets"] == (0, L), model.decoder_module.last_route
+        # threshold activations make no survivor list at all on this route
+        assert model.decoder_module.last_route.get("survivor_list", True) == (fn == "batchtopk")
         model.decoder_module.dense_route = False
         sparse = model(inputs)
         assert model.decoder_module.last_route["dense_targets"] == (L, L)
@@ -200,3 +202,23 @@ def test_dense_pair_route_at_high_density(dev, dtype, case, tying):
     assert sorted(part) == [0, 2]
     for t in part:
         assert orc.rel_l2(part[t].float().cpu(), want[t].float().cpu()) <= TOL[tdt]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("L,T,F", [(2, 300, 520), (1, 77, 250), (3, 64, 1024)], ids=["vector", "element-wise", "vector-small"])
+def test_threshold_dense_gates_in_place_and_counts(dev, dtype, L, T, F):
+    """clt_threshold_dense against the reference's expressions (clt/models/activations.py:177-180 for JumpReLU, F.relu
+    for ReLU): the tensor keeps x where the predicate holds and 0 elsewhere, and the count is the number kept."""
+    g = torch.Generator().manual_seed(L * 100 + T + F)
+    x = torch.randn(L, T, F, generator=g).to(dtype)
+    x[0, 0, :4] = torch.tensor([0.0, -0.0, float("inf"), float("-inf")]).to(dtype)
+    theta = torch.exp(0.5 * torch.randn(L, F, generator=g) - 0.5).to(dtype)
+    theta[0, 0] = 0.0
+    for pred, th in ((nat.PRED_GE_THETA, theta), (nat.PRED_GT_ZERO, None)):
+        buf = x.clone().to(dev)
+        total = engine.threshold_dense(buf, th.to(dev) if th is not None else None, pred)
+        keep = (x >= theta.unsqueeze(1)) if th is not None else (x > 0)
+        want = torch.where(keep, x, torch.zeros_like(x))
+        iv = torch.int32 if dtype == torch.float32 else torch.int16
+        assert torch.equal(buf.cpu().view(iv), want.view(iv))
+        assert int(total) == int(keep.sum())
