@@ -265,6 +265,20 @@ class CrossLayerTranscoder(BaseTranscoder):
         L, d, F = cfg.num_layers, cfg.d_model, cfg.num_features
         if sorted(inputs) != list(range(L)) or sorted(targets) != list(range(L)):
             raise ValueError("loss_and_gradients needs inputs and targets for every layer")
+        dense = None
+        if self.decoder_module.skip_weights is None:
+            dense = self._dense_threshold_activations(inputs, "dense_acts")
+        if dense is not None:
+            # a threshold model in the dense regime: no survivor list, forward and gradients on dense operands
+            acts = dense[1]
+            ws = self._workspace()
+            dec = self.decoder_module
+            rec = dec._decode_dense_pairs(None, (1 << L) - 1, 0, L, ws, dense={l: acts[l] for l in range(L)})
+            dec.last_route = {"sparse_targets": (0, 0), "dense_targets": (0, L), "survivor_list": False}
+            tgt = torch.stack([targets[l].to(device=self.device, dtype=self.dtype).reshape(-1, d) for l in range(L)])
+            mode, mean, std, scale = self._denorm_args(normalization_method, mean_tg, std_tg)
+            loss_l, g, g_model, bias_grad = engine.mse_loss_grad(rec, tgt.contiguous(), ws, mode, mean, std, scale)
+            return loss_l, self._raw_gradients_dense(inputs, None, g, g_model, bias_grad, acts=acts)
         res = self._survivors(inputs)
         if res is None:
             raise ValueError("inputs do not form one [layers, tokens, d_model] batch")
@@ -383,17 +397,19 @@ class CrossLayerTranscoder(BaseTranscoder):
         return engine.encode(stacked_g.contiguous(), stacked_w.contiguous(), None)[0]  # [T, F]
 
     def _raw_gradients_dense(self, inputs: Dict[int, torch.Tensor], surv, g: torch.Tensor, g_model: torch.Tensor,
-                             bias_grad: torch.Tensor):
+                             bias_grad: torch.Tensor, acts: Optional[torch.Tensor] = None):
         """The raw gradients of ``_raw_gradients_from`` at densities the survivor-list kernels were not made for
         (``Decoder.dense_pairs_wanted``: untied or per-source decoders, no skip, no feature affine): autograd's own
         dense formulation behind the reference's dense forward, every product on the MFMA kernel -
         d loss / d activation per source (``_dense_activation_gradient``), gated by list membership (the
         straight-through rule of BatchTopK / TokenTopK, ``input >= threshold`` of JumpReLU, activations.py:68-96,
         192-194), ``dW_enc = dpre.T @ x``, ``dW_dec[s->t] = a[s].T @ g[t]``.  Products are rounded to the model
-        dtype like the reference's autograd results, then kept in fp32."""
+        dtype like the reference's autograd results, then kept in fp32.  ``acts`` [L, T, F]: dense activations of a
+        threshold model in place of a survivor list (every kept element is non-zero there - it passed a positive
+        threshold - so membership is ``acts != 0``)."""
         cfg = self.config
         L, d, F, tying = cfg.num_layers, cfg.d_model, cfg.num_features, cfg.decoder_tying
-        T = surv.T
+        T = surv.T if acts is None else acts.shape[1]
         ws = self._workspace()
         dec = self.decoder_module
         packed = dec.packed()
@@ -411,8 +427,10 @@ class CrossLayerTranscoder(BaseTranscoder):
         else:
             g_t = g_model
         g_t = g_t.transpose(1, 2).contiguous()                                 # [L, d, T]: K = tokens
-        member = SurvivorList(surv.row_ptr, surv.col, torch.ones_like(surv.val), surv.T, surv.F, surv.L, surv.dtype,
-                              surv.status, surv.nnz_hint)
+        member = None
+        if acts is None:
+            member = SurvivorList(surv.row_ptr, surv.col, torch.ones_like(surv.val), surv.T, surv.F, surv.L, surv.dtype,
+                                  surv.status, surv.nnz_hint)
         theta = pre = theta_out = None
         if cfg.activation_fn == "jumprelu" and self.theta_manager.log_threshold is not None:
             w, b = self.encoder_module.stacked()
@@ -420,20 +438,24 @@ class CrossLayerTranscoder(BaseTranscoder):
             theta = self.theta_manager.thresholds(self.dtype)
             theta_out = torch.empty((L, F), dtype=torch.float32, device=dev)
         dact_buf = ws.typed("theta_dact", (T, F), self.dtype)
-        a_buf = ws.typed("dense_sum", (T, F), self.dtype)
-        m_buf = ws.typed("dense_member", (T, F), self.dtype)
+        a_buf = ws.typed("dense_sum", (T, F), self.dtype) if acts is None else None
+        m_buf = ws.typed("dense_member", (T, F), self.dtype) if acts is None else None
         row0 = 0
         for s_ in range(L):
             dact = self._dense_activation_gradient(s_, g_model, packed, dact_buf)
             if theta_out is not None:
                 engine.jumprelu_theta_grad(pre[s_], dact, theta[s_].contiguous(), self.theta_manager.bandwidth, theta_out[s_], ws)
-            engine.accumulate_dense(member, s_, m_buf, True)
-            dpre = dact * m_buf
+            if acts is None:
+                engine.accumulate_dense(member, s_, m_buf, True)
+                dpre = dact * m_buf
+            else:
+                dpre = dact * (acts[s_] != 0)
             db_enc[s_] = dpre.sum(0, dtype=torch.float32)
             dw_enc[s_] = engine.encode(dpre.t().contiguous().unsqueeze(0), x_slab[s_].t().contiguous().unsqueeze(0), None)[0]
             del dpre
-            engine.accumulate_dense(surv, s_, a_buf, True)
-            a_t = a_buf.t().contiguous()                                       # [F, T]
+            if acts is None:
+                engine.accumulate_dense(surv, s_, a_buf, True)
+            a_t = (a_buf if acts is None else acts[s_]).t().contiguous()       # [F, T]
             if tying == "none":
                 n = L - s_
                 dw_dec[row0:row0 + n] = engine.encode(a_t.unsqueeze(0).expand(n, F, T), g_t[s_:], None)
@@ -770,12 +792,9 @@ class CrossLayerTranscoder(BaseTranscoder):
             engine.poison_if(out, full.status)
         return {t: out[t] for t in targets}, full
 
-    def _forward_dense_thresholds(self, inputs: Dict[int, torch.Tensor]) -> Optional[Dict[int, torch.Tensor]]:
-        """The forward of a JumpReLU / ReLU model whose recent batches were dense enough for the decode to run as
-        dense products (``Decoder.dense_pairs_wanted_for`` on the survivor total last seen for this shape): no
-        survivor list is made at all - the pre-activations are stored, gated in place (``clt_threshold_dense``) and
-        multiplied as they are; the number kept travels to the host behind the kernels like the list totals do,
-        so the route follows the density back down.  None: the list route is the one to take."""
+    def _dense_threshold_activations(self, inputs: Dict[int, torch.Tensor], buffer: str):
+        """(layers, dense activations [n, T, F] in workspace buffer ``buffer``) of a JumpReLU / ReLU model when the
+        survivor total last seen for this shape sends the decode to its dense products, else None."""
         cfg = self.config
         fn = cfg.activation_fn
         if fn not in ("jumprelu", "relu") or cfg.skip_connection or torch.cuda.is_current_stream_capturing():
@@ -791,11 +810,9 @@ class CrossLayerTranscoder(BaseTranscoder):
         if key != self._thr_key:
             return None
         self._poll_threshold_runs()
-        dec = self.decoder_module
-        if not dec.dense_pairs_wanted_for(self._thr_last_total / n, T, self.dtype, None):
+        if not self.decoder_module.dense_pairs_wanted_for(self._thr_last_total / n, T, self.dtype, None):
             return None
-        ws = self._workspace()
-        pre = engine.encode(x_slab, w_slab, b_slab, out=ws.typed("pre", (n, T, F), self.dtype))
+        pre = engine.encode(x_slab, w_slab, b_slab, out=self._workspace().typed(buffer, (n, T, F), self.dtype))
         theta = None
         if fn == "jumprelu":
             theta = self.theta_manager.thresholds(self.dtype)
@@ -807,6 +824,20 @@ class CrossLayerTranscoder(BaseTranscoder):
         ev = torch.cuda.Event()
         ev.record()
         self._thr_pending.append((host, ev, key))
+        return layers, pre
+
+    def _forward_dense_thresholds(self, inputs: Dict[int, torch.Tensor]) -> Optional[Dict[int, torch.Tensor]]:
+        """The forward of a JumpReLU / ReLU model whose recent batches were dense enough for the decode to run as
+        dense products (``Decoder.dense_pairs_wanted_for`` on the survivor total last seen for this shape): no
+        survivor list is made at all - the pre-activations are stored, gated in place (``clt_threshold_dense``) and
+        multiplied as they are; the number kept travels to the host behind the kernels like the list totals do,
+        so the route follows the density back down.  None: the list route is the one to take."""
+        got = self._dense_threshold_activations(inputs, "pre")
+        if got is None:
+            return None
+        layers, pre = got
+        dec = self.decoder_module
+        ws = self._workspace()
         src_mask = 0
         for l in layers:
             src_mask |= 1 << l

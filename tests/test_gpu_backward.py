@@ -665,6 +665,13 @@ def test_gradients_on_the_dense_route_at_high_density(dev, dtype, case, tying):
         if name.endswith("log_threshold"):
             bound = 1e-3 if tdt == torch.float32 else 1e-1
         assert err <= bound, (name, err)
+    # threshold activations: once the density of the shape is known no survivor list is made; same gradients
+    torch.cuda.synchronize()
+    loss2, grads2 = model.loss_and_gradients(inputs, tdev)
+    assert model.decoder_module.last_route.get("survivor_list", True) == (fn == "batchtopk")
+    assert float(loss2) == float(loss)
+    for name in grads:
+        assert torch.equal(grads2[name], grads[name]), name
     # the same route under training_step (an optimiser that would otherwise fuse the decoder step) == stepping on
     # the gradients just checked
     a, b = fresh(), fresh()
