@@ -304,7 +304,7 @@ class CrossLayerTranscoder(BaseTranscoder):
         ws = self._workspace()
         mask = (1 << L) - 1
         dec = self.decoder_module
-        if dec.skip_weights is None and dec.dense_pairs_wanted(surv, None):
+        if dec.skip_weights is None and dec.dense_pairs_wanted(surv, None, any_tying=True):
             # so many survivors that the reference's dense products are the cheaper formulation (the decoder step is
             # then not fused: ``dec_w`` is returned and the optimiser applies it)
             return self._raw_gradients_dense(inputs, surv, g, g_model, bias_grad)
@@ -399,7 +399,7 @@ class CrossLayerTranscoder(BaseTranscoder):
     def _raw_gradients_dense(self, inputs: Dict[int, torch.Tensor], surv, g: torch.Tensor, g_model: torch.Tensor,
                              bias_grad: torch.Tensor, acts: Optional[torch.Tensor] = None):
         """The raw gradients of ``_raw_gradients_from`` at densities the survivor-list kernels were not made for
-        (``Decoder.dense_pairs_wanted``: untied or per-source decoders, no skip, no feature affine): autograd's own
+        (``Decoder.dense_pairs_wanted``, any tying; no skip, no feature affine): autograd's own
         dense formulation behind the reference's dense forward, every product on the MFMA kernel -
         d loss / d activation per source (``_dense_activation_gradient``), gated by list membership (the
         straight-through rule of BatchTopK / TokenTopK, ``input >= threshold`` of JumpReLU, activations.py:68-96,
@@ -426,6 +426,7 @@ class CrossLayerTranscoder(BaseTranscoder):
             g_t = torch.flip(torch.cumsum(torch.flip(g, dims=[0]), dim=0), dims=[0]).to(self.dtype)
         else:
             g_t = g_model
+        summed = None       # per-target tying: the running sum of the sources' activations that target s multiplies
         g_t = g_t.transpose(1, 2).contiguous()                                 # [L, d, T]: K = tokens
         member = None
         if acts is None:
@@ -455,7 +456,12 @@ class CrossLayerTranscoder(BaseTranscoder):
             del dpre
             if acts is None:
                 engine.accumulate_dense(surv, s_, a_buf, True)
-            a_t = (a_buf if acts is None else acts[s_]).t().contiguous()       # [F, T]
+            a_s = a_buf if acts is None else acts[s_]
+            if tying == "per_target":
+                # decoder.py:208-246: ``summed_activation += activation_tensor`` in the model dtype, then one product
+                summed = a_s.clone() if summed is None else summed.add_(a_s)
+                a_s = summed
+            a_t = a_s.t().contiguous()                                         # [F, T]
             if tying == "none":
                 n = L - s_
                 dw_dec[row0:row0 + n] = engine.encode(a_t.unsqueeze(0).expand(n, F, T), g_t[s_:], None)
@@ -468,8 +474,10 @@ class CrossLayerTranscoder(BaseTranscoder):
             theta_grad = theta_out * torch.exp(self.theta_manager.log_threshold.detach().float())
         if tying == "none":
             dec_b = bias_grad[torch.tensor([t for s_ in range(L) for t in range(s_, L)], device=bias_grad.device)]
-        else:
+        elif tying == "per_source":
             dec_b = torch.flip(torch.cumsum(torch.flip(bias_grad, dims=[0]), dim=0), dims=[0])
+        else:
+            dec_b = bias_grad
         return {"enc_w": dw_enc, "enc_b": db_enc, "dec_w": dw_dec, "dec_b": dec_b.contiguous(), "theta": theta_grad,
                 "skip": None, "feat_offset": None, "feat_scale": None}
 

@@ -429,7 +429,7 @@ class Decoder(nn.Module):
     # a (source, target) pair goes to the dense product when its gather is priced this many times dearer
     DENSE_PAIR_MARGIN = 1.25
 
-    def dense_pairs_wanted(self, surv: SurvivorList, skip_add: Optional[torch.Tensor]) -> bool:
+    def dense_pairs_wanted(self, surv: SurvivorList, skip_add: Optional[torch.Tensor], any_tying: bool = False) -> bool:
         """Untied and per-source decoders at densities the survivor gather was not made for (a ReLU model, JumpReLU
         thresholds at the start of a training run, a very large k): every active (token, feature) of a source
         fetches a decoder row per target, k T rows of d elements, while the reference's dense product
@@ -437,12 +437,15 @@ class Decoder(nn.Module):
         ``route_rates`` the product wins above roughly 1.5 - 2 % of the features active per token."""
         if surv.nnz_hint is None and surv.status is not None:
             return False                # a threshold list of unknown size (first forward of a shape): the gather
-        return self.dense_pairs_wanted_for(self._survivors_per_layer(surv), surv.T, surv.dtype, skip_add)
+        return self.dense_pairs_wanted_for(self._survivors_per_layer(surv), surv.T, surv.dtype, skip_add, any_tying)
 
-    def dense_pairs_wanted_for(self, per_layer: float, T: int, dtype: torch.dtype, skip_add: Optional[torch.Tensor]) -> bool:
-        """``dense_pairs_wanted`` for ``per_layer`` survivors per source layer in a batch of ``T`` tokens."""
+    def dense_pairs_wanted_for(self, per_layer: float, T: int, dtype: torch.dtype, skip_add: Optional[torch.Tensor],
+                               any_tying: bool = False) -> bool:
+        """``dense_pairs_wanted`` for ``per_layer`` survivors per source layer in a batch of ``T`` tokens.
+        ``any_tying``: decoders tied per target included (their forward has its own rule, ``dense_split``; the
+        gradients ask here)."""
         cfg = self.config
-        if cfg.decoder_tying == "per_target" or not self.dense_route or skip_add is not None:
+        if (cfg.decoder_tying == "per_target" and not any_tying) or not self.dense_route or skip_add is not None:
             return False
         if self.feature_offset is not None or self.feature_scale is not None:
             return False

@@ -605,7 +605,7 @@ def test_threshold_gradient_reduction(dev, dtype, T, F, bandwidth):
     assert int(near.sum()) > 0
 
 
-@pytest.mark.parametrize("tying", ["none", "per_source"])
+@pytest.mark.parametrize("tying", ["none", "per_source", "per_target"])
 @pytest.mark.parametrize("case", ["relu", "jumprelu-low-thresholds", "batchtopk-large-k"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_gradients_on_the_dense_route_at_high_density(dev, dtype, case, tying):
@@ -638,8 +638,13 @@ def test_gradients_on_the_dense_route_at_high_density(dev, dtype, case, tying):
     model = fresh()
     inputs = {l: x[l].to(dev) for l in range(L)}
     tdev = {l: t.to(dev) for l, t in targets.items()}
+    calls = []
+    real = model._raw_gradients_dense
+    model._raw_gradients_dense = lambda *a, **kw: (calls.append(1), real(*a, **kw))[1]
     loss, grads = model.loss_and_gradients(inputs, tdev)
-    assert model.decoder_module.last_route["dense_targets"] == (0, L)
+    assert calls, "the dense gradient route was not taken"
+    if tying != "per_target":       # (decoders tied per target choose target by target in the forward)
+        assert model.decoder_module.last_route["dense_targets"] == (0, L)
     acts = model.get_feature_activations(inputs)
     assert float((acts[0] != 0).float().mean()) > 0.2
     masks, theta, log_theta = None, None, None
@@ -668,7 +673,7 @@ def test_gradients_on_the_dense_route_at_high_density(dev, dtype, case, tying):
     # threshold activations: once the density of the shape is known no survivor list is made; same gradients
     torch.cuda.synchronize()
     loss2, grads2 = model.loss_and_gradients(inputs, tdev)
-    assert model.decoder_module.last_route.get("survivor_list", True) == (fn == "batchtopk")
+    assert model.decoder_module.last_route.get("survivor_list", True) == (fn == "batchtopk" or tying == "per_target")
     assert float(loss2) == float(loss)
     for name in grads:
         assert torch.equal(grads2[name], grads[name]), name
