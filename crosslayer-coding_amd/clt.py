@@ -728,6 +728,13 @@ class CrossLayerTranscoder(BaseTranscoder):
         self._note_no_graph("get_feature_activations")
         cfg = self.config
         topk_family = cfg.activation_fn in ("batchtopk", "topk")
+        got = self._dense_threshold_activations(inputs, "pre")
+        if got is not None:
+            # a threshold model in the dense regime: the gated pre-activations are the answer (fp32 for JumpReLU, as
+            # the reference's ``(x >= theta).float() * x`` is)
+            layers, acts = got
+            dense = acts.float() if cfg.activation_fn == "jumprelu" else acts.clone()
+            return {l: dense[i] for i, l in enumerate(layers)}
         res = self._survivors(inputs)
         if res is not None:
             layers, T, surv = res

@@ -182,10 +182,13 @@ def test_dense_pair_route_at_high_density(dev, dtype, case, tying):
         assert model.decoder_module.last_route["dense_targets"] == (0, L), model.decoder_module.last_route
         # threshold activations make no survivor list at all on this route
         assert model.decoder_module.last_route.get("survivor_list", True) == (fn == "batchtopk")
+        acts_dense = model.get_feature_activations(inputs)        # (threshold models: the gated slab itself)
         model.decoder_module.dense_route = False
         sparse = model(inputs)
         assert model.decoder_module.last_route["dense_targets"] == (L, L)
         acts = {l: a.cpu() for l, a in model.get_feature_activations(inputs).items()}
+        for l in acts:
+            assert acts_dense[l].dtype == acts[l].dtype and torch.equal(acts_dense[l].cpu(), acts[l])
         assert float((acts[0] != 0).float().mean()) > 0.2
         # a subset of layers
         model.decoder_module.dense_route = True
