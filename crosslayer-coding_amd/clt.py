@@ -816,16 +816,24 @@ class CrossLayerTranscoder(BaseTranscoder):
             return None
         if self._thr_last_total is None or not inputs:
             return None
+        # the cheap questions first: this is asked on every forward of a threshold model
+        x0 = next(iter(inputs.values()))
+        if not isinstance(x0, torch.Tensor) or x0.dim() not in (2, 3):
+            return None
+        n, T, F = len(inputs), x0.numel() // max(1, x0.shape[-1]), cfg.num_features
+        key = (fn, tuple(sorted(inputs)), T, self.dtype)
+        if key != self._thr_key:
+            return None
+        self._poll_threshold_runs()
+        if self._thr_last_total is None:
+            return None
+        if not self.decoder_module.dense_pairs_wanted_for(self._thr_last_total / n, T, self.dtype, None):
+            return None
         prep = self.encoder_module.prepare_slab(inputs)
         if prep is None:
             return None
         layers, x_slab, w_slab, b_slab = prep
-        n, T, F = len(layers), x_slab.shape[1], cfg.num_features
-        key = (fn, tuple(layers), T, self.dtype)
-        if key != self._thr_key:
-            return None
-        self._poll_threshold_runs()
-        if not self.decoder_module.dense_pairs_wanted_for(self._thr_last_total / n, T, self.dtype, None):
+        if x_slab.shape[1] != T:
             return None
         pre = engine.encode(x_slab, w_slab, b_slab, out=self._workspace().typed(buffer, (n, T, F), self.dtype))
         theta = None
