@@ -304,9 +304,12 @@ class CrossLayerTranscoder(BaseTranscoder):
         ws = self._workspace()
         mask = (1 << L) - 1
         dec = self.decoder_module
-        if dec.skip_weights is None and dec.dense_pairs_wanted(surv, None, any_tying=True):
-            # so many survivors that the reference's dense products are the cheaper formulation (the decoder step is
-            # then not fused: ``dec_w`` is returned and the optimiser applies it)
+        affine = dec.feature_offset is not None or dec.feature_scale is not None
+        too_wide = d > engine.BACKWARD_MAX_D_MODEL and not affine      # rows beyond what the list kernels hold per lane
+        if dec.skip_weights is None and (too_wide or dec.dense_pairs_wanted(surv, None, any_tying=True)):
+            # so many survivors that the reference's dense products are the cheaper formulation, or a d_model the
+            # survivor-list kernels do not take (the decoder step is then not fused: ``dec_w`` is returned and the
+            # optimiser applies it)
             return self._raw_gradients_dense(inputs, surv, g, g_model, bias_grad)
         off, sc = dec._affine()                     # per-target feature offset / scale of tied decoders, or None
         dval = engine.decode_backward_values(surv, dec.packed(), g, cfg.decoder_tying, mask, ws, feat_scale=sc)

@@ -406,6 +406,10 @@ class Decoder(nn.Module):
         # shapes the MFMA kernel of clt_encode takes (K = F in whole 128-byte stages, 256 x 256 tiles)
         if surv.dtype not in (torch.bfloat16, torch.float16, torch.float32) or T < 256 or d < 256 or d % 4 or F % (128 // esize):
             return t_end
+        if engine.decode_route(T, d, F, cfg.num_layers, cfg.decoder_tying, surv.dtype) == nat.ROUTE_GENERIC:
+            # rows wider than the gather kernels of this tying hold (d_model beyond 2560 in 16-bit elements): the
+            # generic kernel that would serve them is two orders of magnitude slower than the product
+            return t_begin
         gather_rate, mfma_rate = self.route_rates(T, F, d, surv.dtype)
         dense_s = 2.0 * T * F * d / mfma_rate
         per_layer = self._survivors_per_layer(surv)
@@ -453,6 +457,8 @@ class Decoder(nn.Module):
         esize = torch.finfo(dtype).bits // 8
         if dtype not in (torch.bfloat16, torch.float16, torch.float32) or T < 256 or d < 256 or d % 4 or F % (128 // esize):
             return False
+        if engine.decode_route(T, d, F, cfg.num_layers, cfg.decoder_tying, dtype) == nat.ROUTE_GENERIC:
+            return True                 # rows no gather kernel holds (wide and not whole cache lines): the product
         if per_layer < 0.004 * T * F:
             return False                # no plausible pair of rates sends so sparse a batch to the product
         if self.rate_override is None and torch.cuda.is_current_stream_capturing():

@@ -120,6 +120,9 @@ def _wants_sliced_decode(rows: int, slab_bytes: int) -> bool:
 
 # token rows of one tile of the matrix-core encoder: shorter batches are padded to it (see ``encode``)
 ENCODE_MIN_TOKENS = 256
+# widest d_model the gradient kernels that walk survivor lists take (a row is held by one wavefront, up to eight
+# 16-byte pieces per lane in bf16); wider models get their gradients from the dense formulation
+BACKWARD_MAX_D_MODEL = 4096
 # below this many multiply-adds a shape the matrix-core encoder does not take stays on the generic kernel (about
 # 0.2 ms there); above it the operands are zero-padded to a shape it takes (see ``encode``)
 ENCODE_PAD_MIN_MACS = 5e7

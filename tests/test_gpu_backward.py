@@ -689,3 +689,34 @@ def test_gradients_on_the_dense_route_at_high_density(dev, dtype, case, tying):
     for k in sa:
         assert torch.equal(sa[k], sb[k]), k
     assert not torch.equal(sa["encoder_module.encoders.0.weight"].cpu(), sd["encoder_module.encoders.0.weight"])
+
+
+@pytest.mark.parametrize("tying", ["none", "per_target"])
+def test_models_wider_than_the_list_kernels_train_through_the_dense_formulation(dev, tying):
+    """d_model = 4352 > 4096: the gradient kernels that walk survivor lists do not hold such rows; loss and gradients
+    come from the dense formulation at any density, against autograd through the oracle.  Decoders tied per target
+    of that width also decode through the dense products (no gather kernel of that tying holds the rows)."""
+    wl = BASE.scaled("wide", num_layers=2, d_model=4352, num_features=512, tokens=300, k=8, dtype="bfloat16", decoder_tying=tying)
+    model, sd, x, targets = build(wl, dev)
+    L = wl.num_layers
+    inputs = {l: x[l].to(dev) for l in range(L)}
+    calls = []
+    real = model._raw_gradients_dense
+    model._raw_gradients_dense = lambda *a, **kw: (calls.append(1), real(*a, **kw))[1]
+    loss, grads = model.loss_and_gradients(inputs, {l: t.to(dev) for l, t in targets.items()})
+    assert calls
+    if tying == "per_target":
+        assert model.decoder_module.last_route["dense_targets"] == (0, L)
+    masks = {l: (a != 0).cpu() for l, a in model.get_feature_activations(inputs).items()}
+    names = synth.decoder_names(wl)
+    ref_loss, ref = orc.mse_loss_and_gradients(
+        {l: x[l] for l in range(L)}, targets,
+        enc_w=[sd[f"encoder_module.encoders.{l}.weight"] for l in range(L)],
+        enc_b=[sd[f"encoder_module.encoders.{l}.bias_param"] for l in range(L)],
+        dec_w={n: sd[f"decoder_module.decoders.{n}.weight"] for n in names},
+        dec_b={n: sd[f"decoder_module.decoders.{n}.bias_param"] for n in names},
+        activation_fn="batchtopk", num_layers=L, k=wl.k, theta=None, masks=masks, tying=tying, log_threshold=None,
+        model_dtype=torch.bfloat16)
+    assert abs(float(loss) - float(ref_loss)) <= 0.1 * abs(float(ref_loss)) * TOL[torch.bfloat16] * 10
+    for name, gref in ref.items():
+        assert orc.rel_l2(grads[name].float().cpu(), gref) <= 5 * TOL[torch.bfloat16], name
