@@ -87,7 +87,7 @@ class _ReconstructionsWithGraph(torch.autograd.Function):
         return (None, None, None, *grads)
 
 
-MAX_LAYERS = 64     # layers of one model (the kernels' source-layer masks are 64 bits wide)
+MAX_LAYERS = Decoder.MAX_GATHER_LAYERS     # beyond: dense formulations only
 
 
 class CrossLayerTranscoder(BaseTranscoder):
@@ -99,10 +99,12 @@ class CrossLayerTranscoder(BaseTranscoder):
         super().__init__(config)
         require_single_rank(process_group)
         if config.num_layers > MAX_LAYERS:
-            # said here, not by the first forward: the decode and gradient kernels keep the set of layers a batch
-            # has inputs for in one 64-bit word
-            raise NotImplementedError(f"num_layers = {config.num_layers}: the HIP kernels of this build take at most "
-                                      f"{MAX_LAYERS} layers")
+            # said here, not by the first forward: the gather and survivor-list kernels keep the set of layers a batch
+            # has inputs for in one 64-bit word; a deeper model decodes and trains through the dense products, which
+            # cover neither skip connections nor TokenTopK's per-layer counters
+            if config.skip_connection or config.activation_fn == "topk":
+                raise NotImplementedError(f"num_layers = {config.num_layers} > {MAX_LAYERS} together with "
+                                          f"{'skip connections' if config.skip_connection else 'TokenTopK'}: not built")
         self.process_group = process_group
         self.world_size, self.rank = 1, 0
         self.profiler = profiler
@@ -306,6 +308,9 @@ class CrossLayerTranscoder(BaseTranscoder):
         dec = self.decoder_module
         affine = dec.feature_offset is not None or dec.feature_scale is not None
         too_wide = d > engine.BACKWARD_MAX_D_MODEL and not affine      # rows beyond what the list kernels hold per lane
+        if L > MAX_LAYERS and affine:
+            raise NotImplementedError(f"num_layers = {L} > {MAX_LAYERS} with a feature offset / scale: the gradients of "
+                                      "such models come from the dense formulation, which does not cover them")
         if dec.skip_weights is None and (too_wide or dec.dense_pairs_wanted(surv, None, any_tying=True)):
             # so many survivors that the reference's dense products are the cheaper formulation, or a d_model the
             # survivor-list kernels do not take (the decoder step is then not fused: ``dec_w`` is returned and the

@@ -399,6 +399,8 @@ class Decoder(nn.Module):
         decoders have no such sum - each (source, target) pair has its own operand or its own matrix - and go dense
         only at high densities (``dense_pairs_wanted``)."""
         cfg = self.config
+        if cfg.decoder_tying == "per_target" and self._beyond_gather_layers(skip_add, affine_ok=True):
+            return t_begin
         if cfg.decoder_tying != "per_target" or not self.dense_route or skip_add is not None:
             return t_end
         T, F, d = surv.T, surv.F, cfg.d_model
@@ -432,6 +434,21 @@ class Decoder(nn.Module):
 
     # a (source, target) pair goes to the dense product when its gather is priced this many times dearer
     DENSE_PAIR_MARGIN = 1.25
+    # layers the gather and survivor-list kernels take (the set of source layers a batch has inputs for travels
+    # through them as one 64-bit word); deeper models run on the dense formulations only
+    MAX_GATHER_LAYERS = 64
+
+    def _beyond_gather_layers(self, skip_add: Optional[torch.Tensor], affine_ok: bool) -> bool:
+        """True for a model of more layers than the gather kernels take: its decode and gradients are the dense
+        products whatever the density (what the reference runs).  Raises for what those do not cover."""
+        if self.config.num_layers <= self.MAX_GATHER_LAYERS:
+            return False
+        affine = self.feature_offset is not None or self.feature_scale is not None
+        if skip_add is not None or self.skip_weights is not None or (affine and not affine_ok):
+            raise NotImplementedError(
+                f"num_layers = {self.config.num_layers} > {self.MAX_GATHER_LAYERS}: such models run on the dense products, "
+                "which do not cover skip connections" + ("" if affine_ok else " or the per-target feature offset / scale"))
+        return True
 
     def dense_pairs_wanted(self, surv: SurvivorList, skip_add: Optional[torch.Tensor], any_tying: bool = False) -> bool:
         """Untied and per-source decoders at densities the survivor gather was not made for (a ReLU model, JumpReLU
@@ -439,6 +456,8 @@ class Decoder(nn.Module):
         fetches a decoder row per target, k T rows of d elements, while the reference's dense product
         ``a[s] @ W[s->t].T`` (decoder.py:253-316) costs 2 T F d whatever the density.  With the measured rates of
         ``route_rates`` the product wins above roughly 1.5 - 2 % of the features active per token."""
+        if self.config.num_layers > self.MAX_GATHER_LAYERS:
+            return self.dense_pairs_wanted_for(0.0, surv.T, surv.dtype, skip_add, any_tying)
         if surv.nnz_hint is None and surv.status is not None:
             return False                # a threshold list of unknown size (first forward of a shape): the gather
         return self.dense_pairs_wanted_for(self._survivors_per_layer(surv), surv.T, surv.dtype, skip_add, any_tying)
@@ -449,7 +468,11 @@ class Decoder(nn.Module):
         ``any_tying``: decoders tied per target included (their forward has its own rule, ``dense_split``; the
         gradients ask here)."""
         cfg = self.config
-        if (cfg.decoder_tying == "per_target" and not any_tying) or not self.dense_route or skip_add is not None:
+        if cfg.decoder_tying == "per_target" and not any_tying:
+            return False
+        if self._beyond_gather_layers(skip_add, affine_ok=False):
+            return True
+        if not self.dense_route or skip_add is not None:
             return False
         if self.feature_offset is not None or self.feature_scale is not None:
             return False

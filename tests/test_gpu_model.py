@@ -485,3 +485,46 @@ def test_inference_forward_replays_from_a_graph(dev, kw):
             torch.cuda.synchronize()
             for l in want:
                 assert torch.equal(got[l], want[l]), (rep, l)
+
+
+@pytest.mark.parametrize("tying,fn", [("per_target", "batchtopk"), ("per_source", "jumprelu"), ("none", "batchtopk")])
+def test_more_than_64_layers_run_on_the_dense_formulations(dev, tying, fn):
+    """The gather and survivor-list kernels take 64 layers; a deeper model decodes and trains through the dense
+    products at any density.  Forward against the oracle; loss and gradients against autograd through the oracle."""
+    L = 66
+    wl = BASE.scaled("deep", num_layers=L, d_model=32, num_features=64, tokens=20, k=4 if fn == "batchtopk" else None,
+                     activation_fn=fn, decoder_tying=tying)
+    model, sd, x = build(wl, dev)
+    inputs = {l: x[l].to(dev) for l in range(L)}
+    with torch.no_grad():
+        recs = model(inputs)
+        recs = model(inputs)        # (a threshold model knows its density from the second forward on)
+    assert model.decoder_module.last_route["dense_targets"] == (0, L)
+    ref_recs, _ = oracle_forward(wl, sd, x)
+    for t in (0, 1, 31, 64, 65):
+        assert orc.rel_l2(recs[t], ref_recs[t]) <= 1e-5, t
+    g = torch.Generator().manual_seed(6)
+    targets = {l: torch.randn(wl.tokens, wl.d_model, generator=g) for l in range(L)}
+    loss, grads = model.loss_and_gradients(inputs, {l: t.to(dev) for l, t in targets.items()})
+    names = synth.decoder_names(wl)
+    theta = log_theta = masks = None
+    if fn == "jumprelu":
+        theta = torch.exp(sd["theta_manager.log_threshold"].float())
+        log_theta = sd["theta_manager.log_threshold"]
+    ref_loss, ref = orc.mse_loss_and_gradients(
+        {l: x[l] for l in range(L)}, targets,
+        enc_w=[sd[f"encoder_module.encoders.{l}.weight"] for l in range(L)],
+        enc_b=[sd[f"encoder_module.encoders.{l}.bias_param"] for l in range(L)],
+        dec_w={n: sd[f"decoder_module.decoders.{n}.weight"] for n in names},
+        dec_b={n: sd[f"decoder_module.decoders.{n}.bias_param"] for n in names},
+        activation_fn=fn, num_layers=L, k=wl.k, theta=theta, masks=masks, tying=tying, log_threshold=log_theta,
+        model_dtype=torch.float32)
+    assert abs(float(loss) - float(ref_loss)) <= 1e-4 * abs(float(ref_loss))
+    for name in (f"encoder_module.encoders.0.weight", f"encoder_module.encoders.{L - 1}.bias_param",
+                 f"decoder_module.decoders.{names[0]}.weight", f"decoder_module.decoders.{names[-1]}.weight",
+                 f"decoder_module.decoders.{names[len(names) // 2]}.bias_param"):
+        assert orc.rel_l2(grads[name].float().cpu(), ref[name]) <= (1e-3 if name.endswith("log_threshold") else 2e-5), name
+    opt = cca.CLTAdam(model, lr=1e-3)
+    before = model.state_dict()["encoder_module.encoders.3.weight"].clone()
+    model.training_step(inputs, {l: t.to(dev) for l, t in targets.items()}, opt)
+    assert not torch.equal(model.state_dict()["encoder_module.encoders.3.weight"], before)
