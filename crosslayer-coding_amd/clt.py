@@ -100,11 +100,10 @@ class CrossLayerTranscoder(BaseTranscoder):
         require_single_rank(process_group)
         if config.num_layers > MAX_LAYERS:
             # said here, not by the first forward: the gather and survivor-list kernels keep the set of layers a batch
-            # has inputs for in one 64-bit word; a deeper model decodes and trains through the dense products, which
-            # cover neither skip connections nor TokenTopK's per-layer counters
-            if config.skip_connection or config.activation_fn == "topk":
-                raise NotImplementedError(f"num_layers = {config.num_layers} > {MAX_LAYERS} together with "
-                                          f"{'skip connections' if config.skip_connection else 'TokenTopK'}: not built")
+            # has inputs for in one 64-bit word; a deeper model decodes and trains through the dense products
+            # (TokenTopK's selection keeps per-layer counters of the same width)
+            if config.activation_fn == "topk":
+                raise NotImplementedError(f"num_layers = {config.num_layers} > {MAX_LAYERS} together with TokenTopK: not built")
         self.process_group = process_group
         self.world_size, self.rank = 1, 0
         self.profiler = profiler
@@ -267,15 +266,14 @@ class CrossLayerTranscoder(BaseTranscoder):
         L, d, F = cfg.num_layers, cfg.d_model, cfg.num_features
         if sorted(inputs) != list(range(L)) or sorted(targets) != list(range(L)):
             raise ValueError("loss_and_gradients needs inputs and targets for every layer")
-        dense = None
-        if self.decoder_module.skip_weights is None:
-            dense = self._dense_threshold_activations(inputs, "dense_acts")
+        dense = self._dense_threshold_activations(inputs, "dense_acts")
         if dense is not None:
             # a threshold model in the dense regime: no survivor list, forward and gradients on dense operands
             acts = dense[1]
             ws = self._workspace()
             dec = self.decoder_module
-            rec = dec._decode_dense_pairs(None, (1 << L) - 1, 0, L, ws, dense={l: acts[l] for l in range(L)})
+            skip = dec.skip_all_targets(inputs, (1 << L) - 1, acts.shape[1]) if cfg.skip_connection else None
+            rec = dec._decode_dense_pairs(None, (1 << L) - 1, 0, L, ws, dense={l: acts[l] for l in range(L)}, skip_add=skip)
             dec.last_route = {"sparse_targets": (0, 0), "dense_targets": (0, L), "survivor_list": False}
             tgt = torch.stack([targets[l].to(device=self.device, dtype=self.dtype).reshape(-1, d) for l in range(L)])
             mode, mean, std, scale = self._denorm_args(normalization_method, mean_tg, std_tg)
@@ -311,7 +309,7 @@ class CrossLayerTranscoder(BaseTranscoder):
         if L > MAX_LAYERS and affine:
             raise NotImplementedError(f"num_layers = {L} > {MAX_LAYERS} with a feature offset / scale: the gradients of "
                                       "such models come from the dense formulation, which does not cover them")
-        if dec.skip_weights is None and (too_wide or dec.dense_pairs_wanted(surv, None, any_tying=True)):
+        if too_wide or dec.dense_pairs_wanted(surv, None, any_tying=True):
             # so many survivors that the reference's dense products are the cheaper formulation, or a d_model the
             # survivor-list kernels do not take (the decoder step is then not fused: ``dec_w`` is returned and the
             # optimiser applies it)
@@ -486,8 +484,15 @@ class CrossLayerTranscoder(BaseTranscoder):
             dec_b = torch.flip(torch.cumsum(torch.flip(bias_grad, dims=[0]), dim=0), dims=[0])
         else:
             dec_b = bias_grad
+        d_skip = None
+        if dec.skip_weights is not None:
+            # rec[t] += x[s] @ W_skip[s->t].T (untied, every pair) or x[t] @ W_skip[t].T (tied): dW = g[t].T @ x
+            pairs = [(s_, t) for s_ in range(L) for t in range(s_, L)] if tying == "none" else [(t, t) for t in range(L)]
+            d_skip = torch.empty((len(pairs), d, d), dtype=torch.float32, device=dev)
+            for i, (s_, t) in enumerate(pairs):
+                engine.skip_weight_grad(g[t], x_slab[s_], d_skip[i])
         return {"enc_w": dw_enc, "enc_b": db_enc, "dec_w": dw_dec, "dec_b": dec_b.contiguous(), "theta": theta_grad,
-                "skip": None, "feat_offset": None, "feat_scale": None}
+                "skip": d_skip, "feat_offset": None, "feat_scale": None}
 
     @torch.no_grad()
     def loss_and_gradients(self, inputs: Dict[int, torch.Tensor], targets: Dict[int, torch.Tensor],
@@ -820,7 +825,7 @@ class CrossLayerTranscoder(BaseTranscoder):
         survivor total last seen for this shape sends the decode to its dense products, else None."""
         cfg = self.config
         fn = cfg.activation_fn
-        if fn not in ("jumprelu", "relu") or cfg.skip_connection or torch.cuda.is_current_stream_capturing():
+        if fn not in ("jumprelu", "relu") or torch.cuda.is_current_stream_capturing():
             return None
         if self._thr_last_total is None or not inputs:
             return None
@@ -872,8 +877,9 @@ class CrossLayerTranscoder(BaseTranscoder):
         src_mask = 0
         for l in layers:
             src_mask |= 1 << l
+        skip = dec.skip_all_targets(inputs, src_mask, pre.shape[1]) if self.config.skip_connection else None
         out = dec._decode_dense_pairs(None, src_mask, min(layers), max(layers) + 1, ws,
-                                      dense={l: pre[i] for i, l in enumerate(layers)})
+                                      dense={l: pre[i] for i, l in enumerate(layers)}, skip_add=skip)
         dec.last_route = {"sparse_targets": (min(layers), min(layers)), "dense_targets": (min(layers), max(layers) + 1),
                           "survivor_list": False}
         return {t: out[t] for t in layers}

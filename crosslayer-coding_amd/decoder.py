@@ -401,7 +401,7 @@ class Decoder(nn.Module):
         cfg = self.config
         if cfg.decoder_tying == "per_target" and self._beyond_gather_layers(skip_add, affine_ok=True):
             return t_begin
-        if cfg.decoder_tying != "per_target" or not self.dense_route or skip_add is not None:
+        if cfg.decoder_tying != "per_target" or not self.dense_route:
             return t_end
         T, F, d = surv.T, surv.F, cfg.d_model
         esize = torch.finfo(surv.dtype).bits // 8
@@ -444,10 +444,10 @@ class Decoder(nn.Module):
         if self.config.num_layers <= self.MAX_GATHER_LAYERS:
             return False
         affine = self.feature_offset is not None or self.feature_scale is not None
-        if skip_add is not None or self.skip_weights is not None or (affine and not affine_ok):
+        if affine and not affine_ok:
             raise NotImplementedError(
                 f"num_layers = {self.config.num_layers} > {self.MAX_GATHER_LAYERS}: such models run on the dense products, "
-                "which do not cover skip connections" + ("" if affine_ok else " or the per-target feature offset / scale"))
+                "which cover the per-target feature offset / scale only in the forward of decoders tied per target")
         return True
 
     def dense_pairs_wanted(self, surv: SurvivorList, skip_add: Optional[torch.Tensor], any_tying: bool = False) -> bool:
@@ -472,7 +472,7 @@ class Decoder(nn.Module):
             return False
         if self._beyond_gather_layers(skip_add, affine_ok=False):
             return True
-        if not self.dense_route or skip_add is not None:
+        if not self.dense_route:
             return False
         if self.feature_offset is not None or self.feature_scale is not None:
             return False
@@ -492,8 +492,15 @@ class Decoder(nn.Module):
         gather_s = per_layer * d * esize / gather_rate
         return gather_s > self.DENSE_PAIR_MARGIN * 2.0 * T * F * d / mfma_rate
 
+    @staticmethod
+    def _add_skip(out: torch.Tensor, skip_add: Optional[torch.Tensor], t_begin: int, t_end: int) -> None:
+        """out[t] += the skip-connection terms (fp32 [L, T, d], ``skip_all_targets``) of the targets [t_begin, t_end)."""
+        if skip_add is not None and t_end > t_begin:
+            out[t_begin:t_end] = (out[t_begin:t_end].float() + skip_add[t_begin:t_end]).to(out.dtype)
+
     def _decode_dense_pairs(self, surv: Optional[SurvivorList], src_mask: int, t_begin: int, t_end: int, ws,
-                            dense: Optional[Dict[int, torch.Tensor]] = None) -> torch.Tensor:
+                            dense: Optional[Dict[int, torch.Tensor]] = None,
+                            skip_add: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Targets [t_begin, t_end) of untied or per-source decoders as the reference's dense products: per source
         layer the survivors are scattered into a dense [T, F] operand, one launch of the matrix-core kernel
         multiplies it with the decoders of all its targets (checkpoint layout [d, F], bias included, one rounding
@@ -536,6 +543,7 @@ class Decoder(nn.Module):
                 out[lo:t_end] += prod
             else:
                 out[lo:t_end] += prod[0]
+        self._add_skip(out, skip_add, t_begin, t_end)
         return out
 
     def _decode_dense(self, surv: SurvivorList, src_mask: int, t_first: int, t_end: int, out: torch.Tensor, ws) -> None:
@@ -580,13 +588,14 @@ class Decoder(nn.Module):
         t_end = cfg.num_layers if t_end is None else t_end
         if self.dense_pairs_wanted(surv, skip_add):
             self.last_route = {"sparse_targets": (t_begin, t_begin), "dense_targets": (t_begin, t_end)}
-            return self._decode_dense_pairs(surv, src_mask, t_begin, t_end, ws)
+            return self._decode_dense_pairs(surv, src_mask, t_begin, t_end, ws, skip_add=skip_add)
         split = self.dense_split(surv, src_mask, t_begin, t_end, skip_add)
         self.last_route = {"sparse_targets": (t_begin, split), "dense_targets": (split, t_end)}
         out = None
         if split < t_end:
             out = torch.empty((surv.L, surv.T, cfg.d_model), dtype=surv.dtype, device=surv.row_ptr.device)
             self._decode_dense(surv, src_mask, split, t_end, out, ws)
+            self._add_skip(out, skip_add, split, t_end)
             if split == t_begin:
                 return out
         off, sc = self._affine()

@@ -225,3 +225,40 @@ def test_threshold_dense_gates_in_place_and_counts(dev, dtype, L, T, F):
         iv = torch.int32 if dtype == torch.float32 else torch.int16
         assert torch.equal(buf.cpu().view(iv), want.view(iv))
         assert int(total) == int(keep.sum())
+
+
+@pytest.mark.parametrize("tying", ["none", "per_source", "per_target"])
+def test_dense_routes_carry_skip_connections(dev, tying):
+    """A ReLU model with skip connections at 50 % density: reconstructions, loss and every gradient (skip matrices
+    included) of the dense routes against the gather / survivor-list routes of the same model."""
+    wl = synth.Workload("dense-skip", 8, 3, 256, 512, 320, "float32", activation_fn="relu", k=None, decoder_tying=tying)
+    cfg = wl.config()
+    cfg.skip_connection = True
+    x = synth.make_inputs(wl, "cpu")
+    sd = synth.make_state_dict(wl, "cpu", inputs=x)
+    model = cca.CrossLayerTranscoder(cfg, None, dev)
+    missing = [k for k in model.state_dict() if k not in sd]
+    g = torch.Generator().manual_seed(4)
+    for k in missing:                                   # the skip matrices
+        sd[k] = torch.randn(model.state_dict()[k].shape, generator=g) * 0.05
+    model.load_state_dict(sd)
+    model.decoder_module.rate_override = (14.5e12, 1.0e14)
+    L = wl.num_layers
+    inputs = {l: x[l].to(dev) for l in range(L)}
+    targets = {l: torch.randn(wl.tokens, wl.d_model, generator=g).to(dev) for l in range(L)}
+    with torch.no_grad():
+        model(inputs); torch.cuda.synchronize(); model(inputs); torch.cuda.synchronize()
+        dense = model(inputs)
+        assert model.decoder_module.last_route["dense_targets"][1] == L and model.decoder_module.last_route["dense_targets"][0] < L
+    loss_d, grads_d = model.loss_and_gradients(inputs, targets)
+    model.decoder_module.dense_route = False
+    with torch.no_grad():
+        sparse = model(inputs)
+        assert model.decoder_module.last_route["dense_targets"] == (L, L)
+    loss_s, grads_s = model.loss_and_gradients(inputs, targets)
+    for t in range(L):
+        assert orc.rel_l2(dense[t].cpu(), sparse[t].cpu()) <= 1e-5, t
+    assert abs(float(loss_d) - float(loss_s)) <= 1e-5 * abs(float(loss_s))
+    assert any("skip_weights" in k for k in grads_d)
+    for k in grads_s:
+        assert orc.rel_l2(grads_d[k].float().cpu(), grads_s[k].float().cpu()) <= 2e-5, k
