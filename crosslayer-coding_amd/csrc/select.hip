@@ -37,6 +37,7 @@ constexpr int SAMPLE_BLOCKS = 16;        // blocks per problem that gather the s
 constexpr int SCAN_THREADS = 1024;
 constexpr int WBUF = 512;                // candidate entries buffered in LDS per wavefront
 constexpr int PASS_NV = 4;               // 16-byte loads in flight per lane in the pass
+constexpr int TOK_MAX_LAYERS = 1024;         // layers of a TokenTopK problem (per-layer counters in LDS)
 constexpr uint32_t ROW_NONE = 0xFFFFFFFFu;   // row has no candidates
 constexpr uint32_t ROW_DENSE = 0xFFFFFFFEu;  // row did not fit the pool: read it from the matrix
 
@@ -1152,7 +1153,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_token_threshold(
   constexpr int KB = Elem<T>::KEYBITS;
   constexpr int NLEV = KB == 32 ? 3 : 2;
   __shared__ uint32_t lh[NBINS];
-  __shared__ uint32_t cnt_gt[64], cnt_eq[64];
+  __shared__ uint32_t cnt_gt[TOK_MAX_LAYERS], cnt_eq[TOK_MAX_LAYERS];   // per layer of a token's global problem
   const int tid = threadIdx.x;
   // per-layer: problem = (layer, token); global: problem = token
   const int64_t prob = blockIdx.x;
@@ -1185,7 +1186,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_token_threshold(
     prefix_mask |= dm << sh;
   }
   const uint32_t thr = prefix;          // key of the kk-th largest entry; k_rem ties survive
-  if (tid < 64) { cnt_gt[tid] = 0; cnt_eq[tid] = 0; }
+  for (int i = tid; i < TOK_MAX_LAYERS; i += SCAN_THREADS) { cnt_gt[i] = 0; cnt_eq[i] = 0; }
   __syncthreads();
   for (int li = 0; li < nl; ++li) {
     const int64_t l = l0 + li;
@@ -2030,7 +2031,7 @@ extern "C" int clt_tokentopk_select(const void *pre, int64_t T, int64_t F, int64
                                     int32_t *row_ptr, int32_t *col, void *val, void *workspace,
                                     size_t workspace_bytes, void *stream) {
   if (!clt_model_dtype(dtype)) return CLT_ERR_DTYPE;
-  if (T < 0 || F < 0 || L <= 0 || L > 64 || !row_ptr) return CLT_ERR_ARG;
+  if (T < 0 || F < 0 || L <= 0 || L > TOK_MAX_LAYERS || !row_ptr) return CLT_ERR_ARG;
   if (mode != CLT_TOPK_PER_LAYER && mode != CLT_TOPK_GLOBAL) return CLT_ERR_ARG;
   hipStream_t s = (hipStream_t)stream;
   const int64_t R = L * T;

@@ -487,13 +487,16 @@ def test_inference_forward_replays_from_a_graph(dev, kw):
                 assert torch.equal(got[l], want[l]), (rep, l)
 
 
-@pytest.mark.parametrize("tying,fn", [("per_target", "batchtopk"), ("per_source", "jumprelu"), ("none", "batchtopk")])
+@pytest.mark.parametrize("tying,fn", [("per_target", "batchtopk"), ("per_source", "jumprelu"), ("none", "batchtopk"),
+                                      ("per_source", "topk-global")])
 def test_more_than_64_layers_run_on_the_dense_formulations(dev, tying, fn):
     """The gather and survivor-list kernels take 64 layers; a deeper model decodes and trains through the dense
     products at any density.  Forward against the oracle; loss and gradients against autograd through the oracle."""
     L = 66
-    wl = BASE.scaled("deep", num_layers=L, d_model=32, num_features=64, tokens=20, k=4 if fn == "batchtopk" else None,
-                     activation_fn=fn, decoder_tying=tying)
+    mode = "global" if fn == "topk-global" else "per_layer"
+    fn = fn.split("-")[0]
+    wl = BASE.scaled("deep", num_layers=L, d_model=32, num_features=64, tokens=20, k=4 if fn != "jumprelu" else None,
+                     activation_fn=fn, decoder_tying=tying, topk_mode=mode)
     model, sd, x = build(wl, dev)
     inputs = {l: x[l].to(dev) for l in range(L)}
     with torch.no_grad():
@@ -511,6 +514,8 @@ def test_more_than_64_layers_run_on_the_dense_formulations(dev, tying, fn):
     if fn == "jumprelu":
         theta = torch.exp(sd["theta_manager.log_threshold"].float())
         log_theta = sd["theta_manager.log_threshold"]
+    if fn == "topk":
+        masks = {l: (a != 0).cpu() for l, a in model.get_feature_activations(inputs).items()}
     ref_loss, ref = orc.mse_loss_and_gradients(
         {l: x[l] for l in range(L)}, targets,
         enc_w=[sd[f"encoder_module.encoders.{l}.weight"] for l in range(L)],
