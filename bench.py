@@ -545,6 +545,55 @@ def run_evaluator(args):
     }
 
 
+def run_dense_regime(args):
+    """The workload's shape as a JumpReLU model whose encoder biases are raised by ``--dense-regime`` (1.0: about a
+    quarter of the features fire per token, what a run trained from scratch starts at): forward and training step
+    on the dense routes (Decoder.dense_pairs_wanted).  One line: forward ms, training-step ms, density, routes."""
+    import crosslayer_coding_amd as cca
+    from crosslayer_coding_amd import synth
+
+    base = synth.WORKLOADS[args.workload]
+    wl = base.scaled(f"{base.name}-jumprelu-dense", activation_fn="jumprelu", k=None)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    cca._native.load(build_if_missing=False)
+    model, inputs, _ = synth.build_model(wl, dev)
+    with torch.no_grad():
+        for enc in model.encoder_module.encoders:
+            enc.bias_param.add_(args.dense_regime)
+    model.eval()
+    slab = synth.make_targets(wl, dev)
+    targets = {l: slab[l] for l in range(wl.num_layers)}
+
+    def timed(fn, warmup, steps):
+        for _ in range(warmup):
+            fn()
+            torch.cuda.synchronize()       # (the density of a threshold model is known one forward late)
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps * 1e3
+
+    with torch.no_grad():
+        acts = model.get_feature_activations(inputs)
+        density = float(sum((a != 0).float().mean() for a in acts.values())) / len(acts)
+        del acts
+        fwd_ms = timed(lambda: model(inputs), args.warmup, args.steps)
+        fwd_route = dict(model.decoder_module.last_route)
+    opt = cca.CLTAdam(model, lr=1e-4)
+    step_ms = timed(lambda: model.training_step(inputs, targets, opt), max(2, args.warmup // 2), max(3, args.steps // 4))
+    return {
+        "metric": "CLT forward and training step in the dense regime (JumpReLU, encoder biases raised)",
+        "value": wl.tokens / (fwd_ms * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": fwd_ms, "training_step_ms": step_ms, "density": density, "forward_route": fwd_route,
+        "training_route": dict(model.decoder_module.last_route), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": _dtname(wl.dtype), "data": "synthetic",
+        "config": {"workload": f"{wl.name}: L={wl.num_layers} d_model={wl.d_model} F={wl.num_features} T={wl.tokens} "
+                               f"jumprelu, encoder biases + {args.dense_regime}"},
+    }
+
+
 def run_backward(args):
     """Forward, MSE reconstruction loss and the gradients of every encoder / decoder parameter
     (CrossLayerTranscoder.loss_and_gradients); one step = one batch.  No optimizer step."""
@@ -733,6 +782,9 @@ def main():
                     help="time the evaluator's reductions on the survivor list of one batch")
     ap.add_argument("--train-step", action="store_true",
                     help="time full optimisation steps: forward, MSE loss, gradients, Adam update")
+    ap.add_argument("--dense-regime", type=float, default=None, metavar="BIAS_SHIFT",
+                    help="the workload's shape as a JumpReLU model with the encoder biases raised by this much: forward "
+                         "and training step at high density (the dense routes)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one 256 MiB elementwise copy (counter yardstick for profiled runs)")
     args = ap.parse_args()
@@ -743,7 +795,7 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a ROCm GPU", file=sys.stderr)
         sys.exit(2)
-    print(json.dumps(run_theta(args) if args.theta_estimation else run_evaluator(args) if args.evaluator else run_feed(args) if args.feed else run_probe(args) if args.gather_probe else run_backward(args) if (args.backward or args.train_step) else run_gpu(args)))
+    print(json.dumps(run_dense_regime(args) if args.dense_regime is not None else run_theta(args) if args.theta_estimation else run_evaluator(args) if args.evaluator else run_feed(args) if args.feed else run_probe(args) if args.gather_probe else run_backward(args) if (args.backward or args.train_step) else run_gpu(args)))
 
 
 if __name__ == "__main__":
